@@ -1,0 +1,113 @@
+/*
+ * C ABI of the MI355X (gfx950) kernels for llmpalooza's quantized linear-layer
+ * path. One enqueue-only launch per operation on a caller-owned hipStream_t
+ * (passed as void*): nothing here allocates, synchronizes or frees; every
+ * operand and scratch area is the caller's, and stays mapped until a fence
+ * after the launch has completed (src/kernels/ggml/launch.h:4-48,
+ * src/kernels/decode/products.h:48-51 of the reference).
+ *
+ * Return values follow src/kernels/ggml/mxfp8_cutlass.h:75-79:
+ *    0  queued;
+ *   >0  refused before anything was queued (the caller's kRejected);
+ *   <0  the runtime reported an error after work may have been queued (the
+ *       caller's kUnknown: it faults its launch context).
+ * llmp_hip_last_error() names the reason of the calling thread's last
+ * non-zero return.
+ *
+ * Sizes are bytes unless a comment says blocks or elements. "Q8_1 block" is
+ * {f16 d; f16 s; i8 qs[32]} = 36 bytes; Q8_0 is {f16 d; i8 qs[32]} = 34 bytes;
+ * Q4_K is {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} = 144 bytes
+ * (src/format/encoding.cc:110-116).
+ */
+#ifndef LLMP_HIP_H_
+#define LLMP_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml_type values of the weight encodings the kernels read. */
+enum { LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12 };
+/* VecQGlu, src/kernels/ggml/llmp_ops.h:1072. */
+enum { LLMP_GLU_NONE = 0, LLMP_GLU_SWIGLU = 1, LLMP_GLU_SWIGLU_CLAMP = 2, LLMP_GLU_GEGLU = 3 };
+/* Element types of unquantized activations. */
+enum { LLMP_X_F32 = 0, LLMP_X_BF16 = 1, LLMP_X_F16 = 2 };
+
+const char* llmp_hip_last_error(void);
+/* Compute units of the current device (the `sms` argument of the reference's
+ * Scratch/Run pairs). Negative on a runtime error. */
+int llmp_hip_compute_units(void);
+
+/* ------------------------------------------------------------------ llmp.q8_1
+ * Replaces quantize_row_q8_1_cuda as RunQuantizeQ8 calls it
+ * (src/kernels/ggml/vecq.cu:1095-1111; dispatch shape in
+ * third_party/patches/ggml/0010-llmp-q8-dispatch-descriptors.patch:604-611).
+ * x: rows x planes rows of k floats, row_stride / plane_stride floats apart.
+ * out: for each plane then row, padded_k / 32 Q8_1 blocks; blocks past k are zero.
+ * padded_k is k rounded up to 512 (src/kernels/ggml/llmp_ops.cc:2574-2576). */
+int llmp_hip_q8_1_quantize(const float* x, void* out, int64_t k, int64_t padded_k,
+                           int64_t row_stride, int64_t rows, int64_t planes, int64_t plane_stride,
+                           void* stream);
+
+/* ------------------------------------------------------------------ llmp.vecq
+ * The POD of src/kernels/ggml/vecq.h:22-41, field for field. Weight offsets
+ * count the weight type's blocks; activation offsets count Q8_1 blocks. */
+typedef struct llmp_vecq_desc {
+  const void* w;      /* weights (the up projection with a GLU) */
+  const void* g;      /* gate weights, or null */
+  const void* y;      /* Q8_1 activations */
+  const int32_t* ids; /* null: dense or grouped */
+  float* dst;
+  int ncols_x;       /* k */
+  int nrows;         /* n */
+  int stride_row;    /* weight blocks between rows */
+  int stride_expert; /* weight blocks between experts */
+  int y_token;       /* Q8_1 blocks between tokens' rows */
+  int y_slot;        /* between slots' rows (per-slot activations), else 0 */
+  int ids_stride;    /* ids between tokens */
+  int used;
+  int tokens;
+  int dst_token; /* floats */
+  int dst_slot;
+  int glu; /* LLMP_GLU_* */
+  float limit;
+} llmp_vecq_desc;
+
+/* Replaces LaunchVecQ (src/kernels/ggml/vecq.h:43-47, vecq.cu:1023-1094):
+ * variant -1 is the default for the shape; returns 1 for a variant the shape
+ * cannot take, as the reference returns false. tokens 1..16, used * tokens
+ * <= 128 when routed (src/kernels/ggml/llmp_ops.cc:2931-2948). */
+int llmp_hip_vecq(int type, const llmp_vecq_desc* d, int variant, void* stream);
+int llmp_hip_vecq_variants(void);
+const char* llmp_hip_vecq_variant_name(int variant);
+
+/* The same product over unquantized activations: each workgroup quantizes the
+ * tokens' rows to Q8_1 in LDS (the arithmetic of llmp_hip_q8_1_quantize, bit
+ * for bit) instead of reading d->y, which is ignored. x_token / x_slot are
+ * elements between tokens' and slots' rows (x_slot 0: every slot reads the
+ * token's row). This is the reference's in-kernel activation quantization
+ * (src/kernels/ggml/llmp_moe.cu:469-571) for the GGML block types. */
+typedef struct llmp_vecq_source {
+  const void* x;
+  int x_type; /* LLMP_X_* */
+  int64_t x_token;
+  int64_t x_slot;
+} llmp_vecq_source;
+int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant,
+                        void* stream);
+
+/* Test aid: the int32 sums of every (row, block) of a dense one-token product
+ * as the kernel's integer path computes them, added into `sums` (which the
+ * caller zeroes first): sums[(row * blocks + b) * per + i] with per = 1 for
+ * Q8_0 (sum of w * q) and 16 for Q4_K (eight sub-block sums of code * q, then
+ * eight of q; tests/unit/dsv4_fast_test.cc:185-191). */
+int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int32_t* sums, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* LLMP_HIP_H_ */

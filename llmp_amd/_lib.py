@@ -1,0 +1,83 @@
+"""ctypes binding of lib/libllmp_hip.so (include/llmp_hip.h).
+
+There is no fallback: if the library is missing, `load()` raises. torch is
+imported first so that the process holds one HIP runtime.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "lib", "libllmp_hip.so")
+
+TYPE_Q8_0 = 8
+TYPE_Q4_K = 12
+GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
+X_F32, X_BF16, X_F16 = 0, 1, 2
+
+
+class VecQDesc(C.Structure):
+    """llmp_vecq_desc: src/kernels/ggml/vecq.h:22-41 of the reference."""
+    _fields_ = [
+        ("w", C.c_void_p), ("g", C.c_void_p), ("y", C.c_void_p), ("ids", C.c_void_p),
+        ("dst", C.c_void_p),
+        ("ncols_x", C.c_int), ("nrows", C.c_int), ("stride_row", C.c_int),
+        ("stride_expert", C.c_int), ("y_token", C.c_int), ("y_slot", C.c_int),
+        ("ids_stride", C.c_int), ("used", C.c_int), ("tokens", C.c_int),
+        ("dst_token", C.c_int), ("dst_slot", C.c_int), ("glu", C.c_int), ("limit", C.c_float),
+    ]
+
+
+class VecQSource(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
+                ("x_slot", C.c_int64)]
+
+
+_i64, _vp, _int = C.c_int64, C.c_void_p, C.c_int
+
+# name -> (restype, argtypes): every symbol include/llmp_hip.h declares.
+SYMBOLS = {
+    "llmp_hip_last_error": (C.c_char_p, []),
+    "llmp_hip_compute_units": (_int, []),
+    "llmp_hip_q8_1_quantize": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
+    "llmp_hip_vecq": (_int, [_int, C.POINTER(VecQDesc), _int, _vp]),
+    "llmp_hip_vecq_variants": (_int, []),
+    "llmp_hip_vecq_variant_name": (C.c_char_p, [_int]),
+    "llmp_hip_vecq_fused": (_int, [_int, C.POINTER(VecQDesc), C.POINTER(VecQSource), _int, _vp]),
+    "llmp_hip_vecq_block_sums": (_int, [_int, C.POINTER(VecQDesc), _vp, _vp]),
+}
+
+_lib = None
+
+
+class KernelFailure(RuntimeError):
+    """A refusal (rejected: nothing was queued) or a fault (unknown: work may be queued):
+    src/kernels/common/selected_operation.h:26-35 of the reference."""
+
+    def __init__(self, code, detail):
+        super().__init__(f"{'rejected' if code > 0 else 'unknown'} ({code}): {detail}")
+        self.code = code
+        self.rejected = code > 0
+        self.detail = detail
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(SO_PATH):
+        raise ImportError(
+            f"{SO_PATH} is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(make -C llmp_amd/csrc); there is no fallback path")
+    import torch  # noqa: F401  (its HIP runtime first)
+    lib = C.CDLL(SO_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        f = getattr(lib, name)
+        f.restype = res
+        f.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code):
+    if code != 0:
+        raise KernelFailure(code, load().llmp_hip_last_error().decode())

@@ -1,0 +1,68 @@
+// Shared host and device helpers of the gfx950 kernels.
+#ifndef LLMP_AMD_CSRC_COMMON_H_
+#define LLMP_AMD_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace llmp_hip {
+
+// ---- host: status of the calling thread's last refusal or fault.
+void SetError(const char* format, ...) __attribute__((format(printf, 1, 2)));
+// 0 if the last launch was accepted, else -(hipError_t) with the error recorded.
+int LaunchStatus(const char* what);
+int Refuse(int code, const char* format, ...) __attribute__((format(printf, 2, 3)));
+
+constexpr int kWave = 64;
+
+// ---- device: element conversions (src/kernels/device/float_formats.cuh:14-49).
+__device__ __forceinline__ float HalfBitsToFloat(uint32_t bits) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
+}
+__device__ __forceinline__ uint32_t FloatToHalfBits(float v) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));  // nearest even
+}
+__device__ __forceinline__ float Bf16BitsToFloat(uint32_t bits) {
+  return __builtin_bit_cast(float, bits << 16);
+}
+__device__ __forceinline__ uint32_t FloatToBf16Bits(float v) {
+  const uint32_t x = __builtin_bit_cast(uint32_t, v);
+  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x40u;
+  return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+}
+// E8M0: 2^(bits - 127); 0 is 2^-127 (a float subnormal), 0xFF NaN.
+__device__ __forceinline__ float E8m0ToFloat(uint32_t bits) {
+  if (bits == 0xFFu) return __builtin_nanf("");
+  return bits == 0 ? __builtin_bit_cast(float, 0x00400000u) : __builtin_bit_cast(float, bits << 23);
+}
+// OCP E4M3 (bias 7, 0x7F/0xFF NaN, subnormals m * 2^-9).
+__device__ __forceinline__ float E4m3ToFloat(uint32_t bits) {
+  const uint32_t magnitude = bits & 0x7Fu;
+  float v;
+  if (magnitude == 0x7Fu) {
+    v = __builtin_nanf("");
+  } else if (magnitude < 8u) {
+    v = static_cast<float>(magnitude) * 0.001953125f;
+  } else {
+    v = __builtin_bit_cast(float, (magnitude << 20) + (120u << 23));
+  }
+  return (bits & 0x80u) ? -v : v;
+}
+
+__device__ __forceinline__ int Dot4(int a, int b, int c) {
+  return __builtin_amdgcn_sdot4(a, b, c, false);
+}
+
+// A 16-byte and a 4-byte-aligned 16-byte global load of weights, which are
+// read once: non-temporal, so that they do not displace the activations.
+typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+typedef U32x4 U32x4A4 __attribute__((aligned(4)));
+
+template <typename T>
+__device__ __forceinline__ T ShflXor(T v, int mask) {
+  return __shfl_xor(v, mask, kWave);
+}
+
+}  // namespace llmp_hip
+
+#endif  // LLMP_AMD_CSRC_COMMON_H_

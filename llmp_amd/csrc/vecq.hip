@@ -1,0 +1,782 @@
+// llmp.q8_1 and llmp.vecq for gfx950: the Q8_1 activation quantizer and the
+// quantized mat-vec over Q8_0 / Q4_K weights (dense rows, grouped matrices,
+// routed experts; with or without a fused gate/up GLU; 1..16 tokens).
+//
+// Shape of the product kernel. A workgroup is 4 wave64s. The tokens of a pass
+// (P of them) are staged once into LDS as split Q8_1: the codes as a byte
+// stream (16-byte aligned per 32-value block), the block scales as floats and,
+// for Q4_K, the code sums of each 16-value half block. They come either from
+// Q8_1 blocks in memory or, in the fused form, from the unquantized rows,
+// quantized in the workgroup with the quantizer kernel's arithmetic. Then every
+// group of LPR lanes streams one weight row: a lane owns a fixed 16-byte slice
+// of each Q4_K super-block (two half sub-blocks of nibbles) or one pair of Q8_0
+// blocks (68 bytes, 4-byte aligned), loads it straight from global memory a few
+// units ahead of its use, multiplies it with the staged codes by v_dot4_i32_i8
+// and folds the scales in fp32. A (token, row) sum never depends on what else
+// the workgroup computes: per-lane sums in unit order, then a fixed xor
+// butterfly over the row's lanes. No atomics on the result path.
+//
+// Reference behaviour restated here: src/kernels/ggml/vecq.cu:457-665 (kernel
+// forms, pair ownership for routed experts), :186-195 (GLU), :398-418 (Q8_0
+// dot), tests/unit/dsv4_fast_test.cc:167-195 (Q4_K dot).
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr int kMaxPairs = 128;  // used * tokens of a routed product
+constexpr int kThreads = 256;
+constexpr int kQ8Block = 36;
+constexpr int kLdsBudget = 60 * 1024;
+
+// ------------------------------------------------------------- quantizer
+
+// Eight lanes quantize one 32-value block, four consecutive values a lane:
+// amax over the block, d = amax / 127 (IEEE), q = round-half-away(x / d), 0 for
+// a zero block. `sum` is the 32 values added in a 32-lane xor butterfly's order
+// (offsets 16, 8, 4, 2, 1 over one value a lane), whatever the lane mapping.
+struct Q8Block {
+  float d;
+  float sum;
+  uint32_t codes;  // four int8, the first value in the low byte
+};
+
+__device__ __forceinline__ Q8Block QuantizeQ8Block(float x0, float x1, float x2, float x3) {
+#pragma clang fp contract(off)
+  float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
+  amax = fmaxf(amax, ShflXor(amax, 4));
+  amax = fmaxf(amax, ShflXor(amax, 2));
+  amax = fmaxf(amax, ShflXor(amax, 1));
+  const float d = amax / 127.0f;
+  Q8Block out;
+  out.d = d;
+  int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+  if (amax != 0.0f) {
+    q0 = static_cast<int>(roundf(x0 / d));
+    q1 = static_cast<int>(roundf(x1 / d));
+    q2 = static_cast<int>(roundf(x2 / d));
+    q3 = static_cast<int>(roundf(x3 / d));
+  }
+  out.codes = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+  // value 4L + c pairs with 4(L ^ 4) + c at offset 16, 4(L ^ 2) + c at 8, 4(L ^ 1) + c at 4.
+  float s0 = x0, s1 = x1, s2 = x2, s3 = x3;
+#pragma unroll
+  for (int mask = 4; mask >= 1; mask >>= 1) {
+    s0 = s0 + ShflXor(s0, mask);
+    s1 = s1 + ShflXor(s1, mask);
+    s2 = s2 + ShflXor(s2, mask);
+    s3 = s3 + ShflXor(s3, mask);
+  }
+  out.sum = (s0 + s2) + (s1 + s3);
+  return out;
+}
+
+template <int XT>
+__device__ __forceinline__ void Load4(const void* base, int64_t at, int64_t k, float (&v)[4]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int64_t i = at + c;
+    float x = 0.0f;
+    if (i < k) {
+      if constexpr (XT == LLMP_X_F32) {
+        x = static_cast<const float*>(base)[i];
+      } else if constexpr (XT == LLMP_X_BF16) {
+        x = Bf16BitsToFloat(static_cast<const uint16_t*>(base)[i]);
+      } else {
+        x = HalfBitsToFloat(static_cast<const uint16_t*>(base)[i]);
+      }
+    }
+    v[c] = x;
+  }
+}
+
+// grid (ceil(blocks / 32), rows, planes), 256 threads: 32 blocks a workgroup.
+__global__ __launch_bounds__(kThreads) void QuantizeQ8Kernel(const float* __restrict__ x, uint8_t* __restrict__ out,
+                                                            int64_t k, int64_t padded_k, int64_t row_stride,
+                                                            int64_t rows, int64_t plane_stride) {
+  const int lane8 = threadIdx.x & 7;
+  const int64_t block = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int64_t blocks = padded_k / 32;
+  const int64_t row = blockIdx.y;
+  const int64_t plane = blockIdx.z;
+  // Whole 8-lane groups leave together: the shuffles below stay within a group.
+  if (block >= blocks) return;
+  const float* src = x + plane * plane_stride + row * row_stride;
+  float v[4];
+  Load4<LLMP_X_F32>(src, block * 32 + lane8 * 4, k, v);
+  const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+  uint8_t* dst = out + ((plane * rows + row) * blocks + block) * kQ8Block;
+  *reinterpret_cast<uint32_t*>(dst + 4 + lane8 * 4) = q.codes;
+  if (lane8 == 0) *reinterpret_cast<uint32_t*>(dst) = FloatToHalfBits(q.d) | (FloatToHalfBits(q.sum) << 16);
+}
+
+// ------------------------------------------------------------------ vecq
+
+struct VecQArgs {
+  llmp_vecq_desc d;
+  const void* x;  // fused form: unquantized rows
+  int64_t x_token;
+  int64_t x_slot;
+  int kp;         // k rounded up to 512: the staged codes' stride
+  int32_t* dump;  // block sums, or null
+};
+
+__device__ __forceinline__ float Silu(float x) {
+#pragma clang fp contract(off)
+  return x / (1.0f + expf(-x));
+}
+__device__ __forceinline__ float GeluTanh(float x) {
+#pragma clang fp contract(off)
+  return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+}
+// src/kernels/ggml/vecq.cu:186-195
+__device__ __forceinline__ float Glu(int glu, float gate, float up, float limit) {
+#pragma clang fp contract(off)
+  if (glu == LLMP_GLU_GEGLU) return GeluTanh(gate) * up;
+  if (glu == LLMP_GLU_SWIGLU_CLAMP) {
+    gate = fminf(gate, limit);
+    up = fmaxf(fminf(up, limit), -limit);
+  }
+  return Silu(gate) * up;
+}
+
+// The staged activations of a pass.
+struct Staged {
+  const uint8_t* codes;    // [P][kp]
+  const float* scales;     // [P][kp / 32]
+  const uint32_t* halves;  // [P][kp / 32]: Q4_K, per (super-block, lane slice) two int16 sums
+};
+
+// Stages token slot j from Q8_1 blocks in memory: a thread a block.
+template <bool kQ4K>
+__device__ __forceinline__ void StageQ8(const uint8_t* __restrict__ y, int blocks, int kp, int j, uint8_t* codes,
+                                        float* scales, uint32_t* halves) {
+  for (int b = threadIdx.x; b < blocks; b += kThreads) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+    uint4* dst = reinterpret_cast<uint4*>(codes + static_cast<int64_t>(j) * kp + b * 32);
+    dst[0] = make_uint4(w[1], w[2], w[3], w[4]);
+    dst[1] = make_uint4(w[5], w[6], w[7], w[8]);
+    scales[j * (kp / 32) + b] = HalfBitsToFloat(w[0] & 0xFFFFu);
+    if constexpr (kQ4K) {
+      int lo = 0, hi = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lo = Dot4(0x01010101, static_cast<int>(w[1 + i]), lo);
+        hi = Dot4(0x01010101, static_cast<int>(w[5 + i]), hi);
+      }
+      // Sub-block g = b % 8 of its super-block: slice 2(g / 2) + h, half g % 2.
+      auto* h16 = reinterpret_cast<int16_t*>(halves + j * (kp / 32));
+      const int at = ((b & ~7) + ((b & 7) >> 1) * 2) * 2 + (b & 1);
+      h16[at] = static_cast<int16_t>(lo);
+      h16[at + 2] = static_cast<int16_t>(hi);
+    }
+  }
+}
+
+// Stages token slot j from an unquantized row: eight lanes a block.
+template <bool kQ4K, int XT>
+__device__ __forceinline__ void StageX(const void* __restrict__ x, int k, int kp, int j, uint8_t* codes, float* scales,
+                                       uint32_t* halves) {
+  const int lane8 = threadIdx.x & 7;
+  const int blocks = k / 32;
+  for (int b = threadIdx.x >> 3; b < blocks; b += kThreads / 8) {
+    float v[4];
+    Load4<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, v);
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<uint32_t*>(codes + static_cast<int64_t>(j) * kp + b * 32 + lane8 * 4) = q.codes;
+    // The products read the scale as the Q8_1 block stores it: rounded to F16.
+    if (lane8 == 0) scales[j * (kp / 32) + b] = HalfBitsToFloat(FloatToHalfBits(q.d));
+    if constexpr (kQ4K) {
+      int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
+      s += ShflXor(s, 1);
+      s += ShflXor(s, 2);
+      if ((lane8 & 3) == 0) {
+        auto* h16 = reinterpret_cast<int16_t*>(halves + j * (kp / 32));
+        const int h = lane8 >> 2;
+        h16[((b & ~7) + ((b & 7) >> 1) * 2 + h) * 2 + (b & 1)] = static_cast<int16_t>(s);
+      }
+    }
+  }
+}
+
+// ---- Q4_K: a lane's 16-byte slice j of a super-block holds values
+// 16h .. 16h + 15 of sub-blocks 2p (low nibbles) and 2p + 1 (high), p = j / 2,
+// h = j % 2.
+struct Q4KUnit {
+  U32x4 header;  // d, dmin, scales[12]
+  U32x4 codes;
+};
+
+__device__ __forceinline__ Q4KUnit LoadQ4K(const uint8_t* row, int unit) {
+  const uint8_t* block = row + static_cast<int64_t>(unit >> 3) * 144;
+  Q4KUnit u;
+  u.header = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(block));
+  u.codes = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(block + 16 + (unit & 7) * 16));
+  return u;
+}
+
+struct Q4KScales {
+  float dsc0, dsc1, dm0, dm1;
+};
+
+__device__ __forceinline__ Q4KScales DecodeQ4KScales(const U32x4& header, int p) {
+#pragma clang fp contract(off)
+  const int shift = 16 * (p & 1);
+  const uint32_t a = (header.y >> shift) & 0xFFFFu;  // scales[0..3]
+  const uint32_t b = (header.z >> shift) & 0xFFFFu;  // scales[4..7]
+  const uint32_t c = (header.w >> shift) & 0xFFFFu;  // scales[8..11]
+  uint32_t sc, mn;
+  if (p < 2) {
+    sc = a & 0x3F3Fu;
+    mn = b & 0x3F3Fu;
+  } else {
+    sc = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u);
+    mn = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);
+  }
+  const float d = HalfBitsToFloat(header.x & 0xFFFFu);
+  const float dmin = HalfBitsToFloat(header.x >> 16);
+  Q4KScales s;
+  s.dsc0 = d * static_cast<float>(sc & 0xFFu);
+  s.dsc1 = d * static_cast<float>(sc >> 8);
+  s.dm0 = dmin * static_cast<float>(mn & 0xFFu);
+  s.dm1 = dmin * static_cast<float>(mn >> 8);
+  return s;
+}
+
+template <int P, bool kDump>
+__device__ __forceinline__ void DotQ4K(const Q4KUnit& u, int unit, int m, const Staged& act, int kp, float (&acc)[P],
+                                       int32_t* dump) {
+#pragma clang fp contract(off)
+  const int j = unit & 7;
+  const int sb = unit >> 3;
+  const int p = j >> 1;
+  const int h = j & 1;
+  const Q4KScales s = DecodeQ4KScales(u.header, p);
+  const uint32_t raw[4] = {u.codes.x, u.codes.y, u.codes.z, u.codes.w};
+  int lo[4], hi[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    lo[i] = static_cast<int>(raw[i] & 0x0F0F0F0Fu);
+    hi[i] = static_cast<int>((raw[i] >> 4) & 0x0F0F0F0Fu);
+  }
+#pragma unroll
+  for (int t = 0; t < P; ++t) {
+    if (t < m) {
+      const uint8_t* codes = act.codes + static_cast<int64_t>(t) * kp + sb * 256 + p * 64 + h * 16;
+      const uint4 a0 = *reinterpret_cast<const uint4*>(codes);
+      const uint4 a1 = *reinterpret_cast<const uint4*>(codes + 32);
+      const float2 d8 = *reinterpret_cast<const float2*>(act.scales + t * (kp / 32) + sb * 8 + p * 2);
+      const uint32_t sums = act.halves[t * (kp / 32) + sb * 8 + j];
+      int prod0 = Dot4(lo[0], static_cast<int>(a0.x), 0);
+      prod0 = Dot4(lo[1], static_cast<int>(a0.y), prod0);
+      prod0 = Dot4(lo[2], static_cast<int>(a0.z), prod0);
+      prod0 = Dot4(lo[3], static_cast<int>(a0.w), prod0);
+      int prod1 = Dot4(hi[0], static_cast<int>(a1.x), 0);
+      prod1 = Dot4(hi[1], static_cast<int>(a1.y), prod1);
+      prod1 = Dot4(hi[2], static_cast<int>(a1.z), prod1);
+      prod1 = Dot4(hi[3], static_cast<int>(a1.w), prod1);
+      const int sum0 = static_cast<int16_t>(sums & 0xFFFFu);
+      const int sum1 = static_cast<int16_t>(sums >> 16);
+      if (kDump && dump != nullptr) {
+        int32_t* out = dump + static_cast<int64_t>(sb) * 16;
+        atomicAdd(out + 2 * p, prod0);
+        atomicAdd(out + 2 * p + 1, prod1);
+        atomicAdd(out + 8 + 2 * p, sum0);
+        atomicAdd(out + 8 + 2 * p + 1, sum1);
+      }
+      // Spelled out so that every instantiation rounds at the same places.
+      const float t0 = fmaf(s.dsc0, static_cast<float>(prod0), -(s.dm0 * static_cast<float>(sum0)));
+      const float t1 = fmaf(s.dsc1, static_cast<float>(prod1), -(s.dm1 * static_cast<float>(sum1)));
+      acc[t] = fmaf(d8.y, t1, fmaf(d8.x, t0, acc[t]));
+    }
+  }
+}
+
+// ---- Q8_0: a unit is a pair of blocks, 68 bytes at a 4-byte boundary:
+// {d0, q0[0:2]} q0[2:30] {q0[30:32], d1} q1[0:32].
+struct Q8Pair {
+  uint32_t w[17];
+};
+
+__device__ __forceinline__ Q8Pair LoadQ8Pair(const uint8_t* row, int unit) {
+  const uint8_t* at = row + static_cast<int64_t>(unit) * 68;
+  Q8Pair u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const U32x4 v = __builtin_nontemporal_load(reinterpret_cast<const U32x4A4*>(at) + i);
+    u.w[4 * i + 0] = v.x;
+    u.w[4 * i + 1] = v.y;
+    u.w[4 * i + 2] = v.z;
+    u.w[4 * i + 3] = v.w;
+  }
+  u.w[16] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(at) + 16);
+  return u;
+}
+
+template <int P, bool kDump>
+__device__ __forceinline__ void DotQ8Pair(const Q8Pair& u, int unit, int m, const Staged& act, int kp, float (&acc)[P],
+                                          int32_t* dump) {
+#pragma clang fp contract(off)
+  const float d0 = HalfBitsToFloat(u.w[0] & 0xFFFFu);
+  const float d1 = HalfBitsToFloat(u.w[8] >> 16);
+  int q0[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q0[i] = static_cast<int>(__builtin_amdgcn_alignbyte(u.w[i + 1], u.w[i], 2));
+#pragma unroll
+  for (int t = 0; t < P; ++t) {
+    if (t < m) {
+      const uint4* codes = reinterpret_cast<const uint4*>(act.codes + static_cast<int64_t>(t) * kp + unit * 64);
+      const float2 d8 = *reinterpret_cast<const float2*>(act.scales + t * (kp / 32) + unit * 2);
+      int prod0 = 0, prod1 = 0;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint4 a = codes[i];
+        prod0 = Dot4(q0[4 * i + 0], static_cast<int>(a.x), prod0);
+        prod0 = Dot4(q0[4 * i + 1], static_cast<int>(a.y), prod0);
+        prod0 = Dot4(q0[4 * i + 2], static_cast<int>(a.z), prod0);
+        prod0 = Dot4(q0[4 * i + 3], static_cast<int>(a.w), prod0);
+        const uint4 b = codes[2 + i];
+        prod1 = Dot4(static_cast<int>(u.w[9 + 4 * i + 0]), static_cast<int>(b.x), prod1);
+        prod1 = Dot4(static_cast<int>(u.w[9 + 4 * i + 1]), static_cast<int>(b.y), prod1);
+        prod1 = Dot4(static_cast<int>(u.w[9 + 4 * i + 2]), static_cast<int>(b.z), prod1);
+        prod1 = Dot4(static_cast<int>(u.w[9 + 4 * i + 3]), static_cast<int>(b.w), prod1);
+      }
+      if (kDump && dump != nullptr) {
+        atomicAdd(dump + 2 * unit, prod0);
+        atomicAdd(dump + 2 * unit + 1, prod1);
+      }
+      // src/kernels/ggml/vecq.cu:416
+      acc[t] = fmaf(d1 * d8.y, static_cast<float>(prod1), fmaf(d0 * d8.x, static_cast<float>(prod0), acc[t]));
+    }
+  }
+}
+
+// A single Q8_0 block at a 2-byte boundary (rows of an odd block count, or
+// strides that break the pairs' alignment).
+struct Q8Single {
+  uint16_t h[17];
+};
+
+__device__ __forceinline__ Q8Single LoadQ8Single(const uint8_t* row, int unit) {
+  const uint16_t* at = reinterpret_cast<const uint16_t*>(row + static_cast<int64_t>(unit) * 34);
+  Q8Single u;
+#pragma unroll
+  for (int i = 0; i < 17; ++i) u.h[i] = at[i];
+  return u;
+}
+
+template <int P, bool kDump>
+__device__ __forceinline__ void DotQ8Single(const Q8Single& u, int unit, int m, const Staged& act, int kp,
+                                            float (&acc)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+  const float d0 = HalfBitsToFloat(u.h[0]);
+  int q[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = static_cast<int>(u.h[1 + 2 * i] | (static_cast<uint32_t>(u.h[2 + 2 * i]) << 16));
+#pragma unroll
+  for (int t = 0; t < P; ++t) {
+    if (t < m) {
+      const uint4* codes = reinterpret_cast<const uint4*>(act.codes + static_cast<int64_t>(t) * kp + unit * 32);
+      const float d8 = act.scales[t * (kp / 32) + unit];
+      const uint4 a = codes[0];
+      const uint4 b = codes[1];
+      int prod = Dot4(q[0], static_cast<int>(a.x), 0);
+      prod = Dot4(q[1], static_cast<int>(a.y), prod);
+      prod = Dot4(q[2], static_cast<int>(a.z), prod);
+      prod = Dot4(q[3], static_cast<int>(a.w), prod);
+      prod = Dot4(q[4], static_cast<int>(b.x), prod);
+      prod = Dot4(q[5], static_cast<int>(b.y), prod);
+      prod = Dot4(q[6], static_cast<int>(b.z), prod);
+      prod = Dot4(q[7], static_cast<int>(b.w), prod);
+      if (kDump && dump != nullptr) atomicAdd(dump + unit, prod);
+      acc[t] = fmaf(d0 * d8, static_cast<float>(prod), acc[t]);
+    }
+  }
+}
+
+enum Form { kFormQ4K = 0, kFormQ8Pair = 1, kFormQ8Single = 2 };
+
+template <int FORM>
+struct FormTraits;
+template <>
+struct FormTraits<kFormQ4K> {
+  using Unit = Q4KUnit;
+  static constexpr int kBlockBytes = 144;
+  __device__ static Unit Load(const uint8_t* row, int unit) { return LoadQ4K(row, unit); }
+  template <int P, bool kDump>
+  __device__ static void Dot(const Unit& u, int unit, int m, const Staged& a, int kp, float (&acc)[P], int32_t* dump) {
+    DotQ4K<P, kDump>(u, unit, m, a, kp, acc, dump);
+  }
+  __host__ __device__ static int Units(int k) { return k / 256 * 8; }
+  __host__ __device__ static int DumpInts(int k) { return k / 256 * 16; }
+};
+template <>
+struct FormTraits<kFormQ8Pair> {
+  using Unit = Q8Pair;
+  static constexpr int kBlockBytes = 34;
+  __device__ static Unit Load(const uint8_t* row, int unit) { return LoadQ8Pair(row, unit); }
+  template <int P, bool kDump>
+  __device__ static void Dot(const Unit& u, int unit, int m, const Staged& a, int kp, float (&acc)[P], int32_t* dump) {
+    DotQ8Pair<P, kDump>(u, unit, m, a, kp, acc, dump);
+  }
+  __host__ __device__ static int Units(int k) { return k / 64; }
+  __host__ __device__ static int DumpInts(int k) { return k / 32; }
+};
+template <>
+struct FormTraits<kFormQ8Single> {
+  using Unit = Q8Single;
+  static constexpr int kBlockBytes = 34;
+  __device__ static Unit Load(const uint8_t* row, int unit) { return LoadQ8Single(row, unit); }
+  template <int P, bool kDump>
+  __device__ static void Dot(const Unit& u, int unit, int m, const Staged& a, int kp, float (&acc)[P], int32_t* dump) {
+    DotQ8Single<P, kDump>(u, unit, m, a, kp, acc, dump);
+  }
+  __host__ __device__ static int Units(int k) { return k / 32; }
+  __host__ __device__ static int DumpInts(int k) { return k / 32; }
+};
+
+// LPR lanes a row, P tokens a pass, D units in flight a lane.
+// XT < 0: activations are Q8_1 blocks; else the unquantized element type.
+template <int FORM, int LPR, int P, int D, bool kGlu, int XT, bool kDump>
+__global__ __launch_bounds__(kThreads) void VecQKernel(const VecQArgs a) {
+  using T = FormTraits<FORM>;
+  using Unit = typename T::Unit;
+  constexpr bool kQ4K = FORM == kFormQ4K;
+  constexpr int kRowsPerWave = kWave / LPR;
+  constexpr int kRowsPerGroup = kRowsPerWave * (kThreads / kWave);
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int pairs[kMaxPairs];  // token << 8 | slot
+  __shared__ int count;
+
+  const llmp_vecq_desc& d = a.d;
+  const int kp = a.kp;
+  uint8_t* codes = lds;
+  float* scales = reinterpret_cast<float*>(lds + static_cast<int64_t>(P) * kp);
+  uint32_t* halves = reinterpret_cast<uint32_t*>(scales + P * (kp / 32));
+  const Staged act{codes, scales, halves};
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  int expert;
+  if (d.ids == nullptr) {
+    // Dense (one slot), or grouped: slot g's weights are matrix g.
+    expert = blockIdx.y;
+    if (tid < d.tokens) pairs[tid] = (tid << 8) | expert;
+    if (tid == 0) count = d.tokens;
+  } else {
+    // One workgroup row per (token, slot) pair; the first pair naming an
+    // expert owns it and computes every pair that names it, in pair order
+    // (src/kernels/ggml/vecq.cu:514-546, with 64-lane ballots).
+    const int s = blockIdx.y;
+    expert = d.ids[(s / d.used) * d.ids_stride + (s % d.used)];
+    if (wave == 0) {
+      const int total = d.tokens * d.used;
+      int n = 0;
+      bool owner = true;
+      for (int base = 0; base < total && owner; base += kWave) {
+        const int s2 = base + lane;
+        const int t = s2 / d.used;
+        const int u = s2 % d.used;
+        const bool match = s2 < total && d.ids[t * d.ids_stride + u] == expert;
+        const unsigned long long ballot = __ballot(match);
+        if (n == 0 && ballot != 0) owner = base + __ffsll(ballot) - 1 == s;
+        if (owner && match) pairs[n + __popcll(ballot & ((1ull << lane) - 1ull))] = (t << 8) | u;
+        n += __popcll(ballot);
+      }
+      if (lane == 0) count = owner ? n : 0;
+    }
+  }
+  __syncthreads();
+  const int n = count;
+  if (n == 0) return;  // uniform over the workgroup
+
+  const int row = blockIdx.x * kRowsPerGroup + wave * kRowsPerWave + lane / LPR;
+  const int sub = lane % LPR;
+  const bool live = row < d.nrows;
+  const int64_t row_at =
+      (static_cast<int64_t>(expert) * d.stride_expert + static_cast<int64_t>(live ? row : d.nrows - 1) * d.stride_row) *
+      T::kBlockBytes;
+  const uint8_t* wrow = static_cast<const uint8_t*>(d.w) + row_at;
+  const uint8_t* grow = kGlu ? static_cast<const uint8_t*>(d.g) + row_at : nullptr;
+  const int units = T::Units(d.ncols_x);
+  int32_t* dump = kDump && live ? a.dump + static_cast<int64_t>(row) * T::DumpInts(d.ncols_x) : nullptr;
+
+  for (int p0 = 0; p0 < n; p0 += P) {
+    const int m = min(P, n - p0);
+    for (int j = 0; j < m; ++j) {
+      const int pr = pairs[p0 + j];
+      const int token = pr >> 8;
+      const int slot = pr & 0xFF;
+      if constexpr (XT < 0) {
+        const uint8_t* y = static_cast<const uint8_t*>(d.y) +
+                           (static_cast<int64_t>(token) * d.y_token + static_cast<int64_t>(slot) * d.y_slot) * kQ8Block;
+        StageQ8<kQ4K>(y, d.ncols_x / 32, kp, j, codes, scales, halves);
+      } else {
+        const int64_t at = token * a.x_token + slot * a.x_slot;
+        const void* x = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
+                                         : static_cast<const void*>(static_cast<const uint16_t*>(a.x) + at);
+        StageX<kQ4K, XT>(x, d.ncols_x, kp, j, codes, scales, halves);
+      }
+    }
+    __syncthreads();
+
+    float acc[P];
+    float accg[kGlu ? P : 1];
+#pragma unroll
+    for (int t = 0; t < P; ++t) acc[t] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < (kGlu ? P : 1); ++t) accg[t] = 0.0f;
+
+    // D units in flight: the loads of unit i + D are issued before unit i's arithmetic.
+    Unit wu[D];
+    Unit gu[kGlu ? D : 1];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      const int unit = sub + i * LPR;
+      if (unit < units) {
+        wu[i] = T::Load(wrow, unit);
+        if constexpr (kGlu) gu[i] = T::Load(grow, unit);
+      }
+    }
+    for (int base = sub; base < units; base += D * LPR) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        const int unit = base + i * LPR;
+        const Unit w_now = wu[i];
+        Unit g_now;
+        if constexpr (kGlu) g_now = gu[i];
+        const int next = unit + D * LPR;
+        if (next < units) {
+          wu[i] = T::Load(wrow, next);
+          if constexpr (kGlu) gu[i] = T::Load(grow, next);
+        }
+        if (unit < units) {
+          T::template Dot<P, kDump>(w_now, unit, m, act, kp, acc, dump);
+          if constexpr (kGlu) T::template Dot<P, false>(g_now, unit, m, act, kp, accg, nullptr);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+#pragma unroll
+      for (int mask = LPR / 2; mask >= 1; mask >>= 1) {
+        acc[t] += ShflXor(acc[t], mask);
+        if constexpr (kGlu) accg[t] += ShflXor(accg[t], mask);
+      }
+      if (t < m && sub == 0 && live) {
+        const int pr = pairs[p0 + t];
+        float* dst = d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
+        dst[row] = kGlu ? Glu(d.glu, accg[t], acc[t], d.limit) : acc[t];
+      }
+    }
+    __syncthreads();  // the next pass restages
+  }
+}
+
+// ------------------------------------------------------------ host side
+
+struct Variant {
+  const char* name;
+  int lanes;   // a row
+  int pass;    // tokens a pass
+  int flight;  // units a lane keeps in flight
+};
+
+constexpr Variant kVariants[] = {
+    {"lanes8 pass1 flight4", 8, 1, 4},   {"lanes8 pass2 flight3", 8, 2, 3},   {"lanes8 pass4 flight2", 8, 4, 2},
+    {"lanes8 pass8 flight2", 8, 8, 2},   {"lanes16 pass1 flight4", 16, 1, 4}, {"lanes64 pass1 flight2", 64, 1, 2},
+};
+constexpr int kVariantCount = sizeof(kVariants) / sizeof(kVariants[0]);
+
+size_t LdsBytes(int pass, int kp) { return static_cast<size_t>(pass) * (kp + kp / 8 + kp / 8); }
+
+int PaddedK(int k) { return (k + 511) / 512 * 512; }
+
+template <int FORM, int LPR, int P, int D, bool kGlu, int XT>
+void LaunchOne(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+  if (a.dump != nullptr) {
+    if constexpr (P == 1 && !kGlu && XT < 0 && LPR == 8) {
+      hipLaunchKernelGGL((VecQKernel<FORM, LPR, P, D, kGlu, XT, true>), grid, dim3(kThreads), lds, stream, a);
+    }
+    return;
+  }
+  hipLaunchKernelGGL((VecQKernel<FORM, LPR, P, D, kGlu, XT, false>), grid, dim3(kThreads), lds, stream, a);
+}
+
+template <int FORM, int LPR, int P, int D>
+void LaunchSource(const VecQArgs& a, int x_type, dim3 grid, size_t lds, hipStream_t stream) {
+  const bool glu = a.d.g != nullptr;
+  switch (x_type) {
+    case -1:
+      glu ? LaunchOne<FORM, LPR, P, D, true, -1>(a, grid, lds, stream)
+          : LaunchOne<FORM, LPR, P, D, false, -1>(a, grid, lds, stream);
+      break;
+    case LLMP_X_F32:
+      glu ? LaunchOne<FORM, LPR, P, D, true, LLMP_X_F32>(a, grid, lds, stream)
+          : LaunchOne<FORM, LPR, P, D, false, LLMP_X_F32>(a, grid, lds, stream);
+      break;
+    default:
+      glu ? LaunchOne<FORM, LPR, P, D, true, LLMP_X_BF16>(a, grid, lds, stream)
+          : LaunchOne<FORM, LPR, P, D, false, LLMP_X_BF16>(a, grid, lds, stream);
+      break;
+  }
+}
+
+template <int FORM>
+void LaunchVariant(const VecQArgs& a, int x_type, int variant, dim3 grid, size_t lds, hipStream_t stream) {
+  switch (variant) {
+    case 0:
+      LaunchSource<FORM, 8, 1, 4>(a, x_type, grid, lds, stream);
+      break;
+    case 1:
+      LaunchSource<FORM, 8, 2, 3>(a, x_type, grid, lds, stream);
+      break;
+    case 2:
+      LaunchSource<FORM, 8, 4, 2>(a, x_type, grid, lds, stream);
+      break;
+    case 3:
+      LaunchSource<FORM, 8, 8, 2>(a, x_type, grid, lds, stream);
+      break;
+    case 4:
+      LaunchSource<FORM, 16, 1, 4>(a, x_type, grid, lds, stream);
+      break;
+    default:
+      LaunchSource<FORM, 64, 1, 2>(a, x_type, grid, lds, stream);
+      break;
+  }
+}
+
+// The default configuration of a shape: the tokens of a pass first (each pass
+// streams the weights again), then enough lanes a row to fill the device.
+int DefaultVariant(const llmp_vecq_desc& d, int kp) {
+  const int tokens = d.tokens;
+  int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
+  while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
+  switch (pass) {
+    case 8:
+      return 3;
+    case 4:
+      return 2;
+    case 2:
+      return 1;
+    default:
+      return 0;
+  }
+}
+
+int CheckDesc(int type, const llmp_vecq_desc* d) {
+  if (d == nullptr) return Refuse(1, "vecq: null descriptor");
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K) return Refuse(1, "vecq: weight type %d has no kernel", type);
+  const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
+  if (d->w == nullptr || d->dst == nullptr) return Refuse(1, "vecq: null weights or output");
+  if (d->ncols_x <= 0 || d->ncols_x % qk != 0) return Refuse(1, "vecq: k %d is not whole %d-value blocks", d->ncols_x, qk);
+  if (d->nrows <= 0) return Refuse(1, "vecq: no rows");
+  if (d->tokens < 1 || d->tokens > 16) return Refuse(1, "vecq: 1 to 16 tokens, not %d", d->tokens);
+  if (d->used < 1 || d->used > 256) return Refuse(1, "vecq: 1 to 256 slots, not %d", d->used);
+  if (d->ids != nullptr && d->used * d->tokens > kMaxPairs)
+    return Refuse(1, "vecq: %d routed pairs exceed %d", d->used * d->tokens, kMaxPairs);
+  if ((d->glu != LLMP_GLU_NONE) != (d->g != nullptr)) return Refuse(1, "vecq: gate weights exactly with a GLU");
+  if (d->glu < 0 || d->glu > LLMP_GLU_GEGLU) return Refuse(1, "vecq: unknown GLU %d", d->glu);
+  if (d->glu == LLMP_GLU_GEGLU && d->limit != 0.0f) return Refuse(1, "vecq: GeGLU takes no clamp limit");
+  if (d->stride_row < d->ncols_x / qk) return Refuse(1, "vecq: rows overlap");
+  if (reinterpret_cast<uintptr_t>(d->dst) % 4 != 0) return Refuse(1, "vecq: output not 4-byte aligned");
+  const uintptr_t wa = reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g);
+  if (type == LLMP_TYPE_Q4_K && wa % 16 != 0) return Refuse(1, "vecq: Q4_K weights not 16-byte aligned");
+  if (type == LLMP_TYPE_Q8_0 && wa % 2 != 0) return Refuse(1, "vecq: Q8_0 weights not 2-byte aligned");
+  return 0;
+}
+
+int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant, int32_t* dump, void* stream) {
+  if (const int bad = CheckDesc(type, d); bad != 0) return bad;
+  int x_type = -1;
+  VecQArgs a{};
+  a.d = *d;
+  if (x != nullptr) {
+    if (x->x == nullptr || x->x_type < LLMP_X_F32 || x->x_type > LLMP_X_BF16)
+      return Refuse(1, "vecq: unquantized activations of an unknown type");
+    x_type = x->x_type;
+    a.x = x->x;
+    a.x_token = x->x_token;
+    a.x_slot = x->x_slot;
+  } else if (d->y == nullptr || reinterpret_cast<uintptr_t>(d->y) % 4 != 0) {
+    return Refuse(1, "vecq: Q8_1 activations null or not 4-byte aligned");
+  }
+  a.kp = PaddedK(d->ncols_x);
+  a.dump = dump;
+  if (variant < 0) variant = DefaultVariant(*d, a.kp);
+  if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
+  const Variant& v = kVariants[variant];
+  const size_t lds = LdsBytes(v.pass, a.kp);
+  if (lds > static_cast<size_t>(kLdsBudget))
+    return Refuse(1, "vecq: %d tokens of k %d do not fit the staging area", v.pass, d->ncols_x);
+  if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr || variant != 0))
+    return Refuse(1, "vecq: block sums are of a dense one-token product");
+  const int slots = d->ids != nullptr ? d->used * d->tokens : d->used;
+  const int rows_per_group = (kWave / v.lanes) * (kThreads / kWave);
+  const dim3 grid(static_cast<unsigned>((d->nrows + rows_per_group - 1) / rows_per_group),
+                  static_cast<unsigned>(slots));
+  const auto s = static_cast<hipStream_t>(stream);
+  if (type == LLMP_TYPE_Q4_K) {
+    LaunchVariant<kFormQ4K>(a, x_type, variant, grid, lds, s);
+  } else {
+    const bool pairs = d->ncols_x % 64 == 0 && d->stride_row % 2 == 0 && d->stride_expert % 2 == 0 &&
+                       (reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g)) % 4 == 0;
+    if (pairs) {
+      LaunchVariant<kFormQ8Pair>(a, x_type, variant, grid, lds, s);
+    } else {
+      LaunchVariant<kFormQ8Single>(a, x_type, variant, grid, lds, s);
+    }
+  }
+  return LaunchStatus("vecq");
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_q8_1_quantize(const float* x, void* out, int64_t k, int64_t padded_k, int64_t row_stride,
+                                      int64_t rows, int64_t planes, int64_t plane_stride, void* stream) {
+  if (x == nullptr || out == nullptr) return Refuse(1, "q8_1: null operand");
+  if (k <= 0 || rows <= 0 || planes <= 0) return Refuse(1, "q8_1: empty input");
+  if (padded_k < k || padded_k % 32 != 0) return Refuse(1, "q8_1: padded k %lld below k or not whole blocks", (long long)padded_k);
+  if (rows > 65535 || planes > 65535) return Refuse(1, "q8_1: more than 65535 rows or planes");
+  if (reinterpret_cast<uintptr_t>(x) % 4 != 0 || reinterpret_cast<uintptr_t>(out) % 4 != 0)
+    return Refuse(1, "q8_1: operands not 4-byte aligned");
+  const int64_t blocks = padded_k / 32;
+  const dim3 grid(static_cast<unsigned>((blocks + 31) / 32), static_cast<unsigned>(rows), static_cast<unsigned>(planes));
+  hipLaunchKernelGGL(QuantizeQ8Kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), x,
+                     static_cast<uint8_t*>(out), k, padded_k, row_stride, rows, plane_stride);
+  return LaunchStatus("q8_1");
+}
+
+extern "C" int llmp_hip_vecq(int type, const llmp_vecq_desc* d, int variant, void* stream) {
+  return Launch(type, d, nullptr, variant, nullptr, stream);
+}
+
+extern "C" int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant,
+                                   void* stream) {
+  if (x == nullptr) return Refuse(1, "vecq: null source");
+  return Launch(type, d, x, variant, nullptr, stream);
+}
+
+extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int32_t* sums, void* stream) {
+  if (sums == nullptr) return Refuse(1, "vecq: null sums");
+  return Launch(type, d, nullptr, 0, sums, stream);
+}
+
+extern "C" int llmp_hip_vecq_variants(void) { return kVariantCount; }
+
+extern "C" const char* llmp_hip_vecq_variant_name(int variant) {
+  return variant >= 0 && variant < kVariantCount ? kVariants[variant].name : "default";
+}

@@ -1,0 +1,65 @@
+"""Seeded synthetic inputs of the benchmark configurations (numpy, host side).
+
+Weights are byte images of GGML blocks: Q8_0 {f16 d; i8 qs[32]} and Q4_K
+{f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} (src/format/encoding.cc:110-116
+of the reference)."""
+import numpy as np
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def q8_0_weights(n, k, seed):
+    """[n, k/32*34] uint8: codes uniform in [-127, 127], each block's scale
+    max|w| / 127 over 32 draws of N(0, 0.02)."""
+    g = rng(seed)
+    blocks = k // 32
+    out = np.zeros((n, blocks, 34), dtype=np.uint8)
+    amax = np.abs(g.standard_normal((n, blocks, 32), dtype=np.float32) * 0.02).max(axis=-1)
+    out[:, :, 0:2] = (amax / 127.0).astype(np.float16).view(np.uint8).reshape(n, blocks, 2)
+    out[:, :, 2:] = g.integers(-127, 128, size=(n, blocks, 32), dtype=np.int8).view(np.uint8)
+    return out.reshape(n, blocks * 34)
+
+
+def q4_k_weights(n, k, seed):
+    """[n, k/256*144] uint8: 4-bit codes uniform 0..15, 6-bit sub-scales and minimums
+    uniform 0..63, d and dmin sized so that d*63*15 and dmin*63 span the range of 256
+    draws of N(0, 0.02) (about 5.6 and 2.8 standard deviations)."""
+    g = rng(seed)
+    blocks = k // 256
+    out = np.zeros((n, blocks, 144), dtype=np.uint8)
+    d = (0.02 * g.uniform(5.0, 6.2, size=(n, blocks)) / (63.0 * 15.0)).astype(np.float16)
+    dmin = (0.02 * g.uniform(2.4, 3.2, size=(n, blocks)) / 63.0).astype(np.float16)
+    out[:, :, 0:2] = d.view(np.uint8).reshape(n, blocks, 2)
+    out[:, :, 2:4] = dmin.view(np.uint8).reshape(n, blocks, 2)
+    out[:, :, 4:] = g.integers(0, 256, size=(n, blocks, 140), dtype=np.uint8)
+    return out.reshape(n, blocks * 144)
+
+
+def random_blocks(t, n, k, seed):
+    """Every field random (any finite f16 scale up to magnitude 4, any scale byte, any code):
+    the bytes a decoder must take, not a plausible quantization."""
+    g = rng(seed)
+    if t == 8:
+        blocks, size, heads = k // 32, 34, 1
+    else:
+        blocks, size, heads = k // 256, 144, 2
+    out = g.integers(0, 256, size=(n, blocks, size), dtype=np.uint8)
+    scale = (g.uniform(-4.0, 4.0, size=(n, blocks, heads))).astype(np.float16)
+    out[:, :, 0:2 * heads] = scale.view(np.uint8).reshape(n, blocks, 2 * heads)
+    return out.reshape(n, blocks * size)
+
+
+def activations(tokens, k, seed, dtype=np.float32):
+    return rng(seed).standard_normal((tokens, k), dtype=np.float32).astype(dtype)
+
+
+def bf16_bits(x):
+    """float32 -> bfloat16 bits, nearest even (src/kernels/reference/decode.cc:386-392)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def bf16_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)

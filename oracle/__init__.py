@@ -1,0 +1,266 @@
+"""ctypes binding of the CPU oracle (oracle/oracle.c): TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import this
+module. The shipped package never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liboracle.so")
+
+TYPE_Q8_0 = 8
+TYPE_Q4_K = 12
+GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
+CB_3INST, CB_MCG, CB_MUL1 = 0, 1, 2
+Q8_DEVICE, Q8_GGML_CPU = 0, 1
+
+
+def build():
+    subprocess.run(["make", "-C", _HERE, "-B", "liboracle.so"], check=True, capture_output=True)
+
+
+def _load():
+    if not os.path.exists(_SO):
+        build()
+    return C.CDLL(_SO)
+
+
+lib = _load()
+
+
+class VecQDesc(C.Structure):
+    _fields_ = [
+        ("w", C.c_void_p), ("g", C.c_void_p), ("y", C.c_void_p), ("ids", C.c_void_p),
+        ("dst", C.c_void_p),
+        ("ncols_x", C.c_int), ("nrows", C.c_int), ("stride_row", C.c_int),
+        ("stride_expert", C.c_int), ("y_token", C.c_int), ("y_slot", C.c_int),
+        ("ids_stride", C.c_int), ("used", C.c_int), ("tokens", C.c_int),
+        ("dst_token", C.c_int), ("dst_slot", C.c_int), ("glu", C.c_int), ("limit", C.c_float),
+    ]
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _sig(name, res, *args):
+    f = getattr(lib, name)
+    f.restype = res
+    f.argtypes = list(args)
+    return f
+
+
+_i64, _u64, _vp, _int = C.c_int64, C.c_uint64, C.c_void_p, C.c_int
+_sig("orc_f16_to_f32", C.c_float, C.c_uint16)
+_sig("orc_f32_to_f16", C.c_uint16, C.c_float)
+_sig("orc_bf16_to_f32", C.c_float, C.c_uint16)
+_sig("orc_f32_to_bf16", C.c_uint16, C.c_float)
+_sig("orc_e4m3_to_f32", C.c_float, C.c_uint8)
+_sig("orc_e8m0_to_f32", C.c_float, C.c_uint8)
+_sig("orc_f32_to_e4m3", C.c_uint8, C.c_float)
+_sig("orc_q8_1_quantize_row", None, _vp, _i64, _i64, _vp, _int)
+_sig("orc_q8_1_decode_row", None, _vp, _i64, _vp)
+_sig("orc_q4_k_scale_min", None, _vp, _int, _vp, _vp)
+_sig("orc_decode_row", None, _int, _vp, _i64, _vp)
+_sig("orc_block_sums", None, _int, _vp, _vp, _vp)
+_sig("orc_block_product", C.c_double, _int, _vp, _vp)
+_sig("orc_glu", C.c_double, _int, C.c_double, C.c_double, C.c_double)
+_sig("orc_vecq", _int, _int, C.POINTER(VecQDesc), _int, _int)
+_sig("orc_vecq_block_sums", None, _int, _vp, _vp, _int, _int, _int, _vp)
+_sig("orc_mxfp8_scale_code", C.c_uint32, C.c_float)
+_sig("orc_mxfp8_inverse_scale", C.c_float, C.c_uint32)
+_sig("orc_scale_atom_offset", _u64, _u64, _u64, _u64)
+_sig("orc_mxfp8_quantize", None, _vp, _i64, _i64, _i64, _vp, _vp)
+_sig("orc_mxfp8_swizzle", None, _vp, _i64, _i64, _vp)
+_sig("orc_mxfp8_dot", C.c_double, _vp, _vp, _i64, _vp, _vp, _i64, _i64)
+_sig("orc_mxfp8_gemm", None, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _int)
+_sig("orc_mxfp8_gemv", None, _vp, _vp, _i64, _i64, _vp, _i64, _vp)
+_sig("orc_route", None, _vp, _i64, _i64, _i64, _int, C.c_float, _vp, _vp)
+_sig("orc_expert_sort", _int, _vp, _i64, _i64, _vp, _vp)
+_sig("orc_expert_reduce", None, _vp, _vp, _i64, _i64, _i64, _vp)
+_sig("orc_exl3_codebook", C.c_uint16, _int, C.c_uint16)
+_sig("orc_exl3_state", C.c_uint16, _vp, C.c_uint32, C.c_uint32)
+_sig("orc_exl3_placement", None, _vp)
+_sig("orc_exl3_rotated", None, _vp, _i64, _i64, _int, _int, _i64, _i64, _vp)
+_sig("orc_exl3_rows", None, _vp, _vp, _vp, _i64, _i64, _int, _int, _i64, _i64, _vp)
+_sig("orc_exl3_linear", None, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp, _i64, _vp, _int)
+_sig("orc_max_threads", _int)
+
+
+def max_threads():
+    return int(lib.orc_max_threads())
+
+
+def block_bytes(t):
+    return {TYPE_Q8_0: 34, TYPE_Q4_K: 144}[t]
+
+
+def block_elements(t):
+    return {TYPE_Q8_0: 32, TYPE_Q4_K: 256}[t]
+
+
+def padded_k(k):
+    return (k + 511) // 512 * 512
+
+
+def q8_1_quantize(x, flavor=Q8_DEVICE):
+    """float32 [rows, k] -> uint8 [rows, padded_k/32*36]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, k = x.shape
+    pk = padded_k(k)
+    out = np.zeros((rows, pk // 32 * 36), dtype=np.uint8)
+    for r in range(rows):
+        lib.orc_q8_1_quantize_row(_p(x[r]), k, pk, _p(out[r]), flavor)
+    return out
+
+
+def q8_1_decode(blocks, k):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    y = np.zeros(k, dtype=np.float32)
+    lib.orc_q8_1_decode_row(_p(blocks), k, _p(y))
+    return y
+
+
+def decode_rows(t, w, k):
+    """uint8 [rows, k/qk*bs] -> float32 [rows, k]."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    out = np.zeros((w.shape[0], k), dtype=np.float32)
+    for r in range(w.shape[0]):
+        lib.orc_decode_row(t, _p(w[r]), k, _p(out[r]))
+    return out
+
+
+def vecq(t, w, q8, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stride_row=None,
+         stride_expert=0, y_token=None, y_slot=0, glu=GLU_NONE, limit=0.0, experts=0, threads=1):
+    """The llmp.vecq product on the CPU. Returns float32 [tokens, used, nrows]."""
+    qk = block_elements(t)
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    q8 = np.ascontiguousarray(q8, dtype=np.uint8)
+    gate = None if gate is None else np.ascontiguousarray(gate, dtype=np.uint8)
+    ids = None if ids is None else np.ascontiguousarray(ids, dtype=np.int32)
+    dst = np.zeros((tokens, used, nrows), dtype=np.float32)
+    d = VecQDesc()
+    d.w, d.g, d.y, d.ids, d.dst = _p(w), _p(gate), _p(q8), _p(ids), _p(dst)
+    d.ncols_x, d.nrows = k, nrows
+    d.stride_row = k // qk if stride_row is None else stride_row
+    d.stride_expert = stride_expert
+    d.y_token = padded_k(k) // 32 if y_token is None else y_token
+    d.y_slot = y_slot
+    d.ids_stride = used
+    d.used, d.tokens = used, tokens
+    d.dst_token, d.dst_slot = used * nrows, nrows
+    d.glu, d.limit = glu, limit
+    rc = lib.orc_vecq(t, C.byref(d), experts, threads)
+    if rc != 0:
+        raise IndexError("expert id outside the table")
+    return dst
+
+
+def vecq_block_sums(t, w, q8, k, nrows):
+    qk = block_elements(t)
+    per = 1 if t == TYPE_Q8_0 else 16
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    q8 = np.ascontiguousarray(q8, dtype=np.uint8)
+    out = np.zeros((nrows, k // qk, per), dtype=np.int32)
+    lib.orc_vecq_block_sums(t, _p(w), _p(q8), k, nrows, k // qk, _p(out))
+    return out
+
+
+def glu(kind, gate, up, limit=0.0):
+    return lib.orc_glu(kind, float(gate), float(up), float(limit))
+
+
+def mxfp8_scale_bytes(rows, k):
+    return (rows + 127) // 128 * 128 * (k // 32)
+
+
+def mxfp8_quantize(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, k = x.shape
+    codes = np.zeros((rows, k), dtype=np.uint8)
+    scales = np.zeros(mxfp8_scale_bytes(rows, k), dtype=np.uint8)
+    lib.orc_mxfp8_quantize(_p(x), k, k, rows, _p(codes), _p(scales))
+    return codes, scales
+
+
+def mxfp8_swizzle(scales):
+    scales = np.ascontiguousarray(scales, dtype=np.uint8)
+    n, blocks = scales.shape
+    out = np.zeros(mxfp8_scale_bytes(n, blocks * 32), dtype=np.uint8)
+    lib.orc_mxfp8_swizzle(_p(scales), n, blocks, _p(out))
+    return out
+
+
+def mxfp8_dot(a_codes, a_scales, i, b_codes, b_scales, j):
+    k = a_codes.shape[1]
+    return lib.orc_mxfp8_dot(_p(a_codes), _p(a_scales), i, _p(b_codes), _p(b_scales), j, k)
+
+
+def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, threads=1):
+    m, k = a_codes.shape
+    n = b_codes.shape[0]
+    d = np.zeros((m, n), dtype=np.float32)
+    lib.orc_mxfp8_gemm(_p(a_codes), _p(a_scales), _p(b_codes), _p(b_scales), m, n, k, _p(d), threads)
+    return d
+
+
+def mxfp8_gemv(codes, scales, x):
+    n, k = codes.shape
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.zeros((x.shape[0], n), dtype=np.float32)
+    lib.orc_mxfp8_gemv(_p(codes), _p(np.ascontiguousarray(scales)), n, k, _p(x), x.shape[0], _p(y))
+    return y
+
+
+def route(logits, used, normalize=True, scale=1.0):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    tokens, experts = logits.shape
+    ids = np.zeros((tokens, used), dtype=np.int32)
+    w = np.zeros((tokens, used), dtype=np.float32)
+    lib.orc_route(_p(logits), experts, used, tokens, int(normalize), scale, _p(ids), _p(w))
+    return ids, w
+
+
+def expert_sort(ids, experts):
+    ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+    order = np.zeros(ids.size, dtype=np.int32)
+    offsets = np.zeros(experts + 1, dtype=np.int32)
+    if lib.orc_expert_sort(_p(ids), ids.size, experts, _p(order), _p(offsets)) != 0:
+        raise IndexError("expert id outside the table")
+    return order, offsets
+
+
+def expert_reduce(x, w):
+    """x float32 [tokens, used, width], w [tokens, used] -> [tokens, width]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    tokens, used, width = x.shape
+    out = np.zeros((tokens, width), dtype=np.float32)
+    lib.orc_expert_reduce(_p(x), _p(w), width, used, tokens, _p(out))
+    return out
+
+
+def exl3_rotated(trellis, k, n, bits, codebook, first=0, count=None):
+    count = n if count is None else count
+    out = np.zeros((k, count), dtype=np.uint16)
+    lib.orc_exl3_rotated(_p(trellis), k, n, bits, codebook, first, count, _p(out))
+    return out
+
+
+def exl3_rows(trellis, suh, svh, k, n, bits, codebook, first=0, count=None):
+    count = n if count is None else count
+    out = np.zeros((count, k), dtype=np.float32)
+    lib.orc_exl3_rows(_p(trellis), _p(suh), _p(svh), k, n, bits, codebook, first, count, _p(out))
+    return out
+
+
+def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, threads=1):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    m = x.shape[0]
+    y = np.zeros((m, n), dtype=np.float32)
+    lib.orc_exl3_linear(_p(trellis), _p(suh), _p(svh), k, n, bits, codebook, _p(x), m, _p(y), threads)
+    return y

@@ -1,0 +1,683 @@
+/*
+ * CPU oracle for the quantized linear-layer path: TEST INFRASTRUCTURE ONLY
+ * (see oracle.h for what pins each function). Build: make -C oracle.
+ * Compiled with -ffp-contract=off so every float step rounds on its own.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static uint32_t bits_of(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static float float_of(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+static uint16_t load_u16(const uint8_t* p) {
+  uint16_t v;
+  memcpy(&v, p, 2);
+  return v;
+}
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ------------------------------------------------------------ conversions */
+
+/* decode.cc:341-353 */
+float orc_f16_to_f32(uint16_t bits) {
+  const float sign = (bits & 0x8000u) ? -1.0f : 1.0f;
+  const unsigned exponent = (bits >> 10) & 31u;
+  const unsigned mantissa = bits & 1023u;
+  if (exponent == 31) return mantissa ? NAN : sign * INFINITY;
+  if (exponent == 0) return sign * ldexpf((float)mantissa, -24);
+  return sign * ldexpf((float)(1024u + mantissa), (int)exponent - 25);
+}
+
+/* decode.cc:355-382 */
+uint16_t orc_f32_to_f16(float value) {
+  const uint32_t x = bits_of(value);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const uint32_t magnitude = x & 0x7FFFFFFFu;
+  if (magnitude >= 0x7F800000u) return (uint16_t)(sign | (magnitude > 0x7F800000u ? 0x7E00u : 0x7C00u));
+  if (magnitude >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);
+  if (magnitude < 0x38800000u) {
+    const uint32_t exponent = magnitude >> 23;
+    const uint32_t shift = 126u - exponent;
+    if (exponent == 0 || shift > 24) return sign;
+    const uint32_t significand = (magnitude & 0x7FFFFFu) | 0x800000u;
+    uint32_t q = significand >> shift;
+    const uint32_t rest = significand & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1u);
+    if (rest > half || (rest == half && (q & 1u))) ++q;
+    return (uint16_t)(sign | q);
+  }
+  const uint32_t rounded = magnitude + 0xFFFu + ((magnitude >> 13) & 1u);
+  return (uint16_t)(sign | ((rounded - 0x38000000u) >> 13));
+}
+
+/* decode.cc:384-392 */
+float orc_bf16_to_f32(uint16_t bits) { return float_of((uint32_t)bits << 16); }
+uint16_t orc_f32_to_bf16(float value) {
+  const uint32_t x = bits_of(value);
+  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x40u);
+  return (uint16_t)((x + 0x7FFFu + ((x >> 16) & 1u)) >> 16);
+}
+
+/* decode.cc:394-405 */
+float orc_e4m3_to_f32(uint8_t bits) {
+  const float sign = (bits & 0x80u) ? -1.0f : 1.0f;
+  const unsigned exponent = (bits >> 3) & 15u;
+  const unsigned mantissa = bits & 7u;
+  if (exponent == 15 && mantissa == 7) return NAN;
+  if (exponent == 0) return sign * ldexpf((float)mantissa, -9);
+  return sign * ldexpf((float)(8u + mantissa), (int)exponent - 10);
+}
+
+/* decode.cc:417-422 */
+float orc_e8m0_to_f32(uint8_t bits) {
+  if (bits == 0xFF) return NAN;
+  return ldexpf(1.0f, (int)bits - 127);
+}
+
+/* OCP E4M3 from float: nearest, ties to even, saturating to +-448; NaN -> 0x7F. */
+uint8_t orc_f32_to_e4m3(float value) {
+  const uint8_t sign = (bits_of(value) >> 31) ? 0x80u : 0u;
+  if (isnan(value)) return (uint8_t)(sign | 0x7Fu);
+  const float a = fabsf(value);
+  if (a > 448.0f) return (uint8_t)(sign | 0x7Eu);
+  if (a < 0.015625f) { /* below 2^-6: units of 2^-9 */
+    const int q = (int)nearbyintf(a * 512.0f);
+    return (uint8_t)(sign | (uint8_t)q); /* q == 8 is the least normal's encoding */
+  }
+  int e;
+  (void)frexpf(a, &e); /* a = m * 2^e, m in [0.5, 1) */
+  int exponent = e - 1;
+  int q = (int)nearbyintf(ldexpf(a, 3 - exponent)); /* in [8, 16] */
+  if (q == 16) {
+    q = 8;
+    ++exponent;
+  }
+  return (uint8_t)(sign | ((unsigned)(exponent + 7) << 3) | (unsigned)(q - 8));
+}
+
+/* ------------------------------------------------------------------ Q8_1 */
+
+/* The 32 lanes' xor-butterfly sum, offsets 16, 8, 4, 2, 1 (a warp reduction's order). */
+static float butterfly32(const float* x) {
+  float a[32];
+  memcpy(a, x, sizeof(a));
+  for (int h = 16; h >= 1; h /= 2)
+    for (int i = 0; i < h; ++i) a[i] = a[i] + a[i + h];
+  return a[0];
+}
+
+void orc_q8_1_quantize_row(const float* x, int64_t k, int64_t padded_k, uint8_t* out, int flavor) {
+  for (int64_t b = 0; b < padded_k / 32; ++b) {
+    uint8_t* blk = out + b * 36;
+    float v[32];
+    for (int j = 0; j < 32; ++j) {
+      const int64_t i = b * 32 + j;
+      v[j] = i < k ? x[i] : 0.0f;
+    }
+    float amax = 0.0f;
+    for (int j = 0; j < 32; ++j) {
+      const float a = fabsf(v[j]);
+      amax = amax > a ? amax : a;
+    }
+    const float d = amax / 127.0f;
+    int8_t q[32];
+    uint16_t s16;
+    if (flavor == ORC_Q8_GGML_CPU) {
+      /* kv_quant.cuh:35-42 (d, id, codes); s = d * sum(q) as ggml's quantize_row_q8_1_ref. */
+      const float id = d != 0.0f ? 1.0f / d : 0.0f;
+      int sum = 0;
+      for (int j = 0; j < 32; ++j) {
+        q[j] = (int8_t)roundf(v[j] * id);
+        sum += q[j];
+      }
+      s16 = orc_f32_to_f16((float)sum * d);
+    } else {
+      /* llmp_moe.cu:521-536 without fast math: q = roundf(x / d), 0 for a zero block. */
+      for (int j = 0; j < 32; ++j) q[j] = amax == 0.0f ? 0 : (int8_t)roundf(v[j] / d);
+      s16 = orc_f32_to_f16(butterfly32(v));
+    }
+    const uint16_t d16 = orc_f32_to_f16(d);
+    memcpy(blk, &d16, 2);
+    memcpy(blk + 2, &s16, 2);
+    memcpy(blk + 4, q, 32);
+  }
+}
+
+void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y) {
+  for (int64_t b = 0; b < k / 32; ++b) {
+    const uint8_t* x = blocks + b * 36;
+    const float d = orc_f16_to_f32(load_u16(x));
+    for (int j = 0; j < 32; ++j) y[b * 32 + j] = d * (float)(int8_t)x[4 + j];
+  }
+}
+
+/* --------------------------------------------------------- weight blocks */
+
+int orc_block_bytes(int type) { return type == ORC_TYPE_Q8_0 ? 34 : type == ORC_TYPE_Q4_K ? 144 : 0; }
+int orc_block_elements(int type) { return type == ORC_TYPE_Q8_0 ? 32 : type == ORC_TYPE_Q4_K ? 256 : 0; }
+
+/* dsv4_fast_test.cc:180-183 */
+void orc_q4_k_scale_min(const uint8_t* scales, int g, int* scale, int* minimum) {
+  *scale = g < 4 ? scales[g] & 63 : (scales[g + 4] & 15) | ((scales[g - 4] >> 6) << 4);
+  *minimum = g < 4 ? scales[g + 4] & 63 : (scales[g + 4] >> 4) | ((scales[g] >> 6) << 4);
+}
+
+static int q4_k_code(const uint8_t* codes, int g, int i) {
+  return (codes[(g / 2) * 32 + i] >> ((g % 2) * 4)) & 15; /* dsv4_fast_test.cc:187 */
+}
+
+void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
+  if (type == ORC_TYPE_Q8_0) {
+    for (int64_t b = 0; b < k / 32; ++b) {
+      const uint8_t* x = row + b * 34;
+      const float d = orc_f16_to_f32(load_u16(x));
+      for (int j = 0; j < 32; ++j) y[b * 32 + j] = d * (float)(int8_t)x[2 + j];
+    }
+    return;
+  }
+  /* Q4_K: y = d * sc * code - dmin * m (ggml's dequantize_row_q4_K of these bytes). */
+  for (int64_t b = 0; b < k / 256; ++b) {
+    const uint8_t* x = row + b * 144;
+    const float d = orc_f16_to_f32(load_u16(x));
+    const float dmin = orc_f16_to_f32(load_u16(x + 2));
+    for (int g = 0; g < 8; ++g) {
+      int sc, m;
+      orc_q4_k_scale_min(x + 4, g, &sc, &m);
+      const float d1 = d * (float)sc;
+      const float m1 = dmin * (float)m;
+      for (int i = 0; i < 32; ++i) y[b * 256 + g * 32 + i] = d1 * (float)q4_k_code(x + 16, g, i) - m1;
+    }
+  }
+}
+
+void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums) {
+  if (type == ORC_TYPE_Q8_0) {
+    int32_t s = 0;
+    for (int i = 0; i < 32; ++i) s += (int32_t)(int8_t)w[2 + i] * (int32_t)(int8_t)q8[4 + i];
+    sums[0] = s;
+    return;
+  }
+  for (int g = 0; g < 8; ++g) {
+    const uint8_t* a = q8 + g * 36;
+    int32_t product = 0, sum = 0;
+    for (int i = 0; i < 32; ++i) {
+      const int value = (int8_t)a[4 + i];
+      product += q4_k_code(w + 16, g, i) * value;
+      sum += value;
+    }
+    sums[g] = product;
+    sums[8 + g] = sum;
+  }
+}
+
+double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
+  int32_t sums[16];
+  orc_block_sums(type, w, q8, sums);
+  if (type == ORC_TYPE_Q8_0) {
+    /* vecq.cu:415-416: d8_0 * d8_1 * sumi */
+    return (double)orc_f16_to_f32(load_u16(w)) * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
+  }
+  /* dsv4_fast_test.cc:179-193 */
+  const double d = orc_f16_to_f32(load_u16(w));
+  const double dmin = orc_f16_to_f32(load_u16(w + 2));
+  double total = 0;
+  for (int g = 0; g < 8; ++g) {
+    int sc, m;
+    orc_q4_k_scale_min(w + 4, g, &sc, &m);
+    const double d8 = orc_f16_to_f32(load_u16(q8 + g * 36));
+    total += d8 * (d * sc * sums[g] - dmin * m * sums[8 + g]);
+  }
+  return total;
+}
+
+/* -------------------------------------------------------------------- GLU */
+
+static double sigmoid_d(double x) { return 1.0 / (1.0 + exp(-x)); }
+static double silu_d(double x) { return x * sigmoid_d(x); }
+static double gelu_tanh_d(double x) {
+  const double c = sqrt(2.0 / M_PI);
+  return 0.5 * x * (1.0 + tanh(c * x * (1.0 + 0.044715 * x * x)));
+}
+
+/* exec.cc:248-262 */
+double orc_glu(int kind, double gate, double up, double limit) {
+  switch (kind) {
+    case ORC_GLU_SWIGLU:
+      return silu_d(gate) * up;
+    case ORC_GLU_GEGLU:
+      return gelu_tanh_d(gate) * up;
+    case ORC_GLU_SWIGLU_CLAMP: {
+      const double g = gate < limit ? gate : limit;
+      const double u = up < -limit ? -limit : (up > limit ? limit : up);
+      return silu_d(g) * u;
+    }
+    default:
+      return up;
+  }
+}
+
+/* ------------------------------------------------------------------- vecq */
+
+static double row_product(int type, const uint8_t* wrow, const uint8_t* y, int k) {
+  const int qk = orc_block_elements(type);
+  const int bs = orc_block_bytes(type);
+  double s = 0;
+  for (int b = 0; b < k / qk; ++b) s += orc_block_product(type, wrow + (int64_t)b * bs, y + (int64_t)b * (qk / 32) * 36);
+  return s;
+}
+
+int orc_vecq(int type, const orc_vecq_desc* d, int experts, int threads) {
+  const int bs = orc_block_bytes(type);
+  const int routed = d->ids != NULL;
+  const int pairs = routed ? d->tokens * d->used : d->tokens * d->used;
+  for (int p = 0; routed && p < pairs; ++p) {
+    const int id = d->ids[(p / d->used) * d->ids_stride + (p % d->used)];
+    if (experts > 0 && (id < 0 || id >= experts)) return 1;
+  }
+  (void)threads;
+  for (int p = 0; p < pairs; ++p) {
+    const int t = p / d->used;
+    const int u = p % d->used;
+    const int expert = routed ? d->ids[t * d->ids_stride + u] : u;
+    const uint8_t* y = (const uint8_t*)d->y + ((int64_t)t * d->y_token + (int64_t)u * d->y_slot) * 36;
+    float* dst = d->dst + (int64_t)t * d->dst_token + (int64_t)u * d->dst_slot;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+    for (int r = 0; r < d->nrows; ++r) {
+      const int64_t at = ((int64_t)expert * d->stride_expert + (int64_t)r * d->stride_row) * bs;
+      const double up = row_product(type, (const uint8_t*)d->w + at, y, d->ncols_x);
+      double v = up;
+      if (d->g != NULL) {
+        const double gate = row_product(type, (const uint8_t*)d->g + at, y, d->ncols_x);
+        v = orc_glu(d->glu, gate, up, d->limit);
+      }
+      dst[r] = (float)v;
+    }
+  }
+  return 0;
+}
+
+void orc_vecq_block_sums(int type, const void* w, const void* y, int k, int nrows, int stride_row,
+                         int32_t* out) {
+  const int qk = orc_block_elements(type);
+  const int bs = orc_block_bytes(type);
+  const int per = type == ORC_TYPE_Q8_0 ? 1 : 16;
+  const int blocks = k / qk;
+  for (int r = 0; r < nrows; ++r)
+    for (int b = 0; b < blocks; ++b)
+      orc_block_sums(type, (const uint8_t*)w + ((int64_t)r * stride_row + b) * bs,
+                     (const uint8_t*)y + (int64_t)b * (qk / 32) * 36, out + ((int64_t)r * blocks + b) * per);
+}
+
+/* ------------------------------------------------------------------ MXFP8 */
+
+/* mxfp8_quant.cuh:22-29 */
+uint32_t orc_mxfp8_scale_code(float amax) {
+  const uint32_t bits = bits_of(amax * (1.0f / 448.0f));
+  uint32_t e = (bits >> 23) & 0xFFu;
+  if (bits & 0x7FFFFFu) ++e;
+  return e > 253u ? 253u : e;
+}
+/* mxfp8_quant.cuh:33-35 */
+float orc_mxfp8_inverse_scale(uint32_t e) { return float_of((254u - e) << 23); }
+
+/* layout.h:108-113 */
+uint64_t orc_scale_atom_offset(uint64_t row, uint64_t block, uint64_t blocks) {
+  return ((((row / 128) * (blocks / 4)) + (block / 4)) * 512) + ((row % 32) * 16) + (((row % 128) / 32) * 4) +
+         (block % 4);
+}
+
+/* llmp_ops.cu:610-648 */
+void orc_mxfp8_quantize(const float* x, int64_t x_stride, int64_t k, int64_t rows, uint8_t* codes,
+                        uint8_t* scales) {
+  const int64_t blocks = k / 32;
+  const int64_t padded = (rows + 127) / 128 * 128;
+  for (int64_t r = 0; r < padded; ++r) {
+    for (int64_t b = 0; b < blocks; ++b) {
+      const uint64_t at = orc_scale_atom_offset((uint64_t)r, (uint64_t)b, (uint64_t)blocks);
+      if (r >= rows) {
+        scales[at] = 0;
+        continue;
+      }
+      const float* v = x + r * x_stride + b * 32;
+      float amax = 0.0f;
+      for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(v[j]));
+      const uint32_t e = orc_mxfp8_scale_code(amax);
+      const float inverse = orc_mxfp8_inverse_scale(e);
+      for (int j = 0; j < 32; ++j) codes[r * k + b * 32 + j] = orc_f32_to_e4m3(v[j] * inverse);
+      scales[at] = (uint8_t)e;
+    }
+  }
+}
+
+/* llmp_ops.cu:652-663 */
+void orc_mxfp8_swizzle(const uint8_t* in, int64_t n, int64_t blocks, uint8_t* out) {
+  const int64_t padded = (n + 127) / 128 * 128;
+  for (int64_t r = 0; r < padded; ++r)
+    for (int64_t b = 0; b < blocks; ++b)
+      out[orc_scale_atom_offset((uint64_t)r, (uint64_t)b, (uint64_t)blocks)] = r < n ? in[r * blocks + b] : 0;
+}
+
+double orc_mxfp8_dot(const uint8_t* a_codes, const uint8_t* a_scales, int64_t row_a,
+                     const uint8_t* b_codes, const uint8_t* b_scales, int64_t row_b, int64_t k) {
+  const int64_t blocks = k / 32;
+  double total = 0;
+  for (int64_t b = 0; b < blocks; ++b) {
+    const double sa = orc_e8m0_to_f32(a_scales[orc_scale_atom_offset((uint64_t)row_a, (uint64_t)b, (uint64_t)blocks)]);
+    const double sb = orc_e8m0_to_f32(b_scales[orc_scale_atom_offset((uint64_t)row_b, (uint64_t)b, (uint64_t)blocks)]);
+    double s = 0;
+    for (int j = 0; j < 32; ++j)
+      s += (double)orc_e4m3_to_f32(a_codes[row_a * k + b * 32 + j]) * (double)orc_e4m3_to_f32(b_codes[row_b * k + b * 32 + j]);
+    total += s * sa * sb;
+  }
+  return total;
+}
+
+void orc_mxfp8_gemm(const uint8_t* a_codes, const uint8_t* a_scales, const uint8_t* b_codes,
+                    const uint8_t* b_scales, int64_t m, int64_t n, int64_t k, float* d, int threads) {
+  /* Dequantize both operands once (exact in float: an E4M3 value times a power of two,
+   * subnormal results aside), then float-accumulated dot products. */
+  const int64_t blocks = k / 32;
+  float table[256];
+  for (int i = 0; i < 256; ++i) table[i] = orc_e4m3_to_f32((uint8_t)i);
+  float* a = (float*)malloc(sizeof(float) * (size_t)(m * k));
+  float* b = (float*)malloc(sizeof(float) * (size_t)(n * k));
+  for (int64_t r = 0; r < m; ++r)
+    for (int64_t c = 0; c < k; ++c)
+      a[r * k + c] = table[a_codes[r * k + c]] *
+                     orc_e8m0_to_f32(a_scales[orc_scale_atom_offset((uint64_t)r, (uint64_t)(c / 32), (uint64_t)blocks)]);
+  for (int64_t r = 0; r < n; ++r)
+    for (int64_t c = 0; c < k; ++c)
+      b[r * k + c] = table[b_codes[r * k + c]] *
+                     orc_e8m0_to_f32(b_scales[orc_scale_atom_offset((uint64_t)r, (uint64_t)(c / 32), (uint64_t)blocks)]);
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t i = 0; i < m; ++i) {
+    for (int64_t j = 0; j < n; ++j) {
+      const float* ar = a + i * k;
+      const float* br = b + j * k;
+      float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      for (int64_t c = 0; c < k; c += 8)
+        for (int l = 0; l < 8; ++l) acc[l] += ar[c + l] * br[c + l];
+      d[i * n + j] = ((acc[0] + acc[4]) + (acc[2] + acc[6])) + ((acc[1] + acc[5]) + (acc[3] + acc[7]));
+    }
+  }
+  free(a);
+  free(b);
+}
+
+void orc_mxfp8_gemv(const uint8_t* codes, const uint8_t* scales, int64_t n, int64_t k,
+                    const float* x, int64_t tokens, float* y) {
+  const int64_t blocks = k / 32;
+  for (int64_t t = 0; t < tokens; ++t)
+    for (int64_t r = 0; r < n; ++r) {
+      double total = 0;
+      for (int64_t b = 0; b < blocks; ++b) {
+        double s = 0;
+        for (int j = 0; j < 32; ++j) s += (double)orc_e4m3_to_f32(codes[r * k + b * 32 + j]) * (double)x[t * k + b * 32 + j];
+        total += s * (double)orc_e8m0_to_f32(scales[r * blocks + b]);
+      }
+      y[t * n + r] = (float)total;
+    }
+}
+
+/* -------------------------------------------------------------------- MoE */
+
+/* exec.cc:279-315,1728-1818 (kSoftmaxTopK, no bias) */
+void orc_route(const float* logits, int64_t experts, int64_t used, int64_t tokens, int normalize,
+               float scale, int32_t* ids, float* weights) {
+  double* p = (double*)malloc(sizeof(double) * (size_t)experts);
+  int64_t* idx = (int64_t*)malloc(sizeof(int64_t) * (size_t)experts);
+  for (int64_t t = 0; t < tokens; ++t) {
+    const float* l = logits + t * experts;
+    double max = -INFINITY;
+    for (int64_t i = 0; i < experts; ++i) max = max < (double)l[i] ? (double)l[i] : max; /* std::max */
+    if (!isfinite(max)) {
+      for (int64_t i = 0; i < experts; ++i) p[i] = 0.0;
+    } else {
+      double sum = 0.0;
+      for (int64_t i = 0; i < experts; ++i) {
+        p[i] = exp((double)l[i] - max);
+        sum += p[i];
+      }
+      for (int64_t i = 0; i < experts; ++i) p[i] = sum > 0.0 ? p[i] / sum : 0.0;
+    }
+    /* Order(): stable, descending, NaN last (insertion sort keeps equal keys in index order). */
+    for (int64_t i = 0; i < experts; ++i) idx[i] = i;
+    for (int64_t i = 1; i < experts; ++i) {
+      const int64_t v = idx[i];
+      int64_t j = i;
+      while (j > 0) {
+        const double x = p[v], y = p[idx[j - 1]];
+        const int before = (isnan(x) || isnan(y)) ? (!isnan(x) && isnan(y)) : (x > y);
+        if (!before) break;
+        idx[j] = idx[j - 1];
+        --j;
+      }
+      idx[j] = v;
+    }
+    double sum = 0.0;
+    for (int64_t i = 0; i < used; ++i) sum += p[idx[i]];
+    for (int64_t i = 0; i < used; ++i) {
+      double w = p[idx[i]];
+      if (normalize) w /= (sum > 0x1p-14 ? sum : 0x1p-14);
+      ids[t * used + i] = (int32_t)idx[i];
+      weights[t * used + i] = (float)(w * (double)scale);
+    }
+  }
+  free(p);
+  free(idx);
+}
+
+/* exec.cc:1003-1025 */
+int orc_expert_sort(const int32_t* ids, int64_t pairs, int64_t experts, int32_t* order,
+                    int32_t* offsets) {
+  for (int64_t i = 0; i < pairs; ++i)
+    if (ids[i] < 0 || ids[i] >= experts) return 1;
+  int64_t n = 0;
+  for (int64_t e = 0; e < experts; ++e) {
+    offsets[e] = (int32_t)n;
+    for (int64_t i = 0; i < pairs; ++i)
+      if (ids[i] == e) order[n++] = (int32_t)i;
+  }
+  offsets[experts] = (int32_t)n;
+  return 0;
+}
+
+/* exec.cc:1837-1853 in the float arithmetic of llmp_fused.cu:219-235 */
+void orc_expert_reduce(const float* x, const float* w, int64_t width, int64_t used, int64_t tokens,
+                       float* out) {
+  for (int64_t t = 0; t < tokens; ++t)
+    for (int64_t i = 0; i < width; ++i) {
+      float acc = 0.0f;
+      for (int64_t u = 0; u < used; ++u) {
+        const float e = x[(t * used + u) * width + i] * w[t * used + u];
+        acc = u == 0 ? e : acc + e;
+      }
+      out[t * width + i] = acc;
+    }
+}
+
+/* ------------------------------------------------------------------- EXL3 */
+
+static uint32_t lop3(uint32_t x) { return (x & 0x8FFF8FFFu) ^ 0x3B603B60u; } /* decode_exl3.cc:28 */
+static uint16_t half_sum(uint32_t x) {                                       /* decode_exl3.cc:33-37 */
+  const float sum = orc_f16_to_f32((uint16_t)(x & 0xFFFFu)) + orc_f16_to_f32((uint16_t)(x >> 16));
+  return orc_f32_to_f16(sum);
+}
+
+/* decode_exl3.cc:41-66 */
+uint16_t orc_exl3_codebook(int codebook, uint16_t state) {
+  uint32_t x = state;
+  switch (codebook) {
+    case ORC_CB_3INST:
+      x = x * 89226354u + 64248484u;
+      return half_sum(lop3(x));
+    case ORC_CB_MCG:
+      x *= 0xCBAC1FEDu;
+      return half_sum(lop3(x));
+    case ORC_CB_MUL1: {
+      x *= 0x83DCD12Du;
+      const uint32_t sum = (x & 0xFFu) + ((x >> 8) & 0xFFu) + ((x >> 16) & 0xFFu) + (x >> 24) + 0x6400u;
+      const float h = orc_f16_to_f32((uint16_t)(sum & 0xFFFFu));
+      return orc_f32_to_f16(fmaf(h, orc_f16_to_f32(0x1EEEu), orc_f16_to_f32(0xC931u)));
+    }
+    default:
+      return 0x7E00u;
+  }
+}
+
+static uint32_t tile_word(const uint8_t* tile, uint32_t w) {
+  uint32_t v;
+  memcpy(&v, tile + 4 * (size_t)w, 4);
+  return v;
+}
+
+/* decode_exl3.cc:82-96 */
+uint16_t orc_exl3_state(const uint8_t* tile, uint32_t bits, uint32_t t) {
+  const uint32_t words = bits * 256 / 32;
+  const uint32_t b0 = t * bits + bits - 16 + 256 * bits;
+  const uint32_t b1 = b0 + 16;
+  const uint32_t i0 = b0 / 32;
+  const uint32_t i1 = (b1 - 1) / 32;
+  const uint32_t s0 = (i1 + 1) * 32 - b1;
+  const uint64_t merged = ((uint64_t)tile_word(tile, i0 % words) << 32) | tile_word(tile, i1 % words);
+  return (uint16_t)((merged >> s0) & 0xFFFFu);
+}
+
+/* decode_exl3.cc:98-127 */
+void orc_exl3_placement(uint8_t* at) {
+  for (int lane = 0; lane < 32; ++lane) {
+    if (lane & 4) continue;
+    for (int reg = 0; reg < 4; ++reg)
+      for (int high = 0; high < 2; ++high) {
+        const int row = (lane % 4) * 2 + (reg % 2) * 8 + high;
+        const int pair = lane / 8 + (reg / 2) * 4;
+        const int position = 8 * lane + 2 * reg + high;
+        at[position] = (uint8_t)(row * 16 + 2 * pair);
+        at[position + 32] = (uint8_t)(row * 16 + 2 * pair + 1);
+      }
+  }
+}
+
+static const uint16_t* codebook_table(int codebook) {
+  static uint16_t tables[3][65536];
+  static int ready[3];
+#pragma omp critical(orc_codebook)
+  if (!ready[codebook]) {
+    for (uint32_t s = 0; s < 65536; ++s) tables[codebook][s] = orc_exl3_codebook(codebook, (uint16_t)s);
+    ready[codebook] = 1;
+  }
+  return tables[codebook];
+}
+
+/* decode_exl3.cc:157-171: one tile's 256 values, F16 bits, row-major. */
+static void tile_values(const uint8_t* tile, int bits, const uint16_t* table, const uint8_t* place, uint16_t* out) {
+  for (uint32_t t = 0; t < 256; ++t) out[place[t]] = table[orc_exl3_state(tile, (uint32_t)bits, t)];
+}
+
+/* decode_exl3.cc:202-215 */
+void orc_exl3_rotated(const uint8_t* trellis, int64_t k, int64_t n, int bits, int codebook,
+                      int64_t first, int64_t count, uint16_t* out) {
+  uint8_t place[256];
+  orc_exl3_placement(place);
+  const uint16_t* table = codebook_table(codebook);
+  const int64_t tile_bytes = 32 * (int64_t)bits;
+  uint16_t tile[256];
+  for (int64_t kt = 0; kt < k / 16; ++kt)
+    for (int64_t nt = first / 16; nt < (first + count) / 16; ++nt) {
+      tile_values(trellis + (kt * (n / 16) + nt) * tile_bytes, bits, table, place, tile);
+      for (int r = 0; r < 16; ++r) memcpy(&out[(kt * 16 + r) * count + nt * 16 - first], &tile[r * 16], 32);
+    }
+}
+
+/* decode_exl3.cc:173-188 */
+static void hadamard128(double* v) {
+  for (int h = 1; h < 128; h *= 2)
+    for (int i = 0; i < 128; i += 2 * h)
+      for (int j = i; j < i + h; ++j) {
+        const double a = v[j], b = v[j + h];
+        v[j] = a + b;
+        v[j + h] = a - b;
+      }
+}
+
+/* decode_exl3.cc:217-265 */
+void orc_exl3_rows(const uint8_t* trellis, const uint16_t* suh, const uint16_t* svh, int64_t k,
+                   int64_t n, int bits, int codebook, int64_t first, int64_t count, float* out) {
+  const int64_t end = first + count;
+  uint16_t* rot = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)(k * 128));
+  double* block = (double*)malloc(sizeof(double) * (size_t)(k * 128));
+  double* column = (double*)malloc(sizeof(double) * (size_t)k);
+  for (int64_t b = first / 128; b * 128 < end; ++b) {
+    orc_exl3_rotated(trellis, k, n, bits, codebook, b * 128, 128, rot);
+    for (int64_t i = 0; i < k * 128; ++i) block[i] = orc_f16_to_f32(rot[i]);
+    for (int64_t row = 0; row < k; ++row) hadamard128(&block[row * 128]);
+    const int64_t lo = first > b * 128 ? first : b * 128;
+    const int64_t hi = end < (b + 1) * 128 ? end : (b + 1) * 128;
+    for (int64_t c = lo; c < hi; ++c) {
+      const int64_t j = c - b * 128;
+      for (int64_t row = 0; row < k; ++row) column[row] = block[row * 128 + j];
+      for (int64_t kb = 0; kb < k; kb += 128) hadamard128(&column[kb]);
+      const double sv = orc_f16_to_f32(svh[c]);
+      float* y = out + (c - first) * k;
+      for (int64_t row = 0; row < k; ++row) y[row] = (float)(column[row] * (double)orc_f16_to_f32(suh[row]) * sv / 128.0);
+    }
+  }
+  free(rot);
+  free(block);
+  free(column);
+}
+
+void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t* svh, int64_t k,
+                     int64_t n, int bits, int codebook, const uint16_t* x, int64_t m, float* y,
+                     int threads) {
+  const double r = 0.088388347648; /* validate.h:64 */
+  double* xh = (double*)malloc(sizeof(double) * (size_t)(m * k));
+  for (int64_t i = 0; i < m; ++i) {
+    double* row = xh + i * k;
+    for (int64_t c = 0; c < k; ++c) row[c] = (double)orc_f16_to_f32(x[i * k + c]) * (double)orc_f16_to_f32(suh[c]);
+    for (int64_t kb = 0; kb < k; kb += 128) hadamard128(&row[kb]);
+    for (int64_t c = 0; c < k; ++c) row[c] = orc_f16_to_f32(orc_f32_to_f16((float)(row[c] * r)));
+  }
+  (void)codebook_table(codebook);
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t b = 0; b < n / 128; ++b) {
+    uint16_t* rot = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)(k * 128));
+    float* rotf = (float*)malloc(sizeof(float) * (size_t)(k * 128));
+    orc_exl3_rotated(trellis, k, n, bits, codebook, b * 128, 128, rot);
+    for (int64_t i = 0; i < k * 128; ++i) rotf[i] = orc_f16_to_f32(rot[i]);
+    for (int64_t i = 0; i < m; ++i) {
+      double acc[128];
+      for (int j = 0; j < 128; ++j) acc[j] = 0;
+      for (int64_t c = 0; c < k; ++c) {
+        const double xv = xh[i * k + c];
+        const float* wr = rotf + c * 128;
+        for (int j = 0; j < 128; ++j) acc[j] += xv * (double)wr[j];
+      }
+      hadamard128(acc);
+      for (int j = 0; j < 128; ++j) y[i * n + b * 128 + j] = (float)(acc[j] * r * (double)orc_f16_to_f32(svh[b * 128 + j]));
+    }
+    free(rot);
+    free(rotf);
+  }
+  free(xh);
+}

@@ -1,0 +1,189 @@
+"""Parity of llmp.q8_1 and llmp.vecq (HIP, through the C ABI) against the CPU oracle on
+the same seeded inputs. Integer work is compared bit for bit; float outputs to a maximum
+relative error of 1e-3 (the accumulation order is the only difference)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import rel_close
+from llmp_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K = ops.TYPE_Q8_0, ops.TYPE_Q4_K
+TOL = 1e-3
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def make_weights(t, n, k, seed, plausible=True):
+    if plausible:
+        return synth.q8_0_weights(n, k, seed) if t == Q8_0 else synth.q4_k_weights(n, k, seed)
+    return synth.random_blocks(t, n, k, seed)
+
+
+@pytest.mark.parametrize("k,rows", [(4096, 1), (3840, 8), (32, 3), (544, 5)])
+def test_q8_1_quantize_is_bit_exact(device, k, rows):
+    x = synth.activations(rows, k, 11 + k)
+    x[0, : min(k, 40)] = 0.0  # a zero block
+    if rows > 1:
+        x[1] *= 1e-6
+    want = oracle.q8_1_quantize(x)
+    got = ops.quantize_q8_1(dev(x, device)).cpu().numpy()
+    assert got.shape == want.shape
+    assert np.array_equal(got, want)
+
+
+def test_q8_1_planes_and_strides(device):
+    x = synth.activations(2 * 3, 256, 5).reshape(2, 3, 256)
+    wide = np.zeros((2, 3, 300), dtype=np.float32)
+    wide[:, :, :256] = x
+    xd = dev(wide, device)[:, :, :256]
+    got = ops.quantize_q8_1(xd).cpu().numpy()
+    want = oracle.q8_1_quantize(x.reshape(6, 256)).reshape(2, 3, -1)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("t,k,n", [(Q8_0, 4096, 64), (Q4_K, 3840, 40), (Q8_0, 96, 9), (Q4_K, 256, 7)])
+def test_block_sums_are_bit_exact(device, t, k, n):
+    w = make_weights(t, n, k, 21, plausible=False)
+    q8 = oracle.q8_1_quantize(synth.activations(1, k, 22))
+    want = oracle.vecq_block_sums(t, w, q8, k, n)
+    got = ops.vecq_block_sums(t, dev(w, device), dev(q8, device), k, n).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+@pytest.mark.parametrize("k,n", [(4096, 256), (3840, 100), (512, 33), (256, 1)])
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4, 8, 16])
+def test_dense_matches_oracle(device, t, k, n, tokens):
+    w = make_weights(t, n, k, 31 + k + n)
+    x = synth.activations(tokens, k, 32 + tokens)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+def test_every_variant_matches_and_random_bytes_decode(device, t):
+    k, n, tokens = 1024, 50, 5
+    w = make_weights(t, n, k, 41, plausible=False)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
+    want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
+    for variant in range(len(ops.vecq_variants())):
+        got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
+        ok, worst = rel_close(got, want, TOL)
+        assert ok, (variant, worst)
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+@pytest.mark.parametrize("glu", [ops.GLU_SWIGLU, ops.GLU_SWIGLU_CLAMP, ops.GLU_GEGLU])
+@pytest.mark.parametrize("tokens", [1, 4, 8])
+def test_fused_glu_matches_oracle(device, t, glu, tokens):
+    k, n = 1280 if t == Q8_0 else 1280, 72
+    gate = make_weights(t, n, k, 51)
+    up = make_weights(t, n, k, 52)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 53))
+    limit = 0.75 if glu == ops.GLU_SWIGLU_CLAMP else 0.0
+    want = oracle.vecq(t, up, q8, k, n, gate=gate, tokens=tokens, glu=glu, limit=limit)
+    got = ops.vecq(t, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens, glu=glu,
+                   limit=limit).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+@pytest.mark.parametrize("xdtype", ["f32", "bf16"])
+def test_fused_activation_quantization_equals_the_two_step_path(device, t, xdtype):
+    """The in-LDS quantizer is the quantizer kernel's arithmetic: outputs equal bit for bit."""
+    k, n, tokens = 3840, 64, 4
+    w = make_weights(t, n, k, 61)
+    x = synth.activations(tokens, k, 62)
+    if xdtype == "bf16":
+        bits = synth.bf16_bits(x)
+        x = synth.bf16_to_f32(bits)
+        xd = dev(bits.view(np.int16), device).view(torch.bfloat16)
+    else:
+        xd = dev(x, device)
+    q8 = ops.quantize_q8_1(dev(x, device))
+    two = ops.vecq(t, dev(w, device), q8, k, n, tokens=tokens).cpu().numpy()
+    one = ops.vecq_fused(t, dev(w, device), xd, k, n, tokens=tokens).cpu().numpy()
+    assert np.array_equal(one.view(np.uint32), two.view(np.uint32))
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+@pytest.mark.parametrize("tokens,used", [(1, 8), (4, 8), (16, 8), (3, 2)])
+def test_routed_experts_match_oracle(device, t, tokens, used):
+    k, n, experts = 512, 48, 12
+    qk, bs = oracle.block_elements(t), oracle.block_bytes(t)
+    w = make_weights(t, experts * n, k, 71).reshape(experts, n * (k // qk) * bs)
+    g = synth.rng(72)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 73))
+    stride_expert = n * (k // qk)
+    want = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+def test_grouped_matrices_read_their_own_rows(device):
+    t, k, n, groups, tokens = Q8_0, 256, 24, 3, 2
+    qk, bs = 32, 34
+    w = make_weights(t, groups * n, k, 81).reshape(groups, -1)
+    x = synth.activations(tokens * groups, k, 82)
+    q8 = oracle.q8_1_quantize(x)  # [tokens * groups, blocks]: row t * groups + g
+    y_row = ops.padded_k(k) // 32
+    kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // qk), y_token=y_row * groups, y_slot=y_row)
+    want = oracle.vecq(t, w, q8, k, n, **kw)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, **kw).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+def test_tokens_are_independent_and_zero_rows_give_zero(device):
+    """tests/unit/dsv4_fast_test.cc:462-493 of the reference: each token's sums are its
+    one-token product's bit for bit; a zero input row gives zeros."""
+    t, k, n, tokens = Q4_K, 2816, 96, 4
+    gate = make_weights(t, n, k, 91)
+    up = make_weights(t, n, k, 92)
+    x = synth.activations(tokens, k, 93) * 0.5
+    x[0] = 0.0
+    x[3] *= 10
+    wd, gd = dev(up, device), dev(gate, device)
+    q8 = ops.quantize_q8_1(dev(x, device))
+    got = ops.vecq(t, wd, q8, k, n, gate=gd, tokens=tokens, glu=ops.GLU_GEGLU).cpu().numpy()
+    assert np.all(got[0] == 0)
+    for i in range(tokens):
+        solo_q8 = ops.quantize_q8_1(dev(x[i:i + 1], device))
+        solo = ops.vecq(t, wd, solo_q8, k, n, gate=gd, tokens=1, glu=ops.GLU_GEGLU).cpu().numpy()
+        assert np.array_equal(solo[0].view(np.uint32), got[i].view(np.uint32)), i
+
+
+def test_guard_bytes_stay_untouched_and_refusals_queue_nothing(device):
+    """tests/unit/dsv4_fast_test.cc:391-399,494-502 of the reference."""
+    t, k, n = Q8_0, 512, 30
+    w = dev(make_weights(t, n, k, 95), device)
+    q8 = ops.quantize_q8_1(dev(synth.activations(1, k, 96), device))
+    buf = torch.full((64 + n + 64,), float("nan"), dtype=torch.float32, device=device)
+    buf.view(torch.int32).fill_(0x25A5A5A5)
+    out = buf[64:64 + n].view(1, 1, n)
+    ops.vecq(t, w, q8, k, n, out=out)
+    guard = buf.view(torch.int32).cpu().numpy()
+    assert np.all(guard[:64] == 0x25A5A5A5) and np.all(guard[64 + n:] == 0x25A5A5A5)
+    before = buf.clone()
+    with pytest.raises(ops.KernelFailure) as e:
+        ops.vecq(t, w, q8, k, n, glu=ops.GLU_GEGLU, out=out)  # a GLU without gate weights
+    assert e.value.rejected
+    with pytest.raises(ops.KernelFailure):
+        ops.vecq(t, w, q8, k, n, tokens=17, out=out)
+    with pytest.raises(ops.KernelFailure):
+        ops.vecq(t, w, q8, 500, n, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(before.view(torch.int32), buf.view(torch.int32))
