@@ -104,7 +104,8 @@ int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp_vecq_sourc
  * caller zeroes first): sums[(row * blocks + b) * per + i] with per = 1 for
  * Q8_0 (sum of w * q) and 16 for Q4_K (eight sub-block sums of code * q, then
  * eight of q; tests/unit/dsv4_fast_test.cc:185-191). */
-int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int32_t* sums, void* stream);
+int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums,
+                             void* stream);
 
 #ifdef __cplusplus
 }

@@ -43,7 +43,7 @@ SYMBOLS = {
     "llmp_hip_vecq_variants": (_int, []),
     "llmp_hip_vecq_variant_name": (C.c_char_p, [_int]),
     "llmp_hip_vecq_fused": (_int, [_int, C.POINTER(VecQDesc), C.POINTER(VecQSource), _int, _vp]),
-    "llmp_hip_vecq_block_sums": (_int, [_int, C.POINTER(VecQDesc), _vp, _vp]),
+    "llmp_hip_vecq_block_sums": (_int, [_int, C.POINTER(VecQDesc), _int, _vp, _vp]),
 }
 
 _lib = None

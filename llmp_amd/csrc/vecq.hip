@@ -24,75 +24,10 @@
 
 #include "common.h"
 #include "llmp_hip.h"
+#include "vecq_common.h"
 
 namespace llmp_hip {
 namespace {
-
-constexpr int kMaxPairs = 128;  // used * tokens of a routed product
-constexpr int kThreads = 256;
-constexpr int kQ8Block = 36;
-constexpr int kLdsBudget = 60 * 1024;
-
-// ------------------------------------------------------------- quantizer
-
-// Eight lanes quantize one 32-value block, four consecutive values a lane:
-// amax over the block, d = amax / 127 (IEEE), q = round-half-away(x / d), 0 for
-// a zero block. `sum` is the 32 values added in a 32-lane xor butterfly's order
-// (offsets 16, 8, 4, 2, 1 over one value a lane), whatever the lane mapping.
-struct Q8Block {
-  float d;
-  float sum;
-  uint32_t codes;  // four int8, the first value in the low byte
-};
-
-__device__ __forceinline__ Q8Block QuantizeQ8Block(float x0, float x1, float x2, float x3) {
-#pragma clang fp contract(off)
-  float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
-  amax = fmaxf(amax, ShflXor(amax, 4));
-  amax = fmaxf(amax, ShflXor(amax, 2));
-  amax = fmaxf(amax, ShflXor(amax, 1));
-  const float d = amax / 127.0f;
-  Q8Block out;
-  out.d = d;
-  int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-  if (amax != 0.0f) {
-    q0 = static_cast<int>(roundf(x0 / d));
-    q1 = static_cast<int>(roundf(x1 / d));
-    q2 = static_cast<int>(roundf(x2 / d));
-    q3 = static_cast<int>(roundf(x3 / d));
-  }
-  out.codes = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
-  // value 4L + c pairs with 4(L ^ 4) + c at offset 16, 4(L ^ 2) + c at 8, 4(L ^ 1) + c at 4.
-  float s0 = x0, s1 = x1, s2 = x2, s3 = x3;
-#pragma unroll
-  for (int mask = 4; mask >= 1; mask >>= 1) {
-    s0 = s0 + ShflXor(s0, mask);
-    s1 = s1 + ShflXor(s1, mask);
-    s2 = s2 + ShflXor(s2, mask);
-    s3 = s3 + ShflXor(s3, mask);
-  }
-  out.sum = (s0 + s2) + (s1 + s3);
-  return out;
-}
-
-template <int XT>
-__device__ __forceinline__ void Load4(const void* base, int64_t at, int64_t k, float (&v)[4]) {
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int64_t i = at + c;
-    float x = 0.0f;
-    if (i < k) {
-      if constexpr (XT == LLMP_X_F32) {
-        x = static_cast<const float*>(base)[i];
-      } else if constexpr (XT == LLMP_X_BF16) {
-        x = Bf16BitsToFloat(static_cast<const uint16_t*>(base)[i]);
-      } else {
-        x = HalfBitsToFloat(static_cast<const uint16_t*>(base)[i]);
-      }
-    }
-    v[c] = x;
-  }
-}
 
 // grid (ceil(blocks / 32), rows, planes), 256 threads: 32 blocks a workgroup.
 __global__ __launch_bounds__(kThreads) void QuantizeQ8Kernel(const float* __restrict__ x, uint8_t* __restrict__ out,
@@ -112,36 +47,6 @@ __global__ __launch_bounds__(kThreads) void QuantizeQ8Kernel(const float* __rest
   uint8_t* dst = out + ((plane * rows + row) * blocks + block) * kQ8Block;
   *reinterpret_cast<uint32_t*>(dst + 4 + lane8 * 4) = q.codes;
   if (lane8 == 0) *reinterpret_cast<uint32_t*>(dst) = FloatToHalfBits(q.d) | (FloatToHalfBits(q.sum) << 16);
-}
-
-// ------------------------------------------------------------------ vecq
-
-struct VecQArgs {
-  llmp_vecq_desc d;
-  const void* x;  // fused form: unquantized rows
-  int64_t x_token;
-  int64_t x_slot;
-  int kp;         // k rounded up to 512: the staged codes' stride
-  int32_t* dump;  // block sums, or null
-};
-
-__device__ __forceinline__ float Silu(float x) {
-#pragma clang fp contract(off)
-  return x / (1.0f + expf(-x));
-}
-__device__ __forceinline__ float GeluTanh(float x) {
-#pragma clang fp contract(off)
-  return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
-}
-// src/kernels/ggml/vecq.cu:186-195
-__device__ __forceinline__ float Glu(int glu, float gate, float up, float limit) {
-#pragma clang fp contract(off)
-  if (glu == LLMP_GLU_GEGLU) return GeluTanh(gate) * up;
-  if (glu == LLMP_GLU_SWIGLU_CLAMP) {
-    gate = fminf(gate, limit);
-    up = fmaxf(fminf(up, limit), -limit);
-  }
-  return Silu(gate) * up;
 }
 
 // The staged activations of a pass.
@@ -180,27 +85,40 @@ __device__ __forceinline__ void StageQ8(const uint8_t* __restrict__ y, int block
   }
 }
 
-// Stages token slot j from an unquantized row: eight lanes a block.
+// Stages token slot j from an unquantized row: eight lanes a block, the loads of four
+// blocks a lane issued together (one memory round trip for rows up to 4096 values).
 template <bool kQ4K, int XT>
 __device__ __forceinline__ void StageX(const void* __restrict__ x, int k, int kp, int j, uint8_t* codes, float* scales,
                                        uint32_t* halves) {
+  constexpr int kStep = kThreads / 8;  // blocks a sweep of the workgroup
+  constexpr int kAhead = 4;
   const int lane8 = threadIdx.x & 7;
   const int blocks = k / 32;
-  for (int b = threadIdx.x >> 3; b < blocks; b += kThreads / 8) {
-    float v[4];
-    Load4<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, v);
-    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<uint32_t*>(codes + static_cast<int64_t>(j) * kp + b * 32 + lane8 * 4) = q.codes;
-    // The products read the scale as the Q8_1 block stores it: rounded to F16.
-    if (lane8 == 0) scales[j * (kp / 32) + b] = HalfBitsToFloat(FloatToHalfBits(q.d));
-    if constexpr (kQ4K) {
-      int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
-      s += ShflXor(s, 1);
-      s += ShflXor(s, 2);
-      if ((lane8 & 3) == 0) {
-        auto* h16 = reinterpret_cast<int16_t*>(halves + j * (kp / 32));
-        const int h = lane8 >> 2;
-        h16[((b & ~7) + ((b & 7) >> 1) * 2 + h) * 2 + (b & 1)] = static_cast<int16_t>(s);
+  const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
+  for (int b0 = threadIdx.x >> 3; b0 < blocks; b0 += kStep * kAhead) {
+    float v[kAhead][4];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      const int b = b0 + i * kStep;
+      if (b < blocks) Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      const int b = b0 + i * kStep;
+      if (b >= blocks) break;  // whole 8-lane groups leave together
+      const Q8Block q = QuantizeQ8Block(v[i][0], v[i][1], v[i][2], v[i][3]);
+      *reinterpret_cast<uint32_t*>(codes + static_cast<int64_t>(j) * kp + b * 32 + lane8 * 4) = q.codes;
+      // The products read the scale as the Q8_1 block stores it: rounded to F16.
+      if (lane8 == 0) scales[j * (kp / 32) + b] = HalfBitsToFloat(FloatToHalfBits(q.d));
+      if constexpr (kQ4K) {
+        int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
+        s += ShflXor(s, 1);
+        s += ShflXor(s, 2);
+        if ((lane8 & 3) == 0) {
+          auto* h16 = reinterpret_cast<int16_t*>(halves + j * (kp / 32));
+          const int h = lane8 >> 2;
+          h16[((b & ~7) + ((b & 7) >> 1) * 2 + h) * 2 + (b & 1)] = static_cast<int16_t>(s);
+        }
       }
     }
   }
@@ -466,36 +384,7 @@ __global__ __launch_bounds__(kThreads) void VecQKernel(const VecQArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
-  int expert;
-  if (d.ids == nullptr) {
-    // Dense (one slot), or grouped: slot g's weights are matrix g.
-    expert = blockIdx.y;
-    if (tid < d.tokens) pairs[tid] = (tid << 8) | expert;
-    if (tid == 0) count = d.tokens;
-  } else {
-    // One workgroup row per (token, slot) pair; the first pair naming an
-    // expert owns it and computes every pair that names it, in pair order
-    // (src/kernels/ggml/vecq.cu:514-546, with 64-lane ballots).
-    const int s = blockIdx.y;
-    expert = d.ids[(s / d.used) * d.ids_stride + (s % d.used)];
-    if (wave == 0) {
-      const int total = d.tokens * d.used;
-      int n = 0;
-      bool owner = true;
-      for (int base = 0; base < total && owner; base += kWave) {
-        const int s2 = base + lane;
-        const int t = s2 / d.used;
-        const int u = s2 % d.used;
-        const bool match = s2 < total && d.ids[t * d.ids_stride + u] == expert;
-        const unsigned long long ballot = __ballot(match);
-        if (n == 0 && ballot != 0) owner = base + __ffsll(ballot) - 1 == s;
-        if (owner && match) pairs[n + __popcll(ballot & ((1ull << lane) - 1ull))] = (t << 8) | u;
-        n += __popcll(ballot);
-      }
-      if (lane == 0) count = owner ? n : 0;
-    }
-  }
-  __syncthreads();
+  const int expert = ResolvePairs(d, blockIdx.y, pairs, &count);
   const int n = count;
   if (n == 0) return;  // uniform over the workgroup
 
@@ -512,6 +401,18 @@ __global__ __launch_bounds__(kThreads) void VecQKernel(const VecQArgs a) {
 
   for (int p0 = 0; p0 < n; p0 += P) {
     const int m = min(P, n - p0);
+    // D units in flight: the loads of unit i + D are issued before unit i's arithmetic, and
+    // the first D before the activations are staged (they depend on nothing staged).
+    Unit wu[D];
+    Unit gu[kGlu ? D : 1];
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      const int unit = sub + i * LPR;
+      if (unit < units) {
+        wu[i] = T::Load(wrow, unit);
+        if constexpr (kGlu) gu[i] = T::Load(grow, unit);
+      }
+    }
     for (int j = 0; j < m; ++j) {
       const int pr = pairs[p0 + j];
       const int token = pr >> 8;
@@ -536,17 +437,6 @@ __global__ __launch_bounds__(kThreads) void VecQKernel(const VecQArgs a) {
 #pragma unroll
     for (int t = 0; t < (kGlu ? P : 1); ++t) accg[t] = 0.0f;
 
-    // D units in flight: the loads of unit i + D are issued before unit i's arithmetic.
-    Unit wu[D];
-    Unit gu[kGlu ? D : 1];
-#pragma unroll
-    for (int i = 0; i < D; ++i) {
-      const int unit = sub + i * LPR;
-      if (unit < units) {
-        wu[i] = T::Load(wrow, unit);
-        if constexpr (kGlu) gu[i] = T::Load(grow, unit);
-      }
-    }
     for (int base = sub; base < units; base += D * LPR) {
 #pragma unroll
       for (int i = 0; i < D; ++i) {
@@ -595,7 +485,10 @@ struct Variant {
 constexpr Variant kVariants[] = {
     {"lanes8 pass1 flight4", 8, 1, 4},   {"lanes8 pass2 flight3", 8, 2, 3},   {"lanes8 pass4 flight2", 8, 4, 2},
     {"lanes8 pass8 flight2", 8, 8, 2},   {"lanes16 pass1 flight4", 16, 1, 4}, {"lanes64 pass1 flight2", 64, 1, 2},
+    // Q4_K only: a lane a super-block (vecq_flat.hip); `lanes` 0 marks the form.
+    {"flat pass1", 0, 1, 2},             {"flat pass4", 0, 4, 2},
 };
+constexpr int kFlatFirst = 6;
 constexpr int kVariantCount = sizeof(kVariants) / sizeof(kVariants[0]);
 
 size_t LdsBytes(int pass, int kp) { return static_cast<size_t>(pass) * (kp + kp / 8 + kp / 8); }
@@ -658,8 +551,9 @@ void LaunchVariant(const VecQArgs& a, int x_type, int variant, dim3 grid, size_t
 
 // The default configuration of a shape: the tokens of a pass first (each pass
 // streams the weights again), then enough lanes a row to fill the device.
-int DefaultVariant(const llmp_vecq_desc& d, int kp) {
+int DefaultVariant(int type, const llmp_vecq_desc& d, int kp) {
   const int tokens = d.tokens;
+  if (type == LLMP_TYPE_Q4_K && FlatQ4KTakes(d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
   while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
   switch (pass) {
@@ -713,13 +607,20 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   }
   a.kp = PaddedK(d->ncols_x);
   a.dump = dump;
-  if (variant < 0) variant = DefaultVariant(*d, a.kp);
+  if (variant < 0) variant = DefaultVariant(type, *d, a.kp);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
+  if (v.lanes == 0) {
+    if (type != LLMP_TYPE_Q4_K || !FlatQ4KTakes(*d)) return Refuse(1, "vecq: the flat form takes Q4_K rows up to 65536 values");
+    if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
+      return Refuse(1, "vecq: block sums are of a dense one-token product");
+    LaunchFlatQ4K(a, x_type, v.pass, static_cast<hipStream_t>(stream));
+    return LaunchStatus("vecq");
+  }
   const size_t lds = LdsBytes(v.pass, a.kp);
   if (lds > static_cast<size_t>(kLdsBudget))
     return Refuse(1, "vecq: %d tokens of k %d do not fit the staging area", v.pass, d->ncols_x);
-  if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr || variant != 0))
+  if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
     return Refuse(1, "vecq: block sums are of a dense one-token product");
   const int slots = d->ids != nullptr ? d->used * d->tokens : d->used;
   const int rows_per_group = (kWave / v.lanes) * (kThreads / kWave);
@@ -770,9 +671,11 @@ extern "C" int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp
   return Launch(type, d, x, variant, nullptr, stream);
 }
 
-extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int32_t* sums, void* stream) {
+extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums, void* stream) {
   if (sums == nullptr) return Refuse(1, "vecq: null sums");
-  return Launch(type, d, nullptr, 0, sums, stream);
+  if (variant < 0 && d != nullptr) variant = type == LLMP_TYPE_Q4_K && FlatQ4KTakes(*d) ? kFlatFirst : 0;
+  if (variant != 0 && variant != kFlatFirst) return Refuse(1, "vecq: block sums are of the one-token variants");
+  return Launch(type, d, nullptr, variant, sums, stream);
 }
 
 extern "C" int llmp_hip_vecq_variants(void) { return kVariantCount; }

@@ -1,0 +1,176 @@
+// Device code shared by the llmp.vecq kernels: the Q8_1 block quantizer, the launch
+// arguments, the GLU, and the (token, slot) pair list of a workgroup.
+#ifndef LLMP_AMD_CSRC_VECQ_COMMON_H_
+#define LLMP_AMD_CSRC_VECQ_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+
+namespace llmp_hip {
+
+constexpr int kMaxPairs = 128;  // used * tokens of a routed product
+constexpr int kThreads = 256;
+constexpr int kQ8Block = 36;
+constexpr int kLdsBudget = 60 * 1024;
+
+// ------------------------------------------------------------- quantizer
+
+// Eight lanes quantize one 32-value block, four consecutive values a lane:
+// amax over the block, d = amax / 127 (IEEE), q = round-half-away(x / d), 0 for
+// a zero block. `sum` is the 32 values added in a 32-lane xor butterfly's order
+// (offsets 16, 8, 4, 2, 1 over one value a lane), whatever the lane mapping.
+struct Q8Block {
+  float d;
+  float sum;
+  uint32_t codes;  // four int8, the first value in the low byte
+};
+
+__device__ __forceinline__ Q8Block QuantizeQ8Block(float x0, float x1, float x2, float x3) {
+#pragma clang fp contract(off)
+  float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
+  amax = fmaxf(amax, ShflXor(amax, 4));
+  amax = fmaxf(amax, ShflXor(amax, 2));
+  amax = fmaxf(amax, ShflXor(amax, 1));
+  const float d = amax / 127.0f;
+  Q8Block out;
+  out.d = d;
+  int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+  if (amax != 0.0f) {
+    q0 = static_cast<int>(roundf(x0 / d));
+    q1 = static_cast<int>(roundf(x1 / d));
+    q2 = static_cast<int>(roundf(x2 / d));
+    q3 = static_cast<int>(roundf(x3 / d));
+  }
+  out.codes = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+  // value 4L + c pairs with 4(L ^ 4) + c at offset 16, 4(L ^ 2) + c at 8, 4(L ^ 1) + c at 4.
+  float s0 = x0, s1 = x1, s2 = x2, s3 = x3;
+#pragma unroll
+  for (int mask = 4; mask >= 1; mask >>= 1) {
+    s0 = s0 + ShflXor(s0, mask);
+    s1 = s1 + ShflXor(s1, mask);
+    s2 = s2 + ShflXor(s2, mask);
+    s3 = s3 + ShflXor(s3, mask);
+  }
+  out.sum = (s0 + s2) + (s1 + s3);
+  return out;
+}
+
+template <int XT>
+__device__ __forceinline__ void Load4(const void* base, int64_t at, int64_t k, float (&v)[4]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int64_t i = at + c;
+    float x = 0.0f;
+    if (i < k) {
+      if constexpr (XT == LLMP_X_F32) {
+        x = static_cast<const float*>(base)[i];
+      } else if constexpr (XT == LLMP_X_BF16) {
+        x = Bf16BitsToFloat(static_cast<const uint16_t*>(base)[i]);
+      } else {
+        x = HalfBitsToFloat(static_cast<const uint16_t*>(base)[i]);
+      }
+    }
+    v[c] = x;
+  }
+}
+
+// Four consecutive elements at `at`, zero past k; one vector load when `wide` says the
+// row allows it (alignment, checked once a row).
+template <int XT>
+__device__ __forceinline__ void Load4Wide(const void* base, int64_t at, int64_t k, bool wide, float (&v)[4]) {
+  if (wide && at + 4 <= k) {
+    if constexpr (XT == LLMP_X_F32) {
+      const float4 f = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + at);
+      v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+    } else {
+      const uint2 u = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + at);
+      if constexpr (XT == LLMP_X_BF16) {
+        v[0] = Bf16BitsToFloat(u.x & 0xFFFFu), v[1] = Bf16BitsToFloat(u.x >> 16);
+        v[2] = Bf16BitsToFloat(u.y & 0xFFFFu), v[3] = Bf16BitsToFloat(u.y >> 16);
+      } else {
+        v[0] = HalfBitsToFloat(u.x & 0xFFFFu), v[1] = HalfBitsToFloat(u.x >> 16);
+        v[2] = HalfBitsToFloat(u.y & 0xFFFFu), v[3] = HalfBitsToFloat(u.y >> 16);
+      }
+    }
+    return;
+  }
+  Load4<XT>(base, at, k, v);
+}
+
+// ------------------------------------------------------------------ vecq
+
+struct VecQArgs {
+  llmp_vecq_desc d;
+  const void* x;  // fused form: unquantized rows
+  int64_t x_token;
+  int64_t x_slot;
+  int kp;         // k rounded up to 512: the staged codes' stride
+  int32_t* dump;  // block sums, or null
+};
+
+__device__ __forceinline__ float Silu(float x) {
+#pragma clang fp contract(off)
+  return x / (1.0f + expf(-x));
+}
+__device__ __forceinline__ float GeluTanh(float x) {
+#pragma clang fp contract(off)
+  return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+}
+// src/kernels/ggml/vecq.cu:186-195
+__device__ __forceinline__ float Glu(int glu, float gate, float up, float limit) {
+#pragma clang fp contract(off)
+  if (glu == LLMP_GLU_GEGLU) return GeluTanh(gate) * up;
+  if (glu == LLMP_GLU_SWIGLU_CLAMP) {
+    gate = fminf(gate, limit);
+    up = fmaxf(fminf(up, limit), -limit);
+  }
+  return Silu(gate) * up;
+}
+
+
+// The pairs a workgroup computes, in pair order, and its expert: a dense or grouped
+// product's slot is its matrix; of a routed product's pairs, the first naming an expert
+// owns it and computes every pair that names it (src/kernels/ggml/vecq.cu:504-546, with
+// 64-lane ballots). Returns the expert; `count` is 0 for a workgroup that owns nothing.
+// Ends with a workgroup barrier.
+__device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_index, int* pairs, int* count) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  int expert;
+  if (d.ids == nullptr) {
+    expert = slot_index;
+    if (tid < d.tokens) pairs[tid] = (tid << 8) | expert;
+    if (tid == 0) *count = d.tokens;
+  } else {
+    const int s = slot_index;
+    expert = d.ids[(s / d.used) * d.ids_stride + (s % d.used)];
+    if (tid < kWave) {
+      const int total = d.tokens * d.used;
+      int n = 0;
+      bool owner = true;
+      for (int base = 0; base < total && owner; base += kWave) {
+        const int s2 = base + lane;
+        const int t = s2 / d.used;
+        const int u = s2 % d.used;
+        const bool match = s2 < total && d.ids[t * d.ids_stride + u] == expert;
+        const unsigned long long ballot = __ballot(match);
+        if (n == 0 && ballot != 0) owner = base + __ffsll(ballot) - 1 == s;
+        if (owner && match) pairs[n + __popcll(ballot & ((1ull << lane) - 1ull))] = (t << 8) | u;
+        n += __popcll(ballot);
+      }
+      if (lane == 0) *count = owner ? n : 0;
+    }
+  }
+  __syncthreads();
+  return expert;
+}
+
+// The flat Q4_K kernel's launch (vecq_flat.hip). x_type -1: Q8_1 activations.
+bool FlatQ4KTakes(const llmp_vecq_desc& d);
+void LaunchFlatQ4K(const VecQArgs& a, int x_type, int pass, hipStream_t stream);
+
+}  // namespace llmp_hip
+
+#endif  // LLMP_AMD_CSRC_VECQ_COMMON_H_

@@ -95,7 +95,7 @@ def vecq_fused(t, w, x, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stri
     return out
 
 
-def vecq_block_sums(t, w, q8, k, nrows):
+def vecq_block_sums(t, w, q8, k, nrows, variant=-1):
     """The kernel's int32 block sums of a dense one-token product: [nrows, blocks, per]."""
     lib = _lib.load()
     per = 1 if t == TYPE_Q8_0 else 16
@@ -103,7 +103,7 @@ def vecq_block_sums(t, w, q8, k, nrows):
     out = torch.empty((1, 1, nrows), dtype=torch.float32, device=w.device)
     d = _desc(t, w, k, nrows, gate=None, q8=q8, ids=None, tokens=1, used=1, stride_row=None,
               stride_expert=0, y_token=None, y_slot=0, glu=GLU_NONE, limit=0.0, out=out)
-    _lib.check(lib.llmp_hip_vecq_block_sums(t, C.byref(d), _ptr(sums), _stream()))
+    _lib.check(lib.llmp_hip_vecq_block_sums(t, C.byref(d), variant, _ptr(sums), _stream()))
     return sums
 
 
