@@ -1,8 +1,10 @@
 """Benchmark of the quantized mat-vec hot path on one MI355X.
 
-A step is one launch of the fused Q4_K gate/up GEGLU mat-vec (hidden 3840, two 15360-row
-matrices, one bf16 token quantized to Q8_1 inside the kernel) over one of several distinct
-weight copies, rotated so that neither L2 nor the 256 MB Infinity Cache holds them.
+A step is the decode-time gate/up product of one token: llmp.q8_1 (the activation's
+quantization to Q8_1) followed by llmp.vecq, the fused Q4_K gate/up GEGLU mat-vec (hidden
+3840, two 15360-row matrices), over one of several distinct weight copies, rotated so that
+neither L2 nor the 256 MB Infinity Cache holds them. --fused makes it the single launch that
+quantizes the bf16 activation inside the kernel.
 Prints one JSON line; see --help."""
 import argparse
 import json
@@ -55,6 +57,9 @@ def main():
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--fused", action="store_true",
+                    help="a step is one launch that quantizes the activations in the kernel, instead of "
+                         "llmp.q8_1 followed by llmp.vecq over its Q8_1 blocks (the reference's two operations)")
     ap.add_argument("--eager", action="store_true", help="launch each step from Python instead of a graph")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -76,59 +81,75 @@ def main():
     xd = torch.from_numpy(x).to(device).to(torch.bfloat16)
     out = torch.empty((args.tokens, 1, N), dtype=torch.float32, device=device)
 
+    x32 = torch.from_numpy(x).to(device)
+    q8 = ops.quantize_q8_1(x32)
+
     def step(i):
         c = i % copies
+        if not args.fused:
+            ops.quantize_q8_1(x32, out=q8.view(1, args.tokens, -1))
+            ops.vecq(ops.TYPE_Q4_K, ups[c], q8, K, N, gate=gates[c], tokens=args.tokens, glu=ops.GLU_GEGLU,
+                     variant=args.variant, out=out)
+            return
         ops.vecq_fused(ops.TYPE_Q4_K, ups[c], xd, K, N, gate=gates[c], tokens=args.tokens,
                        glu=ops.GLU_GEGLU, variant=args.variant, out=out)
 
-    # Decode steps are replayed as captured graphs (the reference's launch contexts capture
-    # them too, src/kernels/ggml/launch.h:34-48): one graph of W launches, one of K launches.
-    def run(count, first):
-        if args.eager:
-            for i in range(count):
-                step(first + i)
-            return None
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            for i in range(count):
-                step(first + i)
-        return graph
+    def kernel_only(i):
+        c = i % copies
+        ops.vecq(ops.TYPE_Q4_K, ups[c], q8, K, N, gate=gates[c], tokens=args.tokens, glu=ops.GLU_GEGLU,
+                 variant=args.variant, out=out)
 
+    # Decode steps are replayed as captured graphs (the reference's launch contexts capture
+    # them too, src/kernels/ggml/launch.h:34-48): one graph of W steps, one of K steps.
     side = torch.cuda.Stream()
+
+    def timed_region(body, count, first):
+        """Milliseconds of `count` calls of body(i), by HIP events on the launching stream."""
+        graph = None
+        if not args.eager:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(count):
+                    body(first + i)
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        begin.record()
+        if graph is None:
+            for i in range(count):
+                body(first + i)
+        else:
+            graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        return begin.elapsed_time(end), (time.perf_counter() - t0) * 1e3
+
     step(0)
     torch.cuda.synchronize()
-    warm = run(args.warmup, 0)
-    timed = run(args.steps, args.warmup) if not args.eager else None
-    if warm is not None:
-        warm.replay()
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    start.record()
-    if args.eager:
-        run(args.steps, args.warmup)
-    else:
-        timed.replay()
-    stop.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms = start.elapsed_time(stop) / args.steps
+    timed_region(step, args.warmup, 0)
+    total_ms, wall_ms = timed_region(step, args.steps, args.warmup)
+    # The dominant kernel alone (the mat-vec over ready Q8_1 blocks), the same rotation.
+    timed_region(kernel_only if not args.fused else step, args.warmup, 0)
+    kernel_ms, _ = timed_region(kernel_only if not args.fused else step, args.steps, args.warmup)
+    kernel_us = kernel_ms / args.steps * 1e3
+    ms = total_ms / args.steps
     value = WEIGHT_BYTES / (ms * 1e-3) / 1e9
-    achieved = algorithmic_bytes(args.tokens) / (ms * 1e-3) / 1e9
+    achieved = algorithmic_bytes(args.tokens) / (kernel_us * 1e-6) / 1e9
     line = {
         "metric": "Q-matvec weight GB/s at batch 1 (Q4_K fused gate/up GEGLU mat-vec)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 dot (Q4_K x Q8_1), fp32 accumulate", "data": "synthetic",
         "config": {"workload": f"GGML Q4_K fused gate/up GEGLU MMVQ, K={K}, N=2x{N}, batch {args.tokens}, "
-                               "bf16 activations quantized to q8_1 in-kernel, fp32 out",
+                               + ("bf16 activations quantized to q8_1 in-kernel" if args.fused else "fp32 activations through llmp.q8_1")
+                               + ", fp32 out",
                    "weight_copies_rotated": copies, "variant": args.variant, "launch": "eager" if args.eager else "hip graph",
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "VecQKernel<Q4_K, glu, bf16 source>",
+                     "kernel": "VecQFlatQ4K (llmp.vecq, Q4_K, GLU)",
                      "algorithmic_bytes_per_launch": algorithmic_bytes(args.tokens),
-                     "avg_launch_us": round(ms * 1e3, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
+                     "avg_launch_us": round(kernel_us, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(gate, up, x)

@@ -11,7 +11,7 @@
 // cache line is requested once, by neighbouring lanes, and no register holds
 // weights in flight. After s_waitcnt vmcnt(0) each lane reads its own
 // super-block, nine 16-byte reads 144 bytes apart (36 dwords: sixteen lanes'
-// reads fall in distinct banks). A workgroup (8 wave64s) stages its tokens'
+// reads fall in distinct banks). A workgroup (8 wave64s, two a CU) stages its tokens'
 // activations once (quantizing them to Q8_1 itself in the fused form) while the
 // waves' first tiles are in flight; after that one barrier its waves are
 // independent: wave w of the grid takes tiles w, w + waves, .... Sixteen waves a
@@ -27,9 +27,9 @@
 //   [320, 336)  sum(codes) of each sub-block as int16 (read by the test dump).
 // A lane's super-block sum is d * sum_g sc_g * d8_g * prod_g - dmin * sum_g m_g *
 // d8_g * sum_g (tests/unit/dsv4_fast_test.cc:179-193), prod_g eight v_dot4_i32_i8.
-// Row sums: the lanes' partials go to the wave's LDS buffer and one lane a row
-// adds them in super-block order, so a (token, row) value never depends on its
-// neighbours or on which wave computed it.
+// Row sums: a suffix sum over the row's lanes by wave shuffles (a fixed tree), so
+// a (token, row) value never depends on its neighbours or on which wave
+// computed it.
 
 #include <hip/hip_runtime.h>
 
@@ -41,7 +41,7 @@ namespace llmp_hip {
 namespace {
 
 constexpr int kRecord = 336;     // bytes a staged super-block
-constexpr int kGroup = 512;      // threads a workgroup
+constexpr int kGroup = 512;      // threads a workgroup: eight waves, two workgroups a CU
 constexpr int kWaves = kGroup / kWave;
 constexpr int kRing = kWave * 9 * 16;  // bytes of a wave's tile buffer
 constexpr int kChunks = 9;       // 16-byte chunks a super-block
@@ -53,61 +53,104 @@ struct SuperBlock {
 
 // ---- staging into records
 
+// Staging is split in two so that a row's first loads can be queued before the wave's first
+// tile: memory operations complete in order, and a load queued behind a tile would wait for it.
+constexpr int kStep = kGroup / 8;  // blocks a sweep of the workgroup covers, eight lanes a block
+constexpr int kFront = 2;          // sweeps loaded ahead: rows up to 4096 values
+
+struct FrontX {
+  float v[kFront][4];
+};
+
 template <int XT>
-__device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k, uint8_t* token) {
-  constexpr int kStep = kGroup / 8;
-  constexpr int kAhead = 4;
+__device__ __forceinline__ FrontX LoadFrontX(const void* __restrict__ x, int k) {
+  FrontX f;
   const int lane8 = threadIdx.x & 7;
-  const int blocks = k / 32;
   const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
-  for (int b0 = threadIdx.x >> 3; b0 < blocks; b0 += kStep * kAhead) {
-    float v[kAhead][4];
 #pragma unroll
-    for (int i = 0; i < kAhead; ++i) {
-      const int b = b0 + i * kStep;
-      if (b < blocks) Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < kAhead; ++i) {
-      const int b = b0 + i * kStep;
-      if (b >= blocks) break;  // whole 8-lane groups leave together
-      const Q8Block q = QuantizeQ8Block(v[i][0], v[i][1], v[i][2], v[i][3]);
-      uint8_t* record = token + (b >> 3) * kRecord;
-      const int g = b & 7;
-      *reinterpret_cast<uint32_t*>(record + g * 32 + lane8 * 4) = q.codes;
-      int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
-      s += ShflXor(s, 1);
-      s += ShflXor(s, 2);
-      s += ShflXor(s, 4);
-      if (lane8 == 0) {
-        // The products read the scale as a Q8_1 block stores it: rounded to F16.
-        const float d8 = HalfBitsToFloat(FloatToHalfBits(q.d));
-        reinterpret_cast<float*>(record + 256)[g] = d8;
-        reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
-        reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
-      }
-    }
+  for (int i = 0; i < kFront; ++i) {
+    const int b = (threadIdx.x >> 3) + i * kStep;
+    if (b < k / 32) Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, f.v[i]);
+  }
+  return f;
+}
+
+// One block of 32 values, eight lanes: its codes, scale and sums into the record.
+__device__ __forceinline__ void StageBlock(const float (&v)[4], int b, uint8_t* token) {
+  const int lane8 = threadIdx.x & 7;
+  const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+  uint8_t* record = token + (b >> 3) * kRecord;
+  const int g = b & 7;
+  *reinterpret_cast<uint32_t*>(record + g * 32 + lane8 * 4) = q.codes;
+  int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
+  s += ShflXor(s, 1);
+  s += ShflXor(s, 2);
+  s += ShflXor(s, 4);
+  if (lane8 == 0) {
+    // The products read the scale as a Q8_1 block stores it: rounded to F16.
+    const float d8 = HalfBitsToFloat(FloatToHalfBits(q.d));
+    reinterpret_cast<float*>(record + 256)[g] = d8;
+    reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
+    reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
   }
 }
 
-__device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, uint8_t* token) {
-  for (int b = threadIdx.x; b < blocks; b += kGroup) {
+template <int XT>
+__device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k, const FrontX& front, uint8_t* token) {
+  const int lane8 = threadIdx.x & 7;
+  const int blocks = k / 32;
+  const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
+#pragma unroll
+  for (int i = 0; i < kFront; ++i) {
+    const int b = (threadIdx.x >> 3) + i * kStep;
+    if (b < blocks) StageBlock(front.v[i], b, token);  // whole 8-lane groups together
+  }
+  for (int b = (threadIdx.x >> 3) + kFront * kStep; b < blocks; b += kStep) {
+    float v[4];
+    Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v);
+    StageBlock(v, b, token);
+  }
+}
+
+struct FrontQ8 {
+  uint32_t w[9];
+};
+
+__device__ __forceinline__ FrontQ8 LoadFrontQ8(const uint8_t* __restrict__ y, int blocks) {
+  FrontQ8 f;
+  const int b = threadIdx.x;
+  if (b < blocks) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
+#pragma unroll
+    for (int i = 0; i < 9; ++i) f.w[i] = src[i];
+  }
+  return f;
+}
+
+__device__ __forceinline__ void StageQ8Block(const uint32_t (&w)[9], int b, uint8_t* token) {
+  uint8_t* record = token + (b >> 3) * kRecord;
+  const int g = b & 7;
+  uint4* dst = reinterpret_cast<uint4*>(record + g * 32);
+  dst[0] = make_uint4(w[1], w[2], w[3], w[4]);
+  dst[1] = make_uint4(w[5], w[6], w[7], w[8]);
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s = Dot4(0x01010101, static_cast<int>(w[1 + i]), s);
+  const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
+  reinterpret_cast<float*>(record + 256)[g] = d8;
+  reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
+  reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
+}
+
+__device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, const FrontQ8& front,
+                                               uint8_t* token) {
+  if (static_cast<int>(threadIdx.x) < blocks) StageQ8Block(front.w, threadIdx.x, token);
+  for (int b = threadIdx.x + kGroup; b < blocks; b += kGroup) {
     const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
     uint32_t w[9];
 #pragma unroll
     for (int i = 0; i < 9; ++i) w[i] = src[i];
-    uint8_t* record = token + (b >> 3) * kRecord;
-    const int g = b & 7;
-    uint4* dst = reinterpret_cast<uint4*>(record + g * 32);
-    dst[0] = make_uint4(w[1], w[2], w[3], w[4]);
-    dst[1] = make_uint4(w[5], w[6], w[7], w[8]);
-    int s = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s = Dot4(0x01010101, static_cast<int>(w[1 + i]), s);
-    const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
-    reinterpret_cast<float*>(record + 256)[g] = d8;
-    reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
-    reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
+    StageQ8Block(w, b, token);
   }
 }
 
@@ -198,53 +241,45 @@ __device__ __forceinline__ void DotSuperBlock(const SuperBlock& b, const uint8_t
   }
 }
 
-struct Tile {
-  int row0;
-  int half;   // super-blocks of one matrix: rows * nsb
-  int total;  // of both
-};
-
-template <bool kGlu>
-__device__ __forceinline__ Tile TileOf(int index, int rows_per_tile, int nrows, int nsb) {
-  Tile t;
-  t.row0 = index * rows_per_tile;
-  t.half = min(rows_per_tile, nrows - t.row0) * nsb;
-  t.total = kGlu ? 2 * t.half : t.half;
-  return t;
-}
-
 typedef __attribute__((address_space(3))) void* LdsPointer;
 typedef const __attribute__((address_space(1))) void* GlobalPointer;
 
-// Queues the tile's chunks into the wave's buffer: chunk 64 j + lane at byte 16 (64 j + lane).
-// kPacked: rows follow each other without a gap, so a matrix's part of the tile is one range.
-template <bool kGlu, bool kPacked>
-__device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t expert_block, const Tile& tile, int nsb,
-                                          uint8_t* ring, int lane) {
-  const int64_t first = expert_block + static_cast<int64_t>(tile.row0) * d.stride_row;
-  const uint8_t* up = static_cast<const uint8_t*>(d.w) + first * 144;
-  const uint8_t* gate = kGlu ? static_cast<const uint8_t*>(d.g) + first * 144 : nullptr;
-  const int half = tile.half * kChunks;
-  const int total = tile.total * kChunks;
+// Queues one matrix's part of a tile into the wave's buffer at `ring`: chunk c = 64 j + lane
+// of `chunks` lands at byte 16 c. `base` and `ring` are the same in every lane.
+// kPacked: rows follow each other without a gap, so the part is one byte range.
+template <int kLoads, bool kPacked>
+__device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int stride_row, int nsb, uint8_t* ring,
+                                          int lane) {
 #pragma unroll
-  for (int j = 0; j < kChunks; ++j) {
-    int c = j * kWave + lane;
-    if (c < total) {
-      const uint8_t* matrix = up;
-      if (kGlu && c >= half) {
-        matrix = gate;
-        c -= half;
-      }
-      int64_t at;
+  for (int j = 0; j < kLoads; ++j) {
+    const int c = j * kWave + lane;
+    if (c < chunks) {
+      const uint8_t* from;
       if constexpr (kPacked) {
-        at = static_cast<int64_t>(c) * 16;
+        from = base + static_cast<uint32_t>(c) * 16u;
       } else {
         const int f = c / kChunks;
         const int row = f / nsb;
-        at = (static_cast<int64_t>(row) * d.stride_row + (f - row * nsb)) * 144 + (c - f * kChunks) * 16;
+        from = base + (static_cast<int64_t>(row) * stride_row + (f - row * nsb)) * 144 + (c - f * kChunks) * 16;
       }
-      __builtin_amdgcn_global_load_lds((GlobalPointer)(matrix + at), (LdsPointer)(ring + j * kWave * 16), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((GlobalPointer)from, (LdsPointer)(ring + j * kWave * 16), 16, 0, 0);
     }
+  }
+}
+
+// The tile of `rows` rows from `row0`. A matrix's part always starts where a full tile's
+// would (`gate_at` bytes into the buffer), so a lane's place in a tile never changes.
+template <bool kGlu, bool kPacked>
+__device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t expert_block, int row0, int rows, int nsb,
+                                          int gate_at, uint8_t* ring, int lane) {
+  const int64_t first = (expert_block + static_cast<int64_t>(row0) * d.stride_row) * 144;
+  const int chunks = rows * nsb * kChunks;
+  if constexpr (kGlu) {
+    // Each matrix at most 32 super-blocks: 288 chunks, five loads.
+    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, d.stride_row, nsb, ring, lane);
+    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.g) + first, chunks, d.stride_row, nsb, ring + gate_at, lane);
+  } else {
+    FetchPart<kChunks, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, d.stride_row, nsb, ring, lane);
   }
 }
 
@@ -255,9 +290,9 @@ __device__ __forceinline__ void AwaitTile() {
   asm volatile("" ::: "memory");
 }
 
-__device__ __forceinline__ SuperBlock ReadSuperBlock(const uint8_t* ring, int lane) {
+__device__ __forceinline__ SuperBlock ReadSuperBlock(const uint8_t* at) {
   SuperBlock b;
-  const U32x4* mine = reinterpret_cast<const U32x4*>(ring + lane * 144);
+  const U32x4* mine = reinterpret_cast<const U32x4*>(at);
   b.header = mine[0];
 #pragma unroll
   for (int i = 0; i < 8; ++i) b.codes[i] = mine[1 + i];
@@ -279,7 +314,17 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
   const int token_stride = nsb * kRecord;
   const int tiles = (d.nrows + rows_per_tile - 1) / rows_per_tile;
   uint8_t* ring = lds + P * token_stride + wave * kRing;
-  float* partial = reinterpret_cast<float*>(ring);  // [P][64], once the super-blocks are read
+
+  // A lane's place in every tile: its matrix, row and super-block.
+  const int half = rows_per_tile * nsb;
+  const bool gate_lane = kGlu && lane >= half;
+  const int f = gate_lane ? lane - half : lane;
+  const int row = f / nsb;
+  const int sb = f - row * nsb;
+  const bool placed = lane < (kGlu ? 2 * half : half);
+  const int gate_at = half * 144;
+  const uint8_t* my_block = ring + lane * 144;
+  const uint8_t* my_records = lds + sb * kRecord;
 
   // A routed product's workgroup first learns whether it owns its expert.
   int expert = blockIdx.y;
@@ -296,73 +341,83 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
   for (int p0 = 0; p0 < n; p0 += P) {
     const int m = min(P, n - p0);
     if (p0 > 0) __syncthreads();  // the last pass's readers of the records
-    // The wave's first tile leaves before the activations are staged.
-    int index = first_tile;
-    Tile tile{};
-    if (index < tiles) {
-      tile = TileOf<kGlu>(index, rows_per_tile, d.nrows, nsb);
-      FetchTile<kGlu, kPacked>(d, expert_block, tile, nsb, ring, lane);
+    // The activations' first loads, then the wave's first tile, then the staging.
+    const void* rows_x[P];
+    FrontX front_x[XT < 0 ? 1 : P];
+    FrontQ8 front_q[XT < 0 ? P : 1];
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      if (j < m) {
+        const int pr = pairs[p0 + j];
+        const int token = pr >> 8;
+        const int slot = pr & 0xFF;
+        if constexpr (XT < 0) {
+          rows_x[j] = static_cast<const uint8_t*>(d.y) +
+                      (static_cast<int64_t>(token) * d.y_token + static_cast<int64_t>(slot) * d.y_slot) * kQ8Block;
+          front_q[j] = LoadFrontQ8(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32);
+        } else {
+          const int64_t at = token * a.x_token + slot * a.x_slot;
+          rows_x[j] = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
+                                       : static_cast<const void*>(static_cast<const uint16_t*>(a.x) + at);
+          front_x[j] = LoadFrontX<XT>(rows_x[j], d.ncols_x);
+        }
+      }
     }
-    for (int j = 0; j < m; ++j) {
-      const int pr = pairs[p0 + j];
-      const int token = pr >> 8;
-      const int slot = pr & 0xFF;
-      uint8_t* records = lds + j * token_stride;
-      if constexpr (XT < 0) {
-        const uint8_t* y = static_cast<const uint8_t*>(d.y) +
-                           (static_cast<int64_t>(token) * d.y_token + static_cast<int64_t>(slot) * d.y_slot) * kQ8Block;
-        StageRecordsQ8(y, d.ncols_x / 32, records);
-      } else {
-        const int64_t at = token * a.x_token + slot * a.x_slot;
-        const void* x = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
-                                         : static_cast<const void*>(static_cast<const uint16_t*>(a.x) + at);
-        StageRecordsX<XT>(x, d.ncols_x, records);
+    int index = first_tile;
+    if (index < tiles) {
+      const int row0 = index * rows_per_tile;
+      FetchTile<kGlu, kPacked>(d, expert_block, row0, min(rows_per_tile, d.nrows - row0), nsb, gate_at, ring, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < P; ++j) {
+      if (j < m) {
+        uint8_t* records = lds + j * token_stride;
+        if constexpr (XT < 0) {
+          StageRecordsQ8(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_q[j], records);
+        } else {
+          StageRecordsX<XT>(rows_x[j], d.ncols_x, front_x[j], records);
+        }
       }
     }
     __syncthreads();  // the records are staged; from here the waves run alone
 
     while (index < tiles) {
+      const int row0 = index * rows_per_tile;
+      const bool live = placed && row0 + row < d.nrows;
       AwaitTile();
       float out[P];
-      if (lane < tile.total) {
-        const int f = (kGlu && lane >= tile.half) ? lane - tile.half : lane;
-        const int row = f / nsb;
-        const int sb = f - row * nsb;
-        const SuperBlock block = ReadSuperBlock(ring, lane);
-        int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(tile.row0 + row) * nsb + sb) * 16 : nullptr;
-        DotSuperBlock<P, kDump>(block, lds + sb * kRecord, token_stride, m, out, dump);
+      if (live) {
+        const SuperBlock block = ReadSuperBlock(my_block);
+        int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * 16 : nullptr;
+        DotSuperBlock<P, kDump>(block, my_records, token_stride, m, out, dump);
       }
-      // Every lane's reads of the buffer precede these writes in the wave's LDS order.
-      if (lane < tile.total) {
+      // Row sums: a suffix sum over each row's lanes (a fixed tree), the total in the row's
+      // first lane; a gate row's total then moves to its up row's lane.
 #pragma unroll
-        for (int t = 0; t < P; ++t) {
-          if (t < m) partial[t * kWave + lane] = out[t];
+      for (int t = 0; t < P; ++t) {
+        if (t < m) {
+          float v = live ? out[t] : 0.0f;
+          for (int off = 1; off < nsb; off <<= 1) {
+            const float other = __shfl_down(v, off, kWave);
+            if (sb + off < nsb) v += other;
+          }
+          float gate = 0.0f;
+          if constexpr (kGlu) gate = __shfl_down(v, half, kWave);
+          if (live && !gate_lane && sb == 0) {
+            const int pr = pairs[p0 + t];
+            float* dst =
+                d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
+            dst[row0 + row] = kGlu ? Glu(d.glu, gate, v, d.limit) : v;
+          }
         }
       }
-      __builtin_amdgcn_wave_barrier();
-      asm volatile("" ::: "memory");
-      // One lane a (token, row): the row's super-block sums added in order.
-      const int rows = tile.half / nsb;
-      for (int item = lane; item < m * rows; item += kWave) {
-        const int t = item / rows;
-        const int r = item - t * rows;
-        const float* pu = partial + t * kWave + r * nsb;
-        float su = 0.0f, sg = 0.0f;
-        for (int s = 0; s < nsb; ++s) {
-          su += pu[s];
-          if constexpr (kGlu) sg += pu[tile.half + s];
-        }
-        const int pr = pairs[p0 + t];
-        float* dst =
-            d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
-        dst[tile.row0 + r] = kGlu ? Glu(d.glu, sg, su, d.limit) : su;
-      }
-      __builtin_amdgcn_wave_barrier();
-      asm volatile("" ::: "memory");
+      // The next tile may overwrite the buffer: every lane's reads of it were consumed above.
+      // (Queueing these loads before the row sums measured slower.)
       index += tile_step;
       if (index < tiles) {
-        tile = TileOf<kGlu>(index, rows_per_tile, d.nrows, nsb);
-        FetchTile<kGlu, kPacked>(d, expert_block, tile, nsb, ring, lane);
+        const int next0 = index * rows_per_tile;
+        FetchTile<kGlu, kPacked>(d, expert_block, next0, min(rows_per_tile, d.nrows - next0), nsb, gate_at, ring,
+                                 lane);
       }
     }
   }
