@@ -107,6 +107,48 @@ int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp_vecq_sourc
 int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums,
                              void* stream);
 
+/* llmp.vecq over rows sorted by expert (the grouped form of a routed product with more
+ * than 128 (token, slot) pairs; src/kernels/decode/products.h:151-169 and
+ * src/kernels/ggml/moe_cutlass.h:12-27 describe the reference's operand layout): expert e
+ * computes rows offsets[e] .. offsets[e + 1] of the Q8_1 activations d->y (y_token blocks a
+ * row) into the same rows of d->dst (dst_token floats a row) with matrix e of d->w / d->g.
+ * d->ids, used, tokens and the slot strides are ignored. Q4_K only. */
+int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int32_t* offsets, int experts,
+                         int variant, void* stream);
+
+/* ------------------------------------------------------------------ routed experts
+ * llmp.moe.router (src/kernels/ggml/llmp_fused.cu:1307-1407; the definition is kRoute with
+ * kSoftmaxTopK, src/kernels/reference/exec.cc:1728-1818): per token the softmax of its
+ * `experts` logits, the `used` most probable experts (the lower index first among equals; a
+ * row holding a NaN or no finite value picks experts 0 .. used - 1 with zero weights), and
+ * their probabilities, over max(their sum, 2^-14) when `normalize`, times `scale`.
+ * logits [tokens][experts] -> ids, weights [tokens][used]. used <= 64, experts <= 1024. */
+int llmp_hip_moe_router(const float* logits, int experts, int used, int tokens, int normalize,
+                        float scale, int32_t* ids, float* weights, void* stream);
+
+/* llmp.moe.route (src/kernels/ggml/llmp_moe.cu:81-163): ids [tokens][used] (ids_stride
+ * apart) into the route buffer of src/kernels/ggml/moe_layout.h:46-70, int32, in this order:
+ * offsets[experts + 1], scale_rows[experts + 1], position[slots], token[slots],
+ * expert[slots], counts[chunks * experts] (work space; chunks = ceil(tokens / 64)). Rows are
+ * sorted by expert, token order within an expert; an id outside the experts has position -1. */
+int64_t llmp_hip_moe_route_ints(int experts, int used, int tokens);
+int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int experts, int used, int tokens,
+                       int32_t* route, void* stream);
+
+/* llmp.q8_1 with a gather, quantize_row_q8_1_cuda's `ids` argument
+ * (third_party/patches/ggml/0010-llmp-q8-dispatch-descriptors.patch:604-611): output row r
+ * is the Q8_1 of input row rows[r] (row r when rows is null), row_stride floats apart. */
+int llmp_hip_q8_1_quantize_rows(const float* x, const int32_t* rows, void* out, int64_t k,
+                                int64_t padded_k, int64_t row_stride, int64_t count, void* stream);
+
+/* The routed rows' weighted sum (kExpertReduce, src/kernels/reference/exec.cc:1819-1856;
+ * src/kernels/ggml/llmp_fused.cu:200-240 and llmp_moe.cu:390-427 for sorted rows):
+ * out[t][:] = sum_j x[row(t, j)][:] * weights[t][j] in slot order, the first term assigned,
+ * where row(t, j) is t * used + j, or position[t * used + j] when position is given (a
+ * negative position adds nothing). width a multiple of 4. */
+int llmp_hip_moe_combine(const float* x, const float* weights, const int32_t* position, int width,
+                         int used, int tokens, float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,12 @@ SYMBOLS = {
     "llmp_hip_vecq_variant_name": (C.c_char_p, [_int]),
     "llmp_hip_vecq_fused": (_int, [_int, C.POINTER(VecQDesc), C.POINTER(VecQSource), _int, _vp]),
     "llmp_hip_vecq_block_sums": (_int, [_int, C.POINTER(VecQDesc), _int, _vp, _vp]),
+    "llmp_hip_vecq_sorted": (_int, [_int, C.POINTER(VecQDesc), _vp, _int, _int, _vp]),
+    "llmp_hip_moe_router": (_int, [_vp, _int, _int, _int, _int, C.c_float, _vp, _vp, _vp]),
+    "llmp_hip_moe_route_ints": (_i64, [_int, _int, _int]),
+    "llmp_hip_moe_route": (_int, [_vp, _int, _int, _int, _int, _vp, _vp]),
+    "llmp_hip_q8_1_quantize_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
 }
 
 _lib = None

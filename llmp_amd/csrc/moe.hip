@@ -1,0 +1,325 @@
+// The routed-expert operations around llmp.vecq for gfx950: the router (softmax, top-k,
+// renormalized weights), the expert grouping of (token, slot) pairs, the gathering Q8_1
+// quantizer of the sorted rows, and the ordered weighted combine. All deterministic: fixed
+// summation orders, no atomics on results.
+//
+// Reference behaviour restated here: src/kernels/reference/exec.cc:279-315,1728-1856
+// (route and reduce definitions), src/kernels/ggml/llmp_fused.cu:1307-1407 (router kernel),
+// :200-240 (combine), src/kernels/ggml/llmp_moe.cu:81-163 (grouping), :390-427 (sorted
+// combine), src/kernels/ggml/moe_layout.h:46-70 (the route buffer).
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+#include "vecq_common.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr int kRouterWaves = 4;
+constexpr int kRouterSlots = 16;  // experts / 64 at most: up to 1024 experts
+constexpr int kRouteChunk = 64;   // tokens a counting workgroup (moe_layout.h kRouteChunk)
+constexpr int kScaleRows = 128;   // moe_layout.h kScaleRows
+
+__device__ __forceinline__ float WaveSum(float v) {
+#pragma unroll
+  for (int mask = 32; mask >= 1; mask >>= 1) v += ShflXor(v, mask);
+  return v;
+}
+
+// A token a wave: expert lane + 64 i sits in lane `lane`'s slot i.
+__global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float* __restrict__ logits,
+                                                                   int32_t* __restrict__ ids,
+                                                                   float* __restrict__ weights, int tokens, int experts,
+                                                                   int used, int normalize, float scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kRouterWaves + threadIdx.x / kWave;
+  if (t >= tokens) return;  // whole waves
+  const float* l = logits + t * experts;
+  const int slots = (experts + kWave - 1) / kWave;
+  float v[kRouterSlots];
+  float p[kRouterSlots];
+  float most = -INFINITY;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < kRouterSlots; ++i) {
+    const int e = i * kWave + lane;
+    const bool have = i < slots && e < experts;
+    v[i] = have ? l[e] : -INFINITY;
+    nan = nan || (have && v[i] != v[i]);
+    most = fmaxf(most, v[i]);  // ignores NaN, as std::max(max, v) does
+  }
+#pragma unroll
+  for (int mask = 32; mask >= 1; mask >>= 1) most = fmaxf(most, ShflXor(most, mask));
+  nan = __any(nan);
+  // A row with a NaN or no finite maximum has no probabilities: every expert 0, so the first
+  // `used` experts with zero weights (exec.cc:279-299 and the stable order of :303-315).
+  const bool degenerate = nan || !(fabsf(most) < INFINITY);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kRouterSlots; ++i) {
+    const int e = i * kWave + lane;
+    const bool have = i < slots && e < experts;
+    p[i] = have && !degenerate ? expf(v[i] - most) : 0.0f;
+    sum += p[i];
+  }
+  const float total = WaveSum(sum);
+  const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+  // Top `used` by logit (the probabilities' order without their rounding), lower index first
+  // among equals; a degenerate row orders by index alone.
+  float mine = 0.0f;
+  float picked = 0.0f;
+  int my_index = 0;
+  for (int j = 0; j < used; ++j) {
+    float best = -INFINITY;
+    int index = 0x7FFFFFFF;
+    float best_p = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kRouterSlots; ++i) {
+      const int e = i * kWave + lane;
+      const bool have = i < slots && e < experts && p[i] >= 0.0f;  // a pick is marked by -1
+      const float key = degenerate ? 0.0f : v[i];
+      if (have && (index == 0x7FFFFFFF || key > best)) {
+        best = key;
+        index = e;
+        best_p = p[i];
+      }
+    }
+#pragma unroll
+    for (int mask = 32; mask >= 1; mask >>= 1) {
+      const float b = ShflXor(best, mask);
+      const int bi = ShflXor(index, mask);
+      const float bp = ShflXor(best_p, mask);
+      const bool take = bi != 0x7FFFFFFF && (index == 0x7FFFFFFF || b > best || (b == best && bi < index));
+      if (take) {
+        best = b;
+        index = bi;
+        best_p = bp;
+      }
+    }
+    if (index != 0x7FFFFFFF && (index & (kWave - 1)) == lane) {
+#pragma unroll
+      for (int i = 0; i < kRouterSlots; ++i) {
+        if (i == index / kWave) p[i] = -1.0f;
+      }
+    }
+    const float q = best_p * inverse;
+    if (lane == j) {
+      mine = q;
+      my_index = index;
+    }
+    picked += q;  // in pick order
+  }
+  if (lane < used) {
+    ids[t * used + lane] = my_index;
+    const float denominator = normalize ? fmaxf(picked, 6.103515625e-5f) : 1.0f;  // 2^-14
+    weights[t * used + lane] = mine / denominator * scale;
+  }
+}
+
+// ---------------------------------------------------------------- grouping
+
+struct Route {
+  int32_t* offsets;
+  int32_t* scale_rows;
+  int32_t* position;
+  int32_t* token;
+  int32_t* expert;
+  int32_t* counts;
+  int experts, used, tokens, chunks;
+};
+
+// Each workgroup counts its chunk's ids per expert: one thread an expert, the chunk's slots
+// in order (no atomics: a thread owns its counter).
+__global__ void RouteCount(const int32_t* __restrict__ ids, int ids_stride, Route r) {
+  const int c = blockIdx.x;
+  const int t0 = c * kRouteChunk;
+  const int t1 = min(t0 + kRouteChunk, r.tokens);
+  for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
+    int n = 0;
+    for (int t = t0; t < t1; ++t)
+      for (int j = 0; j < r.used; ++j) n += ids[static_cast<int64_t>(t) * ids_stride + j] == e;
+    r.counts[static_cast<int64_t>(c) * r.experts + e] = n;
+  }
+}
+
+// One workgroup: each expert's chunk counts become the chunks' bases, then the experts'
+// offsets and scale rows.
+__global__ void RouteScan(Route r) {
+  extern __shared__ int total[];
+  for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
+    int running = 0;
+    for (int c = 0; c < r.chunks; ++c) {
+      int32_t* at = r.counts + static_cast<int64_t>(c) * r.experts + e;
+      const int v = *at;
+      *at = running;
+      running += v;
+    }
+    total[e] = running;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    r.offsets[0] = 0;
+    r.scale_rows[0] = 0;
+    for (int e = 0; e < r.experts; ++e) {
+      r.offsets[e + 1] = r.offsets[e] + total[e];
+      r.scale_rows[e + 1] = r.scale_rows[e] + (total[e] + kScaleRows - 1) / kScaleRows * kScaleRows;
+    }
+  }
+}
+
+// Each workgroup places its chunk's slots: one thread an expert, its rows in token order.
+__global__ void RouteAssign(const int32_t* __restrict__ ids, int ids_stride, Route r) {
+  const int c = blockIdx.x;
+  const int t0 = c * kRouteChunk;
+  const int t1 = min(t0 + kRouteChunk, r.tokens);
+  for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
+    int row = r.offsets[e] + r.counts[static_cast<int64_t>(c) * r.experts + e];
+    for (int t = t0; t < t1; ++t)
+      for (int j = 0; j < r.used; ++j) {
+        if (ids[static_cast<int64_t>(t) * ids_stride + j] != e) continue;
+        r.position[t * r.used + j] = row;
+        r.token[row] = t;
+        r.expert[row] = e;
+        ++row;
+      }
+  }
+  // Ids outside the experts have no row.
+  for (int i = threadIdx.x; i < (t1 - t0) * r.used; i += blockDim.x) {
+    const int t = t0 + i / r.used;
+    const int j = i % r.used;
+    const int e = ids[static_cast<int64_t>(t) * ids_stride + j];
+    if (e < 0 || e >= r.experts) r.position[t * r.used + j] = -1;
+  }
+}
+
+// ------------------------------------------------------- gathering quantizer
+
+// Output row r is the Q8_1 of input row rows[r] (or r): eight lanes a block.
+__global__ __launch_bounds__(kThreads) void QuantizeGatherKernel(const float* __restrict__ x,
+                                                                const int32_t* __restrict__ rows,
+                                                                uint8_t* __restrict__ out, int64_t k, int64_t padded_k,
+                                                                int64_t row_stride) {
+  const int lane8 = threadIdx.x & 7;
+  const int64_t block = static_cast<int64_t>(blockIdx.x) * 32 + (threadIdx.x >> 3);
+  const int64_t blocks = padded_k / 32;
+  if (block >= blocks) return;  // whole 8-lane groups
+  const int64_t r = blockIdx.y;
+  const int64_t source = rows != nullptr ? rows[r] : r;
+  float v[4];
+  Load4<LLMP_X_F32>(x + source * row_stride, block * 32 + lane8 * 4, k, v);
+  const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+  uint8_t* dst = out + (r * blocks + block) * kQ8Block;
+  *reinterpret_cast<uint32_t*>(dst + 4 + lane8 * 4) = q.codes;
+  if (lane8 == 0) *reinterpret_cast<uint32_t*>(dst) = FloatToHalfBits(q.d) | (FloatToHalfBits(q.sum) << 16);
+}
+
+// ------------------------------------------------------------------ combine
+
+// out[t] = sum_j x[row(t, j)] * w[t, j] in slot order, the first term assigned: four columns
+// a thread. row(t, j) is t * used + j, or position[t * used + j] for sorted rows (a negative
+// position contributes nothing).
+__global__ void CombineKernel(const float4* __restrict__ x, const float* __restrict__ weights,
+                              const int32_t* __restrict__ position, float4* __restrict__ out, int width4, int used,
+                              int64_t total4) {
+#pragma clang fp contract(off)
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const int64_t t = i / width4;
+  const int64_t c4 = i % width4;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  bool first = true;
+  for (int j = 0; j < used; ++j) {
+    int64_t row = t * used + j;
+    if (position != nullptr) {
+      row = position[row];
+      if (row < 0) continue;
+    }
+    const float w = weights[t * used + j];
+    const float4 d = x[row * width4 + c4];
+    const float4 e = make_float4(d.x * w, d.y * w, d.z * w, d.w * w);
+    acc = first ? e : make_float4(acc.x + e.x, acc.y + e.y, acc.z + e.z, acc.w + e.w);
+    first = false;
+  }
+  out[i] = acc;
+}
+
+Route RouteOf(int32_t* base, int experts, int used, int tokens) {
+  const int64_t slots = static_cast<int64_t>(used) * tokens;
+  const int chunks = (tokens + kRouteChunk - 1) / kRouteChunk;
+  Route r;
+  r.offsets = base;
+  r.scale_rows = base + experts + 1;
+  r.position = base + 2 * (experts + 1);
+  r.token = r.position + slots;
+  r.expert = r.token + slots;
+  r.counts = r.expert + slots;
+  r.experts = experts;
+  r.used = used;
+  r.tokens = tokens;
+  r.chunks = chunks;
+  return r;
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_moe_router(const float* logits, int experts, int used, int tokens, int normalize, float scale,
+                                   int32_t* ids, float* weights, void* stream) {
+  if (logits == nullptr || ids == nullptr || weights == nullptr) return Refuse(1, "moe.router: null operand");
+  if (experts < 1 || experts > kRouterSlots * kWave) return Refuse(1, "moe.router: 1 to %d experts", kRouterSlots * kWave);
+  if (used < 1 || used > experts || used > kWave) return Refuse(1, "moe.router: 1 to min(experts, 64) picks, not %d", used);
+  if (tokens < 1) return Refuse(1, "moe.router: no tokens");
+  const dim3 grid(static_cast<unsigned>((tokens + kRouterWaves - 1) / kRouterWaves));
+  hipLaunchKernelGGL(RouterKernel, grid, dim3(kRouterWaves * kWave), 0, static_cast<hipStream_t>(stream), logits, ids,
+                     weights, tokens, experts, used, normalize, scale);
+  return LaunchStatus("moe.router");
+}
+
+extern "C" int64_t llmp_hip_moe_route_ints(int experts, int used, int tokens) {
+  const int64_t slots = static_cast<int64_t>(used) * tokens;
+  const int64_t chunks = (tokens + kRouteChunk - 1) / kRouteChunk;
+  return 2 * (static_cast<int64_t>(experts) + 1) + 3 * slots + chunks * experts;
+}
+
+extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int experts, int used, int tokens,
+                                  int32_t* route, void* stream) {
+  if (ids == nullptr || route == nullptr) return Refuse(1, "moe.route: null operand");
+  if (experts < 1 || used < 1 || tokens < 1 || ids_stride < used) return Refuse(1, "moe.route: empty or overlapping ids");
+  if (static_cast<int64_t>(used) * tokens > (1 << 24)) return Refuse(1, "moe.route: more than 2^24 slots");
+  const Route r = RouteOf(route, experts, used, tokens);
+  const auto s = static_cast<hipStream_t>(stream);
+  const int threads = experts < 256 ? (experts + 63) / 64 * 64 : 256;
+  hipLaunchKernelGGL(RouteCount, dim3(r.chunks), dim3(threads), 0, s, ids, ids_stride, r);
+  if (const int bad = LaunchStatus("moe.route count"); bad != 0) return bad;
+  hipLaunchKernelGGL(RouteScan, dim3(1), dim3(threads), static_cast<size_t>(experts) * sizeof(int), s, r);
+  hipLaunchKernelGGL(RouteAssign, dim3(r.chunks), dim3(threads), 0, s, ids, ids_stride, r);
+  return LaunchStatus("moe.route");
+}
+
+extern "C" int llmp_hip_q8_1_quantize_rows(const float* x, const int32_t* rows, void* out, int64_t k, int64_t padded_k,
+                                           int64_t row_stride, int64_t count, void* stream) {
+  if (x == nullptr || out == nullptr) return Refuse(1, "q8_1: null operand");
+  if (k <= 0 || count <= 0 || count > 65535) return Refuse(1, "q8_1: 1 to 65535 rows");
+  if (padded_k < k || padded_k % 32 != 0) return Refuse(1, "q8_1: padded k below k or not whole blocks");
+  const dim3 grid(static_cast<unsigned>((padded_k / 32 + 31) / 32), static_cast<unsigned>(count));
+  hipLaunchKernelGGL(QuantizeGatherKernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), x, rows,
+                     static_cast<uint8_t*>(out), k, padded_k, row_stride);
+  return LaunchStatus("q8_1 rows");
+}
+
+extern "C" int llmp_hip_moe_combine(const float* x, const float* weights, const int32_t* position, int width, int used,
+                                    int tokens, float* out, void* stream) {
+  if (x == nullptr || weights == nullptr || out == nullptr) return Refuse(1, "moe.combine: null operand");
+  if (width < 4 || width % 4 != 0 || used < 1 || tokens < 1) return Refuse(1, "moe.combine: width a multiple of 4");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)
+    return Refuse(1, "moe.combine: operands not 16-byte aligned");
+  const int64_t total4 = static_cast<int64_t>(tokens) * (width / 4);
+  hipLaunchKernelGGL(CombineKernel, dim3(static_cast<unsigned>((total4 + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), reinterpret_cast<const float4*>(x), weights, position,
+                     reinterpret_cast<float4*>(out), width / 4, used, total4);
+  return LaunchStatus("moe.combine");
+}

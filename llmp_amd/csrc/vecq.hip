@@ -568,7 +568,7 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp) {
   }
 }
 
-int CheckDesc(int type, const llmp_vecq_desc* d) {
+int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K) return Refuse(1, "vecq: weight type %d has no kernel", type);
   const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
@@ -576,7 +576,8 @@ int CheckDesc(int type, const llmp_vecq_desc* d) {
   if (d->ncols_x <= 0 || d->ncols_x % qk != 0) return Refuse(1, "vecq: k %d is not whole %d-value blocks", d->ncols_x, qk);
   if (d->nrows <= 0) return Refuse(1, "vecq: no rows");
   if (d->tokens < 1 || d->tokens > 16) return Refuse(1, "vecq: 1 to 16 tokens, not %d", d->tokens);
-  if (d->used < 1 || d->used > 256) return Refuse(1, "vecq: 1 to 256 slots, not %d", d->used);
+  // A pair packs its slot in 8 bits; sorted rows have no pairs.
+  if (d->used < 1 || (!sorted && d->used > 256)) return Refuse(1, "vecq: 1 to 256 slots, not %d", d->used);
   if (d->ids != nullptr && d->used * d->tokens > kMaxPairs)
     return Refuse(1, "vecq: %d routed pairs exceed %d", d->used * d->tokens, kMaxPairs);
   if ((d->glu != LLMP_GLU_NONE) != (d->g != nullptr)) return Refuse(1, "vecq: gate weights exactly with a GLU");
@@ -590,8 +591,9 @@ int CheckDesc(int type, const llmp_vecq_desc* d) {
   return 0;
 }
 
-int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant, int32_t* dump, void* stream) {
-  if (const int bad = CheckDesc(type, d); bad != 0) return bad;
+int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant, int32_t* dump, void* stream,
+           const int32_t* offsets = nullptr) {
+  if (const int bad = CheckDesc(type, d, offsets != nullptr); bad != 0) return bad;
   int x_type = -1;
   VecQArgs a{};
   a.d = *d;
@@ -607,9 +609,11 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   }
   a.kp = PaddedK(d->ncols_x);
   a.dump = dump;
+  a.offsets = offsets;
   if (variant < 0) variant = DefaultVariant(type, *d, a.kp);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
+  if (offsets != nullptr && v.lanes != 0) return Refuse(1, "vecq: sorted rows take the flat Q4_K form");
   if (v.lanes == 0) {
     if (type != LLMP_TYPE_Q4_K || !FlatQ4KTakes(*d)) return Refuse(1, "vecq: the flat form takes Q4_K rows up to 65536 values");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
@@ -676,6 +680,21 @@ extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int v
   if (variant < 0 && d != nullptr) variant = type == LLMP_TYPE_Q4_K && FlatQ4KTakes(*d) ? kFlatFirst : 0;
   if (variant != 0 && variant != kFlatFirst) return Refuse(1, "vecq: block sums are of the one-token variants");
   return Launch(type, d, nullptr, variant, sums, stream);
+}
+
+extern "C" int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int32_t* offsets, int experts, int variant,
+                                    void* stream) {
+  if (offsets == nullptr || d == nullptr) return Refuse(1, "vecq: null offsets");
+  if (experts < 1 || experts > 65535) return Refuse(1, "vecq: 1 to 65535 experts");
+  if (type != LLMP_TYPE_Q4_K || !FlatQ4KTakes(*d)) return Refuse(1, "vecq: sorted rows take Q4_K weights the flat form takes");
+  llmp_vecq_desc sorted = *d;
+  sorted.ids = nullptr;
+  sorted.used = experts;  // a workgroup row an expert
+  sorted.tokens = 1;      // the row counts come from the offsets
+  sorted.y_slot = 0;
+  sorted.dst_slot = 0;
+  if (variant < 0) variant = kFlatFirst + 1;
+  return Launch(type, &sorted, nullptr, variant, nullptr, stream, offsets);
 }
 
 extern "C" int llmp_hip_vecq_variants(void) { return kVariantCount; }

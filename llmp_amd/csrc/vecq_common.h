@@ -108,6 +108,9 @@ struct VecQArgs {
   int64_t x_slot;
   int kp;         // k rounded up to 512: the staged codes' stride
   int32_t* dump;  // block sums, or null
+  // Sorted rows: expert e computes rows offsets[e] .. offsets[e + 1] of the activations into
+  // the same rows of the output (d.ids unused), or null.
+  const int32_t* offsets;
 };
 
 __device__ __forceinline__ float Silu(float x) {

@@ -326,16 +326,23 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
   const uint8_t* my_block = ring + lane * 144;
   const uint8_t* my_records = lds + sb * kRecord;
 
-  // A routed product's workgroup first learns whether it owns its expert.
+  // A routed product's workgroup first learns whether it owns its expert; one over sorted
+  // rows takes its expert's row range.
   int expert = blockIdx.y;
-  if (d.ids != nullptr) {
+  int sorted_first = 0;
+  if (a.offsets != nullptr) {
+    sorted_first = a.offsets[expert];
+    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+    __syncthreads();
+    if (count == 0) return;  // uniform over the workgroup
+  } else if (d.ids != nullptr) {
     expert = ResolvePairs(d, blockIdx.y, pairs, &count);
     if (count == 0) return;  // uniform over the workgroup
   }
   const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
   const int first_tile = blockIdx.x * kWaves + wave;
   const int tile_step = gridDim.x * kWaves;
-  if (d.ids == nullptr) ResolvePairs(d, blockIdx.y, pairs, &count);
+  if (a.offsets == nullptr && d.ids == nullptr) ResolvePairs(d, blockIdx.y, pairs, &count);
   const int n = count;
 
   for (int p0 = 0; p0 < n; p0 += P) {
@@ -348,7 +355,7 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
-        const int pr = pairs[p0 + j];
+        const int pr = a.offsets != nullptr ? (sorted_first + p0 + j) << 8 : pairs[p0 + j];
         const int token = pr >> 8;
         const int slot = pr & 0xFF;
         if constexpr (XT < 0) {
@@ -404,7 +411,7 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
           float gate = 0.0f;
           if constexpr (kGlu) gate = __shfl_down(v, half, kWave);
           if (live && !gate_lane && sb == 0) {
-            const int pr = pairs[p0 + t];
+            const int pr = a.offsets != nullptr ? (sorted_first + p0 + t) << 8 : pairs[p0 + t];
             float* dst =
                 d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
             dst[row0 + row] = kGlu ? Glu(d.glu, gate, v, d.limit) : v;
@@ -499,10 +506,10 @@ void LaunchFlatQ4K(const VecQArgs& a, int x_type, int pass, hipStream_t stream) 
     const int units = llmp_hip_compute_units();
     g_compute_units = units > 0 ? units : 256;
   }
-  const int slots = d.ids != nullptr ? d.used * d.tokens : d.used;
+  const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
   // What is resident at once: two workgroups a CU, shared by the slots that have work.
-  const int live_slots = d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
+  const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
   int groups = 2 * g_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
   if (groups > (tiles + kWaves - 1) / kWaves) groups = (tiles + kWaves - 1) / kWaves;

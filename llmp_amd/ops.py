@@ -110,3 +110,107 @@ def vecq_block_sums(t, w, q8, k, nrows, variant=-1):
 def vecq_variants():
     lib = _lib.load()
     return [lib.llmp_hip_vecq_variant_name(i).decode() for i in range(lib.llmp_hip_vecq_variants())]
+
+
+def vecq_sorted(t, w, q8, offsets, k, nrows, experts, *, gate=None, stride_row=None, stride_expert=0,
+                glu=GLU_NONE, limit=0.0, variant=-1, out=None):
+    """llmp.vecq over rows sorted by expert: q8 [rows, blocks*36] -> float32 [rows, nrows]."""
+    lib = _lib.load()
+    rows = q8.shape[0]
+    if out is None:
+        out = torch.empty((rows, nrows), dtype=torch.float32, device=w.device)
+    d = _desc(t, w, k, nrows, gate=gate, q8=q8, ids=None, tokens=1, used=1, stride_row=stride_row,
+              stride_expert=stride_expert, y_token=None, y_slot=0, glu=glu, limit=limit, out=out)
+    d.dst_token = nrows
+    _lib.check(lib.llmp_hip_vecq_sorted(t, C.byref(d), _ptr(offsets), experts, variant, _stream()))
+    return out
+
+
+def moe_router(logits, used, normalize=True, scale=1.0):
+    """llmp.moe.router: float32 [tokens, experts] -> (ids int32 [tokens, used], weights float32)."""
+    lib = _lib.load()
+    tokens, experts = logits.shape
+    ids = torch.empty((tokens, used), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((tokens, used), dtype=torch.float32, device=logits.device)
+    _lib.check(lib.llmp_hip_moe_router(_ptr(logits), experts, used, tokens, int(normalize), scale, _ptr(ids),
+                                       _ptr(weights), _stream()))
+    return ids, weights
+
+
+class Route:
+    """Views of llmp.moe.route's buffer (src/kernels/ggml/moe_layout.h:46-70 of the reference)."""
+
+    def __init__(self, buffer, experts, slots):
+        self.buffer = buffer
+        self.offsets = buffer[:experts + 1]
+        self.scale_rows = buffer[experts + 1:2 * (experts + 1)]
+        at = 2 * (experts + 1)
+        self.position = buffer[at:at + slots]
+        self.token = buffer[at + slots:at + 2 * slots]
+        self.expert = buffer[at + 2 * slots:at + 3 * slots]
+
+
+def moe_route(ids, experts):
+    lib = _lib.load()
+    tokens, used = ids.shape
+    ints = lib.llmp_hip_moe_route_ints(experts, used, tokens)
+    buffer = torch.empty(ints, dtype=torch.int32, device=ids.device)
+    _lib.check(lib.llmp_hip_moe_route(_ptr(ids), ids.stride(0), experts, used, tokens, _ptr(buffer), _stream()))
+    return Route(buffer, experts, tokens * used)
+
+
+def quantize_q8_1_rows(x, rows=None, count=None):
+    """llmp.q8_1 with a gather: output row r is input row rows[r]."""
+    lib = _lib.load()
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1
+    k = x.shape[1]
+    count = (x.shape[0] if rows is None else rows.numel()) if count is None else count
+    pk = padded_k(k)
+    out = torch.empty((count, pk // 32 * 36), dtype=torch.uint8, device=x.device)
+    _lib.check(lib.llmp_hip_q8_1_quantize_rows(_ptr(x), _ptr(rows), _ptr(out), k, pk, x.stride(0), count, _stream()))
+    return out
+
+
+def moe_combine(x, weights, position=None):
+    """out[t] = sum_j x[row(t, j)] * weights[t, j] in slot order. x [rows, width]."""
+    lib = _lib.load()
+    tokens, used = weights.shape
+    width = x.shape[-1]
+    out = torch.empty((tokens, width), dtype=torch.float32, device=x.device)
+    _lib.check(lib.llmp_hip_moe_combine(_ptr(x), _ptr(weights), _ptr(position), width, used, tokens, _ptr(out),
+                                        _stream()))
+    return out
+
+
+def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWIGLU, keep=None):
+    """One routed-expert FFN layer (the decomposition of src/ir/decompose.cc:1080-1109 of the
+    reference): route, gate/up with a GLU, down, weighted combine. gate_up is uint8
+    [experts, 2 * ffn rows of hidden] (gate rows first), down uint8 [experts, hidden rows of ffn].
+    Up to 128 (token, slot) pairs go through the routed mat-vec; more are sorted by expert.
+    `keep`, a dict, receives the intermediates (h, hq, y and, when sorted, the route)."""
+    tokens = x.shape[0]
+    qk, bs = BLOCK_ELEMENTS[t], BLOCK_BYTES[t]
+    ids, weights = moe_router(logits, used)
+    gu_stride = 2 * ffn * (hidden // qk)
+    gate = gate_up
+    up = gate_up.view(-1)[ffn * (hidden // qk) * bs:]
+    down_stride = hidden * (ffn // qk)
+    if tokens * used <= 128:
+        q8 = quantize_q8_1(x)
+        h = vecq(t, up, q8, hidden, ffn, gate=gate, ids=ids, tokens=tokens, used=used, stride_expert=gu_stride,
+                 glu=glu)
+        hq = quantize_q8_1(h.view(tokens * used, ffn))
+        blocks = padded_k(ffn) // 32
+        y = vecq(t, down, hq, ffn, hidden, ids=ids, tokens=tokens, used=used, stride_expert=down_stride,
+                 y_token=blocks * used, y_slot=blocks)
+        if keep is not None:
+            keep.update(h=h, hq=hq, y=y)
+        return moe_combine(y.view(tokens * used, hidden), weights), ids, weights
+    route = moe_route(ids, experts)
+    q8 = quantize_q8_1_rows(x, route.token)
+    h = vecq_sorted(t, up, q8, route.offsets, hidden, ffn, experts, gate=gate, stride_expert=gu_stride, glu=glu)
+    hq = quantize_q8_1_rows(h)
+    y = vecq_sorted(t, down, hq, route.offsets, ffn, hidden, experts, stride_expert=down_stride)
+    if keep is not None:
+        keep.update(h=h, hq=hq, y=y, route=route)
+    return moe_combine(y, weights, route.position), ids, weights

@@ -1,0 +1,181 @@
+"""Parity of the routed-expert operations (HIP, through the C ABI) against the CPU oracle:
+router ids bit-exact and weights to 1e-5, grouping bit-exact, the combine bit-exact in its
+float order, and the whole routed FFN layer to 1e-3 (Qwen3-30B-A3B-like shapes)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import rel_close
+from llmp_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+Q4_K = ops.TYPE_Q4_K
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+@pytest.mark.parametrize("tokens,experts,used", [(1, 128, 8), (16, 128, 8), (512, 128, 8), (33, 60, 4), (7, 256, 1),
+                                                 (5, 8, 8)])
+def test_router_matches_oracle(device, tokens, experts, used):
+    logits = synth.rng(7 + tokens).standard_normal((tokens, experts), dtype=np.float32)
+    want_ids, want_w = oracle.route(logits, used)
+    ids, w = ops.moe_router(dev(logits, device), used)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=1e-5, atol=1e-9)
+    np.testing.assert_allclose(w.cpu().numpy().sum(axis=1), 1.0, rtol=1e-5)
+
+
+def test_router_ties_and_degenerate_rows(device):
+    """tests/unit/qwen38_fast_test.cc:975-1037 of the reference: ties go to the lower index;
+    rows of NaN or -inf pick experts 0 .. used - 1 with zero weights."""
+    experts, used = 128, 8
+    logits = np.zeros((6, experts), dtype=np.float32)
+    logits[0, [5, 9, 100]] = 2.0  # three tied leaders, then the zeros in index order
+    logits[1, :] = -np.inf
+    logits[2, 17] = np.nan
+    logits[3, :] = np.inf
+    logits[4, :] = -np.inf
+    logits[4, [3, 70]] = [1.0, 1.5]  # two finite experts: the rest by index with zero weight
+    logits[5] = np.linspace(-3, 3, experts, dtype=np.float32)
+    want_ids, want_w = oracle.route(logits, used)
+    ids, w = ops.moe_router(dev(logits, device), used)
+    ids, w = ids.cpu().numpy(), w.cpu().numpy()
+    assert np.array_equal(ids, want_ids)
+    assert list(ids[0][:3]) == [5, 9, 100] and list(ids[0][3:]) == [0, 1, 2, 3, 4]
+    for row in (1, 2, 3):
+        assert list(ids[row]) == list(range(used)) and np.all(w[row] == 0)
+    assert list(ids[4][:2]) == [70, 3]
+    np.testing.assert_allclose(w, want_w, rtol=1e-5, atol=1e-9)
+    ids2, w2 = ops.moe_router(dev(logits[5:6], device), used, normalize=False, scale=2.5)
+    _, want2 = oracle.route(logits[5:6], used, normalize=False, scale=2.5)
+    np.testing.assert_allclose(w2.cpu().numpy(), want2, rtol=1e-5)
+
+
+@pytest.mark.parametrize("tokens,experts,used", [(1, 128, 8), (16, 128, 8), (512, 128, 8), (130, 7, 3)])
+def test_route_groups_pairs_by_expert_in_token_order(device, tokens, experts, used):
+    g = synth.rng(11 + tokens)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    order, offsets = oracle.expert_sort(ids, experts)
+    route = ops.moe_route(dev(ids, device), experts)
+    assert np.array_equal(route.offsets.cpu().numpy(), offsets)
+    position = route.position.cpu().numpy()
+    # order[row] is the pair at that row: position is its inverse.
+    assert np.array_equal(position[order], np.arange(tokens * used))
+    assert np.array_equal(route.token.cpu().numpy(), order // used)
+    assert np.array_equal(route.expert.cpu().numpy(), ids.reshape(-1)[order])
+    counts = np.diff(offsets)
+    padded = np.concatenate([[0], np.cumsum((counts + 127) // 128 * 128)])
+    assert np.array_equal(route.scale_rows.cpu().numpy(), padded)
+
+
+def test_route_marks_ids_outside_the_experts(device):
+    ids = np.array([[0, 5], [9, 1], [-1, 0]], dtype=np.int32)
+    route = ops.moe_route(dev(ids, device), 4)
+    position = route.position.cpu().numpy()
+    assert position[1] == -1 and position[2] == -1 and position[4] == -1
+    assert np.array_equal(route.offsets.cpu().numpy(), [0, 2, 3, 3, 3])
+
+
+def test_combine_is_the_ordered_float_sum(device):
+    tokens, used, width = 9, 8, 2048
+    g = synth.rng(21)
+    x = g.standard_normal((tokens, used, width), dtype=np.float32)
+    w = g.random((tokens, used), dtype=np.float32)
+    want = oracle.expert_reduce(x, w)
+    got = ops.moe_combine(dev(x.reshape(-1, width), device), dev(w, device)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    closed = (x.astype(np.float64) * w[:, :, None]).sum(axis=1)
+    np.testing.assert_allclose(got, closed, rtol=1e-5, atol=1e-5)
+    # Sorted rows: the same sum through a permutation.
+    perm = g.permutation(tokens * used).astype(np.int32)
+    shuffled = np.zeros_like(x.reshape(-1, width))
+    shuffled[perm] = x.reshape(-1, width)
+    got2 = ops.moe_combine(dev(shuffled, device), dev(w, device), dev(perm, device)).cpu().numpy()
+    assert np.array_equal(got2.view(np.uint32), want.view(np.uint32))
+
+
+def test_gathering_quantizer_is_the_quantizer(device):
+    x = synth.activations(10, 768, 31)
+    rows = np.array([3, 3, 0, 9, 5], dtype=np.int32)
+    got = ops.quantize_q8_1_rows(dev(x, device), dev(rows, device)).cpu().numpy()
+    assert np.array_equal(got, oracle.q8_1_quantize(x[rows]))
+
+
+@pytest.mark.parametrize("tokens", [1, 16, 40])
+def test_routed_ffn_layer_matches_oracle_stage_by_stage(device, tokens):
+    """Qwen3-30B-A3B-like: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K. 40 tokens
+    take the sorted path (320 pairs), 1 and 16 the routed mat-vec. Every stage is compared with
+    the oracle over identical input bytes (the second product over the device's own quantized
+    h: a float rounding of h can move one of its Q8_1 codes by a step, which is a different
+    input, not an error of the product). exec.cc:966-1002,1819-1856 of the reference."""
+    t, hidden, ffn, experts, used = Q4_K, 2048, 768, 128, 8
+    qk, bs = 256, 144
+    gate_up = synth.q4_k_weights(experts * 2 * ffn, hidden, 41).reshape(experts, -1)
+    down = synth.q4_k_weights(experts * hidden, ffn, 42).reshape(experts, -1)
+    logits = synth.rng(43 + tokens).standard_normal((tokens, experts), dtype=np.float32)
+    x = synth.activations(tokens, hidden, 44)
+    keep = {}
+    got, ids, w = ops.moe_ffn(t, dev(logits, device), dev(x, device), dev(gate_up, device), dev(down, device), hidden,
+                              ffn, experts, used, keep=keep)
+    want_ids, want_w = oracle.route(logits, used)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    threads = oracle.max_threads()
+    up = gate_up.reshape(-1)[ffn * (hidden // qk) * bs:]
+    want_h = oracle.vecq(t, up, oracle.q8_1_quantize(x), hidden, ffn, gate=gate_up, ids=want_ids, tokens=tokens,
+                         used=used, stride_expert=2 * ffn * (hidden // qk), glu=oracle.GLU_SWIGLU, experts=experts,
+                         threads=threads).reshape(tokens * used, ffn)
+    h = keep["h"].cpu().numpy().reshape(-1, ffn)
+    hq = keep["hq"].cpu().numpy()
+    y = keep["y"].cpu().numpy().reshape(-1, hidden)
+    pairs = np.arange(tokens * used)
+    if "route" in keep:  # sorted rows: row r holds pair order[r]
+        order, _ = oracle.expert_sort(want_ids, experts)
+        assert np.array_equal(keep["route"].position.cpu().numpy()[order], pairs)
+        pairs = order
+    ok, worst = rel_close(h, want_h[pairs], 1e-3)
+    assert ok, worst
+    assert np.array_equal(hq, oracle.q8_1_quantize(h))
+    blocks = oracle.padded_k(ffn) // 32
+    unsorted_hq = np.zeros_like(hq)
+    unsorted_hq[pairs] = hq
+    want_y = oracle.vecq(t, down, unsorted_hq, ffn, hidden, ids=want_ids, tokens=tokens, used=used,
+                         stride_expert=hidden * (ffn // qk), y_token=blocks * used, y_slot=blocks, experts=experts,
+                         threads=threads).reshape(tokens * used, hidden)
+    ok, worst = rel_close(y, want_y[pairs], 1e-3)
+    assert ok, worst
+    unsorted_y = np.zeros_like(y)
+    unsorted_y[pairs] = y
+    want = oracle.expert_reduce(unsorted_y.reshape(tokens, used, hidden), w.cpu().numpy())
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # End to end against the all-CPU layer: the quantization steps bound it, not float order.
+    cpu_hq = oracle.q8_1_quantize(want_h)
+    cpu_y = oracle.vecq(t, down, cpu_hq, ffn, hidden, ids=want_ids, tokens=tokens, used=used,
+                        stride_expert=hidden * (ffn // qk), y_token=blocks * used, y_slot=blocks, experts=experts,
+                        threads=threads)
+    cpu = oracle.expert_reduce(cpu_y, want_w).astype(np.float64)
+    nmse = np.sum((got.cpu().numpy() - cpu) ** 2) / np.sum(cpu ** 2)
+    assert nmse <= 1e-6, nmse
+
+
+def test_sorted_rows_equal_the_routed_product(device):
+    """The sorted form computes each (token, slot) row with the routed form's arithmetic."""
+    t, hidden, ffn, experts, used, tokens = Q4_K, 1024, 256, 16, 4, 12
+    gate_up = synth.q4_k_weights(experts * 2 * ffn, hidden, 51).reshape(experts, -1)
+    g = synth.rng(52)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    x = synth.activations(tokens, hidden, 53)
+    gd = dev(gate_up, device)
+    up = gd.view(-1)[ffn * (hidden // 256) * 144:]
+    stride = 2 * ffn * (hidden // 256)
+    q8 = ops.quantize_q8_1(dev(x, device))
+    routed = ops.vecq(t, up, q8, hidden, ffn, gate=gd, ids=dev(ids, device), tokens=tokens, used=used,
+                      stride_expert=stride, glu=ops.GLU_SWIGLU).cpu().numpy().reshape(tokens * used, ffn)
+    route = ops.moe_route(dev(ids, device), experts)
+    sq8 = ops.quantize_q8_1_rows(dev(x, device), route.token)
+    sorted_rows = ops.vecq_sorted(t, up, sq8, route.offsets, hidden, ffn, experts, gate=gd, stride_expert=stride,
+                                  glu=ops.GLU_SWIGLU).cpu().numpy()
+    position = route.position.cpu().numpy()
+    assert np.array_equal(sorted_rows[position].view(np.uint32), routed.view(np.uint32))
