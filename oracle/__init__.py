@@ -175,6 +175,7 @@ def glu(kind, gate, up, limit=0.0):
 
 
 def mxfp8_scale_bytes(rows, k):
+    assert k % 128 == 0, "scale atoms hold four 32-value blocks: k must be a multiple of 128"
     return (rows + 127) // 128 * 128 * (k // 32)
 
 

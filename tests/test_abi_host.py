@@ -1,0 +1,87 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/llmp_hip.h declares,
+and its host-side checks refuse bad launches before anything is queued (no GPU call is reached:
+tests/unit/dsv4_fast_test.cc:391-399 of the reference checks the same on its device)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from llmp_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "llmp_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(llmp_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 10
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in _lib.SYMBOLS, f"{name} has no ctypes signature"
+    assert sorted(_lib.SYMBOLS) == names
+
+
+def test_variant_table_is_named():
+    lib = _lib.load()
+    n = lib.llmp_hip_vecq_variants()
+    assert n >= 4
+    names = [lib.llmp_hip_vecq_variant_name(i).decode() for i in range(n)]
+    assert len(set(names)) == n and lib.llmp_hip_vecq_variant_name(-1) == b"default"
+
+
+def desc(**kw):
+    d = _lib.VecQDesc()
+    base = dict(w=0x1000, g=None, y=0x2000, ids=None, dst=0x3000, ncols_x=512, nrows=8, stride_row=2, stride_expert=0,
+                y_token=16, y_slot=0, ids_stride=0, used=1, tokens=1, dst_token=8, dst_slot=0, glu=0, limit=0.0)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(d, k, v)
+    return d
+
+
+@pytest.mark.parametrize("t,kw,why", [
+    (12, dict(ncols_x=500), "whole"),
+    (12, dict(tokens=17), "tokens"),
+    (12, dict(tokens=0), "tokens"),
+    (12, dict(glu=3), "gate"),
+    (12, dict(g=0x4000, glu=0), "gate"),
+    (12, dict(g=0x4000, glu=3, limit=1.0), "GeGLU"),
+    (12, dict(ids=0x5000, used=16, tokens=16), "pairs"),
+    (12, dict(w=None), "null"),
+    (12, dict(w=0x1008), "aligned"),
+    (12, dict(dst=0x3002), "aligned"),
+    (12, dict(stride_row=1), "overlap"),
+    (8, dict(ncols_x=48), "whole"),
+    (8, dict(w=0x1001, stride_row=16), "aligned"),
+    (3, dict(), "type"),
+    (12, dict(used=300), "slots"),
+])
+def test_vecq_refusals_queue_nothing(t, kw, why):
+    lib = _lib.load()
+    code = lib.llmp_hip_vecq(t, C.byref(desc(**kw)), -1, None)
+    assert code > 0
+    assert why in lib.llmp_hip_last_error().decode()
+
+
+def test_other_entry_points_refuse_bad_operands():
+    lib = _lib.load()
+    assert lib.llmp_hip_vecq(12, None, -1, None) > 0
+    assert lib.llmp_hip_vecq(12, C.byref(desc()), 99, None) > 0
+    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=16)), 6, None) > 0  # the flat form is Q4_K's
+    assert lib.llmp_hip_vecq_fused(12, C.byref(desc()), None, -1, None) > 0
+    assert lib.llmp_hip_vecq_block_sums(12, C.byref(desc()), -1, None, None) > 0
+    assert lib.llmp_hip_q8_1_quantize(None, None, 32, 512, 32, 1, 1, 32, None) > 0
+    assert lib.llmp_hip_q8_1_quantize(0x1000, 0x2000, 600, 512, 600, 1, 1, 600, None) > 0
+    assert lib.llmp_hip_moe_router(0x1000, 2000, 8, 1, 1, 1.0, 0x2000, 0x3000, None) > 0
+    assert lib.llmp_hip_moe_router(0x1000, 128, 0, 1, 1, 1.0, 0x2000, 0x3000, None) > 0
+    assert lib.llmp_hip_moe_combine(0x1000, 0x2000, None, 6, 8, 1, 0x3000, None) > 0
+    assert lib.llmp_hip_moe_route(None, 8, 128, 8, 1, 0x1000, None) > 0
+    assert lib.llmp_hip_vecq_sorted(8, C.byref(desc(stride_row=16)), 0x1000, 4, -1, None) > 0
+    assert lib.llmp_hip_moe_route_ints(128, 8, 512) == 2 * 129 + 3 * 4096 + 8 * 128

@@ -1,0 +1,421 @@
+"""Pins of the CPU oracle: the reference's own golden vectors and independent derivations
+(numpy IEEE conversions, closed forms, brute force), so that a dropped term, a wrong index or
+a transposed operand in oracle/oracle.c fails here. No GPU."""
+import math
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import lib
+
+# ---------------------------------------------------------------- conversions
+
+
+def test_f16_decode_is_ieee_exhaustively():
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([lib.orc_f16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_f16_and_bf16_encode_round_to_nearest_even():
+    """tests/unit/reference_decode_test.cc:138-141 of the reference: its sample list, then
+    random bit patterns, against numpy's float16 and the bfloat16 closed form."""
+    samples = [0x00000000, 0x80000000, 0x7F800000, 0xFF800000, 0x477FE000, 0x477FEFFF, 0x477FF000, 0x38800000,
+               0x387FFFFF, 0x33000000, 0x33000001, 0x32FFFFFF, 0x337FFFFF, 0x00000001, 0x3F800000]
+    g = np.random.Generator(np.random.PCG64(3))
+    samples += [int(v) for v in g.integers(0, 2 ** 32, size=20000, dtype=np.uint64)]
+    u = np.array(samples, dtype=np.uint32)
+    f = u.view(np.float32)
+    keep = ~np.isnan(f)
+    with np.errstate(over="ignore"):
+        want16 = f.astype(np.float16).view(np.uint16)
+    for x, w16, ok in zip(f, want16, keep):
+        if not ok:
+            assert math.isnan(lib.orc_f16_to_f32(lib.orc_f32_to_f16(float(x))))
+            continue
+        assert lib.orc_f32_to_f16(float(x)) == int(w16), hex(np.float32(x).view(np.uint32))
+        xb = int(np.float32(x).view(np.uint32))
+        assert lib.orc_f32_to_bf16(float(x)) == ((xb + 0x7FFF + ((xb >> 16) & 1)) >> 16) & 0xFFFF
+    assert lib.orc_bf16_to_f32(0x3FC0) == 1.5
+
+
+def e4m3_closed_form(b):
+    """tests/unit/qwen38_ops_test.cc:101-110 of the reference."""
+    e, m = (b >> 3) & 15, b & 7
+    if e == 15 and m == 7:
+        return math.nan
+    v = m * 2.0 ** -9 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+    return -v if b & 0x80 else v
+
+
+def test_e4m3_and_e8m0_decode():
+    for b in range(256):
+        want = e4m3_closed_form(b)
+        got = lib.orc_e4m3_to_f32(b)
+        assert (math.isnan(got) and math.isnan(want)) or got == want
+        if b == 0xFF:
+            assert math.isnan(lib.orc_e8m0_to_f32(b))
+        else:
+            assert lib.orc_e8m0_to_f32(b) == math.ldexp(1.0, b - 127)
+    assert lib.orc_e4m3_to_f32(0x7E) == 448.0 and lib.orc_e4m3_to_f32(0x01) == 2.0 ** -9
+
+
+def test_e4m3_encode_is_nearest_even_and_saturates():
+    """Brute force: every float maps to the nearest finite E4M3 value, ties to the even code."""
+    values = np.array([e4m3_closed_form(b) for b in range(0x7F)])  # positive finite codes, ascending
+    g = np.random.Generator(np.random.PCG64(4))
+    xs = np.concatenate([g.uniform(-500, 500, 4000), g.uniform(-0.05, 0.05, 4000), values, (values[:-1] + values[1:]) / 2,
+                         [448.0, 449.0, 464.0, 465.0, 1e9, -1e9, 0.0]]).astype(np.float32)
+    for x in xs:
+        got = lib.orc_f32_to_e4m3(float(x))
+        a = abs(float(x))
+        if a >= 448.0:
+            want = 0x7E
+        else:
+            d = np.abs(values - a)
+            best = np.flatnonzero(d == d.min())
+            want = int(best[0]) if len(best) == 1 else int([c for c in best if c % 2 == 0][0])
+        want |= 0x80 if np.signbit(x) else 0
+        assert got == want, (float(x), hex(got), hex(want))
+    assert lib.orc_f32_to_e4m3(float("nan")) & 0x7F == 0x7F
+
+
+# ---------------------------------------------------------------------- Q8_1
+
+
+def test_q8_1_layout_and_values_against_numpy():
+    """Block = {f16 d; f16 s; i8 qs[32]} (src/format/encoding.cc:112 of the reference), d = amax / 127,
+    q = round-half-away(x / d), zero blocks past k (src/ir/op.h:400-405)."""
+    g = np.random.Generator(np.random.PCG64(5))
+    x = g.standard_normal((3, 96)).astype(np.float32)
+    x[0, :32] = 0
+    x[1, 40] = 1000.0
+    got = oracle.q8_1_quantize(x)
+    assert got.shape == (3, 512 // 32 * 36)
+    for r in range(3):
+        blocks = got[r].reshape(-1, 36)
+        assert not blocks[3:].any()
+        for b in range(3):
+            v = x[r, b * 32:(b + 1) * 32]
+            amax = np.abs(v).max()
+            d = np.float32(amax) / np.float32(127.0)
+            assert blocks[b, 0:2].view(np.float16)[0] == np.float16(d)
+            q = np.zeros(32) if amax == 0 else np.trunc(np.abs(v / d) + np.float32(0.5)) * np.sign(v)
+            # (|v / d| + 0.5 truncated is round-half-away unless the sum rounds up: not at these magnitudes)
+            assert np.array_equal(blocks[b, 4:].view(np.int8), q.astype(np.int8))
+            assert abs(float(blocks[b, 2:4].view(np.float16)[0]) - float(v.sum())) <= 2e-3 * max(1.0, abs(v.sum()))
+    # Decode is d * q (tests/unit/reference_decode_test.cc:207-224).
+    back = oracle.q8_1_decode(got[2], 96)
+    assert np.abs(back - x[2]).max() <= np.abs(x[2]).max() / 127 * 0.51
+
+
+def test_q8_1_flavours_differ_only_by_rounding_ties():
+    x = np.random.Generator(np.random.PCG64(6)).standard_normal((64, 4096)).astype(np.float32)
+    a = oracle.q8_1_quantize(x, oracle.Q8_DEVICE).reshape(64, -1, 36)
+    b = oracle.q8_1_quantize(x, oracle.Q8_GGML_CPU).reshape(64, -1, 36)
+    assert np.array_equal(a[:, :, 0:2], b[:, :, 0:2])  # the same scale
+    diff = a[:, :, 4:].view(np.int8).astype(int) - b[:, :, 4:].view(np.int8).astype(int)
+    assert np.abs(diff).max() <= 1
+    assert np.count_nonzero(diff) <= 1e-4 * diff.size  # a handful of codes per million
+
+
+# ------------------------------------------------------------- weight blocks
+
+
+def q4_k_decode_numpy(block):
+    """An independent Q4_K decode: ggml's get_scale_min_k4 packing, nibble j of byte
+    (g / 2) * 32 + i (tests/unit/dsv4_fast_test.cc:176-193 of the reference)."""
+    d, dmin = block[0:4].view(np.float16).astype(np.float32)
+    s = block[4:16].astype(int)
+    qs = block[16:].astype(int)
+    out = np.zeros(256, dtype=np.float64)
+    for g in range(8):
+        if g < 4:
+            sc, m = s[g] & 63, s[g + 4] & 63
+        else:
+            sc, m = (s[g + 4] & 15) | ((s[g - 4] >> 6) << 4), (s[g + 4] >> 4) | ((s[g] >> 6) << 4)
+        codes = (qs[(g // 2) * 32:(g // 2) * 32 + 32] >> (4 * (g % 2))) & 15
+        out[g * 32:(g + 1) * 32] = float(d) * sc * codes - float(dmin) * m
+    return out
+
+
+def test_q4_k_and_q8_0_decode_and_block_sums_by_brute_force():
+    from llmp_amd import synth
+    k = 512
+    for t in (oracle.TYPE_Q4_K, oracle.TYPE_Q8_0):
+        w = synth.random_blocks(t, 5, k, 7)
+        x = np.random.Generator(np.random.PCG64(8)).standard_normal((1, k)).astype(np.float32)
+        q8 = oracle.q8_1_quantize(x)
+        dec = oracle.decode_rows(t, w, k)
+        a = q8[0].reshape(-1, 36)
+        aq = a[:, 4:].view(np.int8).astype(np.int64)
+        ad = a[:, 0:2].view(np.float16).astype(np.float64).reshape(-1)
+        sums = oracle.vecq_block_sums(t, w, q8, k, 5)
+        y = oracle.vecq(t, w, q8, k, 5)[0, 0]
+        for r in range(5):
+            if t == oracle.TYPE_Q4_K:
+                blocks = w[r].reshape(-1, 144)
+                want = np.concatenate([q4_k_decode_numpy(b) for b in blocks])
+                codes = np.stack([((b[16:].astype(int)[(g // 2) * 32:(g // 2) * 32 + 32] >> (4 * (g % 2))) & 15)
+                                  for b in blocks for g in range(8)])
+                prod = (codes * aq[:k // 32]).sum(axis=1).reshape(-1, 8)
+                assert np.array_equal(sums[r, :, :8], prod)
+                assert np.array_equal(sums[r, :, 8:], aq[:k // 32].sum(axis=1).reshape(-1, 8))
+            else:
+                blocks = w[r].reshape(-1, 34)
+                wq = blocks[:, 2:].view(np.int8).astype(np.int64)
+                wd = blocks[:, 0:2].view(np.float16).astype(np.float64).reshape(-1)
+                want = (wq * wd[:, None]).reshape(-1)
+                assert np.array_equal(sums[r, :, 0], (wq * aq[:k // 32]).sum(axis=1))
+            np.testing.assert_allclose(dec[r], want, rtol=1e-6, atol=1e-12)
+            # The product is the FP64 dot of decoded weights and decoded activations.
+            act = (aq[:k // 32] * ad[:k // 32, None]).reshape(-1)
+            np.testing.assert_allclose(y[r], float(np.dot(want, act)), rtol=2e-6, atol=1e-9)
+
+
+def test_hand_built_blocks_have_known_sums():
+    w = np.zeros((1, 34), dtype=np.uint8)
+    w[0, 0:2] = np.array([2.0], dtype=np.float16).view(np.uint8)
+    w[0, 2:] = np.arange(1, 33, dtype=np.int8).view(np.uint8)
+    q8 = np.zeros((1, 16 * 36), dtype=np.uint8)
+    q8[0, 0:2] = np.array([0.5], dtype=np.float16).view(np.uint8)
+    q8[0, 4:36] = np.full(32, 3, dtype=np.int8).view(np.uint8)
+    assert oracle.vecq_block_sums(oracle.TYPE_Q8_0, w, q8, 32, 1)[0, 0, 0] == 3 * 528
+    assert oracle.vecq(oracle.TYPE_Q8_0, w, q8, 32, 1)[0, 0, 0] == 2.0 * 0.5 * 3 * 528
+    # Q4_K: sub-block g has scale g + 1 and minimum 2 g; every code 15 low, 1 high.
+    b = np.zeros((1, 144), dtype=np.uint8)
+    b[0, 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    b[0, 2:4] = np.array([0.5], dtype=np.float16).view(np.uint8)
+    sc = [g + 1 for g in range(8)]
+    mn = [2 * g for g in range(8)]
+    s = np.zeros(12, dtype=int)
+    for g in range(4):
+        s[g] = sc[g] | ((sc[g + 4] >> 4) << 6)
+        s[g + 4] = mn[g] | ((mn[g + 4] >> 4) << 6)
+        s[g + 8] = (sc[g + 4] & 15) | ((mn[g + 4] & 15) << 4)
+    b[0, 4:16] = s
+    b[0, 16:] = 0x1F
+    a = np.zeros((1, 16 * 36), dtype=np.uint8)
+    for g in range(8):
+        a[0, g * 36:g * 36 + 2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+        a[0, g * 36 + 4:g * 36 + 36] = np.full(32, 2, dtype=np.int8).view(np.uint8)
+    sums = oracle.vecq_block_sums(oracle.TYPE_Q4_K, b, a, 256, 1)[0, 0]
+    assert list(sums[:8]) == [15 * 64 if g % 2 == 0 else 64 for g in range(8)]
+    assert list(sums[8:]) == [64] * 8
+    want = sum(1.0 * sc[g] * sums[g] - 0.5 * mn[g] * 64 for g in range(8))
+    assert oracle.vecq(oracle.TYPE_Q4_K, b, a, 256, 1)[0, 0, 0] == want
+
+
+def test_glu_closed_forms():
+    """tests/unit/dsv4_fast_test.cc:401-408 (tanh GELU) and exec.cc:206-214,248-262 of the reference."""
+    for g, u in [(0.3, -1.2), (-2.0, 0.7), (5.0, 5.0), (0.0, 3.0)]:
+        gelu = 0.5 * g * (1 + math.tanh(math.sqrt(2.0 / math.acos(-1.0)) * g * (1 + 0.044715 * g * g)))
+        assert oracle.glu(oracle.GLU_GEGLU, g, u) == pytest.approx(gelu * u, rel=1e-15)
+        assert oracle.glu(oracle.GLU_SWIGLU, g, u) == pytest.approx(g / (1 + math.exp(-g)) * u, rel=1e-15)
+        gc, uc = min(g, 1.0), max(-1.0, min(1.0, u))
+        assert oracle.glu(oracle.GLU_SWIGLU_CLAMP, g, u, 1.0) == pytest.approx(gc / (1 + math.exp(-gc)) * uc, rel=1e-15)
+
+
+def test_vecq_forms_route_to_the_right_rows():
+    """Dense, grouped and routed indexing against an explicit loop over decoded weights."""
+    from llmp_amd import synth
+    t, k, n, experts = oracle.TYPE_Q8_0, 64, 6, 5
+    w = synth.random_blocks(t, experts * n, k, 9).reshape(experts, -1)
+    dec = oracle.decode_rows(t, w.reshape(experts * n, -1), k).reshape(experts, n, k).astype(np.float64)
+    x = np.random.Generator(np.random.PCG64(10)).standard_normal((3, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    act = np.stack([oracle.q8_1_decode(q8[i], k) for i in range(3)]).astype(np.float64)
+    ids = np.array([[4, 0], [1, 1], [2, 3]], dtype=np.int32)
+    got = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=3, used=2, stride_expert=n * (k // 32), experts=experts)
+    for tok in range(3):
+        for u in range(2):
+            np.testing.assert_allclose(got[tok, u], dec[ids[tok, u]] @ act[tok], rtol=1e-6)
+    with pytest.raises(IndexError):
+        oracle.vecq(t, w, q8, k, n, ids=np.array([[5, 0]], dtype=np.int32), tokens=1, used=2,
+                    stride_expert=n * (k // 32), experts=experts)
+
+
+# --------------------------------------------------------------------- MXFP8
+
+
+def test_mxfp8_quantize_invariants():
+    """tests/unit/qwen38_fast_test.cc:179-218 of the reference: each scale the smallest power of two with
+    amax <= 448 * s, each value within half an E4M3 step, padding rows' scales zero."""
+    g = np.random.Generator(np.random.PCG64(11))
+    rows, k = 5, 128
+    x = (g.standard_normal((rows, k)) * np.exp(g.uniform(-8, 8, (rows, 1)))).astype(np.float32)
+    x[0, :32] = 0
+    x[1, 33] = 448.0
+    x[1, 32:64] = np.clip(x[1, 32:64], -448, 448)
+    codes, scales = oracle.mxfp8_quantize(x)
+    blocks = k // 32
+    for r in range(128):
+        for b in range(blocks):
+            e = scales[lib.orc_scale_atom_offset(r, b, blocks)]
+            if r >= rows:
+                assert e == 0
+                continue
+            v = x[r, b * 32:(b + 1) * 32].astype(np.float64)
+            s = 2.0 ** (int(e) - 127)
+            amax = np.abs(v).max()
+            if amax > 0:
+                assert amax <= 448 * s * (1 + 1e-6) and amax > 224 * s * (1 - 1e-6)
+            q = np.array([e4m3_closed_form(int(c)) for c in codes[r, b * 32:(b + 1) * 32]]) * s
+            mag = np.abs(v) / s
+            step = np.where(mag < 2.0 ** -6, 2.0 ** -9, 2.0 ** (np.floor(np.log2(np.maximum(mag, 1e-300))) - 3))
+            assert np.all(np.abs(q - v) <= 0.5 * step * s * (1 + 1e-6))
+    assert lib.orc_mxfp8_scale_code(0.0) == 0 and lib.orc_mxfp8_scale_code(448.0) == 127
+    assert lib.orc_mxfp8_scale_code(449.0) == 128 and lib.orc_mxfp8_inverse_scale(127) == 1.0
+
+
+def test_scale_atoms_and_gemm_are_the_plain_block_scaled_product():
+    """src/format/layout.h:108-113 and tests/unit/reference_decode_test.cc:531-568 of the reference."""
+    assert lib.orc_scale_atom_offset(0, 0, 8) == 0
+    assert lib.orc_scale_atom_offset(1, 0, 8) == 16 and lib.orc_scale_atom_offset(32, 0, 8) == 4
+    assert lib.orc_scale_atom_offset(0, 1, 8) == 1 and lib.orc_scale_atom_offset(0, 4, 8) == 512
+    assert lib.orc_scale_atom_offset(128, 0, 8) == 1024
+    seen = {lib.orc_scale_atom_offset(r, b, 8) for r in range(256) for b in range(8)}
+    assert seen == set(range(256 * 8))  # a bijection onto the padded area
+    g = np.random.Generator(np.random.PCG64(12))
+    m, n, k = 6, 9, 128  # scale atoms take rows of whole groups of four scales
+    a = g.standard_normal((m, k)).astype(np.float32)
+    w = (g.standard_normal((n, k)) * 0.02).astype(np.float32)
+    ac, asc = oracle.mxfp8_quantize(a)
+    wc, wsc = oracle.mxfp8_quantize(w)
+
+    def dequant(codes, scales, rows):
+        out = np.zeros((rows, k))
+        for r in range(rows):
+            for j in range(k):
+                out[r, j] = e4m3_closed_form(int(codes[r, j])) * 2.0 ** (int(scales[lib.orc_scale_atom_offset(r, j // 32, k // 32)]) - 127)
+        return out
+    want = dequant(ac, asc, m) @ dequant(wc, wsc, n).T
+    got = oracle.mxfp8_gemm(ac, asc, wc, wsc)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-7)
+    assert oracle.mxfp8_dot(ac, asc, 2, wc, wsc, 3) == pytest.approx(want[2, 3], rel=1e-12)
+    np.testing.assert_allclose(want, a.astype(np.float64) @ w.astype(np.float64).T, rtol=0.2, atol=0.02)
+    # The swizzle of plain [n][k/32] scales is the same placement.
+    plain = g.integers(100, 140, size=(n, k // 32), dtype=np.uint8)
+    sw = oracle.mxfp8_swizzle(plain)
+    assert all(sw[lib.orc_scale_atom_offset(r, b, k // 32)] == plain[r, b] for r in range(n) for b in range(k // 32))
+    y = oracle.mxfp8_gemv(wc, np.stack([[wsc[lib.orc_scale_atom_offset(r, b, k // 32)] for b in range(k // 32)]
+                                        for r in range(n)]).astype(np.uint8), a)
+    np.testing.assert_allclose(y, a.astype(np.float64) @ dequant(wc, wsc, n).T, rtol=1e-5, atol=1e-7)
+
+
+# ----------------------------------------------------------------------- MoE
+
+
+def test_route_sort_and_reduce_against_numpy():
+    g = np.random.Generator(np.random.PCG64(13))
+    logits = g.standard_normal((9, 32)).astype(np.float32)
+    logits[3, [4, 7]] = logits[3].max() + 1  # a tie for first: the lower index wins
+    ids, w = oracle.route(logits, 4)
+    for t in range(9):
+        l = logits[t].astype(np.float64)
+        p = np.exp(l - l.max())
+        p /= p.sum()
+        order = np.argsort(-p, kind="stable")[:4]
+        assert list(ids[t]) == list(order)
+        np.testing.assert_allclose(w[t], p[order] / p[order].sum(), rtol=1e-6)
+    assert list(ids[3][:2]) == [4, 7]
+    bad = np.full((1, 8), np.nan, dtype=np.float32)
+    ids, w = oracle.route(bad, 3)
+    assert list(ids[0]) == [0, 1, 2] and not w.any()
+    tiny = np.full((1, 8), -1e4, dtype=np.float32)
+    tiny[0, 0] = 0
+    _, w = oracle.route(tiny, 2, normalize=False, scale=3.0)
+    assert w[0, 0] == 3.0 and w[0, 1] == 0.0
+    flat = np.array([3, 1, 3, 0, 1, 3], dtype=np.int32)
+    order, offsets = oracle.expert_sort(flat, 4)
+    assert list(order) == [3, 1, 4, 0, 2, 5] and list(offsets) == [0, 1, 3, 3, 6]
+    with pytest.raises(IndexError):
+        oracle.expert_sort(np.array([4], dtype=np.int32), 4)
+    x = g.standard_normal((2, 3, 8)).astype(np.float32)
+    ww = g.random((2, 3)).astype(np.float32)
+    np.testing.assert_allclose(oracle.expert_reduce(x, ww), (x * ww[:, :, None]).sum(axis=1), rtol=1e-6, atol=1e-7)
+
+
+# ---------------------------------------------------------------------- EXL3
+
+GOLDEN = [(0x0000, 0x3A25, 0x3F60, 0xC2E8), (0x0001, 0xBB5B, 0x304E, 0x3921), (0x1234, 0xC066, 0x3E0F, 0xB89E),
+          (0x8000, 0xB7F8, 0xB915, 0xBAF2), (0xBEEF, 0x424B, 0xC293, 0x3124), (0xFFFF, 0xB110, 0x3ACD, 0xB936)]
+
+
+def test_exl3_codebooks_match_the_reference_golden_vectors():
+    """tests/unit/reference_decode_test.cc:677-682 of the reference: six states, three codebooks."""
+    for state, three_inst, mcg, mul1 in GOLDEN:
+        assert lib.orc_exl3_codebook(oracle.CB_3INST, state) == three_inst
+        assert lib.orc_exl3_codebook(oracle.CB_MCG, state) == mcg
+        assert lib.orc_exl3_codebook(oracle.CB_MUL1, state) == mul1
+    assert lib.orc_exl3_codebook(3, 0) == 0x7E00
+
+
+def test_exl3_tiles_follow_the_independent_derivation():
+    """tests/unit/reference_decode_test.cc:699-747 of the reference: state p is the 16 bits of the tile's
+    circular MSB-first stream ending at bit (p + 1) K; position 8 L + i of a lane without bit 2 lands at row
+    (L % 4) * 2 + {0, 1, 8, 9}[i % 4], column 2 (L / 8 + 4 (i / 4)), lane L + 4's one column right."""
+    kk, nn = 32, 48
+    for bits in range(1, 9):
+        trellis = np.random.Generator(np.random.PCG64(100 + bits)).integers(0, 256, size=(kk // 16) * (nn // 16) * 32 * bits,
+                                                                           dtype=np.uint8)
+        want = np.zeros((kk, nn), dtype=np.uint16)
+        tile_bytes = 32 * bits
+        for kt in range(kk // 16):
+            for nt in range(nn // 16):
+                tile = trellis[(kt * (nn // 16) + nt) * tile_bytes:][:tile_bytes]
+                words = tile.view(np.uint32)
+                length = 256 * bits
+                stream = np.array([(int(words[j // 32]) >> (31 - j % 32)) & 1 for j in range(length)])
+                for p in range(256):
+                    end = (p + 1) * bits
+                    state = 0
+                    for i in range(16):
+                        state = (state << 1) | int(stream[(end + length - 16 + i) % length])
+                    group = p // 8
+                    partner = (group & 4) != 0
+                    lane = group - 4 if partner else group
+                    i = p % 8
+                    row = (lane % 4) * 2 + [0, 1, 8, 9][i % 4]
+                    col = 2 * (lane // 8 + 4 * (i // 4)) + (1 if partner else 0)
+                    want[kt * 16 + row, nt * 16 + col] = lib.orc_exl3_codebook(oracle.CB_MCG, state)
+        got = oracle.exl3_rotated(trellis, kk, nn, bits, oracle.CB_MCG)
+        assert np.array_equal(got, want), bits
+        part = oracle.exl3_rotated(trellis, kk, nn, bits, oracle.CB_MCG, 16, 32)
+        assert np.array_equal(part, want[:, 16:48])
+
+
+def test_exl3_rows_are_the_explicit_hadamard_product():
+    """tests/unit/reference_decode_test.cc:754-814 of the reference: W = diag(suh) H W^ H diag(svh) / 128
+    with explicit Hadamard matrices in F64, bit-equal for 3INST and MCG."""
+    kk, nn = 256, 384
+    idx = np.arange(128)
+    h128 = np.where(np.array([[bin(i & j).count("1") % 2 for j in idx] for i in idx]) == 0, 1.0, -1.0)
+    g = np.random.Generator(np.random.PCG64(200))
+    for bits, codebook in [(4, oracle.CB_3INST), (3, oracle.CB_3INST), (4, oracle.CB_MCG), (6, oracle.CB_MCG)]:
+        trellis = g.integers(0, 256, size=(kk // 16) * (nn // 16) * 32 * bits, dtype=np.uint8)
+        suh = (g.choice([-1.0, 1.0], kk) * g.uniform(0.25, 2.0, kk)).astype(np.float16)
+        svh = (g.choice([-1.0, 1.0], nn) * g.uniform(0.25, 2.0, nn)).astype(np.float16)
+        rot = oracle.exl3_rotated(trellis, kk, nn, bits, codebook).view(np.float16).astype(np.float64)
+        a = np.zeros_like(rot)
+        for kb in range(0, kk, 128):
+            a[kb:kb + 128] = h128 @ rot[kb:kb + 128]
+        w = np.zeros_like(rot)
+        for nb in range(0, nn, 128):
+            w[:, nb:nb + 128] = a[:, nb:nb + 128] @ h128
+        want = (w * suh.astype(np.float64)[:, None] * svh.astype(np.float64)[None, :] / 128.0).T.astype(np.float32)
+        got = oracle.exl3_rows(trellis, suh.view(np.uint16), svh.view(np.uint16), kk, nn, bits, codebook)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        some = oracle.exl3_rows(trellis, suh.view(np.uint16), svh.view(np.uint16), kk, nn, bits, codebook, 100, 200)
+        assert np.array_equal(some, got[100:300])
+        # The linear over these rows: within the F16 rounding of the transformed input
+        # (tests/unit/exl3_trellis_test.cc:519-564: relative RMS 2^-8 a row).
+        x = g.standard_normal((2, kk)).astype(np.float16)
+        y = oracle.exl3_linear(trellis, suh.view(np.uint16), svh.view(np.uint16), kk, nn, bits, codebook, x.view(np.uint16))
+        ref = x.astype(np.float64) @ got.astype(np.float64).T
+        for r in range(2):
+            assert np.sqrt(np.mean((y[r] - ref[r]) ** 2)) <= 2.0 ** -8 * np.sqrt(np.mean(ref[r] ** 2))
