@@ -149,6 +149,44 @@ int llmp_hip_q8_1_quantize_rows(const float* x, const int32_t* rows, void* out, 
 int llmp_hip_moe_combine(const float* x, const float* weights, const int32_t* position, int width,
                          int used, int tokens, float* out, void* stream);
 
+/* ------------------------------------------------------------------ MXFP8
+ * E4M3 codes with one E8M0 scale per 32 values along K. "Atoms" is the scale layout of
+ * src/format/layout.h:108-113 (ScaleAtomOffset; the same as moe_cutlass.h:42-46 SfOffset):
+ * 128-row by 4-scale atoms of 512 bytes, along K first, rows padded to 128, k a multiple of 128.
+ *
+ * llmp.mxfp8.quantize (src/kernels/ggml/llmp_ops.cu:610-648, mxfp8_quant.cuh:19-46): rows of
+ * k F32 or BF16 values, x_stride elements apart, to codes [rows][k] and scales in atoms for
+ * the rows rounded up to 128 (the padding rows' scales zero): RowsLayout of
+ * mxfp8_cutlass.h:42-57 with the two parts passed separately. */
+int llmp_hip_mxfp8_quantize(const void* x, int x_type, int64_t x_stride, int64_t k, int64_t rows,
+                            void* codes, void* scales, void* stream);
+/* llmp.mxfp8.swizzle (llmp_ops.cu:652-663): a weight's scales [n][k / 32] into atoms. */
+int llmp_hip_mxfp8_swizzle(const void* scales, int64_t n, int64_t k, void* out, void* stream);
+/* llmp.mxfp8.mul_mat_vec (llmp_ops.cu:145-224): y[t][r] = sum over blocks of (sum of 32
+ * E4M3(code) * x) * 2^(scale - 127), scales plain [n][k / 32], x F32 [tokens][k], 1..16
+ * tokens, y F32 [tokens][n]. */
+int llmp_hip_mxfp8_gemv(const void* codes, const void* scales, int64_t n, int64_t k, const float* x,
+                        int tokens, float* y, void* stream);
+
+/* llmp.mxfp8.gemm: mxfp8::Gemm / Available / Scratch / Run of
+ * src/kernels/ggml/mxfp8_cutlass.h:56-79, field for field. D[m, n] = A[m, k] * B[n, k]^T,
+ * both operands codes with scales in atoms, F32 accumulation, D F32 or BF16 (rounded once). */
+typedef struct llmp_mxfp8_gemm {
+  int m;
+  int n;
+  int k;
+  const void* a;        /* codes, m rows of k */
+  const void* a_scales; /* atoms */
+  const void* b;        /* codes, n rows of k */
+  const void* b_scales; /* atoms */
+  void* d;              /* m rows of n */
+  int bf16;             /* D in BF16, else F32 */
+  void* scratch;        /* llmp_hip_mxfp8_gemm_scratch bytes, 256-byte aligned (none needed: may be null) */
+} llmp_mxfp8_gemm;
+int llmp_hip_mxfp8_gemm_available(void);
+size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int compute_units);
+int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,6 +27,13 @@ class VecQDesc(C.Structure):
     ]
 
 
+class Mxfp8Gemm(C.Structure):
+    """llmp_mxfp8_gemm: mxfp8::Gemm of src/kernels/ggml/mxfp8_cutlass.h:56-70 of the reference."""
+    _fields_ = [("m", C.c_int), ("n", C.c_int), ("k", C.c_int), ("a", C.c_void_p), ("a_scales", C.c_void_p),
+                ("b", C.c_void_p), ("b_scales", C.c_void_p), ("d", C.c_void_p), ("bf16", C.c_int),
+                ("scratch", C.c_void_p)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -50,6 +57,12 @@ SYMBOLS = {
     "llmp_hip_moe_route": (_int, [_vp, _int, _int, _int, _int, _vp, _vp]),
     "llmp_hip_q8_1_quantize_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
+    "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "llmp_hip_mxfp8_swizzle": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "llmp_hip_mxfp8_gemv": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _vp, _vp]),
+    "llmp_hip_mxfp8_gemm_available": (_int, []),
+    "llmp_hip_mxfp8_gemm_scratch": (C.c_size_t, [C.POINTER(Mxfp8Gemm), _int]),
+    "llmp_hip_mxfp8_gemm_run": (_int, [C.POINTER(Mxfp8Gemm), _int, _vp]),
 }
 
 _lib = None

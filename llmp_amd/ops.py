@@ -8,7 +8,7 @@ import torch
 
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_K,  # noqa: F401
-                   TYPE_Q8_0, X_BF16, X_F16, X_F32, KernelFailure, VecQDesc, VecQSource)
+                   TYPE_Q8_0, X_BF16, X_F16, X_F32, KernelFailure, Mxfp8Gemm, VecQDesc, VecQSource)
 
 BLOCK_BYTES = {TYPE_Q8_0: 34, TYPE_Q4_K: 144}
 BLOCK_ELEMENTS = {TYPE_Q8_0: 32, TYPE_Q4_K: 256}
@@ -214,3 +214,55 @@ def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWI
     if keep is not None:
         keep.update(h=h, hq=hq, y=y, route=route)
     return moe_combine(y, weights, route.position), ids, weights
+
+
+def mxfp8_scale_bytes(rows, k):
+    """SwizzledScaleBytes: src/kernels/ggml/mxfp8_cutlass.h:53-57 of the reference."""
+    return (rows + 127) // 128 * 128 * (k // 32)
+
+
+def mxfp8_quantize(x):
+    """llmp.mxfp8.quantize: float32 / bfloat16 [rows, k] -> (codes uint8 [rows, k], scales uint8 atoms)."""
+    lib = _lib.load()
+    rows, k = x.shape
+    codes = torch.empty((rows, k), dtype=torch.uint8, device=x.device)
+    scales = torch.empty(mxfp8_scale_bytes(rows, k), dtype=torch.uint8, device=x.device)
+    _lib.check(lib.llmp_hip_mxfp8_quantize(_ptr(x), _x_type(x), x.stride(0), k, rows, _ptr(codes), _ptr(scales),
+                                           _stream()))
+    return codes, scales
+
+
+def mxfp8_swizzle(scales):
+    """llmp.mxfp8.swizzle: uint8 [n, k / 32] -> atoms."""
+    lib = _lib.load()
+    n, blocks = scales.shape
+    out = torch.empty(mxfp8_scale_bytes(n, blocks * 32), dtype=torch.uint8, device=scales.device)
+    _lib.check(lib.llmp_hip_mxfp8_swizzle(_ptr(scales), n, blocks * 32, _ptr(out), _stream()))
+    return out
+
+
+def mxfp8_gemv(codes, scales, x):
+    """llmp.mxfp8.mul_mat_vec: codes [n, k], plain scales [n, k / 32], x float32 [tokens, k]."""
+    lib = _lib.load()
+    n, k = codes.shape
+    tokens = x.shape[0]
+    y = torch.empty((tokens, n), dtype=torch.float32, device=x.device)
+    _lib.check(lib.llmp_hip_mxfp8_gemv(_ptr(codes), _ptr(scales), n, k, _ptr(x), tokens, _ptr(y), _stream()))
+    return y
+
+
+def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, bf16=True, out=None):
+    """llmp.mxfp8.gemm: D[m, n] = A[m, k] B[n, k]^T, scales in atoms."""
+    lib = _lib.load()
+    m, k = a_codes.shape
+    n = b_codes.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16 if bf16 else torch.float32, device=a_codes.device)
+    g = Mxfp8Gemm()
+    g.m, g.n, g.k = m, n, k
+    g.a, g.a_scales, g.b, g.b_scales, g.d = (a_codes.data_ptr(), a_scales.data_ptr(), b_codes.data_ptr(),
+                                             b_scales.data_ptr(), out.data_ptr())
+    g.bf16 = int(bf16)
+    g.scratch = None
+    _lib.check(lib.llmp_hip_mxfp8_gemm_run(C.byref(g), lib.llmp_hip_compute_units(), _stream()))
+    return out
