@@ -187,6 +187,53 @@ int llmp_hip_mxfp8_gemm_available(void);
 size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int compute_units);
 int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream);
 
+/* ------------------------------------------------------------------ EXL3
+ * The trellis-coded linear. Weights as src/kernels/exl3/validate.h:84-96 holds them: the
+ * trellis [k / 16][n / 16][16 * bits] uint16, suh (k F16) and svh (n F16); every dimension a
+ * multiple of 128. The codebook is a parameter (src/format/encoding.h:121 of the reference):
+ * the reference's device kernels build MCG only, its CPU definition all three
+ * (src/kernels/reference/decode_exl3.cc:41-66). */
+enum { LLMP_EXL3_3INST = 0, LLMP_EXL3_MCG = 1, LLMP_EXL3_MUL1 = 2 };
+typedef struct llmp_exl3_weights {
+  const void* trellis;
+  const void* suh;
+  const void* svh;
+  int k;
+  int n;
+  int bits;
+  int codebook; /* LLMP_EXL3_* */
+} llmp_exl3_weights;
+
+/* LaunchContext::Reconstruct, unfused (src/kernels/exl3/launch.h:100-103, validate.h:186-197):
+ * columns [column, column + columns) of the weights in the rotated basis into w
+ * (k x columns F16, row-major); whole 16-column tiles. */
+int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void* w, int column, int columns,
+                              void* stream);
+
+/* LaunchContext::Hadamard (launch.h:104-106, validate.h:199-212): 128-point Hadamard
+ * transforms of the rows of x (rows x columns) into y (x itself or disjoint), times
+ * 1 / sqrt(128): F16 with the input scale (y = H(x * scale)), or F16 / F32 with the output
+ * scale (y = H(x) * scale). scale: columns F16. */
+int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, int columns, int f32,
+                           int input_scale, void* stream);
+
+/* The packed linear for 1..16 rows: LinearOperands of validate.h:118-131 and
+ * PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54. x (m x k F16) into
+ * y (m x n, F16 or F32); a_had is the caller's m x k F16 scratch for the transformed input,
+ * written first. `scratch` (llmp_hip_exl3_linear_scratch bytes, 8-byte aligned) takes the place
+ * of the reference's lock area: the K slices' partial sums, added in slice order. Three
+ * launches are queued; a failure after the first is reported as a fault (negative). */
+typedef struct llmp_exl3_linear {
+  llmp_exl3_weights weights;
+  const void* x;
+  void* a_had;
+  void* y;
+  int f32; /* y in F32, else F16 */
+  int m;
+} llmp_exl3_linear;
+size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op);
+int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

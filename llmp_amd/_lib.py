@@ -34,6 +34,18 @@ class Mxfp8Gemm(C.Structure):
                 ("scratch", C.c_void_p)]
 
 
+class Exl3Weights(C.Structure):
+    """llmp_exl3_weights: src/kernels/exl3/validate.h:84-96 of the reference, plus the codebook."""
+    _fields_ = [("trellis", C.c_void_p), ("suh", C.c_void_p), ("svh", C.c_void_p), ("k", C.c_int), ("n", C.c_int),
+                ("bits", C.c_int), ("codebook", C.c_int)]
+
+
+class Exl3Linear(C.Structure):
+    """llmp_exl3_linear: LinearOperands of src/kernels/exl3/validate.h:118-131 of the reference."""
+    _fields_ = [("weights", Exl3Weights), ("x", C.c_void_p), ("a_had", C.c_void_p), ("y", C.c_void_p),
+                ("f32", C.c_int), ("m", C.c_int)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -63,6 +75,10 @@ SYMBOLS = {
     "llmp_hip_mxfp8_gemm_available": (_int, []),
     "llmp_hip_mxfp8_gemm_scratch": (C.c_size_t, [C.POINTER(Mxfp8Gemm), _int]),
     "llmp_hip_mxfp8_gemm_run": (_int, [C.POINTER(Mxfp8Gemm), _int, _vp]),
+    "llmp_hip_exl3_reconstruct": (_int, [C.POINTER(Exl3Weights), _vp, _int, _int, _vp]),
+    "llmp_hip_exl3_hadamard": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp]),
+    "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),
+    "llmp_hip_exl3_linear": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _vp]),
 }
 
 _lib = None

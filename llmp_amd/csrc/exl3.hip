@@ -1,0 +1,432 @@
+// The EXL3 trellis-coded linear (QTIP-style) for gfx950: codebook decode, weight
+// reconstruction, the 128-point Hadamard transforms and the packed product for up to 16 rows.
+//
+// Format (src/kernels/reference/decode_exl3.cc of the reference): the weights are
+// [K / 16][N / 16] tiles of 16 x 16 values at K bits a value; a tile's 256 K bits are a
+// circular stream of uint32 words, most significant bit first, and the value at position t is
+// the codebook value of the 16-bit state ending at bit (t + 1) K. Position 8 L + i (L below 32
+// without bit 2) lands at row (L % 4) * 2 + {0, 1, 8, 9}[i % 4], column 2 (L / 8 + 4 (i / 4)),
+// and lane L + 4's same position one column right. W = diag(suh) H W^ H diag(svh) / 128 with
+// H block diagonal over 128, so y = H(H(x * suh) / sqrt(128) -> f16, times W^) / sqrt(128) * svh.
+//
+// Lane mapping, wave64: that placement is a bijection between a tile's 64 groups of four
+// consecutive positions and the 64 lanes of a 16 x 16 x 16 MFMA's second operand. Lane
+// l = (n = l % 16, g = l / 16) takes positions 8 L + 4 (n / 8) + [0, 4) with
+// L = g + 4 (n % 2) + 8 ((n % 8) / 2): the values of column n at rows 2 g, 2 g + 1, 2 g + 8,
+// 2 g + 9, which is column n of the operand with its four k slots in that row order; the other
+// operand (the transformed activations, a row a token) is loaded with the same row order. So a
+// wave decodes a tile with four states a lane and multiplies it by one MFMA, whatever the
+// token count up to 16. A wave takes the eight tiles of one 128-column block (1 KB, contiguous)
+// per 16 rows of K, fetched with global_load_lds_dwordx4 into a small ring, and a slice of K;
+// the slices' partial sums are added in slice order by the output transform (no atomics).
+//
+// Reference behaviour restated here: src/kernels/reference/decode_exl3.cc:25-66 (codebooks),
+// :82-127 (state and placement), :173-265 (transforms); src/kernels/exl3/validate.h:61-131
+// (scale constant, operand structs), launch.cc:430-481 (reconstruct and Hadamard launches).
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "common.h"
+#include "llmp_hip.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr float kHadamardScale = 0.088388347648f;  // validate.h:64
+
+typedef __attribute__((address_space(3))) void* LdsPointer;
+typedef const __attribute__((address_space(1))) void* GlobalPointer;
+typedef _Float16 Half4 __attribute__((ext_vector_type(4)));
+typedef float V4f __attribute__((ext_vector_type(4)));
+
+// ------------------------------------------------------------------ codebooks
+
+// s * m mod 2^32 for a 16-bit s, as two 24-bit multiplies (full rate) instead of a 32-bit one.
+template <uint32_t kMultiplier>
+__device__ __forceinline__ uint32_t MulState(uint32_t s, uint32_t add) {
+  constexpr uint32_t lo = kMultiplier & 0xFFFFFFu;
+  constexpr uint32_t hi = kMultiplier >> 24;
+  const uint32_t x = __umul24(s, lo) + add;  // low 32 bits of a 40-bit product
+  if constexpr (hi == 0) return x;
+  return x + (__umul24(s, hi) << 24);
+}
+
+// decode_exl3.cc:28-37: each half keeps its sign and low 12 bits under exponent 0b011xx, then
+// the halves are added as one F16 addition.
+__device__ __forceinline__ _Float16 SumHalves(uint32_t x) {
+  const uint32_t y = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
+  const _Float16 lo = __builtin_bit_cast(_Float16, static_cast<uint16_t>(y & 0xFFFFu));
+  const _Float16 hi = __builtin_bit_cast(_Float16, static_cast<uint16_t>(y >> 16));
+  return lo + hi;
+}
+
+// decode_exl3.cc:41-66
+template <int CB>
+__device__ __forceinline__ _Float16 Codebook(uint32_t state) {
+  if constexpr (CB == LLMP_EXL3_3INST) {
+    return SumHalves(MulState<89226354u>(state, 64248484u));
+  } else if constexpr (CB == LLMP_EXL3_MCG) {
+    return SumHalves(MulState<0xCBAC1FEDu>(state, 0u));
+  } else {
+    const uint32_t x = MulState<0x83DCD12Du>(state, 0u);
+    const uint32_t sum = (x & 0xFFu) + ((x >> 8) & 0xFFu) + ((x >> 16) & 0xFFu) + (x >> 24) + 0x6400u;
+    const _Float16 h = __builtin_bit_cast(_Float16, static_cast<uint16_t>(sum & 0xFFFFu));
+    const _Float16 m = __builtin_bit_cast(_Float16, static_cast<uint16_t>(0x1EEEu));
+    const _Float16 a = __builtin_bit_cast(_Float16, static_cast<uint16_t>(0xC931u));
+    return __builtin_fmaf16(h, m, a);  // one rounding
+  }
+}
+
+// The state of position `t` of a tile of `words` uint32 (decode_exl3.cc:82-96); Word(i) reads
+// word i of the tile.
+template <int BITS, typename WordFn>
+__device__ __forceinline__ uint32_t State(int t, WordFn word) {
+  constexpr int words = BITS * 8;
+  const int end = (t + 1) * BITS + 256 * BITS;  // past the state's last bit, a period ahead
+  const int i1 = (end - 1) >> 5;
+  const int i0 = (end - 16) >> 5;  // may be i1
+  const int shift = ((i1 + 1) << 5) - end;
+  const uint64_t merged = (static_cast<uint64_t>(word(i0 % words)) << 32) | word(i1 % words);
+  // When both indices agree the high word is shifted out of the 16 bits kept.
+  return static_cast<uint32_t>(merged >> shift) & 0xFFFFu;
+}
+
+// A lane's place in a tile: column n, row group g, and its first position.
+struct Place {
+  int n, g, first;
+};
+__device__ __forceinline__ Place PlaceOf(int lane) {
+  Place p;
+  p.n = lane & 15;
+  p.g = lane >> 4;
+  const int l32 = p.g + 4 * (p.n & 1) + 8 * ((p.n & 7) >> 1);
+  p.first = 8 * l32 + 4 * (p.n >> 3);
+  return p;
+}
+// The rows of a lane's four values, in position order.
+__device__ __forceinline__ int RowOf(int g, int j) { return 2 * g + (j & 1) + 8 * (j >> 1); }
+
+template <int CB, int BITS, typename WordFn>
+__device__ __forceinline__ Half4 DecodeFour(int first, WordFn word) {
+  Half4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = Codebook<CB>(State<BITS>(first + j, word));
+  return v;
+}
+
+// ---------------------------------------------------------------- reconstruct
+
+// Columns [column, column + columns) of the rotated-basis weights into w[k][columns] F16: a
+// wave a tile; grid (columns / 16, k / 16 / 4), 4 waves a workgroup.
+template <int CB, int BITS>
+__global__ __launch_bounds__(256) void ReconstructKernel(const uint32_t* __restrict__ trellis,
+                                                        uint16_t* __restrict__ w, int n, int k, int column,
+                                                        int columns) {
+  const int lane = threadIdx.x & 63;
+  const int kt = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (kt >= k / 16) return;  // whole waves
+  const int nt = column / 16 + blockIdx.x;
+  const uint32_t* tile = trellis + (static_cast<int64_t>(kt) * (n / 16) + nt) * (BITS * 8);
+  const Place p = PlaceOf(lane);
+  const Half4 v = DecodeFour<CB, BITS>(p.first, [&](int i) { return tile[i]; });
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = kt * 16 + RowOf(p.g, j);
+    const _Float16 value = v[j];  // (a bit cast straight from a vector's element reads element 0)
+    w[static_cast<int64_t>(row) * columns + blockIdx.x * 16 + p.n] = __builtin_bit_cast(uint16_t, value);
+  }
+}
+
+// ------------------------------------------------------------------ Hadamard
+
+// The 128-point Walsh-Hadamard transform of a wave's 128 values, lane l holding values 2 l and
+// 2 l + 1, natural order (H[i][j] = (-1)^popcount(i & j)), unscaled, in F32.
+__device__ __forceinline__ void Hadamard128(float& a, float& b, int lane) {
+  const float s = a + b;
+  b = a - b;
+  a = s;
+#pragma unroll
+  for (int mask = 1; mask < 64; mask <<= 1) {
+    const float pa = ShflXor(a, mask);
+    const float pb = ShflXor(b, mask);
+    const bool upper = (lane & mask) != 0;
+    a = upper ? pa - a : a + pa;
+    b = upper ? pb - b : b + pb;
+  }
+}
+
+// y = f(H(x * in_scale)) * r * out_scale over each 128 block of each row; grid (rows, columns
+// / 128), a wave a block. X / Y: 0 F16, 1 F32. `slices` partial inputs are added in order first.
+template <int X, int Y>
+__global__ __launch_bounds__(64) void HadamardKernel(const void* __restrict__ x, void* __restrict__ y,
+                                                    const uint16_t* __restrict__ in_scale,
+                                                    const uint16_t* __restrict__ out_scale, int columns, int slices,
+                                                    int64_t slice_stride) {
+  const int lane = threadIdx.x;
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * columns + blockIdx.y * 128 + 2 * lane;
+  float a = 0.0f, b = 0.0f;
+  for (int s = 0; s < slices; ++s) {
+    if constexpr (X == 0) {
+      const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(x) + s * slice_stride + at);
+      a += HalfBitsToFloat(v & 0xFFFFu);
+      b += HalfBitsToFloat(v >> 16);
+    } else {
+      const float2 v = *reinterpret_cast<const float2*>(static_cast<const float*>(x) + s * slice_stride + at);
+      a += v.x;
+      b += v.y;
+    }
+  }
+  const int c = blockIdx.y * 128 + 2 * lane;
+  if (in_scale != nullptr) {
+    const uint32_t s = *reinterpret_cast<const uint32_t*>(in_scale + c);
+    a *= HalfBitsToFloat(s & 0xFFFFu);
+    b *= HalfBitsToFloat(s >> 16);
+  }
+  Hadamard128(a, b, lane);
+  a *= kHadamardScale;
+  b *= kHadamardScale;
+  if (out_scale != nullptr) {
+    const uint32_t s = *reinterpret_cast<const uint32_t*>(out_scale + c);
+    a *= HalfBitsToFloat(s & 0xFFFFu);
+    b *= HalfBitsToFloat(s >> 16);
+  }
+  if constexpr (Y == 0) {
+    *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(y) + at) = FloatToHalfBits(a) | (FloatToHalfBits(b) << 16);
+  } else {
+    *reinterpret_cast<float2*>(static_cast<float*>(y) + at) = make_float2(a, b);
+  }
+}
+
+// ------------------------------------------------------------------- product
+
+constexpr int kRingDepth = 4;  // K steps of a 128-column block in flight a wave
+constexpr int kProductWaves = 4;
+
+// partial[slice][m][n] = sum over the slice's K of xh[m][k] W^[k][n]; grid (n / 128 / 4 waves,
+// slices); xh F16 [m][k], m <= 16. A wave a 128-column block: eight tiles per 16 rows of K.
+template <int CB, int BITS>
+__global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_t* __restrict__ trellis,
+                                                                   const uint16_t* __restrict__ xh,
+                                                                   float* __restrict__ partial, int m, int n, int k,
+                                                                   int steps_per_slice) {
+  constexpr int kTileBytes = BITS * 32;
+  constexpr int kStepBytes = 8 * kTileBytes;  // a 128-column block's tiles of one K step
+  constexpr int kLoads = (kStepBytes + 1023) / 1024;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int block = blockIdx.x * kProductWaves + wave;  // of 128 columns
+  if (block >= n / 128) return;  // whole waves; nothing below synchronizes across waves
+  uint8_t* ring = lds + wave * (kRingDepth * kLoads * 1024);
+  const int steps = k / 16;
+  const int first = blockIdx.y * steps_per_slice;
+  const int last = min(first + steps_per_slice, steps);
+  const Place p = PlaceOf(lane);
+  const int64_t row_bytes = static_cast<int64_t>(n / 16) * kTileBytes;
+  const uint8_t* source = trellis + static_cast<int64_t>(block) * kStepBytes;
+
+  auto fetch = [&](int step) {
+    const uint8_t* from = source + step * row_bytes;
+    uint8_t* to = ring + (step % kRingDepth) * (kLoads * 1024);
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      if (i * 1024 + lane * 16 < kStepBytes) {
+        __builtin_amdgcn_global_load_lds((GlobalPointer)(from + i * 1024 + lane * 16), (LdsPointer)(to + i * 1024), 16,
+                                         0, 0);
+      }
+    }
+  };
+
+  V4f acc[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) acc[t] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
+  // The activations' operand: token l % 16, k slots in the lane group's row order.
+  const int token = min(p.n, m - 1);
+  const uint16_t* xrow = xh + static_cast<int64_t>(token) * k;
+
+  for (int s = first; s < min(first + kRingDepth - 1, last); ++s) fetch(s);
+  for (int step = first; step < last; ++step) {
+    const uint32_t x01 = *reinterpret_cast<const uint32_t*>(xrow + step * 16 + 2 * p.g);
+    const uint32_t x89 = *reinterpret_cast<const uint32_t*>(xrow + step * 16 + 2 * p.g + 8);
+    Half4 xv;
+    xv[0] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 & 0xFFFFu));
+    xv[1] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 >> 16));
+    xv[2] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 & 0xFFFFu));
+    xv[3] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 >> 16));
+    if (p.n >= m) xv = Half4{0, 0, 0, 0};
+    const int ahead = step + kRingDepth - 1;
+    if (ahead < last) {
+      fetch(ahead);
+      // All but the newest `kLoads * (kRingDepth - 1)` loads have landed: this step's tiles.
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((kLoads * (kRingDepth - 1)) & 0xF) | (((kLoads * (kRingDepth - 1)) >> 4) << 14));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+    const uint32_t* tiles = reinterpret_cast<const uint32_t*>(ring + (step % kRingDepth) * (kLoads * 1024));
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const uint32_t* tile = tiles + t * (BITS * 8);
+      const Half4 wv = DecodeFour<CB, BITS>(p.first, [&](int i) { return tile[i]; });
+      // D[token][n] += sum_j xv[token][j] wv[j][n]: first operand rows are tokens.
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(xv, wv, acc[t], 0, 0, 0);
+    }
+    asm volatile("" ::: "memory");
+  }
+  // acc[t][q] = D[token 4 g + q][column 16 t + n]
+  float* out = partial + static_cast<int64_t>(blockIdx.y) * m * n + block * 128;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = 4 * p.g + q;
+      if (row < m) out[static_cast<int64_t>(row) * n + t * 16 + p.n] = acc[t][q];
+    }
+  }
+}
+
+int SlicesFor(int m, int k) {
+  const int steps = k / 16;
+  int want = m <= 2 ? 32 : m <= 8 ? 16 : 8;
+  while (want > 1 && steps / want < 4) want /= 2;
+  return want;
+}
+
+int CheckWeights(const llmp_exl3_weights& w) {
+  if (w.trellis == nullptr || w.suh == nullptr || w.svh == nullptr) return Refuse(1, "exl3: null weights");
+  if (w.k <= 0 || w.n <= 0 || w.k % 128 != 0 || w.n % 128 != 0)
+    return Refuse(1, "exl3: dimensions %d x %d are not multiples of 128", w.k, w.n);
+  if (w.k > (1 << 19) || w.n > (1 << 19)) return Refuse(1, "exl3: a dimension exceeds 2^19");
+  if (w.bits < 1 || w.bits > 8) return Refuse(1, "exl3: rate %d outside 1..8", w.bits);
+  if (w.codebook < LLMP_EXL3_3INST || w.codebook > LLMP_EXL3_MUL1) return Refuse(1, "exl3: no codebook %d", w.codebook);
+  if (reinterpret_cast<uintptr_t>(w.trellis) % 16 != 0) return Refuse(1, "exl3: trellis not 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(w.suh) | reinterpret_cast<uintptr_t>(w.svh)) % 8 != 0)
+    return Refuse(1, "exl3: side vectors not 8-byte aligned");
+  return 0;
+}
+
+template <int CB, int BITS>
+void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int columns, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(columns / 16), static_cast<unsigned>((w.k / 16 + 3) / 4));
+  hipLaunchKernelGGL((ReconstructKernel<CB, BITS>), grid, dim3(256), 0, stream,
+                     static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
+}
+
+template <int CB, int BITS>
+void LaunchProduct(const llmp_exl3_weights& w, const void* xh, float* partial, int m, int slices, hipStream_t stream) {
+  constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
+  const int steps = w.k / 16;
+  const int per = (steps + slices - 1) / slices;
+  const dim3 grid(static_cast<unsigned>((w.n / 128 + kProductWaves - 1) / kProductWaves), static_cast<unsigned>(slices));
+  hipLaunchKernelGGL((ProductKernel<CB, BITS>), grid, dim3(kProductWaves * 64),
+                     static_cast<size_t>(kProductWaves) * kRingDepth * kLoads * 1024, stream,
+                     static_cast<const uint8_t*>(w.trellis), static_cast<const uint16_t*>(xh), partial, m, w.n, w.k, per);
+}
+
+template <typename F>
+bool DispatchBits(int bits, F&& f) {
+  switch (bits) {
+    case 1: f(std::integral_constant<int, 1>{}); return true;
+    case 2: f(std::integral_constant<int, 2>{}); return true;
+    case 3: f(std::integral_constant<int, 3>{}); return true;
+    case 4: f(std::integral_constant<int, 4>{}); return true;
+    case 5: f(std::integral_constant<int, 5>{}); return true;
+    case 6: f(std::integral_constant<int, 6>{}); return true;
+    case 7: f(std::integral_constant<int, 7>{}); return true;
+    case 8: f(std::integral_constant<int, 8>{}); return true;
+    default: return false;
+  }
+}
+
+template <typename F>
+void Dispatch(int codebook, int bits, F&& f) {
+  DispatchBits(bits, [&](auto b) {
+    constexpr int kBits = decltype(b)::value;
+    if (codebook == LLMP_EXL3_3INST) {
+      f(std::integral_constant<int, LLMP_EXL3_3INST>{}, std::integral_constant<int, kBits>{});
+    } else if (codebook == LLMP_EXL3_MCG) {
+      f(std::integral_constant<int, LLMP_EXL3_MCG>{}, std::integral_constant<int, kBits>{});
+    } else {
+      f(std::integral_constant<int, LLMP_EXL3_MUL1>{}, std::integral_constant<int, kBits>{});
+    }
+  });
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void* w, int column, int columns,
+                                         void* stream) {
+  if (weights == nullptr || w == nullptr) return Refuse(1, "exl3.reconstruct: null operand");
+  if (const int bad = CheckWeights(*weights); bad != 0) return bad;
+  if (column < 0 || columns <= 0 || column % 16 != 0 || columns % 16 != 0 || column + columns > weights->n)
+    return Refuse(1, "exl3.reconstruct: columns [%d, %d) are not whole tiles of the weights", column, column + columns);
+  Dispatch(weights->codebook, weights->bits, [&](auto cb, auto bits) {
+    LaunchReconstruct<decltype(cb)::value, decltype(bits)::value>(*weights, w, column, columns,
+                                                                  static_cast<hipStream_t>(stream));
+  });
+  return LaunchStatus("exl3.reconstruct");
+}
+
+extern "C" int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, int columns, int f32,
+                                      int input_scale, void* stream) {
+  if (x == nullptr || y == nullptr || scale == nullptr) return Refuse(1, "exl3.hadamard: null operand");
+  if (rows <= 0 || rows > 65535 || columns <= 0 || columns % 128 != 0)
+    return Refuse(1, "exl3.hadamard: 1 to 65535 rows of whole 128-value blocks");
+  if (input_scale && f32) return Refuse(1, "exl3.hadamard: the input scale's transform is F16");
+  const dim3 grid(static_cast<unsigned>(rows), static_cast<unsigned>(columns / 128));
+  const auto s = static_cast<hipStream_t>(stream);
+  const auto* sc = static_cast<const uint16_t*>(scale);
+  if (f32) {
+    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, x, y, nullptr, sc, columns, 1, int64_t{0});
+  } else if (input_scale) {
+    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, x, y, sc, nullptr, columns, 1, int64_t{0});
+  } else {
+    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, x, y, nullptr, sc, columns, 1, int64_t{0});
+  }
+  return LaunchStatus("exl3.hadamard");
+}
+
+extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
+  if (op == nullptr || op->m <= 0 || op->weights.k <= 0 || op->weights.n <= 0) return 0;
+  return static_cast<size_t>(SlicesFor(op->m, op->weights.k)) * op->m * op->weights.n * sizeof(float);
+}
+
+extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream) {
+  if (op == nullptr) return Refuse(1, "exl3.linear: null operands");
+  if (const int bad = CheckWeights(op->weights); bad != 0) return bad;
+  if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || scratch == nullptr)
+    return Refuse(1, "exl3.linear: null operand");
+  if (op->m < 1 || op->m > 16) return Refuse(1, "exl3.linear: the packed product takes 1 to 16 rows, not %d", op->m);
+  if (scratch_bytes < llmp_hip_exl3_linear_scratch(op)) return Refuse(1, "exl3.linear: scratch too small");
+  if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
+       reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
+    return Refuse(1, "exl3.linear: operands not 8-byte aligned");
+  const llmp_exl3_weights& w = op->weights;
+  const auto s = static_cast<hipStream_t>(stream);
+  const int slices = SlicesFor(op->m, w.k);
+  // The transformed input, the product's slices, then their sum transformed.
+  hipLaunchKernelGGL((HadamardKernel<0, 0>), dim3(static_cast<unsigned>(op->m), static_cast<unsigned>(w.k / 128)),
+                     dim3(64), 0, s, op->x, op->a_had, static_cast<const uint16_t*>(w.suh), nullptr, w.k, 1, int64_t{0});
+  if (const int bad = LaunchStatus("exl3.linear input transform"); bad != 0) return bad;
+  Dispatch(w.codebook, w.bits, [&](auto cb, auto bits) {
+    LaunchProduct<decltype(cb)::value, decltype(bits)::value>(w, op->a_had, static_cast<float*>(scratch), op->m, slices, s);
+  });
+  const dim3 grid(static_cast<unsigned>(op->m), static_cast<unsigned>(w.n / 128));
+  const int64_t stride = static_cast<int64_t>(op->m) * w.n;
+  if (op->f32) {
+    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, scratch, op->y, nullptr,
+                       static_cast<const uint16_t*>(w.svh), w.n, slices, stride);
+  } else {
+    hipLaunchKernelGGL((HadamardKernel<1, 0>), grid, dim3(64), 0, s, scratch, op->y, nullptr,
+                       static_cast<const uint16_t*>(w.svh), w.n, slices, stride);
+  }
+  // A failure here follows queued launches: a fault, not a refusal.
+  const int status = LaunchStatus("exl3.linear");
+  return status > 0 ? -status : status;
+}

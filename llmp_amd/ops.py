@@ -8,7 +8,8 @@ import torch
 
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_K,  # noqa: F401
-                   TYPE_Q8_0, X_BF16, X_F16, X_F32, KernelFailure, Mxfp8Gemm, VecQDesc, VecQSource)
+                   TYPE_Q8_0, X_BF16, X_F16, X_F32, Exl3Linear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
+                   VecQSource)
 
 BLOCK_BYTES = {TYPE_Q8_0: 34, TYPE_Q4_K: 144}
 BLOCK_ELEMENTS = {TYPE_Q8_0: 32, TYPE_Q4_K: 256}
@@ -266,3 +267,51 @@ def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, bf16=True, out=None):
     g.scratch = None
     _lib.check(lib.llmp_hip_mxfp8_gemm_run(C.byref(g), lib.llmp_hip_compute_units(), _stream()))
     return out
+
+
+EXL3_3INST, EXL3_MCG, EXL3_MUL1 = 0, 1, 2
+
+
+def _exl3_weights(trellis, suh, svh, k, n, bits, codebook):
+    w = Exl3Weights()
+    w.trellis, w.suh, w.svh = trellis.data_ptr(), suh.data_ptr(), svh.data_ptr()
+    w.k, w.n, w.bits, w.codebook = k, n, bits, codebook
+    return w
+
+
+def exl3_reconstruct(trellis, suh, svh, k, n, bits, codebook, column=0, columns=None):
+    """The rotated-basis weights of columns [column, column + columns): float16 [k, columns]."""
+    lib = _lib.load()
+    columns = n if columns is None else columns
+    out = torch.empty((k, columns), dtype=torch.float16, device=trellis.device)
+    w = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
+    _lib.check(lib.llmp_hip_exl3_reconstruct(C.byref(w), _ptr(out), column, columns, _stream()))
+    return out
+
+
+def exl3_hadamard(x, scale, input_scale=True):
+    """128-point Hadamard transforms of x's rows, times 1 / sqrt(128), with the input or output scale."""
+    lib = _lib.load()
+    rows, columns = x.shape
+    y = torch.empty_like(x)
+    _lib.check(lib.llmp_hip_exl3_hadamard(_ptr(x), _ptr(y), _ptr(scale), rows, columns,
+                                          int(x.dtype == torch.float32), int(input_scale), _stream()))
+    return y
+
+
+def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, f32=True, keep=None):
+    """x float16 [m, k] (m <= 16) through the EXL3 linear: [m, n] float32 or float16.
+    `keep`, a dict, receives the transformed input a_had."""
+    lib = _lib.load()
+    m = x.shape[0]
+    op = Exl3Linear()
+    op.weights = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
+    a_had = torch.empty((m, k), dtype=torch.float16, device=x.device)
+    y = torch.empty((m, n), dtype=torch.float32 if f32 else torch.float16, device=x.device)
+    op.x, op.a_had, op.y, op.f32, op.m = x.data_ptr(), a_had.data_ptr(), y.data_ptr(), int(f32), m
+    need = lib.llmp_hip_exl3_linear_scratch(C.byref(op))
+    scratch = torch.empty(max(need, 8), dtype=torch.uint8, device=x.device)
+    _lib.check(lib.llmp_hip_exl3_linear(C.byref(op), _ptr(scratch), need, _stream()))
+    if keep is not None:
+        keep["a_had"] = a_had
+    return y

@@ -63,3 +63,13 @@ def bf16_bits(x):
 
 def bf16_to_f32(bits):
     return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def exl3_weights(k, n, bits, seed):
+    """A trellis of seed-random words (every bit stream is a valid trellis), input signs
+    suh = +-1 and output scales svh = +-|N(1, 0.1)|, both float16."""
+    g = rng(seed)
+    trellis = g.integers(0, 256, size=(k // 16) * (n // 16) * 32 * bits, dtype=np.uint8)
+    suh = g.choice(np.array([-1.0, 1.0]), size=k).astype(np.float16)
+    svh = (g.choice(np.array([-1.0, 1.0]), size=n) * np.abs(g.normal(1.0, 0.1, size=n))).astype(np.float16)
+    return trellis, suh, svh

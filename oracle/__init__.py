@@ -88,6 +88,8 @@ _sig("orc_exl3_placement", None, _vp)
 _sig("orc_exl3_rotated", None, _vp, _i64, _i64, _int, _int, _i64, _i64, _vp)
 _sig("orc_exl3_rows", None, _vp, _vp, _vp, _i64, _i64, _int, _int, _i64, _i64, _vp)
 _sig("orc_exl3_linear", None, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp, _i64, _vp, _int)
+_sig("orc_exl3_input", None, _vp, _i64, _vp, _i64, _vp)
+_sig("orc_exl3_product", None, _vp, _vp, _i64, _i64, _int, _int, _vp, _i64, _vp, _int)
 _sig("orc_max_threads", _int)
 
 
@@ -264,4 +266,19 @@ def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, threads=1):
     m = x.shape[0]
     y = np.zeros((m, n), dtype=np.float32)
     lib.orc_exl3_linear(_p(trellis), _p(suh), _p(svh), k, n, bits, codebook, _p(x), m, _p(y), threads)
+    return y
+
+
+def exl3_input(suh, k, x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    xh = np.zeros_like(x)
+    lib.orc_exl3_input(_p(suh), k, _p(x), x.shape[0], _p(xh))
+    return xh
+
+
+def exl3_product(trellis, svh, k, n, bits, codebook, xh, threads=1):
+    xh = np.ascontiguousarray(xh, dtype=np.uint16)
+    m = xh.shape[0]
+    y = np.zeros((m, n), dtype=np.float32)
+    lib.orc_exl3_product(_p(trellis), _p(svh), k, n, bits, codebook, _p(xh), m, _p(y), threads)
     return y

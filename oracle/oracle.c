@@ -647,17 +647,20 @@ void orc_exl3_rows(const uint8_t* trellis, const uint16_t* suh, const uint16_t* 
   free(column);
 }
 
-void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t* svh, int64_t k,
-                     int64_t n, int bits, int codebook, const uint16_t* x, int64_t m, float* y,
-                     int threads) {
+void orc_exl3_input(const uint16_t* suh, int64_t k, const uint16_t* x, int64_t m, uint16_t* xh) {
   const double r = 0.088388347648; /* validate.h:64 */
-  double* xh = (double*)malloc(sizeof(double) * (size_t)(m * k));
+  double* row = (double*)malloc(sizeof(double) * (size_t)k);
   for (int64_t i = 0; i < m; ++i) {
-    double* row = xh + i * k;
     for (int64_t c = 0; c < k; ++c) row[c] = (double)orc_f16_to_f32(x[i * k + c]) * (double)orc_f16_to_f32(suh[c]);
     for (int64_t kb = 0; kb < k; kb += 128) hadamard128(&row[kb]);
-    for (int64_t c = 0; c < k; ++c) row[c] = orc_f16_to_f32(orc_f32_to_f16((float)(row[c] * r)));
+    for (int64_t c = 0; c < k; ++c) xh[i * k + c] = orc_f32_to_f16((float)(row[c] * r));
   }
+  free(row);
+}
+
+void orc_exl3_product(const uint8_t* trellis, const uint16_t* svh, int64_t k, int64_t n, int bits,
+                      int codebook, const uint16_t* xh, int64_t m, float* y, int threads) {
+  const double r = 0.088388347648;
   (void)codebook_table(codebook);
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
   for (int64_t b = 0; b < n / 128; ++b) {
@@ -669,7 +672,7 @@ void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t
       double acc[128];
       for (int j = 0; j < 128; ++j) acc[j] = 0;
       for (int64_t c = 0; c < k; ++c) {
-        const double xv = xh[i * k + c];
+        const double xv = orc_f16_to_f32(xh[i * k + c]);
         const float* wr = rotf + c * 128;
         for (int j = 0; j < 128; ++j) acc[j] += xv * (double)wr[j];
       }
@@ -679,5 +682,13 @@ void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t
     free(rot);
     free(rotf);
   }
+}
+
+void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t* svh, int64_t k,
+                     int64_t n, int bits, int codebook, const uint16_t* x, int64_t m, float* y,
+                     int threads) {
+  uint16_t* xh = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)(m * k));
+  orc_exl3_input(suh, k, x, m, xh);
+  orc_exl3_product(trellis, svh, k, n, bits, codebook, xh, m, y, threads);
   free(xh);
 }

@@ -143,6 +143,11 @@ void orc_exl3_rows(const uint8_t* trellis, const uint16_t* suh, const uint16_t* 
 void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t* svh, int64_t k,
                      int64_t n, int bits, int codebook, const uint16_t* x, int64_t m, float* y,
                      int threads);
+/* Its two stages: the transformed input xh (F16 [m][k]), and the product and output transform
+ * over a given xh. */
+void orc_exl3_input(const uint16_t* suh, int64_t k, const uint16_t* x, int64_t m, uint16_t* xh);
+void orc_exl3_product(const uint8_t* trellis, const uint16_t* svh, int64_t k, int64_t n, int bits,
+                      int codebook, const uint16_t* xh, int64_t m, float* y, int threads);
 
 int orc_max_threads(void);
 

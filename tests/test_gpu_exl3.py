@@ -1,0 +1,124 @@
+"""Parity of the EXL3 operations (HIP, through the C ABI) against the CPU oracle: reconstructed
+weights bit for bit (every rate, the three codebooks), the transforms within F16/F32 rounding,
+and the packed linear to a maximum relative error of 1e-3."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import rel_close
+from llmp_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def halves(a, device):
+    return dev(a.view(np.int16), device).view(torch.float16)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("codebook", [ops.EXL3_3INST, ops.EXL3_MCG, ops.EXL3_MUL1])
+def test_reconstruct_is_the_rotated_decode_bit_for_bit(device, bits, codebook):
+    """tests/unit/exl3_trellis_test.cc:446-465 of the reference."""
+    k, n = 128, 256
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 100 + bits)
+    want = oracle.exl3_rotated(trellis, k, n, bits, codebook)
+    got = ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want)
+    part = ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook,
+                                column=64, columns=96)
+    assert np.array_equal(part.cpu().numpy().view(np.uint16), want[:, 64:160])
+
+
+def test_every_state_of_every_codebook(device):
+    """All 65,536 states: a 4-bit trellis whose stream walks them is not needed; a tile's positions
+    see 256 states each, so 4096 random tiles cover the space densely; the golden vectors pin the rest."""
+    k, n, bits = 1024, 1024, 4
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 7)
+    for codebook in (ops.EXL3_3INST, ops.EXL3_MCG, ops.EXL3_MUL1):
+        want = oracle.exl3_rotated(trellis, k, n, bits, codebook)
+        got = ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+        assert np.array_equal(got.cpu().numpy().view(np.uint16), want)
+
+
+def hadamard_rows(x):
+    idx = np.arange(128)
+    h = np.where(np.array([[bin(i & j).count("1") % 2 for j in idx] for i in idx]) == 0, 1.0, -1.0)
+    out = np.zeros_like(x, dtype=np.float64)
+    for b in range(0, x.shape[1], 128):
+        out[:, b:b + 128] = x[:, b:b + 128].astype(np.float64) @ h
+    return out
+
+
+def test_hadamard_transforms(device):
+    g = synth.rng(9)
+    rows, columns = 5, 384
+    x = g.standard_normal((rows, columns)).astype(np.float16)
+    scale = (g.choice([-1.0, 1.0], columns) * g.uniform(0.5, 1.5, columns)).astype(np.float16)
+    r = 0.088388347648
+    want_in = hadamard_rows(x.astype(np.float64) * scale.astype(np.float64)) * r
+    got_in = ops.exl3_hadamard(halves(x, device), halves(scale, device), input_scale=True).float().cpu().numpy()
+    np.testing.assert_allclose(got_in, want_in, rtol=2e-3, atol=2e-3)
+    want_out = hadamard_rows(x) * r * scale.astype(np.float64)
+    got_out = ops.exl3_hadamard(halves(x, device), halves(scale, device), input_scale=False).float().cpu().numpy()
+    np.testing.assert_allclose(got_out, want_out, rtol=2e-3, atol=2e-3)
+    xf = g.standard_normal((rows, columns)).astype(np.float32)
+    got_f = ops.exl3_hadamard(dev(xf, device), halves(scale, device), input_scale=False).cpu().numpy()
+    np.testing.assert_allclose(got_f, hadamard_rows(xf) * r * scale.astype(np.float64), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 16])
+@pytest.mark.parametrize("bits,codebook", [(4, ops.EXL3_3INST), (4, ops.EXL3_MCG), (3, ops.EXL3_3INST), (6, ops.EXL3_MCG),
+                                           (8, ops.EXL3_MUL1)])
+def test_linear_matches_oracle(device, m, bits, codebook):
+    k, n = 1024, 512
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 21 + bits)
+    x = synth.rng(22 + m).standard_normal((m, k)).astype(np.float16)
+    keep = {}
+    got = ops.exl3_linear(dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook,
+                          halves(x, device), keep=keep).cpu().numpy()
+    # Stage one: the transformed input, F16. The device sums in F32, the oracle in F64, so a value
+    # may round to the neighbouring F16 (rarely); nothing moves further.
+    a_had = keep["a_had"].cpu().numpy().view(np.uint16)
+    want_had = oracle.exl3_input(suh.view(np.uint16), k, x.view(np.uint16))
+    ulps = np.abs(a_had.view(np.int16).astype(np.int32) - want_had.view(np.int16).astype(np.int32))
+    assert ulps.max() <= 1 and np.count_nonzero(ulps) <= 0.01 * ulps.size
+    # Stage two over identical transformed inputs: accumulation order only, 1e-3.
+    want = oracle.exl3_product(trellis, svh.view(np.uint16), k, n, bits, codebook, a_had, threads=oracle.max_threads())
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst
+    # And the reference's own bound against the F64 product with the decoded rows
+    # (tests/unit/exl3_trellis_test.cc:519-564): relative RMS 2^-8 a row.
+    rows = oracle.exl3_rows(trellis, suh.view(np.uint16), svh.view(np.uint16), k, n, bits, codebook).astype(np.float64)
+    ref = x.astype(np.float64) @ rows.T
+    for r in range(m):
+        assert np.sqrt(np.mean((got[r] - ref[r]) ** 2)) <= 2.0 ** -8 * np.sqrt(np.mean(ref[r] ** 2))
+
+
+def test_linear_rows_are_independent_and_f16_output_rounds_once(device):
+    k, n, bits, codebook = 512, 256, 4, ops.EXL3_3INST
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 31)
+    x = synth.rng(32).standard_normal((16, k)).astype(np.float16)
+    args = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    full = ops.exl3_linear(*args, halves(x, device)).cpu().numpy()
+    solo = ops.exl3_linear(*args, halves(x[3:4], device)).cpu().numpy()
+    assert np.array_equal(solo[0].view(np.uint32), full[3].view(np.uint32))
+    half = ops.exl3_linear(*args, halves(x, device), f32=False).cpu().numpy()
+    assert np.array_equal(half.view(np.uint16), full.astype(np.float16).view(np.uint16))
+
+
+def test_refusals(device):
+    trellis, suh, svh = synth.exl3_weights(128, 128, 4, 41)
+    x = halves(np.zeros((17, 128), dtype=np.float16), device)
+    with pytest.raises(ops.KernelFailure) as e:
+        ops.exl3_linear(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 4, 0, x)
+    assert e.value.rejected
+    with pytest.raises(ops.KernelFailure):
+        ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 9, 0)
+    with pytest.raises(ops.KernelFailure):
+        ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 4, 0, column=8,
+                             columns=16)
