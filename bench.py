@@ -49,6 +49,115 @@ def cpu_baseline(gate, up, x, budget_s=12.0):
                       f"{elapsed:.1f} s"}
 
 
+def event_us(body, count, warm=5):
+    """Microseconds a call of body(i), by HIP events on the launching stream."""
+    import torch
+    for i in range(warm):
+        body(i)
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for i in range(count):
+        body(warm + i)
+    end.record()
+    torch.cuda.synchronize()
+    return begin.elapsed_time(end) / count * 1e3
+
+
+def other_configs(device, args):
+    """Short measurements of the other benchmark configurations (not the headline line): each
+    over distinct weight copies where the weights are what is streamed."""
+    import numpy as np
+    import torch
+
+    from llmp_amd import ops, synth
+
+    out = {}
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+    # Config 1: Q8_0 mat-vec 4096 x 4096, one F32 token through llmp.q8_1.
+    n = k = 4096
+    w = dev(synth.q8_0_weights(n, k, 201))
+    copies = [w] + [w.clone() for _ in range(-(-ROTATE_BYTES // w.numel()) - 1)]
+    x = dev(synth.activations(1, k, 202))
+    q8 = ops.quantize_q8_1(x)
+    y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
+    us = event_us(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 200)
+    bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
+    out["q8_0_matvec_4096x4096_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
+                                       "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del copies, w
+
+    # Config 2 at batch 4 and 8.
+    gate, up = dev(synth.q4_k_weights(N, K, 101)), dev(synth.q4_k_weights(N, K, 102))
+    count = -(-ROTATE_BYTES // WEIGHT_BYTES)
+    gates = [gate] + [gate.clone() for _ in range(count - 1)]
+    ups = [up] + [up.clone() for _ in range(count - 1)]
+    for tokens in (4, 8):
+        q8 = ops.quantize_q8_1(dev(synth.activations(tokens, K, 203)))
+        y = torch.empty((tokens, 1, N), dtype=torch.float32, device=device)
+        us = event_us(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
+                                         glu=ops.GLU_GEGLU, out=y), 100)
+        out[f"q4_k_gate_up_geglu_b{tokens}"] = {"us": round(us, 2),
+                                                "GB/s": round(algorithmic_bytes(tokens) / us / 1e3, 1)}
+    del gates, ups, gate, up
+    torch.cuda.empty_cache()
+
+    # Config 3: MXFP8 GEMM 2048 x 12288 x 4096, bf16 out, and its activation quantizer.
+    m, n, k = 2048, 12288, 4096
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn((m, k), generator=g).to(device).to(torch.bfloat16)
+    wt = (torch.randn((n, k), generator=g) * 0.02).to(device)
+    ac, asc = ops.mxfp8_quantize(a)
+    wc, wsc = ops.mxfp8_quantize(wt)
+    d = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    us = event_us(lambda i: ops.mxfp8_gemm(ac, asc, wc, wsc, out=d), 30)
+    flops = 2.0 * m * n * k
+    out["mxfp8_gemm_2048x12288x4096"] = {"us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
+                                         "frac_dense_fp8_mfma_peak": round(flops / us / 1e6 / 5033.0, 4)}
+    out["mxfp8_quantize_2048x4096_bf16"] = {"us": round(event_us(lambda i: ops.mxfp8_quantize(a), 30), 1)}
+    del a, wt, ac, asc, wc, wsc, d
+    torch.cuda.empty_cache()
+
+    # Config 4: routed-expert FFN layer, 128 experts top-8, hidden 2048, FFN 768, Q4_K.
+    hidden, ffn, experts, used = 2048, 768, 128, 8
+    gate_up = dev(synth.q4_k_weights(experts * 2 * ffn, hidden, 204).reshape(experts, -1))
+    down = dev(synth.q4_k_weights(experts * hidden, ffn, 205).reshape(experts, -1))
+    expert_bytes = gate_up.numel() // experts + down.numel() // experts
+    for tokens in (1, 16, 512):
+        logits = dev(synth.rng(206).standard_normal((tokens, experts), dtype=np.float32))
+        xs = dev(synth.activations(tokens, hidden, 207))
+        _, ids, _ = ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gate_up, down, hidden, ffn, experts, used)
+        distinct = int(torch.unique(ids).numel())
+        us = event_us(lambda i: ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gate_up, down, hidden, ffn, experts, used),
+                      20 if tokens == 512 else 50)
+        entry = {"us": round(us, 1), "distinct_experts": distinct,
+                 "GB/s_of_touched_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),
+                 "note": "whole layer: router, q8_1, gate/up+GLU, q8_1, down, combine; weights not rotated"}
+        if tokens == 512:
+            entry["TFLOP/s"] = round(tokens * used * 3 * 2.0 * hidden * ffn / us / 1e6, 2)
+        out[f"moe_q4_k_ffn_t{tokens}"] = entry
+    del gate_up, down
+    torch.cuda.empty_cache()
+
+    # Config 5: EXL3 linear 4096 x 14336 at 4 bits, 3INST codebook.
+    k, n, bits = 4096, 14336, 4
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 208)
+    t0 = dev(trellis)
+    trellises = [t0] + [t0.clone() for _ in range(-(-ROTATE_BYTES // t0.numel()) - 1)]
+    suh_d = dev(suh.view(np.int16)).view(torch.float16)
+    svh_d = dev(svh.view(np.int16)).view(torch.float16)
+    for m in (1, 16):
+        xs = dev(synth.rng(209).standard_normal((m, k)).astype(np.float16).view(np.int16)).view(torch.float16)
+        us = event_us(lambda i: ops.exl3_linear(trellises[i % len(trellises)], suh_d, svh_d, k, n, bits, ops.EXL3_3INST,
+                                                xs), 50)
+        bytes_ = t0.numel() + 2 * k + 2 * n + m * (k * 2 + n * 4)
+        out[f"exl3_linear_4096x14336_4bpw_m{m}"] = {"us": round(us, 1), "GB/s": round(bytes_ / us / 1e3, 1),
+                                                    "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                                    "note": "input transform, product, output transform"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -57,6 +166,9 @@ def main():
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations' short measurements")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain device copies of the weights' size (for scaling hardware counters)")
     ap.add_argument("--fused", action="store_true",
                     help="a step is one launch that quantizes the activations in the kernel, instead of "
                          "llmp.q8_1 followed by llmp.vecq over its Q8_1 blocks (the reference's two operations)")
@@ -124,6 +236,14 @@ def main():
         torch.cuda.synchronize()
         return begin.elapsed_time(end), (time.perf_counter() - t0) * 1e3
 
+    if args.calibrate_copy:
+        # A copy of known size: WEIGHT_BYTES read, WEIGHT_BYTES written.
+        whole = torch.cat([gates[0].view(-1), ups[0].view(-1)])
+        target = torch.empty_like(whole)
+        for _ in range(20):
+            target.copy_(whole)
+        torch.cuda.synchronize()
+        del whole, target
     step(0)
     torch.cuda.synchronize()
     timed_region(step, args.warmup, 0)
@@ -151,6 +271,10 @@ def main():
                      "algorithmic_bytes_per_launch": algorithmic_bytes(args.tokens),
                      "avg_launch_us": round(kernel_us, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
     }
+    if not args.no_extras:
+        del gates, ups
+        torch.cuda.empty_cache()
+        line["other_configs"] = other_configs(device, args)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(gate, up, x)
     print(json.dumps(line))
