@@ -158,6 +158,19 @@ def other_configs(device, args):
     return out
 
 
+# HBM bytes per launch of the dominant kernel at batch 1 through the default variant, from two
+# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,476.2 KiB and WRITE_SIZE 60.1 KiB per dispatch,
+# scaled by 1.9988 and 1.0: what the same counters read for --calibrate-copy's copy of 64,800 KiB).
+# Counters cannot be read from inside a run, so other shapes and variants report null.
+PROFILED_TRAFFIC_BYTES = int(round((32476.2 * 1.9988 + 60.1) * 1024))
+
+
+def measured_traffic(args):
+    if args.tokens == 1 and args.variant == -1 and not args.fused:
+        return PROFILED_TRAFFIC_BYTES
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -266,7 +279,7 @@ def main():
                    "weight_copies_rotated": copies, "variant": args.variant, "launch": "eager" if args.eager else "hip graph",
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(args),
                      "kernel": "VecQFlatQ4K (llmp.vecq, Q4_K, GLU)",
                      "algorithmic_bytes_per_launch": algorithmic_bytes(args.tokens),
                      "avg_launch_us": round(kernel_us, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
