@@ -169,11 +169,15 @@ typedef float V4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* LdsPointer;
 typedef const __attribute__((address_space(1))) void* GlobalPointer;
 
-constexpr int kTile = 128;              // rows of either operand a workgroup
+constexpr int kTileM = 256;             // activation rows a workgroup
 constexpr int kStepK = 128;             // codes a K step
-constexpr int kOperandBytes = kTile * kStepK;  // 16 KB
-constexpr int kStageBytes = 2 * kOperandBytes;
-constexpr int kGemmThreads = 256;
+constexpr int kGemmThreads = 512;       // 8 waves: 4 along m, 2 along n
+constexpr int kGroupThreads = 256;      // a group: the four waves with the same position along n
+constexpr int kRingA = 2;               // stages of activation tiles in LDS
+constexpr int kRingB = 3;               // stages of weight tiles
+constexpr int kTileABytes = kTileM * kStepK;  // 32 KB
+constexpr int kLoadsA = kTileABytes / 16 / kGroupThreads;  // 8 a thread of group 1 a stage
+constexpr int kScaleStageBytes = 1024;  // two atoms a stage, either operand
 
 struct GemmArgs {
   const uint8_t* a;         // activations, m rows of k codes
@@ -186,111 +190,235 @@ struct GemmArgs {
   int tiles_m, tiles_n;
 };
 
-// Queues one operand's 128 x 128-byte tile of K step `step` into LDS at `to`: position
-// P = 256 i + thread holds row P / 8's chunk (P % 8) ^ ((row / 2) % 8).
-__device__ __forceinline__ void FetchOperand(const uint8_t* matrix, int row0, int rows, int k, int step, uint8_t* to,
-                                             int tid, int wave) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int p = i * kGemmThreads + tid;
-    const int row = p >> 3;
-    const int chunk = (p & 7) ^ ((row >> 1) & 7);
-    const int source = min(row0 + row, rows - 1);  // rows past the end repeat the last (never stored)
-    const uint8_t* from = matrix + static_cast<int64_t>(source) * k + step * kStepK + chunk * 16;
-    __builtin_amdgcn_global_load_lds((GlobalPointer)from, (LdsPointer)(to + (i * kGemmThreads + wave * 64) * 16), 16, 0,
-                                     0);
-  }
-}
+// LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
+template <int WN>
+struct GemmLds {
+  static constexpr int kTileN = 32 * WN;
+  static constexpr int kTileBBytes = kTileN * kStepK;
+  static constexpr int kA = 0;
+  static constexpr int kB = kA + kRingA * kTileABytes;
+  static constexpr int kAScales = kB + kRingB * kTileBBytes;
+  static constexpr int kBScales = kAScales + kRingA * kScaleStageBytes;
+  static constexpr int kBytes = kBScales + kRingB * kScaleStageBytes;
+};
 
-// Fragment f (16 rows) of an operand tile: lane (r, g) gets its row's chunks g and 4 + g.
-__device__ __forceinline__ V8i ReadFragment(const uint8_t* tile, int f, int r, int g) {
-  const int row = f * 16 + r;
-  const int key = (row >> 1) & 7;
-  const U32x4 lo = *reinterpret_cast<const U32x4*>(tile + (row * 8 + (g ^ key)) * 16);
-  const U32x4 hi = *reinterpret_cast<const U32x4*>(tile + (row * 8 + ((4 + g) ^ key)) * 16);
+// Position p of a ROWS x 128-byte tile in LDS holds row p / 8's 16-byte chunk
+// (p % 8) ^ ((row / 2) % 8). Rows past the operand's end repeat the last (their results are
+// never stored).
+
+// A 16-row fragment: the lane's two 16-byte chunks, at lo and hi bytes into it.
+__device__ __forceinline__ V8i ReadFragment(const uint8_t* fragment, int lo_at, int hi_at) {
+  const U32x4 lo = *reinterpret_cast<const U32x4*>(fragment + lo_at);
+  const U32x4 hi = *reinterpret_cast<const U32x4*>(fragment + hi_at);
   V8i v;
   v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
   v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
   return v;
 }
 
-__global__ __launch_bounds__(kGemmThreads, 2) void GemmKernel(const GemmArgs a) {
+// Waits until at most `left` of this wave's vector-memory operations are outstanding.
+template <int LEFT>
+__device__ __forceinline__ void AwaitLoads() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (LEFT & 15) | ((LEFT >> 4) << 14));
+}
+
+// D tile of 256 activation rows by 32 WN weight rows, K step 128. Wave (wm, wn) of 4 x 2 owns
+// 64 x 16 WN of it: WN x 4 MFMA tiles, the weights as the first operand.
+//
+// The two waves of a SIMD (wn 0 and 1: the hardware places waves 0-3 and 4-7 of a workgroup
+// one on each SIMD) work half a step apart. A step of a wave is a read phase (its 4 + WN
+// fragments and their scales from LDS into registers) and a multiply phase (4 WN MFMAs);
+// every phase ends at a workgroup barrier, and group 1 sits the first phase out, so that
+// while one wave of a SIMD multiplies the other reads: the matrix pipe and LDS both stay
+// busy. Phases, counted from 0: group 0 reads step s in phase 2 s and multiplies in 2 s + 1,
+// group 1 reads in 2 s + 1 and multiplies in 2 s + 2.
+//
+// Tiles come by global_load_lds, issued between the MFMAs of the multiply phases (the only
+// time a wave has issue slots to spare): group 1 brings activations s + 2 while it
+// multiplies step s, into the stage step s used (ring of 2; free since the barrier that ended
+// phase 2 s + 1), and waits for them at the end of its next read phase, before the barrier
+// that opens phase 2 s + 4. Group 0 brings weights s + 2 while it multiplies step s, into the
+// stage step s - 1 used (ring of 3: every weight byte is a compulsory HBM miss for the first
+// workgroup that asks, activations mostly hit L2), and waits for weights s + 1, leaving s + 2
+// in flight, before the barrier that ends its multiply phase.
+template <int WN>
+__global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) {
+  using L = GemmLds<WN>;
+  constexpr int kTileN = L::kTileN;
+  constexpr int kLoadsB = L::kTileBBytes / 16 / kGroupThreads;  // WN a thread of group 0 a stage
+  constexpr int kLoadEvery = WN / 2;  // MFMAs between two loads: 8 loads fit 4 WN MFMAs
+  static_assert(kLoadsB <= kLoadsA && kLoadsA * kLoadEvery <= 4 * WN, "the loads do not fit a multiply phase");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave & 1, wn = wave >> 1;
+  const int wm = wave & 3, wn = wave >> 2;
+  const int group = wn;
   const int r = lane & 15, g = lane >> 4;
 
   // Workgroups go round-robin to the eight XCDs, each with its own L2: give every XCD a
-  // contiguous run of tiles (walking M fastest, so a run shares weight tiles).
+  // contiguous run of tiles, walking m fastest, so the workgroups resident on an XCD share
+  // weight tiles (all m of a few n) and every activation tile.
   int tile = blockIdx.x;
   const int tiles = a.tiles_m * a.tiles_n;
   if (tiles % 8 == 0) tile = (tile % 8) * (tiles / 8) + tile / 8;
   const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
-  const int m0 = tm * kTile, n0 = tn * kTile;
+  const int m0 = tm * kTileM, n0 = tn * kTileN;
   const int steps = a.k / kStepK;
   const int blocks = a.k / 32;
 
-  V4f acc[4][4];
+  // What this thread brings: group 1 the activation tile, group 0 the weight tile; the
+  // group's first wave also the operand's scales, two atoms (128 rows by the step's four
+  // blocks each) a stage. An atom past the operand's padded rows repeats the last.
+  const int loads = group == 1 ? kLoadsA : kLoadsB;
+  const uint8_t* const matrix = group == 1 ? a.a : a.b;
+  // Its position p = 256 i + t of a tile is row 32 i + t / 8, and the chunk there is the same
+  // for every i (the swizzle key of 32 i + t / 8 is that of t / 8).
+  const int thread = tid & (kGroupThreads - 1);
+  const int row_first = (group == 1 ? m0 : n0) + (thread >> 3);
+  const int row_last = (group == 1 ? a.m : a.n) - 1;
+  const uint32_t chunk_from = static_cast<uint32_t>(((thread & 7) ^ ((thread >> 4) & 7)) * 16);
+  const int atom_b0 = n0 / 128;
+  const int atoms = ((group == 1 ? a.m : a.n) + 127) / 128;
+  const int atom_mine = min((group == 1 ? m0 / 128 : atom_b0) + (lane >> 5), atoms - 1);
+  const uint8_t* const from_scale = (group == 1 ? a.a_scales : a.b_scales) +
+                                    static_cast<int64_t>(atom_mine) * (blocks / 4) * 512 + (lane & 31) * 16;
+  const int tile_base = group == 1 ? L::kA : L::kB;
+  const int tile_bytes = group == 1 ? kTileABytes : L::kTileBBytes;
+  const int scale_base = group == 1 ? L::kAScales : L::kBScales;
+  // Load i of this wave of its operand's tile of K step `step` into ring stage `stage`.
+  auto load = [&](int i, int step, int stage) {
+    uint8_t* to = lds + tile_base + stage * tile_bytes + (i * kGroupThreads + wm * 64) * 16;
+    // Recomputed at every use: eight 64-bit addresses kept across the steps would not fit the
+    // register file beside the accumulators and fragments.
+    int row = row_first;
+    asm volatile("" : "+v"(row));
+    const uint32_t from = static_cast<uint32_t>(min(row + 32 * i, row_last)) * static_cast<uint32_t>(a.k) + chunk_from;
+    __builtin_amdgcn_global_load_lds((GlobalPointer)(matrix + step * kStepK + from), (LdsPointer)to, 16, 0, 0);
+  };
+  auto load_scales = [&](int step, int stage) {
+    if (wm == 0) {
+      __builtin_amdgcn_global_load_lds((GlobalPointer)(from_scale + step * 512),
+                                       (LdsPointer)(lds + scale_base + stage * kScaleStageBytes), 16, 0, 0);
+    }
+  };
+
+  // Where a lane's scale bytes sit in a scale stage. Row 16 q + r of an operand has its four
+  // scales at atom q / 8, byte (q % 2) 256 + r 16 + (q % 8) / 2 * 4: a part per 16 rows that
+  // is the same for every lane, plus 16 r + g.
+  auto scale_at = [](int q, int atom0) { return (q / 8 - atom0) * 512 + (q % 2) * 256 + (q % 8) / 2 * 4; };
+  const int scale_lane = r * 16 + g;
+  int scale_x[4], scale_w[WN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int j = 0; j < 4; ++j) scale_x[j] = scale_at(wm * 4 + j, 0);
+#pragma unroll
+  for (int i = 0; i < WN; ++i) scale_w[i] = scale_at(n0 / 16 + wn * WN + i, atom_b0);
+
+  // Lane (r, g) wants its row's chunks g and 4 + g; a fragment's rows are 16 f + r, whose
+  // swizzle key is r's.
+  const int chunk_lo = (r * 8 + (g ^ ((r >> 1) & 7))) * 16;
+  const int chunk_hi = (r * 8 + ((4 + g) ^ ((r >> 1) & 7))) * 16;
+
+  V4f acc[WN][4];
+#pragma unroll
+  for (int i = 0; i < WN; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
+  V8i xf[4], wf[WN];
+  int xscale[4], wscale[WN];
 
-  // A row's four scales of a K step are one dword of the atoms; the lane wants byte g.
-  const int64_t scale_step = 512;  // bytes between a tile's atoms of consecutive K steps
-  const uint8_t* ws[4];
-  const uint8_t* xs[4];
+  // Step s's fragments and scales into registers. Fragment f of a tile is 2 KB further on for
+  // every lane; a lane's scale is one byte.
+  auto read = [&](int stage_a, int stage_b) {
+    const uint8_t* tile_a = lds + L::kA + stage_a * kTileABytes + wm * 4 * 2048;
+    const uint8_t* tile_b = lds + L::kB + stage_b * L::kTileBBytes + wn * WN * 2048;
+    const uint8_t* scales_a = lds + L::kAScales + stage_a * kScaleStageBytes + scale_lane;
+    const uint8_t* scales_b = lds + L::kBScales + stage_b * kScaleStageBytes + scale_lane;
 #pragma unroll
-  for (int f = 0; f < 4; ++f) {
-    ws[f] = a.b_scales + AtomOffset(n0 + wn * 64 + f * 16 + r, 0, blocks);
-    xs[f] = a.a_scales + AtomOffset(m0 + wm * 64 + f * 16 + r, 0, blocks);
-  }
-
-  FetchOperand(a.b, n0, a.n, a.k, 0, lds, tid, wave);
-  FetchOperand(a.a, m0, a.m, a.k, 0, lds + kOperandBytes, tid, wave);
-  for (int step = 0; step < steps; ++step) {
-    uint8_t* now = lds + (step & 1) * kStageBytes;
-    uint8_t* next = lds + ((step + 1) & 1) * kStageBytes;
-    uint32_t wscale[4], xscale[4];
+    for (int j = 0; j < 4; ++j) xscale[j] = scales_a[scale_x[j]];
 #pragma unroll
-    for (int f = 0; f < 4; ++f) {
-      wscale[f] = *reinterpret_cast<const uint32_t*>(ws[f] + step * scale_step) >> (8 * g);
-      xscale[f] = *reinterpret_cast<const uint32_t*>(xs[f] + step * scale_step) >> (8 * g);
-    }
-    if (step + 1 < steps) {
-      FetchOperand(a.b, n0, a.n, a.k, step + 1, next, tid, wave);
-      FetchOperand(a.a, m0, a.m, a.k, step + 1, next + kOperandBytes, tid, wave);
-      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): all but the next step's loads
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-    }
-    __syncthreads();  // every wave's part of this step has landed
-    V8i wf[4];
+    for (int i = 0; i < WN; ++i) wscale[i] = scales_b[scale_w[i]];
 #pragma unroll
-    for (int f = 0; f < 4; ++f) wf[f] = ReadFragment(now, wn * 4 + f, r, g);
+    for (int j = 0; j < 4; ++j) xf[j] = ReadFragment(tile_a + j * 2048, chunk_lo, chunk_hi);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const V8i xf = ReadFragment(now + kOperandBytes, wm * 4 + j, r, g);
+    for (int i = 0; i < WN; ++i) wf[i] = ReadFragment(tile_b + i * 2048, chunk_lo, chunk_hi);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): in registers before the barrier that lets the stage go
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // The 4 WN MFMAs of a step, with this wave's loads of K step `step` into ring stage `stage`
+  // between them. Past the last step the last is asked for again, into a stage nobody reads
+  // any more: no branch on it, and the loads a wave has in flight stay the same number.
+  auto multiply = [&](int step, int stage) {
+    const int bring = min(step, steps - 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf, acc[i][j], 0, 0, 0,
-                                                                      static_cast<int>(wscale[i]), 0,
-                                                                      static_cast<int>(xscale[j]));
+    for (int i = 0; i < WN; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], acc[i][j], 0, 0, 0, wscale[i], 0, xscale[j]);
+        // Pins the MFMA here in program order (the compiler would otherwise sink all of them
+        // below the loads, which have side effects and so keep their place).
+        asm volatile("" : "+v"(acc[i][j]));
+        const int t = i * 4 + j;
+        if (t % kLoadEvery == kLoadEvery - 1 && t / kLoadEvery < kLoadsA) {
+          if (t / kLoadEvery < loads) load(t / kLoadEvery, bring, stage);
+        }
       }
     }
-    __syncthreads();  // this step's buffer may be refilled
-  }
+    load_scales(bring, stage);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-  // acc[i][j][q] = D[m0 + wm 64 + 16 j + r][n0 + wn 64 + 16 i + 4 g + q]
+  // Before the first phase: activations 0 and 1, weights 0 and 1.
+#pragma unroll
+  for (int i = 0; i < kLoadsA; ++i)
+    if (i < loads) load(i, 0, 0);
+  load_scales(0, 0);
+  if (steps > 1) {
+#pragma unroll
+    for (int i = 0; i < kLoadsA; ++i)
+      if (i < loads) load(i, 1, 1);
+    load_scales(1, 1);
+  }
+  AwaitLoads<0>();
+  barrier();
+  if (group == 1) barrier();
+  int stage_b = 0;  // step s's weight stage, s % 3
+  for (int step = 0; step < steps; ++step) {
+    read(step & 1, stage_b);
+    // Group 1: activations step + 1, asked for while multiplying step - 1, have landed.
+    if (group == 1) AwaitLoads<0>();
+    barrier();
+    int to = stage_b + 2;  // (step + 2) % 3
+    if (to >= kRingB) to -= kRingB;
+    multiply(step + 2, group == 1 ? (step & 1) : to);
+    // Group 0: weights step + 1 have landed; step + 2, just asked for, may stay in flight.
+    if (group == 0) {
+      if (wm == 0) {
+        AwaitLoads<kLoadsB + 1>();
+      } else {
+        AwaitLoads<kLoadsB>();
+      }
+    }
+    barrier();
+    if (++stage_b == kRingB) stage_b = 0;
+  }
+  if (group == 0) barrier();
+  AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
+
+  // acc[i][j][q] = D[m0 + wm 64 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int m = m0 + wm * 64 + j * 16 + r;
     if (m >= a.m) continue;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = n0 + wn * 64 + i * 16 + 4 * g;
+    for (int i = 0; i < WN; ++i) {
+      const int n = n0 + wn * 16 * WN + i * 16 + 4 * g;
       if (n >= a.n) continue;  // n is a multiple of 4 (checked on the host)
       const V4f v = acc[i][j];
       if (a.bf16) {
@@ -304,6 +432,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void GemmKernel(const GemmArgs a) 
       }
     }
   }
+}
+
+template <int WN>
+int LaunchGemm(GemmArgs a, hipStream_t stream) {
+  using L = GemmLds<WN>;
+  static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
+  a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
+  static bool sized = false;
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&GemmKernel<WN>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              L::kBytes);
+    sized = true;
+  }
+  hipLaunchKernelGGL((GemmKernel<WN>), dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), L::kBytes,
+                     stream, a);
+  return LaunchStatus("mxfp8.gemm");
 }
 
 }  // namespace
@@ -377,7 +521,6 @@ extern "C" size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int c
 }
 
 extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream) {
-  (void)compute_units;
   if (gemm == nullptr) return Refuse(1, "mxfp8.gemm: null descriptor");
   if (gemm->a == nullptr || gemm->a_scales == nullptr || gemm->b == nullptr || gemm->b_scales == nullptr ||
       gemm->d == nullptr)
@@ -388,6 +531,8 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
   const uintptr_t align = reinterpret_cast<uintptr_t>(gemm->a) | reinterpret_cast<uintptr_t>(gemm->b) |
                           reinterpret_cast<uintptr_t>(gemm->d);
   if (align % 16 != 0) return Refuse(1, "mxfp8.gemm: codes or output not 16-byte aligned");
+  if (static_cast<int64_t>(gemm->m) * gemm->k >= (int64_t{1} << 32) || static_cast<int64_t>(gemm->n) * gemm->k >= (int64_t{1} << 32))
+    return Refuse(1, "mxfp8.gemm: an operand of 4 GiB or more");
   if ((reinterpret_cast<uintptr_t>(gemm->a_scales) | reinterpret_cast<uintptr_t>(gemm->b_scales)) % 4 != 0)
     return Refuse(1, "mxfp8.gemm: scales not 4-byte aligned");
   GemmArgs a;
@@ -400,18 +545,20 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
   a.n = gemm->n;
   a.k = gemm->k;
   a.bf16 = gemm->bf16;
-  a.tiles_m = (gemm->m + kTile - 1) / kTile;
-  a.tiles_n = (gemm->n + kTile - 1) / kTile;
-  const int64_t tiles = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
-  if (tiles > (1 << 30)) return Refuse(1, "mxfp8.gemm: too many tiles");
-  static bool sized = false;
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&GemmKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              2 * kStageBytes);
-    sized = true;
+  a.tiles_m = (gemm->m + kTileM - 1) / kTileM;
+  a.tiles_n = 0;
+  // The weight rows a workgroup takes (192 or 128): whichever leaves the fewest idle
+  // compute units in the last round of workgroups, the larger on a tie.
+  const int cus = compute_units > 0 ? compute_units : 256;
+  int best = 0;
+  int64_t best_cost = 0;
+  for (const int tile_n : {192, 128}) {
+    const int64_t tiles = static_cast<int64_t>(a.tiles_m) * ((gemm->n + tile_n - 1) / tile_n);
+    if (tiles > (1 << 30)) return Refuse(1, "mxfp8.gemm: too many tiles");
+    const int64_t cost = (tiles + cus - 1) / cus * tile_n;
+    if (best == 0 || cost < best_cost) best = tile_n, best_cost = cost;
   }
-  hipLaunchKernelGGL(GemmKernel, dim3(static_cast<unsigned>(tiles)), dim3(kGemmThreads), 2 * kStageBytes,
-                     static_cast<hipStream_t>(stream), a);
-  const int status = LaunchStatus("mxfp8.gemm");
+  const hipStream_t on = static_cast<hipStream_t>(stream);
+  const int status = best == 192 ? LaunchGemm<6>(a, on) : LaunchGemm<4>(a, on);
   return status;  // negative: the launch failed after the checks (the caller's fault path)
 }
