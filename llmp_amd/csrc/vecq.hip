@@ -485,7 +485,8 @@ struct Variant {
 constexpr Variant kVariants[] = {
     {"lanes8 pass1 flight4", 8, 1, 4},   {"lanes8 pass2 flight3", 8, 2, 3},   {"lanes8 pass4 flight2", 8, 4, 2},
     {"lanes8 pass8 flight2", 8, 8, 2},   {"lanes16 pass1 flight4", 16, 1, 4}, {"lanes64 pass1 flight2", 64, 1, 2},
-    // Q4_K only: a lane a super-block (vecq_flat.hip); `lanes` 0 marks the form.
+    // A lane a whole unit of a row, a Q4_K super-block or four Q8_0 blocks (vecq_flat.hip);
+    // `lanes` 0 marks the form.
     {"flat pass1", 0, 1, 2},             {"flat pass4", 0, 4, 2},
 };
 constexpr int kFlatFirst = 6;
@@ -553,7 +554,7 @@ void LaunchVariant(const VecQArgs& a, int x_type, int variant, dim3 grid, size_t
 // streams the weights again), then enough lanes a row to fill the device.
 int DefaultVariant(int type, const llmp_vecq_desc& d, int kp) {
   const int tokens = d.tokens;
-  if (type == LLMP_TYPE_Q4_K && FlatQ4KTakes(d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
+  if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
   while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
   switch (pass) {
@@ -613,12 +614,14 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (variant < 0) variant = DefaultVariant(type, *d, a.kp);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
-  if (offsets != nullptr && v.lanes != 0) return Refuse(1, "vecq: sorted rows take the flat Q4_K form");
+  if (offsets != nullptr && v.lanes != 0) return Refuse(1, "vecq: sorted rows take the flat form");
   if (v.lanes == 0) {
-    if (type != LLMP_TYPE_Q4_K || !FlatQ4KTakes(*d)) return Refuse(1, "vecq: the flat form takes Q4_K rows up to 65536 values");
+    if (!FlatTakes(type, *d))
+      return Refuse(1, "vecq: the flat form takes Q4_K rows up to 16384 values (8192 with a GLU), and Q8_0 rows of whole "
+                       "256 values up to 8192 (4096) at 16-byte boundaries");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
       return Refuse(1, "vecq: block sums are of a dense one-token product");
-    LaunchFlatQ4K(a, x_type, v.pass, static_cast<hipStream_t>(stream));
+    LaunchFlat(type, a, x_type, v.pass, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }
   const size_t lds = LdsBytes(v.pass, a.kp);
@@ -677,7 +680,7 @@ extern "C" int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp
 
 extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums, void* stream) {
   if (sums == nullptr) return Refuse(1, "vecq: null sums");
-  if (variant < 0 && d != nullptr) variant = type == LLMP_TYPE_Q4_K && FlatQ4KTakes(*d) ? kFlatFirst : 0;
+  if (variant < 0 && d != nullptr) variant = FlatTakes(type, *d) ? kFlatFirst : 0;
   if (variant != 0 && variant != kFlatFirst) return Refuse(1, "vecq: block sums are of the one-token variants");
   return Launch(type, d, nullptr, variant, sums, stream);
 }
@@ -686,7 +689,7 @@ extern "C" int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int
                                     void* stream) {
   if (offsets == nullptr || d == nullptr) return Refuse(1, "vecq: null offsets");
   if (experts < 1 || experts > 65535) return Refuse(1, "vecq: 1 to 65535 experts");
-  if (type != LLMP_TYPE_Q4_K || !FlatQ4KTakes(*d)) return Refuse(1, "vecq: sorted rows take Q4_K weights the flat form takes");
+  if (!FlatTakes(type, *d)) return Refuse(1, "vecq: sorted rows take weights the flat form takes");
   llmp_vecq_desc sorted = *d;
   sorted.ids = nullptr;
   sorted.used = experts;  // a workgroup row an expert

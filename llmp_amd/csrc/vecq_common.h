@@ -170,9 +170,10 @@ __device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_in
   return expert;
 }
 
-// The flat Q4_K kernel's launch (vecq_flat.hip). x_type -1: Q8_1 activations.
-bool FlatQ4KTakes(const llmp_vecq_desc& d);
-void LaunchFlatQ4K(const VecQArgs& a, int x_type, int pass, hipStream_t stream);
+// The flat kernels' launch (vecq_flat.hip): whether a product's shape and alignment fit them,
+// and the launch. x_type -1: Q8_1 activations.
+bool FlatTakes(int type, const llmp_vecq_desc& d);
+void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, hipStream_t stream);
 
 }  // namespace llmp_hip
 

@@ -1,32 +1,42 @@
-// llmp.vecq over Q4_K weights, the form the default launches take: one lane owns
-// one whole 144-byte super-block; every wave streams its own tiles through LDS
-// with global-to-LDS loads and never waits for another wave.
+// llmp.vecq in the form the default launches take: one lane owns one whole unit of
+// a weight row (a 144-byte Q4_K super-block, or four Q8_0 blocks: 136 bytes); every
+// wave streams its own tiles through LDS with global-to-LDS loads and never waits
+// for another wave.
 //
 // A tile is R consecutive rows of the weights (of both matrices with a GLU), at
-// most 64 super-blocks: lane t of a wave owns super-block t of the tile's flat
-// list (the up rows' super-blocks, then the gate rows'). With packed rows a
-// matrix's part of the list is one contiguous byte range; the wave fetches the
-// list as 16-byte chunks with global_load_lds_dwordx4, chunk 64 j + lane by its
-// j-th load, which lands at 16 * (64 j + lane) of the wave's LDS buffer: every
-// cache line is requested once, by neighbouring lanes, and no register holds
-// weights in flight. After s_waitcnt vmcnt(0) each lane reads its own
-// super-block, nine 16-byte reads 144 bytes apart (36 dwords: sixteen lanes'
-// reads fall in distinct banks). A workgroup (8 wave64s, two a CU) stages its tokens'
-// activations once (quantizing them to Q8_1 itself in the fused form) while the
-// waves' first tiles are in flight; after that one barrier its waves are
-// independent: wave w of the grid takes tiles w, w + waves, .... Sixteen waves a
-// CU alternate between waiting for a tile and computing one, so a CU always has
-// tiles in flight.
+// most 64 units: lane t of a wave owns unit t of the tile's flat list (the up
+// rows' units, then the gate rows'). With packed rows a matrix's part of the list
+// is one contiguous byte range; the wave fetches the list as 16-byte chunks with
+// global_load_lds_dwordx4, chunk 64 j + lane by its j-th load, which lands at
+// 16 * (64 j + lane) of the wave's LDS buffer: every cache line is requested once,
+// by neighbouring lanes, and no register holds weights in flight. After s_waitcnt
+// vmcnt(0) each lane reads its own unit (Q4_K: nine 16-byte reads 144 bytes apart,
+// 36 dwords, so sixteen lanes' reads fall in distinct banks; Q8_0: seventeen 8-byte
+// reads 136 bytes apart, 34 dwords, likewise for thirty-two lanes). A workgroup
+// (8 wave64s, two a CU) stages its tokens' activations once (quantizing them to
+// Q8_1 itself in the fused form) while the waves' first tiles are in flight; after
+// that one barrier its waves are independent: wave w of the grid takes tiles w,
+// w + waves, .... Sixteen waves a CU alternate between waiting for a tile and
+// computing one, so a CU always has tiles in flight.
 //
-// Staged activations, per token and super-block, a record of 336 bytes (84
-// dwords, so that consecutive super-blocks start 20 banks apart and sixteen
-// lanes' 16-byte reads of the same field never share a bank):
+// Staged activations, Q4_K: per token and super-block a record of 336 bytes (84
+// dwords, so that consecutive super-blocks start 20 banks apart and sixteen lanes'
+// 16-byte reads of the same field never share a bank):
 //   [0, 256)    the 256 int8 codes;
 //   [256, 288)  the eight sub-blocks' scales d8 as floats;
 //   [288, 320)  d8 * sum(codes) of each sub-block as floats (the minimum term);
 //   [320, 336)  sum(codes) of each sub-block as int16 (read by the test dump).
 // A lane's super-block sum is d * sum_g sc_g * d8_g * prod_g - dmin * sum_g m_g *
 // d8_g * sum_g (tests/unit/dsv4_fast_test.cc:179-193), prod_g eight v_dot4_i32_i8.
+//
+// Staged activations, Q8_0: per token and unit a record of 152 bytes: an image of the
+// unit's 136 bytes with the activation codes where the weight codes are and zeros
+// where the four F16 scales are, then the four blocks' scales d8 as floats. A block's
+// 32 weight codes start two bytes into a dword in every other block; against the image
+// the 34 dwords of a unit multiply as they lie, v_dot4_i32_i8 by v_dot4_i32_i8 (the
+// scale bytes meet zeros), and dwords 0-8, 9-16, 17-25 and 26-33 are the four blocks'
+// sums (src/kernels/ggml/vecq.cu:398-418: sum w q times d times d8).
+//
 // Row sums: a suffix sum over the row's lanes by wave shuffles (a fixed tree), so
 // a (token, row) value never depends on its neighbours or on which wave
 // computed it.
@@ -40,18 +50,10 @@
 namespace llmp_hip {
 namespace {
 
-constexpr int kRecord = 336;     // bytes a staged super-block
 constexpr int kGroup = 512;      // threads a workgroup: eight waves, two workgroups a CU
 constexpr int kWaves = kGroup / kWave;
-constexpr int kRing = kWave * 9 * 16;  // bytes of a wave's tile buffer
-constexpr int kChunks = 9;       // 16-byte chunks a super-block
 
-struct SuperBlock {
-  U32x4 header;  // d, dmin, scales[12]
-  U32x4 codes[8];
-};
-
-// ---- staging into records
+// ---- the activations' first loads
 
 // Staging is split in two so that a row's first loads can be queued before the wave's first
 // tile: memory operations complete in order, and a load queued behind a tile would wait for it.
@@ -75,43 +77,6 @@ __device__ __forceinline__ FrontX LoadFrontX(const void* __restrict__ x, int k) 
   return f;
 }
 
-// One block of 32 values, eight lanes: its codes, scale and sums into the record.
-__device__ __forceinline__ void StageBlock(const float (&v)[4], int b, uint8_t* token) {
-  const int lane8 = threadIdx.x & 7;
-  const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
-  uint8_t* record = token + (b >> 3) * kRecord;
-  const int g = b & 7;
-  *reinterpret_cast<uint32_t*>(record + g * 32 + lane8 * 4) = q.codes;
-  int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
-  s += ShflXor(s, 1);
-  s += ShflXor(s, 2);
-  s += ShflXor(s, 4);
-  if (lane8 == 0) {
-    // The products read the scale as a Q8_1 block stores it: rounded to F16.
-    const float d8 = HalfBitsToFloat(FloatToHalfBits(q.d));
-    reinterpret_cast<float*>(record + 256)[g] = d8;
-    reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
-    reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
-  }
-}
-
-template <int XT>
-__device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k, const FrontX& front, uint8_t* token) {
-  const int lane8 = threadIdx.x & 7;
-  const int blocks = k / 32;
-  const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
-#pragma unroll
-  for (int i = 0; i < kFront; ++i) {
-    const int b = (threadIdx.x >> 3) + i * kStep;
-    if (b < blocks) StageBlock(front.v[i], b, token);  // whole 8-lane groups together
-  }
-  for (int b = (threadIdx.x >> 3) + kFront * kStep; b < blocks; b += kStep) {
-    float v[4];
-    Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v);
-    StageBlock(v, b, token);
-  }
-}
-
 struct FrontQ8 {
   uint32_t w[9];
 };
@@ -127,41 +92,74 @@ __device__ __forceinline__ FrontQ8 LoadFrontQ8(const uint8_t* __restrict__ y, in
   return f;
 }
 
-__device__ __forceinline__ void StageQ8Block(const uint32_t (&w)[9], int b, uint8_t* token) {
-  uint8_t* record = token + (b >> 3) * kRecord;
-  const int g = b & 7;
-  uint4* dst = reinterpret_cast<uint4*>(record + g * 32);
-  dst[0] = make_uint4(w[1], w[2], w[3], w[4]);
-  dst[1] = make_uint4(w[5], w[6], w[7], w[8]);
-  int s = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s = Dot4(0x01010101, static_cast<int>(w[1 + i]), s);
-  const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
-  reinterpret_cast<float*>(record + 256)[g] = d8;
-  reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
-  reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
-}
-
-__device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, const FrontQ8& front,
-                                               uint8_t* token) {
-  if (static_cast<int>(threadIdx.x) < blocks) StageQ8Block(front.w, threadIdx.x, token);
-  for (int b = threadIdx.x + kGroup; b < blocks; b += kGroup) {
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
-    uint32_t w[9];
-#pragma unroll
-    for (int i = 0; i < 9; ++i) w[i] = src[i];
-    StageQ8Block(w, b, token);
-  }
-}
-
-// ---- one super-block times the staged tokens
-
 __device__ __forceinline__ float ByteToFloat(uint32_t word, int byte) {
   return static_cast<float>((word >> (8 * byte)) & 0xFFu);  // v_cvt_f32_ubyteN
 }
 
+// ---- Q4_K: a unit is a super-block
+
+struct SuperBlock {
+  U32x4 header;  // d, dmin, scales[12]
+  U32x4 codes[8];
+};
+
+struct FormatQ4K {
+  static constexpr int kUnitBytes = 144;    // of weights a lane
+  static constexpr int kUnitValues = 256;
+  static constexpr int kBlockBytes = 144;   // the descriptor's strides count these
+  static constexpr int kBlockValues = 256;
+  static constexpr int kRecord = 336;       // bytes a staged unit of activations
+  static constexpr int kDumpInts = 16;      // block sums a unit
+  using Unit = SuperBlock;
+
+  static __device__ __forceinline__ Unit Read(const uint8_t* at) {
+    SuperBlock b;
+    const U32x4* mine = reinterpret_cast<const U32x4*>(at);
+    b.header = mine[0];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b.codes[i] = mine[1 + i];
+    return b;
+  }
+
+  // One block of 32 values, eight lanes: its codes, scale and sums into the record.
+  static __device__ __forceinline__ void StageX(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int g = b & 7;
+    *reinterpret_cast<uint32_t*>(record + g * 32 + lane8 * 4) = q.codes;
+    int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
+    s += ShflXor(s, 1);
+    s += ShflXor(s, 2);
+    s += ShflXor(s, 4);
+    if (lane8 == 0) {
+      // The products read the scale as a Q8_1 block stores it: rounded to F16.
+      const float d8 = HalfBitsToFloat(FloatToHalfBits(q.d));
+      reinterpret_cast<float*>(record + 256)[g] = d8;
+      reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
+      reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
+    }
+  }
+
+  // One Q8_1 block (nine dwords), one thread.
+  static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int g = b & 7;
+    uint4* dst = reinterpret_cast<uint4*>(record + g * 32);
+    dst[0] = make_uint4(w[1], w[2], w[3], w[4]);
+    dst[1] = make_uint4(w[5], w[6], w[7], w[8]);
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = Dot4(0x01010101, static_cast<int>(w[1 + i]), s);
+    const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
+    reinterpret_cast<float*>(record + 256)[g] = d8;
+    reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
+    reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
+  }
+
+  // One super-block times the staged tokens.
 template <int P, bool kDump>
-__device__ __forceinline__ void DotSuperBlock(const SuperBlock& b, const uint8_t* records, int token_stride, int m,
+  static __device__ __forceinline__ void Dot(const SuperBlock& b, const uint8_t* records, int token_stride, int m,
                                               float (&out)[P], int32_t* dump) {
 #pragma clang fp contract(off)
   const uint32_t s0 = b.header.y, s1 = b.header.z, s2 = b.header.w;
@@ -240,16 +238,153 @@ __device__ __forceinline__ void DotSuperBlock(const SuperBlock& b, const uint8_t
     }
   }
 }
+};
+
+// ---- Q8_0: a unit is four blocks
+
+struct FourBlocks {
+  uint32_t w[34];  // {f16 d; i8 qs[32]} x 4, as they lie
+};
+
+struct FormatQ8 {
+  static constexpr int kUnitBytes = 136;
+  static constexpr int kUnitValues = 128;
+  static constexpr int kBlockBytes = 34;
+  static constexpr int kBlockValues = 32;
+  static constexpr int kRecord = 152;
+  static constexpr int kDumpInts = 4;
+  using Unit = FourBlocks;
+
+  static __device__ __forceinline__ Unit Read(const uint8_t* at) {
+    FourBlocks u;
+    const uint2* mine = reinterpret_cast<const uint2*>(at);
+#pragma unroll
+    for (int i = 0; i < 17; ++i) {
+      const uint2 v = mine[i];
+      u.w[2 * i] = v.x;
+      u.w[2 * i + 1] = v.y;
+    }
+    return u;
+  }
+
+  // One block of 32 values, eight lanes: the lane's four codes go where the block's weight
+  // codes 4 lane .. 4 lane + 3 lie in the unit, two bytes into it.
+  static __device__ __forceinline__ void StageX(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    uint8_t* record = token + (b >> 2) * kRecord;
+    const int j = b & 3;
+    uint16_t* at = reinterpret_cast<uint16_t*>(record + 34 * j + 2 + lane8 * 4);
+    at[0] = static_cast<uint16_t>(q.codes & 0xFFFFu);
+    at[1] = static_cast<uint16_t>(q.codes >> 16);
+    if (lane8 == 0) {
+      *reinterpret_cast<uint16_t*>(record + 34 * j) = 0;  // against the weight block's scale
+      reinterpret_cast<float*>(record + 136)[j] = HalfBitsToFloat(FloatToHalfBits(q.d));
+    }
+  }
+
+  // One Q8_1 block (nine dwords), one thread. Blocks 1 and 3 of a unit have their codes on a
+  // dword boundary (dwords 9-16 and 26-33); blocks 0 and 2 two bytes into dwords 0 and 17,
+  // their nine dwords ending with the two bytes that face the next block's scale.
+  static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
+    uint8_t* record = token + (b >> 2) * kRecord;
+    const int j = b & 3;
+    uint32_t* image = reinterpret_cast<uint32_t*>(record);
+    if (j & 1) {
+      uint32_t* dst = image + (j == 1 ? 9 : 26);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i] = w[1 + i];
+    } else {
+      uint32_t* dst = image + (j == 0 ? 0 : 17);
+      dst[0] = w[1] << 16;
+#pragma unroll
+      for (int i = 1; i < 8; ++i) dst[i] = (w[i] >> 16) | (w[i + 1] << 16);
+      dst[8] = w[8] >> 16;
+    }
+    reinterpret_cast<float*>(record + 136)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+  }
+
+  // Four blocks times the staged tokens.
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void Dot(const Unit& u, const uint8_t* records, int token_stride, int m,
+                                             float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    const float dw0 = HalfBitsToFloat(u.w[0] & 0xFFFFu);
+    const float dw1 = HalfBitsToFloat(u.w[8] >> 16);
+    const float dw2 = HalfBitsToFloat(u.w[17] & 0xFFFFu);
+    const float dw3 = HalfBitsToFloat(u.w[25] >> 16);
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) {
+        const uint8_t* record = records + t * token_stride;
+        const uint2* image = reinterpret_cast<const uint2*>(record);
+        int s[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 17; ++i) {
+          const uint2 x = image[i];
+          constexpr int kOwner[34] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1, 1, 1, 1, 1,
+                                      2, 2, 2, 2, 2, 2, 2, 2, 2, 3, 3, 3, 3, 3, 3, 3, 3};
+          s[kOwner[2 * i]] = Dot4(static_cast<int>(u.w[2 * i]), static_cast<int>(x.x), s[kOwner[2 * i]]);
+          s[kOwner[2 * i + 1]] = Dot4(static_cast<int>(u.w[2 * i + 1]), static_cast<int>(x.y), s[kOwner[2 * i + 1]]);
+        }
+        const float2 da = *reinterpret_cast<const float2*>(record + 136);
+        const float2 db = *reinterpret_cast<const float2*>(record + 144);
+        if (kDump && dump != nullptr) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dump[j] = s[j];
+        }
+        float v = static_cast<float>(s[0]) * (dw0 * da.x);
+        v = fmaf(static_cast<float>(s[1]), dw1 * da.y, v);
+        v = fmaf(static_cast<float>(s[2]), dw2 * db.x, v);
+        v = fmaf(static_cast<float>(s[3]), dw3 * db.y, v);
+        out[t] = v;
+      }
+    }
+  }
+};
+
+// ---- staging a token's row into records
+
+template <class F, int XT>
+__device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k, const FrontX& front, uint8_t* token) {
+  const int lane8 = threadIdx.x & 7;
+  const int blocks = k / 32;
+  const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
+#pragma unroll
+  for (int i = 0; i < kFront; ++i) {
+    const int b = (threadIdx.x >> 3) + i * kStep;
+    if (b < blocks) F::StageX(front.v[i], b, token);  // whole 8-lane groups together
+  }
+  for (int b = (threadIdx.x >> 3) + kFront * kStep; b < blocks; b += kStep) {
+    float v[4];
+    Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v);
+    F::StageX(v, b, token);
+  }
+}
+
+template <class F>
+__device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, const FrontQ8& front,
+                                               uint8_t* token) {
+  if (static_cast<int>(threadIdx.x) < blocks) F::StageQ8(front.w, threadIdx.x, token);
+  for (int b = threadIdx.x + kGroup; b < blocks; b += kGroup) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+    F::StageQ8(w, b, token);
+  }
+}
 
 typedef __attribute__((address_space(3))) void* LdsPointer;
 typedef const __attribute__((address_space(1))) void* GlobalPointer;
 
 // Queues one matrix's part of a tile into the wave's buffer at `ring`: chunk c = 64 j + lane
 // of `chunks` lands at byte 16 c. `base` and `ring` are the same in every lane.
-// kPacked: rows follow each other without a gap, so the part is one byte range.
+// kPacked: rows follow each other without a gap, so the part is one byte range; else a row's
+// bytes (a whole number of chunks) are `row_bytes` of every `stride_bytes`.
 template <int kLoads, bool kPacked>
-__device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int stride_row, int nsb, uint8_t* ring,
-                                          int lane) {
+__device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int64_t stride_bytes, int row_bytes,
+                                          uint8_t* ring, int lane) {
 #pragma unroll
   for (int j = 0; j < kLoads; ++j) {
     const int c = j * kWave + lane;
@@ -258,9 +393,9 @@ __device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int s
       if constexpr (kPacked) {
         from = base + static_cast<uint32_t>(c) * 16u;
       } else {
-        const int f = c / kChunks;
-        const int row = f / nsb;
-        from = base + (static_cast<int64_t>(row) * stride_row + (f - row * nsb)) * 144 + (c - f * kChunks) * 16;
+        const int byte = c * 16;
+        const int row = byte / row_bytes;
+        from = base + row * stride_bytes + (byte - row * row_bytes);
       }
       __builtin_amdgcn_global_load_lds((GlobalPointer)from, (LdsPointer)(ring + j * kWave * 16), 16, 0, 0);
     }
@@ -269,17 +404,20 @@ __device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int s
 
 // The tile of `rows` rows from `row0`. A matrix's part always starts where a full tile's
 // would (`gate_at` bytes into the buffer), so a lane's place in a tile never changes.
-template <bool kGlu, bool kPacked>
-__device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t expert_block, int row0, int rows, int nsb,
+template <class F, bool kGlu, bool kPacked>
+__device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t expert_block, int row0, int rows, int units,
                                           int gate_at, uint8_t* ring, int lane) {
-  const int64_t first = (expert_block + static_cast<int64_t>(row0) * d.stride_row) * 144;
-  const int chunks = rows * nsb * kChunks;
+  const int64_t first = (expert_block + static_cast<int64_t>(row0) * d.stride_row) * F::kBlockBytes;
+  const int row_bytes = units * F::kUnitBytes;
+  const int chunks = rows * row_bytes / 16;
+  const int64_t stride_bytes = static_cast<int64_t>(d.stride_row) * F::kBlockBytes;
   if constexpr (kGlu) {
-    // Each matrix at most 32 super-blocks: 288 chunks, five loads.
-    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, d.stride_row, nsb, ring, lane);
-    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.g) + first, chunks, d.stride_row, nsb, ring + gate_at, lane);
+    // Each matrix at most 32 units: 288 chunks or fewer, five loads.
+    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
+    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.g) + first, chunks, stride_bytes, row_bytes, ring + gate_at,
+                          lane);
   } else {
-    FetchPart<kChunks, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, d.stride_row, nsb, ring, lane);
+    FetchPart<9, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
   }
 }
 
@@ -290,18 +428,9 @@ __device__ __forceinline__ void AwaitTile() {
   asm volatile("" ::: "memory");
 }
 
-__device__ __forceinline__ SuperBlock ReadSuperBlock(const uint8_t* at) {
-  SuperBlock b;
-  const U32x4* mine = reinterpret_cast<const U32x4*>(at);
-  b.header = mine[0];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) b.codes[i] = mine[1 + i];
-  return b;
-}
-
 // grid (workgroups, slots); LDS: P tokens' records, then a tile buffer a wave.
-template <int P, bool kGlu, int XT, bool kDump, bool kPacked>
-__global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const int rows_per_tile) {
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked>
+__global__ __launch_bounds__(kGroup, 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
@@ -310,21 +439,21 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int nsb = d.ncols_x / 256;
-  const int token_stride = nsb * kRecord;
+  const int nsb = d.ncols_x / F::kUnitValues;  // units a row
+  const int token_stride = nsb * F::kRecord;
   const int tiles = (d.nrows + rows_per_tile - 1) / rows_per_tile;
-  uint8_t* ring = lds + P * token_stride + wave * kRing;
+  uint8_t* ring = lds + P * token_stride + wave * (kWave * F::kUnitBytes);
 
-  // A lane's place in every tile: its matrix, row and super-block.
+  // A lane's place in every tile: its matrix, row and unit of the row.
   const int half = rows_per_tile * nsb;
   const bool gate_lane = kGlu && lane >= half;
   const int f = gate_lane ? lane - half : lane;
   const int row = f / nsb;
   const int sb = f - row * nsb;
   const bool placed = lane < (kGlu ? 2 * half : half);
-  const int gate_at = half * 144;
-  const uint8_t* my_block = ring + lane * 144;
-  const uint8_t* my_records = lds + sb * kRecord;
+  const int gate_at = half * F::kUnitBytes;
+  const uint8_t* my_block = ring + lane * F::kUnitBytes;
+  const uint8_t* my_records = lds + sb * F::kRecord;
 
   // A routed product's workgroup first learns whether it owns its expert; one over sorted
   // rows takes its expert's row range.
@@ -373,16 +502,16 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
     int index = first_tile;
     if (index < tiles) {
       const int row0 = index * rows_per_tile;
-      FetchTile<kGlu, kPacked>(d, expert_block, row0, min(rows_per_tile, d.nrows - row0), nsb, gate_at, ring, lane);
+      FetchTile<F, kGlu, kPacked>(d, expert_block, row0, min(rows_per_tile, d.nrows - row0), nsb, gate_at, ring, lane);
     }
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
         uint8_t* records = lds + j * token_stride;
         if constexpr (XT < 0) {
-          StageRecordsQ8(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_q[j], records);
+          StageRecordsQ8<F>(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_q[j], records);
         } else {
-          StageRecordsX<XT>(rows_x[j], d.ncols_x, front_x[j], records);
+          StageRecordsX<F, XT>(rows_x[j], d.ncols_x, front_x[j], records);
         }
       }
     }
@@ -394,9 +523,9 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
       AwaitTile();
       float out[P];
       if (live) {
-        const SuperBlock block = ReadSuperBlock(my_block);
-        int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * 16 : nullptr;
-        DotSuperBlock<P, kDump>(block, my_records, token_stride, m, out, dump);
+        const typename F::Unit unit = F::Read(my_block);
+        int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * F::kDumpInts : nullptr;
+        F::template Dot<P, kDump>(unit, my_records, token_stride, m, out, dump);
       }
       // Row sums: a suffix sum over each row's lanes (a fixed tree), the total in the row's
       // first lane; a gate row's total then moves to its up row's lane.
@@ -423,7 +552,7 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatQ4K(const VecQArgs a, const
       index += tile_step;
       if (index < tiles) {
         const int next0 = index * rows_per_tile;
-        FetchTile<kGlu, kPacked>(d, expert_block, next0, min(rows_per_tile, d.nrows - next0), nsb, gate_at, ring,
+        FetchTile<F, kGlu, kPacked>(d, expert_block, next0, min(rows_per_tile, d.nrows - next0), nsb, gate_at, ring,
                                  lane);
       }
     }
@@ -436,75 +565,70 @@ struct FlatPlan {
   size_t lds;
 };
 
-FlatPlan PlanFlat(int pass, int nsb, bool glu) {
+template <class F>
+FlatPlan PlanFlat(int pass, int units, bool glu) {
   FlatPlan p;
-  p.rows = (glu ? kWave / 2 : kWave) / nsb;
-  p.lds = static_cast<size_t>(pass) * nsb * kRecord + static_cast<size_t>(kWaves) * kRing;
+  p.rows = (glu ? kWave / 2 : kWave) / units;
+  p.lds = static_cast<size_t>(pass) * units * F::kRecord + static_cast<size_t>(kWaves) * kWave * F::kUnitBytes;
   return p;
 }
 
 constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
 int g_compute_units = 0;
 
-template <int P, bool kGlu, int XT, bool kDump, bool kPacked>
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlatQ4K<P, kGlu, XT, kDump, kPacked>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kFlatLdsLimit));
     sized = true;
   }
-  hipLaunchKernelGGL((VecQFlatQ4K<P, kGlu, XT, kDump, kPacked>), grid, dim3(kGroup), plan.lds, stream, a, plan.rows);
+  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked>), grid, dim3(kGroup), plan.lds, stream, a, plan.rows);
 }
 
-template <int P, bool kGlu, int XT>
+template <class F, int P, bool kGlu, int XT>
 void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
-  const bool packed = a.d.stride_row == a.d.ncols_x / 256;
+  const bool packed = a.d.stride_row == a.d.ncols_x / F::kBlockValues;
   if (a.dump != nullptr) {
-    if constexpr (P == 1 && !kGlu && XT < 0) LaunchK<P, kGlu, XT, true, false>(a, grid, plan, stream);
+    if constexpr (P == 1 && !kGlu && XT < 0) LaunchK<F, P, kGlu, XT, true, false>(a, grid, plan, stream);
     return;
   }
   if (packed) {
-    LaunchK<P, kGlu, XT, false, true>(a, grid, plan, stream);
+    LaunchK<F, P, kGlu, XT, false, true>(a, grid, plan, stream);
   } else {
-    LaunchK<P, kGlu, XT, false, false>(a, grid, plan, stream);
+    LaunchK<F, P, kGlu, XT, false, false>(a, grid, plan, stream);
   }
 }
 
-template <int P>
+template <class F, int P>
 void LaunchP(const VecQArgs& a, int x_type, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   const bool glu = a.d.g != nullptr;
   switch (x_type) {
     case -1:
-      glu ? LaunchT<P, true, -1>(a, grid, plan, stream) : LaunchT<P, false, -1>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, -1>(a, grid, plan, stream) : LaunchT<F, P, false, -1>(a, grid, plan, stream);
       break;
     case LLMP_X_F32:
-      glu ? LaunchT<P, true, LLMP_X_F32>(a, grid, plan, stream) : LaunchT<P, false, LLMP_X_F32>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, LLMP_X_F32>(a, grid, plan, stream)
+          : LaunchT<F, P, false, LLMP_X_F32>(a, grid, plan, stream);
       break;
     default:
-      glu ? LaunchT<P, true, LLMP_X_BF16>(a, grid, plan, stream)
-          : LaunchT<P, false, LLMP_X_BF16>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, LLMP_X_BF16>(a, grid, plan, stream)
+          : LaunchT<F, P, false, LLMP_X_BF16>(a, grid, plan, stream);
       break;
   }
 }
 
-}  // namespace
-
-bool FlatQ4KTakes(const llmp_vecq_desc& d) {
-  const int nsb = d.ncols_x / 256;
-  const bool glu = d.g != nullptr;
-  return nsb >= 1 && nsb <= (glu ? kWave / 2 : kWave) && PlanFlat(1, nsb, glu).lds <= kFlatLdsLimit;
-}
-
-void LaunchFlatQ4K(const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
+template <class F>
+void LaunchF(const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
   const llmp_vecq_desc& d = a.d;
-  const int nsb = d.ncols_x / 256;
+  const int units = d.ncols_x / F::kUnitValues;
   const bool glu = d.g != nullptr;
-  if (pass > 1 && PlanFlat(4, nsb, glu).lds > kFlatLdsLimit) pass = 1;
-  const FlatPlan plan = PlanFlat(pass > 1 ? 4 : 1, nsb, glu);
+  if (pass > 1 && PlanFlat<F>(4, units, glu).lds > kFlatLdsLimit) pass = 1;
+  const FlatPlan plan = PlanFlat<F>(pass > 1 ? 4 : 1, units, glu);
   if (g_compute_units == 0) {
-    const int units = llmp_hip_compute_units();
-    g_compute_units = units > 0 ? units : 256;
+    const int cus = llmp_hip_compute_units();
+    g_compute_units = cus > 0 ? cus : 256;
   }
   const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
@@ -515,9 +639,36 @@ void LaunchFlatQ4K(const VecQArgs& a, int x_type, int pass, hipStream_t stream) 
   if (groups > (tiles + kWaves - 1) / kWaves) groups = (tiles + kWaves - 1) / kWaves;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
   if (pass > 1) {
-    LaunchP<4>(a, x_type, grid, plan, stream);
+    LaunchP<F, 4>(a, x_type, grid, plan, stream);
   } else {
-    LaunchP<1>(a, x_type, grid, plan, stream);
+    LaunchP<F, 1>(a, x_type, grid, plan, stream);
+  }
+}
+
+}  // namespace
+
+// Q4_K rows up to 64 super-blocks (32 with a GLU). Q8_0 rows of whole 256 values up to 64 units
+// (32 with a GLU) whose rows, matrices and experts all start on 16-byte boundaries: the
+// tiles are fetched in 16-byte chunks.
+bool FlatTakes(int type, const llmp_vecq_desc& d) {
+  const bool glu = d.g != nullptr;
+  const int most = glu ? kWave / 2 : kWave;
+  if (type == LLMP_TYPE_Q4_K) {
+    const int units = d.ncols_x / FormatQ4K::kUnitValues;
+    return units >= 1 && units <= most && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
+  }
+  if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
+  const int units = d.ncols_x / FormatQ8::kUnitValues;
+  const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+  return units <= most && d.stride_row % 8 == 0 && d.stride_expert % 8 == 0 && at % 16 == 0 &&
+         PlanFlat<FormatQ8>(1, units, glu).lds <= kFlatLdsLimit;
+}
+
+void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
+  if (type == LLMP_TYPE_Q4_K) {
+    LaunchF<FormatQ4K>(a, x_type, pass, stream);
+  } else {
+    LaunchF<FormatQ8>(a, x_type, pass, stream);
   }
 }
 

@@ -49,9 +49,10 @@ def test_q8_1_planes_and_strides(device):
 
 @pytest.mark.parametrize("t,k,n,variant", [(Q8_0, 4096, 64, 0), (Q4_K, 3840, 40, 0), (Q4_K, 3840, 40, 6),
                                            (Q8_0, 96, 9, 0), (Q4_K, 256, 7, 0), (Q4_K, 256, 7, 6),
-                                           (Q4_K, 2048, 300, 6)])
+                                           (Q4_K, 2048, 300, 6), (Q8_0, 4096, 64, 6), (Q8_0, 256, 7, 6),
+                                           (Q8_0, 3840, 41, 6)])
 def test_block_sums_are_bit_exact(device, t, k, n, variant):
-    """The int32 sums of the rows form (variant 0) and of the flat Q4_K form (variant 6)."""
+    """The int32 sums of the rows form (variant 0) and of the flat form (variant 6)."""
     w = make_weights(t, n, k, 21, plausible=False)
     q8 = oracle.q8_1_quantize(synth.activations(1, k, 22))
     want = oracle.vecq_block_sums(t, w, q8, k, n)
@@ -79,10 +80,6 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
-        if name.startswith("flat") and t != Q4_K:
-            with pytest.raises(ops.KernelFailure):
-                ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
-            continue
         got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
         ok, worst = rel_close(got, want, TOL)
         assert ok, (variant, worst)
