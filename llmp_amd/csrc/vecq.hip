@@ -487,7 +487,8 @@ constexpr Variant kVariants[] = {
     {"lanes8 pass8 flight2", 8, 8, 2},   {"lanes16 pass1 flight4", 16, 1, 4}, {"lanes64 pass1 flight2", 64, 1, 2},
     // A lane a whole unit of a row, a Q4_K super-block or four Q8_0 blocks (vecq_flat.hip);
     // `lanes` 0 marks the form.
-    {"flat pass1", 0, 1, 2},             {"flat pass4", 0, 4, 2},
+    // `flight`: tile buffers a wave.
+    {"flat pass1", 0, 1, 1},             {"flat pass4", 0, 4, 1},             {"flat pass1 two tiles", 0, 1, 2},
 };
 constexpr int kFlatFirst = 6;
 constexpr int kVariantCount = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -621,7 +622,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
                        "256 values up to 8192 (4096) at 16-byte boundaries");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
       return Refuse(1, "vecq: block sums are of a dense one-token product");
-    LaunchFlat(type, a, x_type, v.pass, static_cast<hipStream_t>(stream));
+    LaunchFlat(type, a, x_type, v.pass, v.flight == 2, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }
   const size_t lds = LdsBytes(v.pass, a.kp);

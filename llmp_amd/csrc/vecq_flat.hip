@@ -382,13 +382,23 @@ typedef const __attribute__((address_space(1))) void* GlobalPointer;
 // of `chunks` lands at byte 16 c. `base` and `ring` are the same in every lane.
 // kPacked: rows follow each other without a gap, so the part is one byte range; else a row's
 // bytes (a whole number of chunks) are `row_bytes` of every `stride_bytes`.
+// The same value in every lane, and known to the compiler as such: a pointer that came
+// through LDS or a per-lane load otherwise costs two vector registers wherever it is used.
+__device__ __forceinline__ const uint8_t* Uniform(const uint8_t* p) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 template <int kLoads, bool kPacked>
 __device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int64_t stride_bytes, int row_bytes,
                                           uint8_t* ring, int lane) {
+  base = Uniform(base);
 #pragma unroll
   for (int j = 0; j < kLoads; ++j) {
     const int c = j * kWave + lane;
-    if (c < chunks) {
+    if (j * kWave < chunks && c < chunks) {  // a load is issued exactly when some lane has a chunk
       const uint8_t* from;
       if constexpr (kPacked) {
         from = base + static_cast<uint32_t>(c) * 16u;
@@ -428,9 +438,37 @@ __device__ __forceinline__ void AwaitTile() {
   asm volatile("" ::: "memory");
 }
 
+// The loads FetchTile issues for a tile of `rows` rows: one for every 64 chunks of a part.
+template <class F, bool kGlu>
+__device__ __forceinline__ int TileLoads(int rows, int units) {
+  const int chunks = rows * units * F::kUnitBytes / 16;
+  const int part = min((chunks + kWave - 1) / kWave, kGlu ? 5 : 9);
+  return kGlu ? 2 * part : part;
+}
+
+// All but this wave's `left` latest memory operations are complete (0 to 10; the same in
+// every lane).
+__device__ __forceinline__ void AwaitAllBut(int left) {
+  switch (left) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+    case 9: __builtin_amdgcn_s_waitcnt(0x0F79); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
+  }
+  __builtin_amdgcn_wave_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // grid (workgroups, slots); LDS: P tokens' records, then a tile buffer a wave.
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked>
-__global__ __launch_bounds__(kGroup, 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep>
+__global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
@@ -442,7 +480,10 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlat(const VecQArgs a, const in
   const int nsb = d.ncols_x / F::kUnitValues;  // units a row
   const int token_stride = nsb * F::kRecord;
   const int tiles = (d.nrows + rows_per_tile - 1) / rows_per_tile;
-  uint8_t* ring = lds + P * token_stride + wave * (kWave * F::kUnitBytes);
+  // kDeep: two tile buffers a wave (one workgroup a CU), the next tile in flight while this one
+  // is multiplied.
+  constexpr int kTileBytes = kWave * F::kUnitBytes;
+  uint8_t* ring = lds + P * token_stride + wave * ((kDeep ? 2 : 1) * kTileBytes);
 
   // A lane's place in every tile: its matrix, row and unit of the row.
   const int half = rows_per_tile * nsb;
@@ -517,13 +558,28 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlat(const VecQArgs a, const in
     }
     __syncthreads();  // the records are staged; from here the waves run alone
 
+    int buffer = 0;  // kDeep: the tile buffer the tile `index` is in
     while (index < tiles) {
       const int row0 = index * rows_per_tile;
       const bool live = placed && row0 + row < d.nrows;
-      AwaitTile();
+      const int next = index + tile_step;
+      if constexpr (kDeep) {
+        // The next tile into the other buffer, whose readers finished an iteration ago; then
+        // wait for everything older than its loads: this tile, and the last one's stores.
+        if (next < tiles) {
+          const int next0 = next * rows_per_tile;
+          const int rows = min(rows_per_tile, d.nrows - next0);
+          FetchTile<F, kGlu, kPacked>(d, expert_block, next0, rows, nsb, gate_at, ring + (buffer ^ 1) * kTileBytes, lane);
+          AwaitAllBut(TileLoads<F, kGlu>(rows, nsb));
+        } else {
+          AwaitTile();
+        }
+      } else {
+        AwaitTile();
+      }
       float out[P];
       if (live) {
-        const typename F::Unit unit = F::Read(my_block);
+        const typename F::Unit unit = F::Read(my_block + (kDeep ? buffer * kTileBytes : 0));
         int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * F::kDumpInts : nullptr;
         F::template Dot<P, kDump>(unit, my_records, token_stride, m, out, dump);
       }
@@ -547,13 +603,16 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlat(const VecQArgs a, const in
           }
         }
       }
-      // The next tile may overwrite the buffer: every lane's reads of it were consumed above.
-      // (Queueing these loads before the row sums measured slower.)
-      index += tile_step;
-      if (index < tiles) {
+      index = next;
+      if constexpr (kDeep) {
+        buffer ^= 1;
+        __builtin_amdgcn_wave_barrier();  // every lane has read its unit before the buffer is refilled
+      } else if (index < tiles) {
+        // The next tile may overwrite the buffer: every lane's reads of it were consumed above.
+        // (Queueing these loads before the row sums measured slower.)
         const int next0 = index * rows_per_tile;
         FetchTile<F, kGlu, kPacked>(d, expert_block, next0, min(rows_per_tile, d.nrows - next0), nsb, gate_at, ring,
-                                 lane);
+                                    lane);
       }
     }
   }
@@ -566,32 +625,40 @@ struct FlatPlan {
 };
 
 template <class F>
-FlatPlan PlanFlat(int pass, int units, bool glu) {
+FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   FlatPlan p;
   p.rows = (glu ? kWave / 2 : kWave) / units;
-  p.lds = static_cast<size_t>(pass) * units * F::kRecord + static_cast<size_t>(kWaves) * kWave * F::kUnitBytes;
+  p.lds = static_cast<size_t>(pass) * units * F::kRecord +
+          static_cast<size_t>(deep ? 2 : 1) * kWaves * kWave * F::kUnitBytes;
   return p;
 }
 
 constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
+constexpr size_t kDeepLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 int g_compute_units = 0;
 
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked>
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kFlatLdsLimit));
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(kDeep ? kDeepLdsLimit : kFlatLdsLimit));
     sized = true;
   }
-  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked>), grid, dim3(kGroup), plan.lds, stream, a, plan.rows);
+  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(kGroup), plan.lds, stream, a,
+                     plan.rows);
 }
 
 template <class F, int P, bool kGlu, int XT>
-void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
+void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, bool deep, hipStream_t stream) {
   const bool packed = a.d.stride_row == a.d.ncols_x / F::kBlockValues;
   if (a.dump != nullptr) {
     if constexpr (P == 1 && !kGlu && XT < 0) LaunchK<F, P, kGlu, XT, true, false>(a, grid, plan, stream);
+    return;
+  }
+  if (deep) {
+    if constexpr (P == 1) LaunchK<F, P, kGlu, XT, false, true, true>(a, grid, plan, stream);
     return;
   }
   if (packed) {
@@ -602,30 +669,33 @@ void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t str
 }
 
 template <class F, int P>
-void LaunchP(const VecQArgs& a, int x_type, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
+void LaunchP(const VecQArgs& a, int x_type, dim3 grid, const FlatPlan& plan, bool deep, hipStream_t stream) {
   const bool glu = a.d.g != nullptr;
   switch (x_type) {
     case -1:
-      glu ? LaunchT<F, P, true, -1>(a, grid, plan, stream) : LaunchT<F, P, false, -1>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, -1>(a, grid, plan, deep, stream) : LaunchT<F, P, false, -1>(a, grid, plan, deep, stream);
       break;
     case LLMP_X_F32:
-      glu ? LaunchT<F, P, true, LLMP_X_F32>(a, grid, plan, stream)
-          : LaunchT<F, P, false, LLMP_X_F32>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, LLMP_X_F32>(a, grid, plan, deep, stream)
+          : LaunchT<F, P, false, LLMP_X_F32>(a, grid, plan, deep, stream);
       break;
     default:
-      glu ? LaunchT<F, P, true, LLMP_X_BF16>(a, grid, plan, stream)
-          : LaunchT<F, P, false, LLMP_X_BF16>(a, grid, plan, stream);
+      glu ? LaunchT<F, P, true, LLMP_X_BF16>(a, grid, plan, deep, stream)
+          : LaunchT<F, P, false, LLMP_X_BF16>(a, grid, plan, deep, stream);
       break;
   }
 }
 
 template <class F>
-void LaunchF(const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
+void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
   const llmp_vecq_desc& d = a.d;
   const int units = d.ncols_x / F::kUnitValues;
   const bool glu = d.g != nullptr;
   if (pass > 1 && PlanFlat<F>(4, units, glu).lds > kFlatLdsLimit) pass = 1;
-  const FlatPlan plan = PlanFlat<F>(pass > 1 ? 4 : 1, units, glu);
+  // Two tile buffers a wave: one token a pass, packed rows, one workgroup a CU.
+  deep = deep && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
+         PlanFlat<F>(1, units, glu, true).lds <= kDeepLdsLimit;
+  const FlatPlan plan = PlanFlat<F>(pass > 1 ? 4 : 1, units, glu, deep);
   if (g_compute_units == 0) {
     const int cus = llmp_hip_compute_units();
     g_compute_units = cus > 0 ? cus : 256;
@@ -634,14 +704,14 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
   // What is resident at once: two workgroups a CU, shared by the slots that have work.
   const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
-  int groups = 2 * g_compute_units / (live_slots > 0 ? live_slots : 1);
+  int groups = (deep ? 1 : 2) * g_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
   if (groups > (tiles + kWaves - 1) / kWaves) groups = (tiles + kWaves - 1) / kWaves;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
   if (pass > 1) {
-    LaunchP<F, 4>(a, x_type, grid, plan, stream);
+    LaunchP<F, 4>(a, x_type, grid, plan, deep, stream);
   } else {
-    LaunchP<F, 1>(a, x_type, grid, plan, stream);
+    LaunchP<F, 1>(a, x_type, grid, plan, deep, stream);
   }
 }
 
@@ -664,11 +734,11 @@ bool FlatTakes(int type, const llmp_vecq_desc& d) {
          PlanFlat<FormatQ8>(1, units, glu).lds <= kFlatLdsLimit;
 }
 
-void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, hipStream_t stream) {
+void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
   if (type == LLMP_TYPE_Q4_K) {
-    LaunchF<FormatQ4K>(a, x_type, pass, stream);
+    LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
   } else {
-    LaunchF<FormatQ8>(a, x_type, pass, stream);
+    LaunchF<FormatQ8>(a, x_type, pass, deep, stream);
   }
 }
 
