@@ -489,7 +489,11 @@ constexpr Variant kVariants[] = {
     // `lanes` 0 marks the form.
     // `flight`: tile buffers a wave.
     {"flat pass1", 0, 1, 1},             {"flat pass4", 0, 4, 1},             {"flat pass1 two tiles", 0, 1, 2},
+    // Q4_K sub-block products on the int8 matrix cores, 16 tokens a pass (vecq_mma.hip);
+    // `lanes` -1 marks the form.
+    {"mma pass16", -1, 16, 1},
 };
+constexpr int kMmaVariant = 9;
 constexpr int kFlatFirst = 6;
 constexpr int kVariantCount = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -553,8 +557,11 @@ void LaunchVariant(const VecQArgs& a, int x_type, int variant, dim3 grid, size_t
 
 // The default configuration of a shape: the tokens of a pass first (each pass
 // streams the weights again), then enough lanes a row to fill the device.
-int DefaultVariant(int type, const llmp_vecq_desc& d, int kp) {
+int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   const int tokens = d.tokens;
+  // Several tokens of a dense or grouped product over Q8_1 blocks: the matrix cores. A routed product's pairs
+  // mostly name different experts, one or two tokens each: the flat form.
+  if (tokens > 1 && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
   while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
@@ -612,10 +619,17 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   a.kp = PaddedK(d->ncols_x);
   a.dump = dump;
   a.offsets = offsets;
-  if (variant < 0) variant = DefaultVariant(type, *d, a.kp);
+  if (variant < 0) variant = DefaultVariant(type, *d, a.kp, x != nullptr);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
-  if (offsets != nullptr && v.lanes != 0) return Refuse(1, "vecq: sorted rows take the flat form");
+  if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
+  if (v.lanes < 0) {
+    if (!MmaTakes(type, *d)) return Refuse(1, "vecq: the matrix-core form takes Q4_K rows up to 7168 values");
+    if (x != nullptr) return Refuse(1, "vecq: the matrix-core form takes Q8_1 activations");
+    if (dump != nullptr) return Refuse(1, "vecq: block sums are of the one-token variants");
+    LaunchMma(a, static_cast<hipStream_t>(stream));
+    return LaunchStatus("vecq");
+  }
   if (v.lanes == 0) {
     if (!FlatTakes(type, *d))
       return Refuse(1, "vecq: the flat form takes Q4_K rows up to 16384 values (8192 with a GLU), and Q8_0 rows of whole "
@@ -690,14 +704,16 @@ extern "C" int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int
                                     void* stream) {
   if (offsets == nullptr || d == nullptr) return Refuse(1, "vecq: null offsets");
   if (experts < 1 || experts > 65535) return Refuse(1, "vecq: 1 to 65535 experts");
-  if (!FlatTakes(type, *d)) return Refuse(1, "vecq: sorted rows take weights the flat form takes");
+  if (!FlatTakes(type, *d) && !MmaTakes(type, *d))
+    return Refuse(1, "vecq: sorted rows take weights the flat or the matrix-core form takes");
   llmp_vecq_desc sorted = *d;
   sorted.ids = nullptr;
   sorted.used = experts;  // a workgroup row an expert
   sorted.tokens = 1;      // the row counts come from the offsets
   sorted.y_slot = 0;
   sorted.dst_slot = 0;
-  if (variant < 0) variant = kFlatFirst + 1;
+  // An expert's rows are many tokens of one matrix: the matrix cores where they apply.
+  if (variant < 0) variant = MmaTakes(type, *d) ? kMmaVariant : kFlatFirst + 1;
   return Launch(type, &sorted, nullptr, variant, nullptr, stream, offsets);
 }
 

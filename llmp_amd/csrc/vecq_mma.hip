@@ -1,0 +1,396 @@
+// llmp.vecq over Q4_K weights for 2 to 16 tokens a pass: the sub-block dot products on the
+// int8 matrix cores.
+//
+// v_mfma_i32_16x16x32_i8 multiplies one 32-value sub-block of 16 weight rows with the same
+// sub-block of 16 tokens: the instruction's K is a Q4_K sub-block, so every product comes out
+// as the int32 sum the scalar kernel's eight v_dot4 give, for 256 (token, row) pairs at once.
+// What is left per sub-block is the scaling, in floats, and it is done with exactly the
+// operations of the one-token kernel (vecq_flat.hip) in exactly its order: per super-block
+//   main = fma(float(prod_g), sc_g * d8_g, main), g = 0 .. 7;  mins = m_0 * ds8_0, then
+//   fma(m_g, ds8_g, mins);  out = fma(d, main, -(dmin * mins))
+// and the super-blocks of a row are added in the tree that kernel's wave shuffles form
+// (aligned pairs, then pairs of pairs, ...), so a (token, row) value is bit for bit the
+// one-token product's (src/kernels/ggml/vecq.cu:1150-1166 of the reference asks for that).
+//
+// A lane of the instruction's result holds one weight row (lane % 16) and four tokens
+// (4 (lane / 16) + q): the weights are the second operand. A wave owns 16 rows (of both
+// matrices with a GLU) and half of K; the two waves of a tile split K at the largest power of
+// two below the row's super-blocks, which is the top node of the tree, and meet in LDS. A
+// workgroup is eight waves, four tiles. Weights come straight from global memory into the
+// operand layout (a lane reads its row's header and, per pair of sub-blocks, the eight code
+// bytes of its K group), three super-blocks deep; the tokens' Q8_1 codes and scales are staged
+// in LDS once a workgroup, in the first operand's layout:
+//   codes   [super-block][pair of sub-blocks][K group][token] 16 bytes: the eight codes of
+//           the K group in sub-block 2 p, then in 2 p + 1 (a lane's read is its 16 bytes of a
+//           contiguous 1 KB);
+//   scales  [super-block][token][pair] 4 floats: d8 of 2 p and 2 p + 1, d8 * sum(codes) of
+//           2 p and 2 p + 1.
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+#include "vecq_common.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr int kMmaGroup = 512;
+constexpr int kMmaWaves = kMmaGroup / kWave;
+constexpr int kMmaTokens = 16;                       // a pass
+constexpr int kTilesGroup = kMmaWaves / 2;           // row tiles a workgroup: two waves a tile
+constexpr int kCodesSb = 4 * kMmaTokens * 4 * 16;    // 4096 bytes of codes a super-block
+constexpr int kScalesSb = kMmaTokens * 4 * 16;       // 1024 bytes of scales a super-block
+constexpr int kPartialBytes = kMmaWaves * 2 * kWave * 16;  // a wave's four floats a lane and matrix
+constexpr size_t kMmaLdsLimit = 160 * 1024 - 2048;
+
+typedef int V4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float ByteOf(uint32_t word, int byte) {
+  return static_cast<float>((word >> (8 * byte)) & 0xFFu);  // v_cvt_f32_ubyteN
+}
+
+// A lane's part of one super-block of its weight row: the header and, for each pair of
+// sub-blocks, the eight code bytes of its K group (low nibbles sub-block 2 p, high 2 p + 1).
+struct RowPart {
+  U32x4 header;  // d, dmin, scales[12]
+  uint2 q[4];
+};
+
+__device__ __forceinline__ RowPart LoadRowPart(const uint8_t* row, int sb, int kg) {
+  RowPart part;
+  const uint8_t* at = row + static_cast<int64_t>(sb) * 144;
+  part.header = *reinterpret_cast<const U32x4*>(at);
+#pragma unroll
+  for (int p = 0; p < 4; ++p) part.q[p] = *reinterpret_cast<const uint2*>(at + 16 + 32 * p + 8 * kg);
+  return part;
+}
+
+// The decoded header of a super-block: 6-bit scales and minimums as bytes g of sc[g / 4],
+// mn[g / 4] (the packing of tests/unit/dsv4_fast_test.cc:180-183 of the reference).
+struct Header {
+  uint32_t sc[2], mn[2];
+  float d, dmin;
+};
+
+__device__ __forceinline__ Header Decode(const U32x4& h) {
+  Header out;
+  const uint32_t s0 = h.y, s1 = h.z, s2 = h.w;
+  out.sc[0] = s0 & 0x3F3F3F3Fu;
+  out.sc[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+  out.mn[0] = s1 & 0x3F3F3F3Fu;
+  out.mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+  out.d = HalfBitsToFloat(h.x & 0xFFFFu);
+  out.dmin = HalfBitsToFloat(h.x >> 16);
+  return out;
+}
+
+__device__ __forceinline__ int64_t Pack(uint32_t lo, uint32_t hi) {
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Sums of a row's super-blocks in the order of the one-token kernel's shuffle tree: aligned
+// pairs first, then pairs of pairs, .... The kernel adds each aligned group of four itself
+// (Quad); the groups of four then go through a binary counter's carries, which builds the
+// rest of the same tree: l2 holds a finished group of four waiting for its neighbour, l3 one
+// of eight, l4 one of sixteen. Everything is selects on values the same in every lane, so
+// that the levels stay in registers.
+struct TreeSum {
+  float l2[4], l3[4], l4[4];
+};
+
+__device__ __forceinline__ void Sum4(const float (&a)[4], const float (&b)[4], float (&out)[4]) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int q = 0; q < 4; ++q) out[q] = a[q] + b[q];
+}
+
+// `index`: the group's place counted from the first pushed.
+__device__ __forceinline__ void Push(TreeSum& t, const float (&v)[4], int index) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+#pragma clang fp contract(off)
+    const float c2 = v[q];
+    const float c3 = t.l2[q] + c2;
+    const float c4 = t.l3[q] + c3;
+    t.l2[q] = (index & 1) == 0 ? c2 : t.l2[q];
+    t.l3[q] = (index & 3) == 1 ? c3 : t.l3[q];
+    t.l4[q] = (index & 3) == 3 ? c4 : t.l4[q];
+  }
+}
+
+// The total of `count` pushed groups (1 to 4): the unfinished ones from the smallest up.
+__device__ __forceinline__ void Total(const TreeSum& t, int count, float (&out)[4]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+#pragma clang fp contract(off)
+    float v = 0.0f;
+    bool any = false;
+    if (count & 1) v = t.l2[q], any = true;
+    if (count & 2) v = any ? t.l3[q] + v : t.l3[q], any = true;
+    if (count & 4) v = t.l4[q];  // four groups: nothing else is pending
+    out[q] = v;
+  }
+}
+
+// One super-block of one matrix times the staged tokens: four tokens of this lane's row.
+// `a`: the tokens' codes as first operands, sub-block by sub-block; `entries[4 q + p]`: token
+// q's four scale floats of pair p (in LDS, read a pair at a time).
+__device__ __forceinline__ void DotPart(const RowPart& part, const int64_t (&a)[8], const float4* entries,
+                                        float (&out)[4]) {
+#pragma clang fp contract(off)
+  const Header h = Decode(part.header);
+  float main[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  float mins[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const uint32_t q0 = part.q[p].x, q1 = part.q[p].y;
+    const int64_t lo = Pack(q0 & 0x0F0F0F0Fu, q1 & 0x0F0F0F0Fu);
+    const int64_t hi = Pack((q0 >> 4) & 0x0F0F0F0Fu, (q1 >> 4) & 0x0F0F0F0Fu);
+    const V4i zero = {0, 0, 0, 0};
+    const V4i prod0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[2 * p], lo, zero, 0, 0, 0);
+    const V4i prod1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[2 * p + 1], hi, zero, 0, 0, 0);
+    const float sc0 = ByteOf(h.sc[(2 * p) >> 2], (2 * p) & 3);
+    const float sc1 = ByteOf(h.sc[(2 * p + 1) >> 2], (2 * p + 1) & 3);
+    const float m0 = ByteOf(h.mn[(2 * p) >> 2], (2 * p) & 3);
+    const float m1 = ByteOf(h.mn[(2 * p + 1) >> 2], (2 * p + 1) & 3);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 s = entries[4 * q + p];
+      main[q] = fmaf(static_cast<float>(prod0[q]), sc0 * s.x, main[q]);
+      main[q] = fmaf(static_cast<float>(prod1[q]), sc1 * s.y, main[q]);
+      mins[q] = p == 0 ? m0 * s.z : fmaf(m0, s.z, mins[q]);
+      mins[q] = fmaf(m1, s.w, mins[q]);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) out[q] = fmaf(h.d, main[q], -(h.dmin * mins[q]));
+}
+
+// Stages `m` tokens' Q8_1 rows (one thread a block) into the operand layout. `row_of(j)`: token
+// j's row of Q8_1 blocks.
+template <class RowOf>
+__device__ __forceinline__ void StageTokens(RowOf row_of, int m, int blocks, uint8_t* codes, uint8_t* scales) {
+  for (int index = threadIdx.x; index < m * blocks; index += kMmaGroup) {
+    const int j = index / blocks, b = index - j * blocks;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(j) + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+    const int sb = b >> 3, g = b & 7;
+    uint8_t* to = codes + sb * kCodesSb + ((g >> 1) * 4 * kMmaTokens + j) * 16 + (g & 1) * 8;
+#pragma unroll
+    for (int kg = 0; kg < 4; ++kg)
+      *reinterpret_cast<uint2*>(to + kg * kMmaTokens * 16) = make_uint2(w[1 + 2 * kg], w[2 + 2 * kg]);
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum = Dot4(0x01010101, static_cast<int>(w[1 + i]), sum);
+    const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
+    float* entry = reinterpret_cast<float*>(scales + sb * kScalesSb + (j * 4 + (g >> 1)) * 16);
+    entry[g & 1] = d8;
+    entry[2 + (g & 1)] = d8 * static_cast<float>(sum);
+  }
+}
+
+// grid (workgroups, slots); LDS: codes, scales, the waves' partial sums.
+template <bool kGlu>
+__global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int pairs[kMaxPairs];
+  __shared__ int count;
+
+  const llmp_vecq_desc& d = a.d;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int nsb = d.ncols_x / 256;
+  uint8_t* codes = lds;
+  uint8_t* scales = lds + nsb * kCodesSb;
+  float* partial = reinterpret_cast<float*>(lds + nsb * (kCodesSb + kScalesSb));
+
+  int expert = blockIdx.y;
+  int sorted_first = 0;
+  if (a.offsets != nullptr) {
+    sorted_first = a.offsets[expert];
+    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+    __syncthreads();
+  } else {
+    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
+  }
+  const int n = count;
+  if (n == 0) return;  // uniform over the workgroup
+  const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
+
+  // This wave's half of K: the split is the top node of the row's summation tree.
+  int split = 1;
+  while (split * 2 < nsb) split *= 2;
+  if (nsb == 1) split = 1;
+  const int half = wave & 1;
+  const int first = half == 0 ? 0 : split;
+  const int last = half == 0 ? min(split, nsb) : nsb;
+  const int row_in_tile = lane & 15, kg = lane >> 4;
+  const int tiles = (d.nrows + 15) / 16;
+  const int groups = (tiles + kTilesGroup - 1) / kTilesGroup;
+
+  for (int p0 = 0; p0 < n; p0 += kMmaTokens) {
+    const int m = min(kMmaTokens, n - p0);
+    __syncthreads();  // the last pass's readers of the staged tokens
+    auto row_of = [&](int j) {
+      const int pr = a.offsets != nullptr ? (sorted_first + p0 + j) << 8 : pairs[p0 + j];
+      return static_cast<const uint8_t*>(d.y) +
+             (static_cast<int64_t>(pr >> 8) * d.y_token + static_cast<int64_t>(pr & 0xFF) * d.y_slot) * kQ8Block;
+    };
+    StageTokens(row_of, m, d.ncols_x / 32, codes, scales);
+    __syncthreads();
+
+    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+      const int tile = group * kTilesGroup + (wave >> 1);
+      const int row = min(tile * 16 + row_in_tile, d.nrows - 1);  // rows past the end repeat the last, unstored
+      const uint8_t* up_row =
+          static_cast<const uint8_t*>(d.w) + (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
+      const uint8_t* gate_row =
+          kGlu ? static_cast<const uint8_t*>(d.g) + (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144
+               : nullptr;
+      TreeSum up_sum{}, gate_sum{};
+      RowPart u0, u1, u2, u3, g0, g1, g2, g3;  // three are live at a time
+      auto fetch = [&](int sb, RowPart& u, RowPart& g) {
+        if (sb < last) {
+          u = LoadRowPart(up_row, sb, kg);
+          if constexpr (kGlu) g = LoadRowPart(gate_row, sb, kg);
+        }
+      };
+      auto step = [&](int sb, const RowPart& u, const RowPart& g, float (&up_out)[4], float (&gate_out)[4]) {
+        int64_t acts[8];
+        const uint8_t* mine = codes + sb * kCodesSb + lane * 16;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const U32x4 c = *reinterpret_cast<const U32x4*>(mine + p * (kMmaTokens * 4 * 16));
+          acts[2 * p] = Pack(c.x, c.y);
+          acts[2 * p + 1] = Pack(c.z, c.w);
+        }
+        const float4* entries = reinterpret_cast<const float4*>(scales + sb * kScalesSb) + (4 * kg) * 4;
+        DotPart(u, acts, entries, up_out);
+        if constexpr (kGlu) DotPart(g, acts, entries, gate_out);
+      };
+      int quads = 0;
+      if (tile < tiles) {
+        fetch(first, u0, g0);
+        fetch(first + 1, u1, g1);
+        for (int sb = first; sb < last; sb += 4, ++quads) {
+          const int n = min(4, last - sb);
+          // The group's sum as its values come: (x0 + x1) + (x2 + x3), absent ones left out.
+          float up_quad[4], gate_quad[4], up_next[4], gate_next[4];
+          fetch(sb + 2, u2, g2);
+          step(sb, u0, g0, up_quad, gate_quad);
+          if (n >= 2) {
+            fetch(sb + 3, u3, g3);
+            step(sb + 1, u1, g1, up_next, gate_next);
+            Sum4(up_quad, up_next, up_quad);
+            if constexpr (kGlu) Sum4(gate_quad, gate_next, gate_quad);
+          }
+          if (n >= 3) {
+            float up_rest[4], gate_rest[4];
+            fetch(sb + 4, u0, g0);
+            step(sb + 2, u2, g2, up_rest, gate_rest);
+            if (n >= 4) {
+              fetch(sb + 5, u1, g1);
+              step(sb + 3, u3, g3, up_next, gate_next);
+              Sum4(up_rest, up_next, up_rest);
+              if constexpr (kGlu) Sum4(gate_rest, gate_next, gate_rest);
+            }
+            Sum4(up_quad, up_rest, up_quad);
+            if constexpr (kGlu) Sum4(gate_quad, gate_rest, gate_quad);
+          }
+          Push(up_sum, up_quad, quads);
+          if constexpr (kGlu) Push(gate_sum, gate_quad, quads);
+        }
+      }
+      // The two halves of K meet: the upper half's totals through LDS.
+      float up_total[4] = {0.0f, 0.0f, 0.0f, 0.0f}, gate_total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      const bool has = tile < tiles && last > first;
+      if (has) {
+        Total(up_sum, quads, up_total);
+        if constexpr (kGlu) Total(gate_sum, quads, gate_total);
+      }
+      float4* slot = reinterpret_cast<float4*>(partial) + (wave * 2) * kWave + lane;
+      if (half == 1) {
+        slot[0] = make_float4(up_total[0], up_total[1], up_total[2], up_total[3]);
+        if constexpr (kGlu) slot[kWave] = make_float4(gate_total[0], gate_total[1], gate_total[2], gate_total[3]);
+      }
+      __syncthreads();
+      if (half == 0 && tile < tiles) {
+#pragma clang fp contract(off)
+        if (split < nsb) {
+          const float4* other = reinterpret_cast<const float4*>(partial) + ((wave + 1) * 2) * kWave + lane;
+          const float4 u = other[0];
+          up_total[0] += u.x, up_total[1] += u.y, up_total[2] += u.z, up_total[3] += u.w;
+          if constexpr (kGlu) {
+            const float4 g = other[kWave];
+            gate_total[0] += g.x, gate_total[1] += g.y, gate_total[2] += g.z, gate_total[3] += g.w;
+          }
+        }
+        if (tile * 16 + row_in_tile < d.nrows) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int t = 4 * kg + q;
+            if (t < m) {
+              const int pr = a.offsets != nullptr ? (sorted_first + p0 + t) << 8 : pairs[p0 + t];
+              float* dst = d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
+              dst[tile * 16 + row_in_tile] = kGlu ? Glu(d.glu, gate_total[q], up_total[q], d.limit) : up_total[q];
+            }
+          }
+        }
+      }
+      __syncthreads();  // the partial sums may be overwritten
+    }
+  }
+}
+
+size_t MmaLds(int nsb) { return static_cast<size_t>(nsb) * (kCodesSb + kScalesSb) + kPartialBytes; }
+
+int g_mma_compute_units = 0;
+
+}  // namespace
+
+// Q4_K rows whose sixteen staged tokens fit LDS (k up to 7168).
+bool MmaTakes(int type, const llmp_vecq_desc& d) {
+  if (type != LLMP_TYPE_Q4_K) return false;
+  const int nsb = d.ncols_x / 256;
+  return nsb >= 1 && MmaLds(nsb) <= kMmaLdsLimit;
+}
+
+void LaunchMma(const VecQArgs& a, hipStream_t stream) {
+  const llmp_vecq_desc& d = a.d;
+  const int nsb = d.ncols_x / 256;
+  const size_t lds = MmaLds(nsb);
+  if (g_mma_compute_units == 0) {
+    const int cus = llmp_hip_compute_units();
+    g_mma_compute_units = cus > 0 ? cus : 256;
+  }
+  const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
+  const int tiles = (d.nrows + 15) / 16;
+  const int tile_groups = (tiles + kTilesGroup - 1) / kTilesGroup;
+  const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
+  int groups = g_mma_compute_units / (live_slots > 0 ? live_slots : 1);
+  if (groups < 1) groups = 1;
+  if (groups > tile_groups) groups = tile_groups;
+  const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
+  static bool sized[2] = {false, false};
+  if (d.g != nullptr) {
+    if (!sized[1]) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
+      sized[1] = true;
+    }
+    hipLaunchKernelGGL((VecQMma<true>), grid, dim3(kMmaGroup), lds, stream, a);
+  } else {
+    if (!sized[0]) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
+      sized[0] = true;
+    }
+    hipLaunchKernelGGL((VecQMma<false>), grid, dim3(kMmaGroup), lds, stream, a);
+  }
+}
+
+}  // namespace llmp_hip

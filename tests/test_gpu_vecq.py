@@ -80,6 +80,10 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
+        if name.startswith("mma") and t != Q4_K:  # the matrix-core form is Q4_K's
+            with pytest.raises(ops.KernelFailure):
+                ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
+            continue
         got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
         ok, worst = rel_close(got, want, TOL)
         assert ok, (variant, worst)
