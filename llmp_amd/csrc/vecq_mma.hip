@@ -253,11 +253,15 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
                : nullptr;
       TreeSum up_sum{}, gate_sum{};
       RowPart u0, u1, u2, u3, g0, g1, g2, g3;  // three are live at a time
+      // The loads of super-block sb, queued here and no later: the compiler would otherwise
+      // sink them to their first use, two steps on, and the wave would wait out the whole
+      // memory latency there.
+      // (Past the end the last super-block again: no branch, no copies of what was loaded.)
       auto fetch = [&](int sb, RowPart& u, RowPart& g) {
-        if (sb < last) {
-          u = LoadRowPart(up_row, sb, kg);
-          if constexpr (kGlu) g = LoadRowPart(gate_row, sb, kg);
-        }
+        const int at = min(sb, last - 1);
+        u = LoadRowPart(up_row, at, kg);
+        if constexpr (kGlu) g = LoadRowPart(gate_row, at, kg);
+        __builtin_amdgcn_sched_barrier(0);
       };
       auto step = [&](int sb, const RowPart& u, const RowPart& g, float (&up_out)[4], float (&gate_out)[4]) {
         int64_t acts[8];
