@@ -232,6 +232,32 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
   const int tiles = (d.nrows + 15) / 16;
   const int groups = (tiles + kTilesGroup - 1) / kTilesGroup;
 
+  // This lane's weight rows of the tile its wave takes in a group of tiles (rows past the end
+  // repeat the last, unstored).
+  const uint8_t* up_row = nullptr;
+  const uint8_t* gate_row = nullptr;
+  auto aim = [&](int group) {
+    const int row = min((group * kTilesGroup + (wave >> 1)) * 16 + row_in_tile, d.nrows - 1);
+    const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
+    up_row = static_cast<const uint8_t*>(d.w) + at;
+    if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
+  };
+  RowPart u0, u1, u2, u3, g0, g1, g2, g3;  // three are live at a time
+  // The loads of super-block sb, queued here and no later: the compiler would otherwise sink
+  // them to their first use, two steps on, and the wave would wait out the whole memory latency
+  // there. (Past the end the last super-block again: no branch, no copies of what was loaded.)
+  auto fetch = [&](int sb, RowPart& u, RowPart& g) {
+    const int at = min(sb, last - 1);
+    u = LoadRowPart(up_row, at, kg);
+    if constexpr (kGlu) g = LoadRowPart(gate_row, at, kg);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // A group's first two super-blocks are asked for while the group before it finishes (the
+  // first group's before the tokens are staged).
+  aim(blockIdx.x);
+  fetch(first, u0, g0);
+  fetch(first + 1, u1, g1);
+
   for (int p0 = 0; p0 < n; p0 += kMmaTokens) {
     const int m = min(kMmaTokens, n - p0);
     __syncthreads();  // the last pass's readers of the staged tokens
@@ -245,24 +271,7 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
 
     for (int group = blockIdx.x; group < groups; group += gridDim.x) {
       const int tile = group * kTilesGroup + (wave >> 1);
-      const int row = min(tile * 16 + row_in_tile, d.nrows - 1);  // rows past the end repeat the last, unstored
-      const uint8_t* up_row =
-          static_cast<const uint8_t*>(d.w) + (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
-      const uint8_t* gate_row =
-          kGlu ? static_cast<const uint8_t*>(d.g) + (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144
-               : nullptr;
       TreeSum up_sum{}, gate_sum{};
-      RowPart u0, u1, u2, u3, g0, g1, g2, g3;  // three are live at a time
-      // The loads of super-block sb, queued here and no later: the compiler would otherwise
-      // sink them to their first use, two steps on, and the wave would wait out the whole
-      // memory latency there.
-      // (Past the end the last super-block again: no branch, no copies of what was loaded.)
-      auto fetch = [&](int sb, RowPart& u, RowPart& g) {
-        const int at = min(sb, last - 1);
-        u = LoadRowPart(up_row, at, kg);
-        if constexpr (kGlu) g = LoadRowPart(gate_row, at, kg);
-        __builtin_amdgcn_sched_barrier(0);
-      };
       auto step = [&](int sb, const RowPart& u, const RowPart& g, float (&up_out)[4], float (&gate_out)[4]) {
         int64_t acts[8];
         const uint8_t* mine = codes + sb * kCodesSb + lane * 16;
@@ -278,8 +287,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
       };
       int quads = 0;
       if (tile < tiles) {
-        fetch(first, u0, g0);
-        fetch(first + 1, u1, g1);
         for (int sb = first; sb < last; sb += 4, ++quads) {
           const int n = min(4, last - sb);
           // The group's sum as its values come: (x0 + x1) + (x2 + x3), absent ones left out.
@@ -308,6 +315,14 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
           Push(up_sum, up_quad, quads);
           if constexpr (kGlu) Push(gate_sum, gate_quad, quads);
         }
+      }
+      // The next group's (or the next pass's first group's) first loads.
+      {
+        int next = group + static_cast<int>(gridDim.x);
+        if (next >= groups) next = blockIdx.x;
+        aim(next);
+        fetch(first, u0, g0);
+        fetch(first + 1, u1, g1);
       }
       // The two halves of K meet: the upper half's totals through LDS.
       float up_total[4] = {0.0f, 0.0f, 0.0f, 0.0f}, gate_total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
