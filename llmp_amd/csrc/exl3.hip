@@ -167,6 +167,8 @@ __global__ __launch_bounds__(64) void HadamardKernel(const void* __restrict__ x,
   const int lane = threadIdx.x;
   const int64_t at = static_cast<int64_t>(blockIdx.x) * columns + blockIdx.y * 128 + 2 * lane;
   float a = 0.0f, b = 0.0f;
+  // Added in slice order; unrolled so that eight slices' loads are in flight at a time.
+#pragma unroll 8
   for (int s = 0; s < slices; ++s) {
     if constexpr (X == 0) {
       const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(x) + s * slice_stride + at);
