@@ -28,7 +28,9 @@ __device__ __forceinline__ float WaveSum(float v) {
   return v;
 }
 
-// A token a wave: expert lane + 64 i sits in lane `lane`'s slot i.
+// A token a wave: expert lane + 64 i sits in lane `lane`'s slot i. SLOTS: slots a lane holds (a
+// kernel for 128 experts does not walk the sixteen that 1024 need).
+template <int SLOTS>
 __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float* __restrict__ logits,
                                                                    int32_t* __restrict__ ids,
                                                                    float* __restrict__ weights, int tokens, int experts,
@@ -38,12 +40,12 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float*
   if (t >= tokens) return;  // whole waves
   const float* l = logits + t * experts;
   const int slots = (experts + kWave - 1) / kWave;
-  float v[kRouterSlots];
-  float p[kRouterSlots];
+  float v[SLOTS];
+  float p[SLOTS];
   float most = -INFINITY;
   bool nan = false;
 #pragma unroll
-  for (int i = 0; i < kRouterSlots; ++i) {
+  for (int i = 0; i < SLOTS; ++i) {
     const int e = i * kWave + lane;
     const bool have = i < slots && e < experts;
     v[i] = have ? l[e] : -INFINITY;
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float*
   const bool degenerate = nan || !(fabsf(most) < INFINITY);
   float sum = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kRouterSlots; ++i) {
+  for (int i = 0; i < SLOTS; ++i) {
     const int e = i * kWave + lane;
     const bool have = i < slots && e < experts;
     p[i] = have && !degenerate ? expf(v[i] - most) : 0.0f;
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float*
     int index = 0x7FFFFFFF;
     float best_p = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kRouterSlots; ++i) {
+    for (int i = 0; i < SLOTS; ++i) {
       const int e = i * kWave + lane;
       const bool have = i < slots && e < experts && p[i] >= 0.0f;  // a pick is marked by -1
       const float key = degenerate ? 0.0f : v[i];
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float*
     }
     if (index != 0x7FFFFFFF && (index & (kWave - 1)) == lane) {
 #pragma unroll
-      for (int i = 0; i < kRouterSlots; ++i) {
+      for (int i = 0; i < SLOTS; ++i) {
         if (i == index / kWave) p[i] = -1.0f;
       }
     }
@@ -132,14 +134,25 @@ struct Route {
 
 // Each workgroup counts its chunk's ids per expert: one thread an expert, the chunk's slots
 // in order (no atomics: a thread owns its counter).
+// The chunk's ids into LDS (chunk tokens x used ints): every thread then walks all of them.
+__device__ __forceinline__ int StageChunkIds(const int32_t* __restrict__ ids, int ids_stride, const Route& r, int t0,
+                                             int t1, int32_t* staged) {
+  const int n = (t1 - t0) * r.used;
+  for (int i = threadIdx.x; i < n; i += blockDim.x)
+    staged[i] = ids[static_cast<int64_t>(t0 + i / r.used) * ids_stride + i % r.used];
+  __syncthreads();
+  return n;
+}
+
 __global__ void RouteCount(const int32_t* __restrict__ ids, int ids_stride, Route r) {
+  extern __shared__ int32_t staged[];
   const int c = blockIdx.x;
   const int t0 = c * kRouteChunk;
   const int t1 = min(t0 + kRouteChunk, r.tokens);
+  const int slots = StageChunkIds(ids, ids_stride, r, t0, t1, staged);
   for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
     int n = 0;
-    for (int t = t0; t < t1; ++t)
-      for (int j = 0; j < r.used; ++j) n += ids[static_cast<int64_t>(t) * ids_stride + j] == e;
+    for (int i = 0; i < slots; ++i) n += staged[i] == e;
     r.counts[static_cast<int64_t>(c) * r.experts + e] = n;
   }
 }
@@ -169,28 +182,27 @@ __global__ void RouteScan(Route r) {
   }
 }
 
-// Each workgroup places its chunk's slots: one thread an expert, its rows in token order.
+// Each workgroup places its chunk's slots, one thread a slot: the slot's row is its expert's
+// first row, plus the expert's slots in earlier chunks, plus those before it in this chunk
+// (token order, then slot order: every thread walks the staged ids before its own).
 __global__ void RouteAssign(const int32_t* __restrict__ ids, int ids_stride, Route r) {
+  extern __shared__ int32_t staged[];
   const int c = blockIdx.x;
   const int t0 = c * kRouteChunk;
   const int t1 = min(t0 + kRouteChunk, r.tokens);
-  for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
-    int row = r.offsets[e] + r.counts[static_cast<int64_t>(c) * r.experts + e];
-    for (int t = t0; t < t1; ++t)
-      for (int j = 0; j < r.used; ++j) {
-        if (ids[static_cast<int64_t>(t) * ids_stride + j] != e) continue;
-        r.position[t * r.used + j] = row;
-        r.token[row] = t;
-        r.expert[row] = e;
-        ++row;
-      }
-  }
-  // Ids outside the experts have no row.
-  for (int i = threadIdx.x; i < (t1 - t0) * r.used; i += blockDim.x) {
-    const int t = t0 + i / r.used;
-    const int j = i % r.used;
-    const int e = ids[static_cast<int64_t>(t) * ids_stride + j];
-    if (e < 0 || e >= r.experts) r.position[t * r.used + j] = -1;
+  const int slots = StageChunkIds(ids, ids_stride, r, t0, t1, staged);
+  for (int i = threadIdx.x; i < slots; i += blockDim.x) {
+    const int e = staged[i];
+    if (e < 0 || e >= r.experts) {  // ids outside the experts have no row
+      r.position[t0 * r.used + i] = -1;
+      continue;
+    }
+    int before = 0;
+    for (int j = 0; j < i; ++j) before += staged[j] == e;
+    const int row = r.offsets[e] + r.counts[static_cast<int64_t>(c) * r.experts + e] + before;
+    r.position[t0 * r.used + i] = row;
+    r.token[row] = t0 + i / r.used;
+    r.expert[row] = e;
   }
 }
 
@@ -274,8 +286,18 @@ extern "C" int llmp_hip_moe_router(const float* logits, int experts, int used, i
   if (used < 1 || used > experts || used > kWave) return Refuse(1, "moe.router: 1 to min(experts, 64) picks, not %d", used);
   if (tokens < 1) return Refuse(1, "moe.router: no tokens");
   const dim3 grid(static_cast<unsigned>((tokens + kRouterWaves - 1) / kRouterWaves));
-  hipLaunchKernelGGL(RouterKernel, grid, dim3(kRouterWaves * kWave), 0, static_cast<hipStream_t>(stream), logits, ids,
-                     weights, tokens, experts, used, normalize, scale);
+  const auto s = static_cast<hipStream_t>(stream);
+  const dim3 block(kRouterWaves * kWave);
+  if (experts <= 2 * kWave) {
+    hipLaunchKernelGGL(RouterKernel<2>, grid, block, 0, s, logits, ids, weights, tokens, experts, used, normalize, scale);
+  } else if (experts <= 4 * kWave) {
+    hipLaunchKernelGGL(RouterKernel<4>, grid, block, 0, s, logits, ids, weights, tokens, experts, used, normalize, scale);
+  } else if (experts <= 8 * kWave) {
+    hipLaunchKernelGGL(RouterKernel<8>, grid, block, 0, s, logits, ids, weights, tokens, experts, used, normalize, scale);
+  } else {
+    hipLaunchKernelGGL(RouterKernel<kRouterSlots>, grid, block, 0, s, logits, ids, weights, tokens, experts, used,
+                       normalize, scale);
+  }
   return LaunchStatus("moe.router");
 }
 
@@ -289,14 +311,16 @@ extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int expert
                                   int32_t* route, void* stream) {
   if (ids == nullptr || route == nullptr) return Refuse(1, "moe.route: null operand");
   if (experts < 1 || used < 1 || tokens < 1 || ids_stride < used) return Refuse(1, "moe.route: empty or overlapping ids");
+  if (used > 128) return Refuse(1, "moe.route: more than 128 slots a token");  // a chunk's ids are staged in LDS
   if (static_cast<int64_t>(used) * tokens > (1 << 24)) return Refuse(1, "moe.route: more than 2^24 slots");
   const Route r = RouteOf(route, experts, used, tokens);
   const auto s = static_cast<hipStream_t>(stream);
   const int threads = experts < 256 ? (experts + 63) / 64 * 64 : 256;
-  hipLaunchKernelGGL(RouteCount, dim3(r.chunks), dim3(threads), 0, s, ids, ids_stride, r);
+  const size_t chunk_bytes = static_cast<size_t>(kRouteChunk) * used * sizeof(int32_t);
+  hipLaunchKernelGGL(RouteCount, dim3(r.chunks), dim3(threads), chunk_bytes, s, ids, ids_stride, r);
   if (const int bad = LaunchStatus("moe.route count"); bad != 0) return bad;
   hipLaunchKernelGGL(RouteScan, dim3(1), dim3(threads), static_cast<size_t>(experts) * sizeof(int), s, r);
-  hipLaunchKernelGGL(RouteAssign, dim3(r.chunks), dim3(threads), 0, s, ids, ids_stride, r);
+  hipLaunchKernelGGL(RouteAssign, dim3(r.chunks), dim3(256), chunk_bytes, s, ids, ids_stride, r);
   return LaunchStatus("moe.route");
 }
 
