@@ -16,7 +16,8 @@
 // (4 (lane / 16) + q): the weights are the second operand. A wave owns 16 rows (of both
 // matrices with a GLU) and half of K; the two waves of a tile split K at the largest power of
 // two below the row's super-blocks, which is the top node of the tree, and meet in LDS. A
-// workgroup is eight waves, four tiles. Weights come straight from global memory into the
+// workgroup is eight waves, four tiles (rows of up to eight super-blocks: eight tiles, a wave
+// all of K). Weights come straight from global memory into the
 // operand layout (a lane reads its row's header and, per pair of sub-blocks, the eight code
 // bytes of its K group), three super-blocks deep; the tokens' Q8_1 codes and scales are staged
 // in LDS once a workgroup, in the first operand's layout:
@@ -39,6 +40,7 @@ constexpr int kMmaGroup = 512;
 constexpr int kMmaWaves = kMmaGroup / kWave;
 constexpr int kMmaTokens = 16;                       // a pass
 constexpr int kTilesGroup = kMmaWaves / 2;           // row tiles a workgroup: two waves a tile
+constexpr int kWholeRow = 8;                         // super-blocks a row up to which a wave takes all of K
 constexpr int kCodesSb = 4 * kMmaTokens * 4 * 16;    // 4096 bytes of codes a super-block
 constexpr int kScalesSb = kMmaTokens * 4 * 16;       // 1024 bytes of scales a super-block
 constexpr int kPartialBytes = kMmaWaves * 2 * kWave * 16;  // a wave's four floats a lane and matrix
@@ -221,23 +223,27 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
   if (n == 0) return;  // uniform over the workgroup
   const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
 
-  // This wave's half of K: the split is the top node of the row's summation tree.
+  // This wave's part of K. Rows of up to eight super-blocks: all of it, a tile a wave (too few
+  // steps to be worth two waves and their meeting). Longer rows: a half, split at the top node
+  // of the row's summation tree.
+  const bool whole = nsb <= kWholeRow;
   int split = 1;
   while (split * 2 < nsb) split *= 2;
-  if (nsb == 1) split = 1;
-  const int half = wave & 1;
+  const int half = whole ? 0 : wave & 1;
   const int first = half == 0 ? 0 : split;
-  const int last = half == 0 ? min(split, nsb) : nsb;
+  const int last = whole ? nsb : half == 0 ? min(split, nsb) : nsb;
   const int row_in_tile = lane & 15, kg = lane >> 4;
   const int tiles = (d.nrows + 15) / 16;
-  const int groups = (tiles + kTilesGroup - 1) / kTilesGroup;
+  const int tiles_group = whole ? kMmaWaves : kTilesGroup;
+  const int tile_in_group = whole ? wave : wave >> 1;
+  const int groups = (tiles + tiles_group - 1) / tiles_group;
 
   // This lane's weight rows of the tile its wave takes in a group of tiles (rows past the end
   // repeat the last, unstored).
   const uint8_t* up_row = nullptr;
   const uint8_t* gate_row = nullptr;
   auto aim = [&](int group) {
-    const int row = min((group * kTilesGroup + (wave >> 1)) * 16 + row_in_tile, d.nrows - 1);
+    const int row = min((group * tiles_group + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
     const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
     up_row = static_cast<const uint8_t*>(d.w) + at;
     if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
@@ -270,7 +276,7 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
     __syncthreads();
 
     for (int group = blockIdx.x; group < groups; group += gridDim.x) {
-      const int tile = group * kTilesGroup + (wave >> 1);
+      const int tile = group * tiles_group + tile_in_group;
       TreeSum up_sum{}, gate_sum{};
       auto step = [&](int sb, const RowPart& u, const RowPart& g, float (&up_out)[4], float (&gate_out)[4]) {
         int64_t acts[8];
@@ -336,10 +342,10 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
         slot[0] = make_float4(up_total[0], up_total[1], up_total[2], up_total[3]);
         if constexpr (kGlu) slot[kWave] = make_float4(gate_total[0], gate_total[1], gate_total[2], gate_total[3]);
       }
-      __syncthreads();
+      if (!whole) __syncthreads();
       if (half == 0 && tile < tiles) {
 #pragma clang fp contract(off)
-        if (split < nsb) {
+        if (!whole && split < nsb) {
           const float4* other = reinterpret_cast<const float4*>(partial) + ((wave + 1) * 2) * kWave + lane;
           const float4 u = other[0];
           up_total[0] += u.x, up_total[1] += u.y, up_total[2] += u.z, up_total[3] += u.w;
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
           }
         }
       }
-      __syncthreads();  // the partial sums may be overwritten
+      if (!whole) __syncthreads();  // the partial sums may be overwritten
     }
   }
 }
@@ -388,7 +394,8 @@ void LaunchMma(const VecQArgs& a, hipStream_t stream) {
   }
   const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + 15) / 16;
-  const int tile_groups = (tiles + kTilesGroup - 1) / kTilesGroup;
+  const int tiles_group = nsb <= kWholeRow ? kMmaWaves : kTilesGroup;
+  const int tile_groups = (tiles + tiles_group - 1) / tiles_group;
   const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
   int groups = g_mma_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
