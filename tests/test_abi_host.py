@@ -74,7 +74,10 @@ def test_other_entry_points_refuse_bad_operands():
     lib = _lib.load()
     assert lib.llmp_hip_vecq(12, None, -1, None) > 0
     assert lib.llmp_hip_vecq(12, C.byref(desc()), 99, None) > 0
-    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=16)), 6, None) > 0  # the flat form is Q4_K's
+    # The flat form takes Q8_0 rows of whole 256 values at 16-byte boundaries only; the matrix-core form Q4_K only.
+    assert lib.llmp_hip_vecq(8, C.byref(desc(ncols_x=480, stride_row=15)), 6, None) > 0
+    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=17)), 6, None) > 0
+    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=16, tokens=4)), 9, None) > 0
     assert lib.llmp_hip_vecq_fused(12, C.byref(desc()), None, -1, None) > 0
     assert lib.llmp_hip_vecq_block_sums(12, C.byref(desc()), -1, None, None) > 0
     assert lib.llmp_hip_q8_1_quantize(None, None, 32, 512, 32, 1, 1, 32, None) > 0
@@ -83,5 +86,5 @@ def test_other_entry_points_refuse_bad_operands():
     assert lib.llmp_hip_moe_router(0x1000, 128, 0, 1, 1, 1.0, 0x2000, 0x3000, None) > 0
     assert lib.llmp_hip_moe_combine(0x1000, 0x2000, None, 6, 8, 1, 0x3000, None) > 0
     assert lib.llmp_hip_moe_route(None, 8, 128, 8, 1, 0x1000, None) > 0
-    assert lib.llmp_hip_vecq_sorted(8, C.byref(desc(stride_row=16)), 0x1000, 4, -1, None) > 0
+    assert lib.llmp_hip_vecq_sorted(8, C.byref(desc(ncols_x=480, stride_row=15)), 0x1000, 4, -1, None) > 0
     assert lib.llmp_hip_moe_route_ints(128, 8, 512) == 2 * 129 + 3 * 4096 + 8 * 128
