@@ -141,6 +141,38 @@ def test_routed_experts_match_oracle(device, t, tokens, used):
     assert ok, worst
 
 
+@pytest.mark.parametrize("k,n,tokens", [(2816, 50, 5), (256, 17, 2), (6144, 32, 16), (2048, 130, 9)])
+def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, k, n, tokens):
+    """The int8 matrix-core kernel (variant 9) repeats the flat kernel's float operations and its
+    summation tree: dense with and without a GLU, grouped matrices, and routed experts."""
+    t, mma, flat = Q4_K, 9, 7
+    gate, up = make_weights(t, n, k, 301), make_weights(t, n, k, 302)
+    q8 = ops.quantize_q8_1(dev(synth.activations(tokens, k, 303), device))
+    wd, gd = dev(up, device), dev(gate, device)
+    for kw in (dict(), dict(gate=gd, glu=ops.GLU_SWIGLU)):
+        a = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=mma, **kw).cpu().numpy()
+        b = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=flat, **kw).cpu().numpy()
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), kw.keys()
+    # Three matrices, every token through each (per-slot activations).
+    groups = 3
+    w3 = dev(make_weights(t, groups * n, k, 304).reshape(groups, -1), device)
+    q83 = ops.quantize_q8_1(dev(synth.activations(tokens * groups, k, 305), device))
+    y_row = ops.padded_k(k) // 32
+    kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // 256), y_token=y_row * groups, y_slot=y_row)
+    a = ops.vecq(t, w3, q83, k, n, variant=mma, **kw).cpu().numpy()
+    b = ops.vecq(t, w3, q83, k, n, variant=flat, **kw).cpu().numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    # Routed: two picks a token out of five experts.
+    experts, used = 5, 2
+    w5 = dev(make_weights(t, experts * n, k, 306).reshape(experts, -1), device)
+    g = synth.rng(307)
+    ids = dev(np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32), device)
+    kw = dict(ids=ids, tokens=tokens, used=used, stride_expert=n * (k // 256))
+    a = ops.vecq(t, w5, q8, k, n, variant=mma, **kw).cpu().numpy()
+    b = ops.vecq(t, w5, q8, k, n, variant=flat, **kw).cpu().numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_grouped_matrices_read_their_own_rows(device):
     t, k, n, groups, tokens = Q8_0, 256, 24, 3, 2
     qk, bs = 32, 34
