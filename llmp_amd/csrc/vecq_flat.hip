@@ -57,8 +57,8 @@ constexpr int kWaves = kGroup / kWave;
 
 // Staging is split in two so that a row's first loads can be queued before the wave's first
 // tile: memory operations complete in order, and a load queued behind a tile would wait for it.
-constexpr int kStep = kGroup / 8;  // blocks a sweep of the workgroup covers, eight lanes a block
-constexpr int kFront = 2;          // sweeps loaded ahead: rows up to 4096 values
+// A sweep of the workgroup covers blockDim.x / 8 blocks, eight lanes a block.
+constexpr int kFront = 2;  // sweeps loaded ahead: rows up to 4096 values with eight waves
 
 struct FrontX {
   float v[kFront][4];
@@ -71,7 +71,7 @@ __device__ __forceinline__ FrontX LoadFrontX(const void* __restrict__ x, int k) 
   const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
 #pragma unroll
   for (int i = 0; i < kFront; ++i) {
-    const int b = (threadIdx.x >> 3) + i * kStep;
+    const int b = (threadIdx.x >> 3) + i * static_cast<int>(blockDim.x >> 3);
     if (b < k / 32) Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, f.v[i]);
   }
   return f;
@@ -350,12 +350,13 @@ __device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k,
   const int lane8 = threadIdx.x & 7;
   const int blocks = k / 32;
   const bool wide = reinterpret_cast<uintptr_t>(x) % (XT == LLMP_X_F32 ? 16 : 8) == 0;
+  const int sweep = blockDim.x >> 3;
 #pragma unroll
   for (int i = 0; i < kFront; ++i) {
-    const int b = (threadIdx.x >> 3) + i * kStep;
+    const int b = (threadIdx.x >> 3) + i * sweep;
     if (b < blocks) F::StageX(front.v[i], b, token);  // whole 8-lane groups together
   }
-  for (int b = (threadIdx.x >> 3) + kFront * kStep; b < blocks; b += kStep) {
+  for (int b = (threadIdx.x >> 3) + kFront * sweep; b < blocks; b += sweep) {
     float v[4];
     Load4Wide<XT>(x, static_cast<int64_t>(b) * 32 + lane8 * 4, k, wide, v);
     F::StageX(v, b, token);
@@ -366,7 +367,7 @@ template <class F>
 __device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, const FrontQ8& front,
                                                uint8_t* token) {
   if (static_cast<int>(threadIdx.x) < blocks) F::StageQ8(front.w, threadIdx.x, token);
-  for (int b = threadIdx.x + kGroup; b < blocks; b += kGroup) {
+  for (int b = threadIdx.x + blockDim.x; b < blocks; b += blockDim.x) {
     const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
     uint32_t w[9];
 #pragma unroll
@@ -510,10 +511,15 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
     if (count == 0) return;  // uniform over the workgroup
   }
   const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
-  const int first_tile = blockIdx.x * kWaves + wave;
-  const int tile_step = gridDim.x * kWaves;
-  if (a.offsets == nullptr && d.ids == nullptr) ResolvePairs(d, blockIdx.y, pairs, &count);
-  const int n = count;
+  const int waves = blockDim.x / kWave;  // eight, fewer where a long row's records leave less room
+  const int first_tile = blockIdx.x * waves + wave;
+  const int tile_step = gridDim.x * waves;
+  // A dense or grouped product's pairs are its tokens on the workgroup's matrix: no list.
+  const bool listed = d.ids != nullptr && a.offsets == nullptr;
+  const int n = a.offsets == nullptr && d.ids == nullptr ? d.tokens : count;
+  auto pair_at = [&](int i) {
+    return a.offsets != nullptr ? (sorted_first + i) << 8 : listed ? pairs[i] : (i << 8) | expert;
+  };
 
   for (int p0 = 0; p0 < n; p0 += P) {
     const int m = min(P, n - p0);
@@ -525,7 +531,7 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
-        const int pr = a.offsets != nullptr ? (sorted_first + p0 + j) << 8 : pairs[p0 + j];
+        const int pr = pair_at(p0 + j);
         const int token = pr >> 8;
         const int slot = pr & 0xFF;
         if constexpr (XT < 0) {
@@ -596,7 +602,7 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
           float gate = 0.0f;
           if constexpr (kGlu) gate = __shfl_down(v, half, kWave);
           if (live && !gate_lane && sb == 0) {
-            const int pr = a.offsets != nullptr ? (sorted_first + p0 + t) << 8 : pairs[p0 + t];
+            const int pr = pair_at(p0 + t);
             float* dst =
                 d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
             dst[row0 + row] = kGlu ? Glu(d.glu, gate, v, d.limit) : v;
@@ -621,19 +627,27 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
 // The rows of a tile: as many as a wave's 64 lanes hold (half of them a matrix with a GLU).
 struct FlatPlan {
   int rows;
+  int waves;
   size_t lds;
 };
 
+constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
+constexpr int kFewestWaves = 5;
+
+// Eight waves a workgroup, fewer (down to kFewestWaves) where a long row's records would
+// otherwise push the workgroup past half a CU's LDS.
 template <class F>
 FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   FlatPlan p;
   p.rows = (glu ? kWave / 2 : kWave) / units;
-  p.lds = static_cast<size_t>(pass) * units * F::kRecord +
-          static_cast<size_t>(deep ? 2 : 1) * kWaves * kWave * F::kUnitBytes;
-  return p;
+  p.waves = kWaves;
+  for (;;) {
+    p.lds = static_cast<size_t>(pass) * units * F::kRecord +
+            static_cast<size_t>(deep ? 2 : 1) * p.waves * kWave * F::kUnitBytes;
+    if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
+    --p.waves;
+  }
 }
-
-constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
 constexpr size_t kDeepLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 int g_compute_units = 0;
 
@@ -646,7 +660,7 @@ void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t str
                               static_cast<int>(kDeep ? kDeepLdsLimit : kFlatLdsLimit));
     sized = true;
   }
-  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(kGroup), plan.lds, stream, a,
+  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(plan.waves * kWave), plan.lds, stream, a,
                      plan.rows);
 }
 
@@ -706,7 +720,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
   int groups = (deep ? 1 : 2) * g_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
-  if (groups > (tiles + kWaves - 1) / kWaves) groups = (tiles + kWaves - 1) / kWaves;
+  if (groups > (tiles + plan.waves - 1) / plan.waves) groups = (tiles + plan.waves - 1) / plan.waves;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
   if (pass > 1) {
     LaunchP<F, 4>(a, x_type, grid, plan, deep, stream);

@@ -73,6 +73,23 @@ def test_dense_matches_oracle(device, t, k, n, tokens):
     assert ok, worst
 
 
+@pytest.mark.parametrize("t,k,n", [(Q4_K, 15360, 37), (Q4_K, 16384, 9), (Q4_K, 13056, 70), (Q8_0, 8192, 21),
+                                   (Q8_0, 14336, 12)])
+@pytest.mark.parametrize("tokens", [1, 3])
+def test_long_rows_match_oracle(device, t, k, n, tokens):
+    """Rows whose staged activations leave room for fewer than eight waves' tiles, and rows too
+    long for the streaming form at all."""
+    w = make_weights(t, n, k, 35 + k + n)
+    x = synth.activations(tokens, k, 36 + tokens)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    fused = ops.vecq_fused(t, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+
+
 @pytest.mark.parametrize("t", [Q8_0, Q4_K])
 def test_every_variant_matches_and_random_bytes_decode(device, t):
     k, n, tokens = 1024, 50, 5
