@@ -631,9 +631,9 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
     return LaunchStatus("vecq");
   }
   if (v.lanes == 0) {
-    if (!FlatTakes(type, *d))
-      return Refuse(1, "vecq: the flat form takes Q4_K rows up to 16384 values (8192 with a GLU), and Q8_0 rows of whole "
-                       "256 values up to 8192 (4096) at 16-byte boundaries");
+    if (!FlatTakes(type, *d, dump != nullptr))
+      return Refuse(1, "vecq: the flat form takes Q4_K rows up to 27136 values (8192 with a GLU) and Q8_0 rows of whole "
+                       "256 values up to 32256 (4096) at 16-byte boundaries; block sums, rows up to 64 units");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
       return Refuse(1, "vecq: block sums are of a dense one-token product");
     LaunchFlat(type, a, x_type, v.pass, v.flight == 2, static_cast<hipStream_t>(stream));
@@ -695,7 +695,7 @@ extern "C" int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp
 
 extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums, void* stream) {
   if (sums == nullptr) return Refuse(1, "vecq: null sums");
-  if (variant < 0 && d != nullptr) variant = FlatTakes(type, *d) ? kFlatFirst : 0;
+  if (variant < 0 && d != nullptr) variant = FlatTakes(type, *d, true) ? kFlatFirst : 0;
   if (variant != 0 && variant != kFlatFirst) return Refuse(1, "vecq: block sums are of the one-token variants");
   return Launch(type, d, nullptr, variant, sums, stream);
 }

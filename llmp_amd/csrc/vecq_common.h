@@ -172,7 +172,7 @@ __device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_in
 
 // The flat kernels' launch (vecq_flat.hip): whether a product's shape and alignment fit them,
 // and the launch. x_type -1: Q8_1 activations.
-bool FlatTakes(int type, const llmp_vecq_desc& d);
+bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows = false);
 // `deep`: two tile buffers a wave where the shape allows (one token a pass, packed rows).
 void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream);
 

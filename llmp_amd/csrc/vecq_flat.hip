@@ -624,6 +624,105 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   }
 }
 
+// Rows longer than a wave's 64 units: a row is cut into `split` pieces of `piece` units (the
+// last may be shorter), a wave takes whole rows, a piece a tile, and each lane adds up its
+// units' products over the pieces before the lanes are summed. One token a pass, no GLU.
+// grid (workgroups, slots); LDS: the token's records, then a tile buffer a wave.
+template <class F, int XT>
+__global__ __launch_bounds__(kGroup, 4) void VecQFlatSplit(const VecQArgs a, const int split, const int piece) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int pairs[kMaxPairs];
+  __shared__ int count;
+
+  const llmp_vecq_desc& d = a.d;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int units = d.ncols_x / F::kUnitValues;
+  const int token_stride = units * F::kRecord;
+  uint8_t* ring = lds + token_stride + wave * (kWave * F::kUnitBytes);
+  const uint8_t* my_block = ring + lane * F::kUnitBytes;
+
+  int expert = blockIdx.y;
+  int sorted_first = 0;
+  if (a.offsets != nullptr) {
+    sorted_first = a.offsets[expert];
+    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+    __syncthreads();
+    if (count == 0) return;  // uniform over the workgroup
+  } else if (d.ids != nullptr) {
+    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
+    if (count == 0) return;  // uniform over the workgroup
+  }
+  const bool listed = d.ids != nullptr && a.offsets == nullptr;
+  const int n = a.offsets == nullptr && d.ids == nullptr ? d.tokens : count;
+  const uint8_t* matrix = Uniform(static_cast<const uint8_t*>(d.w) +
+                                  static_cast<int64_t>(expert) * d.stride_expert * F::kBlockBytes);
+  const int64_t row_bytes = static_cast<int64_t>(d.stride_row) * F::kBlockBytes;
+  const int waves = blockDim.x / kWave;
+  const int first_row = blockIdx.x * waves + wave;
+  const int row_step = gridDim.x * waves;
+  auto fetch = [&](int row, int c) {
+    const int here = min(piece, units - c * piece);
+    FetchPart<(kWave * F::kUnitBytes / 16 + kWave - 1) / kWave, true>(
+        matrix + row * row_bytes + c * piece * F::kUnitBytes, here * F::kUnitBytes / 16, 0, 0, ring, lane);
+  };
+
+  for (int p0 = 0; p0 < n; ++p0) {
+    if (p0 > 0) __syncthreads();  // the last pass's readers of the records
+    const int pr = a.offsets != nullptr ? (sorted_first + p0) << 8 : listed ? pairs[p0] : (p0 << 8) | expert;
+    const int token = pr >> 8;
+    const int slot = pr & 0xFF;
+    const void* row_x;
+    FrontX front_x;
+    FrontQ8 front_q;
+    if constexpr (XT < 0) {
+      row_x = static_cast<const uint8_t*>(d.y) +
+              (static_cast<int64_t>(token) * d.y_token + static_cast<int64_t>(slot) * d.y_slot) * kQ8Block;
+      front_q = LoadFrontQ8(static_cast<const uint8_t*>(row_x), d.ncols_x / 32);
+    } else {
+      const int64_t at = token * a.x_token + slot * a.x_slot;
+      row_x = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
+                               : static_cast<const void*>(static_cast<const uint16_t*>(a.x) + at);
+      front_x = LoadFrontX<XT>(row_x, d.ncols_x);
+    }
+    if (first_row < d.nrows) fetch(first_row, 0);
+    if constexpr (XT < 0) {
+      StageRecordsQ8<F>(static_cast<const uint8_t*>(row_x), d.ncols_x / 32, front_q, lds);
+    } else {
+      StageRecordsX<F, XT>(row_x, d.ncols_x, front_x, lds);
+    }
+    __syncthreads();  // the records are staged; from here the waves run alone
+
+    float* dst = d.dst + static_cast<int64_t>(token) * d.dst_token + static_cast<int64_t>(slot) * d.dst_slot;
+    for (int row = first_row; row < d.nrows; row += row_step) {
+      float total = 0.0f;
+      for (int c = 0; c < split; ++c) {
+        AwaitTile();
+        if (lane < min(piece, units - c * piece)) {
+          const typename F::Unit unit = F::Read(my_block);
+          float out[1];
+          F::template Dot<1, false>(unit, lds + (c * piece + lane) * F::kRecord, token_stride, 1, out, nullptr);
+          total += out[0];
+        }
+        // The next tile may overwrite the buffer: every lane's reads of it were consumed above.
+        if (c + 1 < split) {
+          fetch(row, c + 1);
+        } else if (row + row_step < d.nrows) {
+          fetch(row + row_step, 0);
+        }
+      }
+      // A suffix sum over the wave's lanes (a fixed tree), the total in lane 0.
+#pragma unroll
+      for (int off = 1; off < kWave; off <<= 1) {
+        const float other = __shfl_down(total, off, kWave);
+        if (lane + off < kWave) total += other;
+      }
+      if (lane == 0) dst[row] = total;
+    }
+  }
+}
+
 // The rows of a tile: as many as a wave's 64 lanes hold (half of them a matrix with a GLU).
 struct FlatPlan {
   int rows;
@@ -700,11 +799,64 @@ void LaunchP(const VecQArgs& a, int x_type, dim3 grid, const FlatPlan& plan, boo
   }
 }
 
+// A row of more than 64 units in pieces: the fewest pieces, of even length (a Q8_0 unit is 136
+// bytes and a tile is fetched in 16-byte chunks).
+struct SplitPlan {
+  int split;
+  int piece;
+  int waves;
+  size_t lds;
+};
+
+template <class F>
+SplitPlan PlanSplit(int units) {
+  SplitPlan p;
+  p.split = (units + kWave - 1) / kWave;
+  p.piece = ((units + p.split - 1) / p.split + 1) & ~1;
+  p.waves = kWaves;
+  for (;;) {
+    p.lds = static_cast<size_t>(units) * F::kRecord + static_cast<size_t>(p.waves) * kWave * F::kUnitBytes;
+    if (p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
+    --p.waves;
+  }
+}
+
+template <class F, int XT>
+void LaunchS(const VecQArgs& a, dim3 grid, const SplitPlan& plan, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlatSplit<F, XT>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kFlatLdsLimit));
+    sized = true;
+  }
+  hipLaunchKernelGGL((VecQFlatSplit<F, XT>), grid, dim3(plan.waves * kWave), plan.lds, stream, a, plan.split,
+                     plan.piece);
+}
+
 template <class F>
 void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
   const llmp_vecq_desc& d = a.d;
   const int units = d.ncols_x / F::kUnitValues;
   const bool glu = d.g != nullptr;
+  if (units > kWave) {
+    const SplitPlan plan = PlanSplit<F>(units);
+    if (g_compute_units == 0) {
+      const int cus = llmp_hip_compute_units();
+      g_compute_units = cus > 0 ? cus : 256;
+    }
+    const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
+    const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
+    int groups = 2 * g_compute_units / (live_slots > 0 ? live_slots : 1);
+    if (groups < 1) groups = 1;
+    if (groups > (d.nrows + plan.waves - 1) / plan.waves) groups = (d.nrows + plan.waves - 1) / plan.waves;
+    const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
+    switch (x_type) {
+      case -1: LaunchS<F, -1>(a, grid, plan, stream); break;
+      case LLMP_X_F32: LaunchS<F, LLMP_X_F32>(a, grid, plan, stream); break;
+      default: LaunchS<F, LLMP_X_BF16>(a, grid, plan, stream); break;
+    }
+    return;
+  }
   if (pass > 1 && PlanFlat<F>(4, units, glu).lds > kFlatLdsLimit) pass = 1;
   // Two tile buffers a wave: one token a pass, packed rows, one workgroup a CU.
   deep = deep && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
@@ -733,19 +885,23 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
 
 // Q4_K rows up to 64 super-blocks (32 with a GLU). Q8_0 rows of whole 256 values up to 64 units
 // (32 with a GLU) whose rows, matrices and experts all start on 16-byte boundaries: the
-// tiles are fetched in 16-byte chunks.
-bool FlatTakes(int type, const llmp_vecq_desc& d) {
+// tiles are fetched in 16-byte chunks. Without a GLU, and unless `whole_rows` asks for a row
+// in one tile (the block sums), longer rows in pieces, as long as their records fit.
+bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
   const bool glu = d.g != nullptr;
   const int most = glu ? kWave / 2 : kWave;
+  const bool pieces = !glu && !whole_rows;
   if (type == LLMP_TYPE_Q4_K) {
     const int units = d.ncols_x / FormatQ4K::kUnitValues;
-    return units >= 1 && units <= most && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
+    if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
+    return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
   const int units = d.ncols_x / FormatQ8::kUnitValues;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
-  return units <= most && d.stride_row % 8 == 0 && d.stride_expert % 8 == 0 && at % 16 == 0 &&
-         PlanFlat<FormatQ8>(1, units, glu).lds <= kFlatLdsLimit;
+  if (d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || at % 16 != 0) return false;
+  if (units > most) return pieces && PlanSplit<FormatQ8>(units).lds <= kFlatLdsLimit;
+  return PlanFlat<FormatQ8>(1, units, glu).lds <= kFlatLdsLimit;
 }
 
 void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {

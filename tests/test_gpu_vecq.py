@@ -74,11 +74,12 @@ def test_dense_matches_oracle(device, t, k, n, tokens):
 
 
 @pytest.mark.parametrize("t,k,n", [(Q4_K, 15360, 37), (Q4_K, 16384, 9), (Q4_K, 13056, 70), (Q8_0, 8192, 21),
-                                   (Q8_0, 14336, 12)])
+                                   (Q8_0, 14336, 12), (Q8_0, 11008, 19), (Q8_0, 32256, 5), (Q8_0, 32512, 3),
+                                   (Q4_K, 20480, 11), (Q4_K, 27136, 4), (Q4_K, 27392, 3)])
 @pytest.mark.parametrize("tokens", [1, 3])
 def test_long_rows_match_oracle(device, t, k, n, tokens):
-    """Rows whose staged activations leave room for fewer than eight waves' tiles, and rows too
-    long for the streaming form at all."""
+    """Rows whose staged activations leave room for fewer than eight waves' tiles, rows of more
+    than 64 units (streamed in pieces), and rows too long for the streaming form at all."""
     w = make_weights(t, n, k, 35 + k + n)
     x = synth.activations(tokens, k, 36 + tokens)
     q8 = oracle.q8_1_quantize(x)
@@ -156,6 +157,30 @@ def test_routed_experts_match_oracle(device, t, tokens, used):
                    stride_expert=stride_expert).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
+
+
+@pytest.mark.parametrize("t,k", [(Q8_0, 9216), (Q4_K, 18432)])
+def test_routed_and_sorted_long_rows_match_oracle(device, t, k):
+    """Rows streamed in pieces, under routing ids and under sorted-row offsets."""
+    n, experts, tokens, used = 13, 5, 3, 2
+    qk, bs = oracle.block_elements(t), oracle.block_bytes(t)
+    w = make_weights(t, experts * n, k, 75).reshape(experts, n * (k // qk) * bs)
+    g = synth.rng(76)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 77))
+    stride_expert = n * (k // qk)
+    want = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    # The same pairs as rows sorted by expert.
+    order = np.argsort(ids.reshape(-1), kind="stable")
+    offsets = np.concatenate([[0], np.cumsum(np.bincount(ids.reshape(-1), minlength=experts))]).astype(np.int32)
+    rows = np.ascontiguousarray(q8.reshape(tokens, -1)[order // used])
+    sorted_out = ops.vecq_sorted(t, dev(w, device), dev(rows, device), dev(offsets, device), k, n, experts,
+                                 stride_expert=stride_expert).cpu().numpy()
+    assert np.array_equal(sorted_out.view(np.uint32), got.reshape(tokens * used, n)[order].view(np.uint32))
 
 
 @pytest.mark.parametrize("k,n,tokens", [(2816, 50, 5), (256, 17, 2), (6144, 32, 16), (2048, 130, 9)])
