@@ -220,9 +220,10 @@ int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, 
 /* The packed linear for 1..16 rows: LinearOperands of validate.h:118-131 and
  * PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54. x (m x k F16) into
  * y (m x n, F16 or F32); a_had is the caller's m x k F16 scratch for the transformed input,
- * written first. `scratch` (llmp_hip_exl3_linear_scratch bytes, 8-byte aligned) takes the place
- * of the reference's lock area: the K slices' partial sums, added in slice order. Three
- * launches are queued; a failure after the first is reported as a fault (negative). */
+ * which the product's launch writes as it computes it. `scratch` (llmp_hip_exl3_linear_scratch
+ * bytes, 8-byte aligned) takes the place of the reference's lock area: the K slices' partial
+ * sums, added in slice order. Two launches are queued; a failure after the first is reported as
+ * a fault (negative). */
 typedef struct llmp_exl3_linear {
   llmp_exl3_weights weights;
   const void* x;

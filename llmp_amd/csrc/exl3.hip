@@ -43,20 +43,25 @@ typedef float V4f __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------ codebooks
 
-// s * m mod 2^32 for a 16-bit s, as two 24-bit multiplies (full rate) instead of a 32-bit one.
+// s * m + add mod 2^32 for a 16-bit s, as two 24-bit multiplies (full rate; a 32-bit multiply
+// runs at a quarter of it). Written as instructions: the compiler folds the pair back into one
+// 32-bit multiply otherwise.
 template <uint32_t kMultiplier>
 __device__ __forceinline__ uint32_t MulState(uint32_t s, uint32_t add) {
   constexpr uint32_t lo = kMultiplier & 0xFFFFFFu;
   constexpr uint32_t hi = kMultiplier >> 24;
-  const uint32_t x = __umul24(s, lo) + add;  // low 32 bits of a 40-bit product
+  uint32_t x;
+  asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(x) : "v"(s), "s"(lo), "v"(add));  // the product's low 32 bits
   if constexpr (hi == 0) return x;
-  return x + (__umul24(s, hi) << 24);
+  uint32_t top;
+  asm("v_mul_u32_u24 %0, %1, %2" : "=v"(top) : "v"(s), "s"(hi));
+  return x + (top << 24);
 }
 
 // decode_exl3.cc:28-37: each half keeps its sign and low 12 bits under exponent 0b011xx, then
 // the halves are added as one F16 addition.
 __device__ __forceinline__ _Float16 SumHalves(uint32_t x) {
-  const uint32_t y = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
+  const uint32_t y = __builtin_amdgcn_bitop3_b32(x, 0x8FFF8FFFu, 0x3B603B60u, 0x6A);  // (x & mask) ^ bias
   const _Float16 lo = __builtin_bit_cast(_Float16, static_cast<uint16_t>(y & 0xFFFFu));
   const _Float16 hi = __builtin_bit_cast(_Float16, static_cast<uint16_t>(y >> 16));
   return lo + hi;
@@ -108,11 +113,26 @@ __device__ __forceinline__ Place PlaceOf(int lane) {
 // The rows of a lane's four values, in position order.
 __device__ __forceinline__ int RowOf(int g, int j) { return 2 * g + (j & 1) + 8 * (j >> 1); }
 
+// The codebook values of positions first .. first + 3 (first a multiple of four). Up to five
+// bits a value the four states lie within 31 bits of the stream, so within the two words from
+// the first state's first bit: one 64-bit shift brings the last state to bit 0 and the others
+// sit at fixed offsets above it.
 template <int CB, int BITS, typename WordFn>
 __device__ __forceinline__ Half4 DecodeFour(int first, WordFn word) {
   Half4 v;
+  if constexpr (BITS <= 5) {
+    constexpr int words = BITS * 8;
+    const int end0 = (first + 1) * BITS + 256 * BITS;  // past the first state's last bit, a period ahead
+    const int ia = (end0 - 16) >> 5;
+    const int shift = 32 * ia + 64 - (end0 + 3 * BITS);  // 2 .. 45
+    const uint64_t merged = (static_cast<uint64_t>(word(ia % words)) << 32) | word((ia + 1) % words);
+    const uint32_t window = static_cast<uint32_t>(merged >> shift);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) v[j] = Codebook<CB>(State<BITS>(first + j, word));
+    for (int j = 0; j < 4; ++j) v[j] = Codebook<CB>((window >> ((3 - j) * BITS)) & 0xFFFFu);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = Codebook<CB>(State<BITS>(first + j, word));
+  }
   return v;
 }
 
@@ -204,27 +224,36 @@ __global__ __launch_bounds__(64) void HadamardKernel(const void* __restrict__ x,
 // ------------------------------------------------------------------- product
 
 constexpr int kRingDepth = 4;  // K steps of a 128-column block in flight a wave
-constexpr int kProductWaves = 4;
+constexpr int kProductWaves = 8;
+constexpr int kOperandBytes = 16 * 128 * 2;  // a wave's transformed activations of one 128 block of K
+constexpr int kReduceBytes = kProductWaves * 32 * 64 * 4;
 
-// partial[slice][m][n] = sum over the slice's K of xh[m][k] W^[k][n]; grid (n / 128 / 4 waves,
-// slices); xh F16 [m][k], m <= 16. A wave a 128-column block: eight tiles per 16 rows of K.
+// partial[blockIdx.y][m][n] = sum over a K range of xh[m][k] W^[k][n] with xh = H(x * suh) /
+// sqrt(128) as F16; grid (n / 128, outer slices), m <= 16. A workgroup a 128-column block, its
+// eight waves `blocks_per_wave` 128-blocks of K each: a wave transforms its own activations a
+// block at a time (the workgroups of the first column block also write them to a_had), decodes
+// eight tiles per 16 rows of K, and the waves' sums are added in wave order through LDS.
 template <int CB, int BITS>
 __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_t* __restrict__ trellis,
-                                                                   const uint16_t* __restrict__ xh,
+                                                                   const uint16_t* __restrict__ x,
+                                                                   const uint16_t* __restrict__ suh,
+                                                                   uint16_t* __restrict__ a_had,
                                                                    float* __restrict__ partial, int m, int n, int k,
-                                                                   int steps_per_slice) {
+                                                                   int blocks_per_wave) {
   constexpr int kTileBytes = BITS * 32;
   constexpr int kStepBytes = 8 * kTileBytes;  // a 128-column block's tiles of one K step
   constexpr int kLoads = (kStepBytes + 1023) / 1024;
+  constexpr int kRingBytes = kRingDepth * kLoads * 1024;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int block = blockIdx.x * kProductWaves + wave;  // of 128 columns
-  if (block >= n / 128) return;  // whole waves; nothing below synchronizes across waves
-  uint8_t* ring = lds + wave * (kRingDepth * kLoads * 1024);
-  const int steps = k / 16;
-  const int first = blockIdx.y * steps_per_slice;
-  const int last = min(first + steps_per_slice, steps);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int block = blockIdx.x;  // of 128 columns
+  uint8_t* ring = lds + wave * (kRingBytes + kOperandBytes);
+  uint8_t* operand = ring + kRingBytes;  // [token][128] F16
+  const int slice = blockIdx.y * kProductWaves + wave;
+  const int first = min(slice * blocks_per_wave, k / 128) * 8;  // in K steps of 16
+  const int last = min((slice + 1) * blocks_per_wave, k / 128) * 8;
   const Place p = PlaceOf(lane);
   const int64_t row_bytes = static_cast<int64_t>(n / 16) * kTileBytes;
   const uint8_t* source = trellis + static_cast<int64_t>(block) * kStepBytes;
@@ -245,13 +274,31 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_
 #pragma unroll
   for (int t = 0; t < 8; ++t) acc[t] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
   // The activations' operand: token l % 16, k slots in the lane group's row order.
-  const int token = min(p.n, m - 1);
-  const uint16_t* xrow = xh + static_cast<int64_t>(token) * k;
+  const uint8_t* my_operand = operand + min(p.n, m - 1) * 256 + 4 * p.g;
 
   for (int s = first; s < min(first + kRingDepth - 1, last); ++s) fetch(s);
   for (int step = first; step < last; ++step) {
-    const uint32_t x01 = *reinterpret_cast<const uint32_t*>(xrow + step * 16 + 2 * p.g);
-    const uint32_t x89 = *reinterpret_cast<const uint32_t*>(xrow + step * 16 + 2 * p.g + 8);
+    if ((step & 7) == 0) {
+      // The wave's next 128 values of every token, transformed as the input transform does.
+      const int at = (step >> 3) * 128 + 2 * lane;
+      const uint32_t sc = *reinterpret_cast<const uint32_t*>(suh + at);
+      const float sa = HalfBitsToFloat(sc & 0xFFFFu), sb = HalfBitsToFloat(sc >> 16);
+      for (int t = 0; t < m; ++t) {
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(x + static_cast<int64_t>(t) * k + at);
+        float a = HalfBitsToFloat(v & 0xFFFFu) * sa;
+        float b = HalfBitsToFloat(v >> 16) * sb;
+        Hadamard128(a, b, lane);
+        a *= kHadamardScale;
+        b *= kHadamardScale;
+        const uint32_t packed = FloatToHalfBits(a) | (FloatToHalfBits(b) << 16);
+        *reinterpret_cast<uint32_t*>(operand + t * 256 + 4 * lane) = packed;
+        if (block == 0) *reinterpret_cast<uint32_t*>(a_had + static_cast<int64_t>(t) * k + at) = packed;
+      }
+      __builtin_amdgcn_wave_barrier();
+      asm volatile("" ::: "memory");
+    }
+    const uint32_t x01 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32);
+    const uint32_t x89 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32 + 16);
     Half4 xv;
     xv[0] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 & 0xFFFFu));
     xv[1] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 >> 16));
@@ -278,23 +325,38 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_
     }
     asm volatile("" ::: "memory");
   }
-  // acc[t][q] = D[token 4 g + q][column 16 t + n]
-  float* out = partial + static_cast<int64_t>(blockIdx.y) * m * n + block * 128;
+
+  // The waves' sums through LDS (over the rings, which every wave has left), added in wave
+  // order. acc[t][q] = D[token 4 g + q][column 16 t + n].
+  __syncthreads();
+  float* sums = reinterpret_cast<float*>(lds);  // [wave][8 t + q][lane]
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int row = 4 * p.g + q;
-      if (row < m) out[static_cast<int64_t>(row) * n + t * 16 + p.n] = acc[t][q];
-    }
+    for (int q = 0; q < 4; ++q) sums[(wave * 32 + t * 4 + q) * 64 + lane] = acc[t][q];
+  }
+  __syncthreads();
+  float* out = partial + static_cast<int64_t>(blockIdx.y) * m * n + block * 128;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = tid + j * (kProductWaves * 64);  // of 32 x 64
+    float total = sums[e];
+#pragma unroll
+    for (int w = 1; w < kProductWaves; ++w) total += sums[w * 2048 + e];
+    const int tq = e >> 6, l = e & 63;
+    const int row = 4 * (l >> 4) + (tq & 3);
+    if (row < m) out[static_cast<int64_t>(row) * n + (tq >> 2) * 16 + (l & 15)] = total;
   }
 }
 
-int SlicesFor(int m, int k) {
-  const int steps = k / 16;
-  int want = m <= 2 ? 32 : m <= 8 ? 16 : 8;
-  while (want > 1 && steps / want < 4) want /= 2;
-  return want;
+// Outer slices of K: enough workgroups for about 4096 waves, each wave at least one 128 block.
+int SlicesFor(int n, int k) {
+  const int blocks = k / 128;
+  const int column_blocks = n / 128;
+  int want = (4096 / kProductWaves + column_blocks - 1) / column_blocks;
+  const int most = (blocks + kProductWaves - 1) / kProductWaves;
+  if (want > most) want = most;
+  return want < 1 ? 1 : want;
 }
 
 int CheckWeights(const llmp_exl3_weights& w) {
@@ -318,14 +380,23 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
 }
 
 template <int CB, int BITS>
-void LaunchProduct(const llmp_exl3_weights& w, const void* xh, float* partial, int m, int slices, hipStream_t stream) {
+void LaunchProduct(const llmp_exl3_weights& w, const void* x, void* a_had, float* partial, int m, int slices,
+                   hipStream_t stream) {
   constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
-  const int steps = w.k / 16;
-  const int per = (steps + slices - 1) / slices;
-  const dim3 grid(static_cast<unsigned>((w.n / 128 + kProductWaves - 1) / kProductWaves), static_cast<unsigned>(slices));
-  hipLaunchKernelGGL((ProductKernel<CB, BITS>), grid, dim3(kProductWaves * 64),
-                     static_cast<size_t>(kProductWaves) * kRingDepth * kLoads * 1024, stream,
-                     static_cast<const uint8_t*>(w.trellis), static_cast<const uint16_t*>(xh), partial, m, w.n, w.k, per);
+  constexpr int kWork = kProductWaves * (kRingDepth * kLoads * 1024 + kOperandBytes);
+  constexpr int kLds = kWork > kReduceBytes ? kWork : kReduceBytes;
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ProductKernel<CB, BITS>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    sized = true;
+  }
+  const int blocks = w.k / 128;
+  const int per = (blocks + slices * kProductWaves - 1) / (slices * kProductWaves);
+  const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices));
+  hipLaunchKernelGGL((ProductKernel<CB, BITS>), grid, dim3(kProductWaves * 64), kLds, stream,
+                     static_cast<const uint8_t*>(w.trellis), static_cast<const uint16_t*>(x),
+                     static_cast<const uint16_t*>(w.suh), static_cast<uint16_t*>(a_had), partial, m, w.n, w.k, per);
 }
 
 template <typename F>
@@ -396,7 +467,7 @@ extern "C" int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale,
 
 extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
   if (op == nullptr || op->m <= 0 || op->weights.k <= 0 || op->weights.n <= 0) return 0;
-  return static_cast<size_t>(SlicesFor(op->m, op->weights.k)) * op->m * op->weights.n * sizeof(float);
+  return static_cast<size_t>(SlicesFor(op->weights.n, op->weights.k)) * op->m * op->weights.n * sizeof(float);
 }
 
 extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream) {
@@ -411,14 +482,13 @@ extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, s
     return Refuse(1, "exl3.linear: operands not 8-byte aligned");
   const llmp_exl3_weights& w = op->weights;
   const auto s = static_cast<hipStream_t>(stream);
-  const int slices = SlicesFor(op->m, w.k);
-  // The transformed input, the product's slices, then their sum transformed.
-  hipLaunchKernelGGL((HadamardKernel<0, 0>), dim3(static_cast<unsigned>(op->m), static_cast<unsigned>(w.k / 128)),
-                     dim3(64), 0, s, op->x, op->a_had, static_cast<const uint16_t*>(w.suh), nullptr, w.k, 1, int64_t{0});
-  if (const int bad = LaunchStatus("exl3.linear input transform"); bad != 0) return bad;
+  const int slices = SlicesFor(w.n, w.k);
+  // The product of the transformed input in slices of K, then the slices' sum transformed.
   Dispatch(w.codebook, w.bits, [&](auto cb, auto bits) {
-    LaunchProduct<decltype(cb)::value, decltype(bits)::value>(w, op->a_had, static_cast<float*>(scratch), op->m, slices, s);
+    LaunchProduct<decltype(cb)::value, decltype(bits)::value>(w, op->x, op->a_had, static_cast<float*>(scratch), op->m,
+                                                              slices, s);
   });
+  if (const int bad = LaunchStatus("exl3.linear product"); bad != 0) return bad;
   const dim3 grid(static_cast<unsigned>(op->m), static_cast<unsigned>(w.n / 128));
   const int64_t stride = static_cast<int64_t>(op->m) * w.n;
   if (op->f32) {
