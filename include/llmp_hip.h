@@ -222,8 +222,9 @@ int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, 
  * y (m x n, F16 or F32); a_had is the caller's m x k F16 scratch for the transformed input,
  * which the product's launch writes as it computes it. `scratch` (llmp_hip_exl3_linear_scratch
  * bytes, 8-byte aligned) takes the place of the reference's lock area: the K slices' partial
- * sums, added in slice order. Two launches are queued; a failure after the first is reported as
- * a fault (negative). */
+ * sums, added in slice order. Two launches are queued (three above four rows: the input
+ * transform is then a launch of its own); a failure after the first is reported as a fault
+ * (negative). */
 typedef struct llmp_exl3_linear {
   llmp_exl3_weights weights;
   const void* x;

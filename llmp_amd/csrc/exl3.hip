@@ -233,7 +233,9 @@ constexpr int kReduceBytes = kProductWaves * 32 * 64 * 4;
 // eight waves `blocks_per_wave` 128-blocks of K each: a wave transforms its own activations a
 // block at a time (the workgroups of the first column block also write them to a_had), decodes
 // eight tiles per 16 rows of K, and the waves' sums are added in wave order through LDS.
-template <int CB, int BITS>
+// Every column block repeats the transform, which is cheap for a few tokens only: without
+// kFused, x is the transformed input already and a_had is not written.
+template <int CB, int BITS, bool kFused>
 __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_t* __restrict__ trellis,
                                                                    const uint16_t* __restrict__ x,
                                                                    const uint16_t* __restrict__ suh,
@@ -275,10 +277,11 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_
   for (int t = 0; t < 8; ++t) acc[t] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
   // The activations' operand: token l % 16, k slots in the lane group's row order.
   const uint8_t* my_operand = operand + min(p.n, m - 1) * 256 + 4 * p.g;
+  const uint16_t* my_row = x + static_cast<int64_t>(min(p.n, m - 1)) * k + 2 * p.g;
 
   for (int s = first; s < min(first + kRingDepth - 1, last); ++s) fetch(s);
   for (int step = first; step < last; ++step) {
-    if ((step & 7) == 0) {
+    if (kFused && (step & 7) == 0) {
       // The wave's next 128 values of every token, transformed as the input transform does.
       const int at = (step >> 3) * 128 + 2 * lane;
       const uint32_t sc = *reinterpret_cast<const uint32_t*>(suh + at);
@@ -297,8 +300,14 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_
       __builtin_amdgcn_wave_barrier();
       asm volatile("" ::: "memory");
     }
-    const uint32_t x01 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32);
-    const uint32_t x89 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32 + 16);
+    uint32_t x01, x89;
+    if constexpr (kFused) {
+      x01 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32);
+      x89 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32 + 16);
+    } else {
+      x01 = *reinterpret_cast<const uint32_t*>(my_row + step * 16);
+      x89 = *reinterpret_cast<const uint32_t*>(my_row + step * 16 + 8);
+    }
     Half4 xv;
     xv[0] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 & 0xFFFFu));
     xv[1] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 >> 16));
@@ -379,7 +388,9 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
                      static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
 
-template <int CB, int BITS>
+constexpr int kFusedRows = 4;  // up to here the product transforms its input itself
+
+template <int CB, int BITS, bool kFused>
 void LaunchProduct(const llmp_exl3_weights& w, const void* x, void* a_had, float* partial, int m, int slices,
                    hipStream_t stream) {
   constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
@@ -387,14 +398,14 @@ void LaunchProduct(const llmp_exl3_weights& w, const void* x, void* a_had, float
   constexpr int kLds = kWork > kReduceBytes ? kWork : kReduceBytes;
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ProductKernel<CB, BITS>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ProductKernel<CB, BITS, kFused>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     sized = true;
   }
   const int blocks = w.k / 128;
   const int per = (blocks + slices * kProductWaves - 1) / (slices * kProductWaves);
   const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices));
-  hipLaunchKernelGGL((ProductKernel<CB, BITS>), grid, dim3(kProductWaves * 64), kLds, stream,
+  hipLaunchKernelGGL((ProductKernel<CB, BITS, kFused>), grid, dim3(kProductWaves * 64), kLds, stream,
                      static_cast<const uint8_t*>(w.trellis), static_cast<const uint16_t*>(x),
                      static_cast<const uint16_t*>(w.suh), static_cast<uint16_t*>(a_had), partial, m, w.n, w.k, per);
 }
@@ -483,10 +494,22 @@ extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, s
   const llmp_exl3_weights& w = op->weights;
   const auto s = static_cast<hipStream_t>(stream);
   const int slices = SlicesFor(w.n, w.k);
-  // The product of the transformed input in slices of K, then the slices' sum transformed.
+  // The product of the transformed input in slices of K (for more than a few rows the input
+  // is transformed by a launch of its own first), then the slices' sum transformed.
+  const bool fused = op->m <= kFusedRows;
+  if (!fused) {
+    hipLaunchKernelGGL((HadamardKernel<0, 0>), dim3(static_cast<unsigned>(op->m), static_cast<unsigned>(w.k / 128)),
+                       dim3(64), 0, s, op->x, op->a_had, static_cast<const uint16_t*>(w.suh), nullptr, w.k, 1,
+                       int64_t{0});
+    if (const int bad = LaunchStatus("exl3.linear input transform"); bad != 0) return bad;
+  }
   Dispatch(w.codebook, w.bits, [&](auto cb, auto bits) {
-    LaunchProduct<decltype(cb)::value, decltype(bits)::value>(w, op->x, op->a_had, static_cast<float*>(scratch), op->m,
-                                                              slices, s);
+    constexpr int kCb = decltype(cb)::value, kBits = decltype(bits)::value;
+    if (fused) {
+      LaunchProduct<kCb, kBits, true>(w, op->x, op->a_had, static_cast<float*>(scratch), op->m, slices, s);
+    } else {
+      LaunchProduct<kCb, kBits, false>(w, op->a_had, nullptr, static_cast<float*>(scratch), op->m, slices, s);
+    }
   });
   if (const int bad = LaunchStatus("exl3.linear product"); bad != 0) return bad;
   const dim3 grid(static_cast<unsigned>(op->m), static_cast<unsigned>(w.n / 128));
