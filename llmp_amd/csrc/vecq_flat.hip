@@ -157,27 +157,32 @@ struct FormatQ4K {
     reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
   }
 
-  // One super-block times the staged tokens.
+  // The super-block at `at` (LDS) times the staged tokens. With several tokens a pass the
+  // codes are read a pair of sub-blocks at a time, each pair used by every token before the
+  // next is read: the whole super-block and four tokens' operands do not fit the registers.
 template <int P, bool kDump>
-  static __device__ __forceinline__ void Dot(const SuperBlock& b, const uint8_t* records, int token_stride, int m,
-                                              float (&out)[P], int32_t* dump) {
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                                float (&out)[P], int32_t* dump) {
 #pragma clang fp contract(off)
-  const uint32_t s0 = b.header.y, s1 = b.header.z, s2 = b.header.w;
+  const U32x4* mine = reinterpret_cast<const U32x4*>(at);
+  const U32x4 header = mine[0];
+  const uint32_t s0 = header.y, s1 = header.z, s2 = header.w;
   // Bytes g of sc[0], sc[1]: the scales of sub-blocks g and 4 + g; mn likewise.
   const uint32_t sc[2] = {s0 & 0x3F3F3F3Fu, (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u)};
   const uint32_t mn[2] = {s1 & 0x3F3F3F3Fu, ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u)};
-  const float d = HalfBitsToFloat(b.header.x & 0xFFFFu);
-  const float dmin = HalfBitsToFloat(b.header.x >> 16);
+  const float d = HalfBitsToFloat(header.x & 0xFFFFu);
+  const float dmin = HalfBitsToFloat(header.x >> 16);
   float main[P];
 #pragma unroll
   for (int t = 0; t < P; ++t) main[t] = 0.0f;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     // Pair p: 32 bytes, the low nibbles sub-block 2p, the high ones 2p + 1.
+    if constexpr (P > 1) __builtin_amdgcn_sched_barrier(0);
     int lo[8], hi[8];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const U32x4 raw = b.codes[2 * p + i];
+      const U32x4 raw = mine[1 + 2 * p + i];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         lo[4 * i + c] = static_cast<int>(raw[c] & 0x0F0F0F0Fu);
@@ -302,6 +307,12 @@ struct FormatQ8 {
       dst[8] = w[8] >> 16;
     }
     reinterpret_cast<float*>(record + 136)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+  }
+
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+    Dot<P, kDump>(Read(at), records, token_stride, m, out, dump);
   }
 
   // Four blocks times the staged tokens.
@@ -585,9 +596,9 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
       }
       float out[P];
       if (live) {
-        const typename F::Unit unit = F::Read(my_block + (kDeep ? buffer * kTileBytes : 0));
         int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * F::kDumpInts : nullptr;
-        F::template Dot<P, kDump>(unit, my_records, token_stride, m, out, dump);
+        F::template DotAt<P, kDump>(my_block + (kDeep ? buffer * kTileBytes : 0), my_records, token_stride, m, out,
+                                    dump);
       }
       // Row sums: a suffix sum over each row's lanes (a fixed tree), the total in the row's
       // first lane; a gate row's total then moves to its up row's lane.
@@ -700,9 +711,8 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatSplit(const VecQArgs a, con
       for (int c = 0; c < split; ++c) {
         AwaitTile();
         if (lane < min(piece, units - c * piece)) {
-          const typename F::Unit unit = F::Read(my_block);
           float out[1];
-          F::template Dot<1, false>(unit, lds + (c * piece + lane) * F::kRecord, token_stride, 1, out, nullptr);
+          F::template DotAt<1, false>(my_block, lds + (c * piece + lane) * F::kRecord, token_stride, 1, out, nullptr);
           total += out[0];
         }
         // The next tile may overwrite the buffer: every lane's reads of it were consumed above.
@@ -799,6 +809,15 @@ void LaunchP(const VecQArgs& a, int x_type, dim3 grid, const FlatPlan& plan, boo
   }
 }
 
+// The slots of a routed product whose workgroups own an expert, as far as the host can tell:
+// one token's picks are distinct; several tokens' picks repeat, and about five in eight slots
+// own an expert when they are many.
+int LiveSlots(const llmp_vecq_desc& d, int slots) {
+  if (d.tokens == 1) return slots;
+  const int guess = slots * 5 / 8;
+  return guess > d.used ? guess : d.used;
+}
+
 // A row of more than 64 units in pieces: the fewest pieces, of even length (a Q8_0 unit is 136
 // bytes and a tile is fetched in 16-byte chunks).
 struct SplitPlan {
@@ -845,7 +864,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
       g_compute_units = cus > 0 ? cus : 256;
     }
     const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
-    const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
+    const int live_slots = a.offsets == nullptr && d.ids != nullptr ? LiveSlots(d, slots) : slots;
     int groups = 2 * g_compute_units / (live_slots > 0 ? live_slots : 1);
     if (groups < 1) groups = 1;
     if (groups > (d.nrows + plan.waves - 1) / plan.waves) groups = (d.nrows + plan.waves - 1) / plan.waves;
@@ -869,7 +888,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
   // What is resident at once: two workgroups a CU, shared by the slots that have work.
-  const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
+  const int live_slots = a.offsets == nullptr && d.ids != nullptr ? LiveSlots(d, slots) : slots;
   int groups = (deep ? 1 : 2) * g_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
   if (groups > (tiles + plan.waves - 1) / plan.waves) groups = (tiles + plan.waves - 1) / plan.waves;
