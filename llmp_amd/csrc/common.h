@@ -63,6 +63,23 @@ __device__ __forceinline__ T ShflXor(T v, int mask) {
   return __shfl_xor(v, mask, kWave);
 }
 
+// The largest / smallest value over a full wave's 64 lanes, the same in every lane (and known to
+// the compiler as such). Within a row of 16 lanes by data-parallel moves: lane ^ 1, lane ^ 2,
+// then the mirrored half row and the mirrored row, whose lanes already agree within quads and
+// half rows; across the four rows by lane reads.
+__device__ __forceinline__ uint32_t WaveMaxU32(uint32_t v) {
+  v = max(v, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0xB1, 0xF, 0xF, true)));
+  v = max(v, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x4E, 0xF, 0xF, true)));
+  v = max(v, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x141, 0xF, 0xF, true)));
+  v = max(v, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), 0x140, 0xF, 0xF, true)));
+  const uint32_t a = __builtin_amdgcn_readlane(static_cast<int>(v), 0);
+  const uint32_t b = __builtin_amdgcn_readlane(static_cast<int>(v), 16);
+  const uint32_t c = __builtin_amdgcn_readlane(static_cast<int>(v), 32);
+  const uint32_t d = __builtin_amdgcn_readlane(static_cast<int>(v), 48);
+  return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ uint32_t WaveMinU32(uint32_t v) { return ~WaveMaxU32(~v); }
+
 }  // namespace llmp_hip
 
 #endif  // LLMP_AMD_CSRC_COMMON_H_

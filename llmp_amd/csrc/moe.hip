@@ -52,64 +52,65 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void RouterKernel(const float*
     nan = nan || (have && v[i] != v[i]);
     most = fmaxf(most, v[i]);  // ignores NaN, as std::max(max, v) does
   }
-#pragma unroll
-  for (int mask = 32; mask >= 1; mask >>= 1) most = fmaxf(most, ShflXor(most, mask));
+  // The maximum through keys whose unsigned order is the floats' (a NaN is no maximum here).
+  const auto ordered = [](float f) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, f == 0.0f ? 0.0f : f);  // -0 is +0
+    return (bits & 0x80000000u) != 0 ? ~bits : bits | 0x80000000u;
+  };
+  {
+    const uint32_t top = WaveMaxU32(most != most ? 0u : ordered(most));
+    const uint32_t bits = (top & 0x80000000u) != 0 ? top & 0x7FFFFFFFu : ~top;
+    most = __builtin_bit_cast(float, bits);
+  }
   nan = __any(nan);
   // A row with a NaN or no finite maximum has no probabilities: every expert 0, so the first
   // `used` experts with zero weights (exec.cc:279-299 and the stable order of :303-315).
   const bool degenerate = nan || !(fabsf(most) < INFINITY);
   float sum = 0.0f;
+  uint32_t key[SLOTS];  // 0: not an expert, or picked already
 #pragma unroll
   for (int i = 0; i < SLOTS; ++i) {
     const int e = i * kWave + lane;
     const bool have = i < slots && e < experts;
     p[i] = have && !degenerate ? expf(v[i] - most) : 0.0f;
     sum += p[i];
+    key[i] = !have ? 0u : degenerate ? 1u : ordered(v[i]);
   }
   const float total = WaveSum(sum);
   const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
   // Top `used` by logit (the probabilities' order without their rounding), lower index first
-  // among equals; a degenerate row orders by index alone.
+  // among equals; a degenerate row orders by index alone. A pick: the largest key, then the
+  // lowest index among the lanes that hold it.
   float mine = 0.0f;
   float picked = 0.0f;
   int my_index = 0;
   for (int j = 0; j < used; ++j) {
-    float best = -INFINITY;
-    int index = 0x7FFFFFFF;
-    float best_p = 0.0f;
+    uint32_t best = 0u;
+    uint32_t index = 0x7FFFFFFFu;
 #pragma unroll
     for (int i = 0; i < SLOTS; ++i) {
-      const int e = i * kWave + lane;
-      const bool have = i < slots && e < experts && p[i] >= 0.0f;  // a pick is marked by -1
-      const float key = degenerate ? 0.0f : v[i];
-      if (have && (index == 0x7FFFFFFF || key > best)) {
-        best = key;
-        index = e;
-        best_p = p[i];
+      if (key[i] > best) {  // a lane's slots in index order: the first of equals stays
+        best = key[i];
+        index = static_cast<uint32_t>(i * kWave + lane);
       }
     }
+    const uint32_t top = WaveMaxU32(best);
+    const uint32_t chosen = WaveMinU32(best == top ? index : 0x7FFFFFFFu);
+    const int owner = static_cast<int>(chosen & (kWave - 1));
+    const int slot = static_cast<int>(chosen / kWave);
+    float held = 0.0f;
 #pragma unroll
-    for (int mask = 32; mask >= 1; mask >>= 1) {
-      const float b = ShflXor(best, mask);
-      const int bi = ShflXor(index, mask);
-      const float bp = ShflXor(best_p, mask);
-      const bool take = bi != 0x7FFFFFFF && (index == 0x7FFFFFFF || b > best || (b == best && bi < index));
-      if (take) {
-        best = b;
-        index = bi;
-        best_p = bp;
+    for (int i = 0; i < SLOTS; ++i) {
+      if (i == slot) {
+        held = p[i];
+        if (lane == owner) key[i] = 0u;
       }
     }
-    if (index != 0x7FFFFFFF && (index & (kWave - 1)) == lane) {
-#pragma unroll
-      for (int i = 0; i < SLOTS; ++i) {
-        if (i == index / kWave) p[i] = -1.0f;
-      }
-    }
+    const float best_p = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, held), owner));
     const float q = best_p * inverse;
     if (lane == j) {
       mine = q;
-      my_index = index;
+      my_index = static_cast<int>(chosen);
     }
     picked += q;  // in pick order
   }
