@@ -243,17 +243,28 @@ __global__ void CombineKernel(const float4* __restrict__ x, const float* __restr
   const int64_t c4 = i % width4;
   float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   bool first = true;
-  for (int j = 0; j < used; ++j) {
-    int64_t row = t * used + j;
-    if (position != nullptr) {
-      row = position[row];
-      if (row < 0) continue;
+  // Eight slots' loads in flight at a time; the terms are still added in slot order.
+  for (int j0 = 0; j0 < used; j0 += 8) {
+    int64_t row[8];
+    float w[8];
+    float4 d[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int j = min(j0 + u, used - 1);
+      row[u] = t * used + j;
+      w[u] = weights[row[u]];
+      if (position != nullptr) row[u] = position[row[u]];
+      if (j0 + u >= used) row[u] = -1;
     }
-    const float w = weights[t * used + j];
-    const float4 d = x[row * width4 + c4];
-    const float4 e = make_float4(d.x * w, d.y * w, d.z * w, d.w * w);
-    acc = first ? e : make_float4(acc.x + e.x, acc.y + e.y, acc.z + e.z, acc.w + e.w);
-    first = false;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) d[u] = x[max(row[u], int64_t{0}) * width4 + c4];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (row[u] < 0) continue;
+      const float4 e = make_float4(d[u].x * w[u], d[u].y * w[u], d[u].z * w[u], d[u].w * w[u]);
+      acc = first ? e : make_float4(acc.x + e.x, acc.y + e.y, acc.z + e.z, acc.w + e.w);
+      first = false;
+    }
   }
   out[i] = acc;
 }

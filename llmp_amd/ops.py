@@ -197,6 +197,14 @@ def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWI
     up = gate_up.view(-1)[ffn * (hidden // qk) * bs:]
     down_stride = hidden * (ffn // qk)
     if tokens * used <= 128:
+        if keep is None and tokens * used <= 64:
+            # Nobody asks for the intermediates and the pairs are few: each product quantizes
+            # its activations itself (the same arithmetic, two launches fewer).
+            h = vecq_fused(t, up, x, hidden, ffn, gate=gate, ids=ids, tokens=tokens, used=used,
+                           stride_expert=gu_stride, glu=glu)
+            y = vecq_fused(t, down, h, ffn, hidden, ids=ids, tokens=tokens, used=used, stride_expert=down_stride,
+                           x_token=used * ffn, x_slot=ffn)
+            return moe_combine(y.view(tokens * used, hidden), weights), ids, weights
         q8 = quantize_q8_1(x)
         h = vecq(t, up, q8, hidden, ffn, gate=gate, ids=ids, tokens=tokens, used=used, stride_expert=gu_stride,
                  glu=glu)

@@ -150,6 +150,11 @@ def test_routed_ffn_layer_matches_oracle_stage_by_stage(device, tokens):
     unsorted_y[pairs] = y
     want = oracle.expert_reduce(unsorted_y.reshape(tokens, used, hidden), w.cpu().numpy())
     assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # Without a request for the intermediates the products quantize their activations
+    # themselves: the same bits out.
+    plain, _, _ = ops.moe_ffn(t, dev(logits, device), dev(x, device), dev(gate_up, device), dev(down, device), hidden,
+                              ffn, experts, used)
+    assert np.array_equal(plain.cpu().numpy().view(np.uint32), got.cpu().numpy().view(np.uint32))
     # End to end against the all-CPU layer: the quantization steps bound it, not float order.
     cpu_hq = oracle.q8_1_quantize(want_h)
     cpu_y = oracle.vecq(t, down, cpu_hq, ffn, hidden, ids=want_ids, tokens=tokens, used=used,
