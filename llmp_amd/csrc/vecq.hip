@@ -561,7 +561,9 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   const int tokens = d.tokens;
   // Several tokens of a dense or grouped product over Q8_1 blocks: the matrix cores. A routed product's pairs
   // mostly name different experts, one or two tokens each: the flat form.
-  if (tokens > 1 && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
+  // (Q8_0 from four tokens: below that the flat form's second pass costs less than the matrix-core kernel's
+  // scattered weight reads.)
+  if (tokens > (type == LLMP_TYPE_Q8_0 ? 3 : 1) && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
   while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
@@ -624,10 +626,12 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   const Variant& v = kVariants[variant];
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
   if (v.lanes < 0) {
-    if (!MmaTakes(type, *d)) return Refuse(1, "vecq: the matrix-core form takes Q4_K rows up to 7168 values");
+    if (!MmaTakes(type, *d))
+      return Refuse(1, "vecq: the matrix-core form takes Q4_K rows up to 7168 values and Q8_0 rows of whole 128 values "
+                       "up to 8192 at 4-byte boundaries");
     if (x != nullptr) return Refuse(1, "vecq: the matrix-core form takes Q8_1 activations");
     if (dump != nullptr) return Refuse(1, "vecq: block sums are of the one-token variants");
-    LaunchMma(a, static_cast<hipStream_t>(stream));
+    LaunchMma(type, a, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }
   if (v.lanes == 0) {

@@ -176,9 +176,9 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows = false);
 // `deep`: two tile buffers a wave where the shape allows (one token a pass, packed rows).
 void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream);
 
-// The matrix-core kernel for 2 to 16 tokens a pass over Q8_1 activations (vecq_mma.hip).
+// The matrix-core kernels for 2 to 16 tokens a pass over Q8_1 activations (vecq_mma.hip).
 bool MmaTakes(int type, const llmp_vecq_desc& d);
-void LaunchMma(const VecQArgs& a, hipStream_t stream);
+void LaunchMma(int type, const VecQArgs& a, hipStream_t stream);
 
 }  // namespace llmp_hip
 

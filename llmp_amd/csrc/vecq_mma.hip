@@ -371,51 +371,349 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
   }
 }
 
+// ------------------------------------------------------------------ Q8_0
+//
+// The same instruction over Q8_0 blocks: its K is a block, a product the block's int32 sum.
+// The float operations are the one-token kernel's: over a unit of four blocks
+//   v = float(s_0) * (dw_0 * d8_0), then v = fma(float(s_j), dw_j * d8_j, v), j = 1 .. 3,
+// and a row's units are added in that kernel's tree. A tile of 16 rows is taken by four waves,
+// each a quarter of the tree's leaves (the next power of two at or above the row's units, cut in
+// four aligned runs of up to sixteen units), which meet in LDS.
+//
+// A lane reads its row's weights straight into the operand layout: of every pair of blocks
+// (68 bytes, so 4-byte aligned in a row of whole pairs) the eight codes of its K group in the
+// even block lie two bytes into three dwords, those of the odd block in two dwords. The tokens
+// are staged once a workgroup:
+//   codes   [block][K group][token] 8 bytes (a wave's read is a contiguous 512 bytes);
+//   scales  [block][token] F32, a lane reading its four tokens' 16 bytes.
+
+constexpr int kQ8CodesBlock = 4 * kMmaTokens * 8;  // 512 bytes of codes a block
+constexpr int kQ8ScalesBlock = kMmaTokens * 4;     // 64 bytes of scales a block
+constexpr int kQ8Chunks = 4;                       // waves a tile
+constexpr int kQ8Tiles = kMmaWaves / kQ8Chunks;    // tiles a workgroup at a time
+
+struct __attribute__((packed, aligned(4))) Dwords3 {
+  uint32_t a, b, c;
+};
+
+// A lane's part of one unit (four blocks, 136 bytes) of its weight row. The blocks' F16 scales
+// lie in what the row's first and last K group read anyway (bytes 0-1 of a pair in the first's
+// even dwords, bytes 34-35 in the last's) and reach the row's other lanes by a lane exchange:
+// fewer memory requests, which bound this access pattern.
+struct UnitPart {
+  Dwords3 even[2];  // bytes 8 kg .. 8 kg + 11 of each pair: the even block's codes from byte 2
+  uint2 odd[2];     // bytes 36 + 8 kg .. of each pair: the odd block's codes
+};
+
+__device__ __forceinline__ UnitPart LoadUnitPart(const uint8_t* row, int unit, int kg) {
+  UnitPart part;
+  const uint8_t* at = row + static_cast<int64_t>(unit) * 136;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    part.even[i] = *reinterpret_cast<const Dwords3*>(at + 68 * i + 8 * kg);
+    part.odd[i] = *reinterpret_cast<const uint2*>(at + 68 * i + 36 + 8 * kg);
+  }
+  return part;
+}
+
+// One unit of one matrix times the staged tokens: four tokens of this lane's row.
+__device__ __forceinline__ void DotUnit(const UnitPart& part, const uint8_t* codes, const uint8_t* scales, int unit,
+                                        int lane, float (&out)[4]) {
+#pragma clang fp contract(off)
+  const int kg = lane >> 4;
+  // The even blocks' scales from the row's lane of K group 0, the odd blocks' from K group 3's.
+  const uint32_t evens = __shfl((part.even[0].a & 0xFFFFu) | (part.even[1].a << 16), lane & 15, kWave);
+  const uint32_t odds = __shfl((part.even[0].c >> 16) | (part.even[1].c & 0xFFFF0000u), (lane & 15) + 48, kWave);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int64_t weights;
+    const uint32_t both = (j & 1) == 0 ? evens : odds;
+    const float dw = HalfBitsToFloat((j >> 1) == 0 ? both & 0xFFFFu : both >> 16);
+    if ((j & 1) == 0) {
+      const Dwords3& e = part.even[j >> 1];
+      weights = Pack(__builtin_amdgcn_alignbit(e.b, e.a, 16), __builtin_amdgcn_alignbit(e.c, e.b, 16));
+    } else {
+      weights = Pack(part.odd[j >> 1].x, part.odd[j >> 1].y);
+    }
+    const int block = 4 * unit + j;
+    const int64_t tokens = *reinterpret_cast<const int64_t*>(codes + block * kQ8CodesBlock + lane * 8);
+    const float4 d8 = *reinterpret_cast<const float4*>(scales + block * kQ8ScalesBlock + kg * 16);
+    const V4i zero = {0, 0, 0, 0};
+    const V4i prod = __builtin_amdgcn_mfma_i32_16x16x32_i8(tokens, weights, zero, 0, 0, 0);
+    const float d[4] = {d8.x, d8.y, d8.z, d8.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      out[q] = j == 0 ? static_cast<float>(prod[q]) * (dw * d[q]) : fmaf(static_cast<float>(prod[q]), dw * d[q], out[q]);
+    }
+  }
+}
+
+template <class RowOf>
+__device__ __forceinline__ void StageTokensQ8(RowOf row_of, int m, int blocks, uint8_t* codes, uint8_t* scales) {
+  for (int index = threadIdx.x; index < m * blocks; index += kMmaGroup) {
+    const int j = index / blocks, b = index - j * blocks;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(j) + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+#pragma unroll
+    for (int kg = 0; kg < 4; ++kg) {
+      *reinterpret_cast<uint2*>(codes + b * kQ8CodesBlock + (kg * kMmaTokens + j) * 8) =
+          make_uint2(w[1 + 2 * kg], w[2 + 2 * kg]);
+    }
+    *reinterpret_cast<float*>(scales + b * kQ8ScalesBlock + j * 4) = HalfBitsToFloat(w[0] & 0xFFFFu);
+  }
+}
+
+// grid (workgroups, slots); LDS: codes, scales, the waves' partial sums.
+template <bool kGlu>
+__global__ __launch_bounds__(kMmaGroup, 1) void VecQMmaQ8(const VecQArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int pairs[kMaxPairs];
+  __shared__ int count;
+
+  const llmp_vecq_desc& d = a.d;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int blocks = d.ncols_x / 32;
+  const int units = blocks / 4;
+  uint8_t* codes = lds;
+  uint8_t* scales = lds + blocks * kQ8CodesBlock;
+  float4* partial = reinterpret_cast<float4*>(lds + blocks * (kQ8CodesBlock + kQ8ScalesBlock));
+
+  int expert = blockIdx.y;
+  int sorted_first = 0;
+  if (a.offsets != nullptr) {
+    sorted_first = a.offsets[expert];
+    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+    __syncthreads();
+  } else if (d.ids != nullptr) {
+    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
+  }
+  const bool listed = d.ids != nullptr && a.offsets == nullptr;
+  const int n = a.offsets == nullptr && d.ids == nullptr ? d.tokens : count;
+  if (n == 0) return;  // uniform over the workgroup
+  auto pair_at = [&](int i) {
+    return a.offsets != nullptr ? (sorted_first + i) << 8 : listed ? pairs[i] : (i << 8) | expert;
+  };
+  const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
+
+  // This wave's run of the row's units.
+  int leaves = 1;
+  while (leaves < units) leaves *= 2;
+  const int run = max(leaves / kQ8Chunks, 1);
+  const int chunk = wave & (kQ8Chunks - 1);
+  const int first = min(chunk * run, units);
+  const int last = min(first + run, units);
+  const int tile_in_group = wave / kQ8Chunks;
+  const int row_in_tile = lane & 15, kg = lane >> 4;
+  const int tiles = (d.nrows + 15) / 16;
+  const int groups = (tiles + kQ8Tiles - 1) / kQ8Tiles;
+
+  const uint8_t* up_row = nullptr;
+  const uint8_t* gate_row = nullptr;
+  auto aim = [&](int group) {
+    const int row = min((group * kQ8Tiles + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
+    const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 34;
+    up_row = static_cast<const uint8_t*>(d.w) + at;
+    if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
+  };
+  // Four units a matrix in flight; the loads are queued where they are written (past the run's
+  // end the last unit again: no branch).
+  UnitPart u0, u1, u2, u3, g0, g1, g2, g3;
+  auto fetch = [&](int unit, UnitPart& u, UnitPart& g) {
+    const int at = max(min(unit, last - 1), 0);
+    u = LoadUnitPart(up_row, at, kg);
+    if constexpr (kGlu) g = LoadUnitPart(gate_row, at, kg);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  aim(blockIdx.x);
+  fetch(first, u0, g0);
+  fetch(first + 1, u1, g1);
+  fetch(first + 2, u2, g2);
+  fetch(first + 3, u3, g3);
+
+  for (int p0 = 0; p0 < n; p0 += kMmaTokens) {
+    const int m = min(kMmaTokens, n - p0);
+    __syncthreads();  // the last pass's readers of the staged tokens
+    auto row_of = [&](int j) {
+      const int pr = pair_at(p0 + j);
+      return static_cast<const uint8_t*>(d.y) +
+             (static_cast<int64_t>(pr >> 8) * d.y_token + static_cast<int64_t>(pr & 0xFF) * d.y_slot) * kQ8Block;
+    };
+    StageTokensQ8(row_of, m, blocks, codes, scales);
+    __syncthreads();
+
+    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+      const int tile = group * kQ8Tiles + tile_in_group;
+      TreeSum up_sum{}, gate_sum{};
+      int quads = 0;
+      auto step = [&](int unit, const UnitPart& u, const UnitPart& g, float (&up_out)[4], float (&gate_out)[4]) {
+        DotUnit(u, codes, scales, unit, lane, up_out);
+        if constexpr (kGlu) DotUnit(g, codes, scales, unit, lane, gate_out);
+      };
+      if (tile < tiles) {
+        for (int unit = first; unit < last; unit += 4, ++quads) {
+          const int here = min(4, last - unit);
+          // The quad's sum as its values come: (x0 + x1) + (x2 + x3), absent ones left out.
+          float up_quad[4], gate_quad[4], up_next[4], gate_next[4];
+          step(unit, u0, g0, up_quad, gate_quad);
+          fetch(unit + 4, u0, g0);
+          if (here >= 2) {
+            step(unit + 1, u1, g1, up_next, gate_next);
+            Sum4(up_quad, up_next, up_quad);
+            if constexpr (kGlu) Sum4(gate_quad, gate_next, gate_quad);
+          }
+          fetch(unit + 5, u1, g1);
+          if (here >= 3) {
+            float up_rest[4], gate_rest[4];
+            step(unit + 2, u2, g2, up_rest, gate_rest);
+            if (here >= 4) {
+              step(unit + 3, u3, g3, up_next, gate_next);
+              Sum4(up_rest, up_next, up_rest);
+              if constexpr (kGlu) Sum4(gate_rest, gate_next, gate_rest);
+            }
+            Sum4(up_quad, up_rest, up_quad);
+            if constexpr (kGlu) Sum4(gate_quad, gate_rest, gate_quad);
+          }
+          fetch(unit + 6, u2, g2);
+          fetch(unit + 7, u3, g3);
+          Push(up_sum, up_quad, quads);
+          if constexpr (kGlu) Push(gate_sum, gate_quad, quads);
+        }
+      }
+      // The next group's (or the next pass's first group's) first loads.
+      {
+        int next = group + static_cast<int>(gridDim.x);
+        if (next >= groups) next = blockIdx.x;
+        aim(next);
+        fetch(first, u0, g0);
+        fetch(first + 1, u1, g1);
+        fetch(first + 2, u2, g2);
+        fetch(first + 3, u3, g3);
+      }
+      // The four runs meet: (r0 + r1) + (r2 + r3), absent ones left out, through LDS.
+      float up_total[4] = {0.0f, 0.0f, 0.0f, 0.0f}, gate_total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (tile < tiles && last > first) {
+        Total(up_sum, quads, up_total);
+        if constexpr (kGlu) Total(gate_sum, quads, gate_total);
+      }
+      float4* slot = partial + (wave * 2) * kWave + lane;
+      if (chunk != 0) {
+        slot[0] = make_float4(up_total[0], up_total[1], up_total[2], up_total[3]);
+        if constexpr (kGlu) slot[kWave] = make_float4(gate_total[0], gate_total[1], gate_total[2], gate_total[3]);
+      }
+      __syncthreads();
+      if (chunk == 0 && tile < tiles) {
+#pragma clang fp contract(off)
+        auto merge = [&](int matrix, float (&total)[4]) {
+          const float4* other = partial + (wave * 2 + matrix) * kWave + lane;  // this tile's runs follow this wave
+          float rest[4];
+          const bool has1 = run < units, has2 = 2 * run < units, has3 = 3 * run < units;
+          if (has1) {
+            const float4 r1 = other[2 * kWave];
+            total[0] += r1.x, total[1] += r1.y, total[2] += r1.z, total[3] += r1.w;
+          }
+          if (has2) {
+            const float4 r2 = other[4 * kWave];
+            rest[0] = r2.x, rest[1] = r2.y, rest[2] = r2.z, rest[3] = r2.w;
+            if (has3) {
+              const float4 r3 = other[6 * kWave];
+              rest[0] += r3.x, rest[1] += r3.y, rest[2] += r3.z, rest[3] += r3.w;
+            }
+            total[0] += rest[0], total[1] += rest[1], total[2] += rest[2], total[3] += rest[3];
+          }
+        };
+        merge(0, up_total);
+        if constexpr (kGlu) merge(1, gate_total);
+        if (tile * 16 + row_in_tile < d.nrows) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int t = 4 * kg + q;
+            if (t < m) {
+              const int pr = pair_at(p0 + t);
+              float* dst = d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
+              dst[tile * 16 + row_in_tile] = kGlu ? Glu(d.glu, gate_total[q], up_total[q], d.limit) : up_total[q];
+            }
+          }
+        }
+      }
+      __syncthreads();  // the partial sums may be overwritten
+    }
+  }
+}
+
+size_t MmaLdsQ8(int blocks) {
+  return static_cast<size_t>(blocks) * (kQ8CodesBlock + kQ8ScalesBlock) + kPartialBytes;
+}
+
 size_t MmaLds(int nsb) { return static_cast<size_t>(nsb) * (kCodesSb + kScalesSb) + kPartialBytes; }
 
 int g_mma_compute_units = 0;
 
 }  // namespace
 
-// Q4_K rows whose sixteen staged tokens fit LDS (k up to 7168).
+// Q4_K rows whose sixteen staged tokens fit LDS (k up to 7168). Q8_0 rows of whole units of
+// 128 values, up to 64 units (8192 values) as far as they fit LDS, whose rows, matrices and
+// experts start on 4-byte boundaries (a lane reads dwords).
 bool MmaTakes(int type, const llmp_vecq_desc& d) {
-  if (type != LLMP_TYPE_Q4_K) return false;
-  const int nsb = d.ncols_x / 256;
-  return nsb >= 1 && MmaLds(nsb) <= kMmaLdsLimit;
+  if (type == LLMP_TYPE_Q4_K) {
+    const int nsb = d.ncols_x / 256;
+    return nsb >= 1 && MmaLds(nsb) <= kMmaLdsLimit;
+  }
+  if (type != LLMP_TYPE_Q8_0 || d.ncols_x < 128 || d.ncols_x % 128 != 0 || d.ncols_x > 8192) return false;
+  const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+  return d.stride_row % 2 == 0 && d.stride_expert % 2 == 0 && at % 4 == 0 && MmaLdsQ8(d.ncols_x / 32) <= kMmaLdsLimit;
 }
 
-void LaunchMma(const VecQArgs& a, hipStream_t stream) {
+namespace {
+
+template <bool kQ8, bool kGlu>
+void LaunchMmaKernel(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if constexpr (kQ8) {
+    if (!sized) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMmaQ8<kGlu>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
+      sized = true;
+    }
+    hipLaunchKernelGGL((VecQMmaQ8<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
+  } else {
+    if (!sized) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<kGlu>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
+      sized = true;
+    }
+    hipLaunchKernelGGL((VecQMma<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
+  }
+}
+
+}  // namespace
+
+void LaunchMma(int type, const VecQArgs& a, hipStream_t stream) {
   const llmp_vecq_desc& d = a.d;
+  const bool q8 = type == LLMP_TYPE_Q8_0;
   const int nsb = d.ncols_x / 256;
-  const size_t lds = MmaLds(nsb);
+  const size_t lds = q8 ? MmaLdsQ8(d.ncols_x / 32) : MmaLds(nsb);
   if (g_mma_compute_units == 0) {
     const int cus = llmp_hip_compute_units();
     g_mma_compute_units = cus > 0 ? cus : 256;
   }
   const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + 15) / 16;
-  const int tiles_group = nsb <= kWholeRow ? kMmaWaves : kTilesGroup;
+  const int tiles_group = q8 ? kQ8Tiles : nsb <= kWholeRow ? kMmaWaves : kTilesGroup;
   const int tile_groups = (tiles + tiles_group - 1) / tiles_group;
   const int live_slots = a.offsets == nullptr && d.ids != nullptr ? (d.used < slots ? d.used : slots) : slots;
   int groups = g_mma_compute_units / (live_slots > 0 ? live_slots : 1);
   if (groups < 1) groups = 1;
   if (groups > tile_groups) groups = tile_groups;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
-  static bool sized[2] = {false, false};
-  if (d.g != nullptr) {
-    if (!sized[1]) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
-      sized[1] = true;
-    }
-    hipLaunchKernelGGL((VecQMma<true>), grid, dim3(kMmaGroup), lds, stream, a);
+  const bool glu = d.g != nullptr;
+  if (q8) {
+    glu ? LaunchMmaKernel<true, true>(a, grid, lds, stream) : LaunchMmaKernel<true, false>(a, grid, lds, stream);
   } else {
-    if (!sized[0]) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
-      sized[0] = true;
-    }
-    hipLaunchKernelGGL((VecQMma<false>), grid, dim3(kMmaGroup), lds, stream, a);
+    glu ? LaunchMmaKernel<false, true>(a, grid, lds, stream) : LaunchMmaKernel<false, false>(a, grid, lds, stream);
   }
 }
 

@@ -74,10 +74,13 @@ def test_other_entry_points_refuse_bad_operands():
     lib = _lib.load()
     assert lib.llmp_hip_vecq(12, None, -1, None) > 0
     assert lib.llmp_hip_vecq(12, C.byref(desc()), 99, None) > 0
-    # The flat form takes Q8_0 rows of whole 256 values at 16-byte boundaries only; the matrix-core form Q4_K only.
+    # The flat form takes Q8_0 rows of whole 256 values at 16-byte boundaries only; the matrix-core form Q8_0 rows
+    # of whole 128 values, an even number of blocks apart.
     assert lib.llmp_hip_vecq(8, C.byref(desc(ncols_x=480, stride_row=15)), 6, None) > 0
     assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=17)), 6, None) > 0
-    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=16, tokens=4)), 9, None) > 0
+    assert lib.llmp_hip_vecq(8, C.byref(desc(ncols_x=480, stride_row=16, tokens=4)), 9, None) > 0
+    assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=17, tokens=4)), 9, None) > 0
+    assert lib.llmp_hip_vecq(3, C.byref(desc(tokens=4)), 9, None) > 0
     assert lib.llmp_hip_vecq_fused(12, C.byref(desc()), None, -1, None) > 0
     assert lib.llmp_hip_vecq_block_sums(12, C.byref(desc()), -1, None, None) > 0
     assert lib.llmp_hip_q8_1_quantize(None, None, 32, 512, 32, 1, 1, 32, None) > 0

@@ -98,10 +98,6 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
-        if name.startswith("mma") and t != Q4_K:  # the matrix-core form is Q4_K's
-            with pytest.raises(ops.KernelFailure):
-                ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
-            continue
         got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
         ok, worst = rel_close(got, want, TOL)
         assert ok, (variant, worst)
@@ -183,11 +179,14 @@ def test_routed_and_sorted_long_rows_match_oracle(device, t, k):
     assert np.array_equal(sorted_out.view(np.uint32), got.reshape(tokens * used, n)[order].view(np.uint32))
 
 
-@pytest.mark.parametrize("k,n,tokens", [(2816, 50, 5), (256, 17, 2), (6144, 32, 16), (2048, 130, 9)])
-def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, k, n, tokens):
-    """The int8 matrix-core kernel (variant 9) repeats the flat kernel's float operations and its
+@pytest.mark.parametrize("t,k,n,tokens", [(Q4_K, 2816, 50, 5), (Q4_K, 256, 17, 2), (Q4_K, 6144, 32, 16),
+                                          (Q4_K, 2048, 130, 9), (Q8_0, 4096, 50, 5), (Q8_0, 256, 17, 2),
+                                          (Q8_0, 3840, 20, 16), (Q8_0, 1792, 130, 9), (Q8_0, 768, 33, 3)])
+def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, t, k, n, tokens):
+    """The int8 matrix-core kernels (variant 9) repeat the flat kernel's float operations and its
     summation tree: dense with and without a GLU, grouped matrices, and routed experts."""
-    t, mma, flat = Q4_K, 9, 7
+    mma, flat = 9, 7
+    qk = oracle.block_elements(t)
     gate, up = make_weights(t, n, k, 301), make_weights(t, n, k, 302)
     q8 = ops.quantize_q8_1(dev(synth.activations(tokens, k, 303), device))
     wd, gd = dev(up, device), dev(gate, device)
@@ -200,7 +199,7 @@ def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, k, n, tokens)
     w3 = dev(make_weights(t, groups * n, k, 304).reshape(groups, -1), device)
     q83 = ops.quantize_q8_1(dev(synth.activations(tokens * groups, k, 305), device))
     y_row = ops.padded_k(k) // 32
-    kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // 256), y_token=y_row * groups, y_slot=y_row)
+    kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // qk), y_token=y_row * groups, y_slot=y_row)
     a = ops.vecq(t, w3, q83, k, n, variant=mma, **kw).cpu().numpy()
     b = ops.vecq(t, w3, q83, k, n, variant=flat, **kw).cpu().numpy()
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
@@ -209,7 +208,7 @@ def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, k, n, tokens)
     w5 = dev(make_weights(t, experts * n, k, 306).reshape(experts, -1), device)
     g = synth.rng(307)
     ids = dev(np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32), device)
-    kw = dict(ids=ids, tokens=tokens, used=used, stride_expert=n * (k // 256))
+    kw = dict(ids=ids, tokens=tokens, used=used, stride_expert=n * (k // qk))
     a = ops.vecq(t, w5, q8, k, n, variant=mma, **kw).cpu().numpy()
     b = ops.vecq(t, w5, q8, k, n, variant=flat, **kw).cpu().numpy()
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
