@@ -58,9 +58,33 @@ __device__ __forceinline__ int Dot4(int a, int b, int c) {
 typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 typedef U32x4 U32x4A4 __attribute__((aligned(4)));
 
+// The value of lane `lane ^ mask` (every lane of the 2 * mask group active). Within a row of 16
+// lanes by data-parallel moves, which cost a few cycles where a permute through LDS costs its
+// latency: lane ^ 1 and lane ^ 2 are quad permutes, lane ^ 8 a rotation of the row by eight,
+// lane ^ 4 a shift by four either way, each on the banks of four lanes it is right for.
 template <typename T>
 __device__ __forceinline__ T ShflXor(T v, int mask) {
-  return __shfl_xor(v, mask, kWave);
+  static_assert(sizeof(T) == 4, "32-bit values");
+  const int bits = __builtin_bit_cast(int, v);
+  int got;
+  switch (mask) {
+    case 1:
+      got = __builtin_amdgcn_mov_dpp(bits, 0xB1, 0xF, 0xF, true);  // quad_perm:[1,0,3,2]
+      break;
+    case 2:
+      got = __builtin_amdgcn_mov_dpp(bits, 0x4E, 0xF, 0xF, true);  // quad_perm:[2,3,0,1]
+      break;
+    case 4:
+      got = __builtin_amdgcn_update_dpp(bits, bits, 0x104, 0xF, 0x5, false);  // row_shl:4, banks 0 and 2
+      got = __builtin_amdgcn_update_dpp(got, bits, 0x114, 0xF, 0xA, false);   // row_shr:4, banks 1 and 3
+      break;
+    case 8:
+      got = __builtin_amdgcn_mov_dpp(bits, 0x128, 0xF, 0xF, true);  // row_ror:8
+      break;
+    default:
+      return __shfl_xor(v, mask, kWave);
+  }
+  return __builtin_bit_cast(T, got);
 }
 
 // The largest / smallest value over a full wave's 64 lanes, the same in every lane (and known to
