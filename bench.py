@@ -105,7 +105,7 @@ def other_configs(device, args):
     x = dev(synth.activations(1, k, 202))
     q8 = ops.quantize_q8_1(x)
     y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
-    us = event_us(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 200)
+    us = graph_us(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 4 * len(copies))
     bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
     out["q8_0_matvec_4096x4096_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
                                        "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
@@ -119,11 +119,24 @@ def other_configs(device, args):
     for tokens in (4, 8):
         q8 = ops.quantize_q8_1(dev(synth.activations(tokens, K, 203)))
         y = torch.empty((tokens, 1, N), dtype=torch.float32, device=device)
-        us = event_us(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
-                                         glu=ops.GLU_GEGLU, out=y), 100)
+        us = graph_us(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
+                                         glu=ops.GLU_GEGLU, out=y), 4 * count)
         out[f"q4_k_gate_up_geglu_b{tokens}"] = {"us": round(us, 2),
                                                 "GB/s": round(algorithmic_bytes(tokens) / us / 1e3, 1)}
     del gates, ups, gate, up
+    torch.cuda.empty_cache()
+
+    # The same layer's down projection (15360 -> 3840, Q4_K, one token): rows of 60 super-blocks.
+    kd, nd = N, K
+    wdn = dev(synth.q4_k_weights(nd, kd, 104))
+    downs = [wdn] + [wdn.clone() for _ in range(-(-ROTATE_BYTES // wdn.numel()) - 1)]
+    q8 = ops.quantize_q8_1(dev(synth.activations(1, kd, 105)))
+    y = torch.empty((1, 1, nd), dtype=torch.float32, device=device)
+    us = graph_us(lambda i: ops.vecq(ops.TYPE_Q4_K, downs[i % len(downs)], q8, kd, nd, out=y), 4 * len(downs))
+    bytes_ = wdn.numel() + kd * 4 + nd * 4
+    out["q4_k_down_15360x3840_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
+                                      "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del downs, wdn
     torch.cuda.empty_cache()
 
     # Config 3: MXFP8 GEMM 2048 x 12288 x 4096, bf16 out, and its activation quantizer.
@@ -157,8 +170,9 @@ def other_configs(device, args):
         eager = event_us(layer, 20 if tokens == 512 else 50)
         entry = {"us": round(us, 1), "us_launched_from_python": round(eager, 1), "distinct_experts": distinct,
                  "GB/s_of_touched_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),
-                 "note": "whole layer replayed as a HIP graph: router, q8_1, gate/up+GLU, q8_1, down, combine; "
-                         "weights not rotated"}
+                 "note": "whole layer replayed as a HIP graph: router, [q8_1,] gate/up+GLU, [q8_1,] down, combine "
+                         "(up to 64 pairs the products quantize their activations themselves; above 128 "
+                         "pairs the rows are sorted by expert first); weights not rotated"}
         if tokens == 512:
             entry["TFLOP/s"] = round(tokens * used * 3 * 2.0 * hidden * ffn / us / 1e6, 2)
         out[f"moe_q4_k_ffn_t{tokens}"] = entry
@@ -184,10 +198,10 @@ def other_configs(device, args):
 
 
 # HBM bytes per launch of the dominant kernel at batch 1 through the default variant, from two
-# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,476.2 KiB and WRITE_SIZE 60.1 KiB per dispatch,
+# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,475.1 KiB and WRITE_SIZE 60.2 KiB per dispatch,
 # scaled by 1.9988 and 1.0: what the same counters read for --calibrate-copy's copy of 64,800 KiB).
 # Counters cannot be read from inside a run, so other shapes and variants report null.
-PROFILED_TRAFFIC_BYTES = int(round((32476.2 * 1.9988 + 60.1) * 1024))
+PROFILED_TRAFFIC_BYTES = int(round((32475.1 * 1.9988 + 60.2) * 1024))
 
 
 def measured_traffic(args):
