@@ -54,18 +54,44 @@ __device__ __forceinline__ float ByteOf(uint32_t word, int byte) {
 
 // A lane's part of one super-block of its weight row: the header and, for each pair of
 // sub-blocks, the eight code bytes of its K group (low nibbles sub-block 2 p, high 2 p + 1).
+// As loaded, lane (row, j) holds the whole 32 bytes of pair j instead (two 16-byte loads
+// where four 8-byte ones would be needed: these scattered reads cost by the instruction), K
+// group g's eight bytes in q[g]; Transpose exchanges them among the row's four lanes.
 struct RowPart {
   U32x4 header;  // d, dmin, scales[12]
   uint2 q[4];
 };
 
+typedef unsigned Swapped __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ RowPart LoadRowPart(const uint8_t* row, int sb, int kg) {
   RowPart part;
   const uint8_t* at = row + static_cast<int64_t>(sb) * 144;
   part.header = *reinterpret_cast<const U32x4*>(at);
-#pragma unroll
-  for (int p = 0; p < 4; ++p) part.q[p] = *reinterpret_cast<const uint2*>(at + 16 + 32 * p + 8 * kg);
+  const U32x4 lo = *reinterpret_cast<const U32x4*>(at + 16 + 32 * kg);
+  const U32x4 hi = *reinterpret_cast<const U32x4*>(at + 32 + 32 * kg);
+  part.q[0] = make_uint2(lo.x, lo.y);
+  part.q[1] = make_uint2(lo.z, lo.w);
+  part.q[2] = make_uint2(hi.x, hi.y);
+  part.q[3] = make_uint2(hi.z, hi.w);
   return part;
+}
+
+// q[g] of the row's lane j becomes q[j] of its lane g (the lanes of a row are 16 apart): a
+// 4 x 4 transpose in two rounds of row swaps, lanes 32 apart then lanes 16 apart. Every lane
+// of the wave takes part.
+__device__ __forceinline__ void Transpose(RowPart& part) {
+  uint32_t* w = reinterpret_cast<uint32_t*>(part.q);  // q[g] = w[2 g], w[2 g + 1]
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    uint32_t x0 = w[half], x1 = w[2 + half], x2 = w[4 + half], x3 = w[6 + half];
+    const Swapped a = __builtin_amdgcn_permlane32_swap(x0, x2, false, false);
+    const Swapped b = __builtin_amdgcn_permlane32_swap(x1, x3, false, false);
+    x0 = a.x, x2 = a.y, x1 = b.x, x3 = b.y;
+    const Swapped c = __builtin_amdgcn_permlane16_swap(x0, x1, false, false);
+    const Swapped e = __builtin_amdgcn_permlane16_swap(x2, x3, false, false);
+    w[half] = c.x, w[2 + half] = c.y, w[4 + half] = e.x, w[6 + half] = e.y;
+  }
 }
 
 // The decoded header of a super-block: 6-bit scales and minimums as bytes g of sc[g / 4],
@@ -138,9 +164,11 @@ __device__ __forceinline__ void Total(const TreeSum& t, int count, float (&out)[
 // One super-block of one matrix times the staged tokens: four tokens of this lane's row.
 // `a`: the tokens' codes as first operands, sub-block by sub-block; `entries[4 q + p]`: token
 // q's four scale floats of pair p (in LDS, read a pair at a time).
-__device__ __forceinline__ void DotPart(const RowPart& part, const int64_t (&a)[8], const float4* entries,
+__device__ __forceinline__ void DotPart(const RowPart& loaded, const int64_t (&a)[8], const float4* entries,
                                         float (&out)[4]) {
 #pragma clang fp contract(off)
+  RowPart part = loaded;
+  Transpose(part);
   const Header h = Decode(part.header);
   float main[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   float mins[4];
