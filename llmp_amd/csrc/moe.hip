@@ -141,21 +141,33 @@ __device__ __forceinline__ int StageChunkIds(const int32_t* __restrict__ ids, in
   const int n = (t1 - t0) * r.used;
   for (int i = threadIdx.x; i < n; i += blockDim.x)
     staged[i] = ids[static_cast<int64_t>(t0 + i / r.used) * ids_stride + i % r.used];
+  // Padded to whole groups of four with an id nothing equals: the walks read four at a time.
+  if (threadIdx.x < 4 && n + threadIdx.x < ((n + 3) & ~3)) staged[n + threadIdx.x] = INT32_MIN;
   __syncthreads();
   return n;
 }
 
+// How many of staged[0 .. end) equal e, four ids a read (end a multiple of four, or the padded
+// count).
+__device__ __forceinline__ int CountEqual(const int32_t* staged, int end, int e) {
+  const int4* four = reinterpret_cast<const int4*>(staged);
+  int n = 0;
+#pragma unroll 4
+  for (int i = 0; i < end / 4; ++i) {
+    const int4 v = four[i];
+    n += (v.x == e) + (v.y == e) + (v.z == e) + (v.w == e);
+  }
+  return n;
+}
+
 __global__ void RouteCount(const int32_t* __restrict__ ids, int ids_stride, Route r) {
-  extern __shared__ int32_t staged[];
+  extern __shared__ __attribute__((aligned(16))) int32_t staged[];
   const int c = blockIdx.x;
   const int t0 = c * kRouteChunk;
   const int t1 = min(t0 + kRouteChunk, r.tokens);
   const int slots = StageChunkIds(ids, ids_stride, r, t0, t1, staged);
-  for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
-    int n = 0;
-    for (int i = 0; i < slots; ++i) n += staged[i] == e;
-    r.counts[static_cast<int64_t>(c) * r.experts + e] = n;
-  }
+  for (int e = threadIdx.x; e < r.experts; e += blockDim.x)
+    r.counts[static_cast<int64_t>(c) * r.experts + e] = CountEqual(staged, (slots + 3) & ~3, e);
 }
 
 // One workgroup: each expert's chunk counts become the chunks' bases, then the experts'
@@ -164,21 +176,33 @@ __global__ void RouteScan(Route r) {
   extern __shared__ int total[];
   for (int e = threadIdx.x; e < r.experts; e += blockDim.x) {
     int running = 0;
-    for (int c = 0; c < r.chunks; ++c) {
-      int32_t* at = r.counts + static_cast<int64_t>(c) * r.experts + e;
-      const int v = *at;
-      *at = running;
-      running += v;
+    // Eight chunks' counts in flight at a time (a load after a store to the same array would
+    // otherwise wait for it).
+    for (int c0 = 0; c0 < r.chunks; c0 += 8) {
+      int v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = r.counts[static_cast<int64_t>(min(c0 + u, r.chunks - 1)) * r.experts + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (c0 + u < r.chunks) {
+          r.counts[static_cast<int64_t>(c0 + u) * r.experts + e] = running;
+          running += v[u];
+        }
+      }
     }
     total[e] = running;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
+    int offset = 0, scale_row = 0;
     r.offsets[0] = 0;
     r.scale_rows[0] = 0;
     for (int e = 0; e < r.experts; ++e) {
-      r.offsets[e + 1] = r.offsets[e] + total[e];
-      r.scale_rows[e + 1] = r.scale_rows[e] + (total[e] + kScaleRows - 1) / kScaleRows * kScaleRows;
+      offset += total[e];
+      scale_row += (total[e] + kScaleRows - 1) / kScaleRows * kScaleRows;
+      r.offsets[e + 1] = offset;
+      r.scale_rows[e + 1] = scale_row;
     }
   }
 }
@@ -187,7 +211,7 @@ __global__ void RouteScan(Route r) {
 // first row, plus the expert's slots in earlier chunks, plus those before it in this chunk
 // (token order, then slot order: every thread walks the staged ids before its own).
 __global__ void RouteAssign(const int32_t* __restrict__ ids, int ids_stride, Route r) {
-  extern __shared__ int32_t staged[];
+  extern __shared__ __attribute__((aligned(16))) int32_t staged[];
   const int c = blockIdx.x;
   const int t0 = c * kRouteChunk;
   const int t1 = min(t0 + kRouteChunk, r.tokens);
@@ -198,11 +222,107 @@ __global__ void RouteAssign(const int32_t* __restrict__ ids, int ids_stride, Rou
       r.position[t0 * r.used + i] = -1;
       continue;
     }
-    int before = 0;
-    for (int j = 0; j < i; ++j) before += staged[j] == e;
+    int before = CountEqual(staged, i & ~3, e);
+    for (int j = i & ~3; j < i; ++j) before += staged[j] == e;
     const int row = r.offsets[e] + r.counts[static_cast<int64_t>(c) * r.experts + e] + before;
     r.position[t0 * r.used + i] = row;
     r.token[row] = t0 + i / r.used;
+    r.expert[row] = e;
+  }
+}
+
+// The whole grouping by one workgroup, for problems whose ids and per-run counters fit LDS
+// (up to 8192 slots and runs x experts up to 8192): the slots are cut into runs of 64 in slot
+// order; a run's ids are counted per expert with LDS integer atomics (a count does not depend
+// on their order), a thread an expert turns the runs' counts into bases, one thread the
+// experts' totals into offsets, and a thread a slot then takes its expert's first row, plus
+// its run's base, plus the equal ids before it in its run (at most 63 compares).
+// LDS: the ids, padded to fours; runs x experts counters; experts + 1 offsets.
+constexpr int kRouteOneSlots = 8192;
+constexpr int kRouteOneCounters = 8192;
+constexpr int kRouteOneThreads = 1024;
+
+__global__ __launch_bounds__(kRouteOneThreads) void RouteOne(const int32_t* __restrict__ ids, int ids_stride, Route r) {
+  extern __shared__ __attribute__((aligned(16))) int32_t staged[];
+  const int slots = r.tokens * r.used;
+  const int runs = (slots + 63) / 64;
+  int32_t* counters = staged + ((slots + 3) & ~3);  // [run][expert]
+  int32_t* offsets = counters + runs * r.experts;    // [expert + 1]
+  const int tid = threadIdx.x;
+  for (int i = tid; i < slots; i += kRouteOneThreads) staged[i] = ids[static_cast<int64_t>(i / r.used) * ids_stride + i % r.used];
+  if (tid < 4 && slots + tid < ((slots + 3) & ~3)) staged[slots + tid] = INT32_MIN;
+  for (int i = tid; i < runs * r.experts; i += kRouteOneThreads) counters[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < slots; i += kRouteOneThreads) {
+    const int e = staged[i];
+    if (e >= 0 && e < r.experts) atomicAdd(&counters[(i / 64) * r.experts + e], 1);
+  }
+  __syncthreads();
+  for (int e = tid; e < r.experts; e += kRouteOneThreads) {
+    int running = 0;
+    // Sixteen runs' counts read together (a read after a write to the same array would
+    // otherwise wait for it), then their bases written.
+    for (int run0 = 0; run0 < runs; run0 += 16) {
+      int v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = counters[min(run0 + u, runs - 1) * r.experts + e];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        if (run0 + u < runs) {
+          counters[(run0 + u) * r.experts + e] = running;
+          running += v[u];
+        }
+      }
+    }
+    offsets[e + 1] = running;  // the expert's total, for now
+  }
+  __syncthreads();
+  // The experts' totals into offsets: each lane of the first wave a block of consecutive
+  // experts, the blocks' sums scanned across the wave.
+  if (tid < kWave) {
+    const int per = (r.experts + kWave - 1) / kWave;
+    const int e0 = min(tid * per, r.experts), e1 = min(e0 + per, r.experts);
+    int rows = 0, scale_rows = 0;
+    for (int e = e0; e < e1; ++e) {
+      const int total = offsets[e + 1];
+      rows += total;
+      scale_rows += (total + kScaleRows - 1) / kScaleRows * kScaleRows;
+    }
+    int rows_before = rows, scale_before = scale_rows;  // inclusive scans
+#pragma unroll
+    for (int step = 1; step < kWave; step <<= 1) {
+      const int a = __shfl_up(rows_before, step, kWave);
+      const int b = __shfl_up(scale_before, step, kWave);
+      if (tid >= step) rows_before += a, scale_before += b;
+    }
+    int offset = rows_before - rows, scale_row = scale_before - scale_rows;
+    if (tid == 0) {
+      offsets[0] = 0;
+      r.offsets[0] = 0;
+      r.scale_rows[0] = 0;
+    }
+    for (int e = e0; e < e1; ++e) {
+      const int total = offsets[e + 1];
+      offset += total;
+      scale_row += (total + kScaleRows - 1) / kScaleRows * kScaleRows;
+      offsets[e + 1] = offset;
+      r.offsets[e + 1] = offset;
+      r.scale_rows[e + 1] = scale_row;
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < slots; i += kRouteOneThreads) {
+    const int e = staged[i];
+    if (e < 0 || e >= r.experts) {  // ids outside the experts have no row
+      r.position[i] = -1;
+      continue;
+    }
+    const int run0 = i & ~63;
+    int before = CountEqual(staged + run0, (i - run0) & ~3, e);
+    for (int j = i & ~3; j < i; ++j) before += staged[j] == e;
+    const int row = offsets[e] + counters[(i / 64) * r.experts + e] + before;
+    r.position[i] = row;
+    r.token[row] = i / r.used;
     r.expert[row] = e;
   }
 }
@@ -327,8 +447,21 @@ extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int expert
   if (static_cast<int64_t>(used) * tokens > (1 << 24)) return Refuse(1, "moe.route: more than 2^24 slots");
   const Route r = RouteOf(route, experts, used, tokens);
   const auto s = static_cast<hipStream_t>(stream);
+  const int64_t slots = static_cast<int64_t>(used) * tokens;
+  const int64_t runs = (slots + 63) / 64;
+  if (slots <= kRouteOneSlots && runs * experts <= kRouteOneCounters) {
+    const size_t bytes = static_cast<size_t>(((slots + 3) & ~int64_t{3}) + runs * experts + experts + 1) * sizeof(int32_t);
+    static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+    if (!sized) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&RouteOne), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (kRouteOneSlots + kRouteOneCounters + kRouteOneCounters + 4) * 4);
+      sized = true;
+    }
+    hipLaunchKernelGGL(RouteOne, dim3(1), dim3(kRouteOneThreads), bytes, s, ids, ids_stride, r);
+    return LaunchStatus("moe.route");
+  }
   const int threads = experts < 256 ? (experts + 63) / 64 * 64 : 256;
-  const size_t chunk_bytes = static_cast<size_t>(kRouteChunk) * used * sizeof(int32_t);
+  const size_t chunk_bytes = (static_cast<size_t>(kRouteChunk) * used + 4) * sizeof(int32_t);  // padded to fours
   hipLaunchKernelGGL(RouteCount, dim3(r.chunks), dim3(threads), chunk_bytes, s, ids, ids_stride, r);
   if (const int bad = LaunchStatus("moe.route count"); bad != 0) return bad;
   hipLaunchKernelGGL(RouteScan, dim3(1), dim3(threads), static_cast<size_t>(experts) * sizeof(int), s, r);

@@ -54,8 +54,11 @@ def test_router_ties_and_degenerate_rows(device):
     np.testing.assert_allclose(w2.cpu().numpy(), want2, rtol=1e-5)
 
 
-@pytest.mark.parametrize("tokens,experts,used", [(1, 128, 8), (16, 128, 8), (512, 128, 8), (130, 7, 3)])
+@pytest.mark.parametrize("tokens,experts,used", [(1, 128, 8), (16, 128, 8), (512, 128, 8), (130, 7, 3), (1024, 128, 8),
+                                                 (2000, 64, 6), (700, 300, 5), (1100, 256, 8)])
 def test_route_groups_pairs_by_expert_in_token_order(device, tokens, experts, used):
+    """Small problems are grouped by one workgroup, larger ones (more than 8192 slots, or more
+    run counters than fit LDS) by the count / scan / assign launches."""
     g = synth.rng(11 + tokens)
     ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
     order, offsets = oracle.expert_sort(ids, experts)
