@@ -112,7 +112,8 @@ int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int
  * src/kernels/ggml/moe_cutlass.h:12-27 describe the reference's operand layout): expert e
  * computes rows offsets[e] .. offsets[e + 1] of the Q8_1 activations d->y (y_token blocks a
  * row) into the same rows of d->dst (dst_token floats a row) with matrix e of d->w / d->g.
- * d->ids, used, tokens and the slot strides are ignored. Q4_K only. */
+ * d->ids, used, tokens and the slot strides are ignored. Weights the flat or the matrix-core
+ * form takes (the rows form has no sorted variant). */
 int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int32_t* offsets, int experts,
                          int variant, void* stream);
 

@@ -1,0 +1,181 @@
+// The host side of the MI355X kernels in the reference's own C++ vocabulary: the launch
+// interfaces its operator wrappers call (src/kernels/ggml/vecq.h:22-47,
+// src/kernels/ggml/mxfp8_cutlass.h:26-79, src/kernels/exl3/validate.h:84-131 and
+// src/kernels/exl3/linear.h:47-54, src/kernels/selected_operation.h:26-35 of the reference),
+// with the same names, argument meaning and error behaviour, over the C ABI of llmp_hip.h.
+// Header only, C++17, no HIP or torch types: a stream is the void* the reference's
+// NativeStream carries.
+#ifndef LLMP_HIP_HPP_
+#define LLMP_HIP_HPP_
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "llmp_hip.h"
+
+namespace llmp_amd {
+
+// src/kernels/selected_operation.h:26-35: a refusal queues nothing; anything else may have
+// queued work and faults the caller's launch context.
+enum class KernelFailure { kNone, kRejected, kUnknown };
+
+inline KernelFailure FromStatus(int status) {
+  return status == 0 ? KernelFailure::kNone : status > 0 ? KernelFailure::kRejected : KernelFailure::kUnknown;
+}
+inline std::string LastError() { return llmp_hip_last_error(); }
+
+namespace ggml {
+
+// ggml_type values of the encodings these kernels read.
+enum Type : int { kQ8_0 = LLMP_TYPE_Q8_0, kQ4_K = LLMP_TYPE_Q4_K };
+// VecQGlu, src/kernels/ggml/llmp_ops.h:1072.
+enum VecQGlu : int { kNone = LLMP_GLU_NONE, kSwiGlu = LLMP_GLU_SWIGLU, kSwiGluClamp = LLMP_GLU_SWIGLU_CLAMP, kGeGlu = LLMP_GLU_GEGLU };
+
+// What a llmp.vecq launch reads and writes (src/kernels/ggml/vecq.h:22-41). Weight offsets
+// count the weight type's blocks; activation offsets count Q8_1 blocks (36 bytes).
+struct VecQDesc {
+  const void* w = nullptr;
+  const void* g = nullptr;
+  const void* y = nullptr;
+  const std::int32_t* ids = nullptr;
+  float* dst = nullptr;
+  int ncols_x = 0;
+  int nrows = 0;
+  int stride_row = 0;
+  int stride_expert = 0;
+  int y_token = 0;
+  int y_slot = 0;
+  int ids_stride = 0;
+  int used = 1;
+  int tokens = 1;
+  int dst_token = 0;
+  int dst_slot = 0;
+  int glu = 0;
+  float limit = 0.0f;
+};
+
+inline llmp_vecq_desc ToAbi(const VecQDesc& d) {
+  return llmp_vecq_desc{d.w,      d.g,      d.y,          d.ids,  d.dst,    d.ncols_x,   d.nrows,    d.stride_row, d.stride_expert,
+                        d.y_token, d.y_slot, d.ids_stride, d.used, d.tokens, d.dst_token, d.dst_slot, d.glu,        d.limit};
+}
+
+// src/kernels/ggml/vecq.h:43-47: -1 is the default choice for the shape; false for a variant
+// the shape cannot take (and for any other refusal: LastError() names it).
+inline int VecQVariants() { return llmp_hip_vecq_variants(); }
+inline std::string VecQVariantName(int variant) {
+  const char* name = llmp_hip_vecq_variant_name(variant);
+  return name != nullptr ? name : "";
+}
+inline bool LaunchVecQ(int type, const VecQDesc& d, int variant, void* stream) {
+  const llmp_vecq_desc abi = ToAbi(d);
+  return llmp_hip_vecq(type, &abi, variant, stream) == 0;
+}
+
+// quantize_row_q8_1_cuda as RunQuantizeQ8 calls it (src/kernels/ggml/vecq.cu:1095-1111).
+inline KernelFailure QuantizeQ8(const float* x, void* out, std::int64_t k, std::int64_t padded_k, std::int64_t rows,
+                                void* stream) {
+  return FromStatus(llmp_hip_q8_1_quantize(x, out, k, padded_k, k, rows, 1, rows * k, stream));
+}
+// src/kernels/ggml/llmp_ops.cc:2574-2576: rows are padded with zero blocks to a multiple of 512.
+constexpr std::int64_t PaddedK(std::int64_t k) { return (k + 511) / 512 * 512; }
+
+namespace mxfp8 {
+
+// src/kernels/ggml/mxfp8_cutlass.h:28-57.
+inline constexpr std::uint64_t kBlock = 32;
+inline constexpr std::uint64_t kAtomRows = 128;
+constexpr std::uint64_t PaddedRows(std::uint64_t rows) { return (rows + kAtomRows - 1) / kAtomRows * kAtomRows; }
+constexpr std::uint64_t SwizzledScaleBytes(std::uint64_t n, std::uint64_t k) { return PaddedRows(n) * (k / kBlock); }
+
+// src/kernels/ggml/mxfp8_cutlass.h:59-71.
+struct Gemm {
+  int m = 0;
+  int n = 0;
+  int k = 0;
+  const void* a = nullptr;
+  const void* a_scales = nullptr;
+  const void* b = nullptr;
+  const void* b_scales = nullptr;
+  void* d = nullptr;
+  bool bf16 = false;
+  void* scratch = nullptr;
+};
+
+inline llmp_mxfp8_gemm ToAbi(const Gemm& g) {
+  llmp_mxfp8_gemm abi{};
+  abi.m = g.m, abi.n = g.n, abi.k = g.k;
+  abi.a = g.a, abi.a_scales = g.a_scales, abi.b = g.b, abi.b_scales = g.b_scales;
+  abi.d = g.d, abi.bf16 = g.bf16 ? 1 : 0, abi.scratch = g.scratch;
+  return abi;
+}
+
+// src/kernels/ggml/mxfp8_cutlass.h:73-79; `sms` is the device's compute units here.
+inline bool Available() { return llmp_hip_mxfp8_gemm_available() != 0; }
+inline std::size_t Scratch(const Gemm& gemm, int sms) {
+  const llmp_mxfp8_gemm abi = ToAbi(gemm);
+  return llmp_hip_mxfp8_gemm_scratch(&abi, sms);
+}
+inline int Run(const Gemm& gemm, int sms, void* stream) {
+  const llmp_mxfp8_gemm abi = ToAbi(gemm);
+  return llmp_hip_mxfp8_gemm_run(&abi, sms, stream);
+}
+
+}  // namespace mxfp8
+}  // namespace ggml
+
+namespace exl3 {
+
+// src/format/encoding.h:121.
+enum Codebook : int { k3Inst = LLMP_EXL3_3INST, kMcg = LLMP_EXL3_MCG, kMul1 = LLMP_EXL3_MUL1 };
+
+// src/kernels/exl3/validate.h:84-96 (the weights) and :118-131 (LinearOperands): addresses as
+// the reference carries them, uint64.
+struct Weights {
+  std::uint64_t trellis = 0;
+  std::uint64_t suh = 0;
+  std::uint64_t svh = 0;
+  int k = 0;
+  int n = 0;
+  int bits = 0;
+  int codebook = kMcg;
+};
+struct LinearOperands {
+  Weights weights;
+  std::uint64_t x = 0;      // m x k F16
+  std::uint64_t a_had = 0;  // m x k F16 scratch for the transformed input
+  std::uint64_t y = 0;      // m x n
+  bool f32 = false;         // y in F32, else F16
+  int m = 0;
+};
+
+inline llmp_exl3_linear ToAbi(const LinearOperands& o) {
+  llmp_exl3_linear abi{};
+  abi.weights.trellis = reinterpret_cast<const void*>(o.weights.trellis);
+  abi.weights.suh = reinterpret_cast<const void*>(o.weights.suh);
+  abi.weights.svh = reinterpret_cast<const void*>(o.weights.svh);
+  abi.weights.k = o.weights.k, abi.weights.n = o.weights.n;
+  abi.weights.bits = o.weights.bits, abi.weights.codebook = o.weights.codebook;
+  abi.x = reinterpret_cast<const void*>(o.x);
+  abi.a_had = reinterpret_cast<void*>(o.a_had);
+  abi.y = reinterpret_cast<void*>(o.y);
+  abi.f32 = o.f32 ? 1 : 0, abi.m = o.m;
+  return abi;
+}
+
+// The bytes of the partial-sum area a packed linear needs (the reference's lock area,
+// src/kernels/exl3/launch.h:13-36, is the caller's in the same way).
+inline std::size_t ScratchBytes(const LinearOperands& o) {
+  const llmp_exl3_linear abi = ToAbi(o);
+  return llmp_hip_exl3_linear_scratch(&abi);
+}
+// PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54, 1 to 16 rows.
+inline KernelFailure PackedLinear(const LinearOperands& o, void* scratch, std::size_t scratch_bytes, void* stream) {
+  const llmp_exl3_linear abi = ToAbi(o);
+  return FromStatus(llmp_hip_exl3_linear(&abi, scratch, scratch_bytes, stream));
+}
+
+}  // namespace exl3
+}  // namespace llmp_amd
+
+#endif  // LLMP_HIP_HPP_

@@ -1,0 +1,182 @@
+// The C++ host mirror (include/llmp_hip.hpp) exercised the way the reference's unit tests
+// exercise its launch interfaces (tests/unit/dsv4_fast_test.cc:300-520 builds blocks, runs the
+// op and compares with a scalar definition): "host" checks what needs no GPU (refusals queue
+// nothing and name their reason, the layout arithmetic); "device" runs small Q8_0 and Q4_K
+// products, a fused gate/up pair and the Q8_1 quantizer on the GPU and compares them with the
+// CPU oracle (oracle/oracle.h: test infrastructure, linked here as the checker only).
+//
+// Usage: mirror_test host | device. Exit status 0 when every check holds.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "llmp_hip.hpp"
+
+extern "C" {
+#include "oracle.h"
+}
+
+namespace {
+
+int g_failures = 0;
+
+#define EXPECT(condition)                                                     \
+  do {                                                                        \
+    if (!(condition)) {                                                       \
+      std::printf("%s:%d: EXPECT(%s) failed\n", __FILE__, __LINE__, #condition); \
+      ++g_failures;                                                           \
+    }                                                                         \
+  } while (0)
+
+namespace hipk = llmp_amd;
+using hipk::ggml::VecQDesc;
+
+// splitmix64: seeded bytes and floats that do not depend on a library's distributions.
+struct Rng {
+  std::uint64_t state;
+  std::uint64_t Next() {
+    std::uint64_t z = (state += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+  }
+  float Unit() { return static_cast<float>(Next() >> 40) * (1.0f / 16777216.0f); }  // [0, 1)
+  float Normal() {
+    const float u = Unit() + 1e-7f, v = Unit();
+    return std::sqrt(-2.0f * std::log(u)) * std::cos(6.2831853f * v);
+  }
+};
+
+std::uint16_t HalfBits(float v) { return orc_f32_to_f16(v); }
+
+// n rows of k values as Q8_0 / Q4_K blocks with plausible scales and uniform codes.
+std::vector<std::uint8_t> Weights(int type, int n, int k, std::uint64_t seed) {
+  Rng rng{seed};
+  const int bytes = orc_block_bytes(type), elements = orc_block_elements(type);
+  std::vector<std::uint8_t> w(static_cast<std::size_t>(n) * (k / elements) * bytes);
+  for (std::size_t at = 0; at < w.size(); at += bytes) {
+    for (int i = 0; i < bytes; ++i) w[at + i] = static_cast<std::uint8_t>(rng.Next());
+    const std::uint16_t d = HalfBits(0.002f + 0.01f * rng.Unit());
+    std::memcpy(&w[at], &d, 2);
+    if (type == hipk::ggml::kQ4_K) {
+      const std::uint16_t dmin = HalfBits(0.001f + 0.005f * rng.Unit());
+      std::memcpy(&w[at + 2], &dmin, 2);
+    }
+  }
+  return w;
+}
+
+template <typename T>
+T* ToDevice(const std::vector<T>& host) {
+  T* device = nullptr;
+  if (hipMalloc(reinterpret_cast<void**>(&device), host.size() * sizeof(T)) != hipSuccess) return nullptr;
+  if (hipMemcpy(device, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
+  return device;
+}
+
+double WorstRelative(const std::vector<float>& got, const std::vector<float>& want) {
+  double square = 0.0;
+  for (float v : want) square += static_cast<double>(v) * v;
+  const double floor = 1e-3 * std::sqrt(square / want.size());
+  double worst = 0.0;
+  for (std::size_t i = 0; i < want.size(); ++i) {
+    const double error = std::fabs(static_cast<double>(got[i]) - want[i]) / std::fmax(std::fabs(want[i]), floor);
+    worst = std::fmax(worst, error);
+  }
+  return worst;
+}
+
+void HostChecks() {
+  // A refusal queues nothing and names its reason (src/kernels/ggml/vecq.h:43-47: false).
+  VecQDesc d;
+  EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, -1, nullptr));
+  EXPECT(!hipk::LastError().empty());
+  d.w = reinterpret_cast<const void*>(0x1000), d.y = reinterpret_cast<const void*>(0x2000);
+  d.dst = reinterpret_cast<float*>(0x3000);
+  d.ncols_x = 256, d.nrows = 4, d.stride_row = 1, d.y_token = 16, d.dst_token = 4;
+  EXPECT(!hipk::ggml::LaunchVecQ(3, d, -1, nullptr));                          // not a type these kernels read
+  EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, 99, nullptr));          // no such variant
+  d.tokens = 17;
+  EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, -1, nullptr));          // 1 to 16 tokens
+  EXPECT(hipk::ggml::VecQVariants() >= 1);
+  for (int v = 0; v < hipk::ggml::VecQVariants(); ++v) EXPECT(!hipk::ggml::VecQVariantName(v).empty());
+  EXPECT(hipk::FromStatus(0) == hipk::KernelFailure::kNone);
+  EXPECT(hipk::FromStatus(3) == hipk::KernelFailure::kRejected);
+  EXPECT(hipk::FromStatus(-2) == hipk::KernelFailure::kUnknown);
+  // Layout arithmetic of src/kernels/ggml/mxfp8_cutlass.h:33-57.
+  static_assert(hipk::ggml::mxfp8::PaddedRows(1) == 128 && hipk::ggml::mxfp8::PaddedRows(129) == 256);
+  static_assert(hipk::ggml::mxfp8::SwizzledScaleBytes(12288, 4096) == 12288u * 128u);
+  static_assert(hipk::ggml::PaddedK(3840) == 4096 && hipk::ggml::PaddedK(512) == 512);
+  hipk::ggml::mxfp8::Gemm gemm;
+  EXPECT(hipk::ggml::mxfp8::Run(gemm, 256, nullptr) > 0);  // null operands: refused, nothing queued
+  hipk::exl3::LinearOperands linear;
+  EXPECT(hipk::exl3::PackedLinear(linear, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
+}
+
+// One dense product on the GPU against the oracle over the same Q8_1 bytes.
+void DenseProduct(int type, int n, int k, int tokens, bool glu) {
+  const int elements = orc_block_elements(type);
+  const std::vector<std::uint8_t> up = Weights(type, n, k, 11 + n), gate = Weights(type, n, k, 12 + n);
+  Rng rng{static_cast<std::uint64_t>(13 + k)};
+  std::vector<float> x(static_cast<std::size_t>(tokens) * k);
+  for (float& v : x) v = rng.Normal();
+  const std::int64_t padded_k = hipk::ggml::PaddedK(k);
+  std::vector<std::uint8_t> q8(static_cast<std::size_t>(tokens) * (padded_k / 32) * 36);
+  for (int t = 0; t < tokens; ++t)
+    orc_q8_1_quantize_row(&x[static_cast<std::size_t>(t) * k], k, padded_k, &q8[static_cast<std::size_t>(t) * (padded_k / 32) * 36],
+                          ORC_Q8_DEVICE);
+
+  // The quantizer first: its blocks are the oracle's bytes.
+  float* x_device = ToDevice(x);
+  std::uint8_t* q8_device = nullptr;
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&q8_device), q8.size()) == hipSuccess);
+  EXPECT(hipk::ggml::QuantizeQ8(x_device, q8_device, k, padded_k, tokens, nullptr) == hipk::KernelFailure::kNone);
+  std::vector<std::uint8_t> q8_got(q8.size());
+  EXPECT(hipMemcpy(q8_got.data(), q8_device, q8.size(), hipMemcpyDeviceToHost) == hipSuccess);
+  EXPECT(q8_got == q8);
+
+  std::uint8_t* up_device = ToDevice(up);
+  std::uint8_t* gate_device = ToDevice(gate);
+  float* dst_device = nullptr;
+  EXPECT(hipMalloc(reinterpret_cast<void**>(&dst_device), static_cast<std::size_t>(tokens) * n * 4) == hipSuccess);
+  VecQDesc d;
+  d.w = up_device, d.g = glu ? gate_device : nullptr, d.y = q8_device, d.dst = dst_device;
+  d.ncols_x = k, d.nrows = n, d.stride_row = k / elements;
+  d.y_token = static_cast<int>(padded_k / 32), d.tokens = tokens, d.dst_token = n;
+  d.glu = glu ? hipk::ggml::kGeGlu : hipk::ggml::kNone;
+  EXPECT(hipk::ggml::LaunchVecQ(type, d, -1, nullptr));
+  std::vector<float> got(static_cast<std::size_t>(tokens) * n), want(got.size());
+  EXPECT(hipDeviceSynchronize() == hipSuccess);
+  EXPECT(hipMemcpy(got.data(), dst_device, got.size() * 4, hipMemcpyDeviceToHost) == hipSuccess);
+
+  orc_vecq_desc o{};
+  o.w = up.data(), o.g = glu ? gate.data() : nullptr, o.y = q8.data(), o.dst = want.data();
+  o.ncols_x = k, o.nrows = n, o.stride_row = d.stride_row, o.y_token = d.y_token;
+  o.used = 1, o.tokens = tokens, o.dst_token = n, o.glu = glu ? ORC_GLU_GEGLU : ORC_GLU_NONE;
+  EXPECT(orc_vecq(type, &o, 0, 4) == 0);
+  const double worst = WorstRelative(got, want);
+  std::printf("type %d %d x %d, %d tokens%s: worst relative error %.2e\n", type, n, k, tokens, glu ? ", GeGLU" : "", worst);
+  EXPECT(worst <= 1e-3);  // the tolerance of the path: accumulation order only
+  (void)hipFree(x_device), (void)hipFree(q8_device), (void)hipFree(up_device), (void)hipFree(gate_device), (void)hipFree(dst_device);
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  const std::string mode = argc > 1 ? argv[1] : "host";
+  HostChecks();
+  if (mode == "device") {
+    DenseProduct(hipk::ggml::kQ8_0, 96, 4096, 1, false);
+    DenseProduct(hipk::ggml::kQ4_K, 100, 3840, 1, true);
+    DenseProduct(hipk::ggml::kQ4_K, 64, 2048, 8, true);
+    DenseProduct(hipk::ggml::kQ8_0, 40, 1024, 5, false);
+    DenseProduct(hipk::ggml::kQ4_K, 33, 15360, 1, false);
+  }
+  std::printf("%s checks: %d failure(s)\n", mode.c_str(), g_failures);
+  return g_failures == 0 ? 0 : 1;
+}
