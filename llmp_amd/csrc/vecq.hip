@@ -581,7 +581,8 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
 
 int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
-  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K) return Refuse(1, "vecq: weight type %d has no kernel", type);
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_Q4_0)
+    return Refuse(1, "vecq: weight type %d has no kernel", type);
   const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
   if (d->w == nullptr || d->dst == nullptr) return Refuse(1, "vecq: null weights or output");
   if (d->ncols_x <= 0 || d->ncols_x % qk != 0) return Refuse(1, "vecq: k %d is not whole %d-value blocks", d->ncols_x, qk);
@@ -599,6 +600,10 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   const uintptr_t wa = reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g);
   if (type == LLMP_TYPE_Q4_K && wa % 16 != 0) return Refuse(1, "vecq: Q4_K weights not 16-byte aligned");
   if (type == LLMP_TYPE_Q8_0 && wa % 2 != 0) return Refuse(1, "vecq: Q8_0 weights not 2-byte aligned");
+  // Q4_0 runs through the flat form alone: rows of whole 256 values at 16-byte boundaries.
+  if (type == LLMP_TYPE_Q4_0 && !FlatTakes(type, *d))
+    return Refuse(1, "vecq: Q4_0 takes rows of whole 256 values (up to 8192 with a GLU) whose rows, matrices and experts "
+                     "start on 16-byte boundaries");
   return 0;
 }
 
@@ -624,6 +629,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (variant < 0) variant = DefaultVariant(type, *d, a.kp, x != nullptr);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
+  if (type == LLMP_TYPE_Q4_0 && v.lanes != 0) return Refuse(1, "vecq: Q4_0 takes the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
   if (v.lanes < 0) {
     if (!MmaTakes(type, *d))

@@ -354,6 +354,169 @@ struct FormatQ8 {
   }
 };
 
+// ---- Q4_0: a unit is eight blocks of {f16 d; u8 nibbles[16]} (144 bytes, 256 values)
+//
+// Value i of a block is the low nibble of byte i (i < 16) or the high nibble of byte i - 16,
+// minus 8; a block times a Q8_1 block is dw * (sum(code * q) * d8 - 8 * s8) with s8 the
+// activation block's stored sum (tests/unit/dsv4_fast_test.cc:141-164 of the reference). A pair
+// of blocks is 36 bytes, nine dwords: the even block's scale and first two code bytes, three
+// dwords of codes, its last two code bytes and the odd block's scale, then the odd block's four
+// dwords. The staged activations are two images of that layout, one for the low nibbles
+// (values 0-15 of a block) and one for the high (16-31), with zeros where the weight scales lie:
+// masked nibbles and images multiply dword by dword as they lie.
+struct FormatQ40 {
+  static constexpr int kUnitBytes = 144;
+  static constexpr int kUnitValues = 256;
+  static constexpr int kBlockBytes = 18;
+  static constexpr int kBlockValues = 32;
+  static constexpr int kRecord = 352;  // two images of 144 bytes, eight d8, eight s8
+  static constexpr int kDumpInts = 8;
+
+  // The image byte of value v (0 .. 15) of block j of a unit.
+  static __device__ __forceinline__ int ImageAt(int j, int v) { return 36 * (j >> 1) + ((j & 1) ? 20 : 2) + v; }
+
+  // One block of 32 values, eight lanes, four values a lane: lanes 0-3 hold values 0-15 (the low
+  // image), lanes 4-7 values 16-31 (the high image).
+  static __device__ __forceinline__ void StageX(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+    uint8_t* image = record + (lane8 >> 2) * 144;
+    uint16_t* at = reinterpret_cast<uint16_t*>(image + ImageAt(j, 4 * (lane8 & 3)));
+    at[0] = static_cast<uint16_t>(q.codes & 0xFFFFu);
+    at[1] = static_cast<uint16_t>(q.codes >> 16);
+    if ((lane8 & 3) == 0) *reinterpret_cast<uint16_t*>(image + 36 * (j >> 1) + ((j & 1) ? 18 : 0)) = 0;  // against the scale
+    if (lane8 == 0) {
+      reinterpret_cast<float*>(record + 288)[j] = HalfBitsToFloat(FloatToHalfBits(q.d));
+      reinterpret_cast<float*>(record + 320)[j] = HalfBitsToFloat(FloatToHalfBits(q.sum));
+    }
+  }
+
+  // One Q8_1 block (nine dwords), one thread: both images' dwords of the block.
+  static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint32_t* pair = reinterpret_cast<uint32_t*>(record + half * 144) + 9 * (j >> 1);
+      const uint32_t* c = w + 1 + 4 * half;  // the sixteen codes of this half
+      if (j & 1) {
+        // The dword shared with the even block holds only zeros of this block (its scale).
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pair[5 + i] = c[i];
+      } else {
+        pair[0] = c[0] << 16;
+#pragma unroll
+        for (int i = 1; i < 4; ++i) pair[i] = (c[i - 1] >> 16) | (c[i] << 16);
+        pair[4] = c[3] >> 16;
+      }
+    }
+    reinterpret_cast<float*>(record + 288)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+    reinterpret_cast<float*>(record + 320)[j] = HalfBitsToFloat(w[0] >> 16);
+  }
+
+  // The unit at `at` (LDS) times the staged tokens.
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    if constexpr (P > 1) {
+      // Several tokens a pass: a pair of blocks at a time, each pair used by every token before
+      // the next is read (the whole unit's nibbles and the tokens' images do not fit the
+      // registers); the same operations in the same order as below.
+      float v[P];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t* pair = reinterpret_cast<const uint32_t*>(at) + 9 * p;
+        uint32_t lo_codes[9], hi_codes[9];
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+          const uint32_t word = pair[i];
+          lo_codes[i] = word & 0x0F0F0F0Fu;
+          hi_codes[i] = (word >> 4) & 0x0F0F0F0Fu;
+        }
+        const float dw_even = HalfBitsToFloat(pair[0] & 0xFFFFu), dw_odd = HalfBitsToFloat(pair[4] >> 16);
+#pragma unroll
+        for (int t = 0; t < P; ++t) {
+          if (t < m) {
+            const uint8_t* record = records + t * token_stride;
+            const uint32_t* low = reinterpret_cast<const uint32_t*>(record) + 9 * p;
+            const uint32_t* high = reinterpret_cast<const uint32_t*>(record + 144) + 9 * p;
+            int even = 0, odd = 0;
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+              int& s = i >= 5 ? odd : even;
+              s = Dot4(static_cast<int>(lo_codes[i]), static_cast<int>(low[i]), s);
+              s = Dot4(static_cast<int>(hi_codes[i]), static_cast<int>(high[i]), s);
+            }
+            const float2 d8 = *reinterpret_cast<const float2*>(record + 288 + 8 * p);
+            const float2 s8 = *reinterpret_cast<const float2*>(record + 320 + 8 * p);
+            const float term_even = dw_even * (static_cast<float>(even) * d8.x - 8.0f * s8.x);
+            const float term_odd = dw_odd * (static_cast<float>(odd) * d8.y - 8.0f * s8.y);
+            v[t] = p == 0 ? term_even : v[t] + term_even;
+            v[t] = v[t] + term_odd;
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < P; ++t) {
+        if (t < m) out[t] = v[t];
+      }
+      return;
+    }
+    const U32x4* mine = reinterpret_cast<const U32x4*>(at);
+    uint32_t w[36];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      const U32x4 v = mine[i];
+      w[4 * i] = v.x, w[4 * i + 1] = v.y, w[4 * i + 2] = v.z, w[4 * i + 3] = v.w;
+    }
+    float dw[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t word = w[9 * (j >> 1) + ((j & 1) ? 4 : 0)];
+      dw[j] = HalfBitsToFloat((j & 1) ? word >> 16 : word & 0xFFFFu);
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) {
+        const uint8_t* record = records + t * token_stride;
+        const U32x4* low = reinterpret_cast<const U32x4*>(record);
+        const U32x4* high = reinterpret_cast<const U32x4*>(record + 144);
+        int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+          const U32x4 lo = low[i], hi = high[i];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int index = 4 * i + c;
+            const int owner = 2 * (index / 9) + (index % 9 >= 5 ? 1 : 0);  // the block the dword's codes belong to
+            s[owner] = Dot4(static_cast<int>(w[index] & 0x0F0F0F0Fu), static_cast<int>(lo[c]), s[owner]);
+            s[owner] = Dot4(static_cast<int>((w[index] >> 4) & 0x0F0F0F0Fu), static_cast<int>(hi[c]), s[owner]);
+          }
+        }
+        if (kDump && dump != nullptr) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) dump[j] = s[j];
+        }
+        const float4* scales = reinterpret_cast<const float4*>(record + 288);
+        const float4 d8a = scales[0], d8b = scales[1], s8a = scales[2], s8b = scales[3];
+        const float d8[8] = {d8a.x, d8a.y, d8a.z, d8a.w, d8b.x, d8b.y, d8b.z, d8b.w};
+        const float s8[8] = {s8a.x, s8a.y, s8a.z, s8a.w, s8b.x, s8b.y, s8b.z, s8b.w};
+        float v = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float term = dw[j] * (static_cast<float>(s[j]) * d8[j] - 8.0f * s8[j]);
+          v = j == 0 ? term : v + term;
+        }
+        out[t] = v;
+      }
+    }
+  }
+};
+
 // ---- staging a token's row into records
 
 template <class F, int XT>
@@ -915,6 +1078,13 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
+  if (type == LLMP_TYPE_Q4_0) {
+    const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+    if (d.ncols_x % 256 != 0 || d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || at % 16 != 0) return false;
+    const int units = d.ncols_x / FormatQ40::kUnitValues;
+    if (units > most) return pieces && PlanSplit<FormatQ40>(units).lds <= kFlatLdsLimit;
+    return PlanFlat<FormatQ40>(1, units, glu).lds <= kFlatLdsLimit;
+  }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
   const int units = d.ncols_x / FormatQ8::kUnitValues;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
@@ -926,6 +1096,8 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
 void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
   if (type == LLMP_TYPE_Q4_K) {
     LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q4_0) {
+    LaunchF<FormatQ40>(a, x_type, pass, deep, stream);
   } else {
     LaunchF<FormatQ8>(a, x_type, pass, deep, stream);
   }

@@ -7,12 +7,12 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_K,  # noqa: F401
+from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_0, TYPE_Q4_K,  # noqa: F401
                    TYPE_Q8_0, X_BF16, X_F16, X_F32, Exl3Linear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
                    VecQSource)
 
-BLOCK_BYTES = {TYPE_Q8_0: 34, TYPE_Q4_K: 144}
-BLOCK_ELEMENTS = {TYPE_Q8_0: 32, TYPE_Q4_K: 256}
+BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q8_0: 34, TYPE_Q4_K: 144}
+BLOCK_ELEMENTS = {TYPE_Q4_0: 32, TYPE_Q8_0: 32, TYPE_Q4_K: 256}
 
 
 def padded_k(k):
@@ -99,7 +99,7 @@ def vecq_fused(t, w, x, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stri
 def vecq_block_sums(t, w, q8, k, nrows, variant=-1):
     """The kernel's int32 block sums of a dense one-token product: [nrows, blocks, per]."""
     lib = _lib.load()
-    per = 1 if t == TYPE_Q8_0 else 16
+    per = 16 if t == TYPE_Q4_K else 1
     sums = torch.zeros((nrows, k // BLOCK_ELEMENTS[t], per), dtype=torch.int32, device=w.device)
     out = torch.empty((1, 1, nrows), dtype=torch.float32, device=w.device)
     d = _desc(t, w, k, nrows, gate=None, q8=q8, ids=None, tokens=1, used=1, stride_row=None,

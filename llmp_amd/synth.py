@@ -1,8 +1,9 @@
 """Seeded synthetic inputs of the benchmark configurations (numpy, host side).
 
-Weights are byte images of GGML blocks: Q8_0 {f16 d; i8 qs[32]} and Q4_K
+Weights are byte images of GGML blocks: Q8_0 {f16 d; i8 qs[32]}, Q4_K
 {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} (src/format/encoding.cc:110-116
-of the reference)."""
+of the reference) and the legacy 4/5-bit blocks {f16 d; [f16 m;] [u32 high bits;]
+u8 nibbles[16]} as tests/unit/dsv4_fast_test.cc:141-157 reads them."""
 import numpy as np
 
 
@@ -37,11 +38,30 @@ def q4_k_weights(n, k, seed):
     return out.reshape(n, blocks * 144)
 
 
+LEGACY_BYTES = {2: 18, 3: 20, 6: 22, 7: 24}  # Q4_0, Q4_1, Q5_0, Q5_1
+
+
+def legacy_weights(t, n, k, seed):
+    """[n, k/32*bytes] uint8 of a legacy block type: codes uniform, each block's scale the
+    range of 32 draws of N(0, 0.02) over its code range (and a minimum at the low end)."""
+    g = rng(seed)
+    blocks, size = k // 32, LEGACY_BYTES[t]
+    out = g.integers(0, 256, size=(n, blocks, size), dtype=np.uint8)
+    levels = 31.0 if t in (6, 7) else 15.0
+    amax = np.abs(g.standard_normal((n, blocks, 32), dtype=np.float32) * 0.02).max(axis=-1)
+    out[:, :, 0:2] = (2.0 * amax / levels).astype(np.float16).view(np.uint8).reshape(n, blocks, 2)
+    if t in (3, 7):
+        out[:, :, 2:4] = (-amax).astype(np.float16).view(np.uint8).reshape(n, blocks, 2)
+    return out.reshape(n, blocks * size)
+
+
 def random_blocks(t, n, k, seed):
     """Every field random (any finite f16 scale up to magnitude 4, any scale byte, any code):
     the bytes a decoder must take, not a plausible quantization."""
     g = rng(seed)
-    if t == 8:
+    if t in LEGACY_BYTES:
+        blocks, size, heads = k // 32, LEGACY_BYTES[t], 2 if t in (3, 7) else 1
+    elif t == 8:
         blocks, size, heads = k // 32, 34, 1
     else:
         blocks, size, heads = k // 256, 144, 2

@@ -12,6 +12,10 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboracle.so")
 
+TYPE_Q4_0 = 2
+TYPE_Q4_1 = 3
+TYPE_Q5_0 = 6
+TYPE_Q5_1 = 7
 TYPE_Q8_0 = 8
 TYPE_Q4_K = 12
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
@@ -98,11 +102,11 @@ def max_threads():
 
 
 def block_bytes(t):
-    return {TYPE_Q8_0: 34, TYPE_Q4_K: 144}[t]
+    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144}[t]
 
 
 def block_elements(t):
-    return {TYPE_Q8_0: 32, TYPE_Q4_K: 256}[t]
+    return 256 if t == TYPE_Q4_K else 32
 
 
 def padded_k(k):
@@ -164,7 +168,7 @@ def vecq(t, w, q8, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stride_ro
 
 def vecq_block_sums(t, w, q8, k, nrows):
     qk = block_elements(t)
-    per = 1 if t == TYPE_Q8_0 else 16
+    per = 16 if t == TYPE_Q4_K else 1
     w = np.ascontiguousarray(w, dtype=np.uint8)
     q8 = np.ascontiguousarray(q8, dtype=np.uint8)
     out = np.zeros((nrows, k // qk, per), dtype=np.int32)
@@ -261,8 +265,18 @@ def exl3_rows(trellis, suh, svh, k, n, bits, codebook, first=0, count=None):
     return out
 
 
+def _half_bits(x):
+    """F16 values as their bits: a float16 array is reinterpreted, never converted."""
+    x = np.asarray(x)
+    if x.dtype == np.float16:
+        x = x.view(np.uint16)
+    if x.dtype != np.uint16:
+        raise TypeError(f"F16 bits expected, not {x.dtype}")
+    return np.ascontiguousarray(x)
+
+
 def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, threads=1):
-    x = np.ascontiguousarray(x, dtype=np.uint16)
+    x = _half_bits(x)
     m = x.shape[0]
     y = np.zeros((m, n), dtype=np.float32)
     lib.orc_exl3_linear(_p(trellis), _p(suh), _p(svh), k, n, bits, codebook, _p(x), m, _p(y), threads)
@@ -270,14 +284,14 @@ def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, threads=1):
 
 
 def exl3_input(suh, k, x):
-    x = np.ascontiguousarray(x, dtype=np.uint16)
+    x = _half_bits(x)
     xh = np.zeros_like(x)
     lib.orc_exl3_input(_p(suh), k, _p(x), x.shape[0], _p(xh))
     return xh
 
 
 def exl3_product(trellis, svh, k, n, bits, codebook, xh, threads=1):
-    xh = np.ascontiguousarray(xh, dtype=np.uint16)
+    xh = _half_bits(xh)
     m = xh.shape[0]
     y = np.zeros((m, n), dtype=np.float32)
     lib.orc_exl3_product(_p(trellis), _p(svh), k, n, bits, codebook, _p(xh), m, _p(y), threads)

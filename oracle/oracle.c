@@ -173,8 +173,35 @@ void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y) {
 
 /* --------------------------------------------------------- weight blocks */
 
-int orc_block_bytes(int type) { return type == ORC_TYPE_Q8_0 ? 34 : type == ORC_TYPE_Q4_K ? 144 : 0; }
-int orc_block_elements(int type) { return type == ORC_TYPE_Q8_0 ? 32 : type == ORC_TYPE_Q4_K ? 256 : 0; }
+/* src/format/encoding.cc:110-116; the legacy blocks as tests/unit/dsv4_fast_test.cc:141-157 reads
+ * them: {f16 d; [f16 m;] [u32 high bits;] u8 nibbles[16]}. */
+int orc_block_bytes(int type) {
+  switch (type) {
+    case ORC_TYPE_Q4_0: return 18;
+    case ORC_TYPE_Q4_1: return 20;
+    case ORC_TYPE_Q5_0: return 22;
+    case ORC_TYPE_Q5_1: return 24;
+    case ORC_TYPE_Q8_0: return 34;
+    case ORC_TYPE_Q4_K: return 144;
+    default: return 0;
+  }
+}
+int orc_block_elements(int type) { return type == ORC_TYPE_Q4_K ? 256 : orc_block_bytes(type) != 0 ? 32 : 0; }
+
+static int legacy_affine(int type) { return type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_1; }
+static int legacy_five(int type) { return type == ORC_TYPE_Q5_0 || type == ORC_TYPE_Q5_1; }
+static int legacy(int type) {
+  return type == ORC_TYPE_Q4_0 || type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_0 || type == ORC_TYPE_Q5_1;
+}
+/* Code i of a legacy block: dsv4_fast_test.cc:149-158. */
+static int legacy_code(int type, const uint8_t* w, int i) {
+  const int prefix = legacy_affine(type) ? 4 : 2;
+  uint32_t high = 0;
+  if (legacy_five(type)) memcpy(&high, w + prefix, 4);
+  const uint8_t* codes = w + prefix + (legacy_five(type) ? 4 : 0);
+  const int low = i < 16 ? codes[i] & 15 : codes[i - 16] >> 4;
+  return low + (legacy_five(type) ? (int)((high >> i) & 1u) * 16 : 0);
+}
 
 /* dsv4_fast_test.cc:180-183 */
 void orc_q4_k_scale_min(const uint8_t* scales, int g, int* scale, int* minimum) {
@@ -187,6 +214,18 @@ static int q4_k_code(const uint8_t* codes, int g, int i) {
 }
 
 void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
+  if (legacy(type)) {
+    /* ggml's dequantization of these bytes: d * (code - 8 or 16), or d * code + m. */
+    const int bs = orc_block_bytes(type);
+    for (int64_t b = 0; b < k / 32; ++b) {
+      const uint8_t* x = row + b * bs;
+      const float d = orc_f16_to_f32(load_u16(x));
+      const float m = legacy_affine(type) ? orc_f16_to_f32(load_u16(x + 2)) : 0.0f;
+      const int offset = legacy_affine(type) ? 0 : legacy_five(type) ? 16 : 8;
+      for (int j = 0; j < 32; ++j) y[b * 32 + j] = d * (float)(legacy_code(type, x, j) - offset) + m;
+    }
+    return;
+  }
   if (type == ORC_TYPE_Q8_0) {
     for (int64_t b = 0; b < k / 32; ++b) {
       const uint8_t* x = row + b * 34;
@@ -211,6 +250,12 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
 }
 
 void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums) {
+  if (legacy(type)) { /* dsv4_fast_test.cc:154-158 */
+    int32_t s = 0;
+    for (int i = 0; i < 32; ++i) s += legacy_code(type, w, i) * (int32_t)(int8_t)q8[4 + i];
+    sums[0] = s;
+    return;
+  }
   if (type == ORC_TYPE_Q8_0) {
     int32_t s = 0;
     for (int i = 0; i < 32; ++i) s += (int32_t)(int8_t)w[2 + i] * (int32_t)(int8_t)q8[4 + i];
@@ -233,6 +278,17 @@ void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums
 double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
   int32_t sums[16];
   orc_block_sums(type, w, q8, sums);
+  if (legacy(type)) { /* dsv4_fast_test.cc:145-164: the Q8_1 block's s is the rounded sum of its inputs */
+    const float dw = orc_f16_to_f32(load_u16(w));
+    const float da = orc_f16_to_f32(load_u16(q8));
+    const float sa = orc_f16_to_f32(load_u16(q8 + 2));
+    if (legacy_affine(type)) {
+      const float scale = orc_f16_to_f32(orc_f32_to_f16(dw * da));
+      const float minimum = orc_f16_to_f32(orc_f32_to_f16(orc_f16_to_f32(load_u16(w + 2)) * sa));
+      return (double)sums[0] * scale + minimum;
+    }
+    return (double)dw * ((double)sums[0] * da - (legacy_five(type) ? 16.0 : 8.0) * sa);
+  }
   if (type == ORC_TYPE_Q8_0) {
     /* vecq.cu:415-416: d8_0 * d8_1 * sumi */
     return (double)orc_f16_to_f32(load_u16(w)) * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
@@ -320,7 +376,7 @@ void orc_vecq_block_sums(int type, const void* w, const void* y, int k, int nrow
                          int32_t* out) {
   const int qk = orc_block_elements(type);
   const int bs = orc_block_bytes(type);
-  const int per = type == ORC_TYPE_Q8_0 ? 1 : 16;
+  const int per = type == ORC_TYPE_Q4_K ? 16 : 1;
   const int blocks = k / qk;
   for (int r = 0; r < nrows; ++r)
     for (int b = 0; b < blocks; ++b)

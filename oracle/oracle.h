@@ -52,15 +52,16 @@ void orc_q8_1_quantize_row(const float* x, int64_t k, int64_t padded_k, uint8_t*
 void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y);
 
 /* ---- weight blocks: src/format/encoding.cc:110-116 ---- */
-enum { ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12 }; /* ggml_type values */
-int orc_block_bytes(int type);    /* 34 / 144 */
-int orc_block_elements(int type); /* 32 / 256 */
+enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12 }; /* ggml_type values */
+int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144 */
+int orc_block_elements(int type); /* 32, Q4_K 256 */
 /* The Q4_K 6-bit scale and minimum of sub-block g: tests/unit/dsv4_fast_test.cc:180-183. */
 void orc_q4_k_scale_min(const uint8_t* scales12, int g, int* scale, int* minimum);
 /* Decode rows of blocks to floats (the ggml dequantization of those bytes). */
 void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y);
-/* Per-block int32 sums over identical Q8_1 bytes. Q8_0: sums[0] = sum w*q of the
- * 32 values (src/kernels/ggml/vecq.cu:398-418). Q4_K: sums[0..7] = sum code*q per
+/* Per-block int32 sums over identical Q8_1 bytes. Q8_0 and the legacy 4/5-bit blocks:
+ * sums[0] = sum w*q (code*q) of the 32 values (src/kernels/ggml/vecq.cu:398-418,
+ * tests/unit/dsv4_fast_test.cc:154-158). Q4_K: sums[0..7] = sum code*q per
  * sub-block, sums[8..15] = sum q per sub-block (tests/unit/dsv4_fast_test.cc:185-191). */
 void orc_block_sums(int type, const uint8_t* wblock, const uint8_t* q8, int32_t* sums);
 /* One weight block times its Q8_1 blocks in double. */

@@ -40,6 +40,14 @@ def build():
     for kind in (1, 2, 3):
         out[f"q4_k_glu{kind}"] = oracle.vecq(oracle.TYPE_Q4_K, up, q8, k, n, gate=gate, glu=kind, limit=0.05 if kind == 2 else 0.0)
     out["q4_k_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q4_K, up, q8, k, n)
+    # llmp.vecq, Q4_0 (the legacy block that reads the activation blocks' stored sums), 2 tokens.
+    k, n = 256, 16
+    w40 = synth.legacy_weights(oracle.TYPE_Q4_0, n, k, 22)
+    a = synth.activations(2, k, 23)
+    q8 = oracle.q8_1_quantize(a)
+    out["q4_0_w"], out["q4_0_x"] = w40, a
+    out["q4_0_y"] = oracle.vecq(oracle.TYPE_Q4_0, w40, q8, k, n, tokens=2)
+    out["q4_0_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q4_0, w40, q8[:1], k, n)
     # MXFP8: quantizer and one small product.
     xa = synth.activations(5, 256, 17) * 3.0
     xb = synth.activations(8, 256, 18) * 0.02

@@ -53,6 +53,11 @@ def test_device_meets_the_committed_vectors(vectors, device):
     from conftest import rel_close
     from llmp_amd import ops
     v = vectors
+
+    def close(got, want, tol, what):
+        ok, worst = rel_close(got, want, tol)
+        assert ok, (what, worst)
+
     # llmp.q8_1: every byte.
     got = ops.quantize_q8_1(_dev(v["q8_x"], device)).cpu().numpy()
     assert np.array_equal(got, v["q8_blocks"])
@@ -60,24 +65,30 @@ def test_device_meets_the_committed_vectors(vectors, device):
     k, n = 256, 24
     w = _dev(v["q8_0_w"], device)
     q8 = ops.quantize_q8_1(_dev(v["q8_0_x"], device))
-    rel_close(ops.vecq(ops.TYPE_Q8_0, w, q8, k, n, tokens=2).cpu().numpy(), v["q8_0_y"], 1e-3)
+    close(ops.vecq(ops.TYPE_Q8_0, w, q8, k, n, tokens=2).cpu().numpy(), v["q8_0_y"], 1e-3, "q8_0")
     assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q8_0, w, q8[:1], k, n).cpu().numpy(), v["q8_0_sums"])
     # Q4_K with and without each GLU; int32 block sums.
     k, n = 512, 20
     up, gate = _dev(v["q4_k_up"], device), _dev(v["q4_k_gate"], device)
     q8 = ops.quantize_q8_1(_dev(v["q4_k_x"], device))
-    rel_close(ops.vecq(ops.TYPE_Q4_K, up, q8, k, n).cpu().numpy(), v["q4_k_y"], 1e-3)
+    close(ops.vecq(ops.TYPE_Q4_K, up, q8, k, n).cpu().numpy(), v["q4_k_y"], 1e-3, "q4_k")
     for kind in (1, 2, 3):
         got = ops.vecq(ops.TYPE_Q4_K, up, q8, k, n, gate=gate, glu=kind, limit=0.05 if kind == 2 else 0.0).cpu().numpy()
-        rel_close(got, v[f"q4_k_glu{kind}"], 1e-3)
+        close(got, v[f"q4_k_glu{kind}"], 1e-3, f"q4_k glu {kind}")
     assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q4_K, up, q8, k, n).cpu().numpy(), v["q4_k_sums"])
+    # Q4_0 dense, two tokens; int32 block sums.
+    k, n = 256, 16
+    w = _dev(v["q4_0_w"], device)
+    q8 = ops.quantize_q8_1(_dev(v["q4_0_x"], device))
+    close(ops.vecq(ops.TYPE_Q4_0, w, q8, k, n, tokens=2).cpu().numpy(), v["q4_0_y"], 1e-3, "q4_0")
+    assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q4_0, w, q8[:1], k, n).cpu().numpy(), v["q4_0_sums"])
     # MXFP8 quantizer (bytes) and product.
     ac, as_ = ops.mxfp8_quantize(_dev(v["mx_a"], device))
     bc, bs = ops.mxfp8_quantize(_dev(v["mx_b"], device))
     assert np.array_equal(ac.cpu().numpy(), v["mx_a_codes"]) and np.array_equal(as_.cpu().numpy(), v["mx_a_scales"].reshape(-1))
     assert np.array_equal(bc.cpu().numpy(), v["mx_b_codes"]) and np.array_equal(bs.cpu().numpy(), v["mx_b_scales"].reshape(-1))
     d = ops.mxfp8_gemm(ac, as_, bc, bs, bf16=False).cpu().numpy()
-    rel_close(d, v["mx_d"], 1e-3)
+    close(d, v["mx_d"], 1e-3, "mxfp8 gemm")
     # Router.
     ids, weights = ops.moe_router(_dev(v["route_logits"], device), 3)
     assert np.array_equal(ids.cpu().numpy(), v["route_ids"])
@@ -92,5 +103,5 @@ def test_device_meets_the_committed_vectors(vectors, device):
         w = ops.exl3_reconstruct(trellis, suh, svh, k, n, 3, cb).cpu().numpy().view(np.uint16)
         assert np.array_equal(w, v[f"exl3_rotated{cb}"].view(np.uint16).reshape(w.shape))
         y = ops.exl3_linear(trellis, suh, svh, k, n, 3, cb, x).cpu().numpy()
-        rel_close(y, v[f"exl3_y{cb}"], 5e-3)
+        close(y, v[f"exl3_y{cb}"], 5e-3, f"exl3 linear {cb}")
     torch.cuda.synchronize()

@@ -177,6 +177,78 @@ def test_q4_k_and_q8_0_decode_and_block_sums_by_brute_force():
             np.testing.assert_allclose(y[r], float(np.dot(want, act)), rtol=2e-6, atol=1e-9)
 
 
+def legacy_block_numpy(t, block, a):
+    """tests/unit/dsv4_fast_test.cc:141-164 restated with numpy, apart from the oracle's C:
+    (codes, int sum, product) of one legacy block and one Q8_1 block."""
+    affine, five = t in (3, 7), t in (6, 7)
+    prefix = 4 if affine else 2
+    high = int(block[prefix:prefix + 4].view(np.uint32)[0]) if five else 0
+    nib = block[prefix + (4 if five else 0):].astype(np.int64)
+    codes = np.concatenate([nib & 15, nib >> 4])
+    if five:
+        codes = codes + 16 * ((high >> np.arange(32)) & 1)
+    q = a[4:].view(np.int8).astype(np.int64)
+    total = int((codes * q).sum())
+    dw, da, sa = (float(v) for v in (block[0:2].view(np.float16)[0], a[0:2].view(np.float16)[0],
+                                    a[2:4].view(np.float16)[0]))
+    if affine:
+        m = float(block[2:4].view(np.float16)[0])
+        scale = float(np.float16(np.float32(dw) * np.float32(da)))
+        minimum = float(np.float16(np.float32(m) * np.float32(sa)))
+        return codes, total, total * scale + minimum
+    return codes, total, dw * (total * da - (16.0 if five else 8.0) * sa)
+
+
+def test_legacy_blocks_decode_sums_and_products_by_brute_force():
+    from llmp_amd import synth
+    k, n = 256, 4
+    x = np.random.Generator(np.random.PCG64(18)).standard_normal((1, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    acts = q8[0].reshape(-1, 36)
+    for t in (oracle.TYPE_Q4_0, oracle.TYPE_Q4_1, oracle.TYPE_Q5_0, oracle.TYPE_Q5_1):
+        size = oracle.block_bytes(t)
+        assert size == synth.LEGACY_BYTES[t] and oracle.block_elements(t) == 32
+        for w in (synth.random_blocks(t, n, k, 17 + t), synth.legacy_weights(t, n, k, 19 + t)):
+            sums = oracle.vecq_block_sums(t, w, q8, k, n)
+            y = oracle.vecq(t, w, q8, k, n)[0, 0]
+            dec = oracle.decode_rows(t, w, k)
+            for r in range(n):
+                want, row = 0.0, []
+                for b, block in enumerate(w[r].reshape(-1, size)):
+                    codes, total, product = legacy_block_numpy(t, block, acts[b])
+                    assert sums[r, b, 0] == total
+                    want += product
+                    d = float(block[0:2].view(np.float16)[0])
+                    m = float(block[2:4].view(np.float16)[0]) if t in (3, 7) else 0.0
+                    offset = 0 if t in (3, 7) else 16 if t in (6, 7) else 8
+                    row.append(np.float32(d) * (codes - offset).astype(np.float32) + np.float32(m))
+                np.testing.assert_allclose(dec[r], np.concatenate(row), rtol=1e-6, atol=1e-12)
+                np.testing.assert_allclose(y[r], want, rtol=1e-6, atol=1e-9)
+
+
+def test_hand_built_legacy_blocks_have_known_answers():
+    # Q4_0: d = 0.5, code i = i % 16 in both halves (byte i = i | i << 4); activation d = 0.25,
+    # every q = 2, s = 3. sum = 2 * 2 * (0 + .. + 15) = 480; 0.5 * (480 * 0.25 - 8 * 3) = 48.
+    w = np.zeros((1, 18), dtype=np.uint8)
+    w[0, 0:2] = np.array([0.5], dtype=np.float16).view(np.uint8)
+    w[0, 2:] = np.arange(16, dtype=np.uint8) * 17
+    q8 = np.zeros((1, 16 * 36), dtype=np.uint8)
+    q8[0, 0:2] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    q8[0, 2:4] = np.array([3.0], dtype=np.float16).view(np.uint8)
+    q8[0, 4:36] = np.full(32, 2, dtype=np.int8).view(np.uint8)
+    assert oracle.vecq_block_sums(oracle.TYPE_Q4_0, w, q8, 32, 1)[0, 0, 0] == 480
+    assert oracle.vecq(oracle.TYPE_Q4_0, w, q8, 32, 1)[0, 0, 0] == 48.0
+    assert np.array_equal(oracle.decode_rows(oracle.TYPE_Q4_0, w, 32)[0], 0.5 * (np.arange(32) % 16 - 8))
+    # Q5_0 with the high bits of values 0..7 set: codes 16..23 there; offset 16.
+    w5 = np.zeros((1, 22), dtype=np.uint8)
+    w5[0, 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    w5[0, 2:6] = np.array([0xFF], dtype=np.uint32).view(np.uint8)
+    w5[0, 6:] = np.arange(16, dtype=np.uint8) * 17
+    total = 2 * (2 * sum(range(16)) + 16 * 8)
+    assert oracle.vecq_block_sums(oracle.TYPE_Q5_0, w5, q8, 32, 1)[0, 0, 0] == total
+    assert oracle.vecq(oracle.TYPE_Q5_0, w5, q8, 32, 1)[0, 0, 0] == np.float32(total * 0.25 - 16 * 3)
+
+
 def test_hand_built_blocks_have_known_sums():
     w = np.zeros((1, 34), dtype=np.uint8)
     w[0, 0:2] = np.array([2.0], dtype=np.float16).view(np.uint8)
