@@ -17,8 +17,10 @@
  * Sizes are bytes unless a comment says blocks or elements. "Q8_1 block" is
  * {f16 d; f16 s; i8 qs[32]} = 36 bytes; Q8_0 is {f16 d; i8 qs[32]} = 34 bytes;
  * Q4_K is {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]} = 144 bytes
- * (src/format/encoding.cc:110-116); Q4_0 is {f16 d; u8 nibbles[16]} = 18 bytes, value i the
- * low (i < 16) or high nibble of byte i % 16, minus 8 (tests/unit/dsv4_fast_test.cc:141-164).
+ * (src/format/encoding.cc:110-116); the legacy blocks are {f16 d; [f16 m;] [u32 high bits;] u8
+ * nibbles[16]} = 18 (Q4_0), 20 (Q4_1), 22 (Q5_0), 24 (Q5_1) bytes, code i the low (i < 16) or
+ * high nibble of byte i % 16 plus 16 where bit i of the high bits is set
+ * (tests/unit/dsv4_fast_test.cc:141-164).
  */
 #ifndef LLMP_HIP_H_
 #define LLMP_HIP_H_
@@ -31,7 +33,7 @@ extern "C" {
 #endif
 
 /* ggml_type values of the weight encodings the kernels read. */
-enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12 };
+enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12 };
 /* VecQGlu, src/kernels/ggml/llmp_ops.h:1072. */
 enum { LLMP_GLU_NONE = 0, LLMP_GLU_SWIGLU = 1, LLMP_GLU_SWIGLU_CLAMP = 2, LLMP_GLU_GEGLU = 3 };
 /* Element types of unquantized activations. */

@@ -28,7 +28,14 @@ inline std::string LastError() { return llmp_hip_last_error(); }
 namespace ggml {
 
 // ggml_type values of the encodings these kernels read.
-enum Type : int { kQ8_0 = LLMP_TYPE_Q8_0, kQ4_K = LLMP_TYPE_Q4_K };
+enum Type : int {
+  kQ4_0 = LLMP_TYPE_Q4_0,
+  kQ4_1 = LLMP_TYPE_Q4_1,
+  kQ5_0 = LLMP_TYPE_Q5_0,
+  kQ5_1 = LLMP_TYPE_Q5_1,
+  kQ8_0 = LLMP_TYPE_Q8_0,
+  kQ4_K = LLMP_TYPE_Q4_K
+};
 // VecQGlu, src/kernels/ggml/llmp_ops.h:1072.
 enum VecQGlu : int { kNone = LLMP_GLU_NONE, kSwiGlu = LLMP_GLU_SWIGLU, kSwiGluClamp = LLMP_GLU_SWIGLU_CLAMP, kGeGlu = LLMP_GLU_GEGLU };
 

@@ -10,6 +10,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "lib", "libllmp_hip.so")
 
 TYPE_Q4_0 = 2
+TYPE_Q4_1 = 3
+TYPE_Q5_0 = 6
+TYPE_Q5_1 = 7
 TYPE_Q8_0 = 8
 TYPE_Q4_K = 12
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3

@@ -581,7 +581,8 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
 
 int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
-  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_Q4_0)
+  const bool legacy = type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1;
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && !legacy)
     return Refuse(1, "vecq: weight type %d has no kernel", type);
   const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
   if (d->w == nullptr || d->dst == nullptr) return Refuse(1, "vecq: null weights or output");
@@ -600,10 +601,10 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   const uintptr_t wa = reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g);
   if (type == LLMP_TYPE_Q4_K && wa % 16 != 0) return Refuse(1, "vecq: Q4_K weights not 16-byte aligned");
   if (type == LLMP_TYPE_Q8_0 && wa % 2 != 0) return Refuse(1, "vecq: Q8_0 weights not 2-byte aligned");
-  // Q4_0 runs through the flat form alone: rows of whole 256 values at 16-byte boundaries.
-  if (type == LLMP_TYPE_Q4_0 && !FlatTakes(type, *d))
-    return Refuse(1, "vecq: Q4_0 takes rows of whole 256 values (up to 8192 with a GLU) whose rows, matrices and experts "
-                     "start on 16-byte boundaries");
+  // The legacy 4/5-bit blocks run through the flat form alone: rows of whole 256 values at 16-byte boundaries.
+  if (legacy && !FlatTakes(type, *d))
+    return Refuse(1, "vecq: Q4_0, Q4_1, Q5_0 and Q5_1 take rows of whole 256 values (up to 8192 with a GLU) whose rows, "
+                     "matrices and experts start on 16-byte boundaries");
   return 0;
 }
 
@@ -629,7 +630,8 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (variant < 0) variant = DefaultVariant(type, *d, a.kp, x != nullptr);
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
-  if (type == LLMP_TYPE_Q4_0 && v.lanes != 0) return Refuse(1, "vecq: Q4_0 takes the flat variants");
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && v.lanes != 0)
+    return Refuse(1, "vecq: the legacy 4/5-bit blocks take the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
   if (v.lanes < 0) {
     if (!MmaTakes(type, *d))
@@ -642,8 +644,9 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   }
   if (v.lanes == 0) {
     if (!FlatTakes(type, *d, dump != nullptr))
-      return Refuse(1, "vecq: the flat form takes Q4_K rows up to 27136 values (8192 with a GLU) and Q8_0 rows of whole "
-                       "256 values up to 32256 (4096) at 16-byte boundaries; block sums, rows up to 64 units");
+      return Refuse(1, "vecq: the flat form takes rows whose staged activations fit LDS beside three waves' tiles (Q4_K to "
+                       "41216 values, Q8_0 to 46976; 8192 and 4096 with a GLU), Q8_0 and the legacy blocks in whole 256 "
+                       "values at 16-byte boundaries; block sums, rows up to 64 units");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
       return Refuse(1, "vecq: block sums are of a dense one-token product");
     LaunchFlat(type, a, x_type, v.pass, v.flight == 2, static_cast<hipStream_t>(stream));

@@ -517,6 +517,235 @@ struct FormatQ40 {
   }
 };
 
+// ---- Q4_1, Q5_0, Q5_1: a unit is eight blocks of {f16 d; [f16 m;] [u32 high bits;] u8 nibbles[16]}
+//
+// tests/unit/dsv4_fast_test.cc:141-164 of the reference: code i is the low (i < 16) or high
+// nibble of byte i % 16, plus 16 where bit i of the high bits is set; a block times a Q8_1 block
+// is dw * (sum * d8 - 16 * s8) (Q5_0), or sum * f16(dw * d8) + f16(m * s8) for the affine types.
+// As for Q4_0 the staged activations are two images of the unit's byte layout with zeros
+// wherever the unit holds something else than nibbles (no dword holds nibbles of two blocks:
+// at least two header bytes lie between), and for the five-bit types the blocks' codes in
+// plain order as well, against the expanded high bits.
+template <int T>
+struct FormatLegacy {
+  static constexpr bool kAffine = T == 3 || T == 7;
+  static constexpr bool kFive = T == 6 || T == 7;
+  static constexpr int kPrefix = kAffine ? 4 : 2;
+  static constexpr int kCodesAt = kPrefix + (kFive ? 4 : 0);
+  static constexpr int kBlockBytes = kCodesAt + 16;
+  static constexpr int kBlockValues = 32;
+  static constexpr int kUnitBytes = 8 * kBlockBytes;
+  static constexpr int kUnitValues = 256;
+  static constexpr int kDwords = kUnitBytes / 4;
+  static constexpr int kScalesAt = 2 * kUnitBytes;  // eight d8, eight s8
+  static constexpr int kRecord = kScalesAt + 64;
+  static constexpr int kDumpInts = 8;
+
+  // The block whose nibbles dword i of a unit holds, or -1.
+  static constexpr int Owner(int i) {
+    for (int j = 0; j < 8; ++j) {
+      const int first = j * kBlockBytes + kCodesAt;
+      if (4 * i + 3 >= first && 4 * i < first + 16) return j;
+    }
+    return -1;
+  }
+
+  // One block of 32 values, eight lanes, four values a lane: lanes 0-3 hold values 0-15 (the low
+  // image), lanes 4-7 values 16-31 (the high image); each image's first lane zeroes the header.
+  static __device__ __forceinline__ void StageX(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+    uint8_t* image = record + (lane8 >> 2) * kUnitBytes + j * kBlockBytes;
+    uint16_t* at = reinterpret_cast<uint16_t*>(image + kCodesAt + 4 * (lane8 & 3));
+    at[0] = static_cast<uint16_t>(q.codes & 0xFFFFu);
+    at[1] = static_cast<uint16_t>(q.codes >> 16);
+    if ((lane8 & 3) == 0) {
+#pragma unroll
+      for (int i = 0; i < kCodesAt / 2; ++i) reinterpret_cast<uint16_t*>(image)[i] = 0;
+    }
+    if (lane8 == 0) {
+      reinterpret_cast<float*>(record + kScalesAt)[j] = HalfBitsToFloat(FloatToHalfBits(q.d));
+      reinterpret_cast<float*>(record + kScalesAt + 32)[j] = HalfBitsToFloat(FloatToHalfBits(q.sum));
+    }
+  }
+
+  // One Q8_1 block (nine dwords), one thread: the dwords of both images that start within the
+  // block's bytes (a dword that starts in the block before belongs to that block's thread).
+  static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+    const int start = j * kBlockBytes;
+    const int codes = start + kCodesAt;
+    auto value = [&](int v) { return (w[1 + (v >> 2)] >> (8 * (v & 3))) & 0xFFu; };  // v 0 .. 31
+#pragma unroll
+    for (int i = 0; i < (kBlockBytes + 3) / 4 + 1; ++i) {
+      const int at = ((start + 3) & ~3) + 4 * i;  // the dword's first byte
+      if (at < start + kBlockBytes) {
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int v = at + k - codes;
+          if (v >= 0 && v < 16) {
+            lo |= value(v) << (8 * k);
+            hi |= value(16 + v) << (8 * k);
+          }
+        }
+        *reinterpret_cast<uint32_t*>(record + at) = lo;
+        *reinterpret_cast<uint32_t*>(record + kUnitBytes + at) = hi;
+      }
+    }
+    reinterpret_cast<float*>(record + kScalesAt)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+    reinterpret_cast<float*>(record + kScalesAt + 32)[j] = HalfBitsToFloat(w[0] >> 16);
+  }
+
+  // Sixteen high bits (of values 0-15 or 16-31 of block j) as the bytes of 0 or 1 that face
+  // dword i of the unit's image: value v sits at byte first + v of the unit, so the dword's four
+  // bytes take bits 4 k - shift .. of them, k the dword's place among the block's code dwords.
+  // Four bits spread to four bytes by a multiply: bit b of the nibble lands on bit 8 b.
+  static __device__ __forceinline__ uint32_t RaisedMask(uint32_t sixteen, int j, int i) {
+    const int first = j * kBlockBytes + kCodesAt;
+    const int k = i - first / 4, shift = first % 4;
+    return __umul24(((sixteen << shift) >> (4 * k)) & 15u, 0x204081u) & 0x01010101u;
+  }
+
+  // The 16 bits at byte `at` (even) of the unit's dwords.
+  static __device__ __forceinline__ uint32_t HalfAt(const uint32_t (&w)[kDwords], int at) {
+    return (at & 2) ? w[at >> 2] >> 16 : w[at >> 2] & 0xFFFFu;
+  }
+
+  // The unit at `at` (LDS) times the staged tokens.
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    if constexpr (P > 1 || T == 6) {
+      // A block at a time, each used by every token before the next is read: the whole unit's
+      // nibbles and several tokens' images do not fit the registers (nor one token's with
+      // Q5_0's misaligned halves). The same operations in the same order as below.
+      float v[P];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if constexpr (P > 1) __builtin_amdgcn_sched_barrier(0);
+        constexpr int kSpan = (kBlockBytes + 3) / 4 + 1;  // dwords a block's bytes touch, at most
+        const int first = j * kBlockBytes / 4;
+        const int count = ((j + 1) * kBlockBytes + 3) / 4 - first;
+        uint32_t bw[kSpan];
+#pragma unroll
+        for (int i = 0; i < kSpan; ++i) bw[i] = i < count ? reinterpret_cast<const uint32_t*>(at)[first + i] : 0u;
+        auto half_at = [&](int byte) {  // the 16 bits at byte `byte` (even) of the unit
+          const int local = byte - 4 * first;
+          return (local & 2) ? bw[local >> 2] >> 16 : bw[local >> 2] & 0xFFFFu;
+        };
+        const float dw = HalfBitsToFloat(half_at(j * kBlockBytes));
+        const float mw = kAffine ? HalfBitsToFloat(half_at(j * kBlockBytes + 2)) : 0.0f;
+        uint32_t bits = 0;
+        if constexpr (kFive) bits = half_at(j * kBlockBytes + kPrefix) | (half_at(j * kBlockBytes + kPrefix + 2) << 16);
+#pragma unroll
+        for (int t = 0; t < P; ++t) {
+          if (t < m) {
+            const uint8_t* record = records + t * token_stride;
+            const uint32_t* low = reinterpret_cast<const uint32_t*>(record);
+            const uint32_t* high = reinterpret_cast<const uint32_t*>(record + kUnitBytes);
+            int sum = 0, raised = 0;
+#pragma unroll
+            for (int i = 0; i < kSpan; ++i) {
+              if (i < count && Owner(first + i) == j) {
+                const int lo = static_cast<int>(low[first + i]), hi = static_cast<int>(high[first + i]);
+                sum = Dot4(static_cast<int>(bw[i] & 0x0F0F0F0Fu), lo, sum);
+                sum = Dot4(static_cast<int>((bw[i] >> 4) & 0x0F0F0F0Fu), hi, sum);
+                if constexpr (kFive) {
+                  raised = Dot4(static_cast<int>(RaisedMask(bits & 0xFFFFu, j, first + i)), lo, raised);
+                  raised = Dot4(static_cast<int>(RaisedMask(bits >> 16, j, first + i)), hi, raised);
+                }
+              }
+            }
+            sum += 16 * raised;
+            if (kDump && dump != nullptr) dump[j] = sum;
+            const float d8 = reinterpret_cast<const float*>(record + kScalesAt)[j];
+            const float s8 = reinterpret_cast<const float*>(record + kScalesAt + 32)[j];
+            float term;
+            if constexpr (kAffine) {
+              const float scale = HalfBitsToFloat(FloatToHalfBits(dw * d8));
+              const float minimum = HalfBitsToFloat(FloatToHalfBits(mw * s8));
+              term = static_cast<float>(sum) * scale + minimum;
+            } else {
+              term = dw * (static_cast<float>(sum) * d8 - 16.0f * s8);
+            }
+            v[t] = j == 0 ? term : v[t] + term;
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < P; ++t) {
+        if (t < m) out[t] = v[t];
+      }
+      return;
+    }
+    const U32x4* mine = reinterpret_cast<const U32x4*>(at);
+    uint32_t w[kDwords];
+#pragma unroll
+    for (int i = 0; i < kDwords / 4; ++i) {
+      const U32x4 v = mine[i];
+      w[4 * i] = v.x, w[4 * i + 1] = v.y, w[4 * i + 2] = v.z, w[4 * i + 3] = v.w;
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) {
+        const uint8_t* record = records + t * token_stride;
+        const uint32_t* low = reinterpret_cast<const uint32_t*>(record);
+        const uint32_t* high = reinterpret_cast<const uint32_t*>(record + kUnitBytes);
+        int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int raised[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < kDwords; ++i) {
+          constexpr int kNone = -1;
+          const int owner = Owner(i);
+          if (owner != kNone) {
+            const int lo = static_cast<int>(low[i]), hi = static_cast<int>(high[i]);
+            s[owner] = Dot4(static_cast<int>(w[i] & 0x0F0F0F0Fu), lo, s[owner]);
+            s[owner] = Dot4(static_cast<int>((w[i] >> 4) & 0x0F0F0F0Fu), hi, s[owner]);
+            if constexpr (kFive) {
+              const int at_bits = owner * kBlockBytes + kPrefix;
+              raised[owner] = Dot4(static_cast<int>(RaisedMask(HalfAt(w, at_bits), owner, i)), lo, raised[owner]);
+              raised[owner] = Dot4(static_cast<int>(RaisedMask(HalfAt(w, at_bits + 2), owner, i)), hi, raised[owner]);
+            }
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[j] += 16 * raised[j];
+        if (kDump && dump != nullptr) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) dump[j] = s[j];
+        }
+        const float* d8 = reinterpret_cast<const float*>(record + kScalesAt);
+        const float* s8 = d8 + 8;
+        float v = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float dw = HalfBitsToFloat(HalfAt(w, j * kBlockBytes));
+          float term;
+          if constexpr (kAffine) {
+            const float mw = HalfBitsToFloat(HalfAt(w, j * kBlockBytes + 2));
+            const float scale = HalfBitsToFloat(FloatToHalfBits(dw * d8[j]));
+            const float minimum = HalfBitsToFloat(FloatToHalfBits(mw * s8[j]));
+            term = static_cast<float>(s[j]) * scale + minimum;
+          } else {
+            term = dw * (static_cast<float>(s[j]) * d8[j] - 16.0f * s8[j]);
+          }
+          v = j == 0 ? term : v + term;
+        }
+        out[t] = v;
+      }
+    }
+  }
+};
+
+using FormatQ41 = FormatLegacy<3>;
+using FormatQ50 = FormatLegacy<6>;
+using FormatQ51 = FormatLegacy<7>;
+
 // ---- staging a token's row into records
 
 template <class F, int XT>
@@ -596,13 +825,14 @@ __device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t exper
   const int row_bytes = units * F::kUnitBytes;
   const int chunks = rows * row_bytes / 16;
   const int64_t stride_bytes = static_cast<int64_t>(d.stride_row) * F::kBlockBytes;
+  // The loads (1 KB a wave each) of a part: at most 32 units a matrix with a GLU, else 64.
+  constexpr int kLoads = ((kGlu ? kWave / 2 : kWave) * F::kUnitBytes + 1023) / 1024;
   if constexpr (kGlu) {
-    // Each matrix at most 32 units: 288 chunks or fewer, five loads.
-    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
-    FetchPart<5, kPacked>(static_cast<const uint8_t*>(d.g) + first, chunks, stride_bytes, row_bytes, ring + gate_at,
-                          lane);
+    FetchPart<kLoads, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
+    FetchPart<kLoads, kPacked>(static_cast<const uint8_t*>(d.g) + first, chunks, stride_bytes, row_bytes,
+                               ring + gate_at, lane);
   } else {
-    FetchPart<9, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
+    FetchPart<kLoads, kPacked>(static_cast<const uint8_t*>(d.w) + first, chunks, stride_bytes, row_bytes, ring, lane);
   }
 }
 
@@ -617,7 +847,8 @@ __device__ __forceinline__ void AwaitTile() {
 template <class F, bool kGlu>
 __device__ __forceinline__ int TileLoads(int rows, int units) {
   const int chunks = rows * units * F::kUnitBytes / 16;
-  const int part = min((chunks + kWave - 1) / kWave, kGlu ? 5 : 9);
+  constexpr int kLoads = ((kGlu ? kWave / 2 : kWave) * F::kUnitBytes + 1023) / 1024;
+  const int part = min((chunks + kWave - 1) / kWave, kLoads);
   return kGlu ? 2 * part : part;
 }
 
@@ -904,7 +1135,7 @@ struct FlatPlan {
 };
 
 constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
-constexpr int kFewestWaves = 5;
+constexpr int kFewestWaves = 3;
 
 // Eight waves a workgroup, fewer (down to kFewestWaves) where a long row's records would
 // otherwise push the workgroup past half a CU's LDS.
@@ -1041,7 +1272,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   }
   if (pass > 1 && PlanFlat<F>(4, units, glu).lds > kFlatLdsLimit) pass = 1;
   // Two tile buffers a wave: one token a pass, packed rows, one workgroup a CU.
-  deep = deep && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
+  deep = deep && F::kUnitBytes <= 144 && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
          PlanFlat<F>(1, units, glu, true).lds <= kDeepLdsLimit;
   const FlatPlan plan = PlanFlat<F>(pass > 1 ? 4 : 1, units, glu, deep);
   if (g_compute_units == 0) {
@@ -1067,7 +1298,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
 
 // Q4_K rows up to 64 super-blocks (32 with a GLU). Q8_0 rows of whole 256 values up to 64 units
 // (32 with a GLU) whose rows, matrices and experts all start on 16-byte boundaries: the
-// tiles are fetched in 16-byte chunks. Without a GLU, and unless `whole_rows` asks for a row
+// tiles are fetched in 16-byte chunks. The legacy 4/5-bit blocks likewise, in whole 256 values. Without a GLU, and unless `whole_rows` asks for a row
 // in one tile (the block sums), longer rows in pieces, as long as their records fit.
 bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
   const bool glu = d.g != nullptr;
@@ -1078,12 +1309,17 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
-  if (type == LLMP_TYPE_Q4_0) {
+  if (type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
     if (d.ncols_x % 256 != 0 || d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || at % 16 != 0) return false;
-    const int units = d.ncols_x / FormatQ40::kUnitValues;
-    if (units > most) return pieces && PlanSplit<FormatQ40>(units).lds <= kFlatLdsLimit;
-    return PlanFlat<FormatQ40>(1, units, glu).lds <= kFlatLdsLimit;
+    const int units = d.ncols_x / 256;
+    const auto fits = [&](auto format) {
+      using F = decltype(format);
+      if (units > most) return pieces && PlanSplit<F>(units).lds <= kFlatLdsLimit;
+      return PlanFlat<F>(1, units, glu).lds <= kFlatLdsLimit;
+    };
+    return type == LLMP_TYPE_Q4_0 ? fits(FormatQ40{}) : type == LLMP_TYPE_Q4_1 ? fits(FormatQ41{})
+           : type == LLMP_TYPE_Q5_0 ? fits(FormatQ50{}) : fits(FormatQ51{});
   }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
   const int units = d.ncols_x / FormatQ8::kUnitValues;
@@ -1098,6 +1334,12 @@ void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hi
     LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q4_0) {
     LaunchF<FormatQ40>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q4_1) {
+    LaunchF<FormatQ41>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q5_0) {
+    LaunchF<FormatQ50>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q5_1) {
+    LaunchF<FormatQ51>(a, x_type, pass, deep, stream);
   } else {
     LaunchF<FormatQ8>(a, x_type, pass, deep, stream);
   }

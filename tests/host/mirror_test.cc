@@ -99,7 +99,7 @@ void HostChecks() {
   d.w = reinterpret_cast<const void*>(0x1000), d.y = reinterpret_cast<const void*>(0x2000);
   d.dst = reinterpret_cast<float*>(0x3000);
   d.ncols_x = 256, d.nrows = 4, d.stride_row = 1, d.y_token = 16, d.dst_token = 4;
-  EXPECT(!hipk::ggml::LaunchVecQ(3, d, -1, nullptr));                          // not a type these kernels read
+  EXPECT(!hipk::ggml::LaunchVecQ(4, d, -1, nullptr));                          // not a type these kernels read
   EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, 99, nullptr));          // no such variant
   d.tokens = 17;
   EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, -1, nullptr));          // 1 to 16 tokens

@@ -60,7 +60,7 @@ def desc(**kw):
     (12, dict(stride_row=1), "overlap"),
     (8, dict(ncols_x=48), "whole"),
     (8, dict(w=0x1001, stride_row=16), "aligned"),
-    (3, dict(), "type"),
+    (4, dict(), "type"),
     (12, dict(used=300), "slots"),
 ])
 def test_vecq_refusals_queue_nothing(t, kw, why):
@@ -80,7 +80,7 @@ def test_other_entry_points_refuse_bad_operands():
     assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=17)), 6, None) > 0
     assert lib.llmp_hip_vecq(8, C.byref(desc(ncols_x=480, stride_row=16, tokens=4)), 9, None) > 0
     assert lib.llmp_hip_vecq(8, C.byref(desc(stride_row=17, tokens=4)), 9, None) > 0
-    assert lib.llmp_hip_vecq(3, C.byref(desc(tokens=4)), 9, None) > 0
+    assert lib.llmp_hip_vecq(4, C.byref(desc(tokens=4)), 9, None) > 0
     assert lib.llmp_hip_vecq_fused(12, C.byref(desc()), None, -1, None) > 0
     assert lib.llmp_hip_vecq_block_sums(12, C.byref(desc()), -1, None, None) > 0
     assert lib.llmp_hip_q8_1_quantize(None, None, 32, 512, 32, 1, 1, 32, None) > 0

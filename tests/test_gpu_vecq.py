@@ -270,58 +270,63 @@ def test_guard_bytes_stay_untouched_and_refusals_queue_nothing(device):
     assert torch.equal(before.view(torch.int32), buf.view(torch.int32))
 
 
-# ---- Q4_0 through the streaming form (eight blocks of 18 bytes a lane)
+# ---- the legacy 4/5-bit blocks through the streaming form (eight blocks a lane)
 
 Q4_0 = ops.TYPE_Q4_0
+LEGACY = [ops.TYPE_Q4_0, ops.TYPE_Q4_1, ops.TYPE_Q5_0, ops.TYPE_Q5_1]
 
 
+@pytest.mark.parametrize("t", LEGACY)
 @pytest.mark.parametrize("k,n", [(4096, 96), (256, 5), (2816, 33), (15360, 12), (20480, 7)])
 @pytest.mark.parametrize("tokens", [1, 3, 4, 9])
-def test_q4_0_dense_matches_oracle(device, k, n, tokens):
-    """The legacy 4-bit block of tests/unit/dsv4_fast_test.cc:141-164: dw * (sum * d8 - 8 * s8),
-    the activation block's stored sum included. Rows of one tile, of fewer waves, and in pieces."""
-    w = synth.legacy_weights(Q4_0, n, k, 401 + k + n)
+def test_legacy_blocks_dense_match_oracle(device, t, k, n, tokens):
+    """The blocks of tests/unit/dsv4_fast_test.cc:141-164: dw * (sum * d8 - 8 or 16 * s8), or
+    sum * f16(dw * d8) + f16(m * s8), the activation block's stored sum included. Rows of one
+    tile, of fewer waves, and in pieces."""
+    w = synth.legacy_weights(t, n, k, 401 + k + n)
     x = synth.activations(tokens, k, 402 + tokens)
     q8 = oracle.q8_1_quantize(x)
-    want = oracle.vecq(Q4_0, w, q8, k, n, tokens=tokens)
-    got = ops.vecq(Q4_0, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
-    fused = ops.vecq_fused(Q4_0, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
+    fused = ops.vecq_fused(t, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
     assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
     # A token's values do not depend on the tokens beside it (one token a pass and four).
-    alone = ops.vecq(Q4_0, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
+    alone = ops.vecq(t, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
     assert np.array_equal(alone[0].view(np.uint32), got[tokens - 1].view(np.uint32))
 
 
-def test_q4_0_block_sums_and_random_bytes(device):
+@pytest.mark.parametrize("t", LEGACY)
+def test_legacy_block_sums_and_random_bytes(device, t):
     k, n = 2048, 19
-    w = synth.random_blocks(Q4_0, n, k, 411)
+    w = synth.random_blocks(t, n, k, 411)
     q8 = oracle.q8_1_quantize(synth.activations(2, k, 412))
-    want = oracle.vecq_block_sums(Q4_0, w, q8[:1], k, n)
-    got = ops.vecq_block_sums(Q4_0, dev(w, device), dev(q8[:1], device), k, n).cpu().numpy()
+    want = oracle.vecq_block_sums(t, w, q8[:1], k, n)
+    got = ops.vecq_block_sums(t, dev(w, device), dev(q8[:1], device), k, n).cpu().numpy()
     assert np.array_equal(got, want)
-    y = ops.vecq(Q4_0, dev(w, device), dev(q8, device), k, n, tokens=2).cpu().numpy()
-    ok, worst = rel_close(y, oracle.vecq(Q4_0, w, q8, k, n, tokens=2), TOL)
+    y = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=2).cpu().numpy()
+    ok, worst = rel_close(y, oracle.vecq(t, w, q8, k, n, tokens=2), TOL)
     assert ok, worst
 
 
+@pytest.mark.parametrize("t", LEGACY)
 @pytest.mark.parametrize("tokens", [1, 5])
-def test_q4_0_glu_and_routed_match_oracle(device, tokens):
+def test_legacy_blocks_glu_and_routed_match_oracle(device, t, tokens):
     k, n, experts, used = 1024, 40, 6, 2
-    gate, up = synth.legacy_weights(Q4_0, n, k, 421), synth.legacy_weights(Q4_0, n, k, 422)
+    gate, up = synth.legacy_weights(t, n, k, 421), synth.legacy_weights(t, n, k, 422)
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 423))
-    want = oracle.vecq(Q4_0, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_SWIGLU)
-    got = ops.vecq(Q4_0, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens,
+    want = oracle.vecq(t, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_SWIGLU)
+    got = ops.vecq(t, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens,
                    glu=ops.GLU_SWIGLU).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
-    w = synth.legacy_weights(Q4_0, experts * n, k, 424).reshape(experts, -1)
+    w = synth.legacy_weights(t, experts * n, k, 424).reshape(experts, -1)
     g = synth.rng(425)
     ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
     stride_expert = n * (k // 32)
-    want = oracle.vecq(Q4_0, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
-    got = ops.vecq(Q4_0, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+    want = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
                    stride_expert=stride_expert).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
