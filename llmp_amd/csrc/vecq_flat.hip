@@ -694,16 +694,18 @@ struct FormatLegacy {
     for (int t = 0; t < P; ++t) {
       if (t < m) {
         const uint8_t* record = records + t * token_stride;
-        const uint32_t* low = reinterpret_cast<const uint32_t*>(record);
-        const uint32_t* high = reinterpret_cast<const uint32_t*>(record + kUnitBytes);
+        const U32x4* low = reinterpret_cast<const U32x4*>(record);
+        const U32x4* high = reinterpret_cast<const U32x4*>(record + kUnitBytes);
         int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         int raised[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        U32x4 low4 = {0, 0, 0, 0}, high4 = {0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < kDwords; ++i) {
           constexpr int kNone = -1;
           const int owner = Owner(i);
+          if ((i & 3) == 0) low4 = low[i >> 2], high4 = high[i >> 2];
           if (owner != kNone) {
-            const int lo = static_cast<int>(low[i]), hi = static_cast<int>(high[i]);
+            const int lo = static_cast<int>(low4[i & 3]), hi = static_cast<int>(high4[i & 3]);
             s[owner] = Dot4(static_cast<int>(w[i] & 0x0F0F0F0Fu), lo, s[owner]);
             s[owner] = Dot4(static_cast<int>((w[i] >> 4) & 0x0F0F0F0Fu), hi, s[owner]);
             if constexpr (kFive) {
