@@ -191,6 +191,17 @@ int llmp_hip_mxfp8_gemm_available(void);
 size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int compute_units);
 int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream);
 
+/* ------------------------------------------------------------------ KV cache store
+ * llmp.set_rows.quant (SetRowsQuant, src/kernels/ggml/kv_quant.h:28-60,150-158): `rows` rows of k
+ * F32 values (k a multiple of 32, x_stride floats apart, 16-byte aligned) stored as rows
+ * ids[r] (I32 or I64 by index_bytes) of a Q8_0 or Q4_0 destination whose rows are row_bytes
+ * apart. Each block of 32 is quantized with the arithmetic of src/kernels/ggml/kv_quant.cuh:27-69
+ * (GGML's reference quantizers, every step an IEEE operation). The two-dimensional case of
+ * ggml_set_rows's shapes: one plane, no broadcast of the indices. Indices are the caller's to
+ * bound (kv_quant.h:62-63). */
+int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
+                            void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream);
+
 /* ------------------------------------------------------------------ EXL3
  * The trellis-coded linear. Weights as src/kernels/exl3/validate.h:84-96 holds them: the
  * trellis [k / 16][n / 16][16 * bits] uint16, suh (k F16) and svh (n F16); every dimension a

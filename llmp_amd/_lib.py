@@ -73,6 +73,7 @@ SYMBOLS = {
     "llmp_hip_moe_route": (_int, [_vp, _int, _int, _int, _int, _vp, _vp]),
     "llmp_hip_q8_1_quantize_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
+    "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmp_hip_mxfp8_swizzle": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "llmp_hip_mxfp8_gemv": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _vp, _vp]),

@@ -1,0 +1,128 @@
+// llmp.set_rows.quant for gfx950: F32 rows stored into a Q8_0 or Q4_0 cache at given row
+// indices (src/kernels/ggml/kv_quant.h:28-60 of the reference). Each block of 32 values is
+// quantized by one thread with the arithmetic of src/kernels/ggml/kv_quant.cuh:27-69, GGML's
+// reference quantizers step by step: every operation an IEEE one rounded to nearest, none
+// contracted (this unit builds without fast math).
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr int kStoreThreads = 256;  // kQuantStoreThreads, kv_quant.h:78
+
+// kv_quant.cuh:27-43: d = amax / 127, codes round-half-away(x * (1 / d)).
+__device__ __forceinline__ void StoreQ8_0(const float (&x)[32], uint8_t* to) {
+#pragma clang fp contract(off)
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 32; ++j) {
+    const float v = fabsf(x[j]);
+    amax = amax > v ? amax : v;
+  }
+  const float d = amax / 127.0f;
+  const float id = d != 0.0f ? 1.0f / d : 0.0f;
+  uint16_t* out = reinterpret_cast<uint16_t*>(to);
+  out[0] = static_cast<uint16_t>(FloatToHalfBits(d));
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const int q0 = static_cast<int8_t>(roundf(x[2 * j] * id));
+    const int q1 = static_cast<int8_t>(roundf(x[2 * j + 1] * id));
+    out[1 + j] = static_cast<uint16_t>((q0 & 0xFF) | ((q1 & 0xFF) << 8));
+  }
+}
+
+// kv_quant.cuh:45-69: the value of largest magnitude (the first among equals) over -8 as the
+// scale, codes min(15, trunc(x * (1 / d) + 8.5)), value j in byte j's low nibble and value
+// j + 16 in its high one.
+__device__ __forceinline__ void StoreQ4_0(const float (&x)[32], uint8_t* to) {
+#pragma clang fp contract(off)
+  float amax = 0.0f, vmax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 32; ++j) {
+    const float v = x[j];
+    if (amax < fabsf(v)) {
+      amax = fabsf(v);
+      vmax = v;
+    }
+  }
+  float d = vmax / -8.0f;
+  // The quotient as a value of its own before it is rounded to F16: folded into one fused
+  // conversion (vmax * -0.125 + 0) a zero block's scale would come out +0 where 0 / -8 is -0.
+  asm volatile("" : "+v"(d));
+  const float id = d != 0.0f ? 1.0f / d : 0.0f;
+  uint16_t* out = reinterpret_cast<uint16_t*>(to);
+  out[0] = static_cast<uint16_t>(FloatToHalfBits(d));
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    uint32_t pair = 0;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const float x0 = x[2 * j + b] * id;
+      const float x1 = x[16 + 2 * j + b] * id;
+      const int xi0 = min(15, static_cast<int>(static_cast<int8_t>(x0 + 8.5f)));
+      const int xi1 = min(15, static_cast<int>(static_cast<int8_t>(x1 + 8.5f)));
+      pair |= static_cast<uint32_t>((xi0 | (xi1 << 4)) & 0xFF) << (8 * b);
+    }
+    out[1 + j] = static_cast<uint16_t>(pair);
+  }
+}
+
+// A thread a block of 32 values; grid covers rows x blocks.
+template <typename Index>
+__global__ __launch_bounds__(kStoreThreads) void SetRowsQuantKernel(const float* __restrict__ x, int64_t x_stride,
+                                                                   const Index* __restrict__ ids,
+                                                                   uint8_t* __restrict__ destination, int64_t row_bytes,
+                                                                   int blocks, int64_t total, int type) {
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * kStoreThreads + threadIdx.x;
+  if (at >= total) return;
+  const int64_t row = at / blocks;
+  const int block = static_cast<int>(at - row * blocks);
+  const float4* from = reinterpret_cast<const float4*>(x + row * x_stride + block * 32);
+  float v[32];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float4 f = from[i];
+    v[4 * i] = f.x, v[4 * i + 1] = f.y, v[4 * i + 2] = f.z, v[4 * i + 3] = f.w;
+  }
+  uint8_t* to = destination + static_cast<int64_t>(ids[row]) * row_bytes;
+  if (type == LLMP_TYPE_Q8_0) {
+    StoreQ8_0(v, to + block * 34);
+  } else {
+    StoreQ4_0(v, to + block * 18);
+  }
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
+                                       void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream) {
+  if (x == nullptr || ids == nullptr || destination == nullptr) return Refuse(1, "set_rows.quant: null operand");
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_0) return Refuse(1, "set_rows.quant: a Q8_0 or Q4_0 destination");
+  if (index_bytes != 4 && index_bytes != 8) return Refuse(1, "set_rows.quant: I32 or I64 indices");
+  if (k <= 0 || k % 32 != 0 || rows <= 0) return Refuse(1, "set_rows.quant: rows of whole 32-value blocks");
+  const int64_t block_bytes = type == LLMP_TYPE_Q8_0 ? 34 : 18;
+  if (x_stride < k || x_stride % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0)
+    return Refuse(1, "set_rows.quant: source rows overlap or are not 16-byte aligned");
+  if (row_bytes < k / 32 * block_bytes || row_bytes % 2 != 0 || reinterpret_cast<uintptr_t>(destination) % 2 != 0)
+    return Refuse(1, "set_rows.quant: destination rows overlap or are not 2-byte aligned");
+  const int64_t total = rows * (k / 32);
+  if (total > 0xFFFFFFFFll / 32) return Refuse(1, "set_rows.quant: more than 2^32 - 1 values");  // kv_quant.h:150-156
+  const dim3 grid(static_cast<unsigned>((total + kStoreThreads - 1) / kStoreThreads));
+  const auto s = static_cast<hipStream_t>(stream);
+  auto* out = static_cast<uint8_t*>(destination);
+  if (index_bytes == 4) {
+    hipLaunchKernelGGL(SetRowsQuantKernel<int32_t>, grid, dim3(kStoreThreads), 0, s, x, x_stride,
+                       static_cast<const int32_t*>(ids), out, row_bytes, static_cast<int>(k / 32), total, type);
+  } else {
+    hipLaunchKernelGGL(SetRowsQuantKernel<int64_t>, grid, dim3(kStoreThreads), 0, s, x, x_stride,
+                       static_cast<const int64_t*>(ids), out, row_bytes, static_cast<int>(k / 32), total, type);
+  }
+  return LaunchStatus("set_rows.quant");
+}

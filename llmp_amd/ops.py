@@ -128,6 +128,19 @@ def vecq_sorted(t, w, q8, offsets, k, nrows, experts, *, gate=None, stride_row=N
     return out
 
 
+def set_rows_quant(t, x, ids, destination, row_bytes=None):
+    """llmp.set_rows.quant: float32 [rows, k] stored as rows ids[r] (int32 or int64) of a Q8_0 or
+    Q4_0 destination (uint8 [cells, row_bytes])."""
+    lib = _lib.load()
+    rows, k = x.shape
+    if row_bytes is None:
+        row_bytes = destination.stride(0)
+    index_bytes = 8 if ids.dtype == torch.int64 else 4
+    _lib.check(lib.llmp_hip_set_rows_quant(t, _ptr(x), x.stride(0), _ptr(ids), index_bytes, _ptr(destination),
+                                           row_bytes, k, rows, _stream()))
+    return destination
+
+
 def moe_router(logits, used, normalize=True, scale=1.0):
     """llmp.moe.router: float32 [tokens, experts] -> (ids int32 [tokens, used], weights float32)."""
     lib = _lib.load()

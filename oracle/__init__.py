@@ -68,6 +68,7 @@ _sig("orc_e8m0_to_f32", C.c_float, C.c_uint8)
 _sig("orc_f32_to_e4m3", C.c_uint8, C.c_float)
 _sig("orc_q8_1_quantize_row", None, _vp, _i64, _i64, _vp, _int)
 _sig("orc_q8_1_decode_row", None, _vp, _i64, _vp)
+_sig("orc_kv_quantize_row", None, _int, _vp, _i64, _vp)
 _sig("orc_q4_k_scale_min", None, _vp, _int, _vp, _vp)
 _sig("orc_decode_row", None, _int, _vp, _i64, _vp)
 _sig("orc_block_sums", None, _int, _vp, _vp, _vp)
@@ -121,6 +122,17 @@ def q8_1_quantize(x, flavor=Q8_DEVICE):
     out = np.zeros((rows, pk // 32 * 36), dtype=np.uint8)
     for r in range(rows):
         lib.orc_q8_1_quantize_row(_p(x[r]), k, pk, _p(out[r]), flavor)
+    return out
+
+
+def kv_quantize(t, x):
+    """float32 [rows, k] -> uint8 [rows, k/32*bytes] Q8_0 or Q4_0 blocks, GGML's reference
+    quantizers (the KV cache store's arithmetic)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, k = x.shape
+    out = np.zeros((rows, k // 32 * block_bytes(t)), dtype=np.uint8)
+    for r in range(rows):
+        lib.orc_kv_quantize_row(t, _p(x[r]), k, _p(out[r]))
     return out
 
 

@@ -28,6 +28,8 @@ static uint16_t load_u16(const uint8_t* p) {
   return v;
 }
 
+static void store_u16(uint8_t* p, uint16_t v) { memcpy(p, &v, 2); }
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();
@@ -168,6 +170,55 @@ void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y) {
     const uint8_t* x = blocks + b * 36;
     const float d = orc_f16_to_f32(load_u16(x));
     for (int j = 0; j < 32; ++j) y[b * 32 + j] = d * (float)(int8_t)x[4 + j];
+  }
+}
+
+/* ------------------------------------------------ KV cache block quantizers */
+
+/* src/kernels/ggml/kv_quant.cuh:27-43 (quantize_row_q8_0_ref step by step). */
+static void kv_q8_0_block(const float* x, uint8_t* out) {
+  float amax = 0.0f;
+  for (int j = 0; j < 32; ++j) {
+    const float v = fabsf(x[j]);
+    amax = amax > v ? amax : v;
+  }
+  const float d = amax / 127.0f;
+  const float id = d != 0.0f ? 1.0f / d : 0.0f;
+  store_u16(out, orc_f32_to_f16(d));
+  for (int j = 0; j < 32; ++j) out[2 + j] = (uint8_t)(int8_t)roundf(x[j] * id);
+}
+
+/* kv_quant.cuh:45-69 (quantize_row_q4_0_ref step by step). */
+static void kv_q4_0_block(const float* x, uint8_t* out) {
+  float amax = 0.0f, vmax = 0.0f;
+  for (int j = 0; j < 32; ++j) {
+    const float v = x[j];
+    if (amax < fabsf(v)) {
+      amax = fabsf(v);
+      vmax = v;
+    }
+  }
+  const float d = vmax / -8.0f;
+  const float id = d != 0.0f ? 1.0f / d : 0.0f;
+  store_u16(out, orc_f32_to_f16(d));
+  for (int j = 0; j < 16; ++j) {
+    const float x0 = x[j] * id;
+    const float x1 = x[16 + j] * id;
+    int xi0 = (int)(int8_t)(x0 + 8.5f);
+    int xi1 = (int)(int8_t)(x1 + 8.5f);
+    if (xi0 > 15) xi0 = 15;
+    if (xi1 > 15) xi1 = 15;
+    out[2 + j] = (uint8_t)(xi0 | (xi1 << 4));
+  }
+}
+
+void orc_kv_quantize_row(int type, const float* x, int64_t k, uint8_t* out) {
+  for (int64_t b = 0; b < k / 32; ++b) {
+    if (type == ORC_TYPE_Q8_0) {
+      kv_q8_0_block(x + b * 32, out + b * 34);
+    } else {
+      kv_q4_0_block(x + b * 32, out + b * 18);
+    }
   }
 }
 

@@ -51,6 +51,11 @@ void orc_q8_1_quantize_row(const float* x, int64_t k, int64_t padded_k, uint8_t*
 /* d * q of each block: src/kernels/reference/decode.cc:158-170. */
 void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y);
 
+/* ---- KV cache store: src/kernels/ggml/kv_quant.cuh:27-69 (GGML's reference Q8_0 and Q4_0
+ * quantizers step by step, every operation an IEEE one). One row of k floats into k / 32 blocks
+ * of 34 (ORC_TYPE_Q8_0) or 18 (ORC_TYPE_Q4_0) bytes. ---- */
+void orc_kv_quantize_row(int type, const float* x, int64_t k, uint8_t* out);
+
 /* ---- weight blocks: src/format/encoding.cc:110-116 ---- */
 enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12 }; /* ggml_type values */
 int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144 */

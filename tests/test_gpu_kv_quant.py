@@ -1,0 +1,74 @@
+"""llmp.set_rows.quant: F32 rows into a Q8_0 or Q4_0 cache at row indices, each block quantized
+with GGML's reference arithmetic (src/kernels/ggml/kv_quant.cuh:27-69 of the reference): the
+device's bytes are the oracle's."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from llmp_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def corner_rows(k):
+    """Rows that exercise the quantizers' branches: a zero block, equal magnitudes of both
+    signs (the first decides Q4_0's scale), exact half steps, one huge value, tiny values."""
+    g = synth.rng(71)
+    x = g.standard_normal((6, k), dtype=np.float32)
+    x[0, :32] = 0.0
+    x[1, :32] = np.tile(np.array([-3.0, 3.0], dtype=np.float32), 16)
+    x[2, :32] = np.tile(np.array([3.0, -3.0], dtype=np.float32), 16)
+    x[3, :32] = (np.arange(32, dtype=np.float32) - 15.5) * 0.5
+    x[4, 5] = 1.0e6
+    x[5] *= 1.0e-30
+    return x
+
+
+@pytest.mark.parametrize("t", [ops.TYPE_Q8_0, ops.TYPE_Q4_0])
+@pytest.mark.parametrize("index", [torch.int32, torch.int64])
+def test_stored_rows_are_the_reference_quantizers_bytes(device, t, index):
+    k, cells = 256, 40
+    x = np.concatenate([corner_rows(k), synth.activations(9, k, 72) * 3.0])
+    rows = x.shape[0]
+    ids = synth.rng(73).permutation(cells)[:rows]
+    row_bytes = k // 32 * ops.BLOCK_BYTES[t] + 6  # rows a few bytes apart from packed
+    cache = torch.full((cells, row_bytes), 0xA5, dtype=torch.uint8, device=device)
+    ops.set_rows_quant(t, dev(x, device), dev(ids, device).to(index), cache)
+    got = cache.cpu().numpy()
+    want = oracle.kv_quantize(t, x)
+    for r in range(rows):
+        assert np.array_equal(got[ids[r], : want.shape[1]], want[r]), r
+        assert np.all(got[ids[r], want.shape[1]:] == 0xA5)  # nothing past the row's blocks
+    untouched = np.setdiff1d(np.arange(cells), ids)
+    assert np.all(got[untouched] == 0xA5)
+
+
+def test_stored_q8_0_rows_feed_the_mat_vec(device):
+    """A cache row decodes to the values a Q8_0 weight row of the same bytes gives: the store's
+    blocks are the blocks llmp.vecq reads."""
+    k, n = 512, 8
+    x = synth.activations(n, k, 74)
+    cache = torch.zeros((n, k // 32 * 34), dtype=torch.uint8, device=device)
+    ops.set_rows_quant(ops.TYPE_Q8_0, dev(x, device), dev(np.arange(n, dtype=np.int32), device), cache)
+    a = synth.activations(1, k, 75)
+    q8 = oracle.q8_1_quantize(a)
+    got = ops.vecq(ops.TYPE_Q8_0, cache, dev(q8, device), k, n).cpu().numpy()
+    want = oracle.vecq(oracle.TYPE_Q8_0, cache.cpu().numpy(), q8, k, n)
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+def test_refusals(device):
+    x = torch.zeros((2, 64), dtype=torch.float32, device=device)
+    ids = torch.zeros(2, dtype=torch.int32, device=device)
+    cache = torch.zeros((4, 68), dtype=torch.uint8, device=device)
+    with pytest.raises(ops.KernelFailure):
+        ops.set_rows_quant(ops.TYPE_Q4_K, x, ids, cache)
+    with pytest.raises(ops.KernelFailure):
+        ops.set_rows_quant(ops.TYPE_Q8_0, x, ids, cache, row_bytes=40)  # rows would overlap
+    with pytest.raises(ops.KernelFailure):
+        ops.set_rows_quant(ops.TYPE_Q8_0, x[:, :48], ids, cache)  # not whole blocks

@@ -249,6 +249,63 @@ def test_hand_built_legacy_blocks_have_known_answers():
     assert oracle.vecq(oracle.TYPE_Q5_0, w5, q8, 32, 1)[0, 0, 0] == np.float32(total * 0.25 - 16 * 3)
 
 
+def kv_blocks_numpy(t, x):
+    """src/kernels/ggml/kv_quant.cuh:27-69 restated with numpy float32 operations (IEEE, one
+    rounding each), apart from the oracle's C."""
+    f = np.float32
+    out = []
+    for block in x.reshape(-1, 32).astype(np.float32):
+        if t == oracle.TYPE_Q8_0:
+            amax = f(np.max(np.abs(block)))
+            d = f(amax / f(127.0))
+            inv = f(f(1.0) / d) if d != 0 else f(0.0)
+            scaled = (block * inv).astype(np.float32)
+            codes = np.where(scaled >= 0, np.floor(scaled + f(0.5)), np.ceil(scaled - f(0.5)))
+            # roundf is half away from zero; floor(x + 0.5) in float32 can round up a value just below
+            # a half step, so compare in float64, where x + 0.5 is exact.
+            s64 = scaled.astype(np.float64)
+            codes = np.where(s64 >= 0, np.floor(s64 + 0.5), np.ceil(s64 - 0.5))
+            out.append(np.concatenate([np.array([d], dtype=np.float16).view(np.uint8),
+                                       codes.astype(np.int8).view(np.uint8)]))
+        else:
+            first = int(np.argmax(np.abs(block)))  # the first among equals
+            vmax = block[first] if np.abs(block[first]) > 0 else f(0.0)
+            d = f(vmax / f(-8.0))
+            inv = f(f(1.0) / d) if d != 0 else f(0.0)
+            scaled = ((block * inv).astype(np.float32) + f(8.5)).astype(np.float32)
+            codes = np.minimum(15, np.trunc(scaled).astype(np.int64))
+            packed = (codes[:16] | (codes[16:] << 4)).astype(np.uint8)
+            out.append(np.concatenate([np.array([d], dtype=np.float16).view(np.uint8), packed]))
+    return np.concatenate(out)
+
+
+def test_kv_cache_quantizers_by_restatement_and_properties():
+    from llmp_amd import synth
+    g = synth.rng(81)
+    x = g.standard_normal((7, 128), dtype=np.float32) * 2.5
+    x[0, :32] = 0.0
+    x[1, :32] = np.tile(np.array([-3.0, 3.0], dtype=np.float32), 16)
+    x[2, :32] = np.tile(np.array([3.0, -3.0], dtype=np.float32), 16)
+    x[3, :32] = (np.arange(32, dtype=np.float32) - 15.5) * 0.5
+    for t in (oracle.TYPE_Q8_0, oracle.TYPE_Q4_0):
+        got = oracle.kv_quantize(t, x)
+        for r in range(x.shape[0]):
+            assert np.array_equal(got[r], kv_blocks_numpy(t, x[r])), (t, r)
+        # Decoding what was stored lands within half a step of the input (a full step at Q4_0's
+        # clamped upper end), and a zero block stays zero.
+        dec = oracle.decode_rows(t, got, 128)
+        size = oracle.block_bytes(t)
+        d = np.abs(got.reshape(7, -1, size)[:, :, 0:2].copy().view(np.float16).astype(np.float32)).repeat(32, axis=2).reshape(7, 128)
+        bound = d * (0.5 if t == oracle.TYPE_Q8_0 else 1.0) * 1.001 + 1e-7
+        assert np.all(np.abs(dec - x) <= bound + np.abs(x) * 2e-3), t
+        assert np.all(dec[0, :32] == 0.0)
+    # Q4_0 takes its scale from the first value of largest magnitude: -3 first gives d = 0.375,
+    # codes 0 and 15 (clamped from 16); 3 first gives d = -0.375 and the codes swap.
+    q = oracle.kv_quantize(oracle.TYPE_Q4_0, x[1:3, :32])
+    assert q[0, 0:2].view(np.float16)[0] == np.float16(0.375) and q[1, 0:2].view(np.float16)[0] == np.float16(-0.375)
+    assert (q[0, 2] & 15, q[0, 3] & 15) == (0, 15) and (q[1, 2] & 15, q[1, 3] & 15) == (0, 15)
+
+
 def test_hand_built_blocks_have_known_sums():
     w = np.zeros((1, 34), dtype=np.uint8)
     w[0, 0:2] = np.array([2.0], dtype=np.float16).view(np.uint8)
