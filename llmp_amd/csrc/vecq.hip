@@ -562,8 +562,11 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   // Several tokens of a dense or grouped product over Q8_1 blocks: the matrix cores. A routed product's pairs
   // mostly name different experts, one or two tokens each: the flat form.
   // (Q8_0 from four tokens: below that the flat form's second pass costs less than the matrix-core kernel's
-  // scattered weight reads.)
-  if (tokens > (type == LLMP_TYPE_Q8_0 ? 3 : 1) && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
+  // scattered weight reads. Q4_K with a GLU from five: the matrix-core kernel's time does not depend on the
+  // tokens, 25 us at 3840 x 2 x 15360, which the flat form's four-token pass stays under: 18.5 / 22 / 25.5 us at
+  // 2 / 3 / 4 tokens.)
+  const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 3 : d.g != nullptr ? 4 : 1;
+  if (tokens > flat_up_to && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
   while (pass > 1 && LdsBytes(pass, kp) > static_cast<size_t>(kLdsBudget)) pass /= 2;
