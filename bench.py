@@ -227,7 +227,7 @@ def main():
     ap.add_argument("--eager", action="store_true", help="launch each step from Python instead of a graph")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not built (see DESIGN.md, sharding)")
+        sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not built")
 
     import numpy as np
     import torch

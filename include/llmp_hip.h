@@ -20,7 +20,9 @@
  * (src/format/encoding.cc:110-116); the legacy blocks are {f16 d; [f16 m;] [u32 high bits;] u8
  * nibbles[16]} = 18 (Q4_0), 20 (Q4_1), 22 (Q5_0), 24 (Q5_1) bytes, code i the low (i < 16) or
  * high nibble of byte i % 16 plus 16 where bit i of the high bits is set
- * (tests/unit/dsv4_fast_test.cc:141-164).
+ * (tests/unit/dsv4_fast_test.cc:141-164); MXFP4 is {e8m0 e; u8 nibbles[16]} = 17 bytes, value
+ * i the E2M1 value of the low (i < 16) or high nibble of byte i % 16, times 2^(e - 127)
+ * (src/format/encoding.cc:130-138, src/kernels/reference/decode.cc:239-248 and 417-428).
  */
 #ifndef LLMP_HIP_H_
 #define LLMP_HIP_H_
@@ -33,7 +35,7 @@ extern "C" {
 #endif
 
 /* ggml_type values of the weight encodings the kernels read. */
-enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12 };
+enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12, LLMP_TYPE_MXFP4 = 39 };
 /* VecQGlu, src/kernels/ggml/llmp_ops.h:1072. */
 enum { LLMP_GLU_NONE = 0, LLMP_GLU_SWIGLU = 1, LLMP_GLU_SWIGLU_CLAMP = 2, LLMP_GLU_GEGLU = 3 };
 /* Element types of unquantized activations. */

@@ -561,11 +561,11 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   const int tokens = d.tokens;
   // Several tokens of a dense or grouped product over Q8_1 blocks: the matrix cores. A routed product's pairs
   // mostly name different experts, one or two tokens each: the flat form.
-  // (Q8_0 from four tokens: below that the flat form's second pass costs less than the matrix-core kernel's
-  // scattered weight reads. Q4_K with a GLU from five: the matrix-core kernel's time does not depend on the
-  // tokens, 25 us at 3840 x 2 x 15360, which the flat form's four-token pass stays under: 18.5 / 22 / 25.5 us at
-  // 2 / 3 / 4 tokens.)
-  const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 3 : d.g != nullptr ? 4 : 1;
+  // (Measured at 4096 x 14336 and 3840 x 15360, with and without a GLU: the matrix-core kernel's time hardly depends
+  // on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0 (15 / 17 / 20 / 27 us
+  // against 29), four for a Q4_K gate/up pair (19 / 22 / 26 against 25-26) and two for a plain Q4_K product (12
+  // against 13).)
+  const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 5 : d.g != nullptr ? 4 : 2;
   if (tokens > flat_up_to && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
@@ -585,7 +585,7 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
 int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
   const bool legacy = type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1;
-  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && !legacy)
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_MXFP4 && !legacy)
     return Refuse(1, "vecq: weight type %d has no kernel", type);
   const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
   if (d->w == nullptr || d->dst == nullptr) return Refuse(1, "vecq: null weights or output");
@@ -608,6 +608,10 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (legacy && !FlatTakes(type, *d))
     return Refuse(1, "vecq: Q4_0, Q4_1, Q5_0 and Q5_1 take rows of whole 256 values (up to 8192 with a GLU) whose rows, "
                      "matrices and experts start on 16-byte boundaries");
+  // MXFP4 likewise; its 136-byte units come in pairs.
+  if (type == LLMP_TYPE_MXFP4 && !FlatTakes(type, *d))
+    return Refuse(1, "vecq: MXFP4 takes rows of whole 512 values (up to 8192 with a GLU) whose rows, matrices and experts "
+                     "start on 16-byte boundaries");
   return 0;
 }
 
@@ -634,7 +638,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && v.lanes != 0)
-    return Refuse(1, "vecq: the legacy 4/5-bit blocks take the flat variants");
+    return Refuse(1, "vecq: the legacy 4/5-bit blocks and MXFP4 take the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
   if (v.lanes < 0) {
     if (!MmaTakes(type, *d))
@@ -648,7 +652,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (v.lanes == 0) {
     if (!FlatTakes(type, *d, dump != nullptr))
       return Refuse(1, "vecq: the flat form takes rows whose staged activations fit LDS beside three waves' tiles (Q4_K to "
-                       "41216 values, Q8_0 to 46976; 8192 and 4096 with a GLU), Q8_0 and the legacy blocks in whole 256 "
+                       "41216 values, Q8_0 to 46976; 8192 and 4096 with a GLU), Q8_0 and the legacy blocks in whole 256 (MXFP4 512) "
                        "values at 16-byte boundaries; block sums, rows up to 64 units");
     if (dump != nullptr && (d->ids != nullptr || d->tokens != 1 || d->used != 1 || d->g != nullptr))
       return Refuse(1, "vecq: block sums are of a dense one-token product");

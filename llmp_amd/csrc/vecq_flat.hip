@@ -338,6 +338,7 @@ struct FormatQ8 {
           s[kOwner[2 * i]] = Dot4(static_cast<int>(u.w[2 * i]), static_cast<int>(x.x), s[kOwner[2 * i]]);
           s[kOwner[2 * i + 1]] = Dot4(static_cast<int>(u.w[2 * i + 1]), static_cast<int>(x.y), s[kOwner[2 * i + 1]]);
         }
+        if constexpr (P > 1) asm volatile("" : "+v"(s[0]), "+v"(s[1]), "+v"(s[2]), "+v"(s[3]));  // a token's products together
         const float2 da = *reinterpret_cast<const float2*>(record + 136);
         const float2 db = *reinterpret_cast<const float2*>(record + 144);
         if (kDump && dump != nullptr) {
@@ -369,7 +370,9 @@ struct FormatQ40 {
   static constexpr int kUnitValues = 256;
   static constexpr int kBlockBytes = 18;
   static constexpr int kBlockValues = 32;
-  static constexpr int kRecord = 352;  // two images of 144 bytes, eight d8, eight s8
+  // Two images of 144 bytes, eight d8, eight s8, and eight bytes that put the records of a
+  // row's first sixteen units in different LDS banks (90 dwords apart; read 4 or 8 bytes at a time).
+  static constexpr int kRecord = 360;
   static constexpr int kDumpInts = 8;
 
   // The image byte of value v (0 .. 15) of block j of a unit.
@@ -451,6 +454,7 @@ struct FormatQ40 {
               s = Dot4(static_cast<int>(lo_codes[i]), static_cast<int>(low[i]), s);
               s = Dot4(static_cast<int>(hi_codes[i]), static_cast<int>(high[i]), s);
             }
+            asm volatile("" : "+v"(even), "+v"(odd));  // taken here: the products stay with their pair
             const float2 d8 = *reinterpret_cast<const float2*>(record + 288 + 8 * p);
             const float2 s8 = *reinterpret_cast<const float2*>(record + 320 + 8 * p);
             const float term_even = dw_even * (static_cast<float>(even) * d8.x - 8.0f * s8.x);
@@ -483,28 +487,31 @@ struct FormatQ40 {
     for (int t = 0; t < P; ++t) {
       if (t < m) {
         const uint8_t* record = records + t * token_stride;
-        const U32x4* low = reinterpret_cast<const U32x4*>(record);
-        const U32x4* high = reinterpret_cast<const U32x4*>(record + 144);
+        const uint2* low = reinterpret_cast<const uint2*>(record);
+        const uint2* high = reinterpret_cast<const uint2*>(record + 144);
         int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 9; ++i) {
-          const U32x4 lo = low[i], hi = high[i];
+        for (int i = 0; i < 18; ++i) {
+          const uint2 lo = low[i], hi = high[i];
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const int index = 4 * i + c;
+          for (int c = 0; c < 2; ++c) {
+            const int index = 2 * i + c;
             const int owner = 2 * (index / 9) + (index % 9 >= 5 ? 1 : 0);  // the block the dword's codes belong to
-            s[owner] = Dot4(static_cast<int>(w[index] & 0x0F0F0F0Fu), static_cast<int>(lo[c]), s[owner]);
-            s[owner] = Dot4(static_cast<int>((w[index] >> 4) & 0x0F0F0F0Fu), static_cast<int>(hi[c]), s[owner]);
+            s[owner] = Dot4(static_cast<int>(w[index] & 0x0F0F0F0Fu), static_cast<int>(c ? lo.y : lo.x), s[owner]);
+            s[owner] = Dot4(static_cast<int>((w[index] >> 4) & 0x0F0F0F0Fu), static_cast<int>(c ? hi.y : hi.x), s[owner]);
           }
         }
         if (kDump && dump != nullptr) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) dump[j] = s[j];
         }
-        const float4* scales = reinterpret_cast<const float4*>(record + 288);
-        const float4 d8a = scales[0], d8b = scales[1], s8a = scales[2], s8b = scales[3];
-        const float d8[8] = {d8a.x, d8a.y, d8a.z, d8a.w, d8b.x, d8b.y, d8b.z, d8b.w};
-        const float s8[8] = {s8a.x, s8a.y, s8a.z, s8a.w, s8b.x, s8b.y, s8b.z, s8b.w};
+        const float2* scales = reinterpret_cast<const float2*>(record + 288);
+        float d8[8], s8[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float2 d = scales[j], sum = scales[4 + j];
+          d8[2 * j] = d.x, d8[2 * j + 1] = d.y, s8[2 * j] = sum.x, s8[2 * j + 1] = sum.y;
+        }
         float v = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -538,7 +545,9 @@ struct FormatLegacy {
   static constexpr int kUnitValues = 256;
   static constexpr int kDwords = kUnitBytes / 4;
   static constexpr int kScalesAt = 2 * kUnitBytes;  // eight d8, eight s8
-  static constexpr int kRecord = kScalesAt + 64;
+  // Eight more bytes put the records of a row's first sixteen units in different LDS banks
+  // (98, 106 and 114 dwords apart; read 4 or 8 bytes at a time).
+  static constexpr int kRecord = kScalesAt + 64 + 8;
   static constexpr int kDumpInts = 8;
 
   // The block whose nibbles dword i of a unit holds, or -1.
@@ -662,6 +671,7 @@ struct FormatLegacy {
               }
             }
             sum += 16 * raised;
+            asm volatile("" : "+v"(sum));  // taken here: the products stay with their block
             if (kDump && dump != nullptr) dump[j] = sum;
             const float d8 = reinterpret_cast<const float*>(record + kScalesAt)[j];
             const float s8 = reinterpret_cast<const float*>(record + kScalesAt + 32)[j];
@@ -694,18 +704,18 @@ struct FormatLegacy {
     for (int t = 0; t < P; ++t) {
       if (t < m) {
         const uint8_t* record = records + t * token_stride;
-        const U32x4* low = reinterpret_cast<const U32x4*>(record);
-        const U32x4* high = reinterpret_cast<const U32x4*>(record + kUnitBytes);
+        const uint2* low = reinterpret_cast<const uint2*>(record);
+        const uint2* high = reinterpret_cast<const uint2*>(record + kUnitBytes);
         int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         int raised[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        U32x4 low4 = {0, 0, 0, 0}, high4 = {0, 0, 0, 0};
+        uint2 low2 = {0, 0}, high2 = {0, 0};
 #pragma unroll
         for (int i = 0; i < kDwords; ++i) {
           constexpr int kNone = -1;
           const int owner = Owner(i);
-          if ((i & 3) == 0) low4 = low[i >> 2], high4 = high[i >> 2];
+          if ((i & 1) == 0) low2 = low[i >> 1], high2 = high[i >> 1];
           if (owner != kNone) {
-            const int lo = static_cast<int>(low4[i & 3]), hi = static_cast<int>(high4[i & 3]);
+            const int lo = static_cast<int>((i & 1) ? low2.y : low2.x), hi = static_cast<int>((i & 1) ? high2.y : high2.x);
             s[owner] = Dot4(static_cast<int>(w[i] & 0x0F0F0F0Fu), lo, s[owner]);
             s[owner] = Dot4(static_cast<int>((w[i] >> 4) & 0x0F0F0F0Fu), hi, s[owner]);
             if constexpr (kFive) {
@@ -747,6 +757,194 @@ struct FormatLegacy {
 using FormatQ41 = FormatLegacy<3>;
 using FormatQ50 = FormatLegacy<6>;
 using FormatQ51 = FormatLegacy<7>;
+
+// ---- MXFP4: a unit is eight blocks of {e8m0 e; u8 nibbles[16]} (136 bytes, 256 values)
+//
+// src/kernels/reference/decode.cc:239-248 and 417-428 of the reference: value i of a block is
+// the E2M1 value of the low (i < 16) or high nibble of byte 1 + i % 16, times 2^(e - 127), a
+// scale byte of 0xFF making the block NaN; src/kernels/ggml/vecq.cu:421-437: a block times a
+// Q8_1 block is (2^(e - 127) / 2 * d8) * sum(twice the E2M1 values * q). The staged activations
+// are two images of the unit's bytes as for the other four-bit blocks, zeros where the scale
+// bytes lie. A block is 17 bytes, so four of a unit's 34 dwords hold codes of two blocks: their
+// decoded values go to either block's sum under a byte mask.
+struct FormatMxfp4 {
+  static constexpr int kUnitBytes = 136;
+  static constexpr int kUnitValues = 256;
+  static constexpr int kBlockBytes = 17;
+  static constexpr int kBlockValues = 32;
+  static constexpr int kDwords = 34;
+  static constexpr int kImage = 144;  // the unit's 136 bytes, read sixteen at a time
+  static constexpr int kScalesAt = 2 * kImage;
+  // Two images, eight d8, and eight bytes so that the 16 records a 16-unit row's lanes read lie
+  // in different LDS banks (82 dwords apart).
+  static constexpr int kRecord = kScalesAt + 32 + 8;
+  static constexpr int kDumpInts = 8;
+
+  // The bytes of dword i that are codes of block j, as a mask.
+  static constexpr uint32_t CodeMask(int i, int j) {
+    uint32_t m = 0;
+    for (int k = 0; k < 4; ++k) {
+      const int at = 4 * i + k;
+      if (at % 17 != 0 && at / 17 == j) m |= 0xFFu << (8 * k);
+    }
+    return m;
+  }
+
+  // Eight codes of a dword as twice their E2M1 values, int8: the low nibbles' four and the high
+  // nibbles' four. Magnitudes {0, 1, 2, 3, 4, 6, 8, 12} by the code's low three bits, from the
+  // positive and the negative table; the code's fourth bit picks between the two, byte by byte.
+  // (a & mask) | (b & ~mask) in one instruction.
+  static __device__ __forceinline__ uint32_t Merge(uint32_t mask, uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(mask), "v"(a), "v"(b));
+    return r;
+  }
+  static __device__ __forceinline__ void Decode(uint32_t w, uint32_t& lo, uint32_t& hi) {
+    constexpr uint32_t kPosLow = 0x03020100u, kPosHigh = 0x0C080604u;
+    constexpr uint32_t kNegLow = 0xFDFEFF00u, kNegHigh = 0xF4F8FAFCu;
+    constexpr uint32_t kPlaces = 0x03020100u;  // byte k of the positive values; 4 + k, of the negative
+    const uint32_t sel_lo = w & 0x07070707u;
+    const uint32_t sel_hi = (w >> 4) & 0x07070707u;
+    const uint32_t pos_lo = __builtin_amdgcn_perm(kPosHigh, kPosLow, sel_lo);
+    const uint32_t neg_lo = __builtin_amdgcn_perm(kNegHigh, kNegLow, sel_lo);
+    const uint32_t pos_hi = __builtin_amdgcn_perm(kPosHigh, kPosLow, sel_hi);
+    const uint32_t neg_hi = __builtin_amdgcn_perm(kNegHigh, kNegLow, sel_hi);
+    lo = __builtin_amdgcn_perm(neg_lo, pos_lo, Merge(0x04040404u, w >> 1, kPlaces));
+    hi = __builtin_amdgcn_perm(neg_hi, pos_hi, Merge(0x04040404u, w >> 5, kPlaces));
+  }
+
+  // Half the block's scale, 2^(e - 128): NaN for 0xFF, subnormal for 0 and 1.
+  static __device__ __forceinline__ float HalfScale(uint32_t e) {
+    const uint32_t bits = e == 0xFFu ? 0x7FC00000u : e < 2u ? 0x00200000u << e : (e - 1u) << 23;
+    return __uint_as_float(bits);
+  }
+
+  // One block of 32 values, eight lanes, four values a lane: lanes 0-3 hold values 0-15 (the low
+  // image), lanes 4-7 values 16-31 (the high image); each image's first lane zeroes the byte
+  // that faces the scale.
+  static __device__ __forceinline__ void StageX(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+    uint8_t* image = record + (lane8 >> 2) * kImage + 17 * j;
+    uint8_t* at = image + 1 + 4 * (lane8 & 3);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) at[i] = static_cast<uint8_t>(q.codes >> (8 * i));
+    if ((lane8 & 3) == 0) image[0] = 0;
+    if (lane8 == 0) reinterpret_cast<float*>(record + kScalesAt)[j] = HalfBitsToFloat(FloatToHalfBits(q.d));
+  }
+
+  // One Q8_1 block (nine dwords), one thread: sixteen codes into either image from byte
+  // 17 j + 1 on. The three dwords that always lie within the block whole; its first three and
+  // last four bytes one by one (the dwords there are shared with the neighbouring blocks'
+  // threads), whichever of them the dwords covered already: no branches.
+  static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
+    uint8_t* record = token + (b >> 3) * kRecord;
+    const int j = b & 7;
+    const int first = 17 * j + 1;
+    const int lead = (4 - (first & 3)) & 3;  // bytes before the first whole dword
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint8_t* image = record + half * kImage;
+      const uint32_t* c = w + 1 + 4 * half;  // the sixteen codes of this half
+      image[first - 1] = 0;
+#pragma unroll
+      for (int v = 0; v < 3; ++v) image[first + v] = static_cast<uint8_t>(c[0] >> (8 * v));
+#pragma unroll
+      for (int i = 0; i < 3; ++i)
+        *reinterpret_cast<uint32_t*>(image + first + lead + 4 * i) = __builtin_amdgcn_alignbyte(c[i + 1], c[i], lead);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) image[first + 12 + v] = static_cast<uint8_t>(c[3] >> (8 * v));
+    }
+    reinterpret_cast<float*>(record + kScalesAt)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+  }
+
+  // Every code byte of dword i, whatever its block.
+  static constexpr uint32_t Codes(int i) {
+    uint32_t m = 0;
+    for (int j = 0; j < 8; ++j) m |= CodeMask(i, j);
+    return m;
+  }
+
+  // The unit at `at` (LDS) times the staged tokens: a pair of blocks (34 bytes, within nine
+  // dwords) at a time, each pair decoded once and used by every token. A pair's first or last
+  // dword also holds bytes of the pair beside it: the byte masks keep them apart.
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    float v[P];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      __builtin_amdgcn_sched_barrier(0);
+      // The pair's nine dwords begin at dword `first`; they are read eight bytes at a time from
+      // the even dword at or before it (conflict-free in LDS), units and images alike.
+      const int first = 34 * p / 4, from = first & ~1, skip = first - from;
+      const uint2* mine = reinterpret_cast<const uint2*>(at) + from / 2;
+      uint32_t lo[9], hi[9];
+      float scale[2] = {0.0f, 0.0f};
+      {
+        uint32_t w[10];
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+          const uint2 v = mine[i];
+          w[2 * i] = v.x, w[2 * i + 1] = v.y;
+        }
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+          Decode(w[skip + i], lo[i], hi[i]);
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            const int header = 17 * (2 * p + jj);
+            if (header / 4 == first + i) scale[jj] = HalfScale((w[skip + i] >> (8 * (header % 4))) & 0xFFu);
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < P; ++t) {
+        if (t < m) {
+          if constexpr (P > 1) __builtin_amdgcn_sched_barrier(0);  // one token's images at a time
+          const uint8_t* record = records + t * token_stride;
+          const uint2* low2 = reinterpret_cast<const uint2*>(record) + from / 2;
+          const uint2* high2 = reinterpret_cast<const uint2*>(record + kImage) + from / 2;
+          uint32_t low[10], high[10];
+#pragma unroll
+          for (int i = 0; i < 5; ++i) {
+            const uint2 a = low2[i], b = high2[i];
+            low[2 * i] = a.x, low[2 * i + 1] = a.y, high[2 * i] = b.x, high[2 * i + 1] = b.y;
+          }
+          int s[2] = {0, 0};
+#pragma unroll
+          for (int i = 0; i < 9; ++i) {
+            const int a = static_cast<int>(low[skip + i]), b = static_cast<int>(high[skip + i]);
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+              const uint32_t mask = CodeMask(first + i, 2 * p + jj);
+              if (mask == 0) continue;
+              const bool whole = mask == Codes(first + i);
+              s[jj] = Dot4(static_cast<int>(whole ? lo[i] : lo[i] & mask), a, s[jj]);
+              s[jj] = Dot4(static_cast<int>(whole ? hi[i] : hi[i] & mask), b, s[jj]);
+            }
+          }
+          // The sums are taken here, not wherever they are first needed: otherwise the compiler
+          // moves every pair's products to the end and keeps all their operands until then.
+          asm volatile("" : "+v"(s[0]), "+v"(s[1]));
+          if (kDump && dump != nullptr) dump[2 * p] = s[0], dump[2 * p + 1] = s[1];
+          const float2 d8 = *reinterpret_cast<const float2*>(record + kScalesAt + 8 * p);
+          const float even = (scale[0] * d8.x) * static_cast<float>(s[0]);
+          const float odd = (scale[1] * d8.y) * static_cast<float>(s[1]);
+          v[t] = p == 0 ? even : v[t] + even;
+          v[t] = v[t] + odd;
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) out[t] = v[t];
+    }
+  }
+};
 
 // ---- staging a token's row into records
 
@@ -804,10 +1002,15 @@ __device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int64
 #pragma unroll
   for (int j = 0; j < kLoads; ++j) {
     const int c = j * kWave + lane;
-    if (j * kWave < chunks && c < chunks) {  // a load is issued exactly when some lane has a chunk
+    if (j * kWave < chunks && lane < chunks - j * kWave) {  // a load is issued exactly when some lane has a chunk
       const uint8_t* from;
       if constexpr (kPacked) {
-        from = base + static_cast<uint32_t>(c) * 16u;
+        // The load's base in scalar registers, the lane's sixteen bytes the same register for
+        // every load (hidden from the compiler here, or it keeps an address a load alive
+        // across the whole tile loop).
+        uint32_t mine = static_cast<uint32_t>(lane) * 16u;
+        asm volatile("" : "+v"(mine));
+        from = base + j * (kWave * 16) + mine;
       } else {
         const int byte = c * 16;
         const int row = byte / row_bytes;
@@ -891,7 +1094,8 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   // kDeep: two tile buffers a wave (one workgroup a CU), the next tile in flight while this one
   // is multiplied.
   constexpr int kTileBytes = kWave * F::kUnitBytes;
-  uint8_t* ring = lds + P * token_stride + wave * ((kDeep ? 2 : 1) * kTileBytes);
+  // The tile buffers take 16-byte chunks: they start at the next 16-byte boundary after the records.
+  uint8_t* ring = lds + ((P * token_stride + 15) & ~15) + wave * ((kDeep ? 2 : 1) * kTileBytes);
 
   // A lane's place in every tile: its matrix, row and unit of the row.
   const int half = rows_per_tile * nsb;
@@ -1047,7 +1251,7 @@ __global__ __launch_bounds__(kGroup, 4) void VecQFlatSplit(const VecQArgs a, con
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int units = d.ncols_x / F::kUnitValues;
   const int token_stride = units * F::kRecord;
-  uint8_t* ring = lds + token_stride + wave * (kWave * F::kUnitBytes);
+  uint8_t* ring = lds + ((token_stride + 15) & ~15) + wave * (kWave * F::kUnitBytes);
   const uint8_t* my_block = ring + lane * F::kUnitBytes;
 
   int expert = blockIdx.y;
@@ -1147,7 +1351,7 @@ FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   p.rows = (glu ? kWave / 2 : kWave) / units;
   p.waves = kWaves;
   for (;;) {
-    p.lds = static_cast<size_t>(pass) * units * F::kRecord +
+    p.lds = ((static_cast<size_t>(pass) * units * F::kRecord + 15) & ~static_cast<size_t>(15)) +
             static_cast<size_t>(deep ? 2 : 1) * p.waves * kWave * F::kUnitBytes;
     if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
     --p.waves;
@@ -1230,7 +1434,8 @@ SplitPlan PlanSplit(int units) {
   p.piece = ((units + p.split - 1) / p.split + 1) & ~1;
   p.waves = kWaves;
   for (;;) {
-    p.lds = static_cast<size_t>(units) * F::kRecord + static_cast<size_t>(p.waves) * kWave * F::kUnitBytes;
+    p.lds = ((static_cast<size_t>(units) * F::kRecord + 15) & ~static_cast<size_t>(15)) +
+            static_cast<size_t>(p.waves) * kWave * F::kUnitBytes;
     if (p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
     --p.waves;
   }
@@ -1323,6 +1528,14 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     return type == LLMP_TYPE_Q4_0 ? fits(FormatQ40{}) : type == LLMP_TYPE_Q4_1 ? fits(FormatQ41{})
            : type == LLMP_TYPE_Q5_0 ? fits(FormatQ50{}) : fits(FormatQ51{});
   }
+  if (type == LLMP_TYPE_MXFP4) {
+    // A 136-byte unit: rows of an even number of units, everything on 16-byte boundaries.
+    const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+    if (d.ncols_x % 512 != 0 || d.stride_row % 16 != 0 || d.stride_expert % 16 != 0 || at % 16 != 0) return false;
+    const int units = d.ncols_x / 256;
+    if (units > most) return pieces && PlanSplit<FormatMxfp4>(units).lds <= kFlatLdsLimit;
+    return PlanFlat<FormatMxfp4>(1, units, glu).lds <= kFlatLdsLimit;
+  }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
   const int units = d.ncols_x / FormatQ8::kUnitValues;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
@@ -1342,6 +1555,8 @@ void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hi
     LaunchF<FormatQ50>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q5_1) {
     LaunchF<FormatQ51>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_MXFP4) {
+    LaunchF<FormatMxfp4>(a, x_type, pass, deep, stream);
   } else {
     LaunchF<FormatQ8>(a, x_type, pass, deep, stream);
   }

@@ -55,9 +55,21 @@ def legacy_weights(t, n, k, seed):
     return out.reshape(n, blocks * size)
 
 
+def mxfp4_weights(n, k, seed, low=112, high=124):
+    """[n, k/32*17] uint8 of MXFP4 blocks {e8m0 scale; 16 bytes of E2M1 codes}: codes uniform,
+    scale bytes uniform in [low, high) (2^-15 .. 2^-4 by default: weights up to about 0.4)."""
+    g = rng(seed)
+    blocks = k // 32
+    out = g.integers(0, 256, size=(n, blocks, 17), dtype=np.uint8)
+    out[:, :, 0] = g.integers(low, high, size=(n, blocks), dtype=np.uint8)
+    return out.reshape(n, blocks * 17)
+
+
 def random_blocks(t, n, k, seed):
     """Every field random (any finite f16 scale up to magnitude 4, any scale byte, any code):
     the bytes a decoder must take, not a plausible quantization."""
+    if t == 39:
+        return mxfp4_weights(n, k, seed, 90, 150)  # 2^-37 .. 2^22: any code, no overflow
     g = rng(seed)
     if t in LEGACY_BYTES:
         blocks, size, heads = k // 32, LEGACY_BYTES[t], 2 if t in (3, 7) else 1

@@ -18,6 +18,7 @@ TYPE_Q5_0 = 6
 TYPE_Q5_1 = 7
 TYPE_Q8_0 = 8
 TYPE_Q4_K = 12
+TYPE_MXFP4 = 39
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
 CB_3INST, CB_MCG, CB_MUL1 = 0, 1, 2
 Q8_DEVICE, Q8_GGML_CPU = 0, 1
@@ -65,6 +66,7 @@ _sig("orc_bf16_to_f32", C.c_float, C.c_uint16)
 _sig("orc_f32_to_bf16", C.c_uint16, C.c_float)
 _sig("orc_e4m3_to_f32", C.c_float, C.c_uint8)
 _sig("orc_e8m0_to_f32", C.c_float, C.c_uint8)
+_sig("orc_e2m1_to_f32", C.c_float, C.c_uint8)
 _sig("orc_f32_to_e4m3", C.c_uint8, C.c_float)
 _sig("orc_q8_1_quantize_row", None, _vp, _i64, _i64, _vp, _int)
 _sig("orc_q8_1_decode_row", None, _vp, _i64, _vp)
@@ -103,7 +105,7 @@ def max_threads():
 
 
 def block_bytes(t):
-    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144}[t]
+    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17}[t]
 
 
 def block_elements(t):

@@ -234,6 +234,7 @@ int orc_block_bytes(int type) {
     case ORC_TYPE_Q5_1: return 24;
     case ORC_TYPE_Q8_0: return 34;
     case ORC_TYPE_Q4_K: return 144;
+    case ORC_TYPE_MXFP4: return 17; /* encoding.cc:130-138 */
     default: return 0;
   }
 }
@@ -254,6 +255,18 @@ static int legacy_code(int type, const uint8_t* w, int i) {
   return low + (legacy_five(type) ? (int)((high >> i) & 1u) * 16 : 0);
 }
 
+/* decode.cc:424-428: the E2M1 value of a four-bit code. */
+float orc_e2m1_to_f32(uint8_t code) {
+  static const float values[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+  const float v = values[code & 7u];
+  return (code & 8u) ? -v : v;
+}
+/* Code i of a block_mxfp4 {e8m0 e; u8 qs[16]}: byte j holds values j (low nibble) and j + 16
+ * (decode.cc:239-248). */
+static int mxfp4_code(const uint8_t* w, int i) { return i < 16 ? w[1 + i] & 15 : w[1 + i - 16] >> 4; }
+/* Twice the E2M1 value, an integer (the table vecq.cu:424 looks codes up in). */
+static int mxfp4_twice(int code) { return (int)(2.0f * orc_e2m1_to_f32((uint8_t)code)); }
+
 /* dsv4_fast_test.cc:180-183 */
 void orc_q4_k_scale_min(const uint8_t* scales, int g, int* scale, int* minimum) {
   *scale = g < 4 ? scales[g] & 63 : (scales[g + 4] & 15) | ((scales[g - 4] >> 6) << 4);
@@ -265,6 +278,13 @@ static int q4_k_code(const uint8_t* codes, int g, int i) {
 }
 
 void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
+  if (type == ORC_TYPE_MXFP4) { /* decode.cc:239-248 */
+    for (int64_t j = 0; j < k; ++j) {
+      const uint8_t* x = row + j / 32 * 17;
+      y[j] = orc_e2m1_to_f32((uint8_t)mxfp4_code(x, (int)(j % 32))) * orc_e8m0_to_f32(x[0]);
+    }
+    return;
+  }
   if (legacy(type)) {
     /* ggml's dequantization of these bytes: d * (code - 8 or 16), or d * code + m. */
     const int bs = orc_block_bytes(type);
@@ -301,6 +321,12 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
 }
 
 void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums) {
+  if (type == ORC_TYPE_MXFP4) { /* vecq.cu:421-435: the doubled values times the codes */
+    int32_t s = 0;
+    for (int i = 0; i < 32; ++i) s += mxfp4_twice(mxfp4_code(w, i)) * (int32_t)(int8_t)q8[4 + i];
+    sums[0] = s;
+    return;
+  }
   if (legacy(type)) { /* dsv4_fast_test.cc:154-158 */
     int32_t s = 0;
     for (int i = 0; i < 32; ++i) s += legacy_code(type, w, i) * (int32_t)(int8_t)q8[4 + i];
@@ -329,6 +355,9 @@ void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums
 double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
   int32_t sums[16];
   orc_block_sums(type, w, q8, sums);
+  if (type == ORC_TYPE_MXFP4) { /* vecq.cu:426,437: half the block's scale, times d8, times the sum */
+    return (double)orc_e8m0_to_f32(w[0]) * 0.5 * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
+  }
   if (legacy(type)) { /* dsv4_fast_test.cc:145-164: the Q8_1 block's s is the rounded sum of its inputs */
     const float dw = orc_f16_to_f32(load_u16(w));
     const float da = orc_f16_to_f32(load_u16(q8));

@@ -38,6 +38,7 @@ float orc_bf16_to_f32(uint16_t bits);
 uint16_t orc_f32_to_bf16(float value);
 float orc_e4m3_to_f32(uint8_t bits);
 float orc_e8m0_to_f32(uint8_t bits);
+float orc_e2m1_to_f32(uint8_t code); /* decode.cc:424-428 */
 /* Saturating-finite round-to-nearest-even E4M3, what __nv_cvt_float2_to_fp8x2(
  * ..., __NV_SATFINITE, __NV_E4M3) gives (src/kernels/ggml/mxfp8_quant.cuh:38-46). */
 uint8_t orc_f32_to_e4m3(float value);
@@ -57,8 +58,8 @@ void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y);
 void orc_kv_quantize_row(int type, const float* x, int64_t k, uint8_t* out);
 
 /* ---- weight blocks: src/format/encoding.cc:110-116 ---- */
-enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12 }; /* ggml_type values */
-int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144 */
+enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12, ORC_TYPE_MXFP4 = 39 }; /* ggml_type values */
+int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144, MXFP4 17 */
 int orc_block_elements(int type); /* 32, Q4_K 256 */
 /* The Q4_K 6-bit scale and minimum of sub-block g: tests/unit/dsv4_fast_test.cc:180-183. */
 void orc_q4_k_scale_min(const uint8_t* scales12, int g, int* scale, int* minimum);
@@ -67,7 +68,9 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y);
 /* Per-block int32 sums over identical Q8_1 bytes. Q8_0 and the legacy 4/5-bit blocks:
  * sums[0] = sum w*q (code*q) of the 32 values (src/kernels/ggml/vecq.cu:398-418,
  * tests/unit/dsv4_fast_test.cc:154-158). Q4_K: sums[0..7] = sum code*q per
- * sub-block, sums[8..15] = sum q per sub-block (tests/unit/dsv4_fast_test.cc:185-191). */
+ * sub-block, sums[8..15] = sum q per sub-block (tests/unit/dsv4_fast_test.cc:185-191).
+ * MXFP4: sums[0] = sum of twice the E2M1 values times q (vecq.cu:421-435, the values of
+ * src/kernels/reference/decode.cc:424-428). */
 void orc_block_sums(int type, const uint8_t* wblock, const uint8_t* q8, int32_t* sums);
 /* One weight block times its Q8_1 blocks in double. */
 double orc_block_product(int type, const uint8_t* wblock, const uint8_t* q8);

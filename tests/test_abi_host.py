@@ -61,6 +61,10 @@ def desc(**kw):
     (8, dict(ncols_x=48), "whole"),
     (8, dict(w=0x1001, stride_row=16), "aligned"),
     (4, dict(), "type"),
+    (39, dict(ncols_x=768, stride_row=24), "MXFP4"),
+    (39, dict(ncols_x=512, stride_row=24), "MXFP4"),
+    (39, dict(w=0x1004, stride_row=16), "MXFP4"),
+    (2, dict(ncols_x=288, stride_row=9), "Q4_0"),
     (12, dict(used=300), "slots"),
 ])
 def test_vecq_refusals_queue_nothing(t, kw, why):

@@ -117,7 +117,7 @@ def test_gemm_matches_the_product_of_the_quantized_operands(device, m, n, k, bf1
 
 
 def test_gemm_full_size_sampled(device):
-    """BASELINE's shape, M 2048, K 4096, N 12288: sampled entries against the oracle's dot, and
+    """The headline prefill shape, M 2048, K 4096, N 12288: sampled entries against the oracle's dot, and
     linearity in the activations' scales (doubling a row's scales doubles its outputs exactly)."""
     m, n, k = 2048, 12288, 4096
     g = synth.rng(31)

@@ -340,3 +340,87 @@ def test_q4_0_refuses_what_the_streaming_form_does_not_take(device):
         ops.vecq(Q4_0, dev(w, device), dev(q8, device), k, n)
     with pytest.raises(ops.KernelFailure):  # the rows form has no Q4_0
         ops.vecq(Q4_0, dev(synth.legacy_weights(Q4_0, n, 256, 433), device), dev(q8, device), 256, n, variant=0)
+
+
+# ---- MXFP4 through the streaming form (eight 17-byte blocks a lane)
+
+MXFP4 = ops.TYPE_MXFP4
+
+
+@pytest.mark.parametrize("k,n", [(4096, 96), (512, 5), (2560, 33), (15360, 12), (20480, 7)])
+@pytest.mark.parametrize("tokens", [1, 3, 4, 9])
+def test_mxfp4_dense_matches_oracle(device, k, n, tokens):
+    """src/kernels/ggml/vecq.cu:421-437 over the values of src/kernels/reference/decode.cc:239-248:
+    (2^(e - 127) / 2 * d8) * sum(twice the E2M1 values * q). Rows of one tile, of fewer waves, and
+    in pieces; quantized beforehand or in the kernel; a token alone or among others."""
+    w = synth.mxfp4_weights(n, k, 501 + k + n)
+    x = synth.activations(tokens, k, 502 + tokens)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(MXFP4, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    fused = ops.vecq_fused(MXFP4, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    alone = ops.vecq(MXFP4, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
+    assert np.array_equal(alone[0].view(np.uint32), got[tokens - 1].view(np.uint32))
+
+
+def test_mxfp4_block_sums_and_every_scale_byte(device):
+    """The int32 sums bit for bit over random bytes; then every scale byte there is, subnormal
+    (0 and 1) and NaN (0xFF) included, one block a row so that each output is one block's term."""
+    k, n = 2048, 19
+    w = synth.random_blocks(MXFP4, n, k, 511)
+    q8 = oracle.q8_1_quantize(synth.activations(2, k, 512))
+    want = oracle.vecq_block_sums(MXFP4, w, q8[:1], k, n)
+    got = ops.vecq_block_sums(MXFP4, dev(w, device), dev(q8[:1], device), k, n).cpu().numpy()
+    assert np.array_equal(got, want)
+    y = ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n, tokens=2).cpu().numpy()
+    ok, worst = rel_close(y, oracle.vecq(MXFP4, w, q8, k, n, tokens=2), TOL)
+    assert ok, worst
+    k, n = 512, 256
+    w = np.zeros((n, k // 32, 17), dtype=np.uint8)
+    w[:, :, 0] = 127
+    for r in range(n):  # row r: block r % 16 holds codes and scale byte r, the others zeros
+        w[r, r % 16, 0] = r
+        w[r, r % 16, 1:] = synth.rng(513 + r).integers(0, 256, size=16, dtype=np.uint8)
+    w = w.reshape(n, -1)
+    q8 = oracle.q8_1_quantize(synth.activations(1, k, 514) * 1e-3)
+    want = oracle.vecq(MXFP4, w, q8, k, n)[0, 0]
+    got = ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n).cpu().numpy().reshape(-1)
+    assert np.isnan(got[255]) and np.isnan(want[255])
+    # Half the scale times d8 (about 2^-15 here) is exact while it is a normal float: one rounding,
+    # the same bits. Below that (scale bytes under 20) the product is subnormal and loses bits.
+    assert np.array_equal(got[20:255].view(np.uint32), want[20:255].view(np.uint32))
+    assert np.allclose(got[:20], want[:20], rtol=0.1, atol=1e-44) and np.all(np.sign(got[:20]) == np.sign(want[:20]))
+
+
+@pytest.mark.parametrize("tokens", [1, 5])
+def test_mxfp4_glu_and_routed_match_oracle(device, tokens):
+    k, n, experts, used = 1024, 40, 6, 2
+    gate, up = synth.mxfp4_weights(n, k, 521), synth.mxfp4_weights(n, k, 522)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 523))
+    want = oracle.vecq(MXFP4, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_SWIGLU)
+    got = ops.vecq(MXFP4, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens,
+                   glu=ops.GLU_SWIGLU).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    w = synth.mxfp4_weights(experts * n, k, 524).reshape(experts, -1)
+    g = synth.rng(525)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    stride_expert = n * (k // 32)
+    want = oracle.vecq(MXFP4, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+def test_mxfp4_refuses_what_the_streaming_form_does_not_take(device):
+    k, n = 768, 4  # whole 256 values, not whole 512: a row would start off a 16-byte boundary
+    w = synth.mxfp4_weights(n, k, 531)
+    q8 = oracle.q8_1_quantize(synth.activations(1, k, 532))
+    with pytest.raises(ops.KernelFailure):
+        ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n)
+    with pytest.raises(ops.KernelFailure):  # the rows form has no MXFP4
+        ops.vecq(MXFP4, dev(synth.mxfp4_weights(n, 512, 533), device), dev(q8, device), 512, n, variant=0)

@@ -249,6 +249,75 @@ def test_hand_built_legacy_blocks_have_known_answers():
     assert oracle.vecq(oracle.TYPE_Q5_0, w5, q8, 32, 1)[0, 0, 0] == np.float32(total * 0.25 - 16 * 3)
 
 
+def test_mxfp4_values_layout_and_products():
+    """MXFP4 as the reference's own CPU decoder has it (src/kernels/reference/decode.cc:239-248,
+    417-428) and its known answers (tests/unit/reference_decode_test.cc:465-484: bytes of 0x22
+    are ones, scale bytes 0x00 / 0x7F / 0xFE are 2^-127 / 1 / 2^127, 0xFF is NaN); the product
+    of src/kernels/ggml/vecq.cu:421-437 against a numpy restatement and a hand-built block."""
+    from llmp_amd import synth
+    # The E2M1 values, by the format's definition: sign, two exponent bits, one mantissa bit,
+    # bias 1, subnormal at exponent 0.
+    for code in range(16):
+        e, m = (code >> 1) & 3, code & 1
+        magnitude = 0.5 * m if e == 0 else (1.0 + 0.5 * m) * 2.0 ** (e - 1)
+        assert oracle.lib.orc_e2m1_to_f32(code) == (-magnitude if code & 8 else magnitude)
+    assert [oracle.lib.orc_e2m1_to_f32(c) for c in range(8)] == [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    assert oracle.block_bytes(oracle.TYPE_MXFP4) == 17 and oracle.block_elements(oracle.TYPE_MXFP4) == 32
+    # reference_decode_test.cc:465-484
+    k = 128
+    row = np.concatenate([np.concatenate([[e], np.full(16, 0x22)]) for e in (0x00, 0x7F, 0xFE, 0xFF)]).astype(np.uint8)
+    got = oracle.decode_rows(oracle.TYPE_MXFP4, row[None, :], k)[0]
+    assert np.array_equal(got[:32], np.full(32, 2.0 ** -127, dtype=np.float32))
+    assert np.array_equal(got[32:64], np.ones(32, dtype=np.float32))
+    assert np.array_equal(got[64:96], np.full(32, 2.0 ** 127, dtype=np.float32))
+    assert np.all(np.isnan(got[96:]))
+    # Layout: byte j of a block holds values j (low nibble) and j + 16.
+    block = np.zeros(17, dtype=np.uint8)
+    block[0] = 128  # scale 2
+    block[1 + 3] = 0x5 | (0xC << 4)  # value 3 = code 5 (3.0), value 19 = code 12 (-2.0)
+    got = oracle.decode_rows(oracle.TYPE_MXFP4, block[None, :], 32)[0]
+    want = np.zeros(32, dtype=np.float32)
+    want[3], want[19] = 6.0, -4.0
+    assert np.array_equal(got, want)
+    # Products: numpy restatement over random bytes.
+    table = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], dtype=np.int64)
+    k, n = 512, 5
+    x = np.random.Generator(np.random.PCG64(28)).standard_normal((1, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    acts = q8[0].reshape(-1, 36)
+    for w in (synth.random_blocks(oracle.TYPE_MXFP4, n, k, 29), synth.mxfp4_weights(n, k, 30)):
+        sums = oracle.vecq_block_sums(oracle.TYPE_MXFP4, w, q8, k, n)
+        y = oracle.vecq(oracle.TYPE_MXFP4, w, q8, k, n)[0, 0]
+        dec = oracle.decode_rows(oracle.TYPE_MXFP4, w, k)
+        for r in range(n):
+            total, row = 0.0, []
+            for b, blk in enumerate(w[r].reshape(-1, 17)):
+                codes = np.concatenate([blk[1:] & 15, blk[1:] >> 4]).astype(np.int64)
+                q = acts[b][4:].view(np.int8).astype(np.int64)
+                s = int((table[codes] * q).sum())
+                assert sums[r, b, 0] == s
+                scale = 2.0 ** (int(blk[0]) - 127)
+                total += scale * 0.5 * float(acts[b][0:2].view(np.float16)[0]) * s
+                row.append((table[codes] * 0.5 * scale).astype(np.float32))
+            np.testing.assert_array_equal(dec[r], np.concatenate(row))
+            np.testing.assert_allclose(y[r], total, rtol=1e-6, atol=1e-12)
+        # The product is the decoded weights times the decoded activations.
+        dense = dec.astype(np.float64) @ oracle.q8_1_decode(q8[0], k).astype(np.float64)
+        np.testing.assert_allclose(y, dense, rtol=1e-5, atol=1e-9)
+    # By hand: scale byte 126 (0.5), codes i % 16 in both halves; activation d = 0.25, q = 2 against
+    # codes 0..7 (twice their values add up to 36) and -2 against codes 8..15 (-36):
+    # sum = 2 halves * (2 * 36 + -2 * -36) = 288; times 0.5 / 2 * 0.25 = 18.
+    w = np.zeros((1, 17), dtype=np.uint8)
+    w[0, 0] = 126
+    w[0, 1:] = np.arange(16, dtype=np.uint8) * 17
+    q8 = np.zeros((1, 16 * 36), dtype=np.uint8)
+    q8[0, 0:2] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    q = np.where(np.arange(32) % 16 < 8, 2, -2).astype(np.int8)
+    q8[0, 4:36] = q.view(np.uint8)
+    assert oracle.vecq_block_sums(oracle.TYPE_MXFP4, w, q8, 32, 1)[0, 0, 0] == 288
+    assert oracle.vecq(oracle.TYPE_MXFP4, w, q8, 32, 1)[0, 0, 0] == 18.0
+
+
 def kv_blocks_numpy(t, x):
     """src/kernels/ggml/kv_quant.cuh:27-69 restated with numpy float32 operations (IEEE, one
     rounding each), apart from the oracle's C."""
