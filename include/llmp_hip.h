@@ -253,6 +253,26 @@ typedef struct llmp_exl3_linear {
 size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op);
 int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream);
 
+/* exl3.multi_linear.mgemm: MultiLinear of src/kernels/exl3/linear.h:51-53 over the operands of
+ * src/kernels/exl3/validate.h:160-172, a gate and an up linear of the same k, n and rate over
+ * one input (tests/unit/exl3_trellis_test.cc:664-716). x (m x k F16) into y (2 x m x n: the
+ * first linear's rows, then the second's); a_had is 2 x m x k F16 (validate.cc:257-260), each
+ * linear's own transformed input. The reference's three pointer tables have no counterpart:
+ * the launches carry the six addresses. Same launches as llmp_hip_exl3_linear, both linears in
+ * each (one linear after the other where their codebooks differ); `scratch` is
+ * llmp_hip_exl3_multi_linear_scratch bytes. */
+typedef struct llmp_exl3_multi_linear {
+  llmp_exl3_weights first;
+  llmp_exl3_weights second;
+  const void* x;
+  void* a_had;
+  void* y;
+  int f32; /* y in F32, else F16 */
+  int m;
+} llmp_exl3_multi_linear;
+size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op);
+int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, size_t scratch_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -183,6 +183,41 @@ inline KernelFailure PackedLinear(const LinearOperands& o, void* scratch, std::s
   return FromStatus(llmp_hip_exl3_linear(&abi, scratch, scratch_bytes, stream));
 }
 
+// src/kernels/exl3/validate.h:160-172 without the pointer tables (the launches carry the
+// addresses): a gate and an up linear over one input, y the first's m x n rows then the second's.
+struct MultiLinearOperands {
+  Weights first;
+  Weights second;
+  std::uint64_t x = 0;      // m x k F16
+  std::uint64_t a_had = 0;  // 2 x m x k F16 scratch
+  std::uint64_t y = 0;      // 2 x m x n
+  bool f32 = false;
+  int m = 0;
+};
+
+inline llmp_exl3_multi_linear ToAbi(const MultiLinearOperands& o) {
+  LinearOperands one;
+  one.weights = o.first;
+  llmp_exl3_multi_linear abi{};
+  abi.first = ToAbi(one).weights;
+  one.weights = o.second;
+  abi.second = ToAbi(one).weights;
+  abi.x = reinterpret_cast<const void*>(o.x);
+  abi.a_had = reinterpret_cast<void*>(o.a_had);
+  abi.y = reinterpret_cast<void*>(o.y);
+  abi.f32 = o.f32 ? 1 : 0, abi.m = o.m;
+  return abi;
+}
+inline std::size_t ScratchBytes(const MultiLinearOperands& o) {
+  const llmp_exl3_multi_linear abi = ToAbi(o);
+  return llmp_hip_exl3_multi_linear_scratch(&abi);
+}
+// MultiLinear of src/kernels/exl3/linear.h:51-53.
+inline KernelFailure MultiLinear(const MultiLinearOperands& o, void* scratch, std::size_t scratch_bytes, void* stream) {
+  const llmp_exl3_multi_linear abi = ToAbi(o);
+  return FromStatus(llmp_hip_exl3_multi_linear(&abi, scratch, scratch_bytes, stream));
+}
+
 }  // namespace exl3
 }  // namespace llmp_amd
 

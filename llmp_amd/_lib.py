@@ -51,6 +51,13 @@ class Exl3Linear(C.Structure):
                 ("f32", C.c_int), ("m", C.c_int)]
 
 
+class Exl3MultiLinear(C.Structure):
+    """llmp_exl3_multi_linear: MultiLinearOperands of src/kernels/exl3/validate.h:160-172 of the reference,
+    without its pointer tables."""
+    _fields_ = [("first", Exl3Weights), ("second", Exl3Weights), ("x", C.c_void_p), ("a_had", C.c_void_p),
+                ("y", C.c_void_p), ("f32", C.c_int), ("m", C.c_int)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -85,6 +92,8 @@ SYMBOLS = {
     "llmp_hip_exl3_hadamard": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),
     "llmp_hip_exl3_linear": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _vp]),
+    "llmp_hip_exl3_multi_linear_scratch": (C.c_size_t, [C.POINTER(Exl3MultiLinear)]),
+    "llmp_hip_exl3_multi_linear": (_int, [C.POINTER(Exl3MultiLinear), _vp, C.c_size_t, _vp]),
 }
 
 _lib = None

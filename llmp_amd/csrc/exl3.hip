@@ -179,11 +179,24 @@ __device__ __forceinline__ void Hadamard128(float& a, float& b, int lane) {
 
 // y = f(H(x * in_scale)) * r * out_scale over each 128 block of each row; grid (rows, columns
 // / 128), a wave a block. X / Y: 0 F16, 1 F32. `slices` partial inputs are added in order first.
+// One or two transforms a launch (grid z): a linear's, or the two of a gate/up pair.
+struct HadamardSides {
+  const void* x[2];
+  void* y[2];
+  const uint16_t* in_scale[2];
+  const uint16_t* out_scale[2];
+};
+inline HadamardSides OneSide(const void* x, void* y, const uint16_t* in_scale, const uint16_t* out_scale) {
+  return HadamardSides{{x, x}, {y, y}, {in_scale, in_scale}, {out_scale, out_scale}};
+}
+
 template <int X, int Y>
-__global__ __launch_bounds__(64) void HadamardKernel(const void* __restrict__ x, void* __restrict__ y,
-                                                    const uint16_t* __restrict__ in_scale,
-                                                    const uint16_t* __restrict__ out_scale, int columns, int slices,
+__global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, int columns, int slices,
                                                     int64_t slice_stride) {
+  const void* __restrict__ x = sides.x[blockIdx.z];
+  void* __restrict__ y = sides.y[blockIdx.z];
+  const uint16_t* __restrict__ in_scale = sides.in_scale[blockIdx.z];
+  const uint16_t* __restrict__ out_scale = sides.out_scale[blockIdx.z];
   const int lane = threadIdx.x;
   const int64_t at = static_cast<int64_t>(blockIdx.x) * columns + blockIdx.y * 128 + 2 * lane;
   float a = 0.0f, b = 0.0f;
@@ -235,13 +248,22 @@ constexpr int kReduceBytes = kProductWaves * 32 * 64 * 4;
 // eight tiles per 16 rows of K, and the waves' sums are added in wave order through LDS.
 // Every column block repeats the transform, which is cheap for a few tokens only: without
 // kFused, x is the transformed input already and a_had is not written.
+struct ProductSides {  // one or two linears a launch (grid z)
+  const uint8_t* trellis[2];
+  const uint16_t* x[2];
+  const uint16_t* suh[2];
+  uint16_t* a_had[2];
+  float* partial[2];
+};
+
 template <int CB, int BITS, bool kFused>
-__global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const uint8_t* __restrict__ trellis,
-                                                                   const uint16_t* __restrict__ x,
-                                                                   const uint16_t* __restrict__ suh,
-                                                                   uint16_t* __restrict__ a_had,
-                                                                   float* __restrict__ partial, int m, int n, int k,
+__global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const ProductSides sides, int m, int n, int k,
                                                                    int blocks_per_wave) {
+  const uint8_t* __restrict__ trellis = sides.trellis[blockIdx.z];
+  const uint16_t* __restrict__ x = sides.x[blockIdx.z];
+  const uint16_t* __restrict__ suh = sides.suh[blockIdx.z];
+  uint16_t* __restrict__ a_had = sides.a_had[blockIdx.z];
+  float* __restrict__ partial = sides.partial[blockIdx.z];
   constexpr int kTileBytes = BITS * 32;
   constexpr int kStepBytes = 8 * kTileBytes;  // a 128-column block's tiles of one K step
   constexpr int kLoads = (kStepBytes + 1023) / 1024;
@@ -391,7 +413,7 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
 constexpr int kFusedRows = 4;  // up to here the product transforms its input itself
 
 template <int CB, int BITS, bool kFused>
-void LaunchProduct(const llmp_exl3_weights& w, const void* x, void* a_had, float* partial, int m, int slices,
+void LaunchProduct(const llmp_exl3_weights& w, const ProductSides& sides, int count, int m, int slices,
                    hipStream_t stream) {
   constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
   constexpr int kWork = kProductWaves * (kRingDepth * kLoads * 1024 + kOperandBytes);
@@ -404,10 +426,9 @@ void LaunchProduct(const llmp_exl3_weights& w, const void* x, void* a_had, float
   }
   const int blocks = w.k / 128;
   const int per = (blocks + slices * kProductWaves - 1) / (slices * kProductWaves);
-  const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices));
-  hipLaunchKernelGGL((ProductKernel<CB, BITS, kFused>), grid, dim3(kProductWaves * 64), kLds, stream,
-                     static_cast<const uint8_t*>(w.trellis), static_cast<const uint16_t*>(x),
-                     static_cast<const uint16_t*>(w.suh), static_cast<uint16_t*>(a_had), partial, m, w.n, w.k, per);
+  const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices), static_cast<unsigned>(count));
+  hipLaunchKernelGGL((ProductKernel<CB, BITS, kFused>), grid, dim3(kProductWaves * 64), kLds, stream, sides, m, w.n, w.k,
+                     per);
 }
 
 template <typename F>
@@ -467,14 +488,70 @@ extern "C" int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale,
   const auto s = static_cast<hipStream_t>(stream);
   const auto* sc = static_cast<const uint16_t*>(scale);
   if (f32) {
-    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, x, y, nullptr, sc, columns, 1, int64_t{0});
+    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, OneSide(x, y, nullptr, sc), columns, 1, int64_t{0});
   } else if (input_scale) {
-    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, x, y, sc, nullptr, columns, 1, int64_t{0});
+    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, OneSide(x, y, sc, nullptr), columns, 1, int64_t{0});
   } else {
-    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, x, y, nullptr, sc, columns, 1, int64_t{0});
+    hipLaunchKernelGGL((HadamardKernel<0, 0>), grid, dim3(64), 0, s, OneSide(x, y, nullptr, sc), columns, 1, int64_t{0});
   }
   return LaunchStatus("exl3.hadamard");
 }
+
+namespace llmp_hip {
+namespace {
+
+// `count` linears of the same shape, rate and codebook over one input: the transformed input
+// (a launch of its own above a few rows), the products in slices of K, the slices' sums
+// transformed. Linear i writes a_had[i], scratch[i] and y[i].
+int LaunchLinears(const llmp_exl3_weights* const (&w)[2], int count, const void* x, void* const (&a_had)[2],
+                  void* const (&y)[2], float* const (&scratch)[2], bool f32, int m, const char* what, hipStream_t s) {
+  const llmp_exl3_weights& w0 = *w[0];
+  const int slices = SlicesFor(w0.n, w0.k);
+  const bool fused = m <= kFusedRows;
+  const auto* suh0 = static_cast<const uint16_t*>(w[0]->suh);
+  const auto* suh1 = static_cast<const uint16_t*>(w[1]->suh);
+  if (!fused) {
+    const HadamardSides in{{x, x}, {a_had[0], a_had[1]}, {suh0, suh1}, {nullptr, nullptr}};
+    hipLaunchKernelGGL((HadamardKernel<0, 0>),
+                       dim3(static_cast<unsigned>(m), static_cast<unsigned>(w0.k / 128), static_cast<unsigned>(count)),
+                       dim3(64), 0, s, in, w0.k, 1, int64_t{0});
+    if (const int bad = LaunchStatus(what); bad != 0) return bad;
+  }
+  ProductSides sides;
+  for (int i = 0; i < 2; ++i) {
+    sides.trellis[i] = static_cast<const uint8_t*>(w[i]->trellis);
+    sides.x[i] = static_cast<const uint16_t*>(fused ? x : a_had[i]);
+    sides.suh[i] = static_cast<const uint16_t*>(w[i]->suh);
+    sides.a_had[i] = fused ? static_cast<uint16_t*>(a_had[i]) : nullptr;
+    sides.partial[i] = scratch[i];
+  }
+  Dispatch(w0.codebook, w0.bits, [&](auto cb, auto bits) {
+    constexpr int kCb = decltype(cb)::value, kBits = decltype(bits)::value;
+    if (fused) {
+      LaunchProduct<kCb, kBits, true>(w0, sides, count, m, slices, s);
+    } else {
+      LaunchProduct<kCb, kBits, false>(w0, sides, count, m, slices, s);
+    }
+  });
+  if (const int bad = LaunchStatus(what); bad != 0) return bad;
+  const dim3 grid(static_cast<unsigned>(m), static_cast<unsigned>(w0.n / 128), static_cast<unsigned>(count));
+  const int64_t stride = static_cast<int64_t>(m) * w0.n;
+  const HadamardSides out{{scratch[0], scratch[1]},
+                          {y[0], y[1]},
+                          {nullptr, nullptr},
+                          {static_cast<const uint16_t*>(w[0]->svh), static_cast<const uint16_t*>(w[1]->svh)}};
+  if (f32) {
+    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, out, w0.n, slices, stride);
+  } else {
+    hipLaunchKernelGGL((HadamardKernel<1, 0>), grid, dim3(64), 0, s, out, w0.n, slices, stride);
+  }
+  // A failure here follows queued launches: a fault, not a refusal.
+  const int status = LaunchStatus(what);
+  return status > 0 ? -status : status;
+}
+
+}  // namespace
+}  // namespace llmp_hip
 
 extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
   if (op == nullptr || op->m <= 0 || op->weights.k <= 0 || op->weights.n <= 0) return 0;
@@ -491,37 +568,51 @@ extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, s
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
        reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
     return Refuse(1, "exl3.linear: operands not 8-byte aligned");
-  const llmp_exl3_weights& w = op->weights;
+  const llmp_exl3_weights* const w[2] = {&op->weights, &op->weights};
+  void* const a_had[2] = {op->a_had, op->a_had};
+  void* const y[2] = {op->y, op->y};
+  float* const partial[2] = {static_cast<float*>(scratch), static_cast<float*>(scratch)};
+  return LaunchLinears(w, 1, op->x, a_had, y, partial, op->f32 != 0, op->m, "exl3.linear", static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op) {
+  if (op == nullptr || op->m <= 0 || op->first.k <= 0 || op->first.n <= 0) return 0;
+  return 2 * static_cast<size_t>(SlicesFor(op->first.n, op->first.k)) * op->m * op->first.n * sizeof(float);
+}
+
+extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, size_t scratch_bytes,
+                                          void* stream) {
+  if (op == nullptr) return Refuse(1, "exl3.multi_linear: null operands");
+  if (const int bad = CheckWeights(op->first); bad != 0) return bad;
+  if (const int bad = CheckWeights(op->second); bad != 0) return bad;
+  if (op->first.k != op->second.k || op->first.n != op->second.n || op->first.bits != op->second.bits)
+    return Refuse(1, "exl3.multi_linear: the two linears of a multi-GEMM share k, n and K");
+  if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || scratch == nullptr)
+    return Refuse(1, "exl3.multi_linear: null operand");
+  if (op->m < 1 || op->m > 16) return Refuse(1, "exl3.multi_linear: the packed product takes 1 to 16 rows, not %d", op->m);
+  if (scratch_bytes < llmp_hip_exl3_multi_linear_scratch(op)) return Refuse(1, "exl3.multi_linear: scratch too small");
+  if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
+       reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
+    return Refuse(1, "exl3.multi_linear: operands not 8-byte aligned");
   const auto s = static_cast<hipStream_t>(stream);
-  const int slices = SlicesFor(w.n, w.k);
-  // The product of the transformed input in slices of K (for more than a few rows the input
-  // is transformed by a launch of its own first), then the slices' sum transformed.
-  const bool fused = op->m <= kFusedRows;
-  if (!fused) {
-    hipLaunchKernelGGL((HadamardKernel<0, 0>), dim3(static_cast<unsigned>(op->m), static_cast<unsigned>(w.k / 128)),
-                       dim3(64), 0, s, op->x, op->a_had, static_cast<const uint16_t*>(w.suh), nullptr, w.k, 1,
-                       int64_t{0});
-    if (const int bad = LaunchStatus("exl3.linear input transform"); bad != 0) return bad;
+  const int m = op->m, k = op->first.k, n = op->first.n;
+  const size_t out_bytes = static_cast<size_t>(m) * n * (op->f32 ? 4 : 2);
+  float* const part = static_cast<float*>(scratch);
+  const size_t part_floats = static_cast<size_t>(SlicesFor(n, k)) * m * n;
+  const llmp_exl3_weights* const w[2] = {&op->first, &op->second};
+  void* const a_had[2] = {op->a_had, static_cast<uint16_t*>(op->a_had) + static_cast<size_t>(m) * k};
+  void* const y[2] = {op->y, static_cast<uint8_t*>(op->y) + out_bytes};
+  float* const partial[2] = {part, part + part_floats};
+  if (op->first.codebook == op->second.codebook)
+    return LaunchLinears(w, 2, op->x, a_had, y, partial, op->f32 != 0, m, "exl3.multi_linear", s);
+  // Different codebooks decode differently: one linear after the other.
+  for (int i = 0; i < 2; ++i) {
+    const llmp_exl3_weights* const one[2] = {w[i], w[i]};
+    void* const a[2] = {a_had[i], a_had[i]};
+    void* const out[2] = {y[i], y[i]};
+    float* const p[2] = {partial[i], partial[i]};
+    const int status = LaunchLinears(one, 1, op->x, a, out, p, op->f32 != 0, m, "exl3.multi_linear", s);
+    if (status != 0) return i == 0 ? status : (status > 0 ? -status : status);
   }
-  Dispatch(w.codebook, w.bits, [&](auto cb, auto bits) {
-    constexpr int kCb = decltype(cb)::value, kBits = decltype(bits)::value;
-    if (fused) {
-      LaunchProduct<kCb, kBits, true>(w, op->x, op->a_had, static_cast<float*>(scratch), op->m, slices, s);
-    } else {
-      LaunchProduct<kCb, kBits, false>(w, op->a_had, nullptr, static_cast<float*>(scratch), op->m, slices, s);
-    }
-  });
-  if (const int bad = LaunchStatus("exl3.linear product"); bad != 0) return bad;
-  const dim3 grid(static_cast<unsigned>(op->m), static_cast<unsigned>(w.n / 128));
-  const int64_t stride = static_cast<int64_t>(op->m) * w.n;
-  if (op->f32) {
-    hipLaunchKernelGGL((HadamardKernel<1, 1>), grid, dim3(64), 0, s, scratch, op->y, nullptr,
-                       static_cast<const uint16_t*>(w.svh), w.n, slices, stride);
-  } else {
-    hipLaunchKernelGGL((HadamardKernel<1, 0>), grid, dim3(64), 0, s, scratch, op->y, nullptr,
-                       static_cast<const uint16_t*>(w.svh), w.n, slices, stride);
-  }
-  // A failure here follows queued launches: a fault, not a refusal.
-  const int status = LaunchStatus("exl3.linear");
-  return status > 0 ? -status : status;
+  return 0;
 }

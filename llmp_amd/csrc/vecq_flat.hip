@@ -904,7 +904,6 @@ struct FormatMxfp4 {
 #pragma unroll
       for (int t = 0; t < P; ++t) {
         if (t < m) {
-          if constexpr (P > 1) __builtin_amdgcn_sched_barrier(0);  // one token's images at a time
           const uint8_t* record = records + t * token_stride;
           const uint2* low2 = reinterpret_cast<const uint2*>(record) + from / 2;
           const uint2* high2 = reinterpret_cast<const uint2*>(record + kImage) + from / 2;
@@ -1095,7 +1094,9 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   // is multiplied.
   constexpr int kTileBytes = kWave * F::kUnitBytes;
   // The tile buffers take 16-byte chunks: they start at the next 16-byte boundary after the records.
-  uint8_t* ring = lds + ((P * token_stride + 15) & ~15) + wave * ((kDeep ? 2 : 1) * kTileBytes);
+  // (A dense product of fewer tokens than a pass takes stages only those: more room for waves.)
+  const int staged = a.offsets == nullptr && a.d.ids == nullptr && a.d.tokens < P ? a.d.tokens : P;
+  uint8_t* ring = lds + ((staged * token_stride + 15) & ~15) + wave * ((kDeep ? 2 : 1) * kTileBytes);
 
   // A lane's place in every tile: its matrix, row and unit of the row.
   const int half = rows_per_tile * nsb;
@@ -1477,11 +1478,13 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
     }
     return;
   }
-  if (pass > 1 && PlanFlat<F>(4, units, glu).lds > kFlatLdsLimit) pass = 1;
+  // The records a pass stages: four tokens', or a dense product's fewer.
+  const int staged = a.offsets == nullptr && d.ids == nullptr && d.tokens < 4 ? d.tokens : 4;
+  if (pass > 1 && PlanFlat<F>(staged, units, glu).lds > kFlatLdsLimit) pass = 1;
   // Two tile buffers a wave: one token a pass, packed rows, one workgroup a CU.
   deep = deep && F::kUnitBytes <= 144 && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
          PlanFlat<F>(1, units, glu, true).lds <= kDeepLdsLimit;
-  const FlatPlan plan = PlanFlat<F>(pass > 1 ? 4 : 1, units, glu, deep);
+  const FlatPlan plan = PlanFlat<F>(pass > 1 ? staged : 1, units, glu, deep);
   if (g_compute_units == 0) {
     const int cus = llmp_hip_compute_units();
     g_compute_units = cus > 0 ? cus : 256;

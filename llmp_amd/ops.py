@@ -9,7 +9,7 @@ import torch
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q4_K,  # noqa: F401
                    TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1,
-                   TYPE_Q8_0, X_BF16, X_F16, X_F32, Exl3Linear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
+                   TYPE_Q8_0, X_BF16, X_F16, X_F32, Exl3Linear, Exl3MultiLinear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
                    VecQSource)
 
 BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17}
@@ -334,6 +334,27 @@ def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, f32=True, keep=None)
     need = lib.llmp_hip_exl3_linear_scratch(C.byref(op))
     scratch = torch.empty(max(need, 8), dtype=torch.uint8, device=x.device)
     _lib.check(lib.llmp_hip_exl3_linear(C.byref(op), _ptr(scratch), need, _stream()))
+    if keep is not None:
+        keep["a_had"] = a_had
+    return y
+
+
+def exl3_multi_linear(first, second, x, f32=True, keep=None):
+    """exl3.multi_linear: x float16 [m, k] (m <= 16) through a gate and an up linear of the same k, n and
+    rate: [2, m, n]. `first` and `second` are (trellis, suh, svh, k, n, bits, codebook); `keep`, a dict,
+    receives the two transformed inputs a_had [2, m, k]."""
+    lib = _lib.load()
+    m = x.shape[0]
+    k, n = first[3], first[4]
+    op = Exl3MultiLinear()
+    op.first = _exl3_weights(*first)
+    op.second = _exl3_weights(*second)
+    a_had = torch.empty((2, m, k), dtype=torch.float16, device=x.device)
+    y = torch.empty((2, m, n), dtype=torch.float32 if f32 else torch.float16, device=x.device)
+    op.x, op.a_had, op.y, op.f32, op.m = x.data_ptr(), a_had.data_ptr(), y.data_ptr(), int(f32), m
+    need = lib.llmp_hip_exl3_multi_linear_scratch(C.byref(op))
+    scratch = torch.empty(max(need, 8), dtype=torch.uint8, device=x.device)
+    _lib.check(lib.llmp_hip_exl3_multi_linear(C.byref(op), _ptr(scratch), need, _stream()))
     if keep is not None:
         keep["a_had"] = a_had
     return y

@@ -95,3 +95,26 @@ def test_other_entry_points_refuse_bad_operands():
     assert lib.llmp_hip_moe_route(None, 8, 128, 8, 1, 0x1000, None) > 0
     assert lib.llmp_hip_vecq_sorted(8, C.byref(desc(ncols_x=480, stride_row=15)), 0x1000, 4, -1, None) > 0
     assert lib.llmp_hip_moe_route_ints(128, 8, 512) == 2 * 129 + 3 * 4096 + 8 * 128
+
+
+def test_exl3_linears_refuse_bad_operands():
+    lib = _lib.load()
+
+    def weights(k=128, n=128, bits=4, trellis=0x1000):
+        w = _lib.Exl3Weights()
+        w.trellis, w.suh, w.svh, w.k, w.n, w.bits, w.codebook = trellis, 0x2000, 0x3000, k, n, bits, 0
+        return w
+
+    one = _lib.Exl3Linear()
+    one.weights, one.x, one.a_had, one.y, one.f32, one.m = weights(), 0x4000, 0x5000, 0x6000, 1, 17
+    assert lib.llmp_hip_exl3_linear(C.byref(one), 0x7000, 1 << 30, None) > 0 and b"rows" in lib.llmp_hip_last_error()
+    two = _lib.Exl3MultiLinear()
+    two.first, two.second = weights(), weights(bits=3)
+    two.x, two.a_had, two.y, two.f32, two.m = 0x4000, 0x5000, 0x6000, 1, 2
+    assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 1 << 30, None) > 0
+    assert b"share" in lib.llmp_hip_last_error()
+    two.second = weights(n=256)
+    assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 1 << 30, None) > 0
+    two.second = weights()
+    assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 8, None) > 0 and b"scratch" in lib.llmp_hip_last_error()
+    assert lib.llmp_hip_exl3_multi_linear_scratch(C.byref(two)) == 2 * lib.llmp_hip_exl3_linear_scratch(C.byref(one)) // 17 * 2

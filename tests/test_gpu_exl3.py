@@ -122,3 +122,43 @@ def test_refusals(device):
     with pytest.raises(ops.KernelFailure):
         ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 4, 0, column=8,
                              columns=16)
+
+
+@pytest.mark.parametrize("m", [1, 3, 16])
+@pytest.mark.parametrize("codebooks", [(ops.EXL3_3INST, ops.EXL3_3INST), (ops.EXL3_MCG, ops.EXL3_MUL1)])
+@pytest.mark.parametrize("f32", [True, False])
+def test_multi_linear_is_the_two_linears(device, m, codebooks, f32):
+    """exl3.multi_linear (tests/unit/exl3_trellis_test.cc:664-716 of the reference): gate and up over one
+    input, the first linear's rows then the second's, each against its own reference. Here each half
+    is bit for bit the single linear's output (the same arithmetic in one launch), whose parity
+    with the oracle the tests above hold; one half is checked against the oracle directly as well."""
+    k, n, bits = 1024, 384, 4
+    gate, up = synth.exl3_weights(k, n, bits, 51), synth.exl3_weights(k, n, bits, 52)
+    x = synth.rng(53 + m).standard_normal((m, k)).astype(np.float16)
+    first = (dev(gate[0], device), halves(gate[1], device), halves(gate[2], device), k, n, bits, codebooks[0])
+    second = (dev(up[0], device), halves(up[1], device), halves(up[2], device), k, n, bits, codebooks[1])
+    keep = {}
+    got = ops.exl3_multi_linear(first, second, halves(x, device), f32=f32, keep=keep)
+    assert got.shape == (2, m, n)
+    word = torch.int32 if f32 else torch.int16
+    for i, side in enumerate((first, second)):
+        alone = {}
+        want = ops.exl3_linear(*side, halves(x, device), f32=f32, keep=alone)
+        assert torch.equal(got[i].view(word), want.view(word))
+        assert torch.equal(keep["a_had"][i].view(torch.int16), alone["a_had"].view(torch.int16))
+    if f32:
+        a_had = keep["a_had"][1].cpu().numpy().view(np.uint16)
+        want = oracle.exl3_product(up[0], up[2].view(np.uint16), k, n, bits, codebooks[1], a_had,
+                                   threads=oracle.max_threads())
+        ok, worst = rel_close(got[1].cpu().numpy(), want, 1e-3)
+        assert ok, worst
+
+
+def test_multi_linear_refusals(device):
+    a, b = synth.exl3_weights(128, 128, 4, 61), synth.exl3_weights(128, 128, 3, 62)
+    x = halves(np.zeros((2, 128), dtype=np.float16), device)
+    first = (dev(a[0], device), halves(a[1], device), halves(a[2], device), 128, 128, 4, 0)
+    second = (dev(b[0], device), halves(b[1], device), halves(b[2], device), 128, 128, 3, 0)
+    with pytest.raises(ops.KernelFailure) as e:  # the two linears share k, n and the rate
+        ops.exl3_multi_linear(first, second, x)
+    assert e.value.rejected
