@@ -139,6 +139,22 @@ def other_configs(device, args):
     del downs, wdn
     torch.cuda.empty_cache()
 
+    # An MXFP4 gate/up pair (4096 -> 2 x 14336, SwiGLU, one token): the same streaming form, 17-byte blocks.
+    km, nm = 4096, 14336
+    gate = dev(synth.mxfp4_weights(nm, km, 106))
+    count = -(-ROTATE_BYTES // (2 * gate.numel()))
+    gates = [gate] + [gate.clone() for _ in range(count - 1)]
+    ups = [gate.clone() for _ in range(count)]
+    q8 = ops.quantize_q8_1(dev(synth.activations(1, km, 107)))
+    y = torch.empty((1, 1, nm), dtype=torch.float32, device=device)
+    us = graph_us(lambda i: ops.vecq(ops.TYPE_MXFP4, ups[i % count], q8, km, nm, gate=gates[i % count],
+                                     glu=ops.GLU_SWIGLU, out=y), 4 * count)
+    bytes_ = 2 * gate.numel() + km * 4 + nm * 4
+    out["mxfp4_gate_up_swiglu_4096x2x14336_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
+                                                   "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    del gates, ups, gate
+    torch.cuda.empty_cache()
+
     # Config 3: MXFP8 GEMM 2048 x 12288 x 4096, bf16 out, and its activation quantizer.
     m, n, k = 2048, 12288, 4096
     g = torch.Generator().manual_seed(3)
@@ -194,6 +210,61 @@ def other_configs(device, args):
         out[f"exl3_linear_4096x14336_4bpw_m{m}"] = {"us": round(us, 1), "GB/s": round(bytes_ / us / 1e3, 1),
                                                     "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4),
                                                     "note": "input transform, product, output transform, replayed as a HIP graph"}
+    # The same shape's gate and up through exl3.multi_linear (both linears in the same launches).
+    xs = dev(synth.rng(209).standard_normal((1, k)).astype(np.float16).view(np.int16)).view(torch.float16)
+    half = len(trellises) // 2
+    side = lambda i: (trellises[i % len(trellises)], suh_d, svh_d, k, n, bits, ops.EXL3_3INST)
+    us = graph_us(lambda i: ops.exl3_multi_linear(side(i), side(i + half), xs), len(trellises))
+    bytes_ = 2 * (t0.numel() + 2 * k + 2 * n) + k * 2 + 2 * (k * 2 + n * 4)
+    out["exl3_multi_linear_4096x2x14336_4bpw_m1"] = {"us": round(us, 1), "GB/s": round(bytes_ / us / 1e3, 1),
+                                                     "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    return out
+
+
+def block_formats(device):
+    """One gate/up pair (4096 -> 2 x 14336, SwiGLU, one token over ready Q8_1 blocks) in each block type the
+    streaming mat-vec reads, and the KV cache store's two types: `python bench.py --formats`."""
+    import numpy as np
+    import torch
+
+    from llmp_amd import ops, synth
+
+    out = {}
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    k, n = 4096, 14336
+    q8 = ops.quantize_q8_1(dev(synth.activations(1, k, 301)))
+    y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
+    names = {ops.TYPE_Q4_0: "q4_0", ops.TYPE_Q4_1: "q4_1", ops.TYPE_Q5_0: "q5_0", ops.TYPE_Q5_1: "q5_1",
+             ops.TYPE_Q8_0: "q8_0", ops.TYPE_Q4_K: "q4_k", ops.TYPE_MXFP4: "mxfp4"}
+    for t, name in names.items():
+        if t == ops.TYPE_Q4_K:
+            make = lambda seed: synth.q4_k_weights(n, k, seed)
+        elif t == ops.TYPE_Q8_0:
+            make = lambda seed: synth.q8_0_weights(n, k, seed)
+        elif t == ops.TYPE_MXFP4:
+            make = lambda seed: synth.mxfp4_weights(n, k, seed)
+        else:
+            make = lambda seed, t=t: synth.legacy_weights(t, n, k, seed)
+        gate, up = dev(make(302)), dev(make(303))
+        count = -(-ROTATE_BYTES // (2 * gate.numel()))
+        gates = [gate] + [gate.clone() for _ in range(count - 1)]
+        ups = [up] + [up.clone() for _ in range(count - 1)]
+        us = graph_us(lambda i: ops.vecq(t, ups[i % count], q8, k, n, gate=gates[i % count], glu=ops.GLU_SWIGLU, out=y),
+                      4 * count)
+        bytes_ = 2 * gate.numel() + q8.numel() + n * 4
+        out[f"{name}_gate_up_swiglu_4096x2x14336_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
+                                                         "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        del gates, ups, gate, up
+        torch.cuda.empty_cache()
+    # llmp.set_rows.quant: 512 rows of 8192 floats (a layer's K or V rows of a 512-token chunk) into a cache.
+    rows, width, cells = 512, 8192, 4096
+    x = dev(synth.activations(rows, width, 304))
+    ids = dev(synth.rng(305).permutation(cells)[:rows].astype(np.int64))
+    for t, name, size in ((ops.TYPE_Q8_0, "q8_0", 34), (ops.TYPE_Q4_0, "q4_0", 18)):
+        cache = torch.zeros((cells, width // 32 * size), dtype=torch.uint8, device=device)
+        us = graph_us(lambda i: ops.set_rows_quant(t, x, ids, cache), 40)
+        bytes_ = rows * width * 4 + rows * (width // 32 * size)
+        out[f"set_rows_quant_{name}_512x8192"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1)}
     return out
 
 
@@ -219,6 +290,9 @@ def main():
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations' short measurements")
+    ap.add_argument("--formats", action="store_true",
+                    help="instead of the benchmark line: one JSON line with every block type's gate/up mat-vec and "
+                         "the KV cache store")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of the weights' size (for scaling hardware counters)")
     ap.add_argument("--fused", action="store_true",
@@ -235,6 +309,10 @@ def main():
     from llmp_amd import ops, synth
 
     device = torch.device("cuda:0")
+    if args.formats:
+        print(json.dumps({"block_formats": block_formats(device), "data": "synthetic", "launch": "hip graph",
+                          "weight_copies_rotated_bytes": ROTATE_BYTES}))
+        return
     gate = synth.q4_k_weights(N, K, 101)
     up = synth.q4_k_weights(N, K, 102)
     x = synth.bf16_to_f32(synth.bf16_bits(synth.activations(args.tokens, K, 103)))
