@@ -223,7 +223,8 @@ def other_configs(device, args):
 
 def block_formats(device):
     """One gate/up pair (4096 -> 2 x 14336, SwiGLU, one token over ready Q8_1 blocks) in each block type the
-    streaming mat-vec reads, and the KV cache store's two types: `python bench.py --formats`."""
+    streaming mat-vec reads, llmp.decode.vector over five stored encodings, and the KV cache store's two types:
+    `python bench.py --formats`."""
     import numpy as np
     import torch
 
@@ -255,6 +256,21 @@ def block_formats(device):
         out[f"{name}_gate_up_swiglu_4096x2x14336_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
                                                          "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
         del gates, ups, gate, up
+        torch.cuda.empty_cache()
+    # llmp.decode.vector: one F32 input row times a 14336 x 4096 weight in its stored encoding.
+    x = dev(synth.activations(1, k, 306))
+    yd = torch.empty((1, n), dtype=torch.float32, device=device)
+    for decoder in (0, 3, 6, 7, 9):
+        w = synth.decode_weight(decoder, n, k, 307)
+        base = {key: (dev(v) if isinstance(v, np.ndarray) else v) for key, v in w.items() if key != "plain"}
+        bytes_w = base["data"].numel() + (base["scales"].numel() if base.get("scales") is not None else 0)
+        count = max(2, -(-ROTATE_BYTES // bytes_w))
+        ws = [base] + [{**base, "data": base["data"].clone()} for _ in range(count - 1)]
+        us = graph_us(lambda i: ops.decode_vector(decoder, ws[i % count], x, out=yd), 2 * count)
+        bytes_ = bytes_w + k * 4 + n * 4
+        out[f"decode_vector_{ops.DECODERS[decoder].replace('.', '_')}_4096x14336_rows1"] = {
+            "us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1), "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        del ws, base
         torch.cuda.empty_cache()
     # llmp.set_rows.quant: 512 rows of 8192 floats (a layer's K or V rows of a 512-token chunk) into a cache.
     rows, width, cells = 512, 8192, 4096

@@ -273,6 +273,48 @@ typedef struct llmp_exl3_multi_linear {
 size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op);
 int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, size_t scratch_bytes, void* stream);
 
+/* ---------------------------------------------------------------- llmp.decode.vector
+ * RunVector of src/kernels/decode/products.h:96-109: y[t][j] = sum_k W[first + j][k] x[t][k]
+ * (times the weight's tensor scale of row first + j) for t < rows (1 to 16) and j < outputs,
+ * over a weight in its stored encoding; row t of x (F32, 16-byte aligned, x_stride a multiple
+ * of 4 floats) at x + t * x_stride, of y at y + t * y_stride. The decoders are the reference's
+ * (src/kernels/decode/operand.h:26-41, decoders.cuh), the operand its Operand
+ * (operand.h:74-97) field for field; values decode as src/kernels/reference/decode.cc has
+ * them (an undefined block scale, UE4M3 from 0x7F or E8M0 0xFF, is NaN). The affine decoder is
+ * not built (refused). Rows up to 16384 values; four input rows a launch (fewer of long rows),
+ * so 1 to 16 launches are queued and a failure after the first is a fault (negative). */
+enum {
+  LLMP_DECODER_BF16_DENSE = 0,
+  LLMP_DECODER_F16_DENSE = 1,
+  LLMP_DECODER_Q8_0_BLOCKS = 2,       /* GGML's block_q8_0 */
+  LLMP_DECODER_NVFP4_SPLIT = 3,       /* codes k / 2 bytes a row, UE4M3 scales k / 16 a row */
+  LLMP_DECODER_NVFP4_ATOMS = 4,       /* codes as split, scales in CUTLASS's SM1xx atoms */
+  LLMP_DECODER_NVFP4_INTERLEAVED = 5, /* each row's codes, then its scales */
+  LLMP_DECODER_NVFP4_GGML_BLOCKS = 6, /* GGML's block_nvfp4: four scales, then 32 bytes */
+  LLMP_DECODER_MXFP8_SPLIT = 7,       /* E4M3 codes k bytes a row, E8M0 scales k / 32 a row */
+  LLMP_DECODER_MXFP8_ATOMS = 8,
+  LLMP_DECODER_MXFP4_SPLIT = 9,       /* E2M1 codes k / 2 bytes, E8M0 scales k / 32 */
+  LLMP_DECODER_MXFP4_ATOMS = 10,
+  LLMP_DECODER_AFFINE_SPLIT = 11
+};
+typedef struct llmp_decode_operand {
+  const uint8_t* data;       /* kData, or kCodes for the split arrangements */
+  const uint8_t* scales;     /* kBlockScales for the split arrangements */
+  const float* tensor_scale; /* or null: row r takes tensor_scale[r / rows_per_scale] */
+  const uint8_t* biases;     /* affine only */
+  uint32_t k;                /* values a row */
+  uint32_t rows;             /* rows of the matrix */
+  uint32_t rows_per_scale;
+  uint32_t pad;
+  uint64_t row_bytes;        /* bytes of a row of `data` */
+  uint32_t scale_row_bytes;  /* affine only */
+  uint16_t group;            /* affine only */
+  uint8_t bits;              /* affine only */
+  uint8_t scale_type;        /* affine only */
+} llmp_decode_operand;
+int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* weight, uint64_t first, uint64_t outputs,
+                           const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

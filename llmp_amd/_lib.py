@@ -58,6 +58,14 @@ class Exl3MultiLinear(C.Structure):
                 ("y", C.c_void_p), ("f32", C.c_int), ("m", C.c_int)]
 
 
+class DecodeOperand(C.Structure):
+    """llmp_decode_operand: Operand of src/kernels/decode/operand.h:74-97 of the reference."""
+    _fields_ = [("data", C.c_void_p), ("scales", C.c_void_p), ("tensor_scale", C.c_void_p), ("biases", C.c_void_p),
+                ("k", C.c_uint32), ("rows", C.c_uint32), ("rows_per_scale", C.c_uint32), ("pad", C.c_uint32),
+                ("row_bytes", C.c_uint64), ("scale_row_bytes", C.c_uint32), ("group", C.c_uint16),
+                ("bits", C.c_uint8), ("scale_type", C.c_uint8)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -92,6 +100,8 @@ SYMBOLS = {
     "llmp_hip_exl3_hadamard": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),
     "llmp_hip_exl3_linear": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _vp]),
+    "llmp_hip_decode_vector": (_int, [_int, C.POINTER(DecodeOperand), C.c_uint64, C.c_uint64, _vp, C.c_uint64,
+                                      C.c_uint64, _vp, C.c_uint64, _vp]),
     "llmp_hip_exl3_multi_linear_scratch": (C.c_size_t, [C.POINTER(Exl3MultiLinear)]),
     "llmp_hip_exl3_multi_linear": (_int, [C.POINTER(Exl3MultiLinear), _vp, C.c_size_t, _vp]),
 }

@@ -1,0 +1,335 @@
+// llmp.decode.vector for gfx950: products over weights in their stored encodings, a block
+// decoder per encoding and layout under one kernel template (src/kernels/decode/products.h:96-109,
+// decoders.cuh and operand.h of the reference). y[t][j] = tensor_scale(first + j) * sum_k
+// W[first + j][k] x[t][k] for 1 to 16 F32 input rows; every decoder decodes a value as the
+// reference's CPU decoder does (src/kernels/reference/decode.cc), the products are F32.
+//
+// A wave takes two output rows at a time, its lanes the rows' 16-value segments; the pass's
+// input rows are staged in LDS once a workgroup (a segment's 64 bytes every 80, so that the
+// lanes' 16-byte reads fall in different banks) and each staged segment multiplies both rows.
+// E2M1 codes are converted by v_cvt_scalef32_pk_f32_fp4 (two values an instruction), E4M3
+// codes by v_cvt_pk_f32_fp8; a segment's block scale multiplies its sum once. An input row's
+// outputs do not depend on the rows beside it: each row's sums are formed alone, in one order.
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+
+namespace llmp_hip {
+namespace {
+
+typedef float Float2 __attribute__((ext_vector_type(2)));
+typedef uint32_t U32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kDecodeWaves = 8;  // a workgroup's waves with several input rows staged; four with one
+constexpr int kRowsAWave = 2;
+constexpr int kSegmentStride = 80;           // bytes from a staged segment to the next
+constexpr size_t kDecodeLdsLimit = 80 * 1024;  // two workgroups a CU
+
+struct DecodeArgs {
+  llmp_decode_operand w;
+  uint32_t first;
+  uint32_t outputs;
+  uint32_t token0;  // the pass's first input row
+  const float* x;
+  uint64_t x_stride;
+  float* y;
+  uint64_t y_stride;
+};
+
+// operand.h:62-67: row `row`'s scale of block `block` in CUTLASS's scale atoms.
+__device__ __forceinline__ uint64_t AtomAt(uint64_t row, uint64_t block, uint64_t blocks) {
+  return (((row / 128) * (blocks / 4)) + (block / 4)) * 512 + ((row % 32) * 16) + (((row % 128) / 32) * 4) + (block % 4);
+}
+
+// decode.cc:407-411: E4M3's value up to 0x7E, NaN from 0x7F.
+__device__ __forceinline__ float Ue4m3ToFloat(uint32_t bits) {
+  return bits < 0x7Fu ? E4m3ToFloat(bits) : __builtin_nanf("");
+}
+
+// Eight E2M1 codes, value 2 i in byte i's low nibble (decoders.cuh:57-72), into v[0..7].
+__device__ __forceinline__ void Fp4Adjacent(uint32_t word, float* v) {
+  const Float2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+  const Float2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+  const Float2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2);
+  const Float2 d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+  v[0] = a[0], v[1] = a[1], v[2] = b[0], v[3] = b[1], v[4] = c[0], v[5] = c[1], v[6] = d[0], v[7] = d[1];
+}
+// Four bytes of GGML's block_nvfp4: byte j holds values j (low nibble) and j + 8.
+__device__ __forceinline__ void Fp4Halves(uint32_t word, float* low, float* high) {
+  const Float2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+  const Float2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+  const Float2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2);
+  const Float2 d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+  low[0] = a[0], low[1] = b[0], low[2] = c[0], low[3] = d[0];
+  high[0] = a[1], high[1] = b[1], high[2] = c[1], high[3] = d[1];
+}
+__device__ __forceinline__ void Fp8Four(uint32_t word, float* v) {
+  const Float2 a = __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
+  const Float2 b = __builtin_amdgcn_cvt_pk_f32_fp8(word, true);
+  v[0] = a[0], v[1] = a[1], v[2] = b[0], v[3] = b[1];
+}
+
+// Segment `seg` (16 values) of row `row`: the values before the block scale, and that scale.
+template <int D>
+__device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32_t row, uint32_t seg, float (&v)[16],
+                                            float& s) {
+  const uint8_t* data = w.data + static_cast<uint64_t>(row) * w.row_bytes;
+  if constexpr (D == LLMP_DECODER_BF16_DENSE || D == LLMP_DECODER_F16_DENSE) {
+    const U32x4* src = reinterpret_cast<const U32x4*>(data + seg * 32u);
+    const U32x4 a = __builtin_nontemporal_load(src), b = __builtin_nontemporal_load(src + 1);
+    const uint32_t word[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if constexpr (D == LLMP_DECODER_BF16_DENSE) {
+        v[2 * i] = __builtin_bit_cast(float, word[i] << 16);
+        v[2 * i + 1] = __builtin_bit_cast(float, word[i] & 0xFFFF0000u);
+      } else {
+        v[2 * i] = HalfBitsToFloat(word[i] & 0xFFFFu);
+        v[2 * i + 1] = HalfBitsToFloat(word[i] >> 16);
+      }
+    }
+    s = 1.0f;
+  } else if constexpr (D == LLMP_DECODER_Q8_0_BLOCKS) {
+    // block_q8_0 is 34 bytes: only two-byte loads are aligned. A segment is half a block.
+    const uint8_t* block = data + static_cast<uint64_t>(seg / 2u) * 34u;
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(block + 2 + (seg & 1u) * 16u);
+    s = HalfBitsToFloat(*reinterpret_cast<const uint16_t*>(block));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t pair = q[i];
+      v[2 * i] = static_cast<float>(static_cast<int8_t>(pair & 0xFFu));
+      v[2 * i + 1] = static_cast<float>(static_cast<int8_t>(pair >> 8));
+    }
+  } else if constexpr (D == LLMP_DECODER_NVFP4_INTERLEAVED) {
+    // A row is its K / 2 code bytes, then its K / 16 scales: no alignment beyond a byte.
+    const uint8_t* c = data + seg * 8u;
+    const uint32_t lo = c[0] | (c[1] << 8) | (c[2] << 16) | (static_cast<uint32_t>(c[3]) << 24);
+    const uint32_t hi = c[4] | (c[5] << 8) | (c[6] << 16) | (static_cast<uint32_t>(c[7]) << 24);
+    Fp4Adjacent(lo, v);
+    Fp4Adjacent(hi, v + 8);
+    s = Ue4m3ToFloat(data[w.k / 2u + seg]);
+  } else if constexpr (D == LLMP_DECODER_NVFP4_GGML_BLOCKS) {
+    // block_nvfp4: four UE4M3 scales, then 32 bytes; a segment is a 16-value sub-block.
+    const uint8_t* block = data + static_cast<uint64_t>(seg / 4u) * 36u;
+    const uint32_t sub = seg & 3u;
+    const uint32_t* c = reinterpret_cast<const uint32_t*>(block + 4 + sub * 8u);
+    const uint32_t scales = *reinterpret_cast<const uint32_t*>(block);
+    Fp4Halves(c[0], v, v + 8);
+    Fp4Halves(c[1], v + 4, v + 12);
+    s = Ue4m3ToFloat((scales >> (8u * sub)) & 0xFFu);
+  } else if constexpr (D == LLMP_DECODER_MXFP8_SPLIT || D == LLMP_DECODER_MXFP8_ATOMS) {
+    const U32x4 c = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
+    Fp8Four(c.x, v), Fp8Four(c.y, v + 4), Fp8Four(c.z, v + 8), Fp8Four(c.w, v + 12);
+    const uint64_t at = D == LLMP_DECODER_MXFP8_SPLIT ? static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u
+                                                      : AtomAt(row, seg / 2u, w.k / 32u);
+    s = E8m0ToFloat(w.scales[at]);
+  } else {
+    // NVFP4 and MXFP4 codes as rows of K / 2 bytes: a segment is eight bytes.
+    const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
+    Fp4Adjacent(c.x, v);
+    Fp4Adjacent(c.y, v + 8);
+    if constexpr (D == LLMP_DECODER_NVFP4_SPLIT) {
+      s = Ue4m3ToFloat(w.scales[static_cast<uint64_t>(row) * (w.k / 16u) + seg]);
+    } else if constexpr (D == LLMP_DECODER_NVFP4_ATOMS) {
+      s = Ue4m3ToFloat(w.scales[AtomAt(row, seg, w.k / 16u)]);
+    } else if constexpr (D == LLMP_DECODER_MXFP4_SPLIT) {
+      s = E8m0ToFloat(w.scales[static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u]);
+    } else {
+      s = E8m0ToFloat(w.scales[AtomAt(row, seg / 2u, w.k / 32u)]);
+    }
+  }
+}
+
+// grid: workgroups of eight waves, persistent over pairs of output rows; LDS: T input rows.
+template <int D, int T>
+__global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const DecodeArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t segs = a.w.k / 16u;
+  const uint32_t quarters = a.w.k / 4u;  // 16-byte pieces of an input row
+
+  const uint32_t waves = blockDim.x / 64;
+  for (uint32_t c = tid; c < T * quarters; c += blockDim.x) {
+    const uint32_t t = c / quarters, q = c - t * quarters;
+    const float4 piece = *reinterpret_cast<const float4*>(a.x + (a.token0 + t) * a.x_stride + q * 4u);
+    *reinterpret_cast<float4*>(lds + static_cast<size_t>(t * segs + q / 4u) * kSegmentStride + (q & 3u) * 16u) = piece;
+  }
+  __syncthreads();  // the only one: from here the waves run alone
+
+  const uint32_t pairs = (a.outputs + kRowsAWave - 1) / kRowsAWave;
+  for (uint32_t pair = blockIdx.x * waves + wave; pair < pairs; pair += gridDim.x * waves) {
+    const uint32_t out0 = pair * kRowsAWave;
+    float acc[kRowsAWave][T];
+#pragma unroll
+    for (int r = 0; r < kRowsAWave; ++r) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[r][t] = 0.0f;
+    }
+    for (uint32_t seg = lane; seg < segs; seg += 64) {
+      float v[kRowsAWave][16], s[kRowsAWave];
+#pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+        // A lone last row is decoded twice: its second copy's sums are not stored.
+        const uint32_t out = min(out0 + r, a.outputs - 1);
+        LoadSegment<D>(a.w, a.first + out, seg, v[r], s[r]);
+      }
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const float4* xs = reinterpret_cast<const float4*>(lds + static_cast<size_t>(t * segs + seg) * kSegmentStride);
+        const float4 x0 = xs[0], x1 = xs[1], x2 = xs[2], x3 = xs[3];
+        const float x[16] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+        for (int r = 0; r < kRowsAWave; ++r) {
+          float dot = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) dot = fmaf(v[r][i], x[i], dot);
+          acc[r][t] = fmaf(dot, s[r], acc[r][t]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kRowsAWave; ++r) {
+      const uint32_t out = out0 + r;
+      float scale = 1.0f;
+      if (a.w.tensor_scale != nullptr && out < a.outputs) scale = a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale];
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        float total = acc[r][t];
+#pragma unroll
+        for (int mask = 32; mask >= 1; mask >>= 1) total += ShflXor(total, mask);
+        if (lane == 0 && out < a.outputs) a.y[(a.token0 + t) * a.y_stride + out] = total * scale;
+      }
+    }
+  }
+}
+
+size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
+
+template <int D, int T>
+void LaunchDecode(const DecodeArgs& a, int groups, int waves, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDecodeLdsLimit));
+    sized = true;
+  }
+  hipLaunchKernelGGL((DecodeVectorKernel<D, T>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
+                     DecodeLds(T, a.w.k), stream, a);
+}
+
+template <int D>
+void LaunchDecoder(const DecodeArgs& a, int tokens, int groups, int waves, hipStream_t stream) {
+  switch (tokens) {
+    case 1: LaunchDecode<D, 1>(a, groups, waves, stream); break;
+    case 2: LaunchDecode<D, 2>(a, groups, waves, stream); break;
+    case 3: LaunchDecode<D, 3>(a, groups, waves, stream); break;
+    default: LaunchDecode<D, 4>(a, groups, waves, stream); break;
+  }
+}
+
+// The multiple of K a decoder's rows must be (DecoderKMultiple, products.h:88-90): its blocks,
+// scale atoms and 16-value segments.
+uint32_t KMultiple(int decoder) {
+  switch (decoder) {
+    case LLMP_DECODER_Q8_0_BLOCKS: case LLMP_DECODER_MXFP8_SPLIT: case LLMP_DECODER_MXFP4_SPLIT: return 32;
+    case LLMP_DECODER_NVFP4_ATOMS: case LLMP_DECODER_NVFP4_GGML_BLOCKS: return 64;
+    case LLMP_DECODER_MXFP8_ATOMS: case LLMP_DECODER_MXFP4_ATOMS: return 128;
+    default: return 16;
+  }
+}
+// The alignment a decoder's loads of `data` need (products.h:38-43).
+uint32_t DataAlignment(int decoder) {
+  switch (decoder) {
+    case LLMP_DECODER_BF16_DENSE: case LLMP_DECODER_F16_DENSE: case LLMP_DECODER_MXFP8_SPLIT:
+    case LLMP_DECODER_MXFP8_ATOMS: return 16;
+    case LLMP_DECODER_NVFP4_SPLIT: case LLMP_DECODER_NVFP4_ATOMS: case LLMP_DECODER_MXFP4_SPLIT:
+    case LLMP_DECODER_MXFP4_ATOMS: return 8;
+    case LLMP_DECODER_NVFP4_GGML_BLOCKS: return 4;
+    case LLMP_DECODER_Q8_0_BLOCKS: return 2;
+    default: return 1;
+  }
+}
+bool SplitScales(int decoder) {
+  return decoder == LLMP_DECODER_NVFP4_SPLIT || decoder == LLMP_DECODER_NVFP4_ATOMS || decoder == LLMP_DECODER_MXFP8_SPLIT ||
+         decoder == LLMP_DECODER_MXFP8_ATOMS || decoder == LLMP_DECODER_MXFP4_SPLIT || decoder == LLMP_DECODER_MXFP4_ATOMS;
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
+                                      const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
+                                      void* stream) {
+  if (w == nullptr) return Refuse(1, "decode.vector: null operand");
+  if (decoder < 0 || decoder >= LLMP_DECODER_AFFINE_SPLIT)
+    return Refuse(1, "decode.vector: decoder %d has no kernel", decoder);
+  if (w->data == nullptr || x == nullptr || y == nullptr) return Refuse(1, "decode.vector: null operand");
+  if (SplitScales(decoder) && w->scales == nullptr) return Refuse(1, "decode.vector: the layout's block scales are missing");
+  if (w->k == 0 || w->k % KMultiple(decoder) != 0)
+    return Refuse(1, "decode.vector: k %u is not a multiple of the decoder's %u", w->k, KMultiple(decoder));
+  if (rows == 0 || rows > 16 || outputs == 0 || first > w->rows || outputs > w->rows - first)
+    return Refuse(1, "decode.vector: rows %llu (1 to 16), outputs [%llu, %llu) of %u",
+                  static_cast<unsigned long long>(rows), static_cast<unsigned long long>(first),
+                  static_cast<unsigned long long>(first + outputs), w->rows);
+  if (w->tensor_scale != nullptr && w->rows_per_scale == 0) return Refuse(1, "decode.vector: tensor scales of no rows");
+  if (reinterpret_cast<uintptr_t>(w->data) % DataAlignment(decoder) != 0 || w->row_bytes % DataAlignment(decoder) != 0)
+    return Refuse(1, "decode.vector: the weight's rows are not aligned for its decoder's loads (%u bytes)",
+                  DataAlignment(decoder));
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_stride % 4 != 0 || x_stride < w->k || y_stride < outputs ||
+      reinterpret_cast<uintptr_t>(y) % 4 != 0)
+    return Refuse(1, "decode.vector: input rows are 16-byte aligned, a multiple of 4 floats apart and at least k long");
+  // The rows a pass stages must fit LDS: four, or fewer of a long row.
+  int pass = rows < 4 ? static_cast<int>(rows) : 4;
+  while (pass > 1 && DecodeLds(pass, w->k) > kDecodeLdsLimit) --pass;
+  if (DecodeLds(pass, w->k) > kDecodeLdsLimit)
+    return Refuse(1, "decode.vector: a row of %u values does not fit the staging area (16384 at most)", w->k);
+  const int cus = llmp_hip_compute_units();
+  const size_t lds = DecodeLds(pass, w->k);
+  // One input row: four waves a workgroup and more workgroups; several: eight waves share the staged rows.
+  const int waves = pass == 1 ? 4 : kDecodeWaves;
+  int resident = static_cast<int>(160 * 1024 / (lds + 1024));
+  if (resident > 32 / waves) resident = 32 / waves;  // a CU holds 32 waves
+  if (resident < 1) resident = 1;
+  const uint64_t pairs = (outputs + kRowsAWave - 1) / kRowsAWave;
+  uint64_t groups = (pairs + waves - 1) / waves;
+  const uint64_t most = static_cast<uint64_t>(cus > 0 ? cus : 256) * resident;
+  if (groups > most) groups = most;
+  DecodeArgs a;
+  a.w = *w;
+  a.first = static_cast<uint32_t>(first);
+  a.outputs = static_cast<uint32_t>(outputs);
+  a.x = x;
+  a.x_stride = x_stride;
+  a.y = y;
+  a.y_stride = y_stride;
+  const auto s = static_cast<hipStream_t>(stream);
+  for (uint64_t token0 = 0; token0 < rows; token0 += pass) {
+    const int tokens = static_cast<int>(rows - token0 < static_cast<uint64_t>(pass) ? rows - token0 : pass);
+    a.token0 = static_cast<uint32_t>(token0);
+    switch (decoder) {
+#define LLMP_DECODER(ID) \
+  case ID: LaunchDecoder<ID>(a, tokens, static_cast<int>(groups), waves, s); break;
+      LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
+      LLMP_DECODER(LLMP_DECODER_F16_DENSE)
+      LLMP_DECODER(LLMP_DECODER_Q8_0_BLOCKS)
+      LLMP_DECODER(LLMP_DECODER_NVFP4_SPLIT)
+      LLMP_DECODER(LLMP_DECODER_NVFP4_ATOMS)
+      LLMP_DECODER(LLMP_DECODER_NVFP4_INTERLEAVED)
+      LLMP_DECODER(LLMP_DECODER_NVFP4_GGML_BLOCKS)
+      LLMP_DECODER(LLMP_DECODER_MXFP8_SPLIT)
+      LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
+      LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
+      LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+#undef LLMP_DECODER
+    }
+    const int status = LaunchStatus("decode.vector");
+    if (status != 0) return token0 == 0 ? status : (status > 0 ? -status : status);
+  }
+  return 0;
+}

@@ -9,7 +9,7 @@ import torch
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q4_K,  # noqa: F401
                    TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1,
-                   TYPE_Q8_0, X_BF16, X_F16, X_F32, Exl3Linear, Exl3MultiLinear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
+                   TYPE_Q8_0, X_BF16, X_F16, X_F32, DecodeOperand, Exl3Linear, Exl3MultiLinear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
                    VecQSource)
 
 BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17}
@@ -357,4 +357,28 @@ def exl3_multi_linear(first, second, x, f32=True, keep=None):
     _lib.check(lib.llmp_hip_exl3_multi_linear(C.byref(op), _ptr(scratch), need, _stream()))
     if keep is not None:
         keep["a_had"] = a_had
+    return y
+
+
+DECODERS = ("bf16.dense", "f16.dense", "q8_0.blocks", "nvfp4.split", "nvfp4.atoms", "nvfp4.interleaved",
+            "nvfp4.ggml_blocks", "mxfp8.split", "mxfp8.atoms", "mxfp4.split", "mxfp4.atoms", "affine.split")
+
+
+def decode_vector(decoder, weight, x, first=0, outputs=None, out=None):
+    """llmp.decode.vector: float32 x [rows <= 16, k] times a weight in its stored encoding. `weight` is a
+    dict of device tensors: data (uint8 [n, row_bytes]), k, and where the decoder has them scales (uint8)
+    and tensor_scale (float32) with rows_per_scale. Returns float32 [rows, outputs]."""
+    lib = _lib.load()
+    data = weight["data"]
+    op = DecodeOperand()
+    op.data = data.data_ptr()
+    op.scales = weight["scales"].data_ptr() if weight.get("scales") is not None else None
+    op.tensor_scale = weight["tensor_scale"].data_ptr() if weight.get("tensor_scale") is not None else None
+    op.k, op.rows, op.row_bytes = weight["k"], data.shape[0], data.stride(0)
+    op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
+    outputs = data.shape[0] - first if outputs is None else outputs
+    rows = x.shape[0]
+    y = torch.empty((rows, outputs), dtype=torch.float32, device=x.device) if out is None else out
+    _lib.check(lib.llmp_hip_decode_vector(decoder, C.byref(op), first, outputs, _ptr(x), rows, x.stride(0), _ptr(y),
+                                          y.stride(0), _stream()))
     return y

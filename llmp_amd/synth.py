@@ -105,3 +105,57 @@ def exl3_weights(k, n, bits, seed):
     suh = g.choice(np.array([-1.0, 1.0]), size=k).astype(np.float16)
     svh = (g.choice(np.array([-1.0, 1.0]), size=n) * np.abs(g.normal(1.0, 0.1, size=n))).astype(np.float16)
     return trellis, suh, svh
+
+
+def decode_weight(decoder, n, k, seed, tensor_scales=0):
+    """A weight of n rows of k values as decoder `decoder` (its index in the reference's DecoderId,
+    src/kernels/decode/operand.h:26-41) reads it: a dict of data (uint8 [n, row_bytes]), k, and where the
+    layout has them scales (uint8, flat) and, with `tensor_scales` > 0, that many F32 tensor scales. Codes are
+    uniform bytes; block scales are kept in a range whose products stay finite."""
+    g = rng(seed)
+    w = {"k": k}
+
+    def atoms(scales, blocks):  # [n, blocks] -> CUTLASS's scale atoms (src/format/layout.h)
+        rows = (n + 127) // 128 * 128
+        out = np.zeros(rows * blocks, dtype=np.uint8)
+        r, b = np.meshgrid(np.arange(n), np.arange(blocks), indexing="ij")
+        at = ((r // 128) * (blocks // 4) + b // 4) * 512 + (r % 32) * 16 + ((r % 128) // 32) * 4 + b % 4
+        out[at.reshape(-1)] = scales.reshape(-1)
+        return out
+
+    if decoder == 0:  # bf16
+        w["data"] = bf16_bits(g.standard_normal((n, k), dtype=np.float32) * 0.05).view(np.uint8).reshape(n, 2 * k)
+    elif decoder == 1:  # f16
+        w["data"] = (g.standard_normal((n, k), dtype=np.float32) * 0.05).astype(np.float16).view(np.uint8).reshape(n, 2 * k)
+    elif decoder == 2:  # q8_0 blocks
+        w["data"] = q8_0_weights(n, k, seed)
+    elif decoder in (3, 4, 5, 6):  # nvfp4: UE4M3 scales of 16 values, 0x20 .. 0x47 (2^-3 .. 30)
+        codes = g.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+        scales = g.integers(0x20, 0x48, size=(n, k // 16), dtype=np.uint8)
+        if decoder == 3:
+            w["data"], w["scales"] = codes, scales.reshape(-1)
+        elif decoder == 4:
+            w["data"], w["scales"] = codes, atoms(scales, k // 16)
+        elif decoder == 5:
+            w["data"] = np.concatenate([codes, scales], axis=1)
+        else:  # GGML's blocks: value j of a 16-value sub-block in byte j % 8, low nibble below 8
+            v = np.stack([codes & 15, codes >> 4], axis=-1).reshape(n, k // 64, 4, 16)  # codes in value order
+            packed = (v[..., :8] | (v[..., 8:] << 4)).astype(np.uint8).reshape(n, k // 64, 32)
+            w["data"] = np.concatenate([scales.reshape(n, k // 64, 4), packed], axis=-1).reshape(n, k // 64 * 36)
+            w["plain"] = (codes, scales)  # the same values as nvfp4.split holds them
+    elif decoder in (7, 8):  # mxfp8: E8M0 scales of 32 values
+        codes = g.integers(0, 256, size=(n, k), dtype=np.uint8)
+        codes[(codes & 0x7F) == 0x7F] = 0x38  # no NaN codes
+        scales = g.integers(118, 126, size=(n, k // 32), dtype=np.uint8)
+        w["data"], w["scales"] = codes, scales.reshape(-1) if decoder == 7 else atoms(scales, k // 32)
+    elif decoder in (9, 10):  # mxfp4
+        codes = g.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+        scales = g.integers(118, 126, size=(n, k // 32), dtype=np.uint8)
+        w["data"], w["scales"] = codes, scales.reshape(-1) if decoder == 9 else atoms(scales, k // 32)
+    else:
+        raise ValueError("no synthetic weight for this decoder")
+    w["data"] = np.ascontiguousarray(w["data"])
+    if tensor_scales:
+        w["tensor_scale"] = g.uniform(0.5, 2.0, size=tensor_scales).astype(np.float32)
+        w["rows_per_scale"] = n // tensor_scales
+    return w

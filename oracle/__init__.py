@@ -310,3 +310,58 @@ def exl3_product(trellis, svh, k, n, bits, codebook, xh, threads=1):
     y = np.zeros((m, n), dtype=np.float32)
     lib.orc_exl3_product(_p(trellis), _p(svh), k, n, bits, codebook, _p(xh), m, _p(y), threads)
     return y
+
+
+# ---- decode products (src/kernels/decode/products.h of the reference)
+
+DECODERS = ("bf16.dense", "f16.dense", "q8_0.blocks", "nvfp4.split", "nvfp4.atoms", "nvfp4.interleaved",
+            "nvfp4.ggml_blocks", "mxfp8.split", "mxfp8.atoms", "mxfp4.split", "mxfp4.atoms", "affine.split")
+
+
+class DecodeOperand(C.Structure):
+    """src/kernels/decode/operand.h:74-97 of the reference, field for field."""
+    _fields_ = [("data", C.c_void_p), ("scales", C.c_void_p), ("tensor_scale", C.c_void_p), ("biases", C.c_void_p),
+                ("k", C.c_uint32), ("rows", C.c_uint32), ("rows_per_scale", C.c_uint32), ("pad", C.c_uint32),
+                ("row_bytes", C.c_uint64), ("scale_row_bytes", C.c_uint32), ("group", C.c_uint16),
+                ("bits", C.c_uint8), ("scale_type", C.c_uint8)]
+
+
+_sig("orc_ue4m3_to_f32", C.c_float, C.c_uint8)
+_sig("orc_decode_value", C.c_float, _int, C.POINTER(DecodeOperand), _u64, _u64)
+_sig("orc_decode_vector", _int, _int, C.POINTER(DecodeOperand), _u64, _u64, _vp, _u64, _u64, _vp, _u64, _int)
+
+
+def decode_operand(weight):
+    """`weight`: a dict with data (uint8 [rows, row_bytes]), k, and where the decoder has them scales (uint8,
+    flat) and tensor_scale (float32 [rows / rows_per_scale]). The arrays must outlive the operand."""
+    op = DecodeOperand()
+    data = weight["data"]
+    op.data, op.scales, op.tensor_scale = _p(data), _p(weight.get("scales")), _p(weight.get("tensor_scale"))
+    op.k, op.rows = weight["k"], data.shape[0]
+    op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
+    op.row_bytes = data.shape[1]
+    return op
+
+
+def decode_rows_of(decoder, weight):
+    """Every value of the weight, before the tensor scale: float32 [rows, k]."""
+    op = decode_operand(weight)
+    rows, k = weight["data"].shape[0], weight["k"]
+    out = np.empty((rows, k), dtype=np.float32)
+    for r in range(rows):
+        for j in range(k):
+            out[r, j] = lib.orc_decode_value(decoder, C.byref(op), r, j)
+    return out
+
+
+def decode_vector(decoder, weight, x, first=0, outputs=None, threads=1):
+    """llmp.decode.vector on the CPU: float32 x [rows, k] -> [rows, outputs]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    op = decode_operand(weight)
+    outputs = weight["data"].shape[0] - first if outputs is None else outputs
+    y = np.zeros((x.shape[0], outputs), dtype=np.float32)
+    rc = lib.orc_decode_vector(decoder, C.byref(op), first, outputs, _p(x), x.shape[0], x.shape[1], _p(y), outputs,
+                               threads)
+    if rc != 0:
+        raise ValueError("no such decoder")
+    return y

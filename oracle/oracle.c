@@ -386,6 +386,70 @@ double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
   return total;
 }
 
+/* -------------------------------------------------------- decode products */
+
+/* decode.cc:407-411 */
+float orc_ue4m3_to_f32(uint8_t bits) { return bits < 0x7Fu ? orc_e4m3_to_f32(bits) : NAN; }
+
+/* The E2M1 code j of a row of adjacent nibbles (decode.cc:86-91: value 2i in byte i's low nibble). */
+static float fp4_at(const uint8_t* codes, uint64_t j) {
+  const uint8_t b = codes[j / 2];
+  return orc_e2m1_to_f32((uint8_t)((j % 2) ? b >> 4 : b & 15));
+}
+
+float orc_decode_value(int decoder, const orc_decode_operand* w, uint64_t row, uint64_t j) {
+  const uint8_t* data = w->data + row * w->row_bytes;
+  const uint64_t k = w->k;
+  switch (decoder) {
+    case ORC_DECODER_BF16_DENSE: /* decode.cc:52 */
+      return orc_bf16_to_f32(load_u16(data + 2 * j));
+    case ORC_DECODER_F16_DENSE:
+      return orc_f16_to_f32(load_u16(data + 2 * j));
+    case ORC_DECODER_Q8_0_BLOCKS: { /* d * q, ggml's dequantization of these bytes */
+      const uint8_t* block = data + j / 32 * 34;
+      return orc_f16_to_f32(load_u16(block)) * (float)(int8_t)block[2 + j % 32];
+    }
+    case ORC_DECODER_NVFP4_SPLIT: /* decode.cc:296-317 */
+      return fp4_at(data, j) * orc_ue4m3_to_f32(w->scales[row * (k / 16) + j / 16]);
+    case ORC_DECODER_NVFP4_ATOMS:
+      return fp4_at(data, j) * orc_ue4m3_to_f32(w->scales[orc_scale_atom_offset(row, j / 16, k / 16)]);
+    case ORC_DECODER_NVFP4_INTERLEAVED: /* decode.cc:300-304: a row's codes, then its scales */
+      return fp4_at(data, j) * orc_ue4m3_to_f32(data[k / 2 + j / 16]);
+    case ORC_DECODER_NVFP4_GGML_BLOCKS: { /* decode.cc:260-272 */
+      const uint8_t* x = data + j / 64 * 36;
+      const uint64_t sub = (j % 64) / 16, t = j % 16;
+      const uint8_t b = x[4 + sub * 8 + t % 8];
+      return orc_e2m1_to_f32((uint8_t)(t >= 8 ? b >> 4 : b & 15)) * orc_ue4m3_to_f32(x[sub]);
+    }
+    case ORC_DECODER_MXFP8_SPLIT:
+      return orc_e4m3_to_f32(data[j]) * orc_e8m0_to_f32(w->scales[row * (k / 32) + j / 32]);
+    case ORC_DECODER_MXFP8_ATOMS:
+      return orc_e4m3_to_f32(data[j]) * orc_e8m0_to_f32(w->scales[orc_scale_atom_offset(row, j / 32, k / 32)]);
+    case ORC_DECODER_MXFP4_SPLIT:
+      return fp4_at(data, j) * orc_e8m0_to_f32(w->scales[row * (k / 32) + j / 32]);
+    case ORC_DECODER_MXFP4_ATOMS:
+      return fp4_at(data, j) * orc_e8m0_to_f32(w->scales[orc_scale_atom_offset(row, j / 32, k / 32)]);
+    default:
+      return NAN;
+  }
+}
+
+int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
+                      uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
+  if (decoder < 0 || decoder >= ORC_DECODER_AFFINE_SPLIT) return 1;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t j = 0; j < (int64_t)outputs; ++j) {
+    const uint64_t row = first + (uint64_t)j;
+    const double scale = w->tensor_scale != NULL ? (double)w->tensor_scale[row / w->rows_per_scale] : 1.0;
+    for (uint64_t t = 0; t < rows; ++t) {
+      double sum = 0;
+      for (uint64_t c = 0; c < w->k; ++c) sum += (double)orc_decode_value(decoder, w, row, c) * (double)x[t * x_stride + c];
+      y[t * y_stride + (uint64_t)j] = (float)(sum * scale);
+    }
+  }
+  return 0;
+}
+
 /* -------------------------------------------------------------------- GLU */
 
 static double sigmoid_d(double x) { return 1.0 / (1.0 + exp(-x)); }

@@ -75,6 +75,31 @@ void orc_block_sums(int type, const uint8_t* wblock, const uint8_t* q8, int32_t*
 /* One weight block times its Q8_1 blocks in double. */
 double orc_block_product(int type, const uint8_t* wblock, const uint8_t* q8);
 
+/* ---- decode products: src/kernels/decode/products.h:96-109 over the operand of
+ * src/kernels/decode/operand.h:74-97, values as src/kernels/reference/decode.cc decodes them ---- */
+enum {
+  ORC_DECODER_BF16_DENSE = 0, ORC_DECODER_F16_DENSE, ORC_DECODER_Q8_0_BLOCKS, ORC_DECODER_NVFP4_SPLIT,
+  ORC_DECODER_NVFP4_ATOMS, ORC_DECODER_NVFP4_INTERLEAVED, ORC_DECODER_NVFP4_GGML_BLOCKS, ORC_DECODER_MXFP8_SPLIT,
+  ORC_DECODER_MXFP8_ATOMS, ORC_DECODER_MXFP4_SPLIT, ORC_DECODER_MXFP4_ATOMS, ORC_DECODER_AFFINE_SPLIT
+}; /* operand.h:26-41 */
+typedef struct orc_decode_operand { /* operand.h:74-97, field for field */
+  const uint8_t* data;
+  const uint8_t* scales;
+  const float* tensor_scale;
+  const uint8_t* biases;
+  uint32_t k, rows, rows_per_scale, pad;
+  uint64_t row_bytes;
+  uint32_t scale_row_bytes;
+  uint16_t group;
+  uint8_t bits, scale_type;
+} orc_decode_operand;
+float orc_ue4m3_to_f32(uint8_t bits); /* decode.cc:407-411: E4M3's value up to 0x7E, NaN from 0x7F */
+/* Value j of row `row`, before the tensor scale. */
+float orc_decode_value(int decoder, const orc_decode_operand* w, uint64_t row, uint64_t j);
+/* y[t][j] = tensor_scale(first + j) * sum_k W[first + j][k] x[t][k] in double; 1 for an unknown decoder. */
+int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
+                      uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads);
+
 /* ---- GLU: src/kernels/reference/exec.cc:206-214,248-262 ---- */
 enum { ORC_GLU_NONE = 0, ORC_GLU_SWIGLU = 1, ORC_GLU_SWIGLU_CLAMP = 2, ORC_GLU_GEGLU = 3 };
 double orc_glu(int kind, double gate, double up, double limit);

@@ -118,3 +118,29 @@ def test_exl3_linears_refuse_bad_operands():
     two.second = weights()
     assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 8, None) > 0 and b"scratch" in lib.llmp_hip_last_error()
     assert lib.llmp_hip_exl3_multi_linear_scratch(C.byref(two)) == 2 * lib.llmp_hip_exl3_linear_scratch(C.byref(one)) // 17 * 2
+
+
+def test_decode_vector_refuses_bad_operands():
+    lib = _lib.load()
+
+    def operand(**kw):
+        w = _lib.DecodeOperand()
+        base = dict(data=0x1000, scales=0x2000, tensor_scale=None, biases=None, k=256, rows=64, rows_per_scale=64,
+                    row_bytes=128)
+        base.update(kw)
+        for name, value in base.items():
+            setattr(w, name, value)
+        return w
+
+    def run(decoder, w, first=0, outputs=8, x=0x4000, rows=1, x_stride=256, y=0x5000, y_stride=64):
+        return lib.llmp_hip_decode_vector(decoder, C.byref(w), first, outputs, x, rows, x_stride, y, y_stride, None)
+
+    assert run(11, operand()) > 0 and b"no kernel" in lib.llmp_hip_last_error()       # affine
+    assert run(3, operand(), rows=17) > 0 and b"1 to 16" in lib.llmp_hip_last_error()
+    assert run(3, operand(), first=60, outputs=8) > 0
+    assert run(3, operand(scales=None)) > 0 and b"scales" in lib.llmp_hip_last_error()
+    assert run(4, operand(k=32, row_bytes=16)) > 0 and b"multiple" in lib.llmp_hip_last_error()
+    assert run(7, operand(data=0x1008, row_bytes=256)) > 0 and b"aligned" in lib.llmp_hip_last_error()
+    assert run(3, operand(), x=0x4004) > 0
+    assert run(3, operand(), x_stride=258) > 0
+    assert run(9, operand(k=32768, row_bytes=16384), x_stride=32768) > 0 and b"staging" in lib.llmp_hip_last_error()

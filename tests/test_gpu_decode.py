@@ -1,0 +1,120 @@
+"""Parity of llmp.decode.vector (HIP, through the C ABI) against the CPU oracle: every decoder,
+1 to 16 input rows, row windows, strides, tensor scales, undefined block scales. Float outputs to
+a maximum relative error of 1e-3 (the accumulation order is the only difference: both sides
+decode every value exactly)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import rel_close
+from llmp_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+DECODERS = list(range(11))
+
+
+def to_device(weight, device):
+    out = dict(weight)
+    for key in ("data", "scales", "tensor_scale"):
+        if weight.get(key) is not None:
+            out[key] = torch.from_numpy(np.ascontiguousarray(weight[key])).to(device)
+    return out
+
+
+@pytest.mark.parametrize("decoder", DECODERS)
+@pytest.mark.parametrize("rows", [1, 3, 4, 9, 16])
+def test_every_decoder_matches_oracle(device, decoder, rows):
+    n, k = 133, 1024  # an odd number of output rows: the last wave's second row is a copy
+    w = synth.decode_weight(decoder, n, k, 700 + decoder)
+    x = synth.activations(rows, k, 710 + rows)
+    want = oracle.decode_vector(decoder, w, x, threads=oracle.max_threads())
+    got = ops.decode_vector(decoder, to_device(w, device), torch.from_numpy(x).to(device)).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, (oracle.DECODERS[decoder], worst)
+    # An input row's outputs do not depend on the rows beside it (src/kernels/decode/products.h:33-35).
+    alone = ops.decode_vector(decoder, to_device(w, device), torch.from_numpy(x[rows - 1:]).to(device)).cpu().numpy()
+    assert np.array_equal(alone[0].view(np.uint32), got[rows - 1].view(np.uint32))
+
+
+@pytest.mark.parametrize("decoder", [0, 3, 6, 8])
+def test_windows_strides_and_tensor_scales(device, decoder):
+    n, k, rows = 256, 512, 2
+    w = synth.decode_weight(decoder, n, k, 720 + decoder, tensor_scales=4)
+    x = synth.activations(rows, k, 721)
+    wide = np.zeros((rows, k + 8), dtype=np.float32)
+    wide[:, :k] = x
+    xd = torch.from_numpy(wide).to(device)[:, :k]  # rows k + 8 floats apart
+    want = oracle.decode_vector(decoder, w, x, first=60, outputs=77)
+    got = ops.decode_vector(decoder, to_device(w, device), xd, first=60, outputs=77).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst
+    # The tensor scale multiplies each output once: rows 64.. take the second scale.
+    plain = dict(w)
+    plain["tensor_scale"] = None
+    bare = ops.decode_vector(decoder, to_device(plain, device), xd, first=60, outputs=77).cpu().numpy()
+    scale = w["tensor_scale"][(60 + np.arange(77)) // w["rows_per_scale"]]
+    assert np.array_equal((bare * scale).view(np.uint32), got.view(np.uint32))
+
+
+def test_every_code_and_undefined_scales(device):
+    """All 256 E4M3 codes and all 16 E2M1 codes against the oracle's values exactly (one nonzero input
+    a row picks one weight value out); block scales the format leaves undefined are NaN
+    (tests/unit/reference_decode_test.cc:407-484 of the reference)."""
+    k = 256
+    # mxfp8.split: row r holds code r at position r % k, scale 2^0; x is all ones.
+    codes = np.zeros((256, k), dtype=np.uint8)
+    codes[np.arange(256), np.arange(256) % k] = np.arange(256, dtype=np.uint8)
+    w = {"k": k, "data": codes, "scales": np.full(256 * (k // 32), 127, dtype=np.uint8)}
+    x = np.ones((1, k), dtype=np.float32)
+    got = ops.decode_vector(7, to_device(w, device), torch.from_numpy(x).to(device)).cpu().numpy()[0]
+    want = np.array([oracle.lib.orc_e4m3_to_f32(c) for c in range(256)], dtype=np.float32)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    keep = ~np.isnan(want)
+    assert np.array_equal(got[keep], want[keep])
+    # nvfp4.split: row r holds code r % 16 in nibble r of its first bytes, scale 0x38 (1.0).
+    codes = np.zeros((32, k // 2), dtype=np.uint8)
+    for r in range(32):
+        codes[r, r // 2] = (r % 16) << (4 * (r % 2))
+    scales = np.full((32, k // 16), 0x38, dtype=np.uint8)
+    w = {"k": k, "data": codes, "scales": scales.reshape(-1)}
+    got = ops.decode_vector(3, to_device(w, device), torch.from_numpy(x).to(device)).cpu().numpy()[0]
+    want = np.array([oracle.lib.orc_e2m1_to_f32(r % 16) for r in range(32)], dtype=np.float32)
+    assert np.array_equal(got, want)
+    # Undefined scales: UE4M3 from 0x7F up, E8M0 0xFF.
+    for decoder, bad in ((3, 0x7F), (3, 0x80), (3, 0xFF), (6, 0xB8), (9, 0xFF), (7, 0xFF)):
+        w = synth.decode_weight(decoder, 4, k, 730 + decoder)
+        if decoder == 6:
+            w["data"][2, 1] = bad  # row 2's second sub-block scale
+        else:
+            w["scales"] = w["scales"].copy()
+            blocks = k // (16 if decoder == 3 else 32)
+            w["scales"][2 * blocks + 1] = bad
+        got = ops.decode_vector(decoder, to_device(w, device), torch.from_numpy(synth.activations(1, k, 731)).to(device))
+        got = got.cpu().numpy()[0]
+        assert np.isnan(got[2]) and np.all(np.isfinite(got[[0, 1, 3]])), (decoder, bad, got)
+
+
+def test_long_rows_take_fewer_input_rows_a_launch(device):
+    n, k, rows = 12, 8192, 7  # two input rows a launch at this length
+    w = synth.decode_weight(9, n, k, 740)
+    x = synth.activations(rows, k, 741)
+    want = oracle.decode_vector(9, w, x, threads=oracle.max_threads())
+    got = ops.decode_vector(9, to_device(w, device), torch.from_numpy(x).to(device)).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst
+
+
+def test_refusals(device):
+    w = to_device(synth.decode_weight(3, 8, 256, 750), device)
+    x = torch.zeros((17, 256), dtype=torch.float32, device=device)
+    with pytest.raises(ops.KernelFailure) as e:
+        ops.decode_vector(3, w, x)
+    assert e.value.rejected
+    with pytest.raises(ops.KernelFailure):  # the affine decoder is not built
+        ops.decode_vector(11, w, x[:1])
+    with pytest.raises(ops.KernelFailure):  # rows [6, 10) of 8
+        ops.decode_vector(3, w, x[:1], first=6, outputs=4)
+    with pytest.raises(ops.KernelFailure):  # scale atoms take k in whole 64 values
+        ops.decode_vector(4, to_device(synth.decode_weight(3, 8, 32, 751), device), x[:1, :32])

@@ -318,6 +318,75 @@ def test_mxfp4_values_layout_and_products():
     assert oracle.vecq(oracle.TYPE_MXFP4, w, q8, 32, 1)[0, 0, 0] == 18.0
 
 
+def test_decode_products_values_and_layouts():
+    """The decode products' oracle (orc_decode_value, orc_decode_vector) against the reference's known
+    answers and independent restatements: NVFP4 bytes of 0x22 are ones times their block scale in
+    all four layouts, undefined scales NaN (tests/unit/reference_decode_test.cc:407-462); every
+    layout of an encoding holds the same values; the product is the decoded matrix times x."""
+    from llmp_amd import synth
+    scales8 = [0x00, 0x01, 0x38, 0x7E, 0x7F, 0x80, 0xB8, 0xFF]
+    for b in range(256):  # decode.cc:407-411
+        v = oracle.lib.orc_ue4m3_to_f32(b)
+        assert np.isnan(v) == (b >= 0x7F)
+        if b < 0x7F:
+            assert v == oracle.lib.orc_e4m3_to_f32(b)
+    assert oracle.lib.orc_ue4m3_to_f32(0x38) == 1.0 and oracle.lib.orc_ue4m3_to_f32(0x01) == 2.0 ** -9
+    k, n, blocks = 128, 4, 8
+    codes = np.full((n, k // 2), 0x22, dtype=np.uint8)
+    scales = np.array([scales8[i % 8] for i in range(n * blocks)], dtype=np.uint8).reshape(n, blocks)
+    atoms = np.zeros(128 * blocks, dtype=np.uint8)
+    for r in range(n):
+        for b in range(blocks):
+            atoms[oracle.lib.orc_scale_atom_offset(r, b, blocks)] = scales[r, b]
+    ggml = np.concatenate([scales.reshape(n, k // 64, 4), np.full((n, k // 64, 32), 0x22, dtype=np.uint8)],
+                          axis=-1).reshape(n, -1)
+    layouts = {3: {"k": k, "data": codes, "scales": scales.reshape(-1)},
+               4: {"k": k, "data": codes, "scales": atoms},
+               5: {"k": k, "data": np.ascontiguousarray(np.concatenate([codes, scales], axis=1))},
+               6: {"k": k, "data": np.ascontiguousarray(ggml)}}
+    for decoder, w in layouts.items():
+        got = oracle.decode_rows_of(decoder, w)
+        for i in range(n * k):
+            sc = scales.reshape(-1)[i // 16]
+            if sc >= 0x7F:
+                assert np.isnan(got.reshape(-1)[i]), (decoder, i)
+            else:
+                assert got.reshape(-1)[i] == oracle.lib.orc_e4m3_to_f32(sc), (decoder, i)
+    # Random weights: the layouts of one encoding hold the same values; numpy restatements.
+    e2m1 = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], dtype=np.float32)
+    n, k = 130, 256
+    w6 = synth.decode_weight(6, n, k, 41)
+    codes, scales = w6["plain"]
+    nib = np.stack([codes & 15, codes >> 4], axis=-1).reshape(n, k)  # value 2 i in byte i's low nibble
+    ue = np.array([oracle.lib.orc_ue4m3_to_f32(b) for b in range(256)], dtype=np.float32)
+    want = e2m1[nib] * np.repeat(ue[scales], 16, axis=1)
+    assert np.array_equal(oracle.decode_rows_of(6, w6), want)
+    for decoder in (3, 4, 5):
+        w = synth.decode_weight(decoder, n, k, 41)  # the same seed: the same codes and scales
+        assert np.array_equal(oracle.decode_rows_of(decoder, w), want), decoder
+    for split, atoms_id, per in ((7, 8, 32), (9, 10, 32)):
+        a, b = synth.decode_weight(split, n, k, 42), synth.decode_weight(atoms_id, n, k, 42)
+        assert np.array_equal(oracle.decode_rows_of(split, a), oracle.decode_rows_of(atoms_id, b))
+    w9 = synth.decode_weight(9, n, k, 43)
+    nib = np.stack([w9["data"] & 15, w9["data"] >> 4], axis=-1).reshape(n, k)
+    e8 = np.exp2(w9["scales"].reshape(n, k // 32).astype(np.float32) - 127)
+    assert np.array_equal(oracle.decode_rows_of(9, w9), e2m1[nib] * np.repeat(e8, 32, axis=1))
+    w0 = synth.decode_weight(0, 9, 64, 44)
+    assert np.array_equal(oracle.decode_rows_of(0, w0), synth.bf16_to_f32(w0["data"].view(np.uint16)))
+    w1 = synth.decode_weight(1, 9, 64, 45)
+    assert np.array_equal(oracle.decode_rows_of(1, w1), w1["data"].view(np.float16).astype(np.float32))
+    w2 = synth.decode_weight(2, 9, 64, 46)
+    assert np.array_equal(oracle.decode_rows_of(2, w2), oracle.decode_rows(oracle.TYPE_Q8_0, w2["data"], 64))
+    # The product: decoded rows times x, a window of rows, tensor scales once an output.
+    w = synth.decode_weight(6, 64, 128, 47, tensor_scales=2)
+    x = np.random.Generator(np.random.PCG64(48)).standard_normal((3, 128)).astype(np.float32)
+    dense = oracle.decode_rows_of(6, w).astype(np.float64)
+    scale = w["tensor_scale"][np.arange(64) // 32].astype(np.float64)
+    want = (x.astype(np.float64) @ dense.T) * scale
+    np.testing.assert_allclose(oracle.decode_vector(6, w, x), want, rtol=1e-6, atol=1e-9)
+    np.testing.assert_allclose(oracle.decode_vector(6, w, x, first=20, outputs=30), want[:, 20:50], rtol=1e-6, atol=1e-9)
+
+
 def kv_blocks_numpy(t, x):
     """src/kernels/ggml/kv_quant.cuh:27-69 restated with numpy float32 operations (IEEE, one
     rounding each), apart from the oracle's C."""
