@@ -1,7 +1,8 @@
 // The host side of the MI355X kernels in the reference's own C++ vocabulary: the launch
 // interfaces its operator wrappers call (src/kernels/ggml/vecq.h:22-47,
 // src/kernels/ggml/mxfp8_cutlass.h:26-79, src/kernels/exl3/validate.h:84-131 and
-// src/kernels/exl3/linear.h:47-54, src/kernels/selected_operation.h:26-35 of the reference),
+// src/kernels/exl3/linear.h:47-54, src/kernels/decode/products.h:96-109,
+// src/kernels/selected_operation.h:26-35 of the reference),
 // with the same names, argument meaning and error behaviour, over the C ABI of llmp_hip.h.
 // Header only, C++17, no HIP or torch types: a stream is the void* the reference's
 // NativeStream carries.
@@ -131,6 +132,36 @@ inline int Run(const Gemm& gemm, int sms, void* stream) {
 
 }  // namespace mxfp8
 }  // namespace ggml
+
+namespace decode {
+
+// src/kernels/decode/operand.h:26-41.
+enum class DecoderId : std::uint8_t {
+  kBf16Dense, kF16Dense, kQ8_0Blocks, kNvfp4Split, kNvfp4Atoms, kNvfp4Interleaved, kNvfp4GgmlBlocks,
+  kMxfp8Split, kMxfp8Atoms, kMxfp4Split, kMxfp4Atoms, kAffineSplit, kCount
+};
+// src/kernels/decode/operand.h:74-97: the C ABI's operand is that struct field for field.
+using Operand = llmp_decode_operand;
+static_assert(sizeof(Operand) == 64, "Operand descriptor must be 64 bytes");
+
+// The arguments of RunVector (src/kernels/decode/products.h:96-109) once OperandOf has bound the weight.
+struct Product {
+  DecoderId decoder = DecoderId::kBf16Dense;
+  Operand weight{};
+  std::uint64_t first = 0;
+  std::uint64_t outputs = 0;
+  const float* x = nullptr;
+  std::uint64_t rows = 0;
+  std::uint64_t x_stride = 0;
+  float* y = nullptr;
+  std::uint64_t y_stride = 0;
+};
+inline KernelFailure RunVector(const Product& p, void* stream) {
+  return FromStatus(llmp_hip_decode_vector(static_cast<int>(p.decoder), &p.weight, p.first, p.outputs, p.x, p.rows,
+                                           p.x_stride, p.y, p.y_stride, stream));
+}
+
+}  // namespace decode
 
 namespace exl3 {
 

@@ -116,6 +116,10 @@ void HostChecks() {
   EXPECT(hipk::ggml::mxfp8::Run(gemm, 256, nullptr) > 0);  // null operands: refused, nothing queued
   hipk::exl3::LinearOperands linear;
   EXPECT(hipk::exl3::PackedLinear(linear, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
+  hipk::decode::Product product;
+  EXPECT(hipk::decode::RunVector(product, nullptr) == hipk::KernelFailure::kRejected);
+  product.decoder = hipk::decode::DecoderId::kAffineSplit;
+  EXPECT(hipk::decode::RunVector(product, nullptr) == hipk::KernelFailure::kRejected);
   hipk::exl3::MultiLinearOperands multi;
   EXPECT(hipk::exl3::MultiLinear(multi, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
   EXPECT(hipk::exl3::ScratchBytes(multi) == 0);
