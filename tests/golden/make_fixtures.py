@@ -48,6 +48,23 @@ def build():
     out["q4_0_w"], out["q4_0_x"] = w40, a
     out["q4_0_y"] = oracle.vecq(oracle.TYPE_Q4_0, w40, q8, k, n, tokens=2)
     out["q4_0_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q4_0, w40, q8[:1], k, n)
+    # llmp.vecq, MXFP4 (17-byte blocks), 2 tokens.
+    k, n = 512, 12
+    wm = synth.mxfp4_weights(n, k, 24)
+    a = synth.activations(2, k, 25)
+    q8 = oracle.q8_1_quantize(a)
+    out["mxfp4_w"], out["mxfp4_x"] = wm, a
+    out["mxfp4_y"] = oracle.vecq(oracle.TYPE_MXFP4, wm, q8, k, n, tokens=2)
+    out["mxfp4_sums"] = oracle.vecq_block_sums(oracle.TYPE_MXFP4, wm, q8[:1], k, n)
+    # llmp.decode.vector: NVFP4 in GGML's blocks with tensor scales, MXFP8 in scale atoms; 3 input rows.
+    k, n = 256, 20
+    xd = synth.activations(3, k, 26)
+    w6 = synth.decode_weight(6, n, k, 27, tensor_scales=2)
+    out["dec_x"], out["dec6_data"], out["dec6_tensor_scale"] = xd, w6["data"], w6["tensor_scale"]
+    out["dec6_y"] = oracle.decode_vector(6, w6, xd)
+    w8a = synth.decode_weight(8, n, k, 28)
+    out["dec8_data"], out["dec8_scales"] = w8a["data"], w8a["scales"]
+    out["dec8_y"] = oracle.decode_vector(8, w8a, xd, first=3, outputs=11)
     # MXFP8: quantizer and one small product.
     xa = synth.activations(5, 256, 17) * 3.0
     xb = synth.activations(8, 256, 18) * 0.02

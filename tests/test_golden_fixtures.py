@@ -82,6 +82,20 @@ def test_device_meets_the_committed_vectors(vectors, device):
     q8 = ops.quantize_q8_1(_dev(v["q4_0_x"], device))
     close(ops.vecq(ops.TYPE_Q4_0, w, q8, k, n, tokens=2).cpu().numpy(), v["q4_0_y"], 1e-3, "q4_0")
     assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q4_0, w, q8[:1], k, n).cpu().numpy(), v["q4_0_sums"])
+    # MXFP4 dense, two tokens; int32 block sums.
+    k, n = 512, 12
+    w = _dev(v["mxfp4_w"], device)
+    q8 = ops.quantize_q8_1(_dev(v["mxfp4_x"], device))
+    close(ops.vecq(ops.TYPE_MXFP4, w, q8, k, n, tokens=2).cpu().numpy(), v["mxfp4_y"], 1e-3, "mxfp4")
+    assert np.array_equal(ops.vecq_block_sums(ops.TYPE_MXFP4, w, q8[:1], k, n).cpu().numpy(), v["mxfp4_sums"])
+    # Decode products: NVFP4 in GGML's blocks with tensor scales; MXFP8 in scale atoms, a window of rows.
+    k, n = 256, 20
+    xd = _dev(v["dec_x"], device)
+    w6 = {"k": k, "data": _dev(v["dec6_data"], device), "tensor_scale": _dev(v["dec6_tensor_scale"], device),
+          "rows_per_scale": n // 2}
+    close(ops.decode_vector(6, w6, xd).cpu().numpy(), v["dec6_y"], 1e-3, "decode nvfp4.ggml_blocks")
+    w8a = {"k": k, "data": _dev(v["dec8_data"], device), "scales": _dev(v["dec8_scales"], device)}
+    close(ops.decode_vector(8, w8a, xd, first=3, outputs=11).cpu().numpy(), v["dec8_y"], 1e-3, "decode mxfp8.atoms")
     # MXFP8 quantizer (bytes) and product.
     ac, as_ = ops.mxfp8_quantize(_dev(v["mx_a"], device))
     bc, bs = ops.mxfp8_quantize(_dev(v["mx_b"], device))
