@@ -285,10 +285,10 @@ def block_formats(device):
 
 
 # HBM bytes per launch of the dominant kernel at batch 1 through the default variant, from two
-# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,475.1 KiB and WRITE_SIZE 60.2 KiB per dispatch,
+# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,478.4 KiB and WRITE_SIZE 60.1 KiB per dispatch,
 # scaled by 1.9988 and 1.0: what the same counters read for --calibrate-copy's copy of 64,800 KiB).
 # Counters cannot be read from inside a run, so other shapes and variants report null.
-PROFILED_TRAFFIC_BYTES = int(round((32475.1 * 1.9988 + 60.2) * 1024))
+PROFILED_TRAFFIC_BYTES = int(round((32478.4 * 1.9988 + 60.1) * 1024))
 
 
 def measured_traffic(args):
