@@ -161,6 +161,30 @@ inline KernelFailure RunVector(const Product& p, void* stream) {
                                            p.x_stride, p.y, p.y_stride, stream));
 }
 
+// GluProduct and RunVectorGlu (src/kernels/decode/products.h:120-139); `glu` is ir::GluKind's value
+// (src/ir/op.h:455), `limit` GluParams::limit.
+struct GluProduct {
+  DecoderId gate_decoder = DecoderId::kBf16Dense;
+  Operand gate{};
+  std::uint64_t gate_first = 0;
+  DecoderId up_decoder = DecoderId::kBf16Dense;
+  Operand up{};
+  std::uint64_t up_first = 0;
+  std::uint64_t outputs = 0;
+  int glu = 0;
+  float limit = 0.0f;
+  const float* x = nullptr;
+  std::uint64_t rows = 0;
+  std::uint64_t x_stride = 0;
+  float* y = nullptr;
+  std::uint64_t y_stride = 0;
+};
+inline KernelFailure RunVectorGlu(const GluProduct& p, void* stream) {
+  return FromStatus(llmp_hip_decode_vector_glu(static_cast<int>(p.gate_decoder), &p.gate, p.gate_first,
+                                               static_cast<int>(p.up_decoder), &p.up, p.up_first, p.outputs, p.glu,
+                                               p.limit, p.x, p.rows, p.x_stride, p.y, p.y_stride, stream));
+}
+
 }  // namespace decode
 
 namespace exl3 {

@@ -1,6 +1,6 @@
-// llmp.decode.vector for gfx950: products over weights in their stored encodings, a block
-// decoder per encoding and layout under one kernel template (src/kernels/decode/products.h:96-109,
-// decoders.cuh and operand.h of the reference). y[t][j] = tensor_scale(first + j) * sum_k
+// llmp.decode.vector and llmp.decode.vector_glu for gfx950: products over weights in their stored
+// encodings, a block decoder per encoding and layout under one kernel template
+// (src/kernels/decode/products.h:96-139, decoders.cuh, templates.cuh and operand.h of the reference). y[t][j] = tensor_scale(first + j) * sum_k
 // W[first + j][k] x[t][k] for 1 to 16 F32 input rows; every decoder decodes a value as the
 // reference's CPU decoder does (src/kernels/reference/decode.cc), the products are F32.
 //
@@ -29,6 +29,10 @@ constexpr size_t kDecodeLdsLimit = 80 * 1024;  // two workgroups a CU
 
 struct DecodeArgs {
   llmp_decode_operand w;
+  llmp_decode_operand up;  // the GLU form's second weight (w is its gate)
+  uint32_t up_first;
+  int glu;                 // ir::GluKind
+  float limit;
   uint32_t first;
   uint32_t outputs;
   uint32_t token0;  // the pass's first input row
@@ -69,6 +73,25 @@ __device__ __forceinline__ void Fp8Four(uint32_t word, float* v) {
   const Float2 a = __builtin_amdgcn_cvt_pk_f32_fp8(word, false);
   const Float2 b = __builtin_amdgcn_cvt_pk_f32_fp8(word, true);
   v[0] = a[0], v[1] = a[1], v[2] = b[0], v[3] = b[1];
+}
+
+// src/kernels/decode/templates.cuh:73-90 of the reference; ir::GluKind: SwiGLU 0, GeGLU (erf) 1, GeGLU (tanh) 2,
+// SwiGLU with a clamp 3.
+__device__ __forceinline__ float DecodeGlu(int kind, float g, float u, float limit) {
+#pragma clang fp contract(off)
+  switch (kind) {
+    case 1:
+      return 0.5f * g * (1.0f + erff(g * 0.70710678118654752f)) * u;
+    case 2:
+      return 0.5f * g * (1.0f + tanhf(0.79788456080286536f * (g + (0.044715f * g * g * g)))) * u;
+    case 3: {
+      const float gc = fminf(g, limit);
+      const float uc = fminf(fmaxf(u, -limit), limit);
+      return gc / (1.0f + expf(-gc)) * uc;
+    }
+    default:
+      return g / (1.0f + expf(-g)) * u;
+  }
 }
 
 // Segment `seg` (16 values) of row `row`: the values before the block scale, and that scale.
@@ -143,7 +166,8 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
 }
 
 // grid: workgroups of eight waves, persistent over pairs of output rows; LDS: T input rows.
-template <int D, int T>
+// kGlu: a wave's two rows are gate row first + j and up row up_first + j of output j.
+template <int D, int T, bool kGlu>
 __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const DecodeArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x;
@@ -160,9 +184,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
   }
   __syncthreads();  // the only one: from here the waves run alone
 
-  const uint32_t pairs = (a.outputs + kRowsAWave - 1) / kRowsAWave;
+  const uint32_t pairs = kGlu ? a.outputs : (a.outputs + kRowsAWave - 1) / kRowsAWave;
   for (uint32_t pair = blockIdx.x * waves + wave; pair < pairs; pair += gridDim.x * waves) {
-    const uint32_t out0 = pair * kRowsAWave;
+    const uint32_t out0 = kGlu ? pair : pair * kRowsAWave;
     float acc[kRowsAWave][T];
 #pragma unroll
     for (int r = 0; r < kRowsAWave; ++r) {
@@ -173,9 +197,17 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
       float v[kRowsAWave][16], s[kRowsAWave];
 #pragma unroll
       for (int r = 0; r < kRowsAWave; ++r) {
-        // A lone last row is decoded twice: its second copy's sums are not stored.
-        const uint32_t out = min(out0 + r, a.outputs - 1);
-        LoadSegment<D>(a.w, a.first + out, seg, v[r], s[r]);
+        if constexpr (kGlu) {
+          if (r == 0) {
+            LoadSegment<D>(a.w, a.first + out0, seg, v[r], s[r]);
+          } else {
+            LoadSegment<D>(a.up, a.up_first + out0, seg, v[r], s[r]);
+          }
+        } else {
+          // A lone last row is decoded twice: its second copy's sums are not stored.
+          const uint32_t out = min(out0 + r, a.outputs - 1);
+          LoadSegment<D>(a.w, a.first + out, seg, v[r], s[r]);
+        }
       }
 #pragma unroll
       for (int t = 0; t < T; ++t) {
@@ -190,6 +222,21 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
           acc[r][t] = fmaf(dot, s[r], acc[r][t]);
         }
       }
+    }
+    if constexpr (kGlu) {
+      const float gate_scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out0) / a.w.rows_per_scale] : 1.0f;
+      const float up_scale = a.up.tensor_scale != nullptr ? a.up.tensor_scale[(a.up_first + out0) / a.up.rows_per_scale] : 1.0f;
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        float gate = acc[0][t], up = acc[1][t];
+#pragma unroll
+        for (int mask = 32; mask >= 1; mask >>= 1) {
+          gate += ShflXor(gate, mask);
+          up += ShflXor(up, mask);
+        }
+        if (lane == 0) a.y[(a.token0 + t) * a.y_stride + out0] = DecodeGlu(a.glu, gate * gate_scale, up * up_scale, a.limit);
+      }
+      continue;
     }
 #pragma unroll
     for (int r = 0; r < kRowsAWave; ++r) {
@@ -209,25 +256,34 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
 
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
-template <int D, int T>
+template <int D, int T, bool kGlu>
 void LaunchDecode(const DecodeArgs& a, int groups, int waves, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T, kGlu>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDecodeLdsLimit));
     sized = true;
   }
-  hipLaunchKernelGGL((DecodeVectorKernel<D, T>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
+  hipLaunchKernelGGL((DecodeVectorKernel<D, T, kGlu>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
                      DecodeLds(T, a.w.k), stream, a);
 }
 
-template <int D>
-void LaunchDecoder(const DecodeArgs& a, int tokens, int groups, int waves, hipStream_t stream) {
+template <int D, bool kGlu>
+void LaunchTokens(const DecodeArgs& a, int tokens, int groups, int waves, hipStream_t stream) {
   switch (tokens) {
-    case 1: LaunchDecode<D, 1>(a, groups, waves, stream); break;
-    case 2: LaunchDecode<D, 2>(a, groups, waves, stream); break;
-    case 3: LaunchDecode<D, 3>(a, groups, waves, stream); break;
-    default: LaunchDecode<D, 4>(a, groups, waves, stream); break;
+    case 1: LaunchDecode<D, 1, kGlu>(a, groups, waves, stream); break;
+    case 2: LaunchDecode<D, 2, kGlu>(a, groups, waves, stream); break;
+    case 3: LaunchDecode<D, 3, kGlu>(a, groups, waves, stream); break;
+    default: LaunchDecode<D, 4, kGlu>(a, groups, waves, stream); break;
+  }
+}
+
+template <int D>
+void LaunchDecoder(const DecodeArgs& a, bool glu, int tokens, int groups, int waves, hipStream_t stream) {
+  if (glu) {
+    LaunchTokens<D, true>(a, tokens, groups, waves, stream);
+  } else {
+    LaunchTokens<D, false>(a, tokens, groups, waves, stream);
   }
 }
 
@@ -258,63 +314,52 @@ bool SplitScales(int decoder) {
          decoder == LLMP_DECODER_MXFP8_ATOMS || decoder == LLMP_DECODER_MXFP4_SPLIT || decoder == LLMP_DECODER_MXFP4_ATOMS;
 }
 
-}  // namespace
-}  // namespace llmp_hip
-
-using namespace llmp_hip;
-
-extern "C" int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
-                                      const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
-                                      void* stream) {
-  if (w == nullptr) return Refuse(1, "decode.vector: null operand");
-  if (decoder < 0 || decoder >= LLMP_DECODER_AFFINE_SPLIT)
-    return Refuse(1, "decode.vector: decoder %d has no kernel", decoder);
-  if (w->data == nullptr || x == nullptr || y == nullptr) return Refuse(1, "decode.vector: null operand");
-  if (SplitScales(decoder) && w->scales == nullptr) return Refuse(1, "decode.vector: the layout's block scales are missing");
+int CheckOperand(const char* what, int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs) {
+  if (w == nullptr) return Refuse(1, "%s: null operand", what);
+  if (decoder < 0 || decoder >= LLMP_DECODER_AFFINE_SPLIT) return Refuse(1, "%s: decoder %d has no kernel", what, decoder);
+  if (w->data == nullptr) return Refuse(1, "%s: null operand", what);
+  if (SplitScales(decoder) && w->scales == nullptr) return Refuse(1, "%s: the layout's block scales are missing", what);
   if (w->k == 0 || w->k % KMultiple(decoder) != 0)
-    return Refuse(1, "decode.vector: k %u is not a multiple of the decoder's %u", w->k, KMultiple(decoder));
-  if (rows == 0 || rows > 16 || outputs == 0 || first > w->rows || outputs > w->rows - first)
-    return Refuse(1, "decode.vector: rows %llu (1 to 16), outputs [%llu, %llu) of %u",
-                  static_cast<unsigned long long>(rows), static_cast<unsigned long long>(first),
+    return Refuse(1, "%s: k %u is not a multiple of the decoder's %u", what, w->k, KMultiple(decoder));
+  if (outputs == 0 || first > w->rows || outputs > w->rows - first)
+    return Refuse(1, "%s: outputs [%llu, %llu) of %u", what, static_cast<unsigned long long>(first),
                   static_cast<unsigned long long>(first + outputs), w->rows);
-  if (w->tensor_scale != nullptr && w->rows_per_scale == 0) return Refuse(1, "decode.vector: tensor scales of no rows");
+  if (w->tensor_scale != nullptr && w->rows_per_scale == 0) return Refuse(1, "%s: tensor scales of no rows", what);
   if (reinterpret_cast<uintptr_t>(w->data) % DataAlignment(decoder) != 0 || w->row_bytes % DataAlignment(decoder) != 0)
-    return Refuse(1, "decode.vector: the weight's rows are not aligned for its decoder's loads (%u bytes)",
+    return Refuse(1, "%s: the weight's rows are not aligned for its decoder's loads (%u bytes)", what,
                   DataAlignment(decoder));
-  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_stride % 4 != 0 || x_stride < w->k || y_stride < outputs ||
-      reinterpret_cast<uintptr_t>(y) % 4 != 0)
-    return Refuse(1, "decode.vector: input rows are 16-byte aligned, a multiple of 4 floats apart and at least k long");
-  // The rows a pass stages must fit LDS: four, or fewer of a long row.
+  return 0;
+}
+
+// The launches of a product whose operands have been checked: four input rows a pass, or
+// fewer of a long row.
+int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64_t rows, hipStream_t s) {
+  const uint32_t k = a.w.k;
+  if (rows == 0 || rows > 16) return Refuse(1, "%s: rows %llu (1 to 16)", what, static_cast<unsigned long long>(rows));
+  if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || a.x_stride % 4 != 0 || a.x_stride < k || a.y_stride < a.outputs ||
+      reinterpret_cast<uintptr_t>(a.y) % 4 != 0)
+    return Refuse(1, "%s: input rows are 16-byte aligned, a multiple of 4 floats apart and at least k long", what);
   int pass = rows < 4 ? static_cast<int>(rows) : 4;
-  while (pass > 1 && DecodeLds(pass, w->k) > kDecodeLdsLimit) --pass;
-  if (DecodeLds(pass, w->k) > kDecodeLdsLimit)
-    return Refuse(1, "decode.vector: a row of %u values does not fit the staging area (16384 at most)", w->k);
+  while (pass > 1 && DecodeLds(pass, k) > kDecodeLdsLimit) --pass;
+  if (DecodeLds(pass, k) > kDecodeLdsLimit)
+    return Refuse(1, "%s: a row of %u values does not fit the staging area (16384 at most)", what, k);
   const int cus = llmp_hip_compute_units();
-  const size_t lds = DecodeLds(pass, w->k);
+  const size_t lds = DecodeLds(pass, k);
   // One input row: four waves a workgroup and more workgroups; several: eight waves share the staged rows.
   const int waves = pass == 1 ? 4 : kDecodeWaves;
   int resident = static_cast<int>(160 * 1024 / (lds + 1024));
   if (resident > 32 / waves) resident = 32 / waves;  // a CU holds 32 waves
   if (resident < 1) resident = 1;
-  const uint64_t pairs = (outputs + kRowsAWave - 1) / kRowsAWave;
+  const uint64_t pairs = glu ? a.outputs : (a.outputs + kRowsAWave - 1) / kRowsAWave;
   uint64_t groups = (pairs + waves - 1) / waves;
   const uint64_t most = static_cast<uint64_t>(cus > 0 ? cus : 256) * resident;
   if (groups > most) groups = most;
-  DecodeArgs a;
-  a.w = *w;
-  a.first = static_cast<uint32_t>(first);
-  a.outputs = static_cast<uint32_t>(outputs);
-  a.x = x;
-  a.x_stride = x_stride;
-  a.y = y;
-  a.y_stride = y_stride;
-  const auto s = static_cast<hipStream_t>(stream);
   for (uint64_t token0 = 0; token0 < rows; token0 += pass) {
     const int tokens = static_cast<int>(rows - token0 < static_cast<uint64_t>(pass) ? rows - token0 : pass);
     a.token0 = static_cast<uint32_t>(token0);
     switch (decoder) {
 #define LLMP_DECODER(ID) \
-  case ID: LaunchDecoder<ID>(a, tokens, static_cast<int>(groups), waves, s); break;
+  case ID: LaunchDecoder<ID>(a, glu, tokens, static_cast<int>(groups), waves, s); break;
       LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
       LLMP_DECODER(LLMP_DECODER_F16_DENSE)
       LLMP_DECODER(LLMP_DECODER_Q8_0_BLOCKS)
@@ -328,8 +373,48 @@ extern "C" int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* w,
       LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
 #undef LLMP_DECODER
     }
-    const int status = LaunchStatus("decode.vector");
+    const int status = LaunchStatus(what);
     if (status != 0) return token0 == 0 ? status : (status > 0 ? -status : status);
   }
   return 0;
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+using namespace llmp_hip;
+
+extern "C" int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
+                                      const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
+                                      void* stream) {
+  if (const int bad = CheckOperand("decode.vector", decoder, w, first, outputs); bad != 0) return bad;
+  if (x == nullptr || y == nullptr) return Refuse(1, "decode.vector: null operand");
+  DecodeArgs a{};
+  a.w = *w;
+  a.first = static_cast<uint32_t>(first);
+  a.outputs = static_cast<uint32_t>(outputs);
+  a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
+  return LaunchProduct("decode.vector", decoder, false, a, rows, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_operand* gate, uint64_t gate_first,
+                                          int up_decoder, const llmp_decode_operand* up, uint64_t up_first,
+                                          uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
+                                          uint64_t x_stride, float* y, uint64_t y_stride, void* stream) {
+  if (const int bad = CheckOperand("decode.vector_glu gate", gate_decoder, gate, gate_first, outputs); bad != 0) return bad;
+  if (const int bad = CheckOperand("decode.vector_glu up", up_decoder, up, up_first, outputs); bad != 0) return bad;
+  if (gate_decoder != up_decoder)
+    return Refuse(1, "decode.vector_glu: no instantiation for gate decoder %d with up decoder %d", gate_decoder, up_decoder);
+  if (gate->k != up->k) return Refuse(1, "decode.vector_glu: gate's K %u and up's %u differ", gate->k, up->k);
+  if (glu < 0 || glu > 3) return Refuse(1, "decode.vector_glu: unknown GLU");
+  if (x == nullptr || y == nullptr) return Refuse(1, "decode.vector_glu: null operand");
+  DecodeArgs a{};
+  a.w = *gate;
+  a.up = *up;
+  a.first = static_cast<uint32_t>(gate_first);
+  a.up_first = static_cast<uint32_t>(up_first);
+  a.outputs = static_cast<uint32_t>(outputs);
+  a.glu = glu, a.limit = limit;
+  a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
+  return LaunchProduct("decode.vector_glu", gate_decoder, true, a, rows, static_cast<hipStream_t>(stream));
 }

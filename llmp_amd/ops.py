@@ -364,6 +364,31 @@ DECODERS = ("bf16.dense", "f16.dense", "q8_0.blocks", "nvfp4.split", "nvfp4.atom
             "nvfp4.ggml_blocks", "mxfp8.split", "mxfp8.atoms", "mxfp4.split", "mxfp4.atoms", "affine.split")
 
 
+def _decode_operand(weight):
+    data = weight["data"]
+    op = DecodeOperand()
+    op.data = data.data_ptr()
+    op.scales = weight["scales"].data_ptr() if weight.get("scales") is not None else None
+    op.tensor_scale = weight["tensor_scale"].data_ptr() if weight.get("tensor_scale") is not None else None
+    op.k, op.rows, op.row_bytes = weight["k"], data.shape[0], data.stride(0)
+    op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
+    return op
+
+
+def decode_vector_glu(decoder, gate, up, x, glu, limit=0.0, gate_first=0, up_first=0, outputs=None, up_decoder=None):
+    """llmp.decode.vector_glu: glu(gate rows . x, up rows . x), float32 [rows, outputs]; `glu` is the
+    reference's ir::GluKind (0 SwiGLU, 1 GeGLU erf, 2 GeGLU tanh, 3 SwiGLU with a clamp at `limit`)."""
+    lib = _lib.load()
+    g, u = _decode_operand(gate), _decode_operand(up)
+    outputs = gate["data"].shape[0] - gate_first if outputs is None else outputs
+    rows = x.shape[0]
+    y = torch.empty((rows, outputs), dtype=torch.float32, device=x.device)
+    _lib.check(lib.llmp_hip_decode_vector_glu(decoder, C.byref(g), gate_first, decoder if up_decoder is None else up_decoder,
+                                              C.byref(u), up_first, outputs, glu, limit, _ptr(x), rows, x.stride(0),
+                                              _ptr(y), y.stride(0), _stream()))
+    return y
+
+
 def decode_vector(decoder, weight, x, first=0, outputs=None, out=None):
     """llmp.decode.vector: float32 x [rows <= 16, k] times a weight in its stored encoding. `weight` is a
     dict of device tensors: data (uint8 [n, row_bytes]), k, and where the decoder has them scales (uint8)

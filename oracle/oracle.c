@@ -450,6 +450,43 @@ int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, 
   return 0;
 }
 
+/* exec.cc:248-262 with ir::GluKind's numbering (src/ir/op.h:455): SwiGLU 0, GeGLU (erf) 1, GeGLU (tanh) 2, SwiGLU
+ * with a clamp 3. */
+static double decode_glu(int kind, double g, double u, double limit) {
+  switch (kind) {
+    case 1: return 0.5 * g * (1.0 + erf(g / sqrt(2.0))) * u;
+    case 2: return 0.5 * g * (1.0 + tanh(sqrt(2.0 / M_PI) * g * (1.0 + 0.044715 * g * g))) * u;
+    case 3: {
+      const double gc = g < limit ? g : limit;
+      const double uc = u < -limit ? -limit : (u > limit ? limit : u);
+      return gc / (1.0 + exp(-gc)) * uc;
+    }
+    default: return g / (1.0 + exp(-g)) * u;
+  }
+}
+
+int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, const orc_decode_operand* up,
+                          uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
+                          uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
+  if (decoder < 0 || decoder >= ORC_DECODER_AFFINE_SPLIT || glu < 0 || glu > 3 || gate->k != up->k) return 1;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t j = 0; j < (int64_t)outputs; ++j) {
+    const uint64_t grow = gate_first + (uint64_t)j, urow = up_first + (uint64_t)j;
+    const double gs = gate->tensor_scale != NULL ? (double)gate->tensor_scale[grow / gate->rows_per_scale] : 1.0;
+    const double us = up->tensor_scale != NULL ? (double)up->tensor_scale[urow / up->rows_per_scale] : 1.0;
+    for (uint64_t t = 0; t < rows; ++t) {
+      double g = 0, u = 0;
+      for (uint64_t c = 0; c < gate->k; ++c) {
+        const double xv = (double)x[t * x_stride + c];
+        g += (double)orc_decode_value(decoder, gate, grow, c) * xv;
+        u += (double)orc_decode_value(decoder, up, urow, c) * xv;
+      }
+      y[t * y_stride + (uint64_t)j] = (float)decode_glu(glu, g * gs, u * us, (double)limit);
+    }
+  }
+  return 0;
+}
+
 /* -------------------------------------------------------------------- GLU */
 
 static double sigmoid_d(double x) { return 1.0 / (1.0 + exp(-x)); }

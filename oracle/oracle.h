@@ -100,6 +100,12 @@ float orc_decode_value(int decoder, const orc_decode_operand* w, uint64_t row, u
 int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
                       uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads);
 
+/* RunVectorGlu, products.h:120-139: y[t][j] = glu(gate row . x[t], up row . x[t]); glu is ir::GluKind
+ * (src/ir/op.h:455), the functions those of src/kernels/reference/exec.cc:248-262. */
+int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, const orc_decode_operand* up,
+                          uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
+                          uint64_t x_stride, float* y, uint64_t y_stride, int threads);
+
 /* ---- GLU: src/kernels/reference/exec.cc:206-214,248-262 ---- */
 enum { ORC_GLU_NONE = 0, ORC_GLU_SWIGLU = 1, ORC_GLU_SWIGLU_CLAMP = 2, ORC_GLU_GEGLU = 3 };
 double orc_glu(int kind, double gate, double up, double limit);

@@ -118,3 +118,45 @@ def test_refusals(device):
         ops.decode_vector(3, w, x[:1], first=6, outputs=4)
     with pytest.raises(ops.KernelFailure):  # scale atoms take k in whole 64 values
         ops.decode_vector(4, to_device(synth.decode_weight(3, 8, 32, 751), device), x[:1, :32])
+
+
+@pytest.mark.parametrize("decoder", [0, 2, 6, 8, 9])
+@pytest.mark.parametrize("glu", [0, 1, 2, 3])
+@pytest.mark.parametrize("rows", [1, 5])
+def test_vector_glu_matches_oracle(device, decoder, glu, rows):
+    """RunVectorGlu (src/kernels/decode/products.h:120-139 of the reference): the four GLUs of
+    src/kernels/decode/templates.cuh:73-90 over a gate and an up weight with their own tensor scales."""
+    n, k = 96, 512
+    gate = synth.decode_weight(decoder, n, k, 760 + decoder, tensor_scales=2)
+    up = synth.decode_weight(decoder, n, k, 770 + decoder, tensor_scales=3)
+    x = synth.activations(rows, k, 780 + rows) * 0.25
+    limit = 1.5 if glu == 3 else 0.0
+    want = oracle.decode_vector_glu(decoder, gate, up, x, glu, limit, gate_first=8, up_first=3, outputs=70)
+    got = ops.decode_vector_glu(decoder, to_device(gate, device), to_device(up, device), torch.from_numpy(x).to(device),
+                                glu, limit, gate_first=8, up_first=3, outputs=70).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, (oracle.DECODERS[decoder], glu, worst)
+    # The two sums are the plain products': SwiGLU of llmp.decode.vector's outputs, to float rounding.
+    g = ops.decode_vector(decoder, to_device(gate, device), torch.from_numpy(x).to(device), first=8, outputs=70)
+    u = ops.decode_vector(decoder, to_device(up, device), torch.from_numpy(x).to(device), first=3, outputs=70)
+    if glu == 0:
+        silu = g / (1.0 + torch.exp(-g)) * u
+        np.testing.assert_allclose(got, silu.cpu().numpy(), rtol=2e-6, atol=1e-9)
+
+
+def test_vector_glu_of_one_stacked_weight_and_refusals(device):
+    n, k = 64, 256
+    w = synth.decode_weight(3, 2 * n, k, 790)  # gate rows, then up rows, in one weight
+    x = synth.activations(2, k, 791) * 0.25
+    want = oracle.decode_vector_glu(3, w, w, x, 0, gate_first=0, up_first=n, outputs=n)
+    wd = to_device(w, device)
+    xd = torch.from_numpy(x).to(device)
+    got = ops.decode_vector_glu(3, wd, wd, xd, 0, gate_first=0, up_first=n, outputs=n).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst
+    with pytest.raises(ops.KernelFailure):  # an unknown GLU
+        ops.decode_vector_glu(3, wd, wd, xd, 4, outputs=n)
+    with pytest.raises(ops.KernelFailure):  # up rows [100, 164) of 128
+        ops.decode_vector_glu(3, wd, wd, xd, 0, up_first=100, outputs=n)
+    with pytest.raises(ops.KernelFailure):  # a gate and an up of different decoders
+        ops.decode_vector_glu(3, wd, to_device(synth.decode_weight(9, n, k, 792), device), xd, 0, outputs=n, up_decoder=9)

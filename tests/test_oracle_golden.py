@@ -387,6 +387,32 @@ def test_decode_products_values_and_layouts():
     np.testing.assert_allclose(oracle.decode_vector(6, w, x, first=20, outputs=30), want[:, 20:50], rtol=1e-6, atol=1e-9)
 
 
+def test_decode_glu_products_against_closed_forms():
+    """orc_decode_vector_glu: glu(gate . x, up . x) with the four functions of the reference's CPU executor
+    (src/kernels/reference/exec.cc:248-262), here from scipy's erf and numpy, over the oracle's own plain products."""
+    from scipy.special import erf
+    from llmp_amd import synth
+    n, k = 24, 128
+    gate = synth.decode_weight(9, n, k, 51, tensor_scales=2)
+    up = synth.decode_weight(9, n, k, 52)
+    x = np.random.Generator(np.random.PCG64(53)).standard_normal((2, k)).astype(np.float32) * 0.25
+    g = oracle.decode_vector(9, gate, x).astype(np.float64)
+    u = oracle.decode_vector(9, up, x).astype(np.float64)
+    silu = lambda v: v / (1.0 + np.exp(-v))
+    forms = {0: silu(g) * u,
+             1: 0.5 * g * (1.0 + erf(g / np.sqrt(2.0))) * u,
+             2: 0.5 * g * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (g + 0.044715 * g ** 3))) * u,
+             3: silu(np.minimum(g, 0.75)) * np.clip(u, -0.75, 0.75)}
+    for kind, want in forms.items():
+        got = oracle.decode_vector_glu(9, gate, up, x, kind, 0.75 if kind == 3 else 0.0)
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-7)
+    # Row windows of one stacked weight.
+    both = synth.decode_weight(3, 2 * n, k, 54)
+    got = oracle.decode_vector_glu(3, both, both, x, 0, gate_first=0, up_first=n, outputs=n)
+    want = silu(oracle.decode_vector(3, both, x, first=0, outputs=n).astype(np.float64)) * oracle.decode_vector(3, both, x, first=n, outputs=n)
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-7)
+
+
 def kv_blocks_numpy(t, x):
     """src/kernels/ggml/kv_quant.cuh:27-69 restated with numpy float32 operations (IEEE, one
     rounding each), apart from the oracle's C."""
