@@ -324,6 +324,12 @@ int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_operand* gate
                                const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
                                void* stream);
 
+/* RunRows of src/kernels/decode/products.h:172-183: out[i][:] = W[ids[i]][:] as F32 (times the row's tensor
+ * scale) for i < count; ids are device I32; an id outside the matrix writes zeros and sets *bad (a device
+ * I32, or null) to 1. Output rows 16-byte aligned, out_stride (floats) a multiple of 4. */
+int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* weight, const int32_t* ids, uint64_t count, float* out,
+                         uint64_t out_stride, int32_t* bad, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -185,6 +185,21 @@ inline KernelFailure RunVectorGlu(const GluProduct& p, void* stream) {
                                                p.limit, p.x, p.rows, p.x_stride, p.y, p.y_stride, stream));
 }
 
+// RowsGather and RunRows (src/kernels/decode/products.h:172-183).
+struct RowsGather {
+  DecoderId decoder = DecoderId::kBf16Dense;
+  Operand weight{};
+  const std::int32_t* ids = nullptr;
+  std::uint64_t count = 0;
+  float* out = nullptr;
+  std::uint64_t out_stride = 0;
+  std::int32_t* bad = nullptr;
+};
+inline KernelFailure RunRows(const RowsGather& g, void* stream) {
+  return FromStatus(llmp_hip_decode_rows(static_cast<int>(g.decoder), &g.weight, g.ids, g.count, g.out, g.out_stride,
+                                         g.bad, stream));
+}
+
 }  // namespace decode
 
 namespace exl3 {

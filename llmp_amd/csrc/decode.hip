@@ -254,6 +254,34 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
   }
 }
 
+// out[i][:] = W[ids[i]][:] as F32, times the row's tensor scale; an id outside the matrix writes
+// zeros and sets *bad (products.h:172-183). A wave a gathered row, its lanes the segments.
+template <int D>
+__global__ __launch_bounds__(256) void DecodeRowsKernel(const llmp_decode_operand w, const int32_t* __restrict__ ids,
+                                                      uint32_t count, float* __restrict__ out, uint64_t out_stride,
+                                                      int32_t* __restrict__ bad) {
+#pragma clang fp contract(off)
+  const int lane = threadIdx.x & 63;
+  const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (i >= count) return;  // whole waves
+  const int32_t id = ids[i];
+  const bool known = id >= 0 && static_cast<uint32_t>(id) < w.rows;
+  float4* row = reinterpret_cast<float4*>(out + i * out_stride);
+  if (!known && bad != nullptr && lane == 0) *bad = 1;
+  const float scale = known && w.tensor_scale != nullptr ? w.tensor_scale[static_cast<uint32_t>(id) / w.rows_per_scale] : 1.0f;
+  for (uint32_t seg = lane; seg < w.k / 16u; seg += 64) {
+    float v[16] = {};
+    if (known) {
+      float s;
+      LoadSegment<D>(w, static_cast<uint32_t>(id), seg, v, s);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v[j] = (v[j] * s) * scale;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) row[seg * 4u + q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+  }
+}
+
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
 template <int D, int T, bool kGlu>
@@ -417,4 +445,36 @@ extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_op
   a.glu = glu, a.limit = limit;
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
   return LaunchProduct("decode.vector_glu", gate_decoder, true, a, rows, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* w, const int32_t* ids, uint64_t count,
+                                    float* out, uint64_t out_stride, int32_t* bad, void* stream) {
+  if (const int status = CheckOperand("decode.rows", decoder, w, 0, 1); status != 0) return status;
+  if (ids == nullptr || out == nullptr) return Refuse(1, "decode.rows: null operand");
+  if (count == 0 || count > (uint64_t{1} << 31)) return Refuse(1, "decode.rows: 1 to 2^31 rows");
+  if (reinterpret_cast<uintptr_t>(out) % 16 != 0 || out_stride % 4 != 0 || out_stride < w->k ||
+      reinterpret_cast<uintptr_t>(ids) % 4 != 0 || reinterpret_cast<uintptr_t>(bad) % 4 != 0)
+    return Refuse(1, "decode.rows: output rows are 16-byte aligned, a multiple of 4 floats apart and at least k long");
+  const dim3 grid(static_cast<unsigned>((count + 3) / 4));
+  const auto s = static_cast<hipStream_t>(stream);
+  switch (decoder) {
+#define LLMP_DECODER(ID)                                                                                          \
+  case ID:                                                                                                        \
+    hipLaunchKernelGGL((DecodeRowsKernel<ID>), grid, dim3(256), 0, s, *w, ids, static_cast<uint32_t>(count), out, \
+                       out_stride, bad);                                                                          \
+    break;
+    LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_F16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_Q8_0_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_INTERLEAVED)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_GGML_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+#undef LLMP_DECODER
+  }
+  return LaunchStatus("decode.rows");
 }

@@ -407,3 +407,14 @@ def decode_vector(decoder, weight, x, first=0, outputs=None, out=None):
     _lib.check(lib.llmp_hip_decode_vector(decoder, C.byref(op), first, outputs, _ptr(x), rows, x.stride(0), _ptr(y),
                                           y.stride(0), _stream()))
     return y
+
+
+def decode_rows(decoder, weight, ids, bad=None):
+    """llmp.decode.rows: rows ids[i] (int32) of a weight in its stored encoding as float32 [count, k], times their
+    tensor scales; an id outside the matrix gives a row of zeros and sets `bad` (an int32 tensor of one element)."""
+    lib = _lib.load()
+    op = _decode_operand(weight)
+    out = torch.empty((ids.numel(), weight["k"]), dtype=torch.float32, device=ids.device)
+    _lib.check(lib.llmp_hip_decode_rows(decoder, C.byref(op), _ptr(ids), ids.numel(), _ptr(out), out.stride(0),
+                                        _ptr(bad) if bad is not None else None, _stream()))
+    return out

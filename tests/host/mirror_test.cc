@@ -122,6 +122,8 @@ void HostChecks() {
   EXPECT(hipk::decode::RunVector(product, nullptr) == hipk::KernelFailure::kRejected);
   hipk::decode::GluProduct glu_product;
   EXPECT(hipk::decode::RunVectorGlu(glu_product, nullptr) == hipk::KernelFailure::kRejected);
+  hipk::decode::RowsGather gather;
+  EXPECT(hipk::decode::RunRows(gather, nullptr) == hipk::KernelFailure::kRejected);
   hipk::exl3::MultiLinearOperands multi;
   EXPECT(hipk::exl3::MultiLinear(multi, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
   EXPECT(hipk::exl3::ScratchBytes(multi) == 0);

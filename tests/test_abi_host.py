@@ -144,3 +144,13 @@ def test_decode_vector_refuses_bad_operands():
     assert run(3, operand(), x=0x4004) > 0
     assert run(3, operand(), x_stride=258) > 0
     assert run(9, operand(k=32768, row_bytes=16384), x_stride=32768) > 0 and b"staging" in lib.llmp_hip_last_error()
+    gate, up = operand(), operand(k=512, row_bytes=256)
+    glu = lambda gd, ud, kind: lib.llmp_hip_decode_vector_glu(gd, C.byref(gate), 0, ud, C.byref(up), 0, 8, kind, 0.0,
+                                                              0x4000, 1, 512, 0x5000, 64, None)
+    assert glu(3, 3, 0) > 0 and b"differ" in lib.llmp_hip_last_error()            # K 256 against 512
+    assert glu(3, 9, 0) > 0 and b"no instantiation" in lib.llmp_hip_last_error()  # mixed decoders
+    up = operand()
+    assert glu(3, 3, 7) > 0 and b"GLU" in lib.llmp_hip_last_error()
+    rows = lambda **kw: lib.llmp_hip_decode_rows(kw.get("decoder", 3), C.byref(operand()), kw.get("ids", 0x6000),
+                                                 kw.get("count", 4), kw.get("out", 0x7000), kw.get("stride", 256), None, None)
+    assert rows(decoder=11) > 0 and rows(ids=None) > 0 and rows(count=0) > 0 and rows(out=0x7004) > 0 and rows(stride=250) > 0

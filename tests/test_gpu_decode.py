@@ -160,3 +160,22 @@ def test_vector_glu_of_one_stacked_weight_and_refusals(device):
         ops.decode_vector_glu(3, wd, wd, xd, 0, up_first=100, outputs=n)
     with pytest.raises(ops.KernelFailure):  # a gate and an up of different decoders
         ops.decode_vector_glu(3, wd, to_device(synth.decode_weight(9, n, k, 792), device), xd, 0, outputs=n, up_decoder=9)
+
+
+@pytest.mark.parametrize("decoder", DECODERS)
+def test_rows_gather_is_the_decoded_rows_bit_for_bit(device, decoder):
+    """RunRows (src/kernels/decode/products.h:172-183 of the reference): rows by index as F32, times their tensor
+    scale; an id outside the matrix writes zeros and raises the flag."""
+    n, k = 40, 512
+    w = synth.decode_weight(decoder, n, k, 800 + decoder, tensor_scales=4)
+    dense = oracle.decode_rows_of(decoder, w) * w["tensor_scale"][np.arange(n) // w["rows_per_scale"]][:, None]
+    ids = np.array([3, 39, 0, 17, 17, 8, 25], dtype=np.int32)
+    bad = torch.zeros(1, dtype=torch.int32, device=device)
+    got = ops.decode_rows(decoder, to_device(w, device), torch.from_numpy(ids).to(device), bad=bad).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), dense[ids].astype(np.float32).view(np.uint32))
+    assert int(bad.item()) == 0
+    ids = np.array([5, -1, 40, 12], dtype=np.int32)
+    got = ops.decode_rows(decoder, to_device(w, device), torch.from_numpy(ids).to(device), bad=bad).cpu().numpy()
+    assert int(bad.item()) == 1
+    assert np.all(got[1] == 0) and np.all(got[2] == 0)
+    assert np.array_equal(got[[0, 3]].view(np.uint32), dense[[5, 12]].astype(np.float32).view(np.uint32))
