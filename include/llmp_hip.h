@@ -280,8 +280,8 @@ int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, 
  * of 4 floats) at x + t * x_stride, of y at y + t * y_stride. The decoders are the reference's
  * (src/kernels/decode/operand.h:26-41, decoders.cuh), the operand its Operand
  * (operand.h:74-97) field for field; values decode as src/kernels/reference/decode.cc has
- * them (an undefined block scale, UE4M3 from 0x7F or E8M0 0xFF, is NaN). The affine decoder is
- * not built (refused). Rows up to 16384 values; four input rows a launch (fewer of long rows),
+ * them (an undefined block scale, UE4M3 from 0x7F or E8M0 0xFF, is NaN; the affine encoding is
+ * s * q + b rounded once, or s * (q - z)). Rows up to 16384 values; four input rows a launch (fewer of long rows),
  * so 1 to 16 launches are queued and a failure after the first is a fault (negative). */
 enum {
   LLMP_DECODER_BF16_DENSE = 0,
@@ -301,16 +301,16 @@ typedef struct llmp_decode_operand {
   const uint8_t* data;       /* kData, or kCodes for the split arrangements */
   const uint8_t* scales;     /* kBlockScales for the split arrangements */
   const float* tensor_scale; /* or null: row r takes tensor_scale[r / rows_per_scale] */
-  const uint8_t* biases;     /* affine only */
+  const uint8_t* biases;     /* affine only: biases as the scales, or packed zero points */
   uint32_t k;                /* values a row */
   uint32_t rows;             /* rows of the matrix */
   uint32_t rows_per_scale;
   uint32_t pad;
   uint64_t row_bytes;        /* bytes of a row of `data` */
-  uint32_t scale_row_bytes;  /* affine only */
-  uint16_t group;            /* affine only */
-  uint8_t bits;              /* affine only */
-  uint8_t scale_type;        /* affine only */
+  uint32_t scale_row_bytes;  /* affine only: bytes of a row of `scales` (and of the biases) */
+  uint16_t group;            /* affine only: values a group (32, 64, 128) */
+  uint8_t bits;              /* affine only: 4 or 8 bits a code */
+  uint8_t scale_type;        /* affine only: 1 F16, 2 BF16, 3 F32; | 0x80 with zero points */
 } llmp_decode_operand;
 int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* weight, uint64_t first, uint64_t outputs,
                            const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, void* stream);

@@ -142,6 +142,46 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
     Fp4Halves(c[0], v, v + 8);
     Fp4Halves(c[1], v + 4, v + 12);
     s = Ue4m3ToFloat((scales >> (8u * sub)) & 0xFFu);
+  } else if constexpr (D == LLMP_DECODER_AFFINE_SPLIT) {
+    // Unsigned codes of 4 or 8 bits, a scale and a bias (or a zero point) a group of values along the
+    // row; a segment lies within one group. s * q + b rounded once, or s * (q - z)
+    // (src/kernels/reference/decode.cc:197-220).
+#pragma clang fp contract(off)
+    const uint32_t g = seg * 16u / w.group;
+    const uint64_t scale_row = static_cast<uint64_t>(row) * w.scale_row_bytes;
+    const uint32_t scale_type = w.scale_type & 0x7Fu;
+    auto element = [&](const uint8_t* base) {
+      if (scale_type == 3u) return *reinterpret_cast<const float*>(base + scale_row + g * 4u);
+      const uint32_t bits = *reinterpret_cast<const uint16_t*>(base + scale_row + g * 2u);
+      return scale_type == 2u ? __builtin_bit_cast(float, bits << 16) : HalfBitsToFloat(bits);
+    };
+    const float scale = element(w.scales);
+    const bool zero_point = (w.scale_type & 0x80u) != 0;
+    int32_t z = 0;
+    float b = 0.0f;
+    if (zero_point) {
+      const uint64_t zero_row = (static_cast<uint64_t>(w.k / w.group) * w.bits + 7) / 8;
+      const uint8_t* zeros = w.biases + row * zero_row;
+      z = w.bits == 4 ? (zeros[g / 2u] >> (4u * (g & 1u))) & 15u : zeros[g];
+    } else if (w.biases != nullptr) {
+      b = element(w.biases);
+    }
+    uint32_t code[16];
+    if (w.bits == 4) {
+      const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
+#pragma unroll
+      for (int i = 0; i < 16; ++i) code[i] = ((i < 8 ? c.x : c.y) >> (4 * (i % 8))) & 15u;
+    } else {
+      const U32x4 c = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
+#pragma unroll
+      for (int i = 0; i < 16; ++i) code[i] = (c[i / 4] >> (8 * (i % 4))) & 0xFFu;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      v[i] = zero_point ? scale * static_cast<float>(static_cast<int32_t>(code[i]) - z)
+                        : fmaf(scale, static_cast<float>(code[i]), b);
+    }
+    s = 1.0f;
   } else if constexpr (D == LLMP_DECODER_MXFP8_SPLIT || D == LLMP_DECODER_MXFP8_ATOMS) {
     const U32x4 c = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
     Fp8Four(c.x, v), Fp8Four(c.y, v + 4), Fp8Four(c.z, v + 8), Fp8Four(c.w, v + 12);
@@ -325,7 +365,8 @@ uint32_t KMultiple(int decoder) {
     default: return 16;
   }
 }
-// The alignment a decoder's loads of `data` need (products.h:38-43).
+// The alignment a decoder's loads of `data` need (products.h:38-43); the affine decoder's by its
+// code width (16 bytes for 8-bit codes, 8 for 4-bit).
 uint32_t DataAlignment(int decoder) {
   switch (decoder) {
     case LLMP_DECODER_BF16_DENSE: case LLMP_DECODER_F16_DENSE: case LLMP_DECODER_MXFP8_SPLIT:
@@ -344,8 +385,20 @@ bool SplitScales(int decoder) {
 
 int CheckOperand(const char* what, int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs) {
   if (w == nullptr) return Refuse(1, "%s: null operand", what);
-  if (decoder < 0 || decoder >= LLMP_DECODER_AFFINE_SPLIT) return Refuse(1, "%s: decoder %d has no kernel", what, decoder);
+  if (decoder < 0 || decoder > LLMP_DECODER_AFFINE_SPLIT) return Refuse(1, "%s: decoder %d has no kernel", what, decoder);
   if (w->data == nullptr) return Refuse(1, "%s: null operand", what);
+  if (decoder == LLMP_DECODER_AFFINE_SPLIT) {
+    const uint32_t element = w->scale_type & 0x7Fu;
+    if ((w->bits != 4 && w->bits != 8) || (w->group != 32 && w->group != 64 && w->group != 128) || element < 1 || element > 3)
+      return Refuse(1, "%s: affine codes of 4 or 8 bits, groups of 32, 64 or 128 values, F16, BF16 or F32 scales", what);
+    if (w->scales == nullptr || ((w->scale_type & 0x80u) != 0 && w->biases == nullptr))
+      return Refuse(1, "%s: the affine encoding's scales or zero points are missing", what);
+    if (w->k == 0 || w->k % w->group != 0) return Refuse(1, "%s: k %u is not whole groups of %u", what, w->k, w->group);
+    const uint32_t step = element == 3u ? 4u : 2u;
+    if ((reinterpret_cast<uintptr_t>(w->scales) | w->scale_row_bytes) % step != 0 ||
+        ((w->scale_type & 0x80u) == 0 && w->biases != nullptr && reinterpret_cast<uintptr_t>(w->biases) % step != 0))
+      return Refuse(1, "%s: the affine scales are not aligned to their element", what);
+  }
   if (SplitScales(decoder) && w->scales == nullptr) return Refuse(1, "%s: the layout's block scales are missing", what);
   if (w->k == 0 || w->k % KMultiple(decoder) != 0)
     return Refuse(1, "%s: k %u is not a multiple of the decoder's %u", what, w->k, KMultiple(decoder));
@@ -353,9 +406,9 @@ int CheckOperand(const char* what, int decoder, const llmp_decode_operand* w, ui
     return Refuse(1, "%s: outputs [%llu, %llu) of %u", what, static_cast<unsigned long long>(first),
                   static_cast<unsigned long long>(first + outputs), w->rows);
   if (w->tensor_scale != nullptr && w->rows_per_scale == 0) return Refuse(1, "%s: tensor scales of no rows", what);
-  if (reinterpret_cast<uintptr_t>(w->data) % DataAlignment(decoder) != 0 || w->row_bytes % DataAlignment(decoder) != 0)
-    return Refuse(1, "%s: the weight's rows are not aligned for its decoder's loads (%u bytes)", what,
-                  DataAlignment(decoder));
+  const uint32_t alignment = decoder == LLMP_DECODER_AFFINE_SPLIT ? (w->bits == 8 ? 16u : 8u) : DataAlignment(decoder);
+  if (reinterpret_cast<uintptr_t>(w->data) % alignment != 0 || w->row_bytes % alignment != 0)
+    return Refuse(1, "%s: the weight's rows are not aligned for its decoder's loads (%u bytes)", what, alignment);
   return 0;
 }
 
@@ -399,6 +452,7 @@ int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64
       LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
       LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
       LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+      LLMP_DECODER(LLMP_DECODER_AFFINE_SPLIT)
 #undef LLMP_DECODER
     }
     const int status = LaunchStatus(what);
@@ -474,6 +528,7 @@ extern "C" int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* w, c
     LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
     LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
     LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_AFFINE_SPLIT)
 #undef LLMP_DECODER
   }
   return LaunchStatus("decode.rows");

@@ -372,6 +372,10 @@ def _decode_operand(weight):
     op.tensor_scale = weight["tensor_scale"].data_ptr() if weight.get("tensor_scale") is not None else None
     op.k, op.rows, op.row_bytes = weight["k"], data.shape[0], data.stride(0)
     op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
+    if "group" in weight:  # the affine encoding
+        op.biases = weight["biases"].data_ptr() if weight.get("biases") is not None else None
+        op.group, op.bits, op.scale_type = weight["group"], weight["bits"], weight["scale_type"]
+        op.scale_row_bytes = weight["scale_row_bytes"]
     return op
 
 
@@ -395,12 +399,7 @@ def decode_vector(decoder, weight, x, first=0, outputs=None, out=None):
     and tensor_scale (float32) with rows_per_scale. Returns float32 [rows, outputs]."""
     lib = _lib.load()
     data = weight["data"]
-    op = DecodeOperand()
-    op.data = data.data_ptr()
-    op.scales = weight["scales"].data_ptr() if weight.get("scales") is not None else None
-    op.tensor_scale = weight["tensor_scale"].data_ptr() if weight.get("tensor_scale") is not None else None
-    op.k, op.rows, op.row_bytes = weight["k"], data.shape[0], data.stride(0)
-    op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
+    op = _decode_operand(weight)
     outputs = data.shape[0] - first if outputs is None else outputs
     rows = x.shape[0]
     y = torch.empty((rows, outputs), dtype=torch.float32, device=x.device) if out is None else out

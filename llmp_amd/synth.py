@@ -152,9 +152,47 @@ def decode_weight(decoder, n, k, seed, tensor_scales=0):
         codes = g.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
         scales = g.integers(118, 126, size=(n, k // 32), dtype=np.uint8)
         w["data"], w["scales"] = codes, scales.reshape(-1) if decoder == 9 else atoms(scales, k // 32)
+    elif decoder == 11:
+        raise ValueError("affine weights come from affine_weight()")
     else:
         raise ValueError("no synthetic weight for this decoder")
     w["data"] = np.ascontiguousarray(w["data"])
+    if tensor_scales:
+        w["tensor_scale"] = g.uniform(0.5, 2.0, size=tensor_scales).astype(np.float32)
+        w["rows_per_scale"] = n // tensor_scales
+    return w
+
+
+def affine_weight(n, k, seed, bits=4, group=64, scale="f16", zero_point=False, tensor_scales=0):
+    """An MLX-style affine weight as the reference's affine.split decoder reads it (src/kernels/decode/operand.h:
+    74-97): unsigned codes of `bits` bits packed little-endian along the row, a scale and a bias (or, with
+    `zero_point`, a packed zero point) a group of `group` values; scales F16, BF16 or F32."""
+    g = rng(seed)
+    groups = k // group
+    codes = g.integers(0, 1 << bits, size=(n, k), dtype=np.uint8)
+    data = (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8) if bits == 4 else codes
+    sc = g.uniform(0.002, 0.01, size=(n, groups)).astype(np.float32)
+    bias = (-sc * (1 << (bits - 1)) + g.uniform(-0.003, 0.003, size=(n, groups))).astype(np.float32)
+    kind = {"f16": 1, "bf16": 2, "f32": 3}[scale]
+
+    def pack(a):
+        if kind == 3:
+            return np.ascontiguousarray(a).view(np.uint8).reshape(n, -1)
+        if kind == 2:
+            return bf16_bits(a).view(np.uint8).reshape(n, -1)
+        return a.astype(np.float16).view(np.uint8).reshape(n, -1)
+
+    w = {"k": k, "data": np.ascontiguousarray(data), "scales": pack(sc), "group": group, "bits": bits,
+         "scale_type": kind | (0x80 if zero_point else 0), "scale_row_bytes": groups * (4 if kind == 3 else 2)}
+    if zero_point:
+        zeros = g.integers(0, 1 << bits, size=(n, groups), dtype=np.uint8)
+        if bits == 4:
+            padded = np.zeros((n, (groups + 1) // 2 * 2), dtype=np.uint8)
+            padded[:, :groups] = zeros
+            zeros = (padded[:, 0::2] | (padded[:, 1::2] << 4)).astype(np.uint8)
+        w["biases"] = np.ascontiguousarray(zeros)
+    else:
+        w["biases"] = pack(bias)
     if tensor_scales:
         w["tensor_scale"] = g.uniform(0.5, 2.0, size=tensor_scales).astype(np.float32)
         w["rows_per_scale"] = n // tensor_scales

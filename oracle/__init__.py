@@ -340,6 +340,10 @@ def decode_operand(weight):
     op.k, op.rows = weight["k"], data.shape[0]
     op.rows_per_scale = weight.get("rows_per_scale", data.shape[0])
     op.row_bytes = data.shape[1]
+    if "group" in weight:  # the affine encoding
+        op.biases = _p(weight.get("biases"))
+        op.group, op.bits, op.scale_type = weight["group"], weight["bits"], weight["scale_type"]
+        op.scale_row_bytes = weight["scale_row_bytes"]
     return op
 
 

@@ -429,6 +429,33 @@ float orc_decode_value(int decoder, const orc_decode_operand* w, uint64_t row, u
       return fp4_at(data, j) * orc_e8m0_to_f32(w->scales[row * (k / 32) + j / 32]);
     case ORC_DECODER_MXFP4_ATOMS:
       return fp4_at(data, j) * orc_e8m0_to_f32(w->scales[orc_scale_atom_offset(row, j / 32, k / 32)]);
+    case ORC_DECODER_AFFINE_SPLIT: { /* decode.cc:173-220: s * q + b rounded once, or s * (q - z) */
+      const uint64_t g = j / w->group, groups = k / w->group;
+      const int element = w->scale_type & 0x7F; /* 1 F16, 2 BF16, 3 F32 (operand.h:96) */
+      const uint8_t* srow = w->scales + row * w->scale_row_bytes;
+      float sc, b = 0.0f;
+      uint32_t q = 0, z = 0;
+      for (uint32_t i = 0; i < w->bits; ++i) {
+        const uint64_t bit = j * w->bits + i;
+        q |= (uint32_t)((data[bit / 8] >> (bit % 8)) & 1u) << i;
+      }
+      if (element == 3) memcpy(&sc, srow + 4 * g, 4);
+      else sc = element == 2 ? orc_bf16_to_f32(load_u16(srow + 2 * g)) : orc_f16_to_f32(load_u16(srow + 2 * g));
+      if (w->scale_type & 0x80) {
+        const uint8_t* zeros = w->biases + row * ((groups * w->bits + 7) / 8);
+        for (uint32_t i = 0; i < w->bits; ++i) {
+          const uint64_t bit = g * w->bits + i;
+          z |= (uint32_t)((zeros[bit / 8] >> (bit % 8)) & 1u) << i;
+        }
+        return sc * (float)((int32_t)q - (int32_t)z);
+      }
+      if (w->biases != NULL) {
+        const uint8_t* brow = w->biases + row * w->scale_row_bytes;
+        if (element == 3) memcpy(&b, brow + 4 * g, 4);
+        else b = element == 2 ? orc_bf16_to_f32(load_u16(brow + 2 * g)) : orc_f16_to_f32(load_u16(brow + 2 * g));
+      }
+      return fmaf(sc, (float)q, b);
+    }
     default:
       return NAN;
   }
@@ -436,7 +463,7 @@ float orc_decode_value(int decoder, const orc_decode_operand* w, uint64_t row, u
 
 int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
                       uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
-  if (decoder < 0 || decoder >= ORC_DECODER_AFFINE_SPLIT) return 1;
+  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT) return 1;
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
   for (int64_t j = 0; j < (int64_t)outputs; ++j) {
     const uint64_t row = first + (uint64_t)j;
@@ -468,7 +495,7 @@ static double decode_glu(int kind, double g, double u, double limit) {
 int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, const orc_decode_operand* up,
                           uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
                           uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
-  if (decoder < 0 || decoder >= ORC_DECODER_AFFINE_SPLIT || glu < 0 || glu > 3 || gate->k != up->k) return 1;
+  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT || glu < 0 || glu > 3 || gate->k != up->k) return 1;
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
   for (int64_t j = 0; j < (int64_t)outputs; ++j) {
     const uint64_t grow = gate_first + (uint64_t)j, urow = up_first + (uint64_t)j;

@@ -135,7 +135,8 @@ def test_decode_vector_refuses_bad_operands():
     def run(decoder, w, first=0, outputs=8, x=0x4000, rows=1, x_stride=256, y=0x5000, y_stride=64):
         return lib.llmp_hip_decode_vector(decoder, C.byref(w), first, outputs, x, rows, x_stride, y, y_stride, None)
 
-    assert run(11, operand()) > 0 and b"no kernel" in lib.llmp_hip_last_error()       # affine
+    assert run(12, operand()) > 0 and b"no kernel" in lib.llmp_hip_last_error()
+    assert run(11, operand()) > 0 and b"affine" in lib.llmp_hip_last_error()           # no group, width or scale type
     assert run(3, operand(), rows=17) > 0 and b"1 to 16" in lib.llmp_hip_last_error()
     assert run(3, operand(), first=60, outputs=8) > 0
     assert run(3, operand(scales=None)) > 0 and b"scales" in lib.llmp_hip_last_error()
@@ -153,4 +154,4 @@ def test_decode_vector_refuses_bad_operands():
     assert glu(3, 3, 7) > 0 and b"GLU" in lib.llmp_hip_last_error()
     rows = lambda **kw: lib.llmp_hip_decode_rows(kw.get("decoder", 3), C.byref(operand()), kw.get("ids", 0x6000),
                                                  kw.get("count", 4), kw.get("out", 0x7000), kw.get("stride", 256), None, None)
-    assert rows(decoder=11) > 0 and rows(ids=None) > 0 and rows(count=0) > 0 and rows(out=0x7004) > 0 and rows(stride=250) > 0
+    assert rows(decoder=12) > 0 and rows(ids=None) > 0 and rows(count=0) > 0 and rows(out=0x7004) > 0 and rows(stride=250) > 0

@@ -1,4 +1,4 @@
-"""Parity of llmp.decode.vector (HIP, through the C ABI) against the CPU oracle: every decoder,
+"""Parity of llmp.decode.vector, vector_glu and rows (HIP, through the C ABI) against the CPU oracle: every decoder,
 1 to 16 input rows, row windows, strides, tensor scales, undefined block scales. Float outputs to
 a maximum relative error of 1e-3 (the accumulation order is the only difference: both sides
 decode every value exactly)."""
@@ -112,7 +112,7 @@ def test_refusals(device):
     with pytest.raises(ops.KernelFailure) as e:
         ops.decode_vector(3, w, x)
     assert e.value.rejected
-    with pytest.raises(ops.KernelFailure):  # the affine decoder is not built
+    with pytest.raises(ops.KernelFailure):  # an affine operand without its group, width and scale type
         ops.decode_vector(11, w, x[:1])
     with pytest.raises(ops.KernelFailure):  # rows [6, 10) of 8
         ops.decode_vector(3, w, x[:1], first=6, outputs=4)
@@ -179,3 +179,26 @@ def test_rows_gather_is_the_decoded_rows_bit_for_bit(device, decoder):
     assert int(bad.item()) == 1
     assert np.all(got[1] == 0) and np.all(got[2] == 0)
     assert np.array_equal(got[[0, 3]].view(np.uint32), dense[[5, 12]].astype(np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("scale", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("zero_point", [False, True])
+def test_affine_decoder(device, bits, scale, zero_point):
+    """affine.split (src/kernels/decode/decoders.cuh:241-345 of the reference): rows gathered bit for bit, the
+    vector product and its GLU form to 1e-3."""
+    n, k, group = 66, 1024, 64 if bits == 4 else 128
+    w = synth.affine_weight(n, k, 810 + bits, bits=bits, group=group, scale=scale, zero_point=zero_point, tensor_scales=2)
+    wd = {key: (torch.from_numpy(np.ascontiguousarray(v)).to(device) if isinstance(v, np.ndarray) else v) for key, v in w.items()}
+    dense = oracle.decode_rows_of(11, w) * w["tensor_scale"][np.arange(n) // w["rows_per_scale"]][:, None]
+    ids = torch.arange(n, dtype=torch.int32, device=device)
+    got = ops.decode_rows(11, wd, ids).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), dense.astype(np.float32).view(np.uint32))
+    x = synth.activations(3, k, 811)
+    xd = torch.from_numpy(x).to(device)
+    ok, worst = rel_close(ops.decode_vector(11, wd, xd).cpu().numpy(), oracle.decode_vector(11, w, x), 1e-3)
+    assert ok, worst
+    want = oracle.decode_vector_glu(11, w, w, x * 0.25, 2, gate_first=0, up_first=33, outputs=33)
+    got = ops.decode_vector_glu(11, wd, wd, xd * 0.25, 2, gate_first=0, up_first=33, outputs=33).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst

@@ -387,6 +387,42 @@ def test_decode_products_values_and_layouts():
     np.testing.assert_allclose(oracle.decode_vector(6, w, x, first=20, outputs=30), want[:, 20:50], rtol=1e-6, atol=1e-9)
 
 
+def test_affine_decoder_against_a_numpy_restatement():
+    """The affine encoding (src/kernels/reference/decode.cc:173-220): codes of 4 or 8 bits little-endian along the
+    row, s * q + b rounded once or s * (q - z), scales F16 / BF16 / F32 a group; restated with numpy (the fused
+    multiply-add as an exact double product and sum rounded once)."""
+    from llmp_amd import synth
+    n, k, group = 5, 256, 64
+    for bits in (4, 8):
+        for scale in ("f16", "bf16", "f32"):
+            for zero_point in (False, True):
+                w = synth.affine_weight(n, k, 61, bits=bits, group=group, scale=scale, zero_point=zero_point)
+                got = oracle.decode_rows_of(11, w)
+                codes = w["data"] if bits == 8 else np.stack([w["data"] & 15, w["data"] >> 4], axis=-1).reshape(n, k)
+                kind = w["scale_type"] & 0x7F
+
+                def floats(raw):
+                    if kind == 2:
+                        return synth.bf16_to_f32(raw.view(np.uint16)).reshape(n, -1)
+                    return raw.view(np.float16 if kind == 1 else np.float32).astype(np.float32).reshape(n, -1)
+
+                sc = np.repeat(floats(w["scales"]), group, axis=1)
+                if zero_point:
+                    z = w["biases"] if bits == 8 else np.stack([w["biases"] & 15, w["biases"] >> 4], axis=-1).reshape(n, -1)
+                    z = np.repeat(z[:, :k // group].astype(np.int32), group, axis=1)
+                    want = sc * (codes.astype(np.int32) - z).astype(np.float32)
+                else:
+                    b = np.repeat(floats(w["biases"]), group, axis=1)
+                    want = (sc.astype(np.float64) * codes.astype(np.float64) + b.astype(np.float64)).astype(np.float32)
+                assert np.array_equal(got, want), (bits, scale, zero_point)
+    # By hand: 4-bit codes 0..15 in one group of 32 (twice), s = 0.5, b = -4: values -4 .. 3.5.
+    w = {"k": 32, "data": np.array([[(2 * i % 16) | ((2 * i + 1) % 16) << 4 for i in range(16)]], dtype=np.uint8),
+         "scales": np.array([0.5], dtype=np.float16).view(np.uint8).reshape(1, 2),
+         "biases": np.array([-4.0], dtype=np.float16).view(np.uint8).reshape(1, 2),
+         "group": 32, "bits": 4, "scale_type": 1, "scale_row_bytes": 2}
+    assert np.array_equal(oracle.decode_rows_of(11, w)[0], 0.5 * (np.arange(32) % 16) - 4.0)
+
+
 def test_decode_glu_products_against_closed_forms():
     """orc_decode_vector_glu: glu(gate . x, up . x) with the four functions of the reference's CPU executor
     (src/kernels/reference/exec.cc:248-262), here from scipy's erf and numpy, over the oracle's own plain products."""
