@@ -330,6 +330,17 @@ int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_operand* gate
 int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* weight, const int32_t* ids, uint64_t count, float* out,
                          uint64_t out_stride, int32_t* bad, void* stream);
 
+/* RunGrouped of src/kernels/decode/products.h:141-170: for each expert e its pairs p in [offsets[e],
+ * offsets[e + 1]) compute y[pair_out[p] (or p)][j] = sum_k W_e[first + j][k] x[pair_rows[p]][k]. `experts` is a
+ * device array of experts_count operands (any base address each) of the format's decoder, K (`k`) and N
+ * (`n`); offsets (experts_count + 1), pair_rows and pair_out (or null) are device I32 arrays. The device skips
+ * an expert whose operand's K or N is not the format's, a pair past `pairs`, and one naming a row past x_rows or
+ * y_rows (its output row is left untouched). One launch; `rows_hint` (the reference's tile choice) is unused. */
+int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* experts, uint64_t experts_count, uint32_t k, uint32_t n,
+                            uint64_t first, uint64_t outputs, const int32_t* offsets, const int32_t* pair_rows,
+                            const int32_t* pair_out, uint64_t pairs, const float* x, uint64_t x_rows, uint64_t x_stride,
+                            float* y, uint64_t y_rows, uint64_t y_stride, uint64_t rows_hint, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -200,6 +200,33 @@ inline KernelFailure RunRows(const RowsGather& g, void* stream) {
                                          g.bad, stream));
 }
 
+// GroupedProduct and RunGrouped (src/kernels/decode/products.h:141-170); `k` and `n` are the format's.
+struct GroupedProduct {
+  DecoderId decoder = DecoderId::kBf16Dense;
+  std::uint32_t k = 0;
+  std::uint32_t n = 0;
+  const Operand* experts = nullptr;  // device memory
+  std::uint64_t experts_count = 0;
+  std::uint64_t first = 0;
+  std::uint64_t outputs = 0;
+  const std::int32_t* offsets = nullptr;
+  const std::int32_t* pair_rows = nullptr;
+  const std::int32_t* pair_out = nullptr;
+  std::uint64_t pairs = 0;
+  const float* x = nullptr;
+  std::uint64_t x_rows = 0;
+  std::uint64_t x_stride = 0;
+  float* y = nullptr;
+  std::uint64_t y_rows = 0;
+  std::uint64_t y_stride = 0;
+  std::uint64_t rows_hint = 0;
+};
+inline KernelFailure RunGrouped(const GroupedProduct& p, void* stream) {
+  return FromStatus(llmp_hip_decode_grouped(static_cast<int>(p.decoder), p.experts, p.experts_count, p.k, p.n, p.first,
+                                            p.outputs, p.offsets, p.pair_rows, p.pair_out, p.pairs, p.x, p.x_rows,
+                                            p.x_stride, p.y, p.y_rows, p.y_stride, p.rows_hint, stream));
+}
+
 }  // namespace decode
 
 namespace exl3 {

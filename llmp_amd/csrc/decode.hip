@@ -322,6 +322,104 @@ __global__ __launch_bounds__(256) void DecodeRowsKernel(const llmp_decode_operan
   }
 }
 
+// An expert worklist's products (products.h:141-170): expert e = blockIdx.y takes its pairs
+// offsets[e] .. offsets[e + 1], T at a time: their input rows staged, then every wave its output
+// row pairs. An expert whose operand's K or N is not the format's is skipped, as are pairs past
+// `pairs` and pairs naming a row past x_rows or y_rows.
+struct GroupedArgs {
+  const llmp_decode_operand* experts;
+  uint32_t k, n, first, outputs;
+  const int32_t* offsets;
+  const int32_t* pair_rows;
+  const int32_t* pair_out;  // or null: pair p writes row p
+  uint32_t pairs, x_rows, y_rows;
+  const float* x;
+  uint64_t x_stride;
+  float* y;
+  uint64_t y_stride;
+};
+
+template <int D, int T>
+__global__ __launch_bounds__(kDecodeWaves * 64) void DecodeGroupedKernel(const GroupedArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int32_t out_row[T];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t waves = blockDim.x / 64;
+  const llmp_decode_operand w = a.experts[blockIdx.y];
+  if (w.k != a.k || w.rows != a.n) return;  // uniform over the workgroup
+  const uint32_t segs = a.k / 16u, quarters = a.k / 4u;
+  int64_t begin = a.offsets[blockIdx.y], end = a.offsets[blockIdx.y + 1];
+  if (begin < 0) begin = 0;
+  if (end > static_cast<int64_t>(a.pairs)) end = a.pairs;
+  const uint32_t row_pairs = (a.outputs + kRowsAWave - 1) / kRowsAWave;
+  for (int64_t p0 = begin; p0 < end; p0 += T) {
+    const int m = static_cast<int>(end - p0 < T ? end - p0 : T);
+    if (p0 > begin) __syncthreads();  // the last pass's readers of the staged rows
+    // Where each pair's sums go (-1: nowhere), and its input row (zeros for a pair that is skipped).
+    if (tid < m) {
+      const int64_t p = p0 + tid;
+      const int64_t from = a.pair_rows[p];
+      const int64_t to = a.pair_out != nullptr ? a.pair_out[p] : p;
+      out_row[tid] = from >= 0 && from < a.x_rows && to >= 0 && to < a.y_rows ? static_cast<int32_t>(to) : -1;
+    }
+    for (uint32_t c = tid; c < m * quarters; c += blockDim.x) {
+      const uint32_t t = c / quarters, q = c - t * quarters;
+      const int64_t from = a.pair_rows[p0 + t];
+      float4 piece = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (from >= 0 && from < a.x_rows) piece = *reinterpret_cast<const float4*>(a.x + from * a.x_stride + q * 4u);
+      *reinterpret_cast<float4*>(lds + static_cast<size_t>(t * segs + q / 4u) * kSegmentStride + (q & 3u) * 16u) = piece;
+    }
+    __syncthreads();
+    for (uint32_t pair = blockIdx.x * waves + wave; pair < row_pairs; pair += gridDim.x * waves) {
+      const uint32_t out0 = pair * kRowsAWave;
+      float acc[kRowsAWave][T];
+#pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[r][t] = 0.0f;
+      }
+      for (uint32_t seg = lane; seg < segs; seg += 64) {
+        float v[kRowsAWave][16], s[kRowsAWave];
+#pragma unroll
+        for (int r = 0; r < kRowsAWave; ++r) LoadSegment<D>(w, a.first + min(out0 + r, a.outputs - 1), seg, v[r], s[r]);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          if (t < m) {
+            const float4* xs = reinterpret_cast<const float4*>(lds + static_cast<size_t>(t * segs + seg) * kSegmentStride);
+            const float4 x0 = xs[0], x1 = xs[1], x2 = xs[2], x3 = xs[3];
+            const float x[16] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+            for (int r = 0; r < kRowsAWave; ++r) {
+              float dot = 0.0f;
+#pragma unroll
+              for (int i = 0; i < 16; ++i) dot = fmaf(v[r][i], x[i], dot);
+              acc[r][t] = fmaf(dot, s[r], acc[r][t]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+        const uint32_t out = out0 + r;
+        float scale = 1.0f;
+        if (w.tensor_scale != nullptr && out < a.outputs) scale = w.tensor_scale[(a.first + out) / w.rows_per_scale];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          if (t < m) {
+            float total = acc[r][t];
+#pragma unroll
+            for (int mask = 32; mask >= 1; mask >>= 1) total += ShflXor(total, mask);
+            const int32_t to = out_row[t];
+            if (lane == 0 && out < a.outputs && to >= 0) a.y[static_cast<int64_t>(to) * a.y_stride + out] = total * scale;
+          }
+        }
+      }
+    }
+  }
+}
+
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
 template <int D, int T, bool kGlu>
@@ -532,4 +630,87 @@ extern "C" int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* w, c
 #undef LLMP_DECODER
   }
   return LaunchStatus("decode.rows");
+}
+
+namespace llmp_hip {
+namespace {
+
+template <int D, int T>
+void LaunchGrouped(const GroupedArgs& a, dim3 grid, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeGroupedKernel<D, T>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDecodeLdsLimit));
+    sized = true;
+  }
+  hipLaunchKernelGGL((DecodeGroupedKernel<D, T>), grid, dim3(kDecodeWaves * 64), DecodeLds(T, a.k), stream, a);
+}
+
+template <int D>
+void LaunchGroupedDecoder(const GroupedArgs& a, int pass, dim3 grid, hipStream_t stream) {
+  switch (pass) {
+    case 1: LaunchGrouped<D, 1>(a, grid, stream); break;
+    case 2: LaunchGrouped<D, 2>(a, grid, stream); break;
+    default: LaunchGrouped<D, 4>(a, grid, stream); break;
+  }
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+extern "C" int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* experts, uint64_t experts_count, uint32_t k,
+                                       uint32_t n, uint64_t first, uint64_t outputs, const int32_t* offsets,
+                                       const int32_t* pair_rows, const int32_t* pair_out, uint64_t pairs, const float* x,
+                                       uint64_t x_rows, uint64_t x_stride, float* y, uint64_t y_rows, uint64_t y_stride,
+                                       uint64_t rows_hint, void* stream) {
+  (void)rows_hint;  // picks the reference's tile; the passes here are of up to four pairs whatever it is
+  if (decoder < 0 || decoder > LLMP_DECODER_AFFINE_SPLIT) return Refuse(1, "decode.grouped: decoder %d has no kernel", decoder);
+  if (experts == nullptr || offsets == nullptr || pair_rows == nullptr || x == nullptr || y == nullptr)
+    return Refuse(1, "decode.grouped: null operand");
+  if (experts_count == 0 || experts_count > 65535) return Refuse(1, "decode.grouped: 1 to 65535 experts");
+  if (k == 0 || k % KMultiple(decoder) != 0)
+    return Refuse(1, "decode.grouped: k %u is not a multiple of the decoder's %u", k, KMultiple(decoder));
+  if (outputs == 0 || first > n || outputs > n - first)
+    return Refuse(1, "decode.grouped: outputs [%llu, %llu) of %u", static_cast<unsigned long long>(first),
+                  static_cast<unsigned long long>(first + outputs), n);
+  if (pairs == 0 || pairs >= (uint64_t{1} << 31) || x_rows >= (uint64_t{1} << 31) || y_rows >= (uint64_t{1} << 31))
+    return Refuse(1, "decode.grouped: 1 to 2^31 pairs and rows");
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_stride % 4 != 0 || x_stride < k || y_stride < outputs ||
+      reinterpret_cast<uintptr_t>(y) % 4 != 0 || reinterpret_cast<uintptr_t>(experts) % 8 != 0)
+    return Refuse(1, "decode.grouped: input rows are 16-byte aligned, a multiple of 4 floats apart and at least k long");
+  int pass = 4;
+  while (pass > 1 && DecodeLds(pass, k) > kDecodeLdsLimit) pass /= 2;
+  if (DecodeLds(pass, k) > kDecodeLdsLimit)
+    return Refuse(1, "decode.grouped: a row of %u values does not fit the staging area (16384 at most)", k);
+  GroupedArgs a;
+  a.experts = experts;
+  a.k = k, a.n = n, a.first = static_cast<uint32_t>(first), a.outputs = static_cast<uint32_t>(outputs);
+  a.offsets = offsets, a.pair_rows = pair_rows, a.pair_out = pair_out;
+  a.pairs = static_cast<uint32_t>(pairs), a.x_rows = static_cast<uint32_t>(x_rows), a.y_rows = static_cast<uint32_t>(y_rows);
+  a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
+  const int cus = llmp_hip_compute_units();
+  uint64_t groups = 2 * static_cast<uint64_t>(cus > 0 ? cus : 256) / experts_count;
+  const uint64_t most = ((outputs + kRowsAWave - 1) / kRowsAWave + kDecodeWaves - 1) / kDecodeWaves;
+  if (groups > most) groups = most;
+  if (groups < 1) groups = 1;
+  const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(experts_count));
+  const auto s = static_cast<hipStream_t>(stream);
+  switch (decoder) {
+#define LLMP_DECODER(ID) \
+  case ID: LaunchGroupedDecoder<ID>(a, pass, grid, s); break;
+    LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_F16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_Q8_0_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_INTERLEAVED)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_GGML_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_AFFINE_SPLIT)
+#undef LLMP_DECODER
+  }
+  return LaunchStatus("decode.grouped");
 }

@@ -417,3 +417,21 @@ def decode_rows(decoder, weight, ids, bad=None):
     _lib.check(lib.llmp_hip_decode_rows(decoder, C.byref(op), _ptr(ids), ids.numel(), _ptr(out), out.stride(0),
                                         _ptr(bad) if bad is not None else None, _stream()))
     return out
+
+
+def decode_grouped(decoder, experts, k, n, offsets, pair_rows, x, y, pair_out=None, first=0, outputs=None):
+    """llmp.decode.grouped: an expert worklist's products. `experts` is a list of weights (dicts of device tensors,
+    one matrix each); offsets (int32 [experts + 1]), pair_rows and pair_out (int32 [pairs]) are device tensors; `y`
+    (float32 [y_rows, outputs]) is updated in place at the rows the pairs name."""
+    import numpy as np
+    lib = _lib.load()
+    table = (DecodeOperand * len(experts))(*[_decode_operand(w) for w in experts])
+    raw = np.frombuffer(bytes(table), dtype=np.uint8).copy()
+    table_d = torch.from_numpy(raw).to(x.device)  # the operands, in device memory
+    outputs = n - first if outputs is None else outputs
+    _lib.check(lib.llmp_hip_decode_grouped(decoder, _ptr(table_d), len(experts), k, n, first, outputs, _ptr(offsets),
+                                           _ptr(pair_rows), _ptr(pair_out) if pair_out is not None else None,
+                                           pair_rows.numel(), _ptr(x), x.shape[0], x.stride(0), _ptr(y), y.shape[0],
+                                           y.stride(0), 0, _stream()))
+    torch.cuda.current_stream().synchronize()  # table_d must outlive the launch
+    return y

@@ -387,3 +387,22 @@ def decode_vector_glu(decoder, gate, up, x, glu, limit=0.0, gate_first=0, up_fir
     if rc != 0:
         raise ValueError("no such product")
     return y
+
+
+_sig("orc_decode_grouped", _int, _int, C.POINTER(DecodeOperand), _u64, C.c_uint32, C.c_uint32, _u64, _u64, _vp, _vp, _vp,
+     _u64, _vp, _u64, _u64, _vp, _u64, _u64)
+
+
+def decode_grouped(decoder, experts, k, n, offsets, pair_rows, x, y, pair_out=None, first=0, outputs=None):
+    """llmp.decode.grouped on the CPU: `experts` a list of weights, `y` (float32 [y_rows, outputs]) updated in place."""
+    ops_ = (DecodeOperand * len(experts))(*[decode_operand(w) for w in experts])
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    outputs = n - first if outputs is None else outputs
+    offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+    pair_rows = np.ascontiguousarray(pair_rows, dtype=np.int32)
+    pair_out = None if pair_out is None else np.ascontiguousarray(pair_out, dtype=np.int32)
+    rc = lib.orc_decode_grouped(decoder, ops_, len(experts), k, n, first, outputs, _p(offsets), _p(pair_rows), _p(pair_out),
+                                len(pair_rows), _p(x), x.shape[0], x.shape[1], _p(y), y.shape[0], y.shape[1])
+    if rc != 0:
+        raise ValueError("no such decoder")
+    return y

@@ -514,6 +514,33 @@ int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t 
   return 0;
 }
 
+/* products.h:141-170 */
+int orc_decode_grouped(int decoder, const orc_decode_operand* experts, uint64_t experts_count, uint32_t k, uint32_t n,
+                       uint64_t first, uint64_t outputs, const int32_t* offsets, const int32_t* pair_rows,
+                       const int32_t* pair_out, uint64_t pairs, const float* x, uint64_t x_rows, uint64_t x_stride, float* y,
+                       uint64_t y_rows, uint64_t y_stride) {
+  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT) return 1;
+  for (uint64_t e = 0; e < experts_count; ++e) {
+    const orc_decode_operand* w = &experts[e];
+    if (w->k != k || w->rows != n) continue;
+    int64_t begin = offsets[e], end = offsets[e + 1];
+    if (begin < 0) begin = 0;
+    if (end > (int64_t)pairs) end = (int64_t)pairs;
+    for (int64_t p = begin; p < end; ++p) {
+      const int64_t from = pair_rows[p], to = pair_out != NULL ? pair_out[p] : p;
+      if (from < 0 || from >= (int64_t)x_rows || to < 0 || to >= (int64_t)y_rows) continue;
+      for (uint64_t j = 0; j < outputs; ++j) {
+        const uint64_t row = first + j;
+        const double scale = w->tensor_scale != NULL ? (double)w->tensor_scale[row / w->rows_per_scale] : 1.0;
+        double sum = 0;
+        for (uint64_t c = 0; c < k; ++c) sum += (double)orc_decode_value(decoder, w, row, c) * (double)x[(uint64_t)from * x_stride + c];
+        y[(uint64_t)to * y_stride + j] = (float)(sum * scale);
+      }
+    }
+  }
+  return 0;
+}
+
 /* -------------------------------------------------------------------- GLU */
 
 static double sigmoid_d(double x) { return 1.0 / (1.0 + exp(-x)); }

@@ -106,6 +106,13 @@ int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t 
                           uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
                           uint64_t x_stride, float* y, uint64_t y_stride, int threads);
 
+/* RunGrouped, products.h:141-170: an expert worklist's products; experts whose K or N differ, pairs past
+ * `pairs` and pairs naming rows past x_rows or y_rows are skipped. */
+int orc_decode_grouped(int decoder, const orc_decode_operand* experts, uint64_t experts_count, uint32_t k, uint32_t n,
+                       uint64_t first, uint64_t outputs, const int32_t* offsets, const int32_t* pair_rows,
+                       const int32_t* pair_out, uint64_t pairs, const float* x, uint64_t x_rows, uint64_t x_stride, float* y,
+                       uint64_t y_rows, uint64_t y_stride);
+
 /* ---- GLU: src/kernels/reference/exec.cc:206-214,248-262 ---- */
 enum { ORC_GLU_NONE = 0, ORC_GLU_SWIGLU = 1, ORC_GLU_SWIGLU_CLAMP = 2, ORC_GLU_GEGLU = 3 };
 double orc_glu(int kind, double gate, double up, double limit);

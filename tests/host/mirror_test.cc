@@ -124,6 +124,8 @@ void HostChecks() {
   EXPECT(hipk::decode::RunVectorGlu(glu_product, nullptr) == hipk::KernelFailure::kRejected);
   hipk::decode::RowsGather gather;
   EXPECT(hipk::decode::RunRows(gather, nullptr) == hipk::KernelFailure::kRejected);
+  hipk::decode::GroupedProduct grouped;
+  EXPECT(hipk::decode::RunGrouped(grouped, nullptr) == hipk::KernelFailure::kRejected);
   hipk::exl3::MultiLinearOperands multi;
   EXPECT(hipk::exl3::MultiLinear(multi, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
   EXPECT(hipk::exl3::ScratchBytes(multi) == 0);

@@ -155,3 +155,19 @@ def test_decode_vector_refuses_bad_operands():
     rows = lambda **kw: lib.llmp_hip_decode_rows(kw.get("decoder", 3), C.byref(operand()), kw.get("ids", 0x6000),
                                                  kw.get("count", 4), kw.get("out", 0x7000), kw.get("stride", 256), None, None)
     assert rows(decoder=12) > 0 and rows(ids=None) > 0 and rows(count=0) > 0 and rows(out=0x7004) > 0 and rows(stride=250) > 0
+
+
+def test_decode_grouped_refuses_bad_operands():
+    lib = _lib.load()
+
+    def run(decoder=3, experts=0x1000, count=4, k=256, n=64, first=0, outputs=64, offsets=0x2000, rows=0x3000,
+            pairs=8, x=0x4000, x_stride=256, y=0x5000, y_stride=64):
+        return lib.llmp_hip_decode_grouped(decoder, experts, count, k, n, first, outputs, offsets, rows, None, pairs, x,
+                                           16, x_stride, y, 8, y_stride, 0, None)
+
+    assert run(decoder=12) > 0 and b"no kernel" in lib.llmp_hip_last_error()
+    assert run(experts=None) > 0 and run(count=0) > 0 and run(pairs=0) > 0
+    assert run(decoder=4, k=32) > 0 and b"multiple" in lib.llmp_hip_last_error()
+    assert run(first=60, outputs=8) > 0 and b"outputs" in lib.llmp_hip_last_error()
+    assert run(x=0x4004) > 0 and run(x_stride=250) > 0
+    assert run(k=32768, x_stride=32768) > 0 and b"staging" in lib.llmp_hip_last_error()

@@ -202,3 +202,47 @@ def test_affine_decoder(device, bits, scale, zero_point):
     got = ops.decode_vector_glu(11, wd, wd, xd * 0.25, 2, gate_first=0, up_first=33, outputs=33).cpu().numpy()
     ok, worst = rel_close(got, want, 1e-3)
     assert ok, worst
+
+
+@pytest.mark.parametrize("decoder", [0, 3, 6, 8, 11])
+def test_grouped_products_match_oracle(device, decoder):
+    """RunGrouped (src/kernels/decode/products.h:141-170 of the reference): an expert worklist with empty experts,
+    experts of one to nine pairs, output rows by pair or by pair_out, and what the device skips: an operand of
+    another K, pairs naming rows outside x or y (their output rows stay as they were)."""
+    experts, n, k = 7, 48, 512
+    make = (lambda seed: synth.affine_weight(n, k, seed, bits=4, group=64)) if decoder == 11 else \
+           (lambda seed: synth.decode_weight(decoder, n, k, seed, tensor_scales=2))
+    weights = [make(820 + e) for e in range(experts)]
+    weights[5] = (synth.affine_weight(n, 256, 830, bits=4, group=64) if decoder == 11
+                  else synth.decode_weight(decoder, n, 256, 830))  # another K: skipped
+    counts = [3, 0, 9, 1, 4, 2, 5]
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    pairs = int(offsets[-1])
+    g = synth.rng(831)
+    x = synth.activations(10, k, 832)
+    pair_rows = g.integers(0, 10, size=pairs).astype(np.int32)
+    pair_rows[4] = 10   # past x_rows: skipped
+    pair_out = g.permutation(pairs + 3)[:pairs].astype(np.int32)
+    pair_out[7] = pairs + 3  # past y_rows: skipped
+    to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    dev_weights = [{key: (to_dev(v) if isinstance(v, np.ndarray) else v) for key, v in w.items() if key != "plain"}
+                   for w in weights]
+    for out in (None, pair_out):
+        rows_y = pairs if out is None else pairs + 3
+        want = np.full((rows_y, n), 7.0, dtype=np.float32)
+        oracle.decode_grouped(decoder, weights, k, n, offsets, pair_rows, x, want, pair_out=out)
+        y = torch.full((rows_y, n), 7.0, dtype=torch.float32, device=device)
+        ops.decode_grouped(decoder, dev_weights, k, n, to_dev(offsets), to_dev(pair_rows), to_dev(x), y,
+                           pair_out=None if out is None else to_dev(out))
+        got = y.cpu().numpy()
+        untouched = want == 7.0
+        assert np.array_equal(got == 7.0, untouched)
+        ok, worst = rel_close(got[~untouched], want[~untouched], 1e-3)
+        assert ok, worst
+    # A window of output rows.
+    want = np.zeros((pairs, 20), dtype=np.float32)
+    oracle.decode_grouped(decoder, weights, k, n, offsets, pair_rows, x, want, first=9, outputs=20)
+    y = torch.zeros((pairs, 20), dtype=torch.float32, device=device)
+    ops.decode_grouped(decoder, dev_weights, k, n, to_dev(offsets), to_dev(pair_rows), to_dev(x), y, first=9, outputs=20)
+    ok, worst = rel_close(y.cpu().numpy(), want, 1e-3)
+    assert ok, worst
