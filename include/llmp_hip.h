@@ -341,6 +341,13 @@ int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* experts, uin
                             const int32_t* pair_out, uint64_t pairs, const float* x, uint64_t x_rows, uint64_t x_stride,
                             float* y, uint64_t y_rows, uint64_t y_stride, uint64_t rows_hint, void* stream);
 
+/* RunMatrix of src/kernels/decode/products.h:111-118: the same product for 1 to 65535 * 64 input rows on the
+ * matrix cores (`path` 0, MatrixPath::kMma): the decoded weights and the inputs are rounded to the
+ * decoder's matrix element (F16 for F16 and Q8_0 weights, BF16 for the others: products.h:27-33) and
+ * summed in F32. `path` 1 (kFma, for devices without matrix instructions) is refused. One launch. */
+int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* weight, uint64_t first, uint64_t outputs, const float* x,
+                           uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int path, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

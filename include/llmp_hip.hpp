@@ -156,6 +156,12 @@ struct Product {
   float* y = nullptr;
   std::uint64_t y_stride = 0;
 };
+// RunMatrix (src/kernels/decode/products.h:111-118): MatrixPath::kMma is path 0, kFma (refused here) 1.
+enum class MatrixPath : std::uint8_t { kMma, kFma };
+inline KernelFailure RunMatrix(const Product& p, MatrixPath path, void* stream) {
+  return FromStatus(llmp_hip_decode_matrix(static_cast<int>(p.decoder), &p.weight, p.first, p.outputs, p.x, p.rows,
+                                           p.x_stride, p.y, p.y_stride, static_cast<int>(path), stream));
+}
 inline KernelFailure RunVector(const Product& p, void* stream) {
   return FromStatus(llmp_hip_decode_vector(static_cast<int>(p.decoder), &p.weight, p.first, p.outputs, p.x, p.rows,
                                            p.x_stride, p.y, p.y_stride, stream));

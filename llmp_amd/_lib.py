@@ -109,6 +109,8 @@ SYMBOLS = {
     "llmp_hip_decode_grouped": (_int, [_int, _vp, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, _vp, _vp, _vp,
                                        C.c_uint64, _vp, C.c_uint64, C.c_uint64, _vp, C.c_uint64, C.c_uint64, C.c_uint64,
                                        _vp]),
+    "llmp_hip_decode_matrix": (_int, [_int, C.POINTER(DecodeOperand), C.c_uint64, C.c_uint64, _vp, C.c_uint64,
+                                      C.c_uint64, _vp, C.c_uint64, _int, _vp]),
     "llmp_hip_exl3_multi_linear_scratch": (C.c_size_t, [C.POINTER(Exl3MultiLinear)]),
     "llmp_hip_exl3_multi_linear": (_int, [C.POINTER(Exl3MultiLinear), _vp, C.c_size_t, _vp]),
 }

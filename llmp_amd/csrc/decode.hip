@@ -420,6 +420,141 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeGroupedKernel(const G
   }
 }
 
+// ------------------------------------------------------------------ matrix
+// RunMatrix's tensor-core path (products.h:111-118, templates.cuh's Matrix): tiles of 64 outputs by 64
+// input rows, the weights decoded and, like the inputs, rounded to the decoder's matrix element
+// (F16 for F16 and Q8_0 weights, BF16 otherwise), F32 sums on the matrix cores
+// (v_mfma_f32_16x16x32: D[input row][output] += x[input row][k] W[output][k]).
+// A workgroup takes 256 outputs by 64 input rows, a wave 64 of the outputs in four groups of 16; a lane (n = lane % 16, q = lane / 16) decodes segment
+// 4 c + q of output n of each group for chunk c of 64 values of K: its sixteen values are the second operands of
+// two instructions whose k labels run over the four lanes' segments, and the inputs' first
+// operands follow the same labels, so no lane exchange is needed. The inputs' chunk is staged in
+// LDS in the matrix element, rows 144 bytes apart (conflict-free 16-byte reads), in two buffers: the
+// next chunk's inputs and weights are loaded while this one multiplies, one barrier a chunk.
+typedef short Short8 __attribute__((ext_vector_type(8)));
+typedef float Float4 __attribute__((ext_vector_type(4)));
+constexpr int kMatrixTile = 64;        // input rows a workgroup
+constexpr int kMatrixRowBytes = 144;   // 64 two-byte elements and 16 bytes
+
+// Nearest even, by the hardware's conversions (v_cvt_f16_f32, v_cvt_pk_bf16_f32).
+template <bool kHalf>
+__device__ __forceinline__ uint32_t ToElement(float v) {
+  if constexpr (kHalf) {
+    return FloatToHalfBits(v);
+  } else {
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+  }
+}
+
+// G: groups of 16 outputs a wave (a workgroup takes 64 G outputs by 64 input rows).
+template <int D, int G>
+__global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, const uint32_t rows) {
+  constexpr bool kHalf = D == LLMP_DECODER_F16_DENSE || D == LLMP_DECODER_Q8_0_BLOCKS;
+  constexpr int kTileBytes = kMatrixTile * kMatrixRowBytes;
+  __shared__ __attribute__((aligned(16))) uint8_t tiles[2 * kTileBytes];  // this chunk's inputs and the next's
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, q = lane >> 4;
+  const uint32_t out0 = (blockIdx.x * 4 + wave) * (16 * G), t0 = blockIdx.y * kMatrixTile;
+  const uint32_t segs = a.w.k / 16u, chunks = (segs + 3u) / 4u;
+  Float4 acc[G][4];  // [outputs' group][input rows' group]
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  // A chunk's share of a thread: four pieces of four input values, and the lane's segment of each of
+  // its groups of outputs, scaled and rounded to the element (two operands of eight).
+  auto load_inputs = [&](uint32_t chunk, float4 (&piece)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + i * 256;
+      const uint32_t row = c >> 4, column = chunk * 64u + (c & 15u) * 4u;
+      piece[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (t0 + row < rows && column < a.w.k) piece[i] = *reinterpret_cast<const float4*>(a.x + (t0 + row) * a.x_stride + column);
+    }
+  };
+  auto load_weights = [&](uint32_t chunk, Short8 (&b)[G][2]) {
+    const uint32_t seg = chunk * 4u + q;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float v[16] = {};
+      float s = 0.0f;
+      // An output past the last is a copy of it, not stored.
+      if (seg < segs) LoadSegment<D>(a.w, a.first + min(out0 + 16 * g + n, a.outputs - 1), seg, v, s);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b[g][j][i] = static_cast<short>(ToElement<kHalf>(v[8 * j + i] * s));
+      }
+    }
+  };
+
+  float4 piece[4];
+  Short8 b[G][2];
+  load_inputs(0, piece);
+  load_weights(0, b);
+  for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+    uint8_t* tile = tiles + (chunk & 1u) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + i * 256;
+      uint2 packed;
+      packed.x = ToElement<kHalf>(piece[i].x) | (ToElement<kHalf>(piece[i].y) << 16);
+      packed.y = ToElement<kHalf>(piece[i].z) | (ToElement<kHalf>(piece[i].w) << 16);
+      *reinterpret_cast<uint2*>(tile + (c >> 4) * kMatrixRowBytes + (c & 15u) * 8u) = packed;
+    }
+    // One barrier a chunk: this buffer is complete, and the other's readers (the last chunk's) are done.
+    __syncthreads();
+    Short8 next[G][2];
+    if (chunk + 1 < chunks) {  // the next chunk's loads are in flight while this one multiplies
+      load_inputs(chunk + 1, piece);
+      load_weights(chunk + 1, next);
+    }
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const U32x4* mine = reinterpret_cast<const U32x4*>(tile + (16 * m + n) * kMatrixRowBytes + q * 32);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const U32x4 x8 = mine[j];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if constexpr (kHalf) {
+            typedef _Float16 Half8 __attribute__((ext_vector_type(8)));
+            acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(Half8, x8),
+                                                               __builtin_bit_cast(Half8, b[g][j]), acc[g][m], 0, 0, 0);
+          } else {
+            typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));
+            acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(Bf8, x8),
+                                                                __builtin_bit_cast(Bf8, b[g][j]), acc[g][m], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (chunk + 1 < chunks) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) b[g][0] = next[g][0], b[g][1] = next[g][1];
+    }
+  }
+  // acc[g][m][i] = D[input row 16 m + 4 q + i][output 16 g + n].
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const uint32_t out = out0 + 16 * g + n;
+    if (out < a.outputs) {
+      const float scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale] : 1.0f;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t t = t0 + 16 * m + 4 * q + i;
+          if (t < rows) a.y[t * a.y_stride + out] = acc[g][m][i] * scale;
+        }
+      }
+    }
+  }
+}
+
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
 template <int D, int T, bool kGlu>
@@ -713,4 +848,54 @@ extern "C" int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* e
 #undef LLMP_DECODER
   }
   return LaunchStatus("decode.grouped");
+}
+
+extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
+                                      const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
+                                      int path, void* stream) {
+  if (const int bad = CheckOperand("decode.matrix", decoder, w, first, outputs); bad != 0) return bad;
+  if (x == nullptr || y == nullptr) return Refuse(1, "decode.matrix: null operand");
+  if (path != 0) return Refuse(1, "decode.matrix: the FMA path is for devices without matrix cores; this one has them");
+  if (rows == 0 || rows > 65535ull * 64ull) return Refuse(1, "decode.matrix: rows %llu (1 to 4194240)", static_cast<unsigned long long>(rows));
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_stride % 4 != 0 || x_stride < w->k || y_stride < outputs ||
+      reinterpret_cast<uintptr_t>(y) % 4 != 0)
+    return Refuse(1, "decode.matrix: input rows are 16-byte aligned, a multiple of 4 floats apart and at least k long");
+  if (rows * x_stride >= (uint64_t{1} << 32) || rows * y_stride >= (uint64_t{1} << 32))
+    return Refuse(1, "decode.matrix: inputs or outputs of 2^32 values or more");
+  DecodeArgs a{};
+  a.w = *w;
+  a.first = static_cast<uint32_t>(first);
+  a.outputs = static_cast<uint32_t>(outputs);
+  a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
+  // Four groups of 16 outputs a wave (256 a workgroup) where that still leaves two workgroups a CU; else one.
+  const int cus = llmp_hip_compute_units();
+  const uint64_t row_tiles = (rows + kMatrixTile - 1) / kMatrixTile;
+  const bool wide = (outputs + 255) / 256 * row_tiles >= 2 * static_cast<uint64_t>(cus > 0 ? cus : 256);
+  const uint64_t per = wide ? 256 : 64;
+  const dim3 grid(static_cast<unsigned>((outputs + per - 1) / per), static_cast<unsigned>(row_tiles));
+  const auto s = static_cast<hipStream_t>(stream);
+  switch (decoder) {
+#define LLMP_DECODER(ID)                                                                                       \
+  case ID:                                                                                                     \
+    if (wide) {                                                                                                \
+      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 4>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
+    } else {                                                                                                   \
+      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 1>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
+    }                                                                                                          \
+    break;
+    LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_F16_DENSE)
+    LLMP_DECODER(LLMP_DECODER_Q8_0_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_INTERLEAVED)
+    LLMP_DECODER(LLMP_DECODER_NVFP4_GGML_BLOCKS)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP8_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_SPLIT)
+    LLMP_DECODER(LLMP_DECODER_MXFP4_ATOMS)
+    LLMP_DECODER(LLMP_DECODER_AFFINE_SPLIT)
+#undef LLMP_DECODER
+  }
+  return LaunchStatus("decode.matrix");
 }

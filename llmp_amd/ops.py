@@ -435,3 +435,16 @@ def decode_grouped(decoder, experts, k, n, offsets, pair_rows, x, y, pair_out=No
                                            y.stride(0), 0, _stream()))
     torch.cuda.current_stream().synchronize()  # table_d must outlive the launch
     return y
+
+
+def decode_matrix(decoder, weight, x, first=0, outputs=None, path=0, out=None):
+    """llmp.decode.matrix: float32 x [rows, k] (any number of rows) times a weight in its stored encoding on the
+    matrix cores, weights and inputs rounded to the decoder's matrix element. float32 [rows, outputs]."""
+    lib = _lib.load()
+    op = _decode_operand(weight)
+    outputs = weight["data"].shape[0] - first if outputs is None else outputs
+    rows = x.shape[0]
+    y = torch.empty((rows, outputs), dtype=torch.float32, device=x.device) if out is None else out
+    _lib.check(lib.llmp_hip_decode_matrix(decoder, C.byref(op), first, outputs, _ptr(x), rows, x.stride(0), _ptr(y),
+                                          y.stride(0), path, _stream()))
+    return y

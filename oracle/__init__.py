@@ -406,3 +406,18 @@ def decode_grouped(decoder, experts, k, n, offsets, pair_rows, x, y, pair_out=No
     if rc != 0:
         raise ValueError("no such decoder")
     return y
+
+
+_sig("orc_decode_matrix", _int, _int, C.POINTER(DecodeOperand), _u64, _u64, _vp, _u64, _u64, _vp, _u64, _int)
+
+
+def decode_matrix(decoder, weight, x, first=0, outputs=None, threads=1):
+    """llmp.decode.matrix (the tensor-core path's rounding) on the CPU: float32 x [rows, k] -> [rows, outputs]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    op = decode_operand(weight)
+    outputs = weight["data"].shape[0] - first if outputs is None else outputs
+    y = np.zeros((x.shape[0], outputs), dtype=np.float32)
+    rc = lib.orc_decode_matrix(decoder, C.byref(op), first, outputs, _p(x), x.shape[0], x.shape[1], _p(y), outputs, threads)
+    if rc != 0:
+        raise ValueError("no such decoder")
+    return y

@@ -514,6 +514,30 @@ int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t 
   return 0;
 }
 
+/* products.h:27-33: the matrix path rounds weights and inputs to the decoder's matrix element (F16 for F16 and
+ * Q8_0 weights, BF16 otherwise) and sums in F32; here the sums are double. */
+int orc_decode_matrix(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
+                      uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
+  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT) return 1;
+  const int half = decoder == ORC_DECODER_F16_DENSE || decoder == ORC_DECODER_Q8_0_BLOCKS;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t j = 0; j < (int64_t)outputs; ++j) {
+    const uint64_t row = first + (uint64_t)j;
+    const double scale = w->tensor_scale != NULL ? (double)w->tensor_scale[row / w->rows_per_scale] : 1.0;
+    for (uint64_t t = 0; t < rows; ++t) {
+      double sum = 0;
+      for (uint64_t c = 0; c < w->k; ++c) {
+        const float wv = orc_decode_value(decoder, w, row, c), xv = x[t * x_stride + c];
+        const float wr = half ? orc_f16_to_f32(orc_f32_to_f16(wv)) : orc_bf16_to_f32(orc_f32_to_bf16(wv));
+        const float xr = half ? orc_f16_to_f32(orc_f32_to_f16(xv)) : orc_bf16_to_f32(orc_f32_to_bf16(xv));
+        sum += (double)wr * (double)xr;
+      }
+      y[t * y_stride + (uint64_t)j] = (float)(sum * scale);
+    }
+  }
+  return 0;
+}
+
 /* products.h:141-170 */
 int orc_decode_grouped(int decoder, const orc_decode_operand* experts, uint64_t experts_count, uint32_t k, uint32_t n,
                        uint64_t first, uint64_t outputs, const int32_t* offsets, const int32_t* pair_rows,

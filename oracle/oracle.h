@@ -106,6 +106,10 @@ int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t 
                           uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
                           uint64_t x_stride, float* y, uint64_t y_stride, int threads);
 
+/* RunMatrix's tensor-core path, products.h:27-33 and 111-118: weights and inputs rounded to the decoder's
+ * matrix element (F16 for F16 and Q8_0 weights, BF16 otherwise), double sums here. */
+int orc_decode_matrix(int decoder, const orc_decode_operand* w, uint64_t first, uint64_t outputs, const float* x,
+                      uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads);
 /* RunGrouped, products.h:141-170: an expert worklist's products; experts whose K or N differ, pairs past
  * `pairs` and pairs naming rows past x_rows or y_rows are skipped. */
 int orc_decode_grouped(int decoder, const orc_decode_operand* experts, uint64_t experts_count, uint32_t k, uint32_t n,

@@ -120,6 +120,7 @@ void HostChecks() {
   EXPECT(hipk::decode::RunVector(product, nullptr) == hipk::KernelFailure::kRejected);
   product.decoder = hipk::decode::DecoderId::kAffineSplit;
   EXPECT(hipk::decode::RunVector(product, nullptr) == hipk::KernelFailure::kRejected);
+  EXPECT(hipk::decode::RunMatrix(product, hipk::decode::MatrixPath::kMma, nullptr) == hipk::KernelFailure::kRejected);
   hipk::decode::GluProduct glu_product;
   EXPECT(hipk::decode::RunVectorGlu(glu_product, nullptr) == hipk::KernelFailure::kRejected);
   hipk::decode::RowsGather gather;

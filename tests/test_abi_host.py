@@ -171,3 +171,14 @@ def test_decode_grouped_refuses_bad_operands():
     assert run(first=60, outputs=8) > 0 and b"outputs" in lib.llmp_hip_last_error()
     assert run(x=0x4004) > 0 and run(x_stride=250) > 0
     assert run(k=32768, x_stride=32768) > 0 and b"staging" in lib.llmp_hip_last_error()
+
+
+def test_decode_matrix_refuses_bad_operands():
+    lib = _lib.load()
+    w = _lib.DecodeOperand()
+    w.data, w.scales, w.k, w.rows, w.rows_per_scale, w.row_bytes = 0x1000, 0x2000, 256, 64, 64, 128
+    run = lambda **kw: lib.llmp_hip_decode_matrix(kw.get("decoder", 3), C.byref(w), kw.get("first", 0), kw.get("outputs", 8),
+                                                  kw.get("x", 0x4000), kw.get("rows", 100), kw.get("x_stride", 256), 0x5000,
+                                                  64, kw.get("path", 0), None)
+    assert run(path=1) > 0 and b"FMA" in lib.llmp_hip_last_error()
+    assert run(rows=0) > 0 and run(decoder=12) > 0 and run(first=60) > 0 and run(x=0x4004) > 0 and run(x_stride=100) > 0

@@ -246,3 +246,33 @@ def test_grouped_products_match_oracle(device, decoder):
     ops.decode_grouped(decoder, dev_weights, k, n, to_dev(offsets), to_dev(pair_rows), to_dev(x), y, first=9, outputs=20)
     ok, worst = rel_close(y.cpu().numpy(), want, 1e-3)
     assert ok, worst
+
+
+@pytest.mark.parametrize("decoder", list(range(11)) + [11])
+@pytest.mark.parametrize("rows", [1, 17, 130])
+def test_matrix_products_match_oracle(device, decoder, rows):
+    """RunMatrix's tensor-core path (src/kernels/decode/products.h:27-33, 111-118 of the reference): weights and inputs
+    rounded to the decoder's matrix element, F32 sums; partial tiles of outputs, input rows and K."""
+    n, k = 150, 608 if decoder in (0, 1, 3, 5, 11) else 640  # 608 = 9.5 chunks of 64 where the decoder's K allows
+    w = synth.affine_weight(n, k, 840, bits=8, group=32, scale="bf16") if decoder == 11 else \
+        synth.decode_weight(decoder, n, k, 840 + decoder, tensor_scales=3)
+    x = synth.activations(rows, k, 841 + rows)
+    wd = {key: (torch.from_numpy(np.ascontiguousarray(v)).to(device) if isinstance(v, np.ndarray) else v)
+          for key, v in w.items() if key != "plain"}
+    want = oracle.decode_matrix(decoder, w, x, first=7, outputs=139, threads=oracle.max_threads())
+    got = ops.decode_matrix(decoder, wd, torch.from_numpy(x).to(device), first=7, outputs=139).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, (oracle.DECODERS[decoder], worst)
+    # Against the vector product (F32 inputs): the rounding of the inputs to BF16 or F16 is all that differs.
+    if rows == 1:
+        plain = ops.decode_vector(decoder, wd, torch.from_numpy(x).to(device), first=7, outputs=139).cpu().numpy()
+        assert np.abs(got - plain).max() <= 2e-2 * np.abs(plain).max()
+
+
+def test_matrix_refusals(device):
+    w = to_device(synth.decode_weight(3, 8, 256, 850), device)
+    x = torch.zeros((4, 256), dtype=torch.float32, device=device)
+    with pytest.raises(ops.KernelFailure):  # the FMA path is for devices without matrix cores
+        ops.decode_matrix(3, w, x, path=1)
+    with pytest.raises(ops.KernelFailure):
+        ops.decode_matrix(3, w, x, first=6, outputs=4)
