@@ -94,15 +94,89 @@ __device__ __forceinline__ float DecodeGlu(int kind, float g, float u, float lim
   }
 }
 
-// Segment `seg` (16 values) of row `row`: the values before the block scale, and that scale.
+// A segment as loaded, before any arithmetic: its codes (up to 32 bytes; the row-interleaved
+// layout's eight single bytes), its scale's bits and, for the affine encoding, its bias's or zero
+// point's. Loading and decoding are apart so that a kernel can queue several segments' loads,
+// and other work, before it waits for the first.
+struct RawSegment {
+  U32x4 a, b;
+  uint32_t scale, extra;
+};
+
 template <int D>
-__device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32_t row, uint32_t seg, float (&v)[16],
-                                            float& s) {
+__device__ __forceinline__ RawSegment FetchSegment(const llmp_decode_operand& w, uint32_t row, uint32_t seg) {
+  RawSegment r;
+  r.a = U32x4{0, 0, 0, 0}, r.b = U32x4{0, 0, 0, 0}, r.scale = 0, r.extra = 0;
   const uint8_t* data = w.data + static_cast<uint64_t>(row) * w.row_bytes;
   if constexpr (D == LLMP_DECODER_BF16_DENSE || D == LLMP_DECODER_F16_DENSE) {
     const U32x4* src = reinterpret_cast<const U32x4*>(data + seg * 32u);
-    const U32x4 a = __builtin_nontemporal_load(src), b = __builtin_nontemporal_load(src + 1);
-    const uint32_t word[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    r.a = __builtin_nontemporal_load(src), r.b = __builtin_nontemporal_load(src + 1);
+  } else if constexpr (D == LLMP_DECODER_Q8_0_BLOCKS) {
+    // block_q8_0 is 34 bytes: only two-byte loads are aligned. A segment is half a block.
+    const uint8_t* block = data + static_cast<uint64_t>(seg / 2u) * 34u;
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(block + 2 + (seg & 1u) * 16u);
+    r.scale = *reinterpret_cast<const uint16_t*>(block);
+    r.a = U32x4{q[0], q[1], q[2], q[3]}, r.b = U32x4{q[4], q[5], q[6], q[7]};
+  } else if constexpr (D == LLMP_DECODER_NVFP4_INTERLEAVED) {
+    // A row is its K / 2 code bytes, then its K / 16 scales: no alignment beyond a byte.
+    const uint8_t* c = data + seg * 8u;
+    r.a = U32x4{c[0], c[1], c[2], c[3]}, r.b = U32x4{c[4], c[5], c[6], c[7]};
+    r.scale = data[w.k / 2u + seg];
+  } else if constexpr (D == LLMP_DECODER_NVFP4_GGML_BLOCKS) {
+    // block_nvfp4: four UE4M3 scales, then 32 bytes; a segment is a 16-value sub-block.
+    const uint8_t* block = data + static_cast<uint64_t>(seg / 4u) * 36u;
+    const uint32_t* c = reinterpret_cast<const uint32_t*>(block + 4 + (seg & 3u) * 8u);
+    r.a.x = c[0], r.a.y = c[1];
+    r.scale = *reinterpret_cast<const uint32_t*>(block);
+  } else if constexpr (D == LLMP_DECODER_MXFP8_SPLIT || D == LLMP_DECODER_MXFP8_ATOMS) {
+    r.a = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
+    const uint64_t at = D == LLMP_DECODER_MXFP8_SPLIT ? static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u
+                                                      : AtomAt(row, seg / 2u, w.k / 32u);
+    r.scale = w.scales[at];
+  } else if constexpr (D == LLMP_DECODER_AFFINE_SPLIT) {
+    const uint32_t g = seg * 16u / w.group;
+    const uint64_t scale_row = static_cast<uint64_t>(row) * w.scale_row_bytes;
+    const bool wide = (w.scale_type & 0x7Fu) == 3u;
+    auto element = [&](const uint8_t* base) -> uint32_t {
+      return wide ? *reinterpret_cast<const uint32_t*>(base + scale_row + g * 4u)
+                  : *reinterpret_cast<const uint16_t*>(base + scale_row + g * 2u);
+    };
+    r.scale = element(w.scales);
+    if ((w.scale_type & 0x80u) != 0) {
+      const uint64_t zero_row = (static_cast<uint64_t>(w.k / w.group) * w.bits + 7) / 8;
+      r.extra = w.biases[row * zero_row + (w.bits == 4 ? g / 2u : g)];
+    } else if (w.biases != nullptr) {
+      r.extra = element(w.biases);
+    }
+    if (w.bits == 4) {
+      const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
+      r.a.x = c.x, r.a.y = c.y;
+    } else {
+      r.a = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
+    }
+  } else {
+    // NVFP4 and MXFP4 codes as rows of K / 2 bytes: a segment is eight bytes.
+    const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
+    r.a.x = c.x, r.a.y = c.y;
+    if constexpr (D == LLMP_DECODER_NVFP4_SPLIT) {
+      r.scale = w.scales[static_cast<uint64_t>(row) * (w.k / 16u) + seg];
+    } else if constexpr (D == LLMP_DECODER_NVFP4_ATOMS) {
+      r.scale = w.scales[AtomAt(row, seg, w.k / 16u)];
+    } else if constexpr (D == LLMP_DECODER_MXFP4_SPLIT) {
+      r.scale = w.scales[static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u];
+    } else {
+      r.scale = w.scales[AtomAt(row, seg / 2u, w.k / 32u)];
+    }
+  }
+  return r;
+}
+
+// The segment's sixteen values before the block scale, and that scale.
+template <int D>
+__device__ __forceinline__ void DecodeSegment(const llmp_decode_operand& w, uint32_t seg, const RawSegment& r,
+                                              float (&v)[16], float& s) {
+  if constexpr (D == LLMP_DECODER_BF16_DENSE || D == LLMP_DECODER_F16_DENSE) {
+    const uint32_t word[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if constexpr (D == LLMP_DECODER_BF16_DENSE) {
@@ -115,66 +189,46 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
     }
     s = 1.0f;
   } else if constexpr (D == LLMP_DECODER_Q8_0_BLOCKS) {
-    // block_q8_0 is 34 bytes: only two-byte loads are aligned. A segment is half a block.
-    const uint8_t* block = data + static_cast<uint64_t>(seg / 2u) * 34u;
-    const uint16_t* q = reinterpret_cast<const uint16_t*>(block + 2 + (seg & 1u) * 16u);
-    s = HalfBitsToFloat(*reinterpret_cast<const uint16_t*>(block));
+    const uint32_t pair[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const uint32_t pair = q[i];
-      v[2 * i] = static_cast<float>(static_cast<int8_t>(pair & 0xFFu));
-      v[2 * i + 1] = static_cast<float>(static_cast<int8_t>(pair >> 8));
+      v[2 * i] = static_cast<float>(static_cast<int8_t>(pair[i] & 0xFFu));
+      v[2 * i + 1] = static_cast<float>(static_cast<int8_t>(pair[i] >> 8));
     }
+    s = HalfBitsToFloat(r.scale);
   } else if constexpr (D == LLMP_DECODER_NVFP4_INTERLEAVED) {
-    // A row is its K / 2 code bytes, then its K / 16 scales: no alignment beyond a byte.
-    const uint8_t* c = data + seg * 8u;
-    const uint32_t lo = c[0] | (c[1] << 8) | (c[2] << 16) | (static_cast<uint32_t>(c[3]) << 24);
-    const uint32_t hi = c[4] | (c[5] << 8) | (c[6] << 16) | (static_cast<uint32_t>(c[7]) << 24);
-    Fp4Adjacent(lo, v);
-    Fp4Adjacent(hi, v + 8);
-    s = Ue4m3ToFloat(data[w.k / 2u + seg]);
+    Fp4Adjacent(r.a.x | (r.a.y << 8) | (r.a.z << 16) | (r.a.w << 24), v);
+    Fp4Adjacent(r.b.x | (r.b.y << 8) | (r.b.z << 16) | (r.b.w << 24), v + 8);
+    s = Ue4m3ToFloat(r.scale);
   } else if constexpr (D == LLMP_DECODER_NVFP4_GGML_BLOCKS) {
-    // block_nvfp4: four UE4M3 scales, then 32 bytes; a segment is a 16-value sub-block.
-    const uint8_t* block = data + static_cast<uint64_t>(seg / 4u) * 36u;
-    const uint32_t sub = seg & 3u;
-    const uint32_t* c = reinterpret_cast<const uint32_t*>(block + 4 + sub * 8u);
-    const uint32_t scales = *reinterpret_cast<const uint32_t*>(block);
-    Fp4Halves(c[0], v, v + 8);
-    Fp4Halves(c[1], v + 4, v + 12);
-    s = Ue4m3ToFloat((scales >> (8u * sub)) & 0xFFu);
+    Fp4Halves(r.a.x, v, v + 8);
+    Fp4Halves(r.a.y, v + 4, v + 12);
+    s = Ue4m3ToFloat((r.scale >> (8u * (seg & 3u))) & 0xFFu);
+  } else if constexpr (D == LLMP_DECODER_MXFP8_SPLIT || D == LLMP_DECODER_MXFP8_ATOMS) {
+    Fp8Four(r.a.x, v), Fp8Four(r.a.y, v + 4), Fp8Four(r.a.z, v + 8), Fp8Four(r.a.w, v + 12);
+    s = E8m0ToFloat(r.scale);
   } else if constexpr (D == LLMP_DECODER_AFFINE_SPLIT) {
     // Unsigned codes of 4 or 8 bits, a scale and a bias (or a zero point) a group of values along the
     // row; a segment lies within one group. s * q + b rounded once, or s * (q - z)
     // (src/kernels/reference/decode.cc:197-220).
 #pragma clang fp contract(off)
-    const uint32_t g = seg * 16u / w.group;
-    const uint64_t scale_row = static_cast<uint64_t>(row) * w.scale_row_bytes;
     const uint32_t scale_type = w.scale_type & 0x7Fu;
-    auto element = [&](const uint8_t* base) {
-      if (scale_type == 3u) return *reinterpret_cast<const float*>(base + scale_row + g * 4u);
-      const uint32_t bits = *reinterpret_cast<const uint16_t*>(base + scale_row + g * 2u);
-      return scale_type == 2u ? __builtin_bit_cast(float, bits << 16) : HalfBitsToFloat(bits);
+    auto element = [&](uint32_t bits) {
+      return scale_type == 3u ? __builtin_bit_cast(float, bits)
+                              : scale_type == 2u ? __builtin_bit_cast(float, bits << 16) : HalfBitsToFloat(bits);
     };
-    const float scale = element(w.scales);
+    const float scale = element(r.scale);
     const bool zero_point = (w.scale_type & 0x80u) != 0;
-    int32_t z = 0;
-    float b = 0.0f;
-    if (zero_point) {
-      const uint64_t zero_row = (static_cast<uint64_t>(w.k / w.group) * w.bits + 7) / 8;
-      const uint8_t* zeros = w.biases + row * zero_row;
-      z = w.bits == 4 ? (zeros[g / 2u] >> (4u * (g & 1u))) & 15u : zeros[g];
-    } else if (w.biases != nullptr) {
-      b = element(w.biases);
-    }
+    const uint32_t g = seg * 16u / w.group;
+    const int32_t z = zero_point ? (w.bits == 4 ? (r.extra >> (4u * (g & 1u))) & 15u : r.extra) : 0;
+    const float b = !zero_point && w.biases != nullptr ? element(r.extra) : 0.0f;
     uint32_t code[16];
     if (w.bits == 4) {
-      const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
 #pragma unroll
-      for (int i = 0; i < 16; ++i) code[i] = ((i < 8 ? c.x : c.y) >> (4 * (i % 8))) & 15u;
+      for (int i = 0; i < 16; ++i) code[i] = ((i < 8 ? r.a.x : r.a.y) >> (4 * (i % 8))) & 15u;
     } else {
-      const U32x4 c = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
 #pragma unroll
-      for (int i = 0; i < 16; ++i) code[i] = (c[i / 4] >> (8 * (i % 4))) & 0xFFu;
+      for (int i = 0; i < 16; ++i) code[i] = (r.a[i / 4] >> (8 * (i % 4))) & 0xFFu;
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -182,27 +236,22 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
                         : fmaf(scale, static_cast<float>(code[i]), b);
     }
     s = 1.0f;
-  } else if constexpr (D == LLMP_DECODER_MXFP8_SPLIT || D == LLMP_DECODER_MXFP8_ATOMS) {
-    const U32x4 c = __builtin_nontemporal_load(reinterpret_cast<const U32x4*>(data + seg * 16u));
-    Fp8Four(c.x, v), Fp8Four(c.y, v + 4), Fp8Four(c.z, v + 8), Fp8Four(c.w, v + 12);
-    const uint64_t at = D == LLMP_DECODER_MXFP8_SPLIT ? static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u
-                                                      : AtomAt(row, seg / 2u, w.k / 32u);
-    s = E8m0ToFloat(w.scales[at]);
   } else {
-    // NVFP4 and MXFP4 codes as rows of K / 2 bytes: a segment is eight bytes.
-    const U32x2 c = __builtin_nontemporal_load(reinterpret_cast<const U32x2*>(data + seg * 8u));
-    Fp4Adjacent(c.x, v);
-    Fp4Adjacent(c.y, v + 8);
-    if constexpr (D == LLMP_DECODER_NVFP4_SPLIT) {
-      s = Ue4m3ToFloat(w.scales[static_cast<uint64_t>(row) * (w.k / 16u) + seg]);
-    } else if constexpr (D == LLMP_DECODER_NVFP4_ATOMS) {
-      s = Ue4m3ToFloat(w.scales[AtomAt(row, seg, w.k / 16u)]);
-    } else if constexpr (D == LLMP_DECODER_MXFP4_SPLIT) {
-      s = E8m0ToFloat(w.scales[static_cast<uint64_t>(row) * (w.k / 32u) + seg / 2u]);
+    Fp4Adjacent(r.a.x, v);
+    Fp4Adjacent(r.a.y, v + 8);
+    if constexpr (D == LLMP_DECODER_NVFP4_SPLIT || D == LLMP_DECODER_NVFP4_ATOMS) {
+      s = Ue4m3ToFloat(r.scale);
     } else {
-      s = E8m0ToFloat(w.scales[AtomAt(row, seg / 2u, w.k / 32u)]);
+      s = E8m0ToFloat(r.scale);
     }
   }
+}
+
+// Segment `seg` (16 values) of row `row`: the values before the block scale, and that scale.
+template <int D>
+__device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32_t row, uint32_t seg, float (&v)[16],
+                                            float& s) {
+  DecodeSegment<D>(w, seg, FetchSegment<D>(w, row, seg), v, s);
 }
 
 // grid: workgroups of eight waves, persistent over pairs of output rows; LDS: T input rows.
@@ -433,7 +482,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeGroupedKernel(const G
 // next chunk's inputs and weights are loaded while this one multiplies, one barrier a chunk.
 typedef short Short8 __attribute__((ext_vector_type(8)));
 typedef float Float4 __attribute__((ext_vector_type(4)));
-constexpr int kMatrixTile = 64;        // input rows a workgroup
 constexpr int kMatrixRowBytes = 144;   // 64 two-byte elements and 16 bytes
 
 // Nearest even, by the hardware's conversions (v_cvt_f16_f32, v_cvt_pk_bf16_f32).
@@ -446,74 +494,84 @@ __device__ __forceinline__ uint32_t ToElement(float v) {
   }
 }
 
-// G: groups of 16 outputs a wave (a workgroup takes 64 G outputs by 64 input rows).
-template <int D, int G>
+// G: groups of 16 outputs a wave; M: groups of 16 input rows (a workgroup takes 64 G outputs by 16 M input rows).
+// Decoding a segment costs some sixty vector instructions whatever M is, so the large tile is what
+// lets the matrix cores, not the decoding, set the pace; the small one is for products with few tiles, where
+// each wave waits on memory instead: it loads two chunks ahead, the large one (short of registers) one.
+template <int D, int G, int M>
 __global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, const uint32_t rows) {
   constexpr bool kHalf = D == LLMP_DECODER_F16_DENSE || D == LLMP_DECODER_Q8_0_BLOCKS;
-  constexpr int kTileBytes = kMatrixTile * kMatrixRowBytes;
+  constexpr int kAhead = G == 1 ? 2 : 1;
+  constexpr int kTileBytes = 16 * M * kMatrixRowBytes;
   __shared__ __attribute__((aligned(16))) uint8_t tiles[2 * kTileBytes];  // this chunk's inputs and the next's
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, q = lane >> 4;
-  const uint32_t out0 = (blockIdx.x * 4 + wave) * (16 * G), t0 = blockIdx.y * kMatrixTile;
+  const uint32_t out0 = (blockIdx.x * 4 + wave) * (16 * G), t0 = blockIdx.y * (16 * M);
   const uint32_t segs = a.w.k / 16u, chunks = (segs + 3u) / 4u;
-  Float4 acc[G][4];  // [outputs' group][input rows' group]
+  Float4 acc[G][M];  // [outputs' group][input rows' group]
 #pragma unroll
   for (int g = 0; g < G; ++g) {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int m = 0; m < M; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
   }
-  // A chunk's share of a thread: four pieces of four input values, and the lane's segment of each of
-  // its groups of outputs, scaled and rounded to the element (two operands of eight).
-  auto load_inputs = [&](uint32_t chunk, float4 (&piece)[4]) {
+  // A chunk's share of a thread: M pieces of four input values, and the lane's segment of each of
+  // its groups of outputs. Loads without branches: a row past the inputs or a column past K reads a
+  // valid address nearby and is zeroed when it is used; the same for a segment past the row's last.
+  auto load_inputs = [&](uint32_t chunk, float4 (&piece)[M]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < M; ++i) {
       const uint32_t c = tid + i * 256;
-      const uint32_t row = c >> 4, column = chunk * 64u + (c & 15u) * 4u;
-      piece[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      if (t0 + row < rows && column < a.w.k) piece[i] = *reinterpret_cast<const float4*>(a.x + (t0 + row) * a.x_stride + column);
+      const uint32_t row = min(t0 + (c >> 4), rows - 1), column = min(chunk * 64u + (c & 15u) * 4u, a.w.k - 4u);
+      piece[i] = *reinterpret_cast<const float4*>(a.x + static_cast<uint64_t>(row) * a.x_stride + column);
     }
   };
-  auto load_weights = [&](uint32_t chunk, Short8 (&b)[G][2]) {
+  auto fetch_weights = [&](uint32_t chunk, RawSegment (&raw)[G]) {
+    const uint32_t seg = min(chunk * 4u + q, segs - 1);
+#pragma unroll
+    for (int g = 0; g < G; ++g) raw[g] = FetchSegment<D>(a.w, a.first + min(out0 + 16 * g + n, a.outputs - 1), seg);
+  };
+  // Scaled and rounded to the element: two operands of eight a group.
+  auto decode_weights = [&](uint32_t chunk, const RawSegment (&raw)[G], Short8 (&b)[G][2]) {
     const uint32_t seg = chunk * 4u + q;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      float v[16] = {};
-      float s = 0.0f;
-      // An output past the last is a copy of it, not stored.
-      if (seg < segs) LoadSegment<D>(a.w, a.first + min(out0 + 16 * g + n, a.outputs - 1), seg, v, s);
+      float v[16], s;
+      DecodeSegment<D>(a.w, min(seg, segs - 1), raw[g], v, s);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) b[g][j][i] = static_cast<short>(ToElement<kHalf>(v[8 * j + i] * s));
+        for (int i = 0; i < 8; ++i) b[g][j][i] = static_cast<short>(ToElement<kHalf>(seg < segs ? v[8 * j + i] * s : 0.0f));
       }
     }
   };
 
-  float4 piece[4];
+  // Loads run kAhead chunks ahead of their use, in as many sets of registers (by the chunk's parity when
+  // two): a chunk's multiplies are shorter than a trip to memory. Loads past the last chunk read its
+  // addresses and are dropped.
+  float4 piece[kAhead][M];
+  RawSegment raw[kAhead][G];
   Short8 b[G][2];
-  load_inputs(0, piece);
-  load_weights(0, b);
-  for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+  auto step = [&](uint32_t chunk, auto slot) {
+    constexpr int P = decltype(slot)::value, kNext = (P + 1) % kAhead;
     uint8_t* tile = tiles + (chunk & 1u) * kTileBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < M; ++i) {
       const uint32_t c = tid + i * 256;
+      const bool live = t0 + (c >> 4) < rows && chunk * 64u + (c & 15u) * 4u < a.w.k;
       uint2 packed;
-      packed.x = ToElement<kHalf>(piece[i].x) | (ToElement<kHalf>(piece[i].y) << 16);
-      packed.y = ToElement<kHalf>(piece[i].z) | (ToElement<kHalf>(piece[i].w) << 16);
+      packed.x = live ? ToElement<kHalf>(piece[P][i].x) | (ToElement<kHalf>(piece[P][i].y) << 16) : 0u;
+      packed.y = live ? ToElement<kHalf>(piece[P][i].z) | (ToElement<kHalf>(piece[P][i].w) << 16) : 0u;
       *reinterpret_cast<uint2*>(tile + (c >> 4) * kMatrixRowBytes + (c & 15u) * 8u) = packed;
     }
     // One barrier a chunk: this buffer is complete, and the other's readers (the last chunk's) are done.
     __syncthreads();
-    Short8 next[G][2];
-    if (chunk + 1 < chunks) {  // the next chunk's loads are in flight while this one multiplies
-      load_inputs(chunk + 1, piece);
-      load_weights(chunk + 1, next);
-    }
+    load_inputs(chunk + kAhead, piece[P]);
+    if constexpr (kAhead == 1) fetch_weights(chunk + 1, raw[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
+    for (int m = 0; m < M; ++m) {
       const U32x4* mine = reinterpret_cast<const U32x4*>(tile + (16 * m + n) * kMatrixRowBytes + q * 32);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -532,9 +590,23 @@ __global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, co
         }
       }
     }
-    if (chunk + 1 < chunks) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) b[g][0] = next[g][0], b[g][1] = next[g][1];
+    __builtin_amdgcn_sched_barrier(0);  // the loads' first use stays behind the multiplies
+    decode_weights(chunk + 1, raw[kNext], b);
+    if constexpr (kAhead == 2) fetch_weights(chunk + 3, raw[kNext]);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  load_inputs(0, piece[0]);
+  fetch_weights(0, raw[0]);
+  if constexpr (kAhead == 2) {
+    load_inputs(1, piece[1]);
+    fetch_weights(1, raw[1]);
+  }
+  decode_weights(0, raw[0], b);
+  if constexpr (kAhead == 2) fetch_weights(2, raw[0]);
+  for (uint32_t chunk = 0; chunk < chunks; chunk += kAhead) {  // every wave: the same count of barriers
+    step(chunk, std::integral_constant<int, 0>{});
+    if constexpr (kAhead == 2) {
+      if (chunk + 1 < chunks) step(chunk + 1, std::integral_constant<int, 1>{});
     }
   }
   // acc[g][m][i] = D[input row 16 m + 4 q + i][output 16 g + n].
@@ -544,7 +616,7 @@ __global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, co
     if (out < a.outputs) {
       const float scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale] : 1.0f;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
+      for (int m = 0; m < M; ++m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t t = t0 + 16 * m + 4 * q + i;
@@ -867,21 +939,20 @@ extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w,
   a.first = static_cast<uint32_t>(first);
   a.outputs = static_cast<uint32_t>(outputs);
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
-  // Four groups of 16 outputs a wave (256 a workgroup) where that still leaves two workgroups a CU; else one.
+  // Tiles of 256 outputs by 128 input rows where those still give every CU a workgroup; else 64 by 64.
   const int cus = llmp_hip_compute_units();
-  const uint64_t row_tiles = (rows + kMatrixTile - 1) / kMatrixTile;
-  const bool wide = (outputs + 255) / 256 * row_tiles >= 2 * static_cast<uint64_t>(cus > 0 ? cus : 256);
-  const uint64_t per = wide ? 256 : 64;
-  const dim3 grid(static_cast<unsigned>((outputs + per - 1) / per), static_cast<unsigned>(row_tiles));
+  const bool wide = (outputs + 255) / 256 * ((rows + 127) / 128) >= static_cast<uint64_t>(cus > 0 ? cus : 256);
+  const uint64_t per = wide ? 256 : 64, tile = wide ? 128 : 64;
+  const dim3 grid(static_cast<unsigned>((outputs + per - 1) / per), static_cast<unsigned>((rows + tile - 1) / tile));
   const auto s = static_cast<hipStream_t>(stream);
   switch (decoder) {
-#define LLMP_DECODER(ID)                                                                                       \
-  case ID:                                                                                                     \
-    if (wide) {                                                                                                \
-      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 4>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
-    } else {                                                                                                   \
-      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 1>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
-    }                                                                                                          \
+#define LLMP_DECODER(ID)                                                                                          \
+  case ID:                                                                                                        \
+    if (wide) {                                                                                                   \
+      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 4, 8>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
+    } else {                                                                                                      \
+      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 1, 4>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
+    }                                                                                                             \
     break;
     LLMP_DECODER(LLMP_DECODER_BF16_DENSE)
     LLMP_DECODER(LLMP_DECODER_F16_DENSE)
