@@ -272,15 +272,17 @@ def block_formats(device):
             "us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1), "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
         del ws, base
         torch.cuda.empty_cache()
-    # llmp.decode.matrix: 512 F32 input rows times the same NVFP4 and BF16 weights on the matrix cores.
-    xm = dev(synth.activations(512, k, 308))
-    ym = torch.empty((512, n), dtype=torch.float32, device=device)
+    # llmp.decode.matrix: 512 and 2048 F32 input rows times the same NVFP4 and BF16 weights on the matrix cores.
     for decoder in (0, 3):
         w = synth.decode_weight(decoder, n, k, 307)
         base = {key: (dev(v) if isinstance(v, np.ndarray) else v) for key, v in w.items() if key != "plain"}
-        us = event_us(lambda i: ops.decode_matrix(decoder, base, xm, out=ym), 20)
-        out[f"decode_matrix_{ops.DECODERS[decoder].replace('.', '_')}_4096x14336_rows512"] = {
-            "us": round(us, 1), "TFLOP/s": round(2.0 * 512 * n * k / us / 1e6, 1)}
+        for rows in (512, 2048):
+            xm = dev(synth.activations(rows, k, 308))
+            ym = torch.empty((rows, n), dtype=torch.float32, device=device)
+            us = event_us(lambda i: ops.decode_matrix(decoder, base, xm, out=ym), 20)
+            out[f"decode_matrix_{ops.DECODERS[decoder].replace('.', '_')}_4096x14336_rows{rows}"] = {
+                "us": round(us, 1), "TFLOP/s": round(2.0 * rows * n * k / us / 1e6, 1),
+                "frac_bf16_peak": round(2.0 * rows * n * k / us / 1e6 / 2500.0, 4)}
         del base
         torch.cuda.empty_cache()
     # llmp.set_rows.quant: 512 rows of 8192 floats (a layer's K or V rows of a 512-token chunk) into a cache.

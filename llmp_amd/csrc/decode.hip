@@ -49,7 +49,8 @@ __device__ __forceinline__ uint64_t AtomAt(uint64_t row, uint64_t block, uint64_
 
 // decode.cc:407-411: E4M3's value up to 0x7E, NaN from 0x7F.
 __device__ __forceinline__ float Ue4m3ToFloat(uint32_t bits) {
-  return bits < 0x7Fu ? E4m3ToFloat(bits) : __builtin_nanf("");
+  const float value = __builtin_amdgcn_cvt_pk_f32_fp8(bits, false)[0];  // OCP E4M3 on this device; no branches
+  return bits < 0x7Fu ? value : __builtin_nanf("");
 }
 
 // Eight E2M1 codes, value 2 i in byte i's low nibble (decoders.cuh:57-72), into v[0..7].
@@ -627,6 +628,158 @@ __global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, co
   }
 }
 
+// The large product: a workgroup of eight waves takes 256 outputs by 128 input rows. A segment of the
+// weights is decoded once a workgroup, by one thread, into an LDS tile laid out like the inputs' (rows of 64
+// elements, 144 bytes apart), and every wave reads its operands of both sides from LDS: a wave (rows' half
+// w / 4, outputs' quarter w % 4) multiplies 64 rows by 64 outputs. Two stages of both tiles: after a chunk's one
+// barrier a wave queues the loads of the chunk after the next, and decodes the next chunk (loaded a step ago)
+// into the other stage among this chunk's matrix instructions.
+constexpr int kSharedRows = 128, kSharedOutputs = 256;
+constexpr int kSharedInputBytes = kSharedRows * kMatrixRowBytes, kSharedStageBytes = (kSharedRows + kSharedOutputs) * kMatrixRowBytes;
+
+template <int D>
+__global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs a, const uint32_t rows) {
+  constexpr bool kHalf = D == LLMP_DECODER_F16_DENSE || D == LLMP_DECODER_Q8_0_BLOCKS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t stages[];  // two of inputs' tile, weights' tile
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, q = lane >> 4;
+  const uint32_t out0 = blockIdx.x * kSharedOutputs, t0 = blockIdx.y * kSharedRows;
+  const uint32_t row_half = (wave >> 2) * 64, out_quarter = (wave & 3) * 64;
+  const uint32_t segs = a.w.k / 16u, chunks = (segs + 3u) / 4u;
+  Float4 acc[4][4];  // [outputs' group][input rows' group]
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  // A thread's share of a chunk: four pieces of four input values (row c / 16, columns 4 (c % 16) + [0, 4) for
+  // c = tid + 512 i) and two segments of weights (output e / 4, segment e % 4 for e = tid + 512 u). Loads
+  // without branches: past the inputs, the outputs or K they read a valid address nearby, zeroed when staged.
+  struct Share {
+    float4 piece[4];
+    RawSegment raw[2];
+  };
+  auto load = [&](uint32_t chunk, Share& share) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + i * 512;
+      const uint32_t row = min(t0 + (c >> 4), rows - 1), column = min(chunk * 64u + (c & 15u) * 4u, a.w.k - 4u);
+      share.piece[i] = *reinterpret_cast<const float4*>(a.x + static_cast<uint64_t>(row) * a.x_stride + column);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t e = tid + u * 512;
+      share.raw[u] = FetchSegment<D>(a.w, a.first + min(out0 + (e >> 2), a.outputs - 1), min(chunk * 4u + (e & 3u), segs - 1));
+    }
+  };
+  auto stage = [&](uint32_t chunk, const Share& share) {
+    uint8_t* inputs = stages + (chunk & 1u) * kSharedStageBytes;
+    uint8_t* weights = inputs + kSharedInputBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + i * 512;
+      const bool live = t0 + (c >> 4) < rows && chunk * 64u + (c & 15u) * 4u < a.w.k;
+      uint2 packed;
+      packed.x = live ? ToElement<kHalf>(share.piece[i].x) | (ToElement<kHalf>(share.piece[i].y) << 16) : 0u;
+      packed.y = live ? ToElement<kHalf>(share.piece[i].z) | (ToElement<kHalf>(share.piece[i].w) << 16) : 0u;
+      *reinterpret_cast<uint2*>(inputs + (c >> 4) * kMatrixRowBytes + (c & 15u) * 8u) = packed;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t e = tid + u * 512;
+      const uint32_t seg = chunk * 4u + (e & 3u);
+      float v[16], s;
+      DecodeSegment<D>(a.w, min(seg, segs - 1), share.raw[u], v, s);
+      U32x4 half[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t two = ToElement<kHalf>(v[8 * j + 2 * i] * s) | (ToElement<kHalf>(v[8 * j + 2 * i + 1] * s) << 16);
+          half[j][i] = seg < segs ? two : 0u;
+        }
+      }
+      U32x4* to = reinterpret_cast<U32x4*>(weights + (e >> 2) * kMatrixRowBytes + (e & 3u) * 32u);
+      to[0] = half[0], to[1] = half[1];
+    }
+  };
+  auto multiply = [&](uint32_t chunk) {
+    const uint8_t* inputs = stages + (chunk & 1u) * kSharedStageBytes;
+    const uint8_t* weights = inputs + kSharedInputBytes;
+    U32x4 b[4][2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const U32x4* mine = reinterpret_cast<const U32x4*>(weights + (out_quarter + 16 * g + n) * kMatrixRowBytes + q * 32);
+      b[g][0] = mine[0], b[g][1] = mine[1];
+    }
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const U32x4* mine = reinterpret_cast<const U32x4*>(inputs + (row_half + 16 * m + n) * kMatrixRowBytes + q * 32);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const U32x4 x8 = mine[j];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          if constexpr (kHalf) {
+            typedef _Float16 Half8 __attribute__((ext_vector_type(8)));
+            acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(Half8, x8),
+                                                               __builtin_bit_cast(Half8, b[g][j]), acc[g][m], 0, 0, 0);
+          } else {
+            typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));
+            acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(Bf8, x8),
+                                                                __builtin_bit_cast(Bf8, b[g][j]), acc[g][m], 0, 0, 0);
+          }
+        }
+      }
+    }
+  };
+  Share share[2];  // by the chunk's parity
+  load(0, share[0]);
+  load(1, share[1]);
+  stage(0, share[0]);
+  auto step = [&](uint32_t chunk, auto parity) {
+    constexpr int P = decltype(parity)::value;
+    // One barrier a chunk: its stage is complete, and the other stage's readers (the last chunk's) are done.
+    __syncthreads();
+    load(chunk + 2, share[P]);
+    multiply(chunk);
+    stage(chunk + 1, share[1 - P]);
+  };
+  for (uint32_t chunk = 0; chunk < chunks; chunk += 2) {  // every wave: the same count of barriers
+    step(chunk, std::integral_constant<int, 0>{});
+    if (chunk + 1 < chunks) step(chunk + 1, std::integral_constant<int, 1>{});
+  }
+  // acc[g][m][i] = D[input row 16 m + 4 q + i][output 16 g + n] of the wave's 64 by 64.
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const uint32_t out = out0 + out_quarter + 16 * g + n;
+    if (out < a.outputs) {
+      const float scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale] : 1.0f;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t t = t0 + row_half + 16 * m + 4 * q + i;
+          if (t < rows) a.y[t * a.y_stride + out] = acc[g][m][i] * scale;
+        }
+      }
+    }
+  }
+}
+
+template <int D>
+void LaunchMatrixShared(const DecodeArgs& a, dim3 grid, uint32_t rows, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!sized) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeMatrixSharedKernel<D>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kSharedStageBytes);
+    sized = true;
+  }
+  hipLaunchKernelGGL((DecodeMatrixSharedKernel<D>), grid, dim3(512), 2 * kSharedStageBytes, stream, a, rows);
+}
+
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
 template <int D, int T, bool kGlu>
@@ -939,9 +1092,9 @@ extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w,
   a.first = static_cast<uint32_t>(first);
   a.outputs = static_cast<uint32_t>(outputs);
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
-  // Tiles of 256 outputs by 128 input rows where those still give every CU a workgroup; else 64 by 64.
+  // Tiles of 256 outputs by 128 input rows where those still give every other CU a workgroup; else 64 by 64.
   const int cus = llmp_hip_compute_units();
-  const bool wide = (outputs + 255) / 256 * ((rows + 127) / 128) >= static_cast<uint64_t>(cus > 0 ? cus : 256);
+  const bool wide = 2 * ((outputs + 255) / 256 * ((rows + 127) / 128)) >= static_cast<uint64_t>(cus > 0 ? cus : 256);
   const uint64_t per = wide ? 256 : 64, tile = wide ? 128 : 64;
   const dim3 grid(static_cast<unsigned>((outputs + per - 1) / per), static_cast<unsigned>((rows + tile - 1) / tile));
   const auto s = static_cast<hipStream_t>(stream);
@@ -949,7 +1102,7 @@ extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w,
 #define LLMP_DECODER(ID)                                                                                          \
   case ID:                                                                                                        \
     if (wide) {                                                                                                   \
-      hipLaunchKernelGGL((DecodeMatrixKernel<ID, 4, 8>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
+      LaunchMatrixShared<ID>(a, grid, static_cast<uint32_t>(rows), s);                                           \
     } else {                                                                                                      \
       hipLaunchKernelGGL((DecodeMatrixKernel<ID, 1, 4>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
     }                                                                                                             \
