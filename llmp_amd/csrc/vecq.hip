@@ -584,7 +584,8 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
 
 int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
-  const bool legacy = type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1;
+  const bool legacy = type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1 ||
+                      type == LLMP_TYPE_IQ4_NL;  // 18-byte blocks as Q4_0's
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_MXFP4 && !legacy)
     return Refuse(1, "vecq: weight type %d has no kernel", type);
   const int qk = type == LLMP_TYPE_Q4_K ? 256 : 32;
@@ -606,7 +607,7 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (type == LLMP_TYPE_Q8_0 && wa % 2 != 0) return Refuse(1, "vecq: Q8_0 weights not 2-byte aligned");
   // The legacy 4/5-bit blocks run through the flat form alone: rows of whole 256 values at 16-byte boundaries.
   if (legacy && !FlatTakes(type, *d))
-    return Refuse(1, "vecq: Q4_0, Q4_1, Q5_0 and Q5_1 take rows of whole 256 values (up to 8192 with a GLU) whose rows, "
+    return Refuse(1, "vecq: Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL take rows of whole 256 values (up to 8192 with a GLU) whose rows, "
                      "matrices and experts start on 16-byte boundaries");
   // MXFP4 likewise; its 136-byte units come in pairs.
   if (type == LLMP_TYPE_MXFP4 && !FlatTakes(type, *d))

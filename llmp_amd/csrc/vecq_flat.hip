@@ -524,6 +524,95 @@ struct FormatQ40 {
   }
 };
 
+// ---- IQ4_NL: Q4_0's bytes {f16 d; u8 nibbles[16]}, each nibble an index into a codebook of sixteen int8
+//
+// src/kernels/ggml/vecq.cu:375-396 of the reference: a block times a Q8_1 block is (dw * d8) * sum(value[code] * q),
+// the codebook being ggml's kvalues_iq4nl. Units, staged images and tiles are Q4_0's; a dword's eight nibbles
+// become eight values by byte permutes: the code's low three bits pick from the lower and from the upper half
+// of the codebook, its fourth bit between the two, byte by byte.
+struct FormatIq4nl : FormatQ40 {
+  static __device__ __forceinline__ uint32_t Merge(uint32_t mask, uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "s"(mask), "v"(a), "v"(b));  // (a & mask) | (b & ~mask)
+    return r;
+  }
+  static __device__ __forceinline__ void Decode(uint32_t w, uint32_t& lo, uint32_t& hi) {
+    // {-127, -104, -83, -65}, {-49, -35, -22, -10}, {1, 13, 25, 38}, {53, 69, 89, 113}
+    constexpr uint32_t kLower0 = 0xBFAD9881u, kLower1 = 0xF6EADDCFu, kUpper0 = 0x26190D01u, kUpper1 = 0x71594535u;
+    constexpr uint32_t kPlaces = 0x03020100u;  // byte k of the lower half's values; 4 + k, of the upper half's
+    const uint32_t sel_lo = w & 0x07070707u;
+    const uint32_t sel_hi = (w >> 4) & 0x07070707u;
+    const uint32_t lower_lo = __builtin_amdgcn_perm(kLower1, kLower0, sel_lo);
+    const uint32_t upper_lo = __builtin_amdgcn_perm(kUpper1, kUpper0, sel_lo);
+    const uint32_t lower_hi = __builtin_amdgcn_perm(kLower1, kLower0, sel_hi);
+    const uint32_t upper_hi = __builtin_amdgcn_perm(kUpper1, kUpper0, sel_hi);
+    lo = __builtin_amdgcn_perm(upper_lo, lower_lo, Merge(0x04040404u, w >> 1, kPlaces));
+    hi = __builtin_amdgcn_perm(upper_hi, lower_hi, Merge(0x04040404u, w >> 5, kPlaces));
+  }
+
+  // The unit at `at` (LDS) times the staged tokens: a pair of blocks (nine dwords) at a time, each pair used by
+  // every token before the next is read. The dwords that hold a block's scale decode to values that meet the
+  // images' zeros.
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    float v[P];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      __builtin_amdgcn_sched_barrier(0);
+      const uint32_t* pair = reinterpret_cast<const uint32_t*>(at) + 9 * p;
+      uint32_t word[9];
+#pragma unroll
+      for (int i = 0; i < 9; ++i) word[i] = pair[i];
+      const float dw_even = HalfBitsToFloat(word[0] & 0xFFFFu), dw_odd = HalfBitsToFloat(word[4] >> 16);
+      int even[P], odd[P];
+#pragma unroll
+      for (int t = 0; t < P; ++t) even[t] = 0, odd[t] = 0;
+      // The low nibbles against the first image, then the high ones against the second: nine decoded dwords
+      // live at a time, whatever the number of tokens.
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint32_t values[9];
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+          uint32_t lo, hi;
+          Decode(word[i], lo, hi);
+          values[i] = half ? hi : lo;
+        }
+#pragma unroll
+        for (int t = 0; t < P; ++t) {
+          if (t < m) {
+            const uint32_t* image = reinterpret_cast<const uint32_t*>(records + t * token_stride + half * 144) + 9 * p;
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+              int& s = i >= 5 ? odd[t] : even[t];
+              s = Dot4(static_cast<int>(values[i]), static_cast<int>(image[i]), s);
+            }
+            asm volatile("" : "+v"(even[t]), "+v"(odd[t]));  // taken here: the products stay with their pair
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < P; ++t) {
+        if (t < m) {
+          const uint8_t* record = records + t * token_stride;
+          if (kDump && dump != nullptr) dump[2 * p] = even[t], dump[2 * p + 1] = odd[t];
+          const float2 d8 = *reinterpret_cast<const float2*>(record + 288 + 8 * p);
+          const float term_even = (dw_even * d8.x) * static_cast<float>(even[t]);
+          const float term_odd = (dw_odd * d8.y) * static_cast<float>(odd[t]);
+          v[t] = p == 0 ? term_even : v[t] + term_even;
+          v[t] = v[t] + term_odd;
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) out[t] = v[t];
+    }
+  }
+};
+
 // ---- Q4_1, Q5_0, Q5_1: a unit is eight blocks of {f16 d; [f16 m;] [u32 high bits;] u8 nibbles[16]}
 //
 // tests/unit/dsv4_fast_test.cc:141-164 of the reference: code i is the low (i < 16) or high
@@ -1519,7 +1608,8 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
-  if (type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1) {
+  if (type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1 ||
+      type == LLMP_TYPE_IQ4_NL) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
     if (d.ncols_x % 256 != 0 || d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || at % 16 != 0) return false;
     const int units = d.ncols_x / 256;
@@ -1528,7 +1618,7 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
       if (units > most) return pieces && PlanSplit<F>(units).lds <= kFlatLdsLimit;
       return PlanFlat<F>(1, units, glu).lds <= kFlatLdsLimit;
     };
-    return type == LLMP_TYPE_Q4_0 ? fits(FormatQ40{}) : type == LLMP_TYPE_Q4_1 ? fits(FormatQ41{})
+    return type == LLMP_TYPE_Q4_0 ? fits(FormatQ40{}) : type == LLMP_TYPE_IQ4_NL ? fits(FormatIq4nl{}) : type == LLMP_TYPE_Q4_1 ? fits(FormatQ41{})
            : type == LLMP_TYPE_Q5_0 ? fits(FormatQ50{}) : fits(FormatQ51{});
   }
   if (type == LLMP_TYPE_MXFP4) {
@@ -1552,6 +1642,8 @@ void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hi
     LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q4_0) {
     LaunchF<FormatQ40>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_IQ4_NL) {
+    LaunchF<FormatIq4nl>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q4_1) {
     LaunchF<FormatQ41>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q5_0) {

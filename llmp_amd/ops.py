@@ -8,12 +8,12 @@ import torch
 
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q4_K,  # noqa: F401
-                   TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1,
+                   TYPE_IQ4_NL, TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1,
                    TYPE_Q8_0, X_BF16, X_F16, X_F32, DecodeOperand, Exl3Linear, Exl3MultiLinear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
                    VecQSource)
 
-BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17}
-BLOCK_ELEMENTS = {TYPE_Q4_0: 32, TYPE_Q4_1: 32, TYPE_Q5_0: 32, TYPE_Q5_1: 32, TYPE_Q8_0: 32, TYPE_Q4_K: 256, TYPE_MXFP4: 32}
+BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18}
+BLOCK_ELEMENTS = {TYPE_Q4_0: 32, TYPE_Q4_1: 32, TYPE_Q5_0: 32, TYPE_Q5_1: 32, TYPE_Q8_0: 32, TYPE_Q4_K: 256, TYPE_MXFP4: 32, TYPE_IQ4_NL: 32}
 
 
 def padded_k(k):

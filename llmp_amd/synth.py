@@ -38,7 +38,7 @@ def q4_k_weights(n, k, seed):
     return out.reshape(n, blocks * 144)
 
 
-LEGACY_BYTES = {2: 18, 3: 20, 6: 22, 7: 24}  # Q4_0, Q4_1, Q5_0, Q5_1
+LEGACY_BYTES = {2: 18, 3: 20, 6: 22, 7: 24, 20: 18}  # Q4_0, Q4_1, Q5_0, Q5_1; IQ4_NL (Q4_0's bytes)
 
 
 def legacy_weights(t, n, k, seed):
@@ -47,7 +47,7 @@ def legacy_weights(t, n, k, seed):
     g = rng(seed)
     blocks, size = k // 32, LEGACY_BYTES[t]
     out = g.integers(0, 256, size=(n, blocks, size), dtype=np.uint8)
-    levels = 31.0 if t in (6, 7) else 15.0
+    levels = 31.0 if t in (6, 7) else 254.0 if t == 20 else 15.0  # IQ4_NL's codebook spans -127 .. 113
     amax = np.abs(g.standard_normal((n, blocks, 32), dtype=np.float32) * 0.02).max(axis=-1)
     out[:, :, 0:2] = (2.0 * amax / levels).astype(np.float16).view(np.uint8).reshape(n, blocks, 2)
     if t in (3, 7):

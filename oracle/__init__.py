@@ -19,6 +19,7 @@ TYPE_Q5_1 = 7
 TYPE_Q8_0 = 8
 TYPE_Q4_K = 12
 TYPE_MXFP4 = 39
+TYPE_IQ4_NL = 20
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
 CB_3INST, CB_MCG, CB_MUL1 = 0, 1, 2
 Q8_DEVICE, Q8_GGML_CPU = 0, 1
@@ -105,7 +106,7 @@ def max_threads():
 
 
 def block_bytes(t):
-    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17}[t]
+    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18}[t]
 
 
 def block_elements(t):

@@ -235,6 +235,7 @@ int orc_block_bytes(int type) {
     case ORC_TYPE_Q8_0: return 34;
     case ORC_TYPE_Q4_K: return 144;
     case ORC_TYPE_MXFP4: return 17; /* encoding.cc:130-138 */
+    case ORC_TYPE_IQ4_NL: return 18; /* {f16 d; u8 nibbles[16]}: Q4_0's bytes */
     default: return 0;
   }
 }
@@ -254,6 +255,13 @@ static int legacy_code(int type, const uint8_t* w, int i) {
   const int low = i < 16 ? codes[i] & 15 : codes[i - 16] >> 4;
   return low + (legacy_five(type) ? (int)((high >> i) & 1u) * 16 : 0);
 }
+
+/* IQ4_NL (src/kernels/ggml/vecq.cu:375-396 of the reference reads it through ggml's
+ * kvalues_iq4nl, which is not vendored: ggml-common.h of llama.cpp d812350, restated): code i of a
+ * block is the low (i < 16) or high nibble of byte 2 + i % 16, its value the codebook's entry, the
+ * block's values d times those. Parity unpinned: the reference holds no vector for this type. */
+static const int8_t iq4_nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+static int iq4_nl_value(const uint8_t* w, int i) { return iq4_nl_values[i < 16 ? w[2 + i] & 15 : w[2 + i - 16] >> 4]; }
 
 /* decode.cc:424-428: the E2M1 value of a four-bit code. */
 float orc_e2m1_to_f32(uint8_t code) {
@@ -282,6 +290,13 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
     for (int64_t j = 0; j < k; ++j) {
       const uint8_t* x = row + j / 32 * 17;
       y[j] = orc_e2m1_to_f32((uint8_t)mxfp4_code(x, (int)(j % 32))) * orc_e8m0_to_f32(x[0]);
+    }
+    return;
+  }
+  if (type == ORC_TYPE_IQ4_NL) {
+    for (int64_t j = 0; j < k; ++j) {
+      const uint8_t* x = row + j / 32 * 18;
+      y[j] = orc_f16_to_f32(load_u16(x)) * (float)iq4_nl_value(x, (int)(j % 32));
     }
     return;
   }
@@ -327,6 +342,12 @@ void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums
     sums[0] = s;
     return;
   }
+  if (type == ORC_TYPE_IQ4_NL) { /* vecq.cu:379-392: the codebook's values times the codes */
+    int32_t s = 0;
+    for (int i = 0; i < 32; ++i) s += iq4_nl_value(w, i) * (int32_t)(int8_t)q8[4 + i];
+    sums[0] = s;
+    return;
+  }
   if (legacy(type)) { /* dsv4_fast_test.cc:154-158 */
     int32_t s = 0;
     for (int i = 0; i < 32; ++i) s += legacy_code(type, w, i) * (int32_t)(int8_t)q8[4 + i];
@@ -357,6 +378,9 @@ double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
   orc_block_sums(type, w, q8, sums);
   if (type == ORC_TYPE_MXFP4) { /* vecq.cu:426,437: half the block's scale, times d8, times the sum */
     return (double)orc_e8m0_to_f32(w[0]) * 0.5 * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
+  }
+  if (type == ORC_TYPE_IQ4_NL) { /* vecq.cu:394-395: dw * d8, times the sum */
+    return (double)orc_f16_to_f32(load_u16(w)) * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
   }
   if (legacy(type)) { /* dsv4_fast_test.cc:145-164: the Q8_1 block's s is the rounded sum of its inputs */
     const float dw = orc_f16_to_f32(load_u16(w));

@@ -48,6 +48,14 @@ def build():
     out["q4_0_w"], out["q4_0_x"] = w40, a
     out["q4_0_y"] = oracle.vecq(oracle.TYPE_Q4_0, w40, q8, k, n, tokens=2)
     out["q4_0_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q4_0, w40, q8[:1], k, n)
+    # llmp.vecq, IQ4_NL (Q4_0's bytes, ggml's codebook), 2 tokens.
+    k, n = 256, 14
+    wi = synth.legacy_weights(oracle.TYPE_IQ4_NL, n, k, 26)
+    a = synth.activations(2, k, 27)
+    q8 = oracle.q8_1_quantize(a)
+    out["iq4_nl_w"], out["iq4_nl_x"] = wi, a
+    out["iq4_nl_y"] = oracle.vecq(oracle.TYPE_IQ4_NL, wi, q8, k, n, tokens=2)
+    out["iq4_nl_sums"] = oracle.vecq_block_sums(oracle.TYPE_IQ4_NL, wi, q8[:1], k, n)
     # llmp.vecq, MXFP4 (17-byte blocks), 2 tokens.
     k, n = 512, 12
     wm = synth.mxfp4_weights(n, k, 24)

@@ -273,7 +273,7 @@ def test_guard_bytes_stay_untouched_and_refusals_queue_nothing(device):
 # ---- the legacy 4/5-bit blocks through the streaming form (eight blocks a lane)
 
 Q4_0 = ops.TYPE_Q4_0
-LEGACY = [ops.TYPE_Q4_0, ops.TYPE_Q4_1, ops.TYPE_Q5_0, ops.TYPE_Q5_1]
+LEGACY = [ops.TYPE_Q4_0, ops.TYPE_Q4_1, ops.TYPE_Q5_0, ops.TYPE_Q5_1, ops.TYPE_IQ4_NL]  # IQ4_NL: Q4_0's bytes, a codebook
 
 
 @pytest.mark.parametrize("t", LEGACY)
@@ -281,7 +281,8 @@ LEGACY = [ops.TYPE_Q4_0, ops.TYPE_Q4_1, ops.TYPE_Q5_0, ops.TYPE_Q5_1]
 @pytest.mark.parametrize("tokens", [1, 3, 4, 9])
 def test_legacy_blocks_dense_match_oracle(device, t, k, n, tokens):
     """The blocks of tests/unit/dsv4_fast_test.cc:141-164: dw * (sum * d8 - 8 or 16 * s8), or
-    sum * f16(dw * d8) + f16(m * s8), the activation block's stored sum included. Rows of one
+    sum * f16(dw * d8) + f16(m * s8), the activation block's stored sum included; IQ4_NL's
+    (dw * d8) * sum over its codebook's values (src/kernels/ggml/vecq.cu:375-396). Rows of one
     tile, of fewer waves, and in pieces."""
     w = synth.legacy_weights(t, n, k, 401 + k + n)
     x = synth.activations(tokens, k, 402 + tokens)

@@ -226,6 +226,53 @@ def test_legacy_blocks_decode_sums_and_products_by_brute_force():
                 np.testing.assert_allclose(y[r], want, rtol=1e-6, atol=1e-9)
 
 
+def test_iq4_nl_codebook_blocks_by_brute_force_and_known_answers():
+    """IQ4_NL (src/format/encoding.cc:126: 32 values in 18 bytes; src/kernels/ggml/vecq.cu:375-396 of the
+    reference: (dw * d8) * sum(value[code] * q)). Parity unpinned: the codebook is ggml's kvalues_iq4nl, which the
+    reference does not vendor and for which it holds no vector; this pins the oracle's layout and arithmetic
+    against numpy and a hand-built block, and the codebook against what is published of it (sixteen rising int8
+    values from -127 to 113 that sum to -94, the ninth being 1)."""
+    from llmp_amd import synth
+    values = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.int64)
+    t, k, n = oracle.TYPE_IQ4_NL, 256, 4
+    assert oracle.block_bytes(t) == 18 and oracle.block_elements(t) == 32
+    # The codebook as the oracle decodes it: d = 1, code i = i % 16 in both halves.
+    w = np.zeros((1, 18), dtype=np.uint8)
+    w[0, 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    w[0, 2:] = np.arange(16, dtype=np.uint8) * 17
+    book = oracle.decode_rows(t, w, 32)[0]
+    assert np.array_equal(book[:16], book[16:]) and np.all(np.diff(book[:16]) > 0)
+    assert book[0] == -127 and book[8] == 1 and book[15] == 113 and book[:16].sum() == -94
+    assert np.array_equal(book[:16], values)
+    # Every q = 2, d8 = 0.25: sum = 2 * 2 * -94 = -376; (1 * 0.25) * -376 = -94.
+    q8 = np.zeros((1, 36), dtype=np.uint8)
+    q8[0, 0:2] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    q8[0, 2:4] = np.array([3.0], dtype=np.float16).view(np.uint8)  # the stored sum plays no part
+    q8[0, 4:36] = np.full(32, 2, dtype=np.int8).view(np.uint8)
+    assert oracle.vecq_block_sums(t, w, q8, 32, 1)[0, 0, 0] == -376
+    assert oracle.vecq(t, w, q8, 32, 1)[0, 0, 0] == -94.0
+    # Random bytes and plausible blocks against numpy.
+    x = np.random.Generator(np.random.PCG64(58)).standard_normal((1, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    acts = q8[0].reshape(-1, 36)
+    for w in (synth.random_blocks(t, n, k, 59), synth.legacy_weights(t, n, k, 60)):
+        sums = oracle.vecq_block_sums(t, w, q8, k, n)
+        y = oracle.vecq(t, w, q8, k, n)[0, 0]
+        dec = oracle.decode_rows(t, w, k)
+        for r in range(n):
+            want, row = 0.0, []
+            for b, block in enumerate(w[r].reshape(-1, 18)):
+                nib = block[2:].astype(np.int64)
+                v = values[np.concatenate([nib & 15, nib >> 4])]
+                total = int((v * acts[b][4:].view(np.int8).astype(np.int64)).sum())
+                assert sums[r, b, 0] == total
+                d = float(block[0:2].view(np.float16)[0])
+                want += d * float(acts[b][0:2].view(np.float16)[0]) * total
+                row.append(np.float32(d) * v.astype(np.float32))
+            np.testing.assert_allclose(dec[r], np.concatenate(row), rtol=1e-6, atol=1e-12)
+            np.testing.assert_allclose(y[r], want, rtol=1e-6, atol=1e-9)
+
+
 def test_hand_built_legacy_blocks_have_known_answers():
     # Q4_0: d = 0.5, code i = i % 16 in both halves (byte i = i | i << 4); activation d = 0.25,
     # every q = 2, s = 3. sum = 2 * 2 * (0 + .. + 15) = 480; 0.5 * (480 * 0.25 - 8 * 3) = 48.
