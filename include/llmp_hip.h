@@ -24,7 +24,9 @@
  * i the E2M1 value of the low (i < 16) or high nibble of byte i % 16, times 2^(e - 127)
  * (src/format/encoding.cc:130-138, src/kernels/reference/decode.cc:239-248 and 417-428); IQ4_NL is
  * Q4_0's 18 bytes with each nibble an index into ggml's codebook of sixteen int8 values, a value d times the
- * entry (src/format/encoding.cc:126, src/kernels/ggml/vecq.cu:375-396).
+ * entry (src/format/encoding.cc:126, src/kernels/ggml/vecq.cu:375-396); Q5_K is {f16 d; f16 dmin; u8 scales[12];
+ * u8 qh[32]; u8 qs[128]} = 176 bytes, Q4_K with bit g of qh's byte i as the fifth bit of value i of sub-block g
+ * (src/format/encoding.cc:116).
  */
 #ifndef LLMP_HIP_H_
 #define LLMP_HIP_H_
@@ -37,7 +39,7 @@ extern "C" {
 #endif
 
 /* ggml_type values of the weight encodings the kernels read. */
-enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12, LLMP_TYPE_MXFP4 = 39, LLMP_TYPE_IQ4_NL = 20 };
+enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12, LLMP_TYPE_MXFP4 = 39, LLMP_TYPE_IQ4_NL = 20, LLMP_TYPE_Q5_K = 13 };
 /* VecQGlu, src/kernels/ggml/llmp_ops.h:1072. */
 enum { LLMP_GLU_NONE = 0, LLMP_GLU_SWIGLU = 1, LLMP_GLU_SWIGLU_CLAMP = 2, LLMP_GLU_GEGLU = 3 };
 /* Element types of unquantized activations. */

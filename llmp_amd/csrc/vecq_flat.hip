@@ -245,6 +245,103 @@ template <int P, bool kDump>
 }
 };
 
+// ---- Q5_K: Q4_K's header and nibbles with a fifth bit a value
+//
+// {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} = 176 bytes (src/format/encoding.cc:116 of the
+// reference; ggml's dequantize_row_q5_K): bit g of byte i of qh is the fifth bit of value i of sub-block g, so the
+// eight dwords of qh line up with the eight dwords of every pair of sub-blocks, a bit of each byte moved to bit 4
+// of the nibble's byte. The staged activations and the sums over them are Q4_K's.
+struct FormatQ5K : FormatQ4K {
+  static constexpr int kUnitBytes = 176;
+  static constexpr int kBlockBytes = 176;
+
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    const U32x4* mine = reinterpret_cast<const U32x4*>(at);
+    const U32x4 header = mine[0];
+    const uint32_t s0 = header.y, s1 = header.z, s2 = header.w;
+    const uint32_t sc[2] = {s0 & 0x3F3F3F3Fu, (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u)};
+    const uint32_t mn[2] = {s1 & 0x3F3F3F3Fu, ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u)};
+    const float d = HalfBitsToFloat(header.x & 0xFFFFu);
+    const float dmin = HalfBitsToFloat(header.x >> 16);
+    float main[P];
+#pragma unroll
+    for (int t = 0; t < P; ++t) main[t] = 0.0f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      // Pair p: 32 bytes, the low nibbles sub-block 2p, the high ones 2p + 1; their fifth bits are bits 2p and
+      // 2p + 1 of qh's bytes. With several tokens a pass qh is read again for every pair (the clobber keeps the
+      // compiler from holding its eight dwords beside four tokens' operands).
+      if constexpr (P > 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");
+      }
+      const U32x4 high0 = mine[1], high1 = mine[2];
+      const uint32_t qh[8] = {high0.x, high0.y, high0.z, high0.w, high1.x, high1.y, high1.z, high1.w};
+      int lo[8], hi[8];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const U32x4 raw = mine[3 + 2 * p + i];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t h = qh[4 * i + c];
+          const uint32_t fifth_lo = (2 * p <= 4 ? h << (4 - 2 * p) : h >> (2 * p - 4)) & 0x10101010u;
+          const uint32_t fifth_hi = (2 * p + 1 <= 4 ? h << (3 - 2 * p) : h >> (2 * p - 3)) & 0x10101010u;
+          lo[4 * i + c] = static_cast<int>((raw[c] & 0x0F0F0F0Fu) | fifth_lo);
+          hi[4 * i + c] = static_cast<int>(((raw[c] >> 4) & 0x0F0F0F0Fu) | fifth_hi);
+        }
+      }
+      const float sc0 = ByteToFloat(sc[(2 * p) >> 2], (2 * p) & 3);
+      const float sc1 = ByteToFloat(sc[(2 * p + 1) >> 2], (2 * p + 1) & 3);
+#pragma unroll
+      for (int t = 0; t < P; ++t) {
+        if (t < m) {
+          const uint8_t* record = records + t * token_stride;
+          const uint4* a = reinterpret_cast<const uint4*>(record + p * 64);
+          const uint4 a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];
+          const uint32_t first[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+          const uint32_t second[8] = {a2.x, a2.y, a2.z, a2.w, a3.x, a3.y, a3.z, a3.w};
+          const float2 d8 = *reinterpret_cast<const float2*>(record + 256 + p * 8);
+          int prod0 = 0, prod1 = 0;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            prod0 = Dot4(lo[i], static_cast<int>(first[i]), prod0);
+            prod1 = Dot4(hi[i], static_cast<int>(second[i]), prod1);
+          }
+          if constexpr (P > 1) asm volatile("" : "+v"(prod0), "+v"(prod1));  // taken here: the products stay with their pair
+          if (kDump && dump != nullptr) {
+            dump[2 * p] = prod0;
+            dump[2 * p + 1] = prod1;
+            const int16_t* sums = reinterpret_cast<const int16_t*>(record + 320);
+            dump[8 + 2 * p] = sums[2 * p];
+            dump[8 + 2 * p + 1] = sums[2 * p + 1];
+          }
+          main[t] = fmaf(static_cast<float>(prod0), sc0 * d8.x, main[t]);
+          main[t] = fmaf(static_cast<float>(prod1), sc1 * d8.y, main[t]);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) {
+        const float4* ds = reinterpret_cast<const float4*>(records + t * token_stride + 288);
+        const float4 lo4 = ds[0], hi4 = ds[1];
+        float mins = ByteToFloat(mn[0], 0) * lo4.x;
+        mins = fmaf(ByteToFloat(mn[0], 1), lo4.y, mins);
+        mins = fmaf(ByteToFloat(mn[0], 2), lo4.z, mins);
+        mins = fmaf(ByteToFloat(mn[0], 3), lo4.w, mins);
+        mins = fmaf(ByteToFloat(mn[1], 0), hi4.x, mins);
+        mins = fmaf(ByteToFloat(mn[1], 1), hi4.y, mins);
+        mins = fmaf(ByteToFloat(mn[1], 2), hi4.z, mins);
+        mins = fmaf(ByteToFloat(mn[1], 3), hi4.w, mins);
+        out[t] = fmaf(d, main[t], -(dmin * mins));
+      }
+    }
+  }
+};
+
 // ---- Q8_0: a unit is four blocks
 
 struct FourBlocks {
@@ -1608,6 +1705,13 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
+  if (type == LLMP_TYPE_Q5_K) {
+    const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+    if (at % 16 != 0) return false;
+    const int units = d.ncols_x / FormatQ5K::kUnitValues;
+    if (units > most) return pieces && PlanSplit<FormatQ5K>(units).lds <= kFlatLdsLimit;
+    return units >= 1 && PlanFlat<FormatQ5K>(1, units, glu).lds <= kFlatLdsLimit;
+  }
   if (type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1 ||
       type == LLMP_TYPE_IQ4_NL) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
@@ -1640,6 +1744,8 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
 void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
   if (type == LLMP_TYPE_Q4_K) {
     LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q5_K) {
+    LaunchF<FormatQ5K>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q4_0) {
     LaunchF<FormatQ40>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_IQ4_NL) {

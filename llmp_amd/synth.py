@@ -38,6 +38,20 @@ def q4_k_weights(n, k, seed):
     return out.reshape(n, blocks * 144)
 
 
+def q5_k_weights(n, k, seed):
+    """[n, k/256*176] uint8 of Q5_K super-blocks {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]}:
+    5-bit codes, 6-bit sub-scales and minimums uniform, d and dmin sized as for Q4_K."""
+    g = rng(seed)
+    blocks = k // 256
+    out = np.zeros((n, blocks, 176), dtype=np.uint8)
+    d = (0.02 * g.uniform(5.0, 6.2, size=(n, blocks)) / (63.0 * 31.0)).astype(np.float16)
+    dmin = (0.02 * g.uniform(2.4, 3.2, size=(n, blocks)) / 63.0).astype(np.float16)
+    out[:, :, 0:2] = d.view(np.uint8).reshape(n, blocks, 2)
+    out[:, :, 2:4] = dmin.view(np.uint8).reshape(n, blocks, 2)
+    out[:, :, 4:] = g.integers(0, 256, size=(n, blocks, 172), dtype=np.uint8)
+    return out.reshape(n, blocks * 176)
+
+
 LEGACY_BYTES = {2: 18, 3: 20, 6: 22, 7: 24, 20: 18}  # Q4_0, Q4_1, Q5_0, Q5_1; IQ4_NL (Q4_0's bytes)
 
 
@@ -75,6 +89,8 @@ def random_blocks(t, n, k, seed):
         blocks, size, heads = k // 32, LEGACY_BYTES[t], 2 if t in (3, 7) else 1
     elif t == 8:
         blocks, size, heads = k // 32, 34, 1
+    elif t == 13:
+        blocks, size, heads = k // 256, 176, 2
     else:
         blocks, size, heads = k // 256, 144, 2
     out = g.integers(0, 256, size=(n, blocks, size), dtype=np.uint8)

@@ -234,12 +234,13 @@ int orc_block_bytes(int type) {
     case ORC_TYPE_Q5_1: return 24;
     case ORC_TYPE_Q8_0: return 34;
     case ORC_TYPE_Q4_K: return 144;
+    case ORC_TYPE_Q5_K: return 176; /* encoding.cc:116: {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} */
     case ORC_TYPE_MXFP4: return 17; /* encoding.cc:130-138 */
     case ORC_TYPE_IQ4_NL: return 18; /* {f16 d; u8 nibbles[16]}: Q4_0's bytes */
     default: return 0;
   }
 }
-int orc_block_elements(int type) { return type == ORC_TYPE_Q4_K ? 256 : orc_block_bytes(type) != 0 ? 32 : 0; }
+int orc_block_elements(int type) { return type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K ? 256 : orc_block_bytes(type) != 0 ? 32 : 0; }
 
 static int legacy_affine(int type) { return type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_1; }
 static int legacy_five(int type) { return type == ORC_TYPE_Q5_0 || type == ORC_TYPE_Q5_1; }
@@ -284,6 +285,14 @@ void orc_q4_k_scale_min(const uint8_t* scales, int g, int* scale, int* minimum) 
 static int q4_k_code(const uint8_t* codes, int g, int i) {
   return (codes[(g / 2) * 32 + i] >> ((g % 2) * 4)) & 15; /* dsv4_fast_test.cc:187 */
 }
+/* Q5_K (src/kernels/ggml/vecq.cu:74-75 of the reference reads it through ggml's vec_dot_q5_K_q8_1, which is
+ * not vendored: ggml-quants.c of llama.cpp d812350, dequantize_row_q5_K, restated): Q4_K's header and
+ * nibbles, plus bit g of byte i of qh as the fifth bit of value i of sub-block g. Parity unpinned: the
+ * reference holds no vector for this type. The codes of a block of either type: */
+static int k_code(int type, const uint8_t* w, int g, int i) {
+  if (type == ORC_TYPE_Q5_K) return q4_k_code(w + 48, g, i) + 16 * ((w[16 + i] >> g) & 1);
+  return q4_k_code(w + 16, g, i);
+}
 
 void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
   if (type == ORC_TYPE_MXFP4) { /* decode.cc:239-248 */
@@ -320,9 +329,9 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
     }
     return;
   }
-  /* Q4_K: y = d * sc * code - dmin * m (ggml's dequantize_row_q4_K of these bytes). */
+  /* Q4_K, Q5_K: y = d * sc * code - dmin * m (ggml's dequantize_row_q4_K, _q5_K of these bytes). */
   for (int64_t b = 0; b < k / 256; ++b) {
-    const uint8_t* x = row + b * 144;
+    const uint8_t* x = row + b * orc_block_bytes(type);
     const float d = orc_f16_to_f32(load_u16(x));
     const float dmin = orc_f16_to_f32(load_u16(x + 2));
     for (int g = 0; g < 8; ++g) {
@@ -330,7 +339,7 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
       orc_q4_k_scale_min(x + 4, g, &sc, &m);
       const float d1 = d * (float)sc;
       const float m1 = dmin * (float)m;
-      for (int i = 0; i < 32; ++i) y[b * 256 + g * 32 + i] = d1 * (float)q4_k_code(x + 16, g, i) - m1;
+      for (int i = 0; i < 32; ++i) y[b * 256 + g * 32 + i] = d1 * (float)k_code(type, x, g, i) - m1;
     }
   }
 }
@@ -365,7 +374,7 @@ void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums
     int32_t product = 0, sum = 0;
     for (int i = 0; i < 32; ++i) {
       const int value = (int8_t)a[4 + i];
-      product += q4_k_code(w + 16, g, i) * value;
+      product += k_code(type, w, g, i) * value;
       sum += value;
     }
     sums[g] = product;
@@ -659,7 +668,7 @@ void orc_vecq_block_sums(int type, const void* w, const void* y, int k, int nrow
                          int32_t* out) {
   const int qk = orc_block_elements(type);
   const int bs = orc_block_bytes(type);
-  const int per = type == ORC_TYPE_Q4_K ? 16 : 1;
+  const int per = type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K ? 16 : 1;
   const int blocks = k / qk;
   for (int r = 0; r < nrows; ++r)
     for (int b = 0; b < blocks; ++b)

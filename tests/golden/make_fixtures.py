@@ -56,6 +56,14 @@ def build():
     out["iq4_nl_w"], out["iq4_nl_x"] = wi, a
     out["iq4_nl_y"] = oracle.vecq(oracle.TYPE_IQ4_NL, wi, q8, k, n, tokens=2)
     out["iq4_nl_sums"] = oracle.vecq_block_sums(oracle.TYPE_IQ4_NL, wi, q8[:1], k, n)
+    # llmp.vecq, Q5_K (176-byte super-blocks), 2 tokens.
+    k, n = 512, 10
+    w5 = synth.q5_k_weights(n, k, 28)
+    a = synth.activations(2, k, 29)
+    q8 = oracle.q8_1_quantize(a)
+    out["q5_k_w"], out["q5_k_x"] = w5, a
+    out["q5_k_y"] = oracle.vecq(oracle.TYPE_Q5_K, w5, q8, k, n, tokens=2)
+    out["q5_k_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q5_K, w5, q8[:1], k, n)
     # llmp.vecq, MXFP4 (17-byte blocks), 2 tokens.
     k, n = 512, 12
     wm = synth.mxfp4_weights(n, k, 24)

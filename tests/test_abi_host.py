@@ -66,6 +66,8 @@ def desc(**kw):
     (39, dict(w=0x1004, stride_row=16), "MXFP4"),
     (2, dict(ncols_x=288, stride_row=9), "Q4_0"),
     (20, dict(ncols_x=288, stride_row=9), "IQ4_NL"),
+    (13, dict(w=0x1008), "Q5_K"),
+    (13, dict(ncols_x=288), "whole"),
     (12, dict(used=300), "slots"),
 ])
 def test_vecq_refusals_queue_nothing(t, kw, why):

@@ -343,6 +343,71 @@ def test_q4_0_refuses_what_the_streaming_form_does_not_take(device):
         ops.vecq(Q4_0, dev(synth.legacy_weights(Q4_0, n, 256, 433), device), dev(q8, device), 256, n, variant=0)
 
 
+# ---- Q5_K through the streaming form (a 176-byte super-block a lane)
+
+Q5_K = ops.TYPE_Q5_K
+
+
+@pytest.mark.parametrize("k,n", [(4096, 96), (256, 5), (3840, 33), (15360, 12), (20480, 7)])
+@pytest.mark.parametrize("tokens", [1, 3, 4, 9])
+def test_q5_k_dense_matches_oracle(device, k, n, tokens):
+    """Q4_K's products with a fifth bit a code (src/format/encoding.cc:116, src/kernels/ggml/vecq.cu:74-75 of the
+    reference): rows of one tile, of fewer waves, and in pieces; quantizing in the kernel gives the same bits, and a
+    token's values do not depend on the tokens beside it."""
+    w = synth.q5_k_weights(n, k, 601 + k + n)
+    x = synth.activations(tokens, k, 602 + tokens)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(Q5_K, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(Q5_K, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    fused = ops.vecq_fused(Q5_K, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    alone = ops.vecq(Q5_K, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
+    assert np.array_equal(alone[0].view(np.uint32), got[tokens - 1].view(np.uint32))
+
+
+def test_q5_k_block_sums_and_random_bytes(device):
+    k, n = 2048, 19
+    w = synth.random_blocks(Q5_K, n, k, 611)
+    q8 = oracle.q8_1_quantize(synth.activations(2, k, 612))
+    want = oracle.vecq_block_sums(Q5_K, w, q8[:1], k, n)
+    got = ops.vecq_block_sums(Q5_K, dev(w, device), dev(q8[:1], device), k, n).cpu().numpy()
+    assert np.array_equal(got, want)
+    y = ops.vecq(Q5_K, dev(w, device), dev(q8, device), k, n, tokens=2).cpu().numpy()
+    ok, worst = rel_close(y, oracle.vecq(Q5_K, w, q8, k, n, tokens=2), TOL)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("tokens", [1, 5])
+def test_q5_k_glu_and_routed_match_oracle(device, tokens):
+    k, n, experts, used = 1024, 40, 6, 2
+    gate, up = synth.q5_k_weights(n, k, 621), synth.q5_k_weights(n, k, 622)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 623))
+    want = oracle.vecq(Q5_K, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_GEGLU)
+    got = ops.vecq(Q5_K, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens,
+                   glu=ops.GLU_GEGLU).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    w = synth.q5_k_weights(experts * n, k, 624).reshape(experts, -1)
+    g = synth.rng(625)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    stride_expert = n * (k // 256)
+    want = oracle.vecq(Q5_K, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(Q5_K, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+def test_q5_k_refuses_the_other_forms(device):
+    k, n = 512, 8
+    w = synth.q5_k_weights(n, k, 631)
+    q8 = oracle.q8_1_quantize(synth.activations(1, k, 632))
+    with pytest.raises(ops.KernelFailure):  # the rows form has no Q5_K
+        ops.vecq(Q5_K, dev(w, device), dev(q8, device), k, n, variant=0)
+
+
 # ---- MXFP4 through the streaming form (eight 17-byte blocks a lane)
 
 MXFP4 = ops.TYPE_MXFP4

@@ -177,6 +177,69 @@ def test_q4_k_and_q8_0_decode_and_block_sums_by_brute_force():
             np.testing.assert_allclose(y[r], float(np.dot(want, act)), rtol=2e-6, atol=1e-9)
 
 
+def test_q5_k_decode_sums_and_products_by_brute_force_and_known_answers():
+    """Q5_K (src/format/encoding.cc:116 of the reference: 256 values in 176 bytes; ggml's dequantize_row_q5_K):
+    Q4_K's header and nibbles after 32 bytes whose bit g of byte i is the fifth bit of value i of sub-block g.
+    Parity unpinned: ggml is not vendored and the reference holds no Q5_K vector; this pins the oracle's C against
+    numpy's reading of the published layout, the fifth bits alone against Q4_K (a block with qh = 0 is the Q4_K
+    block of the same header and nibbles; with qh = 0xFF every code is 16 more), and a hand-built block."""
+    from llmp_amd import synth
+    t, k, n = oracle.TYPE_Q5_K, 512, 5
+    assert oracle.block_bytes(t) == 176 and oracle.block_elements(t) == 256
+    w = synth.random_blocks(t, n, k, 71)
+    x = np.random.Generator(np.random.PCG64(72)).standard_normal((1, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    a = q8[0].reshape(-1, 36)
+    aq = a[:, 4:].view(np.int8).astype(np.int64)
+    ad = a[:, 0:2].view(np.float16).astype(np.float64).reshape(-1)
+    dec, sums, y = oracle.decode_rows(t, w, k), oracle.vecq_block_sums(t, w, q8, k, n), oracle.vecq(t, w, q8, k, n)[0, 0]
+    for r in range(n):
+        rows, codes = [], []
+        for b in w[r].reshape(-1, 176):
+            four = np.concatenate([b[0:16], b[48:176]])           # the Q4_K block of the same header and nibbles
+            base = q4_k_decode_numpy(four)
+            d = float(b[0:2].view(np.float16)[0])
+            s = b[4:16].astype(int)
+            for g in range(8):
+                sc = s[g] & 63 if g < 4 else (s[g + 4] & 15) | ((s[g - 4] >> 6) << 4)
+                fifth = (b[16:48].astype(int) >> g) & 1
+                base[g * 32:(g + 1) * 32] += d * sc * 16.0 * fifth
+                codes.append(((b[48:].astype(int)[(g // 2) * 32:(g // 2) * 32 + 32] >> (4 * (g % 2))) & 15) + 16 * fifth)
+            rows.append(base)
+        want = np.concatenate(rows)
+        np.testing.assert_allclose(dec[r], want, rtol=1e-5, atol=1e-9)
+        prod = (np.stack(codes) * aq[:k // 32]).sum(axis=1).reshape(-1, 8)
+        assert np.array_equal(sums[r, :, :8], prod)
+        assert np.array_equal(sums[r, :, 8:], aq[:k // 32].sum(axis=1).reshape(-1, 8))
+        act = (aq[:k // 32] * ad[:k // 32, None]).reshape(-1)
+        np.testing.assert_allclose(y[r], float(np.dot(want, act)), rtol=2e-6, atol=1e-9)
+    # qh = 0: the Q4_K block; qh = 0xFF: every code 16 more.
+    five = synth.random_blocks(t, 1, 256, 73)
+    five[0, 16:48] = 0
+    four = np.concatenate([five[0, 0:16], five[0, 48:176]])[None, :]
+    assert np.array_equal(oracle.decode_rows(t, five, 256), oracle.decode_rows(oracle.TYPE_Q4_K, four, 256))
+    q1 = oracle.q8_1_quantize(x[:, :256])
+    low = oracle.vecq_block_sums(t, five, q1, 256, 1)
+    assert np.array_equal(low, oracle.vecq_block_sums(oracle.TYPE_Q4_K, four, q1, 256, 1))
+    five[0, 16:48] = 0xFF
+    high = oracle.vecq_block_sums(t, five, q1, 256, 1)
+    assert np.array_equal(high[0, 0, :8], low[0, 0, :8] + 16 * low[0, 0, 8:])
+    # Hand-built: d = 1, dmin = 0, every sub-scale 1 (bytes 4..7 = 1, bytes 12..15 = 1), nibbles 3, the fifth bit of
+    # sub-block 2 alone set: its values 19, all others 3. Every q = 1 with d8 = 0.5: 0.5 * (7 * 96 + 608) = 640.
+    b = np.zeros((1, 176), dtype=np.uint8)
+    b[0, 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    b[0, 4:8], b[0, 12:16] = 1, 1
+    b[0, 16:48] = 1 << 2
+    b[0, 48:] = 0x33
+    got = oracle.decode_rows(t, b, 256)[0]
+    assert np.array_equal(got, np.where((np.arange(256) // 32) == 2, 19.0, 3.0))
+    q = np.zeros((1, 8 * 36), dtype=np.uint8)
+    for g in range(8):
+        q[0, g * 36:g * 36 + 2] = np.array([0.5], dtype=np.float16).view(np.uint8)
+        q[0, g * 36 + 4:g * 36 + 36] = 1
+    assert oracle.vecq(t, b, q, 256, 1)[0, 0, 0] == 640.0
+
+
 def legacy_block_numpy(t, block, a):
     """tests/unit/dsv4_fast_test.cc:141-164 restated with numpy, apart from the oracle's C:
     (codes, int sum, product) of one legacy block and one Q8_1 block."""
