@@ -236,7 +236,7 @@ def block_formats(device):
     q8 = ops.quantize_q8_1(dev(synth.activations(1, k, 301)))
     y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
     names = {ops.TYPE_Q4_0: "q4_0", ops.TYPE_Q4_1: "q4_1", ops.TYPE_Q5_0: "q5_0", ops.TYPE_Q5_1: "q5_1",
-             ops.TYPE_Q8_0: "q8_0", ops.TYPE_Q4_K: "q4_k", ops.TYPE_MXFP4: "mxfp4", ops.TYPE_IQ4_NL: "iq4_nl", ops.TYPE_Q5_K: "q5_k"}
+             ops.TYPE_Q8_0: "q8_0", ops.TYPE_Q4_K: "q4_k", ops.TYPE_MXFP4: "mxfp4", ops.TYPE_IQ4_NL: "iq4_nl", ops.TYPE_Q5_K: "q5_k", ops.TYPE_Q6_K: "q6_k"}
     for t, name in names.items():
         if t == ops.TYPE_Q4_K:
             make = lambda seed: synth.q4_k_weights(n, k, seed)
@@ -246,6 +246,8 @@ def block_formats(device):
             make = lambda seed: synth.mxfp4_weights(n, k, seed)
         elif t == ops.TYPE_Q5_K:
             make = lambda seed: synth.q5_k_weights(n, k, seed)
+        elif t == ops.TYPE_Q6_K:
+            make = lambda seed: synth.q6_k_weights(n, k, seed)
         else:
             make = lambda seed, t=t: synth.legacy_weights(t, n, k, seed)
         gate, up = dev(make(302)), dev(make(303))

@@ -26,7 +26,9 @@
  * Q4_0's 18 bytes with each nibble an index into ggml's codebook of sixteen int8 values, a value d times the
  * entry (src/format/encoding.cc:126, src/kernels/ggml/vecq.cu:375-396); Q5_K is {f16 d; f16 dmin; u8 scales[12];
  * u8 qh[32]; u8 qs[128]} = 176 bytes, Q4_K with bit g of qh's byte i as the fifth bit of value i of sub-block g
- * (src/format/encoding.cc:116).
+ * (src/format/encoding.cc:116); Q6_K is {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} = 210 bytes, value
+ * 128 h + 32 t + l the nibble t / 2 of ql[64 h + 32 (t % 2) + l] plus 16 times bits 2t, 2t + 1 of qh[32 h + l], minus 32,
+ * times scales[value / 16] times d (src/format/encoding.cc:117).
  */
 #ifndef LLMP_HIP_H_
 #define LLMP_HIP_H_
@@ -39,7 +41,7 @@ extern "C" {
 #endif
 
 /* ggml_type values of the weight encodings the kernels read. */
-enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12, LLMP_TYPE_MXFP4 = 39, LLMP_TYPE_IQ4_NL = 20, LLMP_TYPE_Q5_K = 13 };
+enum { LLMP_TYPE_Q4_0 = 2, LLMP_TYPE_Q4_1 = 3, LLMP_TYPE_Q5_0 = 6, LLMP_TYPE_Q5_1 = 7, LLMP_TYPE_Q8_0 = 8, LLMP_TYPE_Q4_K = 12, LLMP_TYPE_MXFP4 = 39, LLMP_TYPE_IQ4_NL = 20, LLMP_TYPE_Q5_K = 13, LLMP_TYPE_Q6_K = 14 };
 /* VecQGlu, src/kernels/ggml/llmp_ops.h:1072. */
 enum { LLMP_GLU_NONE = 0, LLMP_GLU_SWIGLU = 1, LLMP_GLU_SWIGLU_CLAMP = 2, LLMP_GLU_GEGLU = 3 };
 /* Element types of unquantized activations. */

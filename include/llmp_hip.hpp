@@ -38,7 +38,8 @@ enum Type : int {
   kQ4_K = LLMP_TYPE_Q4_K,
   kMXFP4 = LLMP_TYPE_MXFP4,
   kIQ4_NL = LLMP_TYPE_IQ4_NL,
-  kQ5_K = LLMP_TYPE_Q5_K
+  kQ5_K = LLMP_TYPE_Q5_K,
+  kQ6_K = LLMP_TYPE_Q6_K
 };
 // VecQGlu, src/kernels/ggml/llmp_ops.h:1072.
 enum VecQGlu : int { kNone = LLMP_GLU_NONE, kSwiGlu = LLMP_GLU_SWIGLU, kSwiGluClamp = LLMP_GLU_SWIGLU_CLAMP, kGeGlu = LLMP_GLU_GEGLU };

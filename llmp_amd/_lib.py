@@ -18,6 +18,7 @@ TYPE_Q4_K = 12
 TYPE_MXFP4 = 39
 TYPE_IQ4_NL = 20
 TYPE_Q5_K = 13
+TYPE_Q6_K = 14
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
 X_F32, X_BF16, X_F16 = 0, 1, 2
 

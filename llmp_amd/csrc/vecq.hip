@@ -586,9 +586,10 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (d == nullptr) return Refuse(1, "vecq: null descriptor");
   const bool legacy = type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1 ||
                       type == LLMP_TYPE_IQ4_NL;  // 18-byte blocks as Q4_0's
-  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_Q5_K && type != LLMP_TYPE_MXFP4 && !legacy)
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && type != LLMP_TYPE_Q5_K && type != LLMP_TYPE_Q6_K && type != LLMP_TYPE_MXFP4 &&
+      !legacy)
     return Refuse(1, "vecq: weight type %d has no kernel", type);
-  const int qk = type == LLMP_TYPE_Q4_K || type == LLMP_TYPE_Q5_K ? 256 : 32;
+  const int qk = type == LLMP_TYPE_Q4_K || type == LLMP_TYPE_Q5_K || type == LLMP_TYPE_Q6_K ? 256 : 32;
   if (d->w == nullptr || d->dst == nullptr) return Refuse(1, "vecq: null weights or output");
   if (d->ncols_x <= 0 || d->ncols_x % qk != 0) return Refuse(1, "vecq: k %d is not whole %d-value blocks", d->ncols_x, qk);
   if (d->nrows <= 0) return Refuse(1, "vecq: no rows");
@@ -604,6 +605,9 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   if (reinterpret_cast<uintptr_t>(d->dst) % 4 != 0) return Refuse(1, "vecq: output not 4-byte aligned");
   const uintptr_t wa = reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g);
   if (type == LLMP_TYPE_Q4_K && wa % 16 != 0) return Refuse(1, "vecq: Q4_K weights not 16-byte aligned");
+  if (type == LLMP_TYPE_Q6_K && !FlatTakes(type, *d))
+    return Refuse(1, "vecq: Q6_K takes 16-byte aligned weights, rows up to 16384 values (8192 with a GLU) of which some number "
+                     "fills a tile of 64 lanes (32) with a multiple of eight blocks, matrices and experts of a multiple of eight blocks");
   // Q5_K runs through the flat form alone.
   if (type == LLMP_TYPE_Q5_K && !FlatTakes(type, *d))
     return Refuse(1, "vecq: Q5_K takes 16-byte aligned weights and rows whose staged activations fit LDS (up to 8192 values "
@@ -643,7 +647,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (variant >= kVariantCount) return Refuse(1, "vecq: no variant %d", variant);
   const Variant& v = kVariants[variant];
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && v.lanes != 0)
-    return Refuse(1, "vecq: the legacy 4/5-bit blocks, IQ4_NL, Q5_K and MXFP4 take the flat variants");
+    return Refuse(1, "vecq: the legacy 4/5-bit blocks, IQ4_NL, Q5_K, Q6_K and MXFP4 take the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
   if (v.lanes < 0) {
     if (!MmaTakes(type, *d))

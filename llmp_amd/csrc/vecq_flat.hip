@@ -342,6 +342,98 @@ struct FormatQ5K : FormatQ4K {
   }
 };
 
+// ---- Q6_K: {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} = 210 bytes, 256 values
+//
+// src/format/encoding.cc:117 of the reference; ggml's dequantize_row_q6_K: value 128 h + 32 t + l (h < 2, t < 4,
+// l < 32) is the low (t < 2) or high nibble of ql[64 h + 32 (t & 1) + l] plus 16 times bits 2t, 2t + 1 of
+// qh[32 h + l], minus 32, times scales[value / 16] times d. A block is not a whole number of dwords: a tile is
+// fetched as the same 16-byte chunks (FlatPlan makes a tile's units a multiple of eight, 1680 bytes), a lane's unit
+// then starts 0 or 2 bytes into a dword and every dword it uses is put together from two (v_alignbyte). Codes
+// become signed bytes without a subtraction a byte: x + 0x60 cannot carry for x < 64, and flipping bit 7 of that is
+// x - 32. The staged activations are Q4_K's (the codes in order, d8 a block).
+struct FormatQ6K : FormatQ4K {
+  static constexpr int kUnitBytes = 210;
+  static constexpr int kBlockBytes = 210;
+  static constexpr int kDumpInts = 16;  // the sixteen sub-blocks' sums
+
+  template <int P, bool kDump>
+  static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
+                                               float (&out)[P], int32_t* dump) {
+#pragma clang fp contract(off)
+    const uint32_t shift = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(at)) & 3u;
+    const uint32_t* base = reinterpret_cast<const uint32_t*>(at - shift);
+    // Dwords first .. first + N - 1 of the unit.
+    auto take = [&](int first, auto& dst) {
+      constexpr int N = sizeof(dst) / sizeof(uint32_t);
+      uint32_t raw[N + 1];
+#pragma unroll
+      for (int i = 0; i <= N; ++i) raw[i] = base[first + i];
+#pragma unroll
+      for (int i = 0; i < N; ++i) dst[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], shift);
+    };
+    uint32_t tail[5];  // the sixteen scales, d
+    take(48, tail);
+    const float d = HalfBitsToFloat(tail[4] & 0xFFFFu);
+    float v[P];
+#pragma unroll
+    for (int t = 0; t < P; ++t) v[t] = 0.0f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // One token a pass: the half's 96 bytes at once. Several: a block's 64 at a time, read again for every block
+      // (the clobber keeps the compiler from holding them beside four tokens' operands).
+      uint32_t ql[P > 1 ? 8 : 16], qh[8];
+      if constexpr (P == 1) {
+        take(16 * h, ql);
+        take(32 + 8 * h, qh);
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int block = 4 * h + g;  // of 32 values: two sub-blocks
+        if constexpr (P > 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          asm volatile("" ::: "memory");
+          take(16 * h + 8 * (g & 1), ql);
+          take(32 + 8 * h, qh);
+        }
+        int value[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t low = ql[(P > 1 ? 0 : 8 * (g & 1)) + j];
+          const uint32_t nibbles = (g >> 1) ? (low >> 4) & 0x0F0F0F0Fu : low & 0x0F0F0F0Fu;
+          const uint32_t high = (2 * g <= 4 ? qh[j] << (4 - 2 * g) : qh[j] >> (2 * g - 4)) & 0x30303030u;
+          value[j] = static_cast<int>(((nibbles | high) + 0x60606060u) ^ 0x80808080u);
+        }
+        const uint32_t both = tail[block >> 1] >> (16 * (block & 1));
+        const int sc0 = static_cast<int8_t>(both & 0xFFu), sc1 = static_cast<int8_t>((both >> 8) & 0xFFu);
+#pragma unroll
+        for (int t = 0; t < P; ++t) {
+          if (t < m) {
+            const uint8_t* record = records + t * token_stride;
+            const uint4* a = reinterpret_cast<const uint4*>(record + block * 32);
+            const uint4 a0 = a[0], a1 = a[1];
+            int first = Dot4(value[0], static_cast<int>(a0.x), 0);
+            first = Dot4(value[1], static_cast<int>(a0.y), first);
+            first = Dot4(value[2], static_cast<int>(a0.z), first);
+            first = Dot4(value[3], static_cast<int>(a0.w), first);
+            int second = Dot4(value[4], static_cast<int>(a1.x), 0);
+            second = Dot4(value[5], static_cast<int>(a1.y), second);
+            second = Dot4(value[6], static_cast<int>(a1.z), second);
+            second = Dot4(value[7], static_cast<int>(a1.w), second);
+            if constexpr (P > 1) asm volatile("" : "+v"(first), "+v"(second));  // taken here: the products stay with their block
+            if (kDump && dump != nullptr) dump[2 * block] = first, dump[2 * block + 1] = second;
+            const float d8 = reinterpret_cast<const float*>(record + 256)[block];
+            v[t] = fmaf(d8, static_cast<float>(sc0 * first + sc1 * second), v[t]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < P; ++t) {
+      if (t < m) out[t] = d * v[t];
+    }
+  }
+};
+
 // ---- Q8_0: a unit is four blocks
 
 struct FourBlocks {
@@ -1536,10 +1628,16 @@ template <class F>
 FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   FlatPlan p;
   p.rows = (glu ? kWave / 2 : kWave) / units;
+  // Units that are not whole 16-byte chunks: a tile is a multiple of eight of them (none, if no such tile fits),
+  // and a lane reads up to six bytes past its unit.
+  constexpr bool kOdd = F::kUnitBytes % 16 != 0;
+  if constexpr (kOdd) {
+    while (p.rows > 0 && (p.rows * units) % 8 != 0) --p.rows;
+  }
   p.waves = kWaves;
   for (;;) {
     p.lds = ((static_cast<size_t>(pass) * units * F::kRecord + 15) & ~static_cast<size_t>(15)) +
-            static_cast<size_t>(deep ? 2 : 1) * p.waves * kWave * F::kUnitBytes;
+            static_cast<size_t>(deep ? 2 : 1) * p.waves * kWave * F::kUnitBytes + (kOdd ? 16 : 0);
     if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
     --p.waves;
   }
@@ -1705,6 +1803,16 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
+  if (type == LLMP_TYPE_Q6_K) {
+    // 210-byte blocks: tiles of a multiple of eight units, everything at 16-byte boundaries.
+    const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
+    const int units = d.ncols_x / FormatQ6K::kUnitValues;
+    if (at % 16 != 0 || d.stride_expert % 8 != 0 || units < 1 || units > most) return false;
+    if (d.stride_row != units && (units % 8 != 0 || d.stride_row % 8 != 0)) return false;
+    const FlatPlan plan = PlanFlat<FormatQ6K>(1, units, glu);
+    // Full tiles are whole chunks; so is the last, shorter one if all the rows' blocks are a multiple of eight.
+    return plan.rows >= 1 && (static_cast<int64_t>(d.nrows) * units) % 8 == 0 && plan.lds <= kFlatLdsLimit;
+  }
   if (type == LLMP_TYPE_Q5_K) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
     if (at % 16 != 0) return false;
@@ -1746,6 +1854,8 @@ void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hi
     LaunchF<FormatQ4K>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q5_K) {
     LaunchF<FormatQ5K>(a, x_type, pass, deep, stream);
+  } else if (type == LLMP_TYPE_Q6_K) {
+    LaunchF<FormatQ6K>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_Q4_0) {
     LaunchF<FormatQ40>(a, x_type, pass, deep, stream);
   } else if (type == LLMP_TYPE_IQ4_NL) {

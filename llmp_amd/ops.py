@@ -8,12 +8,12 @@ import torch
 
 from . import _lib
 from ._lib import (GLU_GEGLU, GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, TYPE_Q4_0, TYPE_Q4_1, TYPE_Q4_K,  # noqa: F401
-                   TYPE_IQ4_NL, TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1, TYPE_Q5_K,
+                   TYPE_IQ4_NL, TYPE_MXFP4, TYPE_Q5_0, TYPE_Q5_1, TYPE_Q5_K, TYPE_Q6_K,
                    TYPE_Q8_0, X_BF16, X_F16, X_F32, DecodeOperand, Exl3Linear, Exl3MultiLinear, Exl3Weights, KernelFailure, Mxfp8Gemm, VecQDesc,
                    VecQSource)
 
-BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18, TYPE_Q5_K: 176}
-BLOCK_ELEMENTS = {TYPE_Q4_0: 32, TYPE_Q4_1: 32, TYPE_Q5_0: 32, TYPE_Q5_1: 32, TYPE_Q8_0: 32, TYPE_Q4_K: 256, TYPE_MXFP4: 32, TYPE_IQ4_NL: 32, TYPE_Q5_K: 256}
+BLOCK_BYTES = {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18, TYPE_Q5_K: 176, TYPE_Q6_K: 210}
+BLOCK_ELEMENTS = {TYPE_Q4_0: 32, TYPE_Q4_1: 32, TYPE_Q5_0: 32, TYPE_Q5_1: 32, TYPE_Q8_0: 32, TYPE_Q4_K: 256, TYPE_MXFP4: 32, TYPE_IQ4_NL: 32, TYPE_Q5_K: 256, TYPE_Q6_K: 256}
 
 
 def padded_k(k):
@@ -100,7 +100,7 @@ def vecq_fused(t, w, x, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stri
 def vecq_block_sums(t, w, q8, k, nrows, variant=-1):
     """The kernel's int32 block sums of a dense one-token product: [nrows, blocks, per]."""
     lib = _lib.load()
-    per = 16 if t in (TYPE_Q4_K, TYPE_Q5_K) else 1
+    per = 16 if t in (TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K) else 1
     sums = torch.zeros((nrows, k // BLOCK_ELEMENTS[t], per), dtype=torch.int32, device=w.device)
     out = torch.empty((1, 1, nrows), dtype=torch.float32, device=w.device)
     d = _desc(t, w, k, nrows, gate=None, q8=q8, ids=None, tokens=1, used=1, stride_row=None,

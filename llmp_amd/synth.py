@@ -52,6 +52,17 @@ def q5_k_weights(n, k, seed):
     return out.reshape(n, blocks * 176)
 
 
+def q6_k_weights(n, k, seed):
+    """[n, k/256*210] uint8 of Q6_K super-blocks {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}: 6-bit codes and
+    int8 sub-scales uniform, d sized so that d * 127 * 32 spans the range of 256 draws of N(0, 0.02)."""
+    g = rng(seed)
+    blocks = k // 256
+    out = g.integers(0, 256, size=(n, blocks, 210), dtype=np.uint8)
+    d = (0.02 * g.uniform(5.0, 6.2, size=(n, blocks)) / (127.0 * 32.0)).astype(np.float16)
+    out[:, :, 208:210] = d.view(np.uint8).reshape(n, blocks, 2)
+    return out.reshape(n, blocks * 210)
+
+
 LEGACY_BYTES = {2: 18, 3: 20, 6: 22, 7: 24, 20: 18}  # Q4_0, Q4_1, Q5_0, Q5_1; IQ4_NL (Q4_0's bytes)
 
 
@@ -91,6 +102,11 @@ def random_blocks(t, n, k, seed):
         blocks, size, heads = k // 32, 34, 1
     elif t == 13:
         blocks, size, heads = k // 256, 176, 2
+    elif t == 14:
+        out = rng(seed).integers(0, 256, size=(n, k // 256, 210), dtype=np.uint8)
+        scale = rng(seed + 1).uniform(-4.0, 4.0, size=(n, k // 256, 1)).astype(np.float16)
+        out[:, :, 208:210] = scale.view(np.uint8).reshape(n, k // 256, 2)
+        return out.reshape(n, k // 256 * 210)
     else:
         blocks, size, heads = k // 256, 144, 2
     out = g.integers(0, 256, size=(n, blocks, size), dtype=np.uint8)

@@ -21,6 +21,7 @@ TYPE_Q4_K = 12
 TYPE_MXFP4 = 39
 TYPE_IQ4_NL = 20
 TYPE_Q5_K = 13
+TYPE_Q6_K = 14
 GLU_NONE, GLU_SWIGLU, GLU_SWIGLU_CLAMP, GLU_GEGLU = 0, 1, 2, 3
 CB_3INST, CB_MCG, CB_MUL1 = 0, 1, 2
 Q8_DEVICE, Q8_GGML_CPU = 0, 1
@@ -107,11 +108,11 @@ def max_threads():
 
 
 def block_bytes(t):
-    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18, TYPE_Q5_K: 176}[t]
+    return {TYPE_Q4_0: 18, TYPE_Q4_1: 20, TYPE_Q5_0: 22, TYPE_Q5_1: 24, TYPE_Q8_0: 34, TYPE_Q4_K: 144, TYPE_MXFP4: 17, TYPE_IQ4_NL: 18, TYPE_Q5_K: 176, TYPE_Q6_K: 210}[t]
 
 
 def block_elements(t):
-    return 256 if t in (TYPE_Q4_K, TYPE_Q5_K) else 32
+    return 256 if t in (TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K) else 32
 
 
 def padded_k(k):
@@ -184,7 +185,7 @@ def vecq(t, w, q8, k, nrows, *, gate=None, ids=None, tokens=1, used=1, stride_ro
 
 def vecq_block_sums(t, w, q8, k, nrows):
     qk = block_elements(t)
-    per = 16 if t in (TYPE_Q4_K, TYPE_Q5_K) else 1
+    per = 16 if t in (TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K) else 1
     w = np.ascontiguousarray(w, dtype=np.uint8)
     q8 = np.ascontiguousarray(q8, dtype=np.uint8)
     out = np.zeros((nrows, k // qk, per), dtype=np.int32)

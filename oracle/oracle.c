@@ -234,13 +234,14 @@ int orc_block_bytes(int type) {
     case ORC_TYPE_Q5_1: return 24;
     case ORC_TYPE_Q8_0: return 34;
     case ORC_TYPE_Q4_K: return 144;
+    case ORC_TYPE_Q6_K: return 210; /* encoding.cc:117: {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} */
     case ORC_TYPE_Q5_K: return 176; /* encoding.cc:116: {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} */
     case ORC_TYPE_MXFP4: return 17; /* encoding.cc:130-138 */
     case ORC_TYPE_IQ4_NL: return 18; /* {f16 d; u8 nibbles[16]}: Q4_0's bytes */
     default: return 0;
   }
 }
-int orc_block_elements(int type) { return type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K ? 256 : orc_block_bytes(type) != 0 ? 32 : 0; }
+int orc_block_elements(int type) { return type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K || type == ORC_TYPE_Q6_K ? 256 : orc_block_bytes(type) != 0 ? 32 : 0; }
 
 static int legacy_affine(int type) { return type == ORC_TYPE_Q4_1 || type == ORC_TYPE_Q5_1; }
 static int legacy_five(int type) { return type == ORC_TYPE_Q5_0 || type == ORC_TYPE_Q5_1; }
@@ -255,6 +256,17 @@ static int legacy_code(int type, const uint8_t* w, int i) {
   const uint8_t* codes = w + prefix + (legacy_five(type) ? 4 : 0);
   const int low = i < 16 ? codes[i] & 15 : codes[i - 16] >> 4;
   return low + (legacy_five(type) ? (int)((high >> i) & 1u) * 16 : 0);
+}
+
+/* Q6_K (src/kernels/ggml/vecq.cu:76-77 of the reference reads it through ggml's vec_dot_q6_K_q8_1, which is not
+ * vendored: ggml-quants.c of llama.cpp d812350, dequantize_row_q6_K, restated): value v = 128 h + 32 t + l of a block is
+ * nibble t / 2 of ql[64 h + 32 (t % 2) + l] plus 16 times bits 2t, 2t + 1 of qh[32 h + l], minus 32; it is scaled by
+ * scales[v / 16] (int8) and d. Parity unpinned: the reference holds no vector for this type. */
+static int q6_k_value(const uint8_t* w, int v) {
+  const int h = v / 128, t = (v % 128) / 32, l = v % 32;
+  const int low = w[64 * h + 32 * (t % 2) + l];
+  const int nibble = t / 2 ? low >> 4 : low & 15;
+  return (nibble | (((w[128 + 32 * h + l] >> (2 * t)) & 3) << 4)) - 32;
 }
 
 /* IQ4_NL (src/kernels/ggml/vecq.cu:375-396 of the reference reads it through ggml's
@@ -299,6 +311,14 @@ void orc_decode_row(int type, const uint8_t* row, int64_t k, float* y) {
     for (int64_t j = 0; j < k; ++j) {
       const uint8_t* x = row + j / 32 * 17;
       y[j] = orc_e2m1_to_f32((uint8_t)mxfp4_code(x, (int)(j % 32))) * orc_e8m0_to_f32(x[0]);
+    }
+    return;
+  }
+  if (type == ORC_TYPE_Q6_K) {
+    for (int64_t j = 0; j < k; ++j) {
+      const uint8_t* x = row + j / 256 * 210;
+      const int v = (int)(j % 256);
+      y[j] = orc_f16_to_f32(load_u16(x + 208)) * (float)(int8_t)x[192 + v / 16] * (float)q6_k_value(x, v);
     }
     return;
   }
@@ -351,6 +371,14 @@ void orc_block_sums(int type, const uint8_t* w, const uint8_t* q8, int32_t* sums
     sums[0] = s;
     return;
   }
+  if (type == ORC_TYPE_Q6_K) { /* the sixteen sub-blocks' sums of value times code */
+    for (int j = 0; j < 16; ++j) {
+      int32_t s = 0;
+      for (int i = 0; i < 16; ++i) s += q6_k_value(w, 16 * j + i) * (int32_t)(int8_t)q8[(j / 2) * 36 + 4 + (j % 2) * 16 + i];
+      sums[j] = s;
+    }
+    return;
+  }
   if (type == ORC_TYPE_IQ4_NL) { /* vecq.cu:379-392: the codebook's values times the codes */
     int32_t s = 0;
     for (int i = 0; i < 32; ++i) s += iq4_nl_value(w, i) * (int32_t)(int8_t)q8[4 + i];
@@ -387,6 +415,14 @@ double orc_block_product(int type, const uint8_t* w, const uint8_t* q8) {
   orc_block_sums(type, w, q8, sums);
   if (type == ORC_TYPE_MXFP4) { /* vecq.cu:426,437: half the block's scale, times d8, times the sum */
     return (double)orc_e8m0_to_f32(w[0]) * 0.5 * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
+  }
+  if (type == ORC_TYPE_Q6_K) { /* d * sum over the eight activation blocks of d8 * (sc * sum, both sub-blocks) */
+    double total = 0;
+    for (int b = 0; b < 8; ++b) {
+      const double d8 = orc_f16_to_f32(load_u16(q8 + b * 36));
+      total += d8 * ((double)(int8_t)w[192 + 2 * b] * sums[2 * b] + (double)(int8_t)w[192 + 2 * b + 1] * sums[2 * b + 1]);
+    }
+    return (double)orc_f16_to_f32(load_u16(w + 208)) * total;
   }
   if (type == ORC_TYPE_IQ4_NL) { /* vecq.cu:394-395: dw * d8, times the sum */
     return (double)orc_f16_to_f32(load_u16(w)) * (double)orc_f16_to_f32(load_u16(q8)) * (double)sums[0];
@@ -668,7 +704,7 @@ void orc_vecq_block_sums(int type, const void* w, const void* y, int k, int nrow
                          int32_t* out) {
   const int qk = orc_block_elements(type);
   const int bs = orc_block_bytes(type);
-  const int per = type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K ? 16 : 1;
+  const int per = type == ORC_TYPE_Q4_K || type == ORC_TYPE_Q5_K || type == ORC_TYPE_Q6_K ? 16 : 1;
   const int blocks = k / qk;
   for (int r = 0; r < nrows; ++r)
     for (int b = 0; b < blocks; ++b)

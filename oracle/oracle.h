@@ -21,7 +21,7 @@
  * in the reference tree; no in-tree fixture fixes them. Flavor 0 here is the
  * device definition (IEEE divide, butterfly-ordered sum), flavor 1 the ggml CPU
  * definition (multiply by the reciprocal, s = d * sum(q)).
- * parity unpinned as well: Q5_K's bit layout (ggml's dequantize_row_q5_K restated; no vector in the
+ * parity unpinned as well: Q6_K's and Q5_K's bit layouts (ggml's dequantize_row_q6_K, _q5_K restated; no vector in the
  * reference), pinned only against numpy's reading of the same published layout; the IQ4_NL codebook (ggml's kvalues_iq4nl, restated from llama.cpp's
  * ggml-common.h; the reference reads it from ggml and holds no vector for the type). Its layout and
  * arithmetic are pinned against numpy and a hand-built block.
@@ -62,9 +62,9 @@ void orc_q8_1_decode_row(const uint8_t* blocks, int64_t k, float* y);
 void orc_kv_quantize_row(int type, const float* x, int64_t k, uint8_t* out);
 
 /* ---- weight blocks: src/format/encoding.cc:110-116 ---- */
-enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12, ORC_TYPE_MXFP4 = 39, ORC_TYPE_IQ4_NL = 20, ORC_TYPE_Q5_K = 13 }; /* ggml_type values */
-int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144, MXFP4 17, IQ4_NL 18, Q5_K 176 */
-int orc_block_elements(int type); /* 32, Q4_K and Q5_K 256 */
+enum { ORC_TYPE_Q4_0 = 2, ORC_TYPE_Q4_1 = 3, ORC_TYPE_Q5_0 = 6, ORC_TYPE_Q5_1 = 7, ORC_TYPE_Q8_0 = 8, ORC_TYPE_Q4_K = 12, ORC_TYPE_MXFP4 = 39, ORC_TYPE_IQ4_NL = 20, ORC_TYPE_Q5_K = 13, ORC_TYPE_Q6_K = 14 }; /* ggml_type values */
+int orc_block_bytes(int type);    /* 18 / 20 / 22 / 24 / 34 / 144, MXFP4 17, IQ4_NL 18, Q5_K 176, Q6_K 210 */
+int orc_block_elements(int type); /* 32, the K-quants 256 */
 /* The Q4_K 6-bit scale and minimum of sub-block g: tests/unit/dsv4_fast_test.cc:180-183. */
 void orc_q4_k_scale_min(const uint8_t* scales12, int g, int* scale, int* minimum);
 /* Decode rows of blocks to floats (the ggml dequantization of those bytes). */

@@ -64,6 +64,14 @@ def build():
     out["q5_k_w"], out["q5_k_x"] = w5, a
     out["q5_k_y"] = oracle.vecq(oracle.TYPE_Q5_K, w5, q8, k, n, tokens=2)
     out["q5_k_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q5_K, w5, q8[:1], k, n)
+    # llmp.vecq, Q6_K (210-byte super-blocks), 2 tokens.
+    k, n = 512, 12
+    w6 = synth.q6_k_weights(n, k, 30)
+    a = synth.activations(2, k, 31)
+    q8 = oracle.q8_1_quantize(a)
+    out["q6_k_w"], out["q6_k_x"] = w6, a
+    out["q6_k_y"] = oracle.vecq(oracle.TYPE_Q6_K, w6, q8, k, n, tokens=2)
+    out["q6_k_sums"] = oracle.vecq_block_sums(oracle.TYPE_Q6_K, w6, q8[:1], k, n)
     # llmp.vecq, MXFP4 (17-byte blocks), 2 tokens.
     k, n = 512, 12
     wm = synth.mxfp4_weights(n, k, 24)

@@ -94,6 +94,12 @@ def test_device_meets_the_committed_vectors(vectors, device):
     q8 = ops.quantize_q8_1(_dev(v["q5_k_x"], device))
     close(ops.vecq(ops.TYPE_Q5_K, w, q8, k, n, tokens=2).cpu().numpy(), v["q5_k_y"], 1e-3, "q5_k")
     assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q5_K, w, q8[:1], k, n).cpu().numpy(), v["q5_k_sums"])
+    # Q6_K dense, two tokens; int32 block sums.
+    k, n = 512, 12
+    w = _dev(v["q6_k_w"], device)
+    q8 = ops.quantize_q8_1(_dev(v["q6_k_x"], device))
+    close(ops.vecq(ops.TYPE_Q6_K, w, q8, k, n, tokens=2).cpu().numpy(), v["q6_k_y"], 1e-3, "q6_k")
+    assert np.array_equal(ops.vecq_block_sums(ops.TYPE_Q6_K, w, q8[:1], k, n).cpu().numpy(), v["q6_k_sums"])
     # MXFP4 dense, two tokens; int32 block sums.
     k, n = 512, 12
     w = _dev(v["mxfp4_w"], device)

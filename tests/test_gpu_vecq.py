@@ -408,6 +408,75 @@ def test_q5_k_refuses_the_other_forms(device):
         ops.vecq(Q5_K, dev(w, device), dev(q8, device), k, n, variant=0)
 
 
+# ---- Q6_K through the streaming form (a 210-byte block a lane, every dword put together from two)
+
+Q6_K = ops.TYPE_Q6_K
+
+
+@pytest.mark.parametrize("k,n", [(4096, 96), (2048, 40), (8192, 10), (14336, 7), (5120, 6), (256, 32)])
+@pytest.mark.parametrize("tokens", [1, 3, 4, 9])
+def test_q6_k_dense_matches_oracle(device, k, n, tokens):
+    """src/format/encoding.cc:117, src/kernels/ggml/vecq.cu:76-77 of the reference: tiles of 64, 56, 40 and 32 blocks
+    (a multiple of eight: 1680 bytes), lanes whose block starts 0 or 2 bytes into a dword; quantizing in the kernel
+    gives the same bits, and a token's values do not depend on the tokens beside it."""
+    w = synth.q6_k_weights(n, k, 701 + k + n)
+    x = synth.activations(tokens, k, 702 + tokens)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(Q6_K, w, q8, k, n, tokens=tokens)
+    got = ops.vecq(Q6_K, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    fused = ops.vecq_fused(Q6_K, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    alone = ops.vecq(Q6_K, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
+    assert np.array_equal(alone[0].view(np.uint32), got[tokens - 1].view(np.uint32))
+
+
+def test_q6_k_block_sums_and_random_bytes(device):
+    k, n = 2048, 24
+    w = synth.random_blocks(Q6_K, n, k, 711)
+    q8 = oracle.q8_1_quantize(synth.activations(2, k, 712))
+    want = oracle.vecq_block_sums(Q6_K, w, q8[:1], k, n)
+    got = ops.vecq_block_sums(Q6_K, dev(w, device), dev(q8[:1], device), k, n).cpu().numpy()
+    assert np.array_equal(got, want)
+    y = ops.vecq(Q6_K, dev(w, device), dev(q8, device), k, n, tokens=2).cpu().numpy()
+    ok, worst = rel_close(y, oracle.vecq(Q6_K, w, q8, k, n, tokens=2), TOL)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("tokens", [1, 5])
+def test_q6_k_glu_and_routed_match_oracle(device, tokens):
+    k, n, experts, used = 1024, 40, 6, 2
+    gate, up = synth.q6_k_weights(n, k, 721), synth.q6_k_weights(n, k, 722)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 723))
+    want = oracle.vecq(Q6_K, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_SWIGLU)
+    got = ops.vecq(Q6_K, dev(up, device), dev(q8, device), k, n, gate=dev(gate, device), tokens=tokens,
+                   glu=ops.GLU_SWIGLU).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    w = synth.q6_k_weights(experts * n, k, 724).reshape(experts, -1)
+    g = synth.rng(725)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    stride_expert = n * (k // 256)
+    want = oracle.vecq(Q6_K, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(Q6_K, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+
+
+def test_q6_k_refuses_tiles_that_are_not_whole_chunks(device):
+    q8 = oracle.q8_1_quantize(synth.activations(1, 3840, 732))
+    with pytest.raises(ops.KernelFailure):  # 15 blocks a row: no tile of a multiple of eight blocks in 64 lanes
+        ops.vecq(Q6_K, dev(synth.q6_k_weights(8, 3840, 731), device), dev(q8, device), 3840, 8)
+    q8 = oracle.q8_1_quantize(synth.activations(1, 5120, 734))
+    with pytest.raises(ops.KernelFailure):  # three rows of 20 blocks: the last tile would end within a chunk
+        ops.vecq(Q6_K, dev(synth.q6_k_weights(3, 5120, 733), device), dev(q8, device), 5120, 3)
+    q8 = oracle.q8_1_quantize(synth.activations(1, 4096, 736))
+    with pytest.raises(ops.KernelFailure):  # the rows form has no Q6_K
+        ops.vecq(Q6_K, dev(synth.q6_k_weights(8, 4096, 735), device), dev(q8, device), 4096, 8, variant=0)
+
+
 # ---- MXFP4 through the streaming form (eight 17-byte blocks a lane)
 
 MXFP4 = ops.TYPE_MXFP4

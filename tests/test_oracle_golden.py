@@ -240,6 +240,70 @@ def test_q5_k_decode_sums_and_products_by_brute_force_and_known_answers():
     assert oracle.vecq(t, b, q, 256, 1)[0, 0, 0] == 640.0
 
 
+def q6_k_decode_numpy(block):
+    """ggml's dequantize_row_q6_K, its loops as published (two halves of 128, four groups of 32 each from the same 32
+    bytes of qh), apart from the oracle's index form."""
+    ql, qh, sc = block[0:128].astype(int), block[128:192].astype(int), block[192:208].view(np.int8).astype(int)
+    d = float(block[208:210].view(np.float16)[0])
+    y = np.zeros(256, dtype=np.float64)
+    for half in range(2):
+        lo, hi, s, o = ql[64 * half:], qh[32 * half:], sc[8 * half:], 128 * half
+        for l in range(32):
+            i = l // 16
+            q1 = ((lo[l] & 0xF) | (((hi[l] >> 0) & 3) << 4)) - 32
+            q2 = ((lo[l + 32] & 0xF) | (((hi[l] >> 2) & 3) << 4)) - 32
+            q3 = ((lo[l] >> 4) | (((hi[l] >> 4) & 3) << 4)) - 32
+            q4 = ((lo[l + 32] >> 4) | (((hi[l] >> 6) & 3) << 4)) - 32
+            y[o + l], y[o + l + 32] = d * s[i] * q1, d * s[i + 2] * q2
+            y[o + l + 64], y[o + l + 96] = d * s[i + 4] * q3, d * s[i + 6] * q4
+    return y
+
+
+def test_q6_k_decode_sums_and_products_by_brute_force_and_known_answers():
+    """Q6_K (src/format/encoding.cc:117 of the reference: 256 values in 210 bytes). Parity unpinned: ggml is not
+    vendored and the reference holds no Q6_K vector; this pins the oracle's C against numpy's reading of the published
+    loops, the int32 sums and the product against the FP64 dot of decoded weights and activations, and a hand-built
+    block."""
+    from llmp_amd import synth
+    t, k, n = oracle.TYPE_Q6_K, 512, 5
+    assert oracle.block_bytes(t) == 210 and oracle.block_elements(t) == 256
+    x = np.random.Generator(np.random.PCG64(82)).standard_normal((1, k)).astype(np.float32)
+    q8 = oracle.q8_1_quantize(x)
+    a = q8[0].reshape(-1, 36)
+    aq = a[:, 4:].view(np.int8).astype(np.int64)
+    ad = a[:, 0:2].view(np.float16).astype(np.float64).reshape(-1)
+    act = (aq[:k // 32] * ad[:k // 32, None]).reshape(-1)
+    for w in (synth.random_blocks(t, n, k, 81), synth.q6_k_weights(n, k, 83)):
+        dec, sums, y = oracle.decode_rows(t, w, k), oracle.vecq_block_sums(t, w, q8, k, n), oracle.vecq(t, w, q8, k, n)[0, 0]
+        for r in range(n):
+            blocks = w[r].reshape(-1, 210)
+            want = np.concatenate([q6_k_decode_numpy(b) for b in blocks])
+            np.testing.assert_allclose(dec[r], want, rtol=1e-6, atol=1e-12)
+            for i, b in enumerate(blocks):
+                d, sc = float(b[208:210].view(np.float16)[0]), b[192:208].view(np.int8).astype(np.float64)
+                codes = np.rint(want[256 * i:256 * (i + 1)].reshape(16, 16) / (d * sc[:, None] + (sc[:, None] == 0)))
+                codes = np.where(sc[:, None] == 0, 0, codes).astype(np.int64)
+                got = sums[r, i].astype(np.int64)
+                flat = aq[8 * i:8 * i + 8].reshape(16, 16)
+                live = sc != 0
+                assert np.array_equal(got[live], (codes * flat).sum(axis=1)[live])
+            np.testing.assert_allclose(y[r], float(np.dot(want, act)), rtol=2e-6, atol=1e-9)
+    # Hand-built: d = 0.5, every scale 2, ql = 0x21 everywhere, qh = 0xE4 (bits 2t, 2t + 1 = t): group t of a half has
+    # codes (1 or 2) + 16 t - 32: t = 0, 1 take the low nibble 1, t = 2, 3 the high nibble 2.
+    b = np.zeros((1, 210), dtype=np.uint8)
+    b[0, 0:128], b[0, 128:192], b[0, 192:208] = 0x21, 0xE4, 2
+    b[0, 208:210] = np.array([0.5], dtype=np.float16).view(np.uint8)
+    code = np.array([1 - 32, 1 + 16 - 32, 2 + 32 - 32, 2 + 48 - 32])
+    want = np.tile(np.repeat(code, 32), 2).astype(np.float64)
+    assert np.array_equal(oracle.decode_rows(t, b, 256)[0], want)
+    q = np.zeros((1, 8 * 36), dtype=np.uint8)
+    for g in range(8):
+        q[0, g * 36:g * 36 + 2] = np.array([0.25], dtype=np.float16).view(np.uint8)
+        q[0, g * 36 + 4:g * 36 + 36] = 3
+    assert np.array_equal(oracle.vecq_block_sums(t, b, q, 256, 1)[0, 0], np.tile(np.repeat(code, 2), 2) * 48)
+    assert oracle.vecq(t, b, q, 256, 1)[0, 0, 0] == 0.5 * 0.25 * 2 * 48 * 2 * 2 * code.sum()
+
+
 def legacy_block_numpy(t, block, a):
     """tests/unit/dsv4_fast_test.cc:141-164 restated with numpy, apart from the oracle's C:
     (codes, int sum, product) of one legacy block and one Q8_1 block."""
