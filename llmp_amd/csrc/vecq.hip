@@ -606,8 +606,8 @@ int CheckDesc(int type, const llmp_vecq_desc* d, bool sorted = false) {
   const uintptr_t wa = reinterpret_cast<uintptr_t>(d->w) | reinterpret_cast<uintptr_t>(d->g);
   if (type == LLMP_TYPE_Q4_K && wa % 16 != 0) return Refuse(1, "vecq: Q4_K weights not 16-byte aligned");
   if (type == LLMP_TYPE_Q6_K && !FlatTakes(type, *d))
-    return Refuse(1, "vecq: Q6_K takes 16-byte aligned weights, rows up to 16384 values (8192 with a GLU) of which some number "
-                     "fills a tile of 64 lanes (32) with a multiple of eight blocks, matrices and experts of a multiple of eight blocks");
+    return Refuse(1, "vecq: Q6_K takes 16-byte aligned weights, rows up to 16384 values (8192 with a GLU), packed or of a multiple "
+                     "of eight blocks, matrices and experts of a multiple of eight blocks");
   // Q5_K runs through the flat form alone.
   if (type == LLMP_TYPE_Q5_K && !FlatTakes(type, *d))
     return Refuse(1, "vecq: Q5_K takes 16-byte aligned weights and rows whose staged activations fit LDS (up to 8192 values "

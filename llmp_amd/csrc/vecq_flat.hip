@@ -347,8 +347,8 @@ struct FormatQ5K : FormatQ4K {
 // src/format/encoding.cc:117 of the reference; ggml's dequantize_row_q6_K: value 128 h + 32 t + l (h < 2, t < 4,
 // l < 32) is the low (t < 2) or high nibble of ql[64 h + 32 (t & 1) + l] plus 16 times bits 2t, 2t + 1 of
 // qh[32 h + l], minus 32, times scales[value / 16] times d. A block is not a whole number of dwords: a tile is
-// fetched as the same 16-byte chunks (FlatPlan makes a tile's units a multiple of eight, 1680 bytes), a lane's unit
-// then starts 0 or 2 bytes into a dword and every dword it uses is put together from two (v_alignbyte). Codes
+// fetched as 16-byte chunks from the boundary below its first byte, a lane's unit then starts 0 or 2 bytes into a
+// dword and every dword it uses is put together from two (v_alignbyte). Codes
 // become signed bytes without a subtraction a byte: x + 0x60 cannot carry for x < 64, and flipping bit 7 of that is
 // x - 32. The staged activations are Q4_K's (the codes in order, d8 a block).
 struct FormatQ6K : FormatQ4K {
@@ -1298,14 +1298,32 @@ __device__ __forceinline__ void FetchPart(const uint8_t* base, int chunks, int64
   }
 }
 
+// Where a tile's first byte lies in its buffer: 0 unless the format's units are not whole 16-byte chunks.
+template <class F>
+__device__ __forceinline__ int TileShift(const llmp_vecq_desc& d, int64_t expert_block, int row0) {
+  if constexpr (F::kUnitBytes % 16 != 0) {
+    return static_cast<int>(((expert_block + static_cast<int64_t>(row0) * d.stride_row) * F::kBlockBytes) & 15);
+  } else {
+    return 0;
+  }
+}
+
 // The tile of `rows` rows from `row0`. A matrix's part always starts where a full tile's
 // would (`gate_at` bytes into the buffer), so a lane's place in a tile never changes.
 template <class F, bool kGlu, bool kPacked>
 __device__ __forceinline__ void FetchTile(const llmp_vecq_desc& d, int64_t expert_block, int row0, int rows, int units,
                                           int gate_at, uint8_t* ring, int lane) {
-  const int64_t first = (expert_block + static_cast<int64_t>(row0) * d.stride_row) * F::kBlockBytes;
+  int64_t first = (expert_block + static_cast<int64_t>(row0) * d.stride_row) * F::kBlockBytes;
   const int row_bytes = units * F::kUnitBytes;
-  const int chunks = rows * row_bytes / 16;
+  // Units that are not whole chunks (packed rows): the tile is fetched from the 16-byte boundary below its first
+  // byte and lies that many bytes into the buffer (TileShift); its last chunk ends within the matrix, whose rows'
+  // blocks are a multiple of eight.
+  int shift = 0;
+  if constexpr (F::kUnitBytes % 16 != 0) {
+    shift = static_cast<int>(first & 15);
+    first -= shift;
+  }
+  const int chunks = (shift + rows * row_bytes + 15) / 16;
   const int64_t stride_bytes = static_cast<int64_t>(d.stride_row) * F::kBlockBytes;
   // The loads (1 KB a wave each) of a part: at most 32 units a matrix with a GLU, else 64.
   constexpr int kLoads = ((kGlu ? kWave / 2 : kWave) * F::kUnitBytes + 1023) / 1024;
@@ -1370,7 +1388,10 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   const int tiles = (d.nrows + rows_per_tile - 1) / rows_per_tile;
   // kDeep: two tile buffers a wave (one workgroup a CU), the next tile in flight while this one
   // is multiplied.
-  constexpr int kTileBytes = kWave * F::kUnitBytes;
+  // (Units that are not whole chunks: room for the tile's shift, the gate part's own boundary and a lane's reads
+  // past its unit.)
+  constexpr bool kOdd = F::kUnitBytes % 16 != 0;
+  constexpr int kTileBytes = kWave * F::kUnitBytes + (kOdd ? 80 : 0);
   // The tile buffers take 16-byte chunks: they start at the next 16-byte boundary after the records.
   // (A dense product of fewer tokens than a pass takes stages only those: more room for waves.)
   const int staged = a.offsets == nullptr && a.d.ids == nullptr && a.d.tokens < P ? a.d.tokens : P;
@@ -1383,8 +1404,8 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   const int row = f / nsb;
   const int sb = f - row * nsb;
   const bool placed = lane < (kGlu ? 2 * half : half);
-  const int gate_at = half * F::kUnitBytes;
-  const uint8_t* my_block = ring + lane * F::kUnitBytes;
+  const int gate_at = kOdd ? ((half * F::kUnitBytes + 15) & ~15) + 32 : half * F::kUnitBytes;
+  const uint8_t* my_block = ring + (gate_lane ? gate_at + f * F::kUnitBytes : lane * F::kUnitBytes);
   const uint8_t* my_records = lds + sb * F::kRecord;
 
   // A routed product's workgroup first learns whether it owns its expert; one over sorted
@@ -1476,8 +1497,8 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
       float out[P];
       if (live) {
         int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * F::kDumpInts : nullptr;
-        F::template DotAt<P, kDump>(my_block + (kDeep ? buffer * kTileBytes : 0), my_records, token_stride, m, out,
-                                    dump);
+        F::template DotAt<P, kDump>(my_block + (kDeep ? buffer * kTileBytes : 0) + TileShift<F>(d, expert_block, row0),
+                                    my_records, token_stride, m, out, dump);
       }
       // Row sums: a suffix sum over each row's lanes (a fixed tree), the total in the row's
       // first lane; a gate row's total then moves to its up row's lane.
@@ -1628,16 +1649,13 @@ template <class F>
 FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   FlatPlan p;
   p.rows = (glu ? kWave / 2 : kWave) / units;
-  // Units that are not whole 16-byte chunks: a tile is a multiple of eight of them (none, if no such tile fits),
-  // and a lane reads up to six bytes past its unit.
+  // Units that are not whole 16-byte chunks: a wave's buffer has room for the tile's shift, the gate part's own
+  // boundary and a lane's reads past its unit.
   constexpr bool kOdd = F::kUnitBytes % 16 != 0;
-  if constexpr (kOdd) {
-    while (p.rows > 0 && (p.rows * units) % 8 != 0) --p.rows;
-  }
   p.waves = kWaves;
   for (;;) {
     p.lds = ((static_cast<size_t>(pass) * units * F::kRecord + 15) & ~static_cast<size_t>(15)) +
-            static_cast<size_t>(deep ? 2 : 1) * p.waves * kWave * F::kUnitBytes + (kOdd ? 16 : 0);
+            static_cast<size_t>(deep ? 2 : 1) * p.waves * (kWave * F::kUnitBytes + (kOdd ? 80 : 0));
     if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
     --p.waves;
   }
@@ -1804,14 +1822,13 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
   }
   if (type == LLMP_TYPE_Q6_K) {
-    // 210-byte blocks: tiles of a multiple of eight units, everything at 16-byte boundaries.
+    // 210-byte blocks: matrices and experts at 16-byte boundaries and of a multiple of eight blocks (a tile's
+    // last chunk then ends within its matrix); rows packed, or of a multiple of eight blocks themselves.
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
     const int units = d.ncols_x / FormatQ6K::kUnitValues;
     if (at % 16 != 0 || d.stride_expert % 8 != 0 || units < 1 || units > most) return false;
     if (d.stride_row != units && (units % 8 != 0 || d.stride_row % 8 != 0)) return false;
-    const FlatPlan plan = PlanFlat<FormatQ6K>(1, units, glu);
-    // Full tiles are whole chunks; so is the last, shorter one if all the rows' blocks are a multiple of eight.
-    return plan.rows >= 1 && (static_cast<int64_t>(d.nrows) * units) % 8 == 0 && plan.lds <= kFlatLdsLimit;
+    return (static_cast<int64_t>(d.nrows) * units) % 8 == 0 && PlanFlat<FormatQ6K>(1, units, glu).lds <= kFlatLdsLimit;
   }
   if (type == LLMP_TYPE_Q5_K) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);

@@ -67,7 +67,7 @@ def desc(**kw):
     (2, dict(ncols_x=288, stride_row=9), "Q4_0"),
     (20, dict(ncols_x=288, stride_row=9), "IQ4_NL"),
     (13, dict(w=0x1008), "Q5_K"),
-    (14, dict(ncols_x=3840, stride_row=15), "Q6_K"),
+    (14, dict(ncols_x=3840, stride_row=15, nrows=3), "Q6_K"),
     (13, dict(ncols_x=288), "whole"),
     (12, dict(used=300), "slots"),
 ])

@@ -413,12 +413,14 @@ def test_q5_k_refuses_the_other_forms(device):
 Q6_K = ops.TYPE_Q6_K
 
 
-@pytest.mark.parametrize("k,n", [(4096, 96), (2048, 40), (8192, 10), (14336, 7), (5120, 6), (256, 32)])
+@pytest.mark.parametrize("k,n", [(4096, 96), (2048, 40), (8192, 10), (14336, 7), (5120, 6), (256, 32), (3840, 24),
+                                 (1280, 40), (768, 8)])
 @pytest.mark.parametrize("tokens", [1, 3, 4, 9])
 def test_q6_k_dense_matches_oracle(device, k, n, tokens):
-    """src/format/encoding.cc:117, src/kernels/ggml/vecq.cu:76-77 of the reference: tiles of 64, 56, 40 and 32 blocks
-    (a multiple of eight: 1680 bytes), lanes whose block starts 0 or 2 bytes into a dword; quantizing in the kernel
-    gives the same bits, and a token's values do not depend on the tokens beside it."""
+    """src/format/encoding.cc:117, src/kernels/ggml/vecq.cu:76-77 of the reference: tiles that are whole 16-byte chunks
+    and tiles of 60, 63 and 24 blocks that start 0 to 14 bytes past a boundary, lanes whose block starts 0 or 2 bytes
+    into a dword; quantizing in the kernel gives the same bits, and a token's values do not depend on the tokens
+    beside it."""
     w = synth.q6_k_weights(n, k, 701 + k + n)
     x = synth.activations(tokens, k, 702 + tokens)
     q8 = oracle.q8_1_quantize(x)
@@ -445,8 +447,9 @@ def test_q6_k_block_sums_and_random_bytes(device):
 
 
 @pytest.mark.parametrize("tokens", [1, 5])
-def test_q6_k_glu_and_routed_match_oracle(device, tokens):
-    k, n, experts, used = 1024, 40, 6, 2
+@pytest.mark.parametrize("k", [1024, 3840])
+def test_q6_k_glu_and_routed_match_oracle(device, tokens, k):
+    n, experts, used = 40, 6, 2
     gate, up = synth.q6_k_weights(n, k, 721), synth.q6_k_weights(n, k, 722)
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 723))
     want = oracle.vecq(Q6_K, up, q8, k, n, gate=gate, tokens=tokens, glu=oracle.GLU_SWIGLU)
@@ -467,8 +470,8 @@ def test_q6_k_glu_and_routed_match_oracle(device, tokens):
 
 def test_q6_k_refuses_tiles_that_are_not_whole_chunks(device):
     q8 = oracle.q8_1_quantize(synth.activations(1, 3840, 732))
-    with pytest.raises(ops.KernelFailure):  # 15 blocks a row: no tile of a multiple of eight blocks in 64 lanes
-        ops.vecq(Q6_K, dev(synth.q6_k_weights(8, 3840, 731), device), dev(q8, device), 3840, 8)
+    with pytest.raises(ops.KernelFailure):  # 3 rows of 15 blocks: the matrix ends within a 16-byte chunk
+        ops.vecq(Q6_K, dev(synth.q6_k_weights(3, 3840, 731), device), dev(q8, device), 3840, 3)
     q8 = oracle.q8_1_quantize(synth.activations(1, 5120, 734))
     with pytest.raises(ops.KernelFailure):  # three rows of 20 blocks: the last tile would end within a chunk
         ops.vecq(Q6_K, dev(synth.q6_k_weights(3, 5120, 733), device), dev(q8, device), 5120, 3)
