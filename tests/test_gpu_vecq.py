@@ -480,6 +480,34 @@ def test_q6_k_refuses_tiles_that_are_not_whole_chunks(device):
         ops.vecq(Q6_K, dev(synth.q6_k_weights(8, 4096, 735), device), dev(q8, device), 4096, 8, variant=0)
 
 
+@pytest.mark.parametrize("t", [ops.TYPE_Q5_K, ops.TYPE_Q6_K, ops.TYPE_IQ4_NL])
+@pytest.mark.parametrize("k", [2048, 3840])
+def test_sorted_rows_equal_routed_pairs_for_the_added_types(device, t, k):
+    """Rows sorted by expert (the offsets of llmp.moe.route) against the same pairs under routing ids, bit for bit, and
+    the routed product against the oracle."""
+    n, experts, tokens, used = 16, 5, 6, 2
+    if t == ops.TYPE_IQ4_NL and k % 256:
+        pytest.skip("rows of whole 256 values")
+    make = {ops.TYPE_Q5_K: synth.q5_k_weights, ops.TYPE_Q6_K: synth.q6_k_weights,
+            ops.TYPE_IQ4_NL: lambda n_, k_, seed: synth.legacy_weights(ops.TYPE_IQ4_NL, n_, k_, seed)}[t]
+    w = make(experts * n, k, 801).reshape(experts, -1)
+    g = synth.rng(802)
+    ids = np.stack([g.permutation(experts)[:used] for _ in range(tokens)]).astype(np.int32)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 803))
+    stride_expert = n * (k // oracle.block_elements(t))
+    want = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, ids=dev(ids, device), tokens=tokens, used=used,
+                   stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    order = np.argsort(ids.reshape(-1), kind="stable")
+    offsets = np.concatenate([[0], np.cumsum(np.bincount(ids.reshape(-1), minlength=experts))]).astype(np.int32)
+    rows = np.ascontiguousarray(q8.reshape(tokens, -1)[order // used])
+    sorted_out = ops.vecq_sorted(t, dev(w, device), dev(rows, device), dev(offsets, device), k, n, experts,
+                                 stride_expert=stride_expert).cpu().numpy()
+    assert np.array_equal(sorted_out.view(np.uint32), got.reshape(tokens * used, n)[order].view(np.uint32))
+
+
 # ---- MXFP4 through the streaming form (eight 17-byte blocks a lane)
 
 MXFP4 = ops.TYPE_MXFP4
