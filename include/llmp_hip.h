@@ -210,6 +210,24 @@ int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void
 int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
                             void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream);
 
+/* llmp.set_rows.grouped_quant (SetRowsQuantGroup, src/kernels/ggml/kv_quant.h:82-84, 172-178;
+ * src/kernels/ggml/kv_quant.cc:214-236): two to sixteen such stores in one launch (a layer's K and V rows, or
+ * several layers'), each as llmp_hip_set_rows_quant takes it; `cells` is the destination's number of rows, by
+ * which the call refuses a destination that overlaps another store's destination, values or indices. */
+typedef struct llmp_set_rows_store {
+  int type;        /* LLMP_TYPE_Q8_0 or LLMP_TYPE_Q4_0 */
+  int index_bytes; /* 4 or 8 */
+  const float* x;
+  int64_t x_stride;
+  const void* ids;
+  void* destination;
+  int64_t row_bytes;
+  int64_t k;
+  int64_t rows;
+  int64_t cells;
+} llmp_set_rows_store;
+int llmp_hip_set_rows_quant_group(int count, const llmp_set_rows_store* stores, void* stream);
+
 /* ------------------------------------------------------------------ EXL3
  * The trellis-coded linear. Weights as src/kernels/exl3/validate.h:84-96 holds them: the
  * trellis [k / 16][n / 16][16 * bits] uint16, suh (k F16) and svh (n F16); every dimension a

@@ -69,6 +69,14 @@ class DecodeOperand(C.Structure):
                 ("bits", C.c_uint8), ("scale_type", C.c_uint8)]
 
 
+class SetRowsStore(C.Structure):
+    """llmp_set_rows_store: one member of llmp.set_rows.grouped_quant (src/kernels/ggml/kv_quant.h:172-178 of the
+    reference)."""
+    _fields_ = [("type", C.c_int), ("index_bytes", C.c_int), ("x", C.c_void_p), ("x_stride", C.c_int64),
+                ("ids", C.c_void_p), ("destination", C.c_void_p), ("row_bytes", C.c_int64), ("k", C.c_int64),
+                ("rows", C.c_int64), ("cells", C.c_int64)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -93,6 +101,7 @@ SYMBOLS = {
     "llmp_hip_q8_1_quantize_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
     "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
+    "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmp_hip_mxfp8_swizzle": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "llmp_hip_mxfp8_gemv": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _vp, _vp]),

@@ -96,10 +96,103 @@ __global__ __launch_bounds__(kStoreThreads) void SetRowsQuantKernel(const float*
   }
 }
 
+// Two to sixteen stores in one launch: grid row m is store m, its descriptor in the kernel's arguments
+// (src/kernels/ggml/kv_quant.h:82-84, 172-178 of the reference).
+struct StoreMember {
+  const float* x;
+  const void* ids;
+  uint8_t* destination;
+  int64_t x_stride, row_bytes, total;
+  int blocks, type, index_bytes;
+};
+struct StoreGroup {
+  StoreMember member[16];
+};
+
+__global__ __launch_bounds__(kStoreThreads) void SetRowsQuantGroupKernel(const StoreGroup group) {
+  const StoreMember& s = group.member[blockIdx.y];
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * kStoreThreads + threadIdx.x;
+  if (at >= s.total) return;
+  const int64_t row = at / s.blocks;
+  const int block = static_cast<int>(at - row * s.blocks);
+  const float4* from = reinterpret_cast<const float4*>(s.x + row * s.x_stride + block * 32);
+  float v[32];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float4 f = from[i];
+    v[4 * i] = f.x, v[4 * i + 1] = f.y, v[4 * i + 2] = f.z, v[4 * i + 3] = f.w;
+  }
+  const int64_t id = s.index_bytes == 4 ? static_cast<const int32_t*>(s.ids)[row] : static_cast<const int64_t*>(s.ids)[row];
+  uint8_t* to = s.destination + id * s.row_bytes;
+  if (s.type == LLMP_TYPE_Q8_0) {
+    StoreQ8_0(v, to + block * 34);
+  } else {
+    StoreQ4_0(v, to + block * 18);
+  }
+}
+
+// What one store must satisfy; its count of blocks in *total.
+int CheckStore(const char* op, int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
+               const void* destination, int64_t row_bytes, int64_t k, int64_t rows, int64_t* total) {
+  if (x == nullptr || ids == nullptr || destination == nullptr) return Refuse(1, "%s: null operand", op);
+  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_0) return Refuse(1, "%s: a Q8_0 or Q4_0 destination", op);
+  if (index_bytes != 4 && index_bytes != 8) return Refuse(1, "%s: I32 or I64 indices", op);
+  if (k <= 0 || k % 32 != 0 || rows <= 0) return Refuse(1, "%s: rows of whole 32-value blocks", op);
+  const int64_t block_bytes = type == LLMP_TYPE_Q8_0 ? 34 : 18;
+  if (x_stride < k || x_stride % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0)
+    return Refuse(1, "%s: source rows overlap or are not 16-byte aligned", op);
+  if (row_bytes < k / 32 * block_bytes || row_bytes % 2 != 0 || reinterpret_cast<uintptr_t>(destination) % 2 != 0)
+    return Refuse(1, "%s: destination rows overlap or are not 2-byte aligned", op);
+  *total = rows * (k / 32);
+  if (*total > 0xFFFFFFFFll / 32) return Refuse(1, "%s: more than 2^32 - 1 values", op);  // kv_quant.h:150-156
+  return 0;
+}
+
+bool Meet(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes) {
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + static_cast<uintptr_t>(b_bytes) && b0 < a0 + static_cast<uintptr_t>(a_bytes);
+}
+
 }  // namespace
 }  // namespace llmp_hip
 
 using namespace llmp_hip;
+
+extern "C" int llmp_hip_set_rows_quant_group(int count, const llmp_set_rows_store* stores, void* stream) {
+  const char* op = "set_rows.grouped_quant";
+  if (stores == nullptr) return Refuse(1, "%s: null stores", op);
+  if (count < 2 || count > 16) return Refuse(1, "%s: two through sixteen stores, not %d", op, count);  // kv_quant.cc:216
+  StoreGroup group{};
+  int64_t most = 0;
+  for (int i = 0; i < count; ++i) {
+    const llmp_set_rows_store& s = stores[i];
+    int64_t total = 0;
+    if (const int bad = CheckStore(op, s.type, s.x, s.x_stride, s.ids, s.index_bytes, s.destination, s.row_bytes, s.k,
+                                   s.rows, &total);
+        bad != 0)
+      return bad;
+    if (s.cells <= 0) return Refuse(1, "%s: a destination of no cells", op);
+    group.member[i] = StoreMember{s.x, s.ids, static_cast<uint8_t*>(s.destination), s.x_stride, s.row_bytes, total,
+                                  static_cast<int>(s.k / 32), s.type, s.index_bytes};
+    most = total > most ? total : most;
+  }
+  // No destination meets another store's destination or operands (kv_quant.cc:224-233).
+  for (int i = 0; i < count; ++i) {
+    const llmp_set_rows_store& a = stores[i];
+    const int64_t a_bytes = a.cells * a.row_bytes;
+    for (int j = 0; j < count; ++j) {
+      if (i == j) continue;
+      const llmp_set_rows_store& b = stores[j];
+      const bool meets = (j > i && Meet(a.destination, a_bytes, b.destination, b.cells * b.row_bytes)) ||
+                         Meet(a.destination, a_bytes, b.x, ((b.rows - 1) * b.x_stride + b.k) * 4) ||
+                         Meet(a.destination, a_bytes, b.ids, b.rows * b.index_bytes);
+      if (meets) return Refuse(1, "%s: the destination of store %d overlaps store %d's destination or operands", op, i, j);
+    }
+  }
+  const dim3 grid(static_cast<unsigned>((most + kStoreThreads - 1) / kStoreThreads), static_cast<unsigned>(count));
+  hipLaunchKernelGGL(SetRowsQuantGroupKernel, grid, dim3(kStoreThreads), 0, static_cast<hipStream_t>(stream), group);
+  return LaunchStatus(op);
+}
 
 extern "C" int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
                                        void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream) {

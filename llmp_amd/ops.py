@@ -141,6 +141,18 @@ def set_rows_quant(t, x, ids, destination, row_bytes=None):
     return destination
 
 
+def set_rows_quant_group(stores):
+    """llmp.set_rows.grouped_quant: two to sixteen stores (t, x, ids, destination) in one launch."""
+    lib = _lib.load()
+    table = (_lib.SetRowsStore * len(stores))()
+    for entry, (t, x, ids, destination) in zip(table, stores):
+        entry.type, entry.index_bytes = t, 8 if ids.dtype == torch.int64 else 4
+        entry.x, entry.x_stride, entry.ids = _ptr(x), x.stride(0), _ptr(ids)
+        entry.destination, entry.row_bytes = _ptr(destination), destination.stride(0)
+        entry.k, entry.rows, entry.cells = x.shape[1], x.shape[0], destination.shape[0]
+    _lib.check(lib.llmp_hip_set_rows_quant_group(len(stores), table, _stream()))
+
+
 def moe_router(logits, used, normalize=True, scale=1.0):
     """llmp.moe.router: float32 [tokens, experts] -> (ids int32 [tokens, used], weights float32)."""
     lib = _lib.load()

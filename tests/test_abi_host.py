@@ -186,3 +186,19 @@ def test_decode_matrix_refuses_bad_operands():
                                                   64, kw.get("path", 0), None)
     assert run(path=1) > 0 and b"FMA" in lib.llmp_hip_last_error()
     assert run(rows=0) > 0 and run(decoder=12) > 0 and run(first=60) > 0 and run(x=0x4004) > 0 and run(x_stride=100) > 0
+
+
+def test_grouped_store_refusals_queue_nothing():
+    lib = _lib.load()
+    table = (_lib.SetRowsStore * 2)()
+    for i, entry in enumerate(table):
+        entry.type, entry.index_bytes, entry.x, entry.x_stride, entry.ids = 8, 4, 0x10000, 64, 0x20000
+        entry.destination, entry.row_bytes, entry.k, entry.rows, entry.cells = 0x30000 + 0x1000 * i, 68, 64, 4, 8
+    assert lib.llmp_hip_set_rows_quant_group(1, table, None) > 0 and b"two through sixteen" in lib.llmp_hip_last_error()
+    assert lib.llmp_hip_set_rows_quant_group(2, None, None) > 0
+    table[1].destination = 0x30000 + 100  # inside the first store's 8 x 68 bytes
+    assert lib.llmp_hip_set_rows_quant_group(2, table, None) > 0 and b"overlaps" in lib.llmp_hip_last_error()
+    table[1].destination = 0x10000  # on the first store's values
+    assert lib.llmp_hip_set_rows_quant_group(2, table, None) > 0 and b"overlaps" in lib.llmp_hip_last_error()
+    table[1].destination, table[1].k = 0x40000, 48
+    assert lib.llmp_hip_set_rows_quant_group(2, table, None) > 0 and b"whole 32-value blocks" in lib.llmp_hip_last_error()

@@ -72,3 +72,41 @@ def test_refusals(device):
         ops.set_rows_quant(ops.TYPE_Q8_0, x, ids, cache, row_bytes=40)  # rows would overlap
     with pytest.raises(ops.KernelFailure):
         ops.set_rows_quant(ops.TYPE_Q8_0, x[:, :48], ids, cache)  # not whole blocks
+
+
+def test_grouped_stores_write_what_the_single_stores_write(device):
+    """llmp.set_rows.grouped_quant (src/kernels/ggml/kv_quant.h:172-178 of the reference): a layer's K and V rows and
+    another's, of different widths, types and index types, in one launch; every cache's bytes are the single
+    store's (and so the oracle's)."""
+    g = synth.rng(81)
+    shapes = [(ops.TYPE_Q8_0, 256, 11, torch.int64), (ops.TYPE_Q4_0, 512, 7, torch.int32),
+              (ops.TYPE_Q8_0, 64, 30, torch.int32), (ops.TYPE_Q4_0, 1024, 1, torch.int64)]
+    stores, alone = [], []
+    for t, k, rows, index in shapes:
+        cells = rows + 9
+        x = dev(synth.activations(rows, k, 82 + k) * 2.0, device)
+        ids = dev(g.permutation(cells)[:rows], device).to(index)
+        row_bytes = k // 32 * ops.BLOCK_BYTES[t]
+        stores.append((t, x, ids, torch.full((cells, row_bytes), 0x5A, dtype=torch.uint8, device=device)))
+        alone.append(ops.set_rows_quant(t, x, ids, torch.full((cells, row_bytes), 0x5A, dtype=torch.uint8, device=device)))
+    ops.set_rows_quant_group(stores)
+    for (t, x, ids, cache), single in zip(stores, alone):
+        assert torch.equal(cache, single)
+        want = oracle.kv_quantize(t, x.cpu().numpy())
+        assert np.array_equal(cache.cpu().numpy()[ids.cpu().numpy()], want)
+
+
+def test_grouped_store_refusals(device):
+    x = torch.zeros((4, 64), dtype=torch.float32, device=device)
+    ids = torch.arange(4, dtype=torch.int32, device=device)
+    cache = torch.zeros((8, 68), dtype=torch.uint8, device=device)
+    other = torch.zeros((8, 68), dtype=torch.uint8, device=device)
+    with pytest.raises(ops.KernelFailure):  # two through sixteen
+        ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, cache)])
+    with pytest.raises(ops.KernelFailure):
+        ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, cache)] * 17)
+    with pytest.raises(ops.KernelFailure):  # the same destination twice
+        ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, cache), (ops.TYPE_Q8_0, x, ids, cache)])
+    with pytest.raises(ops.KernelFailure):  # a member that the single store refuses
+        ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, cache), (ops.TYPE_Q4_K, x, ids, other)])
+    assert torch.count_nonzero(cache) == 0 and torch.count_nonzero(other) == 0  # nothing was queued
