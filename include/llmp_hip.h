@@ -228,6 +228,32 @@ typedef struct llmp_set_rows_store {
 } llmp_set_rows_store;
 int llmp_hip_set_rows_quant_group(int count, const llmp_set_rows_store* stores, void* stream);
 
+/* llmp.rope.set_rows_quant (RopeSetRowsQuant, src/kernels/ggml/kv_quant.h:180-192; the kernel's arithmetic
+ * src/kernels/ggml/kv_quant_rope.cu:29-120): a forward NEOX RoPE of `tokens` rows of `heads` heads of head_dim F32
+ * values (the first n_dims channels of a head rotate, channel c with c + n_dims / 2; the rest pass through), each
+ * token's rotated row quantized into row ids[token] of a Q8_0 or Q4_0 destination [cells][heads * head_dim]. The
+ * angle of pair p at position pos[token] is pos * theta_scale^p / freq_factors[p] (theta_scale = freq_base^(-2 /
+ * n_dims), kv_quant.cc:383), scaled by freq_scale, or YaRN's mix of both between corr_dims where ext_factor is not
+ * zero; cosine and sine are scaled by attn_factor (times 1 + 0.1 ln(1 / freq_scale) under YaRN). The rotated
+ * values are F32 results of this device's cosf, sinf and powf: stored codes equal those of a rotation computed in
+ * FP64 except where a value lies within that error of a rounding boundary. */
+typedef struct llmp_rope_store {
+  int type;                  /* LLMP_TYPE_Q8_0 or LLMP_TYPE_Q4_0 */
+  int heads, head_dim, n_dims;
+  const float* x;
+  int64_t x_head_stride;     /* floats */
+  int64_t x_token_stride;    /* floats */
+  const int32_t* pos;        /* a position a token */
+  const float* freq_factors; /* n_dims / 2 of them, or null */
+  const int64_t* ids;        /* a destination row a token */
+  void* destination;
+  int64_t row_bytes;
+  int64_t tokens;
+  float freq_scale, ext_factor, attn_factor, theta_scale;
+  float corr_dims[2];
+} llmp_rope_store;
+int llmp_hip_rope_set_rows_quant(const llmp_rope_store* store, void* stream);
+
 /* ------------------------------------------------------------------ EXL3
  * The trellis-coded linear. Weights as src/kernels/exl3/validate.h:84-96 holds them: the
  * trellis [k / 16][n / 16][16 * bits] uint16, suh (k F16) and svh (n F16); every dimension a

@@ -77,6 +77,15 @@ class SetRowsStore(C.Structure):
                 ("rows", C.c_int64), ("cells", C.c_int64)]
 
 
+class RopeStore(C.Structure):
+    """llmp_rope_store: RopeStore of src/kernels/ggml/kv_quant_rope.cu:55-71 of the reference."""
+    _fields_ = [("type", C.c_int), ("heads", C.c_int), ("head_dim", C.c_int), ("n_dims", C.c_int), ("x", C.c_void_p),
+                ("x_head_stride", C.c_int64), ("x_token_stride", C.c_int64), ("pos", C.c_void_p),
+                ("freq_factors", C.c_void_p), ("ids", C.c_void_p), ("destination", C.c_void_p),
+                ("row_bytes", C.c_int64), ("tokens", C.c_int64), ("freq_scale", C.c_float), ("ext_factor", C.c_float),
+                ("attn_factor", C.c_float), ("theta_scale", C.c_float), ("corr_dims", C.c_float * 2)]
+
+
 class VecQSource(C.Structure):
     _fields_ = [("x", C.c_void_p), ("x_type", C.c_int), ("x_token", C.c_int64),
                 ("x_slot", C.c_int64)]
@@ -102,6 +111,7 @@ SYMBOLS = {
     "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
     "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
     "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
+    "llmp_hip_rope_set_rows_quant": (_int, [C.POINTER(RopeStore), _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmp_hip_mxfp8_swizzle": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "llmp_hip_mxfp8_gemv": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _vp, _vp]),

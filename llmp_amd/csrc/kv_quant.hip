@@ -131,6 +131,53 @@ __global__ __launch_bounds__(kStoreThreads) void SetRowsQuantGroupKernel(const S
   }
 }
 
+// llmp.rope.set_rows_quant: a forward NEOX RoPE of a token's heads, then the store
+// (src/kernels/ggml/kv_quant_rope.cu:29-120 of the reference): a thread a block of 32 values of a token's row. A
+// channel below n_dims is one of the pair (c, c + n_dims / 2); the pair's angle is pos * theta_scale^pair over
+// the frequency factor, YaRN's ramp mixes the interpolated (freq_scale) and the extrapolated angle between the
+// correction dims and raises the magnitude; channels from n_dims on pass through.
+__global__ __launch_bounds__(kStoreThreads) void RopeSetRowsQuantKernel(const llmp_rope_store s, const int64_t total) {
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * kStoreThreads + threadIdx.x;
+  if (at >= total) return;
+  const int blocks_head = s.head_dim / 32, blocks_row = s.heads * blocks_head;
+  const int64_t token = at / blocks_row;
+  const int block = static_cast<int>(at - token * blocks_row);
+  const int head = block / blocks_head;
+  const int first = (block - head * blocks_head) * 32;  // channel within the head
+  const float* x = s.x + head * s.x_head_stride + token * s.x_token_stride;
+  const int half = s.n_dims / 2;
+  const float position = static_cast<float>(s.pos[token]);
+  float magnitude = s.attn_factor;
+  if (s.ext_factor != 0.0f) magnitude *= 1.0f + 0.1f * logf(1.0f / s.freq_scale);
+  float v[32];
+  for (int j = 0; j < 32; ++j) {
+    const int channel = first + j;
+    if (channel >= s.n_dims) {
+      v[j] = x[channel];
+      continue;
+    }
+    const int pair = channel < half ? channel : channel - half;
+    const float factor = s.freq_factors != nullptr ? s.freq_factors[pair] : 1.0f;
+    const float extrapolated = position * powf(s.theta_scale, static_cast<float>(pair)) / factor;
+    const float interpolated = s.freq_scale * extrapolated;
+    float theta = interpolated;
+    if (s.ext_factor != 0.0f) {
+      const float y = (static_cast<float>(pair) - s.corr_dims[0]) / fmaxf(0.001f, s.corr_dims[1] - s.corr_dims[0]);
+      const float ramp = (1.0f - fminf(1.0f, fmaxf(0.0f, y))) * s.ext_factor;
+      theta = interpolated * (1.0f - ramp) + extrapolated * ramp;
+    }
+    const float c = cosf(theta) * magnitude, sn = sinf(theta) * magnitude;
+    const float x0 = x[pair], x1 = x[pair + half];
+    v[j] = channel < half ? x0 * c - x1 * sn : x0 * sn + x1 * c;
+  }
+  uint8_t* to = static_cast<uint8_t*>(s.destination) + s.ids[token] * s.row_bytes;
+  if (s.type == LLMP_TYPE_Q8_0) {
+    StoreQ8_0(v, to + block * 34);
+  } else {
+    StoreQ4_0(v, to + block * 18);
+  }
+}
+
 // What one store must satisfy; its count of blocks in *total.
 int CheckStore(const char* op, int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
                const void* destination, int64_t row_bytes, int64_t k, int64_t rows, int64_t* total) {
@@ -218,4 +265,29 @@ extern "C" int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_strid
                        static_cast<const int64_t*>(ids), out, row_bytes, static_cast<int>(k / 32), total, type);
   }
   return LaunchStatus("set_rows.quant");
+}
+
+extern "C" int llmp_hip_rope_set_rows_quant(const llmp_rope_store* store, void* stream) {
+  const char* op = "rope.set_rows_quant";
+  if (store == nullptr) return Refuse(1, "%s: null store", op);
+  const llmp_rope_store& s = *store;
+  if (s.x == nullptr || s.pos == nullptr || s.ids == nullptr || s.destination == nullptr)
+    return Refuse(1, "%s: null operand", op);
+  if (s.type != LLMP_TYPE_Q8_0 && s.type != LLMP_TYPE_Q4_0) return Refuse(1, "%s: a Q8_0 or Q4_0 destination", op);
+  if (s.heads <= 0 || s.head_dim <= 0 || s.head_dim % 32 != 0 || s.tokens <= 0)
+    return Refuse(1, "%s: heads of whole 32-value blocks", op);  // kv_quant.h:180-185
+  if (s.n_dims <= 0 || s.n_dims % 2 != 0 || s.n_dims > s.head_dim)
+    return Refuse(1, "%s: an even number of rotated dims, at most the head's %d", op, s.head_dim);
+  const int64_t block_bytes = s.type == LLMP_TYPE_Q8_0 ? 34 : 18;
+  const int64_t blocks_row = static_cast<int64_t>(s.heads) * (s.head_dim / 32);
+  if (s.row_bytes < blocks_row * block_bytes || s.row_bytes % 2 != 0 || reinterpret_cast<uintptr_t>(s.destination) % 2 != 0)
+    return Refuse(1, "%s: destination rows overlap or are not 2-byte aligned", op);
+  if (s.x_head_stride < s.head_dim || s.x_token_stride < s.head_dim || reinterpret_cast<uintptr_t>(s.x) % 4 != 0)
+    return Refuse(1, "%s: heads or tokens overlap", op);
+  if (!(s.freq_scale > 0.0f) || !(s.theta_scale > 0.0f)) return Refuse(1, "%s: a positive frequency and angle scale", op);
+  const int64_t total = s.tokens * blocks_row;
+  if (total > 0xFFFFFFFFll / 32) return Refuse(1, "%s: more than 2^32 - 1 values", op);
+  const dim3 grid(static_cast<unsigned>((total + kStoreThreads - 1) / kStoreThreads));
+  hipLaunchKernelGGL(RopeSetRowsQuantKernel, grid, dim3(kStoreThreads), 0, static_cast<hipStream_t>(stream), s, total);
+  return LaunchStatus(op);
 }

@@ -153,6 +153,22 @@ def set_rows_quant_group(stores):
     _lib.check(lib.llmp_hip_set_rows_quant_group(len(stores), table, _stream()))
 
 
+def rope_set_rows_quant(t, x, pos, ids, destination, n_dims, theta_scale, *, freq_scale=1.0, ext_factor=0.0,
+                        attn_factor=1.0, corr_dims=(0.0, 0.0), freq_factors=None):
+    """llmp.rope.set_rows_quant: float32 x [tokens, heads, head_dim] rotated (NEOX) at int32 pos [tokens] and stored
+    as rows ids[token] (int64) of a Q8_0 or Q4_0 destination (uint8 [cells, row_bytes])."""
+    lib = _lib.load()
+    tokens, heads, head_dim = x.shape
+    s = _lib.RopeStore(type=t, heads=heads, head_dim=head_dim, n_dims=n_dims, x=_ptr(x), x_head_stride=x.stride(1),
+                       x_token_stride=x.stride(0), pos=_ptr(pos),
+                       freq_factors=_ptr(freq_factors) if freq_factors is not None else None, ids=_ptr(ids),
+                       destination=_ptr(destination), row_bytes=destination.stride(0), tokens=tokens,
+                       freq_scale=freq_scale, ext_factor=ext_factor, attn_factor=attn_factor, theta_scale=theta_scale)
+    s.corr_dims[0], s.corr_dims[1] = corr_dims
+    _lib.check(lib.llmp_hip_rope_set_rows_quant(C.byref(s), _stream()))
+    return destination
+
+
 def moe_router(logits, used, normalize=True, scale=1.0):
     """llmp.moe.router: float32 [tokens, experts] -> (ids int32 [tokens, used], weights float32)."""
     lib = _lib.load()

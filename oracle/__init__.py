@@ -141,6 +141,45 @@ def kv_quantize(t, x):
     return out
 
 
+def rope_neox(x, pos, n_dims, theta_scale, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0, corr_dims=(0.0, 0.0),
+              freq_factors=None):
+    """float32 x [tokens, heads, head_dim] -> the forward NEOX RoPE's float32 values, as the reference's CPU executor
+    forms them (src/kernels/reference/exec.cc:1343-1484: the mode's default case, offset 0, not the llama3 form): the
+    angle's steps each rounded to F32 (theta_scale^pair from FP64, times the position, over the frequency factor,
+    times the scale; YaRN's ramp between the correction dims), cosine and sine in FP64 times the magnitude, the
+    rotation in FP64, the result rounded to F32. Channels from n_dims on pass through. numpy, not C: test
+    infrastructure like the rest of this package."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    tokens, heads, head_dim = x.shape
+    half = n_dims // 2
+    f32 = np.float32
+    pair = np.arange(half)
+    power = np.power(np.float64(f32(theta_scale)), pair.astype(np.float64)).astype(np.float32)      # exec.cc:1449-1450
+    out = x.copy()
+    magnitude = f32(attn_factor)
+    if ext_factor > 0.0:
+        magnitude = f32(magnitude * f32(f32(1.0) + f32(f32(0.1) * f32(np.log(f32(f32(1.0) / f32(freq_scale)))))))
+    for t in range(tokens):
+        extrap = (f32(pos[t]) * power).astype(np.float32)
+        if freq_factors is not None:
+            extrap = (extrap / np.asarray(freq_factors, dtype=np.float32)[:half]).astype(np.float32)
+        interp = (f32(freq_scale) * extrap).astype(np.float32)
+        theta = interp
+        if ext_factor > 0.0:
+            y = ((pair.astype(np.float32) - f32(corr_dims[0])) / max(f32(0.001), f32(f32(corr_dims[1]) - f32(corr_dims[0])))).astype(np.float32)
+            ramp = ((f32(1.0) - np.minimum(f32(1.0), np.maximum(f32(0.0), y))) * f32(ext_factor)).astype(np.float32)
+            kept = (interp * (f32(1.0) - ramp)).astype(np.float32)
+            mixed = (extrap * ramp).astype(np.float32)
+            theta = (kept + mixed).astype(np.float32)
+        c = np.cos(theta.astype(np.float64)) * np.float64(magnitude)
+        sn = np.sin(theta.astype(np.float64)) * np.float64(magnitude)
+        a = x[t, :, :half].astype(np.float64)
+        b = x[t, :, half:n_dims].astype(np.float64)
+        out[t, :, :half] = (a * c - b * sn).astype(np.float32)
+        out[t, :, half:n_dims] = (a * sn + b * c).astype(np.float32)
+    return out
+
+
 def q8_1_decode(blocks, k):
     blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
     y = np.zeros(k, dtype=np.float32)

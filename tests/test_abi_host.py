@@ -202,3 +202,18 @@ def test_grouped_store_refusals_queue_nothing():
     assert lib.llmp_hip_set_rows_quant_group(2, table, None) > 0 and b"overlaps" in lib.llmp_hip_last_error()
     table[1].destination, table[1].k = 0x40000, 48
     assert lib.llmp_hip_set_rows_quant_group(2, table, None) > 0 and b"whole 32-value blocks" in lib.llmp_hip_last_error()
+
+
+def test_rope_store_refusals_queue_nothing():
+    lib = _lib.load()
+    s = _lib.RopeStore(type=8, heads=2, head_dim=64, n_dims=64, x=0x10000, x_head_stride=64, x_token_stride=128,
+                       pos=0x20000, freq_factors=None, ids=0x30000, destination=0x40000, row_bytes=136, tokens=3,
+                       freq_scale=1.0, ext_factor=0.0, attn_factor=1.0, theta_scale=0.9)
+    for field, value, why in (("n_dims", 66, b"rotated dims"), ("head_dim", 48, b"whole 32-value blocks"),
+                              ("row_bytes", 100, b"overlap"), ("type", 12, b"Q8_0 or Q4_0"), ("pos", None, b"null"),
+                              ("theta_scale", 0.0, b"positive")):
+        old = getattr(s, field)
+        setattr(s, field, value)
+        assert lib.llmp_hip_rope_set_rows_quant(C.byref(s), None) > 0 and why in lib.llmp_hip_last_error(), field
+        setattr(s, field, old)
+    assert lib.llmp_hip_rope_set_rows_quant(None, None) > 0

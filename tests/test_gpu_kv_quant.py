@@ -110,3 +110,65 @@ def test_grouped_store_refusals(device):
     with pytest.raises(ops.KernelFailure):  # a member that the single store refuses
         ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, cache), (ops.TYPE_Q4_K, x, ids, other)])
     assert torch.count_nonzero(cache) == 0 and torch.count_nonzero(other) == 0  # nothing was queued
+
+
+@pytest.mark.parametrize("t", [ops.TYPE_Q8_0, ops.TYPE_Q4_0])
+@pytest.mark.parametrize("yarn", [False, True])
+def test_rope_then_store_matches_the_oracles_rotation_and_quantizer(device, t, yarn):
+    """llmp.rope.set_rows_quant (src/kernels/ggml/kv_quant.h:180-192, kv_quant_rope.cu:29-120 of the reference)
+    against oracle.rope_neox followed by the reference quantizers. The device rotates with F32 cosf / sinf / powf,
+    the oracle as the reference's CPU executor does (FP64 cosine, sine and products): the stored bytes are the
+    oracle's except for a few codes whose value lies at a rounding boundary (at most 1 in 500 bytes may differ here,
+    and every stored value is within 0.6 quantization steps, Q4_0 1.1, of the oracle's rotated value)."""
+    g = synth.rng(95)
+    tokens, heads, head_dim, n_dims, cells = 9, 4, 128, 96, 20
+    whole = synth.activations(tokens, heads * (head_dim + 32), 96).reshape(tokens, heads, head_dim + 32)
+    x = whole[:, :, :head_dim]  # heads 160 floats apart
+    pos = np.array([0, 1, 2, 17, 100, 511, 1024, 2047, 3000], dtype=np.int32)
+    ids = g.permutation(cells)[:tokens].astype(np.int64)
+    theta_scale = float(np.float32(10000.0 ** (-2.0 / n_dims)))
+    ff = g.uniform(0.8, 2.0, size=n_dims // 2).astype(np.float32)
+    kw = dict(freq_scale=0.5, ext_factor=1.0, attn_factor=1.2, corr_dims=(10.0, 30.0)) if yarn else {}
+    rotated = oracle.rope_neox(x, pos, n_dims, theta_scale, freq_factors=ff, **kw)
+    want = oracle.kv_quantize(t, rotated.reshape(tokens, heads * head_dim))
+    xd = dev(whole, device)[:, :, :head_dim]
+    cache = torch.full((cells, want.shape[1] + 4), 0xA5, dtype=torch.uint8, device=device)
+    ops.rope_set_rows_quant(t, xd, dev(pos, device), dev(ids, device), cache, n_dims, theta_scale,
+                            freq_factors=dev(ff, device), **kw)
+    got = cache.cpu().numpy()
+    assert np.all(got[np.setdiff1d(np.arange(cells), ids)] == 0xA5) and np.all(got[:, want.shape[1]:] == 0xA5)
+    stored = got[ids][:, : want.shape[1]]
+    assert np.count_nonzero(stored != want) <= stored.size // 500
+    size = ops.BLOCK_BYTES[t]
+    blocks = stored.reshape(tokens, -1, size)
+    d = blocks[:, :, 0:2].copy().view(np.float16).astype(np.float32)[:, :, 0]
+    if t == ops.TYPE_Q8_0:
+        values = blocks[:, :, 2:].view(np.int8).astype(np.float32) * d[:, :, None]
+    else:
+        nib = blocks[:, :, 2:]
+        values = (np.concatenate([nib & 15, nib >> 4], axis=2).astype(np.float32) - 8.0) * d[:, :, None]
+    error = np.abs(values.reshape(tokens, -1) - rotated.reshape(tokens, -1))
+    step = np.repeat(np.abs(d), 32, axis=1).reshape(tokens, -1)
+    # Half a step, plus the F16 rounding of the scale times the largest code; Q4_0's top value is clamped a step down.
+    assert np.all(error <= (0.6 if t == ops.TYPE_Q8_0 else 1.1) * step + 1e-6)
+    # Position 0 and the channels past n_dims are the plain store's bytes.
+    plain = oracle.kv_quantize(t, x.reshape(tokens, heads * head_dim))
+    if not yarn:
+        assert np.array_equal(stored[0], plain[0])
+
+
+def test_rope_store_refusals(device):
+    x = torch.zeros((2, 2, 64), dtype=torch.float32, device=device)
+    pos = torch.zeros(2, dtype=torch.int32, device=device)
+    ids = torch.arange(2, dtype=torch.int64, device=device)
+    cache = torch.zeros((4, 2 * 2 * 34), dtype=torch.uint8, device=device)
+    for bad in (dict(n_dims=65), dict(n_dims=33), dict(theta_scale=0.0)):
+        args = dict(n_dims=64, theta_scale=0.9)
+        args.update(bad)
+        with pytest.raises(ops.KernelFailure):
+            ops.rope_set_rows_quant(ops.TYPE_Q8_0, x, pos, ids, cache, args["n_dims"], args["theta_scale"])
+    with pytest.raises(ops.KernelFailure):
+        ops.rope_set_rows_quant(ops.TYPE_Q4_K, x, pos, ids, cache, 64, 0.9)
+    with pytest.raises(ops.KernelFailure):  # rows would overlap
+        ops.rope_set_rows_quant(ops.TYPE_Q8_0, x, pos, ids, torch.zeros((4, 100), dtype=torch.uint8, device=device), 64, 0.9)
+    assert torch.count_nonzero(cache) == 0

@@ -922,3 +922,45 @@ def test_exl3_rows_are_the_explicit_hadamard_product():
         ref = x.astype(np.float64) @ got.astype(np.float64).T
         for r in range(2):
             assert np.sqrt(np.mean((y[r] - ref[r]) ** 2)) <= 2.0 ** -8 * np.sqrt(np.mean(ref[r] ** 2))
+
+
+def test_rope_neox_against_complex_rotations_and_yarn_closed_forms():
+    """oracle.rope_neox (src/kernels/reference/exec.cc:1343-1484 of the reference) against an independent form: a
+    pair (c, c + n_dims / 2) as a complex number times exp(i theta); position 0 is the identity; channels past n_dims
+    pass; the frequency factor divides the angle; YaRN with every pair inside the ramp (ramp = 1) keeps the
+    extrapolated angle and raises the magnitude by 1 + 0.1 ln(1 / scale), with every pair past it (ramp = 0) the
+    interpolated one."""
+    g = np.random.Generator(np.random.PCG64(91))
+    tokens, heads, head_dim, n_dims = 5, 3, 64, 48
+    x = g.standard_normal((tokens, heads, head_dim)).astype(np.float32)
+    pos = np.array([0, 1, 7, 300, 4095], dtype=np.int32)
+    theta_scale = np.float32(10000.0 ** (-2.0 / n_dims))
+    half = n_dims // 2
+
+    def rotate(angle, magnitude=1.0):
+        z = (x[:, :, :half].astype(np.float64) + 1j * x[:, :, half:n_dims].astype(np.float64))
+        z = z * np.exp(1j * angle)[:, None, :] * magnitude
+        want = x.astype(np.float64).copy()
+        want[:, :, :half], want[:, :, half:n_dims] = z.real, z.imag
+        return want
+
+    base = pos[:, None].astype(np.float64) * np.float64(theta_scale) ** np.arange(half)[None, :]
+    got = oracle.rope_neox(x, pos, n_dims, theta_scale)
+    # The angle is formed in F32 steps: at position 4095 it is good to about 4095 * 2^-23.
+    np.testing.assert_allclose(got, rotate(base), atol=3e-3, rtol=0)
+    np.testing.assert_allclose(got[:3], rotate(base)[:3], atol=2e-6, rtol=0)
+    assert np.array_equal(got[0], x[0]) and np.array_equal(got[:, :, n_dims:], x[:, :, n_dims:])
+    ff = g.uniform(0.5, 4.0, size=half).astype(np.float32)
+    np.testing.assert_allclose(oracle.rope_neox(x, pos, n_dims, theta_scale, freq_factors=ff)[:3],
+                               rotate(base / ff[None, :])[:3], atol=2e-6, rtol=0)
+    np.testing.assert_allclose(oracle.rope_neox(x, pos, n_dims, theta_scale, freq_scale=0.25)[:3],
+                               rotate(0.25 * base)[:3], atol=2e-6, rtol=0)
+    inside = oracle.rope_neox(x, pos, n_dims, theta_scale, freq_scale=0.25, ext_factor=1.0, attn_factor=1.5,
+                              corr_dims=(100.0, 200.0))
+    np.testing.assert_allclose(inside[:3], rotate(base, 1.5 * (1.0 + 0.1 * np.log(4.0)))[:3], atol=4e-6, rtol=0)
+    past = oracle.rope_neox(x, pos, n_dims, theta_scale, freq_scale=0.25, ext_factor=1.0, attn_factor=1.5,
+                            corr_dims=(-200.0, -100.0))
+    np.testing.assert_allclose(past[:3], rotate(0.25 * base, 1.5 * (1.0 + 0.1 * np.log(4.0)))[:3], atol=4e-6, rtol=0)
+    # Rotations keep a pair's length.
+    n0 = np.hypot(x[:, :, :half], x[:, :, half:n_dims])
+    np.testing.assert_allclose(np.hypot(got[:, :, :half], got[:, :, half:n_dims]), n0, rtol=1e-6)
