@@ -298,6 +298,20 @@ def block_formats(device):
         us = graph_us(lambda i: ops.set_rows_quant(t, x, ids, cache), 40)
         bytes_ = rows * width * 4 + rows * (width // 32 * size)
         out[f"set_rows_quant_{name}_512x8192"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1)}
+    # llmp.set_rows.grouped_quant: the K and the V rows (Q8_0 and Q4_0) in one launch.
+    caches = [torch.zeros((cells, width // 32 * size), dtype=torch.uint8, device=device) for size in (34, 18)]
+    x2 = dev(synth.activations(rows, width, 306))
+    us = graph_us(lambda i: ops.set_rows_quant_group([(ops.TYPE_Q8_0, x, ids, caches[0]), (ops.TYPE_Q4_0, x2, ids, caches[1])]), 40)
+    bytes_ = 2 * rows * width * 4 + rows * (width // 32 * 52)
+    out["set_rows_grouped_quant_q8_0_q4_0_512x8192"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1)}
+    # llmp.rope.set_rows_quant: 512 tokens of 64 heads of 128 values rotated (NEOX) and stored as Q8_0.
+    heads, head_dim = 64, 128
+    xr = x.reshape(rows, heads, head_dim)
+    pos = dev(np.arange(rows, dtype=np.int32) + 1000)
+    theta_scale = float(np.float32(10000.0 ** (-2.0 / head_dim)))
+    us = graph_us(lambda i: ops.rope_set_rows_quant(ops.TYPE_Q8_0, xr, pos, ids, caches[0], head_dim, theta_scale), 40)
+    bytes_ = rows * width * 4 + rows * (width // 32 * 34)
+    out["rope_set_rows_quant_q8_0_512x64x128"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1)}
     return out
 
 

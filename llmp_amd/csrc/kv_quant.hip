@@ -132,31 +132,19 @@ __global__ __launch_bounds__(kStoreThreads) void SetRowsQuantGroupKernel(const S
 }
 
 // llmp.rope.set_rows_quant: a forward NEOX RoPE of a token's heads, then the store
-// (src/kernels/ggml/kv_quant_rope.cu:29-120 of the reference): a thread a block of 32 values of a token's row. A
+// (src/kernels/ggml/kv_quant_rope.cu:29-120 of the reference): a workgroup a token, a thread a block of 32 values of its row. A
 // channel below n_dims is one of the pair (c, c + n_dims / 2); the pair's angle is pos * theta_scale^pair over
 // the frequency factor, YaRN's ramp mixes the interpolated (freq_scale) and the extrapolated angle between the
 // correction dims and raises the magnitude; channels from n_dims on pass through.
-__global__ __launch_bounds__(kStoreThreads) void RopeSetRowsQuantKernel(const llmp_rope_store s, const int64_t total) {
-  const int64_t at = static_cast<int64_t>(blockIdx.x) * kStoreThreads + threadIdx.x;
-  if (at >= total) return;
-  const int blocks_head = s.head_dim / 32, blocks_row = s.heads * blocks_head;
-  const int64_t token = at / blocks_row;
-  const int block = static_cast<int>(at - token * blocks_row);
-  const int head = block / blocks_head;
-  const int first = (block - head * blocks_head) * 32;  // channel within the head
-  const float* x = s.x + head * s.x_head_stride + token * s.x_token_stride;
+// A workgroup a token: the token's n_dims / 2 cosines and sines once, in LDS, for every head's blocks.
+__global__ __launch_bounds__(kStoreThreads) void RopeSetRowsQuantKernel(const llmp_rope_store s) {
+  extern __shared__ float2 rotation[];  // of pair p: magnitude * (cos, sin)
+  const int64_t token = blockIdx.x;
   const int half = s.n_dims / 2;
   const float position = static_cast<float>(s.pos[token]);
   float magnitude = s.attn_factor;
   if (s.ext_factor != 0.0f) magnitude *= 1.0f + 0.1f * logf(1.0f / s.freq_scale);
-  float v[32];
-  for (int j = 0; j < 32; ++j) {
-    const int channel = first + j;
-    if (channel >= s.n_dims) {
-      v[j] = x[channel];
-      continue;
-    }
-    const int pair = channel < half ? channel : channel - half;
+  for (int pair = threadIdx.x; pair < half; pair += kStoreThreads) {
     const float factor = s.freq_factors != nullptr ? s.freq_factors[pair] : 1.0f;
     const float extrapolated = position * powf(s.theta_scale, static_cast<float>(pair)) / factor;
     const float interpolated = s.freq_scale * extrapolated;
@@ -166,15 +154,62 @@ __global__ __launch_bounds__(kStoreThreads) void RopeSetRowsQuantKernel(const ll
       const float ramp = (1.0f - fminf(1.0f, fmaxf(0.0f, y))) * s.ext_factor;
       theta = interpolated * (1.0f - ramp) + extrapolated * ramp;
     }
-    const float c = cosf(theta) * magnitude, sn = sinf(theta) * magnitude;
-    const float x0 = x[pair], x1 = x[pair + half];
-    v[j] = channel < half ? x0 * c - x1 * sn : x0 * sn + x1 * c;
+    rotation[pair] = make_float2(cosf(theta) * magnitude, sinf(theta) * magnitude);
   }
+  __syncthreads();  // every thread: the loop below has no barrier
+  const int blocks_head = s.head_dim / 32, blocks_row = s.heads * blocks_head;
+  const bool wide = half % 32 == 0 && s.x_head_stride % 4 == 0 && s.x_token_stride % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(s.x) % 16 == 0;
   uint8_t* to = static_cast<uint8_t*>(s.destination) + s.ids[token] * s.row_bytes;
-  if (s.type == LLMP_TYPE_Q8_0) {
-    StoreQ8_0(v, to + block * 34);
-  } else {
-    StoreQ4_0(v, to + block * 18);
+  for (int block = threadIdx.x; block < blocks_row; block += kStoreThreads) {
+    const int head = block / blocks_head;
+    const int first = (block - head * blocks_head) * 32;  // channel within the head
+    const float* x = s.x + head * s.x_head_stride + token * s.x_token_stride;
+    float v[32];
+    if (wide) {
+      // The block lies within one half of the rotated channels (or past them): its 32 values and their partners'
+      // as 16-byte loads.
+      const float4* own = reinterpret_cast<const float4*>(x + first);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float4 f = own[i];
+        v[4 * i] = f.x, v[4 * i + 1] = f.y, v[4 * i + 2] = f.z, v[4 * i + 3] = f.w;
+      }
+      if (first < s.n_dims) {
+        const bool lower = first < half;
+        const int pair0 = lower ? first : first - half;
+        const float4* other = reinterpret_cast<const float4*>(x + (lower ? first + half : pair0));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float4 f = other[i];
+          const float partner[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const float2 r = rotation[pair0 + 4 * i + c];
+            const float mine = v[4 * i + c];
+            v[4 * i + c] = lower ? mine * r.x - partner[c] * r.y : partner[c] * r.y + mine * r.x;
+          }
+        }
+      }
+    } else {
+#pragma unroll 8
+      for (int j = 0; j < 32; ++j) {
+        const int channel = first + j;
+        if (channel >= s.n_dims) {
+          v[j] = x[channel];
+          continue;
+        }
+        const int pair = channel < half ? channel : channel - half;
+        const float2 r = rotation[pair];
+        const float x0 = x[pair], x1 = x[pair + half];
+        v[j] = channel < half ? x0 * r.x - x1 * r.y : x0 * r.y + x1 * r.x;
+      }
+    }
+    if (s.type == LLMP_TYPE_Q8_0) {
+      StoreQ8_0(v, to + block * 34);
+    } else {
+      StoreQ4_0(v, to + block * 18);
+    }
   }
 }
 
@@ -287,7 +322,8 @@ extern "C" int llmp_hip_rope_set_rows_quant(const llmp_rope_store* store, void* 
   if (!(s.freq_scale > 0.0f) || !(s.theta_scale > 0.0f)) return Refuse(1, "%s: a positive frequency and angle scale", op);
   const int64_t total = s.tokens * blocks_row;
   if (total > 0xFFFFFFFFll / 32) return Refuse(1, "%s: more than 2^32 - 1 values", op);
-  const dim3 grid(static_cast<unsigned>((total + kStoreThreads - 1) / kStoreThreads));
-  hipLaunchKernelGGL(RopeSetRowsQuantKernel, grid, dim3(kStoreThreads), 0, static_cast<hipStream_t>(stream), s, total);
+  if (s.tokens > 0x7FFFFFFFll || s.n_dims > 8192) return Refuse(1, "%s: more than 2^31 - 1 tokens or 8192 rotated dims", op);
+  hipLaunchKernelGGL(RopeSetRowsQuantKernel, dim3(static_cast<unsigned>(s.tokens)), dim3(kStoreThreads),
+                     static_cast<size_t>(s.n_dims / 2) * sizeof(float2), static_cast<hipStream_t>(stream), s);
   return LaunchStatus(op);
 }

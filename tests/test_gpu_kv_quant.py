@@ -114,14 +114,15 @@ def test_grouped_store_refusals(device):
 
 @pytest.mark.parametrize("t", [ops.TYPE_Q8_0, ops.TYPE_Q4_0])
 @pytest.mark.parametrize("yarn", [False, True])
-def test_rope_then_store_matches_the_oracles_rotation_and_quantizer(device, t, yarn):
+@pytest.mark.parametrize("n_dims", [96, 64])  # halves of 48 (a block spans both) and of 32 (16-byte loads)
+def test_rope_then_store_matches_the_oracles_rotation_and_quantizer(device, t, yarn, n_dims):
     """llmp.rope.set_rows_quant (src/kernels/ggml/kv_quant.h:180-192, kv_quant_rope.cu:29-120 of the reference)
     against oracle.rope_neox followed by the reference quantizers. The device rotates with F32 cosf / sinf / powf,
     the oracle as the reference's CPU executor does (FP64 cosine, sine and products): the stored bytes are the
     oracle's except for a few codes whose value lies at a rounding boundary (at most 1 in 500 bytes may differ here,
     and every stored value is within 0.6 quantization steps, Q4_0 1.1, of the oracle's rotated value)."""
     g = synth.rng(95)
-    tokens, heads, head_dim, n_dims, cells = 9, 4, 128, 96, 20
+    tokens, heads, head_dim, cells = 9, 4, 128, 20
     whole = synth.activations(tokens, heads * (head_dim + 32), 96).reshape(tokens, heads, head_dim + 32)
     x = whole[:, :, :head_dim]  # heads 160 floats apart
     pos = np.array([0, 1, 2, 17, 100, 511, 1024, 2047, 3000], dtype=np.int32)
