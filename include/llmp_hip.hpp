@@ -134,6 +134,28 @@ inline int Run(const Gemm& gemm, int sms, void* stream) {
 }
 
 }  // namespace mxfp8
+
+// The quantizing KV cache stores (src/kernels/ggml/kv_quant.h:150-192 of the reference): SetRowsQuant's
+// two-dimensional case, SetRowsQuantGroup over two to sixteen of them, RopeSetRowsQuant.
+namespace kv {
+
+inline constexpr std::size_t kSetRowsQuantGroupMax = 16;  // kv_quant.h:84
+
+using Store = llmp_set_rows_store;
+using RopeStore = llmp_rope_store;
+
+inline KernelFailure SetRowsQuant(const Store& s, void* stream) {
+  return FromStatus(llmp_hip_set_rows_quant(s.type, s.x, s.x_stride, s.ids, s.index_bytes, s.destination, s.row_bytes,
+                                            s.k, s.rows, stream));
+}
+inline KernelFailure SetRowsQuantGroup(const Store* stores, std::size_t count, void* stream) {
+  return FromStatus(llmp_hip_set_rows_quant_group(static_cast<int>(count), stores, stream));
+}
+inline KernelFailure RopeSetRowsQuant(const RopeStore& s, void* stream) {
+  return FromStatus(llmp_hip_rope_set_rows_quant(&s, stream));
+}
+
+}  // namespace kv
 }  // namespace ggml
 
 namespace decode {

@@ -127,6 +127,15 @@ void HostChecks() {
   EXPECT(hipk::decode::RunRows(gather, nullptr) == hipk::KernelFailure::kRejected);
   hipk::decode::GroupedProduct grouped;
   EXPECT(hipk::decode::RunGrouped(grouped, nullptr) == hipk::KernelFailure::kRejected);
+  // The KV cache stores: refusals without a GPU.
+  hipk::ggml::kv::Store store{};
+  EXPECT(hipk::ggml::kv::SetRowsQuant(store, nullptr) == hipk::KernelFailure::kRejected);
+  hipk::ggml::kv::Store pair[2] = {store, store};
+  EXPECT(hipk::ggml::kv::SetRowsQuantGroup(pair, 1, nullptr) == hipk::KernelFailure::kRejected);
+  EXPECT(hipk::ggml::kv::SetRowsQuantGroup(pair, 2, nullptr) == hipk::KernelFailure::kRejected);
+  hipk::ggml::kv::RopeStore rope{};
+  EXPECT(hipk::ggml::kv::RopeSetRowsQuant(rope, nullptr) == hipk::KernelFailure::kRejected);
+  EXPECT(!hipk::LastError().empty());
   hipk::exl3::MultiLinearOperands multi;
   EXPECT(hipk::exl3::MultiLinear(multi, nullptr, 0, nullptr) == hipk::KernelFailure::kRejected);
   EXPECT(hipk::exl3::ScratchBytes(multi) == 0);
