@@ -192,7 +192,8 @@ typedef struct llmp_mxfp8_gemm {
   const void* b;        /* codes, n rows of k */
   const void* b_scales; /* atoms */
   void* d;              /* m rows of n */
-  int bf16;             /* D in BF16, else F32 */
+  unsigned char bf16;   /* one byte, as the reference's `bool bf16` (mxfp8_cutlass.h:67): non-zero is D in
+                           BF16, else F32; the seven bytes of padding after it are never read */
   void* scratch;        /* llmp_hip_mxfp8_gemm_scratch bytes, 256-byte aligned (none needed: may be null) */
 } llmp_mxfp8_gemm;
 int llmp_hip_mxfp8_gemm_available(void);
@@ -205,10 +206,14 @@ int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void
  * ids[r] (I32 or I64 by index_bytes) of a Q8_0 or Q4_0 destination whose rows are row_bytes
  * apart. Each block of 32 is quantized with the arithmetic of src/kernels/ggml/kv_quant.cuh:27-69
  * (GGML's reference quantizers, every step an IEEE operation). The two-dimensional case of
- * ggml_set_rows's shapes: one plane, no broadcast of the indices. Indices are the caller's to
- * bound (kv_quant.h:62-63). */
+ * ggml_set_rows's shapes only: one plane, one batch, no broadcast of the indices (the reference's
+ * kv_quant_store.cu:27-58 also takes planes and batches; a caller with per-head planes makes one call a
+ * plane, or one grouped call of up to sixteen). `cells` is the destination's number of rows, by which the
+ * call refuses a destination that overlaps the values or the indices. Indices are the caller's to bound
+ * (kv_quant.h:62-63). */
 int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
-                            void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream);
+                            void* destination, int64_t row_bytes, int64_t k, int64_t rows, int64_t cells,
+                            void* stream);
 
 /* llmp.set_rows.grouped_quant (SetRowsQuantGroup, src/kernels/ggml/kv_quant.h:82-84, 172-178;
  * src/kernels/ggml/kv_quant.cc:214-236): two to sixteen such stores in one launch (a layer's K and V rows, or

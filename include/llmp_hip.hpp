@@ -12,6 +12,8 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "llmp_hip.h"
 
@@ -146,7 +148,7 @@ using RopeStore = llmp_rope_store;
 
 inline KernelFailure SetRowsQuant(const Store& s, void* stream) {
   return FromStatus(llmp_hip_set_rows_quant(s.type, s.x, s.x_stride, s.ids, s.index_bytes, s.destination, s.row_bytes,
-                                            s.k, s.rows, stream));
+                                            s.k, s.rows, s.cells, stream));
 }
 inline KernelFailure SetRowsQuantGroup(const Store* stores, std::size_t count, void* stream) {
   return FromStatus(llmp_hip_set_rows_quant_group(static_cast<int>(count), stores, stream));
@@ -347,6 +349,170 @@ inline KernelFailure MultiLinear(const MultiLinearOperands& o, void* scratch, st
 }
 
 }  // namespace exl3
+// ---------------------------------------------------------------------------------------------
+// The implementation registry's entries for these kernels (src/execution/registry.h:131-195 and
+// 297-356 of the reference): what each implementation computes, under the names the planner and
+// its plans use (src/kernels/ggml/capabilities.cc:2486-2489 and 2881-2893,
+// src/kernels/ggml/plan_step.h:201-314, src/kernels/decode/implementations.h:7-13,
+// src/kernels/exl3/implementations.h:8-31). The reference's types hold spans into static tables
+// and IR keys; here the same facts are plain values, so that a binding can build its
+// execution::Implementation from them field by field. "C++ only": nothing of this crosses the C ABI.
+namespace execution {
+
+// registry.h:50-55.
+enum class Rung : std::uint8_t { kNative = 1, kOnChipDecode = 2, kBf16Decode = 5, kPrimitive = 6 };
+// registry.h:75-81.
+enum DeviceFeature : std::uint32_t { kBf16Mma = 1u << 0, kInt8Mma = 1u << 1, kFp8Mma = 1u << 2, kFp4Mma = 1u << 3, kBlockScaledMma = 1u << 4 };
+// The provider's architecture number of the one device this library is built for.
+inline constexpr std::uint32_t kGfx950 = 950;
+// registry.h:91-96.
+struct ShapeRule {
+  std::uint64_t min_rows = 1;
+  std::uint64_t max_rows = ~std::uint64_t{0};
+  std::uint64_t k_multiple = 1;
+  std::uint64_t n_multiple = 1;
+};
+// registry.h:101-170, the fields these implementations set.
+struct Capability {
+  std::string op;                      // the IR operation: ir::Primitive / ir::Fused's name
+  std::vector<std::string> encodings;  // operand 0 (the weight, or the stored destination): any of these
+  std::uint32_t min_arch = kGfx950, max_arch = kGfx950;
+  std::uint32_t needs = 0;  // DeviceFeature bits
+  ShapeRule shape{};
+  Rung rung = Rung::kNative;
+  bool row_invariant = true;  // a row's result never depends on the rows computed beside it
+  bool capturable = true;     // every entry point only queues launches with replay-invariant arguments
+  std::string group;          // "ggml.mul_mat" for the members of upstream's routing
+  std::vector<std::string> launches;  // the entry points (llmp_hip.h) a node of it queues, in order
+};
+// registry.h:322-349.
+struct Implementation {
+  std::string name;
+  std::string source = "llmp_amd";
+  std::string build = "hipcc --offload-arch=gfx950 -O3";
+  std::string variant;
+  std::uint32_t version = 1;
+  Capability capability;
+};
+// registry.h:297-320, the fields a product's query sets.
+struct CapabilityQuery {
+  std::string op;
+  std::string encoding;  // operand 0's
+  std::uint64_t rows = 1, k = 0, n = 0;
+  std::uint32_t arch = kGfx950;
+  std::uint32_t features = kBf16Mma | kInt8Mma | kFp8Mma | kFp4Mma | kBlockScaledMma;
+  bool row_invariant = false;  // required
+  bool capturable = false;     // required
+};
+
+inline const char* const kDecoderNames[] = {"bf16.dense",  "f16.dense",   "q8_0.blocks", "nvfp4.split", "nvfp4.atoms", "nvfp4.interleaved",
+                                            "nvfp4.ggml_blocks", "mxfp8.split", "mxfp8.atoms", "mxfp4.split", "mxfp4.atoms", "affine.split"};
+
+inline std::vector<Implementation> Implementations() {
+  std::vector<Implementation> all;
+  const std::vector<std::string> blocks = {"q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k", "iq4_nl", "mxfp4"};
+  const auto add = [&](std::string name, std::string op, std::vector<std::string> encodings, ShapeRule shape, Rung rung,
+                       std::uint32_t needs, std::vector<std::string> launches, std::string variant, std::string group = "") {
+    Implementation i;
+    i.name = std::move(name);
+    i.variant = std::move(variant);
+    i.capability.op = std::move(op);
+    i.capability.encodings = std::move(encodings);
+    i.capability.shape = shape;
+    i.capability.rung = rung;
+    i.capability.needs = needs;
+    i.capability.launches = std::move(launches);
+    i.capability.group = std::move(group);
+    all.push_back(std::move(i));
+  };
+  const std::uint64_t any = ~std::uint64_t{0};
+  // capabilities.cc:2881-2893 and plan_step.h:201-314: the activation quantizer and the products over its blocks.
+  add("llmp.q8_1", "quantize.block32_q8_sum_f32", {"f32"}, {1, 65535, 1, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize"},
+      "eight lanes a block; rows padded to 512 values");
+  add("llmp.vecq.dense", "mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, kInt8Mma, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "a lane a unit through LDS (1 to 5 tokens), int8 matrix cores above");
+  add("llmp.vecq.glu", "fused.mul_mat_glu", blocks, {1, 16, 256, 1}, Rung::kNative, kInt8Mma, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "gate and up rows in one tile, the GLU in the row's first lane");
+  add("llmp.vecq.experts", "mul_mat_id", blocks, {1, 128, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "up to 128 (token, slot) pairs; the first pair naming an expert owns it");
+  add("llmp.vecq.experts_glu", "fused.mul_mat_id_glu", blocks, {1, 128, 256, 1}, Rung::kNative, 0,
+      {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"}, "up to 128 (token, slot) pairs, fused GLU");
+  add("llmp.vecq.grouped", "fused.grouped_mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "matrix g with input row g: up to 256 groups");
+  add("llmp.vecq.sorted", "mul_mat_id", {"q8_0", "q4_k"}, {129, any, 256, 1}, Rung::kNative, kInt8Mma,
+      {"llmp_hip_moe_route", "llmp_hip_q8_1_quantize_rows", "llmp_hip_vecq_sorted"}, "rows sorted by expert on the int8 matrix cores");
+  // Upstream's routing names (capabilities.cc:2486-2489): the same launches, members of its group.
+  add("ggml.mul_mat.mmvq", "mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "llmp.vecq.dense's launches", "ggml.mul_mat");
+  add("ggml.mul_mat_glu.mmvq_fused", "fused.mul_mat_glu", blocks, {1, 16, 256, 1}, Rung::kNative, 0,
+      {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"}, "llmp.vecq.glu's launches", "ggml.mul_mat");
+  add("llmp.moe.router", "route.softmax_top_k", {"f32"}, {1, any, 1, 1}, Rung::kNative, 0, {"llmp_hip_moe_router"},
+      "a wave a token; up to 1024 experts, 64 picks");
+  add("llmp.moe.combine", "fused.moe_combine", {"f32"}, {1, any, 4, 1}, Rung::kNative, 0, {"llmp_hip_moe_combine"},
+      "ordered float sum over the slots");
+  // MXFP8 (plan_step.h, mxfp8_cutlass.h): the reference's names, "cutlass" included, since plans carry them.
+  add("llmp.mxfp8.mul_mat_vec", "mul_mat", {"mxfp8"}, {1, 16, 32, 1}, Rung::kNative, 0, {"llmp_hip_mxfp8_gemv"}, "a wave a row");
+  add("llmp.mxfp8.quantize", "quantize.mxfp8", {"f32", "bf16"}, {1, any, 128, 1}, Rung::kNative, 0, {"llmp_hip_mxfp8_quantize"},
+      "codes and scale atoms");
+  add("llmp.mxfp8.swizzle", "relayout.scale_atoms", {"e8m0"}, {1, any, 128, 1}, Rung::kNative, 0, {"llmp_hip_mxfp8_swizzle"}, "128 x 4 atoms");
+  add("llmp.mxfp8.gemm.cutlass", "mul_mat", {"mxfp8"}, {1, any, 128, 1}, Rung::kNative, kFp8Mma | kBlockScaledMma,
+      {"llmp_hip_mxfp8_swizzle", "llmp_hip_mxfp8_gemm_run"}, "v_mfma_scale_f32_16x16x128_f8f6f4, 256 x 192 tiles");
+  // The decode templates (decode/implementations.h:7-13): llmp.decode.<template>.<encoding>.<layout>.
+  struct Template {
+    const char* name;
+    const char* op;
+    ShapeRule shape;
+    std::uint32_t needs;
+    const char* launch;
+  };
+  const Template templates[] = {{"vector", "mul_mat", {1, 16, 16, 1}, 0, "llmp_hip_decode_vector"},
+                                {"vector_glu", "fused.mul_mat_glu", {1, 16, 16, 1}, 0, "llmp_hip_decode_vector_glu"},
+                                {"matrix", "mul_mat", {1, 65535ull * 64ull, 16, 1}, kBf16Mma, "llmp_hip_decode_matrix"},
+                                {"grouped", "mul_mat_id", {1, any, 16, 1}, 0, "llmp_hip_decode_grouped"},
+                                {"rows", "get_rows", {1, any, 16, 1}, 0, "llmp_hip_decode_rows"}};
+  for (const Template& t : templates) {
+    for (int d = 0; d < 12; ++d) {
+      const std::string decoder = kDecoderNames[d];
+      add(std::string("llmp.decode.") + t.name + "." + decoder, t.op, {decoder.substr(0, decoder.find('.'))}, t.shape,
+          d < 2 ? Rung::kNative : Rung::kOnChipDecode, t.needs, {t.launch}, std::string("decoder ") + std::to_string(d));
+    }
+  }
+  // EXL3 (exl3/implementations.h:8-31): the packed paths; the reconstruction paths are not built.
+  add("exl3.linear.gemv", "quant_linear", {"exl3"}, {1, 8, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
+      "trellis tiles as the second operand of a 16 x 16 x 16 F16 matrix instruction");
+  add("exl3.linear.gemm", "quant_linear", {"exl3"}, {1, 16, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
+      "the same launches for up to 16 rows");
+  add("exl3.multi_linear.mgemm", "quant_multi_linear", {"exl3"}, {1, 16, 128, 128}, Rung::kOnChipDecode, kBf16Mma,
+      {"llmp_hip_exl3_multi_linear"}, "gate and up in grid z");
+  // The quantizing KV cache stores (kv_quant.h:150-192).
+  add("llmp.set_rows.quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant"}, "a thread a block");
+  add("llmp.set_rows.grouped_quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant_group"},
+      "two to sixteen stores a launch");
+  add("llmp.rope.set_rows_quant", "fused.rope_set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0,
+      {"llmp_hip_rope_set_rows_quant"}, "a workgroup a token");
+  return all;
+}
+
+// Whether `i` computes what `q` asks (registry.h's Candidates filter: operation, operand 0's encoding, device and shape).
+inline bool Computes(const Implementation& i, const CapabilityQuery& q) {
+  const Capability& c = i.capability;
+  if (c.op != q.op || q.arch < c.min_arch || q.arch > c.max_arch || (c.needs & ~q.features) != 0) return false;
+  bool encoding = c.encodings.empty();
+  for (const std::string& e : c.encodings) encoding = encoding || e == q.encoding;
+  if (!encoding) return false;
+  if (q.rows < c.shape.min_rows || q.rows > c.shape.max_rows) return false;
+  if (q.k % c.shape.k_multiple != 0 || q.n % c.shape.n_multiple != 0) return false;
+  return (!q.row_invariant || c.row_invariant) && (!q.capturable || c.capturable);
+}
+inline std::vector<Implementation> Candidates(const CapabilityQuery& q) {
+  std::vector<Implementation> found;
+  for (Implementation& i : Implementations()) {
+    if (Computes(i, q)) found.push_back(std::move(i));
+  }
+  return found;
+}
+
+}  // namespace execution
 }  // namespace llmp_amd
 
 #endif  // LLMP_HIP_HPP_

@@ -38,7 +38,7 @@ class VecQDesc(C.Structure):
 class Mxfp8Gemm(C.Structure):
     """llmp_mxfp8_gemm: mxfp8::Gemm of src/kernels/ggml/mxfp8_cutlass.h:56-70 of the reference."""
     _fields_ = [("m", C.c_int), ("n", C.c_int), ("k", C.c_int), ("a", C.c_void_p), ("a_scales", C.c_void_p),
-                ("b", C.c_void_p), ("b_scales", C.c_void_p), ("d", C.c_void_p), ("bf16", C.c_int),
+                ("b", C.c_void_p), ("b_scales", C.c_void_p), ("d", C.c_void_p), ("bf16", C.c_uint8),
                 ("scratch", C.c_void_p)]
 
 
@@ -109,7 +109,7 @@ SYMBOLS = {
     "llmp_hip_moe_route": (_int, [_vp, _int, _int, _int, _int, _vp, _vp]),
     "llmp_hip_q8_1_quantize_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_moe_combine": (_int, [_vp, _vp, _vp, _int, _int, _int, _vp, _vp]),
-    "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
+    "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
     "llmp_hip_rope_set_rows_quant": (_int, [C.POINTER(RopeStore), _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),

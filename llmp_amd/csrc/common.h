@@ -9,7 +9,14 @@ namespace llmp_hip {
 
 // ---- host: status of the calling thread's last refusal or fault.
 void SetError(const char* format, ...) __attribute__((format(printf, 1, 2)));
-// 0 if the last launch was accepted, else -(hipError_t) with the error recorded.
+// Called by an entry point once its checks have passed, before its first launch: forgets an error that an
+// earlier, unrelated HIP call left on this thread, so that LaunchStatus judges this call's launches only.
+void BeginLaunches();
+// Asks once for `bytes` of dynamic LDS for a kernel that needs more than 64 KB. False: the runtime refused; the
+// reason is recorded, the launch must be skipped, the next LaunchStatus returns the failure and `sized` stays
+// clear so that the next call asks again.
+bool AllowLds(const void* kernel, int bytes, bool* sized);
+// 0 if the launches since BeginLaunches were accepted, else -(hipError_t) with the error recorded.
 int LaunchStatus(const char* what);
 int Refuse(int code, const char* format, ...) __attribute__((format(printf, 2, 3)));
 

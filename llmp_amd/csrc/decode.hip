@@ -772,11 +772,7 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
 template <int D>
 void LaunchMatrixShared(const DecodeArgs& a, dim3 grid, uint32_t rows, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeMatrixSharedKernel<D>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kSharedStageBytes);
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&DecodeMatrixSharedKernel<D>), 2 * kSharedStageBytes, &sized)) return;
   hipLaunchKernelGGL((DecodeMatrixSharedKernel<D>), grid, dim3(512), 2 * kSharedStageBytes, stream, a, rows);
 }
 
@@ -785,11 +781,7 @@ size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * 
 template <int D, int T, bool kGlu>
 void LaunchDecode(const DecodeArgs& a, int groups, int waves, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T, kGlu>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDecodeLdsLimit));
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T, kGlu>), static_cast<int>(kDecodeLdsLimit), &sized)) return;
   hipLaunchKernelGGL((DecodeVectorKernel<D, T, kGlu>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
                      DecodeLds(T, a.w.k), stream, a);
 }
@@ -927,6 +919,7 @@ using namespace llmp_hip;
 extern "C" int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
                                       const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
                                       void* stream) {
+  BeginLaunches();
   if (const int bad = CheckOperand("decode.vector", decoder, w, first, outputs); bad != 0) return bad;
   if (x == nullptr || y == nullptr) return Refuse(1, "decode.vector: null operand");
   DecodeArgs a{};
@@ -941,6 +934,7 @@ extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_op
                                           int up_decoder, const llmp_decode_operand* up, uint64_t up_first,
                                           uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
                                           uint64_t x_stride, float* y, uint64_t y_stride, void* stream) {
+  BeginLaunches();
   if (const int bad = CheckOperand("decode.vector_glu gate", gate_decoder, gate, gate_first, outputs); bad != 0) return bad;
   if (const int bad = CheckOperand("decode.vector_glu up", up_decoder, up, up_first, outputs); bad != 0) return bad;
   if (gate_decoder != up_decoder)
@@ -961,6 +955,7 @@ extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_op
 
 extern "C" int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* w, const int32_t* ids, uint64_t count,
                                     float* out, uint64_t out_stride, int32_t* bad, void* stream) {
+  BeginLaunches();
   if (const int status = CheckOperand("decode.rows", decoder, w, 0, 1); status != 0) return status;
   if (ids == nullptr || out == nullptr) return Refuse(1, "decode.rows: null operand");
   if (count == 0 || count > (uint64_t{1} << 31)) return Refuse(1, "decode.rows: 1 to 2^31 rows");
@@ -998,11 +993,7 @@ namespace {
 template <int D, int T>
 void LaunchGrouped(const GroupedArgs& a, dim3 grid, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&DecodeGroupedKernel<D, T>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDecodeLdsLimit));
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&DecodeGroupedKernel<D, T>), static_cast<int>(kDecodeLdsLimit), &sized)) return;
   hipLaunchKernelGGL((DecodeGroupedKernel<D, T>), grid, dim3(kDecodeWaves * 64), DecodeLds(T, a.k), stream, a);
 }
 
@@ -1023,6 +1014,7 @@ extern "C" int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* e
                                        const int32_t* pair_rows, const int32_t* pair_out, uint64_t pairs, const float* x,
                                        uint64_t x_rows, uint64_t x_stride, float* y, uint64_t y_rows, uint64_t y_stride,
                                        uint64_t rows_hint, void* stream) {
+  BeginLaunches();
   (void)rows_hint;  // picks the reference's tile; the passes here are of up to four pairs whatever it is
   if (decoder < 0 || decoder > LLMP_DECODER_AFFINE_SPLIT) return Refuse(1, "decode.grouped: decoder %d has no kernel", decoder);
   if (experts == nullptr || offsets == nullptr || pair_rows == nullptr || x == nullptr || y == nullptr)
@@ -1078,6 +1070,7 @@ extern "C" int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* e
 extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w, uint64_t first, uint64_t outputs,
                                       const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,
                                       int path, void* stream) {
+  BeginLaunches();
   if (const int bad = CheckOperand("decode.matrix", decoder, w, first, outputs); bad != 0) return bad;
   if (x == nullptr || y == nullptr) return Refuse(1, "decode.matrix: null operand");
   if (path != 0) return Refuse(1, "decode.matrix: the FMA path is for devices without matrix cores; this one has them");

@@ -26,6 +26,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <initializer_list>
+
 #include <type_traits>
 
 #include "common.h"
@@ -403,6 +405,28 @@ int CheckWeights(const llmp_exl3_weights& w) {
   return 0;
 }
 
+// Byte ranges of operands, and the reference's refusal of a written range that meets another
+// (src/kernels/exl3/validate.cc:32-62: "{} overlaps {}"), before anything is queued.
+struct Range {
+  const char* name;
+  uintptr_t base;
+  size_t bytes;
+};
+bool Overlap(const Range& a, const Range& b) {
+  return a.bytes > 0 && b.bytes > 0 && a.base < b.base + b.bytes && b.base < a.base + a.bytes;
+}
+int Disjoint(const char* what, const Range& written, std::initializer_list<Range> others) {
+  for (const Range& other : others) {
+    if (Overlap(written, other)) return Refuse(1, "%s: %s overlaps %s", what, written.name, other.name);
+  }
+  return 0;
+}
+Range TrellisRange(const llmp_exl3_weights& w) {
+  return {"the trellis", reinterpret_cast<uintptr_t>(w.trellis), static_cast<size_t>(w.k) * w.n * w.bits / 8};
+}
+Range SuhRange(const llmp_exl3_weights& w) { return {"suh", reinterpret_cast<uintptr_t>(w.suh), static_cast<size_t>(w.k) * 2}; }
+Range SvhRange(const llmp_exl3_weights& w) { return {"svh", reinterpret_cast<uintptr_t>(w.svh), static_cast<size_t>(w.n) * 2}; }
+
 template <int CB, int BITS>
 void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int columns, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(columns / 16), static_cast<unsigned>((w.k / 16 + 3) / 4));
@@ -419,11 +443,7 @@ void LaunchProduct(const llmp_exl3_weights& w, const ProductSides& sides, int co
   constexpr int kWork = kProductWaves * (kRingDepth * kLoads * 1024 + kOperandBytes);
   constexpr int kLds = kWork > kReduceBytes ? kWork : kReduceBytes;
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&ProductKernel<CB, BITS, kFused>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&ProductKernel<CB, BITS, kFused>), kLds, &sized)) return;
   const int blocks = w.k / 128;
   const int per = (blocks + slices * kProductWaves - 1) / (slices * kProductWaves);
   const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices), static_cast<unsigned>(count));
@@ -467,10 +487,16 @@ using namespace llmp_hip;
 
 extern "C" int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void* w, int column, int columns,
                                          void* stream) {
+  BeginLaunches();
   if (weights == nullptr || w == nullptr) return Refuse(1, "exl3.reconstruct: null operand");
   if (const int bad = CheckWeights(*weights); bad != 0) return bad;
   if (column < 0 || columns <= 0 || column % 16 != 0 || columns % 16 != 0 || column + columns > weights->n)
     return Refuse(1, "exl3.reconstruct: columns [%d, %d) are not whole tiles of the weights", column, column + columns);
+  // validate.cc:379-382: the reconstructed matrix meets none of the weights' tensors.
+  if (const int bad = Disjoint("exl3.reconstruct", {"w", reinterpret_cast<uintptr_t>(w), static_cast<size_t>(weights->k) * columns * 2},
+                               {TrellisRange(*weights), SuhRange(*weights), SvhRange(*weights)});
+      bad != 0)
+    return bad;
   Dispatch(weights->codebook, weights->bits, [&](auto cb, auto bits) {
     LaunchReconstruct<decltype(cb)::value, decltype(bits)::value>(*weights, w, column, columns,
                                                                   static_cast<hipStream_t>(stream));
@@ -480,10 +506,24 @@ extern "C" int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void*
 
 extern "C" int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, int columns, int f32,
                                       int input_scale, void* stream) {
+  BeginLaunches();
   if (x == nullptr || y == nullptr || scale == nullptr) return Refuse(1, "exl3.hadamard: null operand");
   if (rows <= 0 || rows > 65535 || columns <= 0 || columns % 128 != 0)
     return Refuse(1, "exl3.hadamard: 1 to 65535 rows of whole 128-value blocks");
   if (input_scale && f32) return Refuse(1, "exl3.hadamard: the input scale's transform is F16");
+  {
+    // validate.cc:411-416: in place (y == x, F16 only: a lane reads its values before it writes them) or disjoint.
+    const size_t cells = static_cast<size_t>(rows) * columns;
+    const Range xr{"x", reinterpret_cast<uintptr_t>(x), cells * 2};
+    const Range yr{"y", reinterpret_cast<uintptr_t>(y), cells * (f32 ? 4 : 2)};
+    if (x == y && f32) return Refuse(1, "exl3.hadamard: an F32 output cannot be the F16 input");
+    if (x != y) {
+      if (const int bad = Disjoint("exl3.hadamard", yr, {xr}); bad != 0) return bad;
+    }
+    if (const int bad = Disjoint("exl3.hadamard", yr, {{"the scale", reinterpret_cast<uintptr_t>(scale), static_cast<size_t>(columns) * 2}});
+        bad != 0)
+      return bad;
+  }
   const dim3 grid(static_cast<unsigned>(rows), static_cast<unsigned>(columns / 128));
   const auto s = static_cast<hipStream_t>(stream);
   const auto* sc = static_cast<const uint16_t*>(scale);
@@ -559,6 +599,7 @@ extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
 }
 
 extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream) {
+  BeginLaunches();
   if (op == nullptr) return Refuse(1, "exl3.linear: null operands");
   if (const int bad = CheckWeights(op->weights); bad != 0) return bad;
   if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || scratch == nullptr)
@@ -568,6 +609,19 @@ extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, s
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
        reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
     return Refuse(1, "exl3.linear: operands not 8-byte aligned");
+  {
+    // validate.cc:120-126: what the launches write (a_had, y, the partial sums in place of the lock area) meets
+    // nothing they read and not one another.
+    const size_t m = static_cast<size_t>(op->m);
+    const Range x{"x", reinterpret_cast<uintptr_t>(op->x), m * op->weights.k * 2};
+    const Range a_had{"a_had", reinterpret_cast<uintptr_t>(op->a_had), m * op->weights.k * 2};
+    const Range y{"y", reinterpret_cast<uintptr_t>(op->y), m * op->weights.n * (op->f32 ? 4 : 2)};
+    const Range area{"the scratch", reinterpret_cast<uintptr_t>(scratch), llmp_hip_exl3_linear_scratch(op)};
+    const llmp_exl3_weights& w = op->weights;
+    if (const int bad = Disjoint("exl3.linear", a_had, {x, y, TrellisRange(w), SuhRange(w), SvhRange(w), area}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.linear", y, {x, TrellisRange(w), SuhRange(w), SvhRange(w), area}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.linear", area, {x, TrellisRange(w), SuhRange(w), SvhRange(w)}); bad != 0) return bad;
+  }
   const llmp_exl3_weights* const w[2] = {&op->weights, &op->weights};
   void* const a_had[2] = {op->a_had, op->a_had};
   void* const y[2] = {op->y, op->y};
@@ -582,6 +636,7 @@ extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linea
 
 extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, size_t scratch_bytes,
                                           void* stream) {
+  BeginLaunches();
   if (op == nullptr) return Refuse(1, "exl3.multi_linear: null operands");
   if (const int bad = CheckWeights(op->first); bad != 0) return bad;
   if (const int bad = CheckWeights(op->second); bad != 0) return bad;
@@ -594,6 +649,23 @@ extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
        reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
     return Refuse(1, "exl3.multi_linear: operands not 8-byte aligned");
+  {
+    // validate.cc:310-323: a_had, y and the partial sums meet nothing the launches read and not one another.
+    const size_t rows = static_cast<size_t>(op->m);
+    const Range x{"x", reinterpret_cast<uintptr_t>(op->x), rows * op->first.k * 2};
+    const Range a_had{"a_had", reinterpret_cast<uintptr_t>(op->a_had), 2 * rows * op->first.k * 2};
+    const Range y{"y", reinterpret_cast<uintptr_t>(op->y), 2 * rows * op->first.n * (op->f32 ? 4 : 2)};
+    const Range area{"the scratch", reinterpret_cast<uintptr_t>(scratch), llmp_hip_exl3_multi_linear_scratch(op)};
+    for (const llmp_exl3_weights* w : {&op->first, &op->second}) {
+      for (const Range& written : {a_had, y, area}) {
+        if (const int bad = Disjoint("exl3.multi_linear", written, {TrellisRange(*w), SuhRange(*w), SvhRange(*w)}); bad != 0)
+          return bad;
+      }
+    }
+    if (const int bad = Disjoint("exl3.multi_linear", a_had, {x, y, area}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.multi_linear", y, {x, area}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.multi_linear", area, {x}); bad != 0) return bad;
+  }
   const auto s = static_cast<hipStream_t>(stream);
   const int m = op->m, k = op->first.k, n = op->first.n;
   const size_t out_bytes = static_cast<size_t>(m) * n * (op->f32 ? 4 : 2);

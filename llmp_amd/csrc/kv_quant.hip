@@ -241,6 +241,7 @@ bool Meet(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes) {
 using namespace llmp_hip;
 
 extern "C" int llmp_hip_set_rows_quant_group(int count, const llmp_set_rows_store* stores, void* stream) {
+  BeginLaunches();
   const char* op = "set_rows.grouped_quant";
   if (stores == nullptr) return Refuse(1, "%s: null stores", op);
   if (count < 2 || count > 16) return Refuse(1, "%s: two through sixteen stores, not %d", op, count);  // kv_quant.cc:216
@@ -277,18 +278,18 @@ extern "C" int llmp_hip_set_rows_quant_group(int count, const llmp_set_rows_stor
 }
 
 extern "C" int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_stride, const void* ids, int index_bytes,
-                                       void* destination, int64_t row_bytes, int64_t k, int64_t rows, void* stream) {
-  if (x == nullptr || ids == nullptr || destination == nullptr) return Refuse(1, "set_rows.quant: null operand");
-  if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_0) return Refuse(1, "set_rows.quant: a Q8_0 or Q4_0 destination");
-  if (index_bytes != 4 && index_bytes != 8) return Refuse(1, "set_rows.quant: I32 or I64 indices");
-  if (k <= 0 || k % 32 != 0 || rows <= 0) return Refuse(1, "set_rows.quant: rows of whole 32-value blocks");
-  const int64_t block_bytes = type == LLMP_TYPE_Q8_0 ? 34 : 18;
-  if (x_stride < k || x_stride % 4 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0)
-    return Refuse(1, "set_rows.quant: source rows overlap or are not 16-byte aligned");
-  if (row_bytes < k / 32 * block_bytes || row_bytes % 2 != 0 || reinterpret_cast<uintptr_t>(destination) % 2 != 0)
-    return Refuse(1, "set_rows.quant: destination rows overlap or are not 2-byte aligned");
-  const int64_t total = rows * (k / 32);
-  if (total > 0xFFFFFFFFll / 32) return Refuse(1, "set_rows.quant: more than 2^32 - 1 values");  // kv_quant.h:150-156
+                                       void* destination, int64_t row_bytes, int64_t k, int64_t rows, int64_t cells,
+                                       void* stream) {
+  BeginLaunches();
+  const char* op = "set_rows.quant";
+  int64_t total = 0;
+  if (const int bad = CheckStore(op, type, x, x_stride, ids, index_bytes, destination, row_bytes, k, rows, &total); bad != 0)
+    return bad;
+  if (cells <= 0) return Refuse(1, "%s: a destination of no cells", op);
+  // The destination's cells meet neither the values nor the indices the launch reads.
+  if (Meet(destination, cells * row_bytes, x, ((rows - 1) * x_stride + k) * 4) ||
+      Meet(destination, cells * row_bytes, ids, rows * index_bytes))
+    return Refuse(1, "%s: the destination overlaps the values or the indices", op);
   const dim3 grid(static_cast<unsigned>((total + kStoreThreads - 1) / kStoreThreads));
   const auto s = static_cast<hipStream_t>(stream);
   auto* out = static_cast<uint8_t*>(destination);
@@ -303,6 +304,7 @@ extern "C" int llmp_hip_set_rows_quant(int type, const float* x, int64_t x_strid
 }
 
 extern "C" int llmp_hip_rope_set_rows_quant(const llmp_rope_store* store, void* stream) {
+  BeginLaunches();
   const char* op = "rope.set_rows_quant";
   if (store == nullptr) return Refuse(1, "%s: null store", op);
   const llmp_rope_store& s = *store;

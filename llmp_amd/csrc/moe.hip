@@ -413,6 +413,7 @@ using namespace llmp_hip;
 
 extern "C" int llmp_hip_moe_router(const float* logits, int experts, int used, int tokens, int normalize, float scale,
                                    int32_t* ids, float* weights, void* stream) {
+  BeginLaunches();
   if (logits == nullptr || ids == nullptr || weights == nullptr) return Refuse(1, "moe.router: null operand");
   if (experts < 1 || experts > kRouterSlots * kWave) return Refuse(1, "moe.router: 1 to %d experts", kRouterSlots * kWave);
   if (used < 1 || used > experts || used > kWave) return Refuse(1, "moe.router: 1 to min(experts, 64) picks, not %d", used);
@@ -441,6 +442,7 @@ extern "C" int64_t llmp_hip_moe_route_ints(int experts, int used, int tokens) {
 
 extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int experts, int used, int tokens,
                                   int32_t* route, void* stream) {
+  BeginLaunches();
   if (ids == nullptr || route == nullptr) return Refuse(1, "moe.route: null operand");
   if (experts < 1 || used < 1 || tokens < 1 || ids_stride < used) return Refuse(1, "moe.route: empty or overlapping ids");
   if (used > 128) return Refuse(1, "moe.route: more than 128 slots a token");  // a chunk's ids are staged in LDS
@@ -452,11 +454,8 @@ extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int expert
   if (slots <= kRouteOneSlots && runs * experts <= kRouteOneCounters) {
     const size_t bytes = static_cast<size_t>(((slots + 3) & ~int64_t{3}) + runs * experts + experts + 1) * sizeof(int32_t);
     static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-    if (!sized) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&RouteOne), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (kRouteOneSlots + kRouteOneCounters + kRouteOneCounters + 4) * 4);
-      sized = true;
-    }
+    if (!AllowLds(reinterpret_cast<const void*>(&RouteOne), (kRouteOneSlots + kRouteOneCounters + kRouteOneCounters + 4) * 4, &sized))
+      return LaunchStatus("moe.route");
     hipLaunchKernelGGL(RouteOne, dim3(1), dim3(kRouteOneThreads), bytes, s, ids, ids_stride, r);
     return LaunchStatus("moe.route");
   }
@@ -471,6 +470,7 @@ extern "C" int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int expert
 
 extern "C" int llmp_hip_q8_1_quantize_rows(const float* x, const int32_t* rows, void* out, int64_t k, int64_t padded_k,
                                            int64_t row_stride, int64_t count, void* stream) {
+  BeginLaunches();
   if (x == nullptr || out == nullptr) return Refuse(1, "q8_1: null operand");
   if (k <= 0 || count <= 0 || count > 65535) return Refuse(1, "q8_1: 1 to 65535 rows");
   if (padded_k < k || padded_k % 32 != 0) return Refuse(1, "q8_1: padded k below k or not whole blocks");
@@ -482,6 +482,7 @@ extern "C" int llmp_hip_q8_1_quantize_rows(const float* x, const int32_t* rows, 
 
 extern "C" int llmp_hip_moe_combine(const float* x, const float* weights, const int32_t* position, int width, int used,
                                     int tokens, float* out, void* stream) {
+  BeginLaunches();
   if (x == nullptr || weights == nullptr || out == nullptr) return Refuse(1, "moe.combine: null operand");
   if (width < 4 || width % 4 != 0 || used < 1 || tokens < 1) return Refuse(1, "moe.combine: width a multiple of 4");
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)

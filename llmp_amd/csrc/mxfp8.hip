@@ -440,11 +440,7 @@ int LaunchGemm(GemmArgs a, hipStream_t stream) {
   static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
   a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
   static bool sized = false;
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&GemmKernel<WN>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              L::kBytes);
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&GemmKernel<WN>), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
   hipLaunchKernelGGL((GemmKernel<WN>), dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), L::kBytes,
                      stream, a);
   return LaunchStatus("mxfp8.gemm");
@@ -457,6 +453,7 @@ using namespace llmp_hip;
 
 extern "C" int llmp_hip_mxfp8_quantize(const void* x, int x_type, int64_t x_stride, int64_t k, int64_t rows, void* codes,
                                        void* scales, void* stream) {
+  BeginLaunches();
   if (x == nullptr || codes == nullptr || scales == nullptr) return Refuse(1, "mxfp8.quantize: null operand");
   if (k <= 0 || k % 128 != 0) return Refuse(1, "mxfp8.quantize: k %lld is not whole 128-value scale groups", (long long)k);
   if (rows <= 0 || rows > (1 << 24)) return Refuse(1, "mxfp8.quantize: 1 to 2^24 rows");
@@ -479,6 +476,7 @@ extern "C" int llmp_hip_mxfp8_quantize(const void* x, int x_type, int64_t x_stri
 }
 
 extern "C" int llmp_hip_mxfp8_swizzle(const void* scales, int64_t n, int64_t k, void* out, void* stream) {
+  BeginLaunches();
   if (scales == nullptr || out == nullptr) return Refuse(1, "mxfp8.swizzle: null operand");
   if (n <= 0 || k <= 0 || k % 128 != 0) return Refuse(1, "mxfp8.swizzle: k is not whole 128-value scale groups");
   const int64_t padded = (n + 127) / 128 * 128;
@@ -491,6 +489,7 @@ extern "C" int llmp_hip_mxfp8_swizzle(const void* scales, int64_t n, int64_t k, 
 
 extern "C" int llmp_hip_mxfp8_gemv(const void* codes, const void* scales, int64_t n, int64_t k, const float* x,
                                    int tokens, float* y, void* stream) {
+  BeginLaunches();
   if (codes == nullptr || scales == nullptr || x == nullptr || y == nullptr) return Refuse(1, "mxfp8.mul_mat_vec: null operand");
   if (k <= 0 || k % 32 != 0 || n <= 0) return Refuse(1, "mxfp8.mul_mat_vec: k is not whole 32-value blocks");
   if (tokens < 1 || tokens > 16) return Refuse(1, "mxfp8.mul_mat_vec: 1 to 16 tokens, not %d", tokens);
@@ -521,6 +520,7 @@ extern "C" size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int c
 }
 
 extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream) {
+  BeginLaunches();
   if (gemm == nullptr) return Refuse(1, "mxfp8.gemm: null descriptor");
   if (gemm->a == nullptr || gemm->a_scales == nullptr || gemm->b == nullptr || gemm->b_scales == nullptr ||
       gemm->d == nullptr)
@@ -544,7 +544,7 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
   a.m = gemm->m;
   a.n = gemm->n;
   a.k = gemm->k;
-  a.bf16 = gemm->bf16;
+  a.bf16 = gemm->bf16 != 0 ? 1 : 0;
   a.tiles_m = (gemm->m + kTileM - 1) / kTileM;
   a.tiles_n = 0;
   // The weight rows a workgroup takes (192 or 128): whichever leaves the fewest idle

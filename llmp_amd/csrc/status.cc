@@ -8,6 +8,8 @@
 namespace llmp_hip {
 namespace {
 thread_local char g_error[512] = "";
+// A failure met while preparing a launch (the kernel's LDS allowance), reported by the next LaunchStatus.
+thread_local int g_pending = 0;
 }
 
 void SetError(const char* format, ...) {
@@ -25,7 +27,30 @@ int Refuse(int code, const char* format, ...) {
   return code;
 }
 
+void BeginLaunches() {
+  g_pending = 0;
+  (void)hipGetLastError();  // an error an earlier, unrelated call left on this thread is not this call's
+}
+
+bool AllowLds(const void* kernel, int bytes, bool* sized) {
+  if (*sized) return true;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    SetError("allowing a kernel %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+    g_pending = -static_cast<int>(e);
+    return false;  // asked again by the next call: the flag stays clear
+  }
+  *sized = true;
+  return true;
+}
+
 int LaunchStatus(const char* what) {
+  if (g_pending != 0) {
+    const int code = g_pending;
+    g_pending = 0;
+    return code;
+  }
   const hipError_t e = hipGetLastError();
   if (e == hipSuccess) return 0;
   SetError("%s: %s", what, hipGetErrorString(e));

@@ -699,6 +699,7 @@ using namespace llmp_hip;
 
 extern "C" int llmp_hip_q8_1_quantize(const float* x, void* out, int64_t k, int64_t padded_k, int64_t row_stride,
                                       int64_t rows, int64_t planes, int64_t plane_stride, void* stream) {
+  BeginLaunches();
   if (x == nullptr || out == nullptr) return Refuse(1, "q8_1: null operand");
   if (k <= 0 || rows <= 0 || planes <= 0) return Refuse(1, "q8_1: empty input");
   if (padded_k < k || padded_k % 32 != 0) return Refuse(1, "q8_1: padded k %lld below k or not whole blocks", (long long)padded_k);
@@ -713,34 +714,40 @@ extern "C" int llmp_hip_q8_1_quantize(const float* x, void* out, int64_t k, int6
 }
 
 extern "C" int llmp_hip_vecq(int type, const llmp_vecq_desc* d, int variant, void* stream) {
+  BeginLaunches();
   return Launch(type, d, nullptr, variant, nullptr, stream);
 }
 
 extern "C" int llmp_hip_vecq_fused(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int variant,
                                    void* stream) {
+  BeginLaunches();
   if (x == nullptr) return Refuse(1, "vecq: null source");
   return Launch(type, d, x, variant, nullptr, stream);
 }
 
 extern "C" int llmp_hip_vecq_block_sums(int type, const llmp_vecq_desc* d, int variant, int32_t* sums, void* stream) {
+  BeginLaunches();
   if (sums == nullptr) return Refuse(1, "vecq: null sums");
-  if (variant < 0 && d != nullptr) variant = FlatTakes(type, *d, true) ? kFlatFirst : 0;
+  if (const int bad = CheckDesc(type, d); bad != 0) return bad;  // before any plan divides by the row's units
+  if (variant < 0) variant = FlatTakes(type, *d, true) ? kFlatFirst : 0;
   if (variant != 0 && variant != kFlatFirst) return Refuse(1, "vecq: block sums are of the one-token variants");
   return Launch(type, d, nullptr, variant, sums, stream);
 }
 
 extern "C" int llmp_hip_vecq_sorted(int type, const llmp_vecq_desc* d, const int32_t* offsets, int experts, int variant,
                                     void* stream) {
+  BeginLaunches();
   if (offsets == nullptr || d == nullptr) return Refuse(1, "vecq: null offsets");
   if (experts < 1 || experts > 65535) return Refuse(1, "vecq: 1 to 65535 experts");
-  if (!FlatTakes(type, *d) && !MmaTakes(type, *d))
-    return Refuse(1, "vecq: sorted rows take weights the flat or the matrix-core form takes");
   llmp_vecq_desc sorted = *d;
   sorted.ids = nullptr;
   sorted.used = experts;  // a workgroup row an expert
   sorted.tokens = 1;      // the row counts come from the offsets
   sorted.y_slot = 0;
   sorted.dst_slot = 0;
+  if (const int bad = CheckDesc(type, &sorted, true); bad != 0) return bad;  // before any plan divides by the row's units
+  if (!FlatTakes(type, sorted) && !MmaTakes(type, sorted))
+    return Refuse(1, "vecq: sorted rows take weights the flat or the matrix-core form takes");
   // An expert's rows are many tokens of one matrix: the matrix cores where they apply.
   if (variant < 0) variant = MmaTakes(type, *d) ? kMmaVariant : kFlatFirst + 1;
   return Launch(type, &sorted, nullptr, variant, nullptr, stream, offsets);

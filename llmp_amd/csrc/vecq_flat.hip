@@ -1666,12 +1666,7 @@ int g_compute_units = 0;
 template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kDeep ? kDeepLdsLimit : kFlatLdsLimit));
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), static_cast<int>(kDeep ? kDeepLdsLimit : kFlatLdsLimit), &sized)) return;
   hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(plan.waves * kWave), plan.lds, stream, a,
                      plan.rows);
 }
@@ -1747,11 +1742,7 @@ SplitPlan PlanSplit(int units) {
 template <class F, int XT>
 void LaunchS(const VecQArgs& a, dim3 grid, const SplitPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!sized) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQFlatSplit<F, XT>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kFlatLdsLimit));
-    sized = true;
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlatSplit<F, XT>), static_cast<int>(kFlatLdsLimit), &sized)) return;
   hipLaunchKernelGGL((VecQFlatSplit<F, XT>), grid, dim3(plan.waves * kWave), plan.lds, stream, a, plan.split,
                      plan.piece);
 }
@@ -1813,6 +1804,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
 // tiles are fetched in 16-byte chunks. The legacy 4/5-bit blocks likewise, in whole 256 values. Without a GLU, and unless `whole_rows` asks for a row
 // in one tile (the block sums), longer rows in pieces, as long as their records fit.
 bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
+  if (d.ncols_x < 256) return false;  // every format's unit is 256 values: no plan is made for a row without one
   const bool glu = d.g != nullptr;
   const int most = glu ? kWave / 2 : kWave;
   const bool pieces = !glu && !whole_rows;

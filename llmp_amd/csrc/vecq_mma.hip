@@ -701,18 +701,10 @@ template <bool kQ8, bool kGlu>
 void LaunchMmaKernel(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if constexpr (kQ8) {
-    if (!sized) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMmaQ8<kGlu>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
-      sized = true;
-    }
+    if (!AllowLds(reinterpret_cast<const void*>(&VecQMmaQ8<kGlu>), static_cast<int>(kMmaLdsLimit), &sized)) return;
     hipLaunchKernelGGL((VecQMmaQ8<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
   } else {
-    if (!sized) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&VecQMma<kGlu>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMmaLdsLimit));
-      sized = true;
-    }
+    if (!AllowLds(reinterpret_cast<const void*>(&VecQMma<kGlu>), static_cast<int>(kMmaLdsLimit), &sized)) return;
     hipLaunchKernelGGL((VecQMma<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
   }
 }

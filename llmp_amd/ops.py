@@ -137,7 +137,7 @@ def set_rows_quant(t, x, ids, destination, row_bytes=None):
         row_bytes = destination.stride(0)
     index_bytes = 8 if ids.dtype == torch.int64 else 4
     _lib.check(lib.llmp_hip_set_rows_quant(t, _ptr(x), x.stride(0), _ptr(ids), index_bytes, _ptr(destination),
-                                           row_bytes, k, rows, _stream()))
+                                           row_bytes, k, rows, destination.shape[0], _stream()))
     return destination
 
 

@@ -11,7 +11,9 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstddef>
 #include <cstring>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -141,6 +143,94 @@ void HostChecks() {
   EXPECT(hipk::exl3::ScratchBytes(multi) == 0);
 }
 
+// The registry's entries (include/llmp_hip.hpp, namespace execution) against the names the reference's planner and
+// plans use and against what the entry points they list really take: a declared row limit is the entry point's own.
+void RegistryChecks() {
+  namespace ex = hipk::execution;
+  const std::vector<ex::Implementation> all = ex::Implementations();
+  std::set<std::string> names;
+  for (const ex::Implementation& i : all) {
+    EXPECT(names.insert(i.name).second);  // unique in a build (registry.h:323-325)
+    bool well_formed = !i.name.empty();
+    for (const char c : i.name) well_formed = well_formed && ((c >= 'a' && c <= 'z') || (c >= '0' && c <= '9') || c == '.' || c == '_');
+    EXPECT(well_formed);
+    EXPECT(!i.capability.op.empty() && !i.capability.launches.empty() && !i.variant.empty());
+    EXPECT(i.capability.min_arch == ex::kGfx950 && i.capability.max_arch == ex::kGfx950);
+    EXPECT(i.capability.shape.min_rows >= 1 && i.capability.shape.min_rows <= i.capability.shape.max_rows);
+    for (const std::string& launch : i.capability.launches) EXPECT(launch.rfind("llmp_hip_", 0) == 0);
+  }
+  // SURVEY's list of names to keep (plan_step.h:201-314, capabilities.cc:2486-2489 and 2881-2893,
+  // decode/implementations.h:7-13, exl3/implementations.h:8-31).
+  for (const char* name : {"llmp.q8_1", "llmp.vecq.dense", "llmp.vecq.glu", "llmp.vecq.experts", "llmp.vecq.experts_glu", "llmp.vecq.grouped",
+                           "ggml.mul_mat.mmvq", "ggml.mul_mat_glu.mmvq_fused", "llmp.mxfp8.mul_mat_vec", "llmp.mxfp8.quantize",
+                           "llmp.mxfp8.swizzle", "llmp.mxfp8.gemm.cutlass", "llmp.moe.router", "llmp.decode.vector.nvfp4.atoms",
+                           "llmp.decode.vector_glu.mxfp8.split", "llmp.decode.matrix.bf16.dense", "llmp.decode.grouped.affine.split",
+                           "llmp.decode.rows.q8_0.blocks", "exl3.linear.gemv", "exl3.linear.gemm", "exl3.multi_linear.mgemm"})
+    EXPECT(names.count(name) == 1);
+  int decode = 0;
+  for (const std::string& name : names) decode += name.rfind("llmp.decode.", 0) == 0;
+  EXPECT(decode == 5 * 12);  // every built template over every decoder; matrix_fma is refused and not declared
+
+  // Candidates: the config shapes find their implementations, and nothing outside a rule does.
+  ex::CapabilityQuery q;
+  q.op = "fused.mul_mat_glu", q.encoding = "q4_k", q.rows = 1, q.k = 3840, q.n = 15360, q.row_invariant = q.capturable = true;
+  std::vector<ex::Implementation> found = ex::Candidates(q);
+  EXPECT(found.size() == 2 && found[0].name == "llmp.vecq.glu" && found[1].name == "ggml.mul_mat_glu.mmvq_fused");
+  q.rows = 17;
+  EXPECT(ex::Candidates(q).empty());
+  q.rows = 1, q.k = 3840 + 32;
+  EXPECT(ex::Candidates(q).empty());
+  q = ex::CapabilityQuery{};
+  q.op = "mul_mat", q.encoding = "mxfp8", q.rows = 2048, q.k = 4096, q.n = 12288;
+  found = ex::Candidates(q);
+  bool gemm = false;
+  for (const ex::Implementation& i : found) gemm = gemm || i.name == "llmp.mxfp8.gemm.cutlass";
+  EXPECT(gemm);
+  q.features = ex::kBf16Mma;  // a device without block-scaled FP8 matrix instructions
+  for (const ex::Implementation& i : ex::Candidates(q)) EXPECT(i.name != "llmp.mxfp8.gemm.cutlass");
+  q = ex::CapabilityQuery{};
+  q.op = "quant_linear", q.encoding = "exl3", q.rows = 16, q.k = 4096, q.n = 14336;
+  found = ex::Candidates(q);
+  EXPECT(found.size() == 1 && found[0].name == "exl3.linear.gemm");
+  q.arch = 942;
+  EXPECT(ex::Candidates(q).empty());
+
+  // The declared row limits are the entry points' own: one row past a limit is refused by the C ABI.
+  const auto rule = [&](const char* name) {
+    for (const ex::Implementation& i : all)
+      if (i.name == name) return i.capability.shape;
+    ++g_failures;
+    return ex::ShapeRule{};
+  };
+  alignas(16) static std::uint8_t fake[4096];
+  VecQDesc d;
+  d.w = fake, d.y = fake, d.dst = reinterpret_cast<float*>(fake), d.ncols_x = 256, d.nrows = 1, d.stride_row = 1, d.y_token = 16;
+  d.tokens = static_cast<int>(rule("llmp.vecq.dense").max_rows) + 1, d.dst_token = 1;
+  EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, -1, nullptr));
+  EXPECT(hipk::LastError().find("tokens") != std::string::npos);
+  const std::int32_t ids[1] = {0};
+  d.ids = ids, d.tokens = 1, d.used = static_cast<int>(rule("llmp.vecq.experts").max_rows) + 1;
+  EXPECT(!hipk::ggml::LaunchVecQ(hipk::ggml::kQ4_K, d, -1, nullptr));
+  EXPECT(hipk::LastError().find("pairs") != std::string::npos || hipk::LastError().find("slots") != std::string::npos);
+  hipk::exl3::LinearOperands linear;
+  const std::uint64_t at = reinterpret_cast<std::uint64_t>(fake);
+  linear.weights.trellis = at, linear.weights.suh = at, linear.weights.svh = at;
+  linear.weights.k = 128, linear.weights.n = 128, linear.weights.bits = 4;
+  linear.x = at, linear.a_had = at, linear.y = at;
+  linear.m = static_cast<int>(rule("exl3.linear.gemm").max_rows) + 1;
+  EXPECT(hipk::exl3::PackedLinear(linear, fake, sizeof(fake), nullptr) == hipk::KernelFailure::kRejected);
+  EXPECT(hipk::LastError().find("rows") != std::string::npos);
+  EXPECT(rule("llmp.mxfp8.gemm.cutlass").k_multiple == 128);
+  hipk::ggml::mxfp8::Gemm g;
+  g.m = 128, g.n = 128, g.k = 128 + 32, g.a = g.a_scales = g.b = g.b_scales = fake, g.d = fake;
+  EXPECT(hipk::ggml::mxfp8::Run(g, 256, nullptr) > 0);
+  // The descriptor's layout is the reference's (mxfp8_cutlass.h:59-71): `bool bf16` over the C struct's one byte.
+  static_assert(sizeof(hipk::ggml::mxfp8::Gemm) == sizeof(llmp_mxfp8_gemm), "Gemm's size");
+  static_assert(offsetof(hipk::ggml::mxfp8::Gemm, bf16) == offsetof(llmp_mxfp8_gemm, bf16), "bf16's place");
+  static_assert(offsetof(hipk::ggml::mxfp8::Gemm, scratch) == offsetof(llmp_mxfp8_gemm, scratch), "scratch's place");
+  static_assert(sizeof(bool) == sizeof(static_cast<llmp_mxfp8_gemm*>(nullptr)->bf16), "one byte");
+}
+
 // One dense product on the GPU against the oracle over the same Q8_1 bytes.
 void DenseProduct(int type, int n, int k, int tokens, bool glu) {
   const int elements = orc_block_elements(type);
@@ -193,6 +283,7 @@ void DenseProduct(int type, int n, int k, int tokens, bool glu) {
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "host";
   HostChecks();
+  RegistryChecks();
   if (mode == "device") {
     DenseProduct(hipk::ggml::kQ8_0, 96, 4096, 1, false);
     DenseProduct(hipk::ggml::kQ4_K, 100, 3840, 1, true);

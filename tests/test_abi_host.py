@@ -124,6 +124,76 @@ def test_exl3_linears_refuse_bad_operands():
     assert lib.llmp_hip_exl3_multi_linear_scratch(C.byref(two)) == 2 * lib.llmp_hip_exl3_linear_scratch(C.byref(one)) // 17 * 2
 
 
+def test_default_descriptors_are_refused_before_any_plan():
+    """A default-constructed descriptor (k = 0) through the block sums and the sorted rows: refused by the
+    descriptor's checks, for every type, before a plan divides by the row's units."""
+    lib = _lib.load()
+    empty = _lib.VecQDesc()
+    for t in (2, 3, 6, 7, 8, 12, 13, 14, 20, 39):
+        assert lib.llmp_hip_vecq_block_sums(t, C.byref(empty), -1, 0x1000, None) > 0
+        assert lib.llmp_hip_vecq_sorted(t, C.byref(empty), 0x1000, 4, -1, None) > 0
+        nearly = desc(ncols_x=0)
+        assert lib.llmp_hip_vecq_block_sums(t, C.byref(nearly), -1, 0x1000, None) > 0
+        assert lib.llmp_hip_vecq_sorted(t, C.byref(nearly), 0x1000, 4, -1, None) > 0
+        assert b"whole" in lib.llmp_hip_last_error()
+
+
+def test_exl3_refuses_overlapping_operands():
+    """src/kernels/exl3/validate.cc:32-62 and 120-126 of the reference: a written range that meets another
+    operand is refused before anything is queued."""
+    lib = _lib.load()
+
+    def weights(trellis=0x100000, suh=0x200000, svh=0x210000):
+        w = _lib.Exl3Weights()
+        w.trellis, w.suh, w.svh, w.k, w.n, w.bits, w.codebook = trellis, suh, svh, 128, 128, 4, 0
+        return w
+
+    def linear(**kw):
+        op = _lib.Exl3Linear()
+        base = dict(x=0x300000, a_had=0x310000, y=0x320000, f32=1, m=2)
+        base.update(kw)
+        op.weights = weights()
+        for k, v in base.items():
+            setattr(op, k, v)
+        return op
+
+    scratch = 0x400000
+    cases = [(dict(y=0x300000), b"y overlaps x"), (dict(a_had=0x300000), b"a_had overlaps x"),
+             (dict(a_had=0x320000), b"a_had overlaps y"), (dict(y=0x100000 + 64), b"y overlaps the trellis"),
+             (dict(y=0x200000), b"y overlaps suh"), (dict(a_had=0x210000), b"a_had overlaps svh"),
+             (dict(y=scratch + 8), b"y overlaps the scratch"), (dict(x=scratch), b"the scratch overlaps x")]
+    for kw, why in cases:
+        op = linear(**kw)
+        assert lib.llmp_hip_exl3_linear(C.byref(op), scratch, 1 << 20, None) > 0, kw
+        assert why in lib.llmp_hip_last_error(), (kw, lib.llmp_hip_last_error())
+    two = _lib.Exl3MultiLinear()
+    two.first, two.second = weights(), weights(trellis=0x500000)
+    two.x, two.a_had, two.y, two.f32, two.m = 0x300000, 0x310000, 0x310000 + 2 * 2 * 128 * 2 - 8, 1, 2
+    assert lib.llmp_hip_exl3_multi_linear(C.byref(two), scratch, 1 << 20, None) > 0
+    assert b"a_had overlaps y" in lib.llmp_hip_last_error()
+    two.y = 0x500000 + 32
+    assert lib.llmp_hip_exl3_multi_linear(C.byref(two), scratch, 1 << 20, None) > 0
+    assert b"y overlaps the trellis" in lib.llmp_hip_last_error()
+    w = weights()
+    assert lib.llmp_hip_exl3_reconstruct(C.byref(w), 0x100000 + 4096, 0, 16, None) > 0
+    assert b"w overlaps the trellis" in lib.llmp_hip_last_error()
+    # The transform: in place for F16 only; otherwise x, y and the scale apart.
+    assert lib.llmp_hip_exl3_hadamard(0x1000, 0x1000, 0x8000, 2, 128, 1, 0, None) > 0
+    assert lib.llmp_hip_exl3_hadamard(0x1000, 0x1100, 0x8000, 2, 128, 0, 0, None) > 0 and b"y overlaps x" in lib.llmp_hip_last_error()
+    assert lib.llmp_hip_exl3_hadamard(0x1000, 0x8000 + 64, 0x8000, 2, 128, 0, 0, None) > 0
+    assert b"y overlaps the scale" in lib.llmp_hip_last_error()
+
+
+def test_set_rows_quant_refuses_a_destination_over_its_operands():
+    lib = _lib.load()
+    store = lambda **kw: lib.llmp_hip_set_rows_quant(kw.get("t", 8), kw.get("x", 0x10000), 64, kw.get("ids", 0x20000), 4,
+                                                     kw.get("dst", 0x30000), 68, 64, 4, kw.get("cells", 16), None)
+    assert store(cells=0) > 0 and b"no cells" in lib.llmp_hip_last_error()
+    assert store(dst=0x10000 + 512) > 0 and b"overlaps" in lib.llmp_hip_last_error()
+    assert store(dst=0x20000 - 68 * 16 + 2) > 0 and b"overlaps" in lib.llmp_hip_last_error()
+    assert store(t=12) > 0 and b"Q8_0 or Q4_0" in lib.llmp_hip_last_error()
+
+
 def test_decode_vector_refuses_bad_operands():
     lib = _lib.load()
 
