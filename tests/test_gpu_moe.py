@@ -107,10 +107,11 @@ def test_gathering_quantizer_is_the_quantizer(device):
     assert np.array_equal(got, oracle.q8_1_quantize(x[rows]))
 
 
-@pytest.mark.parametrize("tokens", [1, 16, 40])
+@pytest.mark.parametrize("tokens", [1, 16, 40, 512])
 def test_routed_ffn_layer_matches_oracle_stage_by_stage(device, tokens):
-    """Qwen3-30B-A3B-like: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K. 40 tokens
-    take the sorted path (320 pairs), 1 and 16 the routed mat-vec. Every stage is compared with
+    """Qwen3-30B-A3B-like: 128 experts, top-8, hidden 2048, expert FFN 768, Q4_K. 40 and 512 tokens
+    take the sorted path (320 and 4096 pairs: about 2.5 and 32 rows an expert, the latter two and more
+    passes of the matrix-core form), 1 and 16 the routed mat-vec. Every stage is compared with
     the oracle over identical input bytes (the second product over the device's own quantized
     h: a float rounding of h can move one of its Q8_1 codes by a step, which is a different
     input, not an error of the product). exec.cc:966-1002,1819-1856 of the reference."""
