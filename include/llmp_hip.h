@@ -308,6 +308,18 @@ typedef struct llmp_exl3_linear {
 size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op);
 int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream);
 
+/* The same linear for callers that cannot allocate or bring a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose callers always
+ * declare and charge their workspace (src/kernels/ggml/launch.h:4-8). The partial sums go to an array of
+ * LLMP_EXL3_STATIC_SCRATCH_BYTES that the library holds on every device it runs on until the process ends; the
+ * call allocates and frees nothing. A linear whose llmp_hip_exl3_linear_scratch exceeds that is refused (status
+ * 1): pass scratch of your own to llmp_hip_exl3_linear. x, a_had and y are the caller's as before. Every call on
+ * a device shares that device's array: calls that overlap in time on one device (two streams) race; calls on one
+ * stream, or ordered by events, are safe. Nothing in the array needs clearing: every launch overwrites the part
+ * it later reads. Output bits are those of llmp_hip_exl3_linear. */
+#define LLMP_EXL3_STATIC_SCRATCH_BYTES ((size_t)4 << 20) /* config 5 at 16 rows needs 3,670,016 */
+int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* stream);
+
 /* exl3.multi_linear.mgemm: MultiLinear of src/kernels/exl3/linear.h:51-53 over the operands of
  * src/kernels/exl3/validate.h:160-172, a gate and an up linear of the same k, n and rate over
  * one input (tests/unit/exl3_trellis_test.cc:664-716). x (m x k F16) into y (2 x m x n: the

@@ -27,11 +27,17 @@
 #include <hip/hip_runtime.h>
 
 #include <initializer_list>
+#include <mutex>
 
 #include <type_traits>
 
 #include "common.h"
 #include "llmp_hip.h"
+
+// The partial sums of llmp_hip_exl3_linear_static: one array a device, held until the process ends. In host code
+// this name is only a handle for hipGetSymbolAddress; kernels and copies take the address that call returns.
+constexpr size_t kStaticScratchBytes = LLMP_EXL3_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace llmp_hip {
 namespace {
@@ -598,16 +604,21 @@ extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
   return static_cast<size_t>(SlicesFor(op->weights.n, op->weights.k)) * op->m * op->weights.n * sizeof(float);
 }
 
-extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream) {
-  BeginLaunches();
+namespace llmp_hip {
+namespace {
+
+// The checks and launches of the packed linear over `area` (area_bytes of partial sums: the caller's, or this
+// device's static array).
+int LinearOver(const llmp_exl3_linear* op, void* area, size_t area_bytes, hipStream_t stream) {
   if (op == nullptr) return Refuse(1, "exl3.linear: null operands");
   if (const int bad = CheckWeights(op->weights); bad != 0) return bad;
-  if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || scratch == nullptr)
+  if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || area == nullptr)
     return Refuse(1, "exl3.linear: null operand");
   if (op->m < 1 || op->m > 16) return Refuse(1, "exl3.linear: the packed product takes 1 to 16 rows, not %d", op->m);
-  if (scratch_bytes < llmp_hip_exl3_linear_scratch(op)) return Refuse(1, "exl3.linear: scratch too small");
+  if (area_bytes < llmp_hip_exl3_linear_scratch(op))
+    return Refuse(1, "exl3.linear: scratch too small: %zu bytes of partial sums, %zu given", llmp_hip_exl3_linear_scratch(op), area_bytes);
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
-       reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
+       reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(area)) % 8 != 0)
     return Refuse(1, "exl3.linear: operands not 8-byte aligned");
   {
     // validate.cc:120-126: what the launches write (a_had, y, the partial sums in place of the lock area) meets
@@ -616,17 +627,66 @@ extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, s
     const Range x{"x", reinterpret_cast<uintptr_t>(op->x), m * op->weights.k * 2};
     const Range a_had{"a_had", reinterpret_cast<uintptr_t>(op->a_had), m * op->weights.k * 2};
     const Range y{"y", reinterpret_cast<uintptr_t>(op->y), m * op->weights.n * (op->f32 ? 4 : 2)};
-    const Range area{"the scratch", reinterpret_cast<uintptr_t>(scratch), llmp_hip_exl3_linear_scratch(op)};
+    const Range partials{"the scratch", reinterpret_cast<uintptr_t>(area), llmp_hip_exl3_linear_scratch(op)};
     const llmp_exl3_weights& w = op->weights;
-    if (const int bad = Disjoint("exl3.linear", a_had, {x, y, TrellisRange(w), SuhRange(w), SvhRange(w), area}); bad != 0) return bad;
-    if (const int bad = Disjoint("exl3.linear", y, {x, TrellisRange(w), SuhRange(w), SvhRange(w), area}); bad != 0) return bad;
-    if (const int bad = Disjoint("exl3.linear", area, {x, TrellisRange(w), SuhRange(w), SvhRange(w)}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.linear", a_had, {x, y, TrellisRange(w), SuhRange(w), SvhRange(w), partials}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.linear", y, {x, TrellisRange(w), SuhRange(w), SvhRange(w), partials}); bad != 0) return bad;
+    if (const int bad = Disjoint("exl3.linear", partials, {x, TrellisRange(w), SuhRange(w), SvhRange(w)}); bad != 0) return bad;
   }
   const llmp_exl3_weights* const w[2] = {&op->weights, &op->weights};
   void* const a_had[2] = {op->a_had, op->a_had};
   void* const y[2] = {op->y, op->y};
-  float* const partial[2] = {static_cast<float*>(scratch), static_cast<float*>(scratch)};
-  return LaunchLinears(w, 1, op->x, a_had, y, partial, op->f32 != 0, op->m, "exl3.linear", static_cast<hipStream_t>(stream));
+  float* const partial[2] = {static_cast<float*>(area), static_cast<float*>(area)};
+  return LaunchLinears(w, 1, op->x, a_had, y, partial, op->f32 != 0, op->m, "exl3.linear", stream);
+}
+
+// This device's copy of the static array: its address is asked for once a device, with that device current.
+constexpr int kMostDevices = 64;
+std::mutex g_static_lock;
+void* g_static_area[kMostDevices] = {};
+
+int StaticArea(void** area) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) {
+    SetError("exl3.linear_static: %s", hipGetErrorString(e));
+    return -static_cast<int>(e);
+  }
+  if (device < 0 || device >= kMostDevices) return Refuse(1, "exl3.linear_static: device %d beyond the %d this library keeps an area for", device, kMostDevices);
+  std::lock_guard<std::mutex> hold(g_static_lock);
+  if (g_static_area[device] == nullptr) {
+    void* at = nullptr;
+    e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || at == nullptr) {
+      (void)hipGetLastError();
+      SetError("exl3.linear_static: the static area's address: %s", hipGetErrorString(e));
+      return e != hipSuccess ? -static_cast<int>(e) : -1;
+    }
+    g_static_area[device] = at;
+  }
+  *area = g_static_area[device];
+  return 0;
+}
+
+}  // namespace
+}  // namespace llmp_hip
+
+extern "C" int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scratch_bytes, void* stream) {
+  BeginLaunches();
+  return LinearOver(op, scratch, scratch_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* stream) {
+  BeginLaunches();
+  if (op == nullptr) return Refuse(1, "exl3.linear_static: null operands");
+  // The size first: a linear whose partial sums do not fit the static area is refused whatever else holds.
+  const size_t needs = llmp_hip_exl3_linear_scratch(op);
+  if (needs > kStaticScratchBytes)
+    return Refuse(1, "exl3.linear_static: %zu bytes of partial sums exceed the static area's %zu; use llmp_hip_exl3_linear with "
+                     "scratch of the caller's", needs, kStaticScratchBytes);
+  void* area = nullptr;
+  if (const int bad = StaticArea(&area); bad != 0) return bad;
+  return LinearOver(op, area, kStaticScratchBytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op) {

@@ -367,6 +367,19 @@ def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, f32=True, keep=None)
     return y
 
 
+def exl3_linear_static(trellis, suh, svh, k, n, bits, codebook, x, a_had, y):
+    """The same linear through llmp_hip_exl3_linear_static: the partial sums go to the library's static array
+    on this device, the call allocates nothing. x float16 [m, k]; a_had float16 [m, k] and y float32 or
+    float16 [m, n] are the caller's, filled in place."""
+    lib = _lib.load()
+    m = x.shape[0]
+    op = Exl3Linear()
+    op.weights = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
+    op.x, op.a_had, op.y, op.f32, op.m = x.data_ptr(), a_had.data_ptr(), y.data_ptr(), int(y.dtype == torch.float32), m
+    _lib.check(lib.llmp_hip_exl3_linear_static(C.byref(op), _stream()))
+    return y
+
+
 def exl3_multi_linear(first, second, x, f32=True, keep=None):
     """exl3.multi_linear: x float16 [m, k] (m <= 16) through a gate and an up linear of the same k, n and
     rate: [2, m, n]. `first` and `second` are (trellis, suh, svh, k, n, bits, codebook); `keep`, a dict,
