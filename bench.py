@@ -5,7 +5,9 @@ quantization to Q8_1) followed by llmp.vecq, the fused Q4_K gate/up GEGLU mat-ve
 3840, two 15360-row matrices), over one of several distinct weight copies, rotated so that
 neither L2 nor the 256 MB Infinity Cache holds them. --fused makes it the single launch that
 quantizes the bf16 activation inside the kernel.
-Prints one JSON line; see --help."""
+Prints one JSON line; see --help. `other_configs` holds the other four benchmark configurations (Q8_0 mat-vec,
+MXFP8 GEMM, the routed-expert layer at 1, 16 and 512 tokens, the EXL3 linear at 1 and 16 rows), each with the
+roofline of its dominant kernel and the CPU oracle timed beside it; `--only <key>` runs one of them alone."""
 import argparse
 import json
 import os
@@ -87,137 +89,274 @@ def graph_us(body, count, warm=3):
     return begin.elapsed_time(end) / count * 1e3
 
 
-def other_configs(device, args):
-    """Short measurements of the other benchmark configurations (not the headline line): each
-    over distinct weight copies where the weights are what is streamed."""
+MFMA_FP8_PEAK_TFLOPS = 5033.0  # dense FP8, 256 CUs x 2.4 GHz x 8192 flop/clk/CU
+
+# HBM bytes per launch of each configuration's dominant kernel from rocprofv3 --pmc runs of this file
+# (`--only <name> --eager`: FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by 1.9988 and 1.0, what the
+# same counters read for --calibrate-copy's copy of known size). Counters cannot be read from inside a run:
+# a configuration that has not been profiled reports null.
+PROFILED_TRAFFIC = {
+    "q4_k_gate_up_geglu_b1": int(round((32478.4 * 1.9988 + 60.1) * 1024)),
+}
+
+
+def cpu_leg(run, units_per_pass, unit, budget_s, sample, threads, scale=1.0):
+    """The oracle timed on the host cores: `run()` repeated for about budget_s seconds."""
+    run()
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        run()
+        passes += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed >= budget_s:
+            break
+    return {"value": round(units_per_pass * passes / elapsed * scale, 4), "unit": unit, "cores": threads, "kind": "port",
+            "sample": f"{passes} passes of {sample}, {elapsed:.1f} s"}
+
+
+def hbm_roofline(name, kernel, bytes_, us):
+    achieved = bytes_ / us / 1e3
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": PROFILED_TRAFFIC.get(name), "kernel": kernel,
+            "algorithmic_bytes_per_launch": int(bytes_), "avg_launch_us": round(us, 3)}
+
+
+def other_configs(device, args, only=None):
+    """The other benchmark configurations (not the headline line), each with the roofline of its dominant
+    kernel and the oracle timed on the host cores over a bounded sample of the same workload. Weights are
+    what is streamed: every launch reads a copy that neither L2 nor the 256 MB Infinity Cache holds."""
     import numpy as np
     import torch
 
+    import oracle
     from llmp_amd import ops, synth
 
     out = {}
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    want = lambda name: only is None or only == name
+    threads = oracle.max_threads()
+    cpu = not args.no_cpu
+    timed = (lambda body, count: event_us(body, count)) if args.eager else graph_us
 
     # Config 1: Q8_0 mat-vec 4096 x 4096, one F32 token through llmp.q8_1.
-    n = k = 4096
-    w = dev(synth.q8_0_weights(n, k, 201))
-    copies = [w] + [w.clone() for _ in range(-(-ROTATE_BYTES // w.numel()) - 1)]
-    x = dev(synth.activations(1, k, 202))
-    q8 = ops.quantize_q8_1(x)
-    y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
-    us = graph_us(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 4 * len(copies))
-    bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
-    out["q8_0_matvec_4096x4096_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
-                                       "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
-    del copies, w
+    if want("q8_0_matvec_4096x4096_b1"):
+        n = k = 4096
+        w_host = synth.q8_0_weights(n, k, 201)
+        w = dev(w_host)
+        copies = [w] + [w.clone() for _ in range(-(-ROTATE_BYTES // w.numel()) - 1)]
+        x_host = synth.activations(1, k, 202)
+        x = dev(x_host)
+        q8 = ops.quantize_q8_1(x)
+        y = torch.empty((1, 1, n), dtype=torch.float32, device=device)
+
+        def step(i):
+            ops.quantize_q8_1(x, out=q8)
+            ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y)
+
+        step_us = timed(step, 4 * len(copies))
+        us = timed(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 4 * len(copies))
+        bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
+        entry = {"workload": "GGML Q8_0 mat-vec, N=4096, K=4096, batch 1, fp32 activations through llmp.q8_1",
+                 "step_us": round(step_us, 2), "weight_GB/s_of_the_step": round(w.numel() / step_us / 1e3, 1),
+                 "roofline": hbm_roofline("q8_0_matvec_4096x4096_b1", "VecQFlat<FormatQ8> (llmp.vecq, Q8_0)", bytes_, us)}
+        if cpu:
+            q8_host = oracle.q8_1_quantize(x_host)
+            entry["cpu_baseline"] = cpu_leg(lambda: oracle.vecq(oracle.TYPE_Q8_0, w_host, q8_host, k, n, threads=threads),
+                                            w.numel() / 1e9, "GB/s", 3.0, "the whole 4096 x 4096 mat-vec (q8_1 once)", threads)
+        out["q8_0_matvec_4096x4096_b1"] = entry
+        del copies, w
 
     # Config 2 at batch 4 and 8.
-    gate, up = dev(synth.q4_k_weights(N, K, 101)), dev(synth.q4_k_weights(N, K, 102))
-    count = -(-ROTATE_BYTES // WEIGHT_BYTES)
-    gates = [gate] + [gate.clone() for _ in range(count - 1)]
-    ups = [up] + [up.clone() for _ in range(count - 1)]
-    for tokens in (4, 8):
-        q8 = ops.quantize_q8_1(dev(synth.activations(tokens, K, 203)))
-        y = torch.empty((tokens, 1, N), dtype=torch.float32, device=device)
-        us = graph_us(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
-                                         glu=ops.GLU_GEGLU, out=y), 4 * count)
-        out[f"q4_k_gate_up_geglu_b{tokens}"] = {"us": round(us, 2),
-                                                "GB/s": round(algorithmic_bytes(tokens) / us / 1e3, 1)}
-    del gates, ups, gate, up
-    torch.cuda.empty_cache()
+    if want("q4_k_gate_up_geglu_b4") or want("q4_k_gate_up_geglu_b8"):
+        gate_host, up_host = synth.q4_k_weights(N, K, 101), synth.q4_k_weights(N, K, 102)
+        gate, up = dev(gate_host), dev(up_host)
+        count = -(-ROTATE_BYTES // WEIGHT_BYTES)
+        gates = [gate] + [gate.clone() for _ in range(count - 1)]
+        ups = [up] + [up.clone() for _ in range(count - 1)]
+        for tokens in (4, 8):
+            name = f"q4_k_gate_up_geglu_b{tokens}"
+            if not want(name):
+                continue
+            x_host = synth.bf16_to_f32(synth.bf16_bits(synth.activations(tokens, K, 203)))
+            q8 = ops.quantize_q8_1(dev(x_host))
+            y = torch.empty((tokens, 1, N), dtype=torch.float32, device=device)
+            us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
+                                          glu=ops.GLU_GEGLU, out=y), 4 * count)
+            entry = {"workload": f"config 2 at batch {tokens}",
+                     "roofline": hbm_roofline(name, "VecQMma<glu> (llmp.vecq, Q4_K, matrix cores)" if tokens > 4 else
+                                              "VecQFlat<FormatQ4K, 4 tokens a pass, glu>", algorithmic_bytes(tokens), us)}
+            if cpu:
+                q8_host = oracle.q8_1_quantize(x_host)
+                entry["cpu_baseline"] = cpu_leg(
+                    lambda: oracle.vecq(oracle.TYPE_Q4_K, up_host, q8_host, K, N, gate=gate_host, tokens=tokens,
+                                        glu=oracle.GLU_GEGLU, threads=threads),
+                    WEIGHT_BYTES / 1e9, "GB/s", 2.0, f"the whole gate/up pair at {tokens} tokens", threads)
+            out[name] = entry
+        del gates, ups, gate, up
+        torch.cuda.empty_cache()
 
     # The same layer's down projection (15360 -> 3840, Q4_K, one token): rows of 60 super-blocks.
-    kd, nd = N, K
-    wdn = dev(synth.q4_k_weights(nd, kd, 104))
-    downs = [wdn] + [wdn.clone() for _ in range(-(-ROTATE_BYTES // wdn.numel()) - 1)]
-    q8 = ops.quantize_q8_1(dev(synth.activations(1, kd, 105)))
-    y = torch.empty((1, 1, nd), dtype=torch.float32, device=device)
-    us = graph_us(lambda i: ops.vecq(ops.TYPE_Q4_K, downs[i % len(downs)], q8, kd, nd, out=y), 4 * len(downs))
-    bytes_ = wdn.numel() + kd * 4 + nd * 4
-    out["q4_k_down_15360x3840_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
-                                      "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
-    del downs, wdn
-    torch.cuda.empty_cache()
-
-    # An MXFP4 gate/up pair (4096 -> 2 x 14336, SwiGLU, one token): the same streaming form, 17-byte blocks.
-    km, nm = 4096, 14336
-    gate = dev(synth.mxfp4_weights(nm, km, 106))
-    count = -(-ROTATE_BYTES // (2 * gate.numel()))
-    gates = [gate] + [gate.clone() for _ in range(count - 1)]
-    ups = [gate.clone() for _ in range(count)]
-    q8 = ops.quantize_q8_1(dev(synth.activations(1, km, 107)))
-    y = torch.empty((1, 1, nm), dtype=torch.float32, device=device)
-    us = graph_us(lambda i: ops.vecq(ops.TYPE_MXFP4, ups[i % count], q8, km, nm, gate=gates[i % count],
-                                     glu=ops.GLU_SWIGLU, out=y), 4 * count)
-    bytes_ = 2 * gate.numel() + km * 4 + nm * 4
-    out["mxfp4_gate_up_swiglu_4096x2x14336_b1"] = {"us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1),
-                                                   "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
-    del gates, ups, gate
-    torch.cuda.empty_cache()
+    if want("q4_k_down_15360x3840_b1"):
+        kd, nd = N, K
+        wdn = dev(synth.q4_k_weights(nd, kd, 104))
+        downs = [wdn] + [wdn.clone() for _ in range(-(-ROTATE_BYTES // wdn.numel()) - 1)]
+        q8 = ops.quantize_q8_1(dev(synth.activations(1, kd, 105)))
+        y = torch.empty((1, 1, nd), dtype=torch.float32, device=device)
+        us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, downs[i % len(downs)], q8, kd, nd, out=y), 4 * len(downs))
+        out["q4_k_down_15360x3840_b1"] = {"roofline": hbm_roofline("q4_k_down_15360x3840_b1", "VecQFlat<FormatQ4K>",
+                                                                   wdn.numel() + kd * 4 + nd * 4, us)}
+        del downs, wdn
+        torch.cuda.empty_cache()
 
     # Config 3: MXFP8 GEMM 2048 x 12288 x 4096, bf16 out, and its activation quantizer.
-    m, n, k = 2048, 12288, 4096
-    g = torch.Generator().manual_seed(3)
-    a = torch.randn((m, k), generator=g).to(device).to(torch.bfloat16)
-    wt = (torch.randn((n, k), generator=g) * 0.02).to(device)
-    ac, asc = ops.mxfp8_quantize(a)
-    wc, wsc = ops.mxfp8_quantize(wt)
-    d = torch.empty((m, n), dtype=torch.bfloat16, device=device)
-    us = event_us(lambda i: ops.mxfp8_gemm(ac, asc, wc, wsc, out=d), 30)
-    flops = 2.0 * m * n * k
-    out["mxfp8_gemm_2048x12288x4096"] = {"us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
-                                         "frac_dense_fp8_mfma_peak": round(flops / us / 1e6 / 5033.0, 4)}
-    out["mxfp8_quantize_2048x4096_bf16"] = {"us": round(event_us(lambda i: ops.mxfp8_quantize(a), 30), 1)}
-    del a, wt, ac, asc, wc, wsc, d
-    torch.cuda.empty_cache()
+    if want("mxfp8_gemm_2048x12288x4096"):
+        m, n, k = 2048, 12288, 4096
+        g = torch.Generator().manual_seed(3)
+        a_host = torch.randn((m, k), generator=g).to(torch.bfloat16)
+        w_host = torch.randn((n, k), generator=g) * 0.02
+        a = a_host.to(device)
+        wt = w_host.to(device)
+        ac, asc = ops.mxfp8_quantize(a)
+        wc, wsc = ops.mxfp8_quantize(wt)
+        d = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+        us = event_us(lambda i: ops.mxfp8_gemm(ac, asc, wc, wsc, out=d), 30)
+        quant_us = event_us(lambda i: ops.mxfp8_quantize(a), 30)
+        flops = 2.0 * m * n * k
+        achieved = flops / us / 1e6
+        quant_bytes = m * k * 2 + m * k + m * k // 32
+        entry = {"workload": "MXFP8 block-scaled GEMM, M=2048, K=4096, N=12288, E4M3 codes with E8M0 scales per 32, fp32 "
+                             "accumulate, bf16 out; activations quantized per token by llmp.mxfp8.quantize",
+                 "step_us": round(us + quant_us, 1), "TFLOP/s_of_the_step": round(flops / (us + quant_us) / 1e6, 1),
+                 "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                              "frac": round(achieved / MFMA_FP8_PEAK_TFLOPS, 4), "traffic": PROFILED_TRAFFIC.get("mxfp8_gemm_2048x12288x4096"),
+                              "kernel": "GemmKernel (v_mfma_scale_f32_16x16x128_f8f6f4)", "algorithmic_flops_per_launch": int(flops),
+                              "avg_launch_us": round(us, 2)},
+                 "quantize": {"us": round(quant_us, 2), "bytes": quant_bytes, "GB/s": round(quant_bytes / quant_us / 1e3, 1),
+                              "frac_hbm_peak": round(quant_bytes / quant_us / 1e3 / HBM_PEAK_GBPS, 4)}}
+        if cpu:
+            rows = 16  # a bounded sample: the first rows of A against the whole of B
+            a_f32 = a_host[:rows].float().numpy()
+            acodes, ascales = oracle.mxfp8_quantize(a_f32)
+            bcodes, bscales = oracle.mxfp8_quantize(w_host.numpy())
+            entry["cpu_baseline"] = cpu_leg(lambda: oracle.mxfp8_gemm(acodes, ascales, bcodes, bscales, threads=threads),
+                                            2.0 * rows * n * k / 1e12, "TFLOP/s", 4.0,
+                                            f"the first {rows} of the 2048 rows of A against all 12288 rows of B", threads)
+        out["mxfp8_gemm_2048x12288x4096"] = entry
+        del a, wt, ac, asc, wc, wsc, d
+        torch.cuda.empty_cache()
 
-    # Config 4: routed-expert FFN layer, 128 experts top-8, hidden 2048, FFN 768, Q4_K.
-    hidden, ffn, experts, used = 2048, 768, 128, 8
-    gate_up = dev(synth.q4_k_weights(experts * 2 * ffn, hidden, 204).reshape(experts, -1))
-    down = dev(synth.q4_k_weights(experts * hidden, ffn, 205).reshape(experts, -1))
-    expert_bytes = gate_up.numel() // experts + down.numel() // experts
-    for tokens in (1, 16, 512):
-        logits = dev(synth.rng(206).standard_normal((tokens, experts), dtype=np.float32))
-        xs = dev(synth.activations(tokens, hidden, 207))
-        _, ids, _ = ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gate_up, down, hidden, ffn, experts, used)
-        distinct = int(torch.unique(ids).numel())
-        layer = lambda i: ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gate_up, down, hidden, ffn, experts, used)
-        us = graph_us(layer, 10 if tokens == 512 else 20)
-        eager = event_us(layer, 20 if tokens == 512 else 50)
-        entry = {"us": round(us, 1), "us_launched_from_python": round(eager, 1), "distinct_experts": distinct,
-                 "GB/s_of_touched_expert_bytes": round(distinct * expert_bytes / us / 1e3, 1),
-                 "note": "whole layer replayed as a HIP graph: router, [q8_1,] gate/up+GLU, [q8_1,] down, combine "
-                         "(up to 64 pairs the products quantize their activations themselves; above 128 "
-                         "pairs the rows are sorted by expert first); weights not rotated"}
-        if tokens == 512:
-            entry["TFLOP/s"] = round(tokens * used * 3 * 2.0 * hidden * ffn / us / 1e6, 2)
-        out[f"moe_q4_k_ffn_t{tokens}"] = entry
-    del gate_up, down
-    torch.cuda.empty_cache()
+    # Config 4: routed-expert FFN layer, 128 experts top-8, hidden 2048, FFN 768, Q4_K. Sixteen copies of the
+    # experts' weights are rotated: a token's eight experts (21 MB) come from a different copy each launch, so
+    # more than 320 MB pass between two reads of the same bytes.
+    moe_names = [f"moe_q4_k_ffn_t{t}" for t in (1, 16, 512)]
+    if any(want(nm) for nm in moe_names):
+        hidden, ffn, experts, used = 2048, 768, 128, 8
+        gu_host = synth.q4_k_weights(experts * 2 * ffn, hidden, 204).reshape(experts, -1)
+        dn_host = synth.q4_k_weights(experts * hidden, ffn, 205).reshape(experts, -1)
+        gate_up, down = dev(gu_host), dev(dn_host)
+        sets = 16
+        gus = [gate_up] + [gate_up.clone() for _ in range(sets - 1)]
+        dns = [down] + [down.clone() for _ in range(sets - 1)]
+        gu_bytes, dn_bytes = gate_up.numel() // experts, down.numel() // experts
+        qk = 256
+        for tokens in (1, 16, 512):
+            name = f"moe_q4_k_ffn_t{tokens}"
+            if not want(name):
+                continue
+            logits_host = synth.rng(206).standard_normal((tokens, experts), dtype=np.float32)
+            x_host = synth.activations(tokens, hidden, 207)
+            logits, xs = dev(logits_host), dev(x_host)
+            _, ids, _ = ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gate_up, down, hidden, ffn, experts, used)
+            distinct = int(torch.unique(ids).numel())
+            layer = lambda i: ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gus[i % sets], dns[i % sets], hidden, ffn, experts, used)
+            us = timed(layer, 2 * sets)
+            # The dominant kernel alone: the gate/up product with its GLU over ready inputs.
+            pairs = tokens * used
+            h = torch.empty((pairs, ffn), dtype=torch.float32, device=device)
+            gu_stride = 2 * ffn * (hidden // qk)
+            up_of = lambda g: g.view(-1)[ffn * (hidden // qk) * 144:]
+            if pairs <= 64:
+                product = lambda i: ops.vecq_fused(ops.TYPE_Q4_K, up_of(gus[i % sets]), xs, hidden, ffn, gate=gus[i % sets], ids=ids,
+                                                   tokens=tokens, used=used, stride_expert=gu_stride, glu=ops.GLU_SWIGLU,
+                                                   out=h.view(tokens, used, ffn))
+                kernel = "VecQFlat<FormatQ4K, glu, in-kernel q8_1> routed (gate/up)"
+            elif pairs <= 128:
+                q8 = ops.quantize_q8_1(xs)
+                product = lambda i: ops.vecq(ops.TYPE_Q4_K, up_of(gus[i % sets]), q8, hidden, ffn, gate=gus[i % sets], ids=ids,
+                                             tokens=tokens, used=used, stride_expert=gu_stride, glu=ops.GLU_SWIGLU,
+                                             out=h.view(tokens, used, ffn))
+                kernel = "VecQFlat<FormatQ4K, 4 tokens a pass, glu> routed (gate/up)"
+            else:
+                route = ops.moe_route(ids, experts)
+                q8 = ops.quantize_q8_1_rows(xs, route.token)
+                product = lambda i: ops.vecq_sorted(ops.TYPE_Q4_K, up_of(gus[i % sets]), q8, route.offsets, hidden, ffn, experts,
+                                                    gate=gus[i % sets], stride_expert=gu_stride, glu=ops.GLU_SWIGLU, out=h)
+                kernel = "VecQMma<glu> over rows sorted by expert (gate/up)"
+            product_us = timed(product, 2 * sets)
+            product_bytes = distinct * gu_bytes + tokens * hidden * 4 + pairs * ffn * 4
+            layer_bytes = distinct * (gu_bytes + dn_bytes) + tokens * hidden * 4 * 2
+            entry = {"workload": f"MoE expert-grouped Q4_K FFN layer, 128 experts top-8, hidden 2048, expert FFN 768, {tokens} "
+                                 "token(s): router, [q8_1,] gate/up + SwiGLU, [q8_1,] down, ordered weighted combine",
+                     "layer_us": round(us, 1), "distinct_experts": distinct, "expert_weight_sets_rotated": sets,
+                     "layer_algorithmic_bytes": layer_bytes, "layer_GB/s": round(layer_bytes / us / 1e3, 1),
+                     "layer_frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                     "roofline": hbm_roofline(name, kernel, product_bytes, product_us)}
+            if tokens == 512:
+                flops = tokens * used * 3 * 2.0 * hidden * ffn
+                entry["layer_TFLOP/s"] = round(flops / us / 1e6, 2)
+                entry["layer_frac_int8_mfma_peak"] = round(flops / us / 1e6 / 5033.0, 4)
+            if cpu:
+                def cpu_layer():
+                    ids_c, w_c = oracle.route(logits_host, used)
+                    up_c = gu_host.reshape(-1)[ffn * (hidden // qk) * 144:]
+                    h_c = oracle.vecq(oracle.TYPE_Q4_K, up_c, oracle.q8_1_quantize(x_host), hidden, ffn, gate=gu_host, ids=ids_c,
+                                      tokens=tokens, used=used, stride_expert=gu_stride, glu=oracle.GLU_SWIGLU, experts=experts,
+                                      threads=threads)
+                    hq = oracle.q8_1_quantize(h_c.reshape(pairs, ffn))
+                    blocks = oracle.padded_k(ffn) // 32
+                    y_c = oracle.vecq(oracle.TYPE_Q4_K, dn_host, hq, ffn, hidden, ids=ids_c, tokens=tokens, used=used,
+                                      stride_expert=hidden * (ffn // qk), y_token=blocks * used, y_slot=blocks, experts=experts,
+                                      threads=threads)
+                    return oracle.expert_reduce(y_c, w_c)
+                entry["cpu_baseline"] = cpu_leg(cpu_layer, layer_bytes / 1e9, "GB/s", 2.0, f"the whole layer at {tokens} token(s)", threads)
+            out[name] = entry
+        del gus, dns, gate_up, down
+        torch.cuda.empty_cache()
 
     # Config 5: EXL3 linear 4096 x 14336 at 4 bits, 3INST codebook.
-    k, n, bits = 4096, 14336, 4
-    trellis, suh, svh = synth.exl3_weights(k, n, bits, 208)
-    t0 = dev(trellis)
-    trellises = [t0] + [t0.clone() for _ in range(-(-ROTATE_BYTES // t0.numel()) - 1)]
-    suh_d = dev(suh.view(np.int16)).view(torch.float16)
-    svh_d = dev(svh.view(np.int16)).view(torch.float16)
-    for m in (1, 16):
-        xs = dev(synth.rng(209).standard_normal((m, k)).astype(np.float16).view(np.int16)).view(torch.float16)
-        us = graph_us(lambda i: ops.exl3_linear(trellises[i % len(trellises)], suh_d, svh_d, k, n, bits,
-                                                ops.EXL3_3INST, xs), 2 * len(trellises))
-        bytes_ = t0.numel() + 2 * k + 2 * n + m * (k * 2 + n * 4)
-        out[f"exl3_linear_4096x14336_4bpw_m{m}"] = {"us": round(us, 1), "GB/s": round(bytes_ / us / 1e3, 1),
-                                                    "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4),
-                                                    "note": "input transform, product, output transform, replayed as a HIP graph"}
-    # The same shape's gate and up through exl3.multi_linear (both linears in the same launches).
-    xs = dev(synth.rng(209).standard_normal((1, k)).astype(np.float16).view(np.int16)).view(torch.float16)
-    half = len(trellises) // 2
-    side = lambda i: (trellises[i % len(trellises)], suh_d, svh_d, k, n, bits, ops.EXL3_3INST)
-    us = graph_us(lambda i: ops.exl3_multi_linear(side(i), side(i + half), xs), len(trellises))
-    bytes_ = 2 * (t0.numel() + 2 * k + 2 * n) + k * 2 + 2 * (k * 2 + n * 4)
-    out["exl3_multi_linear_4096x2x14336_4bpw_m1"] = {"us": round(us, 1), "GB/s": round(bytes_ / us / 1e3, 1),
-                                                     "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    exl3_names = [f"exl3_linear_4096x14336_4bpw_m{m}" for m in (1, 16)]
+    if any(want(nm) for nm in exl3_names) or want("exl3_multi_linear_4096x2x14336_4bpw_m1"):
+        k, n, bits = 4096, 14336, 4
+        trellis, suh, svh = synth.exl3_weights(k, n, bits, 208)
+        t0 = dev(trellis)
+        trellises = [t0] + [t0.clone() for _ in range(-(-ROTATE_BYTES // t0.numel()) - 1)]
+        suh_d = dev(suh.view(np.int16)).view(torch.float16)
+        svh_d = dev(svh.view(np.int16)).view(torch.float16)
+        for m in (1, 16):
+            name = f"exl3_linear_4096x14336_4bpw_m{m}"
+            if not want(name):
+                continue
+            x_host = synth.rng(209).standard_normal((m, k)).astype(np.float16)
+            xs = dev(x_host.view(np.int16)).view(torch.float16)
+            us = timed(lambda i: ops.exl3_linear(trellises[i % len(trellises)], suh_d, svh_d, k, n, bits,
+                                                 ops.EXL3_3INST, xs), 2 * len(trellises))
+            bytes_ = t0.numel() + 2 * k + 2 * n + m * (k * 2 + n * 4)
+            entry = {"workload": f"EXL3 trellis-coded linear 4096 x 14336, 4 bits a weight, 3INST codebook, {m} row(s) of fp16: "
+                                 "input transform, product, output transform",
+                     "roofline": hbm_roofline(name, "the linear's launches (ProductKernel<3INST, 4> dominant)", bytes_, us)}
+            if cpu:
+                entry["cpu_baseline"] = cpu_leg(
+                    lambda: oracle.exl3_linear(trellis, suh.view(np.uint16), svh.view(np.uint16), k, n, bits, 0, x_host, threads=threads),
+                    t0.numel() / 1e9, "GB/s", 2.5, f"the whole linear at {m} row(s)", threads)
+            out[name] = entry
+        if want("exl3_multi_linear_4096x2x14336_4bpw_m1"):
+            xs = dev(synth.rng(209).standard_normal((1, k)).astype(np.float16).view(np.int16)).view(torch.float16)
+            half = len(trellises) // 2
+            side = lambda i: (trellises[i % len(trellises)], suh_d, svh_d, k, n, bits, ops.EXL3_3INST)
+            us = timed(lambda i: ops.exl3_multi_linear(side(i), side(i + half), xs), len(trellises))
+            bytes_ = 2 * (t0.numel() + 2 * k + 2 * n) + k * 2 + 2 * (k * 2 + n * 4)
+            out["exl3_multi_linear_4096x2x14336_4bpw_m1"] = {"roofline": hbm_roofline("exl3_multi_linear_4096x2x14336_4bpw_m1",
+                                                                                     "exl3.multi_linear's launches", bytes_, us)}
     return out
 
 
@@ -315,16 +454,9 @@ def block_formats(device):
     return out
 
 
-# HBM bytes per launch of the dominant kernel at batch 1 through the default variant, from two
-# rocprofv3 --pmc runs of this file (FETCH_SIZE 32,478.4 KiB and WRITE_SIZE 60.1 KiB per dispatch,
-# scaled by 1.9988 and 1.0: what the same counters read for --calibrate-copy's copy of 64,800 KiB).
-# Counters cannot be read from inside a run, so other shapes and variants report null.
-PROFILED_TRAFFIC_BYTES = int(round((32478.4 * 1.9988 + 60.1) * 1024))
-
-
 def measured_traffic(args):
     if args.tokens == 1 and args.variant == -1 and not args.fused:
-        return PROFILED_TRAFFIC_BYTES
+        return PROFILED_TRAFFIC["q4_k_gate_up_geglu_b1"]
     return None
 
 
@@ -346,6 +478,9 @@ def main():
                     help="a step is one launch that quantizes the activations in the kernel, instead of "
                          "llmp.q8_1 followed by llmp.vecq over its Q8_1 blocks (the reference's two operations)")
     ap.add_argument("--eager", action="store_true", help="launch each step from Python instead of a graph")
+    ap.add_argument("--only", default=None,
+                    help="run one of the other configurations alone (its key in other_configs) and print its entry: "
+                         "what the profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not built")
@@ -356,6 +491,18 @@ def main():
     from llmp_amd import ops, synth
 
     device = torch.device("cuda:0")
+    if args.calibrate_copy:
+        # A copy of known size (WEIGHT_BYTES read, WEIGHT_BYTES written) for scaling the hardware counters.
+        whole = torch.randint(0, 255, (WEIGHT_BYTES,), dtype=torch.uint8, device=device)
+        target = torch.empty_like(whole)
+        for _ in range(20):
+            target.copy_(whole)
+        torch.cuda.synchronize()
+        del whole, target
+    if args.only is not None:
+        print(json.dumps({"other_configs": other_configs(device, args, only=args.only), "data": "synthetic",
+                          "launch": "eager" if args.eager else "hip graph"}))
+        return
     if args.formats:
         print(json.dumps({"block_formats": block_formats(device), "data": "synthetic", "launch": "hip graph",
                           "weight_copies_rotated_bytes": ROTATE_BYTES}))
@@ -413,14 +560,6 @@ def main():
         torch.cuda.synchronize()
         return begin.elapsed_time(end), (time.perf_counter() - t0) * 1e3
 
-    if args.calibrate_copy:
-        # A copy of known size: WEIGHT_BYTES read, WEIGHT_BYTES written.
-        whole = torch.cat([gates[0].view(-1), ups[0].view(-1)])
-        target = torch.empty_like(whole)
-        for _ in range(20):
-            target.copy_(whole)
-        torch.cuda.synchronize()
-        del whole, target
     step(0)
     torch.cuda.synchronize()
     timed_region(step, args.warmup, 0)
