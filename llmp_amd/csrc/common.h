@@ -59,7 +59,6 @@ __device__ __forceinline__ float E4m3ToFloat(uint32_t bits) {
 __device__ __forceinline__ int Dot4(int a, int b, int c) {
   return __builtin_amdgcn_sdot4(a, b, c, false);
 }
-
 // A 16-byte and a 4-byte-aligned 16-byte global load of weights, which are
 // read once: non-temporal, so that they do not displace the activations.
 typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));

@@ -1,0 +1,10 @@
+// llmp.vecq's streaming form (vecq_flat.h) instantiated for: FormatQ5K.
+#include "vecq_flat.h"
+
+namespace llmp_hip {
+
+void LaunchFlatQ5K(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
+  LaunchF<FormatQ5K>(a, x_type, pass, deep, stream);
+}
+
+}  // namespace llmp_hip

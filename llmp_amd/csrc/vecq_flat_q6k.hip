@@ -1,0 +1,10 @@
+// llmp.vecq's streaming form (vecq_flat.h) instantiated for: FormatQ6K.
+#include "vecq_flat.h"
+
+namespace llmp_hip {
+
+void LaunchFlatQ6K(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t stream) {
+  LaunchF<FormatQ6K>(a, x_type, pass, deep, stream);
+}
+
+}  // namespace llmp_hip
