@@ -110,6 +110,78 @@ __global__ void QuantizeKernel(const T* __restrict__ x, int64_t x_stride, uint8_
   scales[at] = static_cast<uint8_t>(e);
 }
 
+// The same quantizer for rows that allow 16-byte loads: eight values a lane, four lanes a block, sixteen lanes
+// the four blocks whose scales are one dword of an atom. Loads and stores are coalesced (a wave reads 512
+// consecutive values and writes their 512 bytes of codes), the block's largest magnitude crosses its quad by
+// data-parallel moves, and the codes come from the hardware's conversion (OCP E4M3, nearest even) after a clamp
+// to +-448, with a NaN's code put in by hand: bit for bit ToE4m3's.
+template <typename T>
+__global__ __launch_bounds__(256) void QuantizeWideKernel(const T* __restrict__ x, int64_t x_stride, uint8_t* __restrict__ codes,
+                                                          uint8_t* __restrict__ scales, int k, int rows, int64_t items) {
+#pragma clang fp contract(off)
+  // One piece of eight values a lane (two, half of the rows apart, with both loads queued first, measured
+  // slower: 7.3 us against 6.7 for 2048 rows of 4096). Whole groups of sixteen lanes share a row: k / 8 is a
+  // multiple of sixteen.
+  constexpr int kPieces = 1;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t half = items / kPieces;
+  if (first >= half) return;
+  const int per_row = k / 8;
+  const int blocks = k / 32;
+  const int lane = threadIdx.x & 63;
+  int r[kPieces], c[kPieces];
+  float v[kPieces][8];
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    const int64_t i = first + p * half;
+    r[p] = static_cast<int>(i / per_row);
+    c[p] = static_cast<int>(i % per_row) * 8;
+    if (r[p] >= rows) continue;
+    const T* from = x + static_cast<int64_t>(r[p]) * x_stride + c[p];
+    if constexpr (sizeof(T) == 4) {
+      const float4 a = reinterpret_cast<const float4*>(from)[0], b = reinterpret_cast<const float4*>(from)[1];
+      v[p][0] = a.x, v[p][1] = a.y, v[p][2] = a.z, v[p][3] = a.w, v[p][4] = b.x, v[p][5] = b.y, v[p][6] = b.z, v[p][7] = b.w;
+    } else {
+      const uint4 raw = *reinterpret_cast<const uint4*>(from);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[p][2 * j] = Bf16BitsToFloat(w[j] & 0xFFFFu), v[p][2 * j + 1] = Bf16BitsToFloat(w[j] >> 16);
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    if (r[p] >= rows) {  // the atoms' padding rows: zero scales, no codes (whole rows: uniform over the group)
+      if ((lane & 15) == 0) *reinterpret_cast<uint32_t*>(scales + AtomOffset(r[p], c[p] / 32, blocks)) = 0;
+      continue;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[p][j]));
+    amax = fmaxf(amax, ShflXor(amax, 1));
+    amax = fmaxf(amax, ShflXor(amax, 2));
+    const uint32_t e = ScaleCode(amax);
+    const float inverse = InverseScale(e);
+    uint32_t word[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = v[p][2 * j] * inverse, b = v[p][2 * j + 1] * inverse;
+      const float ca = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f), cb = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
+      word[j >> 1] = (j & 1) != 0 ? static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, static_cast<int>(word[j >> 1]), true))
+                                  : static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, static_cast<int>(word[j >> 1]), false));
+      // A NaN keeps its sign and takes the format's NaN, whatever the clamp and the conversion made of it.
+      const int at = 16 * (j & 1);
+      if (a != a) word[j >> 1] = (word[j >> 1] & ~(0xFFu << at)) | ((((__builtin_bit_cast(uint32_t, a) >> 24) & 0x80u) | 0x7Fu) << at);
+      if (b != b) word[j >> 1] = (word[j >> 1] & ~(0xFF00u << at)) | ((((__builtin_bit_cast(uint32_t, b) >> 24) & 0x80u) | 0x7Fu) << (at + 8));
+    }
+    *reinterpret_cast<uint2*>(codes + static_cast<int64_t>(r[p]) * k + c[p]) = make_uint2(word[0], word[1]);
+    // The four blocks' scales of these sixteen lanes into one dword: block (lane / 4) % 4 in byte (lane / 4) % 4.
+    uint32_t four = e << (8 * ((lane >> 2) & 3));
+    four |= ShflXor(four, 4);
+    four |= ShflXor(four, 8);
+    if ((lane & 15) == 0) *reinterpret_cast<uint32_t*>(scales + AtomOffset(r[p], c[p] / 32, blocks)) = four;
+  }
+}
+
 // One scale a thread: row r's block b to its place in the atoms (zero for the padding rows).
 __global__ void SwizzleKernel(const uint8_t* __restrict__ in, uint8_t* __restrict__ out, int n, int blocks,
                               int64_t items) {
@@ -463,6 +535,23 @@ extern "C" int llmp_hip_mxfp8_quantize(const void* x, int x_type, int64_t x_stri
   const int64_t items = padded * (k / 32);
   const dim3 grid(static_cast<unsigned>((items + 255) / 256));
   const auto s = static_cast<hipStream_t>(stream);
+  // Rows that start on 16-byte boundaries (and scales on 4-byte ones): eight values a lane.
+  const int64_t element = x_type == LLMP_X_F32 ? 4 : 2;
+  if (reinterpret_cast<uintptr_t>(x) % 16 == 0 && (x_stride * element) % 16 == 0 && reinterpret_cast<uintptr_t>(scales) % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(codes) % 8 == 0) {
+    const int64_t wide_items = padded * (k / 8);
+    const dim3 wide_grid(static_cast<unsigned>((wide_items + 255) / 256));
+    if (x_type == LLMP_X_F32) {
+      hipLaunchKernelGGL(QuantizeWideKernel<float>, wide_grid, dim3(256), 0, s, static_cast<const float*>(x), x_stride,
+                         static_cast<uint8_t*>(codes), static_cast<uint8_t*>(scales), static_cast<int>(k),
+                         static_cast<int>(rows), wide_items);
+    } else {
+      hipLaunchKernelGGL(QuantizeWideKernel<uint16_t>, wide_grid, dim3(256), 0, s, static_cast<const uint16_t*>(x), x_stride,
+                         static_cast<uint8_t*>(codes), static_cast<uint8_t*>(scales), static_cast<int>(k),
+                         static_cast<int>(rows), wide_items);
+    }
+    return LaunchStatus("mxfp8.quantize");
+  }
   if (x_type == LLMP_X_F32) {
     hipLaunchKernelGGL(QuantizeKernel<float>, grid, dim3(256), 0, s, static_cast<const float*>(x), x_stride,
                        static_cast<uint8_t*>(codes), static_cast<uint8_t*>(scales), static_cast<int>(k),

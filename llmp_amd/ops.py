@@ -272,12 +272,15 @@ def mxfp8_scale_bytes(rows, k):
     return (rows + 127) // 128 * 128 * (k // 32)
 
 
-def mxfp8_quantize(x):
-    """llmp.mxfp8.quantize: float32 / bfloat16 [rows, k] -> (codes uint8 [rows, k], scales uint8 atoms)."""
+def mxfp8_quantize(x, out=None):
+    """llmp.mxfp8.quantize: float32 / bfloat16 [rows, k] -> (codes uint8 [rows, k], scales uint8 atoms); `out`,
+    a pair of such tensors, is filled in place."""
     lib = _lib.load()
     rows, k = x.shape
-    codes = torch.empty((rows, k), dtype=torch.uint8, device=x.device)
-    scales = torch.empty(mxfp8_scale_bytes(rows, k), dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = (torch.empty((rows, k), dtype=torch.uint8, device=x.device),
+               torch.empty(mxfp8_scale_bytes(rows, k), dtype=torch.uint8, device=x.device))
+    codes, scales = out
     _lib.check(lib.llmp_hip_mxfp8_quantize(_ptr(x), _x_type(x), x.stride(0), k, rows, _ptr(codes), _ptr(scales),
                                            _stream()))
     return codes, scales
