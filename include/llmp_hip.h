@@ -289,14 +289,15 @@ int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void* w, int col
 int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, int columns, int f32,
                            int input_scale, void* stream);
 
-/* The packed linear for 1..16 rows: LinearOperands of validate.h:118-131 and
- * PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54. x (m x k F16) into
- * y (m x n, F16 or F32); a_had is the caller's m x k F16 scratch for the transformed input,
- * which the product's launch writes as it computes it. `scratch` (llmp_hip_exl3_linear_scratch
- * bytes, 8-byte aligned) takes the place of the reference's lock area: the K slices' partial
- * sums, added in slice order. Two launches are queued (three above four rows: the input
- * transform is then a launch of its own); a failure after the first is reported as a fault
- * (negative). */
+/* The packed linear: LinearOperands of validate.h:118-131 and PackedGemvLinear / PackedGemmLinear of
+ * src/kernels/exl3/linear.h:47-54, 1 to 65536 rows (validate.h:76) in passes of sixteen, each pass streaming
+ * the weights once (upstream's choice, validate.h:254-256, is this path through 144 rows and the
+ * reconstruction above, which is not built: a caller with more rows pays a pass every sixteen). x (m x k F16)
+ * into y (m x n, F16 or F32); a_had is the caller's m x k F16 scratch for the transformed input, which the
+ * launches write as they compute it. `scratch` (llmp_hip_exl3_linear_scratch bytes, 8-byte aligned: one pass's,
+ * shared by the passes in stream order) takes the place of the reference's lock area: the K slices' partial
+ * sums, added in slice order. Two launches a pass are queued (three above four rows: the input transform is
+ * then a launch of its own); a failure after the first is reported as a fault (negative). */
 typedef struct llmp_exl3_linear {
   llmp_exl3_weights weights;
   const void* x;
@@ -326,8 +327,8 @@ int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* stream);
  * first linear's rows, then the second's); a_had is 2 x m x k F16 (validate.cc:257-260), each
  * linear's own transformed input. The reference's three pointer tables have no counterpart:
  * the launches carry the six addresses. Same launches as llmp_hip_exl3_linear, both linears in
- * each (one linear after the other where their codebooks differ); `scratch` is
- * llmp_hip_exl3_multi_linear_scratch bytes. */
+ * each (one linear after the other where their codebooks differ), in the same passes of sixteen rows;
+ * `scratch` is llmp_hip_exl3_multi_linear_scratch bytes. */
 typedef struct llmp_exl3_multi_linear {
   llmp_exl3_weights first;
   llmp_exl3_weights second;

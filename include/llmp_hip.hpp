@@ -307,7 +307,13 @@ inline std::size_t ScratchBytes(const LinearOperands& o) {
   const llmp_exl3_linear abi = ToAbi(o);
   return llmp_hip_exl3_linear_scratch(&abi);
 }
-// PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54, 1 to 16 rows.
+// PackedGemvLinear / PackedGemmLinear of src/kernels/exl3/linear.h:47-54, 1 to 65536 rows in passes of sixteen.
+// UpstreamPath of src/kernels/exl3/validate.h:254-256: the packed path through 144 rows (the reconstruction paths
+// it names above that are not built here; the packed path still takes those rows).
+enum class LinearPath : std::uint8_t { kPacked, kReconstruct, kReconstructFused };
+constexpr LinearPath UpstreamPath(int rows) {
+  return rows >= 1024 ? LinearPath::kReconstructFused : rows > 144 ? LinearPath::kReconstruct : LinearPath::kPacked;
+}
 inline KernelFailure PackedLinear(const LinearOperands& o, void* scratch, std::size_t scratch_bytes, void* stream) {
   const llmp_exl3_linear abi = ToAbi(o);
   return FromStatus(llmp_hip_exl3_linear(&abi, scratch, scratch_bytes, stream));
@@ -480,10 +486,10 @@ inline std::vector<Implementation> Implementations() {
   // EXL3 (exl3/implementations.h:8-31): the packed paths; the reconstruction paths are not built.
   add("exl3.linear.gemv", "quant_linear", {"exl3"}, {1, 8, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
       "trellis tiles as the second operand of a 16 x 16 x 16 F16 matrix instruction");
-  add("exl3.linear.gemm", "quant_linear", {"exl3"}, {1, 16, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
-      "the same launches for up to 16 rows");
-  add("exl3.multi_linear.mgemm", "quant_multi_linear", {"exl3"}, {1, 16, 128, 128}, Rung::kOnChipDecode, kBf16Mma,
-      {"llmp_hip_exl3_multi_linear"}, "gate and up in grid z");
+  add("exl3.linear.gemm", "quant_linear", {"exl3"}, {1, 65536, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
+      "the same launches in passes of sixteen rows");
+  add("exl3.multi_linear.mgemm", "quant_multi_linear", {"exl3"}, {1, 65536, 128, 128}, Rung::kOnChipDecode, kBf16Mma,
+      {"llmp_hip_exl3_multi_linear"}, "gate and up in grid z, passes of sixteen rows");
   // The quantizing KV cache stores (kv_quant.h:150-192).
   add("llmp.set_rows.quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant"}, "a thread a block");
   add("llmp.set_rows.grouped_quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant_group"},

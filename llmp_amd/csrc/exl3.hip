@@ -172,6 +172,7 @@ __global__ __launch_bounds__(256) void ReconstructKernel(const uint32_t* __restr
 // The 128-point Walsh-Hadamard transform of a wave's 128 values, lane l holding values 2 l and
 // 2 l + 1, natural order (H[i][j] = (-1)^popcount(i & j)), unscaled, in F32.
 __device__ __forceinline__ void Hadamard128(float& a, float& b, int lane) {
+#pragma clang fp contract(off)
   const float s = a + b;
   b = a - b;
   a = s;
@@ -201,6 +202,9 @@ inline HadamardSides OneSide(const void* x, void* y, const uint16_t* in_scale, c
 template <int X, int Y>
 __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, int columns, int slices,
                                                     int64_t slice_stride) {
+  // No fused multiply-adds: the transform inside the product kernel rounds every step the same way, so that a
+  // row's transformed input, and with it its output, is the same bits whichever launch computed it.
+#pragma clang fp contract(off)
   const void* __restrict__ x = sides.x[blockIdx.z];
   void* __restrict__ y = sides.y[blockIdx.z];
   const uint16_t* __restrict__ in_scale = sides.in_scale[blockIdx.z];
@@ -267,6 +271,7 @@ struct ProductSides {  // one or two linears a launch (grid z)
 template <int CB, int BITS, bool kFused>
 __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const ProductSides sides, int m, int n, int k,
                                                                    int blocks_per_wave) {
+#pragma clang fp contract(off)
   const uint8_t* __restrict__ trellis = sides.trellis[blockIdx.z];
   const uint16_t* __restrict__ x = sides.x[blockIdx.z];
   const uint16_t* __restrict__ suh = sides.suh[blockIdx.z];
@@ -599,9 +604,15 @@ int LaunchLinears(const llmp_exl3_weights* const (&w)[2], int count, const void*
 }  // namespace
 }  // namespace llmp_hip
 
+// The rows of one pass of the packed product (the matrix instruction's sixteen); more rows take more passes,
+// each streaming the weights again (src/kernels/exl3/validate.h:76: a launch takes 1 to 65536 rows).
+constexpr int kPassRows = 16;
+constexpr int kMostRows = 1 << 16;
+
 extern "C" size_t llmp_hip_exl3_linear_scratch(const llmp_exl3_linear* op) {
   if (op == nullptr || op->m <= 0 || op->weights.k <= 0 || op->weights.n <= 0) return 0;
-  return static_cast<size_t>(SlicesFor(op->weights.n, op->weights.k)) * op->m * op->weights.n * sizeof(float);
+  const int pass = op->m < kPassRows ? op->m : kPassRows;  // the passes share the area
+  return static_cast<size_t>(SlicesFor(op->weights.n, op->weights.k)) * pass * op->weights.n * sizeof(float);
 }
 
 namespace llmp_hip {
@@ -614,7 +625,7 @@ int LinearOver(const llmp_exl3_linear* op, void* area, size_t area_bytes, hipStr
   if (const int bad = CheckWeights(op->weights); bad != 0) return bad;
   if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || area == nullptr)
     return Refuse(1, "exl3.linear: null operand");
-  if (op->m < 1 || op->m > 16) return Refuse(1, "exl3.linear: the packed product takes 1 to 16 rows, not %d", op->m);
+  if (op->m < 1 || op->m > kMostRows) return Refuse(1, "exl3.linear: the packed product takes 1 to %d rows, not %d", kMostRows, op->m);
   if (area_bytes < llmp_hip_exl3_linear_scratch(op))
     return Refuse(1, "exl3.linear: scratch too small: %zu bytes of partial sums, %zu given", llmp_hip_exl3_linear_scratch(op), area_bytes);
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
@@ -634,10 +645,19 @@ int LinearOver(const llmp_exl3_linear* op, void* area, size_t area_bytes, hipStr
     if (const int bad = Disjoint("exl3.linear", partials, {x, TrellisRange(w), SuhRange(w), SvhRange(w)}); bad != 0) return bad;
   }
   const llmp_exl3_weights* const w[2] = {&op->weights, &op->weights};
-  void* const a_had[2] = {op->a_had, op->a_had};
-  void* const y[2] = {op->y, op->y};
   float* const partial[2] = {static_cast<float*>(area), static_cast<float*>(area)};
-  return LaunchLinears(w, 1, op->x, a_had, y, partial, op->f32 != 0, op->m, "exl3.linear", stream);
+  // Sixteen rows a pass, the passes in stream order over the one area of partial sums.
+  for (int row = 0; row < op->m; row += kPassRows) {
+    const int rows = op->m - row < kPassRows ? op->m - row : kPassRows;
+    const size_t in = static_cast<size_t>(row) * op->weights.k * 2;
+    const size_t out = static_cast<size_t>(row) * op->weights.n * (op->f32 ? 4 : 2);
+    void* const a_had[2] = {static_cast<uint8_t*>(op->a_had) + in, static_cast<uint8_t*>(op->a_had) + in};
+    void* const y[2] = {static_cast<uint8_t*>(op->y) + out, static_cast<uint8_t*>(op->y) + out};
+    const int status = LaunchLinears(w, 1, static_cast<const uint8_t*>(op->x) + in, a_had, y, partial, op->f32 != 0, rows,
+                                     "exl3.linear", stream);
+    if (status != 0) return row == 0 ? status : (status > 0 ? -status : status);  // after a queued pass: a fault
+  }
+  return 0;
 }
 
 // This device's copy of the static array: its address is asked for once a device, with that device current.
@@ -691,7 +711,8 @@ extern "C" int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* str
 
 extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op) {
   if (op == nullptr || op->m <= 0 || op->first.k <= 0 || op->first.n <= 0) return 0;
-  return 2 * static_cast<size_t>(SlicesFor(op->first.n, op->first.k)) * op->m * op->first.n * sizeof(float);
+  const int pass = op->m < kPassRows ? op->m : kPassRows;  // the passes share the area
+  return 2 * static_cast<size_t>(SlicesFor(op->first.n, op->first.k)) * pass * op->first.n * sizeof(float);
 }
 
 extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void* scratch, size_t scratch_bytes,
@@ -704,7 +725,8 @@ extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void
     return Refuse(1, "exl3.multi_linear: the two linears of a multi-GEMM share k, n and K");
   if (op->x == nullptr || op->a_had == nullptr || op->y == nullptr || scratch == nullptr)
     return Refuse(1, "exl3.multi_linear: null operand");
-  if (op->m < 1 || op->m > 16) return Refuse(1, "exl3.multi_linear: the packed product takes 1 to 16 rows, not %d", op->m);
+  if (op->m < 1 || op->m > kMostRows)
+    return Refuse(1, "exl3.multi_linear: the packed product takes 1 to %d rows, not %d", kMostRows, op->m);
   if (scratch_bytes < llmp_hip_exl3_multi_linear_scratch(op)) return Refuse(1, "exl3.multi_linear: scratch too small");
   if ((reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->a_had) |
        reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(scratch)) % 8 != 0)
@@ -728,23 +750,36 @@ extern "C" int llmp_hip_exl3_multi_linear(const llmp_exl3_multi_linear* op, void
   }
   const auto s = static_cast<hipStream_t>(stream);
   const int m = op->m, k = op->first.k, n = op->first.n;
-  const size_t out_bytes = static_cast<size_t>(m) * n * (op->f32 ? 4 : 2);
+  const size_t element = op->f32 ? 4 : 2;
   float* const part = static_cast<float*>(scratch);
-  const size_t part_floats = static_cast<size_t>(SlicesFor(n, k)) * m * n;
+  const size_t part_floats = static_cast<size_t>(SlicesFor(n, k)) * (m < kPassRows ? m : kPassRows) * n;
   const llmp_exl3_weights* const w[2] = {&op->first, &op->second};
-  void* const a_had[2] = {op->a_had, static_cast<uint16_t*>(op->a_had) + static_cast<size_t>(m) * k};
-  void* const y[2] = {op->y, static_cast<uint8_t*>(op->y) + out_bytes};
   float* const partial[2] = {part, part + part_floats};
-  if (op->first.codebook == op->second.codebook)
-    return LaunchLinears(w, 2, op->x, a_had, y, partial, op->f32 != 0, m, "exl3.multi_linear", s);
-  // Different codebooks decode differently: one linear after the other.
-  for (int i = 0; i < 2; ++i) {
-    const llmp_exl3_weights* const one[2] = {w[i], w[i]};
-    void* const a[2] = {a_had[i], a_had[i]};
-    void* const out[2] = {y[i], y[i]};
-    float* const p[2] = {partial[i], partial[i]};
-    const int status = LaunchLinears(one, 1, op->x, a, out, p, op->f32 != 0, m, "exl3.multi_linear", s);
-    if (status != 0) return i == 0 ? status : (status > 0 ? -status : status);
+  bool queued = false;
+  // Sixteen rows a pass, the passes in stream order over the one area of partial sums.
+  for (int row = 0; row < m; row += kPassRows) {
+    const int rows = m - row < kPassRows ? m - row : kPassRows;
+    const uint8_t* x = static_cast<const uint8_t*>(op->x) + static_cast<size_t>(row) * k * 2;
+    void* const a_had[2] = {static_cast<uint16_t*>(op->a_had) + static_cast<size_t>(row) * k,
+                            static_cast<uint16_t*>(op->a_had) + (static_cast<size_t>(m) + row) * k};
+    void* const y[2] = {static_cast<uint8_t*>(op->y) + static_cast<size_t>(row) * n * element,
+                        static_cast<uint8_t*>(op->y) + (static_cast<size_t>(m) + row) * n * element};
+    if (op->first.codebook == op->second.codebook) {
+      const int status = LaunchLinears(w, 2, x, a_had, y, partial, op->f32 != 0, rows, "exl3.multi_linear", s);
+      if (status != 0) return !queued ? status : (status > 0 ? -status : status);
+      queued = true;
+      continue;
+    }
+    // Different codebooks decode differently: one linear after the other.
+    for (int i = 0; i < 2; ++i) {
+      const llmp_exl3_weights* const one[2] = {w[i], w[i]};
+      void* const a[2] = {a_had[i], a_had[i]};
+      void* const out[2] = {y[i], y[i]};
+      float* const p[2] = {partial[i], partial[i]};
+      const int status = LaunchLinears(one, 1, x, a, out, p, op->f32 != 0, rows, "exl3.multi_linear", s);
+      if (status != 0) return !queued ? status : (status > 0 ? -status : status);
+      queued = true;
+    }
   }
   return 0;
 }

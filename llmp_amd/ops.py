@@ -353,7 +353,7 @@ def exl3_hadamard(x, scale, input_scale=True):
 
 
 def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, f32=True, keep=None):
-    """x float16 [m, k] (m <= 16) through the EXL3 linear: [m, n] float32 or float16.
+    """x float16 [m, k] through the EXL3 linear (sixteen rows a pass): [m, n] float32 or float16.
     `keep`, a dict, receives the transformed input a_had."""
     lib = _lib.load()
     m = x.shape[0]
@@ -384,7 +384,7 @@ def exl3_linear_static(trellis, suh, svh, k, n, bits, codebook, x, a_had, y):
 
 
 def exl3_multi_linear(first, second, x, f32=True, keep=None):
-    """exl3.multi_linear: x float16 [m, k] (m <= 16) through a gate and an up linear of the same k, n and
+    """exl3.multi_linear: x float16 [m, k] (sixteen rows a pass) through a gate and an up linear of the same k, n and
     rate: [2, m, n]. `first` and `second` are (trellis, suh, svh, k, n, bits, codebook); `keep`, a dict,
     receives the two transformed inputs a_had [2, m, k]."""
     lib = _lib.load()

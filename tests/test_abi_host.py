@@ -110,7 +110,7 @@ def test_exl3_linears_refuse_bad_operands():
         return w
 
     one = _lib.Exl3Linear()
-    one.weights, one.x, one.a_had, one.y, one.f32, one.m = weights(), 0x4000, 0x5000, 0x6000, 1, 17
+    one.weights, one.x, one.a_had, one.y, one.f32, one.m = weights(), 0x4000, 0x5000, 0x6000, 1, 65537
     assert lib.llmp_hip_exl3_linear(C.byref(one), 0x7000, 1 << 30, None) > 0 and b"rows" in lib.llmp_hip_last_error()
     two = _lib.Exl3MultiLinear()
     two.first, two.second = weights(), weights(bits=3)
@@ -121,7 +121,7 @@ def test_exl3_linears_refuse_bad_operands():
     assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 1 << 30, None) > 0
     two.second = weights()
     assert lib.llmp_hip_exl3_multi_linear(C.byref(two), 0x7000, 8, None) > 0 and b"scratch" in lib.llmp_hip_last_error()
-    assert lib.llmp_hip_exl3_multi_linear_scratch(C.byref(two)) == 2 * lib.llmp_hip_exl3_linear_scratch(C.byref(one)) // 17 * 2
+    assert lib.llmp_hip_exl3_multi_linear_scratch(C.byref(two)) == 2 * lib.llmp_hip_exl3_linear_scratch(C.byref(one)) // 16 * 2
 
 
 def test_default_descriptors_are_refused_before_any_plan():

@@ -1,6 +1,8 @@
 """Parity of the EXL3 operations (HIP, through the C ABI) against the CPU oracle: reconstructed
 weights bit for bit (every rate, the three codebooks), the transforms within F16/F32 rounding,
 and the packed linear to a maximum relative error of 1e-3."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -111,12 +113,48 @@ def test_linear_rows_are_independent_and_f16_output_rounds_once(device):
     assert np.array_equal(half.view(np.uint16), full.astype(np.float16).view(np.uint16))
 
 
+@pytest.mark.parametrize("m", [17, 40, 144])
+def test_linear_of_more_than_sixteen_rows_runs_in_passes(device, m):
+    """The packed path is upstream's choice through 144 rows (src/kernels/exl3/validate.h:254-256 of the
+    reference): here sixteen rows a pass. Against the oracle over the device's transformed input, and each pass
+    bit for bit the launch of its sixteen (or fewer) rows alone."""
+    k, n, bits, codebook = 1024, 512, 4, ops.EXL3_3INST
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 71)
+    x = synth.rng(72 + m).standard_normal((m, k)).astype(np.float16)
+    args = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    keep = {}
+    got = ops.exl3_linear(*args, halves(x, device), keep=keep).cpu().numpy()
+    a_had = keep["a_had"].cpu().numpy().view(np.uint16)
+    want_had = oracle.exl3_input(suh.view(np.uint16), k, x.view(np.uint16))
+    ulps = np.abs(a_had.view(np.int16).astype(np.int32) - want_had.view(np.int16).astype(np.int32))
+    assert ulps.max() <= 1 and np.count_nonzero(ulps) <= 0.01 * ulps.size
+    want = oracle.exl3_product(trellis, svh.view(np.uint16), k, n, bits, codebook, a_had, threads=oracle.max_threads())
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, worst
+    for first in range(0, m, 16):
+        alone = ops.exl3_linear(*args, halves(x[first:first + 16], device)).cpu().numpy()
+        assert np.array_equal(alone.view(np.uint32), got[first:first + 16].view(np.uint32)), first
+    if m == 40:
+        up = synth.exl3_weights(k, n, bits, 73)
+        second = (dev(up[0], device), halves(up[1], device), halves(up[2], device), k, n, bits, codebook)
+        both = ops.exl3_multi_linear(args, second, halves(x, device)).cpu().numpy()
+        assert np.array_equal(both[0].view(np.uint32), got.view(np.uint32))
+        alone = ops.exl3_linear(*second, halves(x, device)).cpu().numpy()
+        assert np.array_equal(both[1].view(np.uint32), alone.view(np.uint32))
+
+
 def test_refusals(device):
     trellis, suh, svh = synth.exl3_weights(128, 128, 4, 41)
-    x = halves(np.zeros((17, 128), dtype=np.float16), device)
+    x = halves(np.zeros((2, 128), dtype=np.float16), device)
+    # An in-place linear (a_had and y on x) is refused before anything is queued (validate.cc:120-126).
+    op = ops.Exl3Linear()
+    op.weights = ops._exl3_weights(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 4, 0)
+    op.x, op.a_had, op.y, op.f32, op.m = x.data_ptr(), x.data_ptr(), x.data_ptr(), 0, 2
+    scratch = torch.empty(1 << 16, dtype=torch.uint8, device=device)
+    lib = ops._lib.load()
     with pytest.raises(ops.KernelFailure) as e:
-        ops.exl3_linear(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 4, 0, x)
-    assert e.value.rejected
+        ops._lib.check(lib.llmp_hip_exl3_linear(C.byref(op), scratch.data_ptr(), scratch.numel(), None))
+    assert e.value.rejected and "overlaps" in e.value.detail
     with pytest.raises(ops.KernelFailure):
         ops.exl3_reconstruct(dev(trellis, device), halves(suh, device), halves(svh, device), 128, 128, 9, 0)
     with pytest.raises(ops.KernelFailure):

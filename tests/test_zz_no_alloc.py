@@ -69,7 +69,7 @@ def test_static_scratch_linear_refuses_what_exceeds_its_array(device):
     assert lib.llmp_hip_exl3_linear_scratch(C.byref(op)) > (4 << 20)
     assert lib.llmp_hip_exl3_linear_static(C.byref(op), None) == 1
     assert b"exceed the static area" in lib.llmp_hip_last_error()
-    op.m = 17  # and the linear's own refusals still hold
+    op.m = 65537  # and the linear's own refusals still hold
     w.n = 128
     op.weights = w
     assert lib.llmp_hip_exl3_linear_static(C.byref(op), None) == 1 and b"rows" in lib.llmp_hip_last_error()
