@@ -200,6 +200,37 @@ int llmp_hip_mxfp8_gemm_available(void);
 size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int compute_units);
 int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream);
 
+/* ------------------------------------------------------------------ llmp.moe.gemm
+ * moe::GroupedGemm / GroupedGemmAvailable / GroupedGemmScratch / RunGroupedGemm of
+ * src/kernels/ggml/moe_cutlass.h:48-76, field for field: the block-scaled NVFP4 grouped GEMM over routed rows
+ * sorted by expert. One group an expert e: D_e[M_e, n] = A_e[M_e, k] B_e[n, k]^T, F32 accumulation, D BF16.
+ * A holds every routed row: expert e's rows are rows offsets[e] .. offsets[e + 1] of the codes (E2M1, k / 2 bytes
+ * a row, element 2i in the low nibble); its UE4M3 scales (one per 16 elements) lie in the atoms of
+ * moe_cutlass.h:42-46 (SfOffset, k / 16 scales a row) in a block of rows starting at sf_rows[e] (a multiple of
+ * 128, as llmp_hip_moe_route's scale_rows). B_e is at weights + e * expert_stride: n rows of codes at
+ * codes_offset, their scales at scales_offset in the atoms of n rows. offsets and sf_rows are device arrays of
+ * groups + 1 entries. k a multiple of 64. The scratch is not used (llmp_hip_grouped_gemm_scratch is 0: may be
+ * null). Values are the format's own: E2M1 times UE4M3 is exact in BF16, the products run on the BF16 matrix
+ * instructions (this device's scaled instructions take E8M0 scales per 32, not UE4M3 per 16). */
+typedef struct llmp_grouped_gemm {
+  int groups;
+  int n;
+  int k;
+  const int32_t* offsets;
+  const int32_t* sf_rows;
+  const void* a;
+  const void* a_scales;
+  const void* weights;
+  uint64_t expert_stride;
+  uint64_t codes_offset;
+  uint64_t scales_offset;
+  void* d;
+  void* scratch;
+} llmp_grouped_gemm;
+int llmp_hip_grouped_gemm_available(void);
+size_t llmp_hip_grouped_gemm_scratch(int groups, int compute_units);
+int llmp_hip_grouped_gemm_run(const llmp_grouped_gemm* gemm, int compute_units, void* stream);
+
 /* ------------------------------------------------------------------ KV cache store
  * llmp.set_rows.quant (SetRowsQuant, src/kernels/ggml/kv_quant.h:28-60,150-158): `rows` rows of k
  * F32 values (k a multiple of 32, x_stride floats apart, 16-byte aligned) stored as rows

@@ -137,6 +137,39 @@ inline int Run(const Gemm& gemm, int sms, void* stream) {
 
 }  // namespace mxfp8
 
+namespace moe {
+
+// src/kernels/ggml/moe_cutlass.h:42-64: the scale atoms' offset and the grouped GEMM's operands, whose layout is
+// the C ABI's field for field.
+constexpr std::uint64_t SfOffset(std::uint64_t row, std::uint64_t block, std::uint64_t blocks) {
+  return ((((row / 128) * (blocks / 4)) + (block / 4)) * 512) + ((row % 32) * 16) + (((row % 128) / 32) * 4) + (block % 4);
+}
+struct GroupedGemm {
+  int groups = 0;
+  int n = 0;
+  int k = 0;
+  const std::int32_t* offsets = nullptr;
+  const std::int32_t* sf_rows = nullptr;
+  const void* a = nullptr;
+  const void* a_scales = nullptr;
+  const void* weights = nullptr;
+  std::uint64_t expert_stride = 0;
+  std::uint64_t codes_offset = 0;
+  std::uint64_t scales_offset = 0;
+  void* d = nullptr;
+  void* scratch = nullptr;
+};
+static_assert(sizeof(GroupedGemm) == sizeof(llmp_grouped_gemm), "GroupedGemm's layout is the C ABI's");
+
+// moe_cutlass.h:66-76; `sms` is the device's compute units here.
+inline bool GroupedGemmAvailable() { return llmp_hip_grouped_gemm_available() != 0; }
+inline std::size_t GroupedGemmScratch(int groups, int sms) { return llmp_hip_grouped_gemm_scratch(groups, sms); }
+inline int RunGroupedGemm(const GroupedGemm& gemm, int sms, void* stream) {
+  return llmp_hip_grouped_gemm_run(reinterpret_cast<const llmp_grouped_gemm*>(&gemm), sms, stream);
+}
+
+}  // namespace moe
+
 // The quantizing KV cache stores (src/kernels/ggml/kv_quant.h:150-192 of the reference): SetRowsQuant's
 // two-dimensional case, SetRowsQuantGroup over two to sixteen of them, RopeSetRowsQuant.
 namespace kv {
@@ -454,6 +487,8 @@ inline std::vector<Implementation> Implementations() {
       {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"}, "llmp.vecq.glu's launches", "ggml.mul_mat");
   add("llmp.moe.router", "route.softmax_top_k", {"f32"}, {1, any, 1, 1}, Rung::kNative, 0, {"llmp_hip_moe_router"},
       "a wave a token; up to 1024 experts, 64 picks");
+  add("llmp.moe.experts.cutlass", "mul_mat_id", {"nvfp4"}, {1, any, 64, 1}, Rung::kOnChipDecode, kBf16Mma,
+      {"llmp_hip_moe_route", "llmp_hip_grouped_gemm_run"}, "NVFP4 operands decoded to BF16 (exact), 64 x 64 tiles walked by a fixed grid");
   add("llmp.moe.combine", "fused.moe_combine", {"f32"}, {1, any, 4, 1}, Rung::kNative, 0, {"llmp_hip_moe_combine"},
       "ordered float sum over the slots");
   // MXFP8 (plan_step.h, mxfp8_cutlass.h): the reference's names, "cutlass" included, since plans carry them.

@@ -42,6 +42,13 @@ class Mxfp8Gemm(C.Structure):
                 ("scratch", C.c_void_p)]
 
 
+class GroupedGemm(C.Structure):
+    """llmp_grouped_gemm: moe::GroupedGemm of src/kernels/ggml/moe_cutlass.h:48-64 of the reference."""
+    _fields_ = [("groups", C.c_int), ("n", C.c_int), ("k", C.c_int), ("offsets", C.c_void_p), ("sf_rows", C.c_void_p),
+                ("a", C.c_void_p), ("a_scales", C.c_void_p), ("weights", C.c_void_p), ("expert_stride", C.c_uint64),
+                ("codes_offset", C.c_uint64), ("scales_offset", C.c_uint64), ("d", C.c_void_p), ("scratch", C.c_void_p)]
+
+
 class Exl3Weights(C.Structure):
     """llmp_exl3_weights: src/kernels/exl3/validate.h:84-96 of the reference, plus the codebook."""
     _fields_ = [("trellis", C.c_void_p), ("suh", C.c_void_p), ("svh", C.c_void_p), ("k", C.c_int), ("n", C.c_int),
@@ -118,6 +125,9 @@ SYMBOLS = {
     "llmp_hip_mxfp8_gemm_available": (_int, []),
     "llmp_hip_mxfp8_gemm_scratch": (C.c_size_t, [C.POINTER(Mxfp8Gemm), _int]),
     "llmp_hip_mxfp8_gemm_run": (_int, [C.POINTER(Mxfp8Gemm), _int, _vp]),
+    "llmp_hip_grouped_gemm_available": (_int, []),
+    "llmp_hip_grouped_gemm_scratch": (C.c_size_t, [_int, _int]),
+    "llmp_hip_grouped_gemm_run": (_int, [C.POINTER(GroupedGemm), _int, _vp]),
     "llmp_hip_exl3_reconstruct": (_int, [C.POINTER(Exl3Weights), _vp, _int, _int, _vp]),
     "llmp_hip_exl3_hadamard": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),

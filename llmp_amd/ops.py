@@ -267,6 +267,24 @@ def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWI
     return moe_combine(y, weights, route.position), ids, weights
 
 
+def moe_gemm(a_codes, a_scales, offsets, sf_rows, weights, expert_stride, codes_offset, scales_offset, n, k, out=None):
+    """llmp.moe.gemm (RunGroupedGemm, src/kernels/ggml/moe_cutlass.h:48-76 of the reference): routed rows sorted
+    by expert, NVFP4 codes uint8 [rows, k / 2] with UE4M3 scales in atoms, times each expert's n rows of the
+    same encoding inside `weights`; offsets and sf_rows int32 [groups + 1]. Returns bfloat16 [rows, n]."""
+    lib = _lib.load()
+    rows = a_codes.shape[0]
+    if out is None:
+        out = torch.empty((rows, n), dtype=torch.bfloat16, device=a_codes.device)
+    g = _lib.GroupedGemm()
+    g.groups, g.n, g.k = offsets.numel() - 1, n, k
+    g.offsets, g.sf_rows, g.a, g.a_scales, g.weights = (offsets.data_ptr(), sf_rows.data_ptr(), a_codes.data_ptr(),
+                                                        a_scales.data_ptr(), weights.data_ptr())
+    g.expert_stride, g.codes_offset, g.scales_offset = expert_stride, codes_offset, scales_offset
+    g.d, g.scratch = out.data_ptr(), None
+    _lib.check(lib.llmp_hip_grouped_gemm_run(C.byref(g), lib.llmp_hip_compute_units(), _stream()))
+    return out
+
+
 def mxfp8_scale_bytes(rows, k):
     """SwizzledScaleBytes: src/kernels/ggml/mxfp8_cutlass.h:53-57 of the reference."""
     return (rows + 127) // 128 * 128 * (k // 32)

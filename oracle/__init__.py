@@ -279,6 +279,38 @@ def mxfp8_gemv(codes, scales, x):
     return y
 
 
+def nvfp4_values(codes, scales, rows, k, scale_row0=0):
+    """The values of `rows` rows of NVFP4: E2M1 codes (uint8 [rows, k / 2], element 2i in byte i's low nibble) times
+    the UE4M3 scale of their 16-element block, read from the 128-row by 4-scale atoms of
+    src/kernels/ggml/moe_cutlass.h:42-46 of the reference (orc_scale_atom_offset) at row scale_row0 + r."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint8).reshape(rows, k // 2)
+    e2m1 = np.array([lib.orc_e2m1_to_f32(c) for c in range(16)], dtype=np.float64)
+    ue4m3 = np.array([lib.orc_ue4m3_to_f32(c) for c in range(256)], dtype=np.float64)
+    values = np.empty((rows, k), dtype=np.float64)
+    values[:, 0::2] = e2m1[codes & 15]
+    values[:, 1::2] = e2m1[codes >> 4]
+    blocks = k // 16
+    at = np.array([[lib.orc_scale_atom_offset(scale_row0 + r, b, blocks) for b in range(blocks)] for r in range(rows)],
+                  dtype=np.int64).reshape(rows, blocks)
+    return values * np.repeat(ue4m3[np.asarray(scales, dtype=np.uint8)[at]], 16, axis=1)
+
+
+def grouped_nvfp4_gemm(a_codes, a_scales, offsets, sf_rows, b_codes, b_scales, n, k):
+    """llmp.moe.gemm's definition (src/kernels/ggml/moe_cutlass.h:12-27 of the reference): group e multiplies rows
+    offsets[e] .. offsets[e + 1] of A (scales in a block of rows from sf_rows[e]) by expert e's n rows; b_codes[e]
+    and b_scales[e] are that expert's codes and atoms. Float64 sums of the decoded values: [rows, n]."""
+    rows = int(offsets[-1])
+    out = np.zeros((rows, n), dtype=np.float64)
+    for e in range(len(offsets) - 1):
+        first, count = int(offsets[e]), int(offsets[e + 1] - offsets[e])
+        if count == 0:
+            continue
+        a = nvfp4_values(np.asarray(a_codes)[first:first + count], a_scales, count, k, int(sf_rows[e]))
+        b = nvfp4_values(b_codes[e], b_scales[e], n, k)
+        out[first:first + count] = a @ b.T
+    return out
+
+
 def route(logits, used, normalize=True, scale=1.0):
     logits = np.ascontiguousarray(logits, dtype=np.float32)
     tokens, experts = logits.shape

@@ -163,7 +163,7 @@ void RegistryChecks() {
   // decode/implementations.h:7-13, exl3/implementations.h:8-31).
   for (const char* name : {"llmp.q8_1", "llmp.vecq.dense", "llmp.vecq.glu", "llmp.vecq.experts", "llmp.vecq.experts_glu", "llmp.vecq.grouped",
                            "ggml.mul_mat.mmvq", "ggml.mul_mat_glu.mmvq_fused", "llmp.mxfp8.mul_mat_vec", "llmp.mxfp8.quantize",
-                           "llmp.mxfp8.swizzle", "llmp.mxfp8.gemm.cutlass", "llmp.moe.router", "llmp.decode.vector.nvfp4.atoms",
+                           "llmp.mxfp8.swizzle", "llmp.mxfp8.gemm.cutlass", "llmp.moe.router", "llmp.moe.experts.cutlass", "llmp.decode.vector.nvfp4.atoms",
                            "llmp.decode.vector_glu.mxfp8.split", "llmp.decode.matrix.bf16.dense", "llmp.decode.grouped.affine.split",
                            "llmp.decode.rows.q8_0.blocks", "exl3.linear.gemv", "exl3.linear.gemm", "exl3.multi_linear.mgemm"})
     EXPECT(names.count(name) == 1);
@@ -221,6 +221,12 @@ void RegistryChecks() {
   EXPECT(hipk::exl3::PackedLinear(linear, fake, sizeof(fake), nullptr) == hipk::KernelFailure::kRejected);
   EXPECT(hipk::LastError().find("rows") != std::string::npos);
   EXPECT(rule("llmp.mxfp8.gemm.cutlass").k_multiple == 128);
+  hipk::ggml::moe::GroupedGemm grouped_gemm;
+  grouped_gemm.groups = 2, grouped_gemm.n = 64, grouped_gemm.k = static_cast<int>(rule("llmp.moe.experts.cutlass").k_multiple) + 32;
+  EXPECT(hipk::ggml::moe::GroupedGemmAvailable() && hipk::ggml::moe::GroupedGemmScratch(2, 256) == 0);
+  EXPECT(hipk::ggml::moe::RunGroupedGemm(grouped_gemm, 256, nullptr) > 0);
+  EXPECT(hipk::LastError().find("64-value") != std::string::npos);
+  static_assert(hipk::ggml::moe::SfOffset(129, 5, 8) == ((1 * 2 + 1) * 512 + 1 * 16 + 0 * 4 + 1), "moe_cutlass.h:42-46");
   hipk::ggml::mxfp8::Gemm g;
   g.m = 128, g.n = 128, g.k = 128 + 32, g.a = g.a_scales = g.b = g.b_scales = fake, g.d = fake;
   EXPECT(hipk::ggml::mxfp8::Run(g, 256, nullptr) > 0);

@@ -188,3 +188,55 @@ def test_sorted_rows_equal_the_routed_product(device):
                                   glu=ops.GLU_SWIGLU).cpu().numpy()
     position = route.position.cpu().numpy()
     assert np.array_equal(sorted_rows[position].view(np.uint32), routed.view(np.uint32))
+
+
+def nvfp4_operand(g, rows, k, padded_rows=None):
+    """Random NVFP4 rows: codes uint8 [rows, k / 2] and UE4M3 scales (finite, moderate) in atoms for padded_rows rows."""
+    padded_rows = (rows + 127) // 128 * 128 if padded_rows is None else padded_rows
+    codes = g.integers(0, 256, size=(rows, k // 2), dtype=np.uint8)
+    scales = g.integers(0x20, 0x50, size=padded_rows * (k // 16), dtype=np.uint8)  # 2^-3 .. 2^3
+    return codes, scales
+
+
+@pytest.mark.parametrize("counts,n,k", [([5, 0, 70, 1, 130], 96, 256), ([64, 64], 64, 64), ([3], 200, 1024),
+                                        ([17, 33, 0, 0, 129, 2, 64, 11], 768, 2048)])
+def test_grouped_nvfp4_gemm_matches_its_definition(device, counts, n, k):
+    """llmp.moe.gemm (RunGroupedGemm, src/kernels/ggml/moe_cutlass.h:48-76 of the reference): experts with no rows,
+    one row, partial tiles of rows and of columns, more rows than a tile; D in BF16 within one rounding of the F64
+    product of the decoded operands (both operands decode exactly; F32 accumulation)."""
+    g = synth.rng(91 + n + k)
+    groups = len(counts)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    sf_rows = np.concatenate([[0], np.cumsum((np.array(counts) + 127) // 128 * 128)]).astype(np.int32)
+    rows = int(offsets[-1])
+    a_codes, a_scales = nvfp4_operand(g, rows, k, padded_rows=int(sf_rows[-1]))
+    codes_bytes, scales_bytes = n * (k // 2), (n + 127) // 128 * 128 * (k // 16)
+    scales_offset = (codes_bytes + 255) // 256 * 256
+    expert_stride = (scales_offset + scales_bytes + 255) // 256 * 256
+    weights = np.zeros((groups, expert_stride), dtype=np.uint8)
+    b_codes, b_scales = [], []
+    for e in range(groups):
+        c, s = nvfp4_operand(g, n, k)
+        weights[e, :codes_bytes] = c.reshape(-1)
+        weights[e, scales_offset:scales_offset + scales_bytes] = s
+        b_codes.append(c)
+        b_scales.append(s)
+    want = oracle.grouped_nvfp4_gemm(a_codes, a_scales, offsets, sf_rows, b_codes, b_scales, n, k)
+    guard = torch.full((rows + 2, n), -7.0, dtype=torch.bfloat16, device=device)
+    got = ops.moe_gemm(dev(a_codes, device), dev(a_scales, device), dev(offsets, device), dev(sf_rows, device),
+                       dev(weights, device), expert_stride, 0, scales_offset, n, k, out=guard[1:rows + 1])
+    got = got.float().cpu().numpy().astype(np.float64)
+    rms = np.sqrt(np.mean(want * want))
+    assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-5 * rms), float(np.max(np.abs(got - want)))
+    assert torch.all(guard[0] == -7.0) and torch.all(guard[rows + 1] == -7.0)  # nothing outside the rows is written
+
+
+def test_grouped_nvfp4_gemm_refusals(device):
+    lib = ops._lib.load()
+    g = ops._lib.GroupedGemm()
+    import ctypes as C
+    assert lib.llmp_hip_grouped_gemm_available() == 1 and lib.llmp_hip_grouped_gemm_scratch(128, 256) == 0
+    g.groups, g.n, g.k = 2, 64, 96
+    assert lib.llmp_hip_grouped_gemm_run(C.byref(g), 256, None) > 0 and b"64-value" in lib.llmp_hip_last_error()
+    g.k = 128
+    assert lib.llmp_hip_grouped_gemm_run(C.byref(g), 256, None) > 0 and b"null" in lib.llmp_hip_last_error()

@@ -964,3 +964,38 @@ def test_rope_neox_against_complex_rotations_and_yarn_closed_forms():
     # Rotations keep a pair's length.
     n0 = np.hypot(x[:, :, :half], x[:, :, half:n_dims])
     np.testing.assert_allclose(np.hypot(got[:, :, :half], got[:, :, half:n_dims]), n0, rtol=1e-6)
+
+
+def test_grouped_nvfp4_values_and_product_by_scalar_loops():
+    """llmp.moe.gemm's operands (src/kernels/ggml/moe_cutlass.h:12-46 of the reference): element 2i in byte i's low
+    nibble, one UE4M3 scale per 16 elements at SfOffset in a block of rows from sf_rows[e]. The vectorised decode
+    against scalar loops over the pinned conversions, known answers (bytes of 0x22 are ones, a scale byte of 0x38 is
+    1.0, 0x40 is 2.0), and the product against explicit dot products."""
+    g = np.random.default_rng(5)
+    k, n = 128, 7
+    offsets = np.array([0, 3, 3, 8], dtype=np.int32)
+    sf_rows = np.array([0, 128, 128, 256], dtype=np.int32)
+    a_codes = g.integers(0, 256, size=(8, k // 2), dtype=np.uint8)
+    a_scales = g.integers(0, 0x7F, size=256 * (k // 16), dtype=np.uint8)
+    b_codes = [g.integers(0, 256, size=(n, k // 2), dtype=np.uint8) for _ in range(3)]
+    b_scales = [g.integers(0, 0x7F, size=128 * (k // 16), dtype=np.uint8) for _ in range(3)]
+    ones = oracle.nvfp4_values(np.full((2, k // 2), 0x22, dtype=np.uint8), np.full(128 * (k // 16), 0x38, dtype=np.uint8), 2, k)
+    assert np.array_equal(ones, np.ones((2, k)))
+    twos = oracle.nvfp4_values(np.full((1, k // 2), 0x22, dtype=np.uint8), np.full(128 * (k // 16), 0x40, dtype=np.uint8), 1, k)
+    assert np.array_equal(twos, 2 * np.ones((1, k)))
+
+    def value(codes, scales, r, j, row0):
+        byte = int(codes[r, j // 2])
+        code = byte >> 4 if j % 2 else byte & 15
+        where = ((((row0 + r) // 128) * ((k // 16) // 4)) + ((j // 16) // 4)) * 512 + (((row0 + r) % 32) * 16) + \
+            ((((row0 + r) % 128) // 32) * 4) + ((j // 16) % 4)  # SfOffset, moe_cutlass.h:42-46
+        return float(oracle.lib.orc_e2m1_to_f32(code)) * float(oracle.lib.orc_ue4m3_to_f32(int(scales[where])))
+
+    got = oracle.grouped_nvfp4_gemm(a_codes, a_scales, offsets, sf_rows, b_codes, b_scales, n, k)
+    for e in (0, 2):
+        for r in range(offsets[e], offsets[e + 1]):
+            local = r - offsets[e]
+            a_row = [value(a_codes[offsets[e]:], a_scales, local, j, int(sf_rows[e])) for j in range(k)]
+            for c in (0, n - 1):
+                b_row = [value(b_codes[e], b_scales[e], c, j, 0) for j in range(k)]
+                assert got[r, c] == pytest.approx(sum(x * y for x, y in zip(a_row, b_row)), rel=1e-12, abs=1e-12)
