@@ -262,6 +262,30 @@ struct GemmArgs {
   int tiles_m, tiles_n;
 };
 
+// Timeline instrumentation for tuning, compiled only with -DLLMP_GEMM_TRACE (never into the library): lane 0 of
+// every wave stores the 100 MHz clock at up to eight points of its tile, eight 64-bit words a wave.
+#ifdef LLMP_GEMM_TRACE
+__device__ unsigned long long* g_gemm_trace = nullptr;
+#define GEMM_TRACE(slot)                                                                                          \
+  do {                                                                                                            \
+    if (g_gemm_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
+      g_gemm_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+// ... or the shader clock's counter (slots 1 and 6: the kernel's cycles between them give its clock).
+#define GEMM_TRACE_CYCLES(slot)                                                                                   \
+  do {                                                                                                            \
+    if (g_gemm_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
+      g_gemm_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (slot)] = __builtin_readcyclecounter(); \
+  } while (0)
+#else
+#define GEMM_TRACE(slot) \
+  do {                   \
+  } while (0)
+#define GEMM_TRACE_CYCLES(slot) \
+  do {                          \
+  } while (0)
+#endif
+
 // LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
 template <int WN>
 struct GemmLds {
@@ -321,6 +345,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) 
   constexpr int kLoadEvery = WN / 2;  // MFMAs between two loads: 8 loads fit 4 WN MFMAs
   static_assert(kLoadsB <= kLoadsA && kLoadsA * kLoadEvery <= 4 * WN, "the loads do not fit a multiply phase");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  GEMM_TRACE(0);  // the wave's start
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -457,11 +482,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) 
       if (i < loads) load(i, 1, 1);
     load_scales(1, 1);
   }
+  GEMM_TRACE_CYCLES(1);  // the first two stages asked for
   AwaitLoads<0>();
   barrier();
+  GEMM_TRACE(2);  // ... and landed, for every wave
   if (group == 1) barrier();
   int stage_b = 0;  // step s's weight stage, s % 3
   for (int step = 0; step < steps; ++step) {
+    if (step == 1) GEMM_TRACE(3);
+    if (step == steps / 2) GEMM_TRACE(4);
     read(step & 1, stage_b);
     // Group 1: activations step + 1, asked for while multiplying step - 1, have landed.
     if (group == 1) AwaitLoads<0>();
@@ -480,8 +509,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) 
     barrier();
     if (++stage_b == kRingB) stage_b = 0;
   }
+  GEMM_TRACE(5);  // the last step multiplied
   if (group == 0) barrier();
   AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
+  GEMM_TRACE_CYCLES(6);
 
   // acc[i][j][q] = D[m0 + wm 64 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]
 #pragma unroll
@@ -504,6 +535,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) 
       }
     }
   }
+  GEMM_TRACE(7);  // the tile's stores queued
 }
 
 template <int WN>
@@ -651,3 +683,10 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
   const int status = best == 192 ? LaunchGemm<6>(a, on) : LaunchGemm<4>(a, on);
   return status;  // negative: the launch failed after the checks (the caller's fault path)
 }
+
+#ifdef LLMP_GEMM_TRACE
+// The tuning build's switch: where the GEMM's waves put their timestamps (device memory), or null.
+extern "C" int llmp_hip_gemm_trace_set(unsigned long long* buffer) {
+  return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(llmp_hip::g_gemm_trace), &buffer, sizeof(buffer)));
+}
+#endif

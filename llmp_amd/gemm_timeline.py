@@ -1,0 +1,51 @@
+"""The MXFP8 GEMM's tile timeline: when a workgroup's waves start, have their first stages, pass steps 1 and 16,
+finish the last step and queue their stores, and the shader clock meanwhile. Needs the instrumented build
+(`make -C llmp_amd/csrc trace`).
+
+    python -m llmp_amd.gemm_timeline"""
+import ctypes as C, os, sys
+import numpy as np, torch
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from llmp_amd import _lib
+_lib.SO_PATH = os.path.join(ROOT, "llmp_amd", "lib", "libllmp_hip_trace.so")
+from llmp_amd import ops
+lib = _lib.load()
+lib.llmp_hip_gemm_trace_set.argtypes = [C.c_void_p]
+dev = torch.device("cuda:0")
+m, n, k = 2048, 12288, 4096
+g = torch.Generator().manual_seed(3)
+a = torch.randn((m, k), generator=g).to(dev).to(torch.bfloat16)
+w = (torch.randn((n, k), generator=g) * 0.02).to(dev)
+ac, asc = ops.mxfp8_quantize(a); wc, wsc = ops.mxfp8_quantize(w)
+d = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+for _ in range(5): ops.mxfp8_gemm(ac, asc, wc, wsc, out=d)
+torch.cuda.synchronize()
+b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+b.record()
+for _ in range(20): ops.mxfp8_gemm(ac, asc, wc, wsc, out=d)
+e.record(); torch.cuda.synchronize()
+print(f"gemm {b.elapsed_time(e) / 20 * 1e3:.1f} us (untraced)")
+trace = torch.zeros(512 * 8 * 8, dtype=torch.int64, device=dev)
+assert lib.llmp_hip_gemm_trace_set(trace.data_ptr()) == 0
+for r in range(3):
+    trace.zero_(); torch.cuda.synchronize()
+    ops.mxfp8_gemm(ac, asc, wc, wsc, out=d); torch.cuda.synchronize()
+tr = trace.cpu().numpy().reshape(-1, 8).astype(np.float64)
+lib.llmp_hip_gemm_trace_set(None)
+t0 = tr[:, 0].min()
+names = ["start", "(cycle counter)", "first stages landed", "step 1", "step 16", "last step done", "(cycle counter)", "stores queued"]
+order = np.argsort(tr[:, 0])
+first_round = tr[:, 0] < t0 + 100 * 5.0
+print("waves in the first round:", first_round.sum(), "second:", (~first_round).sum())
+for label, sel in (("first round", first_round), ("second round", ~first_round)):
+    print(label)
+    for j, nm in enumerate(names):
+        if j in (1, 6): continue
+        rel = (tr[sel, j] - t0) / 100
+        print(f"  {nm:22s} min {rel.min():7.2f} median {np.median(rel):7.2f} max {rel.max():7.2f}")
+    per = tr[sel]
+    print(f"  per wave: start->landed {np.median(per[:,2]-per[:,0])/100:.2f}  landed->step1 {np.median(per[:,3]-per[:,2])/100:.2f}  step1->step16 {np.median(per[:,4]-per[:,3])/100:.2f} (15 steps)  step16->last {np.median(per[:,5]-per[:,4])/100:.2f} (16 steps)  last step->stores queued {np.median(per[:,7]-per[:,5])/100:.2f}")
+cyc = tr[:, 6] - tr[:, 1]; us = (tr[:, 5] - tr[:, 2]) / 100
+print("shader cycles between slot 1 and 6: median %.0f; us between 2 and 5: %.2f -> clock about %.2f GHz" % (np.median(cyc), np.median(us), np.median(cyc) / np.median(us) / 1e3))
+print("launch by stamps: %.1f us" % ((tr[:, 7].max() - t0) / 100))
