@@ -1,31 +1,40 @@
-// llmp.vecq over Q4_K weights for 2 to 16 tokens a pass: the sub-block dot products on the
-// int8 matrix cores.
+// llmp.vecq over Q4_K and Q8_0 weights for several tokens a pass: the dot products of the
+// 32-value sub-blocks on the matrix cores.
 //
-// v_mfma_i32_16x16x32_i8 multiplies one 32-value sub-block of 16 weight rows with the same
-// sub-block of 16 tokens: the instruction's K is a Q4_K sub-block, so every product comes out
-// as the int32 sum the scalar kernel's eight v_dot4 give, for 256 (token, row) pairs at once.
-// What is left per sub-block is the scaling, in floats, and it is done with exactly the
-// operations of the one-token kernel (vecq_flat.hip) in exactly its order: per super-block
-//   main = fma(float(prod_g), sc_g * d8_g, main), g = 0 .. 7;  mins = m_0 * ds8_0, then
-//   fma(m_g, ds8_g, mins);  out = fma(d, main, -(dmin * mins))
-// and the super-blocks of a row are added in the tree that kernel's wave shuffles form
-// (aligned pairs, then pairs of pairs, ...), so a (token, row) value is bit for bit the
-// one-token product's (src/kernels/ggml/vecq.cu:1150-1166 of the reference asks for that).
+// Q4_K (the first half of this file). A weight of sub-block g of a super-block is
+// d * sc_g * q - dmin * m_g with q in 0 .. 15 and sc_g, m_g in 0 .. 63. sc_g * q is an integer
+// below 1024 and a Q8_1 code an integer of 8 bits: both are exact in F16, their products and
+// the sum of a sub-block's 32 products are integers below 2^24, exact in the F32 accumulator
+// of v_mfma_f32_16x16x32_f16 in whatever order it adds. So one instruction gives, for 16 weight
+// rows and 16 tokens, the sub-block's int32 sum already multiplied by the row's 6-bit scale
+// and already a float; what is left a (token, row, sub-block) is one fma by the token's block
+// scale d8:
+//   main = P_0 * d8_0, then fma(P_g, d8_g, main), g = 1 .. 7;  out = fma(main, d, out)
+// over a row's super-blocks in order. The minimums' part, sum over g of (dmin * m_g) *
+// (d8_g * sum of the token's codes), is a plain product of a 16 x 8 by an 8 x 16 matrix a
+// super-block: two v_mfma_f32_16x16x4_f32 into an accumulator of its own, subtracted at the
+// end. A (token, row) value depends on nothing but its own token and row (a column of the
+// instruction's result only on its own column of the operand), whatever else the pass holds.
 //
-// A lane of the instruction's result holds one weight row (lane % 16) and four tokens
-// (4 (lane / 16) + q): the weights are the second operand. A wave owns 16 rows (of both
-// matrices with a GLU) and half of K; the two waves of a tile split K at the largest power of
-// two below the row's super-blocks, which is the top node of the tree, and meet in LDS. A
-// workgroup is eight waves, four tiles (rows of up to eight super-blocks: eight tiles, a wave
-// all of K). Weights come straight from global memory into the
-// operand layout (a lane reads its row's header and, per pair of sub-blocks, the eight code
-// bytes of its K group), three super-blocks deep; the tokens' Q8_1 codes and scales are staged
-// in LDS once a workgroup, in the first operand's layout:
-//   codes   [super-block][pair of sub-blocks][K group][token] 16 bytes: the eight codes of
-//           the K group in sub-block 2 p, then in 2 p + 1 (a lane's read is its 16 bytes of a
-//           contiguous 1 KB);
-//   scales  [super-block][token][pair] 4 floats: d8 of 2 p and 2 p + 1, d8 * sum(codes) of
-//           2 p and 2 p + 1.
+// The weights are the instruction's first operand (a lane holds row lane % 16 and eight
+// consecutive values, K group lane / 16, of the sub-block), the tokens its second; a lane of the
+// result holds token lane % 16 and rows 4 (lane / 16) + q. A lane reads its row's header and
+// the 32 bytes of one pair of sub-blocks straight from global memory, three super-blocks deep,
+// and the row's four lanes exchange them into K groups (Transpose); a nibble becomes F16 by
+// or-ing it under 0x6400 (1024 + q, or 1024 + 16 q for a high nibble in place) and one packed
+// fma by the sub-block's scale takes the 1024 off and multiplies: (1024 + q) * sc - 1024 * sc,
+// exact. The row scales d reach the result's layout by one more small product (the column d
+// times a row of ones).
+//
+// The tokens' Q8_1 blocks are staged in LDS once a pass and workgroup, in operand layout:
+//   codes  [super-block][sub-block][token group][K group][token] 16 bytes: eight codes as F16;
+//   d8     [super-block][token group][token] 8 floats, sub-block g at g;
+//   ds8    the same, d8_g * sum(codes) of sub-block g at 2 (g % 4) + g / 4 (a lane reads the
+//          pair of its K group for the two small products).
+// A pass takes up to TG groups of MT tokens (MT 16; 8 or 4 with one group, for rows so long
+// that sixteen tokens do not fit), the weights prepared once for all of them. A wave owns 16
+// rows (of both matrices with a GLU) and all of K (rows of up to eight super-blocks) or one
+// half of it (two waves a tile, meeting in LDS).
 
 #include <hip/hip_runtime.h>
 
@@ -38,19 +47,44 @@ namespace {
 
 constexpr int kMmaGroup = 512;
 constexpr int kMmaWaves = kMmaGroup / kWave;
-constexpr int kMmaTokens = 16;                       // a pass
+constexpr int kMmaTokens = 16;                       // a token group: the instruction's columns
 constexpr int kTilesGroup = kMmaWaves / 2;           // row tiles a workgroup: two waves a tile
 constexpr int kWholeRow = 8;                         // super-blocks a row up to which a wave takes all of K
-constexpr int kCodesSb = 4 * kMmaTokens * 4 * 16;    // 4096 bytes of codes a super-block
-constexpr int kScalesSb = kMmaTokens * 4 * 16;       // 1024 bytes of scales a super-block
 constexpr int kPartialBytes = kMmaWaves * 2 * kWave * 16;  // a wave's four floats a lane and matrix
 constexpr size_t kMmaLdsLimit = 160 * 1024 - 2048;
 
-typedef int V4i __attribute__((ext_vector_type(4)));
+// Timeline instrumentation for tuning, compiled only into a build with -DLLMP_MMA_TRACE (never the
+// library's): lane 0 of every wave stores the 100 MHz clock at up to sixteen points of the Q4_K kernel.
+#ifdef LLMP_MMA_TRACE
+__device__ unsigned long long* g_mma_trace = nullptr;
+// The stamps wait in LDS until the wave ends: a store to global memory at the point itself would wait for the
+// pointer's load behind every weight load in flight, and the wave with it.
+#define MMA_TRACE_AREA __shared__ unsigned long long trace_area[kMmaWaves][16]
+#define MMA_TRACE(slot)                                                                          \
+  do {                                                                                           \
+    if ((threadIdx.x & 63) == 0 && (slot) < 16) trace_area[threadIdx.x / 64][slot] = wall_clock64(); \
+  } while (0)
+#define MMA_TRACE_DUMP                                                                                          \
+  do {                                                                                                          \
+    trace_area[threadIdx.x / 64][15] = wall_clock64();                                                          \
+    if (g_mma_trace != nullptr && (threadIdx.x & 63) < 16)                                                      \
+      g_mma_trace[((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * kMmaWaves + threadIdx.x / 64) * 16 + \
+                  (threadIdx.x & 63)] = trace_area[threadIdx.x / 64][threadIdx.x & 63];                        \
+  } while (0)
+#else
+#define MMA_TRACE_AREA
+#define MMA_TRACE(slot) \
+  do {                  \
+  } while (0)
+#define MMA_TRACE_DUMP \
+  do {                 \
+  } while (0)
+#endif
 
-__device__ __forceinline__ float ByteOf(uint32_t word, int byte) {
-  return static_cast<float>((word >> (8 * byte)) & 0xFFu);  // v_cvt_f32_ubyteN
-}
+typedef int V4i __attribute__((ext_vector_type(4)));
+typedef float V4f __attribute__((ext_vector_type(4)));
+typedef _Float16 H2 __attribute__((ext_vector_type(2)));
+typedef _Float16 H8 __attribute__((ext_vector_type(8)));
 
 // A lane's part of one super-block of its weight row: the header and, for each pair of
 // sub-blocks, the eight code bytes of its K group (low nibbles sub-block 2 p, high 2 p + 1).
@@ -117,9 +151,347 @@ __device__ __forceinline__ int64_t Pack(uint32_t lo, uint32_t hi) {
   return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-// Sums of a row's super-blocks in the order of the one-token kernel's shuffle tree: aligned
-// pairs first, then pairs of pairs, .... The kernel adds each aligned group of four itself
-// (Quad); the groups of four then go through a binary counter's carries, which builds the
+// Two F16 from two bytes of `word` (each below 0x64's reach: the bytes go under 0x64, which
+// makes 1024 + byte): `places` names the byte of the low and of the high half.
+constexpr uint32_t kHalfHigh = 0x64646464u;
+__device__ __forceinline__ H2 Biased(uint32_t word, uint32_t places) {
+  return __builtin_bit_cast(H2, __builtin_amdgcn_perm(kHalfHigh, word, places));
+}
+constexpr uint32_t kBytes01 = 0x04010400u, kBytes23 = 0x04030402u;
+
+__device__ __forceinline__ H2 Both(float v) {
+  const _Float16 h = static_cast<_Float16>(v);
+  return H2{h, h};
+}
+
+// The layout of a pass's staged tokens.
+template <int TG, int MT>
+struct Staged {
+  static constexpr int kCodesSb = 8 * TG * 4 * MT * 16;  // bytes of codes a super-block
+  static constexpr int kCodesBlock = TG * 4 * MT * 16;   // a sub-block of it
+  static constexpr int kCodesGroup = 4 * MT * 16;        // a token group of that
+  static constexpr int kScalesSb = TG * MT * 32;         // bytes of d8 (and of ds8) a super-block
+  static constexpr size_t Bytes(int nsb) { return static_cast<size_t>(nsb) * (kCodesSb + 2 * kScalesSb); }
+};
+
+// One super-block of one matrix times the staged tokens: this lane's token of every group, rows
+// 4 (lane / 16) + q. `codes`, `d8`, `ds8`: this lane's places in the super-block's staged
+// tokens; `groups`: the token groups the pass holds.
+template <int TG, int MT>
+__device__ __forceinline__ void DotPart(const RowPart& loaded, int kg, const uint8_t* codes, const uint8_t* d8,
+                                        const uint8_t* ds8, int groups, V4f (&out)[TG], V4f (&mins)[TG]) {
+  using L = Staged<TG, MT>;
+  RowPart part = loaded;
+  Transpose(part);
+  const Header h = Decode(part.header);
+  const V4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  // The minimums of sub-blocks kg and 4 + kg, and the row scales in the result's layout.
+  const float m0 = h.dmin * static_cast<float>((h.mn[0] >> (8 * kg)) & 0xFFu);
+  const float m1 = h.dmin * static_cast<float>((h.mn[1] >> (8 * kg)) & 0xFFu);
+  const V4f d_rows = __builtin_amdgcn_mfma_f32_16x16x4f32(kg == 0 ? h.d : 0.0f, 1.0f, zero, 0, 0, 0);
+#pragma unroll
+  for (int tg = 0; tg < TG; ++tg) {
+    if (tg < groups) {
+      const float2 s = *reinterpret_cast<const float2*>(ds8 + tg * MT * 32);
+      mins[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m0, s.x, mins[tg], 0, 0, 0);
+      mins[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m1, s.y, mins[tg], 0, 0, 0);
+    }
+  }
+  V4f main[TG];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    // 1024 + sc in both halves, less 1024: the scale of sub-block 2 p, then of 2 p + 1.
+    const uint32_t word = h.sc[p >> 1];
+    const uint32_t place_lo = 2 * (p & 1), place_hi = 2 * (p & 1) + 1;
+    const H2 sc_lo = Biased(word, 0x04000400u | place_lo | (place_lo << 16)) - Both(1024.0f);
+    const H2 sc_hi = Biased(word, 0x04000400u | place_hi | (place_hi << 16)) - Both(1024.0f);
+    const H2 off_lo = sc_lo * Both(-1024.0f);
+    const H2 by_hi = sc_hi * Both(0.0625f);  // a high nibble in place is 16 q
+    const H2 off_hi = sc_hi * Both(-64.0f);
+    H2 lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t w = i == 0 ? part.q[p].x : part.q[p].y;
+      const uint32_t low = w & 0x0F0F0F0Fu, high = w & 0xF0F0F0F0u;
+      lo[2 * i] = __builtin_elementwise_fma(Biased(low, kBytes01), sc_lo, off_lo);
+      lo[2 * i + 1] = __builtin_elementwise_fma(Biased(low, kBytes23), sc_lo, off_lo);
+      hi[2 * i] = __builtin_elementwise_fma(Biased(high, kBytes01), by_hi, off_hi);
+      hi[2 * i + 1] = __builtin_elementwise_fma(Biased(high, kBytes23), by_hi, off_hi);
+    }
+    const H8 w_lo = __builtin_shufflevector(__builtin_shufflevector(lo[0], lo[1], 0, 1, 2, 3),
+                                            __builtin_shufflevector(lo[2], lo[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+    const H8 w_hi = __builtin_shufflevector(__builtin_shufflevector(hi[0], hi[1], 0, 1, 2, 3),
+                                            __builtin_shufflevector(hi[2], hi[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+    for (int tg = 0; tg < TG; ++tg) {
+      if (tg < groups) {
+        const H8 t_lo = *reinterpret_cast<const H8*>(codes + (2 * p) * L::kCodesBlock + tg * L::kCodesGroup);
+        const H8 t_hi = *reinterpret_cast<const H8*>(codes + (2 * p + 1) * L::kCodesBlock + tg * L::kCodesGroup);
+        const V4f p_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, t_lo, zero, 0, 0, 0);
+        const V4f p_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, t_hi, zero, 0, 0, 0);
+        const float2 s = *reinterpret_cast<const float2*>(d8 + tg * MT * 32 + p * 8);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          main[tg][q] = p == 0 ? p_lo[q] * s.x : fmaf(p_lo[q], s.x, main[tg][q]);
+          main[tg][q] = fmaf(p_hi[q], s.y, main[tg][q]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int tg = 0; tg < TG; ++tg) {
+    if (tg < groups) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) out[tg][q] = fmaf(main[tg][q], d_rows[q], out[tg][q]);
+    }
+  }
+}
+
+// Stages `staged` tokens' Q8_1 rows (one thread a block) into the operand layout; tokens past
+// the pass's `m` repeat its last (their columns are computed and dropped). `row_of(j)`: token
+// j's row of Q8_1 blocks.
+template <int TG, int MT, class RowOf>
+__device__ __forceinline__ void StageTokens(RowOf row_of, int m, int staged, int blocks, uint8_t* codes, uint8_t* d8,
+                                            uint8_t* ds8) {
+  using L = Staged<TG, MT>;
+  for (int index = threadIdx.x; index < staged * blocks; index += kMmaGroup) {
+    const int t = index / blocks, b = index - t * blocks;
+    const int tg = t / MT, token = t - tg * MT;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(min(t, m - 1)) + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+    const int sb = b >> 3, g = b & 7;
+    uint8_t* to = codes + sb * L::kCodesSb + g * L::kCodesBlock + tg * L::kCodesGroup + token * 16;
+#pragma unroll
+    for (int kg = 0; kg < 4; ++kg) {
+      // A code plus 128 is a byte: 1024 + 128 + code under 0x64, less 1152.
+      const uint32_t a = w[1 + 2 * kg] ^ 0x80808080u, c = w[2 + 2 * kg] ^ 0x80808080u;
+      const H2 h0 = Biased(a, kBytes01) - Both(1152.0f), h1 = Biased(a, kBytes23) - Both(1152.0f);
+      const H2 h2 = Biased(c, kBytes01) - Both(1152.0f), h3 = Biased(c, kBytes23) - Both(1152.0f);
+      U32x4 packed;
+      packed.x = __builtin_bit_cast(uint32_t, h0), packed.y = __builtin_bit_cast(uint32_t, h1);
+      packed.z = __builtin_bit_cast(uint32_t, h2), packed.w = __builtin_bit_cast(uint32_t, h3);
+      *reinterpret_cast<U32x4*>(to + kg * MT * 16) = packed;
+    }
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum = Dot4(0x01010101, static_cast<int>(w[1 + i]), sum);
+    const float scale = HalfBitsToFloat(w[0] & 0xFFFFu);
+    const int at = sb * L::kScalesSb + (tg * MT + token) * 32;
+    *reinterpret_cast<float*>(d8 + at + g * 4) = scale;
+    *reinterpret_cast<float*>(ds8 + at + (2 * (g & 3) + (g >> 2)) * 4) = scale * static_cast<float>(sum);
+  }
+}
+
+// grid (workgroups, slots); LDS: codes, d8, ds8, the waves' partial sums.
+template <bool kGlu, int TG, int MT>
+__global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
+  using L = Staged<TG, MT>;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int pairs[kMaxPairs];
+  __shared__ int count;
+
+  MMA_TRACE_AREA;
+  MMA_TRACE(0);  // the wave's start
+  const llmp_vecq_desc& d = a.d;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int nsb = d.ncols_x / 256;
+  uint8_t* codes = lds;
+  uint8_t* d8 = lds + nsb * L::kCodesSb;
+  uint8_t* ds8 = d8 + nsb * L::kScalesSb;
+  float4* partial = reinterpret_cast<float4*>(ds8 + nsb * L::kScalesSb);
+
+  int expert = blockIdx.y;
+  int sorted_first = 0;
+  if (a.offsets != nullptr) {
+    sorted_first = a.offsets[expert];
+    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+    __syncthreads();
+  } else {
+    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
+  }
+  const int n = count;
+  if (n == 0) return;  // uniform over the workgroup
+  const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
+  auto pair_at = [&](int i) { return a.offsets != nullptr ? (sorted_first + i) << 8 : pairs[i]; };
+
+  // This wave's part of K. Rows of up to eight super-blocks: all of it, a tile a wave (too few
+  // steps to be worth two waves and their meeting). Longer rows: a half.
+  const bool whole = nsb <= kWholeRow;
+  const int half = whole ? 0 : wave & 1;
+  const int first = half == 0 ? 0 : (nsb + 1) / 2;
+  const int last = whole || half == 1 ? nsb : (nsb + 1) / 2;
+  const int row_in_tile = lane & 15, kg = lane >> 4;
+  const int token_in_group = lane & (MT - 1);
+  const int tiles = (d.nrows + 15) / 16;
+  const int tiles_group = whole ? kMmaWaves : kTilesGroup;
+  const int tile_in_group = whole ? wave : wave >> 1;
+  const int groups = (tiles + tiles_group - 1) / tiles_group;
+  const int my_groups = (groups - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+  const int steps = my_groups * (last - first);  // a pass's
+
+  // The fetches run two steps ahead of the products, through the tiles of a pass in order and
+  // round to the pass's first again (the next pass's, or nobody's).
+  const uint8_t* up_row = nullptr;
+  const uint8_t* gate_row = nullptr;
+  int fetch_group = blockIdx.x, fetch_sb = first;
+  auto aim = [&]() {
+    const int row = min((fetch_group * tiles_group + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
+    const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
+    up_row = static_cast<const uint8_t*>(d.w) + at;
+    if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
+  };
+  // The loads are queued here and no later: the compiler would otherwise sink them to their
+  // first use, two steps on, and the wave would wait out the whole memory latency there.
+  auto fetch = [&](RowPart& u, RowPart& g) {
+    u = LoadRowPart(up_row, fetch_sb, kg);
+    if constexpr (kGlu) g = LoadRowPart(gate_row, fetch_sb, kg);
+    __builtin_amdgcn_sched_barrier(0);
+    if (++fetch_sb == last) {
+      fetch_sb = first;
+      fetch_group += gridDim.x;
+      if (fetch_group >= groups) fetch_group = blockIdx.x;
+      aim();
+    }
+  };
+  RowPart u0, u1, u2, g0, g1, g2;
+  aim();
+  fetch(u0, g0);
+  fetch(u1, g1);
+
+  const uint8_t* my_codes = codes + (kg * MT + token_in_group) * 16;
+  const uint8_t* my_d8 = d8 + token_in_group * 32;
+  const uint8_t* my_ds8 = ds8 + token_in_group * 32 + kg * 8;
+
+  for (int p0 = 0; p0 < n; p0 += TG * MT) {
+    const int m = min(TG * MT, n - p0);
+    const int token_groups = (m + MT - 1) / MT;
+    __syncthreads();  // the last pass's readers of the staged tokens
+    auto row_of = [&](int j) {
+      const int pr = pair_at(p0 + j);
+      return static_cast<const uint8_t*>(d.y) +
+             (static_cast<int64_t>(pr >> 8) * d.y_token + static_cast<int64_t>(pr & 0xFF) * d.y_slot) * kQ8Block;
+    };
+    if (p0 == 0) MMA_TRACE(1);  // the first weights asked for, the pairs known
+    StageTokens<TG, MT>(row_of, m, token_groups * MT, d.ncols_x / 32, codes, d8, ds8);
+    __syncthreads();
+    if (p0 == 0) MMA_TRACE(2);  // the first pass's tokens staged
+
+    V4f up_out[TG], up_mins[TG], gate_out[TG], gate_mins[TG];
+    auto clear = [&]() {
+#pragma unroll
+      for (int tg = 0; tg < TG; ++tg) {
+        up_out[tg] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, up_mins[tg] = up_out[tg];
+        gate_out[tg] = up_out[tg], gate_mins[tg] = up_out[tg];
+      }
+    };
+    clear();
+    int group = blockIdx.x, sb = first;
+    // A tile's rows are done: the two halves of K meet (the upper half's sums through LDS),
+    // and the lower half's wave stores.
+    auto finish = [&]() {
+#pragma clang fp contract(off)
+      const int tile = group * tiles_group + tile_in_group;
+      float4* slot = partial + ((wave >> 1) * 2 * TG) * kWave + lane;  // a tile's
+      if (half == 1) {
+#pragma unroll
+        for (int tg = 0; tg < TG; ++tg) {
+          const V4f u = up_out[tg] - up_mins[tg];
+          slot[(2 * tg) * kWave] = make_float4(u[0], u[1], u[2], u[3]);
+          if constexpr (kGlu) {
+            const V4f g = gate_out[tg] - gate_mins[tg];
+            slot[(2 * tg + 1) * kWave] = make_float4(g[0], g[1], g[2], g[3]);
+          }
+        }
+      }
+      if (!whole) __syncthreads();
+      if (half == 0 && tile < tiles) {
+#pragma unroll
+        for (int tg = 0; tg < TG; ++tg) {
+          V4f u = up_out[tg] - up_mins[tg], g = gate_out[tg] - gate_mins[tg];
+          if (!whole) {
+            const float4 x = slot[(2 * tg) * kWave];
+            u[0] += x.x, u[1] += x.y, u[2] += x.z, u[3] += x.w;
+            if constexpr (kGlu) {
+              const float4 y = slot[(2 * tg + 1) * kWave];
+              g[0] += y.x, g[1] += y.y, g[2] += y.z, g[3] += y.w;
+            }
+          }
+          const int t = tg * MT + row_in_tile;  // this lane's token of the group, when the group has it
+          if (row_in_tile < MT && t < m) {
+            const int pr = pair_at(p0 + t);
+            float* dst = d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int row = tile * 16 + 4 * kg + q;
+              if (row < d.nrows) dst[row] = kGlu ? Glu(d.glu, g[q], u[q], d.limit) : u[q];
+            }
+          }
+        }
+      }
+      if (!whole) __syncthreads();  // the partial sums may be overwritten
+      clear();
+    };
+    auto step = [&](const RowPart& u, const RowPart& g) {
+      DotPart<TG, MT>(u, kg, my_codes + sb * L::kCodesSb, my_d8 + sb * L::kScalesSb, my_ds8 + sb * L::kScalesSb,
+                      token_groups, up_out, up_mins);
+      if constexpr (kGlu)
+        DotPart<TG, MT>(g, kg, my_codes + sb * L::kCodesSb, my_d8 + sb * L::kScalesSb, my_ds8 + sb * L::kScalesSb,
+                        token_groups, gate_out, gate_mins);
+      if (++sb == last) {
+        finish();
+        sb = first;
+        group += gridDim.x;
+      }
+    };
+    for (int s = 0; s < steps; s += 3) {
+      fetch(u2, g2);
+      step(u0, g0);
+      if (p0 == 0) MMA_TRACE(3 + s);  // the first pass's first steps
+      if (s + 1 < steps) {
+        fetch(u0, g0);
+        step(u1, g1);
+        if (p0 == 0) MMA_TRACE(4 + s);
+      }
+      if (s + 2 < steps) {
+        fetch(u1, g1);
+        step(u2, g2);
+        if (p0 == 0) MMA_TRACE(5 + s);
+      }
+    }
+    // The next pass starts at the first tile again, with the buffers in their first roles.
+    if (p0 + TG * MT < n && steps % 3 != 0) {
+      fetch_group = blockIdx.x, fetch_sb = first;
+      aim();
+      fetch(u0, g0);
+      fetch(u1, g1);
+    }
+  }
+  MMA_TRACE_DUMP;  // with the wave's end
+}
+
+// ------------------------------------------------------------------ Q8_0
+//
+// The same instruction over Q8_0 blocks: its K is a block, a product the block's int32 sum.
+// The float operations are the one-token kernel's: over a unit of four blocks
+//   v = float(s_0) * (dw_0 * d8_0), then v = fma(float(s_j), dw_j * d8_j, v), j = 1 .. 3,
+// and a row's units are added in that kernel's tree. A tile of 16 rows is taken by four waves,
+// each a quarter of the tree's leaves (the next power of two at or above the row's units, cut in
+// four aligned runs of up to sixteen units), which meet in LDS.
+//
+// A lane reads its row's weights straight into the operand layout: of every pair of blocks
+// (68 bytes, so 4-byte aligned in a row of whole pairs) the eight codes of its K group in the
+// even block lie two bytes into three dwords, those of the odd block in two dwords. The tokens
+// are staged once a workgroup:
+//   codes   [block][K group][token] 8 bytes (a wave's read is a contiguous 512 bytes);
+//   scales  [block][token] F32, a lane reading its four tokens' 16 bytes.
+
+// Sums of a row's units in the order of the one-token kernel's shuffle tree: aligned
+// pairs first, then pairs of pairs, .... The kernel adds each aligned group of four itself;
+// the groups of four then go through a binary counter's carries, which builds the
 // rest of the same tree: l2 holds a finished group of four waiting for its neighbour, l3 one
 // of eight, l4 one of sixteen. Everything is selects on values the same in every lane, so
 // that the levels stay in registers.
@@ -160,260 +532,6 @@ __device__ __forceinline__ void Total(const TreeSum& t, int count, float (&out)[
     out[q] = v;
   }
 }
-
-// One super-block of one matrix times the staged tokens: four tokens of this lane's row.
-// `a`: the tokens' codes as first operands, sub-block by sub-block; `entries[4 q + p]`: token
-// q's four scale floats of pair p (in LDS, read a pair at a time).
-__device__ __forceinline__ void DotPart(const RowPart& loaded, const int64_t (&a)[8], const float4* entries,
-                                        float (&out)[4]) {
-#pragma clang fp contract(off)
-  RowPart part = loaded;
-  Transpose(part);
-  const Header h = Decode(part.header);
-  float main[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  float mins[4];
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const uint32_t q0 = part.q[p].x, q1 = part.q[p].y;
-    const int64_t lo = Pack(q0 & 0x0F0F0F0Fu, q1 & 0x0F0F0F0Fu);
-    const int64_t hi = Pack((q0 >> 4) & 0x0F0F0F0Fu, (q1 >> 4) & 0x0F0F0F0Fu);
-    const V4i zero = {0, 0, 0, 0};
-    const V4i prod0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[2 * p], lo, zero, 0, 0, 0);
-    const V4i prod1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[2 * p + 1], hi, zero, 0, 0, 0);
-    const float sc0 = ByteOf(h.sc[(2 * p) >> 2], (2 * p) & 3);
-    const float sc1 = ByteOf(h.sc[(2 * p + 1) >> 2], (2 * p + 1) & 3);
-    const float m0 = ByteOf(h.mn[(2 * p) >> 2], (2 * p) & 3);
-    const float m1 = ByteOf(h.mn[(2 * p + 1) >> 2], (2 * p + 1) & 3);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 s = entries[4 * q + p];
-      main[q] = fmaf(static_cast<float>(prod0[q]), sc0 * s.x, main[q]);
-      main[q] = fmaf(static_cast<float>(prod1[q]), sc1 * s.y, main[q]);
-      mins[q] = p == 0 ? m0 * s.z : fmaf(m0, s.z, mins[q]);
-      mins[q] = fmaf(m1, s.w, mins[q]);
-    }
-  }
-#pragma unroll
-  for (int q = 0; q < 4; ++q) out[q] = fmaf(h.d, main[q], -(h.dmin * mins[q]));
-}
-
-// Stages `m` tokens' Q8_1 rows (one thread a block) into the operand layout. `row_of(j)`: token
-// j's row of Q8_1 blocks.
-template <class RowOf>
-__device__ __forceinline__ void StageTokens(RowOf row_of, int m, int blocks, uint8_t* codes, uint8_t* scales) {
-  for (int index = threadIdx.x; index < m * blocks; index += kMmaGroup) {
-    const int j = index / blocks, b = index - j * blocks;
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(j) + static_cast<int64_t>(b) * kQ8Block);
-    uint32_t w[9];
-#pragma unroll
-    for (int i = 0; i < 9; ++i) w[i] = src[i];
-    const int sb = b >> 3, g = b & 7;
-    uint8_t* to = codes + sb * kCodesSb + ((g >> 1) * 4 * kMmaTokens + j) * 16 + (g & 1) * 8;
-#pragma unroll
-    for (int kg = 0; kg < 4; ++kg)
-      *reinterpret_cast<uint2*>(to + kg * kMmaTokens * 16) = make_uint2(w[1 + 2 * kg], w[2 + 2 * kg]);
-    int sum = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) sum = Dot4(0x01010101, static_cast<int>(w[1 + i]), sum);
-    const float d8 = HalfBitsToFloat(w[0] & 0xFFFFu);
-    float* entry = reinterpret_cast<float*>(scales + sb * kScalesSb + (j * 4 + (g >> 1)) * 16);
-    entry[g & 1] = d8;
-    entry[2 + (g & 1)] = d8 * static_cast<float>(sum);
-  }
-}
-
-// grid (workgroups, slots); LDS: codes, scales, the waves' partial sums.
-template <bool kGlu>
-__global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  __shared__ int pairs[kMaxPairs];
-  __shared__ int count;
-
-  const llmp_vecq_desc& d = a.d;
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int nsb = d.ncols_x / 256;
-  uint8_t* codes = lds;
-  uint8_t* scales = lds + nsb * kCodesSb;
-  float* partial = reinterpret_cast<float*>(lds + nsb * (kCodesSb + kScalesSb));
-
-  int expert = blockIdx.y;
-  int sorted_first = 0;
-  if (a.offsets != nullptr) {
-    sorted_first = a.offsets[expert];
-    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
-    __syncthreads();
-  } else {
-    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
-  }
-  const int n = count;
-  if (n == 0) return;  // uniform over the workgroup
-  const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
-
-  // This wave's part of K. Rows of up to eight super-blocks: all of it, a tile a wave (too few
-  // steps to be worth two waves and their meeting). Longer rows: a half, split at the top node
-  // of the row's summation tree.
-  const bool whole = nsb <= kWholeRow;
-  int split = 1;
-  while (split * 2 < nsb) split *= 2;
-  const int half = whole ? 0 : wave & 1;
-  const int first = half == 0 ? 0 : split;
-  const int last = whole ? nsb : half == 0 ? min(split, nsb) : nsb;
-  const int row_in_tile = lane & 15, kg = lane >> 4;
-  const int tiles = (d.nrows + 15) / 16;
-  const int tiles_group = whole ? kMmaWaves : kTilesGroup;
-  const int tile_in_group = whole ? wave : wave >> 1;
-  const int groups = (tiles + tiles_group - 1) / tiles_group;
-
-  // This lane's weight rows of the tile its wave takes in a group of tiles (rows past the end
-  // repeat the last, unstored).
-  const uint8_t* up_row = nullptr;
-  const uint8_t* gate_row = nullptr;
-  auto aim = [&](int group) {
-    const int row = min((group * tiles_group + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
-    const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
-    up_row = static_cast<const uint8_t*>(d.w) + at;
-    if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
-  };
-  RowPart u0, u1, u2, u3, g0, g1, g2, g3;  // three are live at a time
-  // The loads of super-block sb, queued here and no later: the compiler would otherwise sink
-  // them to their first use, two steps on, and the wave would wait out the whole memory latency
-  // there. (Past the end the last super-block again: no branch, no copies of what was loaded.)
-  auto fetch = [&](int sb, RowPart& u, RowPart& g) {
-    const int at = min(sb, last - 1);
-    u = LoadRowPart(up_row, at, kg);
-    if constexpr (kGlu) g = LoadRowPart(gate_row, at, kg);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  // A group's first two super-blocks are asked for while the group before it finishes (the
-  // first group's before the tokens are staged).
-  aim(blockIdx.x);
-  fetch(first, u0, g0);
-  fetch(first + 1, u1, g1);
-
-  for (int p0 = 0; p0 < n; p0 += kMmaTokens) {
-    const int m = min(kMmaTokens, n - p0);
-    __syncthreads();  // the last pass's readers of the staged tokens
-    auto row_of = [&](int j) {
-      const int pr = a.offsets != nullptr ? (sorted_first + p0 + j) << 8 : pairs[p0 + j];
-      return static_cast<const uint8_t*>(d.y) +
-             (static_cast<int64_t>(pr >> 8) * d.y_token + static_cast<int64_t>(pr & 0xFF) * d.y_slot) * kQ8Block;
-    };
-    StageTokens(row_of, m, d.ncols_x / 32, codes, scales);
-    __syncthreads();
-
-    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
-      const int tile = group * tiles_group + tile_in_group;
-      TreeSum up_sum{}, gate_sum{};
-      auto step = [&](int sb, const RowPart& u, const RowPart& g, float (&up_out)[4], float (&gate_out)[4]) {
-        int64_t acts[8];
-        const uint8_t* mine = codes + sb * kCodesSb + lane * 16;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          const U32x4 c = *reinterpret_cast<const U32x4*>(mine + p * (kMmaTokens * 4 * 16));
-          acts[2 * p] = Pack(c.x, c.y);
-          acts[2 * p + 1] = Pack(c.z, c.w);
-        }
-        const float4* entries = reinterpret_cast<const float4*>(scales + sb * kScalesSb) + (4 * kg) * 4;
-        DotPart(u, acts, entries, up_out);
-        if constexpr (kGlu) DotPart(g, acts, entries, gate_out);
-      };
-      int quads = 0;
-      if (tile < tiles) {
-        for (int sb = first; sb < last; sb += 4, ++quads) {
-          const int n = min(4, last - sb);
-          // The group's sum as its values come: (x0 + x1) + (x2 + x3), absent ones left out.
-          float up_quad[4], gate_quad[4], up_next[4], gate_next[4];
-          fetch(sb + 2, u2, g2);
-          step(sb, u0, g0, up_quad, gate_quad);
-          if (n >= 2) {
-            fetch(sb + 3, u3, g3);
-            step(sb + 1, u1, g1, up_next, gate_next);
-            Sum4(up_quad, up_next, up_quad);
-            if constexpr (kGlu) Sum4(gate_quad, gate_next, gate_quad);
-          }
-          if (n >= 3) {
-            float up_rest[4], gate_rest[4];
-            fetch(sb + 4, u0, g0);
-            step(sb + 2, u2, g2, up_rest, gate_rest);
-            if (n >= 4) {
-              fetch(sb + 5, u1, g1);
-              step(sb + 3, u3, g3, up_next, gate_next);
-              Sum4(up_rest, up_next, up_rest);
-              if constexpr (kGlu) Sum4(gate_rest, gate_next, gate_rest);
-            }
-            Sum4(up_quad, up_rest, up_quad);
-            if constexpr (kGlu) Sum4(gate_quad, gate_rest, gate_quad);
-          }
-          Push(up_sum, up_quad, quads);
-          if constexpr (kGlu) Push(gate_sum, gate_quad, quads);
-        }
-      }
-      // The next group's (or the next pass's first group's) first loads.
-      {
-        int next = group + static_cast<int>(gridDim.x);
-        if (next >= groups) next = blockIdx.x;
-        aim(next);
-        fetch(first, u0, g0);
-        fetch(first + 1, u1, g1);
-      }
-      // The two halves of K meet: the upper half's totals through LDS.
-      float up_total[4] = {0.0f, 0.0f, 0.0f, 0.0f}, gate_total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      const bool has = tile < tiles && last > first;
-      if (has) {
-        Total(up_sum, quads, up_total);
-        if constexpr (kGlu) Total(gate_sum, quads, gate_total);
-      }
-      float4* slot = reinterpret_cast<float4*>(partial) + (wave * 2) * kWave + lane;
-      if (half == 1) {
-        slot[0] = make_float4(up_total[0], up_total[1], up_total[2], up_total[3]);
-        if constexpr (kGlu) slot[kWave] = make_float4(gate_total[0], gate_total[1], gate_total[2], gate_total[3]);
-      }
-      if (!whole) __syncthreads();
-      if (half == 0 && tile < tiles) {
-#pragma clang fp contract(off)
-        if (!whole && split < nsb) {
-          const float4* other = reinterpret_cast<const float4*>(partial) + ((wave + 1) * 2) * kWave + lane;
-          const float4 u = other[0];
-          up_total[0] += u.x, up_total[1] += u.y, up_total[2] += u.z, up_total[3] += u.w;
-          if constexpr (kGlu) {
-            const float4 g = other[kWave];
-            gate_total[0] += g.x, gate_total[1] += g.y, gate_total[2] += g.z, gate_total[3] += g.w;
-          }
-        }
-        if (tile * 16 + row_in_tile < d.nrows) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int t = 4 * kg + q;
-            if (t < m) {
-              const int pr = a.offsets != nullptr ? (sorted_first + p0 + t) << 8 : pairs[p0 + t];
-              float* dst = d.dst + static_cast<int64_t>(pr >> 8) * d.dst_token + static_cast<int64_t>(pr & 0xFF) * d.dst_slot;
-              dst[tile * 16 + row_in_tile] = kGlu ? Glu(d.glu, gate_total[q], up_total[q], d.limit) : up_total[q];
-            }
-          }
-        }
-      }
-      if (!whole) __syncthreads();  // the partial sums may be overwritten
-    }
-  }
-}
-
-// ------------------------------------------------------------------ Q8_0
-//
-// The same instruction over Q8_0 blocks: its K is a block, a product the block's int32 sum.
-// The float operations are the one-token kernel's: over a unit of four blocks
-//   v = float(s_0) * (dw_0 * d8_0), then v = fma(float(s_j), dw_j * d8_j, v), j = 1 .. 3,
-// and a row's units are added in that kernel's tree. A tile of 16 rows is taken by four waves,
-// each a quarter of the tree's leaves (the next power of two at or above the row's units, cut in
-// four aligned runs of up to sixteen units), which meet in LDS.
-//
-// A lane reads its row's weights straight into the operand layout: of every pair of blocks
-// (68 bytes, so 4-byte aligned in a row of whole pairs) the eight codes of its K group in the
-// even block lie two bytes into three dwords, those of the odd block in two dwords. The tokens
-// are staged once a workgroup:
-//   codes   [block][K group][token] 8 bytes (a wave's read is a contiguous 512 bytes);
-//   scales  [block][token] F32, a lane reading its four tokens' 16 bytes.
 
 constexpr int kQ8CodesBlock = 4 * kMmaTokens * 8;  // 512 bytes of codes a block
 constexpr int kQ8ScalesBlock = kMmaTokens * 4;     // 64 bytes of scales a block
@@ -676,19 +794,51 @@ size_t MmaLdsQ8(int blocks) {
   return static_cast<size_t>(blocks) * (kQ8CodesBlock + kQ8ScalesBlock) + kPartialBytes;
 }
 
-size_t MmaLds(int nsb) { return static_cast<size_t>(nsb) * (kCodesSb + kScalesSb) + kPartialBytes; }
+// The Q4_K kernel's token groups a pass (TG) and tokens a group (MT) for rows of `nsb`
+// super-blocks when a slot brings up to `tokens` tokens: two groups of sixteen where more than
+// sixteen may come and fit, else the smallest group that holds them all, else the largest that
+// fits. 0 groups: not even four tokens fit.
+struct MmaShape {
+  int groups, tokens;
+  size_t lds;
+};
+
+template <int TG, int MT>
+bool Fits(int nsb, MmaShape* shape) {
+  const size_t partial = nsb <= kWholeRow ? 0 : static_cast<size_t>(kTilesGroup) * 2 * TG * kWave * 16;
+  const size_t lds = Staged<TG, MT>::Bytes(nsb) + partial;
+  if (lds > kMmaLdsLimit) return false;
+  *shape = MmaShape{TG, MT, lds};
+  return true;
+}
+
+MmaShape ShapeFor(int nsb, int tokens) {
+  MmaShape shape{0, 0, 0};
+  if (tokens > 16 && Fits<2, 16>(nsb, &shape)) return shape;
+  if (tokens <= 4 && Fits<1, 4>(nsb, &shape)) return shape;
+  if (tokens <= 8 && Fits<1, 8>(nsb, &shape)) return shape;
+  if (Fits<1, 16>(nsb, &shape) || Fits<1, 8>(nsb, &shape) || Fits<1, 4>(nsb, &shape)) return shape;
+  return shape;
+}
 
 int g_mma_compute_units = 0;
 
 }  // namespace
 
-// Q4_K rows whose sixteen staged tokens fit LDS (k up to 7168). Q8_0 rows of whole units of
-// 128 values, up to 64 units (8192 values) as far as they fit LDS, whose rows, matrices and
-// experts start on 4-byte boundaries (a lane reads dwords).
+#ifdef LLMP_MMA_TRACE
+extern "C" int llmp_hip_trace_set_mma(unsigned long long* buffer) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(g_mma_trace), &buffer, sizeof(buffer)) == hipSuccess ? 0 : -1;
+}
+#endif
+
+// Q4_K rows of which at least eight staged tokens fit LDS (k up to 8448; sixteen up to 4096, two
+// groups of sixteen up to 2048). Q8_0 rows of whole units of 128 values, up to 64 units (8192
+// values) as far as they fit LDS, whose rows, matrices and experts start on 4-byte boundaries (a
+// lane reads dwords).
 bool MmaTakes(int type, const llmp_vecq_desc& d) {
   if (type == LLMP_TYPE_Q4_K) {
     const int nsb = d.ncols_x / 256;
-    return nsb >= 1 && MmaLds(nsb) <= kMmaLdsLimit;
+    return nsb >= 1 && ShapeFor(nsb, 8).groups != 0 && ShapeFor(nsb, 8).tokens >= 8;
   }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x < 128 || d.ncols_x % 128 != 0 || d.ncols_x > 8192) return false;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
@@ -697,16 +847,26 @@ bool MmaTakes(int type, const llmp_vecq_desc& d) {
 
 namespace {
 
-template <bool kQ8, bool kGlu>
-void LaunchMmaKernel(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+template <bool kGlu>
+void LaunchMmaQ8(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if constexpr (kQ8) {
-    if (!AllowLds(reinterpret_cast<const void*>(&VecQMmaQ8<kGlu>), static_cast<int>(kMmaLdsLimit), &sized)) return;
-    hipLaunchKernelGGL((VecQMmaQ8<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
-  } else {
-    if (!AllowLds(reinterpret_cast<const void*>(&VecQMma<kGlu>), static_cast<int>(kMmaLdsLimit), &sized)) return;
-    hipLaunchKernelGGL((VecQMma<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
-  }
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQMmaQ8<kGlu>), static_cast<int>(kMmaLdsLimit), &sized)) return;
+  hipLaunchKernelGGL((VecQMmaQ8<kGlu>), grid, dim3(kMmaGroup), lds, stream, a);
+}
+
+template <bool kGlu, int TG, int MT>
+void LaunchMmaQ4K(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+  static bool sized = false;
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQMma<kGlu, TG, MT>), static_cast<int>(kMmaLdsLimit), &sized)) return;
+  hipLaunchKernelGGL((VecQMma<kGlu, TG, MT>), grid, dim3(kMmaGroup), lds, stream, a);
+}
+
+template <bool kGlu>
+void LaunchMmaQ4KShape(const MmaShape& shape, const VecQArgs& a, dim3 grid, hipStream_t stream) {
+  if (shape.groups == 2) return LaunchMmaQ4K<kGlu, 2, 16>(a, grid, shape.lds, stream);
+  if (shape.tokens == 16) return LaunchMmaQ4K<kGlu, 1, 16>(a, grid, shape.lds, stream);
+  if (shape.tokens == 8) return LaunchMmaQ4K<kGlu, 1, 8>(a, grid, shape.lds, stream);
+  return LaunchMmaQ4K<kGlu, 1, 4>(a, grid, shape.lds, stream);
 }
 
 }  // namespace
@@ -715,7 +875,6 @@ void LaunchMma(int type, const VecQArgs& a, hipStream_t stream) {
   const llmp_vecq_desc& d = a.d;
   const bool q8 = type == LLMP_TYPE_Q8_0;
   const int nsb = d.ncols_x / 256;
-  const size_t lds = q8 ? MmaLdsQ8(d.ncols_x / 32) : MmaLds(nsb);
   if (g_mma_compute_units == 0) {
     const int cus = llmp_hip_compute_units();
     g_mma_compute_units = cus > 0 ? cus : 256;
@@ -731,10 +890,15 @@ void LaunchMma(int type, const VecQArgs& a, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
   const bool glu = d.g != nullptr;
   if (q8) {
-    glu ? LaunchMmaKernel<true, true>(a, grid, lds, stream) : LaunchMmaKernel<true, false>(a, grid, lds, stream);
-  } else {
-    glu ? LaunchMmaKernel<false, true>(a, grid, lds, stream) : LaunchMmaKernel<false, false>(a, grid, lds, stream);
+    const size_t lds = MmaLdsQ8(d.ncols_x / 32);
+    glu ? LaunchMmaQ8<true>(a, grid, lds, stream) : LaunchMmaQ8<false>(a, grid, lds, stream);
+    return;
   }
+  // A slot's tokens: a dense or grouped product's own; sorted rows bring any number an expert, a
+  // routed product up to all its pairs.
+  const int tokens = a.offsets != nullptr ? 32 : d.ids != nullptr ? d.used * d.tokens : d.tokens;
+  const MmaShape shape = ShapeFor(nsb, tokens);
+  glu ? LaunchMmaQ4KShape<true>(shape, a, grid, stream) : LaunchMmaQ4KShape<false>(shape, a, grid, stream);
 }
 
 }  // namespace llmp_hip

@@ -170,7 +170,7 @@ def test_sorted_rows_of_many_passes_match_oracle_and_the_routed_product(device, 
     ok, worst = rel_close(routed, want, TOL)
     assert ok, worst
     default = ops.vecq_sorted(t, upd, sq8, route.offsets, hidden, ffn, experts, stride_expert=stride, **kw).cpu().numpy()
-    ok, worst = rel_close(default[position], routed, 1e-5)  # two forms of the same sums: float order only
+    ok, worst = rel_close(default[position], routed, 1e-5, floor=1.0)  # two forms of the same sums: float order only
     assert ok, worst
 
 

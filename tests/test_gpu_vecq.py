@@ -122,7 +122,8 @@ def test_fused_glu_matches_oracle(device, t, glu, tokens):
 @pytest.mark.parametrize("t", [Q8_0, Q4_K])
 @pytest.mark.parametrize("xdtype", ["f32", "bf16"])
 def test_fused_activation_quantization_equals_the_two_step_path(device, t, xdtype):
-    """The in-LDS quantizer is the quantizer kernel's arithmetic: outputs equal bit for bit."""
+    """The in-LDS quantizer is the quantizer kernel's arithmetic: outputs equal the two-step path's through the
+    same (flat) form bit for bit, and its default form's to float rounding."""
     k, n, tokens = 3840, 64, 4
     w = make_weights(t, n, k, 61)
     x = synth.activations(tokens, k, 62)
@@ -133,9 +134,12 @@ def test_fused_activation_quantization_equals_the_two_step_path(device, t, xdtyp
     else:
         xd = dev(x, device)
     q8 = ops.quantize_q8_1(dev(x, device))
-    two = ops.vecq(t, dev(w, device), q8, k, n, tokens=tokens).cpu().numpy()
+    two = ops.vecq(t, dev(w, device), q8, k, n, tokens=tokens, variant=7).cpu().numpy()
     one = ops.vecq_fused(t, dev(w, device), xd, k, n, tokens=tokens).cpu().numpy()
     assert np.array_equal(one.view(np.uint32), two.view(np.uint32))
+    default = ops.vecq(t, dev(w, device), q8, k, n, tokens=tokens).cpu().numpy()
+    ok, worst = rel_close(default, two, 1e-5, floor=1.0)
+    assert ok, worst
 
 
 @pytest.mark.parametrize("t", [Q8_0, Q4_K])
@@ -179,21 +183,36 @@ def test_routed_and_sorted_long_rows_match_oracle(device, t, k):
     assert np.array_equal(sorted_out.view(np.uint32), got.reshape(tokens * used, n)[order].view(np.uint32))
 
 
+def same_sums(t, a, b):
+    """Q8_0: the matrix-core kernel repeats the flat kernel's float operations and its summation tree, bit for bit.
+    Q4_K: its sub-block sums are the same exact integers, scaled and added in another order (one fma a sub-block
+    on the matrix cores' F32 results): the two forms agree to float rounding."""
+    if t == Q8_0:
+        return np.array_equal(a.view(np.uint32), b.view(np.uint32)), 0.0
+    return rel_close(a, b, 1e-5, floor=1.0)
+
+
 @pytest.mark.parametrize("t,k,n,tokens", [(Q4_K, 2816, 50, 5), (Q4_K, 256, 17, 2), (Q4_K, 6144, 32, 16),
-                                          (Q4_K, 2048, 130, 9), (Q8_0, 4096, 50, 5), (Q8_0, 256, 17, 2),
+                                          (Q4_K, 2048, 130, 9), (Q4_K, 8192, 40, 8), (Q4_K, 768, 100, 13),
+                                          (Q8_0, 4096, 50, 5), (Q8_0, 256, 17, 2),
                                           (Q8_0, 3840, 20, 16), (Q8_0, 1792, 130, 9), (Q8_0, 768, 33, 3)])
-def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, t, k, n, tokens):
-    """The int8 matrix-core kernels (variant 9) repeat the flat kernel's float operations and its
-    summation tree: dense with and without a GLU, grouped matrices, and routed experts."""
+def test_matrix_core_form_against_the_flat_form_and_the_oracle(device, t, k, n, tokens):
+    """The matrix-core kernels (variant 9) against the flat form's four-token passes (one-token arithmetic) and the
+    oracle: dense with and without a GLU, grouped matrices, and routed experts."""
     mma, flat = 9, 7
     qk = oracle.block_elements(t)
     gate, up = make_weights(t, n, k, 301), make_weights(t, n, k, 302)
-    q8 = ops.quantize_q8_1(dev(synth.activations(tokens, k, 303), device))
+    x = synth.activations(tokens, k, 303)
+    q8 = ops.quantize_q8_1(dev(x, device))
     wd, gd = dev(up, device), dev(gate, device)
-    for kw in (dict(), dict(gate=gd, glu=ops.GLU_SWIGLU)):
+    for kw, okw in ((dict(), dict()), (dict(gate=gd, glu=ops.GLU_SWIGLU), dict(gate=gate, glu=oracle.GLU_SWIGLU))):
         a = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=mma, **kw).cpu().numpy()
         b = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=flat, **kw).cpu().numpy()
-        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), kw.keys()
+        ok, worst = same_sums(t, a, b)
+        assert ok, (kw.keys(), worst)
+        want = oracle.vecq(t, up, q8.cpu().numpy(), k, n, tokens=tokens, **okw)
+        ok, worst = rel_close(a.reshape(tokens, n), want.reshape(tokens, n), TOL)
+        assert ok, (kw.keys(), worst)
     # Three matrices, every token through each (per-slot activations).
     groups = 3
     w3 = dev(make_weights(t, groups * n, k, 304).reshape(groups, -1), device)
@@ -202,7 +221,8 @@ def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, t, k, n, toke
     kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // qk), y_token=y_row * groups, y_slot=y_row)
     a = ops.vecq(t, w3, q83, k, n, variant=mma, **kw).cpu().numpy()
     b = ops.vecq(t, w3, q83, k, n, variant=flat, **kw).cpu().numpy()
-    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    ok, worst = same_sums(t, a, b)
+    assert ok, worst
     # Routed: two picks a token out of five experts.
     experts, used = 5, 2
     w5 = dev(make_weights(t, experts * n, k, 306).reshape(experts, -1), device)
@@ -211,7 +231,55 @@ def test_matrix_core_form_equals_the_flat_form_bit_for_bit(device, t, k, n, toke
     kw = dict(ids=ids, tokens=tokens, used=used, stride_expert=n * (k // qk))
     a = ops.vecq(t, w5, q8, k, n, variant=mma, **kw).cpu().numpy()
     b = ops.vecq(t, w5, q8, k, n, variant=flat, **kw).cpu().numpy()
-    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    ok, worst = same_sums(t, a, b)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("k,n,glu", [(2816, 50, False), (3840, 70, True), (8192, 20, True), (768, 33, False)])
+def test_matrix_core_form_values_depend_on_their_own_token_alone(device, k, n, glu):
+    """src/kernels/ggml/vecq.cu:688-693 of the reference, within the matrix-core form: a (token, row) value is the
+    same bits whatever tokens are computed beside it, however many (the kernel stages groups of four, eight or
+    sixteen tokens by the count) and in whatever order."""
+    t, tokens = Q4_K, 16
+    gate, up = make_weights(t, n, k, 311), make_weights(t, n, k, 312)
+    x = synth.activations(tokens, k, 313)
+    x[5] *= 30.0
+    q8 = ops.quantize_q8_1(dev(x, device))
+    wd = dev(up, device)
+    kw = dict(gate=dev(gate, device), glu=ops.GLU_GEGLU) if glu else {}
+    full = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=9, **kw).cpu().numpy().reshape(tokens, n)
+    for count in (2, 3, 4, 7, 8, 9, 13):
+        part = ops.vecq(t, wd, q8[:count].contiguous(), k, n, tokens=count, variant=9, **kw).cpu().numpy()
+        assert np.array_equal(part.reshape(count, n).view(np.uint32), full[:count].view(np.uint32)), count
+    order = synth.rng(314).permutation(tokens)
+    mixed = ops.vecq(t, wd, q8[torch.from_numpy(order).to(device)].contiguous(), k, n, tokens=tokens, variant=9, **kw)
+    assert np.array_equal(mixed.cpu().numpy().reshape(tokens, n).view(np.uint32), full[order].view(np.uint32))
+
+
+def test_matrix_core_form_sub_block_sums_are_exact_integers(device):
+    """With d = 1, dmin = 0 and unit block scales a Q4_K product is the integer sum over sub-blocks of
+    sc * sum(q * code): every partial sum stays below 2^24, so F32 holds it exactly and the kernel must return
+    exactly the integer (a matrix-core product that rounded inside a sub-block would not)."""
+    k, n, tokens = 512, 48, 16
+    g = synth.rng(321)
+    w = synth.q4_k_weights(n, k, 322).reshape(n, k // 256, 144).copy()
+    w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), dtype=np.uint8)
+    w[:, :, 2:4] = 0
+    w[:, :, 4:16] &= 0x0F  # scales and minimums below 16: two super-blocks of 8 x 32 x 15 x 15 x 127 stay below 2^24
+    sc = w[:, :, 4:8].astype(np.int64) & 63  # sub-blocks 0 .. 3; 4 .. 7 are the low nibbles of bytes 12 .. 15
+    sc = np.concatenate([sc, w[:, :, 12:16].astype(np.int64) & 15], axis=2)  # [n, nsb, 8]
+    qs = w[:, :, 16:].reshape(n, k // 256, 4, 32)
+    q = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, k // 256, 8, 32).astype(np.int64)
+    codes = g.integers(-127, 128, size=(tokens, k // 32, 32), dtype=np.int64)
+    q8 = np.zeros((tokens, ops.padded_k(k) // 32, 36), dtype=np.uint8)
+    q8[:, :k // 32, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), dtype=np.uint8)
+    q8[:, :k // 32, 4:] = codes.astype(np.int8).view(np.uint8)
+    sums = np.einsum("rbgk,tbgk->trbg", q, codes.reshape(tokens, k // 256, 8, 32))
+    want = np.einsum("trbg,rbg->tr", sums, sc)
+    assert np.abs(want).max() < 2 ** 24
+    got = ops.vecq(Q4_K, dev(w.reshape(-1), device), dev(q8, device), k, n, tokens=tokens, variant=9).cpu().numpy()
+    assert np.array_equal(got.reshape(tokens, n).astype(np.int64), want)
+    assert np.array_equal(got.reshape(tokens, n), want.astype(np.float32))
 
 
 def test_grouped_matrices_read_their_own_rows(device):
