@@ -12,8 +12,8 @@
 //   main = P_0 * d8_0, then fma(P_g, d8_g, main), g = 1 .. 7;  out = fma(main, d, out)
 // over a row's super-blocks in order. The minimums' part, sum over g of (dmin * m_g) *
 // (d8_g * sum of the token's codes), is a plain product of a 16 x 8 by an 8 x 16 matrix a
-// super-block: two v_mfma_f32_16x16x4_f32 into an accumulator of its own, subtracted at the
-// end. A (token, row) value depends on nothing but its own token and row (a column of the
+// super-block: two v_mfma_f32_16x16x4_f32, with -dmin * m as the operand, into the same
+// accumulator. A (token, row) value depends on nothing but its own token and row (a column of the
 // instruction's result only on its own column of the operand), whatever else the pass holds.
 //
 // The weights are the instruction's first operand (a lane holds row lane % 16 and eight
@@ -31,10 +31,18 @@
 //   d8     [super-block][token group][token] 8 floats, sub-block g at g;
 //   ds8    the same, d8_g * sum(codes) of sub-block g at 2 (g % 4) + g / 4 (a lane reads the
 //          pair of its K group for the two small products).
-// A pass takes up to TG groups of MT tokens (MT 16; 8 or 4 with one group, for rows so long
-// that sixteen tokens do not fit), the weights prepared once for all of them. A wave owns 16
-// rows (of both matrices with a GLU) and all of K (rows of up to eight super-blocks) or one
-// half of it (two waves a tile, meeting in LDS).
+// A pass takes up to TG groups of MT tokens (MT 16, in one, two or, without a GLU and for rows of
+// up to four super-blocks, four groups; 8 or 4 with one group, for rows so long that sixteen
+// tokens do not fit), the weights prepared once for all of them. A wave owns 16 rows (of both
+// matrices with a GLU) and all of K (rows of up to eight super-blocks) or one half of it (two
+// waves a tile, meeting in LDS).
+//
+// On this chip the vector unit and the matrix cores of a SIMD do not run at the same time (448
+// fma and 32 of these products a wave take the sum of their separate times at one, two and four
+// waves a SIMD): a step costs its vector instructions at 4 cycles plus its matrix instructions at
+// 16 (F16) and 32 (F32) cycles, and most of it is preparing the weight operand, which is why a
+// pass takes as many tokens as LDS holds. Sorted rows (an expert's rows, any number) are shared
+// among the workgroups by cost, not by expert: see the kernel.
 
 #include <hip/hip_runtime.h>
 
@@ -64,15 +72,23 @@ __device__ unsigned long long* g_mma_trace = nullptr;
   do {                                                                                           \
     if ((threadIdx.x & 63) == 0 && (slot) < 16) trace_area[threadIdx.x / 64][slot] = wall_clock64(); \
   } while (0)
+#define MMA_TRACE_ADD(slot, value)                                            \
+  do {                                                                        \
+    if ((threadIdx.x & 63) == 0) trace_area[threadIdx.x / 64][slot] += (value); \
+  } while (0)
 #define MMA_TRACE_DUMP                                                                                          \
   do {                                                                                                          \
     trace_area[threadIdx.x / 64][15] = wall_clock64();                                                          \
+    trace_area[threadIdx.x / 64][12] = __builtin_readcyclecounter();                                            \
     if (g_mma_trace != nullptr && (threadIdx.x & 63) < 16)                                                      \
       g_mma_trace[((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * kMmaWaves + threadIdx.x / 64) * 16 + \
                   (threadIdx.x & 63)] = trace_area[threadIdx.x / 64][threadIdx.x & 63];                        \
   } while (0)
 #else
 #define MMA_TRACE_AREA
+#define MMA_TRACE_ADD(slot, value) \
+  do {                             \
+  } while (0)
 #define MMA_TRACE(slot) \
   do {                  \
   } while (0)
@@ -174,149 +190,194 @@ struct Staged {
   static constexpr size_t Bytes(int nsb) { return static_cast<size_t>(nsb) * (kCodesSb + 2 * kScalesSb); }
 };
 
-// One super-block of one matrix times the staged tokens: this lane's token of every group, rows
-// 4 (lane / 16) + q. `codes`, `d8`, `ds8`: this lane's places in the super-block's staged
-// tokens; `groups`: the token groups the pass holds.
-template <int TG, int MT>
-__device__ __forceinline__ void DotPart(const RowPart& loaded, int kg, const uint8_t* codes, const uint8_t* d8,
-                                        const uint8_t* ds8, int groups, V4f (&out)[TG], V4f (&mins)[TG]) {
-  using L = Staged<TG, MT>;
-  RowPart part = loaded;
-  Transpose(part);
-  const Header h = Decode(part.header);
-  const V4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
-  // The minimums of sub-blocks kg and 4 + kg, and the row scales in the result's layout.
-  const float m0 = h.dmin * static_cast<float>((h.mn[0] >> (8 * kg)) & 0xFFu);
-  const float m1 = h.dmin * static_cast<float>((h.mn[1] >> (8 * kg)) & 0xFFu);
-  const V4f d_rows = __builtin_amdgcn_mfma_f32_16x16x4f32(kg == 0 ? h.d : 0.0f, 1.0f, zero, 0, 0, 0);
+// What a lane keeps of one super-block of its row between the pairs of sub-blocks.
+struct Prepared {
+  RowPart part;  // exchanged into K groups
+  uint32_t sc[2];
+  float d;
+};
+
+// The first part of a super-block's step for one matrix: the exchange among the row's lanes, the header, and
+// the product that does not depend on the codes: the minimums' part, subtracted from `out` as it is formed
+// (the operand is -dmin * m).
+template <int TG, int MT, int LIVE>
+__device__ __forceinline__ void Begin(const RowPart& loaded, int kg, const uint8_t* ds8, Prepared& prepared, V4f (&out)[TG]) {
+  prepared.part = loaded;
+  Transpose(prepared.part);
+  const Header h = Decode(prepared.part.header);
+  prepared.sc[0] = h.sc[0], prepared.sc[1] = h.sc[1];
+  prepared.d = h.d;
+  // The minimums of sub-blocks kg and 4 + kg.
+  const float m0 = -h.dmin * static_cast<float>((h.mn[0] >> (8 * kg)) & 0xFFu);
+  const float m1 = -h.dmin * static_cast<float>((h.mn[1] >> (8 * kg)) & 0xFFu);
 #pragma unroll
-  for (int tg = 0; tg < TG; ++tg) {
-    if (tg < groups) {
-      const float2 s = *reinterpret_cast<const float2*>(ds8 + tg * MT * 32);
-      mins[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m0, s.x, mins[tg], 0, 0, 0);
-      mins[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m1, s.y, mins[tg], 0, 0, 0);
+  for (int tg = 0; tg < LIVE; ++tg) {
+    const float2 s = *reinterpret_cast<const float2*>(ds8 + tg * MT * 32);
+    out[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m0, s.x, out[tg], 0, 0, 0);
+    out[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(m1, s.y, out[tg], 0, 0, 0);
+  }
+}
+
+// The F16 operands of pair p of a super-block: sub-block 2 p (the low nibbles) and 2 p + 1.
+__device__ __forceinline__ void Operands(const Prepared& prepared, int p, H8& w_lo, H8& w_hi) {
+  // 1024 + sc in both halves, less 1024: the scale of sub-block 2 p, then of 2 p + 1.
+  const uint32_t word = prepared.sc[p >> 1];
+  const uint32_t place_lo = 2 * (p & 1), place_hi = 2 * (p & 1) + 1;
+  const H2 sc_lo = Biased(word, 0x04000400u | place_lo | (place_lo << 16)) - Both(1024.0f);
+  const H2 sc_hi = Biased(word, 0x04000400u | place_hi | (place_hi << 16)) - Both(1024.0f);
+  const H2 off_lo = sc_lo * Both(-1024.0f);
+  const H2 by_hi = sc_hi * Both(0.0625f);  // a high nibble in place is 16 q
+  const H2 off_hi = sc_hi * Both(-64.0f);
+  H2 lo[4], hi[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t w = i == 0 ? prepared.part.q[p].x : prepared.part.q[p].y;
+    const uint32_t low = w & 0x0F0F0F0Fu, high = w & 0xF0F0F0F0u;
+    lo[2 * i] = __builtin_elementwise_fma(Biased(low, kBytes01), sc_lo, off_lo);
+    lo[2 * i + 1] = __builtin_elementwise_fma(Biased(low, kBytes23), sc_lo, off_lo);
+    hi[2 * i] = __builtin_elementwise_fma(Biased(high, kBytes01), by_hi, off_hi);
+    hi[2 * i + 1] = __builtin_elementwise_fma(Biased(high, kBytes23), by_hi, off_hi);
+  }
+  w_lo = __builtin_shufflevector(__builtin_shufflevector(lo[0], lo[1], 0, 1, 2, 3),
+                                 __builtin_shufflevector(lo[2], lo[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+  w_hi = __builtin_shufflevector(__builtin_shufflevector(hi[0], hi[1], 0, 1, 2, 3),
+                                 __builtin_shufflevector(hi[2], hi[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Pair p of one matrix against the token operands: two products a live group, each an fma by the token's
+// block scale into `main`.
+template <int LIVE>
+__device__ __forceinline__ void Pair(const Prepared& prepared, int p, const H8 (&t_lo)[LIVE], const H8 (&t_hi)[LIVE],
+                                     const float2 (&s)[LIVE], float (&main)[LIVE][4]) {
+  const V4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  H8 w_lo, w_hi;
+  Operands(prepared, p, w_lo, w_hi);
+#pragma unroll
+  for (int tg = 0; tg < LIVE; ++tg) {
+    const V4f a_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, t_lo[tg], zero, 0, 0, 0);
+    const V4f a_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, t_hi[tg], zero, 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      main[tg][q] = p == 0 ? a_lo[q] * s[tg].x : fmaf(a_lo[q], s[tg].x, main[tg][q]);
+      main[tg][q] = fmaf(a_hi[q], s[tg].y, main[tg][q]);
     }
   }
-  V4f main[TG];
+}
+
+// The last part: the super-block's sums times the row scales, which reach the result's layout (rows
+// 4 (lane / 16) + q) by a small product of their own: the column d times a row of ones.
+template <int TG, int LIVE>
+__device__ __forceinline__ void End(const Prepared& prepared, int kg, const float (&main)[LIVE][4], V4f (&out)[TG]) {
+  const V4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+  const V4f rows = __builtin_amdgcn_mfma_f32_16x16x4f32(kg == 0 ? prepared.d : 0.0f, 1.0f, zero, 0, 0, 0);
+#pragma unroll
+  for (int tg = 0; tg < LIVE; ++tg) {
+    const V4f before = out[tg];
+    out[tg] = V4f{fmaf(main[tg][0], rows[0], before[0]), fmaf(main[tg][1], rows[1], before[1]),
+                  fmaf(main[tg][2], rows[2], before[2]), fmaf(main[tg][3], rows[3], before[3])};
+  }
+}
+
+// One super-block of the up (and gate) matrix times the staged tokens: this lane's token of every live group, rows
+// 4 (lane / 16) + q. `codes`, `d8`, `ds8`: this lane's places in the super-block's staged tokens; LIVE: the token
+// groups the pass holds (a constant: a branch a group would cut the step into pieces). A pair of sub-blocks at a
+// time, both matrices against the same token operands (read from LDS once), one matrix after the other, the
+// compiler kept from moving work between them: the matrix cores and the vector unit do not run at the same
+// time on this chip, so there is nothing to gain from interleaving further, and holding more operands and
+// results at once costs registers the kernel does not have.
+template <bool kGlu, int TG, int MT, int LIVE>
+__device__ __forceinline__ void DotStep(const RowPart& up, const RowPart& gate, int kg, const uint8_t* codes, const uint8_t* d8,
+                                        const uint8_t* ds8, V4f (&up_out)[TG], V4f (&gate_out)[TG]) {
+  using L = Staged<TG, MT>;
+  Prepared pu, pg;
+  Begin<TG, MT, LIVE>(up, kg, ds8, pu, up_out);
+  if constexpr (kGlu) Begin<TG, MT, LIVE>(gate, kg, ds8, pg, gate_out);
+  float up_main[LIVE][4], gate_main[LIVE][4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
-    // 1024 + sc in both halves, less 1024: the scale of sub-block 2 p, then of 2 p + 1.
-    const uint32_t word = h.sc[p >> 1];
-    const uint32_t place_lo = 2 * (p & 1), place_hi = 2 * (p & 1) + 1;
-    const H2 sc_lo = Biased(word, 0x04000400u | place_lo | (place_lo << 16)) - Both(1024.0f);
-    const H2 sc_hi = Biased(word, 0x04000400u | place_hi | (place_hi << 16)) - Both(1024.0f);
-    const H2 off_lo = sc_lo * Both(-1024.0f);
-    const H2 by_hi = sc_hi * Both(0.0625f);  // a high nibble in place is 16 q
-    const H2 off_hi = sc_hi * Both(-64.0f);
-    H2 lo[4], hi[4];
+    H8 t_lo[LIVE], t_hi[LIVE];
+    float2 s[LIVE];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t w = i == 0 ? part.q[p].x : part.q[p].y;
-      const uint32_t low = w & 0x0F0F0F0Fu, high = w & 0xF0F0F0F0u;
-      lo[2 * i] = __builtin_elementwise_fma(Biased(low, kBytes01), sc_lo, off_lo);
-      lo[2 * i + 1] = __builtin_elementwise_fma(Biased(low, kBytes23), sc_lo, off_lo);
-      hi[2 * i] = __builtin_elementwise_fma(Biased(high, kBytes01), by_hi, off_hi);
-      hi[2 * i + 1] = __builtin_elementwise_fma(Biased(high, kBytes23), by_hi, off_hi);
+    for (int tg = 0; tg < LIVE; ++tg) {
+      t_lo[tg] = *reinterpret_cast<const H8*>(codes + (2 * p) * L::kCodesBlock + tg * L::kCodesGroup);
+      t_hi[tg] = *reinterpret_cast<const H8*>(codes + (2 * p + 1) * L::kCodesBlock + tg * L::kCodesGroup);
+      s[tg] = *reinterpret_cast<const float2*>(d8 + tg * MT * 32 + p * 8);
     }
-    const H8 w_lo = __builtin_shufflevector(__builtin_shufflevector(lo[0], lo[1], 0, 1, 2, 3),
-                                            __builtin_shufflevector(lo[2], lo[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
-    const H8 w_hi = __builtin_shufflevector(__builtin_shufflevector(hi[0], hi[1], 0, 1, 2, 3),
-                                            __builtin_shufflevector(hi[2], hi[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-    for (int tg = 0; tg < TG; ++tg) {
-      if (tg < groups) {
-        const H8 t_lo = *reinterpret_cast<const H8*>(codes + (2 * p) * L::kCodesBlock + tg * L::kCodesGroup);
-        const H8 t_hi = *reinterpret_cast<const H8*>(codes + (2 * p + 1) * L::kCodesBlock + tg * L::kCodesGroup);
-        const V4f p_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_lo, t_lo, zero, 0, 0, 0);
-        const V4f p_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_hi, t_hi, zero, 0, 0, 0);
-        const float2 s = *reinterpret_cast<const float2*>(d8 + tg * MT * 32 + p * 8);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          main[tg][q] = p == 0 ? p_lo[q] * s.x : fmaf(p_lo[q], s.x, main[tg][q]);
-          main[tg][q] = fmaf(p_hi[q], s.y, main[tg][q]);
-        }
-      }
+    Pair<LIVE>(pu, p, t_lo, t_hi, s, up_main);
+    if constexpr (kGlu) {
+      __builtin_amdgcn_sched_barrier(0);
+      Pair<LIVE>(pg, p, t_lo, t_hi, s, gate_main);
     }
+    __builtin_amdgcn_sched_barrier(0);
   }
-#pragma unroll
-  for (int tg = 0; tg < TG; ++tg) {
-    if (tg < groups) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) out[tg][q] = fmaf(main[tg][q], d_rows[q], out[tg][q]);
-    }
-  }
+  End<TG, LIVE>(pu, kg, up_main, up_out);
+  if constexpr (kGlu) End<TG, LIVE>(pg, kg, gate_main, gate_out);
 }
 
-// Stages `staged` tokens' Q8_1 rows (one thread a block) into the operand layout; tokens past
-// the pass's `m` repeat its last (their columns are computed and dropped). `row_of(j)`: token
-// j's row of Q8_1 blocks.
-template <int TG, int MT, class RowOf>
-__device__ __forceinline__ void StageTokens(RowOf row_of, int m, int staged, int blocks, uint8_t* codes, uint8_t* d8,
-                                            uint8_t* ds8) {
+// One Q8_1 block of a token into the operand layout.
+template <int TG, int MT>
+__device__ __forceinline__ void StageBlock(const uint32_t (&w)[9], int t, int b, uint8_t* codes, uint8_t* d8, uint8_t* ds8) {
   using L = Staged<TG, MT>;
-  for (int index = threadIdx.x; index < staged * blocks; index += kMmaGroup) {
-    const int t = index / blocks, b = index - t * blocks;
-    const int tg = t / MT, token = t - tg * MT;
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(min(t, m - 1)) + static_cast<int64_t>(b) * kQ8Block);
-    uint32_t w[9];
+  const int tg = t / MT, token = t - tg * MT;
+  const int sb = b >> 3, g = b & 7;
+  uint8_t* to = codes + sb * L::kCodesSb + g * L::kCodesBlock + tg * L::kCodesGroup + token * 16;
 #pragma unroll
-    for (int i = 0; i < 9; ++i) w[i] = src[i];
-    const int sb = b >> 3, g = b & 7;
-    uint8_t* to = codes + sb * L::kCodesSb + g * L::kCodesBlock + tg * L::kCodesGroup + token * 16;
-#pragma unroll
-    for (int kg = 0; kg < 4; ++kg) {
-      // A code plus 128 is a byte: 1024 + 128 + code under 0x64, less 1152.
-      const uint32_t a = w[1 + 2 * kg] ^ 0x80808080u, c = w[2 + 2 * kg] ^ 0x80808080u;
-      const H2 h0 = Biased(a, kBytes01) - Both(1152.0f), h1 = Biased(a, kBytes23) - Both(1152.0f);
-      const H2 h2 = Biased(c, kBytes01) - Both(1152.0f), h3 = Biased(c, kBytes23) - Both(1152.0f);
-      U32x4 packed;
-      packed.x = __builtin_bit_cast(uint32_t, h0), packed.y = __builtin_bit_cast(uint32_t, h1);
-      packed.z = __builtin_bit_cast(uint32_t, h2), packed.w = __builtin_bit_cast(uint32_t, h3);
-      *reinterpret_cast<U32x4*>(to + kg * MT * 16) = packed;
-    }
-    int sum = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) sum = Dot4(0x01010101, static_cast<int>(w[1 + i]), sum);
-    const float scale = HalfBitsToFloat(w[0] & 0xFFFFu);
-    const int at = sb * L::kScalesSb + (tg * MT + token) * 32;
-    *reinterpret_cast<float*>(d8 + at + g * 4) = scale;
-    *reinterpret_cast<float*>(ds8 + at + (2 * (g & 3) + (g >> 2)) * 4) = scale * static_cast<float>(sum);
+  for (int kg = 0; kg < 4; ++kg) {
+    // A code plus 128 is a byte: 1024 + 128 + code under 0x64, less 1152.
+    const uint32_t a = w[1 + 2 * kg] ^ 0x80808080u, c = w[2 + 2 * kg] ^ 0x80808080u;
+    const H2 h0 = Biased(a, kBytes01) - Both(1152.0f), h1 = Biased(a, kBytes23) - Both(1152.0f);
+    const H2 h2 = Biased(c, kBytes01) - Both(1152.0f), h3 = Biased(c, kBytes23) - Both(1152.0f);
+    U32x4 packed;
+    packed.x = __builtin_bit_cast(uint32_t, h0), packed.y = __builtin_bit_cast(uint32_t, h1);
+    packed.z = __builtin_bit_cast(uint32_t, h2), packed.w = __builtin_bit_cast(uint32_t, h3);
+    *reinterpret_cast<U32x4*>(to + kg * MT * 16) = packed;
   }
+  int sum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sum = Dot4(0x01010101, static_cast<int>(w[1 + i]), sum);
+  const float scale = HalfBitsToFloat(w[0] & 0xFFFFu);
+  const int at = sb * L::kScalesSb + (tg * MT + token) * 32;
+  *reinterpret_cast<float*>(d8 + at + g * 4) = scale;
+  *reinterpret_cast<float*>(ds8 + at + (2 * (g & 3) + (g >> 2)) * 4) = scale * static_cast<float>(sum);
 }
 
-// grid (workgroups, slots); LDS: codes, d8, ds8, the waves' partial sums.
+constexpr int kStageAhead = 4;  // blocks a thread holds in registers between their loads and their staging
+
+// The work of a workgroup between two stagings of tokens: tokens first .. first + m - 1 of the rows
+// listed for `expert` against its row tiles' groups group_first, group_first + group_step, ...
+// (group_count of them).
+struct Segment {
+  int expert, first, m, group_first, group_step, group_count;
+};
+
+// grid (workgroups, slots), or (workgroups) with `balanced` (sorted rows: the workgroups share the
+// passes of all experts evenly, whatever the experts' row counts); LDS: codes, d8, ds8, the waves'
+// partial sums.
 template <bool kGlu, int TG, int MT>
-__global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
+__global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int balanced) {
   using L = Staged<TG, MT>;
+  constexpr int kDepth = TG <= 2 ? 3 : 2;  // weight buffers: the fetches run kDepth - 1 steps ahead
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
-
+  __shared__ int scan[kMmaGroup / kWave];
   MMA_TRACE_AREA;
+#ifdef LLMP_MMA_TRACE
+  if ((threadIdx.x & 63) < 16) trace_area[threadIdx.x / 64][threadIdx.x & 63] = 0;
+#endif
   MMA_TRACE(0);  // the wave's start
+  MMA_TRACE_ADD(11, static_cast<unsigned long long>(__builtin_readcyclecounter()));  // and its shader clock
+
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int nsb = d.ncols_x / 256;
+  const int blocks = d.ncols_x / 32;
   uint8_t* codes = lds;
   uint8_t* d8 = lds + nsb * L::kCodesSb;
   uint8_t* ds8 = d8 + nsb * L::kScalesSb;
   float4* partial = reinterpret_cast<float4*>(ds8 + nsb * L::kScalesSb);
-
-  int expert = blockIdx.y;
-  int sorted_first = 0;
-  if (a.offsets != nullptr) {
-    sorted_first = a.offsets[expert];
-    if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
-    __syncthreads();
-  } else {
-    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
-  }
-  const int n = count;
-  if (n == 0) return;  // uniform over the workgroup
-  const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
-  auto pair_at = [&](int i) { return a.offsets != nullptr ? (sorted_first + i) << 8 : pairs[i]; };
 
   // This wave's part of K. Rows of up to eight super-blocks: all of it, a tile a wave (too few
   // steps to be worth two waves and their meeting). Longer rows: a half.
@@ -330,66 +391,104 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
   const int tiles_group = whole ? kMmaWaves : kTilesGroup;
   const int tile_in_group = whole ? wave : wave >> 1;
   const int groups = (tiles + tiles_group - 1) / tiles_group;
-  const int my_groups = (groups - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
-  const int steps = my_groups * (last - first);  // a pass's
-
-  // The fetches run two steps ahead of the products, through the tiles of a pass in order and
-  // round to the pass's first again (the next pass's, or nobody's).
-  const uint8_t* up_row = nullptr;
-  const uint8_t* gate_row = nullptr;
-  int fetch_group = blockIdx.x, fetch_sb = first;
-  auto aim = [&]() {
-    const int row = min((fetch_group * tiles_group + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
-    const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
-    up_row = static_cast<const uint8_t*>(d.w) + at;
-    if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
-  };
-  // The loads are queued here and no later: the compiler would otherwise sink them to their
-  // first use, two steps on, and the wave would wait out the whole memory latency there.
-  auto fetch = [&](RowPart& u, RowPart& g) {
-    u = LoadRowPart(up_row, fetch_sb, kg);
-    if constexpr (kGlu) g = LoadRowPart(gate_row, fetch_sb, kg);
-    __builtin_amdgcn_sched_barrier(0);
-    if (++fetch_sb == last) {
-      fetch_sb = first;
-      fetch_group += gridDim.x;
-      if (fetch_group >= groups) fetch_group = blockIdx.x;
-      aim();
-    }
-  };
-  RowPart u0, u1, u2, g0, g1, g2;
-  aim();
-  fetch(u0, g0);
-  fetch(u1, g1);
 
   const uint8_t* my_codes = codes + (kg * MT + token_in_group) * 16;
   const uint8_t* my_d8 = d8 + token_in_group * 32;
   const uint8_t* my_ds8 = ds8 + token_in_group * 32 + kg * 8;
 
-  for (int p0 = 0; p0 < n; p0 += TG * MT) {
-    const int m = min(TG * MT, n - p0);
+  int sorted_first = 0;
+  auto pair_at = [&](int i) { return a.offsets != nullptr ? (sorted_first + i) << 8 : pairs[i]; };
+
+  bool staged_before = false;
+  auto run = [&](const Segment& seg) {
+    const int64_t expert_block = static_cast<int64_t>(seg.expert) * d.stride_expert;
+    const int p0 = seg.first, m = seg.m;
+    const int steps = seg.group_count * (last - first);
+    MMA_TRACE_ADD(13, static_cast<unsigned long long>(steps));  // the wave's steps
+    MMA_TRACE_ADD(14, 1ull);                                     // and segments
+    // The live token groups rounded up to a power of two: one compiled step each.
     const int token_groups = (m + MT - 1) / MT;
-    __syncthreads();  // the last pass's readers of the staged tokens
+    const int live = token_groups <= 1 ? 1 : token_groups <= 2 ? 2 : 4;
+
+    // The tokens' blocks are asked for before the weights (loads return in order, and the tokens are
+    // needed whole before the first step), staged after the first weights are.
+    if (staged_before) __syncthreads();  // the last segment's readers of the staged tokens
+    staged_before = true;
+    const int staged = min(live, TG) * MT * blocks;
     auto row_of = [&](int j) {
-      const int pr = pair_at(p0 + j);
+      const int pr = pair_at(p0 + min(j, m - 1));  // tokens past m repeat the last: computed and dropped
       return static_cast<const uint8_t*>(d.y) +
              (static_cast<int64_t>(pr >> 8) * d.y_token + static_cast<int64_t>(pr & 0xFF) * d.y_slot) * kQ8Block;
     };
-    if (p0 == 0) MMA_TRACE(1);  // the first weights asked for, the pairs known
-    StageTokens<TG, MT>(row_of, m, token_groups * MT, d.ncols_x / 32, codes, d8, ds8);
-    __syncthreads();
-    if (p0 == 0) MMA_TRACE(2);  // the first pass's tokens staged
-
-    V4f up_out[TG], up_mins[TG], gate_out[TG], gate_mins[TG];
-    auto clear = [&]() {
+    uint32_t held[kStageAhead][9];
 #pragma unroll
-      for (int tg = 0; tg < TG; ++tg) {
-        up_out[tg] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, up_mins[tg] = up_out[tg];
-        gate_out[tg] = up_out[tg], gate_mins[tg] = up_out[tg];
+    for (int it = 0; it < kStageAhead; ++it) {
+      const int index = tid + it * kMmaGroup;
+      if (index < staged) {
+        const int t = index / blocks, b = index - t * blocks;
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(t) + static_cast<int64_t>(b) * kQ8Block);
+#pragma unroll
+        for (int i = 0; i < 9; ++i) held[it][i] = src[i];
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // The fetches run kDepth - 1 steps ahead of the products, through the segment's tiles in order.
+    const uint8_t* up_row = nullptr;
+    const uint8_t* gate_row = nullptr;
+    int fetch_group = seg.group_first, fetch_sb = first, fetched = 0;
+    auto aim = [&]() {
+      const int row = min((fetch_group * tiles_group + tile_in_group) * 16 + row_in_tile, d.nrows - 1);
+      const int64_t at = (expert_block + static_cast<int64_t>(row) * d.stride_row) * 144;
+      up_row = static_cast<const uint8_t*>(d.w) + at;
+      if constexpr (kGlu) gate_row = static_cast<const uint8_t*>(d.g) + at;
+    };
+    // The loads are queued here and no later: the compiler would otherwise sink them to their
+    // first use, steps on, and the wave would wait out the whole memory latency there. Past the
+    // segment's end its last part again: a load under a branch would make every wait for loads a wait for
+    // all of them (the count of loads in flight is not known where branches join).
+    auto fetch = [&](RowPart& u, RowPart& g) {
+      u = LoadRowPart(up_row, fetch_sb, kg);
+      if constexpr (kGlu) g = LoadRowPart(gate_row, fetch_sb, kg);
+      __builtin_amdgcn_sched_barrier(0);
+      if (++fetched < steps && ++fetch_sb == last) {
+        fetch_sb = first;
+        fetch_group += seg.group_step;
+        aim();
       }
     };
+    RowPart u0, u1, u2, g0, g1, g2;
+    aim();
+    fetch(u0, g0);
+    if constexpr (kDepth == 3) fetch(u1, g1);
+    MMA_TRACE(1);  // the tokens and the first weights asked for
+
+#pragma unroll
+    for (int it = 0; it < kStageAhead; ++it) {
+      const int index = tid + it * kMmaGroup;
+      if (index < staged) {
+        const int t = index / blocks, b = index - t * blocks;
+        StageBlock<TG, MT>(held[it], t, b, codes, d8, ds8);
+      }
+    }
+    for (int index = tid + kStageAhead * kMmaGroup; index < staged; index += kMmaGroup) {
+      const int t = index / blocks, b = index - t * blocks;
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(row_of(t) + static_cast<int64_t>(b) * kQ8Block);
+      uint32_t w[9];
+#pragma unroll
+      for (int i = 0; i < 9; ++i) w[i] = src[i];
+      StageBlock<TG, MT>(w, t, b, codes, d8, ds8);
+    }
+    __syncthreads();
+    MMA_TRACE(2);  // the tokens staged
+
+    V4f up_out[TG], gate_out[TG];
+    auto clear = [&]() {
+#pragma unroll
+      for (int tg = 0; tg < TG; ++tg) up_out[tg] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, gate_out[tg] = up_out[tg];
+    };
     clear();
-    int group = blockIdx.x, sb = first;
+    int group = seg.group_first, sb = first;
     // A tile's rows are done: the two halves of K meet (the upper half's sums through LDS),
     // and the lower half's wave stores.
     auto finish = [&]() {
@@ -399,10 +498,10 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
       if (half == 1) {
 #pragma unroll
         for (int tg = 0; tg < TG; ++tg) {
-          const V4f u = up_out[tg] - up_mins[tg];
+          const V4f u = up_out[tg];
           slot[(2 * tg) * kWave] = make_float4(u[0], u[1], u[2], u[3]);
           if constexpr (kGlu) {
-            const V4f g = gate_out[tg] - gate_mins[tg];
+            const V4f g = gate_out[tg];
             slot[(2 * tg + 1) * kWave] = make_float4(g[0], g[1], g[2], g[3]);
           }
         }
@@ -411,7 +510,7 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
       if (half == 0 && tile < tiles) {
 #pragma unroll
         for (int tg = 0; tg < TG; ++tg) {
-          V4f u = up_out[tg] - up_mins[tg], g = gate_out[tg] - gate_mins[tg];
+          V4f u = up_out[tg], g = gate_out[tg];
           if (!whole) {
             const float4 x = slot[(2 * tg) * kWave];
             u[0] += x.x, u[1] += x.y, u[2] += x.z, u[3] += x.w;
@@ -436,38 +535,142 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a) {
       clear();
     };
     auto step = [&](const RowPart& u, const RowPart& g) {
-      DotPart<TG, MT>(u, kg, my_codes + sb * L::kCodesSb, my_d8 + sb * L::kScalesSb, my_ds8 + sb * L::kScalesSb,
-                      token_groups, up_out, up_mins);
-      if constexpr (kGlu)
-        DotPart<TG, MT>(g, kg, my_codes + sb * L::kCodesSb, my_d8 + sb * L::kScalesSb, my_ds8 + sb * L::kScalesSb,
-                        token_groups, gate_out, gate_mins);
+      const uint8_t* c = my_codes + sb * L::kCodesSb;
+      const uint8_t* s8 = my_d8 + sb * L::kScalesSb;
+      const uint8_t* ds = my_ds8 + sb * L::kScalesSb;
+      if (TG == 1 || live >= TG) {
+        DotStep<kGlu, TG, MT, TG>(u, g, kg, c, s8, ds, up_out, gate_out);
+      } else if (TG == 4 && live == 2) {
+        DotStep<kGlu, TG, MT, TG == 4 ? 2 : 1>(u, g, kg, c, s8, ds, up_out, gate_out);
+      } else {
+        DotStep<kGlu, TG, MT, 1>(u, g, kg, c, s8, ds, up_out, gate_out);
+      }
       if (++sb == last) {
         finish();
         sb = first;
-        group += gridDim.x;
+        group += seg.group_step;
       }
     };
-    for (int s = 0; s < steps; s += 3) {
-      fetch(u2, g2);
-      step(u0, g0);
-      if (p0 == 0) MMA_TRACE(3 + s);  // the first pass's first steps
-      if (s + 1 < steps) {
-        fetch(u0, g0);
-        step(u1, g1);
-        if (p0 == 0) MMA_TRACE(4 + s);
+    if constexpr (kDepth == 3) {
+      for (int s = 0; s < steps; s += 3) {
+        fetch(u2, g2);
+        step(u0, g0);
+        if (s < 6) MMA_TRACE(3 + s);
+        if (s + 1 < steps) {
+          fetch(u0, g0);
+          step(u1, g1);
+          if (s < 6) MMA_TRACE(4 + s);
+        }
+        if (s + 2 < steps) {
+          fetch(u1, g1);
+          step(u2, g2);
+          if (s < 6) MMA_TRACE(5 + s);
+        }
       }
-      if (s + 2 < steps) {
+    } else {
+      for (int s = 0; s < steps; s += 2) {
         fetch(u1, g1);
-        step(u2, g2);
-        if (p0 == 0) MMA_TRACE(5 + s);
+        step(u0, g0);
+        if (s < 6) MMA_TRACE(3 + s);
+        if (s + 1 < steps) {
+          fetch(u0, g0);
+          step(u1, g1);
+          if (s < 6) MMA_TRACE(4 + s);
+        }
       }
     }
-    // The next pass starts at the first tile again, with the buffers in their first roles.
-    if (p0 + TG * MT < n && steps % 3 != 0) {
-      fetch_group = blockIdx.x, fetch_sb = first;
-      aim();
-      fetch(u0, g0);
-      fetch(u1, g1);
+  };
+
+  if (balanced == 0) {
+    int expert = blockIdx.y;
+    if (a.offsets != nullptr) {
+      sorted_first = a.offsets[expert];
+      if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
+      __syncthreads();
+    } else {
+      expert = ResolvePairs(d, blockIdx.y, pairs, &count);
+    }
+    const int n = count;
+    const int mine = (groups - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    for (int p0 = 0; p0 < n; p0 += TG * MT)
+      run(Segment{expert, p0, min(TG * MT, n - p0), static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x), mine});
+  } else {
+    // Sorted rows, shared evenly: expert e brings ceil(rows / (TG MT)) passes, a pass `groups` groups of
+    // tiles, and a group of a pass costs by the pass's live token groups (Cost). The groups of all passes in
+    // expert order lie end to end on a line of cost, and workgroup w takes the groups that start within its
+    // W-th of the line: a few segments of consecutive groups.
+    const int experts = d.used;
+    constexpr int kPass = TG * MT;
+    auto live_of = [](int m) {
+      const int token_groups = (m + MT - 1) / MT;
+      return token_groups <= 1 ? 1 : token_groups <= 2 ? 2 : 4;
+    };
+    // A step's instructions: about 12 parts for the weights and 7 a live token group.
+    auto cost_of = [](int live) { return 12 + 7 * min(live, TG); };
+    auto expert_cost = [&](int rows) {
+      if (rows <= 0) return 0;
+      const int passes = (rows + kPass - 1) / kPass;
+      return (passes - 1) * cost_of(TG) + cost_of(live_of(rows - (passes - 1) * kPass));
+    };
+    int* walk = pairs;  // [0] all experts' cost, [1] the first expert with groups of this workgroup, [2] the cost
+                        // before it, [3] the last such expert
+    if (tid == 0) walk[0] = 0, walk[1] = experts, walk[2] = 0, walk[3] = -1;
+    __syncthreads();
+    for (int base = 0; base < experts; base += kMmaGroup) {
+      const int e = base + tid;
+      int cost = e < experts ? expert_cost(a.offsets[e + 1] - a.offsets[e]) : 0;
+#pragma unroll
+      for (int delta = kWave / 2; delta >= 1; delta /= 2) cost += ShflXor(cost, delta);
+      if (lane == 0 && cost != 0) atomicAdd(&walk[0], cost);
+    }
+    __syncthreads();
+    const int64_t line = static_cast<int64_t>(walk[0]) * groups;
+    const int64_t from = line * blockIdx.x / gridDim.x, to = line * (blockIdx.x + 1) / gridDim.x;
+    int carried = 0;  // cost of the experts before this round of kMmaGroup
+    for (int base = 0; base < experts; base += kMmaGroup) {
+      const int e = base + tid;
+      const int cost = e < experts ? expert_cost(a.offsets[e + 1] - a.offsets[e]) : 0;
+      int inclusive = cost;  // over the wave, then over the workgroup
+#pragma unroll
+      for (int delta = 1; delta < kWave; delta *= 2) {
+        const int other = __shfl_up(inclusive, delta, kWave);
+        if (lane >= delta) inclusive += other;
+      }
+      __syncthreads();  // the last round's readers of scan
+      if (lane == kWave - 1) scan[wave] = inclusive;
+      __syncthreads();
+      int before = carried;
+      for (int w = 0; w < kMmaGroup / kWave; ++w) {
+        if (w < wave) before += scan[w];
+        carried += scan[w];
+      }
+      const int exclusive = before + inclusive - cost;
+      const bool mine = cost != 0 && max(from, static_cast<int64_t>(exclusive) * groups) <
+                                         min(to, static_cast<int64_t>(exclusive + cost) * groups);
+      if (mine) {
+        atomicMin(&walk[1], e);
+        atomicMax(&walk[3], e);
+      }
+      __syncthreads();
+      if (mine && walk[1] == e) walk[2] = exclusive;
+    }
+    __syncthreads();
+    const int e_first = walk[1], e_last = walk[3];
+    int before = walk[2];
+    __syncthreads();  // pairs is free again
+    for (int e = e_first; e <= e_last; ++e) {
+      sorted_first = a.offsets[e];
+      const int rows = a.offsets[e + 1] - sorted_first;
+      for (int p0 = 0; p0 < rows; p0 += kPass) {
+        const int m = min(kPass, rows - p0);
+        const int cost = cost_of(live_of(m));
+        // The pass's groups start at start, start + cost, ...: those within [from, to).
+        const int64_t start = static_cast<int64_t>(before) * groups;
+        const int g_first = from <= start ? 0 : static_cast<int>((from - start + cost - 1) / cost);
+        const int g_end = to <= start ? 0 : static_cast<int>(min<int64_t>((to - start + cost - 1) / cost, groups));
+        if (g_first < g_end) run(Segment{e, p0, m, g_first, 1, g_end - g_first});
+        before += cost;
+      }
     }
   }
   MMA_TRACE_DUMP;  // with the wave's end
@@ -812,8 +1015,9 @@ bool Fits(int nsb, MmaShape* shape) {
   return true;
 }
 
-MmaShape ShapeFor(int nsb, int tokens) {
+MmaShape ShapeFor(int nsb, int tokens, bool glu) {
   MmaShape shape{0, 0, 0};
+  if (tokens > 32 && !glu && Fits<4, 16>(nsb, &shape)) return shape;  // (with a GLU: more registers than a wave has)
   if (tokens > 16 && Fits<2, 16>(nsb, &shape)) return shape;
   if (tokens <= 4 && Fits<1, 4>(nsb, &shape)) return shape;
   if (tokens <= 8 && Fits<1, 8>(nsb, &shape)) return shape;
@@ -838,7 +1042,7 @@ extern "C" int llmp_hip_trace_set_mma(unsigned long long* buffer) {
 bool MmaTakes(int type, const llmp_vecq_desc& d) {
   if (type == LLMP_TYPE_Q4_K) {
     const int nsb = d.ncols_x / 256;
-    return nsb >= 1 && ShapeFor(nsb, 8).groups != 0 && ShapeFor(nsb, 8).tokens >= 8;
+    return nsb >= 1 && ShapeFor(nsb, 8, true).tokens >= 8;
   }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x < 128 || d.ncols_x % 128 != 0 || d.ncols_x > 8192) return false;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
@@ -855,18 +1059,21 @@ void LaunchMmaQ8(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
 }
 
 template <bool kGlu, int TG, int MT>
-void LaunchMmaQ4K(const VecQArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+void LaunchMmaQ4K(const VecQArgs& a, dim3 grid, size_t lds, int balanced, hipStream_t stream) {
   static bool sized = false;
   if (!AllowLds(reinterpret_cast<const void*>(&VecQMma<kGlu, TG, MT>), static_cast<int>(kMmaLdsLimit), &sized)) return;
-  hipLaunchKernelGGL((VecQMma<kGlu, TG, MT>), grid, dim3(kMmaGroup), lds, stream, a);
+  hipLaunchKernelGGL((VecQMma<kGlu, TG, MT>), grid, dim3(kMmaGroup), lds, stream, a, balanced);
 }
 
 template <bool kGlu>
-void LaunchMmaQ4KShape(const MmaShape& shape, const VecQArgs& a, dim3 grid, hipStream_t stream) {
-  if (shape.groups == 2) return LaunchMmaQ4K<kGlu, 2, 16>(a, grid, shape.lds, stream);
-  if (shape.tokens == 16) return LaunchMmaQ4K<kGlu, 1, 16>(a, grid, shape.lds, stream);
-  if (shape.tokens == 8) return LaunchMmaQ4K<kGlu, 1, 8>(a, grid, shape.lds, stream);
-  return LaunchMmaQ4K<kGlu, 1, 4>(a, grid, shape.lds, stream);
+void LaunchMmaQ4KShape(const MmaShape& shape, const VecQArgs& a, dim3 grid, int balanced, hipStream_t stream) {
+  if constexpr (!kGlu) {
+    if (shape.groups == 4) return LaunchMmaQ4K<kGlu, 4, 16>(a, grid, shape.lds, balanced, stream);
+  }
+  if (shape.groups == 2) return LaunchMmaQ4K<kGlu, 2, 16>(a, grid, shape.lds, balanced, stream);
+  if (shape.tokens == 16) return LaunchMmaQ4K<kGlu, 1, 16>(a, grid, shape.lds, balanced, stream);
+  if (shape.tokens == 8) return LaunchMmaQ4K<kGlu, 1, 8>(a, grid, shape.lds, balanced, stream);
+  return LaunchMmaQ4K<kGlu, 1, 4>(a, grid, shape.lds, balanced, stream);
 }
 
 }  // namespace
@@ -896,9 +1103,13 @@ void LaunchMma(int type, const VecQArgs& a, hipStream_t stream) {
   }
   // A slot's tokens: a dense or grouped product's own; sorted rows bring any number an expert, a
   // routed product up to all its pairs.
-  const int tokens = a.offsets != nullptr ? 32 : d.ids != nullptr ? d.used * d.tokens : d.tokens;
-  const MmaShape shape = ShapeFor(nsb, tokens);
-  glu ? LaunchMmaQ4KShape<true>(shape, a, grid, stream) : LaunchMmaQ4KShape<false>(shape, a, grid, stream);
+  const int tokens = a.offsets != nullptr ? 64 : d.ids != nullptr ? d.used * d.tokens : d.tokens;
+  const MmaShape shape = ShapeFor(nsb, tokens, glu);
+  // Sorted rows: one workgroup a compute unit, the passes of all experts shared among them evenly.
+  const int balanced = a.offsets != nullptr ? 1 : 0;
+  const dim3 shared_grid(static_cast<unsigned>(g_mma_compute_units), 1);
+  glu ? LaunchMmaQ4KShape<true>(shape, a, balanced ? shared_grid : grid, balanced, stream)
+      : LaunchMmaQ4KShape<false>(shape, a, balanced ? shared_grid : grid, balanced, stream);
 }
 
 }  // namespace llmp_hip

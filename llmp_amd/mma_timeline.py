@@ -35,7 +35,7 @@ else:
     tokens = int(sys.argv[2]) if len(sys.argv) > 2 else 512
     hidden, ffn, experts, used = 2048, 768, 128, 8
     per = ffn * (hidden // 256)
-    copies = 3
+    copies = int(sys.argv[3]) if len(sys.argv) > 3 else 3
     w0 = D(synth.q4_k_weights(experts * 2 * ffn, hidden, 71).reshape(experts, -1))
     ws = [w0] + [w0.clone() for _ in range(copies - 1)]
     g = synth.rng(5)
@@ -64,20 +64,29 @@ for r in range(4):
     torch.cuda.synchronize()
     runs.append(trace.cpu().numpy().reshape(-1, 16).copy())
 lib.llmp_hip_trace_set_mma(None)
-names = ["start", "first weights asked for", "tokens staged"] + ["step %d done" % (i + 1) for i in range(12)] + ["wave done"]
+names = ["start", "first weights asked for", "tokens staged"] + ["step %d done" % (i + 1) for i in range(10)] + ["", "", "wave done"]
 tr = runs[-1]
 tr = tr[tr[:, 0] != 0].astype(np.float64)
 t0 = tr[:, 0].min()
 print("waves %d; launch length by the stamps %.2f us" % (len(tr), (tr[:, 15].max() - t0) / 100))
 for s, name in enumerate(names):
+    if not name: continue
     col = tr[:, s]; col = col[col != 0]
     if len(col) == 0: continue
     col = (col - t0) / 100
     print("%-24s waves %5d  min %7.2f  median %7.2f  p90 %7.2f  max %7.2f us" % (name, len(col), col.min(), np.median(col), np.percentile(col, 90), col.max()))
-steps = tr[:, 3:15]
+steps = tr[:, 3:13]
 ok = (steps != 0).all(axis=1)
 if ok.any():
     d = np.diff(steps[ok], axis=1) / 100
-    print("a step (median over waves), steps 2..12: " + " ".join("%.2f" % x for x in np.median(d, axis=0)))
+    print("a step (median over waves), steps 2..10: " + " ".join("%.2f" % x for x in np.median(d, axis=0)))
 done = (tr[:, 15] - t0) / 100
 print("wave done: p10 %.1f p50 %.1f p90 %.1f max %.1f" % tuple(np.percentile(done, [10, 50, 90, 100])))
+count, segments = tr[:, 13], tr[:, 14]
+print("steps a wave: min %d median %d max %d; segments: min %d median %d max %d" % (count.min(), np.median(count), count.max(), segments.min(), np.median(segments), segments.max()))
+for lo in range(0, int(count.max()) + 1, 4):
+    pick = (count >= lo) & (count < lo + 4)
+    if pick.any(): print("  waves of %2d..%2d steps: %4d, done at median %.1f us, segments median %.1f" % (lo, lo + 3, pick.sum(), np.median(done[pick]), np.median(segments[pick])))
+cycles = tr[:, 12] - tr[:, 11]
+span = (tr[:, 15] - tr[:, 0]) / 100
+print("shader clock over a wave's life: median %.2f GHz (min %.2f, max %.2f)" % (np.median(cycles / span) / 1e3, (cycles / span).min() / 1e3, (cycles / span).max() / 1e3))

@@ -17,6 +17,10 @@ pytestmark = pytest.mark.gpu
 
 Q8_0, Q4_K = ops.TYPE_Q8_0, ops.TYPE_Q4_K
 TOL = 1e-3
+# A GLU output is a product of two sums of thousands of terms that cancel: where it comes out under a hundredth of
+# the output's RMS it is held to 1e-5 of the RMS (FP32 accumulation in another order than the oracle's doubles moves
+# it by about 1e-6 of the RMS; the reference's own check, tests/unit/dsv4_fast_test.cc:419, allows 2e-5 absolute).
+GLU_FLOOR = 1e-2
 
 
 def dev(a, device):
@@ -70,11 +74,11 @@ def test_config_2_q4_k_gate_up_geglu_3840_x_15360(device, tokens):
     gd, ud = dev(gate, device), dev(up, device)
     got = ops.vecq(Q4_K, ud, q8_got, k, n, gate=gd, tokens=tokens, glu=ops.GLU_GEGLU).cpu().numpy()
     assert got.shape[-1] == n
-    ok, worst = rel_close(got.reshape(tokens, n), want.reshape(tokens, n), TOL)
+    ok, worst = rel_close(got.reshape(tokens, n), want.reshape(tokens, n), TOL, floor=GLU_FLOOR)
     assert ok, worst
     xd = dev(x, device).to(torch.bfloat16)
     fused = ops.vecq_fused(Q4_K, ud, xd, k, n, gate=gd, tokens=tokens, glu=ops.GLU_GEGLU).cpu().numpy()
-    ok, worst = rel_close(fused.reshape(tokens, n), want.reshape(tokens, n), TOL)
+    ok, worst = rel_close(fused.reshape(tokens, n), want.reshape(tokens, n), TOL, floor=GLU_FLOOR)
     assert ok, worst
     if tokens <= 4:  # the same form at every count: the same bits
         assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
@@ -163,11 +167,11 @@ def test_sorted_rows_of_many_passes_match_oracle_and_the_routed_product(device, 
     for variant in (-1, 7):  # the default (matrix cores) and the flat form's four-token passes
         got = ops.vecq_sorted(t, upd, sq8, route.offsets, hidden, ffn, experts, stride_expert=stride, variant=variant,
                               **kw).cpu().numpy()
-        ok, worst = rel_close(got[position], want, TOL)
+        ok, worst = rel_close(got[position], want, TOL, floor=GLU_FLOOR if glu else 1e-3)
         assert ok, (variant, worst)
     routed = ops.vecq(t, upd, dev(q8, device), hidden, ffn, ids=dev(ids, device), tokens=tokens, used=used,
                       stride_expert=stride, **kw).cpu().numpy().reshape(tokens * used, ffn)
-    ok, worst = rel_close(routed, want, TOL)
+    ok, worst = rel_close(routed, want, TOL, floor=GLU_FLOOR if glu else 1e-3)
     assert ok, worst
     default = ops.vecq_sorted(t, upd, sq8, route.offsets, hidden, ffn, experts, stride_expert=stride, **kw).cpu().numpy()
     ok, worst = rel_close(default[position], routed, 1e-5, floor=1.0)  # two forms of the same sums: float order only
@@ -199,5 +203,5 @@ def test_sorted_rows_beyond_the_routed_form(device):
         order, _ = oracle.expert_sort(ids, experts)
         sq8 = dev(q8[order], device)  # row r of the sorted activations is pair order[r]'s
         got = ops.vecq_sorted(Q4_K, upd, sq8, route.offsets, k, n, experts, stride_expert=stride, **kw).cpu().numpy()
-        ok, worst = rel_close(got, want[order], TOL)
+        ok, worst = rel_close(got, want[order], TOL, floor=GLU_FLOOR if glu else 1e-3)
         assert ok, (k, worst)
