@@ -183,8 +183,8 @@ def other_configs(device, args, only=None):
             us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
                                           glu=ops.GLU_GEGLU, out=y), 4 * count)
             entry = {"workload": f"config 2 at batch {tokens}",
-                     "roofline": hbm_roofline(name, "VecQMma<glu> (llmp.vecq, Q4_K, matrix cores)" if tokens > 4 else
-                                              "VecQFlat<FormatQ4K, 4 tokens a pass, glu>", algorithmic_bytes(tokens), us)}
+                     "roofline": hbm_roofline(name, "VecQRows<glu, %d tokens> (llmp.vecq, Q4_K, a weight row a lane on "
+                                              "v_mfma_i32_4x4x4_16B_i8)" % (4 if tokens <= 4 else 8), algorithmic_bytes(tokens), us)}
             if cpu:
                 q8_host = oracle.q8_1_quantize(x_host)
                 entry["cpu_baseline"] = cpu_leg(

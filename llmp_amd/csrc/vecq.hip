@@ -492,8 +492,12 @@ constexpr Variant kVariants[] = {
     // Q4_K sub-block products on the int8 matrix cores, 16 tokens a pass (vecq_mma.hip);
     // `lanes` -1 marks the form.
     {"mma pass16", -1, 16, 1},
+    // Q4_K, a weight row a lane, 2 to 8 tokens of a dense or grouped product on the 4 x 4 x 4 int8 matrix
+    // instruction (vecq_rows.hip); `lanes` -2 marks the form.
+    {"rows pass8", -2, 8, 1},
 };
 constexpr int kMmaVariant = 9;
+constexpr int kRowsVariant = 10;
 constexpr int kFlatFirst = 6;
 constexpr int kVariantCount = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -561,10 +565,12 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   const int tokens = d.tokens;
   // Several tokens of a dense or grouped product over Q8_1 blocks: the matrix cores. A routed product's pairs
   // mostly name different experts, one or two tokens each: the flat form.
-  // (Measured at 4096 x 14336 and 3840 x 15360, with and without a GLU: the matrix-core kernel's time hardly depends
-  // on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0 (15 / 17 / 20 / 27 us
-  // against 29), four for a Q4_K gate/up pair (19 / 22 / 26 against 25-26) and two for a plain Q4_K product (12
-  // against 13).)
+  // Q4_K, 2 to 8 tokens: a weight row a lane on the 4 x 4 x 4 instruction (at 3840 x 2 x 15360 with a GLU 17.8 us
+  // at two and at four tokens, 21.3 at eight, against the 16 x 16 form's 25 at any count and the flat form's
+  // four-token passes' 18 / 25 / 43). More tokens, and rows that form does not take: the 16 x 16 form, whose time
+  // hardly depends on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0
+  // (15 / 17 / 20 / 27 us against 29 at 4096 x 14336).
+  if (tokens > 1 && !fused && RowsTakes(type, d)) return kRowsVariant;
   const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 5 : d.g != nullptr ? 4 : 2;
   if (tokens > flat_up_to && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
@@ -649,6 +655,15 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && v.lanes != 0)
     return Refuse(1, "vecq: the legacy 4/5-bit blocks, IQ4_NL, Q5_K, Q6_K and MXFP4 take the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
+  if (v.lanes == -2) {
+    if (offsets != nullptr || !RowsTakes(type, *d))
+      return Refuse(1, "vecq: the row-a-lane form takes 2 to 8 tokens of a dense or grouped Q4_K product, rows of 1024 values "
+                       "or more");
+    if (x != nullptr) return Refuse(1, "vecq: the row-a-lane form takes Q8_1 activations");
+    if (dump != nullptr) return Refuse(1, "vecq: block sums are of the one-token variants");
+    LaunchRows(a, static_cast<hipStream_t>(stream));
+    return LaunchStatus("vecq");
+  }
   if (v.lanes < 0) {
     if (!MmaTakes(type, *d))
       return Refuse(1, "vecq: the matrix-core form takes Q4_K rows up to 7168 values and Q8_0 rows of whole 128 values "

@@ -170,6 +170,25 @@ __device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_in
   return expert;
 }
 
+// The decoded header of a super-block: 6-bit scales and minimums as bytes g of sc[g / 4],
+// mn[g / 4] (the packing of tests/unit/dsv4_fast_test.cc:180-183 of the reference).
+struct Q4KHeader {
+  uint32_t sc[2], mn[2];
+  float d, dmin;
+};
+
+__device__ __forceinline__ Q4KHeader DecodeQ4KHeader(const U32x4& h) {
+  Q4KHeader out;
+  const uint32_t s0 = h.y, s1 = h.z, s2 = h.w;
+  out.sc[0] = s0 & 0x3F3F3F3Fu;
+  out.sc[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+  out.mn[0] = s1 & 0x3F3F3F3Fu;
+  out.mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+  out.d = HalfBitsToFloat(h.x & 0xFFFFu);
+  out.dmin = HalfBitsToFloat(h.x >> 16);
+  return out;
+}
+
 // The flat kernels' launch (vecq_flat.hip): whether a product's shape and alignment fit them,
 // and the launch. x_type -1: Q8_1 activations.
 bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows = false);
@@ -179,6 +198,10 @@ void LaunchFlat(int type, const VecQArgs& a, int x_type, int pass, bool deep, hi
 // The matrix-core kernels for 2 to 16 tokens a pass over Q8_1 activations (vecq_mma.hip).
 bool MmaTakes(int type, const llmp_vecq_desc& d);
 void LaunchMma(int type, const VecQArgs& a, hipStream_t stream);
+
+// The row-a-lane kernel for 2 to 8 tokens of a dense or grouped Q4_K product over Q8_1 activations (vecq_rows.hip).
+bool RowsTakes(int type, const llmp_vecq_desc& d);
+void LaunchRows(const VecQArgs& a, hipStream_t stream);
 
 }  // namespace llmp_hip
 

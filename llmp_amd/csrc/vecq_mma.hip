@@ -144,25 +144,6 @@ __device__ __forceinline__ void Transpose(RowPart& part) {
   }
 }
 
-// The decoded header of a super-block: 6-bit scales and minimums as bytes g of sc[g / 4],
-// mn[g / 4] (the packing of tests/unit/dsv4_fast_test.cc:180-183 of the reference).
-struct Header {
-  uint32_t sc[2], mn[2];
-  float d, dmin;
-};
-
-__device__ __forceinline__ Header Decode(const U32x4& h) {
-  Header out;
-  const uint32_t s0 = h.y, s1 = h.z, s2 = h.w;
-  out.sc[0] = s0 & 0x3F3F3F3Fu;
-  out.sc[1] = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
-  out.mn[0] = s1 & 0x3F3F3F3Fu;
-  out.mn[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
-  out.d = HalfBitsToFloat(h.x & 0xFFFFu);
-  out.dmin = HalfBitsToFloat(h.x >> 16);
-  return out;
-}
-
 __device__ __forceinline__ int64_t Pack(uint32_t lo, uint32_t hi) {
   return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
 }
@@ -204,7 +185,7 @@ template <int TG, int MT, int LIVE>
 __device__ __forceinline__ void Begin(const RowPart& loaded, int kg, const uint8_t* ds8, Prepared& prepared, V4f (&out)[TG]) {
   prepared.part = loaded;
   Transpose(prepared.part);
-  const Header h = Decode(prepared.part.header);
+  const Q4KHeader h = DecodeQ4KHeader(prepared.part.header);
   prepared.sc[0] = h.sc[0], prepared.sc[1] = h.sc[1];
   prepared.d = h.d;
   // The minimums of sub-blocks kg and 4 + kg.
@@ -356,7 +337,10 @@ struct Segment {
 template <bool kGlu, int TG, int MT>
 __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int balanced) {
   using L = Staged<TG, MT>;
-  constexpr int kDepth = TG <= 2 ? 3 : 2;  // weight buffers: the fetches run kDepth - 1 steps ahead
+#ifndef MMA_DEPTH1
+#define MMA_DEPTH1 3
+#endif
+  constexpr int kDepth = TG == 1 ? MMA_DEPTH1 : TG == 2 ? 3 : 2;  // weight buffers: the fetches run kDepth - 1 steps ahead
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
@@ -457,10 +441,10 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
         aim();
       }
     };
-    RowPart u0, u1, u2, g0, g1, g2;
+    RowPart ub[kDepth], gb[kDepth];
     aim();
-    fetch(u0, g0);
-    if constexpr (kDepth == 3) fetch(u1, g1);
+#pragma unroll
+    for (int j = 0; j < kDepth - 1; ++j) fetch(ub[j], gb[j]);
     MMA_TRACE(1);  // the tokens and the first weights asked for
 
 #pragma unroll
@@ -551,31 +535,13 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
         group += seg.group_step;
       }
     };
-    if constexpr (kDepth == 3) {
-      for (int s = 0; s < steps; s += 3) {
-        fetch(u2, g2);
-        step(u0, g0);
-        if (s < 6) MMA_TRACE(3 + s);
-        if (s + 1 < steps) {
-          fetch(u0, g0);
-          step(u1, g1);
-          if (s < 6) MMA_TRACE(4 + s);
-        }
-        if (s + 2 < steps) {
-          fetch(u1, g1);
-          step(u2, g2);
-          if (s < 6) MMA_TRACE(5 + s);
-        }
-      }
-    } else {
-      for (int s = 0; s < steps; s += 2) {
-        fetch(u1, g1);
-        step(u0, g0);
-        if (s < 6) MMA_TRACE(3 + s);
-        if (s + 1 < steps) {
-          fetch(u0, g0);
-          step(u1, g1);
-          if (s < 6) MMA_TRACE(4 + s);
+    for (int s = 0; s < steps; s += kDepth) {
+#pragma unroll
+      for (int j = 0; j < kDepth; ++j) {
+        if (j == 0 || s + j < steps) {
+          fetch(ub[(j + kDepth - 1) % kDepth], gb[(j + kDepth - 1) % kDepth]);
+          step(ub[j], gb[j]);
+          if (s < 6 && j < 4) MMA_TRACE(3 + s + j);
         }
       }
     }

@@ -1,0 +1,496 @@
+// llmp.vecq over Q4_K weights for 2 to 8 tokens of a dense or grouped product: a lane a weight row,
+// the dot products on the 4 x 4 x 4 int8 matrix instruction.
+//
+// v_mfma_i32_4x4x4_16B_i8 multiplies, in each of sixteen blocks of four lanes, a 4 x 4 matrix A by a
+// 4 x 4 matrix B over four int8 values: lane 4 b + j supplies column j of B (four values of its own),
+// and A can be one block's, broadcast to all sixteen. With a lane's weight row as its column of B
+// and four tokens' codes as A, one instruction adds four values' products to a 4-token x 64-row
+// tile of int32 sums; eight of them make a sub-block's exact sums for four tokens, with every lane
+// of the result holding its own row. What is left in floats is what the one-token kernel does,
+//   main = float(P_g) * (sc_g * d8_g), then fma over g;  out = fma(main, d, out),
+// but four tokens a lane where the 16 x 16 instructions give sixteen tokens to sixteen rows: at
+// four and eight tokens that is a quarter and a half of their vector work a weight byte. The
+// minimums' part, (dmin * m_g) * (d8_g * sum of the codes), is an outer product a sub-block:
+// v_mfma_f32_4x4x1_16B_f32 into an accumulator of its own.
+//
+// A workgroup is four waves and takes 64 rows at a time, each wave a quarter of K, meeting in LDS.
+// A wave's weights come by global_load_lds_dwordx4 into a ring of its own in LDS, a 64-row
+// super-block (9216 bytes, row after row) a stage, two or three stages deep; a lane then reads
+// its row's 144 bytes (lanes 36 dwords apart: no two on a bank). The tokens' Q8_1 blocks are
+// staged once a workgroup:
+//   codes  [block][half][token] 16 bytes: the block's codes 16 half .. 16 half + 15 (lane t reads
+//          token t's; the instruction broadcasts block t / 4's to all);
+//   d8     [block][token] F32 (read four tokens at a time, the same for every lane);
+//   ds8    [super-block][token] 8 floats, d8 * sum(codes) of sub-block g at g.
+// A (token, row) value depends on its own token and row alone.
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "llmp_hip.h"
+#include "vecq_common.h"
+
+namespace llmp_hip {
+namespace {
+
+constexpr int kRowsGroup = 256;
+constexpr int kRowsWaves = kRowsGroup / kWave;
+constexpr int kTileRows = 64;
+constexpr int kPieceBytes = kTileRows * 144;  // one super-block of a tile's rows
+constexpr int kPieceLoads = kPieceBytes / (kWave * 16);
+constexpr size_t kRowsLdsLimit = 160 * 1024 - 1024;
+
+// Timeline instrumentation for tuning, compiled only into a build with -DLLMP_MMA_TRACE (never the library's):
+// lane 0 of every wave keeps the 100 MHz clock of up to sixteen points in LDS and stores them as the wave ends.
+#ifdef LLMP_MMA_TRACE
+__device__ unsigned long long* g_rows_trace = nullptr;
+#define ROWS_TRACE_AREA __shared__ unsigned long long trace_area[kRowsWaves][16]
+#define ROWS_TRACE(slot)                                                                         \
+  do {                                                                                           \
+    if ((threadIdx.x & 63) == 0 && (slot) < 16)                                                  \
+      LdsWrite8(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&trace_area[threadIdx.x / 64][slot])), wall_clock64()); \
+  } while (0)
+#define ROWS_TRACE_DUMP                                                                                         \
+  do {                                                                                                          \
+    trace_area[threadIdx.x / 64][15] = wall_clock64();                                                          \
+    if (g_rows_trace != nullptr && (threadIdx.x & 63) < 16)                                                     \
+      g_rows_trace[((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * kRowsWaves + threadIdx.x / 64) * 16 + \
+                   (threadIdx.x & 63)] = trace_area[threadIdx.x / 64][threadIdx.x & 63];                       \
+  } while (0)
+#else
+#define ROWS_TRACE_AREA
+#define ROWS_TRACE(slot) \
+  do {                   \
+  } while (0)
+#define ROWS_TRACE_DUMP \
+  do {                  \
+  } while (0)
+#endif
+
+typedef int V4i __attribute__((ext_vector_type(4)));
+typedef float V4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* LdsPointer;
+typedef const __attribute__((address_space(1))) void* GlobalPointer;
+
+template <int LEFT>
+__device__ __forceinline__ void AwaitLoads() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (LEFT & 15) | ((LEFT >> 4) << 14));
+  asm volatile("" ::: "memory");  // what the loads wrote into LDS is read after this
+}
+
+// While a global_load_lds is in flight the compiler makes every wait it inserts a wait for everything: a read or
+// a write of LDS it knows of waits until every load into LDS has landed (it cannot tell which of them the access
+// could alias), and a wait for an ordinary load's register is taken to zero as well (the instruction counts as
+// one that may touch both memories, whose returns are not ordered). The ring would never hold a load in flight
+// while the wave computes. So between the first such load and the drain at a tile's end this kernel touches LDS
+// and global memory only through the instructions written out below, and orders them itself: a wait, then Tie on
+// every register the waited-for instructions wrote (which keeps the compiler from using one earlier).
+typedef uint32_t U32v4 __attribute__((ext_vector_type(4)));
+#define LLMP_TIE(x) asm volatile("" : "+v"(x))
+// (By value: __builtin_bit_cast straight on an element of a vector reads element 0 whatever the index.)
+__device__ __forceinline__ float AsFloat(uint32_t bits) { return __builtin_bit_cast(float, bits); }
+
+template <int OFFSET>
+__device__ __forceinline__ U32v4 LdsRead16(uint32_t at) {
+  U32v4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(OFFSET));
+  return v;
+}
+__device__ __forceinline__ void LdsWaited() { asm volatile("s_waitcnt lgkmcnt(0)"); }
+__device__ __forceinline__ void LdsWrite16(uint32_t at, U32v4 value) { asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(value)); }
+__device__ __forceinline__ void LdsWrite4(uint32_t at, float value) { asm volatile("ds_write_b32 %0, %1" : : "v"(at), "v"(value)); }
+__device__ __forceinline__ void LdsWrite8(uint32_t at, unsigned long long value) {
+  asm volatile("ds_write_b64 %0, %1" : : "v"(at), "v"(value));
+}
+__device__ __forceinline__ U32v4 GlobalLoad16(const void* from) {
+  U32v4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(from));
+  return v;
+}
+__device__ __forceinline__ uint32_t GlobalLoad4(const void* from) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(from));
+  return v;
+}
+// A workgroup barrier for LDS alone: what the waves wrote to LDS is there, loads from global memory stay in flight
+// (__syncthreads waits for those too).
+__device__ __forceinline__ void LdsBarrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)");
+  __builtin_amdgcn_s_barrier();
+}
+
+template <int NT>
+struct Tokens {
+  static constexpr int kCodesBlock = 2 * NT * 16;  // bytes of codes a block
+  static constexpr int kScalesBlock = NT * 4;      // of d8
+  static constexpr int kSumsSb = NT * 32;          // of ds8 a super-block
+  static constexpr size_t Bytes(int blocks) {
+    return static_cast<size_t>(blocks) * (kCodesBlock + kScalesBlock) + static_cast<size_t>(blocks / 8) * kSumsSb;
+  }
+};
+
+// One super-block of one matrix for this lane's row (`row`: the LDS address of its 144 bytes) times the staged
+// tokens. `codes`, `d8`: the LDS addresses of the super-block's, `codes` at this lane's token; `sums`: of this
+// lane's token's eight ds8. Every LDS read is a RingRead (see there): a pair of sub-blocks' token operands are
+// asked for while the pair before is multiplied.
+template <int NT>
+__device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t d8, uint32_t sums, float (&out)[NT],
+                                         V4f (&mins)[NT / 4]) {
+#pragma clang fp contract(off)
+  using T = Tokens<NT>;
+  constexpr int kQuads = NT / 4;
+  U32v4 header = LdsRead16<0>(row);
+  U32v4 qs[8] = {LdsRead16<16>(row), LdsRead16<32>(row), LdsRead16<48>(row), LdsRead16<64>(row),
+                 LdsRead16<80>(row), LdsRead16<96>(row), LdsRead16<112>(row), LdsRead16<128>(row)};
+  U32v4 s_lo = LdsRead16<0>(sums), s_hi = LdsRead16<16>(sums);
+  // Pair p's token operands: the codes of sub-blocks 2 p and 2 p + 1 (two reads each) and their d8 (a read a quad).
+  U32v4 c[2][4], scale[2][2 * kQuads];
+  auto ask = [&](int p, U32v4 (&cs)[4], U32v4 (&ds)[2 * kQuads]) {
+    const uint32_t at = codes + static_cast<uint32_t>(2 * p * T::kCodesBlock);
+    cs[0] = LdsRead16<0>(at), cs[1] = LdsRead16<NT * 16>(at);
+    cs[2] = LdsRead16<T::kCodesBlock>(at), cs[3] = LdsRead16<T::kCodesBlock + NT * 16>(at);
+    const uint32_t dat = d8 + static_cast<uint32_t>(2 * p * T::kScalesBlock);
+    ds[0] = LdsRead16<0>(dat), ds[kQuads] = LdsRead16<T::kScalesBlock>(dat);
+    if constexpr (kQuads >= 2) ds[1] = LdsRead16<16>(dat), ds[kQuads + 1] = LdsRead16<T::kScalesBlock + 16>(dat);
+  };
+  auto landed = [&](U32v4 (&cs)[4], U32v4 (&ds)[2 * kQuads]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) LLMP_TIE(cs[i]);
+#pragma unroll
+    for (int i = 0; i < 2 * kQuads; ++i) LLMP_TIE(ds[i]);
+  };
+  ask(0, c[0], scale[0]);
+  LdsWaited();
+  LLMP_TIE(header);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) LLMP_TIE(qs[i]);
+  LLMP_TIE(s_lo);
+  LLMP_TIE(s_hi);
+  landed(c[0], scale[0]);
+  U32x4 header4;
+  header4.x = header[0], header4.y = header[1], header4.z = header[2], header4.w = header[3];
+  const Q4KHeader h = DecodeQ4KHeader(header4);
+  const float ds8[8] = {AsFloat(s_lo[0]), AsFloat(s_lo[1]), AsFloat(s_lo[2]),
+                        AsFloat(s_lo[3]), AsFloat(s_hi[0]), AsFloat(s_hi[1]),
+                        AsFloat(s_hi[2]), AsFloat(s_hi[3])};
+  uint32_t w[32];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) w[4 * i] = qs[i][0], w[4 * i + 1] = qs[i][1], w[4 * i + 2] = qs[i][2], w[4 * i + 3] = qs[i][3];
+  float main[NT];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const U32v4 (&cs)[4] = c[p & 1];
+    const U32v4 (&ds)[2 * kQuads] = scale[p & 1];
+    if (p < 3) ask(p + 1, c[(p + 1) & 1], scale[(p + 1) & 1]);
+    const uint32_t code[2][8] = {{cs[0][0], cs[0][1], cs[0][2], cs[0][3], cs[1][0], cs[1][1], cs[1][2], cs[1][3]},
+                                 {cs[2][0], cs[2][1], cs[2][2], cs[2][3], cs[3][0], cs[3][1], cs[3][2], cs[3][3]}};
+    // The pair's two (four with eight tokens) chains of products interleaved: a wave is alone on its SIMD, and
+    // a chain alone would wait out every instruction's latency.
+    V4i sum[2][kQuads];
+#pragma unroll
+    for (int upper = 0; upper < 2; ++upper)
+#pragma unroll
+      for (int tq = 0; tq < kQuads; ++tq) sum[upper][tq] = V4i{0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int low = static_cast<int>(w[8 * p + s] & 0x0F0F0F0Fu), high = static_cast<int>((w[8 * p + s] >> 4) & 0x0F0F0F0Fu);
+      if constexpr (kQuads >= 1) {
+        sum[0][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][0], 4, 0, 0);
+        sum[1][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][0], 4, 0, 0);
+      }
+      if constexpr (kQuads >= 2) {
+        sum[0][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][1], 4, 1, 0);
+        sum[1][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][1], 4, 1, 0);
+      }
+    }
+#pragma unroll
+    for (int upper = 0; upper < 2; ++upper) {
+      const int g = 2 * p + upper;
+      const float sc = static_cast<float>((h.sc[g >> 2] >> (8 * (g & 3))) & 0xFFu);
+      const float dm = h.dmin * static_cast<float>((h.mn[g >> 2] >> (8 * (g & 3))) & 0xFFu);
+      if constexpr (kQuads >= 1) mins[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[0], 4, 0, 0);
+      if constexpr (kQuads >= 2) mins[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[1], 4, 1, 0);
+#pragma unroll
+      for (int tq = 0; tq < kQuads; ++tq) {
+        const U32v4 d4 = ds[upper * kQuads + tq];
+        const float token_scale[4] = {AsFloat(d4[0]), AsFloat(d4[1]),
+                                      AsFloat(d4[2]), AsFloat(d4[3])};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float by = sc * token_scale[q];
+          const float product = static_cast<float>(sum[upper][tq][q]);
+          main[4 * tq + q] = g == 0 ? product * by : fmaf(product, by, main[4 * tq + q]);
+        }
+      }
+    }
+    if (p < 3) {
+      LdsWaited();
+      landed(c[(p + 1) & 1], scale[(p + 1) & 1]);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) out[t] = fmaf(main[t], h.d, out[t]);
+}
+
+// grid (workgroups, slots); LDS: the tokens, then the waves' rings (whose first bytes also carry the
+// waves' sums to their meeting).
+template <bool kGlu, int NT, int STAGES>
+__global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
+  using T = Tokens<NT>;
+  constexpr int kMatrices = kGlu ? 2 : 1;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  ROWS_TRACE_AREA;
+#ifdef LLMP_MMA_TRACE
+  if ((threadIdx.x & 63) < 16) trace_area[threadIdx.x / 64][threadIdx.x & 63] = 0;
+#endif
+  ROWS_TRACE(0);  // the wave's start
+
+  const llmp_vecq_desc& d = a.d;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int nsb = d.ncols_x / 256;
+  const int blocks = d.ncols_x / 32;
+  const int slot = blockIdx.y;
+  uint8_t* codes = lds;
+  uint8_t* d8 = codes + blocks * T::kCodesBlock;
+  uint8_t* sums = d8 + blocks * T::kScalesBlock;
+  uint8_t* rings = lds + ((T::Bytes(blocks) + 1023) & ~static_cast<size_t>(1023));
+  uint8_t* ring = rings + wave * (STAGES * kPieceBytes);
+
+  auto lds_address = [](const uint8_t* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); };  // the pointer's low half
+  // The tokens: a thread a block. Their loads are asked for first and held in registers while the first
+  // tile's weights are asked for (loads return in order: the tokens are there while the weights still
+  // come), then staged. No branch around a load or a store: past the last block a thread repeats it, the
+  // same bytes to the same place.
+  const int tokens = d.tokens;
+  constexpr int kHeld = 4;
+  struct HeldBlock {
+    U32v4 lower, upper;  // the codes
+    uint32_t scale;      // d8 and the block's sum as F16
+  };
+  HeldBlock held[kHeld];
+  const int last_block = NT * blocks - 1;
+  auto token_block = [&](int index) {
+    const int t = index / blocks, b = index - t * blocks;
+    const int from = min(t, tokens - 1);  // the tokens a group lacks repeat its last: computed and dropped
+    return static_cast<const uint8_t*>(d.y) +
+           (static_cast<int64_t>(from) * d.y_token + static_cast<int64_t>(slot) * d.y_slot + b) * kQ8Block;
+  };
+  auto ask_block = [&](int index, HeldBlock& block) {
+    const uint8_t* src = token_block(min(index, last_block));
+    block.scale = GlobalLoad4(src);
+    block.lower = GlobalLoad16(src + 4);
+    block.upper = GlobalLoad16(src + 20);
+  };
+  auto stage_block = [&](HeldBlock& block, int index) {
+    LLMP_TIE(block.lower);
+    LLMP_TIE(block.upper);
+    LLMP_TIE(block.scale);
+    index = min(index, last_block);
+    const int t = index / blocks, b = index - t * blocks;
+    LdsWrite16(lds_address(codes) + static_cast<uint32_t>(b * T::kCodesBlock + t * 16), block.lower);
+    LdsWrite16(lds_address(codes) + static_cast<uint32_t>(b * T::kCodesBlock + (NT + t) * 16), block.upper);
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum = Dot4(0x01010101, static_cast<int>(block.lower[i]), sum);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum = Dot4(0x01010101, static_cast<int>(block.upper[i]), sum);
+    const float scale = HalfBitsToFloat(block.scale & 0xFFFFu);
+    LdsWrite4(lds_address(d8) + static_cast<uint32_t>(b * T::kScalesBlock + t * 4), scale);
+    LdsWrite4(lds_address(sums) + static_cast<uint32_t>((b >> 3) * T::kSumsSb + t * 32 + (b & 7) * 4), scale * static_cast<float>(sum));
+  };
+
+  // This wave's quarter of K, and this lane's sixteen bytes of each of a piece's nine loads: byte
+  // 1024 j + 16 lane of the 64 rows x 144 bytes lies in row (that / 144), rows past the matrix's end
+  // repeating its last.
+  const int sb_first = wave * nsb / kRowsWaves, sb_end = (wave + 1) * nsb / kRowsWaves;
+  const int pieces = (sb_end - sb_first) * kMatrices;
+  const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
+  const int64_t matrix_block = static_cast<int64_t>(slot) * d.stride_expert;
+  const int token_lane = min(lane, NT - 1);
+  const uint32_t ring_at = lds_address(ring) + static_cast<uint32_t>(lane) * 144u;  // this lane's row of a stage
+  const uint32_t codes_at = lds_address(codes) + static_cast<uint32_t>(token_lane) * 16u;
+  const uint32_t d8_at = lds_address(d8);
+  const uint32_t sums_at = lds_address(sums) + static_cast<uint32_t>(token_lane) * 32u;
+
+  uint32_t offsets[kPieceLoads];
+  const uint8_t* up_tile = nullptr;
+  const uint8_t* gate_tile = nullptr;
+  auto aim = [&](int tile) {
+    const int row0 = tile * kTileRows;
+#pragma unroll
+    for (int j = 0; j < kPieceLoads; ++j) {
+      const int byte = j * (kWave * 16) + lane * 16;
+      const int row = byte / 144;
+      offsets[j] = static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
+                   static_cast<uint32_t>(byte - row * 144);
+    }
+    const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * 144;
+    up_tile = static_cast<const uint8_t*>(d.w) + at;
+    if constexpr (kGlu) gate_tile = static_cast<const uint8_t*>(d.g) + at;
+  };
+  // Piece i: super-block sb_first + i / kMatrices of the up matrix, then of the gate matrix. Past the
+  // wave's last piece its last again (a load is never skipped: the waits count loads).
+  auto issue = [&](int i) {
+    const int piece = min(i, pieces - 1);
+    const int sb = sb_first + piece / kMatrices;
+    const uint8_t* from = (kGlu && (piece & 1) != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * 144;
+    uint8_t* to = ring + (i % STAGES) * kPieceBytes;
+#pragma unroll
+    for (int j = 0; j < kPieceLoads; ++j)
+      __builtin_amdgcn_global_load_lds((GlobalPointer)(from + offsets[j]), (LdsPointer)(to + j * (kWave * 16)), 16, 0, 0);
+  };
+  // (Every wave has pieces: rows of at least four super-blocks; and every workgroup a tile: the grid is no larger.)
+  auto prologue = [&](int tile) {
+    aim(tile);
+#pragma unroll
+    for (int i = 0; i < STAGES - 1; ++i) issue(i);
+  };
+  // The first tile's first piece is asked for before anything else, the tokens next, the rest of the ring after
+  // them: when all but that rest has landed (loads return in order) the tokens are there, and so is the piece the
+  // wave multiplies first.
+  aim(blockIdx.x);
+  issue(0);
+#pragma unroll
+  for (int it = 0; it < kHeld; ++it) ask_block(tid + it * kRowsGroup, held[it]);
+#pragma unroll
+  for (int i = 1; i < STAGES - 1; ++i) issue(i);
+  ROWS_TRACE(1);  // the tokens and the first weights asked for
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kPieceLoads * (STAGES - 2)));
+#pragma unroll
+  for (int it = 0; it < kHeld; ++it) stage_block(held[it], tid + it * kRowsGroup);
+  for (int index = tid + kHeld * kRowsGroup; index <= last_block; index += kRowsGroup) {  // rows too long for that
+    HeldBlock block;
+    ask_block(index, block);
+    asm volatile("s_waitcnt vmcnt(0)");
+    stage_block(block, index);
+  }
+
+  for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int row0 = tile * kTileRows;
+    if (tile != static_cast<int>(blockIdx.x)) prologue(tile);
+    float up_out[NT], gate_out[NT];
+    V4f up_mins[NT / 4], gate_mins[NT / 4];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) up_out[t] = 0.0f, gate_out[t] = 0.0f;
+#pragma unroll
+    for (int tq = 0; tq < NT / 4; ++tq) up_mins[tq] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, gate_mins[tq] = up_mins[tq];
+    LdsBarrier();  // the tokens are staged
+    ROWS_TRACE(2);
+    {
+      for (int i = 0, sb = sb_first; sb < sb_end; ++sb) {
+        const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * 8 * T::kCodesBlock);
+        const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * 8 * T::kScalesBlock);
+        const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
+        issue(i + STAGES - 1);
+        AwaitLoads<kPieceLoads*(STAGES - 1)>();
+        ROWS_TRACE(3 + i);  // piece i landed (the first ten)
+        PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, up_out, up_mins);
+        ++i;
+        if constexpr (kGlu) {
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
+          issue(i + STAGES - 1);
+          AwaitLoads<kPieceLoads*(STAGES - 1)>();
+          ROWS_TRACE(3 + i);
+          PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, gate_out, gate_mins);
+          ++i;
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+      }
+      ROWS_TRACE(13);  // the last piece multiplied
+      AwaitLoads<0>();  // the repeats past the end: nothing may land in the ring after the sums are there
+    }
+    ROWS_TRACE(14);
+    // The four quarters of K meet: [wave][matrix][token][row] floats at the head of each wave's ring.
+    float* mine = reinterpret_cast<float*>(ring);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma clang fp contract(off)
+      mine[t * kTileRows + lane] = up_out[t] - up_mins[t / 4][t % 4];
+      if constexpr (kGlu) mine[(NT + t) * kTileRows + lane] = gate_out[t] - gate_mins[t / 4][t % 4];
+    }
+    __syncthreads();
+    for (int index = tid; index < tokens * kTileRows; index += kRowsGroup) {
+#pragma clang fp contract(off)
+      const int t = index / kTileRows, r = index - t * kTileRows;
+      auto total = [&](int matrix) {
+        const float* at = reinterpret_cast<const float*>(rings) + (matrix * NT + t) * kTileRows + r;
+        constexpr int kRing = STAGES * kPieceBytes / 4;
+        return (at[0] + at[kRing]) + (at[2 * kRing] + at[3 * kRing]);
+      };
+      const float up = total(0);
+      if (row0 + r < d.nrows) {
+        float* dst = d.dst + static_cast<int64_t>(t) * d.dst_token + static_cast<int64_t>(slot) * d.dst_slot;
+        dst[row0 + r] = kGlu ? Glu(d.glu, total(1), up, d.limit) : up;
+      }
+    }
+    __syncthreads();  // the next tile's first loads land where the sums were
+  }
+  ROWS_TRACE_DUMP;
+}
+
+int g_rows_compute_units = 0;
+
+#ifdef LLMP_MMA_TRACE
+}  // namespace
+extern "C" int llmp_hip_trace_set_rows(unsigned long long* buffer) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(g_rows_trace), &buffer, sizeof(buffer)) == hipSuccess ? 0 : -1;
+}
+namespace {
+#endif
+
+template <int NT>
+int StagesFor(int blocks) {
+  const size_t tokens = (Tokens<NT>::Bytes(blocks) + 1023) & ~static_cast<size_t>(1023);
+  for (int stages = 3; stages >= 2; --stages)
+    if (tokens + static_cast<size_t>(kRowsWaves) * stages * kPieceBytes <= kRowsLdsLimit) return stages;
+  return 0;
+}
+
+template <bool kGlu, int NT, int STAGES>
+void LaunchRowsKernel(const VecQArgs& a, dim3 grid, hipStream_t stream) {
+  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQRows<kGlu, NT, STAGES>), static_cast<int>(kRowsLdsLimit), &sized)) return;
+  const size_t lds = ((Tokens<NT>::Bytes(a.d.ncols_x / 32) + 1023) & ~static_cast<size_t>(1023)) +
+                     static_cast<size_t>(kRowsWaves) * STAGES * kPieceBytes;
+  hipLaunchKernelGGL((VecQRows<kGlu, NT, STAGES>), grid, dim3(kRowsGroup), lds, stream, a);
+}
+
+template <bool kGlu, int NT>
+void LaunchRowsStages(const VecQArgs& a, dim3 grid, hipStream_t stream) {
+  StagesFor<NT>(a.d.ncols_x / 32) == 3 ? LaunchRowsKernel<kGlu, NT, 3>(a, grid, stream)
+                                       : LaunchRowsKernel<kGlu, NT, 2>(a, grid, stream);
+}
+
+}  // namespace
+
+// Q4_K, 2 to 8 tokens of a dense or grouped product (no routing ids) over Q8_1 activations, rows of at
+// least four super-blocks (a wave a quarter of K) whose staged tokens leave room for two stages a wave.
+bool RowsTakes(int type, const llmp_vecq_desc& d) {
+  if (type != LLMP_TYPE_Q4_K || d.ids != nullptr || d.tokens < 2 || d.tokens > 8) return false;
+  const int nsb = d.ncols_x / 256;
+  if (nsb < kRowsWaves) return false;
+  return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
+}
+
+void LaunchRows(const VecQArgs& a, hipStream_t stream) {
+  const llmp_vecq_desc& d = a.d;
+  if (g_rows_compute_units == 0) {
+    const int cus = llmp_hip_compute_units();
+    g_rows_compute_units = cus > 0 ? cus : 256;
+  }
+  const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
+  int groups = g_rows_compute_units / d.used;
+  if (groups < 1) groups = 1;
+  if (groups > tiles) groups = tiles;
+  const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(d.used));
+  const bool glu = d.g != nullptr;
+  if (d.tokens <= 4) {
+    glu ? LaunchRowsStages<true, 4>(a, grid, stream) : LaunchRowsStages<false, 4>(a, grid, stream);
+  } else {
+    glu ? LaunchRowsStages<true, 8>(a, grid, stream) : LaunchRowsStages<false, 8>(a, grid, stream);
+  }
+}
+
+}  // namespace llmp_hip

@@ -4,9 +4,11 @@ steps: the timeline behind the tuning of llmp.vecq's several-token form.
 Needs the instrumented build of the library (`make -C llmp_amd/csrc trace`: lib/libllmp_hip_trace.so; the product
 library carries no instrumentation). Lane 0 of every wave stores the 100 MHz clock at sixteen points.
 
-    python -m llmp_amd.mma_timeline [dense TOKENS | sorted TOKENS]
+    python -m llmp_amd.mma_timeline [dense TOKENS | rows TOKENS | sorted TOKENS]
 
-dense: the Q4_K gate/up pair 3840 -> 2 x 15360 at TOKENS tokens (default 8); sorted: the gate/up pair of 128
+dense: the Q4_K gate/up pair 3840 -> 2 x 15360 at TOKENS tokens (default 8) through the 16 x 16 form; rows: the same
+through the row-a-lane form (stamps: start, loads asked for, tokens staged, pieces 1 .. 10 landed, last piece
+multiplied, loads drained, end); sorted: the gate/up pair of 128
 experts 2048 -> 2 x 768, TOKENS tokens (default 512) routed top-8 and sorted by expert."""
 import ctypes as C, os, sys
 import numpy as np, torch
@@ -17,10 +19,11 @@ _lib.SO_PATH = os.path.join(ROOT, "llmp_amd", "lib", "libllmp_hip_trace.so")
 from llmp_amd import ops, synth
 lib = _lib.load()
 lib.llmp_hip_trace_set_mma.argtypes = [C.c_void_p]
+lib.llmp_hip_trace_set_rows.argtypes = [C.c_void_p]
 which = sys.argv[1] if len(sys.argv) > 1 else "dense"
 dev = torch.device("cuda:0")
 D = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-if which == "dense":
+if which in ("dense", "rows"):
     tokens = int(sys.argv[2]) if len(sys.argv) > 2 else 8
     K, N = 3840, 15360
     g0, u0 = D(synth.q4_k_weights(N, K, 101)), D(synth.q4_k_weights(N, K, 102))
@@ -30,7 +33,7 @@ if which == "dense":
     out = torch.empty((tokens, 1, N), dtype=torch.float32, device=dev)
     def launch(i):
         ops.vecq(ops.TYPE_Q4_K, ups[i % copies], q8, K, N, gate=gates[i % copies], glu=ops.GLU_GEGLU, tokens=tokens,
-                 variant=9, out=out)
+                 variant=9 if which == "dense" else 10, out=out)
 else:
     tokens = int(sys.argv[2]) if len(sys.argv) > 2 else 512
     hidden, ffn, experts, used = 2048, 768, 128, 8
@@ -56,15 +59,17 @@ for i in range(20 * copies): launch(i)
 e.record(); torch.cuda.synchronize()
 print(f"{which} {tokens} tokens: {b.elapsed_time(e) / (20 * copies) * 1e3:.2f} us a launch (eager, untraced)")
 trace = torch.zeros((1 << 15) * 16, dtype=torch.int64, device=dev)
-assert lib.llmp_hip_trace_set_mma(trace.data_ptr()) == 0
+assert lib.llmp_hip_trace_set_mma(trace.data_ptr()) == 0 and lib.llmp_hip_trace_set_rows(trace.data_ptr()) == 0
 runs = []
 for r in range(4):
     trace.zero_(); torch.cuda.synchronize()
     launch(r + 1)
     torch.cuda.synchronize()
     runs.append(trace.cpu().numpy().reshape(-1, 16).copy())
-lib.llmp_hip_trace_set_mma(None)
+lib.llmp_hip_trace_set_mma(None); lib.llmp_hip_trace_set_rows(None)
 names = ["start", "first weights asked for", "tokens staged"] + ["step %d done" % (i + 1) for i in range(10)] + ["", "", "wave done"]
+if which == "rows":
+    names = ["start", "loads asked for", "tokens staged"] + ["piece %d landed" % (i + 1) for i in range(10)] + ["last piece multiplied", "loads drained", "wave done"]
 tr = runs[-1]
 tr = tr[tr[:, 0] != 0].astype(np.float64)
 t0 = tr[:, 0].min()
@@ -75,6 +80,8 @@ for s, name in enumerate(names):
     if len(col) == 0: continue
     col = (col - t0) / 100
     print("%-24s waves %5d  min %7.2f  median %7.2f  p90 %7.2f  max %7.2f us" % (name, len(col), col.min(), np.median(col), np.percentile(col, 90), col.max()))
+if which == "rows":
+    raise SystemExit
 steps = tr[:, 3:13]
 ok = (steps != 0).all(axis=1)
 if ok.any():

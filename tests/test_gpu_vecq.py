@@ -87,8 +87,12 @@ def test_long_rows_match_oracle(device, t, k, n, tokens):
     got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
+    # The form that quantizes in the kernel is the flat form: the same bits as the two steps through it.
+    flat = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=6 if tokens == 1 else 7).cpu().numpy()
+    ok, worst = rel_close(flat, want, TOL)
+    assert ok, worst
     fused = ops.vecq_fused(t, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
-    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(fused.view(np.uint32), flat.view(np.uint32))
 
 
 @pytest.mark.parametrize("t", [Q8_0, Q4_K])
@@ -98,6 +102,10 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
+        if name.startswith("rows") and t != Q4_K:  # the row-a-lane form is Q4_K's alone
+            with pytest.raises(ops.KernelFailure):
+                ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
+            continue
         got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
         ok, worst = rel_close(got, want, TOL)
         assert ok, (variant, worst)
@@ -235,39 +243,45 @@ def test_matrix_core_form_against_the_flat_form_and_the_oracle(device, t, k, n, 
     assert ok, worst
 
 
-@pytest.mark.parametrize("k,n,glu", [(2816, 50, False), (3840, 70, True), (8192, 20, True), (768, 33, False)])
-def test_matrix_core_form_values_depend_on_their_own_token_alone(device, k, n, glu):
-    """src/kernels/ggml/vecq.cu:688-693 of the reference, within the matrix-core form: a (token, row) value is the
-    same bits whatever tokens are computed beside it, however many (the kernel stages groups of four, eight or
-    sixteen tokens by the count) and in whatever order."""
-    t, tokens = Q4_K, 16
+@pytest.mark.parametrize("variant,tokens", [(9, 16), (10, 8)])
+@pytest.mark.parametrize("k,n,glu", [(2816, 50, False), (3840, 70, True), (8192, 20, True), (1024, 133, False)])
+def test_matrix_core_forms_values_depend_on_their_own_token_alone(device, variant, tokens, k, n, glu):
+    """src/kernels/ggml/vecq.cu:688-693 of the reference, within each matrix-core form (9: the 16 x 16 instruction,
+    up to sixteen tokens; 10: a weight row a lane, up to eight): a (token, row) value is the same bits whatever
+    tokens are computed beside it, however many (the kernels stage groups of four, eight or sixteen tokens by the
+    count) and in whatever order."""
+    t = Q4_K
     gate, up = make_weights(t, n, k, 311), make_weights(t, n, k, 312)
-    x = synth.activations(tokens, k, 313)
+    x = synth.activations(16, k, 313)[:tokens]
     x[5] *= 30.0
     q8 = ops.quantize_q8_1(dev(x, device))
     wd = dev(up, device)
     kw = dict(gate=dev(gate, device), glu=ops.GLU_GEGLU) if glu else {}
-    full = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=9, **kw).cpu().numpy().reshape(tokens, n)
+    full = ops.vecq(t, wd, q8, k, n, tokens=tokens, variant=variant, **kw).cpu().numpy().reshape(tokens, n)
     for count in (2, 3, 4, 7, 8, 9, 13):
-        part = ops.vecq(t, wd, q8[:count].contiguous(), k, n, tokens=count, variant=9, **kw).cpu().numpy()
+        if count > tokens:
+            continue
+        part = ops.vecq(t, wd, q8[:count].contiguous(), k, n, tokens=count, variant=variant, **kw).cpu().numpy()
         assert np.array_equal(part.reshape(count, n).view(np.uint32), full[:count].view(np.uint32)), count
     order = synth.rng(314).permutation(tokens)
-    mixed = ops.vecq(t, wd, q8[torch.from_numpy(order).to(device)].contiguous(), k, n, tokens=tokens, variant=9, **kw)
+    mixed = ops.vecq(t, wd, q8[torch.from_numpy(order).to(device)].contiguous(), k, n, tokens=tokens, variant=variant, **kw)
     assert np.array_equal(mixed.cpu().numpy().reshape(tokens, n).view(np.uint32), full[order].view(np.uint32))
 
 
-def test_matrix_core_form_sub_block_sums_are_exact_integers(device):
+@pytest.mark.parametrize("variant,k,tokens", [(9, 512, 16), (10, 1024, 8), (10, 1024, 3)])
+def test_matrix_core_forms_sub_block_sums_are_exact_integers(device, variant, k, tokens):
     """With d = 1, dmin = 0 and unit block scales a Q4_K product is the integer sum over sub-blocks of
     sc * sum(q * code): every partial sum stays below 2^24, so F32 holds it exactly and the kernel must return
     exactly the integer (a matrix-core product that rounded inside a sub-block would not)."""
-    k, n, tokens = 512, 48, 16
+    n = 48
     g = synth.rng(321)
     w = synth.q4_k_weights(n, k, 322).reshape(n, k // 256, 144).copy()
     w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), dtype=np.uint8)
     w[:, :, 2:4] = 0
-    w[:, :, 4:16] &= 0x0F  # scales and minimums below 16: two super-blocks of 8 x 32 x 15 x 15 x 127 stay below 2^24
+    w[:, :, 4:16] &= 0x07  # scales and minimums below 8: four super-blocks of 8 x 32 x 7 x 15 x 127 stay below 2^24
     sc = w[:, :, 4:8].astype(np.int64) & 63  # sub-blocks 0 .. 3; 4 .. 7 are the low nibbles of bytes 12 .. 15
     sc = np.concatenate([sc, w[:, :, 12:16].astype(np.int64) & 15], axis=2)  # [n, nsb, 8]
+    assert sc.max() <= 7
     qs = w[:, :, 16:].reshape(n, k // 256, 4, 32)
     q = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, k // 256, 8, 32).astype(np.int64)
     codes = g.integers(-127, 128, size=(tokens, k // 32, 32), dtype=np.int64)
@@ -277,9 +291,40 @@ def test_matrix_core_form_sub_block_sums_are_exact_integers(device):
     sums = np.einsum("rbgk,tbgk->trbg", q, codes.reshape(tokens, k // 256, 8, 32))
     want = np.einsum("trbg,rbg->tr", sums, sc)
     assert np.abs(want).max() < 2 ** 24
-    got = ops.vecq(Q4_K, dev(w.reshape(-1), device), dev(q8, device), k, n, tokens=tokens, variant=9).cpu().numpy()
+    got = ops.vecq(Q4_K, dev(w.reshape(-1), device), dev(q8, device), k, n, tokens=tokens, variant=variant).cpu().numpy()
     assert np.array_equal(got.reshape(tokens, n).astype(np.int64), want)
     assert np.array_equal(got.reshape(tokens, n), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("k,n,tokens", [(1024, 17, 2), (2816, 130, 5), (6144, 64, 8), (16384, 70, 4), (3840, 200, 7)])
+def test_row_a_lane_form_matches_oracle(device, k, n, tokens):
+    """Variant 10 (Q4_K, a weight row a lane, 2 to 8 tokens): dense with and without a GLU, rows that end within a
+    tile of 64, three grouped matrices; and what it refuses: routed products, one token, nine, short rows."""
+    t, rows = Q4_K, 10
+    gate, up = make_weights(t, n, k, 331), make_weights(t, n, k, 332)
+    q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 333))
+    for kw, okw in ((dict(), dict()), (dict(gate=dev(gate, device), glu=ops.GLU_GEGLU), dict(gate=gate, glu=oracle.GLU_GEGLU))):
+        want = oracle.vecq(t, up, q8, k, n, tokens=tokens, **okw)
+        got = ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=tokens, variant=rows, **kw).cpu().numpy()
+        ok, worst = rel_close(got.reshape(tokens, n), want.reshape(tokens, n), TOL, floor=1e-2 if kw else 1e-3)
+        assert ok, (kw.keys(), worst)
+    groups = 3
+    w3 = make_weights(t, groups * n, k, 334).reshape(groups, -1)
+    q83 = oracle.q8_1_quantize(synth.activations(tokens * groups, k, 335))
+    y_row = ops.padded_k(k) // 32
+    kw = dict(tokens=tokens, used=groups, stride_expert=n * (k // 256), y_token=y_row * groups, y_slot=y_row)
+    want = oracle.vecq(t, w3, q83, k, n, **kw)
+    got = ops.vecq(t, dev(w3, device), dev(q83, device), k, n, variant=rows, **kw).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    ids = dev(np.zeros((tokens, 1), dtype=np.int32), device)
+    for bad in (dict(tokens=tokens, ids=ids, used=1, stride_expert=n * (k // 256)), dict(tokens=1), dict(tokens=9)):
+        with pytest.raises(ops.KernelFailure):
+            ops.vecq(t, dev(up, device), dev(oracle.q8_1_quantize(synth.activations(bad["tokens"], k, 336)), device), k, n,
+                     variant=rows, **bad)
+    with pytest.raises(ops.KernelFailure):  # three super-blocks a row: fewer than the workgroup's four waves
+        ops.vecq(t, dev(make_weights(t, 8, 768, 337), device), dev(oracle.q8_1_quantize(synth.activations(2, 768, 338)), device),
+                 768, 8, tokens=2, variant=rows)
 
 
 def test_grouped_matrices_read_their_own_rows(device):
@@ -297,8 +342,10 @@ def test_grouped_matrices_read_their_own_rows(device):
 
 
 def test_tokens_are_independent_and_zero_rows_give_zero(device):
-    """tests/unit/dsv4_fast_test.cc:462-493 of the reference: each token's sums are its
-    one-token product's bit for bit; a zero input row gives zeros."""
+    """tests/unit/dsv4_fast_test.cc:462-493 of the reference: through the flat form each token's sums are its
+    one-token product's bit for bit; through the default form of four tokens (a weight row a lane) a token's sums
+    are the same bits whatever tokens stand beside it, and close to its one-token product's; a zero input row
+    gives zeros in both."""
     t, k, n, tokens = Q4_K, 2816, 96, 4
     gate = make_weights(t, n, k, 91)
     up = make_weights(t, n, k, 92)
@@ -308,11 +355,20 @@ def test_tokens_are_independent_and_zero_rows_give_zero(device):
     wd, gd = dev(up, device), dev(gate, device)
     q8 = ops.quantize_q8_1(dev(x, device))
     got = ops.vecq(t, wd, q8, k, n, gate=gd, tokens=tokens, glu=ops.GLU_GEGLU).cpu().numpy()
-    assert np.all(got[0] == 0)
+    flat = ops.vecq(t, wd, q8, k, n, gate=gd, tokens=tokens, glu=ops.GLU_GEGLU, variant=7).cpu().numpy()
+    assert np.all(got[0] == 0) and np.all(flat[0] == 0)
     for i in range(tokens):
         solo_q8 = ops.quantize_q8_1(dev(x[i:i + 1], device))
         solo = ops.vecq(t, wd, solo_q8, k, n, gate=gd, tokens=1, glu=ops.GLU_GEGLU).cpu().numpy()
-        assert np.array_equal(solo[0].view(np.uint32), got[i].view(np.uint32)), i
+        assert np.array_equal(solo[0].view(np.uint32), flat[i].view(np.uint32)), i
+        ok, worst = rel_close(got[i], solo[0], 1e-5, floor=1.0)
+        assert ok, (i, worst)
+        # Token i beside another token, in the other place: the default form's own bits again.
+        j = (i + 1) % tokens
+        pair_q8 = ops.quantize_q8_1(dev(x[[j, i]], device))
+        pair = ops.vecq(t, wd, pair_q8, k, n, gate=gd, tokens=2, glu=ops.GLU_GEGLU).cpu().numpy()
+        assert np.array_equal(pair[1].view(np.uint32), got[i].view(np.uint32)), i
+        assert np.array_equal(pair[0].view(np.uint32), got[j].view(np.uint32)), i
 
 
 def test_guard_bytes_stay_untouched_and_refusals_queue_nothing(device):
@@ -359,8 +415,12 @@ def test_legacy_blocks_dense_match_oracle(device, t, k, n, tokens):
     got = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens).cpu().numpy()
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
+    # The form that quantizes in the kernel is the flat form: the same bits as the two steps through it.
+    flat = ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=6 if tokens == 1 else 7).cpu().numpy()
+    ok, worst = rel_close(flat, want, TOL)
+    assert ok, worst
     fused = ops.vecq_fused(t, dev(w, device), dev(x, device), k, n, tokens=tokens).cpu().numpy()
-    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(fused.view(np.uint32), flat.view(np.uint32))
     # A token's values do not depend on the tokens beside it (one token a pass and four).
     alone = ops.vecq(t, dev(w, device), dev(q8[tokens - 1:], device), k, n).cpu().numpy()
     assert np.array_equal(alone[0].view(np.uint32), got[tokens - 1].view(np.uint32))
