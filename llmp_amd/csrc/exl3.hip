@@ -75,6 +75,28 @@ __device__ __forceinline__ _Float16 SumHalves(uint32_t x) {
   return lo + hi;
 }
 
+// Two 3INST or MCG values at once: each one's halves added (the same F16 addition as SumHalves) straight into a
+// half of one dword, by the instruction's operand selects: an instruction a value, and none to pack the results
+// (left to itself the compiler permutes the four halves into two dwords and adds those: three for two values).
+template <int CB>
+__device__ __forceinline__ uint32_t CodebookPair(uint32_t state0, uint32_t state1) {
+  static_assert(CB == LLMP_EXL3_3INST || CB == LLMP_EXL3_MCG, "MUL1 values are not sums of halves");
+  const uint32_t x0 = CB == LLMP_EXL3_3INST ? MulState<89226354u>(state0, 64248484u) : MulState<0xCBAC1FEDu>(state0, 0u);
+  const uint32_t x1 = CB == LLMP_EXL3_3INST ? MulState<89226354u>(state1, 64248484u) : MulState<0xCBAC1FEDu>(state1, 0u);
+  const uint32_t y0 = __builtin_amdgcn_bitop3_b32(x0, 0x8FFF8FFFu, 0x3B603B60u, 0x6A);  // (x & mask) ^ bias
+  const uint32_t y1 = __builtin_amdgcn_bitop3_b32(x1, 0x8FFF8FFFu, 0x3B603B60u, 0x6A);
+  uint32_t pair;
+  // (A wait state after each: the result of an instruction that writes half a register may not be read by the
+  // next one, and inside these statements the compiler does not see that it is.)
+  asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\ts_nop 0"
+      : "=v"(pair)
+      : "v"(y0));
+  asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\ts_nop 0"
+      : "+v"(pair)
+      : "v"(y1));
+  return pair;
+}
+
 // decode_exl3.cc:41-66
 template <int CB>
 __device__ __forceinline__ _Float16 Codebook(uint32_t state) {
@@ -249,6 +271,7 @@ __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, 
 // ------------------------------------------------------------------- product
 
 constexpr int kRingDepth = 4;  // K steps of a 128-column block in flight a wave
+constexpr int kFusedRows = 4;  // up to here the product transforms its input itself
 constexpr int kProductWaves = 8;
 constexpr int kOperandBytes = 16 * 128 * 2;  // a wave's transformed activations of one 128 block of K
 constexpr int kReduceBytes = kProductWaves * 32 * 64 * 4;
@@ -268,6 +291,103 @@ struct ProductSides {  // one or two linears a launch (grid z)
   float* partial[2];
 };
 
+// LDS accesses written as instructions, for the product's loop: while a global_load_lds is in flight the
+// compiler makes every access of LDS it knows of wait until all of them have landed (it cannot tell which the
+// access could alias), the ring's newest fetch included, and the ring would never overlap a fetch with a decode.
+// The loop orders its reads and the loads itself: LdsWaited, then Tie on every register read.
+#define LLMP_TIE(x) asm volatile("" : "+v"(x))
+template <int OFFSET>
+__device__ __forceinline__ uint32_t LdsRead4(uint32_t at) {
+  uint32_t v;
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(OFFSET));
+  return v;
+}
+__device__ __forceinline__ void LdsWrite4(uint32_t at, uint32_t value) { asm volatile("ds_write_b32 %0, %1" : : "v"(at), "v"(value)); }
+__device__ __forceinline__ void LdsWaited() { asm volatile("s_waitcnt lgkmcnt(0)"); }
+// The same for the few loads from global memory into registers inside that loop: the compiler's own wait for one
+// is a wait for every load in flight, the ring's included.
+__device__ __forceinline__ uint32_t GlobalLoad4(const void* from) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(from));
+  return v;
+}
+template <int LEFT>
+__device__ __forceinline__ void LoadsWaited() {
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (LEFT & 0xF) | ((LEFT >> 4) << 14));
+  asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ uint32_t LdsAddress(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
+
+// Where a lane finds the 32 bits of a tile's stream that end at bit `end` (counted a period ahead, so never
+// negative): the word holding the last bit, the word before it (circular), and the shift that brings bit `end`
+// down to bit 0 of the pair.
+template <int BITS>
+struct Window {
+  uint32_t high, low;  // byte offsets in the tile
+  uint32_t shift;
+};
+template <int BITS>
+__device__ __forceinline__ Window<BITS> WindowAt(int end) {
+  constexpr int words = BITS * 8;
+  const int i1 = ((end - 1) >> 5) % words;
+  Window<BITS> w;
+  w.low = static_cast<uint32_t>(i1) * 4u;
+  w.high = static_cast<uint32_t>((i1 + words - 1) % words) * 4u;
+  w.shift = static_cast<uint32_t>((32 - (end & 31)) & 31);
+  return w;
+}
+
+// The windows of a lane's four positions first .. first + 3: one of 16 + 3 BITS bits up to five bits a value
+// (within 32), else one a pair of positions (16 + BITS bits each).
+template <int BITS>
+struct Windows {
+  static constexpr int kCount = BITS <= 5 ? 1 : 2;
+  Window<BITS> w[kCount];
+};
+template <int BITS>
+__device__ __forceinline__ Windows<BITS> WindowsOf(int first) {
+  Windows<BITS> out;
+  if constexpr (BITS <= 5) {
+    out.w[0] = WindowAt<BITS>((first + 4) * BITS + 256 * BITS);
+  } else {
+    out.w[0] = WindowAt<BITS>((first + 2) * BITS + 256 * BITS);
+    out.w[1] = WindowAt<BITS>((first + 4) * BITS + 256 * BITS);
+  }
+  return out;
+}
+
+// The codebook values of a lane's four positions from the words of its windows (high, low a window).
+template <int CB, int BITS>
+__device__ __forceinline__ Half4 DecodeWindows(const Windows<BITS>& at, const uint32_t (&words)[2 * Windows<BITS>::kCount]) {
+  Half4 v;
+  if constexpr (BITS <= 5 && CB != LLMP_EXL3_MUL1) {
+    const uint32_t window = __builtin_amdgcn_alignbit(words[0], words[1], at.w[0].shift);
+    uint2 pairs;
+    pairs.x = CodebookPair<CB>((window >> (3 * BITS)) & 0xFFFFu, (window >> (2 * BITS)) & 0xFFFFu);
+    pairs.y = CodebookPair<CB>((window >> BITS) & 0xFFFFu, window & 0xFFFFu);
+    return __builtin_bit_cast(Half4, pairs);
+  } else if constexpr (BITS <= 5) {
+    const uint32_t window = __builtin_amdgcn_alignbit(words[0], words[1], at.w[0].shift);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = Codebook<CB>((window >> ((3 - j) * BITS)) & 0xFFFFu);
+  } else if constexpr (CB != LLMP_EXL3_MUL1) {
+    uint2 pairs;
+    const uint32_t first = __builtin_amdgcn_alignbit(words[0], words[1], at.w[0].shift);
+    const uint32_t second = __builtin_amdgcn_alignbit(words[2], words[3], at.w[1].shift);
+    pairs.x = CodebookPair<CB>((first >> BITS) & 0xFFFFu, first & 0xFFFFu);
+    pairs.y = CodebookPair<CB>((second >> BITS) & 0xFFFFu, second & 0xFFFFu);
+    return __builtin_bit_cast(Half4, pairs);
+  } else {
+#pragma unroll
+    for (int pair = 0; pair < 2; ++pair) {
+      const uint32_t window = __builtin_amdgcn_alignbit(words[2 * pair], words[2 * pair + 1], at.w[pair].shift);
+      v[2 * pair] = Codebook<CB>((window >> BITS) & 0xFFFFu);
+      v[2 * pair + 1] = Codebook<CB>(window & 0xFFFFu);
+    }
+  }
+  return v;
+}
+
 template <int CB, int BITS, bool kFused>
 __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const ProductSides sides, int m, int n, int k,
                                                                    int blocks_per_wave) {
@@ -280,7 +400,9 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const Produc
   constexpr int kTileBytes = BITS * 32;
   constexpr int kStepBytes = 8 * kTileBytes;  // a 128-column block's tiles of one K step
   constexpr int kLoads = (kStepBytes + 1023) / 1024;
-  constexpr int kRingBytes = kRingDepth * kLoads * 1024;
+  constexpr int kStageBytes = kLoads * 1024;
+  constexpr int kRingBytes = kRingDepth * kStageBytes;
+  constexpr int kWords = 2 * Windows<BITS>::kCount;  // a lane reads of a tile
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -292,12 +414,16 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const Produc
   const int first = min(slice * blocks_per_wave, k / 128) * 8;  // in K steps of 16
   const int last = min((slice + 1) * blocks_per_wave, k / 128) * 8;
   const Place p = PlaceOf(lane);
+  const Windows<BITS> windows = WindowsOf<BITS>(p.first);
   const int64_t row_bytes = static_cast<int64_t>(n / 16) * kTileBytes;
   const uint8_t* source = trellis + static_cast<int64_t>(block) * kStepBytes;
+  const uint32_t ring_at = LdsAddress(ring);
 
+  // Step `step`'s tiles into its stage of the ring; past the wave's last step the last again (a load is never
+  // skipped: the waits count loads).
   auto fetch = [&](int step) {
-    const uint8_t* from = source + step * row_bytes;
-    uint8_t* to = ring + (step % kRingDepth) * (kLoads * 1024);
+    const uint8_t* from = source + min(step, last - 1) * row_bytes;
+    uint8_t* to = ring + (step % kRingDepth) * kStageBytes;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       if (i * 1024 + lane * 16 < kStepBytes) {
@@ -306,68 +432,133 @@ __global__ __launch_bounds__(kProductWaves * 64) void ProductKernel(const Produc
       }
     }
   };
+  // Step `step`'s words of this lane's windows of the eight tiles, asked for (they are there after LdsWaited).
+  auto ask = [&](int step, uint32_t (&words)[8][kWords]) {
+    const uint32_t stage = ring_at + static_cast<uint32_t>((step % kRingDepth) * kStageBytes);
+#pragma unroll
+    for (int w = 0; w < Windows<BITS>::kCount; ++w) {
+      const uint32_t high = stage + windows.w[w].high, low = stage + windows.w[w].low;
+      words[0][2 * w] = LdsRead4<0 * kTileBytes>(high), words[0][2 * w + 1] = LdsRead4<0 * kTileBytes>(low);
+      words[1][2 * w] = LdsRead4<1 * kTileBytes>(high), words[1][2 * w + 1] = LdsRead4<1 * kTileBytes>(low);
+      words[2][2 * w] = LdsRead4<2 * kTileBytes>(high), words[2][2 * w + 1] = LdsRead4<2 * kTileBytes>(low);
+      words[3][2 * w] = LdsRead4<3 * kTileBytes>(high), words[3][2 * w + 1] = LdsRead4<3 * kTileBytes>(low);
+      words[4][2 * w] = LdsRead4<4 * kTileBytes>(high), words[4][2 * w + 1] = LdsRead4<4 * kTileBytes>(low);
+      words[5][2 * w] = LdsRead4<5 * kTileBytes>(high), words[5][2 * w + 1] = LdsRead4<5 * kTileBytes>(low);
+      words[6][2 * w] = LdsRead4<6 * kTileBytes>(high), words[6][2 * w + 1] = LdsRead4<6 * kTileBytes>(low);
+      words[7][2 * w] = LdsRead4<7 * kTileBytes>(high), words[7][2 * w + 1] = LdsRead4<7 * kTileBytes>(low);
+    }
+  };
+  auto landed = [&](uint32_t (&words)[8][kWords]) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+      for (int w = 0; w < kWords; ++w) LLMP_TIE(words[t][w]);
+  };
 
   V4f acc[8];
 #pragma unroll
   for (int t = 0; t < 8; ++t) acc[t] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
   // The activations' operand: token l % 16, k slots in the lane group's row order.
-  const uint8_t* my_operand = operand + min(p.n, m - 1) * 256 + 4 * p.g;
+  const uint32_t my_operand = LdsAddress(operand) + static_cast<uint32_t>(min(p.n, m - 1) * 256 + 4 * p.g);
   const uint16_t* my_row = x + static_cast<int64_t>(min(p.n, m - 1)) * k + 2 * p.g;
 
-  for (int s = first; s < min(first + kRingDepth - 1, last); ++s) fetch(s);
-  for (int step = first; step < last; ++step) {
-    if (kFused && (step & 7) == 0) {
-      // The wave's next 128 values of every token, transformed as the input transform does.
-      const int at = (step >> 3) * 128 + 2 * lane;
-      const uint32_t sc = *reinterpret_cast<const uint32_t*>(suh + at);
-      const float sa = HalfBitsToFloat(sc & 0xFFFFu), sb = HalfBitsToFloat(sc >> 16);
-      for (int t = 0; t < m; ++t) {
-        const uint32_t v = *reinterpret_cast<const uint32_t*>(x + static_cast<int64_t>(t) * k + at);
-        float a = HalfBitsToFloat(v & 0xFFFFu) * sa;
-        float b = HalfBitsToFloat(v >> 16) * sb;
-        Hadamard128(a, b, lane);
-        a *= kHadamardScale;
-        b *= kHadamardScale;
-        const uint32_t packed = FloatToHalfBits(a) | (FloatToHalfBits(b) << 16);
-        *reinterpret_cast<uint32_t*>(operand + t * 256 + 4 * lane) = packed;
-        if (block == 0) *reinterpret_cast<uint32_t*>(a_had + static_cast<int64_t>(t) * k + at) = packed;
-      }
-      __builtin_amdgcn_wave_barrier();
-      asm volatile("" ::: "memory");
-    }
-    uint32_t x01, x89;
-    if constexpr (kFused) {
-      x01 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32);
-      x89 = *reinterpret_cast<const uint32_t*>(my_operand + (step & 7) * 32 + 16);
-    } else {
-      x01 = *reinterpret_cast<const uint32_t*>(my_row + step * 16);
-      x89 = *reinterpret_cast<const uint32_t*>(my_row + step * 16 + 8);
-    }
-    Half4 xv;
-    xv[0] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 & 0xFFFFu));
-    xv[1] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 >> 16));
-    xv[2] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 & 0xFFFFu));
-    xv[3] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 >> 16));
-    if (p.n >= m) xv = Half4{0, 0, 0, 0};
-    const int ahead = step + kRingDepth - 1;
-    if (ahead < last) {
-      fetch(ahead);
-      // All but the newest `kLoads * (kRingDepth - 1)` loads have landed: this step's tiles.
-      __builtin_amdgcn_s_waitcnt(0x0F70 | ((kLoads * (kRingDepth - 1)) & 0xF) | (((kLoads * (kRingDepth - 1)) >> 4) << 14));
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-    }
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-    const uint32_t* tiles = reinterpret_cast<const uint32_t*>(ring + (step % kRingDepth) * (kLoads * 1024));
+  if (first < last) {
+    // The ring runs kRingDepth - 1 steps ahead of the words read, the words one step ahead of the decode. Every
+    // step asks for the same loads in the same order (the next step's two activation words, then a stage of the
+    // ring; with kFused the next block's activations in place of the words), so that a wait can count them.
+    uint32_t words[2][8][kWords];
+    uint32_t xa[2] = {0, 0}, xb[2] = {0, 0};  // a step's activation words (unfused: from global memory)
+    uint32_t held[kFusedRows + 1];             // the next block's scales and activations (fused)
+    auto ask_block = [&](int step) {           // of K step `step`'s 128 block
+      const int at = min(step >> 3, k / 128 - 1) * 128 + 2 * lane;
+      held[0] = GlobalLoad4(suh + at);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const uint32_t* tile = tiles + t * (BITS * 8);
-      const Half4 wv = DecodeFour<CB, BITS>(p.first, [&](int i) { return tile[i]; });
-      // D[token][n] += sum_j xv[token][j] wv[j][n]: first operand rows are tokens.
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(xv, wv, acc[t], 0, 0, 0);
+      for (int t = 0; t < kFusedRows; ++t) held[1 + t] = GlobalLoad4(x + static_cast<int64_t>(min(t, m - 1)) * k + at);
+    };
+    if constexpr (kFused) {
+      ask_block(first);
+    } else {
+      xa[0] = GlobalLoad4(my_row + first * 16);
+      xb[0] = GlobalLoad4(my_row + first * 16 + 8);
     }
-    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int s = 0; s < kRingDepth - 1; ++s) fetch(first + s);
+    LoadsWaited<kLoads*(kRingDepth - 2)>();
+    ask(first, words[0]);
+    auto one = [&](int step, int parity) {
+      uint32_t (&mine)[8][kWords] = words[parity];
+      uint32_t (&next)[8][kWords] = words[parity ^ 1];
+      if (kFused && ((step & 7) == 0 || step == first)) {
+        // The wave's 128 values of every token for this block of K, transformed as the input transform does
+        // (asked for a block ago), and the next block's asked for.
+        const int at = (step >> 3) * 128 + 2 * lane;
+        // (They were asked for before the ring stages the waits have since counted in: they are there.)
+#pragma unroll
+        for (int i = 0; i <= kFusedRows; ++i) LLMP_TIE(held[i]);
+        const float sa = HalfBitsToFloat(held[0] & 0xFFFFu), sb = HalfBitsToFloat(held[0] >> 16);
+        LdsWaited();  // the last block's operand has been read
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < kFusedRows; ++t) {
+          if (t < m) {
+            const uint32_t v = held[1 + t];
+            float a = HalfBitsToFloat(v & 0xFFFFu) * sa;
+            float b = HalfBitsToFloat(v >> 16) * sb;
+            Hadamard128(a, b, lane);
+            a *= kHadamardScale;
+            b *= kHadamardScale;
+            const uint32_t packed = FloatToHalfBits(a) | (FloatToHalfBits(b) << 16);
+            LdsWrite4(LdsAddress(operand) + static_cast<uint32_t>(t * 256 + 4 * lane), packed);
+            if (block == 0) *reinterpret_cast<uint32_t*>(a_had + static_cast<int64_t>(t) * k + at) = packed;
+          }
+        }
+        ask_block(step + 8);
+        LdsWaited();
+        __builtin_amdgcn_wave_barrier();
+      }
+      uint32_t x01, x89;
+      if constexpr (kFused) {
+        const uint32_t at = my_operand + static_cast<uint32_t>((step & 7) * 32);
+        x01 = LdsRead4<0>(at);
+        x89 = LdsRead4<16>(at);
+      } else {
+        xa[parity ^ 1] = GlobalLoad4(my_row + min(step + 1, last - 1) * 16);
+        xb[parity ^ 1] = GlobalLoad4(my_row + min(step + 1, last - 1) * 16 + 8);
+      }
+      // The ring's next stage asked for; the stage after this step's has landed (and this step's activation
+      // words): its words asked for, and this step's words (asked for a step ago) decoded while those come.
+      fetch(step + kRingDepth - 1);
+      LoadsWaited<kLoads*(kRingDepth - 2) + (kFused ? 0 : 2)>();
+      LdsWaited();
+      landed(mine);
+      if constexpr (kFused) {
+        LLMP_TIE(x01);
+        LLMP_TIE(x89);
+      } else {
+        LLMP_TIE(xa[parity]);
+        LLMP_TIE(xb[parity]);
+        x01 = xa[parity], x89 = xb[parity];
+      }
+      ask(step + 1, next);
+      if (p.n >= m) x01 = 0, x89 = 0;
+      Half4 xv;
+      xv[0] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 & 0xFFFFu));
+      xv[1] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x01 >> 16));
+      xv[2] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 & 0xFFFFu));
+      xv[3] = __builtin_bit_cast(_Float16, static_cast<uint16_t>(x89 >> 16));
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const Half4 wv = DecodeWindows<CB, BITS>(windows, mine[t]);
+        // D[token][n] += sum_j xv[token][j] wv[j][n]: first operand rows are tokens.
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(xv, wv, acc[t], 0, 0, 0);
+      }
+    };
+    for (int step = first; step < last; step += 2) {
+      one(step, 0);
+      if (step + 1 < last) one(step + 1, 1);
+    }
+    LdsWaited();  // the words asked for past the end
+    LoadsWaited<0>();
   }
 
   // The waves' sums through LDS (over the rings, which every wave has left), added in wave
@@ -444,8 +635,6 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
   hipLaunchKernelGGL((ReconstructKernel<CB, BITS>), grid, dim3(256), 0, stream,
                      static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
-
-constexpr int kFusedRows = 4;  // up to here the product transforms its input itself
 
 template <int CB, int BITS, bool kFused>
 void LaunchProduct(const llmp_exl3_weights& w, const ProductSides& sides, int count, int m, int slices,
