@@ -34,8 +34,9 @@ __device__ __forceinline__ float Bf16BitsToFloat(uint32_t bits) {
 }
 __device__ __forceinline__ uint32_t FloatToBf16Bits(float v) {
   const uint32_t x = __builtin_bit_cast(uint32_t, v);
-  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x40u;
-  return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+  const uint32_t quiet = (x >> 16) | 0x40u;                          // a NaN keeps its payload's top bits
+  const uint32_t nearest = (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;  // ties to even
+  return __builtin_isnan(v) ? quiet : nearest;
 }
 // E8M0: 2^(bits - 127); 0 is 2^-127 (a float subnormal), 0xFF NaN.
 __device__ __forceinline__ float E8m0ToFloat(uint32_t bits) {

@@ -23,6 +23,9 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 #include "llmp_hip.h"
 
@@ -236,19 +239,12 @@ __global__ __launch_bounds__(256) void GemvKernel(const uint8_t* __restrict__ co
 
 // ------------------------------------------------------------------ GEMM
 
-typedef int V8i __attribute__((ext_vector_type(8)));
-typedef float V4f __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void* LdsPointer;
-typedef const __attribute__((address_space(1))) void* GlobalPointer;
 
 constexpr int kTileM = 256;             // activation rows a workgroup
 constexpr int kStepK = 128;             // codes a K step
-constexpr int kGemmThreads = 512;       // 8 waves: 4 along m, 2 along n
-constexpr int kGroupThreads = 256;      // a group: the four waves with the same position along n
 constexpr int kRingA = 2;               // stages of activation tiles in LDS
 constexpr int kRingB = 3;               // stages of weight tiles
 constexpr int kTileABytes = kTileM * kStepK;  // 32 KB
-constexpr int kLoadsA = kTileABytes / 16 / kGroupThreads;  // 8 a thread of group 1 a stage
 constexpr int kScaleStageBytes = 1024;  // two atoms a stage, either operand
 
 struct GemmArgs {
@@ -302,237 +298,337 @@ struct GemmLds {
 // (p % 8) ^ ((row / 2) % 8). Rows past the operand's end repeat the last (their results are
 // never stored).
 
-// A 16-row fragment: the lane's two 16-byte chunks, at lo and hi bytes into it.
-__device__ __forceinline__ V8i ReadFragment(const uint8_t* fragment, int lo_at, int hi_at) {
-  const U32x4 lo = *reinterpret_cast<const U32x4*>(fragment + lo_at);
-  const U32x4 hi = *reinterpret_cast<const U32x4*>(fragment + hi_at);
-  V8i v;
-  v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
-  v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
-  return v;
-}
-
 // Waits until at most `left` of this wave's vector-memory operations are outstanding.
 template <int LEFT>
 __device__ __forceinline__ void AwaitLoads() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (LEFT & 15) | ((LEFT >> 4) << 14));
 }
 
-// D tile of 256 activation rows by 32 WN weight rows, K step 128. Wave (wm, wn) of 4 x 2 owns
-// 64 x 16 WN of it: WN x 4 MFMA tiles, the weights as the first operand.
+// D tile of 256 activation rows by 32 WN weight rows, K step 128, by WM x 2 waves: wave (wm, wn) owns 256 / WM
+// activation rows by 16 WN weight rows, the weights as the first operand of v_mfma_scale_f32_16x16x128_f8f6f4.
 //
-// The two waves of a SIMD (wn 0 and 1: the hardware places waves 0-3 and 4-7 of a workgroup
-// one on each SIMD) work half a step apart. A step of a wave is a read phase (its 4 + WN
-// fragments and their scales from LDS into registers) and a multiply phase (4 WN MFMAs);
-// every phase ends at a workgroup barrier, and group 1 sits the first phase out, so that
-// while one wave of a SIMD multiplies the other reads: the matrix pipe and LDS both stay
-// busy. Phases, counted from 0: group 0 reads step s in phase 2 s and multiplies in 2 s + 1,
-// group 1 reads in 2 s + 1 and multiplies in 2 s + 2.
+// Tiles come by global_load_lds into rings in LDS, activations 2 stages and weights 3 (every weight byte is a
+// compulsory HBM miss for the first workgroup that asks, activations mostly hit L2). In iteration s, after its
+// barrier: activations s + 2 are asked for (into the stage step s used: every wave read its fragments of it during
+// iteration s - 1), then weights s + 3; the fragments of step s + 1 are read while step s is multiplied, an
+// activation fragment's registers refilled as soon as its row of products is issued, a weight fragment's after its
+// last product; and at the end all loads but the weights just asked for have landed, so that after the next barrier
+// step s + 2 is whole in LDS. One barrier a step; no wave waits for another inside a step.
 //
-// Tiles come by global_load_lds, issued between the MFMAs of the multiply phases (the only
-// time a wave has issue slots to spare): group 1 brings activations s + 2 while it
-// multiplies step s, into the stage step s used (ring of 2; free since the barrier that ended
-// phase 2 s + 1), and waits for them at the end of its next read phase, before the barrier
-// that opens phase 2 s + 4. Group 0 brings weights s + 2 while it multiplies step s, into the
-// stage step s - 1 used (ring of 3: every weight byte is a compulsory HBM miss for the first
-// workgroup that asks, activations mostly hit L2), and waits for weights s + 1, leaving s + 2
-// in flight, before the barrier that ends its multiply phase.
-template <int WN>
-__global__ __launch_bounds__(kGemmThreads, 1) void GemmKernel(const GemmArgs a) {
+// What a step costs, measured with parts of the loop taken out (M 2048, N 12288, K 4096; shader clock 2.0 GHz under
+// this kernel): its 48 products alone 0.99 us a wave that is alone on its SIMD, 41 cycles a product where the matrix
+// pipe's eight passes are 32 (the scales are loaded by an instruction of their own before each product); and nothing
+// else of the same wave is issued meanwhile, so the 16 loads to LDS add 0.19 us (about 20 cycles each), the 42 reads
+// of LDS 0.11, the barrier and the waits 0.09: 1.35 us. Two waves a SIMD (WM = 4) do issue into each other's
+// products, but eight waves read 216 KB of LDS a step where four read 168, and LDS's 128 bytes a cycle then bound the
+// step at 1.29 us; with the smaller tile's poorer tail that is no faster, and four waves are the default.
+//
+// Reads of LDS are written as instructions (the compiler would make each wait for every load into LDS in flight): a
+// wave waits for them itself at the end of an iteration.
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+// (a register number or an instruction's offset field).
+template <class F, int... I>
+__device__ __forceinline__ void StaticForEach(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void StaticFor(F&& f) {
+  StaticForEach(f, std::make_integer_sequence<int, N>{});
+}
+
+// The loop's registers are named, not allocated: left to itself the compiler copies an accumulator before every
+// product whose neighbours are loads (its D and C end up in different registers) and builds each 32-byte operand
+// out of two 16-byte reads with eight moves, all of them on the one pipe that also issues the products.
+//   a[4 t .. 4 t + 3], t = 8 i + j        product (i, j)'s sums (192 of the upper registers at WN = 6); numbers for WM = 2
+//   v[128 + 8 j ..], j < 8                activation fragment j: the lane's chunks g and 4 + g of row 16 j + r
+//   v[192 + 8 i ..], i < WN               weight fragment i
+//   v[240 + j], v[248 + i]                their scales, a byte each
+// The compiler keeps to v0 .. v127 (amdgpu_num_vgpr) and is told once that the kernel uses the rest; what it may
+// not see is listed with each helper.
+#ifndef LLMP_GEMM_WAVES_M
+#define LLMP_GEMM_WAVES_M 2
+#endif
+constexpr int kGemmWavesM = LLMP_GEMM_WAVES_M;
+constexpr int kGemmCompilerVgprs = kGemmWavesM == 2 ? 128 : 64;
+
+// WM waves share the tile's 256 activation rows (2 waves of weights each): 2, a wave a SIMD with 448 registers, or 4, two
+// waves a SIMD with 256 each. A wave's instruction after a matrix product is not issued before the product is (nearly)
+// through the pipe, so a wave that is alone on its SIMD pays for every load and read with the pipe idle; a second wave
+// fills that time, but each of the eight then reads 20 KB of fragments a step where each of four reads 28 KB.
+template <int WM, int WN>
+struct GemmRegs {
+  static constexpr int kXFrags = 16 / WM;                    // 16-row activation fragments a wave
+  static constexpr int kCompilerVgprs = kGemmCompilerVgprs;  // v0 .. for the compiler
+  static_assert(WM == kGemmWavesM, "the attribute that holds the compiler to them is not a template's");
+  static constexpr int kX = kCompilerVgprs;
+  static constexpr int kW = kX + 8 * kXFrags;
+  static constexpr int kXScale = kW + 8 * WN;
+  static constexpr int kWScale = kXScale + kXFrags;
+  static constexpr int kTop = kWScale + WN;
+  static constexpr int kSums = 4 * kXFrags * WN;
+  static_assert(WM == 2 ? (kTop <= 254 && kSums <= 192) : (kTop <= 160 && kSums <= 96), "the register file");
+};
+
+// Fragment registers REG .. REG + 3 from LDS. In flight until the wave's next s_waitcnt lgkmcnt(0).
+template <int REG, int OFFSET>
+__device__ __forceinline__ void LdsToRegs16(uint32_t at) {
+  asm volatile("ds_read_b128 v[%1:%1+3], %0 offset:%2" ::"v"(at), "n"(REG), "n"(OFFSET));
+}
+template <int REG, int OFFSET>
+__device__ __forceinline__ void LdsToReg1(uint32_t at) {
+  asm volatile("ds_read_u8 v[%1], %0 offset:%2" ::"v"(at), "n"(REG), "n"(OFFSET));
+}
+// 16 bytes a lane from `base` + `offset` (a lane's own) to LDS at `to` + 16 lane, without a register between.
+__device__ __forceinline__ void GlobalToLds16(const uint8_t* base, uint32_t offset, uint32_t to) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(to), "v"(offset), "s"(base));
+}
+
+// sums(T) += weights(I) x activations(J), both scaled.
+template <class R, int T, int I, int J>
+__device__ __forceinline__ void ScaledProduct() {
+  asm volatile(
+      "v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%0+3], v[%1:%1+7], v[%2:%2+7], a[%0:%0+3], v[%3], v[%4] op_sel_hi:[0,0,0]" ::"n"(
+          T * 4),
+      "n"(R::kW + 8 * I), "n"(R::kX + 8 * J), "n"(R::kWScale + I), "n"(R::kXScale + J));
+}
+template <int REG>
+__device__ __forceinline__ void ClearSum() {
+  asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(REG));
+}
+template <int REG>
+__device__ __forceinline__ float ReadSum() {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(REG));
+  return v;
+}
+
+template <int WM, int WN>
+__global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCompilerVgprs))) void GemmKernel(
+    const GemmArgs a) {
   using L = GemmLds<WN>;
+  using R = GemmRegs<WM, WN>;
   constexpr int kTileN = L::kTileN;
-  constexpr int kLoadsB = L::kTileBBytes / 16 / kGroupThreads;  // WN a thread of group 0 a stage
-  constexpr int kLoadEvery = WN / 2;  // MFMAs between two loads: 8 loads fit 4 WN MFMAs
-  static_assert(kLoadsB <= kLoadsA && kLoadsA * kLoadEvery <= 4 * WN, "the loads do not fit a multiply phase");
+  constexpr int kThreads = WM * 128;
+  constexpr int kXFrags = R::kXFrags;
+  constexpr int kLoadsA = kTileABytes / 16 / kThreads;     // 8 or 4 a thread a stage
+  constexpr int kLoadsB = L::kTileBBytes / 16 / kThreads;  // WN or half of it
+  static_assert(L::kTileBBytes % (16 * kThreads) == 0 && kLoadsA + 1 + kLoadsB <= kXFrags * WN, "load slots");
+  // The kernel's register counts cover the named ones.
+  if constexpr (WM == 2) {
+    asm volatile("" ::: "v253", "a191");
+  } else {
+    asm volatile("" ::: "v159", "a95");
+  }
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   GEMM_TRACE(0);  // the wave's start
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave & 3, wn = wave >> 2;
-  const int group = wn;
+  const int wm = wave % WM, wn = wave / WM;  // (the two waves of a SIMD, w and w + 4, differ in both)
   const int r = lane & 15, g = lane >> 4;
 
-  // Workgroups go round-robin to the eight XCDs, each with its own L2: give every XCD a
-  // contiguous run of tiles, walking m fastest, so the workgroups resident on an XCD share
-  // weight tiles (all m of a few n) and every activation tile.
   int tile = blockIdx.x;
   const int tiles = a.tiles_m * a.tiles_n;
-  if (tiles % 8 == 0) tile = (tile % 8) * (tiles / 8) + tile / 8;
+  if (tiles % 8 == 0) tile = (tile % 8) * (tiles / 8) + tile / 8;  // an XCD a run of tiles, m fastest
   const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
   const int m0 = tm * kTileM, n0 = tn * kTileN;
   const int steps = a.k / kStepK;
   const int blocks = a.k / 32;
 
-  // What this thread brings: group 1 the activation tile, group 0 the weight tile; the
-  // group's first wave also the operand's scales, two atoms (128 rows by the step's four
-  // blocks each) a stage. An atom past the operand's padded rows repeats the last.
-  const int loads = group == 1 ? kLoadsA : kLoadsB;
-  const uint8_t* const matrix = group == 1 ? a.a : a.b;
-  // Its position p = 256 i + t of a tile is row 32 i + t / 8, and the chunk there is the same
-  // for every i (the swizzle key of 32 i + t / 8 is that of t / 8).
-  const int thread = tid & (kGroupThreads - 1);
-  const int row_first = (group == 1 ? m0 : n0) + (thread >> 3);
-  const int row_last = (group == 1 ? a.m : a.n) - 1;
-  const uint32_t chunk_from = static_cast<uint32_t>(((thread & 7) ^ ((thread >> 4) & 7)) * 16);
+  // What this thread brings of a stage: position T i + tid of either tile (T threads) is row T / 8 i + tid / 8, and the chunk
+  // there is the same for every i.
+  const uint32_t chunk_from = static_cast<uint32_t>(((tid & 7) ^ ((tid >> 4) & 7)) * 16);
+  const int a_row = m0 + (tid >> 3), b_row = n0 + (tid >> 3);
   const int atom_b0 = n0 / 128;
-  const int atoms = ((group == 1 ? a.m : a.n) + 127) / 128;
-  const int atom_mine = min((group == 1 ? m0 / 128 : atom_b0) + (lane >> 5), atoms - 1);
-  const uint8_t* const from_scale = (group == 1 ? a.a_scales : a.b_scales) +
-                                    static_cast<int64_t>(atom_mine) * (blocks / 4) * 512 + (lane & 31) * 16;
-  const int tile_base = group == 1 ? L::kA : L::kB;
-  const int tile_bytes = group == 1 ? kTileABytes : L::kTileBBytes;
-  const int scale_base = group == 1 ? L::kAScales : L::kBScales;
-  // Load i of this wave of its operand's tile of K step `step` into ring stage `stage`.
-  auto load = [&](int i, int step, int stage) {
-    uint8_t* to = lds + tile_base + stage * tile_bytes + (i * kGroupThreads + wm * 64) * 16;
-    // Recomputed at every use: eight 64-bit addresses kept across the steps would not fit the
-    // register file beside the accumulators and fragments.
-    int row = row_first;
-    asm volatile("" : "+v"(row));
-    const uint32_t from = static_cast<uint32_t>(min(row + 32 * i, row_last)) * static_cast<uint32_t>(a.k) + chunk_from;
-    __builtin_amdgcn_global_load_lds((GlobalPointer)(matrix + step * kStepK + from), (LdsPointer)to, 16, 0, 0);
+  const int atoms_a = (a.m + 127) / 128, atoms_b = (a.n + 127) / 128;
+  // The scales: wave 0 the activations', wave 1 the weights', two atoms a stage, 16 bytes a lane.
+  const int atom_mine = wave == 0 ? min(m0 / 128 + (lane >> 5), atoms_a - 1) : min(atom_b0 + (lane >> 5), atoms_b - 1);
+  const uint8_t* const scales_of = wave == 0 ? a.a_scales : a.b_scales;
+  const uint32_t scale_from = static_cast<uint32_t>(atom_mine) * static_cast<uint32_t>(blocks / 4) * 512u + (lane & 31) * 16;
+
+  // Where this thread's chunks of a stage come from, the step's 128 bytes aside (they go into the scalar base):
+  // kept for the whole tile, a vector instruction in the loop takes a matrix instruction's place.
+  uint32_t a_from[kLoadsA], b_from[kLoadsB];
+#pragma unroll
+  for (int i = 0; i < kLoadsA; ++i)
+    a_from[i] = static_cast<uint32_t>(min(a_row + kThreads / 8 * i, a.m - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
+#pragma unroll
+  for (int i = 0; i < kLoadsB; ++i)
+    b_from[i] = static_cast<uint32_t>(min(b_row + kThreads / 8 * i, a.n - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
+  const uint32_t lds_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+  const uint32_t to_mine = lds_at + static_cast<uint32_t>(wave * 64 * 16);
+  auto load_a = [&](int i, int step, int stage) {
+    GlobalToLds16(a.a + step * kStepK, a_from[i], to_mine + static_cast<uint32_t>(L::kA + stage * kTileABytes + i * kThreads * 16));
   };
-  auto load_scales = [&](int step, int stage) {
-    if (wm == 0) {
-      __builtin_amdgcn_global_load_lds((GlobalPointer)(from_scale + step * 512),
-                                       (LdsPointer)(lds + scale_base + stage * kScaleStageBytes), 16, 0, 0);
+  auto load_b = [&](int i, int step, int stage) {
+    GlobalToLds16(a.b + step * kStepK, b_from[i], to_mine + static_cast<uint32_t>(L::kB + stage * L::kTileBBytes + i * kThreads * 16));
+  };
+  // A stage's scales: wave 0 the activations' into stage_a, wave 1 the weights' into stage_b. (A wave-uniform branch
+  // around one load each: the waits below count a wave's loads, and these waves have one more.)
+  auto load_scales = [&](int step_a, int stage_a, int step_b, int stage_b) {
+    if (wave == 0) {
+      GlobalToLds16(scales_of + step_a * 512, scale_from, lds_at + static_cast<uint32_t>(L::kAScales + stage_a * kScaleStageBytes));
+    } else if (wave == 1) {
+      GlobalToLds16(scales_of + step_b * 512, scale_from, lds_at + static_cast<uint32_t>(L::kBScales + stage_b * kScaleStageBytes));
     }
   };
 
-  // Where a lane's scale bytes sit in a scale stage. Row 16 q + r of an operand has its four
-  // scales at atom q / 8, byte (q % 2) 256 + r 16 + (q % 8) / 2 * 4: a part per 16 rows that
-  // is the same for every lane, plus 16 r + g.
   auto scale_at = [](int q, int atom0) { return (q / 8 - atom0) * 512 + (q % 2) * 256 + (q % 8) / 2 * 4; };
   const int scale_lane = r * 16 + g;
-  int scale_x[4], scale_w[WN];
+  // Lane (r, g) wants its row's chunks g and 4 + g; a fragment's rows are 16 f + r, whose swizzle key is r's.
+  const uint32_t chunk_lo = static_cast<uint32_t>((r * 8 + (g ^ ((r >> 1) & 7))) * 16);
+  const uint32_t chunk_hi = static_cast<uint32_t>((r * 8 + ((4 + g) ^ ((r >> 1) & 7))) * 16);
+  const uint32_t frag_a = lds_at + L::kA + static_cast<uint32_t>(wm * kXFrags * 2048);
+  const uint32_t frag_b = lds_at + L::kB + static_cast<uint32_t>(wn * WN * 2048);
+  // A lane's scale bytes: the activations' at a fixed place a fragment from the wave's base, the weights' at
+  // places that depend on the tile (the same for every lane: kept in scalar registers).
+  const uint32_t scale_a_base = lds_at + L::kAScales + static_cast<uint32_t>(scale_at(wm * kXFrags, 0) + scale_lane);
+  const uint32_t scale_b_base = lds_at + L::kBScales + static_cast<uint32_t>(scale_lane);
+  int scale_b_off[WN];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) scale_x[j] = scale_at(wm * 4 + j, 0);
-#pragma unroll
-  for (int i = 0; i < WN; ++i) scale_w[i] = scale_at(n0 / 16 + wn * WN + i, atom_b0);
+  for (int i = 0; i < WN; ++i) scale_b_off[i] = __builtin_amdgcn_readfirstlane(scale_at(n0 / 16 + wn * WN + i, atom_b0));
 
-  // Lane (r, g) wants its row's chunks g and 4 + g; a fragment's rows are 16 f + r, whose
-  // swizzle key is r's.
-  const int chunk_lo = (r * 8 + (g ^ ((r >> 1) & 7))) * 16;
-  const int chunk_hi = (r * 8 + ((4 + g) ^ ((r >> 1) & 7))) * 16;
-
-  V4f acc[WN][4];
-#pragma unroll
-  for (int i = 0; i < WN; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = V4f{0.0f, 0.0f, 0.0f, 0.0f};
-  V8i xf[4], wf[WN];
-  int xscale[4], wscale[WN];
-
-  // Step s's fragments and scales into registers. Fragment f of a tile is 2 KB further on for
-  // every lane; a lane's scale is one byte.
-  auto read = [&](int stage_a, int stage_b) {
-    const uint8_t* tile_a = lds + L::kA + stage_a * kTileABytes + wm * 4 * 2048;
-    const uint8_t* tile_b = lds + L::kB + stage_b * L::kTileBBytes + wn * WN * 2048;
-    const uint8_t* scales_a = lds + L::kAScales + stage_a * kScaleStageBytes + scale_lane;
-    const uint8_t* scales_b = lds + L::kBScales + stage_b * kScaleStageBytes + scale_lane;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) xscale[j] = scales_a[scale_x[j]];
-#pragma unroll
-    for (int i = 0; i < WN; ++i) wscale[i] = scales_b[scale_w[i]];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) xf[j] = ReadFragment(tile_a + j * 2048, chunk_lo, chunk_hi);
-#pragma unroll
-    for (int i = 0; i < WN; ++i) wf[i] = ReadFragment(tile_b + i * 2048, chunk_lo, chunk_hi);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): in registers before the barrier that lets the stage go
-    __builtin_amdgcn_sched_barrier(0);
+  StaticFor<R::kSums>([&](auto t) { ClearSum<decltype(t)::value>(); });
+  // The fragments' registers are refilled in place: an activation fragment's when its row of products has been
+  // issued, a weight fragment's when its last product (in the last row) has.
+  // (The stage's part of an address is added once an iteration, a fragment's is the instruction's offset.)
+  uint32_t a_lo = 0, a_hi = 0, a_scale = 0, b_lo = 0, b_hi = 0, b_scale = 0;
+  auto aim_reads = [&](int stage_a, int stage_b) {
+    a_lo = frag_a + chunk_lo + static_cast<uint32_t>(stage_a * kTileABytes);
+    a_hi = frag_a + chunk_hi + static_cast<uint32_t>(stage_a * kTileABytes);
+    a_scale = scale_a_base + static_cast<uint32_t>(stage_a * kScaleStageBytes);
+    b_lo = frag_b + chunk_lo + static_cast<uint32_t>(stage_b * L::kTileBBytes);
+    b_hi = frag_b + chunk_hi + static_cast<uint32_t>(stage_b * L::kTileBBytes);
+    b_scale = scale_b_base + static_cast<uint32_t>(stage_b * kScaleStageBytes);
   };
-  // The 4 WN MFMAs of a step, with this wave's loads of K step `step` into ring stage `stage`
-  // between them. Past the last step the last is asked for again, into a stage nobody reads
-  // any more: no branch on it, and the loads a wave has in flight stay the same number.
-  auto multiply = [&](int step, int stage) {
-    const int bring = min(step, steps - 1);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < WN; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf[j], acc[i][j], 0, 0, 0, wscale[i], 0, xscale[j]);
-        // Pins the MFMA here in program order (the compiler would otherwise sink all of them
-        // below the loads, which have side effects and so keep their place).
-        asm volatile("" : "+v"(acc[i][j]));
-        const int t = i * 4 + j;
-        if (t % kLoadEvery == kLoadEvery - 1 && t / kLoadEvery < kLoadsA) {
-          if (t / kLoadEvery < loads) load(t / kLoadEvery, bring, stage);
-        }
-      }
-    }
-    load_scales(bring, stage);
-    __builtin_amdgcn_sched_barrier(0);
+  auto read_a = [&](auto jc) {
+    constexpr int j = decltype(jc)::value;
+    LdsToRegs16<R::kX + 8 * j, j * 2048>(a_lo);
+    LdsToRegs16<R::kX + 8 * j + 4, j * 2048>(a_hi);
+    LdsToReg1<R::kXScale + j, (j % 2) * 256 + (j / 2) * 4>(a_scale);
   };
+  auto read_b = [&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+    LdsToRegs16<R::kW + 8 * i, i * 2048>(b_lo);
+    LdsToRegs16<R::kW + 8 * i + 4, i * 2048>(b_hi);
+    LdsToReg1<R::kWScale + i, 0>(b_scale + static_cast<uint32_t>(scale_b_off[i]));
+  };
+  auto read_done = [&]() { asm volatile("s_waitcnt lgkmcnt(0)"); };
   auto barrier = [&]() {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Before the first phase: activations 0 and 1, weights 0 and 1.
+  // Before the first step: activations 0 and 1, weights 0, 1 and 2.
 #pragma unroll
-  for (int i = 0; i < kLoadsA; ++i)
-    if (i < loads) load(i, 0, 0);
-  load_scales(0, 0);
-  if (steps > 1) {
+  for (int i = 0; i < kLoadsA; ++i) load_a(i, 0, 0);
 #pragma unroll
-    for (int i = 0; i < kLoadsA; ++i)
-      if (i < loads) load(i, 1, 1);
-    load_scales(1, 1);
+  for (int i = 0; i < kLoadsB; ++i) load_b(i, 0, 0);
+  load_scales(0, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < kLoadsA; ++i) load_a(i, min(1, steps - 1), 1);
+#pragma unroll
+  for (int i = 0; i < kLoadsB; ++i) load_b(i, min(1, steps - 1), 1);
+  load_scales(min(1, steps - 1), 1, min(1, steps - 1), 1);
+#pragma unroll
+  for (int i = 0; i < kLoadsB; ++i) load_b(i, min(2, steps - 1), 2);
+  if (wave == 1) {
+    GlobalToLds16(scales_of + min(2, steps - 1) * 512, scale_from, lds_at + static_cast<uint32_t>(L::kBScales + 2 * kScaleStageBytes));
   }
-  GEMM_TRACE_CYCLES(1);  // the first two stages asked for
+  GEMM_TRACE_CYCLES(1);  // the first stages asked for
   AwaitLoads<0>();
   barrier();
   GEMM_TRACE(2);  // ... and landed, for every wave
-  if (group == 1) barrier();
+  aim_reads(0, 0);
+  StaticFor<kXFrags>([&](auto j) { read_a(j); });
+  StaticFor<WN>([&](auto i) { read_b(i); });
+  read_done();
+
   int stage_b = 0;  // step s's weight stage, s % 3
   for (int step = 0; step < steps; ++step) {
     if (step == 1) GEMM_TRACE(3);
     if (step == steps / 2) GEMM_TRACE(4);
-    read(step & 1, stage_b);
-    // Group 1: activations step + 1, asked for while multiplying step - 1, have landed.
-    if (group == 1) AwaitLoads<0>();
-    barrier();
-    int to = stage_b + 2;  // (step + 2) % 3
-    if (to >= kRingB) to -= kRingB;
-    multiply(step + 2, group == 1 ? (step & 1) : to);
-    // Group 0: weights step + 1 have landed; step + 2, just asked for, may stay in flight.
-    if (group == 0) {
-      if (wm == 0) {
-        AwaitLoads<kLoadsB + 1>();
-      } else {
-        AwaitLoads<kLoadsB>();
-      }
+    barrier();  // every wave holds step `step`'s fragments; steps up to `step` + 1 (weights: + 2) are whole in LDS
+    const int stage_a = step & 1;
+    const int next_b = stage_b + 1 == kRingB ? 0 : stage_b + 1;  // step + 1's weights
+    const int bring_a = min(step + 2, steps - 1), bring_b = min(step + 3, steps - 1);
+    // An action after every product: the loads first (activations, their scales, weights), and the next step's
+    // fragments into the registers a row (the weights: the last row) has just been multiplied from.
+    aim_reads(stage_a ^ 1, next_b);
+    __builtin_amdgcn_sched_barrier(0);
+    StaticFor<kXFrags>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      StaticFor<WN>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        ScaledProduct<R, kXFrags * i + j, i, j>();
+        constexpr int t = j * WN + i;
+        if constexpr (t < kLoadsA) {
+          load_a(t, bring_a, stage_a);
+        } else if constexpr (t == kLoadsA) {
+          load_scales(bring_a, stage_a, bring_b, stage_b);
+        } else if constexpr (t - kLoadsA - 1 < kLoadsB) {
+          load_b(t - kLoadsA - 1, bring_b, stage_b);
+        }
+        if constexpr (j == kXFrags - 1) read_b(ic);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      read_a(jc);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    read_done();
+    // All but the weights just asked for (and their scales, wave 1) have landed.
+    if (wave == 1) {
+      AwaitLoads<kLoadsB + 1>();
+    } else {
+      AwaitLoads<kLoadsB>();
     }
-    barrier();
     if (++stage_b == kRingB) stage_b = 0;
   }
   GEMM_TRACE(5);  // the last step multiplied
-  if (group == 0) barrier();
   AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
+  // The last products' sums are written passes after their issue: no read of them before.
+  asm volatile("s_nop 15\n\ts_nop 15");
   GEMM_TRACE_CYCLES(6);
 
-  // acc[i][j][q] = D[m0 + wm 64 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int m = m0 + wm * 64 + j * 16 + r;
-    if (m >= a.m) continue;
-#pragma unroll
-    for (int i = 0; i < WN; ++i) {
-      const int n = n0 + wn * 16 * WN + i * 16 + 4 * g;
-      if (n >= a.n) continue;  // n is a multiple of 4 (checked on the host)
-      const V4f v = acc[i][j];
-      if (a.bf16) {
-        uint2 packed;
-        packed.x = FloatToBf16Bits(v[0]) | (FloatToBf16Bits(v[1]) << 16);
-        packed.y = FloatToBf16Bits(v[2]) | (FloatToBf16Bits(v[3]) << 16);
-        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + static_cast<int64_t>(m) * a.n + n) = packed;
-      } else {
-        *reinterpret_cast<float4*>(static_cast<float*>(a.d) + static_cast<int64_t>(m) * a.n + n) =
-            make_float4(v[0], v[1], v[2], v[3]);
-      }
+  // sums(8 i + j)[q] = D[m0 + wm 128 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]. A tile inside the matrix (the
+  // common one) stores without a test an element.
+  const int m_first = m0 + wm * 16 * kXFrags + r, n_first = n0 + wn * 16 * WN + 4 * g;  // n is a multiple of 4 (checked on the host)
+  const int64_t first = static_cast<int64_t>(m_first) * a.n + n_first;
+  const int64_t row_step = static_cast<int64_t>(a.n) * 16;
+  auto store = [&](auto bf16, auto whole) {
+    StaticFor<kXFrags>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+      StaticFor<WN>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int reg = (kXFrags * i + j) * 4;
+        const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
+        if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
+        const int64_t at = first + j * row_step + i * 16;
+        if constexpr (decltype(bf16)::value) {
+          uint2 packed;
+          packed.x = FloatToBf16Bits(v0) | (FloatToBf16Bits(v1) << 16);
+          packed.y = FloatToBf16Bits(v2) | (FloatToBf16Bits(v3) << 16);
+          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + at) = packed;
+        } else {
+          *reinterpret_cast<float4*>(static_cast<float*>(a.d) + at) = make_float4(v0, v1, v2, v3);
+        }
+      });
+    });
+  };
+  const bool whole = m0 + kTileM <= a.m && n0 + kTileN <= a.n;
+  if (a.bf16) {
+    if (whole) {
+      store(std::true_type{}, std::true_type{});
+    } else {
+      store(std::true_type{}, std::false_type{});
+    }
+  } else {
+    if (whole) {
+      store(std::false_type{}, std::true_type{});
+    } else {
+      store(std::false_type{}, std::false_type{});
     }
   }
   GEMM_TRACE(7);  // the tile's stores queued
@@ -544,9 +640,9 @@ int LaunchGemm(GemmArgs a, hipStream_t stream) {
   static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
   a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
   static bool sized = false;
-  if (!AllowLds(reinterpret_cast<const void*>(&GemmKernel<WN>), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
-  hipLaunchKernelGGL((GemmKernel<WN>), dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(kGemmThreads), L::kBytes,
-                     stream, a);
+  if (!AllowLds(reinterpret_cast<const void*>(&GemmKernel<kGemmWavesM, WN>), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
+  hipLaunchKernelGGL((GemmKernel<kGemmWavesM, WN>), dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(kGemmWavesM * 128),
+                     L::kBytes, stream, a);
   return LaunchStatus("mxfp8.gemm");
 }
 

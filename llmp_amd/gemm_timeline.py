@@ -8,7 +8,7 @@ import numpy as np, torch
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 from llmp_amd import _lib
-_lib.SO_PATH = os.path.join(ROOT, "llmp_amd", "lib", "libllmp_hip_trace.so")
+_lib.SO_PATH = os.environ.get("LLMP_TRACE_SO", os.path.join(ROOT, "llmp_amd", "lib", "libllmp_hip_trace.so"))
 from llmp_amd import ops
 lib = _lib.load()
 lib.llmp_hip_gemm_trace_set.argtypes = [C.c_void_p]
@@ -32,6 +32,7 @@ for r in range(3):
     trace.zero_(); torch.cuda.synchronize()
     ops.mxfp8_gemm(ac, asc, wc, wsc, out=d); torch.cuda.synchronize()
 tr = trace.cpu().numpy().reshape(-1, 8).astype(np.float64)
+tr = tr[tr[:, 0] > 0]  # the buffer has room for eight waves a workgroup
 lib.llmp_hip_gemm_trace_set(None)
 t0 = tr[:, 0].min()
 names = ["start", "(cycle counter)", "first stages landed", "step 1", "step 16", "last step done", "(cycle counter)", "stores queued"]
