@@ -91,12 +91,33 @@ def graph_us(body, count, warm=3):
 
 MFMA_FP8_PEAK_TFLOPS = 5033.0  # dense FP8, 256 CUs x 2.4 GHz x 8192 flop/clk/CU
 
-# HBM bytes per launch of each configuration's dominant kernel from rocprofv3 --pmc runs of this file
-# (`--only <name> --eager`: FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by 1.9988 and 1.0, what the
-# same counters read for --calibrate-copy's copy of known size). Counters cannot be read from inside a run:
-# a configuration that has not been profiled reports null.
+# HBM bytes per launch of each configuration's roofline kernel(s), from rocprofv3 --pmc runs of this file
+# (`--only <name> --no-cpu --eager --calibrate-copy`: FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what
+# the same counters read for --calibrate-copy's copy of known size: FETCH_SIZE reads half the bytes fetched, factor
+# 2.0014, WRITE_SIZE all of them, factor 1.0010). Counters cannot be read from inside a run: a configuration that has
+# not been profiled reports null.
+def _traffic(fetch_kib, write_kib):
+    return int(round((fetch_kib * 2.0014 + write_kib * 1.0010) * 1024))
+
+
 PROFILED_TRAFFIC = {
     "q4_k_gate_up_geglu_b1": int(round((32478.4 * 1.9988 + 60.1) * 1024)),
+    "q8_0_matvec_4096x4096_b1": _traffic(8768.0, 16.0),
+    # A weight row a lane asks for 144 bytes a row a load, ragged against the 64-byte units HBM is fetched in; the
+    # unit two neighbouring super-blocks share is fetched for each (the second request comes while the first is in
+    # flight): 1.4 times the algorithmic bytes.
+    "q4_k_gate_up_geglu_b4": _traffic(45506.7, 240.0),
+    "q4_k_gate_up_geglu_b8": _traffic(46231.1, 960.0),
+    "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
+    # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through
+    # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
+    "mxfp8_gemm_2048x12288x4096": _traffic(93107.9, 49162.0),
+    "moe_q4_k_ffn_t1": _traffic(7028.8, 24.0),        # the gate/up launch
+    "moe_q4_k_ffn_t16": _traffic(76343.9, 457.9),     # the gate/up launch
+    "moe_q4_k_ffn_t512": _traffic(182457.3, 12338.4),  # the gate/up launch: the experts' tokens once a segment of rows
+    "exl3_linear_4096x14336_4bpw_m1": _traffic(14475.9 + 143.5, 232.0 + 56.0),  # product + output transform
+    "exl3_linear_4096x14336_4bpw_m16": _traffic(14906.0 + 114.5 + 1921.5, 3584.0 + 128.0 + 896.0),
+    "exl3_multi_linear_4096x2x14336_4bpw_m1": _traffic(28815.7 + 255.5, 464.0 + 112.0),
 }
 
 

@@ -341,6 +341,25 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     for (int j = 0; j < kPieceLoads; ++j)
       __builtin_amdgcn_global_load_lds((GlobalPointer)(from + offsets[j]), (LdsPointer)(to + j * (kWave * 16)), 16, 0, 0);
   };
+  // Before piece i is multiplied: the piece STAGES - 1 ahead is asked for, and all but the STAGES - 1 youngest
+  // pieces have landed. At the tile's end nothing is asked for (a repeat of the last piece would be read from HBM
+  // again: the copies of the weights are rotated) and the wait is for what is left.
+  auto next_piece = [&](int i) {
+    const int left = pieces - 1 - i;  // pieces after this one
+    if (left >= STAGES - 1) {
+      issue(i + STAGES - 1);
+      AwaitLoads<kPieceLoads*(STAGES - 1)>();
+    } else {
+      static_assert(STAGES <= 4, "a wait for each count of pieces left");
+      if (STAGES > 3 && left == 2) {
+        AwaitLoads<kPieceLoads * 2>();
+      } else if (STAGES > 2 && left == 1) {
+        AwaitLoads<kPieceLoads>();
+      } else {
+        AwaitLoads<0>();
+      }
+    }
+  };
   // (Every wave has pieces: rows of at least four super-blocks; and every workgroup a tile: the grid is no larger.)
   auto prologue = [&](int tile) {
     aim(tile);
@@ -383,23 +402,20 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
         const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * 8 * T::kCodesBlock);
         const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * 8 * T::kScalesBlock);
         const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
-        issue(i + STAGES - 1);
-        AwaitLoads<kPieceLoads*(STAGES - 1)>();
+        next_piece(i);
         ROWS_TRACE(3 + i);  // piece i landed (the first ten)
         PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, up_out, up_mins);
         ++i;
         if constexpr (kGlu) {
           __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
-          issue(i + STAGES - 1);
-          AwaitLoads<kPieceLoads*(STAGES - 1)>();
+          next_piece(i);
           ROWS_TRACE(3 + i);
           PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, gate_out, gate_mins);
           ++i;
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);
       }
-      ROWS_TRACE(13);  // the last piece multiplied
-      AwaitLoads<0>();  // the repeats past the end: nothing may land in the ring after the sums are there
+      ROWS_TRACE(13);  // the last piece multiplied (nothing is in flight: its wait was for every load)
     }
     ROWS_TRACE(14);
     // The four quarters of K meet: [wave][matrix][token][row] floats at the head of each wave's ring.
