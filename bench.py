@@ -104,9 +104,8 @@ PROFILED_TRAFFIC = {
     "q4_k_gate_up_geglu_b1": int(round((32478.4 * 1.9988 + 60.1) * 1024)),
     "q8_0_matvec_4096x4096_b1": _traffic(8768.0, 16.0),
     # A weight row a lane asks for 144 bytes a row a load, ragged against the 64-byte units HBM is fetched in; the
-    # unit two neighbouring super-blocks share is fetched for each (the second request comes while the first is in
-    # flight): 1.4 times the algorithmic bytes.
-    "q4_k_gate_up_geglu_b4": _traffic(45506.7, 240.0),
+    # unit two neighbouring super-blocks share is often fetched for each: 1.3 to 1.4 times the algorithmic bytes.
+    "q4_k_gate_up_geglu_b4": _traffic(43591.1, 240.0),
     "q4_k_gate_up_geglu_b8": _traffic(46231.1, 960.0),
     "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
     # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through

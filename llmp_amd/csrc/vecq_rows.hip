@@ -330,12 +330,18 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     up_tile = static_cast<const uint8_t*>(d.w) + at;
     if constexpr (kGlu) gate_tile = static_cast<const uint8_t*>(d.g) + at;
   };
-  // Piece i: super-block sb_first + i / kMatrices of the up matrix, then of the gate matrix. Past the
+  // Piece i, in the order the loop below multiplies them: two super-blocks of the up matrix, the same two of the
+  // gate matrix, the next two (an odd one out last, up then gate). Past the
   // wave's last piece its last again (a load is never skipped: the waits count loads).
   auto issue = [&](int i) {
     const int piece = min(i, pieces - 1);
-    const int sb = sb_first + piece / kMatrices;
-    const uint8_t* from = (kGlu && (piece & 1) != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * 144;
+    int gate = 0, sb = sb_first + piece;
+    if constexpr (kGlu) {
+      const int paired = (sb_end - sb_first) / 2 * 4;  // pieces of whole pairs of super-blocks
+      gate = piece < paired ? (piece & 3) >> 1 : piece - paired;
+      sb = sb_first + (piece < paired ? (piece >> 2) * 2 + (piece & 1) : sb_end - sb_first - 1);
+    }
+    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * 144;
     uint8_t* to = ring + (i % STAGES) * kPieceBytes;
 #pragma unroll
     for (int j = 0; j < kPieceLoads; ++j)
@@ -398,22 +404,26 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     LdsBarrier();  // the tokens are staged
     ROWS_TRACE(2);
     {
-      for (int i = 0, sb = sb_first; sb < sb_end; ++sb) {
+      // Two super-blocks of the up matrix, then the same two of the gate matrix: neighbours in a row share a 64-byte
+      // unit of HBM more often than not, and the sooner the second asks for it the likelier L2 still has it.
+      const int count = sb_end - sb_first;
+      int i = 0;
+      auto piece_dot = [&](int sb, float (&out)[NT], V4f (&mins)[NT / 4]) {
         const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * 8 * T::kCodesBlock);
         const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * 8 * T::kScalesBlock);
         const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
         next_piece(i);
         ROWS_TRACE(3 + i);  // piece i landed (the first ten)
-        PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, up_out, up_mins);
+        PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
         ++i;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
+      };
+      for (int n = 0; n < count; n += kMatrices) {
+        const int width = min(kMatrices, count - n);
+        for (int w = 0; w < width; ++w) piece_dot(sb_first + n + w, up_out, up_mins);
         if constexpr (kGlu) {
-          __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
-          next_piece(i);
-          ROWS_TRACE(3 + i);
-          PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, gate_out, gate_mins);
-          ++i;
+          for (int w = 0; w < width; ++w) piece_dot(sb_first + n + w, gate_out, gate_mins);
         }
-        __builtin_amdgcn_s_waitcnt(0xC07F);
       }
       ROWS_TRACE(13);  // the last piece multiplied (nothing is in flight: its wait was for every load)
     }
