@@ -12,8 +12,8 @@ from llmp_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "llmp_hip.h")).read()
+def declared_symbols(header="llmp_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(llmp_hip_[a-z0-9_]+)\s*\(", text)))
 
@@ -26,6 +26,15 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
         assert name in _lib.SYMBOLS, f"{name} has no ctypes signature"
     assert sorted(_lib.SYMBOLS) == names
+
+
+def test_library_exports_the_provider_and_launch_context():
+    """include/llmp_hip_launch.h: bound from C++ (include/llmp_hip_launch.hpp), so exported names are what is checked."""
+    lib = _lib.load()
+    names = declared_symbols("llmp_hip_launch.h")
+    assert len(names) >= 35
+    for name in names:
+        assert hasattr(lib, name), name
 
 
 def test_variant_table_is_named():
