@@ -419,7 +419,7 @@ struct Capability {
   std::uint32_t needs = 0;  // DeviceFeature bits
   ShapeRule shape{};
   Rung rung = Rung::kNative;
-  bool row_invariant = true;  // a row's result never depends on the rows computed beside it
+  bool row_invariant = true;  // every row computes what its one-row launch computes, bit for bit (usable in verify plans)
   bool capturable = true;     // every entry point only queues launches with replay-invariant arguments
   std::string group;          // "ggml.mul_mat" for the members of upstream's routing
   std::vector<std::string> launches;  // the entry points (llmp_hip.h) a node of it queues, in order
@@ -468,10 +468,24 @@ inline std::vector<Implementation> Implementations() {
   // capabilities.cc:2881-2893 and plan_step.h:201-314: the activation quantizer and the products over its blocks.
   add("llmp.q8_1", "quantize.block32_q8_sum_f32", {"f32"}, {1, 65535, 1, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize"},
       "eight lanes a block; rows padded to 512 values");
+  // The default choice of form follows the token count (a weight row a lane or the F16 matrix cores for Q4_K above one
+  // token): a row's bits then differ from its one-row launch's in the last place, as upstream's multi-column kernel's
+  // do, so these are not candidates of a row-invariant plan.
+  const auto follows_rows = [&]() { all.back().capability.row_invariant = false; };
   add("llmp.vecq.dense", "mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, kInt8Mma, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
-      "a lane a unit through LDS (1 to 5 tokens), int8 matrix cores above");
+      "variant -1: a lane a unit through LDS, a weight row a lane (Q4_K, 2 to 8 tokens), matrix cores above");
+  follows_rows();
   add("llmp.vecq.glu", "fused.mul_mat_glu", blocks, {1, 16, 256, 1}, Rung::kNative, kInt8Mma, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
-      "gate and up rows in one tile, the GLU in the row's first lane");
+      "variant -1: gate and up rows in one tile, the GLU in the row's first lane");
+  follows_rows();
+  // The reference's row-invariant products (docs/decisions.md D-092, src/kernels/ggml/mmvq_rows.cu): the one-token
+  // launch's arithmetic for every token, the weights read once for four.
+  add("llmp.mul_mat.mmvq_rows", "mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "variant 7 (flat pass4): passes of four tokens, each the one-token product bit for bit");
+  add("llmp.mul_mat_glu.mmvq_rows", "fused.mul_mat_glu", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "variant 7 (flat pass4) with the GLU");
+  add("llmp.mul_mat_id.mmvq_rows", "mul_mat_id", blocks, {1, 128, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
+      "variant 7 (flat pass4) over up to 128 (token, slot) pairs");
   add("llmp.vecq.experts", "mul_mat_id", blocks, {1, 128, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
       "up to 128 (token, slot) pairs; the first pair naming an expert owns it");
   add("llmp.vecq.experts_glu", "fused.mul_mat_id_glu", blocks, {1, 128, 256, 1}, Rung::kNative, 0,
@@ -479,12 +493,15 @@ inline std::vector<Implementation> Implementations() {
   add("llmp.vecq.grouped", "fused.grouped_mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
       "matrix g with input row g: up to 256 groups");
   add("llmp.vecq.sorted", "mul_mat_id", {"q8_0", "q4_k"}, {129, any, 256, 1}, Rung::kNative, kInt8Mma,
-      {"llmp_hip_moe_route", "llmp_hip_q8_1_quantize_rows", "llmp_hip_vecq_sorted"}, "rows sorted by expert on the int8 matrix cores");
+      {"llmp_hip_moe_route", "llmp_hip_q8_1_quantize_rows", "llmp_hip_vecq_sorted"}, "rows sorted by expert on the matrix cores");
+  follows_rows();
   // Upstream's routing names (capabilities.cc:2486-2489): the same launches, members of its group.
   add("ggml.mul_mat.mmvq", "mul_mat", blocks, {1, 16, 256, 1}, Rung::kNative, 0, {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"},
       "llmp.vecq.dense's launches", "ggml.mul_mat");
+  follows_rows();
   add("ggml.mul_mat_glu.mmvq_fused", "fused.mul_mat_glu", blocks, {1, 16, 256, 1}, Rung::kNative, 0,
       {"llmp_hip_q8_1_quantize", "llmp_hip_vecq"}, "llmp.vecq.glu's launches", "ggml.mul_mat");
+  follows_rows();
   add("llmp.moe.router", "route.softmax_top_k", {"f32"}, {1, any, 1, 1}, Rung::kNative, 0, {"llmp_hip_moe_router"},
       "a wave a token; up to 1024 experts, 64 picks");
   add("llmp.moe.experts.cutlass", "mul_mat_id", {"nvfp4"}, {1, any, 64, 1}, Rung::kOnChipDecode, kBf16Mma,

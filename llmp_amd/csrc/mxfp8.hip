@@ -282,6 +282,17 @@ __device__ unsigned long long* g_gemm_trace = nullptr;
   } while (0)
 #endif
 
+// For the tuning build only (make trace EXTRA=-DLLMP_GEMM_WITHOUT=<bits>): parts of GemmKernel's loop left out, to time
+// what each costs. Results are wrong; nothing faults (what is left out is never a wait that guards an address).
+//   1 the loads to LDS after the prologue   2 the reads of fragments and scales from LDS   4 the step's barrier
+//   8 the wait for the step's loads         16 the tile's stores
+#ifndef LLMP_GEMM_WITHOUT
+#define LLMP_GEMM_WITHOUT 0
+#endif
+#if LLMP_GEMM_WITHOUT != 0 && !defined(LLMP_GEMM_TRACE)
+#error "LLMP_GEMM_WITHOUT is for the tuning build"
+#endif
+
 // LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
 template <int WN>
 struct GemmLds {
@@ -550,7 +561,8 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
   for (int step = 0; step < steps; ++step) {
     if (step == 1) GEMM_TRACE(3);
     if (step == steps / 2) GEMM_TRACE(4);
-    barrier();  // every wave holds step `step`'s fragments; steps up to `step` + 1 (weights: + 2) are whole in LDS
+    if constexpr ((LLMP_GEMM_WITHOUT & 4) == 0) barrier();
+    // Every wave holds step `step`'s fragments; steps up to `step` + 1 (weights: + 2) are whole in LDS
     const int stage_a = step & 1;
     const int next_b = stage_b + 1 == kRingB ? 0 : stage_b + 1;  // step + 1's weights
     const int bring_a = min(step + 2, steps - 1), bring_b = min(step + 3, steps - 1);
@@ -564,25 +576,28 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
         constexpr int i = decltype(ic)::value;
         ScaledProduct<R, kXFrags * i + j, i, j>();
         constexpr int t = j * WN + i;
-        if constexpr (t < kLoadsA) {
+        if constexpr ((LLMP_GEMM_WITHOUT & 1) != 0) {
+        } else if constexpr (t < kLoadsA) {
           load_a(t, bring_a, stage_a);
         } else if constexpr (t == kLoadsA) {
           load_scales(bring_a, stage_a, bring_b, stage_b);
         } else if constexpr (t - kLoadsA - 1 < kLoadsB) {
           load_b(t - kLoadsA - 1, bring_b, stage_b);
         }
-        if constexpr (j == kXFrags - 1) read_b(ic);
+        if constexpr (j == kXFrags - 1 && (LLMP_GEMM_WITHOUT & 2) == 0) read_b(ic);
         __builtin_amdgcn_sched_barrier(0);
       });
-      read_a(jc);
+      if constexpr ((LLMP_GEMM_WITHOUT & 2) == 0) read_a(jc);
       __builtin_amdgcn_sched_barrier(0);
     });
     read_done();
     // All but the weights just asked for (and their scales, wave 1) have landed.
-    if (wave == 1) {
-      AwaitLoads<kLoadsB + 1>();
-    } else {
-      AwaitLoads<kLoadsB>();
+    if constexpr ((LLMP_GEMM_WITHOUT & 8) == 0) {
+      if (wave == 1) {
+        AwaitLoads<kLoadsB + 1>();
+      } else {
+        AwaitLoads<kLoadsB>();
+      }
     }
     if (++stage_b == kRingB) stage_b = 0;
   }
@@ -605,6 +620,7 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
         constexpr int reg = (kXFrags * i + j) * 4;
         const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
         if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
+        if ((LLMP_GEMM_WITHOUT & 16) != 0 && v0 != 12345.678f) return;  // (the sums are still read and converted)
         const int64_t at = first + j * row_step + i * 16;
         if constexpr (decltype(bf16)::value) {
           uint2 packed;

@@ -162,7 +162,7 @@ void RegistryChecks() {
   // SURVEY's list of names to keep (plan_step.h:201-314, capabilities.cc:2486-2489 and 2881-2893,
   // decode/implementations.h:7-13, exl3/implementations.h:8-31).
   for (const char* name : {"llmp.q8_1", "llmp.vecq.dense", "llmp.vecq.glu", "llmp.vecq.experts", "llmp.vecq.experts_glu", "llmp.vecq.grouped",
-                           "ggml.mul_mat.mmvq", "ggml.mul_mat_glu.mmvq_fused", "llmp.mxfp8.mul_mat_vec", "llmp.mxfp8.quantize",
+                           "ggml.mul_mat.mmvq", "ggml.mul_mat_glu.mmvq_fused", "llmp.mul_mat.mmvq_rows", "llmp.mul_mat_id.mmvq_rows", "llmp.mxfp8.mul_mat_vec", "llmp.mxfp8.quantize",
                            "llmp.mxfp8.swizzle", "llmp.mxfp8.gemm.cutlass", "llmp.moe.router", "llmp.moe.experts.cutlass", "llmp.decode.vector.nvfp4.atoms",
                            "llmp.decode.vector_glu.mxfp8.split", "llmp.decode.matrix.bf16.dense", "llmp.decode.grouped.affine.split",
                            "llmp.decode.rows.q8_0.blocks", "exl3.linear.gemv", "exl3.linear.gemm", "exl3.multi_linear.mgemm"})
@@ -174,8 +174,14 @@ void RegistryChecks() {
   // Candidates: the config shapes find their implementations, and nothing outside a rule does.
   ex::CapabilityQuery q;
   q.op = "fused.mul_mat_glu", q.encoding = "q4_k", q.rows = 1, q.k = 3840, q.n = 15360, q.row_invariant = q.capturable = true;
+  // A row-invariant plan (docs/decisions.md D-092 of the reference) takes the product whose every row is its one-row
+  // launch bit for bit, not the default whose form follows the row count.
   std::vector<ex::Implementation> found = ex::Candidates(q);
-  EXPECT(found.size() == 2 && found[0].name == "llmp.vecq.glu" && found[1].name == "ggml.mul_mat_glu.mmvq_fused");
+  EXPECT(found.size() == 1 && found[0].name == "llmp.mul_mat_glu.mmvq_rows");
+  q.row_invariant = false;
+  found = ex::Candidates(q);
+  EXPECT(found.size() == 3 && found[0].name == "llmp.vecq.glu" && found[1].name == "llmp.mul_mat_glu.mmvq_rows" &&
+         found[2].name == "ggml.mul_mat_glu.mmvq_fused");
   q.rows = 17;
   EXPECT(ex::Candidates(q).empty());
   q.rows = 1, q.k = 3840 + 32;
