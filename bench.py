@@ -141,6 +141,24 @@ def hbm_roofline(name, kernel, bytes_, us):
             "algorithmic_bytes_per_launch": int(bytes_), "avg_launch_us": round(us, 3)}
 
 
+def read_only_launch(device, bytes_, kernel_us, eager=False):
+    """The yardstick beside a streaming kernel's time: a launch that only reads as many bytes (llmp_hip_stream_read,
+    eight 16-byte loads in flight a lane) over copies rotated like the weights, timed the same way."""
+    import torch
+
+    from llmp_amd import ops
+
+    size = (int(bytes_) + 15) // 16 * 16
+    copies = [torch.randint(0, 255, (size,), dtype=torch.uint8, device=device) for _ in range(-(-ROTATE_BYTES // size) + 1)]
+    sink = ops.stream_read(copies[0])
+    body = lambda i: ops.stream_read(copies[i % len(copies)], sink)
+    us = event_us(body, 8 * len(copies)) if eager else graph_us(body, 8 * len(copies))
+    del copies
+    torch.cuda.empty_cache()
+    return {"us": round(us, 3), "GB/s": round(size / us / 1e3, 1), "frac_hbm_peak": round(size / us / 1e3 / HBM_PEAK_GBPS, 4),
+            "kernel_over_read_only": round(kernel_us / us, 3)}
+
+
 def other_configs(device, args, only=None):
     """The other benchmark configurations (not the headline line), each with the roofline of its dominant
     kernel and the oracle timed on the host cores over a bounded sample of the same workload. Weights are
@@ -178,7 +196,8 @@ def other_configs(device, args, only=None):
         bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
         entry = {"workload": "GGML Q8_0 mat-vec, N=4096, K=4096, batch 1, fp32 activations through llmp.q8_1",
                  "step_us": round(step_us, 2), "weight_GB/s_of_the_step": round(w.numel() / step_us / 1e3, 1),
-                 "roofline": hbm_roofline("q8_0_matvec_4096x4096_b1", "VecQFlat<FormatQ8> (llmp.vecq, Q8_0)", bytes_, us)}
+                 "roofline": hbm_roofline("q8_0_matvec_4096x4096_b1", "VecQFlat<FormatQ8> (llmp.vecq, Q8_0)", bytes_, us),
+                 "read_only_launch": read_only_launch(device, bytes_, us, args.eager)}
         if cpu:
             q8_host = oracle.q8_1_quantize(x_host)
             entry["cpu_baseline"] = cpu_leg(lambda: oracle.vecq(oracle.TYPE_Q8_0, w_host, q8_host, k, n, threads=threads),
@@ -607,9 +626,11 @@ def main():
                      "algorithmic_bytes_per_launch": algorithmic_bytes(args.tokens),
                      "avg_launch_us": round(kernel_us, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
     }
+    del gates, ups
+    torch.cuda.empty_cache()
+    # Beside the roofline: what a launch that only reads the same bytes takes on this box (not part of `value`).
+    line["read_only_launch"] = read_only_launch(device, algorithmic_bytes(args.tokens), kernel_us, args.eager)
     if not args.no_extras:
-        del gates, ups
-        torch.cuda.empty_cache()
         line["other_configs"] = other_configs(device, args)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(gate, up, x)

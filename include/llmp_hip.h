@@ -447,6 +447,14 @@ int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* experts, uin
 int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* weight, uint64_t first, uint64_t outputs, const float* x,
                            uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int path, void* stream);
 
+/* ------------------------------------------------------------ a yardstick
+ * No counterpart in the reference: a launch that only reads `bytes` (whole 16-byte chunks at a 16-byte boundary),
+ * eight loads in flight a lane, folded into `sink` (llmp_hip_stream_read_sink(cus) bytes, the caller's). What it
+ * takes is what the launch latency and the memory system leave of the HBM peak at that size: the benchmark prints
+ * it beside each streaming kernel's time. */
+size_t llmp_hip_stream_read_sink(int compute_units);
+int llmp_hip_stream_read(const void* data, size_t bytes, void* sink, int compute_units, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -104,6 +104,8 @@ _i64, _vp, _int = C.c_int64, C.c_void_p, C.c_int
 SYMBOLS = {
     "llmp_hip_last_error": (C.c_char_p, []),
     "llmp_hip_compute_units": (_int, []),
+    "llmp_hip_stream_read_sink": (C.c_size_t, [_int]),
+    "llmp_hip_stream_read": (_int, [_vp, C.c_size_t, _vp, _int, _vp]),
     "llmp_hip_q8_1_quantize": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_vecq": (_int, [_int, C.POINTER(VecQDesc), _int, _vp]),
     "llmp_hip_vecq_variants": (_int, []),

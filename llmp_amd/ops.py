@@ -290,6 +290,17 @@ def mxfp8_scale_bytes(rows, k):
     return (rows + 127) // 128 * 128 * (k // 32)
 
 
+def stream_read(data, sink=None):
+    """A launch that only reads `data` (a uint8 tensor of whole 16-byte chunks): the yardstick beside the streaming
+    kernels' times. Returns the sink (reuse it across calls)."""
+    lib = _lib.load()
+    cus = lib.llmp_hip_compute_units()
+    if sink is None:
+        sink = torch.empty(lib.llmp_hip_stream_read_sink(cus), dtype=torch.uint8, device=data.device)
+    _lib.check(lib.llmp_hip_stream_read(_ptr(data), data.numel() * data.element_size(), _ptr(sink), cus, _stream()))
+    return sink
+
+
 def mxfp8_quantize(x, out=None):
     """llmp.mxfp8.quantize: float32 / bfloat16 [rows, k] -> (codes uint8 [rows, k], scales uint8 atoms); `out`,
     a pair of such tensors, is filled in place."""
