@@ -268,7 +268,7 @@ def other_configs(device, args, only=None):
                  "step_us": round(us + quant_us, 1), "TFLOP/s_of_the_step": round(flops / (us + quant_us) / 1e6, 1),
                  "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(achieved / MFMA_FP8_PEAK_TFLOPS, 4), "traffic": PROFILED_TRAFFIC.get("mxfp8_gemm_2048x12288x4096"),
-                              "kernel": "GemmKernel (v_mfma_scale_f32_16x16x128_f8f6f4)", "algorithmic_flops_per_launch": int(flops),
+                              "kernel": "GemmKernel192 (v_mfma_scale_f32_16x16x128_f8f6f4)", "algorithmic_flops_per_launch": int(flops),
                               "avg_launch_us": round(us, 2)},
                  "quantize": {"us": round(quant_us, 2), "bytes": quant_bytes, "GB/s": round(quant_bytes / quant_us / 1e3, 1),
                               "frac_hbm_peak": round(quant_bytes / quant_us / 1e3 / HBM_PEAK_GBPS, 4)}}

@@ -242,8 +242,7 @@ __global__ __launch_bounds__(256) void GemvKernel(const uint8_t* __restrict__ co
 
 constexpr int kTileM = 256;             // activation rows a workgroup
 constexpr int kStepK = 128;             // codes a K step
-constexpr int kRingA = 2;               // stages of activation tiles in LDS
-constexpr int kRingB = 3;               // stages of weight tiles
+constexpr int kRingB = 3;               // stages of weight tiles in LDS (of activation tiles: two or three, GemmLds)
 constexpr int kTileABytes = kTileM * kStepK;  // 32 KB
 constexpr int kScaleStageBytes = 1024;  // two atoms a stage, either operand
 
@@ -294,8 +293,9 @@ __device__ unsigned long long* g_gemm_trace = nullptr;
 #endif
 
 // LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
-template <int WN>
+template <int WN, int RA>
 struct GemmLds {
+  static constexpr int kRingA = RA;
   static constexpr int kTileN = 32 * WN;
   static constexpr int kTileBBytes = kTileN * kStepK;
   static constexpr int kA = 0;
@@ -330,7 +330,7 @@ __device__ __forceinline__ void AwaitLoads() {
 // this kernel): its 48 products alone 0.99 us a wave that is alone on its SIMD, 41 cycles a product where the matrix
 // pipe's eight passes are 32 (the scales are loaded by an instruction of their own before each product); and nothing
 // else of the same wave is issued meanwhile, so the 16 loads to LDS add 0.19 us (about 20 cycles each), the 42 reads
-// of LDS 0.11, the barrier and the waits 0.09: 1.35 us. Two waves a SIMD (WM = 4) do issue into each other's
+// of LDS 0.11, the barrier and the waits 0.09: 1.35 us. Two waves a SIMD (eight waves a tile) do issue into each other's
 // products, but eight waves read 216 KB of LDS a step where four read 168, and LDS's 128 bytes a cycle then bound the
 // step at 1.29 us; with the smaller tile's poorer tail that is no faster, and four waves are the default.
 //
@@ -357,11 +357,8 @@ __device__ __forceinline__ void StaticFor(F&& f) {
 //   v[240 + j], v[248 + i]                their scales, a byte each
 // The compiler keeps to v0 .. v127 (amdgpu_num_vgpr) and is told once that the kernel uses the rest; what it may
 // not see is listed with each helper.
-#ifndef LLMP_GEMM_WAVES_M
-#define LLMP_GEMM_WAVES_M 2
-#endif
-constexpr int kGemmWavesM = LLMP_GEMM_WAVES_M;
-constexpr int kGemmCompilerVgprs = kGemmWavesM == 2 ? 128 : 64;
+// v0 .. for the compiler: 128 of them with four waves a workgroup, 64 with eight.
+constexpr int GemmCompilerVgprs(int wm) { return wm == 2 ? 128 : 64; }
 
 // WM waves share the tile's 256 activation rows (2 waves of weights each): 2, a wave a SIMD with 448 registers, or 4, two
 // waves a SIMD with 256 each. A wave's instruction after a matrix product is not issued before the product is (nearly)
@@ -370,8 +367,7 @@ constexpr int kGemmCompilerVgprs = kGemmWavesM == 2 ? 128 : 64;
 template <int WM, int WN>
 struct GemmRegs {
   static constexpr int kXFrags = 16 / WM;                    // 16-row activation fragments a wave
-  static constexpr int kCompilerVgprs = kGemmCompilerVgprs;  // v0 .. for the compiler
-  static_assert(WM == kGemmWavesM, "the attribute that holds the compiler to them is not a template's");
+  static constexpr int kCompilerVgprs = GemmCompilerVgprs(WM);  // v0 .. for the compiler
   static constexpr int kX = kCompilerVgprs;
   static constexpr int kW = kX + 8 * kXFrags;
   static constexpr int kXScale = kW + 8 * WN;
@@ -414,10 +410,9 @@ __device__ __forceinline__ float ReadSum() {
   return v;
 }
 
-template <int WM, int WN>
-__global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCompilerVgprs))) void GemmKernel(
-    const GemmArgs a) {
-  using L = GemmLds<WN>;
+template <int WM, int WN, int RA>
+__device__ __forceinline__ void GemmTile(const GemmArgs& a) {
+  using L = GemmLds<WN, RA>;
   using R = GemmRegs<WM, WN>;
   constexpr int kTileN = L::kTileN;
   constexpr int kThreads = WM * 128;
@@ -532,22 +527,24 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Before the first step: activations 0 and 1, weights 0, 1 and 2.
+  // Before the first step: activations 0 .. RA - 1, weights 0, 1 and 2, each with its scales.
+  StaticFor<(RA > kRingB ? RA : kRingB)>([&](auto sc) {
+    constexpr int stage = decltype(sc)::value;
+    const int step = min(stage, steps - 1);
+    if constexpr (stage < RA) {
 #pragma unroll
-  for (int i = 0; i < kLoadsA; ++i) load_a(i, 0, 0);
+      for (int i = 0; i < kLoadsA; ++i) load_a(i, step, stage);
+    }
+    if constexpr (stage < kRingB) {
 #pragma unroll
-  for (int i = 0; i < kLoadsB; ++i) load_b(i, 0, 0);
-  load_scales(0, 0, 0, 0);
-#pragma unroll
-  for (int i = 0; i < kLoadsA; ++i) load_a(i, min(1, steps - 1), 1);
-#pragma unroll
-  for (int i = 0; i < kLoadsB; ++i) load_b(i, min(1, steps - 1), 1);
-  load_scales(min(1, steps - 1), 1, min(1, steps - 1), 1);
-#pragma unroll
-  for (int i = 0; i < kLoadsB; ++i) load_b(i, min(2, steps - 1), 2);
-  if (wave == 1) {
-    GlobalToLds16(scales_of + min(2, steps - 1) * 512, scale_from, lds_at + static_cast<uint32_t>(L::kBScales + 2 * kScaleStageBytes));
-  }
+      for (int i = 0; i < kLoadsB; ++i) load_b(i, step, stage);
+    }
+    if (wave == 0) {
+      if constexpr (stage < RA) load_scales(step, stage, step, stage);
+    } else if (wave == 1) {
+      if constexpr (stage < kRingB) load_scales(step, stage, step, stage);
+    }
+  });
   GEMM_TRACE_CYCLES(1);  // the first stages asked for
   AwaitLoads<0>();
   barrier();
@@ -557,18 +554,20 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
   StaticFor<WN>([&](auto i) { read_b(i); });
   read_done();
 
+  int stage_a = 0;  // step s's activation stage, s % RA
   int stage_b = 0;  // step s's weight stage, s % 3
   for (int step = 0; step < steps; ++step) {
     if (step == 1) GEMM_TRACE(3);
     if (step == steps / 2) GEMM_TRACE(4);
     if constexpr ((LLMP_GEMM_WITHOUT & 4) == 0) barrier();
-    // Every wave holds step `step`'s fragments; steps up to `step` + 1 (weights: + 2) are whole in LDS
-    const int stage_a = step & 1;
+    // Every wave holds step `step`'s fragments; steps up to `step` + RA - 1 (weights: + 2) are whole in LDS or on
+    // their way, step + 1 whole.
+    const int next_a = stage_a + 1 == RA ? 0 : stage_a + 1;      // step + 1's activations
     const int next_b = stage_b + 1 == kRingB ? 0 : stage_b + 1;  // step + 1's weights
-    const int bring_a = min(step + 2, steps - 1), bring_b = min(step + 3, steps - 1);
+    const int bring_a = min(step + RA, steps - 1), bring_b = min(step + 3, steps - 1);
     // An action after every product: the loads first (activations, their scales, weights), and the next step's
     // fragments into the registers a row (the weights: the last row) has just been multiplied from.
-    aim_reads(stage_a ^ 1, next_b);
+    aim_reads(next_a, next_b);
     __builtin_amdgcn_sched_barrier(0);
     StaticFor<kXFrags>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
@@ -591,15 +590,18 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
       __builtin_amdgcn_sched_barrier(0);
     });
     read_done();
-    // All but the weights just asked for (and their scales, wave 1) have landed.
+    // Step + 2 has landed: with two activation stages all but the weights just asked for (and their scales, wave 1),
+    // with three everything asked for before this iteration (loads complete in the order they were asked for).
     if constexpr ((LLMP_GEMM_WITHOUT & 8) == 0) {
-      if (wave == 1) {
-        AwaitLoads<kLoadsB + 1>();
+      constexpr int kLeft = RA == 2 ? kLoadsB : kLoadsA + kLoadsB;
+      if (wave == 1 || (RA > 2 && wave == 0)) {
+        AwaitLoads<kLeft + 1>();
       } else {
-        AwaitLoads<kLoadsB>();
+        AwaitLoads<kLeft>();
       }
     }
-    if (++stage_b == kRingB) stage_b = 0;
+    stage_a = next_a;
+    stage_b = next_b;
   }
   GEMM_TRACE(5);  // the last step multiplied
   AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
@@ -650,15 +652,33 @@ __global__ __launch_bounds__(WM * 128, 1) __attribute__((amdgpu_num_vgpr(kGemmCo
   GEMM_TRACE(7);  // the tile's stores queued
 }
 
-template <int WN>
-int LaunchGemm(GemmArgs a, hipStream_t stream) {
-  using L = GemmLds<WN>;
+// The two tile shapes, four waves each, one a SIMD. (Eight waves of 64 x 64 on the 256 x 128 tile with three
+// activation stages, two waves a SIMD issuing into each other's products, take 1.10 us a step against this form's
+// 1.03: eight waves read 176 KB of LDS a step.) A kernel's register attribute cannot depend on a template's argument:
+// one kernel a shape.
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel192(const GemmArgs a) {
+  GemmTile<2, 6, 2>(a);
+}
+#ifndef LLMP_GEMM_EIGHT_WAVES
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel128(const GemmArgs a) {
+  GemmTile<2, 4, 2>(a);
+}
+constexpr int kWavesM128 = 2, kRingA128 = 2;
+#else  // the tuning build's (make trace EXTRA=-DLLMP_GEMM_EIGHT_WAVES): that form, and the 256 x 128 tile wherever it ties
+__global__ __launch_bounds__(512, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(4)))) void GemmKernel128(const GemmArgs a) {
+  GemmTile<4, 4, 3>(a);
+}
+constexpr int kWavesM128 = 4, kRingA128 = 3;
+#endif
+
+template <int WM, int WN, int RA>
+int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, hipStream_t stream) {
+  using L = GemmLds<WN, RA>;
   static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
   a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
   static bool sized = false;
-  if (!AllowLds(reinterpret_cast<const void*>(&GemmKernel<kGemmWavesM, WN>), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
-  hipLaunchKernelGGL((GemmKernel<kGemmWavesM, WN>), dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(kGemmWavesM * 128),
-                     L::kBytes, stream, a);
+  if (!AllowLds(reinterpret_cast<const void*>(kernel), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(WM * 128), L::kBytes, stream, a);
   return LaunchStatus("mxfp8.gemm");
 }
 
@@ -789,10 +809,14 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
     const int64_t tiles = static_cast<int64_t>(a.tiles_m) * ((gemm->n + tile_n - 1) / tile_n);
     if (tiles > (1 << 30)) return Refuse(1, "mxfp8.gemm: too many tiles");
     const int64_t cost = (tiles + cus - 1) / cus * tile_n;
+#ifndef LLMP_GEMM_EIGHT_WAVES
     if (best == 0 || cost < best_cost) best = tile_n, best_cost = cost;
+#else
+    if (best == 0 || cost <= best_cost) best = tile_n, best_cost = cost;
+#endif
   }
   const hipStream_t on = static_cast<hipStream_t>(stream);
-  const int status = best == 192 ? LaunchGemm<6>(a, on) : LaunchGemm<4>(a, on);
+  const int status = best == 192 ? LaunchGemm<2, 6, 2>(GemmKernel192, a, on) : LaunchGemm<kWavesM128, 4, kRingA128>(GemmKernel128, a, on);
   return status;  // negative: the launch failed after the checks (the caller's fault path)
 }
 
