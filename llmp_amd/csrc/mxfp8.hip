@@ -261,18 +261,25 @@ struct GemmArgs {
 // every wave stores the 100 MHz clock at up to eight points of its tile, eight 64-bit words a wave.
 #ifdef LLMP_GEMM_TRACE
 __device__ unsigned long long* g_gemm_trace = nullptr;
-#define GEMM_TRACE(slot)                                                                                          \
-  do {                                                                                                            \
-    if (g_gemm_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
-      g_gemm_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (slot)] = wall_clock64(); \
+// The wave's eight slots, asked for once at the kernel's start (read at every stamp, the pointer's two loads and
+// their waits would be part of every step that is timed).
+#define GEMM_TRACE_BEGIN                                                                                     \
+  unsigned long long* gemm_trace_slots = g_gemm_trace;                                                       \
+  if (gemm_trace_slots != nullptr)                                                                           \
+    gemm_trace_slots += (static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8
+#define GEMM_TRACE(slot)                                                                     \
+  do {                                                                                       \
+    if (gemm_trace_slots != nullptr && (threadIdx.x & 63) == 0) gemm_trace_slots[slot] = wall_clock64(); \
   } while (0)
 // ... or the shader clock's counter (slots 1 and 6: the kernel's cycles between them give its clock).
-#define GEMM_TRACE_CYCLES(slot)                                                                                   \
-  do {                                                                                                            \
-    if (g_gemm_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
-      g_gemm_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (slot)] = __builtin_readcyclecounter(); \
+#define GEMM_TRACE_CYCLES(slot)                                                                               \
+  do {                                                                                                        \
+    if (gemm_trace_slots != nullptr && (threadIdx.x & 63) == 0) gemm_trace_slots[slot] = __builtin_readcyclecounter(); \
   } while (0)
 #else
+#define GEMM_TRACE_BEGIN \
+  do {                   \
+  } while (0)
 #define GEMM_TRACE(slot) \
   do {                   \
   } while (0)
@@ -326,11 +333,11 @@ __device__ __forceinline__ void AwaitLoads() {
 // last product; and at the end all loads but the weights just asked for have landed, so that after the next barrier
 // step s + 2 is whole in LDS. One barrier a step; no wave waits for another inside a step.
 //
-// What a step costs, measured with parts of the loop taken out (M 2048, N 12288, K 4096; shader clock 2.0 GHz under
-// this kernel): its 48 products alone 0.99 us a wave that is alone on its SIMD, 41 cycles a product where the matrix
-// pipe's eight passes are 32 (the scales are loaded by an instruction of their own before each product); and nothing
-// else of the same wave is issued meanwhile, so the 16 loads to LDS add 0.19 us (about 20 cycles each), the 42 reads
-// of LDS 0.11, the barrier and the waits 0.09: 1.35 us. Two waves a SIMD (eight waves a tile) do issue into each other's
+// What a step costs, measured with parts of the loop taken out (M 2048, N 12288, K 4096; the shader clock is 1.9 GHz
+// under this kernel): its 48 products alone 0.87-0.95 us a wave that is alone on its SIMD (the pipe takes a product
+// every 32 cycles from one wave; with random codes in every CU the clock does not hold 2.4 GHz); and nothing else of
+// the same wave is issued meanwhile, so the 16 loads to LDS add 0.19 us (about 20 cycles each), the 42 reads of LDS
+// 0.10, the barrier and the waits 0.15: 1.26-1.35 us. Two waves a SIMD (eight waves a tile) do issue into each other's
 // products, but eight waves read 216 KB of LDS a step where four read 168, and LDS's 128 bytes a cycle then bound the
 // step at 1.29 us; with the smaller tile's poorer tail that is no faster, and four waves are the default.
 //
@@ -427,6 +434,7 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     asm volatile("" ::: "v159", "a95");
   }
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  GEMM_TRACE_BEGIN;
   GEMM_TRACE(0);  // the wave's start
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -671,6 +679,39 @@ __global__ __launch_bounds__(512, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
 constexpr int kWavesM128 = 4, kRingA128 = 3;
 #endif
 
+#ifdef LLMP_GEMM_TRACE
+// The tuning build's probe of the matrix pipe alone: the 256 x 192 kernel's 48 products of a step, from the same
+// named registers, `iters` times over with nothing between them, four waves a workgroup (one a SIMD). The
+// fragments are filled from `data` (126 dwords a lane: zeros and random codes draw different power), the scales
+// are 1. Lane 0 of the first wave writes the shader counter's ticks over the loop to `ticks`.
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void ProductsProbeKernel(
+    const uint32_t* __restrict__ data, int iters, unsigned long long* ticks, float* sink) {
+  using R = GemmRegs<2, 6>;
+  asm volatile("" ::: "v253", "a191");
+  StaticFor<R::kXScale - R::kX>([&](auto rc) {
+    constexpr int reg = R::kX + decltype(rc)::value;
+    const uint32_t v = data[decltype(rc)::value * 256 + threadIdx.x];
+    asm volatile("v_mov_b32 v[%0], %1" ::"n"(reg), "v"(v));
+  });
+  StaticFor<R::kTop - R::kXScale>([&](auto rc) {
+    constexpr int reg = R::kXScale + decltype(rc)::value;
+    asm volatile("v_mov_b32 v[%0], 127" ::"n"(reg));
+  });
+  StaticFor<R::kSums>([&](auto t) { ClearSum<decltype(t)::value>(); });
+  asm volatile("s_nop 7");
+  const unsigned long long t0 = __builtin_readcyclecounter();
+  for (int it = 0; it < iters; ++it) {
+    StaticFor<8>([&](auto jc) {
+      StaticFor<6>([&](auto ic) { ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>(); });
+    });
+  }
+  const unsigned long long t1 = __builtin_readcyclecounter();
+  asm volatile("s_nop 15\n\ts_nop 15");
+  sink[blockIdx.x * 256 + threadIdx.x] = ReadSum<0>() + ReadSum<191>();
+  if (blockIdx.x == 0 && threadIdx.x == 0) ticks[0] = t1 - t0;
+}
+#endif
+
 template <int WM, int WN, int RA>
 int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, hipStream_t stream) {
   using L = GemmLds<WN, RA>;
@@ -824,5 +865,14 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
 // The tuning build's switch: where the GEMM's waves put their timestamps (device memory), or null.
 extern "C" int llmp_hip_gemm_trace_set(unsigned long long* buffer) {
   return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(llmp_hip::g_gemm_trace), &buffer, sizeof(buffer)));
+}
+// The products probe on `workgroups` workgroups: data 126 x 256 dwords, ticks one 64-bit word, sink 256 floats a
+// workgroup.
+extern "C" int llmp_hip_gemm_probe_products(const void* data, int iters, int workgroups, void* ticks, void* sink, void* stream) {
+  BeginLaunches();
+  if (data == nullptr || ticks == nullptr || sink == nullptr || iters < 1 || workgroups < 1) return Refuse(1, "probe: arguments");
+  hipLaunchKernelGGL(ProductsProbeKernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint32_t*>(data), iters, static_cast<unsigned long long*>(ticks), static_cast<float*>(sink));
+  return LaunchStatus("probe");
 }
 #endif

@@ -2,7 +2,8 @@
 finish the last step and queue their stores, and the shader clock meanwhile. Needs the instrumented build
 (`make -C llmp_amd/csrc trace`).
 
-    python -m llmp_amd.gemm_timeline"""
+    python -m llmp_amd.gemm_timeline
+    python -m llmp_amd.gemm_timeline probe      # the matrix pipe alone: a step's 48 products from registers, in a loop"""
 import ctypes as C, os, sys
 import numpy as np, torch
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -13,6 +14,29 @@ from llmp_amd import ops
 lib = _lib.load()
 lib.llmp_hip_gemm_trace_set.argtypes = [C.c_void_p]
 dev = torch.device("cuda:0")
+if len(sys.argv) > 1 and sys.argv[1] == "probe":
+    # The matrix pipe alone: the kernel's 48 products of a step from registers, nothing between them, on every CU.
+    lib.llmp_hip_gemm_probe_products.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    cus = lib.llmp_hip_compute_units()
+    ticks = torch.zeros(1, dtype=torch.int64, device=dev)
+    sink = torch.zeros(cus * 256, dtype=torch.float32, device=dev)
+    g = torch.Generator().manual_seed(5)
+    codes = torch.randint(0, 256, (126 * 256 * 4,), generator=g, dtype=torch.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x38  # no NaN codes
+    for name, data in (("zeros", torch.zeros(126 * 256, dtype=torch.int32)), ("random E4M3 codes", codes.view(torch.int32))):
+        data = data.to(dev)
+        for groups in (cus, 1):
+            iters = 20000
+            b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, ticks.data_ptr(), sink.data_ptr(), None) == 0
+            b.record()
+            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, ticks.data_ptr(), sink.data_ptr(), None) == 0
+            e.record(); torch.cuda.synchronize()
+            ns = b.elapsed_time(e) * 1e6 / (48 * iters)
+            t = int(ticks.item()) / (48 * iters)
+            print(f"{name:18s} {groups:3d} workgroups: {t:.2f} ticks of the shader counter a product, {ns:.2f} ns a product -> {t / ns:.2f} GHz, "
+                  f"{groups * 4 * 65536 / ns / 1e6:.2f} PFLOP/s")
+    sys.exit(0)
 m, n, k = 2048, 12288, 4096
 g = torch.Generator().manual_seed(3)
 a = torch.randn((m, k), generator=g).to(dev).to(torch.bfloat16)
