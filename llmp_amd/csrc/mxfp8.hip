@@ -426,7 +426,15 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
   constexpr int kXFrags = R::kXFrags;
   constexpr int kLoadsA = kTileABytes / 16 / kThreads;     // 8 or 4 a thread a stage
   constexpr int kLoadsB = L::kTileBBytes / 16 / kThreads;  // WN or half of it
-  static_assert(L::kTileBBytes % (16 * kThreads) == 0 && kLoadsA + 1 + kLoadsB <= kXFrags * WN, "load slots");
+  // A load after every kLoadEvery-th product: a CU's path to LDS takes 64 bytes a cycle, its four waves' loads after
+  // every product would ask for 128 (1 KB a wave every 32 cycles) and hold the next products back.
+  constexpr int kLoadEveryMost = kXFrags * WN / (kLoadsA + 1 + kLoadsB);
+#ifndef LLMP_GEMM_LOAD_EVERY
+  constexpr int kLoadEvery = kLoadEveryMost;
+#else
+  constexpr int kLoadEvery = LLMP_GEMM_LOAD_EVERY < kLoadEveryMost ? LLMP_GEMM_LOAD_EVERY : kLoadEveryMost;
+#endif
+  static_assert(L::kTileBBytes % (16 * kThreads) == 0 && (kLoadsA + 1 + kLoadsB) * kLoadEvery <= kXFrags * WN, "load slots");
   // The kernel's register counts cover the named ones.
   if constexpr (WM == 2) {
     asm volatile("" ::: "v253", "a191");
@@ -583,13 +591,14 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
         constexpr int i = decltype(ic)::value;
         ScaledProduct<R, kXFrags * i + j, i, j>();
         constexpr int t = j * WN + i;
+        constexpr int q = t % kLoadEvery == 0 ? t / kLoadEvery : kLoadsA + 1 + kLoadsB;  // the load after product t
         if constexpr ((LLMP_GEMM_WITHOUT & 1) != 0) {
-        } else if constexpr (t < kLoadsA) {
-          load_a(t, bring_a, stage_a);
-        } else if constexpr (t == kLoadsA) {
+        } else if constexpr (q < kLoadsA) {
+          load_a(q, bring_a, stage_a);
+        } else if constexpr (q == kLoadsA) {
           load_scales(bring_a, stage_a, bring_b, stage_b);
-        } else if constexpr (t - kLoadsA - 1 < kLoadsB) {
-          load_b(t - kLoadsA - 1, bring_b, stage_b);
+        } else if constexpr (q - kLoadsA - 1 < kLoadsB) {
+          load_b(q - kLoadsA - 1, bring_b, stage_b);
         }
         if constexpr (j == kXFrags - 1 && (LLMP_GEMM_WITHOUT & 2) == 0) read_b(ic);
         __builtin_amdgcn_sched_barrier(0);
@@ -700,10 +709,36 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   StaticFor<R::kSums>([&](auto t) { ClearSum<decltype(t)::value>(); });
   asm volatile("s_nop 7");
   const unsigned long long t0 = __builtin_readcyclecounter();
+  // LLMP_GEMM_PROBE_BETWEEN: one more instruction of the same wave after every product (what it costs the pipe):
+  //   1 a vector move   2 a 16-byte read of LDS into registers no product uses   3 the same into the activation
+  //   fragment the product has just been issued from   4 a 16-byte load a lane from `data` to LDS
+#ifndef LLMP_GEMM_PROBE_BETWEEN
+#define LLMP_GEMM_PROBE_BETWEEN 0
+#endif
+  __shared__ __attribute__((aligned(16))) uint8_t probe_lds[4096];
+  const uint32_t probe_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x & 63) * 16;
+  const uint32_t probe_to =
+      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x >> 6) * 1024);
+  const uint32_t probe_from = threadIdx.x * 16;
+  auto between = [&](auto jc) {
+    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 1) {
+      asm volatile("v_mov_b32 v120, v121" ::: "v120");
+    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 2) {
+      asm volatile("ds_read_b128 v[120:123], %0" ::"v"(probe_at) : "v120", "v121", "v122", "v123");
+    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 3) {
+      LdsToRegs16<R::kX + 8 * decltype(jc)::value, 0>(probe_at);
+    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 4) {
+      GlobalToLds16(reinterpret_cast<const uint8_t*>(data), probe_from, probe_to);
+    }
+  };
   for (int it = 0; it < iters; ++it) {
     StaticFor<8>([&](auto jc) {
-      StaticFor<6>([&](auto ic) { ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>(); });
+      StaticFor<6>([&](auto ic) {
+        ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>();
+        between(jc);
+      });
     });
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)");
   }
   const unsigned long long t1 = __builtin_readcyclecounter();
   asm volatile("s_nop 15\n\ts_nop 15");
