@@ -358,30 +358,42 @@ __device__ __forceinline__ void StaticFor(F&& f) {
 // The loop's registers are named, not allocated: left to itself the compiler copies an accumulator before every
 // product whose neighbours are loads (its D and C end up in different registers) and builds each 32-byte operand
 // out of two 16-byte reads with eight moves, all of them on the one pipe that also issues the products.
-//   a[4 t .. 4 t + 3], t = 8 i + j        product (i, j)'s sums (192 of the upper registers at WN = 6); numbers for WM = 2
-//   v[128 + 8 j ..], j < 8                activation fragment j: the lane's chunks g and 4 + g of row 16 j + r
-//   v[192 + 8 i ..], i < WN               weight fragment i
-//   v[240 + j], v[248 + i]                their scales, a byte each
-// The compiler keeps to v0 .. v127 (amdgpu_num_vgpr) and is told once that the kernel uses the rest; what it may
+// With four waves a workgroup (WM = 2, WN = 6):
+//   a[4 t .. 4 t + 3], t = 8 i + j        product (i, j)'s sums (192 of the upper registers)
+//   v[64 + 8 b ..], b < 9                 activation fragment j < 7 in b = j: the lane's chunks g and 4 + g of row
+//                                         16 j + r; fragment 7 in b = 7 on even steps and b = 8 on odd ones
+//   v[136 + 48 p + 8 i ..], i < 6         weight fragment i of a step of parity p
+//   v[232 + b], v[241 + 6 p + i]          their scales, a byte each
+// The second set lets the next step's weight fragments and last activation fragment be read at any time in a step,
+// so a step's 42 reads of LDS go one after a product, none in a burst at the step's end. With eight waves (WM = 4)
+// there is one set: a fragment's registers are refilled when its last product has been issued.
+// The compiler keeps to v0 .. v63 (amdgpu_num_vgpr) and is told once that the kernel uses the rest; what it may
 // not see is listed with each helper.
-// v0 .. for the compiler: 128 of them with four waves a workgroup, 64 with eight.
-constexpr int GemmCompilerVgprs(int wm) { return wm == 2 ? 128 : 64; }
+constexpr int GemmCompilerVgprs(int) { return 64; }
 
 // WM waves share the tile's 256 activation rows (2 waves of weights each): 2, a wave a SIMD with 448 registers, or 4, two
-// waves a SIMD with 256 each. A wave's instruction after a matrix product is not issued before the product is (nearly)
-// through the pipe, so a wave that is alone on its SIMD pays for every load and read with the pipe idle; a second wave
-// fills that time, but each of the eight then reads 20 KB of fragments a step where each of four reads 28 KB.
+// waves a SIMD with 256 each; each of the eight then reads 20 KB of fragments a step where each of four reads 28 KB.
 template <int WM, int WN>
 struct GemmRegs {
   static constexpr int kXFrags = 16 / WM;                    // 16-row activation fragments a wave
+  static constexpr bool kTwice = WM == 2;                    // two sets of weight fragments, two places for the last activation fragment
+  static constexpr int kXBuffers = kXFrags + (kTwice ? 1 : 0);
+  static constexpr int kWSets = kTwice ? 2 : 1;
   static constexpr int kCompilerVgprs = GemmCompilerVgprs(WM);  // v0 .. for the compiler
   static constexpr int kX = kCompilerVgprs;
-  static constexpr int kW = kX + 8 * kXFrags;
-  static constexpr int kXScale = kW + 8 * WN;
-  static constexpr int kWScale = kXScale + kXFrags;
-  static constexpr int kTop = kWScale + WN;
+  static constexpr int kW = kX + 8 * kXBuffers;
+  static constexpr int kXScale = kW + 8 * WN * kWSets;
+  static constexpr int kWScale = kXScale + kXBuffers;
+  static constexpr int kTop = kWScale + WN * kWSets;
   static constexpr int kSums = 4 * kXFrags * WN;
   static_assert(WM == 2 ? (kTop <= 254 && kSums <= 192) : (kTop <= 160 && kSums <= 96), "the register file");
+  static_assert(!kTwice || WN >= 4, "a row of products has a slot for each of four reads");
+  // Where fragment j (i) of a step of parity p lies, and its scale.
+  static constexpr int XBuffer(int j, int p) { return kTwice && j == kXFrags - 1 ? j + p : j; }
+  static constexpr int X(int j, int p) { return kX + 8 * XBuffer(j, p); }
+  static constexpr int XScale(int j, int p) { return kXScale + XBuffer(j, p); }
+  static constexpr int W(int i, int p) { return kW + 8 * (i + (kTwice ? p * WN : 0)); }
+  static constexpr int WScale(int i, int p) { return kWScale + i + (kTwice ? p * WN : 0); }
 };
 
 // Fragment registers REG .. REG + 3 from LDS. In flight until the wave's next s_waitcnt lgkmcnt(0).
@@ -398,13 +410,13 @@ __device__ __forceinline__ void GlobalToLds16(const uint8_t* base, uint32_t offs
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(to), "v"(offset), "s"(base));
 }
 
-// sums(T) += weights(I) x activations(J), both scaled.
-template <class R, int T, int I, int J>
+// sums(T) += weights(I) x activations(J) of a step of parity P, both scaled.
+template <class R, int T, int I, int J, int P = 0>
 __device__ __forceinline__ void ScaledProduct() {
   asm volatile(
       "v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%0+3], v[%1:%1+7], v[%2:%2+7], a[%0:%0+3], v[%3], v[%4] op_sel_hi:[0,0,0]" ::"n"(
           T * 4),
-      "n"(R::kW + 8 * I), "n"(R::kX + 8 * J), "n"(R::kWScale + I), "n"(R::kXScale + J));
+      "n"(R::W(I, P)), "n"(R::X(J, P)), "n"(R::WScale(I, P)), "n"(R::XScale(J, P)));
 }
 template <int REG>
 __device__ __forceinline__ void ClearSum() {
@@ -524,17 +536,33 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     b_hi = frag_b + chunk_hi + static_cast<uint32_t>(stage_b * L::kTileBBytes);
     b_scale = scale_b_base + static_cast<uint32_t>(stage_b * kScaleStageBytes);
   };
-  auto read_a = [&](auto jc) {
-    constexpr int j = decltype(jc)::value;
-    LdsToRegs16<R::kX + 8 * j, j * 2048>(a_lo);
-    LdsToRegs16<R::kX + 8 * j + 4, j * 2048>(a_hi);
-    LdsToReg1<R::kXScale + j, (j % 2) * 256 + (j / 2) * 4>(a_scale);
+  // Fragment j (i) of the step the reads are aimed at, into the registers of parity p: its lower chunk, its upper
+  // chunk and scale byte, or both.
+  auto read_a_lo = [&](auto jc, auto pc) {
+    constexpr int j = decltype(jc)::value, p = decltype(pc)::value;
+    LdsToRegs16<R::X(j, p), j * 2048>(a_lo);
   };
-  auto read_b = [&](auto ic) {
-    constexpr int i = decltype(ic)::value;
-    LdsToRegs16<R::kW + 8 * i, i * 2048>(b_lo);
-    LdsToRegs16<R::kW + 8 * i + 4, i * 2048>(b_hi);
-    LdsToReg1<R::kWScale + i, 0>(b_scale + static_cast<uint32_t>(scale_b_off[i]));
+  auto read_a_hi = [&](auto jc, auto pc) {
+    constexpr int j = decltype(jc)::value, p = decltype(pc)::value;
+    LdsToRegs16<R::X(j, p) + 4, j * 2048>(a_hi);
+    LdsToReg1<R::XScale(j, p), (j % 2) * 256 + (j / 2) * 4>(a_scale);
+  };
+  auto read_b_lo = [&](auto ic, auto pc) {
+    constexpr int i = decltype(ic)::value, p = decltype(pc)::value;
+    LdsToRegs16<R::W(i, p), i * 2048>(b_lo);
+  };
+  auto read_b_hi = [&](auto ic, auto pc) {
+    constexpr int i = decltype(ic)::value, p = decltype(pc)::value;
+    LdsToRegs16<R::W(i, p) + 4, i * 2048>(b_hi);
+    LdsToReg1<R::WScale(i, p), 0>(b_scale + static_cast<uint32_t>(scale_b_off[i]));
+  };
+  auto read_a = [&](auto jc, auto pc) {
+    read_a_lo(jc, pc);
+    read_a_hi(jc, pc);
+  };
+  auto read_b = [&](auto ic, auto pc) {
+    read_b_lo(ic, pc);
+    read_b_hi(ic, pc);
   };
   auto read_done = [&]() { asm volatile("s_waitcnt lgkmcnt(0)"); };
   auto barrier = [&]() {
@@ -566,13 +594,18 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
   barrier();
   GEMM_TRACE(2);  // ... and landed, for every wave
   aim_reads(0, 0);
-  StaticFor<kXFrags>([&](auto j) { read_a(j); });
-  StaticFor<WN>([&](auto i) { read_b(i); });
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+  StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
+  StaticFor<WN>([&](auto i) { read_b(i, Even{}); });
   read_done();
 
   int stage_a = 0;  // step s's activation stage, s % RA
   int stage_b = 0;  // step s's weight stage, s % 3
-  for (int step = 0; step < steps; ++step) {
+  // One step, its fragments in the registers of parity P, the next step's read into those of the other parity.
+  auto multiply = [&](auto pc, int step) {
+    constexpr int P = decltype(pc)::value;
+    using Next = std::integral_constant<int, R::kTwice ? 1 - P : 0>;
     if (step == 1) GEMM_TRACE(3);
     if (step == steps / 2) GEMM_TRACE(4);
     if constexpr ((LLMP_GEMM_WITHOUT & 4) == 0) barrier();
@@ -581,15 +614,17 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     const int next_a = stage_a + 1 == RA ? 0 : stage_a + 1;      // step + 1's activations
     const int next_b = stage_b + 1 == kRingB ? 0 : stage_b + 1;  // step + 1's weights
     const int bring_a = min(step + RA, steps - 1), bring_b = min(step + 3, steps - 1);
-    // An action after every product: the loads first (activations, their scales, weights), and the next step's
-    // fragments into the registers a row (the weights: the last row) has just been multiplied from.
+    // After a product at most one load (activations, their scales, weights) and one read of the next step's
+    // fragments. With two sets of registers: in row j the activation fragment row j - 1 was multiplied from (in row
+    // 0 the last fragment, into its other place), and in the first WN rows a weight fragment each, into the other set.
+    // With one: a fragment's registers are refilled when its row (the weights: the last row) has been issued.
     aim_reads(next_a, next_b);
     __builtin_amdgcn_sched_barrier(0);
     StaticFor<kXFrags>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
       StaticFor<WN>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        ScaledProduct<R, kXFrags * i + j, i, j>();
+        ScaledProduct<R, kXFrags * i + j, i, j, P>();
         constexpr int t = j * WN + i;
         constexpr int q = t % kLoadEvery == 0 ? t / kLoadEvery : kLoadsA + 1 + kLoadsB;  // the load after product t
         if constexpr ((LLMP_GEMM_WITHOUT & 1) != 0) {
@@ -600,10 +635,19 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
         } else if constexpr (q - kLoadsA - 1 < kLoadsB) {
           load_b(q - kLoadsA - 1, bring_b, stage_b);
         }
-        if constexpr (j == kXFrags - 1 && (LLMP_GEMM_WITHOUT & 2) == 0) read_b(ic);
+        if constexpr ((LLMP_GEMM_WITHOUT & 2) != 0) {
+        } else if constexpr (R::kTwice) {
+          using Before = std::integral_constant<int, j == 0 ? kXFrags - 1 : j - 1>;
+          if constexpr (i == 0) read_a_lo(Before{}, Next{});
+          if constexpr (i == 1) read_a_hi(Before{}, Next{});
+          if constexpr (i == 2 && j < WN) read_b_lo(jc, Next{});
+          if constexpr (i == 3 && j < WN) read_b_hi(jc, Next{});
+        } else if constexpr (j == kXFrags - 1) {
+          read_b(ic, Next{});
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr ((LLMP_GEMM_WITHOUT & 2) == 0) read_a(jc);
+      if constexpr ((LLMP_GEMM_WITHOUT & 2) == 0 && !R::kTwice) read_a(jc, Next{});
       __builtin_amdgcn_sched_barrier(0);
     });
     read_done();
@@ -619,6 +663,10 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     }
     stage_a = next_a;
     stage_b = next_b;
+  };
+  for (int step = 0; step < steps; step += 2) {
+    multiply(Even{}, step);
+    if (step + 1 < steps) multiply(Odd{}, step + 1);
   }
   GEMM_TRACE(5);  // the last step multiplied
   AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
@@ -699,7 +747,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   asm volatile("" ::: "v253", "a191");
   StaticFor<R::kXScale - R::kX>([&](auto rc) {
     constexpr int reg = R::kX + decltype(rc)::value;
-    const uint32_t v = data[decltype(rc)::value * 256 + threadIdx.x];
+    const uint32_t v = data[decltype(rc)::value % 126 * 256 + threadIdx.x];
     asm volatile("v_mov_b32 v[%0], %1" ::"n"(reg), "v"(v));
   });
   StaticFor<R::kTop - R::kXScale>([&](auto rc) {
@@ -711,7 +759,8 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   const unsigned long long t0 = __builtin_readcyclecounter();
   // LLMP_GEMM_PROBE_BETWEEN: one more instruction of the same wave after every product (what it costs the pipe):
   //   1 a vector move   2 a 16-byte read of LDS into registers no product uses   3 the same into the activation
-  //   fragment the product has just been issued from   4 a 16-byte load a lane from `data` to LDS
+  //   fragment the product has just been issued from   4 a 16-byte load a lane from `data` to LDS   5 that load
+  //   after every third product
 #ifndef LLMP_GEMM_PROBE_BETWEEN
 #define LLMP_GEMM_PROBE_BETWEEN 0
 #endif
@@ -720,14 +769,14 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   const uint32_t probe_to =
       __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x >> 6) * 1024);
   const uint32_t probe_from = threadIdx.x * 16;
-  auto between = [&](auto jc) {
+  auto between = [&](auto jc, auto ic) {
     if constexpr (LLMP_GEMM_PROBE_BETWEEN == 1) {
       asm volatile("v_mov_b32 v120, v121" ::: "v120");
     } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 2) {
       asm volatile("ds_read_b128 v[120:123], %0" ::"v"(probe_at) : "v120", "v121", "v122", "v123");
     } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 3) {
-      LdsToRegs16<R::kX + 8 * decltype(jc)::value, 0>(probe_at);
-    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 4) {
+      LdsToRegs16<R::X(decltype(jc)::value, 0), 0>(probe_at);
+    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 4 || (LLMP_GEMM_PROBE_BETWEEN == 5 && decltype(ic)::value % 3 == 0)) {
       GlobalToLds16(reinterpret_cast<const uint8_t*>(data), probe_from, probe_to);
     }
   };
@@ -735,7 +784,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
     StaticFor<8>([&](auto jc) {
       StaticFor<6>([&](auto ic) {
         ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>();
-        between(jc);
+        between(jc, ic);
       });
     });
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)");

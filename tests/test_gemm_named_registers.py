@@ -12,7 +12,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 # kernel -> (the compiler's registers v0 .. below this, the highest named register, the sums' registers)
-SHAPES = {"GemmKernel192": (128, 253, 192), "GemmKernel128": (128, 251, 128)}
+SHAPES = {"GemmKernel192": (64, 252, 192), "GemmKernel128": (64, 216, 128)}
 
 
 def kernels(assembly):
