@@ -258,15 +258,16 @@ struct GemmArgs {
 };
 
 // Timeline instrumentation for tuning, compiled only with -DLLMP_GEMM_TRACE (never into the library): lane 0 of
-// every wave stores the 100 MHz clock at up to eight points of its tile, eight 64-bit words a wave.
+// every wave stores the 100 MHz clock at up to eight points of its first tile and of its later ones (the last of
+// them stays), sixteen 64-bit words a wave.
 #ifdef LLMP_GEMM_TRACE
 __device__ unsigned long long* g_gemm_trace = nullptr;
-// The wave's eight slots, asked for once at the kernel's start (read at every stamp, the pointer's two loads and
+// The wave's sixteen slots, asked for once at the kernel's start (read at every stamp, the pointer's two loads and
 // their waits would be part of every step that is timed).
 #define GEMM_TRACE_BEGIN                                                                                     \
   unsigned long long* gemm_trace_slots = g_gemm_trace;                                                       \
   if (gemm_trace_slots != nullptr)                                                                           \
-    gemm_trace_slots += (static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8
+    gemm_trace_slots += (static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 16
 #define GEMM_TRACE(slot)                                                                     \
   do {                                                                                       \
     if (gemm_trace_slots != nullptr && (threadIdx.x & 63) == 0) gemm_trace_slots[slot] = wall_clock64(); \
@@ -410,13 +411,18 @@ __device__ __forceinline__ void GlobalToLds16(const uint8_t* base, uint32_t offs
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(to), "v"(offset), "s"(base));
 }
 
-// sums(T) += weights(I) x activations(J) of a step of parity P, both scaled.
-template <class R, int T, int I, int J, int P = 0>
+// sums(T) += weights(I) x activations(J) of a step of parity P, both scaled; FIRST: sums(T) = that product.
+template <class R, int T, int I, int J, int P = 0, bool FIRST = false>
 __device__ __forceinline__ void ScaledProduct() {
-  asm volatile(
-      "v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%0+3], v[%1:%1+7], v[%2:%2+7], a[%0:%0+3], v[%3], v[%4] op_sel_hi:[0,0,0]" ::"n"(
-          T * 4),
-      "n"(R::W(I, P)), "n"(R::X(J, P)), "n"(R::WScale(I, P)), "n"(R::XScale(J, P)));
+  if constexpr (FIRST) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%0+3], v[%1:%1+7], v[%2:%2+7], 0, v[%3], v[%4] op_sel_hi:[0,0,0]" ::"n"(T * 4),
+                 "n"(R::W(I, P)), "n"(R::X(J, P)), "n"(R::WScale(I, P)), "n"(R::XScale(J, P)));
+  } else {
+    asm volatile(
+        "v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%0+3], v[%1:%1+7], v[%2:%2+7], a[%0:%0+3], v[%3], v[%4] op_sel_hi:[0,0,0]" ::"n"(
+            T * 4),
+        "n"(R::W(I, P)), "n"(R::X(J, P)), "n"(R::WScale(I, P)), "n"(R::XScale(J, P)));
+  }
 }
 template <int REG>
 __device__ __forceinline__ void ClearSum() {
@@ -429,8 +435,16 @@ __device__ __forceinline__ float ReadSum() {
   return v;
 }
 
+// Two floats to BF16 (nearest, ties to even; a NaN stays a quiet NaN) in one dword, `lo` in the low half: one
+// instruction where the shifts and adds take six a value, 192 values a lane a tile.
+__device__ __forceinline__ uint32_t PackBf16(float lo, float hi) {
+  uint32_t packed;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(packed) : "v"(lo), "v"(hi));
+  return packed;
+}
+
 template <int WM, int WN, int RA>
-__device__ __forceinline__ void GemmTile(const GemmArgs& a) {
+__device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   using L = GemmLds<WN, RA>;
   using R = GemmRegs<WM, WN>;
   constexpr int kTileN = L::kTileN;
@@ -462,41 +476,63 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
   const int wm = wave % WM, wn = wave / WM;  // (the two waves of a SIMD, w and w + 4, differ in both)
   const int r = lane & 15, g = lane >> 4;
 
-  int tile = blockIdx.x;
+  // This workgroup's tiles: positions blockIdx.x, + gridDim.x, ... of the launch's order (an XCD a run of tiles, m
+  // fastest), one after the other: `mine` of them.
   const int tiles = a.tiles_m * a.tiles_n;
-  if (tiles % 8 == 0) tile = (tile % 8) * (tiles / 8) + tile / 8;  // an XCD a run of tiles, m fastest
-  const int tm = tile % a.tiles_m, tn = tile / a.tiles_m;
-  const int m0 = tm * kTileM, n0 = tn * kTileN;
   const int steps = a.k / kStepK;
   const int blocks = a.k / 32;
+  const int mine = (tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+  auto origin = [&](int ord, int& m0, int& n0) {
+    int tile = static_cast<int>(blockIdx.x) + ord * static_cast<int>(gridDim.x);
+    if (tiles % 8 == 0) tile = (tile % 8) * (tiles / 8) + tile / 8;
+    m0 = tile % a.tiles_m * kTileM;
+    n0 = tile / a.tiles_m * kTileN;
+  };
+  const int atoms_a = (a.m + 127) / 128, atoms_b = (a.n + 127) / 128;
 
   // What this thread brings of a stage: position T i + tid of either tile (T threads) is row T / 8 i + tid / 8, and the chunk
-  // there is the same for every i.
-  const uint32_t chunk_from = static_cast<uint32_t>(((tid & 7) ^ ((tid >> 4) & 7)) * 16);
-  const int a_row = m0 + (tid >> 3), b_row = n0 + (tid >> 3);
-  const int atom_b0 = n0 / 128;
-  const int atoms_a = (a.m + 127) / 128, atoms_b = (a.n + 127) / 128;
+  // there is the same for every i. Where its chunks come from, the step's 128 bytes aside (they go into the scalar
+  // base), is kept for the whole tile: a vector instruction in the loop takes a matrix instruction's place.
   // The scales: wave 0 the activations', wave 1 the weights', two atoms a stage, 16 bytes a lane.
-  const int atom_mine = wave == 0 ? min(m0 / 128 + (lane >> 5), atoms_a - 1) : min(atom_b0 + (lane >> 5), atoms_b - 1);
+  const uint32_t chunk_from = static_cast<uint32_t>(((tid & 7) ^ ((tid >> 4) & 7)) * 16);
   const uint8_t* const scales_of = wave == 0 ? a.a_scales : a.b_scales;
-  const uint32_t scale_from = static_cast<uint32_t>(atom_mine) * static_cast<uint32_t>(blocks / 4) * 512u + (lane & 31) * 16;
-
-  // Where this thread's chunks of a stage come from, the step's 128 bytes aside (they go into the scalar base):
-  // kept for the whole tile, a vector instruction in the loop takes a matrix instruction's place.
-  uint32_t a_from[kLoadsA], b_from[kLoadsB];
-#pragma unroll
-  for (int i = 0; i < kLoadsA; ++i)
-    a_from[i] = static_cast<uint32_t>(min(a_row + kThreads / 8 * i, a.m - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
-#pragma unroll
-  for (int i = 0; i < kLoadsB; ++i)
-    b_from[i] = static_cast<uint32_t>(min(b_row + kThreads / 8 * i, a.n - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
+  // Load i's rows lie 32 k bytes (T / 8 rows) after load i - 1's, but never past the operand's last row: one
+  // register for the first load's place and one for the last row's, an add and a minimum a load (vector instructions
+  // that are issued while a product runs), not a register a load.
+  uint32_t a_from = 0, b_from = 0, scale_from = 0;
+  const uint32_t a_last = static_cast<uint32_t>(a.m - 1) * static_cast<uint32_t>(a.k) + chunk_from;
+  const uint32_t b_last = static_cast<uint32_t>(a.n - 1) * static_cast<uint32_t>(a.k) + chunk_from;
+  const uint32_t load_stride = static_cast<uint32_t>(kThreads / 8) * static_cast<uint32_t>(a.k);
+  auto aim_loads = [&](int ord) {
+    int m0, n0;
+    origin(ord, m0, n0);
+    a_from = static_cast<uint32_t>(min(m0 + (tid >> 3), a.m - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
+    b_from = static_cast<uint32_t>(min(n0 + (tid >> 3), a.n - 1)) * static_cast<uint32_t>(a.k) + chunk_from;
+    const int atom_mine = wave == 0 ? min(m0 / 128 + (lane >> 5), atoms_a - 1) : min(n0 / 128 + (lane >> 5), atoms_b - 1);
+    scale_from = static_cast<uint32_t>(atom_mine) * static_cast<uint32_t>(blocks / 4) * 512u + (lane & 31) * 16;
+  };
   const uint32_t lds_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
   const uint32_t to_mine = lds_at + static_cast<uint32_t>(wave * 64 * 16);
   auto load_a = [&](int i, int step, int stage) {
-    GlobalToLds16(a.a + step * kStepK, a_from[i], to_mine + static_cast<uint32_t>(L::kA + stage * kTileABytes + i * kThreads * 16));
+    GlobalToLds16(a.a + step * kStepK, min(a_from + static_cast<uint32_t>(i) * load_stride, a_last),
+                  to_mine + static_cast<uint32_t>(L::kA + stage * kTileABytes + i * kThreads * 16));
   };
   auto load_b = [&](int i, int step, int stage) {
-    GlobalToLds16(a.b + step * kStepK, b_from[i], to_mine + static_cast<uint32_t>(L::kB + stage * L::kTileBBytes + i * kThreads * 16));
+    GlobalToLds16(a.b + step * kStepK, min(b_from + static_cast<uint32_t>(i) * load_stride, b_last),
+                  to_mine + static_cast<uint32_t>(L::kB + stage * L::kTileBBytes + i * kThreads * 16));
+  };
+  // The same in the loop, where a load whose place is computed just before it would wait for that result with the
+  // next product behind it: each load leaves the next one's place in `load_from`.
+  uint32_t load_from = 0;
+  auto load_a_ahead = [&](int i, int step, int stage) {
+    GlobalToLds16(a.a + step * kStepK, i == 0 ? a_from : load_from,
+                  to_mine + static_cast<uint32_t>(L::kA + stage * kTileABytes + i * kThreads * 16));
+    if (i + 1 < kLoadsA) load_from = min(a_from + static_cast<uint32_t>(i + 1) * load_stride, a_last);
+  };
+  auto load_b_ahead = [&](int i, int step, int stage) {
+    GlobalToLds16(a.b + step * kStepK, i == 0 ? b_from : load_from,
+                  to_mine + static_cast<uint32_t>(L::kB + stage * L::kTileBBytes + i * kThreads * 16));
+    if (i + 1 < kLoadsB) load_from = min(b_from + static_cast<uint32_t>(i + 1) * load_stride, b_last);
   };
   // A stage's scales: wave 0 the activations' into stage_a, wave 1 the weights' into stage_b. (A wave-uniform branch
   // around one load each: the waits below count a wave's loads, and these waves have one more.)
@@ -520,10 +556,13 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
   const uint32_t scale_a_base = lds_at + L::kAScales + static_cast<uint32_t>(scale_at(wm * kXFrags, 0) + scale_lane);
   const uint32_t scale_b_base = lds_at + L::kBScales + static_cast<uint32_t>(scale_lane);
   int scale_b_off[WN];
+  auto aim_weight_scales = [&](int ord) {
+    int m0, n0;
+    origin(ord, m0, n0);
 #pragma unroll
-  for (int i = 0; i < WN; ++i) scale_b_off[i] = __builtin_amdgcn_readfirstlane(scale_at(n0 / 16 + wn * WN + i, atom_b0));
+    for (int i = 0; i < WN; ++i) scale_b_off[i] = __builtin_amdgcn_readfirstlane(scale_at(n0 / 16 + wn * WN + i, n0 / 128));
+  };
 
-  StaticFor<R::kSums>([&](auto t) { ClearSum<decltype(t)::value>(); });
   // The fragments' registers are refilled in place: an activation fragment's when its row of products has been
   // issued, a weight fragment's when its last product (in the last row) has.
   // (The stage's part of an address is added once an iteration, a fragment's is the instruction's offset.)
@@ -571,43 +610,39 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Before the first step: activations 0 .. RA - 1, weights 0, 1 and 2, each with its scales.
-  StaticFor<(RA > kRingB ? RA : kRingB)>([&](auto sc) {
-    constexpr int stage = decltype(sc)::value;
-    const int step = min(stage, steps - 1);
-    if constexpr (stage < RA) {
+  // A tile's first stages: activations 0 .. RA - 1, weights 0, 1 and 2, each with its scales.
+  auto first_loads = [&]() {
+    StaticFor<(RA > kRingB ? RA : kRingB)>([&](auto sc) {
+      constexpr int stage = decltype(sc)::value;
+      const int step = min(stage, steps - 1);
+      if constexpr (stage < RA) {
 #pragma unroll
-      for (int i = 0; i < kLoadsA; ++i) load_a(i, step, stage);
-    }
-    if constexpr (stage < kRingB) {
+        for (int i = 0; i < kLoadsA; ++i) load_a(i, step, stage);
+      }
+      if constexpr (stage < kRingB) {
 #pragma unroll
-      for (int i = 0; i < kLoadsB; ++i) load_b(i, step, stage);
-    }
-    if (wave == 0) {
-      if constexpr (stage < RA) load_scales(step, stage, step, stage);
-    } else if (wave == 1) {
-      if constexpr (stage < kRingB) load_scales(step, stage, step, stage);
-    }
-  });
-  GEMM_TRACE_CYCLES(1);  // the first stages asked for
-  AwaitLoads<0>();
-  barrier();
-  GEMM_TRACE(2);  // ... and landed, for every wave
-  aim_reads(0, 0);
+        for (int i = 0; i < kLoadsB; ++i) load_b(i, step, stage);
+      }
+      if (wave == 0) {
+        if constexpr (stage < RA) load_scales(step, stage, step, stage);
+      } else if (wave == 1) {
+        if constexpr (stage < kRingB) load_scales(step, stage, step, stage);
+      }
+    });
+  };
   using Even = std::integral_constant<int, 0>;
   using Odd = std::integral_constant<int, 1>;
-  StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
-  StaticFor<WN>([&](auto i) { read_b(i, Even{}); });
-  read_done();
 
   int stage_a = 0;  // step s's activation stage, s % RA
   int stage_b = 0;  // step s's weight stage, s % 3
   // One step, its fragments in the registers of parity P, the next step's read into those of the other parity.
-  auto multiply = [&](auto pc, int step) {
+  int ord = 0;  // the tile that is multiplied
+  auto multiply = [&](auto pc, auto firstc, int step) {
     constexpr int P = decltype(pc)::value;
+    constexpr bool kFirst = decltype(firstc)::value;  // the tile's first step starts its sums, the others add to them
     using Next = std::integral_constant<int, R::kTwice ? 1 - P : 0>;
-    if (step == 1) GEMM_TRACE(3);
-    if (step == steps / 2) GEMM_TRACE(4);
+    if (step == 1) GEMM_TRACE(3 + 8 * min(ord, 1));
+    if (step == steps / 2) GEMM_TRACE(4 + 8 * min(ord, 1));
     if constexpr ((LLMP_GEMM_WITHOUT & 4) == 0) barrier();
     // Every wave holds step `step`'s fragments; steps up to `step` + RA - 1 (weights: + 2) are whole in LDS or on
     // their way, step + 1 whole.
@@ -624,16 +659,16 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
       constexpr int j = decltype(jc)::value;
       StaticFor<WN>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        ScaledProduct<R, kXFrags * i + j, i, j, P>();
+        ScaledProduct<R, kXFrags * i + j, i, j, P, kFirst>();
         constexpr int t = j * WN + i;
         constexpr int q = t % kLoadEvery == 0 ? t / kLoadEvery : kLoadsA + 1 + kLoadsB;  // the load after product t
         if constexpr ((LLMP_GEMM_WITHOUT & 1) != 0) {
         } else if constexpr (q < kLoadsA) {
-          load_a(q, bring_a, stage_a);
+          load_a_ahead(q, bring_a, stage_a);
         } else if constexpr (q == kLoadsA) {
           load_scales(bring_a, stage_a, bring_b, stage_b);
         } else if constexpr (q - kLoadsA - 1 < kLoadsB) {
-          load_b(q - kLoadsA - 1, bring_b, stage_b);
+          load_b_ahead(q - kLoadsA - 1, bring_b, stage_b);
         }
         if constexpr ((LLMP_GEMM_WITHOUT & 2) != 0) {
         } else if constexpr (R::kTwice) {
@@ -664,57 +699,89 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
     stage_a = next_a;
     stage_b = next_b;
   };
-  for (int step = 0; step < steps; step += 2) {
-    multiply(Even{}, step);
-    if (step + 1 < steps) multiply(Odd{}, step + 1);
-  }
-  GEMM_TRACE(5);  // the last step multiplied
-  AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
-  // The last products' sums are written passes after their issue: no read of them before.
-  asm volatile("s_nop 15\n\ts_nop 15");
-  GEMM_TRACE_CYCLES(6);
-
-  // sums(8 i + j)[q] = D[m0 + wm 128 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]. A tile inside the matrix (the
-  // common one) stores without a test an element.
-  const int m_first = m0 + wm * 16 * kXFrags + r, n_first = n0 + wn * 16 * WN + 4 * g;  // n is a multiple of 4 (checked on the host)
-  const int64_t first = static_cast<int64_t>(m_first) * a.n + n_first;
-  const int64_t row_step = static_cast<int64_t>(a.n) * 16;
-  auto store = [&](auto bf16, auto whole) {
-    StaticFor<kXFrags>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      StaticFor<WN>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        constexpr int reg = (kXFrags * i + j) * 4;
-        const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
-        if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
-        if ((LLMP_GEMM_WITHOUT & 16) != 0 && v0 != 12345.678f) return;  // (the sums are still read and converted)
-        const int64_t at = first + j * row_step + i * 16;
-        if constexpr (decltype(bf16)::value) {
-          uint2 packed;
-          packed.x = FloatToBf16Bits(v0) | (FloatToBf16Bits(v1) << 16);
-          packed.y = FloatToBf16Bits(v2) | (FloatToBf16Bits(v3) << 16);
-          *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + at) = packed;
-        } else {
-          *reinterpret_cast<float4*>(static_cast<float*>(a.d) + at) = make_float4(v0, v1, v2, v3);
-        }
+  // A finished tile's sums to D: sums(8 i + j)[q] = D[m0 + wm 128 + 16 j + r][n0 + wn 16 WN + 16 i + 4 g + q]. A tile
+  // inside the matrix (the common one) stores without a test an element. The sums stay as they are: the next tile's
+  // first products do not add to them.
+  auto store_tile = [&](int of) {
+    int m0, n0;
+    origin(of, m0, n0);
+    const int m_first = m0 + wm * 16 * kXFrags + r, n_first = n0 + wn * 16 * WN + 4 * g;  // n is a multiple of 4 (checked on the host)
+    const int64_t first = static_cast<int64_t>(m_first) * a.n + n_first;
+    const int64_t row_step = static_cast<int64_t>(a.n) * 16;
+    auto store = [&](auto bf16, auto whole) {
+      StaticFor<kXFrags>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        StaticFor<WN>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          constexpr int reg = (kXFrags * i + j) * 4;
+          const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
+          if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
+          if ((LLMP_GEMM_WITHOUT & 16) != 0 && v0 != 12345.678f) return;  // (the sums are still read and converted)
+          const int64_t at = first + j * row_step + i * 16;
+          if constexpr (decltype(bf16)::value) {
+            uint2 packed;
+            packed.x = PackBf16(v0, v1);
+            packed.y = PackBf16(v2, v3);
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + at) = packed;
+          } else {
+            *reinterpret_cast<float4*>(static_cast<float*>(a.d) + at) = make_float4(v0, v1, v2, v3);
+          }
+        });
       });
-    });
+    };
+    const bool whole = m0 + kTileM <= a.m && n0 + kTileN <= a.n;
+    if (a.bf16) {
+      if (whole) {
+        store(std::true_type{}, std::true_type{});
+      } else {
+        store(std::true_type{}, std::false_type{});
+      }
+    } else {
+      if (whole) {
+        store(std::false_type{}, std::true_type{});
+      } else {
+        store(std::false_type{}, std::false_type{});
+      }
+    }
   };
-  const bool whole = m0 + kTileM <= a.m && n0 + kTileN <= a.n;
-  if (a.bf16) {
-    if (whole) {
-      store(std::true_type{}, std::true_type{});
-    } else {
-      store(std::true_type{}, std::false_type{});
+
+  aim_loads(0);
+  first_loads();
+  GEMM_TRACE_CYCLES(1);  // the first stages asked for
+  for (; ord < mine; ++ord) {
+    aim_weight_scales(ord);
+    // The tile's first stages have landed (they were asked for ahead of the tile before's stores, which this wait
+    // counts as well), for every wave.
+    AwaitLoads<0>();
+    barrier();
+    GEMM_TRACE(2 + 8 * min(ord, 1));
+    aim_reads(0, 0);
+    StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
+    StaticFor<WN>([&](auto i) { read_b(i, Even{}); });
+    read_done();
+    stage_a = 0;
+    stage_b = 0;
+    multiply(Even{}, std::true_type{}, 0);
+    int step = 1;
+    for (; step + 1 < steps; step += 2) {
+      multiply(Odd{}, std::false_type{}, step);
+      multiply(Even{}, std::false_type{}, step + 1);
     }
-  } else {
-    if (whole) {
-      store(std::false_type{}, std::true_type{});
-    } else {
-      store(std::false_type{}, std::false_type{});
+    if (step < steps) multiply(Odd{}, std::false_type{}, step);
+    GEMM_TRACE(5 + 8 * min(ord, 1));  // the tile's last step multiplied
+    // The next tile's first stages are asked for ahead of this tile's stores: they land while the stores are taken.
+    // (This wave's loads still on their way, the last step asked for again, go to places of its own and land first.)
+    if (ord + 1 < mine) {
+      aim_loads(ord + 1);
+      first_loads();
     }
+    // The last products' sums are written passes after their issue: no read of them before.
+    asm volatile("s_nop 15\n\ts_nop 15");
+    GEMM_TRACE_CYCLES(6 + 8 * min(ord, 1));
+    store_tile(ord);
+    GEMM_TRACE(7 + 8 * min(ord, 1));  // the tile's stores queued
   }
-  GEMM_TRACE(7);  // the tile's stores queued
+  AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
 }
 
 // The two tile shapes, four waves each, one a SIMD. (Eight waves of 64 x 64 on the 256 x 128 tile with three
@@ -722,16 +789,16 @@ __device__ __forceinline__ void GemmTile(const GemmArgs& a) {
 // 1.03: eight waves read 176 KB of LDS a step.) A kernel's register attribute cannot depend on a template's argument:
 // one kernel a shape.
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel192(const GemmArgs a) {
-  GemmTile<2, 6, 2>(a);
+  GemmTiles<2, 6, 2>(a);
 }
 #ifndef LLMP_GEMM_EIGHT_WAVES
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel128(const GemmArgs a) {
-  GemmTile<2, 4, 2>(a);
+  GemmTiles<2, 4, 2>(a);
 }
 constexpr int kWavesM128 = 2, kRingA128 = 2;
 #else  // the tuning build's (make trace EXTRA=-DLLMP_GEMM_EIGHT_WAVES): that form, and the 256 x 128 tile wherever it ties
 __global__ __launch_bounds__(512, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(4)))) void GemmKernel128(const GemmArgs a) {
-  GemmTile<4, 4, 3>(a);
+  GemmTiles<4, 4, 3>(a);
 }
 constexpr int kWavesM128 = 4, kRingA128 = 3;
 #endif
@@ -796,14 +863,16 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
 }
 #endif
 
+// A workgroup a compute unit, each through its share of the tiles (fewer workgroups where there are fewer tiles).
 template <int WM, int WN, int RA>
-int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, hipStream_t stream) {
+int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, int compute_units, hipStream_t stream) {
   using L = GemmLds<WN, RA>;
   static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
   a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
   static bool sized = false;
   if (!AllowLds(reinterpret_cast<const void*>(kernel), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
-  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(a.tiles_m * a.tiles_n)), dim3(WM * 128), L::kBytes, stream, a);
+  const int tiles = a.tiles_m * a.tiles_n;
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles < compute_units ? tiles : compute_units)), dim3(WM * 128), L::kBytes, stream, a);
   return LaunchStatus("mxfp8.gemm");
 }
 
@@ -941,7 +1010,7 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
 #endif
   }
   const hipStream_t on = static_cast<hipStream_t>(stream);
-  const int status = best == 192 ? LaunchGemm<2, 6, 2>(GemmKernel192, a, on) : LaunchGemm<kWavesM128, 4, kRingA128>(GemmKernel128, a, on);
+  const int status = best == 192 ? LaunchGemm<2, 6, 2>(GemmKernel192, a, cus, on) : LaunchGemm<kWavesM128, 4, kRingA128>(GemmKernel128, a, cus, on);
   return status;  // negative: the launch failed after the checks (the caller's fault path)
 }
 

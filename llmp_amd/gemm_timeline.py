@@ -50,27 +50,29 @@ b.record()
 for _ in range(20): ops.mxfp8_gemm(ac, asc, wc, wsc, out=d)
 e.record(); torch.cuda.synchronize()
 print(f"gemm {b.elapsed_time(e) / 20 * 1e3:.1f} us (untraced)")
-trace = torch.zeros(512 * 8 * 8, dtype=torch.int64, device=dev)
+trace = torch.zeros(512 * 8 * 16, dtype=torch.int64, device=dev)
 assert lib.llmp_hip_gemm_trace_set(trace.data_ptr()) == 0
 for r in range(3):
     trace.zero_(); torch.cuda.synchronize()
     ops.mxfp8_gemm(ac, asc, wc, wsc, out=d); torch.cuda.synchronize()
-tr = trace.cpu().numpy().reshape(-1, 8).astype(np.float64)
+tr = trace.cpu().numpy().reshape(-1, 16).astype(np.float64)
 tr = tr[tr[:, 0] > 0]  # the buffer has room for eight waves a workgroup
 lib.llmp_hip_gemm_trace_set(None)
 t0 = tr[:, 0].min()
+print("waves:", len(tr), "(a workgroup a CU, its tiles one after the other)")
 names = ["start", "(cycle counter)", "first stages landed", "step 1", "step 16", "last step done", "(cycle counter)", "stores queued"]
-order = np.argsort(tr[:, 0])
-first_round = tr[:, 0] < t0 + 100 * 5.0
-print("waves in the first round:", first_round.sum(), "second:", (~first_round).sum())
-for label, sel in (("first round", first_round), ("second round", ~first_round)):
+for label, base in (("first tile", 0), ("last tile", 8)):
     print(label)
     for j, nm in enumerate(names):
-        if j in (1, 6): continue
-        rel = (tr[sel, j] - t0) / 100
+        if j in (1, 6) or (base and j in (0, 2)): continue
+        rel = (tr[:, base + j] - t0) / 100
         print(f"  {nm:22s} min {rel.min():7.2f} median {np.median(rel):7.2f} max {rel.max():7.2f}")
-    per = tr[sel]
-    print(f"  per wave: start->landed {np.median(per[:,2]-per[:,0])/100:.2f}  landed->step1 {np.median(per[:,3]-per[:,2])/100:.2f}  step1->step16 {np.median(per[:,4]-per[:,3])/100:.2f} (15 steps)  step16->last {np.median(per[:,5]-per[:,4])/100:.2f} (16 steps)  last step->stores queued {np.median(per[:,7]-per[:,5])/100:.2f}")
+    per = tr[:, base:base + 8]
+    if base == 0:
+        print(f"  per wave: start->landed {np.median(per[:,2]-per[:,0])/100:.2f}  landed->step1 {np.median(per[:,3]-per[:,2])/100:.2f}", end="")
+    else:
+        print(f"  per wave: first tile's stores queued->step1 {np.median(per[:,3]-tr[:,7])/100:.2f}", end="")
+    print(f"  step1->step16 {np.median(per[:,4]-per[:,3])/100:.2f} (15 steps)  step16->last {np.median(per[:,5]-per[:,4])/100:.2f} (16 steps)  last step->stores queued {np.median(per[:,7]-per[:,5])/100:.2f}")
 cyc = tr[:, 6] - tr[:, 1]; us = (tr[:, 5] - tr[:, 2]) / 100
-print("shader cycles between slot 1 and 6: median %.0f; us between 2 and 5: %.2f -> clock about %.2f GHz" % (np.median(cyc), np.median(us), np.median(cyc) / np.median(us) / 1e3))
-print("launch by stamps: %.1f us" % ((tr[:, 7].max() - t0) / 100))
+print("first tile: shader cycles between slot 1 and 6: median %.0f; us between 2 and 5: %.2f -> clock about %.2f GHz" % (np.median(cyc), np.median(us), np.median(cyc) / np.median(us) / 1e3))
+print("launch by stamps: %.1f us" % ((tr[:, 15].max() - t0) / 100))

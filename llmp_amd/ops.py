@@ -334,8 +334,10 @@ def mxfp8_gemv(codes, scales, x):
     return y
 
 
-def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, bf16=True, out=None):
-    """llmp.mxfp8.gemm: D[m, n] = A[m, k] B[n, k]^T, scales in atoms."""
+def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, bf16=True, out=None, compute_units=None):
+    """llmp.mxfp8.gemm: D[m, n] = A[m, k] B[n, k]^T, scales in atoms. `compute_units`: the count the reference's run
+    call passes (the device's by default); the launch has no more workgroups than that, each through its share of
+    the tiles."""
     lib = _lib.load()
     m, k = a_codes.shape
     n = b_codes.shape[0]
@@ -347,7 +349,8 @@ def mxfp8_gemm(a_codes, a_scales, b_codes, b_scales, bf16=True, out=None):
                                              b_scales.data_ptr(), out.data_ptr())
     g.bf16 = int(bf16)
     g.scratch = None
-    _lib.check(lib.llmp_hip_mxfp8_gemm_run(C.byref(g), lib.llmp_hip_compute_units(), _stream()))
+    cus = lib.llmp_hip_compute_units() if compute_units is None else int(compute_units)
+    _lib.check(lib.llmp_hip_mxfp8_gemm_run(C.byref(g), cus, _stream()))
     return out
 
 

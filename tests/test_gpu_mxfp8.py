@@ -116,6 +116,25 @@ def test_gemm_matches_the_product_of_the_quantized_operands(device, m, n, k, bf1
     assert np.sum((got - exact) ** 2) / np.sum(exact ** 2) <= 3e-3
 
 
+@pytest.mark.parametrize("m,n,k", [(520, 400, 384), (300, 700, 128), (257, 260, 256), (600, 392, 640)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm_workgroups_that_take_several_tiles(device, m, n, k, bf16):
+    """A workgroup goes through its tiles one after the other, the next tile's first steps asked for while the last
+    steps of this one are multiplied (with one or two K steps a tile, two or three tiles ahead). Whichever workgroup
+    takes a tile, its sums are the same: one, two, three or five workgroups against a workgroup a tile, bit for bit,
+    and that against the oracle."""
+    a, w, (ac, asc), (wc, wsc) = quantized_operands(m, n, k, 60 + m)
+    ops_in = (dev(ac, device), dev(asc, device), dev(wc, device), dev(wsc, device))
+    each = ops.mxfp8_gemm(*ops_in, bf16=bf16, compute_units=4096).cpu()
+    want = oracle.mxfp8_gemm(ac, asc, wc, wsc, threads=oracle.max_threads())
+    got = each.float().numpy()
+    scale = np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), 2e-2 * scale))
+    for cus in (1, 2, 3, 5):
+        few = ops.mxfp8_gemm(*ops_in, bf16=bf16, compute_units=cus).cpu()
+        assert torch.equal(few.view(torch.int16 if bf16 else torch.int32), each.view(torch.int16 if bf16 else torch.int32)), cus
+
+
 def test_gemm_full_size_sampled(device):
     """The headline prefill shape, M 2048, K 4096, N 12288: sampled entries against the oracle's dot, and
     linearity in the activations' scales (doubling a row's scales doubles its outputs exactly)."""
