@@ -809,7 +809,7 @@ constexpr int kWavesM128 = 4, kRingA128 = 3;
 // fragments are filled from `data` (126 dwords a lane: zeros and random codes draw different power), the scales
 // are 1. Lane 0 of the first wave writes the shader counter's ticks over the loop to `ticks`.
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void ProductsProbeKernel(
-    const uint32_t* __restrict__ data, int iters, unsigned long long* ticks, float* sink) {
+    const uint32_t* __restrict__ data, int iters, int stream_slots, unsigned long long* ticks, float* sink) {
   using R = GemmRegs<2, 6>;
   asm volatile("" ::: "v253", "a191");
   StaticFor<R::kXScale - R::kX>([&](auto rc) {
@@ -827,7 +827,8 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   // LLMP_GEMM_PROBE_BETWEEN: one more instruction of the same wave after every product (what it costs the pipe):
   //   1 a vector move   2 a 16-byte read of LDS into registers no product uses   3 the same into the activation
   //   fragment the product has just been issued from   4 a 16-byte load a lane from `data` to LDS   5 that load
-  //   after every third product
+  //   after every third product   6 after every third product a load of bytes that no workgroup has asked for
+  //   before (64 KB an iteration a workgroup from `stream_slots` slots of `data`), the iteration before's in flight
 #ifndef LLMP_GEMM_PROBE_BETWEEN
 #define LLMP_GEMM_PROBE_BETWEEN 0
 #endif
@@ -836,6 +837,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   const uint32_t probe_to =
       __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x >> 6) * 1024);
   const uint32_t probe_from = threadIdx.x * 16;
+  const uint8_t* stream_from = reinterpret_cast<const uint8_t*>(data);
   auto between = [&](auto jc, auto ic) {
     if constexpr (LLMP_GEMM_PROBE_BETWEEN == 1) {
       asm volatile("v_mov_b32 v120, v121" ::: "v120");
@@ -845,17 +847,26 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
       LdsToRegs16<R::X(decltype(jc)::value, 0), 0>(probe_at);
     } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 4 || (LLMP_GEMM_PROBE_BETWEEN == 5 && decltype(ic)::value % 3 == 0)) {
       GlobalToLds16(reinterpret_cast<const uint8_t*>(data), probe_from, probe_to);
+    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6 && decltype(ic)::value % 3 == 0) {
+      GlobalToLds16(stream_from + (decltype(jc)::value * 2 + decltype(ic)::value / 3) * 4096, probe_from, probe_to);
     }
   };
   for (int it = 0; it < iters; ++it) {
+    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6)
+      stream_from = reinterpret_cast<const uint8_t*>(data) + static_cast<size_t>((blockIdx.x * 61u + static_cast<unsigned>(it)) % static_cast<unsigned>(stream_slots)) * 65536;
     StaticFor<8>([&](auto jc) {
       StaticFor<6>([&](auto ic) {
         ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>();
         between(jc, ic);
       });
     });
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)");
+    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6) {
+      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)");
+    }
   }
+  asm volatile("s_waitcnt vmcnt(0)");
   const unsigned long long t1 = __builtin_readcyclecounter();
   asm volatile("s_nop 15\n\ts_nop 15");
   sink[blockIdx.x * 256 + threadIdx.x] = ReadSum<0>() + ReadSum<191>();
@@ -1019,13 +1030,16 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
 extern "C" int llmp_hip_gemm_trace_set(unsigned long long* buffer) {
   return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(llmp_hip::g_gemm_trace), &buffer, sizeof(buffer)));
 }
-// The products probe on `workgroups` workgroups: data 126 x 256 dwords, ticks one 64-bit word, sink 256 floats a
-// workgroup.
-extern "C" int llmp_hip_gemm_probe_products(const void* data, int iters, int workgroups, void* ticks, void* sink, void* stream) {
+// The products probe on `workgroups` workgroups: data 126 x 256 dwords (or `stream_slots` x 64 KB where that is
+// more: what its streaming variant reads), ticks one 64-bit word, sink 256 floats a workgroup.
+extern "C" int llmp_hip_gemm_probe_products(const void* data, int iters, int workgroups, int stream_slots, void* ticks, void* sink,
+                                            void* stream) {
   BeginLaunches();
-  if (data == nullptr || ticks == nullptr || sink == nullptr || iters < 1 || workgroups < 1) return Refuse(1, "probe: arguments");
+  if (data == nullptr || ticks == nullptr || sink == nullptr || iters < 1 || workgroups < 1 || stream_slots < 1)
+    return Refuse(1, "probe: arguments");
   hipLaunchKernelGGL(ProductsProbeKernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint32_t*>(data), iters, static_cast<unsigned long long*>(ticks), static_cast<float*>(sink));
+                     static_cast<const uint32_t*>(data), iters, stream_slots, static_cast<unsigned long long*>(ticks),
+                     static_cast<float*>(sink));
   return LaunchStatus("probe");
 }
 #endif

@@ -16,7 +16,9 @@ lib.llmp_hip_gemm_trace_set.argtypes = [C.c_void_p]
 dev = torch.device("cuda:0")
 if len(sys.argv) > 1 and sys.argv[1] == "probe":
     # The matrix pipe alone: the kernel's 48 products of a step from registers, nothing between them, on every CU.
-    lib.llmp_hip_gemm_probe_products.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.llmp_hip_gemm_probe_products.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    # (A build with -DLLMP_GEMM_PROBE_BETWEEN=6 streams `slots` x 64 KB of `data`: LLMP_PROBE_STREAM_MB says how much.)
+    slots = max(1, int(os.environ.get("LLMP_PROBE_STREAM_MB", "0")) * 16)
     cus = lib.llmp_hip_compute_units()
     ticks = torch.zeros(1, dtype=torch.int64, device=dev)
     sink = torch.zeros(cus * 256, dtype=torch.float32, device=dev)
@@ -25,12 +27,14 @@ if len(sys.argv) > 1 and sys.argv[1] == "probe":
     codes[(codes & 0x7F) == 0x7F] = 0x38  # no NaN codes
     for name, data in (("zeros", torch.zeros(126 * 256, dtype=torch.int32)), ("random E4M3 codes", codes.view(torch.int32))):
         data = data.to(dev)
+        if slots > 1:
+            data = data.repeat(-(-slots * 65536 // (data.numel() * 4)))
         for groups in (cus, 1):
-            iters = 20000
+            iters = 20000 if slots == 1 else 2000
             b, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, ticks.data_ptr(), sink.data_ptr(), None) == 0
+            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, slots, ticks.data_ptr(), sink.data_ptr(), None) == 0
             b.record()
-            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, ticks.data_ptr(), sink.data_ptr(), None) == 0
+            assert lib.llmp_hip_gemm_probe_products(data.data_ptr(), iters, groups, slots, ticks.data_ptr(), sink.data_ptr(), None) == 0
             e.record(); torch.cuda.synchronize()
             ns = b.elapsed_time(e) * 1e6 / (48 * iters)
             t = int(ticks.item()) / (48 * iters)
