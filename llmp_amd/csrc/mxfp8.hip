@@ -326,21 +326,27 @@ __device__ __forceinline__ void AwaitLoads() {
 // D tile of 256 activation rows by 32 WN weight rows, K step 128, by WM x 2 waves: wave (wm, wn) owns 256 / WM
 // activation rows by 16 WN weight rows, the weights as the first operand of v_mfma_scale_f32_16x16x128_f8f6f4.
 //
-// Tiles come by global_load_lds into rings in LDS, activations 2 stages and weights 3 (every weight byte is a
-// compulsory HBM miss for the first workgroup that asks, activations mostly hit L2). In iteration s, after its
-// barrier: activations s + 2 are asked for (into the stage step s used: every wave read its fragments of it during
-// iteration s - 1), then weights s + 3; the fragments of step s + 1 are read while step s is multiplied, an
-// activation fragment's registers refilled as soon as its row of products is issued, a weight fragment's after its
-// last product; and at the end all loads but the weights just asked for have landed, so that after the next barrier
-// step s + 2 is whole in LDS. One barrier a step; no wave waits for another inside a step.
+// A workgroup a compute unit goes through its tiles one after the other (two each at M 2048, N 12288). Tiles come
+// by global_load_lds into rings in LDS, activations 2 stages and weights 3 (every weight byte is a compulsory HBM
+// miss for the first workgroup that asks, activations mostly hit L2). In iteration s, after its barrier: activations
+// s + 2 are asked for (into the stage step s used: every wave read its fragments of it during iteration s - 1), then
+// weights s + 3, a load after every third product (a CU's path to LDS takes 64 bytes a cycle; its four waves' loads
+// after every product would ask for 128); the fragments of step s + 1 are read while step s is multiplied, one read
+// after a product (GemmRegs); and at the end all loads but the weights just asked for have landed, so that after the
+// next barrier step s + 2 is whole in LDS. One barrier a step; no wave waits for another inside a step. A tile's
+// first products start its sums (no clearing), and the next tile's first stages are asked for ahead of this tile's
+// stores, which take about 4 us to be accepted (every CU stores its 98 KB at once; stores marked nontemporal made a
+// launch 107 us instead of 91).
 //
-// What a step costs, measured with parts of the loop taken out (M 2048, N 12288, K 4096; the shader clock is 1.9 GHz
-// under this kernel): its 48 products alone 0.87-0.95 us a wave that is alone on its SIMD (the pipe takes a product
-// every 32 cycles from one wave; with random codes in every CU the clock does not hold 2.4 GHz); and nothing else of
-// the same wave is issued meanwhile, so the 16 loads to LDS add 0.19 us (about 20 cycles each), the 42 reads of LDS
-// 0.10, the barrier and the waits 0.15: 1.26-1.35 us. Two waves a SIMD (eight waves a tile) do issue into each other's
-// products, but eight waves read 216 KB of LDS a step where four read 168, and LDS's 128 bytes a cycle then bound the
-// step at 1.29 us; with the smaller tile's poorer tail that is no faster, and four waves are the default.
+// What bounds a step (M 2048, N 12288, K 4096; the tuning build's probe and ablations): one wave a SIMD issues a
+// product every 32 cycles, and a vector move, a read of LDS or (every third product) a load to LDS between two
+// products costs 0.3 to 1.2 cycles: they are issued while the product runs. But the clock does not hold: 2.4 GHz on
+// zeros, 1.97 GHz with random codes in every CU's products, and 1.35-1.4 GHz when the operands also stream from L2
+// at this kernel's rate (64 KB a workgroup a step): 2.7-2.8 PFLOP/s is what the device's power allows with operands
+// arriving. The loop here runs at 1.04-1.12 us a step, 2.9-3.1 PFLOP/s while it multiplies, at 1.85-1.9 GHz with its
+// pipes 0.75 busy: cycles taken out of it (loads 140 a step, reads of LDS 95, barrier and waits 110 of 2070) come back
+// as a lower clock. Two waves a SIMD (eight waves a tile) read 216 KB of LDS a step where four read 168, and LDS's
+// 128 bytes a cycle then bound the step; four waves are the default.
 //
 // Reads of LDS are written as instructions (the compiler would make each wait for every load into LDS in flight): a
 // wave waits for them itself at the end of an iteration.
