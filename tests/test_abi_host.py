@@ -37,6 +37,15 @@ def test_library_exports_the_provider_and_launch_context():
         assert hasattr(lib, name), name
 
 
+def test_library_exports_the_memory_provider():
+    """include/llmp_hip_memory.h: bound from C++ (include/llmp_hip_memory.hpp), so exported names are what is checked."""
+    lib = _lib.load()
+    names = declared_symbols("llmp_hip_memory.h")
+    assert len(names) >= 21
+    for name in names:
+        assert hasattr(lib, name), name
+
+
 def test_variant_table_is_named():
     lib = _lib.load()
     n = lib.llmp_hip_vecq_variants()
