@@ -584,34 +584,44 @@ def main():
     # them too, src/kernels/ggml/launch.h:34-48): one graph of W steps, one of K steps.
     side = torch.cuda.Stream()
 
-    def timed_region(body, count, first):
-        """Milliseconds of `count` calls of body(i), by HIP events on the launching stream."""
-        graph = None
-        if not args.eager:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(count):
-                    body(first + i)
-        torch.cuda.synchronize()
-        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        begin.record()
-        if graph is None:
+    def capture(body, count, first):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
             for i in range(count):
                 body(first + i)
+        return graph
+
+    def timed_region(body):
+        """Milliseconds of the K timed calls of body(i), by HIP events on the launching stream, right behind its W
+        warm-up calls: both graphs are captured first (capturing is host work of milliseconds with the device idle,
+        and the W warm-up steps are to run just ahead of the timed ones, not ahead of that gap)."""
+        warm = timed = None
+        if not args.eager:
+            warm = capture(body, args.warmup, 0) if args.warmup > 0 else None
+            timed = capture(body, args.steps, args.warmup)
+        torch.cuda.synchronize()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if args.eager:
+            for i in range(args.warmup):
+                body(i)
+        elif warm is not None:
+            warm.replay()
+        t0 = time.perf_counter()
+        begin.record()
+        if args.eager:
+            for i in range(args.steps):
+                body(args.warmup + i)
         else:
-            graph.replay()
+            timed.replay()
         end.record()
         torch.cuda.synchronize()
         return begin.elapsed_time(end), (time.perf_counter() - t0) * 1e3
 
     step(0)
     torch.cuda.synchronize()
-    timed_region(step, args.warmup, 0)
-    total_ms, wall_ms = timed_region(step, args.steps, args.warmup)
+    total_ms, wall_ms = timed_region(step)
     # The dominant kernel alone (the mat-vec over ready Q8_1 blocks), the same rotation.
-    timed_region(kernel_only if not args.fused else step, args.warmup, 0)
-    kernel_ms, _ = timed_region(kernel_only if not args.fused else step, args.steps, args.warmup)
+    kernel_ms, _ = timed_region(kernel_only if not args.fused else step)
     kernel_us = kernel_ms / args.steps * 1e3
     ms = total_ms / args.steps
     value = WEIGHT_BYTES / (ms * 1e-3) / 1e9
