@@ -135,6 +135,25 @@ def test_gemm_workgroups_that_take_several_tiles(device, m, n, k, bf16):
         assert torch.equal(few.view(torch.int16 if bf16 else torch.int32), each.view(torch.int16 if bf16 else torch.int32)), cus
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm_nan_codes_and_scales_stay_in_their_rows_and_columns(device, bf16):
+    """E4M3's NaN code (0x7F) in an activation row, and an undefined scale (0xFF) on a weight row: every output of
+    that row (that column) is a NaN, in F32 and after the bf16 packing, and every other output keeps its bits."""
+    m, n, k = 130, 200, 256
+    a, w, (ac, asc), (wc, wsc) = quantized_operands(m, n, k, 77)
+    clean = ops.mxfp8_gemm(dev(ac, device), dev(asc, device), dev(wc, device), dev(wsc, device), bf16=bf16).float().cpu().numpy()
+    ac2 = ac.copy()
+    ac2[5, 131] = 0x7F
+    wsc2 = wsc.copy()
+    wsc2[oracle.lib.orc_scale_atom_offset(9, 3, k // 32)] = 0xFF
+    got = ops.mxfp8_gemm(dev(ac2, device), dev(asc, device), dev(wc, device), dev(wsc2, device), bf16=bf16).float().cpu().numpy()
+    bad = np.zeros((m, n), dtype=bool)
+    bad[5, :] = True
+    bad[:, 9] = True
+    assert np.all(np.isnan(got[bad]))
+    assert np.array_equal(got[~bad].view(np.uint32), clean[~bad].view(np.uint32))
+
+
 def test_gemm_full_size_sampled(device):
     """The headline prefill shape, M 2048, K 4096, N 12288: sampled entries against the oracle's dot, and
     linearity in the activations' scales (doubling a row's scales doubles its outputs exactly)."""
