@@ -198,6 +198,8 @@ typedef struct llmp_mxfp8_gemm {
 } llmp_mxfp8_gemm;
 int llmp_hip_mxfp8_gemm_available(void);
 size_t llmp_hip_mxfp8_gemm_scratch(const llmp_mxfp8_gemm* gemm, int compute_units);
+/* `compute_units` (the reference's `sms`; 0 or less: 256): the launch has at most that many workgroups, each going
+ * through its share of the tiles one after the other. The sums do not depend on it. */
 int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void* stream);
 
 /* ------------------------------------------------------------------ llmp.moe.gemm
