@@ -761,6 +761,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     AwaitLoads<0>();
     barrier();
     GEMM_TRACE(2 + 8 * min(ord, 1));
+    if (ord > 0) GEMM_TRACE_CYCLES(9);  // (the first tile's counter is read when its loads have been asked for)
     aim_reads(0, 0);
     StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
     StaticFor<WN>([&](auto i) { read_b(i, Even{}); });

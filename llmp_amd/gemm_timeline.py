@@ -79,4 +79,6 @@ for label, base in (("first tile", 0), ("last tile", 8)):
     print(f"  step1->step16 {np.median(per[:,4]-per[:,3])/100:.2f} (15 steps)  step16->last {np.median(per[:,5]-per[:,4])/100:.2f} (16 steps)  last step->stores queued {np.median(per[:,7]-per[:,5])/100:.2f}")
 cyc = tr[:, 6] - tr[:, 1]; us = (tr[:, 5] - tr[:, 2]) / 100
 print("first tile: shader cycles between slot 1 and 6: median %.0f; us between 2 and 5: %.2f -> clock about %.2f GHz" % (np.median(cyc), np.median(us), np.median(cyc) / np.median(us) / 1e3))
+cyc = tr[:, 14] - tr[:, 9]; us = (tr[:, 13] - tr[:, 10]) / 100
+print("last tile: shader cycles between its first stages landed and its last step: median %.0f in %.2f us -> clock about %.2f GHz" % (np.median(cyc), np.median(us), np.median(cyc) / np.median(us) / 1e3))
 print("launch by stamps: %.1f us" % ((tr[:, 15].max() - t0) / 100))
