@@ -4,8 +4,8 @@
  * its paging engine (src/providers/device_memory.h:118-157) and its CUDA build implements them over
  * the driver's VMM calls (src/providers/cuda/cuda_device_memory.cc:42-215). Here the primitives are
  * hipMemAddressReserve / hipMemAddressFree, hipMemCreate / hipMemRelease, hipMemMap / hipMemUnmap and
- * hipMemSetAccess; the rules over them are the reference's VmmProvider's, the same for every
- * implementation (device_memory.h:30-45):
+ * hipMemSetAccess; the contract over them is the one the reference states for every implementation
+ * (device_memory.h:30-45), kept by the books of llmp_amd/csrc/vmm_ledger.h:
  *   - a reservation is address space only, a non-zero multiple of the granularity;
  *   - backing is created in one allocation class, a multiple of the granularity, filled with nothing
  *     a caller may rely on;
@@ -15,8 +15,8 @@
  *   - backing is released only when unmapped, a reservation freed only when nothing is mapped in it.
  * Nothing here pages on demand: touching address space whose backing is absent is a bug.
  *
- * Identities are 64-bit, generation-checked and never reused: a stale one names nothing. 0 is no
- * identity.
+ * Identities are 64-bit numbers from one counter, never handed out twice: a stale one names nothing,
+ * and a reservation's never names a backing. 0 is no identity.
  *
  * Return values, as in llmp_hip_launch.h: 0 done; > 0 refused or failed with nothing changed, one
  * of LLMP_PROVIDER_* (the reference's ProviderError, device_memory.h:84-95); < 0 a primitive's

@@ -24,7 +24,7 @@ struct AllocationClass {
   std::uint64_t granularity = 0;
 };
 enum class Access : std::uint8_t { kNone, kRead, kReadWrite };
-using ReservationId = std::uint64_t;  // generation-checked, never reused; 0 is none
+using ReservationId = std::uint64_t;  // never handed out twice; 0 is none
 using BackingId = std::uint64_t;
 struct AddressRange {
   std::uint64_t base = 0;

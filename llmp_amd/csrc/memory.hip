@@ -1,6 +1,6 @@
-// The HIP device-memory provider behind include/llmp_hip_memory.h: the primitives of the reference's
-// CudaDeviceMemory (src/providers/cuda/cuda_device_memory.cc:42-144) on HIP's virtual memory management calls,
-// under the shared rules of vmm_rules.h. Host code only.
+// The HIP device-memory provider behind include/llmp_hip_memory.h: what the reference's CudaDeviceMemory does with the
+// CUDA driver (src/providers/cuda/cuda_device_memory.cc:42-144) done with HIP's virtual memory management calls, as the
+// Backend of the books kept in vmm_ledger.h. Host code only.
 #include <hip/hip_runtime.h>
 
 #include <memory>
@@ -11,13 +11,13 @@
 #include "common.h"
 #include "llmp_hip.h"
 #include "llmp_hip_memory.h"
-#include "vmm_rules.h"
+#include "vmm_ledger.h"
 
 using llmp_hip::vmm::Access;
 using llmp_hip::vmm::AllocationClass;
 using llmp_hip::vmm::Error;
 using llmp_hip::vmm::Kind;
-using llmp_hip::vmm::Rules;
+using llmp_hip::vmm::Ledger;
 using llmp_hip::vmm::Status;
 
 namespace llmp_hip {
@@ -65,37 +65,36 @@ hipMemAllocationProp Properties(const AllocationClass& allocation_class) {
   return prop;
 }
 
-class HipDeviceMemory final : public Rules {
+class HipBackend final : public vmm::Backend {
  public:
-  HipDeviceMemory(int device, std::vector<AllocationClass> classes, std::uint64_t granularity)
-      : Rules(std::move(classes), granularity), device_(device) {}
+  HipBackend(int device, std::vector<AllocationClass> classes, std::uint64_t granularity)
+      : device_(device), classes_(std::move(classes)), granularity_(granularity) {}
 
- protected:
-  Status DoReserve(std::uint64_t size, std::uint64_t* base) override {
+  Status ReserveSpace(std::uint64_t size, std::uint64_t* base) override {
     if (Status current = Current(); !current) return current;
     void* at = nullptr;
-    if (Status reserved = Outcome(hipMemAddressReserve(&at, size, Granularity(), nullptr, 0), "hipMemAddressReserve"); !reserved) return reserved;
+    if (Status reserved = Outcome(hipMemAddressReserve(&at, size, granularity_, nullptr, 0), "hipMemAddressReserve"); !reserved) return reserved;
     *base = reinterpret_cast<std::uint64_t>(at);
     return vmm::Ok();
   }
-  Status DoFree(std::uint64_t base, std::uint64_t size) override {
+  Status FreeSpace(std::uint64_t base, std::uint64_t size) override {
     return Outcome(hipMemAddressFree(reinterpret_cast<void*>(base), size), "hipMemAddressFree");
   }
-  Status DoCreate(const AllocationClass& allocation_class, std::uint64_t size, Handle* handle) override {
+  Status CreateBlock(const AllocationClass& allocation_class, std::uint64_t size, std::uint64_t* handle) override {
     if (Status current = Current(); !current) return current;
     const hipMemAllocationProp prop = Properties(allocation_class);
     hipMemGenericAllocationHandle_t made = nullptr;
     if (Status created = Outcome(hipMemCreate(&made, size, &prop, 0), "hipMemCreate"); !created) return created;
-    *handle = reinterpret_cast<Handle>(made);
+    *handle = reinterpret_cast<std::uint64_t>(made);
     return vmm::Ok();
   }
-  Status DoRelease(Handle handle, std::uint64_t) override {
+  Status ReleaseBlock(std::uint64_t handle) override {
     return Outcome(hipMemRelease(reinterpret_cast<hipMemGenericAllocationHandle_t>(handle)), "hipMemRelease");
   }
-  Status DoMap(std::uint64_t address, std::uint64_t size, Handle handle) override {
+  Status Attach(std::uint64_t address, std::uint64_t size, std::uint64_t handle) override {
     return Outcome(hipMemMap(reinterpret_cast<void*>(address), size, 0, reinterpret_cast<hipMemGenericAllocationHandle_t>(handle), 0), "hipMemMap");
   }
-  Status DoSetAccess(std::uint64_t address, std::uint64_t size, Access access, bool host) override {
+  Status Protect(std::uint64_t address, std::uint64_t size, Access access, bool host) override {
     hipMemAccessFlags flags = hipMemAccessFlagsProtNone;
     if (access == Access::kRead) {
       flags = hipMemAccessFlagsProtRead;
@@ -104,7 +103,7 @@ class HipDeviceMemory final : public Rules {
     }
     // The device always; the CPU on the host node when the range holds host backing (cuda_device_memory.cc:112-123).
     std::vector<hipMemAccessDesc> descriptors;
-    for (const AllocationClass& allocation_class : Classes()) {
+    for (const AllocationClass& allocation_class : classes_) {
       if (allocation_class.kind == Kind::kDevice || host) {
         hipMemAccessDesc descriptor = {};
         descriptor.location = Properties(allocation_class).location;
@@ -114,13 +113,15 @@ class HipDeviceMemory final : public Rules {
     }
     return Outcome(hipMemSetAccess(reinterpret_cast<void*>(address), size, descriptors.data(), descriptors.size()), "hipMemSetAccess");
   }
-  Status DoUnmap(std::uint64_t address, std::uint64_t size) override {
+  Status Detach(std::uint64_t address, std::uint64_t size) override {
     return Outcome(hipMemUnmap(reinterpret_cast<void*>(address), size), "hipMemUnmap");
   }
 
  private:
   Status Current() { return Outcome(hipSetDevice(device_), "hipSetDevice"); }
   int device_;
+  std::vector<AllocationClass> classes_;
+  std::uint64_t granularity_;
 };
 
 // The C ABI's return value for a status, its reason recorded for llmp_hip_last_error.
@@ -148,7 +149,11 @@ int Code(const Status& status) {
 }  // namespace llmp_hip
 
 struct llmp_hip_memory {
-  std::unique_ptr<llmp_hip::HipDeviceMemory> provider;
+  llmp_hip_memory(int device, const std::vector<AllocationClass>& classes, std::uint64_t granularity)
+      : backend(device, classes, granularity), books(&backend, classes, granularity), provider(&books) {}
+  llmp_hip::HipBackend backend;
+  Ledger books;
+  Ledger* provider;
 };
 
 using llmp_hip::Code;
@@ -157,13 +162,17 @@ using llmp_hip::Refuse;
 extern "C" int llmp_hip_memory_open(int device, llmp_hip_memory** out) {
   if (out == nullptr) return Refuse(LLMP_PROVIDER_INVALID, "memory: null result");
   *out = nullptr;
+#if defined(LLMP_HIP_MEMORY_ON_DEVICE) && !defined(LLMP_HIP_MEMORY_FAULT_CAUSE_SHOWN)
+#error "LLMP_HIP_MEMORY_ON_DEVICE switches on calls whose one run on an MI355X ended with the GPU faulted; define LLMP_HIP_MEMORY_FAULT_CAUSE_SHOWN as well only once that fault's cause has been shown and fixed"
+#endif
 #ifndef LLMP_HIP_MEMORY_ON_DEVICE
-  // Switched off: the one run of these primitives on an MI355X (two mappings in a reservation, access granted, host
+  // Switched off: the one run of these calls on an MI355X (two mappings in a reservation, access granted, host
   // copies through them) ended with the GPU faulted, before any kernel of this library ran, and the cause has not
-  // been shown. Until it is, no provider is opened and no virtual memory call is made; the rules of vmm_rules.h are
-  // tested on the CPU (tests/host/memory_test.cc, rules).
+  // been shown. Until it is, no provider is opened and no virtual memory call is made; the books of vmm_ledger.h are
+  // tested on the CPU (tests/host/memory_test.cc, rules). A consumer that pages meanwhile allocates with hipMalloc and
+  // copies, with no remapping.
   (void)device;
-  return Refuse(LLMP_PROVIDER_UNSUPPORTED, "memory: the HIP virtual memory primitives are switched off in this build (-DLLMP_HIP_MEMORY_ON_DEVICE)");
+  return Refuse(LLMP_PROVIDER_UNSUPPORTED, "memory: the HIP virtual memory calls are switched off in this build");
 #else
   int devices = 0;
   if (const hipError_t e = hipGetDeviceCount(&devices); e != hipSuccess || device < 0 || device >= devices) {
@@ -188,7 +197,7 @@ extern "C" int llmp_hip_memory_open(int device, llmp_hip_memory** out) {
     allocation_class.granularity = granularity;
     common = std::lcm(common, static_cast<std::uint64_t>(granularity));
   }
-  *out = new llmp_hip_memory{std::make_unique<llmp_hip::HipDeviceMemory>(device, std::move(classes), common)};
+  *out = new llmp_hip_memory(device, classes, common);
   return 0;
 #endif
 }

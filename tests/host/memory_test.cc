@@ -1,7 +1,7 @@
 // The device-memory provider (include/llmp_hip_memory.h, .hpp), as the reference's tests drive its
 // (tests/unit/device_memory_test.cc of the reference is the model: the shared rules over a provider whose primitives
 // can be told to fail, then the real device).
-//   memory_test rules    the rules of llmp_amd/csrc/vmm_rules.h on the CPU, over primitives that count, fail and lose
+//   memory_test rules    the books of llmp_amd/csrc/vmm_ledger.h on the CPU, over a backend that counts, fails and loses
 //                        outcomes on request (no GPU, no HIP call)
 //   memory_test host     what the C ABI refuses without a device
 //   memory_test device   reservations, backing, mappings and access on the GPU: bytes written through one mapping read
@@ -14,7 +14,7 @@
 #include <string>
 #include <vector>
 
-#include "../../llmp_amd/csrc/vmm_rules.h"
+#include "../../llmp_amd/csrc/vmm_ledger.h"
 #include "llmp_hip_memory.hpp"
 
 namespace {
@@ -34,20 +34,73 @@ using llmp_hip::vmm::Error;
 using llmp_hip::vmm::Kind;
 using llmp_hip::vmm::Status;
 
-// Primitives that keep books: address space handed out upwards from 1 << 40, handles counted up, every live range,
-// handle and mapping remembered, so that a rule that let a wrong call through shows. `fail_next` makes the next
-// primitive fail with that error once.
-class Counting final : public llmp_hip::vmm::Rules {
+// A backend that keeps books of its own: address space handed out upwards from 1 << 40, handles counted up, every live
+// range, handle and mapping remembered, so that a rule that let a wrong call through shows. `fail_next` makes the next
+// call fail with that error once. The ledger under test sits on top of it and is reached through `->`.
+class Counting final : public llmp_hip::vmm::Backend {
  public:
   static constexpr std::uint64_t kGranule = 1 << 16;
-  Counting()
-      : Rules({AllocationClass{Kind::kDevice, 0, kGranule / 2}, AllocationClass{Kind::kHost, 1, kGranule}}, kGranule) {}
+  Counting() : ledger_(this, {AllocationClass{Kind::kDevice, 0, kGranule / 2}, AllocationClass{Kind::kHost, 1, kGranule}}, kGranule) {}
   Error fail_next = Error::kOk;
   std::set<std::uint64_t> ranges, handles;
-  std::vector<std::string> calls;  // what reached the primitives
+  std::vector<std::string> calls;  // what reached the backend
   std::set<std::uint64_t> mapped;  // addresses of live mappings
 
- protected:
+  // The ledger's operations under the names the checks below use.
+  Status Reserve(std::uint64_t size, std::uint64_t* id) { return ledger_.Reserve(size, id); }
+  Status RangeOf(std::uint64_t id, std::uint64_t* base, std::uint64_t* size) const { return ledger_.RangeOf(id, base, size); }
+  Status Free(std::uint64_t id) { return ledger_.Free(id); }
+  Status Create(std::size_t c, std::uint64_t size, std::uint64_t* id) { return ledger_.Create(c, size, id); }
+  Status Release(std::uint64_t id) { return ledger_.Release(id); }
+  Status Map(std::uint64_t r, std::uint64_t offset, std::uint64_t b) { return ledger_.Map(r, offset, b); }
+  Status SetAccess(std::uint64_t r, std::uint64_t offset, std::uint64_t size, Access a) { return ledger_.SetAccess(r, offset, size, a); }
+  Status Unmap(std::uint64_t r, std::uint64_t offset, std::uint64_t size) { return ledger_.Unmap(r, offset, size); }
+  std::uint64_t MappedAt(std::uint64_t r, std::uint64_t offset) const { return ledger_.MappedAt(r, offset); }
+  bool UndeterminedReservation(std::uint64_t id) const { return ledger_.UndeterminedReservation(id); }
+  bool UndeterminedBacking(std::uint64_t id) const { return ledger_.UndeterminedBacking(id); }
+  std::uint64_t UndeterminedBytes() const { return ledger_.UndeterminedBytes(); }
+  std::size_t reservations() const { return ledger_.reservations(); }
+  std::size_t backings() const { return ledger_.backings(); }
+  std::uint64_t created_backings() const { return ledger_.created_backings(); }
+  std::uint64_t released_backings() const { return ledger_.released_backings(); }
+
+  Status ReserveSpace(std::uint64_t size, std::uint64_t* base) override {
+    if (Status s = Take("reserve"); !s) return s;
+    *base = next_;
+    next_ += size + kGranule;
+    ranges.insert(*base);
+    return llmp_hip::vmm::Ok();
+  }
+  Status FreeSpace(std::uint64_t base, std::uint64_t) override {
+    if (Status s = Take("free"); !s) return s;
+    CHECK(ranges.erase(base) == 1);
+    return llmp_hip::vmm::Ok();
+  }
+  Status CreateBlock(const AllocationClass&, std::uint64_t, std::uint64_t* handle) override {
+    if (Status s = Take("create"); !s) return s;
+    *handle = ++last_handle_;
+    handles.insert(*handle);
+    return llmp_hip::vmm::Ok();
+  }
+  Status ReleaseBlock(std::uint64_t handle) override {
+    if (Status s = Take("release"); !s) return s;
+    CHECK(handles.erase(handle) == 1);
+    return llmp_hip::vmm::Ok();
+  }
+  Status Attach(std::uint64_t address, std::uint64_t, std::uint64_t handle) override {
+    if (Status s = Take("map"); !s) return s;
+    CHECK(handles.count(handle) == 1);
+    CHECK(mapped.insert(address).second);
+    return llmp_hip::vmm::Ok();
+  }
+  Status Protect(std::uint64_t, std::uint64_t, Access, bool host) override { return Take(host ? "access host" : "access device"); }
+  Status Detach(std::uint64_t address, std::uint64_t size) override {
+    if (Status s = Take("unmap"); !s) return s;
+    for (auto at = mapped.lower_bound(address); at != mapped.end() && *at < address + size;) at = mapped.erase(at);
+    return llmp_hip::vmm::Ok();
+  }
+
+ private:
   Status Take(const char* what) {
     calls.push_back(what);
     if (fail_next == Error::kOk) return llmp_hip::vmm::Ok();
@@ -55,45 +108,9 @@ class Counting final : public llmp_hip::vmm::Rules {
     fail_next = Error::kOk;
     return Status{e, std::string(what) + " was told to fail", e == Error::kUnknown ? 999 : 0};
   }
-  Status DoReserve(std::uint64_t size, std::uint64_t* base) override {
-    if (Status s = Take("reserve"); !s) return s;
-    *base = next_;
-    next_ += size + kGranule;
-    ranges.insert(*base);
-    return llmp_hip::vmm::Ok();
-  }
-  Status DoFree(std::uint64_t base, std::uint64_t) override {
-    if (Status s = Take("free"); !s) return s;
-    CHECK(ranges.erase(base) == 1);
-    return llmp_hip::vmm::Ok();
-  }
-  Status DoCreate(const AllocationClass&, std::uint64_t, Handle* handle) override {
-    if (Status s = Take("create"); !s) return s;
-    *handle = ++last_handle_;
-    handles.insert(*handle);
-    return llmp_hip::vmm::Ok();
-  }
-  Status DoRelease(Handle handle, std::uint64_t) override {
-    if (Status s = Take("release"); !s) return s;
-    CHECK(handles.erase(handle) == 1);
-    return llmp_hip::vmm::Ok();
-  }
-  Status DoMap(std::uint64_t address, std::uint64_t, Handle handle) override {
-    if (Status s = Take("map"); !s) return s;
-    CHECK(handles.count(handle) == 1);
-    CHECK(mapped.insert(address).second);
-    return llmp_hip::vmm::Ok();
-  }
-  Status DoSetAccess(std::uint64_t, std::uint64_t, Access, bool host) override { return Take(host ? "access host" : "access device"); }
-  Status DoUnmap(std::uint64_t address, std::uint64_t size) override {
-    if (Status s = Take("unmap"); !s) return s;
-    for (auto at = mapped.lower_bound(address); at != mapped.end() && *at < address + size;) at = mapped.erase(at);
-    return llmp_hip::vmm::Ok();
-  }
-
- private:
   std::uint64_t next_ = std::uint64_t{1} << 40;
-  Handle last_handle_ = 0;
+  std::uint64_t last_handle_ = 0;
+  llmp_hip::vmm::Ledger ledger_;
 };
 
 void RulesChecks() {
@@ -165,7 +182,7 @@ void RulesChecks() {
   CHECK(m.Release(b3).error == Error::kUnknown && m.Release(b3).error == Error::kUndetermined);
   m.fail_next = Error::kUnknown;
   CHECK(m.Free(r2).error == Error::kUnknown && m.Free(r2).error == Error::kUndetermined);
-  // Identities are never reused: a new reservation in a freed slot has another name.
+  // Identities are never reused: a reservation made after one was freed has another name.
   std::uint64_t r3 = 0, r4 = 0;
   CHECK(m.Reserve(G, &r3) && m.Free(r3) && m.Reserve(G, &r4) && r4 != r3 && m.RangeOf(r3, &base, &size).error == Error::kInvalid);
   CHECK(m.Free(r4));
