@@ -95,7 +95,7 @@ def graph_us(body, count, warm=3):
 SETTLE_REPLAYS = 20
 
 
-MFMA_FP8_PEAK_TFLOPS = 5033.0  # dense FP8, 256 CUs x 2.4 GHz x 8192 flop/clk/CU
+MFMA_FP8_PEAK_TFLOPS = 5000.0  # dense FP8 (and int8), the published figure
 
 # HBM bytes per launch of each configuration's roofline kernel(s), from rocprofv3 --pmc runs of this file
 # (`--only <name> --no-cpu --eager --calibrate-copy`: FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what
@@ -349,7 +349,7 @@ def other_configs(device, args, only=None):
             if tokens == 512:
                 flops = tokens * used * 3 * 2.0 * hidden * ffn
                 entry["layer_TFLOP/s"] = round(flops / us / 1e6, 2)
-                entry["layer_frac_int8_mfma_peak"] = round(flops / us / 1e6 / 5033.0, 4)
+                entry["layer_frac_int8_mfma_peak"] = round(flops / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 4)
             if cpu:
                 def cpu_layer():
                     ids_c, w_c = oracle.route(logits_host, used)
@@ -366,6 +366,40 @@ def other_configs(device, args, only=None):
                 entry["cpu_baseline"] = cpu_leg(cpu_layer, layer_bytes / 1e9, "GB/s", 2.0, f"the whole layer at {tokens} token(s)", threads)
             out[name] = entry
         del gus, dns, gate_up, down
+        torch.cuda.empty_cache()
+
+    # llmp.moe.gemm (the reference's NVFP4 grouped expert product) on config 4's shape: 512 tokens' 4096 rows sorted by
+    # expert over 128 experts, each expert's 768 x 2048 (gate or up) and 2048 x 768 (down) weights. Not a BASELINE
+    # config: timed so that its cost is known.
+    if want("moe_gemm_nvfp4_128_experts_t512"):
+        experts, used, tokens = 128, 8, 512
+        g = synth.rng(230)
+        logits_host = g.standard_normal((tokens, experts), dtype=np.float32)
+        _, ids, _ = (None, ops.moe_router(dev(logits_host), used)[0], None)
+        counts = torch.bincount(ids.view(-1).to(torch.int64), minlength=experts).cpu().numpy()
+        offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        sf_rows = np.concatenate([[0], np.cumsum((counts + 127) // 128 * 128)]).astype(np.int32)
+        rows = int(offsets[-1])
+        entry = {"workload": "llmp.moe.gemm: NVFP4 (E2M1 codes, UE4M3 scales a 16) rows sorted by expert, 128 experts, "
+                             f"{rows} rows, bf16 out; not a BASELINE config", "shapes": {}}
+        for n, k in ((768, 2048), (2048, 768)):
+            a_codes = dev(g.integers(0, 256, size=(rows, k // 2), dtype=np.uint8))
+            a_scales = dev(g.integers(0x20, 0x50, size=int(sf_rows[-1]) * (k // 16), dtype=np.uint8))
+            codes_bytes, scales_bytes = n * (k // 2), (n + 127) // 128 * 128 * (k // 16)
+            scales_offset = (codes_bytes + 255) // 256 * 256
+            expert_stride = (scales_offset + scales_bytes + 255) // 256 * 256
+            weights = g.integers(0, 256, size=(experts, expert_stride), dtype=np.uint8)
+            weights[:, scales_offset:] = g.integers(0x20, 0x50, size=(experts, expert_stride - scales_offset), dtype=np.uint8)
+            wd = dev(weights)
+            wds = [wd] + [wd.clone() for _ in range(3)]
+            d = torch.empty((rows, n), dtype=torch.bfloat16, device=device)
+            od, sd = dev(offsets), dev(sf_rows)
+            us = timed(lambda i: ops.moe_gemm(a_codes, a_scales, od, sd, wds[i % 4], expert_stride, 0, scales_offset, n, k, out=d), 8)
+            flops = 2.0 * rows * n * k
+            entry["shapes"][f"n{n}_k{k}"] = {"us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1),
+                                             "frac_bf16_mfma_peak": round(flops / us / 1e6 / 2500.0, 4),
+                                             "weight_GB/s": round(experts * (codes_bytes + scales_bytes) / us / 1e3, 1)}
+        out["moe_gemm_nvfp4_128_experts_t512"] = entry
         torch.cuda.empty_cache()
 
     # Config 5: EXL3 linear 4096 x 14336 at 4 bits, 3INST codebook.

@@ -353,6 +353,13 @@ int llmp_hip_exl3_linear(const llmp_exl3_linear* op, void* scratch, size_t scrat
  * it later reads. Output bits are those of llmp_hip_exl3_linear. */
 #define LLMP_EXL3_STATIC_SCRATCH_BYTES ((size_t)4 << 20) /* config 5 at 16 rows needs 3,670,016 */
 int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* stream);
+/* What the first llmp_hip_exl3_linear_static call on a device and for a (codebook, bits) does besides launching:
+ * taking the static array's address and asking the runtime once for the product kernels' dynamic LDS. Neither is
+ * a launch, so a stream capture may refuse or be invalidated by them: a caller that captures calls this first,
+ * outside any capture, with the device current (only op->weights is read; no stream, nothing is queued), or makes
+ * its first call of each such linear eagerly. Like its sibling it has no counterpart in the reference. Returns
+ * as the launchers do. */
+int llmp_hip_exl3_linear_static_prepare(const llmp_exl3_linear* op);
 
 /* exl3.multi_linear.mgemm: MultiLinear of src/kernels/exl3/linear.h:51-53 over the operands of
  * src/kernels/exl3/validate.h:160-172, a gate and an up linear of the same k, n and rate over

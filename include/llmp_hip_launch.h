@@ -18,7 +18,9 @@
  *
  * Threads, as in the reference (device_execution.h:17-24, launch.h:28-32): the provider's calls
  * are safe for distinct streams and fences from any threads, and llmp_hip_execution_query may run
- * beside any other call; a launch context is used by one thread at a time.
+ * beside any other call; one thread drives a stream at a time (queueing on it, recording its fences,
+ * destroying it: a record that ran beside another thread's submission on the same stream could mark
+ * that work as fenced); a launch context is used by one thread at a time.
  */
 #ifndef LLMP_HIP_LAUNCH_H_
 #define LLMP_HIP_LAUNCH_H_

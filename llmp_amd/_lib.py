@@ -135,6 +135,7 @@ SYMBOLS = {
     "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),
     "llmp_hip_exl3_linear": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _vp]),
     "llmp_hip_exl3_linear_static": (_int, [C.POINTER(Exl3Linear), _vp]),
+    "llmp_hip_exl3_linear_static_prepare": (_int, [C.POINTER(Exl3Linear)]),
     "llmp_hip_decode_vector": (_int, [_int, C.POINTER(DecodeOperand), C.c_uint64, C.c_uint64, _vp, C.c_uint64,
                                       C.c_uint64, _vp, C.c_uint64, _vp]),
     "llmp_hip_decode_vector_glu": (_int, [_int, C.POINTER(DecodeOperand), C.c_uint64, _int, C.POINTER(DecodeOperand),

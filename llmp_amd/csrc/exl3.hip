@@ -636,14 +636,26 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
                      static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
 
+template <int BITS>
+constexpr int ProductLds() {
+  constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
+  constexpr int kWork = kProductWaves * (kRingDepth * kLoads * 1024 + kOperandBytes);
+  return kWork > kReduceBytes ? kWork : kReduceBytes;
+}
+// More than 64 KB of dynamic LDS must be asked for once a kernel instance: a runtime call that is no launch, so a
+// caller that captures makes it beforehand (llmp_hip_exl3_linear_static_prepare).
+template <int CB, int BITS, bool kFused>
+bool g_product_sized = false;
+template <int CB, int BITS, bool kFused>
+bool SizeProduct() {
+  return AllowLds(reinterpret_cast<const void*>(&ProductKernel<CB, BITS, kFused>), ProductLds<BITS>(), &g_product_sized<CB, BITS, kFused>);
+}
+
 template <int CB, int BITS, bool kFused>
 void LaunchProduct(const llmp_exl3_weights& w, const ProductSides& sides, int count, int m, int slices,
                    hipStream_t stream) {
-  constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
-  constexpr int kWork = kProductWaves * (kRingDepth * kLoads * 1024 + kOperandBytes);
-  constexpr int kLds = kWork > kReduceBytes ? kWork : kReduceBytes;
-  static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&ProductKernel<CB, BITS, kFused>), kLds, &sized)) return;
+  constexpr int kLds = ProductLds<BITS>();
+  if (!SizeProduct<CB, BITS, kFused>()) return;
   const int blocks = w.k / 128;
   const int per = (blocks + slices * kProductWaves - 1) / (slices * kProductWaves);
   const dim3 grid(static_cast<unsigned>(w.n / 128), static_cast<unsigned>(slices), static_cast<unsigned>(count));
@@ -896,6 +908,19 @@ extern "C" int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* str
   void* area = nullptr;
   if (const int bad = StaticArea(&area); bad != 0) return bad;
   return LinearOver(op, area, kStaticScratchBytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int llmp_hip_exl3_linear_static_prepare(const llmp_exl3_linear* op) {
+  BeginLaunches();
+  if (op == nullptr) return Refuse(1, "exl3.linear_static_prepare: null operands");
+  if (const int bad = llmp_hip::CheckWeights(op->weights); bad != 0) return bad;
+  void* area = nullptr;
+  if (const int bad = StaticArea(&area); bad != 0) return bad;
+  llmp_hip::Dispatch(op->weights.codebook, op->weights.bits, [&](auto cb, auto bits) {
+    (void)llmp_hip::SizeProduct<decltype(cb)::value, decltype(bits)::value, true>();
+    (void)llmp_hip::SizeProduct<decltype(cb)::value, decltype(bits)::value, false>();
+  });
+  return LaunchStatus("exl3.linear_static_prepare");
 }
 
 extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op) {

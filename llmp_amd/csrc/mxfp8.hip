@@ -257,49 +257,6 @@ struct GemmArgs {
   int tiles_m, tiles_n;
 };
 
-// Timeline instrumentation for tuning, compiled only with -DLLMP_GEMM_TRACE (never into the library): lane 0 of
-// every wave stores the 100 MHz clock at up to eight points of its first tile and of its later ones (the last of
-// them stays), sixteen 64-bit words a wave.
-#ifdef LLMP_GEMM_TRACE
-__device__ unsigned long long* g_gemm_trace = nullptr;
-// The wave's sixteen slots, asked for once at the kernel's start (read at every stamp, the pointer's two loads and
-// their waits would be part of every step that is timed).
-#define GEMM_TRACE_BEGIN                                                                                     \
-  unsigned long long* gemm_trace_slots = g_gemm_trace;                                                       \
-  if (gemm_trace_slots != nullptr)                                                                           \
-    gemm_trace_slots += (static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 16
-#define GEMM_TRACE(slot)                                                                     \
-  do {                                                                                       \
-    if (gemm_trace_slots != nullptr && (threadIdx.x & 63) == 0) gemm_trace_slots[slot] = wall_clock64(); \
-  } while (0)
-// ... or the shader clock's counter (slots 1 and 6: the kernel's cycles between them give its clock).
-#define GEMM_TRACE_CYCLES(slot)                                                                               \
-  do {                                                                                                        \
-    if (gemm_trace_slots != nullptr && (threadIdx.x & 63) == 0) gemm_trace_slots[slot] = __builtin_readcyclecounter(); \
-  } while (0)
-#else
-#define GEMM_TRACE_BEGIN \
-  do {                   \
-  } while (0)
-#define GEMM_TRACE(slot) \
-  do {                   \
-  } while (0)
-#define GEMM_TRACE_CYCLES(slot) \
-  do {                          \
-  } while (0)
-#endif
-
-// For the tuning build only (make trace EXTRA=-DLLMP_GEMM_WITHOUT=<bits>): parts of GemmKernel's loop left out, to time
-// what each costs. Results are wrong; nothing faults (what is left out is never a wait that guards an address).
-//   1 the loads to LDS after the prologue   2 the reads of fragments and scales from LDS   4 the step's barrier
-//   8 the wait for the step's loads         16 the tile's stores
-#ifndef LLMP_GEMM_WITHOUT
-#define LLMP_GEMM_WITHOUT 0
-#endif
-#if LLMP_GEMM_WITHOUT != 0 && !defined(LLMP_GEMM_TRACE)
-#error "LLMP_GEMM_WITHOUT is for the tuning build"
-#endif
-
 // LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
 template <int WN, int RA>
 struct GemmLds {
@@ -338,7 +295,7 @@ __device__ __forceinline__ void AwaitLoads() {
 // stores, which take about 4 us to be accepted (every CU stores its 98 KB at once; stores marked nontemporal made a
 // launch 107 us instead of 91).
 //
-// What bounds a step (M 2048, N 12288, K 4096; the tuning build's probe and ablations): one wave a SIMD issues a
+// What bounds a step (M 2048, N 12288, K 4096; measured with a probe of the matrix pipe and with parts of the loop left out): one wave a SIMD issues a
 // product every 32 cycles, and a vector move, a read of LDS or (every third product) a load to LDS between two
 // products costs 0.3 to 1.2 cycles: they are issued while the product runs. But the clock does not hold: 2.4 GHz on
 // zeros, 1.97 GHz with random codes in every CU's products, and 1.35-1.4 GHz when the operands also stream from L2
@@ -461,11 +418,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   // A load after every kLoadEvery-th product: a CU's path to LDS takes 64 bytes a cycle, its four waves' loads after
   // every product would ask for 128 (1 KB a wave every 32 cycles) and hold the next products back.
   constexpr int kLoadEveryMost = kXFrags * WN / (kLoadsA + 1 + kLoadsB);
-#ifndef LLMP_GEMM_LOAD_EVERY
   constexpr int kLoadEvery = kLoadEveryMost;
-#else
-  constexpr int kLoadEvery = LLMP_GEMM_LOAD_EVERY < kLoadEveryMost ? LLMP_GEMM_LOAD_EVERY : kLoadEveryMost;
-#endif
   static_assert(L::kTileBBytes % (16 * kThreads) == 0 && (kLoadsA + 1 + kLoadsB) * kLoadEvery <= kXFrags * WN, "load slots");
   // The kernel's register counts cover the named ones.
   if constexpr (WM == 2) {
@@ -474,8 +427,6 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     asm volatile("" ::: "v159", "a95");
   }
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  GEMM_TRACE_BEGIN;
-  GEMM_TRACE(0);  // the wave's start
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -647,9 +598,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     constexpr int P = decltype(pc)::value;
     constexpr bool kFirst = decltype(firstc)::value;  // the tile's first step starts its sums, the others add to them
     using Next = std::integral_constant<int, R::kTwice ? 1 - P : 0>;
-    if (step == 1) GEMM_TRACE(3 + 8 * min(ord, 1));
-    if (step == steps / 2) GEMM_TRACE(4 + 8 * min(ord, 1));
-    if constexpr ((LLMP_GEMM_WITHOUT & 4) == 0) barrier();
+    barrier();
     // Every wave holds step `step`'s fragments; steps up to `step` + RA - 1 (weights: + 2) are whole in LDS or on
     // their way, step + 1 whole.
     const int next_a = stage_a + 1 == RA ? 0 : stage_a + 1;      // step + 1's activations
@@ -668,16 +617,14 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
         ScaledProduct<R, kXFrags * i + j, i, j, P, kFirst>();
         constexpr int t = j * WN + i;
         constexpr int q = t % kLoadEvery == 0 ? t / kLoadEvery : kLoadsA + 1 + kLoadsB;  // the load after product t
-        if constexpr ((LLMP_GEMM_WITHOUT & 1) != 0) {
-        } else if constexpr (q < kLoadsA) {
+        if constexpr (q < kLoadsA) {
           load_a_ahead(q, bring_a, stage_a);
         } else if constexpr (q == kLoadsA) {
           load_scales(bring_a, stage_a, bring_b, stage_b);
         } else if constexpr (q - kLoadsA - 1 < kLoadsB) {
           load_b_ahead(q - kLoadsA - 1, bring_b, stage_b);
         }
-        if constexpr ((LLMP_GEMM_WITHOUT & 2) != 0) {
-        } else if constexpr (R::kTwice) {
+        if constexpr (R::kTwice) {
           using Before = std::integral_constant<int, j == 0 ? kXFrags - 1 : j - 1>;
           if constexpr (i == 0) read_a_lo(Before{}, Next{});
           if constexpr (i == 1) read_a_hi(Before{}, Next{});
@@ -688,19 +635,17 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
         }
         __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr ((LLMP_GEMM_WITHOUT & 2) == 0 && !R::kTwice) read_a(jc, Next{});
+      if constexpr (!R::kTwice) read_a(jc, Next{});
       __builtin_amdgcn_sched_barrier(0);
     });
     read_done();
     // Step + 2 has landed: with two activation stages all but the weights just asked for (and their scales, wave 1),
     // with three everything asked for before this iteration (loads complete in the order they were asked for).
-    if constexpr ((LLMP_GEMM_WITHOUT & 8) == 0) {
-      constexpr int kLeft = RA == 2 ? kLoadsB : kLoadsA + kLoadsB;
-      if (wave == 1 || (RA > 2 && wave == 0)) {
-        AwaitLoads<kLeft + 1>();
-      } else {
-        AwaitLoads<kLeft>();
-      }
+    constexpr int kLeft = RA == 2 ? kLoadsB : kLoadsA + kLoadsB;
+    if (wave == 1 || (RA > 2 && wave == 0)) {
+      AwaitLoads<kLeft + 1>();
+    } else {
+      AwaitLoads<kLeft>();
     }
     stage_a = next_a;
     stage_b = next_b;
@@ -722,7 +667,6 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
           constexpr int reg = (kXFrags * i + j) * 4;
           const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
           if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
-          if ((LLMP_GEMM_WITHOUT & 16) != 0 && v0 != 12345.678f) return;  // (the sums are still read and converted)
           const int64_t at = first + j * row_step + i * 16;
           if constexpr (decltype(bf16)::value) {
             uint2 packed;
@@ -753,15 +697,12 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
 
   aim_loads(0);
   first_loads();
-  GEMM_TRACE_CYCLES(1);  // the first stages asked for
   for (; ord < mine; ++ord) {
     aim_weight_scales(ord);
     // The tile's first stages have landed (they were asked for ahead of the tile before's stores, which this wait
     // counts as well), for every wave.
     AwaitLoads<0>();
     barrier();
-    GEMM_TRACE(2 + 8 * min(ord, 1));
-    if (ord > 0) GEMM_TRACE_CYCLES(9);  // (the first tile's counter is read when its loads have been asked for)
     aim_reads(0, 0);
     StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
     StaticFor<WN>([&](auto i) { read_b(i, Even{}); });
@@ -775,7 +716,6 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
       multiply(Even{}, std::false_type{}, step + 1);
     }
     if (step < steps) multiply(Odd{}, std::false_type{}, step);
-    GEMM_TRACE(5 + 8 * min(ord, 1));  // the tile's last step multiplied
     // The next tile's first stages are asked for ahead of this tile's stores: they land while the stores are taken.
     // (This wave's loads still on their way, the last step asked for again, go to places of its own and land first.)
     if (ord + 1 < mine) {
@@ -784,9 +724,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     }
     // The last products' sums are written passes after their issue: no read of them before.
     asm volatile("s_nop 15\n\ts_nop 15");
-    GEMM_TRACE_CYCLES(6 + 8 * min(ord, 1));
     store_tile(ord);
-    GEMM_TRACE(7 + 8 * min(ord, 1));  // the tile's stores queued
   }
   AwaitLoads<0>();  // nothing may land in LDS after the workgroup has gone
 }
@@ -798,88 +736,11 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel192(const GemmArgs a) {
   GemmTiles<2, 6, 2>(a);
 }
-#ifndef LLMP_GEMM_EIGHT_WAVES
 __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernel128(const GemmArgs a) {
   GemmTiles<2, 4, 2>(a);
 }
 constexpr int kWavesM128 = 2, kRingA128 = 2;
-#else  // the tuning build's (make trace EXTRA=-DLLMP_GEMM_EIGHT_WAVES): that form, and the 256 x 128 tile wherever it ties
-__global__ __launch_bounds__(512, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(4)))) void GemmKernel128(const GemmArgs a) {
-  GemmTiles<4, 4, 3>(a);
-}
-constexpr int kWavesM128 = 4, kRingA128 = 3;
-#endif
 
-#ifdef LLMP_GEMM_TRACE
-// The tuning build's probe of the matrix pipe alone: the 256 x 192 kernel's 48 products of a step, from the same
-// named registers, `iters` times over with nothing between them, four waves a workgroup (one a SIMD). The
-// fragments are filled from `data` (126 dwords a lane: zeros and random codes draw different power), the scales
-// are 1. Lane 0 of the first wave writes the shader counter's ticks over the loop to `ticks`.
-__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void ProductsProbeKernel(
-    const uint32_t* __restrict__ data, int iters, int stream_slots, unsigned long long* ticks, float* sink) {
-  using R = GemmRegs<2, 6>;
-  asm volatile("" ::: "v253", "a191");
-  StaticFor<R::kXScale - R::kX>([&](auto rc) {
-    constexpr int reg = R::kX + decltype(rc)::value;
-    const uint32_t v = data[decltype(rc)::value % 126 * 256 + threadIdx.x];
-    asm volatile("v_mov_b32 v[%0], %1" ::"n"(reg), "v"(v));
-  });
-  StaticFor<R::kTop - R::kXScale>([&](auto rc) {
-    constexpr int reg = R::kXScale + decltype(rc)::value;
-    asm volatile("v_mov_b32 v[%0], 127" ::"n"(reg));
-  });
-  StaticFor<R::kSums>([&](auto t) { ClearSum<decltype(t)::value>(); });
-  asm volatile("s_nop 7");
-  const unsigned long long t0 = __builtin_readcyclecounter();
-  // LLMP_GEMM_PROBE_BETWEEN: one more instruction of the same wave after every product (what it costs the pipe):
-  //   1 a vector move   2 a 16-byte read of LDS into registers no product uses   3 the same into the activation
-  //   fragment the product has just been issued from   4 a 16-byte load a lane from `data` to LDS   5 that load
-  //   after every third product   6 after every third product a load of bytes that no workgroup has asked for
-  //   before (64 KB an iteration a workgroup from `stream_slots` slots of `data`), the iteration before's in flight
-#ifndef LLMP_GEMM_PROBE_BETWEEN
-#define LLMP_GEMM_PROBE_BETWEEN 0
-#endif
-  __shared__ __attribute__((aligned(16))) uint8_t probe_lds[4096];
-  const uint32_t probe_at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x & 63) * 16;
-  const uint32_t probe_to =
-      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(probe_lds)) + (threadIdx.x >> 6) * 1024);
-  const uint32_t probe_from = threadIdx.x * 16;
-  const uint8_t* stream_from = reinterpret_cast<const uint8_t*>(data);
-  auto between = [&](auto jc, auto ic) {
-    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 1) {
-      asm volatile("v_mov_b32 v120, v121" ::: "v120");
-    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 2) {
-      asm volatile("ds_read_b128 v[120:123], %0" ::"v"(probe_at) : "v120", "v121", "v122", "v123");
-    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 3) {
-      LdsToRegs16<R::X(decltype(jc)::value, 0), 0>(probe_at);
-    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 4 || (LLMP_GEMM_PROBE_BETWEEN == 5 && decltype(ic)::value % 3 == 0)) {
-      GlobalToLds16(reinterpret_cast<const uint8_t*>(data), probe_from, probe_to);
-    } else if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6 && decltype(ic)::value % 3 == 0) {
-      GlobalToLds16(stream_from + (decltype(jc)::value * 2 + decltype(ic)::value / 3) * 4096, probe_from, probe_to);
-    }
-  };
-  for (int it = 0; it < iters; ++it) {
-    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6)
-      stream_from = reinterpret_cast<const uint8_t*>(data) + static_cast<size_t>((blockIdx.x * 61u + static_cast<unsigned>(it)) % static_cast<unsigned>(stream_slots)) * 65536;
-    StaticFor<8>([&](auto jc) {
-      StaticFor<6>([&](auto ic) {
-        ScaledProduct<R, 8 * decltype(ic)::value + decltype(jc)::value, decltype(ic)::value, decltype(jc)::value>();
-        between(jc, ic);
-      });
-    });
-    if constexpr (LLMP_GEMM_PROBE_BETWEEN == 6) {
-      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)");
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)");
-  const unsigned long long t1 = __builtin_readcyclecounter();
-  asm volatile("s_nop 15\n\ts_nop 15");
-  sink[blockIdx.x * 256 + threadIdx.x] = ReadSum<0>() + ReadSum<191>();
-  if (blockIdx.x == 0 && threadIdx.x == 0) ticks[0] = t1 - t0;
-}
-#endif
 
 // A workgroup a compute unit, each through its share of the tiles (fewer workgroups where there are fewer tiles).
 template <int WM, int WN, int RA>
@@ -1021,32 +882,10 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
     const int64_t tiles = static_cast<int64_t>(a.tiles_m) * ((gemm->n + tile_n - 1) / tile_n);
     if (tiles > (1 << 30)) return Refuse(1, "mxfp8.gemm: too many tiles");
     const int64_t cost = (tiles + cus - 1) / cus * tile_n;
-#ifndef LLMP_GEMM_EIGHT_WAVES
     if (best == 0 || cost < best_cost) best = tile_n, best_cost = cost;
-#else
-    if (best == 0 || cost <= best_cost) best = tile_n, best_cost = cost;
-#endif
   }
   const hipStream_t on = static_cast<hipStream_t>(stream);
   const int status = best == 192 ? LaunchGemm<2, 6, 2>(GemmKernel192, a, cus, on) : LaunchGemm<kWavesM128, 4, kRingA128>(GemmKernel128, a, cus, on);
   return status;  // negative: the launch failed after the checks (the caller's fault path)
 }
 
-#ifdef LLMP_GEMM_TRACE
-// The tuning build's switch: where the GEMM's waves put their timestamps (device memory), or null.
-extern "C" int llmp_hip_gemm_trace_set(unsigned long long* buffer) {
-  return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(llmp_hip::g_gemm_trace), &buffer, sizeof(buffer)));
-}
-// The products probe on `workgroups` workgroups: data 126 x 256 dwords (or `stream_slots` x 64 KB where that is
-// more: what its streaming variant reads), ticks one 64-bit word, sink 256 floats a workgroup.
-extern "C" int llmp_hip_gemm_probe_products(const void* data, int iters, int workgroups, int stream_slots, void* ticks, void* sink,
-                                            void* stream) {
-  BeginLaunches();
-  if (data == nullptr || ticks == nullptr || sink == nullptr || iters < 1 || workgroups < 1 || stream_slots < 1)
-    return Refuse(1, "probe: arguments");
-  hipLaunchKernelGGL(ProductsProbeKernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint32_t*>(data), iters, stream_slots, static_cast<unsigned long long*>(ticks),
-                     static_cast<float*>(sink));
-  return LaunchStatus("probe");
-}
-#endif

@@ -59,22 +59,6 @@ namespace {
 constexpr int kGroup = 512;      // threads a workgroup: eight waves, two workgroups a CU
 constexpr int kWaves = kGroup / kWave;
 
-// Timeline instrumentation for tuning, compiled only into a build with -DLLMP_VECQ_TRACE (never the library's):
-// lane 0 of every wave of a dense launch stores the 100 MHz clock at up to eight points of its run, eight 64-bit
-// words a wave.
-#ifdef LLMP_VECQ_TRACE
-__device__ unsigned long long* g_trace = nullptr;
-#define LLMP_TRACE(slot)                                                                                     \
-  do {                                                                                                       \
-    if (g_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
-      g_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 8 + (slot)] = wall_clock64(); \
-  } while (0)
-#else
-#define LLMP_TRACE(slot) \
-  do {                   \
-  } while (0)
-#endif
-
 // ---- the activations' first loads
 
 // Staging is split in two so that a row's first loads can be queued before the wave's first
@@ -1401,7 +1385,6 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
 
-  LLMP_TRACE(0);  // the wave's start
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -1496,12 +1479,9 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
         }
       }
     }
-    LLMP_TRACE(1);  // the first tile queued, the wave's part of the records staged
     __syncthreads();  // the records are staged; from here the waves run alone
-    LLMP_TRACE(2);
 
     int buffer = 0;  // kDeep: the tile buffer the tile `index` is in
-    [[maybe_unused]] int trace_slot = 3;  // 3, 5: the first and second tile landed; 4, 6: their rows stored
     while (index < tiles) {
       const int row0 = index * rows_per_tile;
       const bool live = placed && row0 + row < d.nrows;
@@ -1520,8 +1500,6 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
       } else {
         AwaitTile();
       }
-      if (trace_slot < 7) LLMP_TRACE(trace_slot);
-      ++trace_slot;
       float out[P];
       if (live) {
         int32_t* dump = kDump ? a.dump + (static_cast<int64_t>(row0 + row) * nsb + sb) * F::kDumpInts : nullptr;
@@ -1548,8 +1526,6 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
           }
         }
       }
-      if (trace_slot < 7) LLMP_TRACE(trace_slot);
-      ++trace_slot;
       index = next;
       if constexpr (kDeep) {
         buffer ^= 1;
@@ -1563,7 +1539,6 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
       }
     }
   }
-  LLMP_TRACE(7);  // the wave's end
 }
 
 // Rows longer than a wave's 64 units: a row is cut into `split` pieces of `piece` units (the

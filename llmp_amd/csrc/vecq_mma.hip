@@ -61,42 +61,6 @@ constexpr int kWholeRow = 8;                         // super-blocks a row up to
 constexpr int kPartialBytes = kMmaWaves * 2 * kWave * 16;  // a wave's four floats a lane and matrix
 constexpr size_t kMmaLdsLimit = 160 * 1024 - 2048;
 
-// Timeline instrumentation for tuning, compiled only into a build with -DLLMP_MMA_TRACE (never the
-// library's): lane 0 of every wave stores the 100 MHz clock at up to sixteen points of the Q4_K kernel.
-#ifdef LLMP_MMA_TRACE
-__device__ unsigned long long* g_mma_trace = nullptr;
-// The stamps wait in LDS until the wave ends: a store to global memory at the point itself would wait for the
-// pointer's load behind every weight load in flight, and the wave with it.
-#define MMA_TRACE_AREA __shared__ unsigned long long trace_area[kMmaWaves][16]
-#define MMA_TRACE(slot)                                                                          \
-  do {                                                                                           \
-    if ((threadIdx.x & 63) == 0 && (slot) < 16) trace_area[threadIdx.x / 64][slot] = wall_clock64(); \
-  } while (0)
-#define MMA_TRACE_ADD(slot, value)                                            \
-  do {                                                                        \
-    if ((threadIdx.x & 63) == 0) trace_area[threadIdx.x / 64][slot] += (value); \
-  } while (0)
-#define MMA_TRACE_DUMP                                                                                          \
-  do {                                                                                                          \
-    trace_area[threadIdx.x / 64][15] = wall_clock64();                                                          \
-    trace_area[threadIdx.x / 64][12] = __builtin_readcyclecounter();                                            \
-    if (g_mma_trace != nullptr && (threadIdx.x & 63) < 16)                                                      \
-      g_mma_trace[((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * kMmaWaves + threadIdx.x / 64) * 16 + \
-                  (threadIdx.x & 63)] = trace_area[threadIdx.x / 64][threadIdx.x & 63];                        \
-  } while (0)
-#else
-#define MMA_TRACE_AREA
-#define MMA_TRACE_ADD(slot, value) \
-  do {                             \
-  } while (0)
-#define MMA_TRACE(slot) \
-  do {                  \
-  } while (0)
-#define MMA_TRACE_DUMP \
-  do {                 \
-  } while (0)
-#endif
-
 typedef int V4i __attribute__((ext_vector_type(4)));
 typedef float V4f __attribute__((ext_vector_type(4)));
 typedef _Float16 H2 __attribute__((ext_vector_type(2)));
@@ -337,20 +301,11 @@ struct Segment {
 template <bool kGlu, int TG, int MT>
 __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int balanced) {
   using L = Staged<TG, MT>;
-#ifndef MMA_DEPTH1
-#define MMA_DEPTH1 3
-#endif
-  constexpr int kDepth = TG == 1 ? MMA_DEPTH1 : TG == 2 ? 3 : 2;  // weight buffers: the fetches run kDepth - 1 steps ahead
+  constexpr int kDepth = TG == 1 ? 3 : TG == 2 ? 3 : 2;  // weight buffers: the fetches run kDepth - 1 steps ahead
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
   __shared__ int scan[kMmaGroup / kWave];
-  MMA_TRACE_AREA;
-#ifdef LLMP_MMA_TRACE
-  if ((threadIdx.x & 63) < 16) trace_area[threadIdx.x / 64][threadIdx.x & 63] = 0;
-#endif
-  MMA_TRACE(0);  // the wave's start
-  MMA_TRACE_ADD(11, static_cast<unsigned long long>(__builtin_readcyclecounter()));  // and its shader clock
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
@@ -388,8 +343,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
     const int64_t expert_block = static_cast<int64_t>(seg.expert) * d.stride_expert;
     const int p0 = seg.first, m = seg.m;
     const int steps = seg.group_count * (last - first);
-    MMA_TRACE_ADD(13, static_cast<unsigned long long>(steps));  // the wave's steps
-    MMA_TRACE_ADD(14, 1ull);                                     // and segments
     // The live token groups rounded up to a power of two: one compiled step each.
     const int token_groups = (m + MT - 1) / MT;
     const int live = token_groups <= 1 ? 1 : token_groups <= 2 ? 2 : 4;
@@ -445,7 +398,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
     aim();
 #pragma unroll
     for (int j = 0; j < kDepth - 1; ++j) fetch(ub[j], gb[j]);
-    MMA_TRACE(1);  // the tokens and the first weights asked for
 
 #pragma unroll
     for (int it = 0; it < kStageAhead; ++it) {
@@ -464,7 +416,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
       StageBlock<TG, MT>(w, t, b, codes, d8, ds8);
     }
     __syncthreads();
-    MMA_TRACE(2);  // the tokens staged
 
     V4f up_out[TG], gate_out[TG];
     auto clear = [&]() {
@@ -541,7 +492,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
         if (j == 0 || s + j < steps) {
           fetch(ub[(j + kDepth - 1) % kDepth], gb[(j + kDepth - 1) % kDepth]);
           step(ub[j], gb[j]);
-          if (s < 6 && j < 4) MMA_TRACE(3 + s + j);
         }
       }
     }
@@ -639,7 +589,6 @@ __global__ __launch_bounds__(kMmaGroup, 1) void VecQMma(const VecQArgs a, int ba
       }
     }
   }
-  MMA_TRACE_DUMP;  // with the wave's end
 }
 
 // ------------------------------------------------------------------ Q8_0
@@ -995,11 +944,6 @@ int g_mma_compute_units = 0;
 
 }  // namespace
 
-#ifdef LLMP_MMA_TRACE
-extern "C" int llmp_hip_trace_set_mma(unsigned long long* buffer) {
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_mma_trace), &buffer, sizeof(buffer)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 // Q4_K rows of which at least eight staged tokens fit LDS (k up to 8448; sixteen up to 4096, two
 // groups of sixteen up to 2048). Q8_0 rows of whole units of 128 values, up to 64 units (8192

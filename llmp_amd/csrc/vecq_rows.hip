@@ -40,33 +40,6 @@ constexpr int kPieceBytes = kTileRows * 144;  // one super-block of a tile's row
 constexpr int kPieceLoads = kPieceBytes / (kWave * 16);
 constexpr size_t kRowsLdsLimit = 160 * 1024 - 1024;
 
-// Timeline instrumentation for tuning, compiled only into a build with -DLLMP_MMA_TRACE (never the library's):
-// lane 0 of every wave keeps the 100 MHz clock of up to sixteen points in LDS and stores them as the wave ends.
-#ifdef LLMP_MMA_TRACE
-__device__ unsigned long long* g_rows_trace = nullptr;
-#define ROWS_TRACE_AREA __shared__ unsigned long long trace_area[kRowsWaves][16]
-#define ROWS_TRACE(slot)                                                                         \
-  do {                                                                                           \
-    if ((threadIdx.x & 63) == 0 && (slot) < 16)                                                  \
-      LdsWrite8(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&trace_area[threadIdx.x / 64][slot])), wall_clock64()); \
-  } while (0)
-#define ROWS_TRACE_DUMP                                                                                         \
-  do {                                                                                                          \
-    trace_area[threadIdx.x / 64][15] = wall_clock64();                                                          \
-    if (g_rows_trace != nullptr && (threadIdx.x & 63) < 16)                                                     \
-      g_rows_trace[((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * kRowsWaves + threadIdx.x / 64) * 16 + \
-                   (threadIdx.x & 63)] = trace_area[threadIdx.x / 64][threadIdx.x & 63];                       \
-  } while (0)
-#else
-#define ROWS_TRACE_AREA
-#define ROWS_TRACE(slot) \
-  do {                   \
-  } while (0)
-#define ROWS_TRACE_DUMP \
-  do {                  \
-  } while (0)
-#endif
-
 typedef int V4i __attribute__((ext_vector_type(4)));
 typedef float V4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* LdsPointer;
@@ -239,11 +212,6 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   using T = Tokens<NT>;
   constexpr int kMatrices = kGlu ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  ROWS_TRACE_AREA;
-#ifdef LLMP_MMA_TRACE
-  if ((threadIdx.x & 63) < 16) trace_area[threadIdx.x / 64][threadIdx.x & 63] = 0;
-#endif
-  ROWS_TRACE(0);  // the wave's start
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
@@ -381,7 +349,6 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   for (int it = 0; it < kHeld; ++it) ask_block(tid + it * kRowsGroup, held[it]);
 #pragma unroll
   for (int i = 1; i < STAGES - 1; ++i) issue(i);
-  ROWS_TRACE(1);  // the tokens and the first weights asked for
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kPieceLoads * (STAGES - 2)));
 #pragma unroll
   for (int it = 0; it < kHeld; ++it) stage_block(held[it], tid + it * kRowsGroup);
@@ -402,7 +369,6 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
 #pragma unroll
     for (int tq = 0; tq < NT / 4; ++tq) up_mins[tq] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, gate_mins[tq] = up_mins[tq];
     LdsBarrier();  // the tokens are staged
-    ROWS_TRACE(2);
     {
       // Two super-blocks of the up matrix, then the same two of the gate matrix: neighbours in a row share a 64-byte
       // unit of HBM more often than not, and the sooner the second asks for it the likelier L2 still has it.
@@ -413,7 +379,6 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
         const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * 8 * T::kScalesBlock);
         const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
         next_piece(i);
-        ROWS_TRACE(3 + i);  // piece i landed (the first ten)
         PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
         ++i;
         __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
@@ -425,9 +390,7 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
           for (int w = 0; w < width; ++w) piece_dot(sb_first + n + w, gate_out, gate_mins);
         }
       }
-      ROWS_TRACE(13);  // the last piece multiplied (nothing is in flight: its wait was for every load)
     }
-    ROWS_TRACE(14);
     // The four quarters of K meet: [wave][matrix][token][row] floats at the head of each wave's ring.
     float* mine = reinterpret_cast<float*>(ring);
 #pragma unroll
@@ -453,18 +416,10 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     }
     __syncthreads();  // the next tile's first loads land where the sums were
   }
-  ROWS_TRACE_DUMP;
 }
 
 int g_rows_compute_units = 0;
 
-#ifdef LLMP_MMA_TRACE
-}  // namespace
-extern "C" int llmp_hip_trace_set_rows(unsigned long long* buffer) {
-  return hipMemcpyToSymbol(HIP_SYMBOL(g_rows_trace), &buffer, sizeof(buffer)) == hipSuccess ? 0 : -1;
-}
-namespace {
-#endif
 
 template <int NT>
 int StagesFor(int blocks) {

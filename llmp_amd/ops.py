@@ -415,6 +415,15 @@ def exl3_linear_static(trellis, suh, svh, k, n, bits, codebook, x, a_had, y):
     return y
 
 
+def exl3_linear_static_prepare(trellis, suh, svh, k, n, bits, codebook):
+    """llmp_hip_exl3_linear_static_prepare: the set-up that is no launch (the static array's address on this device,
+    the product kernels' dynamic LDS), to be done outside a stream capture."""
+    lib = _lib.load()
+    op = Exl3Linear()
+    op.weights = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
+    _lib.check(lib.llmp_hip_exl3_linear_static_prepare(C.byref(op)))
+
+
 def exl3_multi_linear(first, second, x, f32=True, keep=None):
     """exl3.multi_linear: x float16 [m, k] (sixteen rows a pass) through a gate and an up linear of the same k, n and
     rate: [2, m, n]. `first` and `second` are (trellis, suh, svh, k, n, bits, codebook); `keep`, a dict,

@@ -207,7 +207,9 @@ def nvfp4_operand(g, rows, k, padded_rows=None):
 
 
 @pytest.mark.parametrize("counts,n,k", [([5, 0, 70, 1, 130], 96, 256), ([64, 64], 64, 64), ([3], 200, 1024),
-                                        ([17, 33, 0, 0, 129, 2, 64, 11], 768, 2048)])
+                                        ([17, 33, 0, 0, 129, 2, 64, 11], 768, 2048),
+                                        # 128 experts as the reference's layers have them, most without a row
+                                        ([(7 * e) % 41 if e % 5 == 0 else (1 if e % 17 == 3 else 0) for e in range(128)], 256, 512)])
 def test_grouped_nvfp4_gemm_matches_its_definition(device, counts, n, k):
     """llmp.moe.gemm (RunGroupedGemm, src/kernels/ggml/moe_cutlass.h:48-76 of the reference): experts with no rows,
     one row, partial tiles of rows and of columns, more rows than a tile; D in BF16 within one rounding of the F64

@@ -32,13 +32,19 @@ def test_static_scratch_linear_equals_the_linear_on_two_calls_in_a_row(device):
         a_had = torch.zeros((m, k), dtype=torch.float16, device=device)
         y = torch.full((m, n), 7.0, dtype=torch.float32 if f32 else torch.float16, device=device)
         cases.append((weights, halves(x, device), a_had, y, f32, (trellis, suh, svh, x)))
+    # The set-up that is no launch (the array's address, the kernels' LDS attribute) first: what it takes from the
+    # runtime, a code object's load included, is taken here and not by the calls that are counted below.
+    for weights, *_ in cases:
+        ops.exl3_linear_static_prepare(*weights)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]  # hipMemGetInfo: sees what the library or the runtime would take too
     # Two calls in a row on one stream, sharing the device's static array; nothing is allocated between them.
     for weights, x, a_had, y, _, _ in cases:
         ops.exl3_linear_static(*weights, x, a_had, y)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     for weights, x, a_had, y, f32, host in cases:
         keep = {}
         want = ops.exl3_linear(*weights, x, f32=f32, keep=keep)
@@ -58,6 +64,31 @@ def test_static_scratch_linear_equals_the_linear_on_two_calls_in_a_row(device):
     ops.exl3_linear_static(*weights, x, a_had, y)
     torch.cuda.synchronize()
     assert torch.equal(first.view(torch.int16), y.view(torch.int16))
+
+
+def test_static_scratch_linear_captured_in_a_graph_replays_bit_for_bit(device):
+    """Prepared outside the capture, captured through the launch context's thread-local capture, replayed twice with
+    a different x each time and eager work between: every replay is bit for bit the eager linear."""
+    bits, codebook, k, n, m = 4, ops.EXL3_3INST, 1024, 512, 2
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 95)
+    weights = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    ops.exl3_linear_static_prepare(*weights)
+    x = torch.zeros((m, k), dtype=torch.float16, device=device)
+    a_had = torch.zeros((m, k), dtype=torch.float16, device=device)
+    y = torch.zeros((m, n), dtype=torch.float32, device=device)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side, capture_error_mode="thread_local"):
+        ops.exl3_linear_static(*weights, x, a_had, y)
+    for seed in (96, 97):
+        fresh = halves(synth.rng(seed).standard_normal((m, k)).astype(np.float16), device)
+        x.copy_(fresh)
+        want = ops.exl3_linear(*weights, fresh, f32=True)  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int32), want.view(torch.int32))
 
 
 def test_static_scratch_linear_refuses_what_exceeds_its_array(device):
