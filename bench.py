@@ -402,6 +402,42 @@ def other_configs(device, args, only=None):
         out["moe_gemm_nvfp4_128_experts_t512"] = entry
         torch.cuda.empty_cache()
 
+    # The attention that reads the quantized KV cache (ggml.flash_attn_ext.vec_q8_0, a "next" row of the path: not a
+    # BASELINE config), at config 2's model's decode shape: 16 heads over 8 KV heads of 256, one query row, 8192 cells.
+    for kind, t in (("q8_0", ops.TYPE_Q8_0), ("q4_0", ops.TYPE_Q4_0)):
+        name = f"attn_vec_{kind}_d256_h16_kv8_cells8192_rows1"
+        if not want(name):
+            continue
+        d_, heads, kv_heads, cells = 256, 16, 8, 8192
+        g = synth.rng(240)
+        k_host = oracle.kv_quantize(t, g.standard_normal((cells * kv_heads, d_), dtype=np.float32)).reshape(cells, -1)
+        v_host = oracle.kv_quantize(t, g.standard_normal((cells * kv_heads, d_), dtype=np.float32)).reshape(cells, -1)
+        q_host = g.standard_normal((heads, 1, d_), dtype=np.float32)
+        mask_host = np.zeros((2, cells), dtype=np.float16)
+        mask_host[:, cells - 37:] = -np.inf
+        kd, vd = dev(k_host), dev(v_host)
+        copies = max(2, -(-ROTATE_BYTES // (2 * kd.numel())))
+        ks = [kd] + [kd.clone() for _ in range(copies - 1)]
+        vs = [vd] + [vd.clone() for _ in range(copies - 1)]
+        qd, md = dev(q_host), dev(mask_host.view(np.int16)).view(torch.float16)
+        out_d = torch.empty((1, heads, d_), dtype=torch.float32, device=device)
+        scratch = torch.empty(8 << 20, dtype=torch.uint8, device=device)
+        scale = 1.0 / 16.0
+        us = timed(lambda i: ops.attn_vec_quant(t, qd, ks[i % copies], vs[i % copies], md, d_, heads, kv_heads, cells, scale,
+                                                out=out_d, scratch=scratch), 4 * copies)
+        bytes_ = 2 * kd.numel() + heads * d_ * 8 + cells * 2
+        entry = {"workload": f"attention over a {kind.upper()} KV cache, head size 256, 16 heads over 8 KV heads, 1 query row, "
+                             "8192 cells (both launches: the splits and their combination); not a BASELINE config",
+                 "roofline": hbm_roofline(name, "AttnVecQuantKernel + AttnCombineKernel", bytes_, us)}
+        if cpu:
+            entry["cpu_baseline"] = cpu_leg(
+                lambda: oracle.attention_quant(t, q_host, k_host, v_host, d_, heads, kv_heads, 1, cells, scale, mask=mask_host,
+                                               threads=threads),
+                bytes_ / 1e9, "GB/s", 2.0, "the whole attention", threads)
+        out[name] = entry
+        del ks, vs, kd, vd
+        torch.cuda.empty_cache()
+
     # Config 5: EXL3 linear 4096 x 14336 at 4 bits, 3INST codebook.
     exl3_names = [f"exl3_linear_4096x14336_4bpw_m{m}" for m in (1, 16)]
     if any(want(nm) for nm in exl3_names) or want("exl3_multi_linear_4096x2x14336_4bpw_m1"):

@@ -292,6 +292,37 @@ typedef struct llmp_rope_store {
 } llmp_rope_store;
 int llmp_hip_rope_set_rows_quant(const llmp_rope_store* store, void* stream);
 
+/* ggml.flash_attn_ext.vec_q8_0 / vec_q4_0 (FlashAttnVecQuant over a checked ggml_flash_attn_ext node,
+ * src/kernels/ggml/kv_quant.h:9-26, 146-160; the checks of src/kernels/ggml/kv_quant.cc:81-170): attention that
+ * reads K and V as the Q8_0 or Q4_0 blocks the stores above wrote, nothing expanded into device memory.
+ * Q F32, value (d, row, head) at q[d + row * q_row_stride + head * q_head_stride] (ggml's [D, rows, heads]); K
+ * and V of one block type, the row of (cell, KV head) at cell * cell_stride + head * head_stride bytes (whole
+ * blocks; the reference's view [D, cells, KV heads] of a cache that holds a cell's heads together); an F16 mask
+ * row of `cells` values a query row, added to the scaled scores (-inf hides a cell); optional F32 sinks, one a
+ * head, in the softmax's denominator; output F32 [rows][heads][D] (ggml's [D, heads, rows]). head_dim 64 or 256
+ * (512 for Q8_0), cells a multiple of 256, heads a multiple of kv_heads by at most 8, a positive finite scale,
+ * softcap 0 or a positive one at head_dim 256 (score = softcap * tanh(score / softcap) before the mask), no
+ * ALiBi. The queries pass through Q8_1 for the K product, as in the reference's kernel; sums are F32. A query
+ * row that sees no cell (and has no sink) is zeros. The cells are split over workgroups whose partial results go
+ * through `scratch` (llmp_hip_attn_vec_quant_scratch bytes for the same `cus`, the device's compute units; 0
+ * where the operands would be refused) and are combined by a second launch. Returns as the launchers above. */
+typedef struct llmp_attn_vec_quant {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* mask;
+  const void* sinks; /* or NULL */
+  void* out;
+  int64_t q_row_stride, q_head_stride; /* floats */
+  int64_t k_cell_stride, k_head_stride, v_cell_stride, v_head_stride; /* bytes */
+  int64_t mask_row_stride; /* halves */
+  int32_t type; /* LLMP_TYPE_Q8_0 or LLMP_TYPE_Q4_0 */
+  int32_t head_dim, heads, kv_heads, rows, cells;
+  float scale, softcap;
+} llmp_attn_vec_quant;
+size_t llmp_hip_attn_vec_quant_scratch(const llmp_attn_vec_quant* op, int cus);
+int llmp_hip_attn_vec_quant(const llmp_attn_vec_quant* op, void* scratch, size_t scratch_bytes, int cus, void* stream);
+
 /* ------------------------------------------------------------------ EXL3
  * The trellis-coded linear. Weights as src/kernels/exl3/validate.h:84-96 holds them: the
  * trellis [k / 16][n / 16][16 * bits] uint16, suh (k F16) and svh (n F16); every dimension a

@@ -84,6 +84,17 @@ class SetRowsStore(C.Structure):
                 ("rows", C.c_int64), ("cells", C.c_int64)]
 
 
+class AttnVecQuant(C.Structure):
+    """llmp_attn_vec_quant: the operands of ggml.flash_attn_ext.vec_q8_0 / vec_q4_0 (src/kernels/ggml/kv_quant.h:146-160
+    of the reference)."""
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("mask", C.c_void_p), ("sinks", C.c_void_p),
+                ("out", C.c_void_p), ("q_row_stride", C.c_int64), ("q_head_stride", C.c_int64),
+                ("k_cell_stride", C.c_int64), ("k_head_stride", C.c_int64), ("v_cell_stride", C.c_int64),
+                ("v_head_stride", C.c_int64), ("mask_row_stride", C.c_int64), ("type", C.c_int32),
+                ("head_dim", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32), ("rows", C.c_int32),
+                ("cells", C.c_int32), ("scale", C.c_float), ("softcap", C.c_float)]
+
+
 class RopeStore(C.Structure):
     """llmp_rope_store: RopeStore of src/kernels/ggml/kv_quant_rope.cu:55-71 of the reference."""
     _fields_ = [("type", C.c_int), ("heads", C.c_int), ("head_dim", C.c_int), ("n_dims", C.c_int), ("x", C.c_void_p),
@@ -121,6 +132,8 @@ SYMBOLS = {
     "llmp_hip_set_rows_quant": (_int, [_int, _vp, _i64, _vp, _int, _vp, _i64, _i64, _i64, _i64, _vp]),
     "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
     "llmp_hip_rope_set_rows_quant": (_int, [C.POINTER(RopeStore), _vp]),
+    "llmp_hip_attn_vec_quant_scratch": (C.c_size_t, [C.POINTER(AttnVecQuant), _int]),
+    "llmp_hip_attn_vec_quant": (_int, [C.POINTER(AttnVecQuant), _vp, C.c_size_t, _int, _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmp_hip_mxfp8_swizzle": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "llmp_hip_mxfp8_gemv": (_int, [_vp, _vp, _i64, _i64, _vp, _int, _vp, _vp]),

@@ -267,6 +267,35 @@ def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWI
     return moe_combine(y, weights, route.position), ids, weights
 
 
+def attn_vec_quant(t, q, k_cache, v_cache, mask, head_dim, heads, kv_heads, cells, scale, *, softcap=0.0, sinks=None,
+                   cell_stride=None, head_stride=None, out=None, scratch=None):
+    """ggml.flash_attn_ext.vec_q8_0 / vec_q4_0: q float32 [heads, rows, head_dim]; k_cache, v_cache uint8 holding
+    the row of (cell, KV head) at cell * cell_stride + head * head_stride bytes (default: a cell's heads together);
+    mask float16 [>= rows, cells]. Returns float32 [rows, heads, head_dim]."""
+    lib = _lib.load()
+    rows = q.shape[1]
+    row_bytes = head_dim // 32 * BLOCK_BYTES[t]
+    head_stride = row_bytes if head_stride is None else head_stride
+    cell_stride = row_bytes * kv_heads if cell_stride is None else cell_stride
+    if out is None:
+        out = torch.empty((rows, heads, head_dim), dtype=torch.float32, device=q.device)
+    op = _lib.AttnVecQuant()
+    op.q, op.k, op.v, op.mask, op.out = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), mask.data_ptr(), out.data_ptr()
+    op.sinks = sinks.data_ptr() if sinks is not None else None
+    op.q_row_stride, op.q_head_stride = q.stride(1), q.stride(0)
+    op.k_cell_stride = op.v_cell_stride = cell_stride
+    op.k_head_stride = op.v_head_stride = head_stride
+    op.mask_row_stride = mask.stride(0)
+    op.type, op.head_dim, op.heads, op.kv_heads, op.rows, op.cells = t, head_dim, heads, kv_heads, rows, cells
+    op.scale, op.softcap = scale, softcap
+    cus = lib.llmp_hip_compute_units()
+    need = lib.llmp_hip_attn_vec_quant_scratch(C.byref(op), cus)
+    if scratch is None:
+        scratch = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.llmp_hip_attn_vec_quant(C.byref(op), _ptr(scratch), scratch.numel(), cus, _stream()))
+    return out
+
+
 def moe_gemm(a_codes, a_scales, offsets, sf_rows, weights, expert_stride, codes_offset, scales_offset, n, k, out=None):
     """llmp.moe.gemm (RunGroupedGemm, src/kernels/ggml/moe_cutlass.h:48-76 of the reference): routed rows sorted
     by expert, NVFP4 codes uint8 [rows, k / 2] with UE4M3 scales in atoms, times each expert's n rows of the

@@ -63,6 +63,8 @@ def _sig(name, res, *args):
 
 
 _i64, _u64, _vp, _int = C.c_int64, C.c_uint64, C.c_void_p, C.c_int
+_sig("orc_attention_quant", None, _int, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float,
+     C.c_float, _int, _vp, _int)
 _sig("orc_f16_to_f32", C.c_float, C.c_uint16)
 _sig("orc_f32_to_f16", C.c_uint16, C.c_float)
 _sig("orc_bf16_to_f32", C.c_float, C.c_uint16)
@@ -138,6 +140,26 @@ def kv_quantize(t, x):
     out = np.zeros((rows, k // 32 * block_bytes(t)), dtype=np.uint8)
     for r in range(rows):
         lib.orc_kv_quantize_row(t, _p(x[r]), k, _p(out[r]))
+    return out
+
+
+def attention_quant(t, q, k, v, d, heads, kv_heads, rows, cells, scale, *, mask=None, sinks=None, softcap=0.0,
+                    cell_stride=None, head_stride=None, q8_1_q=False, threads=1):
+    """Attention over a Q8_0 / Q4_0 KV cache decoded exactly (the reference executor's kAttention in double).
+    q float32 [heads, rows, d]; k, v uint8 with (cell, kv head)'s row at cell * cell_stride + head * head_stride
+    (default: a cell's heads together); mask float16 [>= rows, cells]; returns float32 [rows, heads, d]."""
+    row_bytes = d // 32 * block_bytes(t)
+    head_stride = row_bytes if head_stride is None else head_stride
+    cell_stride = row_bytes * kv_heads if cell_stride is None else cell_stride
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    out = np.zeros((rows, heads, d), dtype=np.float32)
+    mask_bits = None if mask is None else np.ascontiguousarray(mask).view(np.uint16)
+    if mask_bits is not None:
+        assert mask_bits.shape[1] == cells and mask_bits.shape[0] >= rows
+    sk = None if sinks is None else np.ascontiguousarray(sinks, dtype=np.float32)
+    lib.orc_attention_quant(t, _p(q), _p(k), _p(v), cell_stride, head_stride, _p(mask_bits) if mask_bits is not None else None,
+                            _p(sk) if sk is not None else None, d, heads, kv_heads, rows, cells, scale, softcap,
+                            int(q8_1_q), _p(out), threads)
     return out
 
 

@@ -1076,3 +1076,76 @@ void orc_exl3_linear(const uint8_t* trellis, const uint16_t* suh, const uint16_t
   orc_exl3_product(trellis, svh, k, n, bits, codebook, xh, m, y, threads);
   free(xh);
 }
+
+/* ------------------------------------------------------------------ attention over a quantized KV cache
+ * The reference executor's attention (src/kernels/reference/exec.cc:1027-1085, SoftmaxRow :279-299) over K and V
+ * rows stored as Q8_0 or Q4_0 blocks, decoded exactly (orc_decode_row), everything else in double: what the
+ * reference's own test holds its quantized vector attention to (tests/unit/kv_quant_gpu_test.cc:826-950, NMSE
+ * 5e-4). q F32 [heads][rows][d] (a head's rows together, as ggml's [D, rows, heads]); k, v uint8, the row of
+ * (cell, kv head) at cell * cell_stride + head * head_stride bytes; mask F16 bits [mask_rows][cells] or NULL;
+ * sinks F32 [heads] or NULL; out F32 [rows][heads][d] (ggml's [D, heads, rows]). No ALiBi (slope 1).
+ * q8_1_q != 0: each query row is first quantized to Q8_1 and decoded again, which is what the device multiplies K
+ * with (kv_quant.h:16-19 of the reference: "quantizing Q to Q8_1 in shared memory for the K product"): the
+ * comparison that leaves accumulation order alone. */
+void orc_attention_quant(int type, const float* q, const uint8_t* k, const uint8_t* v, int64_t cell_stride,
+                         int64_t head_stride, const uint16_t* mask, const float* sinks, int64_t d, int64_t heads,
+                         int64_t kv_heads, int64_t rows, int64_t cells, float scale, float softcap, int q8_1_q,
+                         float* out, int threads) {
+  const int64_t group = heads / kv_heads;
+#pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(dynamic)
+  for (int64_t h = 0; h < heads; ++h) {
+    const int64_t kh = h / group;
+    float* kd = (float*)malloc((size_t)(cells * d) * sizeof(float));
+    float* vd = (float*)malloc((size_t)(cells * d) * sizeof(float));
+    double* s = (double*)malloc((size_t)cells * sizeof(double));
+    float* qrow = (float*)malloc((size_t)d * sizeof(float));
+    uint8_t* q8 = (uint8_t*)malloc((size_t)((d + 511) / 512 * 512 / 32 * 36));
+    for (int64_t c = 0; c < cells; ++c) {
+      orc_decode_row(type, k + c * cell_stride + kh * head_stride, d, kd + c * d);
+      orc_decode_row(type, v + c * cell_stride + kh * head_stride, d, vd + c * d);
+    }
+    for (int64_t iq = 0; iq < rows; ++iq) {
+      const float* qsrc = q + (h * rows + iq) * d;
+      if (q8_1_q) {
+        orc_q8_1_quantize_row(qsrc, d, (d + 511) / 512 * 512, q8, 0);
+        orc_q8_1_decode_row(q8, d, qrow);
+      } else {
+        memcpy(qrow, qsrc, (size_t)d * sizeof(float));
+      }
+      double max = -INFINITY;
+      for (int64_t c = 0; c < cells; ++c) {
+        double dot = 0.0;
+        for (int64_t j = 0; j < d; ++j) dot += (double)qrow[j] * (double)kd[c * d + j];
+        double score = dot * (double)scale;
+        if (softcap > 0.0f) score = (double)softcap * tanh(score / (double)softcap);
+        if (mask != NULL) score += (double)orc_f16_to_f32(mask[iq * cells + c]);
+        s[c] = score;
+        if (score > max) max = score;
+      }
+      if (sinks != NULL && (double)sinks[h] > max) max = (double)sinks[h];
+      float* o = out + (iq * heads + h) * d;
+      if (!isfinite(max)) { /* a row with nothing finite (and no sink) is zero */
+        for (int64_t j = 0; j < d; ++j) o[j] = 0.0f;
+        continue;
+      }
+      double sum = sinks != NULL ? exp((double)sinks[h] - max) : 0.0;
+      for (int64_t c = 0; c < cells; ++c) {
+        s[c] = exp(s[c] - max);
+        sum += s[c];
+      }
+      for (int64_t j = 0; j < d; ++j) {
+        double acc = 0.0;
+        for (int64_t c = 0; c < cells; ++c) {
+          const double p = sum > 0.0 ? s[c] / sum : 0.0;
+          if (p != 0.0) acc += p * (double)vd[c * d + j];
+        }
+        o[j] = (float)acc;
+      }
+    }
+    free(kd);
+    free(vd);
+    free(s);
+    free(qrow);
+    free(q8);
+  }
+}

@@ -204,6 +204,13 @@ void orc_exl3_input(const uint16_t* suh, int64_t k, const uint16_t* x, int64_t m
 void orc_exl3_product(const uint8_t* trellis, const uint16_t* svh, int64_t k, int64_t n, int bits,
                       int codebook, const uint16_t* xh, int64_t m, float* y, int threads);
 
+/* Attention over a Q8_0 or Q4_0 KV cache decoded exactly, in double (exec.cc:1027-1085 of the reference); with
+ * q8_1_q the query rows pass through Q8_1 first, as the device's K product takes them. Layouts in oracle.c. */
+void orc_attention_quant(int type, const float* q, const uint8_t* k, const uint8_t* v, int64_t cell_stride,
+                         int64_t head_stride, const uint16_t* mask, const float* sinks, int64_t d, int64_t heads,
+                         int64_t kv_heads, int64_t rows, int64_t cells, float scale, float softcap, int q8_1_q,
+                         float* out, int threads);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

@@ -999,3 +999,81 @@ def test_grouped_nvfp4_values_and_product_by_scalar_loops():
             for c in (0, n - 1):
                 b_row = [value(b_codes[e], b_scales[e], c, j, 0) for j in range(k)]
                 assert got[r, c] == pytest.approx(sum(x * y for x, y in zip(a_row, b_row)), rel=1e-12, abs=1e-12)
+
+
+@pytest.mark.parametrize("t", [oracle.TYPE_Q8_0, oracle.TYPE_Q4_0])
+def test_attention_over_a_quantized_cache_against_numpy_and_closed_forms(t):
+    """orc_attention_quant (the reference executor's kAttention, src/kernels/reference/exec.cc:1027-1085, over Q8_0 /
+    Q4_0 rows): against an independent numpy softmax attention over the rows decoded by the pinned block decoders
+    (grouped heads, an F16 mask with -inf cells and finite biases, a softcap, sinks, pitched cells); and against what
+    the mathematics fixes: equal keys give the mean of the seen values, one seen cell gives that cell's value, a row
+    that sees nothing is zero, a large sink empties the output."""
+    g = np.random.default_rng(31 + t)
+    d, heads, kv_heads, rows, cells = 64, 6, 2, 3, 40
+    row_bytes = d // 32 * oracle.block_bytes(t)
+    keys = g.standard_normal((cells, kv_heads, d)).astype(np.float32)
+    vals = g.standard_normal((cells, kv_heads, d)).astype(np.float32)
+    pitch = row_bytes * kv_heads + 2 * oracle.block_bytes(t)  # a gap of two blocks after every cell
+    k_cache = np.zeros((cells, pitch), dtype=np.uint8)
+    v_cache = np.zeros((cells, pitch), dtype=np.uint8)
+    k_cache[:, :row_bytes * kv_heads] = oracle.kv_quantize(t, keys.reshape(cells * kv_heads, d)).reshape(cells, -1)
+    v_cache[:, :row_bytes * kv_heads] = oracle.kv_quantize(t, vals.reshape(cells * kv_heads, d)).reshape(cells, -1)
+    kd = oracle.decode_rows(t, k_cache[:, :row_bytes * kv_heads].reshape(cells * kv_heads, row_bytes), d).reshape(cells, kv_heads, d).astype(np.float64)
+    vd = oracle.decode_rows(t, v_cache[:, :row_bytes * kv_heads].reshape(cells * kv_heads, row_bytes), d).reshape(cells, kv_heads, d).astype(np.float64)
+    q = g.standard_normal((heads, rows, d)).astype(np.float32)
+    mask = np.full((rows + 1, cells), -np.inf, dtype=np.float16)
+    for r in range(rows):
+        mask[r, :cells - 7 + r] = 0.0
+        mask[r, 1:cells - 7 + r:5] = -0.75
+    sinks = g.standard_normal(heads).astype(np.float32)
+    scale, softcap = 0.125, 3.0
+
+    def numpy_attention(use_mask, use_sinks, cap):
+        out = np.zeros((rows, heads, d))
+        for h in range(heads):
+            kh = h // (heads // kv_heads)
+            for r in range(rows):
+                s = (kd[:, kh, :] @ q[h, r].astype(np.float64)) * scale
+                if cap > 0:
+                    s = cap * np.tanh(s / cap)
+                if use_mask:
+                    s = s + mask[r].astype(np.float64)
+                m = max(s.max(), float(sinks[h])) if use_sinks else s.max()
+                e = np.exp(s - m)
+                total = e.sum() + (np.exp(float(sinks[h]) - m) if use_sinks else 0.0)
+                out[r, h] = (e / total) @ vd[:, kh, :]
+        return out
+
+    for use_mask, use_sinks, cap in ((True, False, 0.0), (True, True, softcap), (False, False, softcap)):
+        got = oracle.attention_quant(t, q, k_cache, v_cache, d, heads, kv_heads, rows, cells, scale,
+                                     mask=mask if use_mask else None, sinks=sinks if use_sinks else None, softcap=cap,
+                                     cell_stride=pitch, head_stride=row_bytes)
+        np.testing.assert_allclose(got, numpy_attention(use_mask, use_sinks, cap), rtol=2e-6, atol=2e-7)
+    # Equal keys: every seen cell weighs the same, the output is the mean of the seen values.
+    same = np.repeat(k_cache[:1], cells, axis=0)
+    got = oracle.attention_quant(t, q, same, v_cache, d, heads, kv_heads, rows, cells, scale, mask=mask,
+                                 cell_stride=pitch, head_stride=row_bytes)
+    for r in range(rows):
+        seen = np.isfinite(mask[r].astype(np.float64))
+        w = np.exp(mask[r].astype(np.float64)[seen])
+        want = (w / w.sum()) @ vd[seen][:, 0, :]
+        np.testing.assert_allclose(got[r, 0], want, rtol=2e-6, atol=2e-7)
+    # One seen cell: its value row, whatever the scores; none: zeros; a huge sink: nearly nothing.
+    one = np.full((rows, cells), -np.inf, dtype=np.float16)
+    one[:, 5] = 0.0
+    one[2, :] = -np.inf
+    got = oracle.attention_quant(t, q, k_cache, v_cache, d, heads, kv_heads, rows, cells, scale, mask=one,
+                                 cell_stride=pitch, head_stride=row_bytes)
+    np.testing.assert_allclose(got[0, 4], vd[5, 1], rtol=1e-6, atol=1e-7)
+    assert np.all(got[2] == 0.0)
+    big = oracle.attention_quant(t, q, k_cache, v_cache, d, heads, kv_heads, rows, cells, scale, mask=mask,
+                                 sinks=np.full(heads, 80.0, dtype=np.float32), cell_stride=pitch, head_stride=row_bytes)
+    assert np.abs(big).max() < 1e-20
+    # Through Q8_1: the same attention over the decoded quantized queries.
+    blocks = oracle.q8_1_quantize(q.reshape(heads * rows, d))
+    q8 = np.stack([oracle.q8_1_decode(row, d) for row in blocks]).reshape(heads, rows, d)
+    a = oracle.attention_quant(t, q, k_cache, v_cache, d, heads, kv_heads, rows, cells, scale, mask=mask, q8_1_q=True,
+                               cell_stride=pitch, head_stride=row_bytes)
+    b = oracle.attention_quant(t, q8, k_cache, v_cache, d, heads, kv_heads, rows, cells, scale, mask=mask,
+                               cell_stride=pitch, head_stride=row_bytes)
+    assert np.array_equal(a, b)
