@@ -73,13 +73,21 @@ __device__ __forceinline__ void AttnFor(F&& f) {
 
 // `bytes` a lane from `from` (a lane's own address) to LDS at `to` + bytes * lane, no register between. In flight
 // until the wave's vmcnt says otherwise.
+// `base` the same in every lane (scalar registers), `offset` a lane's own.
 template <int BYTES, int OFFSET>
-__device__ __forceinline__ void ToLds(const uint8_t* from, uint32_t to) {
+__device__ __forceinline__ void ToLds(const uint8_t* base, uint32_t offset, uint32_t to) {
   if constexpr (BYTES == 16) {
-    asm volatile("s_add_u32 m0, %0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(to), "v"(from), "n"(OFFSET) : "memory", "scc");
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(to), "v"(offset), "s"(base), "n"(OFFSET) : "memory", "scc");
   } else {
-    asm volatile("s_add_u32 m0, %0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(to), "v"(from), "n"(OFFSET) : "memory", "scc");
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(to), "v"(offset), "s"(base), "n"(OFFSET) : "memory", "scc");
   }
+}
+// The same pointer known to the compiler as the same in every lane.
+__device__ __forceinline__ const uint8_t* UniformPointer(const uint8_t* p) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
 template <int LEFT>
@@ -94,19 +102,34 @@ struct AttnArgs {
   int splits, split_cells, group, rows_a_pass;
 };
 
+// Over a wave's 64 lanes, the same in every lane: within a row of 16 lanes by data-parallel moves (lane ^ 1, lane ^ 2,
+// the mirrored half row, the mirrored row), across the four rows by lane reads; no permute through LDS.
+template <int CONTROL>
+__device__ __forceinline__ float Dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CONTROL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float LaneValue(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float WaveMax(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  v = fmaxf(v, Dpp<0xB1>(v));
+  v = fmaxf(v, Dpp<0x4E>(v));
+  v = fmaxf(v, Dpp<0x141>(v));
+  v = fmaxf(v, Dpp<0x140>(v));
+  return fmaxf(fmaxf(LaneValue(v, 0), LaneValue(v, 16)), fmaxf(LaneValue(v, 32), LaneValue(v, 48)));
 }
 __device__ __forceinline__ float WaveSum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  v += Dpp<0xB1>(v);
+  v += Dpp<0x4E>(v);
+  v += Dpp<0x141>(v);
+  v += Dpp<0x140>(v);
+  return (LaneValue(v, 0) + LaneValue(v, 16)) + (LaneValue(v, 32) + LaneValue(v, 48));
 }
 
 // grid (splits, KV heads, passes of rows); 256 threads.
-template <int TYPE, int D>
+// NQ: the queries the loops are unrolled for, at least the pass's; those beyond it multiply images of zeros and are
+// never written out.
+template <int TYPE, int D, int NQ>
 __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const AttnArgs a) {
   using G = AttnGeo<TYPE, D>;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -119,34 +142,6 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   const int rows_here = min(a.rows_a_pass, d.rows - row0);
   const int nq = a.group * rows_here;  // query q: head kv_head * group + q / rows_here, row row0 + q % rows_here
 
-  // ---- the queries: Q8_1 blocks (eight lanes a block), laid out as images of a K row.
-  for (int i = tid; i < G::kQueries / 4; i += kAttnThreads) reinterpret_cast<uint32_t*>(lds)[i] = 0;
-  __syncthreads();
-  for (int b = tid >> 3; b < nq * G::kBlocks; b += kAttnThreads >> 3) {  // whole 8-lane groups together
-    const int q = b / G::kBlocks, blk = b - q * G::kBlocks;
-    const int head = kv_head * a.group + q / rows_here, row = row0 + q % rows_here;
-    const float* src = static_cast<const float*>(d.q) + head * d.q_head_stride + row * d.q_row_stride + blk * 32 + (tid & 7) * 4;
-    const float4 x = *reinterpret_cast<const float4*>(src);
-    const Q8Block packed = QuantizeQ8Block(x.x, x.y, x.z, x.w);
-    uint8_t* mine = lds + q * G::kQuery;
-    const int lane8 = tid & 7;
-    // Values 4 lane8 .. + 3 of the block: against the row's codes (Q4_0: the low nibbles hold values 0 to 15, the
-    // high ones 16 to 31 of the same bytes).
-    const int at = G::kQ8 ? blk * G::kBlock + 2 + 4 * lane8 : (lane8 >> 2) * G::kRow + blk * G::kBlock + 2 + 4 * (lane8 & 3);
-    *reinterpret_cast<uint16_t*>(mine + at) = static_cast<uint16_t>(packed.codes);
-    *reinterpret_cast<uint16_t*>(mine + at + 2) = static_cast<uint16_t>(packed.codes >> 16);
-    int total = Dot4(0x01010101, static_cast<int>(packed.codes), 0);
-    total += ShflXor(total, 1);
-    total += ShflXor(total, 2);
-    total += ShflXor(total, 4);
-    if (lane8 == 0) {
-      float* scales = reinterpret_cast<float*>(mine + G::kImage);
-      scales[blk] = HalfBitsToFloat(FloatToHalfBits(packed.d));  // the scale as a Q8_1 block stores it
-      scales[G::kBlocks + blk] = static_cast<float>(total);
-    }
-  }
-  __syncthreads();
-
   // ---- this wave's tiles of the split.
   const uint32_t lds_at = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)));
   uint8_t* const mine = lds + G::kQueries + wave * G::kWaveBytes;
@@ -156,16 +151,23 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   float* const probs = reinterpret_cast<float*>(mine + 2 * G::kTileBytes);  // [query][cell of the tile]
   const int cell_first = split * a.split_cells;
   const int tiles = min(a.split_cells, d.cells - cell_first) / G::kTile;
-  // A lane's piece of every load: piece p = 64 i + lane of a tile is row p / (pieces a row), piece p % (...).
+  // A lane's piece of every load: piece p = 64 i + lane of a tile is row p / (pieces a row), piece p % (...): where
+  // it lies from the tile's first row is the same for every tile (a register a load; the tile's place is scalar).
   constexpr int kPieces = G::kRow / G::kPiece;
-  auto fetch = [&](const void* base, int64_t cell_stride, int64_t head_stride, int tile, uint32_t to) {
-    const uint8_t* from = static_cast<const uint8_t*>(base) + kv_head * head_stride;
+  uint32_t k_from[G::kLoads], v_from[G::kLoads];
+#pragma unroll
+  for (int i = 0; i < G::kLoads; ++i) {
+    const int p = i * kWave + lane;
+    const int r = p / kPieces, c = p - r * kPieces;
+    k_from[i] = static_cast<uint32_t>(r * d.k_cell_stride + c * G::kPiece);
+    v_from[i] = static_cast<uint32_t>(r * d.v_cell_stride + c * G::kPiece);
+  }
+  auto fetch = [&](const void* base, int64_t cell_stride, int64_t head_stride, const uint32_t (&from)[G::kLoads], int tile, uint32_t to) {
     const int cell0 = cell_first + tile * G::kTile;
+    const uint8_t* first = UniformPointer(static_cast<const uint8_t*>(base) + kv_head * head_stride + cell0 * cell_stride);
     AttnFor<G::kLoads>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      const int p = i * kWave + lane;
-      const int r = p / kPieces, c = p - r * kPieces;
-      ToLds<G::kPiece, i * kWave * G::kPiece>(from + (cell0 + r) * cell_stride + c * G::kPiece, to);
+      ToLds<G::kPiece, i * kWave * G::kPiece>(first, from[i], to);
     });
   };
 
@@ -174,20 +176,83 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   const uint32_t mask_at = mine_at + 2 * G::kTileBytes + kMostQueries * G::kTile * 4;
   const uint16_t* const mask_tile = reinterpret_cast<const uint16_t*>(mine + 2 * G::kTileBytes + kMostQueries * G::kTile * 4);
   auto fetch_keys = [&](int tile) {
-    fetch(d.k, d.k_cell_stride, d.k_head_stride, tile, mine_at);
+    fetch(d.k, d.k_cell_stride, d.k_head_stride, k_from, tile, mine_at);
     const int cell0 = cell_first + tile * G::kTile;
     AttnFor<kMostQueries>([&](auto rc) {
       constexpr int r = decltype(rc)::value;
       const int row = row0 + min(r, rows_here - 1);
-      if (lane < G::kTile / 2)
-        ToLds<4, r * G::kTile * 2>(
-            reinterpret_cast<const uint8_t*>(static_cast<const uint16_t*>(d.mask) + row * d.mask_row_stride + cell0 + 2 * lane), mask_at);
+      const uint8_t* first = UniformPointer(reinterpret_cast<const uint8_t*>(static_cast<const uint16_t*>(d.mask) + row * d.mask_row_stride + cell0));
+      if (lane < G::kTile / 2) ToLds<4, r * G::kTile * 2>(first, static_cast<uint32_t>(4 * lane), mask_at);
     });
   };
 
-  float top[kMostQueries], sum[kMostQueries], corr[kMostQueries], acc[kMostQueries][G::kPer];
+  // The queries' loads first, then the wave's first tiles, then the staging: the loads are written as instructions
+  // and waited for by count (they are older than the tiles' loads), so that the tiles are on their way while the
+  // queries are quantized.
+  typedef float F4 __attribute__((ext_vector_type(4)));
+  constexpr int kGroups = kAttnThreads >> 3;                                         // 8-lane groups, a block each a sweep
+  constexpr int kSweeps = (kMostQueries * G::kBlocks + kGroups - 1) / kGroups;
+  F4 held[kSweeps];
 #pragma unroll
-  for (int q = 0; q < kMostQueries; ++q) {
+  for (int i = 0; i < kSweeps; ++i) {
+    const int b = (tid >> 3) + i * kGroups;
+    held[i] = F4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (b < nq * G::kBlocks) {
+      const int q = b / G::kBlocks, blk = b - q * G::kBlocks;
+      const int head = kv_head * a.group + q / rows_here, row = row0 + q % rows_here;
+      const float* src = static_cast<const float*>(d.q) + head * d.q_head_stride + row * d.q_row_stride + blk * 32 + (tid & 7) * 4;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(held[i]) : "v"(src) : "memory");
+    }
+  }
+  for (int i = tid; i < G::kQueries / 4; i += kAttnThreads) reinterpret_cast<uint32_t*>(lds)[i] = 0;
+  if (wave < tiles) {
+    fetch_keys(wave);
+    fetch(d.v, d.v_cell_stride, d.v_head_stride, v_from, wave, mine_at + G::kTileBytes);
+  }
+  // The queries have landed once no more than the tiles' loads are outstanding (the registers are tied to the wait).
+  if (wave < tiles) {
+    if constexpr (kSweeps == 1) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(held[0]) : "n"(G::kLoadsWithMask + G::kLoads));
+    if constexpr (kSweeps == 2) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(held[0]), "+v"(held[1]) : "n"(G::kLoadsWithMask + G::kLoads));
+    if constexpr (kSweeps == 4)
+      asm volatile("s_waitcnt vmcnt(%4)" : "+v"(held[0]), "+v"(held[1]), "+v"(held[2]), "+v"(held[3]) : "n"(G::kLoadsWithMask + G::kLoads));
+  } else {
+    if constexpr (kSweeps == 1) asm volatile("s_waitcnt vmcnt(0)" : "+v"(held[0]));
+    if constexpr (kSweeps == 2) asm volatile("s_waitcnt vmcnt(0)" : "+v"(held[0]), "+v"(held[1]));
+    if constexpr (kSweeps == 4) asm volatile("s_waitcnt vmcnt(0)" : "+v"(held[0]), "+v"(held[1]), "+v"(held[2]), "+v"(held[3]));
+  }
+  static_assert(kSweeps == 1 || kSweeps == 2 || kSweeps == 4, "the sweeps the waits are written for");
+  __syncthreads();  // the images are zero
+
+  // ---- the queries: Q8_1 blocks (eight lanes a block), laid out as images of a K row.
+#pragma unroll
+  for (int i = 0; i < kSweeps; ++i) {
+    const int b = (tid >> 3) + i * kGroups;
+    if (b < nq * G::kBlocks) {  // whole 8-lane groups together
+      const int q = b / G::kBlocks, blk = b - q * G::kBlocks;
+      const Q8Block packed = QuantizeQ8Block(held[i].x, held[i].y, held[i].z, held[i].w);
+      uint8_t* image = lds + q * G::kQuery;
+      const int lane8 = tid & 7;
+      // Values 4 lane8 .. + 3 of the block: against the row's codes (Q4_0: the low nibbles hold values 0 to 15, the
+      // high ones 16 to 31 of the same bytes).
+      const int at = G::kQ8 ? blk * G::kBlock + 2 + 4 * lane8 : (lane8 >> 2) * G::kRow + blk * G::kBlock + 2 + 4 * (lane8 & 3);
+      *reinterpret_cast<uint16_t*>(image + at) = static_cast<uint16_t>(packed.codes);
+      *reinterpret_cast<uint16_t*>(image + at + 2) = static_cast<uint16_t>(packed.codes >> 16);
+      int total = Dot4(0x01010101, static_cast<int>(packed.codes), 0);
+      total += ShflXor(total, 1);
+      total += ShflXor(total, 2);
+      total += ShflXor(total, 4);
+      if (lane8 == 0) {
+        float* scales = reinterpret_cast<float*>(image + G::kImage);
+        scales[blk] = HalfBitsToFloat(FloatToHalfBits(packed.d));  // the scale as a Q8_1 block stores it
+        scales[G::kBlocks + blk] = static_cast<float>(total);
+      }
+    }
+  }
+  __syncthreads();
+
+  float top[NQ], sum[NQ], corr[NQ], acc[NQ][G::kPer];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
     top[q] = -INFINITY;
     sum[q] = 0.0f;
     corr[q] = 0.0f;
@@ -202,37 +267,56 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   const int v_codes_at = v_scale_at + 2 + (G::kQ8 ? v_in : v_in % 16);
   const int v_shift = G::kQ8 ? 0 : (v_in / 16) * 4;
 
-  if (wave < tiles) {
-    fetch_keys(wave);
-    fetch(d.v, d.v_cell_stride, d.v_head_stride, wave, mine_at + G::kTileBytes);
-  }
   for (int tile = wave; tile < tiles; tile += kAttnWaves) {
     AwaitAllBut<G::kLoads>();  // K and the mask have landed, V may be on its way
     __builtin_amdgcn_wave_barrier();
     // The mask's values into registers: their place is refilled before they are used.
-    float bias[kMostQueries];
+    float bias[NQ];
 #pragma unroll
-    for (int q = 0; q < kMostQueries; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       bias[q] = 0.0f;
-      if (q < nq && lane < G::kTile) bias[q] = HalfBitsToFloat(mask_tile[(q % rows_here) * G::kTile + lane]);
+      if (lane < G::kTile) bias[q] = HalfBitsToFloat(mask_tile[(q % rows_here) * G::kTile + lane]);
     }
     // ---- scores: a lane a cell.
-    float score[kMostQueries];
-    int part[kMostQueries];
+    float score[NQ];
+    int part[NQ];
 #pragma unroll
-    for (int q = 0; q < kMostQueries; ++q) score[q] = 0.0f, part[q] = 0;
+    for (int q = 0; q < NQ; ++q) score[q] = 0.0f, part[q] = 0;
     if (lane < G::kTile) {
       const uint8_t* row = k_tile + lane * G::kRow;
+      // One or two queries' images stay in registers from tile to tile (the compiler finds their reads the same in
+      // every iteration); more do not fit, so their place is hidden from it here and they are read again a tile.
+      uint32_t images_at = 0;
+      if constexpr (NQ > 2) asm volatile("" : "+v"(images_at));
+      const uint8_t* images = lds + images_at;
       uint32_t kd[G::kRead];
+      uint32_t low[NQ][G::kRead], high[G::kQ8 ? 1 : NQ][G::kRead];  // the images' dwords beside the row's
       float dk = 0.0f;
       AttnFor<G::kDwords>([&](auto wc) {
         constexpr int w = decltype(wc)::value;
+        // (The reads of LDS stay with their group of dwords: hoisted to the front of the unrolled row they take
+        // more registers than there are.)
+        if constexpr (w % (2 * G::kRead) == 0 && w > 0) __builtin_amdgcn_sched_barrier(0);
         if constexpr (w % G::kRead == 0) {
           if constexpr (G::kWide) {
             const uint4 x = *reinterpret_cast<const uint4*>(row + 4 * w);
             kd[0] = x.x, kd[1] = x.y, kd[2] = x.z, kd[3] = x.w;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+              const uint4 y = *reinterpret_cast<const uint4*>(images + q * G::kQuery + 4 * w);
+              low[q][0] = y.x, low[q][1] = y.y, low[q][2] = y.z, low[q][3] = y.w;
+              if constexpr (!G::kQ8) {
+                const uint4 z = *reinterpret_cast<const uint4*>(images + q * G::kQuery + G::kRow + 4 * w);
+                high[q][0] = z.x, high[q][1] = z.y, high[q][2] = z.z, high[q][3] = z.w;
+              }
+            }
           } else {
             kd[0] = *reinterpret_cast<const uint32_t*>(row + 4 * w);
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+              low[q][0] = *reinterpret_cast<const uint32_t*>(images + q * G::kQuery + 4 * w);
+              if constexpr (!G::kQ8) high[q][0] = *reinterpret_cast<const uint32_t*>(images + q * G::kQuery + G::kRow + 4 * w);
+            }
           }
         }
         const uint32_t x = kd[w % G::kRead];
@@ -240,25 +324,28 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
         // A scale in the dword's upper half is the next block's: it takes effect once this block's sum is scaled.
         if constexpr (G::HasScale(w) && G::ScaleBlock(w) == blk) dk = HalfBitsToFloat((x >> G::ScaleShift(w)) & 0xFFFFu);
 #pragma unroll
-        for (int q = 0; q < kMostQueries; ++q) {
-          if (q < nq) {
-            const uint8_t* image = lds + q * G::kQuery;
-            if constexpr (G::kQ8) {
-              part[q] = Dot4(static_cast<int>(x), *reinterpret_cast<const int*>(image + 4 * w), part[q]);
-            } else {
-              part[q] = Dot4(static_cast<int>(x & 0x0F0F0F0Fu), *reinterpret_cast<const int*>(image + 4 * w), part[q]);
-              part[q] = Dot4(static_cast<int>((x >> 4) & 0x0F0F0F0Fu), *reinterpret_cast<const int*>(image + G::kRow + 4 * w), part[q]);
-            }
-            if constexpr (G::LastOf(w)) {
-              const float* scales = reinterpret_cast<const float*>(image + G::kImage);
-              // Q4_0: values are codes minus 8, so eight times the query's code sum comes off.
-              const float whole = G::kQ8 ? static_cast<float>(part[q]) : static_cast<float>(part[q]) - 8.0f * scales[G::kBlocks + blk];
-              score[q] += (dk * scales[blk]) * whole;
-              part[q] = 0;
-            }
+        for (int q = 0; q < NQ; ++q) {
+          if constexpr (G::kQ8) {
+            part[q] = Dot4(static_cast<int>(x), static_cast<int>(low[q][w % G::kRead]), part[q]);
+          } else {
+            part[q] = Dot4(static_cast<int>(x & 0x0F0F0F0Fu), static_cast<int>(low[q][w % G::kRead]), part[q]);
+            part[q] = Dot4(static_cast<int>((x >> 4) & 0x0F0F0F0Fu), static_cast<int>(high[q][w % G::kRead]), part[q]);
+          }
+          if constexpr (G::LastOf(w)) {
+            const float* scales = reinterpret_cast<const float*>(images + q * G::kQuery + G::kImage);
+            // Q4_0: values are codes minus 8, so eight times the query's code sum comes off.
+            const float whole = G::kQ8 ? static_cast<float>(part[q]) : static_cast<float>(part[q]) - 8.0f * scales[G::kBlocks + blk];
+            score[q] += (dk * scales[blk]) * whole;
+            part[q] = 0;
           }
         }
         if constexpr (G::HasScale(w) && G::ScaleBlock(w) != blk) dk = HalfBitsToFloat((x >> G::ScaleShift(w)) & 0xFFFFu);
+        // The sums are taken where they are computed: pure as they are, the compiler otherwise moves every product
+        // to the row's end and keeps all the row's and images' dwords until then.
+        if constexpr ((w + 1) % G::kRead == 0 || w + 1 == G::kDwords) {
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) asm volatile("" : "+v"(part[q]), "+v"(score[q]));
+        }
       });
     }
     // K's buffer is free: the wave's next tile of K on its way.
@@ -268,21 +355,19 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
     if (next < tiles) fetch_keys(next);
     // ---- online softmax over the tile.
 #pragma unroll
-    for (int q = 0; q < kMostQueries; ++q) {
-      if (q < nq) {
-        float s = score[q] * d.scale;
-        if (capped) s = d.softcap * tanhf(s * cap_inverse);
-        s = lane < G::kTile ? s + bias[q] : -INFINITY;
-        const float peak = fmaxf(top[q], WaveMax(s));
-        const float p = peak == -INFINITY ? 0.0f : __expf(s - peak);
-        const float keep = peak == -INFINITY ? 1.0f : __expf(top[q] - peak);  // exp(-inf) is 0: a first tile keeps nothing
-        sum[q] = sum[q] * keep + WaveSum(p);
-        corr[q] *= keep;
+    for (int q = 0; q < NQ; ++q) {
+      float s = score[q] * d.scale;
+      if (capped) s = d.softcap * tanhf(s * cap_inverse);
+      s = lane < G::kTile ? s + bias[q] : -INFINITY;
+      const float peak = fmaxf(top[q], WaveMax(s));
+      const float p = peak == -INFINITY ? 0.0f : __expf(s - peak);
+      const float keep = peak == -INFINITY ? 1.0f : __expf(top[q] - peak);  // exp(-inf) is 0: a first tile keeps nothing
+      sum[q] = sum[q] * keep + WaveSum(p);
+      corr[q] *= keep;
 #pragma unroll
-        for (int j = 0; j < G::kPer; ++j) acc[q][j] *= keep;
-        top[q] = peak;
-        if (lane < G::kTile) probs[q * G::kTile + lane] = p;
-      }
+      for (int j = 0; j < G::kPer; ++j) acc[q][j] *= keep;
+      top[q] = peak;
+      if (lane < G::kTile) probs[q * G::kTile + lane] = p;
     }
     if (next < tiles) {
       AwaitAllBut<G::kLoadsWithMask>();  // V has landed (the next K and mask may be on their way)
@@ -291,30 +376,35 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
     }
     __builtin_amdgcn_wave_barrier();
     // ---- values: a lane kPer consecutive values of every row of the tile.
-#pragma unroll 2
-    for (int c = 0; c < G::kTile; ++c) {
-      const uint8_t* row = v_tile + c * G::kRow;
-      const float dv = HalfBitsToFloat(*reinterpret_cast<const uint16_t*>(row + v_scale_at));
-      float value[G::kPer];
-      if constexpr (G::kPer == 1) {
-        const uint32_t byte = row[v_codes_at];
-        value[0] = G::kQ8 ? static_cast<float>(byte ^ 0x80u) : static_cast<float>((byte >> v_shift) & 0xFu);
-      } else {
+#pragma unroll 1
+    for (int c4 = 0; c4 < G::kTile; c4 += 4) {
+      float4 four_probs[NQ];  // the probabilities of four cells, broadcast
 #pragma unroll
-        for (int j = 0; j < G::kPer; j += 4) {
-          uint32_t four = *reinterpret_cast<const uint16_t*>(row + v_codes_at + j) |
-                          (static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(row + v_codes_at + j + 2)) << 16);
-          four = G::kQ8 ? four ^ 0x80808080u : (four >> v_shift) & 0x0F0F0F0Fu;
-          value[j] = static_cast<float>(four & 0xFFu);
-          value[j + 1] = static_cast<float>((four >> 8) & 0xFFu);
-          value[j + 2] = static_cast<float>((four >> 16) & 0xFFu);
-          value[j + 3] = static_cast<float>(four >> 24);
+      for (int q = 0; q < NQ; ++q) four_probs[q] = *reinterpret_cast<const float4*>(probs + q * G::kTile + c4);
+#pragma unroll
+      for (int cc = 0; cc < 4; ++cc) {
+        const uint8_t* row = v_tile + (c4 + cc) * G::kRow;
+        const float dv = HalfBitsToFloat(*reinterpret_cast<const uint16_t*>(row + v_scale_at));
+        float value[G::kPer];
+        if constexpr (G::kPer == 1) {
+          const uint32_t byte = row[v_codes_at];
+          value[0] = G::kQ8 ? static_cast<float>(byte ^ 0x80u) : static_cast<float>((byte >> v_shift) & 0xFu);
+        } else {
+#pragma unroll
+          for (int j = 0; j < G::kPer; j += 4) {
+            uint32_t four = *reinterpret_cast<const uint16_t*>(row + v_codes_at + j) |
+                            (static_cast<uint32_t>(*reinterpret_cast<const uint16_t*>(row + v_codes_at + j + 2)) << 16);
+            four = G::kQ8 ? four ^ 0x80808080u : (four >> v_shift) & 0x0F0F0F0Fu;
+            value[j] = static_cast<float>(four & 0xFFu);
+            value[j + 1] = static_cast<float>((four >> 8) & 0xFFu);
+            value[j + 2] = static_cast<float>((four >> 16) & 0xFFu);
+            value[j + 3] = static_cast<float>(four >> 24);
+          }
         }
-      }
 #pragma unroll
-      for (int q = 0; q < kMostQueries; ++q) {
-        if (q < nq) {
-          const float weight = probs[q * G::kTile + c] * dv;
+        for (int q = 0; q < NQ; ++q) {
+          const float p = cc == 0 ? four_probs[q].x : cc == 1 ? four_probs[q].y : cc == 2 ? four_probs[q].z : four_probs[q].w;
+          const float weight = p * dv;
           corr[q] += weight;
 #pragma unroll
           for (int j = 0; j < G::kPer; ++j) acc[q][j] = fmaf(weight, value[j], acc[q][j]);
@@ -323,7 +413,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
     }
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-    if (next < tiles) fetch(d.v, d.v_cell_stride, d.v_head_stride, next, mine_at + G::kTileBytes);
+    if (next < tiles) fetch(d.v, d.v_cell_stride, d.v_head_stride, v_from, next, mine_at + G::kTileBytes);
   }
   AwaitAllBut<0>();
   __syncthreads();
@@ -332,7 +422,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   constexpr float kOffset = G::kQ8 ? 128.0f : 8.0f;
   float* const meet = reinterpret_cast<float*>(lds + G::kQueries);  // [wave][query][D + 2]
 #pragma unroll
-  for (int q = 0; q < kMostQueries; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     if (q < nq) {
       float* out = meet + (wave * kMostQueries + q) * (D + 2);
       if (lane == 0) out[0] = top[q], out[1] = sum[q];
@@ -361,21 +451,26 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
   }
 }
 
-// grid (heads, rows); D threads: the splits' partial results into one row of the output.
+// grid (heads, rows); D threads: the splits' partial results into one row of the output. The splits' maxima and sums
+// through LDS (a thread a split), then every thread its value over the splits, eight loads at a time.
+constexpr int kMostSplits = 512;
 template <int D>
 __global__ __launch_bounds__(D) void AttnCombineKernel(const AttnArgs a) {
+  __shared__ float peaks[kMostSplits], totals[kMostSplits];
   const llmp_attn_vec_quant& d = a.d;
   const int head = blockIdx.x, row = blockIdx.y, j = threadIdx.x;
   const float* from = a.partial + (static_cast<int64_t>(row) * d.heads + head) * a.splits * (D + 2);
+  for (int s = j; s < a.splits; s += D) peaks[s] = from[s * (D + 2)], totals[s] = from[s * (D + 2) + 1];
+  __syncthreads();
   const bool sunk = d.sinks != nullptr;
   float peak = sunk ? static_cast<const float*>(d.sinks)[head] : -INFINITY;
-  for (int s = 0; s < a.splits; ++s) peak = fmaxf(peak, from[s * (D + 2)]);
+  for (int s = 0; s < a.splits; ++s) peak = fmaxf(peak, peaks[s]);
   float total = sunk ? __expf(static_cast<const float*>(d.sinks)[head] - peak) : 0.0f, value = 0.0f;
+#pragma unroll 8
   for (int s = 0; s < a.splits; ++s) {
-    const float* part = from + s * (D + 2);
-    const float keep = part[0] == -INFINITY ? 0.0f : __expf(part[0] - peak);
-    total += part[1] * keep;
-    value += part[2 + j] * keep;
+    const float keep = peaks[s] == -INFINITY ? 0.0f : __expf(peaks[s] - peak);
+    total += totals[s] * keep;
+    value += from[s * (D + 2) + 2 + j] * keep;
   }
   // A row that sees nothing (and has no sink) is zero, as the reference's SoftmaxRow has it.
   static_cast<float*>(d.out)[(static_cast<int64_t>(row) * d.heads + head) * D + j] =
@@ -386,13 +481,27 @@ struct AttnPlan {
   int group, rows_a_pass, passes, splits, split_cells;
 };
 
-template <int TYPE, int D>
-void LaunchAttn(const AttnArgs& args, const AttnPlan& plan, hipStream_t stream) {
+template <int TYPE, int D, int NQ>
+void LaunchAttnFor(const AttnArgs& args, const AttnPlan& plan, hipStream_t stream) {
   using G = AttnGeo<TYPE, D>;
   static bool sized = false;
-  if (!AllowLds(reinterpret_cast<const void*>(&AttnVecQuantKernel<TYPE, D>), G::kLds, &sized)) return;
+  if (!AllowLds(reinterpret_cast<const void*>(&AttnVecQuantKernel<TYPE, D, NQ>), G::kLds, &sized)) return;
   const dim3 grid(static_cast<unsigned>(plan.splits), static_cast<unsigned>(args.d.kv_heads), static_cast<unsigned>(plan.passes));
-  hipLaunchKernelGGL((AttnVecQuantKernel<TYPE, D>), grid, dim3(kAttnThreads), G::kLds, stream, args);
+  hipLaunchKernelGGL((AttnVecQuantKernel<TYPE, D, NQ>), grid, dim3(kAttnThreads), G::kLds, stream, args);
+}
+
+template <int TYPE, int D>
+void LaunchAttn(const AttnArgs& args, const AttnPlan& plan, hipStream_t stream) {
+  const int queries = plan.group * plan.rows_a_pass;  // of a full pass
+  if (queries <= 1) {
+    LaunchAttnFor<TYPE, D, 1>(args, plan, stream);
+  } else if (queries <= 2) {
+    LaunchAttnFor<TYPE, D, 2>(args, plan, stream);
+  } else if (queries <= 4) {
+    LaunchAttnFor<TYPE, D, 4>(args, plan, stream);
+  } else {
+    LaunchAttnFor<TYPE, D, 8>(args, plan, stream);
+  }
   hipLaunchKernelGGL((AttnCombineKernel<D>), dim3(static_cast<unsigned>(args.d.heads), static_cast<unsigned>(args.d.rows)), dim3(D), 0,
                      stream, args);
 }
@@ -445,6 +554,7 @@ int PlanAttn(const llmp_attn_vec_quant* op, int cus, AttnPlan* plan) {
   int splits = (2 * (cus > 0 ? cus : 256) + others - 1) / others;
   const int most = (tiles + kAttnWaves - 1) / kAttnWaves;
   if (splits > most) splits = most;
+  if (splits > kMostSplits) splits = kMostSplits;
   if (splits < 1) splits = 1;
   const int tiles_a_split = (tiles + splits - 1) / splits;
   plan->split_cells = tiles_a_split * tile;
