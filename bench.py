@@ -237,7 +237,22 @@ def other_configs(device, args, only=None):
                                         glu=oracle.GLU_GEGLU, threads=threads),
                     WEIGHT_BYTES / 1e9, "GB/s", 2.0, f"the whole gate/up pair at {tokens} tokens", threads)
             out[name] = entry
+            # The same over weights relaid out at import into 64-row tiles (lossless; the kernel's reads become whole
+            # 64-byte units): beside the reference's layout, not in place of it.
+            tiled_name = name + "_tiles64"
+            tiled_variant = ops.vecq_variants().index("rows pass8 tiles64")
+            if only is None or only in (name, tiled_name):
+                if "gates_tiled" not in locals():
+                    gates_tiled = [ops.relayout_q4_k_tiles64(g_, N, K) for g_ in gates]
+                    ups_tiled = [ops.relayout_q4_k_tiles64(u_, N, K) for u_ in ups]
+                us_tiled = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, ups_tiled[i % count], q8, K, N, gate=gates_tiled[i % count],
+                                                    tokens=tokens, glu=ops.GLU_GEGLU, variant=tiled_variant, out=y), 4 * count)
+                out[tiled_name] = {"workload": f"config 2 at batch {tokens}, weights relaid out at import (llmp_hip_relayout_q4_k_tiles64)",
+                                   "roofline": hbm_roofline(tiled_name, "VecQRows<glu, %d tokens> over 64-row tiles" % (4 if tokens <= 4 else 8),
+                                                            algorithmic_bytes(tokens), us_tiled)}
         del gates, ups, gate, up
+        if "gates_tiled" in locals():
+            del gates_tiled, ups_tiled
         torch.cuda.empty_cache()
 
     # The same layer's down projection (15360 -> 3840, Q4_K, one token): rows of 60 super-blocks.

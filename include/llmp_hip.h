@@ -95,6 +95,17 @@ int llmp_hip_vecq(int type, const llmp_vecq_desc* d, int variant, void* stream);
 int llmp_hip_vecq_variants(void);
 const char* llmp_hip_vecq_variant_name(int variant);
 
+/* An import-time relayout for this device, lossless and undone by inverse != 0 (the reference does its
+ * platform-specific relayouts at import, src/import/expert_relayout.h:4-17: a table rewritten into the tile order
+ * its products read). Q4_K rows (nrows x blocks_per_row super-blocks, packed) in tiles of 64 rows: within a tile
+ * the blocks lie super-block after super-block, a super-block's 64 rows together, so that the 9216 bytes a wave of
+ * the row-a-lane product reads at a time are consecutive (over the reference's row-major blocks that read fetches
+ * 1.3 to 1.4 times its bytes: 144-byte pieces are ragged against HBM's 64-byte units). A 64-row tile covers the same
+ * bytes in both layouts, so a table of experts or matrices is relaid out in one call (nrows = all its rows) as long
+ * as every matrix is whole tiles. llmp_hip_vecq's variant "rows pass8 tiles64" reads the result; every other variant
+ * reads the reference's layout. src and dst at 16-byte boundaries, not overlapping. */
+int llmp_hip_relayout_q4_k_tiles64(const void* src, void* dst, int64_t nrows, int64_t blocks_per_row, int inverse, void* stream);
+
 /* The same product over unquantized activations: each workgroup quantizes the
  * tokens' rows to Q8_1 in LDS (the arithmetic of llmp_hip_q8_1_quantize, bit
  * for bit) instead of reading d->y, which is ignored. x_token / x_slot are

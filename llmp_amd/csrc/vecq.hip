@@ -495,6 +495,9 @@ constexpr Variant kVariants[] = {
     // Q4_K, a weight row a lane, 2 to 8 tokens of a dense or grouped product on the 4 x 4 x 4 int8 matrix
     // instruction (vecq_rows.hip); `lanes` -2 marks the form.
     {"rows pass8", -2, 8, 1},
+    // The same over weights relaid out at import into 64-row tiles (llmp_hip_relayout_q4_k_tiles64); `lanes` -3.
+    // Never a default: the layout is the caller's to declare.
+    {"rows pass8 tiles64", -3, 8, 1},
 };
 constexpr int kMmaVariant = 9;
 constexpr int kRowsVariant = 10;
@@ -655,6 +658,14 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (type != LLMP_TYPE_Q8_0 && type != LLMP_TYPE_Q4_K && v.lanes != 0)
     return Refuse(1, "vecq: the legacy 4/5-bit blocks, IQ4_NL, Q5_K, Q6_K and MXFP4 take the flat variants");
   if (offsets != nullptr && v.lanes > 0) return Refuse(1, "vecq: sorted rows take the flat or the matrix-core form");
+  if (v.lanes == -3) {
+    if (offsets != nullptr || x != nullptr || dump != nullptr || !RowsTiledTakes(type, *d))
+      return Refuse(1, "vecq: the row-a-lane form over relaid-out weights takes what the row-a-lane form takes, in whole tiles of "
+                       "64 packed rows");
+    a.tiled = 1;
+    LaunchRows(a, static_cast<hipStream_t>(stream));
+    return LaunchStatus("vecq");
+  }
   if (v.lanes == -2) {
     if (offsets != nullptr || !RowsTakes(type, *d))
       return Refuse(1, "vecq: the row-a-lane form takes 2 to 8 tokens of a dense or grouped Q4_K product, rows of 1024 values "

@@ -111,6 +111,9 @@ struct VecQArgs {
   // Sorted rows: expert e computes rows offsets[e] .. offsets[e + 1] of the activations into
   // the same rows of the output (d.ids unused), or null.
   const int32_t* offsets;
+  // The row-a-lane form over weights the importer relaid out (llmp_hip_relayout_q4_k_tiles64): within every 64
+  // rows the blocks lie super-block after super-block, a super-block's 64 rows together.
+  int tiled = 0;
 };
 
 __device__ __forceinline__ float Silu(float x) {
@@ -201,6 +204,7 @@ void LaunchMma(int type, const VecQArgs& a, hipStream_t stream);
 
 // The row-a-lane kernel for 2 to 8 tokens of a dense or grouped Q4_K product over Q8_1 activations (vecq_rows.hip).
 bool RowsTakes(int type, const llmp_vecq_desc& d);
+bool RowsTiledTakes(int type, const llmp_vecq_desc& d);
 void LaunchRows(const VecQArgs& a, hipStream_t stream);
 
 }  // namespace llmp_hip

@@ -291,8 +291,10 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     for (int j = 0; j < kPieceLoads; ++j) {
       const int byte = j * (kWave * 16) + lane * 16;
       const int row = byte / 144;
-      offsets[j] = static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
-                   static_cast<uint32_t>(byte - row * 144);
+      // (Relaid-out weights: a piece is 9216 consecutive bytes, every 64-byte unit of HBM asked for once.)
+      offsets[j] = a.tiled != 0 ? static_cast<uint32_t>(byte)
+                                : static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
+                                      static_cast<uint32_t>(byte - row * 144);
     }
     const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * 144;
     up_tile = static_cast<const uint8_t*>(d.w) + at;
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       gate = piece < paired ? (piece & 3) >> 1 : piece - paired;
       sb = sb_first + (piece < paired ? (piece >> 2) * 2 + (piece & 1) : sb_end - sb_first - 1);
     }
-    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * 144;
+    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * (a.tiled != 0 ? kPieceBytes : 144);
     uint8_t* to = ring + (i % STAGES) * kPieceBytes;
 #pragma unroll
     for (int j = 0; j < kPieceLoads; ++j)
@@ -444,6 +446,22 @@ void LaunchRowsStages(const VecQArgs& a, dim3 grid, hipStream_t stream) {
                                        : LaunchRowsKernel<kGlu, NT, 2>(a, grid, stream);
 }
 
+// 16 bytes a thread: block (row, sb) of the row-major matrix is block (sb, row % 64) of its 64-row tile.
+__global__ void RelayoutTiles64Kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t chunks, int nsb, int inverse) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= chunks) return;
+  const int64_t block = i / 9;
+  const int part = static_cast<int>(i - block * 9);
+  const int64_t row = block / nsb;
+  const int sb = static_cast<int>(block - row * nsb);
+  const int64_t tiled = ((row / kTileRows) * nsb + sb) * kTileRows + row % kTileRows;
+  if (inverse != 0) {
+    dst[block * 9 + part] = src[tiled * 9 + part];
+  } else {
+    dst[tiled * 9 + part] = src[block * 9 + part];
+  }
+}
+
 }  // namespace
 
 // Q4_K, 2 to 8 tokens of a dense or grouped product (no routing ids) over Q8_1 activations, rows of at
@@ -453,6 +471,12 @@ bool RowsTakes(int type, const llmp_vecq_desc& d) {
   const int nsb = d.ncols_x / 256;
   if (nsb < kRowsWaves) return false;
   return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
+}
+
+// The same over relaid-out weights: whole tiles of packed rows.
+bool RowsTiledTakes(int type, const llmp_vecq_desc& d) {
+  return RowsTakes(type, d) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
+         d.stride_expert % (kTileRows * (d.ncols_x / 256)) == 0;
 }
 
 void LaunchRows(const VecQArgs& a, hipStream_t stream) {
@@ -475,3 +499,19 @@ void LaunchRows(const VecQArgs& a, hipStream_t stream) {
 }
 
 }  // namespace llmp_hip
+
+extern "C" int llmp_hip_relayout_q4_k_tiles64(const void* src, void* dst, int64_t nrows, int64_t blocks_per_row, int inverse, void* stream) {
+  using namespace llmp_hip;
+  BeginLaunches();
+  if (src == nullptr || dst == nullptr || src == dst) return Refuse(1, "relayout: null operands, or in place");
+  if (nrows < 1 || nrows % kTileRows != 0 || blocks_per_row < 1 || blocks_per_row > INT32_MAX)
+    return Refuse(1, "relayout: rows in whole tiles of %d and at least a block a row, not %lld x %lld", kTileRows, (long long)nrows, (long long)blocks_per_row);
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16 != 0) return Refuse(1, "relayout: operands at 16-byte boundaries");
+  const uintptr_t a = reinterpret_cast<uintptr_t>(src), b = reinterpret_cast<uintptr_t>(dst);
+  const uint64_t bytes = static_cast<uint64_t>(nrows) * static_cast<uint64_t>(blocks_per_row) * 144u;
+  if (a < b + bytes && b < a + bytes) return Refuse(1, "relayout: the source and the destination overlap");
+  const int64_t chunks = static_cast<int64_t>(bytes / 16);
+  hipLaunchKernelGGL(RelayoutTiles64Kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), chunks, static_cast<int>(blocks_per_row), inverse);
+  return LaunchStatus("relayout");
+}

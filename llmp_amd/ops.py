@@ -109,6 +109,15 @@ def vecq_block_sums(t, w, q8, k, nrows, variant=-1):
     return sums
 
 
+def relayout_q4_k_tiles64(w, nrows, k, inverse=False):
+    """The import-time relayout the variant "rows pass8 tiles64" reads: uint8 Q4_K rows (nrows x k / 256 super-blocks,
+    packed) into 64-row tiles, a super-block's 64 rows together; inverse=True undoes it. Returns a new tensor."""
+    lib = _lib.load()
+    out = torch.empty_like(w)
+    _lib.check(lib.llmp_hip_relayout_q4_k_tiles64(_ptr(w), _ptr(out), nrows, k // 256, int(inverse), _stream()))
+    return out
+
+
 def vecq_variants():
     lib = _lib.load()
     return [lib.llmp_hip_vecq_variant_name(i).decode() for i in range(lib.llmp_hip_vecq_variants())]

@@ -102,7 +102,8 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
-        if name.startswith("rows") and t != Q4_K:  # the row-a-lane form is Q4_K's alone
+        if name.startswith("rows") and (t != Q4_K or name.endswith("tiles64")):
+            # the row-a-lane form is Q4_K's alone, and its relaid-out variant takes whole tiles of 64 rows
             with pytest.raises(ops.KernelFailure):
                 ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
             continue
@@ -718,3 +719,40 @@ def test_mxfp4_refuses_what_the_streaming_form_does_not_take(device):
         ops.vecq(MXFP4, dev(w, device), dev(q8, device), k, n)
     with pytest.raises(ops.KernelFailure):  # the rows form has no MXFP4
         ops.vecq(MXFP4, dev(synth.mxfp4_weights(n, 512, 533), device), dev(q8, device), 512, n, variant=0)
+
+
+@pytest.mark.parametrize("tokens,glu", [(2, ops.GLU_NONE), (4, ops.GLU_GEGLU), (8, ops.GLU_SWIGLU)])
+def test_relaid_out_rows_equal_the_row_a_lane_form_bit_for_bit(device, tokens, glu):
+    """llmp_hip_relayout_q4_k_tiles64 permutes whole blocks inside 64-row tiles and its inverse puts them back; the
+    variant that reads the result multiplies the same blocks with the same arithmetic as the row-a-lane form over the
+    reference's layout: equal bits, and the oracle's values. Dense and grouped (two matrices, two input rows)."""
+    k, n, used = 1280, 192, 2
+    names = ops.vecq_variants()
+    rows_variant, tiled_variant = names.index("rows pass8"), names.index("rows pass8 tiles64")
+    up = make_weights(Q4_K, used * n, k, 301)
+    gate = make_weights(Q4_K, used * n, k, 302) if glu != ops.GLU_NONE else None
+    q8 = oracle.q8_1_quantize(synth.activations(tokens * used, k, 303))
+    ud, qd = dev(up, device), dev(q8, device)
+    gd = dev(gate, device) if gate is not None else None
+    ut = ops.relayout_q4_k_tiles64(ud, used * n, k)
+    gt = ops.relayout_q4_k_tiles64(gd, used * n, k) if gd is not None else None
+    assert not torch.equal(ut, ud)
+    assert torch.equal(ops.relayout_q4_k_tiles64(ut, used * n, k, inverse=True), ud)
+    # What the layout is: block (row, sb) at block (sb, row % 64) of its tile.
+    nsb = k // 256
+    native, tiled = up.reshape(-1, nsb, 144), ut.cpu().numpy().reshape(-1, nsb, 64, 144)
+    for row, sb in ((0, 0), (63, nsb - 1), (64, 1), (used * n - 1, 2)):
+        assert np.array_equal(tiled[row // 64, sb, row % 64], native[row, sb])
+    blocks = oracle.padded_k(k) // 32
+    common = dict(tokens=tokens, used=used, stride_expert=n * nsb, y_token=blocks * used, y_slot=blocks, glu=glu)
+    want = ops.vecq(Q4_K, ud, qd, k, n, gate=gd, variant=rows_variant, **common)
+    got = ops.vecq(Q4_K, ut, qd, k, n, gate=gt, variant=tiled_variant, **common)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    ref = oracle.vecq(Q4_K, up, q8, k, n, gate=gate, tokens=tokens, used=used, stride_expert=n * nsb, y_token=blocks * used,
+                      y_slot=blocks, glu=glu)
+    ok, worst = rel_close(got.cpu().numpy(), ref, TOL)
+    assert ok, worst
+    # Rows that are not whole tiles are refused, nothing queued.
+    with pytest.raises(ops.KernelFailure) as refused:
+        ops.vecq(Q4_K, ut, qd, k, n - 8, gate=gt, variant=tiled_variant, **common)
+    assert refused.value.rejected
