@@ -330,6 +330,17 @@ def other_configs(device, args, only=None):
             distinct = int(torch.unique(ids).numel())
             layer = lambda i: ops.moe_ffn(ops.TYPE_Q4_K, logits, xs, gus[i % sets], dns[i % sets], hidden, ffn, experts, used)
             us = timed(layer, 2 * sets)
+            chain_us = None
+            if tokens == 1:
+                # One token: the layer in one launch (llmp_hip_moe_token), bit for bit the four operations' result.
+                chain_us = us
+                state = ops.MoeTokenState(used, ffn, device)
+                y1 = torch.empty(hidden, dtype=torch.float32, device=device)
+                us = timed(lambda i: ops.moe_token(ops.TYPE_Q4_K, logits.view(-1), xs.view(-1), gus[i % sets], dns[i % sets], hidden, ffn,
+                                                   experts, used, state, launches=2, out=y1), 2 * sets)
+                one_us = timed(lambda i: ops.moe_token(ops.TYPE_Q4_K, logits.view(-1), xs.view(-1), gus[i % sets], dns[i % sets], hidden,
+                                                       ffn, experts, used, state, launches=1, out=y1), 2 * sets)
+                assert int(state.sync[2]) == 0, "a workgroup gave up waiting at the layer's meeting"
             # The dominant kernel alone: the gate/up product with its GLU over ready inputs.
             pairs = tokens * used
             h = torch.empty((pairs, ffn), dtype=torch.float32, device=device)
@@ -356,11 +367,15 @@ def other_configs(device, args, only=None):
             product_bytes = distinct * gu_bytes + tokens * hidden * 4 + pairs * ffn * 4
             layer_bytes = distinct * (gu_bytes + dn_bytes) + tokens * hidden * 4 * 2
             entry = {"workload": f"MoE expert-grouped Q4_K FFN layer, 128 experts top-8, hidden 2048, expert FFN 768, {tokens} "
-                                 "token(s): router, [q8_1,] gate/up + SwiGLU, [q8_1,] down, ordered weighted combine",
+                                 "token(s): router, [q8_1,] gate/up + SwiGLU, [q8_1,] down, ordered weighted combine (one token: llmp_hip_moe_token)",
                      "layer_us": round(us, 1), "distinct_experts": distinct, "expert_weight_sets_rotated": sets,
                      "layer_algorithmic_bytes": layer_bytes, "layer_GB/s": round(layer_bytes / us / 1e3, 1),
                      "layer_frac_hbm_peak": round(layer_bytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                      "roofline": hbm_roofline(name, kernel, product_bytes, product_us)}
+            if chain_us is not None:
+                entry["layer_launches"] = "two (llmp_hip_moe_token: router + gate/up + SwiGLU; down + combine)"
+                entry["layer_us_as_one_launch_meeting_inside"] = round(one_us, 1)
+                entry["layer_us_as_four_operations"] = round(chain_us, 1)
             if tokens == 512:
                 flops = tokens * used * 3 * 2.0 * hidden * ffn
                 entry["layer_TFLOP/s"] = round(flops / us / 1e6, 2)

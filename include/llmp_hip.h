@@ -158,6 +158,47 @@ int64_t llmp_hip_moe_route_ints(int experts, int used, int tokens);
 int llmp_hip_moe_route(const int32_t* ids, int ids_stride, int experts, int used, int tokens,
                        int32_t* route, void* stream);
 
+/* One token through a routed-expert FFN layer (Q4_K experts) in one or two launches: llmp.moe.router, the picked experts'
+ * gate/up products with their GLU, their down products and the ordered weighted sum, which the reference's graph holds
+ * as kRoute, kMatMulId, kGlu, kMatMulId and kExpertReduce (src/ir/decompose.cc:1080-1109) and the entry points above
+ * run as four launches. It has no single counterpart in the reference: it is those operations fused for the decode
+ * step, where each launch costs more than its bytes. Results are bit for bit llmp_hip_moe_router's ids and weights
+ * and llmp_hip_vecq_fused (gate/up with the GLU; down) followed by llmp_hip_moe_combine.
+ * logits F32 [experts]; x the token's `hidden` activations (x_type LLMP_X_F32 or LLMP_X_BF16); gate_up: an expert's
+ * 2 * ffn rows of `hidden` values, the gate's rows first, gate_up_stride blocks an expert; down: hidden rows of ffn
+ * values, down_stride blocks an expert; out F32 [hidden]; ids, weights [used]: the router's result, written; h F32
+ * [used][ffn]: scratch for the activated values (llmp_hip_moe_token_scratch bytes). used <= 8, hidden and ffn whole
+ * super-blocks (hidden <= 8192).
+ * launches 1: the two halves meet inside the launch at `sync`, 16 + 4 * cus bytes of device memory that are zero
+ * before their first use and need no reset between calls or graph replays with the same `cus` (each workgroup keeps
+ * the number of meetings it has come to in a word of its own from byte 16 on); word 2 of it is set to 1 if
+ * a workgroup ever gave up waiting (the results of that call are then wrong; it never happens while the whole grid,
+ * `cus` workgroups, is resident, which takes a device this call has to itself: no other kernel of another stream
+ * holding compute units for long). launches 2: the same two halves as two launches, `sync` unused: the faster of the
+ * two on an MI355X (16.7 us against 19.3 at 128 experts, top 8, hidden 2048, ffn 768; the four operations 20 us):
+ * agent-scope stores and loads take longer to cross the device than a launch boundary does. Calls that share h, ids,
+ * weights or sync must not overlap. */
+typedef struct llmp_moe_token {
+  const float* logits;
+  const void* x;
+  const void* gate_up;
+  const void* down;
+  float* out;
+  int32_t* ids;
+  float* weights;
+  float* h;
+  void* sync;
+  int64_t gate_up_stride, down_stride; /* blocks an expert */
+  int32_t type;                        /* LLMP_TYPE_Q4_K */
+  int32_t x_type;
+  int32_t experts, used, hidden, ffn;
+  int32_t glu;       /* LLMP_GLU_* */
+  int32_t normalize; /* the router's: weights over their sum */
+  float limit, route_scale;
+} llmp_moe_token;
+size_t llmp_hip_moe_token_scratch(const llmp_moe_token* op);
+int llmp_hip_moe_token(const llmp_moe_token* op, int launches, int cus, void* stream);
+
 /* llmp.q8_1 with a gather, quantize_row_q8_1_cuda's `ids` argument
  * (third_party/patches/ggml/0010-llmp-q8-dispatch-descriptors.patch:604-611): output row r
  * is the Q8_1 of input row rows[r] (row r when rows is null), row_stride floats apart. */

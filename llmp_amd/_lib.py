@@ -84,6 +84,15 @@ class SetRowsStore(C.Structure):
                 ("rows", C.c_int64), ("cells", C.c_int64)]
 
 
+class MoeToken(C.Structure):
+    """llmp_moe_token: one token's routed-expert FFN layer in one launch."""
+    _fields_ = [("logits", C.c_void_p), ("x", C.c_void_p), ("gate_up", C.c_void_p), ("down", C.c_void_p), ("out", C.c_void_p),
+                ("ids", C.c_void_p), ("weights", C.c_void_p), ("h", C.c_void_p), ("sync", C.c_void_p),
+                ("gate_up_stride", C.c_int64), ("down_stride", C.c_int64), ("type", C.c_int32), ("x_type", C.c_int32),
+                ("experts", C.c_int32), ("used", C.c_int32), ("hidden", C.c_int32), ("ffn", C.c_int32), ("glu", C.c_int32),
+                ("normalize", C.c_int32), ("limit", C.c_float), ("route_scale", C.c_float)]
+
+
 class AttnVecQuant(C.Structure):
     """llmp_attn_vec_quant: the operands of ggml.flash_attn_ext.vec_q8_0 / vec_q4_0 (src/kernels/ggml/kv_quant.h:146-160
     of the reference)."""
@@ -133,6 +142,8 @@ SYMBOLS = {
     "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
     "llmp_hip_rope_set_rows_quant": (_int, [C.POINTER(RopeStore), _vp]),
     "llmp_hip_relayout_q4_k_tiles64": (_int, [_vp, _vp, C.c_int64, C.c_int64, _int, _vp]),
+    "llmp_hip_moe_token_scratch": (C.c_size_t, [C.POINTER(MoeToken)]),
+    "llmp_hip_moe_token": (_int, [C.POINTER(MoeToken), _int, _int, _vp]),
     "llmp_hip_attn_vec_quant_scratch": (C.c_size_t, [C.POINTER(AttnVecQuant), _int]),
     "llmp_hip_attn_vec_quant": (_int, [C.POINTER(AttnVecQuant), _vp, C.c_size_t, _int, _vp]),
     "llmp_hip_mxfp8_quantize": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),

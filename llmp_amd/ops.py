@@ -305,6 +305,35 @@ def attn_vec_quant(t, q, k_cache, v_cache, mask, head_dim, heads, kv_heads, cell
     return out
 
 
+class MoeTokenState:
+    """What llmp_hip_moe_token keeps between calls on a device: the meeting words (zero before their first use), the
+    activated values' scratch, and the router's result."""
+
+    def __init__(self, used, ffn, device):
+        self.sync = torch.zeros(4 + 1024, dtype=torch.int32, device=device)
+        self.h = torch.empty((used, ffn), dtype=torch.float32, device=device)
+        self.ids = torch.empty(used, dtype=torch.int32, device=device)
+        self.weights = torch.empty(used, dtype=torch.float32, device=device)
+
+
+def moe_token(t, logits, x, gate_up, down, hidden, ffn, experts, used, state, *, glu=GLU_SWIGLU, limit=0.0, launches=2, out=None):
+    """One token's routed-expert FFN layer in two launches, or one with the halves meeting inside it (llmp_hip_moe_token): logits float32 [experts], x float32 or
+    bfloat16 [hidden]; gate_up, down as moe_ffn takes them. Returns float32 [hidden]; state.ids and state.weights hold
+    the router's result."""
+    lib = _lib.load()
+    qk = BLOCK_ELEMENTS[t]
+    if out is None:
+        out = torch.empty(hidden, dtype=torch.float32, device=x.device)
+    op = _lib.MoeToken()
+    op.logits, op.x, op.gate_up, op.down, op.out = logits.data_ptr(), x.data_ptr(), gate_up.data_ptr(), down.data_ptr(), out.data_ptr()
+    op.ids, op.weights, op.h, op.sync = state.ids.data_ptr(), state.weights.data_ptr(), state.h.data_ptr(), state.sync.data_ptr()
+    op.gate_up_stride, op.down_stride = 2 * ffn * (hidden // qk), hidden * (ffn // qk)
+    op.type, op.x_type, op.experts, op.used, op.hidden, op.ffn = t, _x_type(x), experts, used, hidden, ffn
+    op.glu, op.normalize, op.limit, op.route_scale = glu, 1, limit, 1.0
+    _lib.check(lib.llmp_hip_moe_token(C.byref(op), launches, lib.llmp_hip_compute_units(), _stream()))
+    return out
+
+
 def moe_gemm(a_codes, a_scales, offsets, sf_rows, weights, expert_stride, codes_offset, scales_offset, n, k, out=None):
     """llmp.moe.gemm (RunGroupedGemm, src/kernels/ggml/moe_cutlass.h:48-76 of the reference): routed rows sorted
     by expert, NVFP4 codes uint8 [rows, k / 2] with UE4M3 scales in atoms, times each expert's n rows of the

@@ -250,3 +250,63 @@ def test_grouped_nvfp4_gemm_refusals(device):
     assert lib.llmp_hip_grouped_gemm_run(C.byref(g), 256, None) > 0 and b"64-value" in lib.llmp_hip_last_error()
     g.k = 128
     assert lib.llmp_hip_grouped_gemm_run(C.byref(g), 256, None) > 0 and b"null" in lib.llmp_hip_last_error()
+
+
+@pytest.mark.parametrize("launches", [2, 1])
+@pytest.mark.parametrize("hidden,ffn,experts,used,x_dtype", [(2048, 768, 128, 8, "f32"), (1024, 512, 16, 4, "bf16"), (512, 256, 8, 1, "f32")])
+def test_one_token_layer_in_one_launch_equals_the_four_operations(device, launches, hidden, ffn, experts, used, x_dtype):
+    """llmp_hip_moe_token (router, gate/up with the GLU, down, ordered weighted sum in one launch, or its two halves as
+    two): the router's ids and weights and the layer's output are bit for bit those of llmp.moe.router,
+    llmp_hip_vecq_fused twice and llmp.moe.combine, and within 1e-3 of the oracle's layer; three calls in a row over the
+    same meeting words (no reset between them) give the same bits, and no workgroup ever gave up waiting."""
+    t = Q4_K
+    gate_up = synth.q4_k_weights(experts * 2 * ffn, hidden, 401).reshape(experts, -1)
+    down = synth.q4_k_weights(experts * hidden, ffn, 402).reshape(experts, -1)
+    logits = synth.rng(403).standard_normal((1, experts), dtype=np.float32)
+    x = synth.activations(1, hidden, 404)
+    if x_dtype == "bf16":
+        x = synth.bf16_to_f32(synth.bf16_bits(x))
+    gd, dd, ld = dev(gate_up, device), dev(down, device), dev(logits, device)
+    xd = dev(x, device) if x_dtype == "f32" else dev(x, device).to(torch.bfloat16)
+    want, ids, weights = ops.moe_ffn(t, ld, xd if x_dtype == "f32" else dev(x, device), gd, dd, hidden, ffn, experts, used)
+    state = ops.MoeTokenState(used, ffn, device)
+    outs = []
+    for _ in range(3):
+        outs.append(ops.moe_token(t, ld.view(-1), xd.view(-1), gd, dd, hidden, ffn, experts, used, state, launches=launches).clone())
+    torch.cuda.synchronize()
+    words = state.sync.cpu().numpy()
+    assert words[2] == 0, "a workgroup gave up waiting at the meeting"
+    assert np.all(words[4:4 + 8] == (3 if launches == 1 else 0))  # a word a workgroup: the meetings it has come to
+    assert torch.equal(state.ids, ids.view(-1)) and torch.equal(state.weights.view(torch.int32), weights.view(-1).view(torch.int32))
+    for got in outs:
+        assert torch.equal(got.view(torch.int32), want.view(-1).view(torch.int32))
+    # And the oracle's layer over the same inputs (the activated values quantized again before the down product).
+    ids_c, w_c = oracle.route(logits, used)
+    qk = 256
+    up_c = gate_up.reshape(-1)[ffn * (hidden // qk) * 144:]
+    h_c = oracle.vecq(oracle.TYPE_Q4_K, up_c, oracle.q8_1_quantize(x), hidden, ffn, gate=gate_up, ids=ids_c, tokens=1, used=used,
+                      stride_expert=2 * ffn * (hidden // qk), glu=oracle.GLU_SWIGLU, experts=experts)
+    hq = oracle.q8_1_quantize(h_c.reshape(used, ffn))
+    blocks = oracle.padded_k(ffn) // 32
+    y_c = oracle.vecq(oracle.TYPE_Q4_K, down, hq, ffn, hidden, ids=ids_c, tokens=1, used=used, stride_expert=hidden * (ffn // qk),
+                      y_token=blocks * used, y_slot=blocks, experts=experts)
+    ref = oracle.expert_reduce(y_c, w_c).reshape(-1)
+    ok, worst = rel_close(outs[0].cpu().numpy(), ref, 2e-3, floor=1e-2)
+    assert ok, worst
+
+
+def test_one_token_layer_refusals(device):
+    import ctypes as C
+    lib = ops._lib.load()
+    op = ops._lib.MoeToken()
+    for name in ("logits", "x", "gate_up", "down", "out", "ids", "weights", "h", "sync"):
+        setattr(op, name, 0x10000)
+    op.type, op.x_type, op.experts, op.used, op.hidden, op.ffn, op.glu, op.normalize = Q4_K, ops.X_F32, 128, 8, 2048, 768, ops.GLU_SWIGLU, 1
+    op.gate_up_stride, op.down_stride = 2 * 768 * 8, 2048 * 3
+    for field, value, what in (("used", 9, b"picks"), ("hidden", 2000, b"super-blocks"), ("type", ops.TYPE_Q8_0, b"Q4_K"),
+                               ("glu", ops.GLU_NONE, b"a GLU"), ("down_stride", 100, b"stride"), ("sync", None, b"null")):
+        saved = getattr(op, field)
+        setattr(op, field, value)
+        assert lib.llmp_hip_moe_token(C.byref(op), 1, 256, None) == 1 and what in lib.llmp_hip_last_error(), (field, lib.llmp_hip_last_error())
+        setattr(op, field, saved)
+    assert lib.llmp_hip_moe_token(C.byref(op), 3, 256, None) == 1
