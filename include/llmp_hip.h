@@ -508,8 +508,10 @@ int llmp_hip_decode_vector(int decoder, const llmp_decode_operand* weight, uint6
 /* RunVectorGlu of src/kernels/decode/products.h:120-139: y[t][j] = glu(gate row gate_first + j . x[t],
  * up row up_first + j . x[t]), each with its weight's tensor scale; one weight may be both (a
  * stacked gate and up). `glu` is ir::GluKind (src/ir/op.h:455): 0 SwiGLU, 1 GeGLU (erf), 2 GeGLU
- * (tanh), 3 SwiGLU with gate <= limit and |up| <= limit (src/kernels/decode/templates.cuh:73-90). The two weights share K
- * and, here, the decoder (the reference has a short list of mixed pairs: refused). */
+ * (tanh), 3 SwiGLU with gate <= limit and |up| <= limit (src/kernels/decode/templates.cuh:73-90). The two weights share K;
+ * their decoders are the same, or one of the six mixed pairs the reference instantiates
+ * (src/kernels/decode/implementations.cc:73-81: an MXFP8, NVFP4, MXFP4 or affine split gate with a BF16 up, an NVFP4
+ * or MXFP4 split gate with a Q8_0 up); any other pair is refused, as there. */
 int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_operand* gate, uint64_t gate_first, int up_decoder,
                                const llmp_decode_operand* up, uint64_t up_first, uint64_t outputs, int glu, float limit,
                                const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride,

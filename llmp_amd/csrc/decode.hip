@@ -256,8 +256,9 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
 }
 
 // grid: workgroups of eight waves, persistent over pairs of output rows; LDS: T input rows.
-// kGlu: a wave's two rows are gate row first + j and up row up_first + j of output j.
-template <int D, int T, bool kGlu>
+// kGlu: a wave's two rows are gate row first + j and up row up_first + j of output j; the up weight's decoder DU may
+// differ from the gate's D (the pairs src/kernels/decode/implementations.cc:73-81 of the reference lists).
+template <int D, int T, bool kGlu, int DU = D>
 __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const DecodeArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int tid = threadIdx.x;
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
           if (r == 0) {
             LoadSegment<D>(a.w, a.first + out0, seg, v[r], s[r]);
           } else {
-            LoadSegment<D>(a.up, a.up_first + out0, seg, v[r], s[r]);
+            LoadSegment<DU>(a.up, a.up_first + out0, seg, v[r], s[r]);
           }
         } else {
           // A lone last row is decoded twice: its second copy's sums are not stored.
@@ -778,12 +779,33 @@ void LaunchMatrixShared(const DecodeArgs& a, dim3 grid, uint32_t rows, hipStream
 
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
 
-template <int D, int T, bool kGlu>
+template <int D, int T, bool kGlu, int DU = D>
 void LaunchDecode(const DecodeArgs& a, int groups, int waves, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T, kGlu>), static_cast<int>(kDecodeLdsLimit), &sized)) return;
-  hipLaunchKernelGGL((DecodeVectorKernel<D, T, kGlu>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
+  if (!AllowLds(reinterpret_cast<const void*>(&DecodeVectorKernel<D, T, kGlu, DU>), static_cast<int>(kDecodeLdsLimit), &sized)) return;
+  hipLaunchKernelGGL((DecodeVectorKernel<D, T, kGlu, DU>), dim3(static_cast<unsigned>(groups)), dim3(waves * 64),
                      DecodeLds(T, a.w.k), stream, a);
+}
+
+// The GLU of two different decoders.
+template <int D, int DU>
+void LaunchMixedGlu(const DecodeArgs& a, int tokens, int groups, int waves, hipStream_t stream) {
+  switch (tokens) {
+    case 1: LaunchDecode<D, 1, true, DU>(a, groups, waves, stream); break;
+    case 2: LaunchDecode<D, 2, true, DU>(a, groups, waves, stream); break;
+    case 3: LaunchDecode<D, 3, true, DU>(a, groups, waves, stream); break;
+    default: LaunchDecode<D, 4, true, DU>(a, groups, waves, stream); break;
+  }
+}
+// The mixed pairs the reference instantiates (decode_mixed.cu by src/kernels/decode/implementations.cc:73-81): a
+// block-scaled or affine gate with a BF16 or Q8_0 up.
+constexpr int kMixedGlu[6][2] = {{LLMP_DECODER_MXFP8_SPLIT, LLMP_DECODER_BF16_DENSE},  {LLMP_DECODER_NVFP4_SPLIT, LLMP_DECODER_Q8_0_BLOCKS},
+                                 {LLMP_DECODER_NVFP4_SPLIT, LLMP_DECODER_BF16_DENSE},  {LLMP_DECODER_MXFP4_SPLIT, LLMP_DECODER_BF16_DENSE},
+                                 {LLMP_DECODER_MXFP4_SPLIT, LLMP_DECODER_Q8_0_BLOCKS}, {LLMP_DECODER_AFFINE_SPLIT, LLMP_DECODER_BF16_DENSE}};
+bool MixedGluBuilt(int gate, int up) {
+  for (const auto& pair : kMixedGlu)
+    if (pair[0] == gate && pair[1] == up) return true;
+  return false;
 }
 
 template <int D, bool kGlu>
@@ -864,7 +886,7 @@ int CheckOperand(const char* what, int decoder, const llmp_decode_operand* w, ui
 
 // The launches of a product whose operands have been checked: four input rows a pass, or
 // fewer of a long row.
-int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64_t rows, hipStream_t s) {
+int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64_t rows, hipStream_t s, int up_decoder = -1) {
   const uint32_t k = a.w.k;
   if (rows == 0 || rows > 16) return Refuse(1, "%s: rows %llu (1 to 16)", what, static_cast<unsigned long long>(rows));
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || a.x_stride % 4 != 0 || a.x_stride < k || a.y_stride < a.outputs ||
@@ -888,6 +910,20 @@ int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64
   for (uint64_t token0 = 0; token0 < rows; token0 += pass) {
     const int tokens = static_cast<int>(rows - token0 < static_cast<uint64_t>(pass) ? rows - token0 : pass);
     a.token0 = static_cast<uint32_t>(token0);
+    if (up_decoder >= 0 && up_decoder != decoder) {
+#define LLMP_MIXED(G, U) \
+  if (decoder == G && up_decoder == U) LaunchMixedGlu<G, U>(a, tokens, static_cast<int>(groups), waves, s);
+      LLMP_MIXED(LLMP_DECODER_MXFP8_SPLIT, LLMP_DECODER_BF16_DENSE)
+      LLMP_MIXED(LLMP_DECODER_NVFP4_SPLIT, LLMP_DECODER_Q8_0_BLOCKS)
+      LLMP_MIXED(LLMP_DECODER_NVFP4_SPLIT, LLMP_DECODER_BF16_DENSE)
+      LLMP_MIXED(LLMP_DECODER_MXFP4_SPLIT, LLMP_DECODER_BF16_DENSE)
+      LLMP_MIXED(LLMP_DECODER_MXFP4_SPLIT, LLMP_DECODER_Q8_0_BLOCKS)
+      LLMP_MIXED(LLMP_DECODER_AFFINE_SPLIT, LLMP_DECODER_BF16_DENSE)
+#undef LLMP_MIXED
+      const int status = LaunchStatus(what);
+      if (status != 0) return token0 == 0 ? status : (status > 0 ? -status : status);
+      continue;
+    }
     switch (decoder) {
 #define LLMP_DECODER(ID) \
   case ID: LaunchDecoder<ID>(a, glu, tokens, static_cast<int>(groups), waves, s); break;
@@ -937,7 +973,7 @@ extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_op
   BeginLaunches();
   if (const int bad = CheckOperand("decode.vector_glu gate", gate_decoder, gate, gate_first, outputs); bad != 0) return bad;
   if (const int bad = CheckOperand("decode.vector_glu up", up_decoder, up, up_first, outputs); bad != 0) return bad;
-  if (gate_decoder != up_decoder)
+  if (gate_decoder != up_decoder && !MixedGluBuilt(gate_decoder, up_decoder))
     return Refuse(1, "decode.vector_glu: no instantiation for gate decoder %d with up decoder %d", gate_decoder, up_decoder);
   if (gate->k != up->k) return Refuse(1, "decode.vector_glu: gate's K %u and up's %u differ", gate->k, up->k);
   if (glu < 0 || glu > 3) return Refuse(1, "decode.vector_glu: unknown GLU");
@@ -950,7 +986,7 @@ extern "C" int llmp_hip_decode_vector_glu(int gate_decoder, const llmp_decode_op
   a.outputs = static_cast<uint32_t>(outputs);
   a.glu = glu, a.limit = limit;
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
-  return LaunchProduct("decode.vector_glu", gate_decoder, true, a, rows, static_cast<hipStream_t>(stream));
+  return LaunchProduct("decode.vector_glu", gate_decoder, true, a, rows, static_cast<hipStream_t>(stream), up_decoder);
 }
 
 extern "C" int llmp_hip_decode_rows(int decoder, const llmp_decode_operand* w, const int32_t* ids, uint64_t count,

@@ -467,18 +467,18 @@ def decode_vector(decoder, weight, x, first=0, outputs=None, threads=1):
     return y
 
 
-_sig("orc_decode_vector_glu", _int, _int, C.POINTER(DecodeOperand), _u64, C.POINTER(DecodeOperand), _u64, _u64, _int,
+_sig("orc_decode_vector_glu", _int, _int, C.POINTER(DecodeOperand), _u64, _int, C.POINTER(DecodeOperand), _u64, _u64, _int,
      C.c_float, _vp, _u64, _u64, _vp, _u64, _int)
 
 
-def decode_vector_glu(decoder, gate, up, x, glu, limit=0.0, gate_first=0, up_first=0, outputs=None, threads=1):
+def decode_vector_glu(decoder, gate, up, x, glu, limit=0.0, gate_first=0, up_first=0, outputs=None, threads=1, up_decoder=None):
     """llmp.decode.vector_glu on the CPU; `glu` is the reference's ir::GluKind (0 SwiGLU, 1 GeGLU erf, 2 GeGLU
     tanh, 3 SwiGLU with a clamp)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     g, u = decode_operand(gate), decode_operand(up)
     outputs = gate["data"].shape[0] - gate_first if outputs is None else outputs
     y = np.zeros((x.shape[0], outputs), dtype=np.float32)
-    rc = lib.orc_decode_vector_glu(decoder, C.byref(g), gate_first, C.byref(u), up_first, outputs, glu, limit, _p(x),
+    rc = lib.orc_decode_vector_glu(decoder, C.byref(g), gate_first, decoder if up_decoder is None else up_decoder, C.byref(u), up_first, outputs, glu, limit, _p(x),
                                    x.shape[0], x.shape[1], _p(y), outputs, threads)
     if rc != 0:
         raise ValueError("no such product")

@@ -561,10 +561,12 @@ static double decode_glu(int kind, double g, double u, double limit) {
   }
 }
 
-int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, const orc_decode_operand* up,
-                          uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
-                          uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
-  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT || glu < 0 || glu > 3 || gate->k != up->k) return 1;
+int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, int up_decoder,
+                          const orc_decode_operand* up, uint64_t up_first, uint64_t outputs, int glu, float limit,
+                          const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads) {
+  if (decoder < 0 || decoder > ORC_DECODER_AFFINE_SPLIT || up_decoder < 0 || up_decoder > ORC_DECODER_AFFINE_SPLIT || glu < 0 ||
+      glu > 3 || gate->k != up->k)
+    return 1;
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
   for (int64_t j = 0; j < (int64_t)outputs; ++j) {
     const uint64_t grow = gate_first + (uint64_t)j, urow = up_first + (uint64_t)j;
@@ -575,7 +577,7 @@ int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t 
       for (uint64_t c = 0; c < gate->k; ++c) {
         const double xv = (double)x[t * x_stride + c];
         g += (double)orc_decode_value(decoder, gate, grow, c) * xv;
-        u += (double)orc_decode_value(decoder, up, urow, c) * xv;
+        u += (double)orc_decode_value(up_decoder, up, urow, c) * xv;
       }
       y[t * y_stride + (uint64_t)j] = (float)decode_glu(glu, g * gs, u * us, (double)limit);
     }

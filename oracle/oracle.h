@@ -106,9 +106,9 @@ int orc_decode_vector(int decoder, const orc_decode_operand* w, uint64_t first, 
 
 /* RunVectorGlu, products.h:120-139: y[t][j] = glu(gate row . x[t], up row . x[t]); glu is ir::GluKind
  * (src/ir/op.h:455), the functions those of src/kernels/reference/exec.cc:248-262. */
-int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, const orc_decode_operand* up,
-                          uint64_t up_first, uint64_t outputs, int glu, float limit, const float* x, uint64_t rows,
-                          uint64_t x_stride, float* y, uint64_t y_stride, int threads);
+int orc_decode_vector_glu(int decoder, const orc_decode_operand* gate, uint64_t gate_first, int up_decoder,
+                          const orc_decode_operand* up, uint64_t up_first, uint64_t outputs, int glu, float limit,
+                          const float* x, uint64_t rows, uint64_t x_stride, float* y, uint64_t y_stride, int threads);
 
 /* RunMatrix's tensor-core path, products.h:27-33 and 111-118: weights and inputs rounded to the decoder's
  * matrix element (F16 for F16 and Q8_0 weights, BF16 otherwise), double sums here. */

@@ -158,8 +158,27 @@ def test_vector_glu_of_one_stacked_weight_and_refusals(device):
         ops.decode_vector_glu(3, wd, wd, xd, 4, outputs=n)
     with pytest.raises(ops.KernelFailure):  # up rows [100, 164) of 128
         ops.decode_vector_glu(3, wd, wd, xd, 0, up_first=100, outputs=n)
-    with pytest.raises(ops.KernelFailure):  # a gate and an up of different decoders
+    with pytest.raises(ops.KernelFailure):  # a gate and an up of two decoders that are no pair the reference builds
         ops.decode_vector_glu(3, wd, to_device(synth.decode_weight(9, n, k, 792), device), xd, 0, outputs=n, up_decoder=9)
+
+
+@pytest.mark.parametrize("gate_decoder,up_decoder", [(7, 0), (3, 2), (3, 0), (9, 0), (9, 2), (11, 0)])
+@pytest.mark.parametrize("rows", [1, 6])
+def test_vector_glu_of_two_decoders(device, gate_decoder, up_decoder, rows):
+    """The six mixed pairs the reference instantiates (src/kernels/decode/implementations.cc:73-81): a block-scaled or
+    affine gate with a BF16 or Q8_0 up, each weight decoded by its own decoder, against the oracle."""
+    n, k = 80, 512
+    gate = synth.affine_weight(n, k, 806, bits=4, group=64, tensor_scales=2) if gate_decoder == 11 else \
+        synth.decode_weight(gate_decoder, n, k, 795 + gate_decoder, tensor_scales=2)
+    up = synth.decode_weight(up_decoder, n, k, 796 + up_decoder)
+    x = synth.activations(rows, k, 797 + rows) * 0.25
+    for glu in (0, 2):
+        want = oracle.decode_vector_glu(gate_decoder, gate, up, x, glu, gate_first=5, up_first=2, outputs=64, up_decoder=up_decoder)
+        on = lambda w: {key: (torch.from_numpy(np.ascontiguousarray(v)).to(device) if isinstance(v, np.ndarray) else v) for key, v in w.items()}
+        got = ops.decode_vector_glu(gate_decoder, on(gate), on(up), torch.from_numpy(x).to(device), glu,
+                                    gate_first=5, up_first=2, outputs=64, up_decoder=up_decoder).cpu().numpy()
+        ok, worst = rel_close(got, want, 1e-3)
+        assert ok, (gate_decoder, up_decoder, glu, worst)
 
 
 @pytest.mark.parametrize("decoder", DECODERS)
