@@ -111,8 +111,11 @@ PROFILED_TRAFFIC = {
     "q8_0_matvec_4096x4096_b1": _traffic(8768.0, 16.0),
     # A weight row a lane asks for 144 bytes a row a load, ragged against the 64-byte units HBM is fetched in; the
     # unit two neighbouring super-blocks share is often fetched for each: 1.3 to 1.4 times the algorithmic bytes.
-    "q4_k_gate_up_geglu_b4": _traffic(43591.1, 240.0),
-    "q4_k_gate_up_geglu_b8": _traffic(46231.1, 960.0),
+    "q4_k_gate_up_geglu_b4": _traffic(43611.5, 240.0),
+    "q4_k_gate_up_geglu_b8": _traffic(43637.9, 480.0),
+    # The same kernel over weights relaid out into 64-row tiles: a wave's 9216 bytes are consecutive.
+    "q4_k_gate_up_geglu_b4_tiles64": _traffic(32567.8, 240.0),
+    "q4_k_gate_up_geglu_b8_tiles64": _traffic(32649.7, 480.0),
     "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
     # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through
     # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
@@ -120,6 +123,8 @@ PROFILED_TRAFFIC = {
     "moe_q4_k_ffn_t1": _traffic(7028.8, 24.0),        # the gate/up launch
     "moe_q4_k_ffn_t16": _traffic(76343.9, 457.9),     # the gate/up launch
     "moe_q4_k_ffn_t512": _traffic(182457.3, 12338.4),  # the gate/up launch: the experts' tokens once a segment of rows
+    "attn_vec_q8_0_d256_h16_kv8_cells8192_rows1": _traffic(17578.0 + 273.5, 528.0 + 16.0),  # the splits + their combination
+    "attn_vec_q4_0_d256_h16_kv8_cells8192_rows1": _traffic(9387.0 + 273.5, 528.0 + 16.0),
     "exl3_linear_4096x14336_4bpw_m1": _traffic(14475.9 + 143.5, 232.0 + 56.0),  # product + output transform
     "exl3_linear_4096x14336_4bpw_m16": _traffic(14906.0 + 114.5 + 1921.5, 3584.0 + 128.0 + 896.0),
     "exl3_multi_linear_4096x2x14336_4bpw_m1": _traffic(28815.7 + 255.5, 464.0 + 112.0),
@@ -212,7 +217,7 @@ def other_configs(device, args, only=None):
         del copies, w
 
     # Config 2 at batch 4 and 8.
-    if want("q4_k_gate_up_geglu_b4") or want("q4_k_gate_up_geglu_b8"):
+    if any(want(f"q4_k_gate_up_geglu_b{t}{suffix}") for t in (4, 8) for suffix in ("", "_tiles64")):
         gate_host, up_host = synth.q4_k_weights(N, K, 101), synth.q4_k_weights(N, K, 102)
         gate, up = dev(gate_host), dev(up_host)
         count = -(-ROTATE_BYTES // WEIGHT_BYTES)
@@ -220,28 +225,29 @@ def other_configs(device, args, only=None):
         ups = [up] + [up.clone() for _ in range(count - 1)]
         for tokens in (4, 8):
             name = f"q4_k_gate_up_geglu_b{tokens}"
-            if not want(name):
+            if not want(name) and not want(name + "_tiles64"):
                 continue
             x_host = synth.bf16_to_f32(synth.bf16_bits(synth.activations(tokens, K, 203)))
             q8 = ops.quantize_q8_1(dev(x_host))
             y = torch.empty((tokens, 1, N), dtype=torch.float32, device=device)
-            us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
-                                          glu=ops.GLU_GEGLU, out=y), 4 * count)
-            entry = {"workload": f"config 2 at batch {tokens}",
-                     "roofline": hbm_roofline(name, "VecQRows<glu, %d tokens> (llmp.vecq, Q4_K, a weight row a lane on "
-                                              "v_mfma_i32_4x4x4_16B_i8)" % (4 if tokens <= 4 else 8), algorithmic_bytes(tokens), us)}
-            if cpu:
-                q8_host = oracle.q8_1_quantize(x_host)
-                entry["cpu_baseline"] = cpu_leg(
-                    lambda: oracle.vecq(oracle.TYPE_Q4_K, up_host, q8_host, K, N, gate=gate_host, tokens=tokens,
-                                        glu=oracle.GLU_GEGLU, threads=threads),
-                    WEIGHT_BYTES / 1e9, "GB/s", 2.0, f"the whole gate/up pair at {tokens} tokens", threads)
-            out[name] = entry
+            if want(name):
+                us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, ups[i % count], q8, K, N, gate=gates[i % count], tokens=tokens,
+                                              glu=ops.GLU_GEGLU, out=y), 4 * count)
+                entry = {"workload": f"config 2 at batch {tokens}",
+                         "roofline": hbm_roofline(name, "VecQRows<glu, %d tokens> (llmp.vecq, Q4_K, a weight row a lane on "
+                                                  "v_mfma_i32_4x4x4_16B_i8)" % (4 if tokens <= 4 else 8), algorithmic_bytes(tokens), us)}
+                if cpu:
+                    q8_host = oracle.q8_1_quantize(x_host)
+                    entry["cpu_baseline"] = cpu_leg(
+                        lambda: oracle.vecq(oracle.TYPE_Q4_K, up_host, q8_host, K, N, gate=gate_host, tokens=tokens,
+                                            glu=oracle.GLU_GEGLU, threads=threads),
+                        WEIGHT_BYTES / 1e9, "GB/s", 2.0, f"the whole gate/up pair at {tokens} tokens", threads)
+                out[name] = entry
             # The same over weights relaid out at import into 64-row tiles (lossless; the kernel's reads become whole
             # 64-byte units): beside the reference's layout, not in place of it.
             tiled_name = name + "_tiles64"
             tiled_variant = ops.vecq_variants().index("rows pass8 tiles64")
-            if only is None or only in (name, tiled_name):
+            if want(tiled_name):
                 if "gates_tiled" not in locals():
                     gates_tiled = [ops.relayout_q4_k_tiles64(g_, N, K) for g_ in gates]
                     ups_tiled = [ops.relayout_q4_k_tiles64(u_, N, K) for u_ in ups]
