@@ -737,6 +737,8 @@ def main():
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 dot (Q4_K x Q8_1), fp32 accumulate", "data": "synthetic",
+        "parity": "int32 sub-block sums bit-exact; fp32 outputs |got - want| <= 1e-3 * max(|want|, 1e-3 * rms(want)) "
+                  "against the CPU oracle (a relative bound with an RMS floor, looser than a strict max-rel 1e-3)",
         "config": {"workload": f"GGML Q4_K fused gate/up GEGLU MMVQ, K={K}, N=2x{N}, batch {args.tokens}, "
                                + ("bf16 activations quantized to q8_1 in-kernel" if args.fused else "fp32 activations through llmp.q8_1")
                                + ", fp32 out",

@@ -548,6 +548,16 @@ inline std::vector<Implementation> Implementations() {
       "two to sixteen stores a launch");
   add("llmp.rope.set_rows_quant", "fused.rope_set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0,
       {"llmp_hip_rope_set_rows_quant"}, "a workgroup a token");
+  // The attention that reads those caches (kv_quant.h:9-26, 146-160): not row invariant (the query rows of a pass
+  // share their workgroup's online softmax tiles, each row's values its own).
+  for (const char* kind : {"q8_0", "q4_0"}) {
+    add(std::string("ggml.flash_attn_ext.vec_") + kind, "flash_attn_ext", {kind}, {1, any, 64, 1}, Rung::kNative, 0,
+        {"llmp_hip_attn_vec_quant"}, "a lane a cell for K, a lane D / 64 values for V, the cells split over workgroups");
+  }
+  // One token through a routed-expert layer: the router, the experts' products, their GLU and the ordered sum fused
+  // (no single counterpart in the reference: ir/decompose.cc:1080-1109 holds the five operations).
+  add("llmp.moe.token", "fused.moe_ffn_token", {"q4_k"}, {1, 1, 256, 256}, Rung::kNative, 0, {"llmp_hip_moe_token"},
+      "two launches: router + gate/up + GLU; down + combine");
   return all;
 }
 
