@@ -398,6 +398,15 @@ typedef struct llmp_exl3_weights {
 int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void* w, int column, int columns,
                               void* stream);
 
+/* LaunchContext::Reconstruct with ReconstructOperands::fused (src/kernels/exl3/launch.cc:425-448, validate.h:183-193;
+ * the definition src/kernels/reference/decode.h:37-43): the same columns of the weights themselves,
+ * W = diag(suh) H What H diag(svh) / 128 with H the 128-point transform over each block of 128 inputs and of 128
+ * outputs, into w (k x columns F16, row-major, at a 16-byte boundary), for the reconstruction path's plain GEMM from
+ * 1,024 rows. Whole 128-column blocks. The transforms run in F32 and a value is rounded to F16 once (the
+ * reference's kernel rounds every butterfly to F16). */
+int llmp_hip_exl3_reconstruct_fused(const llmp_exl3_weights* weights, void* w, int column, int columns,
+                                    void* stream);
+
 /* LaunchContext::Hadamard (launch.h:104-106, validate.h:199-212): 128-point Hadamard
  * transforms of the rows of x (rows x columns) into y (x itself or disjoint), times
  * 1 / sqrt(128): F16 with the input scale (y = H(x * scale)), or F16 / F32 with the output

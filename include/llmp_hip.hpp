@@ -535,7 +535,8 @@ inline std::vector<Implementation> Implementations() {
           d < 2 ? Rung::kNative : Rung::kOnChipDecode, t.needs, {t.launch}, std::string("decoder ") + std::to_string(d));
     }
   }
-  // EXL3 (exl3/implementations.h:8-31): the packed paths; the reconstruction paths are not built.
+  // EXL3 (exl3/implementations.h:8-31): the packed paths; of the reconstruction paths the two reconstruction
+  // kernels are entry points (llmp_hip_exl3_reconstruct, _fused), the plain GEMM after them is the caller's library's.
   add("exl3.linear.gemv", "quant_linear", {"exl3"}, {1, 8, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
       "trellis tiles as the second operand of a 16 x 16 x 16 F16 matrix instruction");
   add("exl3.linear.gemm", "quant_linear", {"exl3"}, {1, 65536, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},

@@ -268,6 +268,79 @@ __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, 
   }
 }
 
+// ------------------------------------------------------- reconstruct, transformed
+
+// Columns [column, column + columns) of the weights themselves, W = diag(suh) H What H diag(svh) / 128 with H the
+// 128-point transform over each block of 128 inputs and of 128 outputs, into w[k][columns] F16 (the reference's
+// reconstruct_had_kernel, launch.cc:440-448; the definition decode.h:37-43). A workgroup of four waves a block of 128
+// inputs by 128 outputs; grid (columns / 128, k / 128); LDS 128 x 129 floats. The rotated values are decoded into
+// LDS (exact), every column is transformed along the inputs and every row along the outputs in F32 by the wave's
+// butterfly (lane l holds elements l and l + 64 of a vector: the transform does not change when the bits of its
+// index are permuted on both sides, and this assignment reads LDS without bank conflicts both ways), and the block
+// is rounded to F16 once, after the scales: the reference's kernel rounds every butterfly to F16.
+constexpr int kHadBlockPitch = 129;
+constexpr int kHadBlockLds = 128 * kHadBlockPitch * 4;
+
+template <int CB, int BITS>
+__global__ __launch_bounds__(256) void ReconstructHadKernel(const uint32_t* __restrict__ trellis,
+                                                           const uint16_t* __restrict__ suh,
+                                                           const uint16_t* __restrict__ svh,
+                                                           uint16_t* __restrict__ w, int n, int column, int columns) {
+#pragma clang fp contract(off)
+  extern __shared__ __attribute__((aligned(16))) float had_block[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int k0 = blockIdx.y * 128;
+  const int c0 = blockIdx.x * 128;  // within the slice
+  const Place p = PlaceOf(lane);
+  // Sixteen of the block's 64 tiles a wave.
+#pragma unroll 2
+  for (int t = wave * 16; t < wave * 16 + 16; ++t) {
+    const int kt = t >> 3, nt = t & 7;
+    const uint32_t* tile =
+        trellis + (static_cast<int64_t>(k0 / 16 + kt) * (n / 16) + (column + c0) / 16 + nt) * (BITS * 8);
+    const Half4 v = DecodeFour<CB, BITS>(p.first, [&](int i) { return tile[i]; });
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const _Float16 value = v[j];
+      had_block[(kt * 16 + RowOf(p.g, j)) * kHadBlockPitch + nt * 16 + p.n] = static_cast<float>(value);
+    }
+  }
+  __syncthreads();
+  // Along the inputs: a wave 32 columns.
+  for (int j = wave * 32; j < wave * 32 + 32; ++j) {
+    float a = had_block[lane * kHadBlockPitch + j];
+    float b = had_block[(lane + 64) * kHadBlockPitch + j];
+    Hadamard128(a, b, lane);
+    had_block[lane * kHadBlockPitch + j] = a;
+    had_block[(lane + 64) * kHadBlockPitch + j] = b;
+  }
+  __syncthreads();
+  // Along the outputs, then the scales: a wave 32 rows.
+  const float sv_a = HalfBitsToFloat(svh[column + c0 + lane]) * (1.0f / 128.0f);
+  const float sv_b = HalfBitsToFloat(svh[column + c0 + lane + 64]) * (1.0f / 128.0f);
+  for (int i = wave * 32; i < wave * 32 + 32; ++i) {
+    float a = had_block[i * kHadBlockPitch + lane];
+    float b = had_block[i * kHadBlockPitch + lane + 64];
+    Hadamard128(a, b, lane);
+    const float su = HalfBitsToFloat(suh[k0 + i]);
+    had_block[i * kHadBlockPitch + lane] = a * (su * sv_a);
+    had_block[i * kHadBlockPitch + lane + 64] = b * (su * sv_b);
+  }
+  __syncthreads();
+  // Sixteen bytes a thread: a row is sixteen threads' worth.
+  const int part = threadIdx.x & 15;
+  for (int i = threadIdx.x >> 4; i < 128; i += 16) {
+    const float* from = had_block + i * kHadBlockPitch + part * 8;
+    U32x4 out;
+    out.x = FloatToHalfBits(from[0]) | (FloatToHalfBits(from[1]) << 16);
+    out.y = FloatToHalfBits(from[2]) | (FloatToHalfBits(from[3]) << 16);
+    out.z = FloatToHalfBits(from[4]) | (FloatToHalfBits(from[5]) << 16);
+    out.w = FloatToHalfBits(from[6]) | (FloatToHalfBits(from[7]) << 16);
+    *reinterpret_cast<U32x4*>(w + static_cast<int64_t>(k0 + i) * columns + c0 + part * 8) = out;
+  }
+}
+
 // ------------------------------------------------------------------- product
 
 constexpr int kRingDepth = 4;  // K steps of a 128-column block in flight a wave
@@ -636,6 +709,17 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
                      static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
 
+template <int CB, int BITS>
+bool g_reconstruct_had_sized = false;
+template <int CB, int BITS>
+void LaunchReconstructHad(const llmp_exl3_weights& w, void* out, int column, int columns, hipStream_t stream) {
+  if (!AllowLds(reinterpret_cast<const void*>(&ReconstructHadKernel<CB, BITS>), kHadBlockLds, &g_reconstruct_had_sized<CB, BITS>)) return;
+  const dim3 grid(static_cast<unsigned>(columns / 128), static_cast<unsigned>(w.k / 128));
+  hipLaunchKernelGGL((ReconstructHadKernel<CB, BITS>), grid, dim3(256), kHadBlockLds, stream,
+                     static_cast<const uint32_t*>(w.trellis), static_cast<const uint16_t*>(w.suh),
+                     static_cast<const uint16_t*>(w.svh), static_cast<uint16_t*>(out), w.n, column, columns);
+}
+
 template <int BITS>
 constexpr int ProductLds() {
   constexpr int kLoads = (BITS * 32 * 8 + 1023) / 1024;
@@ -714,6 +798,27 @@ extern "C" int llmp_hip_exl3_reconstruct(const llmp_exl3_weights* weights, void*
                                                                   static_cast<hipStream_t>(stream));
   });
   return LaunchStatus("exl3.reconstruct");
+}
+
+extern "C" int llmp_hip_exl3_reconstruct_fused(const llmp_exl3_weights* weights, void* w, int column, int columns,
+                                               void* stream) {
+  BeginLaunches();
+  if (weights == nullptr || w == nullptr) return Refuse(1, "exl3.reconstruct_fused: null operand");
+  if (const int bad = CheckWeights(*weights); bad != 0) return bad;
+  // validate.cc:367-372: 128-column blocks inside the matrix.
+  if (column < 0 || columns < 128 || column % 128 != 0 || columns % 128 != 0 || column > weights->n - columns)
+    return Refuse(1, "exl3.reconstruct_fused: columns [%d, %lld) of %d: 128-column blocks inside the matrix", column,
+                  static_cast<long long>(column) + columns, weights->n);
+  if (reinterpret_cast<uintptr_t>(w) % 16 != 0) return Refuse(1, "exl3.reconstruct_fused: w at a 16-byte boundary");
+  if (const int bad = Disjoint("exl3.reconstruct_fused", {"w", reinterpret_cast<uintptr_t>(w), static_cast<size_t>(weights->k) * columns * 2},
+                               {TrellisRange(*weights), SuhRange(*weights), SvhRange(*weights)});
+      bad != 0)
+    return bad;
+  Dispatch(weights->codebook, weights->bits, [&](auto cb, auto bits) {
+    LaunchReconstructHad<decltype(cb)::value, decltype(bits)::value>(*weights, w, column, columns,
+                                                                     static_cast<hipStream_t>(stream));
+  });
+  return LaunchStatus("exl3.reconstruct_fused");
 }
 
 extern "C" int llmp_hip_exl3_hadamard(const void* x, void* y, const void* scale, int rows, int columns, int f32,

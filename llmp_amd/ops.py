@@ -431,13 +431,15 @@ def _exl3_weights(trellis, suh, svh, k, n, bits, codebook):
     return w
 
 
-def exl3_reconstruct(trellis, suh, svh, k, n, bits, codebook, column=0, columns=None):
-    """The rotated-basis weights of columns [column, column + columns): float16 [k, columns]."""
+def exl3_reconstruct(trellis, suh, svh, k, n, bits, codebook, column=0, columns=None, fused=False):
+    """Columns [column, column + columns) as float16 [k, columns]: the rotated-basis weights, or (fused, the
+    reference's ReconstructOperands::fused) the weights themselves, both transforms and side vectors applied."""
     lib = _lib.load()
     columns = n if columns is None else columns
     out = torch.empty((k, columns), dtype=torch.float16, device=trellis.device)
     w = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
-    _lib.check(lib.llmp_hip_exl3_reconstruct(C.byref(w), _ptr(out), column, columns, _stream()))
+    launch = lib.llmp_hip_exl3_reconstruct_fused if fused else lib.llmp_hip_exl3_reconstruct
+    _lib.check(launch(C.byref(w), _ptr(out), column, columns, _stream()))
     return out
 
 

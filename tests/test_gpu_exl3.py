@@ -47,6 +47,36 @@ def test_every_state_of_every_codebook(device):
         assert np.array_equal(got.cpu().numpy().view(np.uint16), want)
 
 
+@pytest.mark.parametrize("bits,codebook", [(4, ops.EXL3_3INST), (3, ops.EXL3_MCG), (6, ops.EXL3_MUL1), (1, ops.EXL3_3INST),
+                                           (8, ops.EXL3_MCG)])
+def test_fused_reconstruction_is_the_weights(device, bits, codebook):
+    """ReconstructOperands::fused (tests/unit/exl3_trellis_test.cc:467-518 of the reference): the weights with both
+    transforms and side vectors applied, against the oracle's W in F64. The reference's bounds (relative L2 of a
+    128 x 128 block 2^-7, any value within 2^-4 of its block's RMS) are for F16 butterflies; this kernel's transforms
+    are F32 with one rounding to F16, so every value is also held to one F16 step of the oracle's (and F32's own error, which is of the block's size, not the value's)."""
+    k, n = 384, 512
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 300 + bits)
+    want = oracle.exl3_rows(trellis, suh, svh, k, n, bits, codebook).T  # [k][n]
+    args = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    got16 = ops.exl3_reconstruct(*args, fused=True)
+    got = got16.float().cpu().numpy().astype(np.float64)
+    for kb in range(0, k, 128):
+        for nb in range(0, n, 128):
+            w, g = want[kb:kb + 128, nb:nb + 128], got[kb:kb + 128, nb:nb + 128]
+            rms = np.sqrt(np.mean(w.astype(np.float64) ** 2))
+            assert np.sqrt(np.mean((g - w) ** 2)) / rms <= 2.0 ** -7
+            assert np.abs(g - w).max() / rms <= 2.0 ** -4
+    step = np.maximum(np.spacing(np.abs(want).astype(np.float16)).astype(np.float64), 2.0 ** -24)
+    assert np.all(np.abs(got - want) <= step + 2e-6 * np.abs(want).max())  # F32's own error is of the block's size
+    assert np.mean(got.astype(np.float16) != want.astype(np.float16)) < 2e-3  # ties and F32's last bits
+    # A slice is the same columns of the whole.
+    part = ops.exl3_reconstruct(*args, column=128, columns=256, fused=True)
+    assert torch.equal(part, got16[:, 128:384])
+    for column, columns in ((64, 128), (0, 64), (384, 256)):
+        with pytest.raises(ops.KernelFailure):
+            ops.exl3_reconstruct(*args, column=column, columns=columns, fused=True)
+
+
 def hadamard_rows(x):
     idx = np.arange(128)
     h = np.where(np.array([[bin(i & j).count("1") % 2 for j in idx] for i in idx]) == 0, 1.0, -1.0)
