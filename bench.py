@@ -405,8 +405,8 @@ def other_configs(device, args, only=None):
         torch.cuda.empty_cache()
 
     # llmp.moe.gemm (the reference's NVFP4 grouped expert product) on config 4's shape: 512 tokens' 4096 rows sorted by
-    # expert over 128 experts, each expert's 768 x 2048 (gate or up) and 2048 x 768 (down) weights. Not a BASELINE
-    # config: timed so that its cost is known.
+    # expert over 128 experts, each expert's 768 x 2048 (gate or up) and 2048 x 768 (down) weights. Not one of the
+    # benchmark's five configurations: timed so that its cost is known.
     if want("moe_gemm_nvfp4_128_experts_t512"):
         experts, used, tokens = 128, 8, 512
         g = synth.rng(230)
@@ -417,7 +417,7 @@ def other_configs(device, args, only=None):
         sf_rows = np.concatenate([[0], np.cumsum((counts + 127) // 128 * 128)]).astype(np.int32)
         rows = int(offsets[-1])
         entry = {"workload": "llmp.moe.gemm: NVFP4 (E2M1 codes, UE4M3 scales a 16) rows sorted by expert, 128 experts, "
-                             f"{rows} rows, bf16 out; not a BASELINE config", "shapes": {}}
+                             f"{rows} rows, bf16 out; not one of the benchmark's five configurations", "shapes": {}}
         for n, k in ((768, 2048), (2048, 768)):
             a_codes = dev(g.integers(0, 256, size=(rows, k // 2), dtype=np.uint8))
             a_scales = dev(g.integers(0x20, 0x50, size=int(sf_rows[-1]) * (k // 16), dtype=np.uint8))
@@ -438,8 +438,8 @@ def other_configs(device, args, only=None):
         out["moe_gemm_nvfp4_128_experts_t512"] = entry
         torch.cuda.empty_cache()
 
-    # The attention that reads the quantized KV cache (ggml.flash_attn_ext.vec_q8_0, a "next" row of the path: not a
-    # BASELINE config), at config 2's model's decode shape: 16 heads over 8 KV heads of 256, one query row, 8192 cells.
+    # The attention that reads the quantized KV cache (ggml.flash_attn_ext.vec_q8_0, beside the path: not one of
+    # the benchmark's five configurations), at config 2's model's decode shape: 16 heads over 8 KV heads of 256, one query row, 8192 cells.
     for kind, t in (("q8_0", ops.TYPE_Q8_0), ("q4_0", ops.TYPE_Q4_0)):
         name = f"attn_vec_{kind}_d256_h16_kv8_cells8192_rows1"
         if not want(name):
@@ -463,7 +463,7 @@ def other_configs(device, args, only=None):
                                                 out=out_d, scratch=scratch), 4 * copies)
         bytes_ = 2 * kd.numel() + heads * d_ * 8 + cells * 2
         entry = {"workload": f"attention over a {kind.upper()} KV cache, head size 256, 16 heads over 8 KV heads, 1 query row, "
-                             "8192 cells (both launches: the splits and their combination); not a BASELINE config",
+                             "8192 cells (both launches: the splits and their combination); not one of the benchmark's five configurations",
                  "roofline": hbm_roofline(name, "AttnVecQuantKernel + AttnCombineKernel", bytes_, us)}
         if cpu:
             entry["cpu_baseline"] = cpu_leg(

@@ -159,7 +159,7 @@ void RegistryChecks() {
     EXPECT(i.capability.shape.min_rows >= 1 && i.capability.shape.min_rows <= i.capability.shape.max_rows);
     for (const std::string& launch : i.capability.launches) EXPECT(launch.rfind("llmp_hip_", 0) == 0);
   }
-  // SURVEY's list of names to keep (plan_step.h:201-314, capabilities.cc:2486-2489 and 2881-2893,
+  // The reference's names that a binding must keep (plan_step.h:201-314, capabilities.cc:2486-2489 and 2881-2893,
   // decode/implementations.h:7-13, exl3/implementations.h:8-31).
   for (const char* name : {"llmp.q8_1", "llmp.vecq.dense", "llmp.vecq.glu", "llmp.vecq.experts", "llmp.vecq.experts_glu", "llmp.vecq.grouped",
                            "ggml.mul_mat.mmvq", "ggml.mul_mat_glu.mmvq_fused", "llmp.mul_mat.mmvq_rows", "llmp.mul_mat_id.mmvq_rows", "llmp.mxfp8.mul_mat_vec", "llmp.mxfp8.quantize",
