@@ -263,8 +263,9 @@ int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_units, void
  * moe_cutlass.h:42-46 (SfOffset, k / 16 scales a row) in a block of rows starting at sf_rows[e] (a multiple of
  * 128, as llmp_hip_moe_route's scale_rows). B_e is at weights + e * expert_stride: n rows of codes at
  * codes_offset, their scales at scales_offset in the atoms of n rows. offsets and sf_rows are device arrays of
- * groups + 1 entries. k a multiple of 64. The scratch is not used (llmp_hip_grouped_gemm_scratch is 0: may be
- * null). Values are the format's own: E2M1 times UE4M3 is exact in BF16, the products run on the BF16 matrix
+ * groups + 1 entries. k a multiple of 64; the codes (a, weights, expert_stride, codes_offset) at 16-byte and the
+ * scales (a_scales, scales_offset) at 4-byte boundaries. The scratch is not used (llmp_hip_grouped_gemm_scratch is 0: may be
+ * null). Values are the format's own: E2M1 times UE4M3 is exact in F16, the products run on the F16 matrix
  * instructions (this device's scaled instructions take E8M0 scales per 32, not UE4M3 per 16). */
 typedef struct llmp_grouped_gemm {
   int groups;

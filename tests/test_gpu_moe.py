@@ -241,6 +241,42 @@ def test_grouped_nvfp4_gemm_matches_its_definition(device, counts, n, k):
     assert torch.all(guard[0] == -7.0) and torch.all(guard[rows + 1] == -7.0)  # nothing outside the rows is written
 
 
+def test_grouped_nvfp4_gemm_scales_that_are_not_numbers(device):
+    """A UE4M3 scale byte from 0x7F on is NaN (src/kernels/reference/decode.cc:407-411 of the reference): exactly the
+    outputs whose row or column holds one are NaN, the others are as without it."""
+    g = synth.rng(77)
+    counts, n, k = [20, 40], 128, 256
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    sf_rows = np.array([0, 128, 256], dtype=np.int32)
+    rows = int(offsets[-1])
+    a_codes, a_scales = nvfp4_operand(g, rows, k, padded_rows=256)
+    codes_bytes, scales_bytes = n * (k // 2), 128 * (k // 16)
+    weights = np.zeros((2, codes_bytes + scales_bytes), dtype=np.uint8)
+    b_codes, b_scales = [], []
+    for e in range(2):
+        c, s = nvfp4_operand(g, n, k)
+        b_codes.append(c)
+        b_scales.append(s)
+    sf = lambda row, block: (((row // 128) * (k // 64)) + block // 4) * 512 + (row % 32) * 16 + ((row % 128) // 32) * 4 + block % 4
+    a_scales[sf(128 + 7, 5)] = 0x7F   # group 1's row 7
+    a_scales[sf(3, 0)] = 0x93         # group 0's row 3
+    b_scales[1][sf(100, 15)] = 0xFF   # expert 1's column 100
+    b_scales[0][sf(0, 9)] = 0x80      # expert 0's column 0
+    for e in range(2):
+        weights[e, :codes_bytes] = b_codes[e].reshape(-1)
+        weights[e, codes_bytes:] = b_scales[e]
+    want = oracle.grouped_nvfp4_gemm(a_codes, a_scales, offsets, sf_rows, b_codes, b_scales, n, k)
+    got = ops.moe_gemm(dev(a_codes, device), dev(a_scales, device), dev(offsets, device), dev(sf_rows, device),
+                       dev(weights, device), codes_bytes + scales_bytes, 0, codes_bytes, n, k)
+    got = got.float().cpu().numpy().astype(np.float64)
+    expect_nan = np.zeros((rows, n), dtype=bool)
+    expect_nan[3, :] = expect_nan[20 + 7, :] = True
+    expect_nan[:20, 0] = expect_nan[20:, 100] = True
+    assert np.array_equal(np.isnan(want), expect_nan) and np.array_equal(np.isnan(got), expect_nan)
+    fine = ~expect_nan
+    assert np.all(np.abs(got[fine] - want[fine]) <= 2.0 ** -8 * np.abs(want[fine]) + 1e-5 * np.sqrt(np.mean(want[fine] ** 2)))
+
+
 def test_grouped_nvfp4_gemm_refusals(device):
     lib = ops._lib.load()
     g = ops._lib.GroupedGemm()
