@@ -476,7 +476,7 @@ def other_configs(device, args, only=None):
 
     # Config 5: EXL3 linear 4096 x 14336 at 4 bits, 3INST codebook.
     exl3_names = [f"exl3_linear_4096x14336_4bpw_m{m}" for m in (1, 16)]
-    if any(want(nm) for nm in exl3_names) or want("exl3_multi_linear_4096x2x14336_4bpw_m1"):
+    if any(want(nm) for nm in exl3_names) or want("exl3_multi_linear_4096x2x14336_4bpw_m1") or want("exl3_linear_4096x14336_4bpw_m2048_reconstructed"):
         k, n, bits = 4096, 14336, 4
         trellis, suh, svh = synth.exl3_weights(k, n, bits, 208)
         t0 = dev(trellis)
@@ -500,6 +500,30 @@ def other_configs(device, args, only=None):
                     lambda: oracle.exl3_linear(trellis, suh.view(np.uint16), svh.view(np.uint16), k, n, bits, 0, x_host, threads=threads),
                     t0.numel() / 1e9, "GB/s", 2.5, f"the whole linear at {m} row(s)", threads)
             out[name] = entry
+        # The same linear at a prefill's rows through the fused reconstruction path (the reference's choice from 1,024
+        # rows): the weights to F16 once, then a plain F16 product.
+        if want("exl3_linear_4096x14336_4bpw_m2048_reconstructed"):
+            m = 2048
+            xs = dev(synth.rng(210).standard_normal((m, k)).astype(np.float16).view(np.int16)).view(torch.float16)
+            lib = ops._lib.load()
+            wbuf = torch.empty(k * n * 2, dtype=torch.uint8, device=device)
+            both_us = event_us(lambda i: ops.exl3_linear_reconstructed(trellises[i % len(trellises)], suh_d, svh_d, k, n, bits,
+                                                                       ops.EXL3_3INST, xs, f32=False, fused=True, w=wbuf), 20, warm=40)
+            wt = torch.empty((k, n), dtype=torch.float16, device=device)
+            recon_us = event_us(lambda i: ops.exl3_reconstruct(trellises[i % len(trellises)], suh_d, svh_d, k, n, bits,
+                                                               ops.EXL3_3INST, fused=True), 20, warm=20)
+            del wt
+            flops = 2.0 * m * k * n
+            product_us = both_us - recon_us
+            out["exl3_linear_4096x14336_4bpw_m2048_reconstructed"] = {
+                "workload": "EXL3 linear 4096 x 14336, 4 bits a weight, 2048 rows of fp16 through the fused reconstruction path: "
+                            "the weights to fp16 (both transforms applied), then a plain fp16 product, fp32 sums, fp16 out",
+                "path_us": round(both_us, 1), "reconstruction_us": round(recon_us, 1),
+                "TFLOP/s_of_the_path": round(flops / both_us / 1e6, 1),
+                "roofline": {"bound": "mfma", "achieved": round(flops / product_us / 1e6, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                             "frac": round(flops / product_us / 1e6 / 2500.0, 4), "traffic": None,
+                             "kernel": "GemmKernelHalf (v_mfma_f32_16x16x32_f16): the path's time less the reconstruction's",
+                             "algorithmic_flops_per_launch": int(flops), "avg_launch_us": round(product_us, 2)}}
         if want("exl3_multi_linear_4096x2x14336_4bpw_m1"):
             xs = dev(synth.rng(209).standard_normal((1, k)).astype(np.float16).view(np.int16)).view(torch.float16)
             half = len(trellises) // 2

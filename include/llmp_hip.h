@@ -454,6 +454,22 @@ int llmp_hip_exl3_linear_static(const llmp_exl3_linear* op, void* stream);
  * as the launchers do. */
 int llmp_hip_exl3_linear_static_prepare(const llmp_exl3_linear* op);
 
+/* The reconstruction paths of one linear (ReconstructedLinear, src/kernels/exl3/linear.h:57-60 and linear.cc:87-190,
+ * over ReconstructedOperands, validate.h:263-277; upstream's choice from 145 rows, fused from 1,024): the weights
+ * are reconstructed to F16 a slice of up to 32,768 columns at a time into `w` (llmp_hip_exl3_reconstructed_scratch
+ * bytes: k x min(n, 32,768) halves, ReconstructScratchBytes) and each slice is multiplied by a plain F16 product with
+ * F32 sums into its columns of y. fused: the weights themselves (llmp_hip_exl3_reconstruct_fused's values) times x.
+ * Not fused: the rotated weights times the transformed input (written to op->a_had, m x k halves), then the output's
+ * transform over y in place. The reference's product is cuBLASLt's (recon_gemm.h); this one is the library's own
+ * (the MXFP8 product's loop over F16 operands), which reads both operands along K, so `w` holds a slice column by
+ * column (columns x k), not k x columns: it is scratch of this call, not an interface. x, y, w (and a_had) at
+ * 16-byte boundaries, apart from each other and from the weights. No bias (the reference's add_kernel_hhh is not
+ * built). Results are the linear's definition within F16 rounding of the reconstructed weights (the reference's
+ * bound: 2^-8 of a row's RMS), not bit for bit the packed path's. */
+size_t llmp_hip_exl3_reconstructed_scratch(const llmp_exl3_weights* weights);
+int llmp_hip_exl3_linear_reconstructed(const llmp_exl3_linear* op, void* w, size_t w_bytes, int fused, int compute_units,
+                                       void* stream);
+
 /* exl3.multi_linear.mgemm: MultiLinear of src/kernels/exl3/linear.h:51-53 over the operands of
  * src/kernels/exl3/validate.h:160-172, a gate and an up linear of the same k, n and rate over
  * one input (tests/unit/exl3_trellis_test.cc:664-716). x (m x k F16) into y (2 x m x n: the

@@ -535,14 +535,18 @@ inline std::vector<Implementation> Implementations() {
           d < 2 ? Rung::kNative : Rung::kOnChipDecode, t.needs, {t.launch}, std::string("decoder ") + std::to_string(d));
     }
   }
-  // EXL3 (exl3/implementations.h:8-31): the packed paths; of the reconstruction paths the two reconstruction
-  // kernels are entry points (llmp_hip_exl3_reconstruct, _fused), the plain GEMM after them is the caller's library's.
+  // EXL3 (exl3/implementations.h:8-31): the packed paths and the reconstruction paths.
   add("exl3.linear.gemv", "quant_linear", {"exl3"}, {1, 8, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
       "trellis tiles as the second operand of a 16 x 16 x 16 F16 matrix instruction");
   add("exl3.linear.gemm", "quant_linear", {"exl3"}, {1, 65536, 128, 128}, Rung::kOnChipDecode, kBf16Mma, {"llmp_hip_exl3_linear"},
       "the same launches in passes of sixteen rows");
   add("exl3.multi_linear.mgemm", "quant_multi_linear", {"exl3"}, {1, 65536, 128, 128}, Rung::kOnChipDecode, kBf16Mma,
       {"llmp_hip_exl3_multi_linear"}, "gate and up in grid z, passes of sixteen rows");
+  // (Upstream's choice of path by rows, UpstreamPath above; the entry point itself takes any number from one.)
+  add("exl3.linear.reconstruct", "quant_linear", {"exl3"}, {145, 65536, 128, 128}, Rung::kBf16Decode, kBf16Mma,
+      {"llmp_hip_exl3_linear_reconstructed"}, "input transform, rotated weights to F16 and an F16 product a slice, output transform");
+  add("exl3.linear.reconstruct_fused", "quant_linear", {"exl3"}, {1024, 65536, 128, 128}, Rung::kBf16Decode, kBf16Mma,
+      {"llmp_hip_exl3_linear_reconstructed"}, "the weights themselves to F16 and an F16 product a slice");
   // The quantizing KV cache stores (kv_quant.h:150-192).
   add("llmp.set_rows.quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant"}, "a thread a block");
   add("llmp.set_rows.grouped_quant", "set_rows", {"q8_0", "q4_0"}, {1, any, 32, 1}, Rung::kNative, 0, {"llmp_hip_set_rows_quant_group"},

@@ -157,6 +157,8 @@ SYMBOLS = {
     "llmp_hip_grouped_gemm_run": (_int, [C.POINTER(GroupedGemm), _int, _vp]),
     "llmp_hip_exl3_reconstruct": (_int, [C.POINTER(Exl3Weights), _vp, _int, _int, _vp]),
     "llmp_hip_exl3_reconstruct_fused": (_int, [C.POINTER(Exl3Weights), _vp, _int, _int, _vp]),
+    "llmp_hip_exl3_reconstructed_scratch": (C.c_size_t, [C.POINTER(Exl3Weights)]),
+    "llmp_hip_exl3_linear_reconstructed": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _int, _int, _vp]),
     "llmp_hip_exl3_hadamard": (_int, [_vp, _vp, _vp, _int, _int, _int, _int, _vp]),
     "llmp_hip_exl3_linear_scratch": (C.c_size_t, [C.POINTER(Exl3Linear)]),
     "llmp_hip_exl3_linear": (_int, [C.POINTER(Exl3Linear), _vp, C.c_size_t, _vp]),

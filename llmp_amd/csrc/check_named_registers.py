@@ -1,4 +1,4 @@
-"""The MXFP8 GEMM names the registers of its loop (fragments, scales and sums) in its instructions and holds the
+"""The MXFP8 GEMM (and its F16 sibling, the same loop) names the registers of its loop (fragments, scales and sums) in its instructions and holds the
 compiler to the registers below them. Nothing in the language enforces that split, so this build step reads the
 compiler's assembly of the kernel: no instruction that the compiler wrote may touch a named register, nothing may
 spill, and the kernel's register counts must cover the named ones. Needs hipcc, no GPU. Run by the library's build
@@ -13,7 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 # kernel -> (the compiler's registers v0 .. below this, the highest named register, the sums' registers)
-SHAPES = {"GemmKernel192": (64, 252, 192), "GemmKernel128": (64, 216, 128)}
+SHAPES = {"GemmKernel192": (64, 252, 192), "GemmKernel128": (64, 216, 128),
+          "GemmKernelHalf192": (64, 252, 192), "GemmKernelHalf128": (64, 216, 128)}
 
 
 def kernels(assembly):
@@ -52,7 +53,7 @@ def check():
                 continue
             if not text or text[0] in ";." or text.endswith(":"):
                 continue
-            products += "v_mfma_scale" in text
+            products += "v_mfma_scale" in text or "v_mfma_f32_16x16x32_f16" in text
             if own:
                 continue
             code = text.split(";")[0]

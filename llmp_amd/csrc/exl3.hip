@@ -202,9 +202,11 @@ __device__ __forceinline__ void Hadamard128(float& a, float& b, int lane) {
   for (int mask = 1; mask < 64; mask <<= 1) {
     const float pa = ShflXor(a, mask);
     const float pb = ShflXor(b, mask);
-    const bool upper = (lane & mask) != 0;
-    a = upper ? pa - a : a + pa;
-    b = upper ? pb - b : b + pb;
+    // The partner's value plus or minus this lane's: one fused operation with a sign of one, which rounds as the
+    // addition or subtraction does (the product is exact), where a choice between the two takes three.
+    const float sign = (lane & mask) != 0 ? -1.0f : 1.0f;
+    a = __builtin_fmaf(a, sign, pa);
+    b = __builtin_fmaf(b, sign, pb);
   }
 }
 
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, 
 // Columns [column, column + columns) of the weights themselves, W = diag(suh) H What H diag(svh) / 128 with H the
 // 128-point transform over each block of 128 inputs and of 128 outputs, into w[k][columns] F16 (the reference's
 // reconstruct_had_kernel, launch.cc:440-448; the definition decode.h:37-43). A workgroup of four waves a block of 128
-// inputs by 128 outputs; grid (columns / 128, k / 128); LDS 128 x 129 floats. The rotated values are decoded into
+// inputs by 128 outputs; LDS 128 x 129 floats. The rotated values are decoded into
 // LDS (exact), every column is transformed along the inputs and every row along the outputs in F32 by the wave's
 // butterfly (lane l holds elements l and l + 64 of a vector: the transform does not change when the bits of its
 // index are permuted on both sides, and this assignment reads LDS without bank conflicts both ways), and the block
@@ -281,63 +283,120 @@ __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, 
 constexpr int kHadBlockPitch = 129;
 constexpr int kHadBlockLds = 128 * kHadBlockPitch * 4;
 
-template <int CB, int BITS>
+// kTransform false: the rotated values as they are (the reconstruction without the transforms, through the same
+// block). kTransposed: w[columns][k] instead, a column's inputs together, which is how the product below reads its
+// second operand (both operands' rows along K).
+template <int CB, int BITS, bool kTransform, bool kTransposed>
 __global__ __launch_bounds__(256) void ReconstructHadKernel(const uint32_t* __restrict__ trellis,
                                                            const uint16_t* __restrict__ suh,
                                                            const uint16_t* __restrict__ svh,
-                                                           uint16_t* __restrict__ w, int n, int column, int columns) {
+                                                           uint16_t* __restrict__ w, int n, int k, int column, int columns) {
 #pragma clang fp contract(off)
   extern __shared__ __attribute__((aligned(16))) float had_block[];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int k0 = blockIdx.y * 128;
-  const int c0 = blockIdx.x * 128;  // within the slice
   const Place p = PlaceOf(lane);
-  // Sixteen of the block's 64 tiles a wave.
-#pragma unroll 2
-  for (int t = wave * 16; t < wave * 16 + 16; ++t) {
+  // Sixteen of a block's 64 tiles a wave. A lane's four states lie within three consecutive words of a tile's
+  // stream, the same three in every tile: they are asked for from all sixteen tiles before the first is decoded (a
+  // tile after the other, each decode would wait for its own loads), and a workgroup goes through its blocks (every
+  // gridDim.x-th, columns fastest) with the next block's words asked for ahead of this block's transforms.
+  constexpr int kWords = BITS * 8;
+  const int word0 = (((p.first + 1) * BITS + 256 * BITS - 16) >> 5) % kWords;
+  const int blocks_n = columns / 128;
+  const int blocks = blocks_n * (k / 128);
+  uint32_t words[16][3];
+  auto ask = [&](int block) {
+    const int k_at = (block / blocks_n) * 128, c_at = (block % blocks_n) * 128;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int t = wave * 16 + u;
+      const int kt = t >> 3, nt = t & 7;
+      const uint32_t* tile =
+          trellis + (static_cast<int64_t>(k_at / 16 + kt) * (n / 16) + (column + c_at) / 16 + nt) * kWords;
+#pragma unroll
+      for (int i = 0; i < 3; ++i) words[u][i] = tile[(word0 + i) % kWords];
+    }
+  };
+  if (static_cast<int>(blockIdx.x) < blocks) ask(blockIdx.x);
+  for (int block = blockIdx.x; block < blocks; block += gridDim.x) {
+  const int k0 = (block / blocks_n) * 128;
+  const int c0 = (block % blocks_n) * 128;  // within the slice
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int t = wave * 16 + u;
     const int kt = t >> 3, nt = t & 7;
-    const uint32_t* tile =
-        trellis + (static_cast<int64_t>(k0 / 16 + kt) * (n / 16) + (column + c0) / 16 + nt) * (BITS * 8);
-    const Half4 v = DecodeFour<CB, BITS>(p.first, [&](int i) { return tile[i]; });
+    const Half4 v = DecodeFour<CB, BITS>(p.first, [&](int i) {
+      const int d = (i - word0 + kWords) % kWords;
+      return d == 0 ? words[u][0] : d == 1 ? words[u][1] : words[u][2];
+    });
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const _Float16 value = v[j];
       had_block[(kt * 16 + RowOf(p.g, j)) * kHadBlockPitch + nt * 16 + p.n] = static_cast<float>(value);
     }
   }
+  // (A block past the last is the last again: no load under a branch.)
+  ask(min(block + static_cast<int>(gridDim.x), blocks - 1));
   __syncthreads();
-  // Along the inputs: a wave 32 columns.
-  for (int j = wave * 32; j < wave * 32 + 32; ++j) {
-    float a = had_block[lane * kHadBlockPitch + j];
-    float b = had_block[(lane + 64) * kHadBlockPitch + j];
-    Hadamard128(a, b, lane);
-    had_block[lane * kHadBlockPitch + j] = a;
-    had_block[(lane + 64) * kHadBlockPitch + j] = b;
+  if constexpr (kTransform) {
+    // Along the inputs: a wave 32 columns, four at a time (their exchanges between lanes then overlap).
+    for (int j0 = wave * 32; j0 < wave * 32 + 32; j0 += 4) {
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = had_block[lane * kHadBlockPitch + j0 + u];
+        b[u] = had_block[(lane + 64) * kHadBlockPitch + j0 + u];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) Hadamard128(a[u], b[u], lane);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        had_block[lane * kHadBlockPitch + j0 + u] = a[u];
+        had_block[(lane + 64) * kHadBlockPitch + j0 + u] = b[u];
+      }
+    }
+    __syncthreads();
+    // Along the outputs, then the scales: a wave 32 rows.
+    const float sv_a = HalfBitsToFloat(svh[column + c0 + lane]) * (1.0f / 128.0f);
+    const float sv_b = HalfBitsToFloat(svh[column + c0 + lane + 64]) * (1.0f / 128.0f);
+    for (int i0 = wave * 32; i0 < wave * 32 + 32; i0 += 4) {
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = had_block[(i0 + u) * kHadBlockPitch + lane];
+        b[u] = had_block[(i0 + u) * kHadBlockPitch + lane + 64];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) Hadamard128(a[u], b[u], lane);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float su = HalfBitsToFloat(suh[k0 + i0 + u]);
+        had_block[(i0 + u) * kHadBlockPitch + lane] = a[u] * (su * sv_a);
+        had_block[(i0 + u) * kHadBlockPitch + lane + 64] = b[u] * (su * sv_b);
+      }
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  // Along the outputs, then the scales: a wave 32 rows.
-  const float sv_a = HalfBitsToFloat(svh[column + c0 + lane]) * (1.0f / 128.0f);
-  const float sv_b = HalfBitsToFloat(svh[column + c0 + lane + 64]) * (1.0f / 128.0f);
-  for (int i = wave * 32; i < wave * 32 + 32; ++i) {
-    float a = had_block[i * kHadBlockPitch + lane];
-    float b = had_block[i * kHadBlockPitch + lane + 64];
-    Hadamard128(a, b, lane);
-    const float su = HalfBitsToFloat(suh[k0 + i]);
-    had_block[i * kHadBlockPitch + lane] = a * (su * sv_a);
-    had_block[i * kHadBlockPitch + lane + 64] = b * (su * sv_b);
-  }
-  __syncthreads();
-  // Sixteen bytes a thread: a row is sixteen threads' worth.
+  // Sixteen bytes a thread: a row (a column, transposed) is sixteen threads' worth.
   const int part = threadIdx.x & 15;
   for (int i = threadIdx.x >> 4; i < 128; i += 16) {
-    const float* from = had_block + i * kHadBlockPitch + part * 8;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = kTransposed ? had_block[(part * 8 + e) * kHadBlockPitch + i] : had_block[i * kHadBlockPitch + part * 8 + e];
+    }
     U32x4 out;
-    out.x = FloatToHalfBits(from[0]) | (FloatToHalfBits(from[1]) << 16);
-    out.y = FloatToHalfBits(from[2]) | (FloatToHalfBits(from[3]) << 16);
-    out.z = FloatToHalfBits(from[4]) | (FloatToHalfBits(from[5]) << 16);
-    out.w = FloatToHalfBits(from[6]) | (FloatToHalfBits(from[7]) << 16);
-    *reinterpret_cast<U32x4*>(w + static_cast<int64_t>(k0 + i) * columns + c0 + part * 8) = out;
+    out.x = FloatToHalfBits(v[0]) | (FloatToHalfBits(v[1]) << 16);
+    out.y = FloatToHalfBits(v[2]) | (FloatToHalfBits(v[3]) << 16);
+    out.z = FloatToHalfBits(v[4]) | (FloatToHalfBits(v[5]) << 16);
+    out.w = FloatToHalfBits(v[6]) | (FloatToHalfBits(v[7]) << 16);
+    if constexpr (kTransposed) {
+      *reinterpret_cast<U32x4*>(w + static_cast<int64_t>(c0 + i) * k + k0 + part * 8) = out;
+    } else {
+      *reinterpret_cast<U32x4*>(w + static_cast<int64_t>(k0 + i) * columns + c0 + part * 8) = out;
+    }
+  }
+  __syncthreads();  // the block's readers, before the next is decoded into it
   }
 }
 
@@ -709,15 +768,20 @@ void LaunchReconstruct(const llmp_exl3_weights& w, void* out, int column, int co
                      static_cast<const uint32_t*>(w.trellis), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
 
-template <int CB, int BITS>
+template <int CB, int BITS, bool kTransform, bool kTransposed>
 bool g_reconstruct_had_sized = false;
-template <int CB, int BITS>
+template <int CB, int BITS, bool kTransform, bool kTransposed>
 void LaunchReconstructHad(const llmp_exl3_weights& w, void* out, int column, int columns, hipStream_t stream) {
-  if (!AllowLds(reinterpret_cast<const void*>(&ReconstructHadKernel<CB, BITS>), kHadBlockLds, &g_reconstruct_had_sized<CB, BITS>)) return;
-  const dim3 grid(static_cast<unsigned>(columns / 128), static_cast<unsigned>(w.k / 128));
-  hipLaunchKernelGGL((ReconstructHadKernel<CB, BITS>), grid, dim3(256), kHadBlockLds, stream,
+  if (!AllowLds(reinterpret_cast<const void*>(&ReconstructHadKernel<CB, BITS, kTransform, kTransposed>), kHadBlockLds,
+                &g_reconstruct_had_sized<CB, BITS, kTransform, kTransposed>))
+    return;
+  // Two workgroups a compute unit are resident (LDS): that many go through the blocks.
+  const int blocks = (columns / 128) * (w.k / 128);
+  const int cus = llmp_hip_compute_units() > 0 ? llmp_hip_compute_units() : 256;
+  const dim3 grid(static_cast<unsigned>(blocks < 2 * cus ? blocks : 2 * cus));
+  hipLaunchKernelGGL((ReconstructHadKernel<CB, BITS, kTransform, kTransposed>), grid, dim3(256), kHadBlockLds, stream,
                      static_cast<const uint32_t*>(w.trellis), static_cast<const uint16_t*>(w.suh),
-                     static_cast<const uint16_t*>(w.svh), static_cast<uint16_t*>(out), w.n, column, columns);
+                     static_cast<const uint16_t*>(w.svh), static_cast<uint16_t*>(out), w.n, w.k, column, columns);
 }
 
 template <int BITS>
@@ -815,8 +879,8 @@ extern "C" int llmp_hip_exl3_reconstruct_fused(const llmp_exl3_weights* weights,
       bad != 0)
     return bad;
   Dispatch(weights->codebook, weights->bits, [&](auto cb, auto bits) {
-    LaunchReconstructHad<decltype(cb)::value, decltype(bits)::value>(*weights, w, column, columns,
-                                                                     static_cast<hipStream_t>(stream));
+    LaunchReconstructHad<decltype(cb)::value, decltype(bits)::value, true, false>(*weights, w, column, columns,
+                                                                                  static_cast<hipStream_t>(stream));
   });
   return LaunchStatus("exl3.reconstruct_fused");
 }
@@ -1026,6 +1090,88 @@ extern "C" int llmp_hip_exl3_linear_static_prepare(const llmp_exl3_linear* op) {
     (void)llmp_hip::SizeProduct<decltype(cb)::value, decltype(bits)::value, false>();
   });
   return LaunchStatus("exl3.linear_static_prepare");
+}
+
+namespace llmp_hip {
+// mxfp8.hip: D[m][n] = A[m][k] B[n][k]^T over F16 operands, F32 sums.
+int LaunchHalfGemm(const void* a_rows, const void* b_rows, void* d, int m, int n, int k, int64_t ldd, bool f16_out,
+                   int compute_units, hipStream_t stream);
+}  // namespace llmp_hip
+
+constexpr int kReconstructSlice = 32768;  // validate.h:257-261: columns a slice of the reconstruction
+
+extern "C" size_t llmp_hip_exl3_reconstructed_scratch(const llmp_exl3_weights* weights) {
+  if (weights == nullptr || weights->k <= 0 || weights->n <= 0) return 0;
+  const int columns = weights->n < kReconstructSlice ? weights->n : kReconstructSlice;
+  return static_cast<size_t>(weights->k) * columns * 2;
+}
+
+extern "C" int llmp_hip_exl3_linear_reconstructed(const llmp_exl3_linear* op, void* w, size_t w_bytes, int fused,
+                                                  int compute_units, void* stream) {
+  BeginLaunches();
+  if (op == nullptr || w == nullptr) return Refuse(1, "exl3.linear_reconstructed: null operands");
+  const llmp_exl3_weights& weights = op->weights;
+  if (const int bad = llmp_hip::CheckWeights(weights); bad != 0) return bad;
+  if (op->x == nullptr || op->y == nullptr || (!fused && op->a_had == nullptr)) return Refuse(1, "exl3.linear_reconstructed: null operand");
+  if (op->m < 1 || op->m > 65536) return Refuse(1, "exl3.linear_reconstructed: 1 to 65536 rows, not %d", op->m);
+  if (static_cast<int64_t>(op->m) * weights.k * 2 >= (int64_t{1} << 32)) return Refuse(1, "exl3.linear_reconstructed: an input of 4 GiB or more");
+  const size_t needs = llmp_hip_exl3_reconstructed_scratch(&weights);
+  if (w_bytes < needs) return Refuse(1, "exl3.linear_reconstructed: %zu bytes of weight scratch, %zu needed", w_bytes, needs);
+  const uintptr_t aligned = reinterpret_cast<uintptr_t>(op->x) | reinterpret_cast<uintptr_t>(op->y) | reinterpret_cast<uintptr_t>(w) |
+                            (fused ? 0 : reinterpret_cast<uintptr_t>(op->a_had));
+  if (aligned % 16 != 0) return Refuse(1, "exl3.linear_reconstructed: operands not 16-byte aligned");
+  {
+    // validate.cc:508-539: the scratch the path writes meets nothing it later reads or writes, and nothing it writes
+    // holds the weights.
+    const size_t cells = static_cast<size_t>(op->m) * weights.k;
+    const llmp_hip::Range x{"x", reinterpret_cast<uintptr_t>(op->x), cells * 2};
+    const llmp_hip::Range xh{"xh", fused ? 0 : reinterpret_cast<uintptr_t>(op->a_had), fused ? 0 : cells * 2};
+    const llmp_hip::Range wr{"w", reinterpret_cast<uintptr_t>(w), needs};
+    const llmp_hip::Range y{"y", reinterpret_cast<uintptr_t>(op->y), static_cast<size_t>(op->m) * weights.n * (op->f32 ? 4 : 2)};
+    if (const int bad = llmp_hip::Disjoint("exl3.linear_reconstructed", wr, {x, xh, y}); bad != 0) return bad;
+    if (const int bad = llmp_hip::Disjoint("exl3.linear_reconstructed", xh, {x, y}); bad != 0) return bad;
+    if (const int bad = llmp_hip::Disjoint("exl3.linear_reconstructed", y, {x}); bad != 0) return bad;
+    for (const llmp_hip::Range& written : {xh, wr, y}) {
+      if (const int bad = llmp_hip::Disjoint("exl3.linear_reconstructed", written,
+                                             {llmp_hip::TrellisRange(weights), llmp_hip::SuhRange(weights), llmp_hip::SvhRange(weights)});
+          bad != 0)
+        return bad;
+    }
+  }
+  const auto s = static_cast<hipStream_t>(stream);
+  const auto* suh = static_cast<const uint16_t*>(weights.suh);
+  const auto* svh = static_cast<const uint16_t*>(weights.svh);
+  const void* product_input = op->x;
+  if (!fused) {
+    // The input's transform, y = H(x * suh) / sqrt(128), as the packed path's.
+    hipLaunchKernelGGL((llmp_hip::HadamardKernel<0, 0>), dim3(static_cast<unsigned>(op->m), static_cast<unsigned>(weights.k / 128)), dim3(64),
+                       0, s, llmp_hip::OneSide(op->x, op->a_had, suh, nullptr), weights.k, 1, int64_t{0});
+    product_input = op->a_had;
+  }
+  for (int column = 0; column < weights.n; column += kReconstructSlice) {
+    const int columns = weights.n - column < kReconstructSlice ? weights.n - column : kReconstructSlice;
+    // The slice's weights, a column's inputs together (the product reads both operands along K).
+    llmp_hip::Dispatch(weights.codebook, weights.bits, [&](auto cb, auto bits) {
+      if (fused) {
+        llmp_hip::LaunchReconstructHad<decltype(cb)::value, decltype(bits)::value, true, true>(weights, w, column, columns, s);
+      } else {
+        llmp_hip::LaunchReconstructHad<decltype(cb)::value, decltype(bits)::value, false, true>(weights, w, column, columns, s);
+      }
+    });
+    void* y_at = op->f32 ? static_cast<void*>(static_cast<float*>(op->y) + column) : static_cast<void*>(static_cast<uint16_t*>(op->y) + column);
+    if (const int bad = llmp_hip::LaunchHalfGemm(product_input, w, y_at, op->m, columns, weights.k, weights.n, !op->f32, compute_units, s); bad != 0)
+      return bad;
+  }
+  if (!fused) {
+    // The output's transform in place, y = H(y) / sqrt(128) * svh.
+    const dim3 grid(static_cast<unsigned>(op->m), static_cast<unsigned>(weights.n / 128));
+    if (op->f32) {
+      hipLaunchKernelGGL((llmp_hip::HadamardKernel<1, 1>), grid, dim3(64), 0, s, llmp_hip::OneSide(op->y, op->y, nullptr, svh), weights.n, 1, int64_t{0});
+    } else {
+      hipLaunchKernelGGL((llmp_hip::HadamardKernel<0, 0>), grid, dim3(64), 0, s, llmp_hip::OneSide(op->y, op->y, nullptr, svh), weights.n, 1, int64_t{0});
+    }
+  }
+  return LaunchStatus("exl3.linear_reconstructed");
 }
 
 extern "C" size_t llmp_hip_exl3_multi_linear_scratch(const llmp_exl3_multi_linear* op) {

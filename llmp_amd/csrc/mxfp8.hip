@@ -252,9 +252,10 @@ struct GemmArgs {
   const uint8_t* b;         // weights, n rows of k codes
   const uint8_t* b_scales;  // atoms
   void* d;
-  int m, n, k;
-  int bf16;
+  int m, n, k;  // k: bytes of a row of either operand (the codes of a step are 128 of them)
+  int bf16;     // D's elements: 0 F32, 1 BF16, 2 F16
   int tiles_m, tiles_n;
+  int64_t ldd;  // elements between D's rows
 };
 
 // LDS of GemmKernel<WN>: activation tiles, weight tiles, activation scales, weight scales.
@@ -387,6 +388,20 @@ __device__ __forceinline__ void ScaledProduct() {
         "n"(R::W(I, P)), "n"(R::X(J, P)), "n"(R::WScale(I, P)), "n"(R::XScale(J, P)));
   }
 }
+// The same for F16 operands (a step's 128 bytes a row are 64 values: the fragment's lower chunk is one product's K,
+// its upper chunk the next one's): two v_mfma_f32_16x16x32_f16 into the same sums, no scales.
+template <class R, int T, int I, int J, int P = 0, bool FIRST = false>
+__device__ __forceinline__ void HalfProduct() {
+  if constexpr (FIRST) {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%0:%0+3], v[%1:%1+3], v[%2:%2+3], 0\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%0:%0+3], v[%1+4:%1+7], v[%2+4:%2+7], a[%0:%0+3]" ::"n"(T * 4),
+                 "n"(R::W(I, P)), "n"(R::X(J, P)));
+  } else {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%0:%0+3], v[%1:%1+3], v[%2:%2+3], a[%0:%0+3]\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%0:%0+3], v[%1+4:%1+7], v[%2+4:%2+7], a[%0:%0+3]" ::"n"(T * 4),
+                 "n"(R::W(I, P)), "n"(R::X(J, P)));
+  }
+}
 template <int REG>
 __device__ __forceinline__ void ClearSum() {
   asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(REG));
@@ -406,7 +421,8 @@ __device__ __forceinline__ uint32_t PackBf16(float lo, float hi) {
   return packed;
 }
 
-template <int WM, int WN, int RA>
+// kHalf: the operands are rows of F16 values and there are no scales (the reconstruction paths' product).
+template <int WM, int WN, int RA, bool kHalf = false>
 __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   using L = GemmLds<WN, RA>;
   using R = GemmRegs<WM, WN>;
@@ -494,6 +510,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   // A stage's scales: wave 0 the activations' into stage_a, wave 1 the weights' into stage_b. (A wave-uniform branch
   // around one load each: the waits below count a wave's loads, and these waves have one more.)
   auto load_scales = [&](int step_a, int stage_a, int step_b, int stage_b) {
+    if constexpr (kHalf) return;
     if (wave == 0) {
       GlobalToLds16(scales_of + step_a * 512, scale_from, lds_at + static_cast<uint32_t>(L::kAScales + stage_a * kScaleStageBytes));
     } else if (wave == 1) {
@@ -541,7 +558,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   auto read_a_hi = [&](auto jc, auto pc) {
     constexpr int j = decltype(jc)::value, p = decltype(pc)::value;
     LdsToRegs16<R::X(j, p) + 4, j * 2048>(a_hi);
-    LdsToReg1<R::XScale(j, p), (j % 2) * 256 + (j / 2) * 4>(a_scale);
+    if constexpr (!kHalf) LdsToReg1<R::XScale(j, p), (j % 2) * 256 + (j / 2) * 4>(a_scale);
   };
   auto read_b_lo = [&](auto ic, auto pc) {
     constexpr int i = decltype(ic)::value, p = decltype(pc)::value;
@@ -550,7 +567,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   auto read_b_hi = [&](auto ic, auto pc) {
     constexpr int i = decltype(ic)::value, p = decltype(pc)::value;
     LdsToRegs16<R::W(i, p) + 4, i * 2048>(b_hi);
-    LdsToReg1<R::WScale(i, p), 0>(b_scale + static_cast<uint32_t>(scale_b_off[i]));
+    if constexpr (!kHalf) LdsToReg1<R::WScale(i, p), 0>(b_scale + static_cast<uint32_t>(scale_b_off[i]));
   };
   auto read_a = [&](auto jc, auto pc) {
     read_a_lo(jc, pc);
@@ -580,10 +597,12 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
 #pragma unroll
         for (int i = 0; i < kLoadsB; ++i) load_b(i, step, stage);
       }
-      if (wave == 0) {
-        if constexpr (stage < RA) load_scales(step, stage, step, stage);
-      } else if (wave == 1) {
-        if constexpr (stage < kRingB) load_scales(step, stage, step, stage);
+      if constexpr (!kHalf) {
+        if (wave == 0) {
+          if constexpr (stage < RA) load_scales(step, stage, step, stage);
+        } else if (wave == 1) {
+          if constexpr (stage < kRingB) load_scales(step, stage, step, stage);
+        }
       }
     });
   };
@@ -614,7 +633,11 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
       constexpr int j = decltype(jc)::value;
       StaticFor<WN>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        ScaledProduct<R, kXFrags * i + j, i, j, P, kFirst>();
+        if constexpr (kHalf) {
+          HalfProduct<R, kXFrags * i + j, i, j, P, kFirst>();
+        } else {
+          ScaledProduct<R, kXFrags * i + j, i, j, P, kFirst>();
+        }
         constexpr int t = j * WN + i;
         constexpr int q = t % kLoadEvery == 0 ? t / kLoadEvery : kLoadsA + 1 + kLoadsB;  // the load after product t
         if constexpr (q < kLoadsA) {
@@ -642,7 +665,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     // Step + 2 has landed: with two activation stages all but the weights just asked for (and their scales, wave 1),
     // with three everything asked for before this iteration (loads complete in the order they were asked for).
     constexpr int kLeft = RA == 2 ? kLoadsB : kLoadsA + kLoadsB;
-    if (wave == 1 || (RA > 2 && wave == 0)) {
+    if (!kHalf && (wave == 1 || (RA > 2 && wave == 0))) {
       AwaitLoads<kLeft + 1>();
     } else {
       AwaitLoads<kLeft>();
@@ -657,9 +680,9 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
     int m0, n0;
     origin(of, m0, n0);
     const int m_first = m0 + wm * 16 * kXFrags + r, n_first = n0 + wn * 16 * WN + 4 * g;  // n is a multiple of 4 (checked on the host)
-    const int64_t first = static_cast<int64_t>(m_first) * a.n + n_first;
-    const int64_t row_step = static_cast<int64_t>(a.n) * 16;
-    auto store = [&](auto bf16, auto whole) {
+    const int64_t first = static_cast<int64_t>(m_first) * a.ldd + n_first;
+    const int64_t row_step = a.ldd * 16;
+    auto store = [&](auto kind, auto whole) {
       StaticFor<kXFrags>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         StaticFor<WN>([&](auto ic) {
@@ -668,10 +691,15 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
           const float v0 = ReadSum<reg>(), v1 = ReadSum<reg + 1>(), v2 = ReadSum<reg + 2>(), v3 = ReadSum<reg + 3>();
           if (!decltype(whole)::value && (m_first + 16 * j >= a.m || n_first + 16 * i >= a.n)) return;
           const int64_t at = first + j * row_step + i * 16;
-          if constexpr (decltype(bf16)::value) {
+          if constexpr (decltype(kind)::value == 1) {
             uint2 packed;
             packed.x = PackBf16(v0, v1);
             packed.y = PackBf16(v2, v3);
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + at) = packed;
+          } else if constexpr (decltype(kind)::value == 2) {
+            uint2 packed;
+            packed.x = FloatToHalfBits(v0) | (FloatToHalfBits(v1) << 16);
+            packed.y = FloatToHalfBits(v2) | (FloatToHalfBits(v3) << 16);
             *reinterpret_cast<uint2*>(static_cast<uint16_t*>(a.d) + at) = packed;
           } else {
             *reinterpret_cast<float4*>(static_cast<float*>(a.d) + at) = make_float4(v0, v1, v2, v3);
@@ -680,17 +708,34 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
       });
     };
     const bool whole = m0 + kTileM <= a.m && n0 + kTileN <= a.n;
-    if (a.bf16) {
-      if (whole) {
-        store(std::true_type{}, std::true_type{});
+    using F32Out = std::integral_constant<int, 0>;
+    using Bf16Out = std::integral_constant<int, 1>;
+    using F16Out = std::integral_constant<int, 2>;
+    if constexpr (kHalf) {  // F16 or F32
+      if (a.bf16 == 2) {
+        if (whole) {
+          store(F16Out{}, std::true_type{});
+        } else {
+          store(F16Out{}, std::false_type{});
+        }
       } else {
-        store(std::true_type{}, std::false_type{});
+        if (whole) {
+          store(F32Out{}, std::true_type{});
+        } else {
+          store(F32Out{}, std::false_type{});
+        }
+      }
+    } else if (a.bf16) {
+      if (whole) {
+        store(Bf16Out{}, std::true_type{});
+      } else {
+        store(Bf16Out{}, std::false_type{});
       }
     } else {
       if (whole) {
-        store(std::false_type{}, std::true_type{});
+        store(F32Out{}, std::true_type{});
       } else {
-        store(std::false_type{}, std::false_type{});
+        store(F32Out{}, std::false_type{});
       }
     }
   };
@@ -698,7 +743,7 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   aim_loads(0);
   first_loads();
   for (; ord < mine; ++ord) {
-    aim_weight_scales(ord);
+    if constexpr (!kHalf) aim_weight_scales(ord);
     // The tile's first stages have landed (they were asked for ahead of the tile before's stores, which this wait
     // counts as well), for every wave.
     AwaitLoads<0>();
@@ -740,15 +785,22 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompiler
   GemmTiles<2, 4, 2>(a);
 }
 constexpr int kWavesM128 = 2, kRingA128 = 2;
+// The same two shapes over F16 operands.
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernelHalf192(const GemmArgs a) {
+  GemmTiles<2, 6, 2, true>(a);
+}
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_num_vgpr(GemmCompilerVgprs(2)))) void GemmKernelHalf128(const GemmArgs a) {
+  GemmTiles<2, 4, 2, true>(a);
+}
 
 
 // A workgroup a compute unit, each through its share of the tiles (fewer workgroups where there are fewer tiles).
-template <int WM, int WN, int RA>
+template <int WM, int WN, int RA, bool kHalf = false>
 int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, int compute_units, hipStream_t stream) {
   using L = GemmLds<WN, RA>;
   static_assert(L::kBytes <= 160 * 1024, "the stages do not fit a CU's LDS");
   a.tiles_n = (a.n + L::kTileN - 1) / L::kTileN;
-  static bool sized = false;
+  static bool sized = false;  // (one a kernel: the template's arguments name it)
   if (!AllowLds(reinterpret_cast<const void*>(kernel), L::kBytes, &sized)) return LaunchStatus("mxfp8.gemm");
   const int tiles = a.tiles_m * a.tiles_n;
   hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles < compute_units ? tiles : compute_units)), dim3(WM * 128), L::kBytes, stream, a);
@@ -756,6 +808,37 @@ int LaunchGemm(void (*kernel)(const GemmArgs), GemmArgs a, int compute_units, hi
 }
 
 }  // namespace
+
+// D[m][n] (rows ldd elements apart; F16 if f16_out, else F32) = A[m][k] B[n][k]^T over F16 operands whose rows follow
+// each other, F32 sums: the MXFP8 product's loop with two F16 products where it has a scaled one. k a multiple of 64,
+// n of 4, operands and D at 16-byte boundaries (the caller's checks). Queues one launch.
+int LaunchHalfGemm(const void* a_rows, const void* b_rows, void* d, int m, int n, int k, int64_t ldd, bool f16_out,
+                   int compute_units, hipStream_t stream) {
+  GemmArgs a;
+  a.a = static_cast<const uint8_t*>(a_rows);
+  a.a_scales = nullptr;
+  a.b = static_cast<const uint8_t*>(b_rows);
+  a.b_scales = nullptr;
+  a.d = d;
+  a.m = m;
+  a.n = n;
+  a.k = 2 * k;
+  a.bf16 = f16_out ? 2 : 0;
+  a.ldd = ldd;
+  a.tiles_m = (m + kTileM - 1) / kTileM;
+  a.tiles_n = 0;
+  const int cus = compute_units > 0 ? compute_units : 256;
+  int best = 0;
+  int64_t best_cost = 0;
+  for (const int tile_n : {192, 128}) {
+    const int64_t tiles = static_cast<int64_t>(a.tiles_m) * ((n + tile_n - 1) / tile_n);
+    const int64_t cost = (tiles + cus - 1) / cus * tile_n;
+    if (best == 0 || cost < best_cost) best = tile_n, best_cost = cost;
+  }
+  return best == 192 ? LaunchGemm<2, 6, 2, true>(GemmKernelHalf192, a, cus, stream)
+                     : LaunchGemm<kWavesM128, 4, kRingA128, true>(GemmKernelHalf128, a, cus, stream);
+}
+
 }  // namespace llmp_hip
 
 using namespace llmp_hip;
@@ -871,6 +954,7 @@ extern "C" int llmp_hip_mxfp8_gemm_run(const llmp_mxfp8_gemm* gemm, int compute_
   a.n = gemm->n;
   a.k = gemm->k;
   a.bf16 = gemm->bf16 != 0 ? 1 : 0;
+  a.ldd = gemm->n;
   a.tiles_m = (gemm->m + kTileM - 1) / kTileM;
   a.tiles_n = 0;
   // The weight rows a workgroup takes (192 or 128): whichever leaves the fewest idle

@@ -471,6 +471,25 @@ def exl3_linear(trellis, suh, svh, k, n, bits, codebook, x, f32=True, keep=None)
     return y
 
 
+def exl3_linear_reconstructed(trellis, suh, svh, k, n, bits, codebook, x, f32=True, fused=True, w=None):
+    """The same linear through a reconstruction path (the reference's ReconstructedLinear, upstream's choice from 145
+    rows; fused from 1,024): the weights reconstructed to float16 a slice at a time into the scratch `w`, a plain
+    float16 product with float32 sums a slice. x float16 [m, k]: [m, n] float32 or float16."""
+    lib = _lib.load()
+    m = x.shape[0]
+    op = Exl3Linear()
+    op.weights = _exl3_weights(trellis, suh, svh, k, n, bits, codebook)
+    a_had = torch.empty((m, k), dtype=torch.float16, device=x.device)
+    y = torch.empty((m, n), dtype=torch.float32 if f32 else torch.float16, device=x.device)
+    op.x, op.a_had, op.y, op.f32, op.m = x.data_ptr(), a_had.data_ptr(), y.data_ptr(), int(f32), m
+    need = lib.llmp_hip_exl3_reconstructed_scratch(C.byref(op.weights))
+    if w is None:
+        w = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _lib.check(lib.llmp_hip_exl3_linear_reconstructed(C.byref(op), _ptr(w), w.numel() * w.element_size(), int(fused),
+                                                      lib.llmp_hip_compute_units(), _stream()))
+    return y
+
+
 def exl3_linear_static(trellis, suh, svh, k, n, bits, codebook, x, a_had, y):
     """The same linear through llmp_hip_exl3_linear_static: the partial sums go to the library's static array
     on this device, the call allocates nothing. x float16 [m, k]; a_had float16 [m, k] and y float32 or

@@ -198,6 +198,9 @@ void RegistryChecks() {
   q.op = "quant_linear", q.encoding = "exl3", q.rows = 16, q.k = 4096, q.n = 14336;
   found = ex::Candidates(q);
   EXPECT(found.size() == 1 && found[0].name == "exl3.linear.gemm");
+  q.rows = 2048;  // the packed path still computes it; the reconstruction paths are candidates from their rows on
+  found = ex::Candidates(q);
+  EXPECT(found.size() == 3);
   q.arch = 942;
   EXPECT(ex::Candidates(q).empty());
 

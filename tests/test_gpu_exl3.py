@@ -173,6 +173,55 @@ def test_linear_of_more_than_sixteen_rows_runs_in_passes(device, m):
         assert np.array_equal(both[1].view(np.uint32), alone.view(np.uint32))
 
 
+@pytest.mark.parametrize("m,k,n,bits,codebook", [(200, 1024, 512, 4, ops.EXL3_3INST), (300, 256, 384, 3, ops.EXL3_MCG),
+                                                 (1, 128, 128, 5, ops.EXL3_MUL1), (130, 128, 32768 + 256, 2, ops.EXL3_3INST)])
+@pytest.mark.parametrize("fused", [True, False])
+def test_reconstruction_paths_of_the_linear(device, m, k, n, bits, codebook, fused):
+    """ReconstructedLinear (src/kernels/exl3/linear.cc:87-190 of the reference; its test
+    tests/unit/exl3_trellis_test.cc:519-564): the weights reconstructed to F16 a slice at a time, a plain F16 product
+    with F32 sums a slice; partial tiles of rows, two slices of columns. Against the F64 product with the decoded
+    rows within the reference's bounds (2^-8 of a row's RMS; any output within 2^-5 of it), and stage by stage over
+    the device's own reconstructed weights (and transformed input): what is left is the order of F32 sums, 1e-3."""
+    trellis, suh, svh = synth.exl3_weights(k, n, bits, 500 + bits)
+    x = synth.rng(501 + m).standard_normal((m, k)).astype(np.float16)
+    args = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, bits, codebook)
+    got = ops.exl3_linear_reconstructed(*args, halves(x, device), f32=True, fused=fused).cpu().numpy().astype(np.float64)
+    rows = oracle.exl3_rows(trellis, suh.view(np.uint16), svh.view(np.uint16), k, n, bits, codebook).astype(np.float64)
+    ref = x.astype(np.float64) @ rows.T
+    for r in range(m):
+        rms = np.sqrt(np.mean(ref[r] ** 2))
+        assert np.sqrt(np.mean((got[r] - ref[r]) ** 2)) <= 2.0 ** -8 * rms
+        assert np.abs(got[r] - ref[r]).max() <= 2.0 ** -5 * rms
+    if fused:
+        w = np.concatenate([ops.exl3_reconstruct(*args, column=c, columns=min(32768, n - c), fused=True).float().cpu().numpy()
+                            for c in range(0, n, 32768)], axis=1).astype(np.float64)
+        want = x.astype(np.float64) @ w
+        ok, worst = rel_close(got, want, 1e-3)
+        assert ok, worst
+    else:
+        # The same definition as the packed path's: its output over the same rows agrees to the sums' order and the
+        # rounding of the transformed input (one F16 step of a value in a hundred).
+        packed = np.concatenate([ops.exl3_linear(*args, halves(x[i:i + 16], device)).cpu().numpy() for i in range(0, m, 16)])
+        ok, worst = rel_close(got, packed.astype(np.float64), 2e-3)
+        assert ok, worst
+    half = ops.exl3_linear_reconstructed(*args, halves(x, device), f32=False, fused=fused).float().cpu().numpy()
+    for r in range(0, m, 7):
+        rms = np.sqrt(np.mean(ref[r] ** 2))
+        assert np.sqrt(np.mean((half[r] - ref[r]) ** 2)) <= 2.0 ** -8 * rms
+
+
+def test_reconstruction_path_refusals(device):
+    k, n = 256, 256
+    trellis, suh, svh = synth.exl3_weights(k, n, 4, 41)
+    args = (dev(trellis, device), halves(suh, device), halves(svh, device), k, n, 4, 0)
+    x = halves(synth.rng(1).standard_normal((8, k)).astype(np.float16), device)
+    with pytest.raises(ops.KernelFailure) as e:
+        ops.exl3_linear_reconstructed(*args, x, w=torch.empty(1024, dtype=torch.uint8, device=device))
+    assert e.value.rejected and "scratch" in e.value.detail
+    with pytest.raises(ops.KernelFailure):
+        ops.exl3_linear_reconstructed(*args, x[:0])
+
+
 def test_refusals(device):
     trellis, suh, svh = synth.exl3_weights(128, 128, 4, 41)
     x = halves(np.zeros((2, 128), dtype=np.float16), device)
