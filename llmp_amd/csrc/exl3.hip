@@ -210,6 +210,34 @@ __device__ __forceinline__ void Hadamard128(float& a, float& b, int lane) {
   }
 }
 
+// The same transform of four vectors a wave, one a row of sixteen lanes: lane l of a row holds elements l + 16 e,
+// e = 0 .. 7. (The transform does not change when the bits of its index are permuted on both sides.) The three index
+// bits that e holds are butterflies within the lane, the four that l holds exchanges within the row, which are
+// data-parallel moves: nothing passes through LDS, and a value costs twelve operations where the wave-wide form
+// takes over twenty. `sign[b]`: -1 where bit b of l is set, else 1.
+__device__ __forceinline__ void Hadamard128Rows(float (&x)[8], const float (&sign)[4]) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int bit = 1; bit < 8; bit <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if ((e & bit) == 0) {
+        const float sum = x[e] + x[e | bit];
+        x[e | bit] = x[e] - x[e | bit];
+        x[e] = sum;
+      }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float other = ShflXor(x[e], 1 << b);
+      x[e] = __builtin_fmaf(x[e], sign[b], other);
+    }
+  }
+}
+
 // y = f(H(x * in_scale)) * r * out_scale over each 128 block of each row; grid (rows, columns
 // / 128), a wave a block. X / Y: 0 F16, 1 F32. `slices` partial inputs are added in order first.
 // One or two transforms a launch (grid z): a linear's, or the two of a gate/up pair.
@@ -276,10 +304,9 @@ __global__ __launch_bounds__(64) void HadamardKernel(const HadamardSides sides, 
 // 128-point transform over each block of 128 inputs and of 128 outputs, into w[k][columns] F16 (the reference's
 // reconstruct_had_kernel, launch.cc:440-448; the definition decode.h:37-43). A workgroup of four waves a block of 128
 // inputs by 128 outputs; LDS 128 x 129 floats. The rotated values are decoded into
-// LDS (exact), every column is transformed along the inputs and every row along the outputs in F32 by the wave's
-// butterfly (lane l holds elements l and l + 64 of a vector: the transform does not change when the bits of its
-// index are permuted on both sides, and this assignment reads LDS without bank conflicts both ways), and the block
-// is rounded to F16 once, after the scales: the reference's kernel rounds every butterfly to F16.
+// LDS (exact), every column is transformed along the inputs and every row along the outputs in F32 (four vectors a
+// wave at a time, Hadamard128Rows), and the block is rounded to F16 once, after the scales: the reference's kernel
+// rounds every butterfly to F16.
 constexpr int kHadBlockPitch = 129;
 constexpr int kHadBlockLds = 128 * kHadBlockPitch * 4;
 
@@ -296,6 +323,10 @@ __global__ __launch_bounds__(256) void ReconstructHadKernel(const uint32_t* __re
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const Place p = PlaceOf(lane);
+  const int l16 = lane & 15, row4 = lane >> 4;
+  float sign[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) sign[b] = (l16 >> b) & 1 ? -1.0f : 1.0f;
   // Sixteen of a block's 64 tiles a wave. A lane's four states lie within three consecutive words of a tile's
   // stream, the same three in every tile: they are asked for from all sixteen tiles before the first is decoded (a
   // tile after the other, each decode would wait for its own loads), and a workgroup goes through its blocks (every
@@ -339,41 +370,28 @@ __global__ __launch_bounds__(256) void ReconstructHadKernel(const uint32_t* __re
   ask(min(block + static_cast<int>(gridDim.x), blocks - 1));
   __syncthreads();
   if constexpr (kTransform) {
-    // Along the inputs: a wave 32 columns, four at a time (their exchanges between lanes then overlap).
-    for (int j0 = wave * 32; j0 < wave * 32 + 32; j0 += 4) {
-      float a[4], b[4];
+    // Along the inputs: a wave 32 columns, four at a time, one a row of sixteen lanes (Hadamard128Rows).
+    for (int j = wave * 32 + row4; j < wave * 32 + 32; j += 4) {
+      float x[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        a[u] = had_block[lane * kHadBlockPitch + j0 + u];
-        b[u] = had_block[(lane + 64) * kHadBlockPitch + j0 + u];
-      }
+      for (int e = 0; e < 8; ++e) x[e] = had_block[(l16 + 16 * e) * kHadBlockPitch + j];
+      Hadamard128Rows(x, sign);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) Hadamard128(a[u], b[u], lane);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        had_block[lane * kHadBlockPitch + j0 + u] = a[u];
-        had_block[(lane + 64) * kHadBlockPitch + j0 + u] = b[u];
-      }
+      for (int e = 0; e < 8; ++e) had_block[(l16 + 16 * e) * kHadBlockPitch + j] = x[e];
     }
     __syncthreads();
     // Along the outputs, then the scales: a wave 32 rows.
-    const float sv_a = HalfBitsToFloat(svh[column + c0 + lane]) * (1.0f / 128.0f);
-    const float sv_b = HalfBitsToFloat(svh[column + c0 + lane + 64]) * (1.0f / 128.0f);
-    for (int i0 = wave * 32; i0 < wave * 32 + 32; i0 += 4) {
-      float a[4], b[4];
+    float sv[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        a[u] = had_block[(i0 + u) * kHadBlockPitch + lane];
-        b[u] = had_block[(i0 + u) * kHadBlockPitch + lane + 64];
-      }
+    for (int e = 0; e < 8; ++e) sv[e] = HalfBitsToFloat(svh[column + c0 + l16 + 16 * e]) * (1.0f / 128.0f);
+    for (int i = wave * 32 + row4; i < wave * 32 + 32; i += 4) {
+      float x[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) Hadamard128(a[u], b[u], lane);
+      for (int e = 0; e < 8; ++e) x[e] = had_block[i * kHadBlockPitch + l16 + 16 * e];
+      Hadamard128Rows(x, sign);
+      const float su = HalfBitsToFloat(suh[k0 + i]);
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float su = HalfBitsToFloat(suh[k0 + i0 + u]);
-        had_block[(i0 + u) * kHadBlockPitch + lane] = a[u] * (su * sv_a);
-        had_block[(i0 + u) * kHadBlockPitch + lane + 64] = b[u] * (su * sv_b);
-      }
+      for (int e = 0; e < 8; ++e) had_block[i * kHadBlockPitch + l16 + 16 * e] = x[e] * (su * sv[e]);
     }
     __syncthreads();
   }
