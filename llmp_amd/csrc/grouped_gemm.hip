@@ -161,9 +161,15 @@ __global__ __launch_bounds__(kThreads, 3) void GroupedNvfp4Kernel(const GroupedA
     }
     __syncthreads();
     const int total = s_before[kChunk];
-    // This workgroup's tiles of the chunk: every gridDim.x-th of the whole list.
-    int t = (static_cast<int>(blockIdx.x) - base % static_cast<int>(gridDim.x) + static_cast<int>(gridDim.x)) % static_cast<int>(gridDim.x);
-    for (; t < total; t += gridDim.x) {
+    // This workgroup's tiles of the chunk: every gridDim.x-th place of the whole list, a place p holding tile
+    // (p % 8) * ceil(total / 8) + p / 8. Workgroups go to the device's eight dies in turn, so with a grid that is a multiple of
+    // eight (the usual compute-unit counts) a die takes a run of consecutive tiles: a group's tiles, which read the same rows of A, share that
+    // die's L2 (spread over the dies, every die fetched A for itself: 1.4 times the bytes).
+    const int run = (total + 7) / 8;
+    int place = (static_cast<int>(blockIdx.x) - base % static_cast<int>(gridDim.x) + static_cast<int>(gridDim.x)) % static_cast<int>(gridDim.x);
+    for (; place < 8 * run; place += gridDim.x) {
+      const int t = (place & 7) * run + (place >> 3);
+      if (t >= total) continue;
       // The last group whose tiles start at or before t (groups without tiles share their start with the next).
       int lo = 0, hi = count - 1;
       while (lo < hi) {
@@ -269,7 +275,7 @@ __global__ __launch_bounds__(kThreads, 3) void GroupedNvfp4Kernel(const GroupedA
         }
       }
     }
-    base += total;
+    base += 8 * run;
   }
 }
 
