@@ -352,17 +352,11 @@ def other_configs(device, args, only=None):
             h = torch.empty((pairs, ffn), dtype=torch.float32, device=device)
             gu_stride = 2 * ffn * (hidden // qk)
             up_of = lambda g: g.view(-1)[ffn * (hidden // qk) * 144:]
-            if pairs <= 64:
+            if pairs <= 128:
                 product = lambda i: ops.vecq_fused(ops.TYPE_Q4_K, up_of(gus[i % sets]), xs, hidden, ffn, gate=gus[i % sets], ids=ids,
                                                    tokens=tokens, used=used, stride_expert=gu_stride, glu=ops.GLU_SWIGLU,
                                                    out=h.view(tokens, used, ffn))
-                kernel = "VecQFlat<FormatQ4K, glu, in-kernel q8_1> routed (gate/up)"
-            elif pairs <= 128:
-                q8 = ops.quantize_q8_1(xs)
-                product = lambda i: ops.vecq(ops.TYPE_Q4_K, up_of(gus[i % sets]), q8, hidden, ffn, gate=gus[i % sets], ids=ids,
-                                             tokens=tokens, used=used, stride_expert=gu_stride, glu=ops.GLU_SWIGLU,
-                                             out=h.view(tokens, used, ffn))
-                kernel = "VecQFlat<FormatQ4K, 4 tokens a pass, glu> routed (gate/up)"
+                kernel = "VecQFlat<FormatQ4K, glu, in-kernel q8_1> routed (gate/up; four tokens a pass from two tokens on)"
             else:
                 route = ops.moe_route(ids, experts)
                 q8 = ops.quantize_q8_1_rows(xs, route.token)

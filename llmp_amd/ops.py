@@ -248,7 +248,7 @@ def moe_ffn(t, logits, x, gate_up, down, hidden, ffn, experts, used, glu=GLU_SWI
     up = gate_up.view(-1)[ffn * (hidden // qk) * bs:]
     down_stride = hidden * (ffn // qk)
     if tokens * used <= 128:
-        if keep is None and tokens * used <= 64:
+        if keep is None and tokens * used <= 128:
             # Nobody asks for the intermediates and the pairs are few: each product quantizes
             # its activations itself (the same arithmetic, two launches fewer).
             h = vecq_fused(t, up, x, hidden, ffn, gate=gate, ids=ids, tokens=tokens, used=used,
