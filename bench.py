@@ -116,6 +116,8 @@ PROFILED_TRAFFIC = {
     # The same kernel over weights relaid out into 64-row tiles: a wave's 9216 bytes are consecutive.
     "q4_k_gate_up_geglu_b4_tiles64": _traffic(32567.8, 240.0),
     "q4_k_gate_up_geglu_b8_tiles64": _traffic(32649.7, 480.0),
+    "q8_0_gate_up_swiglu_4096x2x14336_b8": _traffic(88119.6, 448.0),
+    "q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64": _traffic(61151.1, 448.0),
     "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
     # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through
     # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
@@ -259,6 +261,39 @@ def other_configs(device, args, only=None):
         del gates, ups, gate, up
         if "gates_tiled" in locals():
             del gates_tiled, ups_tiled
+        torch.cuda.empty_cache()
+
+    # Q8_0 at 8 tokens (config 1's block type on a Llama-like gate/up pair, 4096 -> 2 x 14336, SwiGLU): the default form
+    # over the file's layout (the 16-token matrix form) and the row-a-lane form over weights relaid out at import.
+    if want("q8_0_gate_up_swiglu_4096x2x14336_b8") or want("q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64"):
+        k8, n8, tokens = 4096, 14336, 8
+        pair_bytes = 2 * n8 * (k8 // 32) * 34
+        count = -(-ROTATE_BYTES // pair_bytes)
+        gates8 = [dev(synth.q8_0_weights(n8, k8, 231))]
+        ups8 = [dev(synth.q8_0_weights(n8, k8, 232))]
+        gates8 += [gates8[0].clone() for _ in range(count - 1)]
+        ups8 += [ups8[0].clone() for _ in range(count - 1)]
+        q8 = ops.quantize_q8_1(dev(synth.activations(tokens, k8, 233)))
+        y = torch.empty((tokens, 1, n8), dtype=torch.float32, device=device)
+        bytes_ = pair_bytes + tokens * (k8 // 32) * 36 + tokens * n8 * 4
+        if want("q8_0_gate_up_swiglu_4096x2x14336_b8"):
+            us = timed(lambda i: ops.vecq(ops.TYPE_Q8_0, ups8[i % count], q8, k8, n8, gate=gates8[i % count], tokens=tokens,
+                                          glu=ops.GLU_SWIGLU, out=y), 2 * count)
+            out["q8_0_gate_up_swiglu_4096x2x14336_b8"] = {
+                "workload": "Q8_0 gate/up pair 4096 -> 2 x 14336 with SwiGLU at 8 tokens, the file's layout; not one of the benchmark's five configurations",
+                "roofline": hbm_roofline("q8_0_gate_up_swiglu_4096x2x14336_b8", "VecQMmaQ8<glu> (Q8_0 blocks on v_mfma_i32_16x16x32_i8, a lane reading its row's codes from device memory)", bytes_, us)}
+        if want("q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64"):
+            tiled_variant = ops.vecq_variants().index("rows pass8 tiles64")
+            gates8t = [ops.relayout_q8_0_tiles64(g_, n8, k8) for g_ in gates8]
+            ups8t = [ops.relayout_q8_0_tiles64(u_, n8, k8) for u_ in ups8]
+            us = timed(lambda i: ops.vecq(ops.TYPE_Q8_0, ups8t[i % count], q8, k8, n8, gate=gates8t[i % count], tokens=tokens,
+                                          glu=ops.GLU_SWIGLU, variant=tiled_variant, out=y), 2 * count)
+            out["q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64"] = {
+                "workload": "the same over weights relaid out at import (llmp_hip_relayout_q8_0_tiles64)",
+                "roofline": hbm_roofline("q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64",
+                                         "VecQRows<glu, 8 tokens, Q8_0> over 64-row tiles (a weight row a lane on v_mfma_i32_4x4x4_16B_i8)", bytes_, us)}
+            del gates8t, ups8t
+        del gates8, ups8
         torch.cuda.empty_cache()
 
     # The same layer's down projection (15360 -> 3840, Q4_K, one token): rows of 60 super-blocks.

@@ -105,6 +105,16 @@ const char* llmp_hip_vecq_variant_name(int variant);
  * as every matrix is whole tiles. llmp_hip_vecq's variant "rows pass8 tiles64" reads the result; every other variant
  * reads the reference's layout. src and dst at 16-byte boundaries, not overlapping. */
 int llmp_hip_relayout_q4_k_tiles64(const void* src, void* dst, int64_t nrows, int64_t blocks_per_row, int inverse, void* stream);
+/* The same for Q8_0 rows (nrows x blocks_per_row blocks of 34 bytes, packed; blocks_per_row a multiple of four), the
+ * split the reference's importer notes call for (codes and scales apart, the codes at 16-byte boundaries): a tile's
+ * piece is four blocks of each of its 64 rows, 8704 bytes: the rows' codes (row r's 128 at 128 r, its 16-byte chunk c
+ * at place c ^ (r % 8), so that lanes reading one chunk of eight rows use every bank of LDS once), then the rows' four
+ * F16 scales, 8 bytes a row. The same bytes in all, lossless, undone by inverse != 0. llmp_hip_vecq's variant
+ * "rows pass8 tiles64" reads it for Q8_0 products of 2 to 8 tokens (a weight row a lane on the 4 x 4 x 4 int8 matrix
+ * instruction, the weights read once: where the reference's layout goes through the four-token passes or the
+ * 16-token matrix form, 1.3 to 1.7 times slower at 4 to 8 tokens). The rows at 2-byte, the tiles at 16-byte
+ * boundaries (inverse: the other way round), not overlapping. */
+int llmp_hip_relayout_q8_0_tiles64(const void* src, void* dst, int64_t nrows, int64_t blocks_per_row, int inverse, void* stream);
 
 /* The same product over unquantized activations: each workgroup quantizes the
  * tokens' rows to Q8_1 in LDS (the arithmetic of llmp_hip_q8_1_quantize, bit

@@ -142,6 +142,7 @@ SYMBOLS = {
     "llmp_hip_set_rows_quant_group": (_int, [_int, C.POINTER(SetRowsStore), _vp]),
     "llmp_hip_rope_set_rows_quant": (_int, [C.POINTER(RopeStore), _vp]),
     "llmp_hip_relayout_q4_k_tiles64": (_int, [_vp, _vp, C.c_int64, C.c_int64, _int, _vp]),
+    "llmp_hip_relayout_q8_0_tiles64": (_int, [_vp, _vp, C.c_int64, C.c_int64, _int, _vp]),
     "llmp_hip_moe_token_scratch": (C.c_size_t, [C.POINTER(MoeToken)]),
     "llmp_hip_moe_token": (_int, [C.POINTER(MoeToken), _int, _int, _vp]),
     "llmp_hip_attn_vec_quant_scratch": (C.c_size_t, [C.POINTER(AttnVecQuant), _int]),

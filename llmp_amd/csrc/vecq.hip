@@ -662,7 +662,7 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
     if (offsets != nullptr || x != nullptr || dump != nullptr || !RowsTiledTakes(type, *d))
       return Refuse(1, "vecq: the row-a-lane form over relaid-out weights takes what the row-a-lane form takes, in whole tiles of "
                        "64 packed rows");
-    a.tiled = 1;
+    a.tiled = type == LLMP_TYPE_Q8_0 ? 2 : 1;
     LaunchRows(a, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }

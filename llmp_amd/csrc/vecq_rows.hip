@@ -205,20 +205,94 @@ __device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t 
   for (int t = 0; t < NT; ++t) out[t] = fmaf(main[t], h.d, out[t]);
 }
 
+// Q8_0 over weights relaid out into 64-row tiles (llmp_hip_relayout_q8_0_tiles64): a piece is four blocks of each
+// of 64 rows, the codes first (row r's 128 at 128 r, its 16-byte chunk c at place c ^ (r % 8): eight lanes' 16-byte
+// reads of one chunk then cover all 32 banks), then the rows' four F16 scales, 8 bytes a row from byte 8192. The
+// codes are whole dwords as they lie (no 34-byte blocks to realign), and a dword goes into the instruction as it is.
+// `stage`: the LDS address of the piece; `swizzle[c]`: this lane's 128 r + 16 (c ^ (r % 8)); `codes`, `d8`: as PieceDot's.
+//   out[t] = fma(float(sum of block b's products with token t), dw_b * d8_b[t], out[t]), b = 0 .. 3.
+template <int NT>
+__device__ __forceinline__ void PieceDotQ8(uint32_t stage, const uint32_t (&swizzle)[8], uint32_t scales_at, uint32_t codes, uint32_t d8,
+                                           float (&out)[NT]) {
+#pragma clang fp contract(off)
+  using T = Tokens<NT>;
+  constexpr int kQuads = NT / 4;
+  U32v4 w[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) w[c] = LdsRead16<0>(stage + swizzle[c]);
+  uint2 row_scales;
+  asm volatile("ds_read_b64 %0, %1" : "=v"(row_scales) : "v"(stage + scales_at));
+  U32v4 cs[2][2], ds[2][kQuads];
+  auto ask = [&](int b, U32v4 (&c2)[2], U32v4 (&d2)[kQuads]) {
+    const uint32_t at = codes + static_cast<uint32_t>(b * T::kCodesBlock);
+    c2[0] = LdsRead16<0>(at), c2[1] = LdsRead16<NT * 16>(at);
+    const uint32_t dat = d8 + static_cast<uint32_t>(b * T::kScalesBlock);
+    d2[0] = LdsRead16<0>(dat);
+    if constexpr (kQuads >= 2) d2[1] = LdsRead16<16>(dat);
+  };
+  auto landed = [&](U32v4 (&c2)[2], U32v4 (&d2)[kQuads]) {
+    LLMP_TIE(c2[0]);
+    LLMP_TIE(c2[1]);
+#pragma unroll
+    for (int i = 0; i < kQuads; ++i) LLMP_TIE(d2[i]);
+  };
+  ask(0, cs[0], ds[0]);
+  LdsWaited();
+#pragma unroll
+  for (int c = 0; c < 8; ++c) LLMP_TIE(w[c]);
+  LLMP_TIE(row_scales.x);
+  LLMP_TIE(row_scales.y);
+  landed(cs[0], ds[0]);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const U32v4 (&c2)[2] = cs[b & 1];
+    const U32v4 (&d2)[kQuads] = ds[b & 1];
+    if (b < 3) ask(b + 1, cs[(b + 1) & 1], ds[(b + 1) & 1]);
+    V4i sum[kQuads];
+#pragma unroll
+    for (int tq = 0; tq < kQuads; ++tq) sum[tq] = V4i{0, 0, 0, 0};
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int code = static_cast<int>(c2[half][s]), weight = static_cast<int>(w[2 * b + half][s]);
+        if constexpr (kQuads >= 1) sum[0] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, weight, sum[0], 4, 0, 0);
+        if constexpr (kQuads >= 2) sum[1] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, weight, sum[1], 4, 1, 0);
+      }
+    }
+    const uint32_t pair = b < 2 ? row_scales.x : row_scales.y;
+    const float dw = HalfBitsToFloat((b & 1) != 0 ? pair >> 16 : pair & 0xFFFFu);
+#pragma unroll
+    for (int tq = 0; tq < kQuads; ++tq) {
+      const U32v4 d4 = d2[tq];
+      const float token_scale[4] = {AsFloat(d4[0]), AsFloat(d4[1]), AsFloat(d4[2]), AsFloat(d4[3])};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) out[4 * tq + q] = fmaf(static_cast<float>(sum[tq][q]), dw * token_scale[q], out[4 * tq + q]);
+    }
+    if (b < 3) {
+      LdsWaited();
+      landed(cs[(b + 1) & 1], ds[(b + 1) & 1]);
+    }
+  }
+}
+
+constexpr int kQ8PieceBytes = kTileRows * 136;  // a relaid-out Q8_0 piece in device memory: 8192 bytes of codes, 512 of scales
+
 // grid (workgroups, slots); LDS: the tokens, then the waves' rings (whose first bytes also carry the
-// waves' sums to their meeting).
-template <bool kGlu, int NT, int STAGES>
+// waves' sums to their meeting). FMT 0: Q4_K (a unit a super-block); 1: Q8_0 relaid out (a unit four blocks).
+template <bool kGlu, int NT, int STAGES, int FMT = 0>
 __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   using T = Tokens<NT>;
   constexpr int kMatrices = kGlu ? 2 : 1;
+  constexpr int kUnitBlocks = FMT == 0 ? 8 : 4;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int nsb = d.ncols_x / 256;
   const int blocks = d.ncols_x / 32;
+  const int nsb = blocks / kUnitBlocks;  // units a row
   const int slot = blockIdx.y;
   uint8_t* codes = lds;
   uint8_t* d8 = codes + blocks * T::kCodesBlock;
@@ -277,7 +351,11 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
   const int64_t matrix_block = static_cast<int64_t>(slot) * d.stride_expert;
   const int token_lane = min(lane, NT - 1);
-  const uint32_t ring_at = lds_address(ring) + static_cast<uint32_t>(lane) * 144u;  // this lane's row of a stage
+  const uint32_t ring_at = lds_address(ring) + (FMT == 0 ? static_cast<uint32_t>(lane) * 144u : 0u);  // this lane's row of a stage (Q8_0: the stage)
+  uint32_t swizzle[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) swizzle[c] = static_cast<uint32_t>(lane * 128 + ((c ^ (lane & 7)) << 4));
+  const uint32_t scales_at = 8192u + static_cast<uint32_t>(lane) * 8u;
   const uint32_t codes_at = lds_address(codes) + static_cast<uint32_t>(token_lane) * 16u;
   const uint32_t d8_at = lds_address(d8);
   const uint32_t sums_at = lds_address(sums) + static_cast<uint32_t>(token_lane) * 32u;
@@ -292,11 +370,17 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       const int byte = j * (kWave * 16) + lane * 16;
       const int row = byte / 144;
       // (Relaid-out weights: a piece is 9216 consecutive bytes, every 64-byte unit of HBM asked for once.)
-      offsets[j] = a.tiled != 0 ? static_cast<uint32_t>(byte)
-                                : static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
-                                      static_cast<uint32_t>(byte - row * 144);
+      if constexpr (FMT != 0) {
+        // The piece's last 512 bytes (the scales) by the lower half of the wave, the upper half the same again
+        // (into the stage's spare 512 bytes).
+        offsets[j] = j < 8 ? static_cast<uint32_t>(byte) : 8192u + static_cast<uint32_t>(lane & 31) * 16u;
+      } else {
+        offsets[j] = a.tiled != 0 ? static_cast<uint32_t>(byte)
+                                  : static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
+                                        static_cast<uint32_t>(byte - row * 144);
+      }
     }
-    const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * 144;
+    const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * (FMT == 0 ? 144 : 34);
     up_tile = static_cast<const uint8_t*>(d.w) + at;
     if constexpr (kGlu) gate_tile = static_cast<const uint8_t*>(d.g) + at;
   };
@@ -311,7 +395,7 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       gate = piece < paired ? (piece & 3) >> 1 : piece - paired;
       sb = sb_first + (piece < paired ? (piece >> 2) * 2 + (piece & 1) : sb_end - sb_first - 1);
     }
-    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * (a.tiled != 0 ? kPieceBytes : 144);
+    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * (FMT != 0 ? kQ8PieceBytes : a.tiled != 0 ? kPieceBytes : 144);
     uint8_t* to = ring + (i % STAGES) * kPieceBytes;
 #pragma unroll
     for (int j = 0; j < kPieceLoads; ++j)
@@ -377,11 +461,15 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       const int count = sb_end - sb_first;
       int i = 0;
       auto piece_dot = [&](int sb, float (&out)[NT], V4f (&mins)[NT / 4]) {
-        const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * 8 * T::kCodesBlock);
-        const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * 8 * T::kScalesBlock);
+        const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * kUnitBlocks * T::kCodesBlock);
+        const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * kUnitBlocks * T::kScalesBlock);
         const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
         next_piece(i);
-        PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
+        if constexpr (FMT == 0) {
+          PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
+        } else {
+          PieceDotQ8<NT>(ring_at + (i % STAGES) * kPieceBytes, swizzle, scales_at, sb_codes, sb_d8, out);
+        }
         ++i;
         __builtin_amdgcn_s_waitcnt(0xC07F);  // the stage about to be refilled has been read
       };
@@ -431,19 +519,52 @@ int StagesFor(int blocks) {
   return 0;
 }
 
-template <bool kGlu, int NT, int STAGES>
+template <bool kGlu, int NT, int STAGES, int FMT>
 void LaunchRowsKernel(const VecQArgs& a, dim3 grid, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&VecQRows<kGlu, NT, STAGES>), static_cast<int>(kRowsLdsLimit), &sized)) return;
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQRows<kGlu, NT, STAGES, FMT>), static_cast<int>(kRowsLdsLimit), &sized)) return;
   const size_t lds = ((Tokens<NT>::Bytes(a.d.ncols_x / 32) + 1023) & ~static_cast<size_t>(1023)) +
                      static_cast<size_t>(kRowsWaves) * STAGES * kPieceBytes;
-  hipLaunchKernelGGL((VecQRows<kGlu, NT, STAGES>), grid, dim3(kRowsGroup), lds, stream, a);
+  hipLaunchKernelGGL((VecQRows<kGlu, NT, STAGES, FMT>), grid, dim3(kRowsGroup), lds, stream, a);
 }
 
 template <bool kGlu, int NT>
 void LaunchRowsStages(const VecQArgs& a, dim3 grid, hipStream_t stream) {
-  StagesFor<NT>(a.d.ncols_x / 32) == 3 ? LaunchRowsKernel<kGlu, NT, 3>(a, grid, stream)
-                                       : LaunchRowsKernel<kGlu, NT, 2>(a, grid, stream);
+  const bool three = StagesFor<NT>(a.d.ncols_x / 32) == 3;
+  if (a.tiled == 2) {
+    three ? LaunchRowsKernel<kGlu, NT, 3, 1>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 1>(a, grid, stream);
+  } else {
+    three ? LaunchRowsKernel<kGlu, NT, 3, 0>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 0>(a, grid, stream);
+  }
+}
+
+// A thread a row's unit of four blocks (136 bytes): into its tile's piece (see PieceDotQ8), or back.
+__global__ void RelayoutQ8Tiles64Kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int64_t units_all, int units, int inverse) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= units_all) return;
+  const int64_t row = i / units;
+  const int unit = static_cast<int>(i - row * units);
+  const int r = static_cast<int>(row % kTileRows);
+  const uint16_t* native = src + (inverse != 0 ? 0 : i * 68);
+  uint16_t* native_to = dst + (inverse != 0 ? i * 68 : 0);
+  const int64_t piece = ((row / kTileRows) * units + unit) * (kQ8PieceBytes / 2);  // in halfwords
+  for (int b = 0; b < 4; ++b) {
+    const int64_t scale_at = piece + 4096 + r * 4 + b;
+    if (inverse != 0) {
+      native_to[17 * b] = src[scale_at];
+    } else {
+      dst[scale_at] = native[17 * b];
+    }
+    for (int h = 0; h < 16; ++h) {  // the block's codes, two a halfword: chunk 2 b + h / 8, halfword h % 8 of it
+      const int c = 2 * b + (h >> 3);
+      const int64_t code_at = piece + r * 64 + ((c ^ (r & 7)) << 3) + (h & 7);
+      if (inverse != 0) {
+        native_to[17 * b + 1 + h] = src[code_at];
+      } else {
+        dst[code_at] = native[17 * b + 1 + h];
+      }
+    }
+  }
 }
 
 // 16 bytes a thread: block (row, sb) of the row-major matrix is block (sb, row % 64) of its 64-row tile.
@@ -473,8 +594,14 @@ bool RowsTakes(int type, const llmp_vecq_desc& d) {
   return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
 }
 
-// The same over relaid-out weights: whole tiles of packed rows.
+// The same over relaid-out weights: whole tiles of packed rows. Q8_0 has this form alone (rows of whole units of four
+// blocks, at least four of them).
 bool RowsTiledTakes(int type, const llmp_vecq_desc& d) {
+  if (type == LLMP_TYPE_Q8_0) {
+    if (d.ids != nullptr || d.tokens < 2 || d.tokens > 8 || d.ncols_x % 128 != 0 || d.ncols_x / 128 < kRowsWaves) return false;
+    if ((d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) == 0) return false;
+    return d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 32 && d.stride_expert % (kTileRows * (d.ncols_x / 32)) == 0;
+  }
   return RowsTakes(type, d) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
          d.stride_expert % (kTileRows * (d.ncols_x / 256)) == 0;
 }
@@ -513,5 +640,24 @@ extern "C" int llmp_hip_relayout_q4_k_tiles64(const void* src, void* dst, int64_
   const int64_t chunks = static_cast<int64_t>(bytes / 16);
   hipLaunchKernelGGL(RelayoutTiles64Kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint4*>(src), static_cast<uint4*>(dst), chunks, static_cast<int>(blocks_per_row), inverse);
+  return LaunchStatus("relayout");
+}
+
+extern "C" int llmp_hip_relayout_q8_0_tiles64(const void* src, void* dst, int64_t nrows, int64_t blocks_per_row, int inverse, void* stream) {
+  using namespace llmp_hip;
+  BeginLaunches();
+  if (src == nullptr || dst == nullptr || src == dst) return Refuse(1, "relayout: null operands, or in place");
+  if (nrows < 1 || nrows % kTileRows != 0 || blocks_per_row < 4 || blocks_per_row % 4 != 0 || blocks_per_row > INT32_MAX)
+    return Refuse(1, "relayout: rows in whole tiles of %d and of whole units of four blocks, not %lld x %lld", kTileRows, (long long)nrows,
+                  (long long)blocks_per_row);
+  // The native rows at 2-byte boundaries (their blocks are 34 bytes), the tiles at 16-byte ones (their chunks are read whole).
+  if (reinterpret_cast<uintptr_t>(inverse != 0 ? dst : src) % 2 != 0 || reinterpret_cast<uintptr_t>(inverse != 0 ? src : dst) % 16 != 0)
+    return Refuse(1, "relayout: the rows at 2-byte, the tiles at 16-byte boundaries");
+  const uintptr_t a = reinterpret_cast<uintptr_t>(src), b = reinterpret_cast<uintptr_t>(dst);
+  const uint64_t bytes = static_cast<uint64_t>(nrows) * static_cast<uint64_t>(blocks_per_row) * 34u;
+  if (a < b + bytes && b < a + bytes) return Refuse(1, "relayout: the source and the destination overlap");
+  const int64_t units_all = nrows * (blocks_per_row / 4);
+  hipLaunchKernelGGL(RelayoutQ8Tiles64Kernel, dim3(static_cast<unsigned>((units_all + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), units_all, static_cast<int>(blocks_per_row / 4), inverse);
   return LaunchStatus("relayout");
 }

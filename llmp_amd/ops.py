@@ -118,6 +118,15 @@ def relayout_q4_k_tiles64(w, nrows, k, inverse=False):
     return out
 
 
+def relayout_q8_0_tiles64(w, nrows, k, inverse=False):
+    """The same for uint8 Q8_0 rows (nrows x k / 32 blocks, packed; k a multiple of 128): 64-row tiles, four blocks of a
+    tile's rows a piece, codes and scales apart. Returns a new tensor."""
+    lib = _lib.load()
+    out = torch.empty_like(w)
+    _lib.check(lib.llmp_hip_relayout_q8_0_tiles64(_ptr(w), _ptr(out), nrows, k // 32, int(inverse), _stream()))
+    return out
+
+
 def vecq_variants():
     lib = _lib.load()
     return [lib.llmp_hip_vecq_variant_name(i).decode() for i in range(lib.llmp_hip_vecq_variants())]

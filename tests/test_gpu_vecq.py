@@ -756,3 +756,52 @@ def test_relaid_out_rows_equal_the_row_a_lane_form_bit_for_bit(device, tokens, g
     with pytest.raises(ops.KernelFailure) as refused:
         ops.vecq(Q4_K, ut, qd, k, n - 8, gate=gt, variant=tiled_variant, **common)
     assert refused.value.rejected
+
+
+@pytest.mark.parametrize("tokens,glu,k", [(2, ops.GLU_NONE, 640), (4, ops.GLU_GEGLU, 1536), (8, ops.GLU_SWIGLU, 1536), (7, ops.GLU_NONE, 4096)])
+def test_q8_0_rows_form_over_relaid_out_weights(device, tokens, glu, k):
+    """llmp_hip_relayout_q8_0_tiles64 (codes and scales apart, 64-row tiles, four blocks a piece) and the row-a-lane
+    variant that reads it for Q8_0: the layout is what the header says, the inverse gives the file's bytes back, the
+    products are the oracle's (integer block sums on the matrix instruction are exact; what is left is the order of
+    the float sums, 1e-3), a token's values do not depend on the tokens beside it, and shapes the form does not take
+    are refused. Dense and grouped (two matrices, two input rows)."""
+    n, used = 192, 2
+    tiled_variant = ops.vecq_variants().index("rows pass8 tiles64")
+    up = make_weights(Q8_0, used * n, k, 311)
+    gate = make_weights(Q8_0, used * n, k, 312) if glu != ops.GLU_NONE else None
+    q8 = oracle.q8_1_quantize(synth.activations(tokens * used, k, 313))
+    ud, qd = dev(up, device), dev(q8, device)
+    ut = ops.relayout_q8_0_tiles64(ud, used * n, k)
+    gt = ops.relayout_q8_0_tiles64(dev(gate, device), used * n, k) if gate is not None else None
+    assert not torch.equal(ut, ud)
+    assert torch.equal(ops.relayout_q8_0_tiles64(ut, used * n, k, inverse=True), ud)
+    units = k // 128
+    native = up.reshape(-1, units, 4, 34)                      # [row][unit][block][d, 32 codes]
+    tiled = ut.cpu().numpy().reshape(-1, units, 8704)          # [tile][unit][piece]
+    for row, unit in ((0, 0), (63, units - 1), (64, 1), (used * n - 1, 2), (77, 3)):
+        piece, r = tiled[row // 64, unit], row % 64
+        for b in range(4):
+            assert np.array_equal(piece[8192 + r * 8 + 2 * b:8192 + r * 8 + 2 * b + 2], native[row, unit, b, :2])
+            for half in range(2):
+                c = 2 * b + half
+                at = r * 128 + ((c ^ (r & 7)) << 4)
+                assert np.array_equal(piece[at:at + 16], native[row, unit, b, 2 + 16 * half:18 + 16 * half])
+    blocks = oracle.padded_k(k) // 32
+    common = dict(used=used, stride_expert=n * (k // 32), y_token=blocks * used, y_slot=blocks, glu=glu)
+    got = ops.vecq(Q8_0, ut, qd, k, n, gate=gt, variant=tiled_variant, tokens=tokens, **common)
+    ref = oracle.vecq(Q8_0, up, q8, k, n, gate=gate, tokens=tokens, **common)
+    ok, worst = rel_close(got.cpu().numpy(), ref, TOL)
+    assert ok, worst
+    # The default form over the file's layout computes the same definition.
+    same = ops.vecq(Q8_0, ud, qd, k, n, gate=dev(gate, device) if gate is not None else None, tokens=tokens, **common)
+    ok, worst = rel_close(got.cpu().numpy(), same.cpu().numpy(), TOL)
+    assert ok, worst
+    # Two of the tokens alone (another instance of the kernel where the count crosses four): the same bits.
+    pair = ops.vecq(Q8_0, ut, qd, k, n, gate=gt, variant=tiled_variant, tokens=2, **common)
+    assert torch.equal(pair.view(torch.int32), got[:2].view(torch.int32))
+    for bad in (dict(nrows=n - 8), dict(tokens=1), dict(tokens=9)):
+        with pytest.raises(ops.KernelFailure) as refused:
+            ops.vecq(Q8_0, ut, qd, k, bad.get("nrows", n), gate=gt, variant=tiled_variant, tokens=bad.get("tokens", tokens), **common)
+        assert refused.value.rejected
+    with pytest.raises(ops.KernelFailure):  # the file's layout has no row-a-lane form for Q8_0
+        ops.vecq(Q8_0, ud, qd, k, n, variant=ops.vecq_variants().index("rows pass8"), tokens=tokens, **common)
