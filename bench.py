@@ -116,8 +116,8 @@ PROFILED_TRAFFIC = {
     # The same kernel over weights relaid out into 64-row tiles: a wave's 9216 bytes are consecutive.
     "q4_k_gate_up_geglu_b4_tiles64": _traffic(32567.8, 240.0),
     "q4_k_gate_up_geglu_b8_tiles64": _traffic(32649.7, 480.0),
-    "q8_0_gate_up_swiglu_4096x2x14336_b8": _traffic(88119.6, 448.0),
-    "q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64": _traffic(61151.1, 448.0),
+    "q8_0_gate_up_swiglu_4096x2x14336_b8": _traffic(78810.1, 448.0),
+    "q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64": _traffic(61149.7, 448.0),
     "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
     # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through
     # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
@@ -264,7 +264,7 @@ def other_configs(device, args, only=None):
         torch.cuda.empty_cache()
 
     # Q8_0 at 8 tokens (config 1's block type on a Llama-like gate/up pair, 4096 -> 2 x 14336, SwiGLU): the default form
-    # over the file's layout (the 16-token matrix form) and the row-a-lane form over weights relaid out at import.
+    # over the file's layout and the row-a-lane form over weights relaid out at import.
     if want("q8_0_gate_up_swiglu_4096x2x14336_b8") or want("q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64"):
         k8, n8, tokens = 4096, 14336, 8
         pair_bytes = 2 * n8 * (k8 // 32) * 34
@@ -281,7 +281,7 @@ def other_configs(device, args, only=None):
                                           glu=ops.GLU_SWIGLU, out=y), 2 * count)
             out["q8_0_gate_up_swiglu_4096x2x14336_b8"] = {
                 "workload": "Q8_0 gate/up pair 4096 -> 2 x 14336 with SwiGLU at 8 tokens, the file's layout; not one of the benchmark's five configurations",
-                "roofline": hbm_roofline("q8_0_gate_up_swiglu_4096x2x14336_b8", "VecQMmaQ8<glu> (Q8_0 blocks on v_mfma_i32_16x16x32_i8, a lane reading its row's codes from device memory)", bytes_, us)}
+                "roofline": hbm_roofline("q8_0_gate_up_swiglu_4096x2x14336_b8", "VecQRows<glu, 8 tokens, Q8_0 in the file's layout> (a weight row a lane on v_mfma_i32_4x4x4_16B_i8)", bytes_, us)}
         if want("q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64"):
             tiled_variant = ops.vecq_variants().index("rows pass8 tiles64")
             gates8t = [ops.relayout_q8_0_tiles64(g_, n8, k8) for g_ in gates8]

@@ -573,7 +573,15 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   // four-token passes' 18 / 25 / 43). More tokens, and rows that form does not take: the 16 x 16 form, whose time
   // hardly depends on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0
   // (15 / 17 / 20 / 27 us against 29 at 4096 x 14336).
-  if (tokens > 1 && !fused && RowsTakes(type, d)) return kRowsVariant;
+  if (tokens > 1 && !fused && type == LLMP_TYPE_Q4_K && RowsTakes(type, d)) return kRowsVariant;
+  // Q8_0: the same form, whose time hardly depends on the tokens (4096 x 14336: 16.2-17.4 us at 2 to 8 tokens against
+  // 19 / 22 / 31 for the four-token passes and the 16 x 16 form), wherever its 64-row tiles fill the device; with
+  // fewer tiles from five tokens, where the flat form would take a second pass (4096 x 4096: 14.5-14.8 us at 5 to 8
+  // tokens against 15.6-19.4, but 13.4 against 8.4-12.6 at 2 to 4).
+  if (tokens > 1 && !fused && type == LLMP_TYPE_Q8_0 && RowsTakes(type, d)) {
+    const int64_t tiles = static_cast<int64_t>((d.nrows + 63) / 64) * d.used;
+    if (tiles >= 128 ? tokens >= (d.g != nullptr ? 3 : 2) : tokens >= 5) return kRowsVariant;
+  }
   const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 5 : d.g != nullptr ? 4 : 2;
   if (tokens > flat_up_to && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
@@ -669,9 +677,10 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
   if (v.lanes == -2) {
     if (offsets != nullptr || !RowsTakes(type, *d))
       return Refuse(1, "vecq: the row-a-lane form takes 2 to 8 tokens of a dense or grouped Q4_K product, rows of 1024 values "
-                       "or more");
+                       "or more, or of a Q8_0 product, rows of whole 256 values, 512 or more, at 16-byte boundaries");
     if (x != nullptr) return Refuse(1, "vecq: the row-a-lane form takes Q8_1 activations");
     if (dump != nullptr) return Refuse(1, "vecq: block sums are of the one-token variants");
+    a.tiled = type == LLMP_TYPE_Q8_0 ? 3 : 0;
     LaunchRows(a, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }

@@ -276,10 +276,84 @@ __device__ __forceinline__ void PieceDotQ8(uint32_t stage, const uint32_t (&swiz
   }
 }
 
+// Q8_0 in the file's layout: a lane's row of a piece is 144 bytes fetched from the 16-byte boundary at or below its
+// unit of four 34-byte blocks, which begins `shift` bytes (0 or 8, the same for every row: rows are whole 16-byte
+// chunks apart) into it. Blocks 1 and 3 of a unit have their codes on dword boundaries; blocks 0 and 2 have them two
+// bytes off, and every dword of theirs is put together from two (v_alignbyte).
+template <int NT>
+__device__ __forceinline__ void PieceDotQ8Native(uint32_t row, uint32_t codes, uint32_t d8, float (&out)[NT]) {
+#pragma clang fp contract(off)
+  using T = Tokens<NT>;
+  constexpr int kQuads = NT / 4;
+  uint2 raw[17];
+#pragma unroll
+  for (int i = 0; i < 17; ++i) asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(raw[i]) : "v"(row), "n"(8 * i));
+  U32v4 cs[2][2], ds[2][kQuads];
+  auto ask = [&](int b, U32v4 (&c2)[2], U32v4 (&d2)[kQuads]) {
+    const uint32_t at = codes + static_cast<uint32_t>(b * T::kCodesBlock);
+    c2[0] = LdsRead16<0>(at), c2[1] = LdsRead16<NT * 16>(at);
+    const uint32_t dat = d8 + static_cast<uint32_t>(b * T::kScalesBlock);
+    d2[0] = LdsRead16<0>(dat);
+    if constexpr (kQuads >= 2) d2[1] = LdsRead16<16>(dat);
+  };
+  auto landed = [&](U32v4 (&c2)[2], U32v4 (&d2)[kQuads]) {
+    LLMP_TIE(c2[0]);
+    LLMP_TIE(c2[1]);
+#pragma unroll
+    for (int i = 0; i < kQuads; ++i) LLMP_TIE(d2[i]);
+  };
+  ask(0, cs[0], ds[0]);
+  LdsWaited();
+  uint32_t d[34];
+#pragma unroll
+  for (int i = 0; i < 17; ++i) {
+    LLMP_TIE(raw[i].x);
+    LLMP_TIE(raw[i].y);
+    d[2 * i] = raw[i].x, d[2 * i + 1] = raw[i].y;
+  }
+  landed(cs[0], ds[0]);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const U32v4 (&c2)[2] = cs[b & 1];
+    const U32v4 (&d2)[kQuads] = ds[b & 1];
+    if (b < 3) ask(b + 1, cs[(b + 1) & 1], ds[(b + 1) & 1]);
+    // Block b begins at byte 34 b: dword 8 b + b / 2, on its boundary (b even) or two bytes past it (b odd); its
+    // codes follow its two bytes of scale.
+    const int first = 8 * b + b / 2;
+    uint32_t weight[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      weight[s] = (b & 1) != 0 ? d[first + 1 + s] : __builtin_amdgcn_alignbyte(d[first + 1 + s], d[first + s], 2);
+    }
+    const float dw = HalfBitsToFloat((b & 1) != 0 ? d[first] >> 16 : d[first] & 0xFFFFu);
+    V4i sum[kQuads];
+#pragma unroll
+    for (int tq = 0; tq < kQuads; ++tq) sum[tq] = V4i{0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int code = static_cast<int>(c2[s >> 2][s & 3]);
+      if constexpr (kQuads >= 1) sum[0] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[0], 4, 0, 0);
+      if constexpr (kQuads >= 2) sum[1] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[1], 4, 1, 0);
+    }
+#pragma unroll
+    for (int tq = 0; tq < kQuads; ++tq) {
+      const U32v4 d4 = d2[tq];
+      const float token_scale[4] = {AsFloat(d4[0]), AsFloat(d4[1]), AsFloat(d4[2]), AsFloat(d4[3])};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) out[4 * tq + q] = fmaf(static_cast<float>(sum[tq][q]), dw * token_scale[q], out[4 * tq + q]);
+    }
+    if (b < 3) {
+      LdsWaited();
+      landed(cs[(b + 1) & 1], ds[(b + 1) & 1]);
+    }
+  }
+}
+
 constexpr int kQ8PieceBytes = kTileRows * 136;  // a relaid-out Q8_0 piece in device memory: 8192 bytes of codes, 512 of scales
 
 // grid (workgroups, slots); LDS: the tokens, then the waves' rings (whose first bytes also carry the
-// waves' sums to their meeting). FMT 0: Q4_K (a unit a super-block); 1: Q8_0 relaid out (a unit four blocks).
+// waves' sums to their meeting). FMT 0: Q4_K (a unit a super-block); 1: Q8_0 relaid out (a unit four blocks); 2: Q8_0
+// in the file's layout.
 template <bool kGlu, int NT, int STAGES, int FMT = 0>
 __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   using T = Tokens<NT>;
@@ -351,7 +425,7 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
   const int64_t matrix_block = static_cast<int64_t>(slot) * d.stride_expert;
   const int token_lane = min(lane, NT - 1);
-  const uint32_t ring_at = lds_address(ring) + (FMT == 0 ? static_cast<uint32_t>(lane) * 144u : 0u);  // this lane's row of a stage (Q8_0: the stage)
+  const uint32_t ring_at = lds_address(ring) + (FMT != 1 ? static_cast<uint32_t>(lane) * 144u : 0u);  // this lane's row of a stage (Q8_0 relaid out: the stage)
   uint32_t swizzle[8];
 #pragma unroll
   for (int c = 0; c < 8; ++c) swizzle[c] = static_cast<uint32_t>(lane * 128 + ((c ^ (lane & 7)) << 4));
@@ -370,7 +444,11 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       const int byte = j * (kWave * 16) + lane * 16;
       const int row = byte / 144;
       // (Relaid-out weights: a piece is 9216 consecutive bytes, every 64-byte unit of HBM asked for once.)
-      if constexpr (FMT != 0) {
+      if constexpr (FMT == 2) {
+        // A row's 144 bytes from the 16-byte boundary at or below its unit (issue adds the unit's place).
+        offsets[j] = static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 34u +
+                     static_cast<uint32_t>(byte - row * 144);
+      } else if constexpr (FMT == 1) {
         // The piece's last 512 bytes (the scales) by the lower half of the wave, the upper half the same again
         // (into the stage's spare 512 bytes).
         offsets[j] = j < 8 ? static_cast<uint32_t>(byte) : 8192u + static_cast<uint32_t>(lane & 31) * 16u;
@@ -395,7 +473,9 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       gate = piece < paired ? (piece & 3) >> 1 : piece - paired;
       sb = sb_first + (piece < paired ? (piece >> 2) * 2 + (piece & 1) : sb_end - sb_first - 1);
     }
-    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) + static_cast<int64_t>(sb) * (FMT != 0 ? kQ8PieceBytes : a.tiled != 0 ? kPieceBytes : 144);
+    const uint8_t* from = (gate != 0 ? gate_tile : up_tile) +
+                          (FMT == 2 ? static_cast<int64_t>(sb) * 136 & ~int64_t{15}
+                                    : static_cast<int64_t>(sb) * (FMT == 1 ? kQ8PieceBytes : a.tiled != 0 ? kPieceBytes : 144));
     uint8_t* to = ring + (i % STAGES) * kPieceBytes;
 #pragma unroll
     for (int j = 0; j < kPieceLoads; ++j)
@@ -467,6 +547,8 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
         next_piece(i);
         if constexpr (FMT == 0) {
           PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
+        } else if constexpr (FMT == 2) {
+          PieceDotQ8Native<NT>(ring_at + (i % STAGES) * kPieceBytes + static_cast<uint32_t>((sb & 1) * 8), sb_codes, sb_d8, out);
         } else {
           PieceDotQ8<NT>(ring_at + (i % STAGES) * kPieceBytes, swizzle, scales_at, sb_codes, sb_d8, out);
         }
@@ -533,6 +615,8 @@ void LaunchRowsStages(const VecQArgs& a, dim3 grid, hipStream_t stream) {
   const bool three = StagesFor<NT>(a.d.ncols_x / 32) == 3;
   if (a.tiled == 2) {
     three ? LaunchRowsKernel<kGlu, NT, 3, 1>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 1>(a, grid, stream);
+  } else if (a.tiled == 3) {
+    three ? LaunchRowsKernel<kGlu, NT, 3, 2>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 2>(a, grid, stream);
   } else {
     three ? LaunchRowsKernel<kGlu, NT, 3, 0>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 0>(a, grid, stream);
   }
@@ -586,8 +670,17 @@ __global__ void RelayoutTiles64Kernel(const uint4* __restrict__ src, uint4* __re
 }  // namespace
 
 // Q4_K, 2 to 8 tokens of a dense or grouped product (no routing ids) over Q8_1 activations, rows of at
-// least four super-blocks (a wave a quarter of K) whose staged tokens leave room for two stages a wave.
+// least four super-blocks (a wave a quarter of K) whose staged tokens leave room for two stages a wave. Q8_0: rows of
+// whole 256 values (an even number of four-block units, so that a row's last 16-byte chunk ends inside the row), at
+// least four units, every row and matrix at a 16-byte boundary.
 bool RowsTakes(int type, const llmp_vecq_desc& d) {
+  if (type == LLMP_TYPE_Q8_0) {
+    if (d.ids != nullptr || d.tokens < 2 || d.tokens > 8 || d.ncols_x % 256 != 0 || d.ncols_x / 128 < kRowsWaves) return false;
+    if (d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || reinterpret_cast<uintptr_t>(d.w) % 16 != 0 ||
+        (d.g != nullptr && reinterpret_cast<uintptr_t>(d.g) % 16 != 0))
+      return false;
+    return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
+  }
   if (type != LLMP_TYPE_Q4_K || d.ids != nullptr || d.tokens < 2 || d.tokens > 8) return false;
   const int nsb = d.ncols_x / 256;
   if (nsb < kRowsWaves) return false;
@@ -602,7 +695,7 @@ bool RowsTiledTakes(int type, const llmp_vecq_desc& d) {
     if ((d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) == 0) return false;
     return d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 32 && d.stride_expert % (kTileRows * (d.ncols_x / 32)) == 0;
   }
-  return RowsTakes(type, d) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
+  return type == LLMP_TYPE_Q4_K && RowsTakes(type, d) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
          d.stride_expert % (kTileRows * (d.ncols_x / 256)) == 0;
 }
 

@@ -102,8 +102,8 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
-        if name.startswith("rows") and (t != Q4_K or name.endswith("tiles64")):
-            # the row-a-lane form is Q4_K's alone, and its relaid-out variant takes whole tiles of 64 rows
+        if name.endswith("tiles64"):
+            # the relaid-out variant takes whole tiles of 64 rows (and the layout it is named for)
             with pytest.raises(ops.KernelFailure):
                 ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
             continue
@@ -803,5 +803,19 @@ def test_q8_0_rows_form_over_relaid_out_weights(device, tokens, glu, k):
         with pytest.raises(ops.KernelFailure) as refused:
             ops.vecq(Q8_0, ut, qd, k, bad.get("nrows", n), gate=gt, variant=tiled_variant, tokens=bad.get("tokens", tokens), **common)
         assert refused.value.rejected
-    with pytest.raises(ops.KernelFailure):  # the file's layout has no row-a-lane form for Q8_0
-        ops.vecq(Q8_0, ud, qd, k, n, variant=ops.vecq_variants().index("rows pass8"), tokens=tokens, **common)
+    # The row-a-lane form over the file's layout (rows of whole 256 values): the same arithmetic, the same bits.
+    rows_variant = ops.vecq_variants().index("rows pass8")
+    gd = dev(gate, device) if gate is not None else None
+    if k % 256 == 0:
+        native = ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=rows_variant, tokens=tokens, **common)
+        assert torch.equal(native.view(torch.int32), got.view(torch.int32))
+        # Fewer rows than whole tiles, and rows apart (a pitch of eight blocks more): the form's own edges.
+        pitched = torch.zeros((used * n, k // 32 + 8, 34), dtype=torch.uint8, device=device)
+        pitched[:, :k // 32] = ud.view(used * n, k // 32, 34)
+        wide = dict(common, stride_expert=n * (k // 32 + 8))
+        short = ops.vecq(Q8_0, pitched.view(-1), qd, k, n - 24, variant=rows_variant, tokens=tokens, stride_row=k // 32 + 8, **dict(wide, glu=ops.GLU_NONE))
+        plain = got if glu == ops.GLU_NONE else ops.vecq(Q8_0, ut, qd, k, n, variant=tiled_variant, tokens=tokens, **dict(common, glu=ops.GLU_NONE))
+        assert torch.equal(short.view(torch.int32), plain[:, :, :n - 24].contiguous().view(torch.int32))
+    else:
+        with pytest.raises(ops.KernelFailure):
+            ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=rows_variant, tokens=tokens, **common)
