@@ -573,16 +573,22 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   // four-token passes' 18 / 25 / 43). More tokens, and rows that form does not take: the 16 x 16 form, whose time
   // hardly depends on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0
   // (15 / 17 / 20 / 27 us against 29 at 4096 x 14336).
-  if (tokens > 1 && !fused && type == LLMP_TYPE_Q4_K && RowsTakes(type, d)) return kRowsVariant;
-  // Q8_0: the same form, whose time hardly depends on the tokens (4096 x 14336: 16.2-17.4 us at 2 to 8 tokens against
-  // 19 / 22 / 31 for the four-token passes and the 16 x 16 form), wherever its 64-row tiles fill the device; with
-  // fewer tiles from five tokens, where the flat form would take a second pass (4096 x 4096: 14.5-14.8 us at 5 to 8
-  // tokens against 15.6-19.4, but 13.4 against 8.4-12.6 at 2 to 4).
-  if (tokens > 1 && !fused && type == LLMP_TYPE_Q8_0 && RowsTakes(type, d)) {
+  // The row-a-lane form's time hardly depends on the tokens, but it takes 64 rows a workgroup of four waves: a matrix
+  // of fewer than 128 such tiles leaves most of the device without one, and the flat form's four-token pass is the
+  // faster up to four tokens (Q4_K 15360 x 3840, 60 tiles: 13.8 us against 24.5 at two tokens, 25 both at four;
+  // 4096 x 4096: 7.0 / 8.9 against 10.5 at two and four, 14.4 against 12.3 at eight).
+  // Q8_0: the same (4096 x 14336: 16.2-17.4 us at 2 to 8 tokens against 19 / 22 / 31 for the four-token passes and
+  // the 16 x 16 form; 4096 x 4096: 14.5-14.8 us at 5 to 8 tokens against 15.6-19.4, but 13.4 against 8.4-12.6 at 2 to
+  // 4); with a GLU the pair's two-token pass is as fast, so from three.
+  if (tokens > 1 && !fused && (type == LLMP_TYPE_Q4_K || type == LLMP_TYPE_Q8_0) && RowsTakes(type, d)) {
     const int64_t tiles = static_cast<int64_t>((d.nrows + 63) / 64) * d.used;
-    if (tiles >= 128 ? tokens >= (d.g != nullptr ? 3 : 2) : tokens >= 5) return kRowsVariant;
+    const int from = type == LLMP_TYPE_Q8_0 && d.g != nullptr ? 3 : 2;
+    if (tiles >= 128 ? tokens >= from : tokens >= 5) return kRowsVariant;
   }
-  const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 5 : d.g != nullptr ? 4 : 2;
+  // (A plain Q4_K product of few rows: the four-token pass up to four tokens, 9.0 us against the 16 x 16 form's 13.1
+  // at 4096 x 4096.)
+  const bool few_rows = static_cast<int64_t>((d.nrows + 63) / 64) * d.used < 128;
+  const int flat_up_to = type == LLMP_TYPE_Q8_0 ? 5 : d.g != nullptr || few_rows ? 4 : 2;
   if (tokens > flat_up_to && d.ids == nullptr && !fused && MmaTakes(type, d)) return kMmaVariant;
   if (FlatTakes(type, d)) return tokens > 1 ? kFlatFirst + 1 : kFlatFirst;
   int pass = tokens >= 5 ? 8 : tokens >= 3 ? 4 : tokens >= 2 ? 2 : 1;
