@@ -494,10 +494,16 @@ constexpr Variant kVariants[] = {
     {"mma pass16", -1, 16, 1},
     // Q4_K, a weight row a lane, 2 to 8 tokens of a dense or grouped product on the 4 x 4 x 4 int8 matrix
     // instruction (vecq_rows.hip); `lanes` -2 marks the form.
-    {"rows pass8", -2, 8, 1},
+    // `flight`: the units of a row in a piece, 0 for the launcher's choice (see the variants that follow the next).
+    {"rows pass8", -2, 8, 0},
     // The same over weights relaid out at import into 64-row tiles (llmp_hip_relayout_q4_k_tiles64); `lanes` -3.
     // Never a default: the layout is the caller's to declare.
     {"rows pass8 tiles64", -3, 8, 1},
+    // The row-a-lane form over the file's layout with its tile named: 64 rows (a piece a unit of each), or 32 or 16 (a
+    // piece two or four units of each row, for matrices of few rows).
+    {"rows pass8 rows64", -2, 8, 1},
+    {"rows pass8 rows32", -2, 8, 2},
+    {"rows pass8 rows16", -2, 8, 4},
 };
 constexpr int kMmaVariant = 9;
 constexpr int kRowsVariant = 10;
@@ -573,17 +579,19 @@ int DefaultVariant(int type, const llmp_vecq_desc& d, int kp, bool fused) {
   // four-token passes' 18 / 25 / 43). More tokens, and rows that form does not take: the 16 x 16 form, whose time
   // hardly depends on the tokens; the flat form's four-token pass stays under it up to five tokens for Q8_0
   // (15 / 17 / 20 / 27 us against 29 at 4096 x 14336).
-  // The row-a-lane form's time hardly depends on the tokens, but it takes 64 rows a workgroup of four waves: a matrix
-  // of fewer than 128 such tiles leaves most of the device without one, and the flat form's four-token pass is the
-  // faster up to four tokens (Q4_K 15360 x 3840, 60 tiles: 13.8 us against 24.5 at two tokens, 25 both at four;
-  // 4096 x 4096: 7.0 / 8.9 against 10.5 at two and four, 14.4 against 12.3 at eight).
+  // The row-a-lane form's time hardly depends on the tokens. Its tiles are 64 rows a workgroup of four waves, or 32 or
+  // 16 where the matrix has too few rows to give most compute units a tile of 64 (Q4_K 15360 x 3840, 60 tiles of 64:
+  // 12.8 / 12.6 / 19 us at two, four and eight tokens in tiles of 16 against 24.8 / 24.5 / 34 in tiles of 64 and the
+  // flat form's four-token passes' 13.7 / 25 / 44; 4096 x 4096: 7.0 / 7.1 / 8.0 against 10.5 / 10.5 / 12.4 and
+  // 7.0 / 9.0 / 14.5). At two tokens the four-token pass is as fast, here a tenth faster (5120 x 5120: 8.0 against
+  // 9.2 us) and there a tenth slower; the row-a-lane form from two tokens keeps a token's bits the same at every count.
   // Q8_0: the same (4096 x 14336: 16.2-17.4 us at 2 to 8 tokens against 19 / 22 / 31 for the four-token passes and
-  // the 16 x 16 form; 4096 x 4096: 14.5-14.8 us at 5 to 8 tokens against 15.6-19.4, but 13.4 against 8.4-12.6 at 2 to
-  // 4); with a GLU the pair's two-token pass is as fast, so from three.
+  // the 16 x 16 form; 14336 x 4096 in tiles of 16 rows: 17 us at 2 to 4 tokens and 22 at 5 to 8 against 26 / 35 / 44
+  // / 54-82).
   if (tokens > 1 && !fused && (type == LLMP_TYPE_Q4_K || type == LLMP_TYPE_Q8_0) && RowsTakes(type, d)) {
-    const int64_t tiles = static_cast<int64_t>((d.nrows + 63) / 64) * d.used;
-    const int from = type == LLMP_TYPE_Q8_0 && d.g != nullptr ? 3 : 2;
-    if (tiles >= 128 ? tokens >= from : tokens >= 5) return kRowsVariant;
+    // (More than eight tokens are launches of eight: for rows too long for the 16 x 16 form. Q4_K 15360 x 3840 at
+    // sixteen tokens: 2 x 19 us against the four-token passes' 82.)
+    if (tokens <= 8 || !MmaTakes(type, d)) return kRowsVariant;
   }
   // (A plain Q4_K product of few rows: the four-token pass up to four tokens, 9.0 us against the 16 x 16 form's 13.1
   // at 4096 x 4096.)
@@ -681,12 +689,14 @@ int Launch(int type, const llmp_vecq_desc* d, const llmp_vecq_source* x, int var
     return LaunchStatus("vecq");
   }
   if (v.lanes == -2) {
-    if (offsets != nullptr || !RowsTakes(type, *d))
-      return Refuse(1, "vecq: the row-a-lane form takes 2 to 8 tokens of a dense or grouped Q4_K product, rows of 1024 values "
-                       "or more, or of a Q8_0 product, rows of whole 256 values, 512 or more, at 16-byte boundaries");
+    if (offsets != nullptr || !RowsTakes(type, *d, v.flight > 0 ? v.flight : 1))
+      return Refuse(1, "vecq: the row-a-lane form takes 2 to 16 tokens of a dense or grouped Q4_K product, rows of 1024 values "
+                       "or more, or of a Q8_0 product, rows of whole 256 values, 512 or more, at 16-byte boundaries; tiles of 32 "
+                       "or 16 rows, rows of two or four times that");
     if (x != nullptr) return Refuse(1, "vecq: the row-a-lane form takes Q8_1 activations");
     if (dump != nullptr) return Refuse(1, "vecq: block sums are of the one-token variants");
     a.tiled = type == LLMP_TYPE_Q8_0 ? 3 : 0;
+    a.parts = v.flight;
     LaunchRows(a, static_cast<hipStream_t>(stream));
     return LaunchStatus("vecq");
   }

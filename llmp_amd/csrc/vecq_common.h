@@ -114,6 +114,10 @@ struct VecQArgs {
   // The row-a-lane form over weights the importer relaid out (llmp_hip_relayout_q4_k_tiles64): within every 64
   // rows the blocks lie super-block after super-block, a super-block's 64 rows together.
   int tiled = 0;
+  // The row-a-lane form: units of each wave's quarter of a row whose tokens are staged at a time (0: the whole row's).
+  int span = 0;
+  // and the super-blocks of a row in a piece: 1 (tiles of 64 rows), 2 or 4 (of 32 or 16, Q4_K); 0: the launcher's choice.
+  int parts = 0;
 };
 
 __device__ __forceinline__ float Silu(float x) {
@@ -203,7 +207,8 @@ bool MmaTakes(int type, const llmp_vecq_desc& d);
 void LaunchMma(int type, const VecQArgs& a, hipStream_t stream);
 
 // The row-a-lane kernel for 2 to 8 tokens of a dense or grouped Q4_K product over Q8_1 activations (vecq_rows.hip).
-bool RowsTakes(int type, const llmp_vecq_desc& d);
+constexpr int kRowsTokensMost = 16;  // of the row-a-lane form (the operation's most): eight a launch
+bool RowsTakes(int type, const llmp_vecq_desc& d, int parts = 1);  // parts: the units of a row in a piece (tiles of 64 / parts rows)
 bool RowsTiledTakes(int type, const llmp_vecq_desc& d);
 void LaunchRows(const VecQArgs& a, hipStream_t stream);
 

@@ -106,9 +106,12 @@ struct Tokens {
 // tokens. `codes`, `d8`: the LDS addresses of the super-block's, `codes` at this lane's token; `sums`: of this
 // lane's token's eight ds8. Every LDS read is a RingRead (see there): a pair of sub-blocks' token operands are
 // asked for while the pair before is multiplied.
-template <int NT>
+// CBSZ: the matrix instructions' broadcast of the tokens, 4 from the wave's first lanes to all of it, 3 or 2 from the
+// first lanes of every half or quarter of the wave to that half or quarter (whose lanes then stand at a super-block
+// of their own: `codes`, `d8`, `sums` are this lane's); `live`: 1, or 0 for a lane whose super-block does not count.
+template <int NT, int CBSZ = 4>
 __device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t d8, uint32_t sums, float (&out)[NT],
-                                         V4f (&mins)[NT / 4]) {
+                                         V4f (&mins)[NT / 4], float live = 1.0f) {
 #pragma clang fp contract(off)
   using T = Tokens<NT>;
   constexpr int kQuads = NT / 4;
@@ -142,7 +145,8 @@ __device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t 
   landed(c[0], scale[0]);
   U32x4 header4;
   header4.x = header[0], header4.y = header[1], header4.z = header[2], header4.w = header[3];
-  const Q4KHeader h = DecodeQ4KHeader(header4);
+  Q4KHeader h = DecodeQ4KHeader(header4);
+  if constexpr (CBSZ != 4) h.d *= live, h.dmin *= live;
   const float ds8[8] = {AsFloat(s_lo[0]), AsFloat(s_lo[1]), AsFloat(s_lo[2]),
                         AsFloat(s_lo[3]), AsFloat(s_hi[0]), AsFloat(s_hi[1]),
                         AsFloat(s_hi[2]), AsFloat(s_hi[3])};
@@ -168,12 +172,12 @@ __device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t 
     for (int s = 0; s < 8; ++s) {
       const int low = static_cast<int>(w[8 * p + s] & 0x0F0F0F0Fu), high = static_cast<int>((w[8 * p + s] >> 4) & 0x0F0F0F0Fu);
       if constexpr (kQuads >= 1) {
-        sum[0][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][0], 4, 0, 0);
-        sum[1][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][0], 4, 0, 0);
+        sum[0][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][0], CBSZ, 0, 0);
+        sum[1][0] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][0], CBSZ, 0, 0);
       }
       if constexpr (kQuads >= 2) {
-        sum[0][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][1], 4, 1, 0);
-        sum[1][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][1], 4, 1, 0);
+        sum[0][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[0][s]), low, sum[0][1], CBSZ, 1, 0);
+        sum[1][1] = __builtin_amdgcn_mfma_i32_4x4x4i8(static_cast<int>(code[1][s]), high, sum[1][1], CBSZ, 1, 0);
       }
     }
 #pragma unroll
@@ -181,8 +185,8 @@ __device__ __forceinline__ void PieceDot(uint32_t row, uint32_t codes, uint32_t 
       const int g = 2 * p + upper;
       const float sc = static_cast<float>((h.sc[g >> 2] >> (8 * (g & 3))) & 0xFFu);
       const float dm = h.dmin * static_cast<float>((h.mn[g >> 2] >> (8 * (g & 3))) & 0xFFu);
-      if constexpr (kQuads >= 1) mins[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[0], 4, 0, 0);
-      if constexpr (kQuads >= 2) mins[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[1], 4, 1, 0);
+      if constexpr (kQuads >= 1) mins[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[0], CBSZ, 0, 0);
+      if constexpr (kQuads >= 2) mins[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds8[g], dm, mins[1], CBSZ, 1, 0);
 #pragma unroll
       for (int tq = 0; tq < kQuads; ++tq) {
         const U32v4 d4 = ds[upper * kQuads + tq];
@@ -280,8 +284,9 @@ __device__ __forceinline__ void PieceDotQ8(uint32_t stage, const uint32_t (&swiz
 // unit of four 34-byte blocks, which begins `shift` bytes (0 or 8, the same for every row: rows are whole 16-byte
 // chunks apart) into it. Blocks 1 and 3 of a unit have their codes on dword boundaries; blocks 0 and 2 have them two
 // bytes off, and every dword of theirs is put together from two (v_alignbyte).
-template <int NT>
-__device__ __forceinline__ void PieceDotQ8Native(uint32_t row, uint32_t codes, uint32_t d8, float (&out)[NT]) {
+// CBSZ, `live`: as PieceDot's.
+template <int NT, int CBSZ = 4>
+__device__ __forceinline__ void PieceDotQ8Native(uint32_t row, uint32_t codes, uint32_t d8, float (&out)[NT], float live = 1.0f) {
 #pragma clang fp contract(off)
   using T = Tokens<NT>;
   constexpr int kQuads = NT / 4;
@@ -325,15 +330,16 @@ __device__ __forceinline__ void PieceDotQ8Native(uint32_t row, uint32_t codes, u
     for (int s = 0; s < 8; ++s) {
       weight[s] = (b & 1) != 0 ? d[first + 1 + s] : __builtin_amdgcn_alignbyte(d[first + 1 + s], d[first + s], 2);
     }
-    const float dw = HalfBitsToFloat((b & 1) != 0 ? d[first] >> 16 : d[first] & 0xFFFFu);
+    float dw = HalfBitsToFloat((b & 1) != 0 ? d[first] >> 16 : d[first] & 0xFFFFu);
+    if constexpr (CBSZ != 4) dw *= live;
     V4i sum[kQuads];
 #pragma unroll
     for (int tq = 0; tq < kQuads; ++tq) sum[tq] = V4i{0, 0, 0, 0};
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int code = static_cast<int>(c2[s >> 2][s & 3]);
-      if constexpr (kQuads >= 1) sum[0] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[0], 4, 0, 0);
-      if constexpr (kQuads >= 2) sum[1] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[1], 4, 1, 0);
+      if constexpr (kQuads >= 1) sum[0] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[0], CBSZ, 0, 0);
+      if constexpr (kQuads >= 2) sum[1] = __builtin_amdgcn_mfma_i32_4x4x4i8(code, static_cast<int>(weight[s]), sum[1], CBSZ, 1, 0);
     }
 #pragma unroll
     for (int tq = 0; tq < kQuads; ++tq) {
@@ -353,25 +359,37 @@ constexpr int kQ8PieceBytes = kTileRows * 136;  // a relaid-out Q8_0 piece in de
 
 // grid (workgroups, slots); LDS: the tokens, then the waves' rings (whose first bytes also carry the
 // waves' sums to their meeting). FMT 0: Q4_K (a unit a super-block); 1: Q8_0 relaid out (a unit four blocks); 2: Q8_0
-// in the file's layout.
-template <bool kGlu, int NT, int STAGES, int FMT = 0>
+// in the file's layout; 3, 4: Q4_K, and 5, 6: Q8_0 in the file's layout, in tiles of 32 and 16 rows (for matrices of
+// few rows, whose 64-row tiles would leave most of the device idle): a piece is two or four consecutive units of each
+// row, a half or a quarter of the wave's lanes at each, the lanes' sums meeting at the tile's end.
+// kSpans: the tokens staged a span of the row at a time (below).
+template <bool kGlu, int NT, int STAGES, int FMT = 0, bool kSpans = false>
 __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   using T = Tokens<NT>;
   constexpr int kMatrices = kGlu ? 2 : 1;
-  constexpr int kUnitBlocks = FMT == 0 ? 8 : 4;
+  constexpr bool kQ4K = FMT == 0 || FMT == 3 || FMT == 4;
+  constexpr bool kNative8 = FMT == 2 || FMT >= 5;
+  constexpr int kParts = FMT == 3 || FMT == 5 ? 2 : FMT == 4 || FMT == 6 ? 4 : 1;  // units of a row that a piece holds
+  constexpr int kRows = kTileRows / kParts;                // rows a tile
+  constexpr int kUnitBlocks = kQ4K ? 8 : 4;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int blocks = d.ncols_x / 32;
-  const int nsb = blocks / kUnitBlocks;  // units a row
+  const int nsb = d.ncols_x / 32 / kUnitBlocks;  // units a row
+  // Rows whose tokens do not fit LDS beside the rings are taken in spans, the span's tokens staged anew (for every
+  // tile: long rows are the down projections' few tiles), the sums carried in registers. A span is `a.span` units of
+  // every wave's own quarter of the row, so a wave adds its units in the row's order whatever the spans: the same
+  // bits as one span gives.
+  const int spans = kSpans ? ((nsb + kRowsWaves - 1) / kRowsWaves + a.span - 1) / a.span : 1;
+  const int staged_blocks = (kSpans ? kRowsWaves * a.span : nsb) * kUnitBlocks;  // the room for tokens
   const int slot = blockIdx.y;
   uint8_t* codes = lds;
-  uint8_t* d8 = codes + blocks * T::kCodesBlock;
-  uint8_t* sums = d8 + blocks * T::kScalesBlock;
-  uint8_t* rings = lds + ((T::Bytes(blocks) + 1023) & ~static_cast<size_t>(1023));
+  uint8_t* d8 = codes + staged_blocks * T::kCodesBlock;
+  uint8_t* sums = d8 + staged_blocks * T::kScalesBlock;
+  uint8_t* rings = lds + ((T::Bytes(staged_blocks) + 1023) & ~static_cast<size_t>(1023));
   uint8_t* ring = rings + wave * (STAGES * kPieceBytes);
 
   auto lds_address = [](const uint8_t* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); };  // the pointer's low half
@@ -386,9 +404,28 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
     uint32_t scale;      // d8 and the block's sum as F16
   };
   HeldBlock held[kHeld];
-  const int last_block = NT * blocks - 1;
+  // The span at hand: how far into the quarters it starts, this wave's units of it, and the unit that the first
+  // staged one of this wave is (the staged tokens of a wave's units follow those of the wave before).
+  const int blocks = staged_blocks, last_block = NT * blocks - 1;
+  const int quarter_first = wave * nsb / kRowsWaves, quarter_end = (wave + 1) * nsb / kRowsWaves;
+  int span_at = 0, sb_first = quarter_first, sb_end = quarter_end, staged_from = 0;
+  int pieces = (sb_end - sb_first + kParts - 1) / kParts * kMatrices;
+  auto set_span = [&](int span) {
+    span_at = span * a.span;
+    sb_first = quarter_first + span_at;
+    sb_end = min(sb_first + a.span, quarter_end);
+    staged_from = sb_first - wave * a.span;
+    pieces = (sb_end - sb_first + kParts - 1) / kParts * kMatrices;
+  };
+  if constexpr (kSpans) set_span(0);
   auto token_block = [&](int index) {
-    const int t = index / blocks, b = index - t * blocks;
+    const int t = index / blocks;
+    int b = index - t * blocks;
+    if constexpr (kSpans) {  // the staged unit's place in the row: its wave's quarter, the span's start, its own
+      const int unit = b / kUnitBlocks, of_wave = unit / a.span;
+      const int in_row = min(of_wave * nsb / kRowsWaves + span_at + (unit - of_wave * a.span), nsb - 1);
+      b = in_row * kUnitBlocks + (b - unit * kUnitBlocks);
+    }
     const int from = min(t, tokens - 1);  // the tokens a group lacks repeat its last: computed and dropped
     return static_cast<const uint8_t*>(d.y) +
            (static_cast<int64_t>(from) * d.y_token + static_cast<int64_t>(slot) * d.y_slot + b) * kQ8Block;
@@ -420,11 +457,10 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   // This wave's quarter of K, and this lane's sixteen bytes of each of a piece's nine loads: byte
   // 1024 j + 16 lane of the 64 rows x 144 bytes lies in row (that / 144), rows past the matrix's end
   // repeating its last.
-  const int sb_first = wave * nsb / kRowsWaves, sb_end = (wave + 1) * nsb / kRowsWaves;
-  const int pieces = (sb_end - sb_first) * kMatrices;
-  const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
+  const int tiles = (d.nrows + kRows - 1) / kRows;
   const int64_t matrix_block = static_cast<int64_t>(slot) * d.stride_expert;
-  const int token_lane = min(lane, NT - 1);
+  const int part = lane / kRows;  // which of a piece's super-blocks of its row this lane multiplies
+  const int token_lane = min(lane & (kRows - 1), NT - 1);
   const uint32_t ring_at = lds_address(ring) + (FMT != 1 ? static_cast<uint32_t>(lane) * 144u : 0u);  // this lane's row of a stage (Q8_0 relaid out: the stage)
   uint32_t swizzle[8];
 #pragma unroll
@@ -435,30 +471,38 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   const uint32_t sums_at = lds_address(sums) + static_cast<uint32_t>(token_lane) * 32u;
 
   uint32_t offsets[kPieceLoads];
+  [[maybe_unused]] uint32_t odd_first[kPieceLoads];  // (narrow Q8_0 tiles: what a piece whose first unit is an odd one adds)
   const uint8_t* up_tile = nullptr;
   const uint8_t* gate_tile = nullptr;
   auto aim = [&](int tile) {
-    const int row0 = tile * kTileRows;
+    const int row0 = tile * kRows;
 #pragma unroll
     for (int j = 0; j < kPieceLoads; ++j) {
       const int byte = j * (kWave * 16) + lane * 16;
-      const int row = byte / 144;
+      const int row = byte / 144;  // the lane that reads these 144 bytes of the stage
       // (Relaid-out weights: a piece is 9216 consecutive bytes, every 64-byte unit of HBM asked for once.)
-      if constexpr (FMT == 2) {
-        // A row's 144 bytes from the 16-byte boundary at or below its unit (issue adds the unit's place).
-        offsets[j] = static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 34u +
-                     static_cast<uint32_t>(byte - row * 144);
+      if constexpr (kNative8) {
+        // A row's 144 bytes from the 16-byte boundary at or below its unit (issue adds the place of the piece's first
+        // unit). Narrow tiles: unit u of the piece lies 136 u bytes on, its boundary 0, 128, 272, 400 on where the
+        // first unit begins at a boundary (an even unit), 0, 144, 272, 416 where it begins 8 bytes past one.
+        const int u = row / kRows;
+        offsets[j] = static_cast<uint32_t>(min(row0 + (row & (kRows - 1)), d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 34u +
+                     static_cast<uint32_t>((u * 136 & ~15) + (byte - row * 144));
+        odd_first[j] = static_cast<uint32_t>((u & 1) * 16);
       } else if constexpr (FMT == 1) {
         // The piece's last 512 bytes (the scales) by the lower half of the wave, the upper half the same again
         // (into the stage's spare 512 bytes).
         offsets[j] = j < 8 ? static_cast<uint32_t>(byte) : 8192u + static_cast<uint32_t>(lane & 31) * 16u;
+      } else if constexpr (kQ4K && kParts > 1) {
+        offsets[j] = static_cast<uint32_t>(min(row0 + (row & (kRows - 1)), d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
+                     static_cast<uint32_t>(row / kRows * 144 + (byte - row * 144));
       } else {
         offsets[j] = a.tiled != 0 ? static_cast<uint32_t>(byte)
                                   : static_cast<uint32_t>(min(row0 + row, d.nrows - 1) - row0) * static_cast<uint32_t>(d.stride_row) * 144u +
                                         static_cast<uint32_t>(byte - row * 144);
       }
     }
-    const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * (FMT == 0 ? 144 : 34);
+    const int64_t at = (matrix_block + static_cast<int64_t>(row0) * d.stride_row) * (kQ4K ? 144 : 34);
     up_tile = static_cast<const uint8_t*>(d.w) + at;
     if constexpr (kGlu) gate_tile = static_cast<const uint8_t*>(d.g) + at;
   };
@@ -467,19 +511,25 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   // wave's last piece its last again (a load is never skipped: the waits count loads).
   auto issue = [&](int i) {
     const int piece = min(i, pieces - 1);
-    int gate = 0, sb = sb_first + piece;
+    const int count = (sb_end - sb_first + kParts - 1) / kParts;
+    int gate = 0, sb = piece;
     if constexpr (kGlu) {
-      const int paired = (sb_end - sb_first) / 2 * 4;  // pieces of whole pairs of super-blocks
+      const int paired = count / 2 * 4;  // pieces of whole pairs of super-blocks
       gate = piece < paired ? (piece & 3) >> 1 : piece - paired;
-      sb = sb_first + (piece < paired ? (piece >> 2) * 2 + (piece & 1) : sb_end - sb_first - 1);
+      sb = piece < paired ? (piece >> 2) * 2 + (piece & 1) : count - 1;
     }
+    // (Narrow tiles: the last piece of a quarter that is no whole number of pieces starts early, see piece_dot.)
+    sb = sb_first + (kParts == 1 ? sb : min(kParts * sb, sb_end - sb_first - kParts));
     const uint8_t* from = (gate != 0 ? gate_tile : up_tile) +
-                          (FMT == 2 ? static_cast<int64_t>(sb) * 136 & ~int64_t{15}
+                          (kNative8 ? static_cast<int64_t>(sb) * 136 & ~int64_t{15}
                                     : static_cast<int64_t>(sb) * (FMT == 1 ? kQ8PieceBytes : a.tiled != 0 ? kPieceBytes : 144));
     uint8_t* to = ring + (i % STAGES) * kPieceBytes;
+    [[maybe_unused]] const uint32_t odd = (sb & 1) != 0 ? ~0u : 0u;
 #pragma unroll
-    for (int j = 0; j < kPieceLoads; ++j)
-      __builtin_amdgcn_global_load_lds((GlobalPointer)(from + offsets[j]), (LdsPointer)(to + j * (kWave * 16)), 16, 0, 0);
+    for (int j = 0; j < kPieceLoads; ++j) {
+      const uint32_t offset = kNative8 && kParts > 1 ? offsets[j] + (odd_first[j] & odd) : offsets[j];
+      __builtin_amdgcn_global_load_lds((GlobalPointer)(from + offset), (LdsPointer)(to + j * (kWave * 16)), 16, 0, 0);
+    }
   };
   // Before piece i is multiplied: the piece STAGES - 1 ahead is asked for, and all but the STAGES - 1 youngest
   // pieces have landed. At the tile's end nothing is asked for (a repeat of the last piece would be read from HBM
@@ -518,35 +568,60 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kPieceLoads * (STAGES - 2)));
 #pragma unroll
   for (int it = 0; it < kHeld; ++it) stage_block(held[it], tid + it * kRowsGroup);
-  for (int index = tid + kHeld * kRowsGroup; index <= last_block; index += kRowsGroup) {  // rows too long for that
-    HeldBlock block;
-    ask_block(index, block);
+  for (int index = tid + kHeld * kRowsGroup; index <= last_block; index += kHeld * kRowsGroup) {  // rows too long for that
+#pragma unroll
+    for (int it = 0; it < kHeld; ++it) ask_block(index + it * kRowsGroup, held[it]);
     asm volatile("s_waitcnt vmcnt(0)");
-    stage_block(block, index);
+#pragma unroll
+    for (int it = 0; it < kHeld; ++it) stage_block(held[it], index + it * kRowsGroup);
   }
 
   for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int row0 = tile * kTileRows;
-    if (tile != static_cast<int>(blockIdx.x)) prologue(tile);
+    const int row0 = tile * kRows;
     float up_out[NT], gate_out[NT];
     V4f up_mins[NT / 4], gate_mins[NT / 4];
 #pragma unroll
     for (int t = 0; t < NT; ++t) up_out[t] = 0.0f, gate_out[t] = 0.0f;
 #pragma unroll
     for (int tq = 0; tq < NT / 4; ++tq) up_mins[tq] = V4f{0.0f, 0.0f, 0.0f, 0.0f}, gate_mins[tq] = up_mins[tq];
+    for (int span = 0; span < spans; ++span) {
+    if (tile != static_cast<int>(blockIdx.x) || span != 0) {
+      if constexpr (kSpans) {
+        __syncthreads();  // the tokens' readers are done with the span before
+        set_span(span);
+        for (int index = tid; index <= last_block; index += kHeld * kRowsGroup) {
+#pragma unroll
+          for (int it = 0; it < kHeld; ++it) ask_block(index + it * kRowsGroup, held[it]);
+          asm volatile("s_waitcnt vmcnt(0)");
+#pragma unroll
+          for (int it = 0; it < kHeld; ++it) stage_block(held[it], index + it * kRowsGroup);
+        }
+      }
+      prologue(tile);
+    }
     LdsBarrier();  // the tokens are staged
     {
       // Two super-blocks of the up matrix, then the same two of the gate matrix: neighbours in a row share a 64-byte
       // unit of HBM more often than not, and the sooner the second asks for it the likelier L2 still has it.
-      const int count = sb_end - sb_first;
+      const int count = (sb_end - sb_first + kParts - 1) / kParts;
       int i = 0;
-      auto piece_dot = [&](int sb, float (&out)[NT], V4f (&mins)[NT / 4]) {
-        const uint32_t sb_codes = codes_at + static_cast<uint32_t>(sb * kUnitBlocks * T::kCodesBlock);
-        const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(sb * kUnitBlocks * T::kScalesBlock);
-        const uint32_t sb_sums = sums_at + static_cast<uint32_t>(sb * T::kSumsSb);
+      auto piece_dot = [&](int step, float (&out)[NT], V4f (&mins)[NT / 4]) {
+        // Narrow tiles: the piece starts kParts super-blocks a step on, the last one kParts before the quarter's end,
+        // where the lanes at super-blocks that the step before had do not count.
+        const int start = kParts == 1 ? step : min(kParts * step, sb_end - sb_first - kParts);
+        const int sb = sb_first + start + part;
+        [[maybe_unused]] const float live = start + part >= kParts * step ? 1.0f : 0.0f;
+        const int staged_unit = sb - staged_from;
+        const uint32_t sb_codes = codes_at + static_cast<uint32_t>(staged_unit * kUnitBlocks * T::kCodesBlock);
+        const uint32_t sb_d8 = d8_at + static_cast<uint32_t>(staged_unit * kUnitBlocks * T::kScalesBlock);
+        const uint32_t sb_sums = sums_at + static_cast<uint32_t>(staged_unit * T::kSumsSb);
         next_piece(i);
         if constexpr (FMT == 0) {
           PieceDot<NT>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins);
+        } else if constexpr (kQ4K && kParts > 1) {
+          PieceDot<NT, kParts == 2 ? 3 : 2>(ring_at + (i % STAGES) * kPieceBytes, sb_codes, sb_d8, sb_sums, out, mins, live);
+        } else if constexpr (kNative8 && kParts > 1) {
+          PieceDotQ8Native<NT, kParts == 2 ? 3 : 2>(ring_at + (i % STAGES) * kPieceBytes + static_cast<uint32_t>((sb & 1) * 8), sb_codes, sb_d8, out, live);
         } else if constexpr (FMT == 2) {
           PieceDotQ8Native<NT>(ring_at + (i % STAGES) * kPieceBytes + static_cast<uint32_t>((sb & 1) * 8), sb_codes, sb_d8, out);
         } else {
@@ -557,26 +632,34 @@ __global__ __launch_bounds__(kRowsGroup, 2) void VecQRows(const VecQArgs a) {
       };
       for (int n = 0; n < count; n += kMatrices) {
         const int width = min(kMatrices, count - n);
-        for (int w = 0; w < width; ++w) piece_dot(sb_first + n + w, up_out, up_mins);
+        for (int w = 0; w < width; ++w) piece_dot(n + w, up_out, up_mins);
         if constexpr (kGlu) {
-          for (int w = 0; w < width; ++w) piece_dot(sb_first + n + w, gate_out, gate_mins);
+          for (int w = 0; w < width; ++w) piece_dot(n + w, gate_out, gate_mins);
         }
       }
     }
+    }
     // The four quarters of K meet: [wave][matrix][token][row] floats at the head of each wave's ring.
+    // (Narrow tiles: the lanes of a row first, halves of the wave then quarters; every lane of a row ends with the sum.)
     float* mine = reinterpret_cast<float*>(ring);
+    auto of_row = [&](float mine_alone) {
+#pragma clang fp contract(off)
+      if constexpr (kParts >= 2) mine_alone += __shfl_xor(mine_alone, 32);
+      if constexpr (kParts >= 4) mine_alone += __shfl_xor(mine_alone, 16);
+      return mine_alone;
+    };
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma clang fp contract(off)
-      mine[t * kTileRows + lane] = up_out[t] - up_mins[t / 4][t % 4];
-      if constexpr (kGlu) mine[(NT + t) * kTileRows + lane] = gate_out[t] - gate_mins[t / 4][t % 4];
+      mine[t * kRows + (lane & (kRows - 1))] = of_row(up_out[t] - up_mins[t / 4][t % 4]);
+      if constexpr (kGlu) mine[(NT + t) * kRows + (lane & (kRows - 1))] = of_row(gate_out[t] - gate_mins[t / 4][t % 4]);
     }
     __syncthreads();
-    for (int index = tid; index < tokens * kTileRows; index += kRowsGroup) {
+    for (int index = tid; index < tokens * kRows; index += kRowsGroup) {
 #pragma clang fp contract(off)
-      const int t = index / kTileRows, r = index - t * kTileRows;
+      const int t = index / kRows, r = index - t * kRows;
       auto total = [&](int matrix) {
-        const float* at = reinterpret_cast<const float*>(rings) + (matrix * NT + t) * kTileRows + r;
+        const float* at = reinterpret_cast<const float*>(rings) + (matrix * NT + t) * kRows + r;
         constexpr int kRing = STAGES * kPieceBytes / 4;
         return (at[0] + at[kRing]) + (at[2 * kRing] + at[3 * kRing]);
       };
@@ -601,24 +684,82 @@ int StagesFor(int blocks) {
   return 0;
 }
 
-template <bool kGlu, int NT, int STAGES, int FMT>
-void LaunchRowsKernel(const VecQArgs& a, dim3 grid, hipStream_t stream) {
+// The units of a wave's quarter that a span takes, for rows of `units` units of `unit_blocks` blocks: 0 where the whole
+// row's tokens fit beside the rings, else those of the fewest spans that do (every wave with a unit or more in every
+// span), -1 if none.
+// `parts`: the units that a wave's share of a span is at least (a piece's units in narrow tiles), and that a span is a
+// multiple of: a unit then meets the same lane whatever the spans, and the sums the same order.
+template <int NT>
+int SpanFor(int units, int unit_blocks, int parts = 1) {
+  const int shortest = units / kRowsWaves, longest = (units + kRowsWaves - 1) / kRowsWaves;
+  if (shortest < parts) return -1;
+  if (StagesFor<NT>(units * unit_blocks) != 0) return 0;
+  for (int spans = 2; spans <= shortest; ++spans) {
+    const int span = ((longest + spans - 1) / spans + parts - 1) / parts * parts;  // whole pieces in all but the last
+    if (shortest - (spans - 1) * span < parts) continue;
+    if (StagesFor<NT>(kRowsWaves * span * unit_blocks) != 0) return span;
+  }
+  return -1;
+}
+
+// Tiles of 64 rows, or of 32 or 16 (the file's layouts) where that many more workgroups still find a compute
+// unit each and the rows are long enough for a piece of two or four super-blocks a wave and span.
+int RowsParts(const VecQArgs& a, int cus) {
+  const llmp_vecq_desc& d = a.d;
+  if (a.tiled != 0 && a.tiled != 3) return 1;
+  const int64_t tiles = static_cast<int64_t>((d.nrows + kTileRows - 1) / kTileRows) * d.used;
+  const int unit_blocks = a.tiled == 3 ? 4 : 8, units = d.ncols_x / 32 / unit_blocks;
+  for (int parts = 4; parts > 1; parts /= 2) {
+    if (tiles * parts > cus) continue;
+    if ((d.tokens <= 4 ? SpanFor<4>(units, unit_blocks, parts) : SpanFor<8>(units, unit_blocks, parts)) >= 0) return parts;
+  }
+  return 1;
+}
+
+template <bool kGlu, int NT, int STAGES, int FMT, bool kSpans = false>
+void LaunchRowsKernel(const VecQArgs& a, int staged_blocks, dim3 grid, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&VecQRows<kGlu, NT, STAGES, FMT>), static_cast<int>(kRowsLdsLimit), &sized)) return;
-  const size_t lds = ((Tokens<NT>::Bytes(a.d.ncols_x / 32) + 1023) & ~static_cast<size_t>(1023)) +
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQRows<kGlu, NT, STAGES, FMT, kSpans>), static_cast<int>(kRowsLdsLimit), &sized)) return;
+  const size_t lds = ((Tokens<NT>::Bytes(staged_blocks) + 1023) & ~static_cast<size_t>(1023)) +
                      static_cast<size_t>(kRowsWaves) * STAGES * kPieceBytes;
-  hipLaunchKernelGGL((VecQRows<kGlu, NT, STAGES, FMT>), grid, dim3(kRowsGroup), lds, stream, a);
+  hipLaunchKernelGGL((VecQRows<kGlu, NT, STAGES, FMT, kSpans>), grid, dim3(kRowsGroup), lds, stream, a);
+}
+
+// Three stages a wave where they fit beside the whole row's tokens, else two; two with spans.
+template <bool kGlu, int NT, int FMT>
+void LaunchRowsFormat(const VecQArgs& a, int staged_blocks, dim3 grid, hipStream_t stream) {
+  if (a.span > 0) {
+    LaunchRowsKernel<kGlu, NT, 2, FMT, true>(a, staged_blocks, grid, stream);
+  } else if (StagesFor<NT>(staged_blocks) == 3) {
+    LaunchRowsKernel<kGlu, NT, 3, FMT>(a, staged_blocks, grid, stream);
+  } else {
+    LaunchRowsKernel<kGlu, NT, 2, FMT>(a, staged_blocks, grid, stream);
+  }
 }
 
 template <bool kGlu, int NT>
-void LaunchRowsStages(const VecQArgs& a, dim3 grid, hipStream_t stream) {
-  const bool three = StagesFor<NT>(a.d.ncols_x / 32) == 3;
-  if (a.tiled == 2) {
-    three ? LaunchRowsKernel<kGlu, NT, 3, 1>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 1>(a, grid, stream);
-  } else if (a.tiled == 3) {
-    three ? LaunchRowsKernel<kGlu, NT, 3, 2>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 2>(a, grid, stream);
-  } else {
-    three ? LaunchRowsKernel<kGlu, NT, 3, 0>(a, grid, stream) : LaunchRowsKernel<kGlu, NT, 2, 0>(a, grid, stream);
+void LaunchRowsStages(const VecQArgs& whole, dim3 grid, hipStream_t stream) {
+  VecQArgs a = whole;
+  const int unit_blocks = a.tiled >= 2 ? 4 : 8;
+  const int units = a.d.ncols_x / 32 / unit_blocks;
+  a.span = SpanFor<NT>(units, unit_blocks, a.parts);
+  const int staged_blocks = (a.span > 0 ? kRowsWaves * a.span : units) * unit_blocks;
+  const int format = a.tiled == 2 ? 1 : a.tiled == 3 ? (a.parts == 2 ? 5 : a.parts == 4 ? 6 : 2) : a.tiled == 0 ? (a.parts == 2 ? 3 : a.parts == 4 ? 4 : 0) : 0;
+  switch (format) {
+    case 1:
+      return LaunchRowsFormat<kGlu, NT, 1>(a, staged_blocks, grid, stream);
+    case 2:
+      return LaunchRowsFormat<kGlu, NT, 2>(a, staged_blocks, grid, stream);
+    case 3:
+      return LaunchRowsFormat<kGlu, NT, 3>(a, staged_blocks, grid, stream);
+    case 4:
+      return LaunchRowsFormat<kGlu, NT, 4>(a, staged_blocks, grid, stream);
+    case 5:
+      return LaunchRowsFormat<kGlu, NT, 5>(a, staged_blocks, grid, stream);
+    case 6:
+      return LaunchRowsFormat<kGlu, NT, 6>(a, staged_blocks, grid, stream);
+    default:
+      return LaunchRowsFormat<kGlu, NT, 0>(a, staged_blocks, grid, stream);
   }
 }
 
@@ -673,18 +814,21 @@ __global__ void RelayoutTiles64Kernel(const uint4* __restrict__ src, uint4* __re
 // least four super-blocks (a wave a quarter of K) whose staged tokens leave room for two stages a wave. Q8_0: rows of
 // whole 256 values (an even number of four-block units, so that a row's last 16-byte chunk ends inside the row), at
 // least four units, every row and matrix at a 16-byte boundary.
-bool RowsTakes(int type, const llmp_vecq_desc& d) {
+bool RowsTakes(int type, const llmp_vecq_desc& whole, int parts) {
+  // Nine to kRowsTokensMost tokens are launches of eight or fewer each.
+  llmp_vecq_desc d = whole;
+  if (d.tokens > 8 && d.tokens <= kRowsTokensMost) d.tokens = 8;
   if (type == LLMP_TYPE_Q8_0) {
     if (d.ids != nullptr || d.tokens < 2 || d.tokens > 8 || d.ncols_x % 256 != 0 || d.ncols_x / 128 < kRowsWaves) return false;
     if (d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || reinterpret_cast<uintptr_t>(d.w) % 16 != 0 ||
         (d.g != nullptr && reinterpret_cast<uintptr_t>(d.g) % 16 != 0))
       return false;
-    return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
+    return (d.tokens <= 4 ? SpanFor<4>(d.ncols_x / 128, 4, parts) : SpanFor<8>(d.ncols_x / 128, 4, parts)) >= 0;
   }
   if (type != LLMP_TYPE_Q4_K || d.ids != nullptr || d.tokens < 2 || d.tokens > 8) return false;
   const int nsb = d.ncols_x / 256;
   if (nsb < kRowsWaves) return false;
-  return (d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) != 0;
+  return (d.tokens <= 4 ? SpanFor<4>(nsb, 8, parts) : SpanFor<8>(nsb, 8, parts)) >= 0;
 }
 
 // The same over relaid-out weights: whole tiles of packed rows. Q8_0 has this form alone (rows of whole units of four
@@ -692,20 +836,36 @@ bool RowsTakes(int type, const llmp_vecq_desc& d) {
 bool RowsTiledTakes(int type, const llmp_vecq_desc& d) {
   if (type == LLMP_TYPE_Q8_0) {
     if (d.ids != nullptr || d.tokens < 2 || d.tokens > 8 || d.ncols_x % 128 != 0 || d.ncols_x / 128 < kRowsWaves) return false;
-    if ((d.tokens <= 4 ? StagesFor<4>(d.ncols_x / 32) : StagesFor<8>(d.ncols_x / 32)) == 0) return false;
+    if ((d.tokens <= 4 ? SpanFor<4>(d.ncols_x / 128, 4) : SpanFor<8>(d.ncols_x / 128, 4)) < 0) return false;
     return d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 32 && d.stride_expert % (kTileRows * (d.ncols_x / 32)) == 0;
   }
-  return type == LLMP_TYPE_Q4_K && RowsTakes(type, d) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
+  return type == LLMP_TYPE_Q4_K && RowsTakes(type, d, 1) && d.nrows % kTileRows == 0 && d.stride_row == d.ncols_x / 256 &&
          d.stride_expert % (kTileRows * (d.ncols_x / 256)) == 0;
 }
 
-void LaunchRows(const VecQArgs& a, hipStream_t stream) {
+void LaunchRows(const VecQArgs& whole, hipStream_t stream) {
+  VecQArgs a = whole;
   const llmp_vecq_desc& d = a.d;
   if (g_rows_compute_units == 0) {
     const int cus = llmp_hip_compute_units();
     g_rows_compute_units = cus > 0 ? cus : 256;
   }
-  const int tiles = (d.nrows + kTileRows - 1) / kTileRows;
+  if (a.parts == 0) a.parts = RowsParts(a, g_rows_compute_units);
+  if (d.tokens > 8) {
+    // Equal shares of eight tokens or fewer, a launch each (the weights read once a launch): for rows too long for the
+    // 16 x 16 form, whose other choice is a pass for every four tokens.
+    const int launches = (d.tokens + 7) / 8, share = (d.tokens + launches - 1) / launches;
+    for (int first = 0; first < d.tokens; first += share) {
+      VecQArgs some = a;
+      some.d.tokens = min(share, d.tokens - first);
+      some.d.y = static_cast<const uint8_t*>(d.y) + static_cast<int64_t>(first) * d.y_token * kQ8Block;
+      some.d.dst = d.dst + static_cast<int64_t>(first) * d.dst_token;
+      LaunchRows(some, stream);
+    }
+    return;
+  }
+  const int tile_rows = kTileRows / a.parts;
+  const int tiles = (d.nrows + tile_rows - 1) / tile_rows;
   int groups = g_rows_compute_units / d.used;
   if (groups < 1) groups = 1;
   if (groups > tiles) groups = tiles;

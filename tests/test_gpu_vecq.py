@@ -102,8 +102,10 @@ def test_every_variant_matches_and_random_bytes_decode(device, t):
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 42))
     want = oracle.vecq(t, w, q8, k, n, tokens=tokens)
     for variant, name in enumerate(ops.vecq_variants()):
-        if name.endswith("tiles64"):
-            # the relaid-out variant takes whole tiles of 64 rows (and the layout it is named for)
+        units_a_wave = k // (256 if t == Q4_K else 128) // 4
+        if name.endswith("tiles64") or (name.endswith("rows32") and units_a_wave < 2) or (name.endswith("rows16") and units_a_wave < 4):
+            # the relaid-out variant takes whole tiles of 64 rows (and the layout it is named for); tiles of 32 and 16
+            # rows take rows of two and four units a wave (a unit is 256 values of Q4_K, 128 of Q8_0)
             with pytest.raises(ops.KernelFailure):
                 ops.vecq(t, dev(w, device), dev(q8, device), k, n, tokens=tokens, variant=variant)
             continue
@@ -297,18 +299,36 @@ def test_matrix_core_forms_sub_block_sums_are_exact_integers(device, variant, k,
     assert np.array_equal(got.reshape(tokens, n), want.astype(np.float32))
 
 
-@pytest.mark.parametrize("k,n,tokens", [(1024, 17, 2), (2816, 130, 5), (6144, 64, 8), (16384, 70, 4), (3840, 200, 7)])
+@pytest.mark.parametrize("k,n,tokens", [(1024, 17, 2), (2816, 130, 5), (6144, 64, 8), (16384, 70, 4), (3840, 200, 7),
+                                        (15360, 70, 8), (20480, 130, 6), (32768, 64, 3), (9472, 20, 8)])
 def test_row_a_lane_form_matches_oracle(device, k, n, tokens):
     """Variant 10 (Q4_K, a weight row a lane, 2 to 8 tokens): dense with and without a GLU, rows that end within a
-    tile of 64, three grouped matrices; and what it refuses: routed products, one token, nine, short rows."""
+    tile of 64, three grouped matrices, more than eight tokens, rows whose tokens are staged a span at a time (15360 and 20480 values at 5 to
+    8 tokens, 32768 at 3, 9472 in two uneven spans); and what it refuses: routed products, one token, 17, short
+    rows."""
     t, rows = Q4_K, 10
     gate, up = make_weights(t, n, k, 331), make_weights(t, n, k, 332)
     q8 = oracle.q8_1_quantize(synth.activations(tokens, k, 333))
+    names = ops.vecq_variants()
+    assert names[rows] == "rows pass8"
     for kw, okw in ((dict(), dict()), (dict(gate=dev(gate, device), glu=ops.GLU_GEGLU), dict(gate=gate, glu=oracle.GLU_GEGLU))):
         want = oracle.vecq(t, up, q8, k, n, tokens=tokens, **okw)
         got = ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=tokens, variant=rows, **kw).cpu().numpy()
         ok, worst = rel_close(got.reshape(tokens, n), want.reshape(tokens, n), TOL, floor=1e-2 if kw else 1e-3)
         assert ok, (kw.keys(), worst)
+        # The tiles by name: 64 rows, and 32 and 16 where every wave has two and four super-blocks of a row.
+        for parts, name in ((1, "rows pass8 rows64"), (2, "rows pass8 rows32"), (4, "rows pass8 rows16")):
+            # (37 super-blocks a row are quarters of 9 and 10; eight tokens of them are staged in spans, and no span of
+            # whole four-unit pieces leaves the shortest quarter four units for the last span.)
+            if k // 256 // 4 < parts or (k == 9472 and tokens == 8 and parts == 4):
+                with pytest.raises(ops.KernelFailure):
+                    ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=tokens, variant=names.index(name), **kw)
+                continue
+            got = ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=tokens, variant=names.index(name), **kw)
+            ok, worst = rel_close(got.cpu().numpy().reshape(tokens, n), want.reshape(tokens, n), TOL, floor=1e-2 if kw else 1e-3)
+            assert ok, (name, kw.keys(), worst)
+            two = ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=2, variant=names.index(name), **kw)
+            assert torch.equal(two.view(torch.int32), got[:2].view(torch.int32)), name
     groups = 3
     w3 = make_weights(t, groups * n, k, 334).reshape(groups, -1)
     q83 = oracle.q8_1_quantize(synth.activations(tokens * groups, k, 335))
@@ -319,7 +339,19 @@ def test_row_a_lane_form_matches_oracle(device, k, n, tokens):
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
     ids = dev(np.zeros((tokens, 1), dtype=np.int32), device)
-    for bad in (dict(tokens=tokens, ids=ids, used=1, stride_expert=n * (k // 256)), dict(tokens=1), dict(tokens=9)):
+    # Nine tokens and more (to the operation's 16) are launches of eight or fewer each: every token the bits it has among eight.
+    many = min(tokens + 9, 16)
+    x_many = synth.activations(many, k, 339)
+    q8_many = dev(oracle.q8_1_quantize(x_many), device)
+    got = ops.vecq(t, dev(up, device), q8_many, k, n, tokens=many, variant=rows)
+    share = -(-many // -(-many // 8))
+    for first in range(0, many, share):
+        some = min(share, many - first)
+        alone = ops.vecq(t, dev(up, device), dev(oracle.q8_1_quantize(x_many[first:first + some]), device), k, n, tokens=some, variant=rows)
+        assert torch.equal(alone.view(torch.int32), got[first:first + some].view(torch.int32)), first
+    ok, worst = rel_close(got.cpu().numpy().reshape(many, n), oracle.vecq(t, up, oracle.q8_1_quantize(x_many), k, n, tokens=many).reshape(many, n), TOL)
+    assert ok, worst
+    for bad in (dict(tokens=tokens, ids=ids, used=1, stride_expert=n * (k // 256)), dict(tokens=1), dict(tokens=17)):
         with pytest.raises(ops.KernelFailure):
             ops.vecq(t, dev(up, device), dev(oracle.q8_1_quantize(synth.activations(bad["tokens"], k, 336)), device), k, n,
                      variant=rows, **bad)
@@ -728,7 +760,7 @@ def test_relaid_out_rows_equal_the_row_a_lane_form_bit_for_bit(device, tokens, g
     reference's layout: equal bits, and the oracle's values. Dense and grouped (two matrices, two input rows)."""
     k, n, used = 1280, 192, 2
     names = ops.vecq_variants()
-    rows_variant, tiled_variant = names.index("rows pass8"), names.index("rows pass8 tiles64")
+    rows_variant, tiled_variant = names.index("rows pass8 rows64"), names.index("rows pass8 tiles64")
     up = make_weights(Q4_K, used * n, k, 301)
     gate = make_weights(Q4_K, used * n, k, 302) if glu != ops.GLU_NONE else None
     q8 = oracle.q8_1_quantize(synth.activations(tokens * used, k, 303))
@@ -758,7 +790,8 @@ def test_relaid_out_rows_equal_the_row_a_lane_form_bit_for_bit(device, tokens, g
     assert refused.value.rejected
 
 
-@pytest.mark.parametrize("tokens,glu,k", [(2, ops.GLU_NONE, 640), (4, ops.GLU_GEGLU, 1536), (8, ops.GLU_SWIGLU, 1536), (7, ops.GLU_NONE, 4096)])
+@pytest.mark.parametrize("tokens,glu,k", [(2, ops.GLU_NONE, 640), (4, ops.GLU_GEGLU, 1536), (8, ops.GLU_SWIGLU, 1536), (7, ops.GLU_NONE, 4096),
+                                           (8, ops.GLU_NONE, 14336), (6, ops.GLU_SWIGLU, 9472)])
 def test_q8_0_rows_form_over_relaid_out_weights(device, tokens, glu, k):
     """llmp_hip_relayout_q8_0_tiles64 (codes and scales apart, 64-row tiles, four blocks a piece) and the row-a-lane
     variant that reads it for Q8_0: the layout is what the header says, the inverse gives the file's bytes back, the
@@ -803,12 +836,23 @@ def test_q8_0_rows_form_over_relaid_out_weights(device, tokens, glu, k):
         with pytest.raises(ops.KernelFailure) as refused:
             ops.vecq(Q8_0, ut, qd, k, bad.get("nrows", n), gate=gt, variant=tiled_variant, tokens=bad.get("tokens", tokens), **common)
         assert refused.value.rejected
-    # The row-a-lane form over the file's layout (rows of whole 256 values): the same arithmetic, the same bits.
-    rows_variant = ops.vecq_variants().index("rows pass8")
+    # The row-a-lane form over the file's layout (rows of whole 256 values) in tiles of 64 rows: the same arithmetic,
+    # the same bits. In tiles of 32 and 16 rows (and the launcher's choice among the three) the sums meet in another
+    # order: the oracle's values, and a token's own whatever the tokens beside it.
+    rows_variant = ops.vecq_variants().index("rows pass8 rows64")
     gd = dev(gate, device) if gate is not None else None
     if k % 256 == 0:
         native = ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=rows_variant, tokens=tokens, **common)
         assert torch.equal(native.view(torch.int32), got.view(torch.int32))
+        for name in ("rows pass8", "rows pass8 rows32", "rows pass8 rows16"):
+            narrow_variant = ops.vecq_variants().index(name)
+            if k // 512 < (4 if name.endswith("rows16") else 2 if name.endswith("rows32") else 1):
+                continue  # a wave's quarter of a row is at least a piece: two units are 1024 values a row, four 2048
+            narrow = ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=narrow_variant, tokens=tokens, **common)
+            ok, worst = rel_close(narrow.cpu().numpy(), ref, TOL)
+            assert ok, (name, worst)
+            two = ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=narrow_variant, tokens=2, **common)
+            assert torch.equal(two.view(torch.int32), narrow[:2].view(torch.int32)), name
         # Fewer rows than whole tiles, and rows apart (a pitch of eight blocks more): the form's own edges.
         pitched = torch.zeros((used * n, k // 32 + 8, 34), dtype=torch.uint8, device=device)
         pitched[:, :k // 32] = ud.view(used * n, k // 32, 34)
