@@ -119,6 +119,9 @@ PROFILED_TRAFFIC = {
     "q8_0_gate_up_swiglu_4096x2x14336_b8": _traffic(78810.1, 448.0),
     "q8_0_gate_up_swiglu_4096x2x14336_b8_tiles64": _traffic(61149.7, 448.0),
     "q4_k_down_15360x3840_b1": _traffic(16320.6, 30.0),
+    # Tiles of 16 rows: 576-byte runs of a row, and every workgroup's own copy of the tokens where L2 misses.
+    "q4_k_down_15360x3840_b4": _traffic(16805.5, 60.0),
+    "q4_k_down_15360x3840_b8": _traffic(17157.2, 120.0),
     # The GEMM's tiles re-read the operands (each activation tile by 64 workgroups, each weight tile by 8) through
     # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
     "mxfp8_gemm_2048x12288x4096": _traffic(93182.8, 49173.6),
@@ -296,16 +299,24 @@ def other_configs(device, args, only=None):
         del gates8, ups8
         torch.cuda.empty_cache()
 
-    # The same layer's down projection (15360 -> 3840, Q4_K, one token): rows of 60 super-blocks.
-    if want("q4_k_down_15360x3840_b1"):
+    # The same layer's down projection (15360 -> 3840, Q4_K): rows of 60 super-blocks, 60 tiles of 64 rows. One token, and
+    # four and eight (the row-a-lane form in tiles of 16 rows, eight tokens staged in two spans of the row).
+    down_keys = ("q4_k_down_15360x3840_b1", "q4_k_down_15360x3840_b4", "q4_k_down_15360x3840_b8")
+    if any(want(key) for key in down_keys):
         kd, nd = N, K
         wdn = dev(synth.q4_k_weights(nd, kd, 104))
         downs = [wdn] + [wdn.clone() for _ in range(-(-ROTATE_BYTES // wdn.numel()) - 1)]
-        q8 = ops.quantize_q8_1(dev(synth.activations(1, kd, 105)))
-        y = torch.empty((1, 1, nd), dtype=torch.float32, device=device)
-        us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, downs[i % len(downs)], q8, kd, nd, out=y), 4 * len(downs))
-        out["q4_k_down_15360x3840_b1"] = {"roofline": hbm_roofline("q4_k_down_15360x3840_b1", "VecQFlat<FormatQ4K>",
-                                                                   wdn.numel() + kd * 4 + nd * 4, us)}
+        for key, tokens, kernel in zip(down_keys, (1, 4, 8), ("VecQFlat<FormatQ4K>", "VecQRows<4 tokens, Q4_K in tiles of 16 rows>",
+                                                               "VecQRows<8 tokens, Q4_K in tiles of 16 rows, spans>")):
+            if not want(key):
+                continue
+            q8 = ops.quantize_q8_1(dev(synth.activations(tokens, kd, 105)))
+            y = torch.empty((tokens, 1, nd), dtype=torch.float32, device=device)
+            us = timed(lambda i: ops.vecq(ops.TYPE_Q4_K, downs[i % len(downs)], q8, kd, nd, tokens=tokens, out=y), 4 * len(downs))
+            bytes_ = wdn.numel() + (kd * 4 + nd * 4 if tokens == 1 else tokens * (kd // 32) * 36 + tokens * nd * 4)
+            out[key] = {"roofline": hbm_roofline(key, kernel, bytes_, us)}
+            if tokens > 1:
+                out[key]["workload"] = f"config 2's down projection at {tokens} tokens; not one of the benchmark's five configurations"
         del downs, wdn
         torch.cuda.empty_cache()
 
