@@ -480,11 +480,13 @@ def other_configs(device, args, only=None):
 
     # The attention that reads the quantized KV cache (ggml.flash_attn_ext.vec_q8_0, beside the path: not one of
     # the benchmark's five configurations), at config 2's model's decode shape: 16 heads over 8 KV heads of 256, one query row, 8192 cells.
-    for kind, t in (("q8_0", ops.TYPE_Q8_0), ("q4_0", ops.TYPE_Q4_0)):
-        name = f"attn_vec_{kind}_d256_h16_kv8_cells8192_rows1"
+    # (And at 32768 cells, where a wave has several tiles and the next one's loads run under the products.)
+    for kind, t, cells in (("q8_0", ops.TYPE_Q8_0, 8192), ("q4_0", ops.TYPE_Q4_0, 8192), ("q8_0", ops.TYPE_Q8_0, 32768),
+                           ("q4_0", ops.TYPE_Q4_0, 32768)):
+        name = f"attn_vec_{kind}_d256_h16_kv8_cells{cells}_rows1"
         if not want(name):
             continue
-        d_, heads, kv_heads, cells = 256, 16, 8, 8192
+        d_, heads, kv_heads = 256, 16, 8
         g = synth.rng(240)
         k_host = oracle.kv_quantize(t, g.standard_normal((cells * kv_heads, d_), dtype=np.float32)).reshape(cells, -1)
         v_host = oracle.kv_quantize(t, g.standard_normal((cells * kv_heads, d_), dtype=np.float32)).reshape(cells, -1)
@@ -503,7 +505,7 @@ def other_configs(device, args, only=None):
                                                 out=out_d, scratch=scratch), 4 * copies)
         bytes_ = 2 * kd.numel() + heads * d_ * 8 + cells * 2
         entry = {"workload": f"attention over a {kind.upper()} KV cache, head size 256, 16 heads over 8 KV heads, 1 query row, "
-                             "8192 cells (both launches: the splits and their combination); not one of the benchmark's five configurations",
+                             f"{cells} cells (both launches: the splits and their combination); not one of the benchmark's five configurations",
                  "roofline": hbm_roofline(name, "AttnVecQuantKernel + AttnCombineKernel", bytes_, us)}
         if cpu:
             entry["cpu_baseline"] = cpu_leg(

@@ -92,6 +92,33 @@ def test_config_2_q4_k_gate_up_geglu_3840_x_15360(device, tokens):
         assert np.array_equal(flipped.reshape(tokens, n)[::-1].view(np.uint32), got.reshape(tokens, n).view(np.uint32))
 
 
+@pytest.mark.parametrize("t,k,n", [(Q4_K, 15360, 3840), (Q8_0, 14336, 4096)])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 8, 16])
+def test_down_projection_at_full_size(device, t, k, n, tokens):
+    """Config 2's down projection (15360 -> 3840, Q4_K: rows of 60 super-blocks, 60 tiles of 64 rows) and a Q8_0 one of
+    the same kind (14336 -> 4096) at 1 to 16 tokens: the default forms (the flat form at one token, the row-a-lane form
+    in tiles of 16 rows at 2 to 8, eight tokens in spans, sixteen in two launches) within 1e-3 of the oracle, and the
+    same shape through the flat form's four-token passes, an independent kernel, within 1e-3 as well; a token's values
+    do not move with the tokens beside it."""
+    w = (synth.q4_k_weights if t == Q4_K else synth.q8_0_weights)(n, k, 111)
+    x = synth.activations(tokens, k, 112)
+    q8 = oracle.q8_1_quantize(x)
+    want = oracle.vecq(t, w, q8, k, n, tokens=tokens, threads=oracle.max_threads()).reshape(tokens, n)
+    wd, qd = dev(w, device), dev(q8, device)
+    got = ops.vecq(t, wd, qd, k, n, tokens=tokens)
+    ok, worst = rel_close(got.cpu().numpy().reshape(tokens, n), want, TOL)
+    assert ok, worst
+    flat = ops.vecq(t, wd, qd, k, n, tokens=tokens, variant=ops.vecq_variants().index("flat pass4" if tokens > 1 else "flat pass1"))
+    ok, worst = rel_close(flat.cpu().numpy().reshape(tokens, n), want, TOL)
+    assert ok, worst
+    if tokens > 1:
+        flipped = ops.vecq(t, wd, qd.flip(0).contiguous(), k, n, tokens=tokens)
+        assert torch.equal(flipped.flip(0).view(torch.int32), got.view(torch.int32))
+    if tokens in (4, 8):  # among fewer tokens (another instance of the kernel, the whole row staged at once): the same bits
+        fewer = ops.vecq(t, wd, qd[:tokens // 2].contiguous(), k, n, tokens=tokens // 2)
+        assert torch.equal(fewer.view(torch.int32), got[:tokens // 2].view(torch.int32))
+
+
 def test_config_2_block_sums_at_full_size(device):
     """The eight products and eight sums of every super-block of the 15360 x 3840 gate matrix, bit for bit."""
     k, n = 3840, 15360
