@@ -3,10 +3,11 @@
 // nothing expanded into device memory. The reference launches GGML's vector kernel; this is a gfx950 kernel with the
 // same operands and the same outline (Q quantized to Q8_1 in LDS for the K product; an online softmax; F32 output).
 //
-// A workgroup of four waves takes one KV head, a run of cells (a split) and up to eight queries that share that KV
-// head (the head's group of query heads times a few rows), so K and V are read once for all of them. A wave takes
-// tiles of 64 cells (32 at D 512): its K and V rows come by global_load_lds as 16-byte (4-byte at D 64) pieces,
-// packed rows in LDS, every cache line asked for once. K product: a lane a cell; the row's dwords multiply, as they
+// A workgroup of four waves (eight at D 256) takes one KV head, a run of cells (a split) and up to eight queries that
+// share that KV head (the head's group of query heads times a few rows), so K and V are read once for all of them. A
+// wave takes tiles of 64 cells (32 at D 256 and 512): its K and V rows come by global_load_lds as 16-byte (4-byte at
+// D 64) pieces, packed rows in LDS, every cache line asked for once. K product: a lane a cell (two lanes a cell, half
+// a row each, in tiles of 32); the row's dwords multiply, as they
 // lie, with an image of the quantized query that holds its codes where the row holds codes and zeros where it holds
 // the blocks' scales (Q4_0: one image for the low nibbles, one for the high), v_dot4_i32_i8 by v_dot4_i32_i8; every
 // dword holds codes of one block only, so a block's integer sum is complete at a known dword and is scaled there. V
@@ -27,8 +28,10 @@
 namespace llmp_hip {
 namespace {
 
-constexpr int kAttnWaves = 4;
-constexpr int kAttnThreads = kAttnWaves * kWave;
+// Waves a workgroup and cells a tile by head size: 4 waves of 64 cells at D 64, 8 of 32 at D 256 (two waves a SIMD:
+// the tile's vector work of one wave runs under the other's waits), 4 of 32 at D 512.
+constexpr int AttnWavesOf(int head_dim) { return head_dim == 256 ? 8 : 4; }
+constexpr int AttnTileOf(int head_dim) { return head_dim >= 256 ? 32 : 64; }
 constexpr int kMostQueries = 8;  // queries of a workgroup: a KV head's query heads times rows
 
 template <int TYPE, int D>
@@ -41,9 +44,17 @@ struct AttnGeo {
   static constexpr bool kWide = kRow % 16 == 0;       // rows of whole 16-byte pieces (D 256, 512)
   static constexpr int kPiece = kWide ? 16 : 4;       // bytes a lane brings a load
   static constexpr int kRead = kWide ? 4 : 1;         // dwords a read of LDS
-  static constexpr int kTile = D == 512 ? 32 : 64;    // cells a tile
+  static constexpr int kWaves = AttnWavesOf(D);
+  static constexpr int kThreads = kWaves * kWave;
+  static constexpr int kTile = AttnTileOf(D);         // cells a tile
   static constexpr int kTileBytes = kTile * kRow;
-  static constexpr int kLoads = kTileBytes / (kWave * kPiece);  // loads a tile of K or of V
+  static constexpr int kLoads = (kTileBytes + kWave * kPiece - 1) / (kWave * kPiece);  // loads a tile of K or of V
+  static constexpr int kLastLanes = (kTileBytes - (kLoads - 1) * kWave * kPiece) / kPiece;  // lanes of the last one
+  // A tile of 32 cells leaves half the wave without a cell: the K product then splits a row between two lanes (whole
+  // blocks each). (The V product keeps a lane at D / 64 values of every cell: twice the values of half the cells has
+  // two rows' reads of LDS in the same banks, and took longer.)
+  static constexpr int kHalves = kWave / kTile;       // lanes a cell in the K product
+  static constexpr int kHalfRow = kRow / kHalves, kHalfDwords = kDwords / kHalves, kHalfBlocks = kBlocks / kHalves;
   static constexpr int kPer = D / kWave;              // values of a V row a lane
   static constexpr int kImage = (kQ8 ? 1 : 2) * kRow; // bytes of a query's image(s)
   static constexpr int kQuery = kImage + kBlocks * 8; // ... and its blocks' scales and code sums
@@ -51,11 +62,11 @@ struct AttnGeo {
   static constexpr int kMaskBytes = kMostQueries * kTile * 2;                   // a tile's mask values, a row a query row
   static constexpr int kWaveBytes = 2 * kTileBytes + kMostQueries * kTile * 4 + kMaskBytes;  // K, V, probabilities, mask
   static constexpr int kLoadsWithMask = kLoads + kMostQueries;  // a tile of K and its mask rows
-  static constexpr int kLds = kQueries + kAttnWaves * kWaveBytes;
-  static_assert(kTileBytes % (kWave * kPiece) == 0 && kRow % 4 == 0 && kPer >= 1 && 32 % kPer == 0, "geometry");
+  static constexpr int kLds = kQueries + kWaves * kWaveBytes;
+  static_assert(kTileBytes % kPiece == 0 && kRow % 4 == 0 && kPer >= 1 && 32 % kPer == 0 && kHalfRow % kBlock == 0 && (kHalves == 1 || kHalfRow % 8 == 0), "geometry");
   // The block whose codes dword w holds: its last byte's, unless that byte is a scale's.
   static constexpr int BlockOf(int w) { return (4 * w + 3) % kBlock >= 2 ? (4 * w + 3) / kBlock : (4 * w) / kBlock; }
-  static constexpr bool LastOf(int w) { return w + 1 == kDwords || BlockOf(w + 1) != BlockOf(w); }
+  static constexpr bool LastOf(int w) { return w + 1 == kHalfDwords || BlockOf(w + 1) != BlockOf(w); }
   // Whether dword w holds a block's scale, and in which half.
   static constexpr bool HasScale(int w) { return (4 * w) % kBlock == 0 || (4 * w + 2) % kBlock == 0; }
   static constexpr int ScaleShift(int w) { return (4 * w) % kBlock == 0 ? 0 : 16; }
@@ -130,8 +141,9 @@ __device__ __forceinline__ float WaveSum(float v) {
 // NQ: the queries the loops are unrolled for, at least the pass's; those beyond it multiply images of zeros and are
 // never written out.
 template <int TYPE, int D, int NQ>
-__global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const AttnArgs a) {
+__global__ __launch_bounds__(AttnWavesOf(D) * kWave, 1) void AttnVecQuantKernel(const AttnArgs a) {
   using G = AttnGeo<TYPE, D>;
+  constexpr int kAttnWaves = G::kWaves, kAttnThreads = G::kThreads;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const llmp_attn_vec_quant& d = a.d;
   const int tid = threadIdx.x;
@@ -167,7 +179,9 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
     const uint8_t* first = UniformPointer(static_cast<const uint8_t*>(base) + kv_head * head_stride + cell0 * cell_stride);
     AttnFor<G::kLoads>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      ToLds<G::kPiece, i * kWave * G::kPiece>(first, from[i], to);
+      // (The last load of a tile that is no whole number of loads is the lower lanes' alone: an instruction all the
+      // same, counted by the waits like the others.)
+      if (i + 1 < G::kLoads || G::kLastLanes == kWave || lane < G::kLastLanes) ToLds<G::kPiece, i * kWave * G::kPiece>(first, from[i], to);
     });
   };
 
@@ -282,33 +296,41 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
     int part[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) score[q] = 0.0f, part[q] = 0;
-    if (lane < G::kTile) {
-      const uint8_t* row = k_tile + lane * G::kRow;
+    {
+      // (A tile of 32 cells: lanes 32 to 63 take the rows' upper halves, whole blocks like the lower ones.)
+      const int k_half = lane / G::kTile;
+      const uint8_t* row = k_tile + (lane & (G::kTile - 1)) * G::kRow + k_half * G::kHalfRow;
       // One or two queries' images stay in registers from tile to tile (the compiler finds their reads the same in
       // every iteration); more do not fit, so their place is hidden from it here and they are read again a tile.
       uint32_t images_at = 0;
       if constexpr (NQ > 2) asm volatile("" : "+v"(images_at));
-      const uint8_t* images = lds + images_at;
+      const uint8_t* images = lds + images_at + k_half * G::kHalfRow;
+      const int scales_from = k_half * G::kHalfBlocks;
       uint32_t kd[G::kRead];
       uint32_t low[NQ][G::kRead], high[G::kQ8 ? 1 : NQ][G::kRead];  // the images' dwords beside the row's
       float dk = 0.0f;
-      AttnFor<G::kDwords>([&](auto wc) {
+      AttnFor<G::kHalfDwords>([&](auto wc) {
         constexpr int w = decltype(wc)::value;
         // (The reads of LDS stay with their group of dwords: hoisted to the front of the unrolled row they take
         // more registers than there are.)
         if constexpr (w % (2 * G::kRead) == 0 && w > 0) __builtin_amdgcn_sched_barrier(0);
         if constexpr (w % G::kRead == 0) {
           if constexpr (G::kWide) {
-            const uint4 x = *reinterpret_cast<const uint4*>(row + 4 * w);
-            kd[0] = x.x, kd[1] = x.y, kd[2] = x.z, kd[3] = x.w;
+            // (Half rows begin at 8-byte boundaries: two 8-byte reads each. A row's last read may run past its half.)
+            auto four = [](const uint8_t* at, uint32_t (&into)[G::kRead]) {
+              if constexpr (G::kHalfRow % 16 == 0) {
+                const uint4 x = *reinterpret_cast<const uint4*>(at);
+                into[0] = x.x, into[1] = x.y, into[2] = x.z, into[3] = x.w;
+              } else {
+                const uint2 x = *reinterpret_cast<const uint2*>(at), y = *reinterpret_cast<const uint2*>(at + 8);
+                into[0] = x.x, into[1] = x.y, into[2] = y.x, into[3] = y.y;
+              }
+            };
+            four(row + 4 * w, kd);
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
-              const uint4 y = *reinterpret_cast<const uint4*>(images + q * G::kQuery + 4 * w);
-              low[q][0] = y.x, low[q][1] = y.y, low[q][2] = y.z, low[q][3] = y.w;
-              if constexpr (!G::kQ8) {
-                const uint4 z = *reinterpret_cast<const uint4*>(images + q * G::kQuery + G::kRow + 4 * w);
-                high[q][0] = z.x, high[q][1] = z.y, high[q][2] = z.z, high[q][3] = z.w;
-              }
+              four(images + q * G::kQuery + 4 * w, low[q]);
+              if constexpr (!G::kQ8) four(images + q * G::kQuery + G::kRow + 4 * w, high[q]);
             }
           } else {
             kd[0] = *reinterpret_cast<const uint32_t*>(row + 4 * w);
@@ -332,7 +354,7 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
             part[q] = Dot4(static_cast<int>((x >> 4) & 0x0F0F0F0Fu), static_cast<int>(high[q][w % G::kRead]), part[q]);
           }
           if constexpr (G::LastOf(w)) {
-            const float* scales = reinterpret_cast<const float*>(images + q * G::kQuery + G::kImage);
+            const float* scales = reinterpret_cast<const float*>(lds + images_at + q * G::kQuery + G::kImage) + scales_from;
             // Q4_0: values are codes minus 8, so eight times the query's code sum comes off.
             const float whole = G::kQ8 ? static_cast<float>(part[q]) : static_cast<float>(part[q]) - 8.0f * scales[G::kBlocks + blk];
             score[q] += (dk * scales[blk]) * whole;
@@ -342,11 +364,15 @@ __global__ __launch_bounds__(kAttnThreads, 1) void AttnVecQuantKernel(const Attn
         if constexpr (G::HasScale(w) && G::ScaleBlock(w) != blk) dk = HalfBitsToFloat((x >> G::ScaleShift(w)) & 0xFFFFu);
         // The sums are taken where they are computed: pure as they are, the compiler otherwise moves every product
         // to the row's end and keeps all the row's and images' dwords until then.
-        if constexpr ((w + 1) % G::kRead == 0 || w + 1 == G::kDwords) {
+        if constexpr ((w + 1) % G::kRead == 0 || w + 1 == G::kHalfDwords) {
 #pragma unroll
           for (int q = 0; q < NQ; ++q) asm volatile("" : "+v"(part[q]), "+v"(score[q]));
         }
       });
+    }
+    if constexpr (G::kHalves == 2) {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) score[q] += __shfl_xor(score[q], 32);  // a cell's two half rows
     }
     // K's buffer is free: the wave's next tile of K on its way.
     const int next = tile + kAttnWaves;
@@ -487,7 +513,7 @@ void LaunchAttnFor(const AttnArgs& args, const AttnPlan& plan, hipStream_t strea
   static bool sized = false;
   if (!AllowLds(reinterpret_cast<const void*>(&AttnVecQuantKernel<TYPE, D, NQ>), G::kLds, &sized)) return;
   const dim3 grid(static_cast<unsigned>(plan.splits), static_cast<unsigned>(args.d.kv_heads), static_cast<unsigned>(plan.passes));
-  hipLaunchKernelGGL((AttnVecQuantKernel<TYPE, D, NQ>), grid, dim3(kAttnThreads), G::kLds, stream, args);
+  hipLaunchKernelGGL((AttnVecQuantKernel<TYPE, D, NQ>), grid, dim3(G::kThreads), G::kLds, stream, args);
 }
 
 template <int TYPE, int D>
@@ -505,8 +531,6 @@ void LaunchAttn(const AttnArgs& args, const AttnPlan& plan, hipStream_t stream) 
   hipLaunchKernelGGL((AttnCombineKernel<D>), dim3(static_cast<unsigned>(args.d.heads), static_cast<unsigned>(args.d.rows)), dim3(D), 0,
                      stream, args);
 }
-
-int TileOf(int head_dim) { return head_dim == 512 ? 32 : 64; }
 
 // 0 and the plan, or a refusal: every check of the reference's CheckFlashAttnVecQuant (src/kernels/ggml/kv_quant.cc:81-170)
 // that applies to these operands, and this kernel's own.
@@ -548,11 +572,11 @@ int PlanAttn(const llmp_attn_vec_quant* op, int cus, AttnPlan* plan) {
   plan->rows_a_pass = op->rows < kMostQueries / group ? op->rows : (kMostQueries / group < 1 ? 1 : kMostQueries / group);
   plan->passes = (op->rows + plan->rows_a_pass - 1) / plan->rows_a_pass;
   // Splits: about two workgroups a compute unit over the launch, each at least a tile a wave where the cells allow.
-  const int tile = TileOf(op->head_dim);
+  const int tile = AttnTileOf(op->head_dim), waves = AttnWavesOf(op->head_dim);
   const int tiles = op->cells / tile;
   const int others = op->kv_heads * plan->passes;
   int splits = (2 * (cus > 0 ? cus : 256) + others - 1) / others;
-  const int most = (tiles + kAttnWaves - 1) / kAttnWaves;
+  const int most = (tiles + waves - 1) / waves;
   if (splits > most) splits = most;
   if (splits > kMostSplits) splits = kMostSplits;
   if (splits < 1) splits = 1;
