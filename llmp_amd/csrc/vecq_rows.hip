@@ -72,9 +72,6 @@ __device__ __forceinline__ U32v4 LdsRead16(uint32_t at) {
 __device__ __forceinline__ void LdsWaited() { asm volatile("s_waitcnt lgkmcnt(0)"); }
 __device__ __forceinline__ void LdsWrite16(uint32_t at, U32v4 value) { asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(value)); }
 __device__ __forceinline__ void LdsWrite4(uint32_t at, float value) { asm volatile("ds_write_b32 %0, %1" : : "v"(at), "v"(value)); }
-__device__ __forceinline__ void LdsWrite8(uint32_t at, unsigned long long value) {
-  asm volatile("ds_write_b64 %0, %1" : : "v"(at), "v"(value));
-}
 __device__ __forceinline__ U32v4 GlobalLoad16(const void* from) {
   U32v4 v;
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(from));
@@ -703,16 +700,23 @@ int SpanFor(int units, int unit_blocks, int parts = 1) {
 }
 
 // Tiles of 64 rows, or of 32 or 16 (the file's layouts) where that many more workgroups still find a compute
-// unit each and the rows are long enough for a piece of two or four super-blocks a wave and span.
+// unit each and the rows are long enough for a piece of two or four units a wave and span. Measured at 4 tokens of
+// Q4_K rows of 4096 values, tiles of 64 / 32 / 16 rows: 80 tiles 10.6 / 7.9 / 10.1 us, 128 tiles 10.9 / 8.6 / 10.9,
+// 160 tiles 11.2 / 12.8 / 14.1, 256 tiles 13.3 / 13.9 / 18.3.
 int RowsParts(const VecQArgs& a, int cus) {
   const llmp_vecq_desc& d = a.d;
   if (a.tiled != 0 && a.tiled != 3) return 1;
   const int64_t tiles = static_cast<int64_t>((d.nrows + kTileRows - 1) / kTileRows) * d.used;
   const int unit_blocks = a.tiled == 3 ? 4 : 8, units = d.ncols_x / 32 / unit_blocks;
+  auto takes = [&](int parts) { return (d.tokens <= 4 ? SpanFor<4>(units, unit_blocks, parts) : SpanFor<8>(units, unit_blocks, parts)) >= 0; };
   for (int parts = 4; parts > 1; parts /= 2) {
-    if (tiles * parts > cus) continue;
-    if ((d.tokens <= 4 ? SpanFor<4>(units, unit_blocks, parts) : SpanFor<8>(units, unit_blocks, parts)) >= 0) return parts;
+    if (tiles * parts <= cus && takes(parts)) return parts;
   }
+  // More tiles than compute units: the workgroups go through them in rounds, and half tiles end the last round
+  // sooner where that saves a fifth of the rounds (320 tiles on 256 units: three rounds of half tiles for two of
+  // whole ones, 18.6 us against 20.4 at 4096 x 20480).
+  const int64_t rounds = (tiles + cus - 1) / cus, half_rounds = (2 * tiles + cus - 1) / cus;
+  if (5 * half_rounds <= 8 * rounds && takes(2)) return 2;
   return 1;
 }
 
