@@ -630,6 +630,15 @@ def block_formats(device):
         bytes_ = bytes_w + k * 4 + n * 4
         out[f"decode_vector_{ops.DECODERS[decoder].replace('.', '_')}_4096x14336_rows1"] = {
             "us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1), "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        # The same at 4 and 16 input rows (a launch for every four rows).
+        for rows in (4, 16):
+            xr = dev(synth.activations(rows, k, 306))
+            yr = torch.empty((rows, n), dtype=torch.float32, device=device)
+            us = graph_us(lambda i: ops.decode_vector(decoder, ws[i % count], xr, out=yr), 2 * count)
+            bytes_ = bytes_w + rows * (k * 4 + n * 4)
+            out[f"decode_vector_{ops.DECODERS[decoder].replace('.', '_')}_4096x14336_rows{rows}"] = {
+                "us": round(us, 2), "GB/s": round(bytes_ / us / 1e3, 1), "frac_hbm_peak": round(bytes_ / us / 1e3 / HBM_PEAK_GBPS, 4),
+                "TFLOP/s": round(2.0 * rows * n * k / us / 1e6, 1)}
         del ws, base
         torch.cuda.empty_cache()
     # llmp.decode.matrix: 512 and 2048 F32 input rows times the same NVFP4 and BF16 weights on the matrix cores.
