@@ -22,7 +22,8 @@ namespace {
 typedef float Float2 __attribute__((ext_vector_type(2)));
 typedef uint32_t U32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kDecodeWaves = 8;  // a workgroup's waves with several input rows staged; four with one
+constexpr int kDecodeWaves = 16;  // a workgroup's waves with several input rows staged; four with one
+constexpr int kGroupedWaves = 8;  // of the expert worklist's kernel
 constexpr int kRowsAWave = 2;
 constexpr int kSegmentStride = 80;           // bytes from a staged segment to the next
 constexpr size_t kDecodeLdsLimit = 80 * 1024;  // two workgroups a CU
@@ -255,7 +256,7 @@ __device__ __forceinline__ void LoadSegment(const llmp_decode_operand& w, uint32
   DecodeSegment<D>(w, seg, FetchSegment<D>(w, row, seg), v, s);
 }
 
-// grid: workgroups of eight waves, persistent over pairs of output rows; LDS: T input rows.
+// grid: workgroups of four waves (one input row) or sixteen, persistent over pairs of output rows; LDS: T input rows.
 // kGlu: a wave's two rows are gate row first + j and up row up_first + j of output j; the up weight's decoder DU may
 // differ from the gate's D (the pairs src/kernels/decode/implementations.cc:73-81 of the reference lists).
 template <int D, int T, bool kGlu, int DU = D>
@@ -275,29 +276,134 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
   }
   __syncthreads();  // the only one: from here the waves run alone
 
+  if constexpr (T <= 3) {
+    // One to three input rows: four or eight waves a workgroup and two or more workgroups a CU; their number hides the
+    // loads (at three rows 22 us for MXFP8 4096 x 14336 against 24 with the loads ahead).
+    const uint32_t pairs = kGlu ? a.outputs : (a.outputs + kRowsAWave - 1) / kRowsAWave;
+    for (uint32_t pair = blockIdx.x * waves + wave; pair < pairs; pair += gridDim.x * waves) {
+      const uint32_t out0 = kGlu ? pair : pair * kRowsAWave;
+      float acc[kRowsAWave][T];
+  #pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+  #pragma unroll
+        for (int t = 0; t < T; ++t) acc[r][t] = 0.0f;
+      }
+      for (uint32_t seg = lane; seg < segs; seg += 64) {
+        float v[kRowsAWave][16], s[kRowsAWave];
+  #pragma unroll
+        for (int r = 0; r < kRowsAWave; ++r) {
+          if constexpr (kGlu) {
+            if (r == 0) {
+              LoadSegment<D>(a.w, a.first + out0, seg, v[r], s[r]);
+            } else {
+              LoadSegment<DU>(a.up, a.up_first + out0, seg, v[r], s[r]);
+            }
+          } else {
+            // A lone last row is decoded twice: its second copy's sums are not stored.
+            const uint32_t out = min(out0 + r, a.outputs - 1);
+            LoadSegment<D>(a.w, a.first + out, seg, v[r], s[r]);
+          }
+        }
+  #pragma unroll
+        for (int t = 0; t < T; ++t) {
+          const float4* xs = reinterpret_cast<const float4*>(lds + static_cast<size_t>(t * segs + seg) * kSegmentStride);
+          const float4 x0 = xs[0], x1 = xs[1], x2 = xs[2], x3 = xs[3];
+          const float x[16] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+  #pragma unroll
+          for (int r = 0; r < kRowsAWave; ++r) {
+            float dot = 0.0f;
+  #pragma unroll
+            for (int i = 0; i < 16; ++i) dot = fmaf(v[r][i], x[i], dot);
+            acc[r][t] = fmaf(dot, s[r], acc[r][t]);
+          }
+        }
+      }
+      if constexpr (kGlu) {
+        const float gate_scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out0) / a.w.rows_per_scale] : 1.0f;
+        const float up_scale = a.up.tensor_scale != nullptr ? a.up.tensor_scale[(a.up_first + out0) / a.up.rows_per_scale] : 1.0f;
+  #pragma unroll
+        for (int t = 0; t < T; ++t) {
+          float gate = acc[0][t], up = acc[1][t];
+  #pragma unroll
+          for (int mask = 32; mask >= 1; mask >>= 1) {
+            gate += ShflXor(gate, mask);
+            up += ShflXor(up, mask);
+          }
+          if (lane == 0) a.y[(a.token0 + t) * a.y_stride + out0] = DecodeGlu(a.glu, gate * gate_scale, up * up_scale, a.limit);
+        }
+        continue;
+      }
+  #pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+        const uint32_t out = out0 + r;
+        float scale = 1.0f;
+        if (a.w.tensor_scale != nullptr && out < a.outputs) scale = a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale];
+  #pragma unroll
+        for (int t = 0; t < T; ++t) {
+          float total = acc[r][t];
+  #pragma unroll
+          for (int mask = 32; mask >= 1; mask >>= 1) total += ShflXor(total, mask);
+          if (lane == 0 && out < a.outputs) a.y[(a.token0 + t) * a.y_stride + out] = total * scale;
+        }
+      }
+    }
+    return;
+  }
+  // The wave's work as one run of steps, (pair of rows, 64 segments) each: a step's two segments are asked for two
+  // steps before they are multiplied (several input rows: the staged rows fill LDS and a CU holds one workgroup),
+  // past the last step the last again, so that no load sits under a branch (three steps ahead measured the same).
+  // What a lane adds, and in which order, is what the plain loop over its pairs and segments adds.
   const uint32_t pairs = kGlu ? a.outputs : (a.outputs + kRowsAWave - 1) / kRowsAWave;
-  for (uint32_t pair = blockIdx.x * waves + wave; pair < pairs; pair += gridDim.x * waves) {
-    const uint32_t out0 = kGlu ? pair : pair * kRowsAWave;
-    float acc[kRowsAWave][T];
+  const uint32_t first_pair = blockIdx.x * waves + wave, pair_step = gridDim.x * waves;
+  if (first_pair >= pairs) return;
+  const uint32_t seg_steps = (segs + 63u) / 64u;
+  const uint32_t total = ((pairs - first_pair + pair_step - 1) / pair_step) * seg_steps;
+  struct Step {
+    RawSegment raw[kRowsAWave];
+  };
+  auto fetch = [&](uint32_t it) {
+    it = min(it, total - 1);
+    const uint32_t p = it / seg_steps;
+    const uint32_t out0 = kGlu ? first_pair + p * pair_step : (first_pair + p * pair_step) * kRowsAWave;
+    const uint32_t seg = min((it - p * seg_steps) * 64u + lane, segs - 1);
+    Step step;
 #pragma unroll
     for (int r = 0; r < kRowsAWave; ++r) {
-#pragma unroll
-      for (int t = 0; t < T; ++t) acc[r][t] = 0.0f;
+      if constexpr (kGlu) {
+        if (r == 0) {
+          step.raw[r] = FetchSegment<D>(a.w, a.first + out0, seg);
+        } else {
+          step.raw[r] = FetchSegment<DU>(a.up, a.up_first + out0, seg);
+        }
+      } else {
+        // A lone last row is decoded twice: its second copy's sums are not stored.
+        step.raw[r] = FetchSegment<D>(a.w, a.first + min(out0 + r, a.outputs - 1), seg);
+      }
     }
-    for (uint32_t seg = lane; seg < segs; seg += 64) {
+    return step;
+  };
+  float acc[kRowsAWave][T];
+#pragma unroll
+  for (int r = 0; r < kRowsAWave; ++r) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[r][t] = 0.0f;
+  }
+  auto multiply = [&](uint32_t it, const Step& step) {
+    const uint32_t p = it / seg_steps, part = it - p * seg_steps;
+    const uint32_t out0 = kGlu ? first_pair + p * pair_step : (first_pair + p * pair_step) * kRowsAWave;
+    const uint32_t seg = part * 64u + lane;
+    if (seg < segs) {
       float v[kRowsAWave][16], s[kRowsAWave];
 #pragma unroll
       for (int r = 0; r < kRowsAWave; ++r) {
         if constexpr (kGlu) {
           if (r == 0) {
-            LoadSegment<D>(a.w, a.first + out0, seg, v[r], s[r]);
+            DecodeSegment<D>(a.w, seg, step.raw[r], v[r], s[r]);
           } else {
-            LoadSegment<DU>(a.up, a.up_first + out0, seg, v[r], s[r]);
+            DecodeSegment<DU>(a.up, seg, step.raw[r], v[r], s[r]);
           }
         } else {
-          // A lone last row is decoded twice: its second copy's sums are not stored.
-          const uint32_t out = min(out0 + r, a.outputs - 1);
-          LoadSegment<D>(a.w, a.first + out, seg, v[r], s[r]);
+          DecodeSegment<D>(a.w, seg, step.raw[r], v[r], s[r]);
         }
       }
 #pragma unroll
@@ -314,6 +420,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
         }
       }
     }
+    if (part + 1 < seg_steps) return;
+    // The pair's last step: the lanes' sums meet and the outputs are stored.
     if constexpr (kGlu) {
       const float gate_scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out0) / a.w.rows_per_scale] : 1.0f;
       const float up_scale = a.up.tensor_scale != nullptr ? a.up.tensor_scale[(a.up_first + out0) / a.up.rows_per_scale] : 1.0f;
@@ -326,21 +434,34 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void DecodeVectorKernel(const De
           up += ShflXor(up, mask);
         }
         if (lane == 0) a.y[(a.token0 + t) * a.y_stride + out0] = DecodeGlu(a.glu, gate * gate_scale, up * up_scale, a.limit);
+        acc[0][t] = 0.0f, acc[1][t] = 0.0f;
       }
-      continue;
+    } else {
+#pragma unroll
+      for (int r = 0; r < kRowsAWave; ++r) {
+        const uint32_t out = out0 + r;
+        float scale = 1.0f;
+        if (a.w.tensor_scale != nullptr && out < a.outputs) scale = a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          float total_sum = acc[r][t];
+#pragma unroll
+          for (int mask = 32; mask >= 1; mask >>= 1) total_sum += ShflXor(total_sum, mask);
+          if (lane == 0 && out < a.outputs) a.y[(a.token0 + t) * a.y_stride + out] = total_sum * scale;
+          acc[r][t] = 0.0f;
+        }
+      }
     }
-#pragma unroll
-    for (int r = 0; r < kRowsAWave; ++r) {
-      const uint32_t out = out0 + r;
-      float scale = 1.0f;
-      if (a.w.tensor_scale != nullptr && out < a.outputs) scale = a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale];
-#pragma unroll
-      for (int t = 0; t < T; ++t) {
-        float total = acc[r][t];
-#pragma unroll
-        for (int mask = 32; mask >= 1; mask >>= 1) total += ShflXor(total, mask);
-        if (lane == 0 && out < a.outputs) a.y[(a.token0 + t) * a.y_stride + out] = total * scale;
-      }
+  };
+  Step even = fetch(0), odd = fetch(1);
+  for (uint32_t it = 0; it < total; it += 2) {
+    const Step now = even;
+    even = fetch(it + 2);
+    multiply(it, now);
+    if (it + 1 < total) {
+      const Step then = odd;
+      odd = fetch(it + 3);
+      multiply(it + 1, then);
     }
   }
 }
@@ -391,7 +512,7 @@ struct GroupedArgs {
 };
 
 template <int D, int T>
-__global__ __launch_bounds__(kDecodeWaves * 64) void DecodeGroupedKernel(const GroupedArgs a) {
+__global__ __launch_bounds__(kGroupedWaves * 64) void DecodeGroupedKernel(const GroupedArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int32_t out_row[T];
   const int tid = threadIdx.x;
@@ -898,8 +1019,10 @@ int LaunchProduct(const char* what, int decoder, bool glu, DecodeArgs& a, uint64
     return Refuse(1, "%s: a row of %u values does not fit the staging area (16384 at most)", what, k);
   const int cus = llmp_hip_compute_units();
   const size_t lds = DecodeLds(pass, k);
-  // One input row: four waves a workgroup and more workgroups; several: eight waves share the staged rows.
-  const int waves = pass == 1 ? 4 : kDecodeWaves;
+  // One input row: four waves a workgroup and more workgroups; two or three: eight; four: sixteen waves share the
+  // staged rows (which then fill LDS: one workgroup a CU, its loads two steps ahead: MXFP8 4096 x 14336 at four rows
+  // 34.5 -> 22.8 us, at sixteen 135 -> 88; NVFP4 30 -> 19.6 and 117 -> 74).
+  const int waves = pass == 1 ? 4 : pass < 4 ? 8 : kDecodeWaves;
   int resident = static_cast<int>(160 * 1024 / (lds + 1024));
   if (resident > 32 / waves) resident = 32 / waves;  // a CU holds 32 waves
   if (resident < 1) resident = 1;
@@ -1030,7 +1153,7 @@ template <int D, int T>
 void LaunchGrouped(const GroupedArgs& a, dim3 grid, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!AllowLds(reinterpret_cast<const void*>(&DecodeGroupedKernel<D, T>), static_cast<int>(kDecodeLdsLimit), &sized)) return;
-  hipLaunchKernelGGL((DecodeGroupedKernel<D, T>), grid, dim3(kDecodeWaves * 64), DecodeLds(T, a.k), stream, a);
+  hipLaunchKernelGGL((DecodeGroupedKernel<D, T>), grid, dim3(kGroupedWaves * 64), DecodeLds(T, a.k), stream, a);
 }
 
 template <int D>
@@ -1078,7 +1201,7 @@ extern "C" int llmp_hip_decode_grouped(int decoder, const llmp_decode_operand* e
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
   const int cus = llmp_hip_compute_units();
   uint64_t groups = 2 * static_cast<uint64_t>(cus > 0 ? cus : 256) / experts_count;
-  const uint64_t most = ((outputs + kRowsAWave - 1) / kRowsAWave + kDecodeWaves - 1) / kDecodeWaves;
+  const uint64_t most = ((outputs + kRowsAWave - 1) / kRowsAWave + kGroupedWaves - 1) / kGroupedWaves;
   if (groups > most) groups = most;
   if (groups < 1) groups = 1;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(experts_count));
