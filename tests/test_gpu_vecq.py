@@ -339,6 +339,22 @@ def test_row_a_lane_form_matches_oracle(device, k, n, tokens):
     ok, worst = rel_close(got, want, TOL)
     assert ok, worst
     ids = dev(np.zeros((tokens, 1), dtype=np.int32), device)
+    # Rows apart (a pitch of two super-blocks more) and fewer rows than the matrix holds, through every tile that takes
+    # the shape: the values of the packed matrix's rows.
+    nsb = k // 256
+    pitched = torch.zeros((n, nsb + 2, 144), dtype=torch.uint8, device=device)
+    pitched[:, :nsb] = dev(up, device).view(n, nsb, 144)
+    packed = ops.vecq(t, dev(up, device), dev(q8, device), k, n, tokens=tokens, variant=names.index("rows pass8 rows64"))
+    for name in ("rows pass8", "rows pass8 rows64", "rows pass8 rows32", "rows pass8 rows16"):
+        try:
+            apart = ops.vecq(t, pitched.view(-1), dev(q8, device), k, n - 5, tokens=tokens, stride_row=nsb + 2, variant=names.index(name))
+        except ops.KernelFailure as refused:  # a tile the rows are too short for (checked above)
+            assert refused.rejected and name.endswith(("rows32", "rows16")), name
+            continue
+        ok, worst = rel_close(apart.cpu().numpy().reshape(tokens, n - 5), packed.cpu().numpy().reshape(tokens, n)[:, :n - 5], TOL)
+        assert ok, (name, worst)
+        if name.endswith("rows64"):
+            assert torch.equal(apart.view(torch.int32), packed[:, :, :n - 5].contiguous().view(torch.int32))
     # Nine tokens and more (to the operation's 16) are launches of eight or fewer each: every token the bits it has among eight.
     many = min(tokens + 9, 16)
     x_many = synth.activations(many, k, 339)
@@ -860,6 +876,11 @@ def test_q8_0_rows_form_over_relaid_out_weights(device, tokens, glu, k):
         short = ops.vecq(Q8_0, pitched.view(-1), qd, k, n - 24, variant=rows_variant, tokens=tokens, stride_row=k // 32 + 8, **dict(wide, glu=ops.GLU_NONE))
         plain = got if glu == ops.GLU_NONE else ops.vecq(Q8_0, ut, qd, k, n, variant=tiled_variant, tokens=tokens, **dict(common, glu=ops.GLU_NONE))
         assert torch.equal(short.view(torch.int32), plain[:, :, :n - 24].contiguous().view(torch.int32))
+        # The same edges in the narrower tiles (the launcher's choice here): the oracle's values.
+        narrow_short = ops.vecq(Q8_0, pitched.view(-1), qd, k, n - 24, tokens=tokens, stride_row=k // 32 + 8,
+                                variant=ops.vecq_variants().index("rows pass8"), **dict(wide, glu=ops.GLU_NONE))
+        ok, worst = rel_close(narrow_short.cpu().numpy(), plain[:, :, :n - 24].cpu().numpy(), TOL)
+        assert ok, worst
     else:
         with pytest.raises(ops.KernelFailure):
             ops.vecq(Q8_0, ud, qd, k, n, gate=gd, variant=rows_variant, tokens=tokens, **common)
