@@ -37,6 +37,34 @@ def test_q8_1_quantize_is_bit_exact(device, k, rows):
     assert np.array_equal(got, want)
 
 
+def test_q8_1_quantize_ties_and_near_ties_are_bit_exact(device):
+    """Quotients x / d on and beside k + 1/2 (the device multiplies by a reciprocal where that cannot change the rounded
+    integer and divides otherwise), scales that are powers of two and not, blocks of tiny and huge values, a block whose
+    largest magnitude is subnormal: the oracle's codes, scales and sums, bit for bit."""
+    g = synth.rng(77)
+    rows, k = 24, 1024
+    x = np.zeros((rows, k), dtype=np.float32)
+    for r in range(rows):
+        for b in range(k // 32):
+            amax = np.float32([127.0, 63.5, 254.0, 1.0, 3.0, 100.0, 0.37, 12.7][(r + b) % 8])
+            d = np.float32(amax / np.float32(127.0))
+            halves = (g.integers(-126, 126, size=32).astype(np.float32) + np.float32(0.5)) * d
+            nudge = g.integers(-2, 3, size=32)
+            block = halves.copy()
+            for _ in range(2):  # up to two units in the last place either way
+                block = np.where(nudge > 0, np.nextafter(block, np.float32(np.inf)), np.where(nudge < 0, np.nextafter(block, np.float32(-np.inf)), block))
+                nudge = nudge - np.sign(nudge)
+            block[g.integers(0, 32)] = amax * (1 if b % 2 else -1)
+            x[r, b * 32:(b + 1) * 32] = block
+    x[20] *= np.float32(1e-30)
+    x[21] *= np.float32(1e30)
+    x[22] *= np.float32(1e-38)
+    x[23, :32] = np.float32(1e-41)  # subnormal: its scale's reciprocal is not finite
+    want = oracle.q8_1_quantize(x)
+    got = ops.quantize_q8_1(dev(x, device)).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 def test_q8_1_planes_and_strides(device):
     x = synth.activations(2 * 3, 256, 5).reshape(2, 3, 256)
     wide = np.zeros((2, 3, 300), dtype=np.float32)
