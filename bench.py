@@ -128,8 +128,10 @@ PROFILED_TRAFFIC = {
     "moe_q4_k_ffn_t1": _traffic(7028.8, 24.0),        # the gate/up launch
     "moe_q4_k_ffn_t16": _traffic(76343.9, 457.9),     # the gate/up launch
     "moe_q4_k_ffn_t512": _traffic(182457.3, 12338.4),  # the gate/up launch: the experts' tokens once a segment of rows
-    "attn_vec_q8_0_d256_h16_kv8_cells8192_rows1": _traffic(17578.0 + 273.5, 528.0 + 16.0),  # the splits + their combination
-    "attn_vec_q4_0_d256_h16_kv8_cells8192_rows1": _traffic(9387.0 + 273.5, 528.0 + 16.0),
+    "attn_vec_q8_0_d256_h16_kv8_cells8192_rows1": _traffic(17562.0 + 279.5, 528.0 + 16.0),  # the splits + their combination
+    "attn_vec_q4_0_d256_h16_kv8_cells8192_rows1": _traffic(9369.5 + 279.5, 528.0 + 16.0),
+    "attn_vec_q8_0_d256_h16_kv8_cells32768_rows1": _traffic(73938.5 + 537.5, 1056.0 + 16.0),
+    "attn_vec_q4_0_d256_h16_kv8_cells32768_rows1": _traffic(40693.4 + 537.5, 1056.0 + 16.0),
     "exl3_linear_4096x14336_4bpw_m1": _traffic(14475.9 + 143.5, 232.0 + 56.0),  # product + output transform
     "exl3_linear_4096x14336_4bpw_m16": _traffic(14906.0 + 114.5 + 1921.5, 3584.0 + 128.0 + 896.0),
     "exl3_multi_linear_4096x2x14336_4bpw_m1": _traffic(28815.7 + 255.5, 464.0 + 112.0),
