@@ -478,7 +478,7 @@ __global__ __launch_bounds__(AttnWavesOf(D) * kWave, 1) void AttnVecQuantKernel(
 }
 
 // grid (heads, rows); D threads: the splits' partial results into one row of the output. The splits' maxima and sums
-// through LDS (a thread a split), then every thread its value over the splits, eight loads at a time.
+// through LDS (a thread a split), then every thread its value over the splits, in split order.
 constexpr int kMostSplits = 512;
 template <int D>
 __global__ __launch_bounds__(D) void AttnCombineKernel(const AttnArgs a) {
@@ -492,7 +492,9 @@ __global__ __launch_bounds__(D) void AttnCombineKernel(const AttnArgs a) {
   float peak = sunk ? static_cast<const float*>(d.sinks)[head] : -INFINITY;
   for (int s = 0; s < a.splits; ++s) peak = fmaxf(peak, peaks[s]);
   float total = sunk ? __expf(static_cast<const float*>(d.sinks)[head] - peak) : 0.0f, value = 0.0f;
-#pragma unroll 8
+  // (Thirty-two loads in flight: a launch of sixteen workgroups is a chain of round trips, and eight at a time made
+  // four of them at 32 splits. Asking for them ahead of the maxima's trip through LDS measured slower.)
+#pragma unroll 32
   for (int s = 0; s < a.splits; ++s) {
     const float keep = peaks[s] == -INFINITY ? 0.0f : __expf(peaks[s] - peak);
     total += totals[s] * keep;
