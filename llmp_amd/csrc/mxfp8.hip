@@ -745,8 +745,17 @@ __device__ __forceinline__ void GemmTiles(const GemmArgs& a) {
   for (; ord < mine; ++ord) {
     if constexpr (!kHalf) aim_weight_scales(ord);
     // The tile's first stages have landed (they were asked for ahead of the tile before's stores, which this wait
-    // counts as well), for every wave.
-    AwaitLoads<0>();
+    // counts as well), for every wave. The launch's first tile has no stores behind it and starts like a step: its
+    // third stage of weights, asked for last, may still be on its way (the first step's own wait takes it in).
+    if (ord == 0 && RA == 2) {
+      if (!kHalf && wave == 1) {
+        AwaitLoads<kLoadsB + 1>();
+      } else {
+        AwaitLoads<kLoadsB>();
+      }
+    } else {
+      AwaitLoads<0>();
+    }
     barrier();
     aim_reads(0, 0);
     StaticFor<kXFrags>([&](auto j) { read_a(j, Even{}); });
