@@ -177,6 +177,36 @@ __device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_in
   return expert;
 }
 
+// The same list for a routed product whose workgroups share an expert's work instead: every pair's workgroups
+// get the pairs that name their pair's expert, in pair order, and `rank`, their own pair's place among them. An
+// expert that n pairs name then has n pairs' workgroups, each taking a share of its rows against all n tokens: the
+// weights are still read once, and the workgroups an expert gets grow with the tokens it serves. Ends with a
+// workgroup barrier.
+__device__ __forceinline__ int SharePairs(const llmp_vecq_desc& d, int slot_index, int* pairs, int* count, int* rank) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int s = slot_index;
+  const int expert = d.ids[(s / d.used) * d.ids_stride + (s % d.used)];
+  if (tid < kWave) {
+    const int total = d.tokens * d.used;
+    int n = 0;
+    for (int base = 0; base < total; base += kWave) {
+      const int s2 = base + lane;
+      const int t = s2 / d.used;
+      const int u = s2 % d.used;
+      const bool match = s2 < total && d.ids[t * d.ids_stride + u] == expert;
+      const unsigned long long ballot = __ballot(match);
+      const int at = n + __popcll(ballot & ((1ull << lane) - 1ull));
+      if (match) pairs[at] = (t << 8) | u;
+      if (s2 == s) *rank = at;
+      n += __popcll(ballot);
+    }
+    if (lane == 0) *count = n;
+  }
+  __syncthreads();
+  return expert;
+}
+
 // The decoded header of a super-block: 6-bit scales and minimums as bytes g of sc[g / 4],
 // mn[g / 4] (the packing of tests/unit/dsv4_fast_test.cc:180-183 of the reference).
 struct Q4KHeader {

@@ -1384,6 +1384,7 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
+  __shared__ int rank_among;
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
@@ -1418,19 +1419,22 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   // rows takes its expert's row range.
   int expert = blockIdx.y;
   int sorted_first = 0;
+  int rank = 0, sharers = 1;
   if (a.offsets != nullptr) {
     sorted_first = a.offsets[expert];
     if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
     __syncthreads();
     if (count == 0) return;  // uniform over the workgroup
   } else if (d.ids != nullptr) {
-    expert = ResolvePairs(d, blockIdx.y, pairs, &count);
-    if (count == 0) return;  // uniform over the workgroup
+    // The pairs that name this pair's expert share its tiles: `count` pairs' workgroups, this pair's at `rank`.
+    expert = SharePairs(d, blockIdx.y, pairs, &count, &rank_among);
+    sharers = count;
+    rank = rank_among;
   }
   const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
   const int waves = blockDim.x / kWave;  // eight, fewer where a long row's records leave less room
-  const int first_tile = blockIdx.x * waves + wave;
-  const int tile_step = gridDim.x * waves;
+  const int first_tile = (rank * gridDim.x + blockIdx.x) * waves + wave;
+  const int tile_step = sharers * gridDim.x * waves;
   // A dense or grouped product's pairs are its tokens on the workgroup's matrix: no list.
   const bool listed = d.ids != nullptr && a.offsets == nullptr;
   const int n = a.offsets == nullptr && d.ids == nullptr ? d.tokens : count;
@@ -1790,9 +1794,9 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   }
   const int slots = a.offsets != nullptr ? d.used : d.ids != nullptr ? d.used * d.tokens : d.used;
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
-  // What is resident at once: two workgroups a CU, shared by the slots that have work.
-  const int live_slots = a.offsets == nullptr && d.ids != nullptr ? LiveSlots(d, slots) : slots;
-  int groups = (deep ? 1 : 2) * g_compute_units / (live_slots > 0 ? live_slots : 1);
+  // What is resident at once: two workgroups a CU, shared by the slots (every pair of a routed product has work:
+  // the pairs that name an expert share it).
+  int groups = (deep ? 1 : 2) * g_compute_units / (slots > 0 ? slots : 1);
   if (groups < 1) groups = 1;
   if (groups > (tiles + plan.waves - 1) / plan.waves) groups = (tiles + plan.waves - 1) / plan.waves;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));
