@@ -180,30 +180,28 @@ __device__ __forceinline__ int ResolvePairs(const llmp_vecq_desc& d, int slot_in
 // The same list for a routed product whose workgroups share an expert's work instead: every pair's workgroups
 // get the pairs that name their pair's expert, in pair order, and `rank`, their own pair's place among them. An
 // expert that n pairs name then has n pairs' workgroups, each taking a share of its rows against all n tokens: the
-// weights are still read once, and the workgroups an expert gets grow with the tokens it serves. Ends with a
-// workgroup barrier.
+// weights are still read once, and the workgroups an expert gets grow with the tokens it serves. Every wave works
+// the list out for itself from one round of loads (the pairs' experts, two a lane) and writes the same words to
+// `pairs`, so no wave waits for another here: a wave reads back what it wrote itself.
 __device__ __forceinline__ int SharePairs(const llmp_vecq_desc& d, int slot_index, int* pairs, int* count, int* rank) {
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
+  const int lane = threadIdx.x & (kWave - 1);
   const int s = slot_index;
-  const int expert = d.ids[(s / d.used) * d.ids_stride + (s % d.used)];
-  if (tid < kWave) {
-    const int total = d.tokens * d.used;
-    int n = 0;
-    for (int base = 0; base < total; base += kWave) {
-      const int s2 = base + lane;
-      const int t = s2 / d.used;
-      const int u = s2 % d.used;
-      const bool match = s2 < total && d.ids[t * d.ids_stride + u] == expert;
-      const unsigned long long ballot = __ballot(match);
-      const int at = n + __popcll(ballot & ((1ull << lane) - 1ull));
-      if (match) pairs[at] = (t << 8) | u;
-      if (s2 == s) *rank = at;
-      n += __popcll(ballot);
-    }
-    if (lane == 0) *count = n;
-  }
-  __syncthreads();
+  const int total = d.tokens * d.used;
+  const int s0 = lane, s1 = kWave + lane;
+  const int t0 = s0 / d.used, u0 = s0 - t0 * d.used;
+  const int t1 = s1 / d.used, u1 = s1 - t1 * d.used;
+  const int id0 = s0 < total ? d.ids[t0 * d.ids_stride + u0] : 0;
+  const int id1 = s1 < total ? d.ids[t1 * d.ids_stride + u1] : 0;
+  const int expert = s < kWave ? __builtin_amdgcn_readlane(id0, s) : __builtin_amdgcn_readlane(id1, s - kWave);
+  const bool match0 = s0 < total && id0 == expert;
+  const bool match1 = s1 < total && id1 == expert;
+  const unsigned long long named0 = __ballot(match0), named1 = __ballot(match1);
+  const unsigned long long below = (1ull << lane) - 1ull;
+  const int n0 = __popcll(named0);
+  if (match0) pairs[__popcll(named0 & below)] = (t0 << 8) | u0;
+  if (match1) pairs[n0 + __popcll(named1 & below)] = (t1 << 8) | u1;
+  *count = n0 + __popcll(named1);
+  *rank = s < kWave ? __popcll(named0 & ((1ull << s) - 1ull)) : n0 + __popcll(named1 & ((1ull << (s - kWave)) - 1ull));
   return expert;
 }
 

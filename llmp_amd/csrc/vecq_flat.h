@@ -1384,7 +1384,6 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
-  __shared__ int rank_among;
 
   const llmp_vecq_desc& d = a.d;
   const int tid = threadIdx.x;
@@ -1419,7 +1418,7 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   // rows takes its expert's row range.
   int expert = blockIdx.y;
   int sorted_first = 0;
-  int rank = 0, sharers = 1;
+  int rank = 0, sharers = 1, routed_pairs = 0;
   if (a.offsets != nullptr) {
     sorted_first = a.offsets[expert];
     if (tid == 0) count = a.offsets[expert + 1] - sorted_first;
@@ -1427,9 +1426,8 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
     if (count == 0) return;  // uniform over the workgroup
   } else if (d.ids != nullptr) {
     // The pairs that name this pair's expert share its tiles: `count` pairs' workgroups, this pair's at `rank`.
-    expert = SharePairs(d, blockIdx.y, pairs, &count, &rank_among);
-    sharers = count;
-    rank = rank_among;
+    expert = SharePairs(d, blockIdx.y, pairs, &sharers, &rank);
+    routed_pairs = sharers;
   }
   const int64_t expert_block = static_cast<int64_t>(expert) * d.stride_expert;
   const int waves = blockDim.x / kWave;  // eight, fewer where a long row's records leave less room
@@ -1437,7 +1435,7 @@ __global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs
   const int tile_step = sharers * gridDim.x * waves;
   // A dense or grouped product's pairs are its tokens on the workgroup's matrix: no list.
   const bool listed = d.ids != nullptr && a.offsets == nullptr;
-  const int n = a.offsets == nullptr && d.ids == nullptr ? d.tokens : count;
+  const int n = a.offsets != nullptr ? count : d.ids != nullptr ? routed_pairs : d.tokens;
   auto pair_at = [&](int i) {
     return a.offsets != nullptr ? (sorted_first + i) << 8 : listed ? pairs[i] : (i << 8) | expert;
   };
