@@ -126,7 +126,7 @@ PROFILED_TRAFFIC = {
     # L2s of 4 MB an XCD: 191 MB fetched for 59 MB of operands, 50 MB written.
     "mxfp8_gemm_2048x12288x4096": _traffic(93182.8, 49173.6),
     "moe_q4_k_ffn_t1": _traffic(7028.8, 24.0),        # the gate/up launch
-    "moe_q4_k_ffn_t16": _traffic(76343.9, 457.9),     # the gate/up launch
+    "moe_q4_k_ffn_t16": _traffic(76769.0, 469.8),     # the gate/up launch
     "moe_q4_k_ffn_t512": _traffic(182457.3, 12338.4),  # the gate/up launch: the experts' tokens once a segment of rows
     "attn_vec_q8_0_d256_h16_kv8_cells8192_rows1": _traffic(17562.0 + 279.5, 528.0 + 16.0),  # the splits + their combination
     "attn_vec_q4_0_d256_h16_kv8_cells8192_rows1": _traffic(9369.5 + 279.5, 528.0 + 16.0),
