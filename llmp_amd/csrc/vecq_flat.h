@@ -1380,7 +1380,7 @@ __device__ __forceinline__ void AwaitAllBut(int left) {
 
 // grid (workgroups, slots); LDS: P tokens' records, then a tile buffer a wave.
 template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep>
-__global__ __launch_bounds__(kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
+__global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
   __shared__ int count;
@@ -1646,9 +1646,11 @@ struct FlatPlan {
   int rows;
   int waves;
   size_t lds;
+  bool wide = false;  // one workgroup of up to sixteen waves a CU instead of two of up to eight
 };
 
 constexpr size_t kFlatLdsLimit = 80 * 1024;  // two workgroups share a CU's 160 KB
+constexpr size_t kWideLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 constexpr int kFewestWaves = 3;
 
 // Eight waves a workgroup, fewer (down to kFewestWaves) where a long row's records would
@@ -1664,17 +1666,33 @@ FlatPlan PlanFlat(int pass, int units, bool glu, bool deep = false) {
   for (;;) {
     p.lds = ((static_cast<size_t>(pass) * units * F::kRecord + 15) & ~static_cast<size_t>(15)) +
             static_cast<size_t>(deep ? 2 : 1) * p.waves * (kWave * F::kUnitBytes + (kOdd ? 80 : 0));
-    if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) return p;
+    if (deep || p.lds <= kFlatLdsLimit || p.waves == kFewestWaves) break;
     --p.waves;
   }
+  if (deep || p.waves == kWaves) return p;
+  // A long row's records are staged once a workgroup: two workgroups a CU hold them twice and have room for fewer
+  // than sixteen tiles between them. One workgroup of up to sixteen waves holds them once: more tiles in flight a
+  // CU (15360 values: 15 tiles against 12, and the 3840 rows of a down projection are then one tile a wave).
+  const size_t records = (static_cast<size_t>(pass) * units * F::kRecord + 15) & ~static_cast<size_t>(15);
+  const size_t tile = kWave * F::kUnitBytes + (kOdd ? 80 : 0);
+  if (records >= kWideLdsLimit) return p;
+  int wide = static_cast<int>((kWideLdsLimit - records) / tile);
+  if (wide > 2 * kWaves) wide = 2 * kWaves;
+  if (wide > 2 * p.waves) {
+    p.waves = wide;
+    p.lds = records + wide * tile;
+    p.wide = true;
+  }
+  return p;
 }
+inline bool PlanFits(const FlatPlan& p) { return p.lds <= (p.wide ? kWideLdsLimit : kFlatLdsLimit); }
 constexpr size_t kDeepLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 int g_compute_units = 0;
 
 template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), static_cast<int>(kDeep ? kDeepLdsLimit : kFlatLdsLimit), &sized)) return;
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), static_cast<int>(kDeepLdsLimit), &sized)) return;
   hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(plan.waves * kWave), plan.lds, stream, a,
                      plan.rows);
 }
@@ -1781,7 +1799,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   }
   // The records a pass stages: four tokens', or a dense product's fewer.
   const int staged = a.offsets == nullptr && d.ids == nullptr && d.tokens < 4 ? d.tokens : 4;
-  if (pass > 1 && PlanFlat<F>(staged, units, glu).lds > kFlatLdsLimit) pass = 1;
+  if (pass > 1 && !PlanFits(PlanFlat<F>(staged, units, glu))) pass = 1;
   // Two tile buffers a wave: one token a pass, packed rows, one workgroup a CU.
   deep = deep && F::kUnitBytes <= 144 && pass == 1 && a.dump == nullptr && d.stride_row == d.ncols_x / F::kBlockValues &&
          PlanFlat<F>(1, units, glu, true).lds <= kDeepLdsLimit;
@@ -1794,7 +1812,7 @@ void LaunchF(const VecQArgs& a, int x_type, int pass, bool deep, hipStream_t str
   const int tiles = (d.nrows + plan.rows - 1) / plan.rows;
   // What is resident at once: two workgroups a CU, shared by the slots (every pair of a routed product has work:
   // the pairs that name an expert share it).
-  int groups = (deep ? 1 : 2) * g_compute_units / (slots > 0 ? slots : 1);
+  int groups = (deep || plan.wide ? 1 : 2) * g_compute_units / (slots > 0 ? slots : 1);
   if (groups < 1) groups = 1;
   if (groups > (tiles + plan.waves - 1) / plan.waves) groups = (tiles + plan.waves - 1) / plan.waves;
   const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(slots));

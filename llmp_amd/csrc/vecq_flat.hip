@@ -15,7 +15,7 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
   if (type == LLMP_TYPE_Q4_K) {
     const int units = d.ncols_x / FormatQ4K::kUnitValues;
     if (units > most) return pieces && PlanSplit<FormatQ4K>(units).lds <= kFlatLdsLimit;
-    return units >= 1 && PlanFlat<FormatQ4K>(1, units, glu).lds <= kFlatLdsLimit;
+    return units >= 1 && PlanFits(PlanFlat<FormatQ4K>(1, units, glu));
   }
   if (type == LLMP_TYPE_Q6_K) {
     // 210-byte blocks: matrices and experts at 16-byte boundaries and of a multiple of eight blocks (a tile's
@@ -24,14 +24,14 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     const int units = d.ncols_x / FormatQ6K::kUnitValues;
     if (at % 16 != 0 || d.stride_expert % 8 != 0 || units < 1 || units > most) return false;
     if (d.stride_row != units && (units % 8 != 0 || d.stride_row % 8 != 0)) return false;
-    return (static_cast<int64_t>(d.nrows) * units) % 8 == 0 && PlanFlat<FormatQ6K>(1, units, glu).lds <= kFlatLdsLimit;
+    return (static_cast<int64_t>(d.nrows) * units) % 8 == 0 && PlanFits(PlanFlat<FormatQ6K>(1, units, glu));
   }
   if (type == LLMP_TYPE_Q5_K) {
     const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
     if (at % 16 != 0) return false;
     const int units = d.ncols_x / FormatQ5K::kUnitValues;
     if (units > most) return pieces && PlanSplit<FormatQ5K>(units).lds <= kFlatLdsLimit;
-    return units >= 1 && PlanFlat<FormatQ5K>(1, units, glu).lds <= kFlatLdsLimit;
+    return units >= 1 && PlanFits(PlanFlat<FormatQ5K>(1, units, glu));
   }
   if (type == LLMP_TYPE_Q4_0 || type == LLMP_TYPE_Q4_1 || type == LLMP_TYPE_Q5_0 || type == LLMP_TYPE_Q5_1 ||
       type == LLMP_TYPE_IQ4_NL) {
@@ -41,7 +41,7 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     const auto fits = [&](auto format) {
       using F = decltype(format);
       if (units > most) return pieces && PlanSplit<F>(units).lds <= kFlatLdsLimit;
-      return PlanFlat<F>(1, units, glu).lds <= kFlatLdsLimit;
+      return PlanFits(PlanFlat<F>(1, units, glu));
     };
     return type == LLMP_TYPE_Q4_0 ? fits(FormatQ40{}) : type == LLMP_TYPE_IQ4_NL ? fits(FormatIq4nl{}) : type == LLMP_TYPE_Q4_1 ? fits(FormatQ41{})
            : type == LLMP_TYPE_Q5_0 ? fits(FormatQ50{}) : fits(FormatQ51{});
@@ -52,14 +52,14 @@ bool FlatTakes(int type, const llmp_vecq_desc& d, bool whole_rows) {
     if (d.ncols_x % 512 != 0 || d.stride_row % 16 != 0 || d.stride_expert % 16 != 0 || at % 16 != 0) return false;
     const int units = d.ncols_x / 256;
     if (units > most) return pieces && PlanSplit<FormatMxfp4>(units).lds <= kFlatLdsLimit;
-    return PlanFlat<FormatMxfp4>(1, units, glu).lds <= kFlatLdsLimit;
+    return PlanFits(PlanFlat<FormatMxfp4>(1, units, glu));
   }
   if (type != LLMP_TYPE_Q8_0 || d.ncols_x % 256 != 0) return false;
   const int units = d.ncols_x / FormatQ8::kUnitValues;
   const uintptr_t at = reinterpret_cast<uintptr_t>(d.w) | reinterpret_cast<uintptr_t>(d.g);
   if (d.stride_row % 8 != 0 || d.stride_expert % 8 != 0 || at % 16 != 0) return false;
   if (units > most) return pieces && PlanSplit<FormatQ8>(units).lds <= kFlatLdsLimit;
-  return PlanFlat<FormatQ8>(1, units, glu).lds <= kFlatLdsLimit;
+  return PlanFits(PlanFlat<FormatQ8>(1, units, glu));
 }
 
 // One launcher a format, each in its own translation unit (vecq_flat_*.hip).
