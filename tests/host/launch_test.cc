@@ -120,7 +120,7 @@ void DeviceChecks() {
   for (std::size_t at = 0; at < weights.size(); at += 34) {
     for (int i = 0; i < 34; ++i) weights[at + i] = static_cast<std::uint8_t>(rng.Next());
     weights[at] = static_cast<std::uint8_t>(rng.Next());
-    weights[at + 1] = 0x1F + static_cast<std::uint8_t>(rng.Next() % 4);  // half scales around 2^-8
+    weights[at + 1] = 0x1F + static_cast<std::uint8_t>(rng.Next() % 4);  // half scales near 2^-8
   }
   std::vector<float> tokens[4];
   for (auto& token : tokens) {
