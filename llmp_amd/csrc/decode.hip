@@ -756,51 +756,61 @@ __global__ __launch_bounds__(256) void DecodeMatrixKernel(const DecodeArgs a, co
 // w / 4, outputs' quarter w % 4) multiplies 64 rows by 64 outputs. Two stages of both tiles: after a chunk's one
 // barrier a wave queues the loads of the chunk after the next, and decodes the next chunk (loaded a step ago)
 // into the other stage among this chunk's matrix instructions.
-constexpr int kSharedRows = 128, kSharedOutputs = 256;
-constexpr int kSharedInputBytes = kSharedRows * kMatrixRowBytes, kSharedStageBytes = (kSharedRows + kSharedOutputs) * kMatrixRowBytes;
+// MR: groups of 16 input rows a wave (4: the tile is 128 input rows; 8: 256, where the inputs have that many and the
+// tiles still fill the device: a decoded segment then serves twice the matrix instructions, and a wave reads 24
+// operands of LDS for 64 instructions instead of 16 for 32).
+constexpr int kSharedOutputs = 256;
+constexpr int SharedStageBytes(int mr) { return (32 * mr + kSharedOutputs) * kMatrixRowBytes; }
 
-template <int D>
+template <int D, int MR>
 __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs a, const uint32_t rows) {
   constexpr bool kHalf = D == LLMP_DECODER_F16_DENSE || D == LLMP_DECODER_Q8_0_BLOCKS;
+  constexpr int kSharedRows = 32 * MR;
+  constexpr int kSharedInputBytes = kSharedRows * kMatrixRowBytes, kSharedStageBytes = SharedStageBytes(MR);
   extern __shared__ __attribute__((aligned(16))) uint8_t stages[];  // two of inputs' tile, weights' tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 15, q = lane >> 4;
   const uint32_t out0 = blockIdx.x * kSharedOutputs, t0 = blockIdx.y * kSharedRows;
-  const uint32_t row_half = (wave >> 2) * 64, out_quarter = (wave & 3) * 64;
+  const uint32_t row_half = (wave >> 2) * (16 * MR), out_quarter = (wave & 3) * 64;
   const uint32_t segs = a.w.k / 16u, chunks = (segs + 3u) / 4u;
-  Float4 acc[4][4];  // [outputs' group][input rows' group]
+  Float4 acc[4][MR];  // [outputs' group][input rows' group]
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int m = 0; m < MR; ++m) acc[g][m] = Float4{0.0f, 0.0f, 0.0f, 0.0f};
   }
-  // A thread's share of a chunk: four pieces of four input values (row c / 16, columns 4 (c % 16) + [0, 4) for
+  // A thread's share of a chunk: MR pieces of four input values (row c / 16, columns 4 (c % 16) + [0, 4) for
   // c = tid + 512 i) and two segments of weights (output e / 4, segment e % 4 for e = tid + 512 u). Loads
   // without branches: past the inputs, the outputs or K they read a valid address nearby, zeroed when staged.
   struct Share {
-    float4 piece[4];
+    float4 piece[MR];
     RawSegment raw[2];
   };
-  auto load = [&](uint32_t chunk, Share& share) {
+  auto load_inputs = [&](uint32_t chunk, Share& share) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MR; ++i) {
       const uint32_t c = tid + i * 512;
       const uint32_t row = min(t0 + (c >> 4), rows - 1), column = min(chunk * 64u + (c & 15u) * 4u, a.w.k - 4u);
       share.piece[i] = *reinterpret_cast<const float4*>(a.x + static_cast<uint64_t>(row) * a.x_stride + column);
     }
+  };
+  auto load_weights = [&](uint32_t chunk, Share& share) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const uint32_t e = tid + u * 512;
       share.raw[u] = FetchSegment<D>(a.w, a.first + min(out0 + (e >> 2), a.outputs - 1), min(chunk * 4u + (e & 3u), segs - 1));
     }
   };
-  auto stage = [&](uint32_t chunk, const Share& share) {
+  auto load = [&](uint32_t chunk, Share& share) {
+    load_inputs(chunk, share);
+    load_weights(chunk, share);
+  };
+  auto stage_inputs = [&](uint32_t chunk, const Share& share) {
     uint8_t* inputs = stages + (chunk & 1u) * kSharedStageBytes;
-    uint8_t* weights = inputs + kSharedInputBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MR; ++i) {
       const uint32_t c = tid + i * 512;
       const bool live = t0 + (c >> 4) < rows && chunk * 64u + (c & 15u) * 4u < a.w.k;
       uint2 packed;
@@ -808,6 +818,9 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
       packed.y = live ? ToElement<kHalf>(share.piece[i].z) | (ToElement<kHalf>(share.piece[i].w) << 16) : 0u;
       *reinterpret_cast<uint2*>(inputs + (c >> 4) * kMatrixRowBytes + (c & 15u) * 8u) = packed;
     }
+  };
+  auto stage_weights = [&](uint32_t chunk, const Share& share) {
+    uint8_t* weights = stages + (chunk & 1u) * kSharedStageBytes + kSharedInputBytes;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const uint32_t e = tid + u * 512;
@@ -827,31 +840,41 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
       to[0] = half[0], to[1] = half[1];
     }
   };
+  auto stage = [&](uint32_t chunk, const Share& share) {
+    stage_inputs(chunk, share);
+    stage_weights(chunk, share);
+  };
   auto multiply = [&](uint32_t chunk) {
     const uint8_t* inputs = stages + (chunk & 1u) * kSharedStageBytes;
     const uint8_t* weights = inputs + kSharedInputBytes;
-    U32x4 b[4][2];
+    // A half of the chunk's K at a time: the outputs' four operands stay, the rows' pass by.
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const U32x4* mine = reinterpret_cast<const U32x4*>(weights + (out_quarter + 16 * g + n) * kMatrixRowBytes + q * 32);
-      b[g][0] = mine[0], b[g][1] = mine[1];
-    }
+    for (int j = 0; j < 2; ++j) {
+      U32x4 b[4];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const U32x4* mine = reinterpret_cast<const U32x4*>(inputs + (row_half + 16 * m + n) * kMatrixRowBytes + q * 32);
+      for (int g = 0; g < 4; ++g)
+        b[g] = reinterpret_cast<const U32x4*>(weights + (out_quarter + 16 * g + n) * kMatrixRowBytes + q * 32)[j];
+      // (The rows' operands are read one group ahead of their use and no further: left to itself the compiler
+      // reads all of them first and the tall tile's registers spill.)
+      auto rows_operand = [&](int m) {
+        return reinterpret_cast<const U32x4*>(inputs + (row_half + 16 * m + n) * kMatrixRowBytes + q * 32)[j];
+      };
+      U32x4 ahead = rows_operand(0);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const U32x4 x8 = mine[j];
+      for (int m = 0; m < MR; ++m) {
+        const U32x4 x8 = ahead;
+        if (m + 1 < MR) ahead = rows_operand(m + 1);
+        if constexpr (MR > 4) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           if constexpr (kHalf) {
             typedef _Float16 Half8 __attribute__((ext_vector_type(8)));
             acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(Half8, x8),
-                                                               __builtin_bit_cast(Half8, b[g][j]), acc[g][m], 0, 0, 0);
+                                                               __builtin_bit_cast(Half8, b[g]), acc[g][m], 0, 0, 0);
           } else {
             typedef __bf16 Bf8 __attribute__((ext_vector_type(8)));
             acc[g][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(Bf8, x8),
-                                                                __builtin_bit_cast(Bf8, b[g][j]), acc[g][m], 0, 0, 0);
+                                                                __builtin_bit_cast(Bf8, b[g]), acc[g][m], 0, 0, 0);
           }
         }
       }
@@ -859,15 +882,29 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
   };
   Share share[2];  // by the chunk's parity
   load(0, share[0]);
-  load(1, share[1]);
+  if constexpr (MR > 4) {
+    load_weights(1, share[1]);
+  } else {
+    load(1, share[1]);
+  }
   stage(0, share[0]);
   auto step = [&](uint32_t chunk, auto parity) {
     constexpr int P = decltype(parity)::value;
     // One barrier a chunk: its stage is complete, and the other stage's readers (the last chunk's) are done.
     __syncthreads();
-    load(chunk + 2, share[P]);
-    multiply(chunk);
-    stage(chunk + 1, share[1 - P]);
+    if constexpr (MR > 4) {
+      // The tall tile's registers hold one chunk's inputs, not two: the next chunk's are asked for here, a chunk's
+      // multiplies ahead of their staging, into the set the weights' loads two chunks ahead do not use.
+      load_weights(chunk + 2, share[P]);
+      load_inputs(chunk + 1, share[0]);
+      multiply(chunk);
+      stage_inputs(chunk + 1, share[0]);
+      stage_weights(chunk + 1, share[1 - P]);
+    } else {
+      load(chunk + 2, share[P]);
+      multiply(chunk);
+      stage(chunk + 1, share[1 - P]);
+    }
   };
   for (uint32_t chunk = 0; chunk < chunks; chunk += 2) {  // every wave: the same count of barriers
     step(chunk, std::integral_constant<int, 0>{});
@@ -880,7 +917,7 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
     if (out < a.outputs) {
       const float scale = a.w.tensor_scale != nullptr ? a.w.tensor_scale[(a.first + out) / a.w.rows_per_scale] : 1.0f;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
+      for (int m = 0; m < MR; ++m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t t = t0 + row_half + 16 * m + 4 * q + i;
@@ -891,11 +928,11 @@ __global__ __launch_bounds__(512) void DecodeMatrixSharedKernel(const DecodeArgs
   }
 }
 
-template <int D>
+template <int D, int MR>
 void LaunchMatrixShared(const DecodeArgs& a, dim3 grid, uint32_t rows, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&DecodeMatrixSharedKernel<D>), 2 * kSharedStageBytes, &sized)) return;
-  hipLaunchKernelGGL((DecodeMatrixSharedKernel<D>), grid, dim3(512), 2 * kSharedStageBytes, stream, a, rows);
+  if (!AllowLds(reinterpret_cast<const void*>(&DecodeMatrixSharedKernel<D, MR>), 2 * SharedStageBytes(MR), &sized)) return;
+  hipLaunchKernelGGL((DecodeMatrixSharedKernel<D, MR>), grid, dim3(512), 2 * SharedStageBytes(MR), stream, a, rows);
 }
 
 size_t DecodeLds(int tokens, uint32_t k) { return static_cast<size_t>(tokens) * (k / 16u) * kSegmentStride; }
@@ -1246,15 +1283,20 @@ extern "C" int llmp_hip_decode_matrix(int decoder, const llmp_decode_operand* w,
   a.x = x, a.x_stride = x_stride, a.y = y, a.y_stride = y_stride;
   // Tiles of 256 outputs by 128 input rows where those still give every other CU a workgroup; else 64 by 64.
   const int cus = llmp_hip_compute_units();
-  const bool wide = 2 * ((outputs + 255) / 256 * ((rows + 127) / 128)) >= static_cast<uint64_t>(cus > 0 ? cus : 256);
-  const uint64_t per = wide ? 256 : 64, tile = wide ? 128 : 64;
+  const uint64_t units = static_cast<uint64_t>(cus > 0 ? cus : 256);
+  const bool wide = 2 * ((outputs + 255) / 256 * ((rows + 127) / 128)) >= units;
+  // Tiles of 256 input rows where the inputs have them and the tiles still give every CU one.
+  const bool tall = wide && rows >= 256 && (outputs + 255) / 256 * ((rows + 255) / 256) >= units;
+  const uint64_t per = wide ? 256 : 64, tile = tall ? 256 : wide ? 128 : 64;
   const dim3 grid(static_cast<unsigned>((outputs + per - 1) / per), static_cast<unsigned>((rows + tile - 1) / tile));
   const auto s = static_cast<hipStream_t>(stream);
   switch (decoder) {
 #define LLMP_DECODER(ID)                                                                                          \
   case ID:                                                                                                        \
-    if (wide) {                                                                                                   \
-      LaunchMatrixShared<ID>(a, grid, static_cast<uint32_t>(rows), s);                                           \
+    if (tall) {                                                                                                   \
+      LaunchMatrixShared<ID, 8>(a, grid, static_cast<uint32_t>(rows), s);                                        \
+    } else if (wide) {                                                                                            \
+      LaunchMatrixShared<ID, 4>(a, grid, static_cast<uint32_t>(rows), s);                                        \
     } else {                                                                                                      \
       hipLaunchKernelGGL((DecodeMatrixKernel<ID, 1, 4>), grid, dim3(256), 0, s, a, static_cast<uint32_t>(rows)); \
     }                                                                                                             \

@@ -305,6 +305,23 @@ def test_matrix_large_tiles_match_oracle(device, decoder):
     assert ok, (oracle.DECODERS[decoder], worst)
 
 
+@pytest.mark.parametrize("decoder", list(range(12)))
+def test_matrix_tall_tiles_match_oracle(device, decoder):
+    """Enough outputs and input rows for a tile of 256 outputs by 256 input rows on every compute unit (17 by 16
+    tiles), with partial tiles of both and of K."""
+    n, rows = 4140, 3900
+    k = 160 if decoder in (0, 1, 3, 5, 11) else 256 if decoder in (8, 10) else 192
+    w = synth.affine_weight(n, k, 880, bits=4, group=32, scale="f16") if decoder == 11 else \
+        synth.decode_weight(decoder, n, k, 880 + decoder, tensor_scales=5)
+    x = synth.activations(rows, k, 881)
+    wd = {key: (torch.from_numpy(np.ascontiguousarray(v)).to(device) if isinstance(v, np.ndarray) else v)
+          for key, v in w.items() if key != "plain"}
+    want = oracle.decode_matrix(decoder, w, x, first=7, outputs=4100, threads=oracle.max_threads())
+    got = ops.decode_matrix(decoder, wd, torch.from_numpy(x).to(device), first=7, outputs=4100).cpu().numpy()
+    ok, worst = rel_close(got, want, 1e-3)
+    assert ok, (oracle.DECODERS[decoder], worst)
+
+
 def test_matrix_refusals(device):
     w = to_device(synth.decode_weight(3, 8, 256, 850), device)
     x = torch.zeros((4, 256), dtype=torch.float32, device=device)
