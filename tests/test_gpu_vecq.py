@@ -198,6 +198,37 @@ def test_routed_experts_match_oracle(device, t, tokens, used):
     assert ok, worst
 
 
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+@pytest.mark.parametrize("routing", ["one expert", "one a pair", "two experts, unequal"])
+def test_routed_pairs_that_share_an_expert(device, t, routing):
+    """The pairs that name an expert share its rows (every pair's workgroups at work on a share of them, each
+    against all of the expert's tokens): whatever the picks, a pair's values are the oracle's and, bit for bit, those
+    of its own token alone through its expert as a dense product."""
+    tokens, used, k, n = 16, 8, 1024, 203  # 128 pairs; several tiles a share, the last partial
+    experts = {"one expert": 3, "one a pair": 128, "two experts, unequal": 5}[routing]
+    qk, bs = oracle.block_elements(t), oracle.block_bytes(t)
+    w = make_weights(t, experts * n, k, 91).reshape(experts, n * (k // qk) * bs)
+    pair = np.arange(tokens * used)
+    if routing == "one expert":
+        ids = np.full(tokens * used, 2)
+    elif routing == "one a pair":
+        ids = synth.rng(92).permutation(experts)[pair]
+    else:
+        ids = np.where(pair % 7 == 3, 4, 1)  # 18 pairs name one, 110 the other
+    ids = ids.reshape(tokens, used).astype(np.int32)
+    x = synth.activations(tokens, k, 93)
+    q8 = oracle.q8_1_quantize(x)
+    stride_expert = n * (k // qk)
+    want = oracle.vecq(t, w, q8, k, n, ids=ids, tokens=tokens, used=used, stride_expert=stride_expert, experts=experts)
+    wd, q8d = dev(w, device), dev(q8, device)
+    got = ops.vecq(t, wd, q8d, k, n, ids=dev(ids, device), tokens=tokens, used=used, stride_expert=stride_expert).cpu().numpy()
+    ok, worst = rel_close(got, want, TOL)
+    assert ok, worst
+    for token, slot in ((0, 0), (5, 3), (15, 7)):
+        alone = ops.vecq(t, wd[ids[token, slot]].contiguous(), q8d[token:token + 1].contiguous(), k, n, tokens=1).cpu().numpy()
+        assert np.array_equal(alone.reshape(n).view(np.uint32), got[token, slot].view(np.uint32)), (token, slot)
+
+
 @pytest.mark.parametrize("t,k", [(Q8_0, 9216), (Q4_K, 18432)])
 def test_routed_and_sorted_long_rows_match_oracle(device, t, k):
     """Rows streamed in pieces, under routing ids and under sorted-row offsets."""
