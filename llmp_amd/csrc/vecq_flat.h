@@ -49,6 +49,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "llmp_hip.h"
 #include "vecq_common.h"
@@ -97,6 +99,54 @@ __device__ __forceinline__ FrontQ8 LoadFrontQ8(const uint8_t* __restrict__ y, in
   }
   return f;
 }
+
+// The same loads written as instructions, always issued (a thread past the row's blocks reads the last block
+// again): the compiler neither counts them nor waits for them, so the kernel's own wait, after the first tile's
+// loads are queued, decides when they are read (AwaitFront). Loads the compiler knows of were waited for where
+// they were issued, a trip to memory before the first tile's loads, and again with every tile load landed
+// (their number is not known at compile time) before the staging that should run under them.
+typedef uint32_t FrontWords __attribute__((ext_vector_type(4)));
+struct FrontQ8Asm {
+  FrontWords a, b;  // the block's first eight words
+  uint32_t c;       // its ninth
+};
+__device__ __forceinline__ FrontQ8Asm LoadFrontQ8Asm(const uint8_t* __restrict__ y, int blocks) {
+  FrontQ8Asm f;
+  const int b = min(static_cast<int>(threadIdx.x), blocks - 1);
+  const uint8_t* src = y + static_cast<int64_t>(b) * kQ8Block;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(f.a) : "v"(src) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(f.b) : "v"(src) : "memory");
+  asm volatile("global_load_dword %0, %1, off offset:32" : "=v"(f.c) : "v"(src) : "memory");
+  return f;
+}
+// The front loads have landed once no more than `later` memory operations issued after them are outstanding (a
+// wave's memory operations complete in order); `later` must not exceed the number actually issued since.
+__device__ __forceinline__ void AwaitFront(FrontQ8Asm& f, int later) {
+  // One statement for every count: the registers go in and come out of it where they are. (A switch over ten
+  // statements let the compiler copy the registers on its way into a case, ahead of the wait, while the loads were
+  // still on their way.)
+  const int n = __builtin_amdgcn_readfirstlane(later);
+  asm volatile(
+      "s_cmp_lt_u32 %3, 10\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(10)\n\ts_branch 11f\n"
+      "1:\ts_cmp_lt_u32 %3, 9\n\ts_cbranch_scc1 2f\n\ts_waitcnt vmcnt(9)\n\ts_branch 11f\n"
+      "2:\ts_cmp_lt_u32 %3, 8\n\ts_cbranch_scc1 3f\n\ts_waitcnt vmcnt(8)\n\ts_branch 11f\n"
+      "3:\ts_cmp_lt_u32 %3, 7\n\ts_cbranch_scc1 4f\n\ts_waitcnt vmcnt(7)\n\ts_branch 11f\n"
+      "4:\ts_cmp_lt_u32 %3, 6\n\ts_cbranch_scc1 5f\n\ts_waitcnt vmcnt(6)\n\ts_branch 11f\n"
+      "5:\ts_cmp_lt_u32 %3, 5\n\ts_cbranch_scc1 6f\n\ts_waitcnt vmcnt(5)\n\ts_branch 11f\n"
+      "6:\ts_cmp_lt_u32 %3, 4\n\ts_cbranch_scc1 7f\n\ts_waitcnt vmcnt(4)\n\ts_branch 11f\n"
+      "7:\ts_cmp_lt_u32 %3, 3\n\ts_cbranch_scc1 8f\n\ts_waitcnt vmcnt(3)\n\ts_branch 11f\n"
+      "8:\ts_cmp_lt_u32 %3, 2\n\ts_cbranch_scc1 9f\n\ts_waitcnt vmcnt(2)\n\ts_branch 11f\n"
+      "9:\ts_cmp_lt_u32 %3, 1\n\ts_cbranch_scc1 10f\n\ts_waitcnt vmcnt(1)\n\ts_branch 11f\n"
+      "10:\ts_waitcnt vmcnt(0)\n"
+      "11:"
+      : "+v"(f.a), "+v"(f.b), "+v"(f.c)
+      : "s"(n)
+      : "scc", "memory");
+}
+__device__ __forceinline__ uint32_t FlatLdsAddress(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
+__device__ __forceinline__ void FlatLdsWrite16(uint32_t at, FrontWords v) { asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(v) : "memory"); }
+__device__ __forceinline__ void FlatLdsWrite4(uint32_t at, uint32_t v) { asm volatile("ds_write_b32 %0, %1" : : "v"(at), "v"(v) : "memory"); }
+__device__ __forceinline__ void FlatLdsWrite2(uint32_t at, uint32_t v) { asm volatile("ds_write_b16 %0, %1" : : "v"(at), "v"(v) : "memory"); }
 
 __device__ __forceinline__ float ByteToFloat(uint32_t word, int byte) {
   return static_cast<float>((word >> (8 * byte)) & 0xFFu);  // v_cvt_f32_ubyteN
@@ -161,6 +211,28 @@ struct FormatQ4K {
     reinterpret_cast<float*>(record + 256)[g] = d8;
     reinterpret_cast<float*>(record + 288)[g] = d8 * static_cast<float>(s);
     reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
+  }
+
+  // The same with the record written by instructions the compiler does not take for accesses of LDS: it would hold
+  // them back until every load into LDS in flight has landed.
+  static constexpr bool kStagesUnderLoads = true;
+  static __device__ __forceinline__ void StageQ8Asm(const FrontQ8Asm& f, int b, uint8_t* token) {
+    const uint32_t record = FlatLdsAddress(token) + static_cast<uint32_t>((b >> 3) * kRecord);
+    const int g = b & 7;
+    FlatLdsWrite16(record + g * 32, FrontWords{f.a.y, f.a.z, f.a.w, f.b.x});
+    FlatLdsWrite16(record + g * 32 + 16, FrontWords{f.b.y, f.b.z, f.b.w, f.c});
+    int s = Dot4(0x01010101, static_cast<int>(f.a.y), 0);
+    s = Dot4(0x01010101, static_cast<int>(f.a.z), s);
+    s = Dot4(0x01010101, static_cast<int>(f.a.w), s);
+    s = Dot4(0x01010101, static_cast<int>(f.b.x), s);
+    s = Dot4(0x01010101, static_cast<int>(f.b.y), s);
+    s = Dot4(0x01010101, static_cast<int>(f.b.z), s);
+    s = Dot4(0x01010101, static_cast<int>(f.b.w), s);
+    s = Dot4(0x01010101, static_cast<int>(f.c), s);
+    const float d8 = HalfBitsToFloat(f.a.x & 0xFFFFu);
+    FlatLdsWrite4(record + 256 + g * 4, __builtin_bit_cast(uint32_t, d8));
+    FlatLdsWrite4(record + 288 + g * 4, __builtin_bit_cast(uint32_t, d8 * static_cast<float>(s)));
+    FlatLdsWrite2(record + 320 + g * 2, static_cast<uint32_t>(s));
   }
 
   // The super-block at `at` (LDS) times the staged tokens. With several tokens a pass the
@@ -502,6 +574,26 @@ struct FormatQ8 {
       dst[8] = w[8] >> 16;
     }
     reinterpret_cast<float*>(record + 136)[j] = HalfBitsToFloat(w[0] & 0xFFFFu);
+  }
+
+  // The same by instructions (see FormatQ4K::StageQ8Asm).
+  static constexpr bool kStagesUnderLoads = true;
+  static __device__ __forceinline__ void StageQ8Asm(const FrontQ8Asm& f, int b, uint8_t* token) {
+    const uint32_t w[9] = {f.a.x, f.a.y, f.a.z, f.a.w, f.b.x, f.b.y, f.b.z, f.b.w, f.c};
+    const uint32_t record = FlatLdsAddress(token) + static_cast<uint32_t>((b >> 2) * kRecord);
+    const int j = b & 3;
+    if (j & 1) {
+      const uint32_t dst = record + 4 * (j == 1 ? 9 : 26);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) FlatLdsWrite4(dst + 4 * i, w[1 + i]);
+    } else {
+      const uint32_t dst = record + 4 * (j == 0 ? 0 : 17);
+      FlatLdsWrite4(dst, w[1] << 16);
+#pragma unroll
+      for (int i = 1; i < 8; ++i) FlatLdsWrite4(dst + 4 * i, (w[i] >> 16) | (w[i + 1] << 16));
+      FlatLdsWrite4(dst + 32, w[8] >> 16);
+    }
+    FlatLdsWrite4(record + 136 + 4 * j, __builtin_bit_cast(uint32_t, HalfBitsToFloat(w[0] & 0xFFFFu)));
   }
 
   template <int P, bool kDump>
@@ -1249,6 +1341,27 @@ __device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k,
   }
 }
 
+// Formats whose records of Q8_1 activations are staged by instructions, under the first tile's loads.
+template <class F, class = void>
+struct StagesUnderLoads : std::false_type {};
+template <class F>
+struct StagesUnderLoads<F, std::void_t<decltype(F::kStagesUnderLoads)>> : std::bool_constant<F::kStagesUnderLoads> {};
+
+// The front block by instructions; the row's further blocks (rows of more blocks than the workgroup has threads)
+// as the compiler orders them.
+template <class F>
+__device__ __forceinline__ void StageRecordsQ8Asm(const uint8_t* __restrict__ y, int blocks, const FrontQ8Asm& front,
+                                                  uint8_t* token) {
+  if (static_cast<int>(threadIdx.x) < blocks) F::StageQ8Asm(front, threadIdx.x, token);
+  for (int b = threadIdx.x + blockDim.x; b < blocks; b += blockDim.x) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(y + static_cast<int64_t>(b) * kQ8Block);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = src[i];
+    F::StageQ8(w, b, token);
+  }
+}
+
 template <class F>
 __device__ __forceinline__ void StageRecordsQ8(const uint8_t* __restrict__ y, int blocks, const FrontQ8& front,
                                                uint8_t* token) {
@@ -1379,7 +1492,12 @@ __device__ __forceinline__ void AwaitAllBut(int left) {
 }
 
 // grid (workgroups, slots); LDS: P tokens' records, then a tile buffer a wave.
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep>
+// kUnder: the Q8_1 activations' records are staged under the first tile's loads (loads and LDS writes by
+// instructions, a barrier for LDS alone), for launches whose waves take one tile each: the launch is then one trip
+// to memory, and the trip for the activations and their staging no longer stand in front of it and behind it. With
+// two tiles a wave it measured slower (the gate/up pair 14.7 to 15.2 us against 14.2): there the waves do better
+// entering the first products together.
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep, bool kUnder = false>
 __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
@@ -1444,9 +1562,11 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
     const int m = min(P, n - p0);
     if (p0 > 0) __syncthreads();  // the last pass's readers of the records
     // The activations' first loads, then the wave's first tile, then the staging.
+    constexpr bool kAsmFront = kUnder;
     const void* rows_x[P];
     FrontX front_x[XT < 0 ? 1 : P];
-    FrontQ8 front_q[XT < 0 ? P : 1];
+    FrontQ8 front_q[XT < 0 && !kAsmFront ? P : 1];
+    FrontQ8Asm front_a[kAsmFront ? P : 1];
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
@@ -1456,7 +1576,11 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
         if constexpr (XT < 0) {
           rows_x[j] = static_cast<const uint8_t*>(d.y) +
                       (static_cast<int64_t>(token) * d.y_token + static_cast<int64_t>(slot) * d.y_slot) * kQ8Block;
-          front_q[j] = LoadFrontQ8(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32);
+          if constexpr (kAsmFront) {
+            front_a[j] = LoadFrontQ8Asm(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32);
+          } else {
+            front_q[j] = LoadFrontQ8(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32);
+          }
         } else {
           const int64_t at = token * a.x_token + slot * a.x_slot;
           rows_x[j] = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
@@ -1466,22 +1590,40 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
       }
     }
     int index = first_tile;
+    int tile_loads = 0;  // no more than the loads the first tile's fetch issues
     if (index < tiles) {
       const int row0 = index * rows_per_tile;
       FetchTile<F, kGlu, kPacked>(d, expert_block, row0, min(rows_per_tile, d.nrows - row0), nsb, gate_at, ring, lane);
+      tile_loads = TileLoads<F, kGlu>(min(rows_per_tile, d.nrows - row0), nsb);
+    }
+    if constexpr (kAsmFront) {
+      // The activations' blocks have landed once only the tile's loads, issued after them, are outstanding.
+#pragma unroll
+      for (int j = 0; j < P; ++j) {
+        if (j < m) AwaitFront(front_a[j], tile_loads);
+      }
     }
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
         uint8_t* records = lds + j * token_stride;
-        if constexpr (XT < 0) {
+        if constexpr (kAsmFront) {
+          StageRecordsQ8Asm<F>(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_a[j], records);
+        } else if constexpr (XT < 0) {
           StageRecordsQ8<F>(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_q[j], records);
         } else {
           StageRecordsX<F, XT>(rows_x[j], d.ncols_x, front_x[j], records);
         }
       }
     }
-    __syncthreads();  // the records are staged; from here the waves run alone
+    // The records are staged; from here the waves run alone. (A barrier for LDS alone where the staging ran under
+    // the tile's loads: __syncthreads would wait for those to land as well.)
+    if constexpr (kAsmFront) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+    } else {
+      __syncthreads();
+    }
 
     int buffer = 0;  // kDeep: the tile buffer the tile `index` is in
     while (index < tiles) {
@@ -1689,11 +1831,11 @@ inline bool PlanFits(const FlatPlan& p) { return p.lds <= (p.wide ? kWideLdsLimi
 constexpr size_t kDeepLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 int g_compute_units = 0;
 
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false>
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false, bool kUnder = false>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
-  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), static_cast<int>(kDeepLdsLimit), &sized)) return;
-  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep>), grid, dim3(plan.waves * kWave), plan.lds, stream, a,
+  if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep, kUnder>), static_cast<int>(kDeepLdsLimit), &sized)) return;
+  hipLaunchKernelGGL((VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep, kUnder>), grid, dim3(plan.waves * kWave), plan.lds, stream, a,
                      plan.rows);
 }
 
@@ -1707,6 +1849,14 @@ void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, bool deep, hipS
   if (deep) {
     if constexpr (P == 1) LaunchK<F, P, kGlu, XT, false, true, true>(a, grid, plan, stream);
     return;
+  }
+  if constexpr (P == 1 && XT < 0 && StagesUnderLoads<F>::value) {
+    // One tile a wave at most: the records staged under its loads.
+    const int tiles = (a.d.nrows + plan.rows - 1) / plan.rows;
+    if (packed && tiles <= static_cast<int>(grid.x) * plan.waves) {
+      LaunchK<F, P, kGlu, XT, false, true, false, true>(a, grid, plan, stream);
+      return;
+    }
   }
   if (packed) {
     LaunchK<F, P, kGlu, XT, false, true>(a, grid, plan, stream);
