@@ -143,6 +143,73 @@ __device__ __forceinline__ void AwaitFront(FrontQ8Asm& f, int later) {
       : "s"(n)
       : "scc", "memory");
 }
+// The unquantized activations' front pieces the same way: a lane's four values of a block as they lie in memory
+// (sixteen bytes of F32, eight of BF16 or F16; the row aligned to that), always loaded (a lane past the row's blocks
+// reads the last block's piece again), converted after the wait.
+typedef uint32_t FrontPair __attribute__((ext_vector_type(2)));
+template <int XT>
+struct FrontXAsm {
+  FrontWords w[kFront];  // F32
+  FrontPair h[kFront];   // the 16-bit types
+};
+template <int XT>
+__device__ __forceinline__ FrontXAsm<XT> LoadFrontXAsm(const void* __restrict__ x, int k) {
+  FrontXAsm<XT> f;
+  const int lane8 = threadIdx.x & 7;
+#pragma unroll
+  for (int i = 0; i < kFront; ++i) {
+    const int b = min(static_cast<int>(threadIdx.x >> 3) + i * static_cast<int>(blockDim.x >> 3), k / 32 - 1);
+    const int64_t at = static_cast<int64_t>(b) * 32 + lane8 * 4;
+    if constexpr (XT == LLMP_X_F32) {
+      const float* src = static_cast<const float*>(x) + at;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(f.w[i]) : "v"(src) : "memory");
+    } else {
+      const uint16_t* src = static_cast<const uint16_t*>(x) + at;
+      asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(f.h[i]) : "v"(src) : "memory");
+    }
+  }
+  return f;
+}
+#define LLMP_WAIT_CHAIN                                                                            \
+  "s_cmp_lt_u32 %2, 10\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(10)\n\ts_branch 11f\n"               \
+  "1:\ts_cmp_lt_u32 %2, 9\n\ts_cbranch_scc1 2f\n\ts_waitcnt vmcnt(9)\n\ts_branch 11f\n"             \
+  "2:\ts_cmp_lt_u32 %2, 8\n\ts_cbranch_scc1 3f\n\ts_waitcnt vmcnt(8)\n\ts_branch 11f\n"             \
+  "3:\ts_cmp_lt_u32 %2, 7\n\ts_cbranch_scc1 4f\n\ts_waitcnt vmcnt(7)\n\ts_branch 11f\n"             \
+  "4:\ts_cmp_lt_u32 %2, 6\n\ts_cbranch_scc1 5f\n\ts_waitcnt vmcnt(6)\n\ts_branch 11f\n"             \
+  "5:\ts_cmp_lt_u32 %2, 5\n\ts_cbranch_scc1 6f\n\ts_waitcnt vmcnt(5)\n\ts_branch 11f\n"             \
+  "6:\ts_cmp_lt_u32 %2, 4\n\ts_cbranch_scc1 7f\n\ts_waitcnt vmcnt(4)\n\ts_branch 11f\n"             \
+  "7:\ts_cmp_lt_u32 %2, 3\n\ts_cbranch_scc1 8f\n\ts_waitcnt vmcnt(3)\n\ts_branch 11f\n"             \
+  "8:\ts_cmp_lt_u32 %2, 2\n\ts_cbranch_scc1 9f\n\ts_waitcnt vmcnt(2)\n\ts_branch 11f\n"             \
+  "9:\ts_cmp_lt_u32 %2, 1\n\ts_cbranch_scc1 10f\n\ts_waitcnt vmcnt(1)\n\ts_branch 11f\n"            \
+  "10:\ts_waitcnt vmcnt(0)\n"                                                                       \
+  "11:"
+template <int XT>
+__device__ __forceinline__ void AwaitFrontX(FrontXAsm<XT>& f, int later) {
+  static_assert(kFront == 2, "the registers this wait ties");
+  const int n = __builtin_amdgcn_readfirstlane(later);
+  if constexpr (XT == LLMP_X_F32) {
+    asm volatile(LLMP_WAIT_CHAIN : "+v"(f.w[0]), "+v"(f.w[1]) : "s"(n) : "scc", "memory");
+  } else {
+    asm volatile(LLMP_WAIT_CHAIN : "+v"(f.h[0]), "+v"(f.h[1]) : "s"(n) : "scc", "memory");
+  }
+}
+#undef LLMP_WAIT_CHAIN
+template <int XT>
+__device__ __forceinline__ void FrontValues(const FrontXAsm<XT>& f, int i, float (&v)[4]) {
+  const FrontPair w = f.h[i];
+  if constexpr (XT == LLMP_X_F32) {
+    // (Through scalars: __builtin_bit_cast of a vector's component reads its first component with this compiler.)
+    const uint32_t x0 = f.w[i].x, x1 = f.w[i].y, x2 = f.w[i].z, x3 = f.w[i].w;
+    v[0] = __builtin_bit_cast(float, x0), v[1] = __builtin_bit_cast(float, x1);
+    v[2] = __builtin_bit_cast(float, x2), v[3] = __builtin_bit_cast(float, x3);
+  } else if constexpr (XT == LLMP_X_BF16) {
+    v[0] = Bf16BitsToFloat(w.x & 0xFFFFu), v[1] = Bf16BitsToFloat(w.x >> 16);
+    v[2] = Bf16BitsToFloat(w.y & 0xFFFFu), v[3] = Bf16BitsToFloat(w.y >> 16);
+  } else {
+    v[0] = HalfBitsToFloat(w.x & 0xFFFFu), v[1] = HalfBitsToFloat(w.x >> 16);
+    v[2] = HalfBitsToFloat(w.y & 0xFFFFu), v[3] = HalfBitsToFloat(w.y >> 16);
+  }
+}
 __device__ __forceinline__ uint32_t FlatLdsAddress(const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); }
 __device__ __forceinline__ void FlatLdsWrite16(uint32_t at, FrontWords v) { asm volatile("ds_write_b128 %0, %1" : : "v"(at), "v"(v) : "memory"); }
 __device__ __forceinline__ void FlatLdsWrite4(uint32_t at, uint32_t v) { asm volatile("ds_write_b32 %0, %1" : : "v"(at), "v"(v) : "memory"); }
@@ -196,6 +263,26 @@ struct FormatQ4K {
       reinterpret_cast<int16_t*>(record + 320)[g] = static_cast<int16_t>(s);
     }
   }
+
+  // StageX with the record written by instructions (see StageQ8Asm below).
+  static __device__ __forceinline__ void StageXAsm(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    const uint32_t record = FlatLdsAddress(token) + static_cast<uint32_t>((b >> 3) * kRecord);
+    const int g = b & 7;
+    FlatLdsWrite4(record + g * 32 + lane8 * 4, q.codes);
+    int s = Dot4(0x01010101, static_cast<int>(q.codes), 0);
+    s += ShflXor(s, 1);
+    s += ShflXor(s, 2);
+    s += ShflXor(s, 4);
+    if (lane8 == 0) {
+      const float d8 = HalfBitsToFloat(FloatToHalfBits(q.d));
+      FlatLdsWrite4(record + 256 + g * 4, __builtin_bit_cast(uint32_t, d8));
+      FlatLdsWrite4(record + 288 + g * 4, __builtin_bit_cast(uint32_t, d8 * static_cast<float>(s)));
+      FlatLdsWrite2(record + 320 + g * 2, static_cast<uint32_t>(s));
+    }
+  }
+  static constexpr bool kStagesXUnderLoads = true;
 
   // One Q8_1 block (nine dwords), one thread.
   static __device__ __forceinline__ void StageQ8(const uint32_t (&w)[9], int b, uint8_t* token) {
@@ -332,6 +419,9 @@ template <int P, bool kDump>
 struct FormatQ5K : FormatQ4K {
   static constexpr int kUnitBytes = 176;
   static constexpr int kBlockBytes = 176;
+  // (Staging under the tile's loads is Q4_K's and Q8_0's own: not inherited.)
+  static constexpr bool kStagesUnderLoads = false;
+  static constexpr bool kStagesXUnderLoads = false;
 
   template <int P, bool kDump>
   static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
@@ -432,6 +522,8 @@ struct FormatQ5K : FormatQ4K {
 struct FormatQ6K : FormatQ4K {
   static constexpr int kUnitBytes = 210;
   static constexpr int kBlockBytes = 210;
+  static constexpr bool kStagesUnderLoads = false;
+  static constexpr bool kStagesXUnderLoads = false;
   static constexpr int kDumpInts = 16;  // the sixteen sub-blocks' sums
 
   template <int P, bool kDump>
@@ -1341,6 +1433,28 @@ __device__ __forceinline__ void StageRecordsX(const void* __restrict__ x, int k,
   }
 }
 
+template <class F, class = void>
+struct StagesXUnderLoads : std::false_type {};
+template <class F>
+struct StagesXUnderLoads<F, std::void_t<decltype(F::kStagesXUnderLoads)>> : std::bool_constant<F::kStagesXUnderLoads> {};
+
+// The front pieces quantized and their records written by instructions; every block of the row is a front block
+// (the launcher sees to it).
+template <class F, int XT>
+__device__ __forceinline__ void StageRecordsXAsm(const FrontXAsm<XT>& front, int k, uint8_t* token) {
+  const int blocks = k / 32;
+  const int sweep = blockDim.x >> 3;
+#pragma unroll
+  for (int i = 0; i < kFront; ++i) {
+    const int b = (threadIdx.x >> 3) + i * sweep;
+    if (b < blocks) {  // whole 8-lane groups together
+      float v[4];
+      FrontValues<XT>(front, i, v);
+      F::StageXAsm(v, b, token);
+    }
+  }
+}
+
 // Formats whose records of Q8_1 activations are staged by instructions, under the first tile's loads.
 template <class F, class = void>
 struct StagesUnderLoads : std::false_type {};
@@ -1492,12 +1606,14 @@ __device__ __forceinline__ void AwaitAllBut(int left) {
 }
 
 // grid (workgroups, slots); LDS: P tokens' records, then a tile buffer a wave.
-// kUnder: the Q8_1 activations' records are staged under the first tile's loads (loads and LDS writes by
-// instructions, a barrier for LDS alone), for launches whose waves take one tile each: the launch is then one trip
-// to memory, and the trip for the activations and their staging no longer stand in front of it and behind it. With
-// two tiles a wave it measured slower (the gate/up pair 14.7 to 15.2 us against 14.2): there the waves do better
-// entering the first products together.
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep, bool kUnder = false>
+// kUnder (1 or 2): the activations' records are staged under the first tile's loads: the activations loaded and
+// the records written by instructions, and with 1 a barrier for LDS alone. Over Q8_1 activations it is for launches
+// whose waves take one tile each: the launch is then one trip to memory, and the trip for the activations and their
+// staging no longer stand in front of it and behind it; with two tiles a wave it measured slower (the gate/up pair
+// 14.7 to 15.2 us against 14.2: there the waves do better entering the first products together). Over unquantized
+// activations the staging is their quantization, some four hundred vector instructions a wave, and running it under
+// the loads pays whatever the tiles a wave (the gate/up pair 16.5 -> 14.6-14.9 us; 2 keeps the full barrier).
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep, int kUnder = 0>
 __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void VecQFlat(const VecQArgs a, const int rows_per_tile) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   __shared__ int pairs[kMaxPairs];
@@ -1562,9 +1678,11 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
     const int m = min(P, n - p0);
     if (p0 > 0) __syncthreads();  // the last pass's readers of the records
     // The activations' first loads, then the wave's first tile, then the staging.
-    constexpr bool kAsmFront = kUnder;
+    constexpr bool kAsmFront = kUnder != 0 && XT < 0;
+    constexpr bool kAsmX = kUnder != 0 && XT >= 0;
     const void* rows_x[P];
-    FrontX front_x[XT < 0 ? 1 : P];
+    FrontX front_x[XT < 0 || kAsmX ? 1 : P];
+    FrontXAsm<XT < 0 ? 0 : XT> front_xa[kAsmX ? P : 1];
     FrontQ8 front_q[XT < 0 && !kAsmFront ? P : 1];
     FrontQ8Asm front_a[kAsmFront ? P : 1];
 #pragma unroll
@@ -1585,7 +1703,11 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
           const int64_t at = token * a.x_token + slot * a.x_slot;
           rows_x[j] = XT == LLMP_X_F32 ? static_cast<const void*>(static_cast<const float*>(a.x) + at)
                                        : static_cast<const void*>(static_cast<const uint16_t*>(a.x) + at);
-          front_x[j] = LoadFrontX<XT>(rows_x[j], d.ncols_x);
+          if constexpr (kAsmX) {
+            front_xa[j] = LoadFrontXAsm<XT>(rows_x[j], d.ncols_x);
+          } else {
+            front_x[j] = LoadFrontX<XT>(rows_x[j], d.ncols_x);
+          }
         }
       }
     }
@@ -1603,6 +1725,12 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
         if (j < m) AwaitFront(front_a[j], tile_loads);
       }
     }
+    if constexpr (kAsmX) {
+#pragma unroll
+      for (int j = 0; j < P; ++j) {
+        if (j < m) AwaitFrontX(front_xa[j], tile_loads);
+      }
+    }
 #pragma unroll
     for (int j = 0; j < P; ++j) {
       if (j < m) {
@@ -1611,6 +1739,8 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
           StageRecordsQ8Asm<F>(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_a[j], records);
         } else if constexpr (XT < 0) {
           StageRecordsQ8<F>(static_cast<const uint8_t*>(rows_x[j]), d.ncols_x / 32, front_q[j], records);
+        } else if constexpr (kAsmX) {
+          StageRecordsXAsm<F, XT>(front_xa[j], d.ncols_x, records);
         } else {
           StageRecordsX<F, XT>(rows_x[j], d.ncols_x, front_x[j], records);
         }
@@ -1618,7 +1748,7 @@ __global__ __launch_bounds__(kDeep ? kGroup : 2 * kGroup, kDeep ? 2 : 4) void Ve
     }
     // The records are staged; from here the waves run alone. (A barrier for LDS alone where the staging ran under
     // the tile's loads: __syncthreads would wait for those to land as well.)
-    if constexpr (kAsmFront) {
+    if constexpr (kUnder == 1) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
     } else {
@@ -1831,7 +1961,7 @@ inline bool PlanFits(const FlatPlan& p) { return p.lds <= (p.wide ? kWideLdsLimi
 constexpr size_t kDeepLdsLimit = 160 * 1024 - 1024;  // one workgroup, beside the kernel's own few words
 int g_compute_units = 0;
 
-template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false, bool kUnder = false>
+template <class F, int P, bool kGlu, int XT, bool kDump, bool kPacked, bool kDeep = false, int kUnder = 0>
 void LaunchK(const VecQArgs& a, dim3 grid, const FlatPlan& plan, hipStream_t stream) {
   static bool sized = false;  // more than 64 KB of dynamic LDS must be asked for once
   if (!AllowLds(reinterpret_cast<const void*>(&VecQFlat<F, P, kGlu, XT, kDump, kPacked, kDeep, kUnder>), static_cast<int>(kDeepLdsLimit), &sized)) return;
@@ -1854,7 +1984,25 @@ void LaunchT(const VecQArgs& a, dim3 grid, const FlatPlan& plan, bool deep, hipS
     // One tile a wave at most: the records staged under its loads.
     const int tiles = (a.d.nrows + plan.rows - 1) / plan.rows;
     if (packed && tiles <= static_cast<int>(grid.x) * plan.waves) {
-      LaunchK<F, P, kGlu, XT, false, true, false, true>(a, grid, plan, stream);
+      LaunchK<F, P, kGlu, XT, false, true, false, 1>(a, grid, plan, stream);
+      return;
+    }
+  }
+  if constexpr (P == 1 && XT >= 0 && StagesXUnderLoads<F>::value) {
+    // Unquantized activations quantized under the first tile's loads: rows whose blocks are all front blocks,
+    // aligned for the pieces' loads.
+    const int tiles = (a.d.nrows + plan.rows - 1) / plan.rows;
+    const int64_t align = XT == LLMP_X_F32 ? 16 : 8, width = XT == LLMP_X_F32 ? 4 : 2;
+    const bool aligned = reinterpret_cast<uintptr_t>(a.x) % align == 0 && (a.x_token * width) % align == 0 &&
+                         (a.x_slot * width) % align == 0;
+    const bool front = a.d.ncols_x / 32 <= kFront * (plan.waves * kWave / 8);
+    if (packed && aligned && front && a.d.ncols_x >= 32) {
+      // One tile a wave: the barrier for LDS alone; more: the full barrier, which keeps the waves together.
+      if (tiles <= static_cast<int>(grid.x) * plan.waves) {
+        LaunchK<F, P, kGlu, XT, false, true, false, 1>(a, grid, plan, stream);
+      } else {
+        LaunchK<F, P, kGlu, XT, false, true, false, 2>(a, grid, plan, stream);
+      }
       return;
     }
   }
