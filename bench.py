@@ -1,10 +1,12 @@
 """Benchmark of the quantized mat-vec hot path on one MI355X.
 
-A step is the decode-time gate/up product of one token: llmp.q8_1 (the activation's
-quantization to Q8_1) followed by llmp.vecq, the fused Q4_K gate/up GEGLU mat-vec (hidden
-3840, two 15360-row matrices), over one of several distinct weight copies, rotated so that
-neither L2 nor the 256 MB Infinity Cache holds them. --fused makes it the single launch that
-quantizes the bf16 activation inside the kernel.
+A step is the decode-time gate/up product of one token: the activation's quantization to Q8_1
+(llmp.q8_1) and the fused Q4_K gate/up GEGLU mat-vec over its blocks (llmp.vecq; hidden 3840, two
+15360-row matrices), over one of several distinct weight copies, rotated so that neither L2 nor
+the 256 MB Infinity Cache holds them. By default the step is one launch, which quantizes the bf16
+activation inside the kernel under its first tile's loads (the same bits out); --two-launches
+makes it the reference's two operations, llmp.q8_1 followed by llmp.vecq, which the default run
+times beside it (`two_launch_step`).
 Prints one JSON line; see --help. `other_configs` holds the other four benchmark configurations (Q8_0 mat-vec,
 MXFP8 GEMM, the routed-expert layer at 1, 16 and 512 tokens, the EXL3 linear at 1 and 16 rows), each with the
 roofline of its dominant kernel and the CPU oracle timed beside it; `--only <key>` runs one of them alone."""
@@ -108,6 +110,7 @@ def _traffic(fetch_kib, write_kib):
 
 PROFILED_TRAFFIC = {
     "q4_k_gate_up_geglu_b1": int(round((32478.4 * 1.9988 + 60.1) * 1024)),
+    "q4_k_gate_up_geglu_b1_one_launch": int(round((32505.0 * 1.9988 + 60.1) * 1024)),
     "q8_0_matvec_4096x4096_b1": _traffic(8768.0, 16.0),
     # A weight row a lane asks for 144 bytes a row a load, ragged against the 64-byte units HBM is fetched in; the
     # unit two neighbouring super-blocks share is often fetched for each: 1.3 to 1.4 times the algorithmic bytes.
@@ -683,8 +686,8 @@ def block_formats(device):
 
 
 def measured_traffic(args):
-    if args.tokens == 1 and args.variant == -1 and not args.fused:
-        return PROFILED_TRAFFIC["q4_k_gate_up_geglu_b1"]
+    if args.tokens == 1 and args.variant == -1:
+        return PROFILED_TRAFFIC["q4_k_gate_up_geglu_b1_one_launch" if args.fused else "q4_k_gate_up_geglu_b1"]
     return None
 
 
@@ -702,9 +705,10 @@ def main():
                          "the KV cache store")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of the weights' size (for scaling hardware counters)")
-    ap.add_argument("--fused", action="store_true",
-                    help="a step is one launch that quantizes the activations in the kernel, instead of "
-                         "llmp.q8_1 followed by llmp.vecq over its Q8_1 blocks (the reference's two operations)")
+    ap.add_argument("--two-launches", action="store_true",
+                    help="a step is llmp.q8_1 followed by llmp.vecq over its Q8_1 blocks (the reference's two "
+                         "operations) instead of the one launch that quantizes the activations in the kernel")
+    ap.add_argument("--fused", action="store_true", help="the default since the one launch became the faster step; kept for old command lines")
     ap.add_argument("--eager", action="store_true", help="launch each step from Python instead of a graph")
     ap.add_argument("--only", default=None,
                     help="run one of the other configurations alone (its key in other_configs) and print its entry: "
@@ -712,6 +716,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not built")
+    args.fused = not args.two_launches
 
     import numpy as np
     import torch
@@ -748,15 +753,18 @@ def main():
     x32 = torch.from_numpy(x).to(device)
     q8 = ops.quantize_q8_1(x32)
 
-    def step(i):
+    def two_launches(i):
         c = i % copies
-        if not args.fused:
-            ops.quantize_q8_1(x32, out=q8.view(1, args.tokens, -1))
-            ops.vecq(ops.TYPE_Q4_K, ups[c], q8, K, N, gate=gates[c], tokens=args.tokens, glu=ops.GLU_GEGLU,
-                     variant=args.variant, out=out)
-            return
+        ops.quantize_q8_1(x32, out=q8.view(1, args.tokens, -1))
+        ops.vecq(ops.TYPE_Q4_K, ups[c], q8, K, N, gate=gates[c], tokens=args.tokens, glu=ops.GLU_GEGLU,
+                 variant=args.variant, out=out)
+
+    def one_launch(i):
+        c = i % copies
         ops.vecq_fused(ops.TYPE_Q4_K, ups[c], xd, K, N, gate=gates[c], tokens=args.tokens,
                        glu=ops.GLU_GEGLU, variant=args.variant, out=out)
+
+    step = one_launch if args.fused else two_launches
 
     def kernel_only(i):
         c = i % copies
@@ -806,6 +814,9 @@ def main():
     # The dominant kernel alone (the mat-vec over ready Q8_1 blocks), the same rotation.
     kernel_ms, _ = timed_region(kernel_only if not args.fused else step)
     kernel_us = kernel_ms / args.steps * 1e3
+    # Beside it, the other form of the step and the mat-vec over ready Q8_1 blocks alone (not part of `value`).
+    other_ms, _ = timed_region(two_launches if args.fused else one_launch)
+    matvec_ms, _ = timed_region(kernel_only) if args.fused else (kernel_ms, None)
     ms = total_ms / args.steps
     value = WEIGHT_BYTES / (ms * 1e-3) / 1e9
     achieved = algorithmic_bytes(args.tokens) / (kernel_us * 1e-6) / 1e9
@@ -817,16 +828,21 @@ def main():
         "parity": "int32 sub-block sums bit-exact; fp32 outputs |got - want| <= 1e-3 * max(|want|, 1e-3 * rms(want)) "
                   "against the CPU oracle (a relative bound with an RMS floor, looser than a strict max-rel 1e-3)",
         "config": {"workload": f"GGML Q4_K fused gate/up GEGLU MMVQ, K={K}, N=2x{N}, batch {args.tokens}, "
-                               + ("bf16 activations quantized to q8_1 in-kernel" if args.fused else "fp32 activations through llmp.q8_1")
+                               + ("bf16 activations quantized to q8_1 in the kernel, one launch" if args.fused else "fp32 activations through llmp.q8_1, two launches")
                                + ", fp32 out",
                    "weight_copies_rotated": copies, "variant": args.variant, "launch": "eager" if args.eager else "hip graph",
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(args),
-                     "kernel": "VecQFlatQ4K (llmp.vecq, Q4_K, GLU)",
+                     "kernel": "VecQFlat<FormatQ4K, glu, bf16 activations quantized under the first tile's loads> (the step's one launch)"
+                               if args.fused else "VecQFlatQ4K (llmp.vecq, Q4_K, GLU)",
                      "algorithmic_bytes_per_launch": algorithmic_bytes(args.tokens),
                      "avg_launch_us": round(kernel_us, 3), "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
     }
+    other = {"us": round(other_ms / args.steps * 1e3, 3),
+             "GB/s": round(WEIGHT_BYTES / (other_ms / args.steps * 1e-3) / 1e9, 1),
+             "matvec_over_ready_q8_1_us": round(matvec_ms / args.steps * 1e3, 3)}
+    line["two_launch_step" if args.fused else "one_launch_step"] = other
     del gates, ups
     torch.cuda.empty_cache()
     # Beside the roofline: what a launch that only reads the same bytes takes on this box (not part of `value`).
