@@ -213,10 +213,12 @@ def other_configs(device, args, only=None):
             ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y)
 
         step_us = timed(step, 4 * len(copies))
+        one_launch_us = timed(lambda i: ops.vecq_fused(ops.TYPE_Q8_0, copies[i % len(copies)], x, k, n, out=y), 4 * len(copies))
         us = timed(lambda i: ops.vecq(ops.TYPE_Q8_0, copies[i % len(copies)], q8, k, n, out=y), 4 * len(copies))
         bytes_ = n * (k // 32) * 34 + k * 4 + n * 4
         entry = {"workload": "GGML Q8_0 mat-vec, N=4096, K=4096, batch 1, fp32 activations through llmp.q8_1",
                  "step_us": round(step_us, 2), "weight_GB/s_of_the_step": round(w.numel() / step_us / 1e3, 1),
+                 "step_us_as_one_launch": round(one_launch_us, 2),
                  "roofline": hbm_roofline("q8_0_matvec_4096x4096_b1", "VecQFlat<FormatQ8> (llmp.vecq, Q8_0)", bytes_, us),
                  "read_only_launch": read_only_launch(device, bytes_, us, args.eager)}
         if cpu:

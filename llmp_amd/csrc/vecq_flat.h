@@ -647,6 +647,22 @@ struct FormatQ8 {
     }
   }
 
+  // StageX with the record written by instructions (see FormatQ4K::StageQ8Asm).
+  static constexpr bool kStagesXUnderLoads = true;
+  static __device__ __forceinline__ void StageXAsm(const float (&v)[4], int b, uint8_t* token) {
+    const int lane8 = threadIdx.x & 7;
+    const Q8Block q = QuantizeQ8Block(v[0], v[1], v[2], v[3]);
+    const uint32_t record = FlatLdsAddress(token) + static_cast<uint32_t>((b >> 2) * kRecord);
+    const int j = b & 3;
+    const uint32_t at = record + 34 * j + 2 + lane8 * 4;
+    FlatLdsWrite2(at, q.codes & 0xFFFFu);
+    FlatLdsWrite2(at + 2, q.codes >> 16);
+    if (lane8 == 0) {
+      FlatLdsWrite2(record + 34 * j, 0u);  // against the weight block's scale
+      FlatLdsWrite4(record + 136 + 4 * j, __builtin_bit_cast(uint32_t, HalfBitsToFloat(FloatToHalfBits(q.d))));
+    }
+  }
+
   // One Q8_1 block (nine dwords), one thread. Blocks 1 and 3 of a unit have their codes on a
   // dword boundary (dwords 9-16 and 26-33); blocks 0 and 2 two bytes into dwords 0 and 17,
   // their nine dwords ending with the two bytes that face the next block's scale.
