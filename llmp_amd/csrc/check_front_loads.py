@@ -14,7 +14,7 @@ import tempfile
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-SOURCES = ("vecq_flat_q4k.hip", "vecq_flat_q8.hip")
+SOURCES = ("vecq_flat_q4k.hip", "vecq_flat_q8.hip", "vecq_flat_q5k.hip", "vecq_flat_q6k.hip")
 WAIT = re.compile(r"s_cmp_lt_u32 s\d+, 10\b")  # the first instruction of the wait's chain
 
 

@@ -419,9 +419,6 @@ template <int P, bool kDump>
 struct FormatQ5K : FormatQ4K {
   static constexpr int kUnitBytes = 176;
   static constexpr int kBlockBytes = 176;
-  // (Staging under the tile's loads is Q4_K's and Q8_0's own: not inherited.)
-  static constexpr bool kStagesUnderLoads = false;
-  static constexpr bool kStagesXUnderLoads = false;
 
   template <int P, bool kDump>
   static __device__ __forceinline__ void DotAt(const uint8_t* at, const uint8_t* records, int token_stride, int m,
@@ -522,8 +519,6 @@ struct FormatQ5K : FormatQ4K {
 struct FormatQ6K : FormatQ4K {
   static constexpr int kUnitBytes = 210;
   static constexpr int kBlockBytes = 210;
-  static constexpr bool kStagesUnderLoads = false;
-  static constexpr bool kStagesXUnderLoads = false;
   static constexpr int kDumpInts = 16;  // the sixteen sub-blocks' sums
 
   template <int P, bool kDump>
