@@ -1,4 +1,4 @@
-"""The one-token block product (vecq_flat.h) loads its activations' first blocks by instructions the compiler does
+"""The one-token block product (vecq_flat.h; and the one-token expert layer, moe_token.hip) loads its activations' first blocks by instructions the compiler does
 not track, so that it can wait for them by count after the first tile's loads are queued. Between such a load and
 that wait the destination registers hold nothing yet, and the compiler, which takes them for ordinary values, is free
 to copy or spill them. Nothing in the language forbids that, so this build step reads the compiler's assembly of every
@@ -14,8 +14,9 @@ import tempfile
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-SOURCES = ("vecq_flat_q4k.hip", "vecq_flat_q8.hip", "vecq_flat_q5k.hip", "vecq_flat_q6k.hip")
-WAIT = re.compile(r"s_cmp_lt_u32 s\d+, 10\b")  # the first instruction of the wait's chain
+SOURCES = ("vecq_flat_q4k.hip", "vecq_flat_q8.hip", "vecq_flat_q5k.hip", "vecq_flat_q6k.hip", "moe_token.hip")
+# The first instruction of the wait's chain, or (the one-token expert layer's second launch) a plain wait for all.
+WAIT = re.compile(r"s_cmp_lt_u32 s\d+, 10\b|^s_waitcnt vmcnt\(0\)$")
 
 
 def registers(code):
@@ -49,7 +50,7 @@ def check_kernel(name, body):
                 pending[r] = code
             loads += 1
             continue
-        if own and WAIT.search(code):
+        if own and WAIT.search(code.strip()):
             pending = {}
             continue
         if own and pending and re.match(r"s_(cmp|cbranch|waitcnt|branch)", code):
@@ -75,7 +76,7 @@ def check():
                 check=True, capture_output=True, timeout=1200)
             with open(out) as f:
                 assembly = f.read()
-        for m in re.finditer(r"^(_ZN\S*VecQFlat\S*):", assembly, re.M):
+        for m in re.finditer(r"^(_ZN\S*(?:VecQFlat|MoeTokenKernel)\S*):", assembly, re.M):
             body = assembly[m.end():assembly.index("s_endpgm", m.end())]
             if check_kernel(m.group(1), body) > 0:
                 kernels += 1

@@ -68,6 +68,9 @@ __global__ __launch_bounds__(kTokenThreads, 1) void MoeTokenKernel(const MoeToke
   uint8_t* const ring = lds + records + wave * (kWave * F::kUnitBytes);
   float* const meet = reinterpret_cast<float*>(lds + records + kTokenWaves * (kWave * F::kUnitBytes));  // [slot][row of the tile]
 
+  constexpr int kHeldSweeps = 4;
+  FrontWords held[kHeldSweeps];
+  const bool h_ahead = a.phase == 2 && d.ffn / 32 <= kHeldSweeps * (kWave >> 3);
   // ---- the token's experts: routed here, or (second launch of two) read back.
   if (a.phase != 2) {
     if (tid == 0) generation = __hip_atomic_load(words + 4 + blockIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -84,11 +87,38 @@ __global__ __launch_bounds__(kTokenThreads, 1) void MoeTokenKernel(const MoeToke
         }
       }
     }
-  } else if (tid < d.used) {
-    picked[tid] = d.ids[tid];
-    picked_weight[tid] = d.weights[tid];
+  } else {
+    // The second launch of two: a wave's slot's h (the launch before wrote it) is asked for here, ahead of the
+    // picks' loads (one trip to memory for both) and of the tile's, by instructions; quantized after the tile's
+    // loads are queued, with its records written by instructions, it no longer waits for the tile to land and
+    // then for a trip to memory a sweep (the compiler holds a write to LDS back while a load into LDS is in flight,
+    // so every sweep's loads waited for the one before). Rows of up to kHeldSweeps x 8 blocks.
+    // (One straight run of instructions from the loads to their wait, every lane taking part with its index held
+    // within bounds: a branch between them gave the compiler a place to copy the registers before the data was
+    // there, which the build's check of the assembly refuses.)
+    const int slot = min(wave, d.used - 1);
+#pragma unroll
+    for (int i = 0; i < kHeldSweeps; ++i) {
+      const int b = min((lane >> 3) + i * (kWave >> 3), d.ffn / 32 - 1);
+      const float* from = d.h + slot * d.ffn + b * 32 + (lane & 7) * 4;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(held[i]) : "v"(from) : "memory");
+    }
+    uint32_t pick, pick_weight;
+    {
+      const int32_t* from_ids = d.ids + min(tid, d.used - 1);
+      const float* from_weights = d.weights + min(tid, d.used - 1);
+      asm volatile("global_load_dword %0, %1, off" : "=&v"(pick) : "v"(from_ids) : "memory");
+      asm volatile("global_load_dword %0, %1, off" : "=&v"(pick_weight) : "v"(from_weights) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(held[0]), "+v"(held[1]), "+v"(held[2]), "+v"(held[3]), "+v"(pick), "+v"(pick_weight)
+                 :
+                 : "memory");
+    if (tid < d.used) {
+      picked[tid] = static_cast<int>(pick);
+      picked_weight[tid] = __builtin_bit_cast(float, pick_weight);
+    }
   }
-
   if (a.phase != 2) {
     // ---- first phase: the token's records, then h = GLU(gate x, up x) of every slot.
     const FrontX front = LoadFrontX<XT>(d.x, d.hidden);
@@ -176,7 +206,18 @@ __global__ __launch_bounds__(kTokenThreads, 1) void MoeTokenKernel(const MoeToke
   }
   // This wave's slot's h into its own records: eight lanes a block, the quantizer of llmp.q8_1.
   uint8_t* const my_records = lds + wave * (nsb_b * F::kRecord);
-  if (wave < d.used) {
+  if (h_ahead && wave < d.used) {
+#pragma unroll
+    for (int i = 0; i < kHeldSweeps; ++i) {
+      const int b = (lane >> 3) + i * (kWave >> 3);
+      if (b < d.ffn / 32) {  // whole 8-lane groups together
+        const uint32_t x0 = held[i].x, x1 = held[i].y, x2 = held[i].z, x3 = held[i].w;
+        const float v[4] = {__builtin_bit_cast(float, x0), __builtin_bit_cast(float, x1), __builtin_bit_cast(float, x2),
+                            __builtin_bit_cast(float, x3)};
+        F::StageXAsm(v, b, my_records);
+      }
+    }
+  } else if (wave < d.used) {
     const float* from = d.h + wave * d.ffn;
     for (int b = lane >> 3; b < d.ffn / 32; b += kWave >> 3) {
       float v[4];
